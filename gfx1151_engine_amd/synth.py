@@ -1,0 +1,85 @@
+"""Seeded synthetic tensors in the engine's on-disk byte layouts (numpy, host side).
+
+q4cp blob  (hgn dtype 5, reference src/hgn.h:2-9,219-240):
+    [64 B: 16 x f32 codebook][rows*cols/2 B codes, row-major, low nibble first]
+    [rows x scale_stride B: cols/32 fp16 scales, record padded to 16 B]
+Q4_K rows  (GGUF type 12, reference src/gguf.h:408-441): cols/256 super-blocks of 144 B:
+    [fp16 d][fp16 dmin][12 B packed 6-bit scales/mins][128 B codes]
+"""
+import numpy as np
+
+ZP8_CODEBOOK = np.arange(16, dtype=np.float32) - 8.0  # zero-point 8: w = (code - 8) * scale
+
+
+def q4cp_scale_stride(cols):
+    return ((cols // 32 * 2) + 15) & ~15
+
+
+def q4cp_blob_bytes(rows, cols):
+    return 64 + rows * cols // 2 + rows * q4cp_scale_stride(cols)
+
+
+def make_q4cp(rng, rows, cols, codebook=None, scale_std=0.01, scales=None, codes=None):
+    """Random q4cp blob. scales: fp16 |N(0,1)|*scale_std unless given ([rows][cols/32] float16)."""
+    assert cols % 32 == 0
+    cb = ZP8_CODEBOOK if codebook is None else np.asarray(codebook, np.float32)
+    ss = q4cp_scale_stride(cols)
+    blob = np.zeros(q4cp_blob_bytes(rows, cols), np.uint8)
+    blob[:64] = cb.view(np.uint8)
+    nb = rows * cols // 2
+    blob[64:64 + nb] = (rng.integers(0, 256, nb, dtype=np.uint8) if codes is None
+                        else np.asarray(codes, np.uint8).reshape(-1))
+    if scales is None:
+        scales = (np.abs(rng.standard_normal((rows, cols // 32), dtype=np.float32)) * scale_std
+                  ).astype(np.float16)
+    rec = np.zeros((rows, ss // 2), np.float16)
+    rec[:, :cols // 32] = scales
+    blob[64 + nb:] = rec.view(np.uint8).reshape(-1)
+    return blob
+
+
+def q4k_row_bytes(cols):
+    return cols // 256 * 144
+
+
+def pack_scale_min_k4(sc, mn):
+    """Inverse of get_scale_min_k4: 8 six-bit scales + 8 six-bit mins -> 12 bytes."""
+    sc = np.asarray(sc, np.uint8)
+    mn = np.asarray(mn, np.uint8)
+    q = np.zeros(sc.shape[:-1] + (12,), np.uint8)
+    for j in range(4):
+        q[..., j] = (sc[..., j] & 63) | ((sc[..., j + 4] >> 4) << 6)
+        q[..., j + 4] = (mn[..., j] & 63) | ((mn[..., j + 4] >> 4) << 6)
+        q[..., j + 8] = (sc[..., j + 4] & 0xF) | ((mn[..., j + 4] & 0xF) << 4)
+    return q
+
+
+def make_q4k(rng, rows, cols, scale_std=0.01):
+    """Random Q4_K rows: d,dmin = fp16(|N(0,1)|*scale_std); sub-scales/mins uniform [0,63]."""
+    assert cols % 256 == 0
+    nb = rows * cols // 256
+    blk = np.zeros((nb, 144), np.uint8)
+    dd = (np.abs(rng.standard_normal((nb, 2), dtype=np.float32)) * scale_std).astype(np.float16)
+    blk[:, 0:4] = dd.view(np.uint8)
+    sc = rng.integers(0, 64, (nb, 8), dtype=np.uint8)
+    mn = rng.integers(0, 64, (nb, 8), dtype=np.uint8)
+    blk[:, 4:16] = pack_scale_min_k4(sc, mn)
+    blk[:, 16:] = rng.integers(0, 256, (nb, 128), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+def f32_to_bf16_bits(a):
+    """Round-to-nearest-even f32 -> bf16 bit patterns (uint16)."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    r = ((u >> 16) & 1) + 0x7FFF
+    return ((u + r) >> 16).astype(np.uint16)
+
+
+def bf16_round(a):
+    return (f32_to_bf16_bits(a).astype(np.uint32) << 16).view(np.float32)
+
+
+def zipf_bias(rng, E, s=1.1, beta=1.0):
+    """Per-expert logit bias b_e = -beta*s*ln(rank_e) under a random rank permutation."""
+    rank = rng.permutation(E) + 1
+    return (-beta * s * np.log(rank)).astype(np.float32)

@@ -1,0 +1,437 @@
+/*
+ * moe_oracle.c — CPU oracle for the routed-expert MoE layer.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file restates, in plain C, the arithmetic of
+ * the reference engine's CPU path so that the HIP kernels can be checked
+ * against it.  Nothing in the product library links, loads or calls it; only
+ * tests, the smoke check and the benchmark's cpu_baseline leg do.
+ *
+ * Reference files followed (paths relative to the reference tree):
+ *   src/hgn.h:77-84      fp16 -> f32
+ *   src/hgn.h:219-261    q4cp blob layout, q4cp_parse / q4cp_row
+ *   src/gguf.h:328-336   scale_min_k4
+ *   src/gguf.h:408-441   Q4_K dequant_row
+ *   src/ref.cpp:55-56    sigmoid / silu
+ *   src/ref.cpp:68-77    matvec: fp64 sequential accumulate, f32 result
+ *   src/ref.cpp:563-637  Model::moe (router, top-k, experts, shared expert)
+ *   src/gpu/parts/10_ple_io.inc:784-825  expert-sorted permutation + tiles
+ *
+ * Pinning status of every function is listed in oracle/README.md; each one is
+ * checked in tests/ against the reference's own code built under oracle/_ref
+ * and against closed forms / brute force.  None is "parity unpinned".
+ *
+ * One deliberate addition: std::partial_sort in src/ref.cpp:587 leaves the
+ * order of equal probabilities unspecified.  The oracle fixes it to "lowest
+ * expert index first", the rule the reference's GPU router states
+ * (src/gpu/parts/20_kernels_gemv.inc:1488-1494,1545).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ---- weight format tags (shared with the library header by value) ---- */
+enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12 };
+
+/* src/hgn.h:77-84 and src/gguf.h:318-325 (same function twice in the reference) */
+ORC_API float orc_fp16_to_f32(uint16_t h) {
+  uint32_t s = (h >> 15) & 1u, e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+  float v;
+  if (e == 0) v = (float)m * 0x1p-24f;
+  else if (e == 31) v = m ? NAN : INFINITY;
+  else v = ldexpf((float)(1024 + m), (int)e - 25);
+  return s ? -v : v;
+}
+
+static inline float bf16_to_f32(uint16_t b) { /* src/hgn.h:86-91 */
+  uint32_t u = (uint32_t)b << 16;
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+/* ---- q4cp: [64 B codebook][rows*cols/2 codes][rows x scale_stride] ---- */
+ORC_API uint64_t orc_q4cp_scale_stride(uint64_t cols) { /* src/hgn.h:231 */
+  return ((cols / 32 * 2) + 15) & ~15ULL;
+}
+ORC_API uint64_t orc_q4cp_blob_bytes(uint64_t rows, uint64_t cols) { /* src/hgn.h:232 */
+  return 64 + rows * cols / 2 + rows * orc_q4cp_scale_stride(cols);
+}
+
+/* src/hgn.h:249-261: one row -> out[cols] */
+ORC_API void orc_q4cp_row(const uint8_t* blob, uint64_t rows, uint64_t cols, uint64_t row,
+                          float* out) {
+  const float* cb = (const float*)blob;
+  const uint8_t* codes = blob + 64 + row * (cols / 2);
+  const uint64_t ss = orc_q4cp_scale_stride(cols);
+  const uint8_t* srec = blob + 64 + rows * cols / 2 + row * ss;
+  for (uint64_t g = 0; g < cols / 32; g++) {
+    uint16_t sh;
+    memcpy(&sh, srec + 2 * g, 2);
+    const float s = orc_fp16_to_f32(sh);
+    for (uint64_t j = 0; j < 32; j++) {
+      const uint64_t i = g * 32 + j;
+      const uint8_t byte = codes[i / 2];
+      const uint8_t nib = (j % 2 == 0) ? (byte & 0xf) : (byte >> 4);
+      out[i] = cb[nib] * s;
+    }
+  }
+}
+
+ORC_API void orc_q4cp_rows(const uint8_t* blob, uint64_t rows, uint64_t cols, uint64_t row0,
+                           uint64_t nrows, float* out) {
+  for (uint64_t r = 0; r < nrows; r++) orc_q4cp_row(blob, rows, cols, row0 + r, out + r * cols);
+}
+
+/* ---- GGUF Q4_K: 144-byte super-blocks of 256 elements ---- */
+ORC_API void orc_scale_min_k4(int j, const uint8_t* q, uint8_t* d, uint8_t* m) { /* gguf.h:328-336 */
+  if (j < 4) {
+    *d = q[j] & 63;
+    *m = q[j + 4] & 63;
+  } else {
+    *d = (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4);
+    *m = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+  }
+}
+
+/* src/gguf.h:408-441, Q4_K branch.  The products d*sc, dmin*m and (d*sc)*q are
+ * exact in f32 (11-bit fp16 significand times a 6-bit and a 4-bit integer), so
+ * the value is one correctly rounded f32 subtraction whatever the contraction
+ * setting of the compiler. */
+ORC_API void orc_q4k_row(const uint8_t* src, float* y, uint64_t k) {
+  for (uint64_t b = 0; b < k / 256; b++, src += 144) {
+    uint16_t dh, mh;
+    memcpy(&dh, src, 2);
+    memcpy(&mh, src + 2, 2);
+    const float d = orc_fp16_to_f32(dh), dmin = orc_fp16_to_f32(mh);
+    const uint8_t* sc = src + 4;
+    const uint8_t* ql = src + 16;
+    float* yy = y + b * 256;
+    int is = 0;
+    for (int j = 0; j < 256; j += 64) {
+      uint8_t s0, m0, s1, m1;
+      orc_scale_min_k4(is + 0, sc, &s0, &m0);
+      orc_scale_min_k4(is + 1, sc, &s1, &m1);
+      const float d1 = d * s0, dm1 = dmin * m0, d2 = d * s1, dm2 = dmin * m1;
+      for (int l = 0; l < 32; l++) *yy++ = d1 * (float)(ql[l] & 0xF) - dm1;
+      for (int l = 0; l < 32; l++) *yy++ = d2 * (float)(ql[l] >> 4) - dm2;
+      ql += 32;
+      is += 2;
+    }
+  }
+}
+ORC_API uint64_t orc_q4k_row_bytes(uint64_t k) { return k / 256 * 144; } /* gguf.h:79-84 */
+
+/* ---- generic "row r of a weight matrix" in any supported storage ---- */
+typedef struct {
+  int dtype;            /* ORC_F32 / ORC_BF16 / ORC_Q4CP / ORC_Q4K */
+  const uint8_t* data;  /* f32/bf16: row-major; q4cp: whole blob; q4k: row-major raw blocks */
+  uint64_t rows, cols;  /* logical matrix (q4cp: rows of the whole blob) */
+} orc_mat;
+
+static void mat_row(const orc_mat* W, uint64_t r, float* out) {
+  switch (W->dtype) {
+    case ORC_F32: memcpy(out, W->data + r * W->cols * 4, W->cols * 4); break;
+    case ORC_BF16: {
+      const uint16_t* p = (const uint16_t*)W->data + r * W->cols;
+      for (uint64_t c = 0; c < W->cols; c++) out[c] = bf16_to_f32(p[c]);
+      break;
+    }
+    case ORC_Q4CP: orc_q4cp_row(W->data, W->rows, W->cols, r, out); break;
+    case ORC_Q4K: orc_q4k_row(W->data + r * orc_q4k_row_bytes(W->cols), out, W->cols); break;
+    default: memset(out, 0, W->cols * 4);
+  }
+}
+
+/* src/ref.cpp:75-77,85-87: acc (double) += (double)w * x, c ascending, then (float) */
+static inline float dot_f64(const float* w, const float* x, uint64_t n) {
+  double acc = 0;
+  for (uint64_t c = 0; c < n; c++) acc += (double)w[c] * x[c];
+  return (float)acc;
+}
+
+static inline float sigmoidf_ref(float x) { return 1.f / (1.f + expf(-x)); } /* ref.cpp:55 */
+static inline float siluf_ref(float x) { return x / (1.f + expf(-x)); }      /* ref.cpp:56 */
+
+/* ---- router: src/ref.cpp:565-594 -------------------------------------- */
+/* logits[E] (f32, already the (float) of the fp64 dot) -> probs, ids, weights.
+ * ids are in selection order (descending probability, ties -> lowest index). */
+ORC_API void orc_softmax_topk(const float* logits, int E, int k, float* probs, int* ids,
+                              float* ws) {
+  double mx = -1e300;
+  for (int i = 0; i < E; i++) mx = fmax(mx, (double)logits[i]);
+  double se = 0;
+  for (int i = 0; i < E; i++) {
+    probs[i] = (float)exp((double)logits[i] - mx);
+    se += probs[i];
+  }
+  for (int i = 0; i < E; i++) probs[i] = (float)(probs[i] / se);
+  /* k rounds of arg-max over what is left; strict '>' keeps the lowest index */
+  uint8_t* taken = (uint8_t*)calloc((size_t)E, 1);
+  for (int j = 0; j < k; j++) {
+    int best = -1;
+    for (int i = 0; i < E; i++)
+      if (!taken[i] && (best < 0 || probs[i] > probs[best])) best = i;
+    ids[j] = best;
+    taken[best] = 1;
+  }
+  free(taken);
+  double wsum = 0;
+  for (int j = 0; j < k; j++) wsum += probs[ids[j]];
+  for (int j = 0; j < k; j++) ws[j] = (float)(probs[ids[j]] / wsum);
+}
+
+/* router logits for T tokens: logits[t][e] = (float) sum_c (double)W[e][c]*x[t][c] */
+ORC_API void orc_router_logits(const orc_mat* Wr, const float* x, int T, float* logits) {
+  const int E = (int)Wr->rows;
+  const uint64_t d = Wr->cols;
+#pragma omp parallel
+  {
+    float* wr = (float*)malloc(d * 4);
+#pragma omp for schedule(static)
+    for (int e = 0; e < E; e++) {
+      mat_row(Wr, (uint64_t)e, wr);
+      for (int t = 0; t < T; t++) logits[(size_t)t * E + e] = dot_f64(wr, x + (size_t)t * d, d);
+    }
+    free(wr);
+  }
+}
+
+/* ids/ws rows are id_stride wide (the reference pads to 16), first k valid. */
+ORC_API void orc_router(const orc_mat* Wr, const float* bias, const float* x, int T, int k,
+                        int id_stride, float* logits_out, int* ids, float* ws) {
+  const int E = (int)Wr->rows;
+  float* logits = logits_out ? logits_out : (float*)malloc((size_t)T * E * 4);
+  orc_router_logits(Wr, x, T, logits);
+  if (bias) /* synthetic skew only: added in f32 to the f32 logit */
+    for (int t = 0; t < T; t++)
+      for (int e = 0; e < E; e++) logits[(size_t)t * E + e] += bias[e];
+#pragma omp parallel
+  {
+    float* probs = (float*)malloc((size_t)E * 4);
+#pragma omp for schedule(static)
+    for (int t = 0; t < T; t++)
+      orc_softmax_topk(logits + (size_t)t * E, E, k, probs, ids + (size_t)t * id_stride,
+                       ws + (size_t)t * id_stride);
+    free(probs);
+  }
+  if (!logits_out) free(logits);
+}
+
+/* ---- expert-sorted permutation: 10_ple_io.inc:784-811 (stable sort by expert) ---- */
+ORC_API void orc_route(const int* ids, const float* ws, int P, int k, int E, int id_stride,
+                       int* tokidx, float* pw, int* eoff, int* pairids) {
+  int* cnt = (int*)calloc((size_t)E + 1, sizeof(int));
+  for (int p = 0; p < P * k; p++) cnt[ids[(p / k) * id_stride + p % k] + 1]++;
+  eoff[0] = 0;
+  for (int e = 0; e < E; e++) eoff[e + 1] = eoff[e] + cnt[e + 1];
+  int* cur = (int*)malloc((size_t)E * sizeof(int));
+  memcpy(cur, eoff, (size_t)E * sizeof(int));
+  for (int p = 0; p < P * k; p++) { /* ascending original pair index = stable */
+    const int t = p / k, s = p % k, e = ids[t * id_stride + s];
+    const int q = cur[e]++;
+    tokidx[q] = t;
+    pw[q] = ws[t * id_stride + s];
+    if (pairids) {
+      int rank = 0;
+      for (int j = 0; j < k; j++) rank += ids[t * id_stride + j] < e;
+      pairids[t * k + rank] = q;
+    }
+  }
+  free(cur);
+  free(cnt);
+}
+
+/* 10_ple_io.inc:813-825: split every expert's run into <=cap slot tiles */
+ORC_API int orc_tiles(const int* eoff, int E, int cap, int* tiles /* [n][3] */) {
+  int n = 0;
+  for (int e = 0; e < E; e++) {
+    const int first = eoff[e], ne = eoff[e + 1] - first;
+    for (int j = 0; j * cap < ne; j++) {
+      tiles[3 * n + 0] = e;
+      tiles[3 * n + 1] = first + j * cap;
+      tiles[3 * n + 2] = ne - j * cap < cap ? ne - j * cap : cap;
+      n++;
+    }
+  }
+  return n;
+}
+
+/* ---- the layer: src/ref.cpp:596-636 ----------------------------------- */
+typedef struct {
+  int d, mid, E, k;
+  orc_mat router;          /* [E][d] */
+  const float* router_bias;/* optional [E] synthetic skew, may be NULL */
+  /* routed experts: either fused gate_up [E*2*mid][d] (q4cp) or separate gate/up [E*mid][d] */
+  orc_mat gate_up;         /* dtype<0 => use gate/up */
+  orc_mat gate, up;
+  orc_mat down;            /* [E*d][mid] */
+  /* shared expert (dense, one expert's shape) */
+  orc_mat sh_gate, sh_up, sh_down; /* [mid][d],[mid][d],[d][mid] */
+  orc_mat sh_sg;           /* [1][d] */
+  int has_shared;
+} orc_layer;
+
+static void expert_rows_gate_up(const orc_layer* L, int e, int r, float* out) {
+  /* row r in [0, 2*mid): gate rows first, then up rows (ref.cpp:613-615) */
+  if (L->gate_up.data) mat_row(&L->gate_up, (uint64_t)e * 2 * L->mid + r, out);
+  else if (r < L->mid) mat_row(&L->gate, (uint64_t)e * L->mid + r, out);
+  else mat_row(&L->up, (uint64_t)e * L->mid + (r - L->mid), out);
+}
+
+/*
+ * y[T][d] for the tokens listed in tok_list (n_list of them; NULL => all T).
+ * Per token the arithmetic is exactly Model::moe's; the loops are reordered
+ * (expert-major, each weight row dequantised once and used for every token
+ * routed to it) which changes no value: every dot product is an independent
+ * fp64 chain, and each token's f32 accumulation still runs in rank order.
+ * ids/ws are outputs ([T][id_stride]); hid_out (optional) is [T][k][mid].
+ */
+ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int* tok_list,
+                           int n_list, int id_stride, int* ids, float* ws, float* hid_out,
+                           float* y) {
+  const int d = L->d, mid = L->mid, E = L->E, k = L->k;
+  orc_router(&L->router, L->router_bias, x, T, k, id_stride, NULL, ids, ws);
+  const int n = tok_list ? n_list : T;
+  /* pair list grouped by expert (only tokens in the list) */
+  int* cnt = (int*)calloc((size_t)E + 1, sizeof(int));
+  for (int i = 0; i < n; i++) {
+    const int t = tok_list ? tok_list[i] : i;
+    for (int s = 0; s < k; s++) cnt[ids[t * id_stride + s] + 1]++;
+  }
+  for (int e = 0; e < E; e++) cnt[e + 1] += cnt[e];
+  int* cur = (int*)malloc((size_t)E * sizeof(int));
+  memcpy(cur, cnt, (size_t)E * sizeof(int));
+  int* pair_i = (int*)malloc((size_t)n * k * sizeof(int)); /* list index */
+  int* pair_s = (int*)malloc((size_t)n * k * sizeof(int)); /* rank */
+  for (int i = 0; i < n; i++) {
+    const int t = tok_list ? tok_list[i] : i;
+    for (int s = 0; s < k; s++) {
+      const int q = cur[ids[t * id_stride + s]]++;
+      pair_i[q] = i;
+      pair_s[q] = s;
+    }
+  }
+  free(cur);
+  /* per (list index, rank): guv[2*mid], hid[mid], dn[d] */
+  float* guv = (float*)malloc((size_t)n * k * 2 * mid * 4);
+  float* hid = (float*)malloc((size_t)n * k * mid * 4);
+  float* dn = (float*)malloc((size_t)n * k * d * 4);
+#pragma omp parallel
+  {
+    float* wr = (float*)malloc((size_t)(d > mid ? d : mid) * 4);
+#pragma omp for schedule(dynamic, 16) collapse(2)
+    for (int e = 0; e < E; e++)
+      for (int r = 0; r < 2 * mid; r++) {
+        if (cnt[e] == cnt[e + 1]) continue;
+        expert_rows_gate_up(L, e, r, wr);
+        for (int q = cnt[e]; q < cnt[e + 1]; q++) {
+          const int i = pair_i[q], t = tok_list ? tok_list[i] : i;
+          guv[((size_t)i * k + pair_s[q]) * 2 * mid + r] = dot_f64(wr, x + (size_t)t * d, d);
+        }
+      }
+#pragma omp for schedule(static)
+    for (int i = 0; i < n * k; i++)
+      for (int r = 0; r < mid; r++)
+        hid[(size_t)i * mid + r] =
+            siluf_ref(guv[(size_t)i * 2 * mid + r]) * guv[(size_t)i * 2 * mid + mid + r];
+#pragma omp for schedule(dynamic, 16) collapse(2)
+    for (int e = 0; e < E; e++)
+      for (int r = 0; r < d; r++) {
+        if (cnt[e] == cnt[e + 1]) continue;
+        mat_row(&L->down, (uint64_t)e * d + r, wr);
+        for (int q = cnt[e]; q < cnt[e + 1]; q++) {
+          const size_t ps = (size_t)pair_i[q] * k + pair_s[q];
+          dn[ps * d + r] = dot_f64(wr, hid + ps * mid, mid);
+        }
+      }
+    free(wr);
+  }
+  /* ref.cpp:621: acc[r] += w * (float)a2, ranks in order, f32 */
+#pragma omp parallel for schedule(static)
+  for (int i = 0; i < n; i++) {
+    const int t = tok_list ? tok_list[i] : i;
+    float* yt = y + (size_t)t * d;
+    for (int r = 0; r < d; r++) {
+      float acc = 0.f;
+      for (int s = 0; s < k; s++) acc += ws[t * id_stride + s] * dn[((size_t)i * k + s) * d + r];
+      yt[r] = acc;
+    }
+  }
+  if (hid_out)
+    for (int i = 0; i < n; i++) {
+      const int t = tok_list ? tok_list[i] : i;
+      memcpy(hid_out + (size_t)t * k * mid, hid + (size_t)i * k * mid, (size_t)k * mid * 4);
+    }
+  free(guv);
+  free(hid);
+  free(dn);
+  free(pair_i);
+  free(pair_s);
+  free(cnt);
+  if (!L->has_shared) return;
+  /* shared expert, ref.cpp:623-636 */
+  float* g1 = (float*)malloc((size_t)n * mid * 4);
+  float* u1 = (float*)malloc((size_t)n * mid * 4);
+  float* sg = (float*)malloc((size_t)n * 4);
+#pragma omp parallel
+  {
+    float* wr = (float*)malloc((size_t)(d > mid ? d : mid) * 4);
+#pragma omp for schedule(static)
+    for (int r = 0; r < mid; r++) {
+      mat_row(&L->sh_gate, (uint64_t)r, wr);
+      for (int i = 0; i < n; i++) {
+        const int t = tok_list ? tok_list[i] : i;
+        g1[(size_t)i * mid + r] = dot_f64(wr, x + (size_t)t * d, d);
+      }
+      mat_row(&L->sh_up, (uint64_t)r, wr);
+      for (int i = 0; i < n; i++) {
+        const int t = tok_list ? tok_list[i] : i;
+        u1[(size_t)i * mid + r] = dot_f64(wr, x + (size_t)t * d, d);
+      }
+    }
+#pragma omp single
+    {
+      mat_row(&L->sh_sg, 0, wr);
+      for (int i = 0; i < n; i++) {
+        const int t = tok_list ? tok_list[i] : i;
+        sg[i] = sigmoidf_ref(dot_f64(wr, x + (size_t)t * d, d));
+      }
+    }
+#pragma omp for schedule(static)
+    for (int i = 0; i < n * mid; i++) g1[i] = siluf_ref(g1[i]) * u1[i];
+#pragma omp for schedule(static)
+    for (int r = 0; r < d; r++) {
+      mat_row(&L->sh_down, (uint64_t)r, wr);
+      for (int i = 0; i < n; i++) {
+        const int t = tok_list ? tok_list[i] : i;
+        const float ey = dot_f64(wr, g1 + (size_t)i * mid, mid);
+        y[(size_t)t * d + r] = y[(size_t)t * d + r] + sg[i] * ey; /* ref.cpp:636 */
+      }
+    }
+    free(wr);
+  }
+  free(g1);
+  free(u1);
+  free(sg);
+}
+
+ORC_API int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}
+ORC_API void orc_set_threads(int n) {
+#ifdef _OPENMP
+  omp_set_num_threads(n);
+#else
+  (void)n;
+#endif
+}

@@ -1,0 +1,282 @@
+"""ctypes binding of oracle/libmoe_oracle.so and (when built) oracle/_ref/libmoe_ref.so.
+
+TEST INFRASTRUCTURE ONLY: the checker for the HIP path, never the thing shipped or measured
+(except as bench.py's labelled cpu_baseline).  numpy arrays in, numpy arrays out.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+F32, BF16, Q4CP, Q4K = 1, 0, 5, 12
+
+
+def build(force=False):
+    """Compile the oracle (and the reference shim when /root/reference exists)."""
+    args = ["make", "-C", _HERE] + (["-B"] if force else [])
+    subprocess.run(args, check=True, stdout=subprocess.DEVNULL)
+
+
+class _Mat(C.Structure):
+    _fields_ = [("dtype", C.c_int), ("data", C.c_void_p), ("rows", C.c_uint64), ("cols", C.c_uint64)]
+
+
+class _Layer(C.Structure):
+    _fields_ = [("d", C.c_int), ("mid", C.c_int), ("E", C.c_int), ("k", C.c_int),
+                ("router", _Mat), ("router_bias", C.c_void_p),
+                ("gate_up", _Mat), ("gate", _Mat), ("up", _Mat), ("down", _Mat),
+                ("sh_gate", _Mat), ("sh_up", _Mat), ("sh_down", _Mat), ("sh_sg", _Mat),
+                ("has_shared", C.c_int)]
+
+
+_lib = None
+_ref = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        path = os.path.join(_HERE, "libmoe_oracle.so")
+        if not os.path.exists(path):
+            build()
+        _lib = C.CDLL(path)
+        _lib.orc_fp16_to_f32.restype = C.c_float
+        _lib.orc_fp16_to_f32.argtypes = [C.c_uint16]
+        _lib.orc_q4cp_scale_stride.restype = C.c_uint64
+        _lib.orc_q4cp_scale_stride.argtypes = [C.c_uint64]
+        _lib.orc_q4cp_blob_bytes.restype = C.c_uint64
+        _lib.orc_q4cp_blob_bytes.argtypes = [C.c_uint64, C.c_uint64]
+        _lib.orc_q4k_row_bytes.restype = C.c_uint64
+        _lib.orc_q4k_row_bytes.argtypes = [C.c_uint64]
+        _lib.orc_num_threads.restype = C.c_int
+    return _lib
+
+
+def ref():
+    """The reference's own code (oracle/_ref/libmoe_ref.so) or None when not built."""
+    global _ref
+    if _ref is None:
+        path = os.path.join(_HERE, "_ref", "libmoe_ref.so")
+        if not os.path.exists(path):
+            return None
+        _ref = C.CDLL(path)
+        _ref.ref_fp16_to_f32.restype = C.c_float
+        _ref.ref_fp16_to_f32.argtypes = [C.c_uint16]
+        _ref.ref_q4k_row_bytes.restype = C.c_uint64
+        _ref.ref_q4k_row_bytes.argtypes = [C.c_uint64]
+    return _ref
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def _c(a, dt):
+    a = np.ascontiguousarray(a, dtype=dt)
+    return a
+
+
+class Mat:
+    """A weight matrix in one of the supported storages; keeps its bytes alive."""
+
+    def __init__(self, dtype, data, rows, cols):
+        self.dtype, self.rows, self.cols = dtype, int(rows), int(cols)
+        self.data = np.ascontiguousarray(data)
+        if dtype == Q4CP:
+            assert self.data.dtype == np.uint8 and self.data.size == lib().orc_q4cp_blob_bytes(rows, cols)
+        elif dtype == Q4K:
+            assert self.data.dtype == np.uint8 and self.data.size == rows * lib().orc_q4k_row_bytes(cols)
+        elif dtype == F32:
+            assert self.data.dtype == np.float32 and self.data.size == rows * cols
+        elif dtype == BF16:
+            assert self.data.dtype == np.uint16 and self.data.size == rows * cols
+
+    def c(self):
+        return _Mat(self.dtype, self.data.ctypes.data, self.rows, self.cols)
+
+    def dequant(self, row0=0, nrows=None):
+        nrows = self.rows - row0 if nrows is None else nrows
+        if self.dtype == Q4CP:
+            return q4cp_rows(self.data, self.rows, self.cols, row0, nrows)
+        if self.dtype == Q4K:
+            rb = lib().orc_q4k_row_bytes(self.cols)
+            return q4k_rows(self.data[row0 * rb:(row0 + nrows) * rb], nrows, self.cols)
+        if self.dtype == F32:
+            return self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].copy()
+        u = self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].astype(np.uint32) << 16
+        return u.view(np.float32)
+
+
+_NULL = _Mat(-1, None, 0, 0)
+
+
+def fp16_to_f32(h):
+    return float(lib().orc_fp16_to_f32(int(h)))
+
+
+def q4cp_rows(blob, rows, cols, row0, nrows):
+    blob = _c(blob, np.uint8)
+    out = np.empty((nrows, cols), np.float32)
+    lib().orc_q4cp_rows(_p(blob), C.c_uint64(rows), C.c_uint64(cols), C.c_uint64(row0),
+                        C.c_uint64(nrows), _p(out))
+    return out
+
+
+def q4k_rows(raw, nrows, k):
+    raw = _c(raw, np.uint8)
+    rb = lib().orc_q4k_row_bytes(k)
+    assert raw.size == nrows * rb
+    out = np.empty((nrows, k), np.float32)
+    for r in range(nrows):
+        lib().orc_q4k_row(C.c_void_p(raw.ctypes.data + r * rb), C.c_void_p(out.ctypes.data + r * k * 4),
+                          C.c_uint64(k))
+    return out
+
+
+def scale_min_k4(j, q12):
+    q12 = _c(q12, np.uint8)
+    d, m = C.c_uint8(), C.c_uint8()
+    lib().orc_scale_min_k4(int(j), _p(q12), C.byref(d), C.byref(m))
+    return d.value, m.value
+
+
+def softmax_topk(logits, k):
+    logits = _c(logits, np.float32)
+    E = logits.size
+    probs = np.empty(E, np.float32)
+    ids = np.empty(k, np.int32)
+    ws = np.empty(k, np.float32)
+    lib().orc_softmax_topk(_p(logits), E, k, _p(probs), _p(ids), _p(ws))
+    return probs, ids, ws
+
+
+def router(Wr, x, k, bias=None, id_stride=16):
+    """-> logits [T][E] f32, ids [T][id_stride] i32, ws [T][id_stride] f32 (first k valid)."""
+    x = _c(x, np.float32).reshape(-1, Wr.cols)
+    T, E = x.shape[0], Wr.rows
+    logits = np.empty((T, E), np.float32)
+    ids = np.zeros((T, id_stride), np.int32)
+    ws = np.zeros((T, id_stride), np.float32)
+    b = _c(bias, np.float32) if bias is not None else None
+    m = Wr.c()
+    lib().orc_router(C.byref(m), _p(b), _p(x), T, k, id_stride, _p(logits), _p(ids), _p(ws))
+    return logits, ids, ws
+
+
+def route(ids, ws, k, E):
+    """Expert-sorted permutation -> tokidx, pw, eoff, pairids."""
+    ids = _c(ids, np.int32)
+    ws = _c(ws, np.float32)
+    P, stride = ids.shape
+    tokidx = np.empty(P * k, np.int32)
+    pw = np.empty(P * k, np.float32)
+    eoff = np.empty(E + 1, np.int32)
+    pairids = np.empty(P * k, np.int32)
+    lib().orc_route(_p(ids), _p(ws), P, k, E, stride, _p(tokidx), _p(pw), _p(eoff), _p(pairids))
+    return tokidx, pw, eoff, pairids
+
+
+def tiles(eoff, cap):
+    eoff = _c(eoff, np.int32)
+    E = eoff.size - 1
+    out = np.empty((int(eoff[-1]) // cap + E + 1, 3), np.int32)
+    lib().orc_tiles.restype = C.c_int
+    n = lib().orc_tiles(_p(eoff), E, cap, _p(out))
+    return out[:n].copy()
+
+
+class Layer:
+    """One MoE layer's weights for the oracle (numpy-backed)."""
+
+    def __init__(self, d, mid, E, k, router, down, gate_up=None, gate=None, up=None,
+                 shared=None, router_bias=None):
+        self.d, self.mid, self.E, self.k = d, mid, E, k
+        self.router, self.down, self.gate_up, self.gate, self.up = router, down, gate_up, gate, up
+        self.shared = shared  # (sh_gate, sh_up, sh_down, sh_sg) or None
+        self.router_bias = _c(router_bias, np.float32) if router_bias is not None else None
+
+    def c(self):
+        L = _Layer()
+        L.d, L.mid, L.E, L.k = self.d, self.mid, self.E, self.k
+        L.router = self.router.c()
+        L.router_bias = self.router_bias.ctypes.data if self.router_bias is not None else None
+        L.gate_up = self.gate_up.c() if self.gate_up is not None else _NULL
+        L.gate = self.gate.c() if self.gate is not None else _NULL
+        L.up = self.up.c() if self.up is not None else _NULL
+        L.down = self.down.c()
+        if self.shared is not None:
+            L.sh_gate, L.sh_up, L.sh_down, L.sh_sg = (m.c() for m in self.shared)
+            L.has_shared = 1
+        else:
+            L.sh_gate = L.sh_up = L.sh_down = L.sh_sg = _NULL
+            L.has_shared = 0
+        return L
+
+
+def moe_layer(layer, x, tok_list=None, id_stride=16, want_hid=False):
+    """y [T][d] (rows outside tok_list are left NaN), ids, ws, hid?"""
+    x = _c(x, np.float32).reshape(-1, layer.d)
+    T = x.shape[0]
+    ids = np.zeros((T, id_stride), np.int32)
+    ws = np.zeros((T, id_stride), np.float32)
+    y = np.full((T, layer.d), np.nan, np.float32)
+    hid = np.full((T, layer.k, layer.mid), np.nan, np.float32) if want_hid else None
+    tl = _c(tok_list, np.int32) if tok_list is not None else None
+    L = layer.c()
+    lib().orc_moe_layer(C.byref(L), _p(x), T, _p(tl), 0 if tl is None else tl.size, id_stride,
+                        _p(ids), _p(ws), _p(hid), _p(y))
+    return (y, ids, ws, hid) if want_hid else (y, ids, ws)
+
+
+def num_threads():
+    return lib().orc_num_threads()
+
+
+def set_threads(n):
+    lib().orc_set_threads(int(n))
+
+
+# ---- the reference's own code (only where oracle/_ref is built) ----
+
+def ref_q4cp_rows(blob, rows, cols, row0, nrows):
+    blob = _c(blob, np.uint8)
+    out = np.empty((nrows, cols), np.float32)
+    rc = ref().ref_q4cp_rows(_p(blob), C.c_uint64(rows), C.c_uint64(cols), C.c_uint64(row0),
+                             C.c_uint64(nrows), _p(out))
+    assert rc == 0
+    return out
+
+
+def ref_q4k_rows(raw, nrows, k):
+    raw = _c(raw, np.uint8)
+    rb = ref().ref_q4k_row_bytes(C.c_uint64(k))
+    out = np.empty((nrows, k), np.float32)
+    for r in range(nrows):
+        rc = ref().ref_q4k_row(C.c_void_p(raw.ctypes.data + r * rb),
+                               C.c_void_p(out.ctypes.data + r * k * 4), C.c_uint64(k))
+        assert rc == 0
+    return out
+
+
+def ref_scale_min_k4(j, q12):
+    q12 = _c(q12, np.uint8)
+    d, m = C.c_uint8(), C.c_uint8()
+    ref().ref_scale_min_k4(int(j), _p(q12), C.byref(d), C.byref(m))
+    return d.value, m.value
+
+
+def ref_moe_token(layer, x):
+    """Model::moe of the reference for one token.  Router/shared tensors must be BF16 or Q4CP,
+    routed experts q4cp with fused gate_up."""
+    x = _c(x, np.float32).reshape(layer.d)
+    y = np.empty(layer.d, np.float32)
+    sh_gate, sh_up, sh_down, sh_sg = layer.shared
+    assert sh_gate.dtype == sh_up.dtype == sh_down.dtype
+    rc = ref().ref_moe_token(layer.d, layer.mid, layer.E, layer.k, C.c_uint32(layer.router.dtype),
+                             _p(layer.router.data), _p(layer.gate_up.data), _p(layer.down.data),
+                             C.c_uint32(sh_gate.dtype), _p(sh_gate.data), _p(sh_up.data),
+                             _p(sh_down.data), C.c_uint32(sh_sg.dtype), _p(sh_sg.data), _p(x), _p(y))
+    assert rc == 0
+    return y
