@@ -1,0 +1,223 @@
+"""ctypes binding of libmi355moe.so (include/mi355_moe.h).
+
+PyTorch supplies device memory and the stream only; every computation is a call through the
+C ABI.  Loading fails loudly when the library has not been built — there is no fallback path.
+"""
+import ctypes as C
+import os
+
+import torch
+
+from .build import LIB
+
+F32, BF16, Q4CP = 1, 0, 5
+GGML_Q4_K = 12
+
+
+class MoeError(RuntimeError):
+    pass
+
+
+class WView(C.Structure):
+    _fields_ = [("dtype", C.c_int), ("data", C.c_void_p), ("rows", C.c_uint64), ("cols", C.c_uint64),
+                ("scale_stride", C.c_uint64)]
+
+
+class GgExperts(C.Structure):
+    _fields_ = [("gate", C.c_void_p), ("up", C.c_void_p), ("down", C.c_void_p), ("tgu", C.c_int),
+                ("tdn", C.c_int)]
+
+
+class Config(C.Structure):
+    _fields_ = [("d", C.c_int), ("mid", C.c_int), ("experts", C.c_int), ("topk", C.c_int),
+                ("layers", C.c_int), ("max_tokens", C.c_int), ("id_stride", C.c_int)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB):
+            raise MoeError(f"{LIB} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
+        _lib = C.CDLL(LIB)
+        _lib.moe_version.restype = C.c_char_p
+        _lib.moe_status_string.restype = C.c_char_p
+    return _lib
+
+
+def check(rc, what=""):
+    if rc != 0:
+        raise MoeError(f"{what}: status {rc} ({lib().moe_status_string(C.c_int(rc)).decode()})")
+
+
+def stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def q4cp_scale_stride(cols):
+    return ((cols // 32 * 2) + 15) & ~15
+
+
+def wview(t, dtype, rows, cols):
+    """A weight tensor (torch uint8 / float32 / bfloat16 on the GPU) as the engine's WView."""
+    ss = q4cp_scale_stride(cols) if dtype == Q4CP else 0
+    v = WView(dtype, t.data_ptr(), rows, cols, ss)
+    v._keep = t
+    return v
+
+
+def u64(v):
+    return C.c_uint64(int(v))
+
+
+# ---- stage-level calls ----
+
+def q4cp_dequant_rows(blob, rows, cols, row0, nrows):
+    out = torch.empty((nrows, cols), dtype=torch.float32, device=blob.device)
+    check(lib().moe_q4cp_dequant_rows(ptr(blob), u64(rows), u64(cols), u64(row0), u64(nrows), ptr(out),
+                                      stream()), "moe_q4cp_dequant_rows")
+    return out
+
+
+def q4k_dequant_rows(raw, nrows, cols):
+    out = torch.empty((nrows, cols), dtype=torch.float32, device=raw.device)
+    check(lib().moe_q4k_dequant_rows(ptr(raw), u64(nrows), u64(cols), ptr(out), stream()),
+          "moe_q4k_dequant_rows")
+    return out
+
+
+def router_logits(W, x, bias=None, mode=0):
+    P = x.shape[0]
+    out = torch.empty((P, W.rows), dtype=torch.float32, device=x.device)
+    check(lib().moe_router_logits(C.byref(W), ptr(bias), ptr(x), P, ptr(out), mode, stream()),
+          "moe_router_logits")
+    return out
+
+
+def router_topk(logits, k, id_stride=16):
+    P, E = logits.shape
+    ids = torch.zeros((P, id_stride), dtype=torch.int32, device=logits.device)
+    ws = torch.zeros((P, id_stride), dtype=torch.float32, device=logits.device)
+    check(lib().moe_router_topk(ptr(logits), ptr(ids), ptr(ws), P, E, k, id_stride, stream()),
+          "moe_router_topk")
+    return ids, ws
+
+
+class Routing:
+    """GpuMoeRouting: init(capacity, experts) / run(...)."""
+
+    def __init__(self, capacity_pairs, experts):
+        self.h = C.c_void_p()
+        self.experts = experts
+        check(lib().moe_routing_create(capacity_pairs, experts, C.byref(self.h)), "moe_routing_create")
+
+    def run(self, ids, ws, k, want_pairids=True):
+        P, stride = ids.shape
+        dev = ids.device
+        n = P * k
+        tokidx = torch.full((max(n, 1),), -1, dtype=torch.int32, device=dev)
+        pw = torch.zeros((max(n, 1),), dtype=torch.float32, device=dev)
+        eoff = torch.full((self.experts + 1,), -1, dtype=torch.int32, device=dev)
+        pairids = torch.full((max(n, 1),), -1, dtype=torch.int32, device=dev) if want_pairids else None
+        check(lib().moe_routing_run(self.h, ptr(ids), ptr(ws), ptr(tokidx), ptr(pw), ptr(eoff), ptr(pairids),
+                                    P, k, self.experts, stride, stream()), "moe_routing_run")
+        return tokidx[:n], pw[:n], eoff, (pairids[:n] if want_pairids else None)
+
+    def close(self):
+        if self.h:
+            check(lib().moe_routing_destroy(self.h), "moe_routing_destroy")
+            self.h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def tiles(eoff, cap, pairs):
+    E = eoff.numel() - 1
+    max_tiles = (pairs + cap - 1) // cap + E
+    t = torch.zeros((max_tiles, 3), dtype=torch.int32, device=eoff.device)
+    n = torch.zeros((1,), dtype=torch.int32, device=eoff.device)
+    check(lib().moe_tiles(ptr(eoff), ptr(t), ptr(n), E, cap, stream()), "moe_tiles")
+    return t, n
+
+
+def q4cp_gemv_gate_up(gu, x, ids, kpt, mid):
+    P = x.shape[0]
+    hid = torch.empty((P * kpt, mid), dtype=torch.float32, device=x.device)
+    check(lib().moe_q4cp_gemv_gate_up(C.byref(gu), ptr(x), u64(x.stride(0)), ptr(ids), ids.shape[1], kpt, P,
+                                      mid, ptr(hid), stream()), "moe_q4cp_gemv_gate_up")
+    return hid
+
+
+def q4cp_gemv_down_topk(dn, hid, ids, ws, kpt, d, ey=None, sg=None):
+    P = ids.shape[0]
+    out = torch.empty((P, d), dtype=torch.float32, device=hid.device)
+    check(lib().moe_q4cp_gemv_down_topk(C.byref(dn), ptr(hid), ptr(ids), ptr(ws), ids.shape[1], kpt, P, d,
+                                        ptr(ey), ptr(sg), ptr(out), u64(d), stream()),
+          "moe_q4cp_gemv_down_topk")
+    return out
+
+
+# ---- model level ----
+
+class Moe:
+    """moe_ctx: weights are borrowed torch tensors (kept alive here), scratch lives in the context."""
+
+    def __init__(self, d, mid, experts, topk, layers=1, max_tokens=32, id_stride=16):
+        self.cfg = Config(d, mid, experts, topk, layers, max_tokens, id_stride)
+        self.h = C.c_void_p()
+        self._keep = []
+        check(lib().moe_create(C.byref(self.cfg), C.byref(self.h)), "moe_create")
+
+    def set_router(self, layer, W, bias=None):
+        self._keep += [W, bias]
+        check(lib().moe_set_router(self.h, layer, C.byref(W), ptr(bias)), "moe_set_router")
+
+    def set_experts_q4cp(self, layer, gate_up, down):
+        self._keep += [gate_up, down]
+        check(lib().moe_set_experts_q4cp(self.h, layer, C.byref(gate_up), C.byref(down)),
+              "moe_set_experts_q4cp")
+
+    def set_experts_gguf(self, layer, gate, up, down, tgu=GGML_Q4_K, tdn=GGML_Q4_K):
+        self._keep += [gate, up, down]
+        gg = GgExperts(gate.data_ptr(), up.data_ptr(), down.data_ptr(), tgu, tdn)
+        check(lib().moe_set_experts_gguf(self.h, layer, C.byref(gg)), "moe_set_experts_gguf")
+
+    def set_shared(self, layer, gate_proj, up_proj, down_proj, shared_gate, gguf_type=0):
+        self._keep += [gate_proj, up_proj, down_proj, shared_gate]
+        check(lib().moe_set_shared(self.h, layer, C.byref(gate_proj), C.byref(up_proj), C.byref(down_proj),
+                                   C.byref(shared_gate), gguf_type), "moe_set_shared")
+
+    def forward(self, layer, x, y=None):
+        P = x.shape[0]
+        if y is None:
+            y = torch.empty((P, self.cfg.d), dtype=torch.float32, device=x.device)
+        check(lib().moe_forward(self.h, layer, ptr(x), P, ptr(y), stream()), "moe_forward")
+        return y
+
+    def last_routing(self, P):
+        S = self.cfg.id_stride
+        ids = torch.empty((P, S), dtype=torch.int32, device="cuda")
+        ws = torch.empty((P, S), dtype=torch.float32, device="cuda")
+        check(lib().moe_get_routing(self.h, P, ptr(ids), ptr(ws), stream()), "moe_get_routing")
+        return ids, ws
+
+    def close(self):
+        if self.h:
+            check(lib().moe_destroy(self.h), "moe_destroy")
+            self.h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

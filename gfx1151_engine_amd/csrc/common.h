@@ -1,0 +1,62 @@
+// Shared helpers of libmi355moe (gfx950 only, wave64).
+#pragma once
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi355_moe.h"
+
+#define MOE_API extern "C" __attribute__((visibility("default")))
+#define MOE_WAVE 64
+
+static inline hipStream_t moe_s(moe_stream_t s) { return (hipStream_t)s; }
+
+// After a launch: hand a launch error back as a positive hipError_t.
+#define MOE_LAUNCH_CHECK()                     \
+  do {                                         \
+    hipError_t e__ = hipGetLastError();        \
+    if (e__ != hipSuccess) return (int)e__;    \
+  } while (0)
+#define MOE_HIP(call)                          \
+  do {                                         \
+    hipError_t e__ = (call);                   \
+    if (e__ != hipSuccess) return (int)e__;    \
+  } while (0)
+
+static inline bool moe_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// q4cp view -> operand pointers (reference: xcodes(), 40_model.inc:1599-1602)
+struct Q4cpOps {
+  const uint8_t* codes;
+  const uint8_t* scales;
+  const float* cb;
+  uint64_t cols, scale_stride;
+};
+static inline Q4cpOps q4cp_ops(const moe_wview* w) {
+  Q4cpOps o;
+  o.cb = (const float*)w->data;
+  o.codes = w->data + 64;
+  o.scales = w->data + 64 + w->rows * w->cols / 2;
+  o.cols = w->cols;
+  o.scale_stride = w->scale_stride ? w->scale_stride : (((w->cols / 32 * 2) + 15) & ~15ULL);
+  return o;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int o = 32; o; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); }

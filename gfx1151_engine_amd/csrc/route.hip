@@ -1,0 +1,199 @@
+// Expert-sorted token permutation: wavefront ballots build, per 64-token wave, one membership
+// bit mask per expert in LDS; popcounts of those masks give counts, and prefix sums over
+// waves / blocks / experts give every pair its slot.  Stable: inside an expert pairs are in
+// ascending token order, exactly what the reference's stable radix sort yields.
+// (reference: src/gpu/parts/10_ple_io.inc:784-861)
+#include "common.h"
+
+struct moe_routing {
+  int capacity_pairs, experts, max_blocks;
+  int* blockcnt;  // [max_blocks][experts] pairs of block b that go to expert e
+  int* blockoff;  // [max_blocks][experts] exclusive prefix over blocks
+};
+
+namespace {
+constexpr int RT_WAVES = 4, RT_TOK = 64 * RT_WAVES, RT_MAXE = 1024;
+
+// masks[w][e]: bit l set <=> token (block*256 + w*64 + l) routes to expert e.
+__device__ __forceinline__ void build_masks(const int* __restrict__ ids, int P, int k, int E,
+                                            int id_stride, int nbits,
+                                            unsigned long long (*masks)[RT_MAXE]) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < RT_WAVES * E; i += blockDim.x) masks[i / E][i % E] = 0ull;
+  __syncthreads();
+  const int tok = blockIdx.x * RT_TOK + threadIdx.x;
+  for (int s = 0; s < k; s++) {
+    const int key = tok < P ? ids[(size_t)tok * id_stride + s] : -1;
+    const bool valid = key >= 0 && key < E;
+    unsigned long long eq = __ballot(valid);
+    for (int b = 0; b < nbits; b++) {
+      const bool bit = (key >> b) & 1;
+      const unsigned long long bal = __ballot(bit);
+      eq &= bit ? bal : ~bal;
+    }
+    // the lowest lane of every equal-key set records the set; keys differ between leaders
+    if (valid && (unsigned)lane == (unsigned)__ffsll((long long)eq) - 1u) masks[w][key] |= eq;
+  }
+  __syncthreads();
+}
+
+__global__ void __launch_bounds__(256) k_route_count(const int* __restrict__ ids, int P, int k, int E,
+                                                     int id_stride, int nbits,
+                                                     int* __restrict__ blockcnt) {
+  __shared__ unsigned long long masks[RT_WAVES][RT_MAXE];
+  build_masks(ids, P, k, E, id_stride, nbits, masks);
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    int c = 0;
+#pragma unroll
+    for (int w = 0; w < RT_WAVES; w++) c += __popcll(masks[w][e]);
+    blockcnt[(size_t)blockIdx.x * E + e] = c;
+  }
+}
+
+// One block, one thread per expert: prefix over blocks, then an LDS prefix scan over experts.
+__global__ void __launch_bounds__(RT_MAXE) k_route_scan(const int* __restrict__ blockcnt,
+                                                        int* __restrict__ blockoff,
+                                                        int* __restrict__ eoff, int nblk, int E) {
+  __shared__ int wsum[RT_MAXE / 64];
+  const int e = threadIdx.x, lane = e & 63, w = e >> 6;
+  int run = 0;
+  if (e < E)
+    for (int b = 0; b < nblk; b++) {
+      const int c = blockcnt[(size_t)b * E + e];
+      blockoff[(size_t)b * E + e] = run;
+      run += c;
+    }
+  // inclusive scan inside the wave
+  int inc = run;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += v;
+  }
+  if (lane == 63) wsum[w] = inc;
+  __syncthreads();
+  int base = 0;
+  for (int i = 0; i < w; i++) base += wsum[i];
+  if (e < E) eoff[e] = base + inc - run;
+  if (e == E - 1) eoff[E] = base + inc;
+}
+
+__global__ void __launch_bounds__(256) k_route_scatter(const int* __restrict__ ids,
+                                                       const float* __restrict__ ws, int P, int k,
+                                                       int E, int id_stride, int nbits,
+                                                       const int* __restrict__ blockoff,
+                                                       const int* __restrict__ eoff,
+                                                       int* __restrict__ tokidx, float* __restrict__ pw,
+                                                       int* __restrict__ pairids) {
+  __shared__ unsigned long long masks[RT_WAVES][RT_MAXE];
+  build_masks(ids, P, k, E, id_stride, nbits, masks);
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int tok = blockIdx.x * RT_TOK + threadIdx.x;
+  if (tok >= P) return;
+  const unsigned long long below = lane ? (~0ull >> (64 - lane)) : 0ull;
+  for (int s = 0; s < k; s++) {
+    const int key = ids[(size_t)tok * id_stride + s];
+    if (key < 0 || key >= E) continue;
+    int pos = eoff[key] + blockoff[(size_t)blockIdx.x * E + key];
+    for (int i = 0; i < w; i++) pos += __popcll(masks[i][key]);
+    pos += __popcll(masks[w][key] & below);
+    tokidx[pos] = tok;
+    pw[pos] = ws[(size_t)tok * id_stride + s];
+    if (pairids) {
+      int rank = 0;
+      for (int j = 0; j < k; j++) rank += ids[(size_t)tok * id_stride + j] < key;
+      pairids[(size_t)tok * k + rank] = pos;
+    }
+  }
+}
+
+// Tiles in expert order: thread e owns expert e, LDS scan of the per-expert tile counts.
+__global__ void __launch_bounds__(RT_MAXE) k_tiles(const int* __restrict__ eoff,
+                                                   moe_tile* __restrict__ tiles,
+                                                   int* __restrict__ total, int E, int cap) {
+  __shared__ int wsum[RT_MAXE / 64];
+  const int e = threadIdx.x, lane = e & 63, w = e >> 6;
+  const int first = e < E ? eoff[e] : 0;
+  const int ne = e < E ? eoff[e + 1] - first : 0;
+  const int count = (ne + cap - 1) / cap;
+  int inc = count;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += v;
+  }
+  if (lane == 63) wsum[w] = inc;
+  __syncthreads();
+  int base = 0;
+  for (int i = 0; i < w; i++) base += wsum[i];
+  const int begin = base + inc - count;
+  if (e == RT_MAXE - 1) *total = begin + count;
+  for (int j = 0; j < count; j++) {
+    moe_tile t;
+    t.expert = e;
+    t.first = first + j * cap;
+    t.count = min(cap, ne - j * cap);
+    tiles[begin + j] = t;
+  }
+}
+}  // namespace
+
+MOE_API int moe_routing_create(int capacity_pairs, int experts, moe_routing** out) {
+  if (!out || capacity_pairs < 1 || experts < 1) return MOE_E_INVALID;
+  if (experts > RT_MAXE) return MOE_E_UNSUPPORTED;
+  moe_routing* r = new (std::nothrow) moe_routing();
+  if (!r) return (int)hipErrorOutOfMemory;
+  r->capacity_pairs = capacity_pairs;
+  r->experts = experts;
+  r->max_blocks = (capacity_pairs + RT_TOK - 1) / RT_TOK;  // >= ceil(P/256) for any k >= 1
+  r->blockcnt = r->blockoff = nullptr;
+  const size_t bytes = (size_t)r->max_blocks * experts * sizeof(int);
+  hipError_t e = hipMalloc(&r->blockcnt, bytes);
+  if (e == hipSuccess) e = hipMalloc(&r->blockoff, bytes);
+  if (e != hipSuccess) {
+    if (r->blockcnt) (void)hipFree(r->blockcnt);
+    delete r;
+    return (int)e;
+  }
+  *out = r;
+  return MOE_OK;
+}
+
+MOE_API int moe_routing_destroy(moe_routing* r) {
+  if (!r) return MOE_OK;
+  hipError_t e1 = hipFree(r->blockcnt), e2 = hipFree(r->blockoff);
+  delete r;
+  return e1 != hipSuccess ? (int)e1 : (int)e2;
+}
+
+MOE_API int moe_routing_run(moe_routing* r, const int* ids, const float* ws, int* tokidx, float* pw,
+                            int* eoff, int* pairids, int P, int k, int experts, int id_stride,
+                            moe_stream_t st) {
+  if (!r || !eoff || (P > 0 && (!ids || !ws || !tokidx || !pw))) return MOE_E_INVALID;
+  if (P < 0 || k < 1 || id_stride < k || experts != r->experts) return MOE_E_INVALID;
+  if ((int64_t)P * k > r->capacity_pairs) return MOE_E_STATE;
+  int nbits = 0;
+  for (int v = experts - 1; v; v >>= 1) nbits++;
+  const int nblk = (P + RT_TOK - 1) / RT_TOK;
+  if (nblk > 0) {
+    k_route_count<<<nblk, 256, 0, moe_s(st)>>>(ids, P, k, experts, id_stride, nbits, r->blockcnt);
+    MOE_LAUNCH_CHECK();
+  }
+  k_route_scan<<<1, RT_MAXE, 0, moe_s(st)>>>(r->blockcnt, r->blockoff, eoff, nblk, experts);
+  MOE_LAUNCH_CHECK();
+  if (nblk > 0) {
+    k_route_scatter<<<nblk, 256, 0, moe_s(st)>>>(ids, ws, P, k, experts, id_stride, nbits,
+                                                 r->blockoff, eoff, tokidx, pw, pairids);
+    MOE_LAUNCH_CHECK();
+  }
+  return MOE_OK;
+}
+
+MOE_API int moe_tiles(const int* eoff, moe_tile* tiles, int* ntiles, int experts, int cap,
+                      moe_stream_t st) {
+  if (!eoff || !tiles || !ntiles || cap < 1 || experts < 1) return MOE_E_INVALID;
+  if (experts > RT_MAXE) return MOE_E_UNSUPPORTED;
+  k_tiles<<<1, RT_MAXE, 0, moe_s(st)>>>(eoff, tiles, ntiles, experts, cap);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}

@@ -1,0 +1,263 @@
+// Router: logits with the CPU path's fp64 accumulation, fp64 softmax, top-k, renormalised weights.
+// (reference: src/ref.cpp:68-77,565-594; src/gpu/parts/20_kernels_gemv.inc:1433-1562)
+#include "common.h"
+
+namespace {
+
+template <bool BF16>
+__device__ __forceinline__ float load_w(const void* W, uint64_t i) {
+  if (BF16) return bf16_bits_to_f32(((const uint16_t*)W)[i]);
+  return ((const float*)W)[i];
+}
+
+// ---- sequential order: bit-identical to `acc += (double)w*x` for c = 0..d-1 ----
+// Block = 64 tokens x 64 experts, thread = 4 x 4 independent fp64 chains.  The f32*f32 product
+// is exact in fp64, so fma(w, x, acc) equals the reference's multiply-then-add.
+constexpr int RL_T = 64, RL_E = 64, RL_K = 32;
+template <bool BF16>
+__global__ void __launch_bounds__(256) k_router_logits_seq(const void* __restrict__ W,
+                                                           const float* __restrict__ bias,
+                                                           const float* __restrict__ x, int P, int E,
+                                                           int d, float* __restrict__ logits) {
+  __shared__ float Xs[RL_K][RL_T + 1];
+  __shared__ float Ws[RL_K][RL_E + 1];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int e0 = blockIdx.x * RL_E, t0 = blockIdx.y * RL_T;
+  double acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = 0.0;
+  for (int c0 = 0; c0 < d; c0 += RL_K) {
+    // stage 64 rows x 32 columns of each operand (zero outside the matrix)
+#pragma unroll
+    for (int it = 0; it < (RL_T * RL_K) / 256; it++) {
+      const int i = tid + it * 256, r = i / RL_K, c = i % RL_K;
+      const int t = t0 + r, e = e0 + r, cc = c0 + c;
+      Xs[c][r] = (t < P && cc < d) ? x[(size_t)t * d + cc] : 0.f;
+      Ws[c][r] = (e < E && cc < d) ? load_w<BF16>(W, (uint64_t)e * d + cc) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int c = 0; c < RL_K; c++) {
+      double wv[4], xv[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) wv[i] = (double)Ws[c][tx + 16 * i];
+#pragma unroll
+      for (int j = 0; j < 4; j++) xv[j] = (double)Xs[c][ty + 16 * j];
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = fma(wv[i], xv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int t = t0 + ty + 16 * j;
+    if (t >= P) continue;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int e = e0 + tx + 16 * i;
+      if (e >= E) continue;
+      float v = (float)acc[i][j];
+      if (bias) v += bias[e];
+      logits[(size_t)t * E + e] = v;
+    }
+  }
+}
+
+// ---- lane-parallel order for small P: one wave per weight row, lanes stride the columns,
+// per-lane fp64 chains, fixed butterfly.  The fp64 sum differs from the sequential one only in
+// its last bits, so the f32 logit differs with probability ~1e-8 per value.
+// Row E (if Wx given) is the shared-expert gate vector: out_x[t] = its logit.
+template <bool BF16, int TT>
+__global__ void __launch_bounds__(256) k_router_logits_par(const void* __restrict__ W,
+                                                           const float* __restrict__ bias,
+                                                           const void* __restrict__ Wx, bool wx_bf16,
+                                                           const float* __restrict__ x, int P, int E,
+                                                           int d, float* __restrict__ logits,
+                                                           float* __restrict__ out_x) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row > E || (row == E && !Wx)) return;
+  const bool extra = row == E;
+  const void* Wr = extra ? Wx : W;
+  const uint64_t base = extra ? 0 : (uint64_t)row * d;
+  const bool bf = extra ? wx_bf16 : BF16;
+  for (int t0 = 0; t0 < P; t0 += TT) {
+    double acc[TT];
+#pragma unroll
+    for (int i = 0; i < TT; i++) acc[i] = 0.0;
+    for (int c = lane * 4; c < d; c += 256) {
+      float w[4];
+      if (bf) {
+        const uint2 u = *(const uint2*)((const uint16_t*)Wr + base + c);
+        w[0] = __uint_as_float(u.x << 16);
+        w[1] = __uint_as_float(u.x & 0xffff0000u);
+        w[2] = __uint_as_float(u.y << 16);
+        w[3] = __uint_as_float(u.y & 0xffff0000u);
+      } else {
+        const float4 f = *(const float4*)((const float*)Wr + base + c);
+        w[0] = f.x; w[1] = f.y; w[2] = f.z; w[3] = f.w;
+      }
+#pragma unroll
+      for (int i = 0; i < TT; i++) {
+        if (t0 + i < P) {
+          const float4 xv = *(const float4*)(x + (size_t)(t0 + i) * d + c);
+          acc[i] = fma((double)w[0], (double)xv.x, acc[i]);
+          acc[i] = fma((double)w[1], (double)xv.y, acc[i]);
+          acc[i] = fma((double)w[2], (double)xv.z, acc[i]);
+          acc[i] = fma((double)w[3], (double)xv.w, acc[i]);
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TT; i++) {
+      const double s = wave_sum(acc[i]);
+      if (lane == 0 && t0 + i < P) {
+        float v = (float)s;
+        if (extra) out_x[t0 + i] = v;
+        else {
+          if (bias) v += bias[row];
+          logits[(size_t)(t0 + i) * E + row] = v;
+        }
+      }
+    }
+  }
+}
+
+// ---- softmax + top-k, one wave per token (E <= 64*NPL) ----
+template <int NPL>
+__global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ logits,
+                                                     int* __restrict__ ids, float* __restrict__ ws,
+                                                     int P, int E, int k, int id_stride) {
+  __shared__ float pbuf[4][64 * NPL];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int tok = blockIdx.x * 4 + wv;
+  if (tok >= P) return;
+  const float* lg = logits + (size_t)tok * E;
+  float v[NPL];
+  float mxf = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = lane + 64 * j;
+    v[j] = e < E ? lg[e] : -INFINITY;
+    mxf = fmaxf(mxf, v[j]);
+  }
+  const double mx = (double)wave_max(mxf);
+  // p = (float)exp((double)logit - mx)
+  float p[NPL];
+  bool exact = true;  // all partial sums representable -> any summation order gives the same fp64
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = lane + 64 * j;
+    p[j] = e < E ? (float)exp((double)v[j] - mx) : 0.f;
+    exact = exact && (p[j] == 0.f || p[j] >= 0x1p-20f);
+  }
+  double se;
+  if (__all(exact)) {
+    double s = 0.0;
+#pragma unroll
+    for (int j = 0; j < NPL; j++) s += (double)p[j];
+    se = wave_sum(s);
+  } else {
+    // very wide logit range: replay the reference's index order on one lane
+#pragma unroll
+    for (int j = 0; j < NPL; j++) pbuf[wv][lane + 64 * j] = p[j];
+    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_wave_barrier();
+    double s = 0.0;
+    if (lane == 0)
+      for (int e = 0; e < E; e++) s += (double)pbuf[wv][e];
+    se = __shfl(s, 0, 64);
+  }
+  float sc[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = lane + 64 * j;
+    sc[j] = e < E ? (float)((double)p[j] / se) : -1.f;
+  }
+  // k rounds of arg-max: larger probability first, equal probabilities -> lower index
+  double wsum = 0.0;
+  float mine = 0.f;  // lane r keeps the r-th selected probability
+  for (int r = 0; r < k; r++) {
+    float bv = -2.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < NPL; j++)
+      if (sc[j] > bv) {
+        bv = sc[j];
+        bi = lane + 64 * j;
+      }
+#pragma unroll
+    for (int o = 32; o; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > bv || (ov == bv && oi < bi)) {
+        bv = ov;
+        bi = oi;
+      }
+    }
+    wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
+    if (lane == r) mine = bv;
+    if (lane == 0) ids[(size_t)tok * id_stride + r] = bi;
+    if ((bi & 63) == lane) {
+#pragma unroll
+      for (int j = 0; j < NPL; j++)
+        if (j == (bi >> 6)) sc[j] = -1.f;
+    }
+  }
+  if (lane < k) ws[(size_t)tok * id_stride + lane] = (float)((double)mine / wsum);
+}
+
+}  // namespace
+
+MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float* x, int P,
+                              float* logits, int mode, moe_stream_t st) {
+  if (!W || !W->data || !x || !logits) return MOE_E_INVALID;
+  if (W->dtype != MOE_DT_F32 && W->dtype != MOE_DT_BF16) return MOE_E_UNSUPPORTED;
+  if (P < 0 || W->rows == 0 || W->cols == 0 || W->rows > (1u << 20) || W->cols > (1u << 24))
+    return MOE_E_INVALID;
+  if (P == 0) return MOE_OK;
+  const int E = (int)W->rows, d = (int)W->cols;
+  const bool bf = W->dtype == MOE_DT_BF16;
+  const bool par = mode == 0 && P <= 32 && d % 4 == 0 && moe_aligned(x, 16) && moe_aligned(W->data, 16);
+  if (par) {
+    dim3 g((E + 3) / 4);
+    if (bf) k_router_logits_par<true, 4><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
+    else k_router_logits_par<false, 4><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
+  } else {
+    dim3 g((E + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
+    if (bf) k_router_logits_seq<true><<<g, 256, 0, moe_s(st)>>>(W->data, bias, x, P, E, d, logits);
+    else k_router_logits_seq<false><<<g, 256, 0, moe_s(st)>>>(W->data, bias, x, P, E, d, logits);
+  }
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// Internal: small-P logits plus the shared-expert gate row in the same launch.
+int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
+                            int P, float* logits, float* out_x, hipStream_t st) {
+  const int E = (int)W->rows, d = (int)W->cols;
+  const bool bf = W->dtype == MOE_DT_BF16;
+  const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
+  dim3 g((E + 1 + 3) / 4);
+  if (bf) k_router_logits_par<true, 4><<<g, 256, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x);
+  else k_router_logits_par<false, 4><<<g, 256, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+MOE_API int moe_router_topk(const float* logits, int* ids, float* ws, int P, int E, int k,
+                            int id_stride, moe_stream_t st) {
+  if (!logits || !ids || !ws) return MOE_E_INVALID;
+  if (P < 0 || E < 1 || k < 1 || k > E || k > 64 || id_stride < k) return MOE_E_INVALID;
+  if (E > 1024) return MOE_E_UNSUPPORTED;
+  if (P == 0) return MOE_OK;
+  dim3 g((P + 3) / 4);
+  if (E <= 512) k_router_topk<8><<<g, 256, 0, moe_s(st)>>>(logits, ids, ws, P, E, k, id_stride);
+  else k_router_topk<16><<<g, 256, 0, moe_s(st)>>>(logits, ids, ws, P, E, k, id_stride);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}

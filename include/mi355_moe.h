@@ -1,0 +1,154 @@
+/*
+ * mi355_moe.h — C ABI of libmi355moe.so: the routed-expert MoE layer of gfx1151-engine
+ * (router top-k, 4-bit expert GEMV / grouped GEMM, SwiGLU, weighted combine, shared expert)
+ * for one AMD Instinct MI355X (gfx950).
+ *
+ * Every entry point names the reference symbol it stands in for (file:line inside the reference
+ * tree).  Conventions kept from the reference:
+ *   - the caller owns every buffer; weights are borrowed, read-only device memory in the
+ *     engine's on-disk byte layouts (hgn q4cp blobs, GGUF raw blocks);
+ *   - every call only enqueues work on the given HIP stream, never synchronises the host, never
+ *     allocates (contexts allocate once, at creation) and is safe under HIP graph capture;
+ *   - router rows are `id_stride` ints/floats wide, the first k valid (the engine uses 16);
+ *   - one host thread drives a context at a time (contexts share scratch between calls).
+ * Return value: 0 = ok, < 0 = moe_status (unsupported / invalid arguments: nothing was enqueued),
+ * > 0 = a hipError_t from the runtime.  Nothing throws across this boundary.
+ */
+#ifndef MI355_MOE_H
+#define MI355_MOE_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* moe_stream_t; /* hipStream_t */
+
+enum moe_status {
+  MOE_OK = 0,
+  MOE_E_UNSUPPORTED = -1, /* shape / type the kernels do not cover (reference: `return false`) */
+  MOE_E_INVALID = -2,     /* null pointer, misaligned pointer, inconsistent sizes */
+  MOE_E_STATE = -3        /* context not ready (weights missing, capacity exceeded) */
+};
+
+/* hgn tensor dtypes (src/hgn.h:2-23) and ggml types (src/gguf.h:42-64) used on this path */
+enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5 };
+enum { MOE_GGML_Q4_K = 12 };
+
+/* WView (src/gpu/parts/30_host_util.inc:772-780): a weight tensor as it lies in memory.
+ * q4cp: data = [64 B codebook][rows*cols/2 codes][rows x scale_stride]. */
+typedef struct moe_wview {
+  int dtype;
+  const uint8_t* data;
+  uint64_t rows, cols, scale_stride;
+} moe_wview;
+
+/* GgExperts (30_host_util.inc:348-351): GGUF ffn_{gate,up,down}_exps raw blocks, [K,N,E]. */
+typedef struct moe_gg_experts {
+  const uint8_t *gate, *up, *down;
+  int tgu, tdn; /* ggml types */
+} moe_gg_experts;
+
+/* MoeTile (src/gpu/parts/10_ple_io.inc:813) */
+typedef struct moe_tile {
+  int expert, first, count;
+} moe_tile;
+
+const char* moe_version(void);
+const char* moe_status_string(int status);
+
+/* ---- weights: dequantisation (bit-exact with the reference's CPU formulas) ---- */
+
+/* hgn::Checkpoint::q4cp_row (src/hgn.h:249-261) for rows [row0, row0+nrows) of a q4cp blob:
+ * out[r][c] = cb[nibble] * f32(fp16 scale[r][c/32]).  out: f32 [nrows][cols]. */
+int moe_q4cp_dequant_rows(const uint8_t* blob, uint64_t rows, uint64_t cols, uint64_t row0,
+                          uint64_t nrows, float* out, moe_stream_t st);
+/* gguf::dequant_row, Q4_K branch (src/gguf.h:408-441) for nrows raw rows of `cols` elements. */
+int moe_q4k_dequant_rows(const uint8_t* raw, uint64_t nrows, uint64_t cols, float* out,
+                         moe_stream_t st);
+
+/* ---- router ---- */
+
+/* Router logits, the reference CPU arithmetic (src/ref.cpp:70-77 via :566): per (token, expert)
+ * one fp64 accumulation over c = 0..d-1 rounded to f32; replaces gemv()/gemm() on
+ * mlp.gate.weight (src/gpu/parts/40_model.inc:1809,4023).  W: [E][d] f32 or bf16.
+ * bias (optional, [E]) is added in f32 afterwards.  mode 0 = automatic (exact sequential order
+ * for P > 32, lane-parallel fp64 order for P <= 32), 1 = force the sequential order. */
+int moe_router_logits(const moe_wview* W, const float* bias, const float* x, int P, float* logits,
+                      int mode, moe_stream_t st);
+/* k_router_topk / k_router_topk_w32 (src/gpu/parts/20_kernels_gemv.inc:1433,1496) with the CPU
+ * path's arithmetic (src/ref.cpp:575-594): fp64 softmax -> f32 probabilities, k rounds of
+ * arg-max (ties -> lowest index), weights renormalised over the selected k. */
+int moe_router_topk(const float* logits, int* ids, float* ws, int P, int E, int k, int id_stride,
+                    moe_stream_t st);
+
+/* ---- expert-sorted token permutation ---- */
+
+/* GpuMoeRouting (10_ple_io.inc:827-861): init() -> create, run() -> run.  Stable by expert:
+ * tokidx[p] token of pair p, pw[p] its router weight, eoff[e]..eoff[e+1] expert e's pairs,
+ * pairids[t*k+rank] pair of token t's rank-th expert in ascending expert id (may be NULL). */
+typedef struct moe_routing moe_routing;
+int moe_routing_create(int capacity_pairs, int experts, moe_routing** out);
+int moe_routing_destroy(moe_routing* r);
+int moe_routing_run(moe_routing* r, const int* ids, const float* ws, int* tokidx, float* pw,
+                    int* eoff, int* pairids, int P, int k, int experts, int id_stride,
+                    moe_stream_t st);
+/* k_moe_tiles (10_ple_io.inc:815): split each expert's run into <= cap pair tiles, expert order.
+ * tiles must hold (pairs+cap-1)/cap + experts entries. */
+int moe_tiles(const int* eoff, moe_tile* tiles, int* ntiles, int experts, int cap, moe_stream_t st);
+
+/* ---- decode / small-batch path (P*k slots, each token's experts read in place) ---- */
+
+/* k_q4cp_gemv_gg + k_silu_mul_g (20_kernels_gemv.inc:1608,1680) fused: for slot = (tok, s),
+ * expert e = ids[tok*id_stride+s]: hid[slot][r] = silu(W_e[r].x_tok) * (W_e[mid+r].x_tok).
+ * gu: q4cp view of the fused gate_up tensor [E*2*mid][d].  x: f32 [P][x_stride]. */
+int moe_q4cp_gemv_gate_up(const moe_wview* gu, const float* x, uint64_t x_stride, const int* ids,
+                          int id_stride, int kpt, int P, int mid, float* hid, moe_stream_t st);
+/* k_q4cp_gemv_gd_topk_h16 (20_kernels_gemv.inc:1771): out[tok][r] = sum_s ws[tok][s] *
+ * (W_{e_s}[r] . hid[tok*kpt+s]) in slot order, overwriting out (no atomics).  If ey/sg are given,
+ * k_axpy_sg (40_model.inc:8897) is folded in: out += sigmoid(sg[tok]) * ey[tok]. */
+int moe_q4cp_gemv_down_topk(const moe_wview* dn, const float* hid, const int* ids, const float* ws,
+                            int id_stride, int kpt, int P, int d, const float* ey, const float* sg,
+                            float* out, uint64_t out_stride, moe_stream_t st);
+/* moe_gg_gemv (src/gpu/parts/26_kernels_moe_gguf.inc:893): GGUF raw-block experts, small P.
+ * Supported: tgu = tdn = Q4_K, d % 256 == 0, mid % 256 == 0. */
+int moe_gg_gemv(int tgu, int tdn, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+                const float* x, const int* ids, const float* ws, float* hid, float* out, int P,
+                int d, int mid, int kpt, int id_stride, moe_stream_t st);
+
+/* ---- model level ---- */
+
+typedef struct moe_config {
+  int d, mid, experts, topk;
+  int layers;     /* number of layer slots */
+  int max_tokens; /* scratch is sized for this many rows (reference: maxbatch_cap) */
+  int id_stride;  /* 0 -> 16 */
+} moe_config;
+
+typedef struct moe_ctx moe_ctx;
+int moe_create(const moe_config* cfg, moe_ctx** out);
+int moe_destroy(moe_ctx* ctx);
+/* weights of one layer; all pointers are device memory owned by the caller.
+ * router: mlp.gate.weight [E][d] (f32 / bf16); router_bias optional (synthetic skew).
+ * hgn: gate_up [E*2*mid][d] and down [E*d][mid] q4cp views (40_model.inc:1826-1829).
+ * gguf: GgExperts (40_model.inc:1823).  Exactly one of hgn / gguf per layer.
+ * shared expert: gate_proj/up_proj [mid][d], down_proj [d][mid], shared_expert_gate [1][d]
+ * (40_model.inc:1848-1857); dtype q4cp, f32 or bf16; sh_gguf_type != 0 means gate/up/down are
+ * raw GGUF rows of that ggml type. */
+int moe_set_router(moe_ctx* ctx, int layer, const moe_wview* gate_w, const float* router_bias);
+int moe_set_experts_q4cp(moe_ctx* ctx, int layer, const moe_wview* gate_up, const moe_wview* down);
+int moe_set_experts_gguf(moe_ctx* ctx, int layer, const moe_gg_experts* gg);
+int moe_set_shared(moe_ctx* ctx, int layer, const moe_wview* gate_proj, const moe_wview* up_proj,
+                   const moe_wview* down_proj, const moe_wview* shared_gate, int sh_gguf_type);
+/* GpuModel::moe (40_model.inc:1806) for P == 1 and GpuModel::moe_b (40_model.inc:4018) for a
+ * batch: y[P][d] = routed experts (top-k, renormalised) + sigmoid-gated shared expert.
+ * x, y: f32 [P][d]; y is fully overwritten. */
+int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_stream_t st);
+/* Copy the last call's router output (the reference keeps it in d_topids / d_topw,
+ * 40_model.inc:1811) into caller buffers [P][id_stride] (device memory; async on st). */
+int moe_get_routing(moe_ctx* ctx, int P, int* ids_out, float* ws_out, moe_stream_t st);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

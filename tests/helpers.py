@@ -1,0 +1,88 @@
+"""Shared builders for the tests: seeded layers in the engine's byte layouts, for the oracle
+(numpy) and for the HIP library (torch tensors on the GPU) from the same bytes."""
+import numpy as np
+
+from gfx1151_engine_amd import synth as S
+from oracle import oracle as O
+
+
+def bits(a):
+    return np.ascontiguousarray(a, np.float32).view(np.uint32)
+
+
+def max_abs_rel(y, ref):
+    """max |y - ref| / max |ref|: the layer tolerance is stated on this number."""
+    return float(np.abs(y.astype(np.float64) - ref.astype(np.float64)).max() / np.abs(ref).max())
+
+
+class HostLayer:
+    """One synthetic MoE layer as host bytes (the 'file' side)."""
+
+    def __init__(self, rng, d, mid, E, k, fmt="q4cp", router_dtype="f32", codebook=None, scale_std=0.01,
+                 router_std=0.02, shared=True, bias=None):
+        self.d, self.mid, self.E, self.k, self.fmt = d, mid, E, k, fmt
+        rw = (rng.standard_normal((E, d), dtype=np.float32) * router_std)
+        if router_dtype == "bf16":
+            self.router = S.f32_to_bf16_bits(rw)
+            self.router_dt = O.BF16
+        else:
+            self.router = rw
+            self.router_dt = O.F32
+        self.bias = bias
+        if fmt == "q4cp":
+            self.gate_up = S.make_q4cp(rng, E * 2 * mid, d, codebook=codebook, scale_std=scale_std)
+            self.down = S.make_q4cp(rng, E * d, mid, codebook=codebook, scale_std=scale_std)
+        else:
+            self.gate = S.make_q4k(rng, E * mid, d, scale_std=scale_std)
+            self.up = S.make_q4k(rng, E * mid, d, scale_std=scale_std)
+            self.down = S.make_q4k(rng, E * d, mid, scale_std=scale_std)
+        self.shared = None
+        if shared:
+            mk = (lambda r, c: S.make_q4cp(rng, r, c, codebook=codebook, scale_std=scale_std)) if fmt == "q4cp" \
+                else (lambda r, c: S.make_q4k(rng, r, c, scale_std=scale_std))
+            self.shared = [mk(mid, d), mk(mid, d), mk(d, mid),
+                           rng.standard_normal((1, d), dtype=np.float32) * router_std]
+
+    def oracle_layer(self):
+        d, mid, E, k = self.d, self.mid, self.E, self.k
+        wt = O.Q4CP if self.fmt == "q4cp" else O.Q4K
+        sh = None
+        if self.shared is not None:
+            sh = [O.Mat(wt, self.shared[0], mid, d), O.Mat(wt, self.shared[1], mid, d),
+                  O.Mat(wt, self.shared[2], d, mid), O.Mat(O.F32, self.shared[3], 1, d)]
+        router = O.Mat(self.router_dt, self.router, E, d)
+        if self.fmt == "q4cp":
+            return O.Layer(d, mid, E, k, router, O.Mat(wt, self.down, E * d, mid),
+                           gate_up=O.Mat(wt, self.gate_up, E * 2 * mid, d), shared=sh, router_bias=self.bias)
+        return O.Layer(d, mid, E, k, router, O.Mat(wt, self.down, E * d, mid),
+                       gate=O.Mat(wt, self.gate, E * mid, d), up=O.Mat(wt, self.up, E * mid, d), shared=sh,
+                       router_bias=self.bias)
+
+    def to_gpu(self, max_tokens=32):
+        """-> (capi.Moe context with this layer registered as layer 0, dict of device tensors)."""
+        import torch
+        from gfx1151_engine_amd import capi
+        d, mid, E, k = self.d, self.mid, self.E, self.k
+        dev = {}
+
+        def up(name, a):
+            t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+            dev[name] = t
+            return t
+        m = capi.Moe(d, mid, E, k, layers=1, max_tokens=max_tokens)
+        rt = up("router", self.router.view(np.int16) if self.router_dt == O.BF16 else self.router)
+        m.set_router(0, capi.wview(rt, capi.BF16 if self.router_dt == O.BF16 else capi.F32, E, d),
+                     up("bias", self.bias) if self.bias is not None else None)
+        if self.fmt == "q4cp":
+            m.set_experts_q4cp(0, capi.wview(up("gate_up", self.gate_up), capi.Q4CP, E * 2 * mid, d),
+                               capi.wview(up("down", self.down), capi.Q4CP, E * d, mid))
+        else:
+            m.set_experts_gguf(0, up("gate", self.gate), up("up", self.up), up("down", self.down))
+        if self.shared is not None:
+            wt = capi.Q4CP if self.fmt == "q4cp" else 0
+            m.set_shared(0, capi.wview(up("shg", self.shared[0]), wt, mid, d),
+                         capi.wview(up("shu", self.shared[1]), wt, mid, d),
+                         capi.wview(up("shd", self.shared[2]), wt, d, mid),
+                         capi.wview(up("shsg", self.shared[3]), capi.F32, 1, d),
+                         0 if self.fmt == "q4cp" else capi.GGML_Q4_K)
+        return m, dev

@@ -1,0 +1,286 @@
+"""CPU-only: pins the oracle (oracle/moe_oracle.c) against
+ (1) golden vectors produced by the reference's own code (tests/golden/*.npz),
+ (2) the reference's own code directly where oracle/_ref is built (this container),
+ (3) closed forms, invariants and brute force that a dropped term / wrong index would break."""
+import numpy as np
+import pytest
+
+from gfx1151_engine_amd import synth as S
+from helpers import HostLayer, bits
+
+
+def same_bits(a, b):
+    a, b = bits(a), np.asarray(b, np.uint32)
+    nan = (np.isnan(a.view(np.float32)) & np.isnan(b.view(np.float32)))
+    return bool(((a == b) | nan).all())
+
+
+# ---------- fp16 ----------
+def test_fp16_all_patterns_golden(oracle, golden):
+    want = golden("fp16_table.npz")["bits"]
+    got = np.array([oracle.fp16_to_f32(h) for h in range(65536)], np.float32)
+    assert same_bits(got, want)
+
+
+def test_fp16_matches_numpy(oracle):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([oracle.fp16_to_f32(int(x)) for x in h], np.float32)
+    ok = np.isfinite(want)
+    assert (bits(got[ok]) == bits(want[ok])).all()
+
+
+# ---------- q4cp ----------
+def test_q4cp_golden(oracle, golden):
+    g = golden("q4cp_rows.npz")
+    for i in range(int(g["n"])):
+        rows, cols = (int(v) for v in g[f"shape{i}"])
+        got = oracle.q4cp_rows(g[f"blob{i}"], rows, cols, 0, rows)
+        assert same_bits(got, g[f"bits{i}"]), f"case {i}"
+
+
+def test_q4cp_layout_closed_form(oracle):
+    """Independent numpy decode of the byte layout: codebook, low nibble first, padded scale record."""
+    rng = np.random.default_rng(5)
+    rows, cols = 7, 640
+    cb = rng.uniform(-2, 2, 16).astype(np.float32)
+    blob = S.make_q4cp(rng, rows, cols, codebook=cb, scale_std=0.5)
+    ss = 48  # 40 B of scales padded to 16 B
+    assert S.q4cp_scale_stride(cols) == ss == oracle.lib().orc_q4cp_scale_stride(cols)
+    assert blob.size == 64 + rows * cols // 2 + rows * ss == oracle.lib().orc_q4cp_blob_bytes(rows, cols)
+    codes = blob[64:64 + rows * cols // 2].reshape(rows, cols // 2)
+    nib = np.stack([codes & 0xF, codes >> 4], axis=-1).reshape(rows, cols)
+    sc = blob[64 + rows * cols // 2:].reshape(rows, ss)[:, :cols // 16].copy().view(np.float16).astype(np.float32)
+    want = cb[nib] * np.repeat(sc, 32, axis=1)
+    assert same_bits(oracle.q4cp_rows(blob, rows, cols, 0, rows), bits(want))
+    # row offset argument
+    assert same_bits(oracle.q4cp_rows(blob, rows, cols, 3, 2), bits(want[3:5]))
+
+
+def test_q4cp_vs_reference_build(oracle):
+    if oracle.ref() is None:
+        pytest.skip("oracle/_ref not built here")
+    rng = np.random.default_rng(11)
+    for rows, cols in [(9, 640), (3, 3072), (16, 32)]:
+        blob = S.make_q4cp(rng, rows, cols, codebook=rng.standard_normal(16).astype(np.float32), scale_std=1.0)
+        assert same_bits(oracle.q4cp_rows(blob, rows, cols, 0, rows),
+                         bits(oracle.ref_q4cp_rows(blob, rows, cols, 0, rows)))
+
+
+# ---------- Q4_K ----------
+def test_q4k_golden(oracle, golden):
+    g = golden("q4k_rows.npz")
+    for i in range(int(g["n"])):
+        rows, cols = (int(v) for v in g[f"shape{i}"])
+        assert same_bits(oracle.q4k_rows(g[f"raw{i}"], rows, cols), g[f"bits{i}"]), f"case {i}"
+    for i in range(g["k4_q"].shape[0]):
+        for j in range(8):
+            assert oracle.scale_min_k4(j, g["k4_q"][i]) == tuple(int(v) for v in g["k4_sm"][i, j])
+
+
+def test_q4k_scale_pack_roundtrip_bruteforce(oracle):
+    """All 64 x 64 (scale, min) values in every one of the 8 positions survive pack -> unpack."""
+    vals = np.arange(64, dtype=np.uint8)
+    for j in range(8):
+        for m in (0, 21, 63):
+            sc = np.zeros((64, 8), np.uint8)
+            mn = np.full((64, 8), m, np.uint8)
+            sc[:, j] = vals
+            q = S.pack_scale_min_k4(sc, mn)
+            for v in range(64):
+                assert oracle.scale_min_k4(j, q[v]) == (v, m)
+            q = S.pack_scale_min_k4(mn, sc)
+            for v in range(64):
+                assert oracle.scale_min_k4(j, q[v]) == (m, v)
+
+
+def test_q4k_closed_form(oracle):
+    """y = d*sc*q - dmin*m with the documented element order (low nibbles then high nibbles of 32 bytes)."""
+    rng = np.random.default_rng(3)
+    raw = S.make_q4k(rng, 1, 512)
+    y = oracle.q4k_rows(raw, 1, 512)[0]
+    for b in range(2):
+        blk = raw[b * 144:(b + 1) * 144]
+        d, dmin = (float(v) for v in blk[:4].copy().view(np.float16).astype(np.float32))
+        for j in range(4):
+            s0, m0 = oracle.scale_min_k4(2 * j, blk[4:16])
+            s1, m1 = oracle.scale_min_k4(2 * j + 1, blk[4:16])
+            qs = blk[16 + 32 * j:16 + 32 * j + 32]
+            lo = np.float32(d * s0) * (qs & 0xF).astype(np.float32) - np.float32(dmin * m0)
+            hi = np.float32(d * s1) * (qs >> 4).astype(np.float32) - np.float32(dmin * m1)
+            got = y[b * 256 + 64 * j: b * 256 + 64 * j + 64]
+            assert same_bits(got[:32], bits(lo)) and same_bits(got[32:], bits(hi))
+
+
+def test_q4k_vs_reference_build(oracle):
+    if oracle.ref() is None:
+        pytest.skip("oracle/_ref not built here")
+    rng = np.random.default_rng(12)
+    raw = S.make_q4k(rng, 5, 1024, scale_std=1.0)
+    assert same_bits(oracle.q4k_rows(raw, 5, 1024), bits(oracle.ref_q4k_rows(raw, 5, 1024)))
+    assert oracle.lib().orc_q4k_row_bytes(3072) == oracle.ref().ref_q4k_row_bytes(3072) == 1728
+
+
+# ---------- router ----------
+def test_router_matches_float64_numpy(oracle):
+    rng = np.random.default_rng(21)
+    E, d, k, T = 64, 96, 10, 9
+    W = rng.standard_normal((E, d)).astype(np.float32) * 0.3
+    x = rng.standard_normal((T, d)).astype(np.float32)
+    logits, ids, ws = oracle.router(oracle.Mat(oracle.F32, W, E, d), x, k)
+    # sequential fp64 accumulation == math.fsum to within the last f32 bit; check exact order on a small case
+    for t in range(T):
+        for e in range(0, E, 7):
+            acc = 0.0
+            for c in range(d):
+                acc += float(W[e, c]) * float(x[t, c])
+            assert np.float32(acc) == logits[t, e]
+        p = np.exp(logits[t].astype(np.float64) - logits[t].max())
+        p = (p.astype(np.float32).astype(np.float64) / p.astype(np.float32).astype(np.float64).sum()).astype(np.float32)
+        order = np.lexsort((np.arange(E), -p))[:k]  # value desc, index asc
+        assert (ids[t, :k] == order).all()
+        w = (p[order].astype(np.float64) / p[order].astype(np.float64).sum()).astype(np.float32)
+        assert (bits(ws[t, :k]) == bits(w)).all()
+        assert abs(float(ws[t, :k].sum()) - 1.0) < 1e-6 and len(set(ids[t, :k])) == k
+
+
+def test_router_ties_and_special_cases(oracle):
+    E, k = 32, 5
+    # uniform logits: every probability equal -> lowest indices, equal weights
+    p, ids, ws = oracle.softmax_topk(np.zeros(E, np.float32), k)
+    assert list(ids) == [0, 1, 2, 3, 4] and np.allclose(ws, 0.2) and np.allclose(p, 1.0 / E)
+    # one-hot: that expert first with weight ~1, the rest tie -> lowest indices
+    lg = np.zeros(E, np.float32)
+    lg[17] = 30.0
+    p, ids, ws = oracle.softmax_topk(lg, k)
+    assert list(ids) == [17, 0, 1, 2, 3] and ws[0] > 0.999
+    # k == E returns a permutation sorted by logit
+    lg = np.random.default_rng(2).standard_normal(E).astype(np.float32)
+    p, ids, ws = oracle.softmax_topk(lg, E)
+    assert (np.diff(lg[ids]) <= 0).all() and sorted(ids) == list(range(E))
+    # pairs of equal logits: lower index wins
+    lg = np.repeat(np.arange(16, dtype=np.float32), 2)[::-1].copy()
+    p, ids, ws = oracle.softmax_topk(lg, 6)
+    assert list(ids) == [0, 1, 2, 3, 4, 5]
+
+
+# ---------- permutation ----------
+def test_route_invariants_and_bruteforce(oracle):
+    rng = np.random.default_rng(31)
+    P, E, k = 300, 40, 6
+    ids = np.zeros((P, 16), np.int32)
+    ws = np.zeros((P, 16), np.float32)
+    for t in range(P):
+        ids[t, :k] = rng.choice(E - 3, k, replace=False)  # experts E-3.. stay empty
+        ws[t, :k] = rng.random(k)
+    tokidx, pw, eoff, pairids = oracle.route(ids, ws, k, E)
+    assert eoff[0] == 0 and eoff[E] == P * k and (np.diff(eoff) >= 0).all()
+    flat = [(ids[t, s], t * k + s) for t in range(P) for s in range(k)]
+    order = sorted(flat)  # stable sort by (expert, original pair index)
+    for q, (e, p0) in enumerate(order):
+        t, s = divmod(p0, k)
+        assert tokidx[q] == t and pw[q] == ws[t, s] and eoff[e] <= q < eoff[e + 1]
+    assert sorted(pairids) == list(range(P * k))
+    for t in range(0, P, 17):
+        es = [ids[t, s] for s in range(k)]
+        for rank, e in enumerate(sorted(es)):
+            q = pairids[t * k + rank]
+            assert tokidx[q] == t and eoff[e] <= q < eoff[e + 1]
+    tl = oracle.tiles(eoff, 64)
+    assert tl[:, 2].sum() == P * k and (tl[:, 2] <= 64).all() and (tl[:, 2] > 0).all()
+    assert (np.diff(tl[:, 0]) >= 0).all()
+
+
+# ---------- the layer ----------
+def test_layer_golden_from_reference_moe(oracle, golden):
+    """Model::moe of the reference (src/ref.cpp:563-637) on tiny synthetic checkpoints: bit-identical y."""
+    g = golden("moe_layer.npz")
+    for i in range(int(g["n"])):
+        d, mid, E, k, sh_dt = (int(v) for v in g[f"cfg{i}"])
+        O = oracle
+        sh = [O.Mat(sh_dt, g[f"shg{i}"], mid, d), O.Mat(sh_dt, g[f"shu{i}"], mid, d),
+              O.Mat(sh_dt, g[f"shd{i}"], d, mid), O.Mat(O.BF16, g[f"sg{i}"], 1, d)]
+        L = O.Layer(d, mid, E, k, O.Mat(O.BF16, g[f"router{i}"], E, d), O.Mat(O.Q4CP, g[f"dn{i}"], E * d, mid),
+                    gate_up=O.Mat(O.Q4CP, g[f"gu{i}"], E * 2 * mid, d), shared=sh)
+        y, ids, ws = O.moe_layer(L, g[f"x{i}"])
+        assert (bits(y) == g[f"ybits{i}"]).all(), f"case {i}"
+        # token subset path gives the same rows
+        y2, _, _ = O.moe_layer(L, g[f"x{i}"], tok_list=[4, 1])
+        assert (bits(y2[[1, 4]]) == g[f"ybits{i}"][[1, 4]]).all() and np.isnan(y2[0]).all()
+
+
+def test_layer_vs_reference_build_random(oracle):
+    if oracle.ref() is None:
+        pytest.skip("oracle/_ref not built here")
+    rng = np.random.default_rng(41)
+    d, mid, E, k = 160, 96, 10, 4
+    hl = HostLayer(rng, d, mid, E, k, router_dtype="bf16", scale_std=0.05, router_std=0.3)
+    L = hl.oracle_layer()
+    # the reference's matvec has no f32 branch: give it the shared gate as bf16 (same values)
+    sg16 = S.f32_to_bf16_bits(hl.shared[3])
+    L.shared[3] = oracle.Mat(oracle.BF16, sg16, 1, d)
+    x = rng.standard_normal((3, d)).astype(np.float32)
+    y, ids, ws = oracle.moe_layer(L, x)
+    for t in range(3):
+        assert (bits(oracle.ref_moe_token(L, x[t])) == bits(y[t])).all()
+
+
+def test_layer_textbook_special_cases(oracle):
+    """Identity-like weights: one expert, codebook value 1 on the diagonal groups -> hand-computable."""
+    O = oracle
+    d = mid = 32
+    E, k = 2, 1
+    cb = np.zeros(16, np.float32)
+    cb[1] = 1.0
+    # expert 0: gate row r = e_r (code 1 at column r), up the same, down identity; expert 1: zeros
+    def eye_codes(rows):
+        c = np.zeros((rows, 16), np.uint8)
+        for r in range(rows):
+            col = r % 32
+            c[r, col // 2] = 1 << (4 * (col % 2))
+        return c
+    gu_codes = np.zeros((E * 2 * mid, 16), np.uint8)
+    gu_codes[:2 * mid] = eye_codes(2 * mid)
+    dn_codes = np.zeros((E * d, 16), np.uint8)
+    dn_codes[:d] = eye_codes(d)
+    one = np.ones((E * 2 * mid, 1), np.float16)
+    gu = S.make_q4cp(None, E * 2 * mid, d, codebook=cb, scales=one, codes=gu_codes)
+    dn = S.make_q4cp(None, E * d, mid, codebook=cb, scales=np.ones((E * d, 1), np.float16), codes=dn_codes)
+    Wr = np.zeros((E, d), np.float32)
+    Wr[0, 0] = 50.0  # x[0] > 0 -> expert 0
+    L = O.Layer(d, mid, E, k, O.Mat(O.F32, Wr, E, d), O.Mat(O.Q4CP, dn, E * d, mid),
+                gate_up=O.Mat(O.Q4CP, gu, E * 2 * mid, d))
+    x = np.linspace(0.5, 2.0, d, dtype=np.float32)[None]
+    y, ids, ws = O.moe_layer(L, x)
+    assert ids[0, 0] == 0 and ws[0, 0] == 1.0
+    want = (x[0] / (1 + np.exp(-x[0].astype(np.float64)))).astype(np.float32) * x[0]  # silu(x)*x
+    assert np.allclose(y[0], want, rtol=1e-6)
+    # zero activations: silu(0)*0 = 0 everywhere
+    y0, _, _ = O.moe_layer(L, np.zeros((1, d), np.float32))
+    assert (y0 == 0).all()
+
+
+def test_layer_matches_float64_numpy_q4k(oracle):
+    """Q4_K layer against an independent numpy float64 evaluation from the dequantised matrices."""
+    O = oracle
+    rng = np.random.default_rng(51)
+    d, mid, E, k = 256, 256, 6, 3
+    hl = HostLayer(rng, d, mid, E, k, fmt="q4k", scale_std=0.02, router_std=0.2)
+    L = hl.oracle_layer()
+    x = rng.standard_normal((4, d)).astype(np.float32)
+    y, ids, ws = O.moe_layer(L, x)
+    G, U, D = L.gate.dequant().astype(np.float64), L.up.dequant().astype(np.float64), L.down.dequant().astype(np.float64)
+    shg, shu, shd, sg = (m.dequant().astype(np.float64) for m in L.shared)
+    for t in range(4):
+        xt = x[t].astype(np.float64)
+        acc = np.zeros(d)
+        for s in range(k):
+            e = ids[t, s]
+            g = G[e * mid:(e + 1) * mid] @ xt
+            u = U[e * mid:(e + 1) * mid] @ xt
+            h = g / (1 + np.exp(-g)) * u
+            acc += float(ws[t, s]) * (D[e * d:(e + 1) * d] @ h)
+        g, u = shg @ xt, shu @ xt
+        ey = shd @ (g / (1 + np.exp(-g)) * u)
+        want = acc + ey / (1 + np.exp(-(sg @ xt)))
+        assert np.abs(y[t] - want).max() <= 2e-5 * np.abs(want).max()
