@@ -167,6 +167,52 @@ def q4cp_gemv_down_topk(dn, hid, ids, ws, kpt, d, ey=None, sg=None):
     return out
 
 
+class LutW(C.Structure):
+    _fields_ = [("w", C.c_void_p), ("w_up", C.c_void_p), ("sc", C.c_void_p), ("sc_up", C.c_void_p),
+                ("cb", C.c_void_p), ("sstride", C.c_int), ("e_rows", C.c_int), ("up_off", C.c_int)]
+
+
+LUT_Q4CP = 100
+
+
+def lut_q4cp_view(blob, rows, cols, e_rows, up_off):
+    p = LutW()
+    check(lib().moe_lut_q4cp_view(ptr(blob), u64(rows), u64(cols), u64(0), e_rows, up_off, C.byref(p)),
+          "moe_lut_q4cp_view")
+    p._keep = blob
+    return p
+
+
+def f32_to_f16(x):
+    out = torch.empty(x.shape, dtype=torch.float16, device=x.device)
+    check(lib().moe_f32_to_f16(ptr(x), ptr(out), u64(x.numel()), stream()), "moe_f32_to_f16")
+    return out
+
+
+def lut_up(p, x16, tokidx, tiles_t, ntiles, mid, npairs):
+    hid = torch.full((npairs, mid), float("nan"), dtype=torch.float16, device=x16.device)
+    check(lib().moe_lut_up(LUT_Q4CP, C.byref(p), ptr(x16), ptr(tokidx), ptr(tiles_t), ptr(ntiles),
+                           tiles_t.shape[0], ptr(hid), mid, x16.shape[1], stream()), "moe_lut_up")
+    return hid
+
+
+def lut_down(p, hid16, tiles_t, ntiles, d, f16=True):
+    npairs = hid16.shape[0]
+    pairs = torch.full((npairs, d), float("nan"), dtype=torch.float16 if f16 else torch.float32,
+                       device=hid16.device)
+    check(lib().moe_lut_down(LUT_Q4CP, C.byref(p), ptr(hid16), ptr(tiles_t), ptr(ntiles), tiles_t.shape[0],
+                             ptr(pairs), d, hid16.shape[1], 1 if f16 else 0, stream()), "moe_lut_down")
+    return pairs
+
+
+def reduce_pw_sg(pairs, pairids, pw, P, K, ey=None, sg=None):
+    D = pairs.shape[1]
+    out = torch.empty((P, D), dtype=torch.float32, device=pairs.device)
+    check(lib().moe_reduce_pw_sg(ptr(pairs), 1 if pairs.dtype == torch.float16 else 0, ptr(pairids), ptr(pw),
+                                 ptr(ey), ptr(sg), ptr(out), P, D, K, stream()), "moe_reduce_pw_sg")
+    return out
+
+
 # ---- model level ----
 
 class Moe:

@@ -25,8 +25,20 @@ struct moe_ctx {
   int* ids = nullptr;         // [T][id_stride]
   float* ws = nullptr;        // [T][id_stride]
   float* sh_logit = nullptr;  // [T]
-  float* hid32 = nullptr;     // [T][k+1][mid] f32 (small-batch path)
+  float* hid32 = nullptr;     // [min(T,small_max)][k+1][mid] f32 (small-batch path)
   int small_max = 32;         // batches up to this size take the in-place GEMV path
+  // batch path (allocated only when max_tokens > small_max)
+  moe_routing* routing = nullptr;
+  __half* x16 = nullptr;      // [T][d]
+  int* tokidx = nullptr;      // [(k+1)T] routed pairs then the shared expert's P pairs
+  float* pw = nullptr;        // [(k+1)T]
+  int* eoff = nullptr;        // [E+1]
+  int* pairids = nullptr;     // [T*k]
+  moe_tile* tiles = nullptr;  // [max_tiles]
+  int* ntiles = nullptr;
+  int max_tiles = 0;
+  __half* hid16 = nullptr;    // [(k+1)T][mid]
+  __half* pairs16 = nullptr;  // [(k+1)T][d]
 };
 
 MOE_API const char* moe_version(void) { return "mi355moe 0.1 (gfx950)"; }
@@ -44,7 +56,9 @@ MOE_API const char* moe_status_string(int status) {
 MOE_API int moe_destroy(moe_ctx* c) {
   if (!c) return MOE_OK;
   int rc = MOE_OK;
-  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->hid32};
+  if (c->routing) rc = moe_routing_destroy(c->routing);
+  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->hid32, c->x16, c->tokidx, c->pw, c->eoff,
+                  c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16};
   for (void* b : bufs)
     if (b) {
       hipError_t e = hipFree(b);
@@ -74,7 +88,26 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   if (e == hipSuccess) e = hipMalloc(&c->ids, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ws, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->sh_logit, T * 4);
-  if (e == hipSuccess) e = hipMalloc(&c->hid32, T * (size_t)(cfg->topk + 1) * cfg->mid * 4);
+  const size_t Ts = T < (size_t)c->small_max ? T : (size_t)c->small_max;
+  if (e == hipSuccess) e = hipMalloc(&c->hid32, Ts * (size_t)(cfg->topk + 1) * cfg->mid * 4);
+  if (e == hipSuccess && T > (size_t)c->small_max) {
+    const size_t k1 = (size_t)cfg->topk + 1, d = cfg->d, mid = cfg->mid;
+    c->max_tiles = (int)((T * cfg->topk + 127) / 128 + E + (T + 127) / 128);
+    int rc = moe_routing_create((int)(T * cfg->topk), cfg->experts, &c->routing);
+    if (rc != MOE_OK) {
+      moe_destroy(c);
+      return rc;
+    }
+    e = hipMalloc(&c->x16, T * d * 2);
+    if (e == hipSuccess) e = hipMalloc(&c->tokidx, k1 * T * 4);
+    if (e == hipSuccess) e = hipMalloc(&c->pw, k1 * T * 4);
+    if (e == hipSuccess) e = hipMalloc(&c->eoff, (E + 2) * 4);
+    if (e == hipSuccess) e = hipMalloc(&c->pairids, T * cfg->topk * 4);
+    if (e == hipSuccess) e = hipMalloc(&c->tiles, (size_t)c->max_tiles * sizeof(moe_tile));
+    if (e == hipSuccess) e = hipMalloc(&c->ntiles, 4);
+    if (e == hipSuccess) e = hipMalloc(&c->hid16, k1 * T * mid * 2);
+    if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);
+  }
   if (e != hipSuccess) {
     moe_destroy(c);
     return (int)e;
@@ -182,6 +215,48 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
                              c->sh_logit, x, c->ids, c->ws, c->hid32, y, P, g.d, g.mid, g.topk, g.id_stride, st);
 }
 
+// Batches: expert-sorted permutation, MFMA grouped GEMMs over <=128-pair tiles (the shared expert
+// rides along as expert index E over all tokens), f16 pair buffer, deterministic weighted combine.
+// Returns MOE_E_UNSUPPORTED (before enqueuing anything) for shapes / formats the GEMM does not cover.
+static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
+  const moe_config& g = c->cfg;
+  if (!L.has_q4cp) return MOE_E_UNSUPPORTED;
+  if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
+  if (g.mid % 128 || g.d % 256 || g.d % 64 || g.mid % 64) return MOE_E_UNSUPPORTED;
+  moe_lutw gu, dn, sgu{}, sdn{};
+  moe_lut_q4cp_view(L.gate_up.data, L.gate_up.rows, L.gate_up.cols, L.gate_up.scale_stride, 2 * g.mid, g.mid, &gu);
+  moe_lut_q4cp_view(L.down.data, L.down.rows, L.down.cols, L.down.scale_stride, g.d, 0, &dn);
+  if (L.has_shared) {
+    moe_lutw t;
+    moe_lut_q4cp_view(L.sh_gate.data, L.sh_gate.rows, L.sh_gate.cols, L.sh_gate.scale_stride, g.mid, 0, &sgu);
+    moe_lut_q4cp_view(L.sh_up.data, L.sh_up.rows, L.sh_up.cols, L.sh_up.scale_stride, g.mid, 0, &t);
+    sgu.w_up = t.w;
+    sgu.sc_up = t.sc;
+    // one codebook per LutW: gate and up of the shared expert must agree (they come from one quantiser)
+    moe_lut_q4cp_view(L.sh_down.data, L.sh_down.rows, L.sh_down.cols, L.sh_down.scale_stride, g.d, 0, &sdn);
+  }
+  int rc;
+  if ((rc = moe_router_logits_seq(&L.router, L.router_bias, x, P, c->logits, st))) return rc;
+  if (L.has_shared && (rc = moe_router_logits_seq(&L.sh_sg, nullptr, x, P, c->sh_logit, st))) return rc;
+  if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
+  if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
+                            g.experts, g.id_stride, st)))
+    return rc;
+  const int sh_first = L.has_shared ? P * g.topk : -1;
+  if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, sh_first, c->tokidx, st)))
+    return rc;
+  if ((rc = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, st))) return rc;
+  const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
+  if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,
+                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, st)))
+    return rc;
+  if ((rc = moe_launch_gemm_q4cp(false, &dn, L.has_shared ? &sdn : nullptr, g.experts, c->hid16, nullptr,
+                                 c->tiles, c->ntiles, max_tiles, c->pairs16, g.d, g.mid, true, st)))
+    return rc;
+  return moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
+                           sh_first, y, P, g.d, g.topk, st);
+}
+
 MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, moe_stream_t st) {
   MoeLayer* L = layer_of(c, layer);
   if (!L || !x || !y || P < 0) return MOE_E_INVALID;
@@ -189,5 +264,14 @@ MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, 
   if (P > c->cfg.max_tokens) return MOE_E_STATE;
   if (!moe_aligned(x, 16) || !moe_aligned(y, 16)) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
-  return forward_small(c, *L, x, P, y, moe_s(st));
+  if (P <= c->small_max) return forward_small(c, *L, x, P, y, moe_s(st));
+  const int rc = forward_batch(c, *L, x, P, y, moe_s(st));
+  if (rc != MOE_E_UNSUPPORTED) return rc;
+  // formats the grouped GEMM does not cover yet: the in-place path, 32 rows at a time
+  for (int t0 = 0; t0 < P; t0 += c->small_max) {
+    const int n = P - t0 < c->small_max ? P - t0 : c->small_max;
+    const int r2 = forward_small(c, *L, x + (size_t)t0 * c->cfg.d, n, y + (size_t)t0 * c->cfg.d, moe_s(st));
+    if (r2) return r2;
+  }
+  return MOE_OK;
 }

@@ -16,3 +16,13 @@ int moe_launch_q4k_gemv(const uint8_t* gate, const uint8_t* up, const uint8_t* d
                         const float* sh_logit, const float* x, const int* ids, const float* ws,
                         float* hid, float* out, int P, int d, int mid, int kpt, int id_stride,
                         hipStream_t st);
+int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
+                         const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
+                         int max_tiles, void* out, int m, int k, bool f16out, hipStream_t st);
+int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E, int cap, int P,
+                            int sh_first, int* tokidx, hipStream_t st);
+int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
+                      const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
+                      hipStream_t st);
+int moe_router_logits_seq(const moe_wview* W, const float* bias, const float* x, int P, float* logits,
+                          hipStream_t st);

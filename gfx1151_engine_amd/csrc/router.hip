@@ -236,6 +236,17 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
   return MOE_OK;
 }
 
+// Internal: sequential-order logits for any P (also used for the one-row shared-expert gate).
+int moe_router_logits_seq(const moe_wview* W, const float* bias, const float* x, int P, float* logits,
+                          hipStream_t st) {
+  const int E = (int)W->rows, d = (int)W->cols;
+  dim3 g((E + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
+  if (W->dtype == MOE_DT_BF16) k_router_logits_seq<true><<<g, 256, 0, st>>>(W->data, bias, x, P, E, d, logits);
+  else k_router_logits_seq<false><<<g, 256, 0, st>>>(W->data, bias, x, P, E, d, logits);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
 // Internal: small-P logits plus the shared-expert gate row in the same launch.
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, hipStream_t st) {

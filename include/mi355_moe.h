@@ -116,6 +116,38 @@ int moe_gg_gemv(int tgu, int tdn, const uint8_t* gate, const uint8_t* up, const 
                 const float* x, const int* ids, const float* ws, float* hid, float* out, int P,
                 int d, int mid, int kpt, int id_stride, moe_stream_t st);
 
+/* ---- prefill path: grouped GEMM on MFMA over expert-sorted tiles ---- */
+
+/* LutW (src/gpu/parts/27_kernels_moe_lut.inc:75-83): q4cp operand planes of an expert tensor.
+ * Expert e's gate rows start at row e*e_rows of (w, sc), its up rows at row e*e_rows + up_off of
+ * (w_up, sc_up); down tensors use (w, sc) only. */
+typedef struct moe_lutw {
+  const uint8_t *w, *w_up, *sc, *sc_up;
+  const float* cb;
+  int sstride, e_rows, up_off;
+} moe_lutw;
+enum { MOE_LUT_Q4CP = 100 }; /* moelut::kQ4CP (27_kernels_moe_lut.inc:33) */
+/* lut_q4cp_view (27_kernels_moe_lut.inc:811) */
+int moe_lut_q4cp_view(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t scale_stride,
+                      int e_rows, int up_off, moe_lutw* out);
+/* k_f32_to_f16_v4 (26_kernels_moe_gguf.inc:389): round-to-nearest-even, n % 4 == 0 */
+int moe_f32_to_f16(const float* x, void* x16, uint64_t n, moe_stream_t st);
+/* moe_lut_up (27_kernels_moe_lut.inc:660): hid16[pair][m] = f16(silu(gate) * up) for every tile
+ * (tiles hold <= 128 pairs); x16: f16 [P][k] gathered through tokidx; m % 128 == 0, k % 64 == 0. */
+int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* tokidx,
+               const moe_tile* tiles, const int* ntiles, int max_tiles, void* hid16, int m, int k,
+               moe_stream_t st);
+/* moe_lut_down (27_kernels_moe_lut.inc:765): pairs[pair][m] (unweighted; f32, or f16 if f16 != 0)
+ * = W_e[m][k] . hid16[pair]; m % 256 == 0, k % 64 == 0. */
+int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
+                 const int* ntiles, int max_tiles, void* pairs, int m, int k, int f16,
+                 moe_stream_t st);
+/* k_moe_reduce_pw / k_moe_reduce_pw_sg (src/gpu/parts/24_kernels_moe_lt.inc:82,104):
+ * out[t] = sum_s pw[pid_s] * pairs[pid_s] in pairids order (+ sigmoid(sg[t]) * ey[t] if given). */
+int moe_reduce_pw_sg(const void* pairs, int pairs_f16, const int* pairids, const float* pw,
+                     const float* ey, const float* sg, float* out, int P, int D, int K,
+                     moe_stream_t st);
+
 /* ---- model level ---- */
 
 typedef struct moe_config {

@@ -1,0 +1,113 @@
+"""GPU parity of the batch (prefill) path: MFMA grouped GEMM stages against fp64 evaluations of the
+oracle's dequantised weights, and the whole layer against the oracle within max-abs-rel 2e-3."""
+import numpy as np
+import pytest
+
+from gfx1151_engine_amd import synth as S
+from helpers import HostLayer, max_abs_rel
+
+pytestmark = pytest.mark.gpu
+TOL_LAYER = 2e-3  # north-star tolerance: f16 MFMA operands, f32 accumulation, vs the fp64/f32 CPU path
+
+
+def gpu(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from gfx1151_engine_amd import capi as c
+    c.lib()
+    return c
+
+
+def make_routing(rng, P, E, k, counts=None):
+    ids = np.zeros((P, 16), np.int32)
+    ws = np.zeros((P, 16), np.float32)
+    for t in range(P):
+        ids[t, :k] = rng.choice(E, k, replace=False)
+        w = rng.random(k).astype(np.float32) + 0.1
+        ws[t, :k] = w / w.sum()
+    return ids, ws
+
+
+@pytest.mark.parametrize("d,mid,E,k,P,cb", [(256, 128, 6, 2, 300, "zp8"), (3072, 768, 8, 4, 200, "zp8"),
+                                            (512, 256, 5, 3, 150, "random")])
+def test_grouped_gemm_stages(capi, oracle, d, mid, E, k, P, cb):
+    """up -> hid16, down -> pairs, reduce -> y, each against fp64 from the oracle's weights.
+    Expert 0 is left empty and one expert gets a 1-pair tile and a 129-pair run (tile edge cases,
+    reference: tools/ktest.cu:2588-2592 uses counts {0,1,63,64,65,2})."""
+    import torch
+    rng = np.random.default_rng(d + P)
+    codebook = None if cb == "zp8" else rng.uniform(-2, 2, 16).astype(np.float32)
+    gu = S.make_q4cp(rng, E * 2 * mid, d, codebook=codebook, scale_std=0.02)
+    dn = S.make_q4cp(rng, E * d, mid, codebook=codebook, scale_std=0.02)
+    x = rng.standard_normal((P, d), dtype=np.float32)
+    ids, ws = make_routing(rng, P, E - 1, k)
+    ids[:, :k] += 1  # expert 0 empty
+    x16 = capi.f32_to_f16(gpu(x))
+    assert (x16.cpu().numpy() == x.astype(np.float16)).all()
+    r = capi.Routing(P * k, E)
+    tokidx, pw, eoff, pairids = r.run(gpu(ids), gpu(ws), k)
+    tiles_t, ntiles = capi.tiles(eoff, 128, P * k)
+    pgu = capi.lut_q4cp_view(gpu(gu), E * 2 * mid, d, 2 * mid, mid)
+    pdn = capi.lut_q4cp_view(gpu(dn), E * d, mid, d, 0)
+    hid = capi.lut_up(pgu, x16, tokidx, tiles_t, ntiles, mid, P * k)
+    pairs = capi.lut_down(pdn, hid, tiles_t, ntiles, d, f16=False)
+    pairs16 = capi.lut_down(pdn, hid, tiles_t, ntiles, d, f16=True)
+    y = capi.reduce_pw_sg(pairs, pairids, pw, P, k)
+    hid, pairs, pairs16, y = hid.cpu().numpy(), pairs.cpu().numpy(), pairs16.cpu().numpy(), y.cpu().numpy()
+    assert not np.isnan(hid).any() and not np.isnan(pairs).any(), "every pair row must be written"
+    tokidx, pw, eoff = tokidx.cpu().numpy(), pw.cpu().numpy(), eoff.cpu().numpy()
+    GU = oracle.q4cp_rows(gu, E * 2 * mid, d, 0, E * 2 * mid).astype(np.float64)
+    DN = oracle.q4cp_rows(dn, E * d, mid, 0, E * d).astype(np.float64)
+    x64 = x.astype(np.float16).astype(np.float64)
+    yref = np.zeros((P, d))
+    for e in range(E):
+        sl = slice(eoff[e], eoff[e + 1])
+        if sl.start == sl.stop:
+            continue
+        xe = x64[tokidx[sl]]
+        g = xe @ GU[e * 2 * mid:e * 2 * mid + mid].T
+        u = xe @ GU[e * 2 * mid + mid:(e + 1) * 2 * mid].T
+        h = g / (1 + np.exp(-g)) * u
+        assert np.abs(hid[sl] - h).max() <= 3e-3 * np.abs(h).max(), e
+        pr = hid[sl].astype(np.float64) @ DN[e * d:(e + 1) * d].T
+        assert np.abs(pairs[sl] - pr).max() <= 2e-3 * np.abs(pr).max(), e
+        assert np.abs(pairs16[sl] - pr).max() <= 3e-3 * np.abs(pr).max(), e
+        np.add.at(yref, tokidx[sl], pw[sl, None].astype(np.float64) * pairs[sl].astype(np.float64))
+    assert np.abs(y - yref).max() <= 1e-5 * np.abs(yref).max()
+    r.close()
+
+
+@pytest.mark.parametrize("d,mid,E,k,T,skew", [(512, 256, 16, 4, 333, False), (3072, 768, 64, 10, 700, True),
+                                              (1024, 256, 8, 3, 33, False)])
+def test_batch_layer_vs_oracle(oracle, d, mid, E, k, T, skew):
+    rng = np.random.default_rng(d * 3 + T)
+    bias = S.zipf_bias(rng, E, 1.1, 1.0) if skew else None
+    hl = HostLayer(rng, d, mid, E, k, bias=bias)
+    x = S.bf16_round(rng.standard_normal((T, d), dtype=np.float32))
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    y = m.forward(0, gpu(x))
+    ids, ws = m.last_routing(T)
+    y, ids, ws = y.cpu().numpy(), ids.cpu().numpy(), ws.cpu().numpy()
+    assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
+    assert (ws[:, :k].view(np.uint32) == wo[:, :k].view(np.uint32)).all(), "sequential-order router weights are bit-exact"
+    err = max_abs_rel(y, yo)
+    assert err <= TOL_LAYER, err
+    m.close()
+
+
+def test_batch_equals_small_path_statistically(oracle):
+    """Same layer through the MFMA path (T=40) and the f32 in-place path (two calls of 20)."""
+    rng = np.random.default_rng(5)
+    hl = HostLayer(rng, 1024, 256, 12, 4)
+    x = rng.standard_normal((40, 1024), dtype=np.float32)
+    m, dev = hl.to_gpu(max_tokens=64)
+    xb = gpu(x)
+    yb = m.forward(0, xb).cpu().numpy()
+    ys = np.concatenate([m.forward(0, xb[:20].contiguous()).cpu().numpy(), m.forward(0, xb[20:].contiguous()).cpu().numpy()])
+    assert max_abs_rel(yb, ys) <= TOL_LAYER
+    m.close()
