@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""Benchmark of the routed-expert MoE layer on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|decode|verify|q4k_prefill|q4k_decode|stack]
+
+One step = one pass of the MoE layer (moe_forward) over one batch of synthetic input that is
+already resident in HBM.  Prints ONE JSON line: whole-layer throughput, the roofline figure of the
+dominant kernel (timed live with HIP events on the launch stream) and the CPU oracle timed on the
+host cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="prefill")
+    ap.add_argument("--tokens", type=int, default=0, help="override the batch size of the workload")
+    ap.add_argument("--layers", type=int, default=48, help="stack workload: number of resident layers")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from gfx1151_engine_amd import capi, workloads as W
+    from gfx1151_engine_amd import synth as S
+    capi.lib()
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    d, mid, E, k = 3072, 768, 512, 10
+    wl = a.workload
+    fmt = "q4k" if wl.startswith("q4k") else "q4cp"
+    kind = wl.replace("q4k_", "")
+    T = a.tokens or {"prefill": 16384 if fmt == "q4cp" else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
+    nlayers = a.layers if kind == "stack" else 1
+
+    layers = [W.DeviceLayer(1000 + l, d, mid, E, k, fmt) for l in range(nlayers)]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(99)
+    extra = {}
+    if kind == "prefill":
+        x = torch.randn((T, d), device="cuda", generator=g).to(torch.bfloat16).to(torch.float32)
+        bias, beta = W.calibrate_zipf(layers[0].router, x, k)
+        layers[0].bias = bias
+        xs = [x]
+        extra["zipf_beta"] = round(beta, 4)
+    elif kind == "verify":
+        xs = [W.verify_batch(layers[0].router, d, T, seed=5 + i) for i in range(64)]
+    else:
+        # decode: rotate 64 different tokens so that no cache level can hold the experts of a step
+        xs = [torch.randn((T, d), device="cuda", generator=g) for _ in range(64)]
+    m = capi.Moe(d, mid, E, k, layers=nlayers, max_tokens=T)
+    for l, L in enumerate(layers):
+        L.register(m, l)
+    y = torch.empty((T, d), dtype=torch.float32, device="cuda")
+
+    def step(i):
+        if kind == "stack":
+            for l in range(nlayers):
+                m.forward(l, xs[(i * nlayers + l) % len(xs)], y)
+        else:
+            m.forward(0, xs[i % len(xs)], y)
+
+    for i in range(a.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    # whole-job timing: K steps between two synchronisations, HIP events on the launch stream
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(a.steps):
+        step(a.warmup + i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    ms = e0.elapsed_time(e1) / a.steps
+
+    # per-stage timing (HIP events recorded by the library between its kernels, same stream)
+    m.profile(True)
+    stage = {}
+    nprof = max(5, min(a.steps, 20))
+    for i in range(nprof):
+        lsel = i % nlayers
+        m.forward(lsel, xs[i % len(xs)], y)
+        for kk, v in m.profile_read().items():
+            stage[kk] = stage.get(kk, 0.0) + v / nprof
+    m.profile(False)
+
+    # routing statistics of the last step (for the algorithmic byte / flop counts)
+    ids, _ = m.last_routing(T)
+    ids = ids[:, :k].cpu().numpy()
+    eb = layers[0].expert_bytes()
+    uniq = int(np.unique(ids).size)
+    cnt = np.bincount(ids.reshape(-1), minlength=E)
+    pairs = T * k
+    res = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
+           "host_ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "data": "synthetic", "stage_ms": {kk: round(v, 5) for kk, v in stage.items()}}
+    cfg = {"workload": wl, "tokens": T, "d_model": d, "moe_mid": mid, "experts": E, "topk": k, "shared_experts": 1,
+           "format": "q4cp g32 zero-point 8" if fmt == "q4cp" else "GGUF Q4_K", "layers": nlayers, **extra}
+    if kind == "prefill":
+        flop_tok = k * 6 * d * mid + 6 * d * mid + 2 * d * E + 2 * d
+        up_flop = (pairs + T) * 2 * (2 * mid) * d  # gate+up GEMM incl. shared expert, one launch
+        up_s = stage["up"] * 1e-3
+        res.update({"metric": "moe_layer_prefill_tokens_per_s", "unit": "tok/s", "value": round(T / (ms * 1e-3), 1),
+                    "dtype": "f16",
+                    "layer_tflops": round(flop_tok * T / (ms * 1e-3) / 1e12, 2),
+                    "roofline": {"bound": "mfma", "kernel": "k_moe_gemm (gate/up + SwiGLU)",
+                                 "achieved": round(up_flop / up_s / 1e12, 2), "peak": MFMA_F16_PEAK_TFLOPS,
+                                 "unit": "TFLOP/s", "frac": round(up_flop / up_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                                 "traffic": None}})
+        cfg.update({"hottest_over_mean": round(float(cnt.max() / cnt.mean()), 2), "empty_experts": int((cnt == 0).sum())})
+    else:
+        # algorithmic bytes of a step: unique experts + shared expert + fp32 router + gate vector + x/y
+        step_bytes = nlayers * ((uniq if kind != "stack" else k) + 1) * eb + nlayers * (E * d * 4 + d * 4 + T * 2 * d * 4)
+        if kind == "stack":
+            uniq = k
+        gu_bytes = (uniq + 1) * 2 * mid * (eb // (2 * mid + d) if False else 0)  # placeholder, fixed below
+        if fmt == "q4cp":
+            gu_row = d // 2 + S.q4cp_scale_stride(d)
+        else:
+            gu_row = S.q4k_row_bytes(d)
+        gu_bytes = (uniq + 1) * 2 * mid * gu_row
+        up_s = stage["up"] * 1e-3
+        res.update({"metric": "moe_layer_decode_hbm_GB_per_s", "unit": "GB/s",
+                    "value": round(step_bytes / (ms * 1e-3) / 1e9, 1), "dtype": "f32",
+                    "tokens_per_s": round(T / (ms * 1e-3), 1),
+                    "roofline": {"bound": "hbm", "kernel": "gate/up GEMV + SwiGLU",
+                                 "achieved": round(gu_bytes / up_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                 "frac": round(gu_bytes / up_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None}})
+        cfg.update({"unique_experts": uniq, "step_bytes": int(step_bytes)})
+    res["config"] = cfg
+
+    if not a.no_cpu:
+        from oracle import oracle as O
+        ol = layers[0].oracle_layer()
+        if kind == "prefill":
+            nsamp = 32
+            hot = int(np.argmax(cnt))
+            toks = np.concatenate([np.where((ids == hot).any(1))[0][:8], np.arange(nsamp)])[:nsamp]
+            xc = xs[0][torch.from_numpy(toks).cuda()].cpu().numpy()
+        else:
+            nsamp = T
+            xc = xs[0].cpu().numpy()
+        t0 = time.perf_counter()
+        yo, io, wo = O.moe_layer(ol, xc)
+        cpu_s = time.perf_counter() - t0
+        yg = torch.empty((nsamp, d), dtype=torch.float32, device="cuda")
+        m2 = None
+        if kind == "prefill":
+            m.forward(0, xs[0], y)
+            yg = y[torch.from_numpy(toks).cuda()]
+        else:
+            m.forward(0, xs[0], yg)
+        yg = yg.cpu().numpy()
+        err = float(np.abs(yg.astype(np.float64) - yo).max() / np.abs(yo).max())
+        if kind == "prefill":
+            cpu = {"value": round(nsamp / cpu_s, 3), "unit": "tok/s"}
+        else:
+            cb = (int(np.unique(io[:, :k]).size) + 1) * eb + E * d * 4 + d * 4 + T * 2 * d * 4
+            cpu = {"value": round(cb / cpu_s / 1e9, 4), "unit": "GB/s"}
+        cpu.update({"cores": O.num_threads(), "kind": "port", "seconds": round(cpu_s, 3),
+                    "sample": f"{nsamp} tokens of the same batch through the OpenMP restatement of src/ref.cpp Model::moe",
+                    "max_abs_rel_vs_gpu": err})
+        res["cpu_baseline"] = cpu
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

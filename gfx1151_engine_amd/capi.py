@@ -250,6 +250,15 @@ class Moe:
         check(lib().moe_forward(self.h, layer, ptr(x), P, ptr(y), stream()), "moe_forward")
         return y
 
+    def profile(self, on=True):
+        check(lib().moe_profile_enable(self.h, 1 if on else 0), "moe_profile_enable")
+
+    def profile_read(self):
+        """-> dict stage -> ms of the last forward (router, route, up, down, reduce)."""
+        ms = (C.c_float * 5)()
+        check(lib().moe_profile_read(self.h, ms), "moe_profile_read")
+        return dict(zip(("router", "route", "up", "down", "reduce"), [float(v) for v in ms]))
+
     def last_routing(self, P):
         S = self.cfg.id_stride
         ids = torch.empty((P, S), dtype=torch.int32, device="cuda")

@@ -39,7 +39,20 @@ struct moe_ctx {
   int max_tiles = 0;
   __half* hid16 = nullptr;    // [(k+1)T][mid]
   __half* pairs16 = nullptr;  // [(k+1)T][d]
+  // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
+  bool profile = false;
+  hipEvent_t ev[MOE_PROF_STAGES + 1] = {};
+  int ev_n = 0;            // events recorded by the last call
+  int ev_stage[MOE_PROF_STAGES] = {};
 };
+
+static void prof_mark(moe_ctx* c, int stage_done, hipStream_t st) {
+  // event i closes stage ev_stage[i-1]; event 0 opens the call
+  if (!c->profile || c->ev_n > MOE_PROF_STAGES) return;
+  if (hipEventRecord(c->ev[c->ev_n], st) != hipSuccess) return;
+  if (c->ev_n > 0) c->ev_stage[c->ev_n - 1] = stage_done;
+  c->ev_n++;
+}
 
 MOE_API const char* moe_version(void) { return "mi355moe 0.1 (gfx950)"; }
 
@@ -57,6 +70,8 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (!c) return MOE_OK;
   int rc = MOE_OK;
   if (c->routing) rc = moe_routing_destroy(c->routing);
+  for (hipEvent_t e : c->ev)
+    if (e) (void)hipEventDestroy(e);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->hid32, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16};
   for (void* b : bufs)
@@ -108,6 +123,7 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
     if (e == hipSuccess) e = hipMalloc(&c->hid16, k1 * T * mid * 2);
     if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);
   }
+  for (int i = 0; i <= MOE_PROF_STAGES && e == hipSuccess; i++) e = hipEventCreate(&c->ev[i]);
   if (e != hipSuccess) {
     moe_destroy(c);
     return (int)e;
@@ -181,6 +197,26 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
   return MOE_OK;
 }
 
+MOE_API int moe_profile_enable(moe_ctx* c, int on) {
+  if (!c) return MOE_E_INVALID;
+  c->profile = on != 0;
+  c->ev_n = 0;
+  return MOE_OK;
+}
+
+MOE_API int moe_profile_read(moe_ctx* c, float* ms) {
+  if (!c || !ms) return MOE_E_INVALID;
+  for (int i = 0; i < MOE_PROF_STAGES; i++) ms[i] = 0.f;
+  if (c->ev_n < 2) return MOE_E_STATE;
+  MOE_HIP(hipEventSynchronize(c->ev[c->ev_n - 1]));
+  for (int i = 1; i < c->ev_n; i++) {
+    float t = 0.f;
+    MOE_HIP(hipEventElapsedTime(&t, c->ev[i - 1], c->ev[i]));
+    ms[c->ev_stage[i - 1]] += t;
+  }
+  return MOE_OK;
+}
+
 MOE_API int moe_get_routing(moe_ctx* c, int P, int* ids_out, float* ws_out, moe_stream_t st) {
   if (!c || P < 0 || P > c->cfg.max_tokens) return MOE_E_INVALID;
   const size_t n = (size_t)P * c->cfg.id_stride * 4;
@@ -196,18 +232,24 @@ MOE_API int moe_get_routing(moe_ctx* c, int P, int* ids_out, float* ws_out, moe_
 static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
   const moe_config& g = c->cfg;
   int rc;
+  c->ev_n = 0;
+  prof_mark(c, 0, st);
   if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
                                     c->logits, c->sh_logit, st)))
     return rc;
   if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
+  prof_mark(c, MOE_PROF_ROUTER, st);
   if (L.has_q4cp) {
     if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
     if ((rc = moe_launch_gemv_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
                                  L.has_shared ? &L.sh_up : nullptr, x, (uint64_t)g.d, c->ids, g.id_stride,
                                  g.topk, P, g.mid, c->hid32, st)))
       return rc;
-    return moe_launch_gemv_dn(&L.down, L.has_shared ? &L.sh_down : nullptr, c->sh_logit, nullptr, nullptr,
-                              c->hid32, c->ids, c->ws, g.id_stride, g.topk, P, g.d, y, (uint64_t)g.d, st);
+    prof_mark(c, MOE_PROF_UP, st);
+    rc = moe_launch_gemv_dn(&L.down, L.has_shared ? &L.sh_down : nullptr, c->sh_logit, nullptr, nullptr,
+                            c->hid32, c->ids, c->ws, g.id_stride, g.topk, P, g.d, y, (uint64_t)g.d, st);
+    prof_mark(c, MOE_PROF_DOWN, st);
+    return rc;
   }
   if (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
   return moe_launch_q4k_gemv(L.gg.gate, L.gg.up, L.gg.down, L.has_shared ? L.sh_gate.data : nullptr,
@@ -236,9 +278,12 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     moe_lut_q4cp_view(L.sh_down.data, L.sh_down.rows, L.sh_down.cols, L.sh_down.scale_stride, g.d, 0, &sdn);
   }
   int rc;
+  c->ev_n = 0;
+  prof_mark(c, 0, st);
   if ((rc = moe_router_logits_seq(&L.router, L.router_bias, x, P, c->logits, st))) return rc;
   if (L.has_shared && (rc = moe_router_logits_seq(&L.sh_sg, nullptr, x, P, c->sh_logit, st))) return rc;
   if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
+  prof_mark(c, MOE_PROF_ROUTER, st);
   if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
                             g.experts, g.id_stride, st)))
     return rc;
@@ -246,15 +291,20 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, sh_first, c->tokidx, st)))
     return rc;
   if ((rc = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, st))) return rc;
+  prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
   if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,
                                  c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, st)))
     return rc;
+  prof_mark(c, MOE_PROF_UP, st);
   if ((rc = moe_launch_gemm_q4cp(false, &dn, L.has_shared ? &sdn : nullptr, g.experts, c->hid16, nullptr,
                                  c->tiles, c->ntiles, max_tiles, c->pairs16, g.d, g.mid, true, st)))
     return rc;
-  return moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
-                           sh_first, y, P, g.d, g.topk, st);
+  prof_mark(c, MOE_PROF_DOWN, st);
+  rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
+                         sh_first, y, P, g.d, g.topk, st);
+  prof_mark(c, MOE_PROF_REDUCE, st);
+  return rc;
 }
 
 MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, moe_stream_t st) {

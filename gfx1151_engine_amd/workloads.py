@@ -1,0 +1,149 @@
+"""Full-size synthetic MoE layers generated directly in HBM (torch is only the allocator / RNG).
+
+Byte layouts are the engine's: hgn q4cp blobs and GGUF Q4_K raw blocks.  The CPU oracle is fed the
+very same bytes, read back from the device, so both sides see identical weights.
+"""
+import numpy as np
+import torch
+
+from . import capi
+from . import synth as S
+
+
+def _gen(seed):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    return g
+
+
+def q4cp_blob(g, rows, cols, scale_std=0.01):
+    """uint8 tensor [64 + rows*cols/2 + rows*ss]: zero-point-8 codebook, uniform codes, fp16 |N|*std scales."""
+    ss = S.q4cp_scale_stride(cols)
+    nb = rows * cols // 2
+    blob = torch.empty(64 + nb + rows * ss, dtype=torch.uint8, device="cuda")
+    blob[:64] = torch.from_numpy(S.ZP8_CODEBOOK.view(np.uint8).copy()).cuda()
+    step = 1 << 28
+    for i in range(0, nb, step):
+        n = min(step, nb - i)
+        blob[64 + i:64 + i + n] = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    rec = blob[64 + nb:].view(rows, ss)
+    rec.zero_()
+    G = cols // 32
+    crow = max(1, (1 << 26) // G)
+    for r0 in range(0, rows, crow):
+        r1 = min(rows, r0 + crow)
+        sc = (torch.randn((r1 - r0, G), device="cuda", generator=g).abs() * scale_std).to(torch.float16)
+        rec[r0:r1, :G * 2] = sc.view(torch.uint8)
+    return blob
+
+
+def q4k_rows(g, rows, cols, scale_std=0.01):
+    """uint8 tensor of rows*cols/256 Q4_K super-blocks (144 B): d,dmin fp16 |N|*std; 6-bit sub-scales/mins
+    uniform [0,63]; codes uniform."""
+    nb = rows * cols // 256
+    blk = torch.empty((nb, 144), dtype=torch.uint8, device="cuda")
+    dd = (torch.randn((nb, 2), device="cuda", generator=g).abs() * scale_std).to(torch.float16)
+    blk[:, 0:4] = dd.view(torch.uint8)
+    sc = torch.randint(0, 64, (nb, 8), dtype=torch.uint8, device="cuda", generator=g)
+    mn = torch.randint(0, 64, (nb, 8), dtype=torch.uint8, device="cuda", generator=g)
+    q = torch.empty((nb, 12), dtype=torch.uint8, device="cuda")
+    for j in range(4):
+        q[:, j] = (sc[:, j] & 63) | ((sc[:, j + 4] >> 4) << 6)
+        q[:, j + 4] = (mn[:, j] & 63) | ((mn[:, j + 4] >> 4) << 6)
+        q[:, j + 8] = (sc[:, j + 4] & 0xF) | ((mn[:, j + 4] & 0xF) << 4)
+    blk[:, 4:16] = q
+    step = max(1, (1 << 28) // 128)
+    for i in range(0, nb, step):
+        n = min(step, nb - i)
+        blk[i:i + n, 16:] = torch.randint(0, 256, (n, 128), dtype=torch.uint8, device="cuda", generator=g)
+    return blk.view(-1)
+
+
+class DeviceLayer:
+    """One layer's weights in HBM + registration into a capi.Moe context."""
+
+    def __init__(self, seed, d=3072, mid=768, E=512, k=10, fmt="q4cp", bias=None):
+        g = _gen(seed)
+        self.d, self.mid, self.E, self.k, self.fmt = d, mid, E, k, fmt
+        self.router = torch.randn((E, d), device="cuda", generator=g) * 0.02
+        self.sh_sg = torch.randn((1, d), device="cuda", generator=g) * 0.02
+        self.bias = bias
+        if fmt == "q4cp":
+            self.gate_up = q4cp_blob(g, E * 2 * mid, d)
+            self.down = q4cp_blob(g, E * d, mid)
+            self.sh = [q4cp_blob(g, mid, d), q4cp_blob(g, mid, d), q4cp_blob(g, d, mid)]
+        else:
+            self.gate = q4k_rows(g, E * mid, d)
+            self.up = q4k_rows(g, E * mid, d)
+            self.down = q4k_rows(g, E * d, mid)
+            self.sh = [q4k_rows(g, mid, d), q4k_rows(g, mid, d), q4k_rows(g, d, mid)]
+
+    def expert_bytes(self):
+        d, mid = self.d, self.mid
+        if self.fmt == "q4cp":
+            return 2 * mid * (d // 2 + S.q4cp_scale_stride(d)) + d * (mid // 2 + S.q4cp_scale_stride(mid))
+        return 2 * mid * S.q4k_row_bytes(d) + d * S.q4k_row_bytes(mid)
+
+    def register(self, m, layer=0):
+        d, mid, E = self.d, self.mid, self.E
+        m.set_router(layer, capi.wview(self.router, capi.F32, E, d), self.bias)
+        if self.fmt == "q4cp":
+            m.set_experts_q4cp(layer, capi.wview(self.gate_up, capi.Q4CP, E * 2 * mid, d),
+                               capi.wview(self.down, capi.Q4CP, E * d, mid))
+            wt, gt = capi.Q4CP, 0
+        else:
+            m.set_experts_gguf(layer, self.gate, self.up, self.down)
+            wt, gt = 0, capi.GGML_Q4_K
+        m.set_shared(layer, capi.wview(self.sh[0], wt, mid, d), capi.wview(self.sh[1], wt, mid, d),
+                     capi.wview(self.sh[2], wt, d, mid), capi.wview(self.sh_sg, capi.F32, 1, d), gt)
+
+    def oracle_layer(self):
+        """The same bytes, copied to the host, as an oracle layer (test / cpu_baseline use only)."""
+        from oracle import oracle as O
+        d, mid, E, k = self.d, self.mid, self.E, self.k
+        wt = O.Q4CP if self.fmt == "q4cp" else O.Q4K
+        h = lambda t: t.cpu().numpy()
+        sh = [O.Mat(wt, h(self.sh[0]), mid, d), O.Mat(wt, h(self.sh[1]), mid, d), O.Mat(wt, h(self.sh[2]), d, mid),
+              O.Mat(O.F32, h(self.sh_sg), 1, d)]
+        router = O.Mat(O.F32, h(self.router), E, d)
+        bias = h(self.bias) if self.bias is not None else None
+        if self.fmt == "q4cp":
+            return O.Layer(d, mid, E, k, router, O.Mat(wt, h(self.down), E * d, mid),
+                           gate_up=O.Mat(wt, h(self.gate_up), E * 2 * mid, d), shared=sh, router_bias=bias)
+        return O.Layer(d, mid, E, k, router, O.Mat(wt, h(self.down), E * d, mid),
+                       gate=O.Mat(wt, h(self.gate), E * mid, d), up=O.Mat(wt, h(self.up), E * mid, d),
+                       shared=sh, router_bias=bias)
+
+
+def calibrate_zipf(router, x, k, s=1.1, target=12.0, seed=3):
+    """Per-expert logit bias b_e = -beta*s*ln(rank_e) (random rank permutation), beta chosen so that the
+    hottest expert receives ~target x the mean pair count.  Uses plain torch only to pick beta."""
+    E = router.shape[0]
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    rank = (torch.randperm(E, generator=g) + 1).to(torch.float32).cuda()
+    logits = x @ router.T
+    lo, hi = 0.0, 4.0
+    for _ in range(20):
+        beta = 0.5 * (lo + hi)
+        b = -beta * s * torch.log(rank)
+        top = torch.topk(logits + b, k, dim=1).indices
+        cnt = torch.bincount(top.reshape(-1), minlength=E).float()
+        ratio = (cnt.max() / cnt.mean()).item()
+        if ratio < target:
+            lo = beta
+        else:
+            hi = beta
+    beta = 0.5 * (lo + hi)
+    return (-beta * s * torch.log(rank)).contiguous(), beta
+
+
+def verify_batch(router, d, T=20, share=0.3, k=10, seed=5):
+    """Activations for a speculative-verify batch: ~share of the tokens are small perturbations of a
+    template token, so their router logits reproduce its top-k set."""
+    g = _gen(seed)
+    x = torch.randn((T, d), device="cuda", generator=g)
+    n = int(round(share * T))
+    for i in range(1, n):
+        x[i] = x[0] + 1e-3 * torch.randn((d,), device="cuda", generator=g)
+    return x

@@ -176,6 +176,15 @@ int moe_set_shared(moe_ctx* ctx, int layer, const moe_wview* gate_proj, const mo
  * batch: y[P][d] = routed experts (top-k, renormalised) + sigmoid-gated shared expert.
  * x, y: f32 [P][d]; y is fully overwritten. */
 int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_stream_t st);
+/* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
+ * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP
+ * events between its stages; moe_profile_read waits for the last one and fills
+ * ms[MOE_PROF_STAGES] (router = logits + top-k; route = permutation + tiles + f16 conversion;
+ * up / down = the expert GEMM or GEMV kernels; reduce = weighted combine). */
+enum { MOE_PROF_ROUTER = 0, MOE_PROF_ROUTE = 1, MOE_PROF_UP = 2, MOE_PROF_DOWN = 3, MOE_PROF_REDUCE = 4,
+       MOE_PROF_STAGES = 5 };
+int moe_profile_enable(moe_ctx* ctx, int on);
+int moe_profile_read(moe_ctx* ctx, float* ms);
 /* Copy the last call's router output (the reference keeps it in d_topids / d_topw,
  * 40_model.inc:1811) into caller buffers [P][id_stride] (device memory; async on st). */
 int moe_get_routing(moe_ctx* ctx, int P, int* ids_out, float* ws_out, moe_stream_t st);
