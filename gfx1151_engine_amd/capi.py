@@ -183,10 +183,20 @@ def lut_q4cp_view(blob, rows, cols, e_rows, up_off):
     return p
 
 
-def f32_to_f16(x):
+def f32_to_f16(x, layout=1):
     out = torch.empty(x.shape, dtype=torch.float16, device=x.device)
-    check(lib().moe_f32_to_f16(ptr(x), ptr(out), u64(x.numel()), stream()), "moe_f32_to_f16")
+    check(lib().moe_f32_to_f16(ptr(x), ptr(out), u64(x.numel()), layout, stream()), "moe_f32_to_f16")
     return out
+
+
+ILV = [0, 4, 1, 5, 2, 6, 3, 7]  # layout 1: position p of a group of 8 holds element ILV[p]
+
+
+def from_layout1(t):
+    """Undo the interleaved f16 activation order (last dim, groups of 8) -> natural order."""
+    inv = [ILV.index(e) for e in range(8)]
+    s = t.shape
+    return t.reshape(*s[:-1], s[-1] // 8, 8)[..., inv].reshape(s)
 
 
 def lut_up(p, x16, tokidx, tiles_t, ntiles, mid, npairs):

@@ -264,7 +264,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const moe_config& g = c->cfg;
   if (!L.has_q4cp) return MOE_E_UNSUPPORTED;
   if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
-  if (g.mid % 128 || g.d % 256 || g.d % 64 || g.mid % 64) return MOE_E_UNSUPPORTED;
+  if (g.d % 128 || g.mid % 128) return MOE_E_UNSUPPORTED;
   moe_lutw gu, dn, sgu{}, sdn{};
   moe_lut_q4cp_view(L.gate_up.data, L.gate_up.rows, L.gate_up.cols, L.gate_up.scale_stride, 2 * g.mid, g.mid, &gu);
   moe_lut_q4cp_view(L.down.data, L.down.rows, L.down.cols, L.down.scale_stride, g.d, 0, &dn);
@@ -280,8 +280,9 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   int rc;
   c->ev_n = 0;
   prof_mark(c, 0, st);
-  if ((rc = moe_router_logits_seq(&L.router, L.router_bias, x, P, c->logits, st))) return rc;
-  if (L.has_shared && (rc = moe_router_logits_seq(&L.sh_sg, nullptr, x, P, c->sh_logit, st))) return rc;
+  if ((rc = moe_router_logits_seq(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
+                                  c->sh_logit, st)))
+    return rc;
   if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
   prof_mark(c, MOE_PROF_ROUTER, st);
   if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
@@ -290,7 +291,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const int sh_first = L.has_shared ? P * g.topk : -1;
   if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, sh_first, c->tokidx, st)))
     return rc;
-  if ((rc = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, st))) return rc;
+  if ((rc = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, 1, st))) return rc;
   prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
   if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,

@@ -1,12 +1,15 @@
 // Prefill: grouped expert GEMM on q4cp weights with CDNA4 MFMA (v_mfma_f32_32x32x16_f16).
 //
-// One block = one tile of up to 128 (token, expert) pairs of ONE expert x one block of weight
-// rows.  Activations (f16) are gathered through tokidx into LDS; raw 4-bit codes and fp16 scales
-// are staged in LDS as they lie in the blob and dequantised in registers straight into the MFMA
-// B-operand layout: one 32-bit code word = 8 consecutive K of one weight row = one lane's operand.
-// The unpack yields the K order [0,4,1,5,2,6,3,7] inside each group of 8, so the activation tile
-// is written to LDS in that same order (a dot product does not care, as long as both sides agree).
-// gate/up: both row sets are accumulated by the same wave, SwiGLU runs on the accumulators.
+// One block (4 waves) = one tile of up to 128 (token, expert) pairs of ONE expert x 512 weight rows
+// (gate/up: 256 gate + the matching 256 up rows, SwiGLU on the accumulators).  Each wave owns
+// 128 pairs x 128 weight rows, so one activation fragment read from LDS feeds four MFMAs: LDS
+// bandwidth, not the matrix pipe, is what a narrower wave tile runs out of first.
+// Activations (f16), raw 4-bit codes and fp16 scales go global -> LDS directly (no registers),
+// double-buffered, one barrier per 64-wide K stage.  Codes are dequantised in registers straight
+// into the MFMA B-operand layout: one 32-bit code word = 8 consecutive K of one weight row = one
+// lane's operand.  The unpack yields the K order [0,4,1,5,2,6,3,7] inside each group of 8, so
+// f16 activations are kept in that same "interleaved" order (a dot product does not care as long
+// as both sides agree): moe_f32_to_f16(layout 1) and the gate/up epilogue write it.
 // (reference: src/gpu/parts/27_kernels_moe_lut.inc:75-83,110-640,660-821; weights are
 //  w = f16(cb[n] * scale), F32 accumulation over the whole K, as in :16)
 #include "common.h"
@@ -18,10 +21,14 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+constexpr int NT = 256;        // 4 waves, each 128 pairs x 128 weight rows
 constexpr int BM = 128;        // pairs per tile (4 MFMA row fragments)
 constexpr int BK = 64;         // K per stage
-constexpr int A_LD = BK + 8;   // f16 elements per LDS activation row (144 B: conflict-free b128 reads)
-constexpr int WROWS = 256;     // weight rows per block (up: 128 gate + 128 up)
+constexpr int WROWS = 512;     // weight rows per block (up: 256 gate + 256 up)
+constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chunk c of row m at slot c ^ (m & 7)
+constexpr int W_BYTES = WROWS * 32;       // 16 KB  [row][32 B]
+constexpr int S_BYTES = WROWS * 16;       //  8 KB  [row][8 scales], refreshed every 4 stages
+constexpr int SMEM_BYTES = 2 * (A_BYTES + W_BYTES + S_BYTES) + 64 + BM * 4;
 
 struct LutDev {
   const uint8_t *w, *w_up, *sc, *sc_up;
@@ -67,17 +74,193 @@ __device__ __forceinline__ half8 deq8_table(uint32_t w, float s, const float* cb
   return r.v;
 }
 
+// position of element e (0..7) inside its interleaved group of 8
+__device__ __forceinline__ int ilv_pos(int e) { return ((e & 3) << 1) | (e >> 2); }
+
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+// 64 lanes x 16 B: global (per-lane address) -> LDS (wave-uniform base, lane l lands at base + 16 l)
+__device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, LDS_PTR(lds_base), 16, 0, 0);
+}
+
+// MF = live 32-row fragments of the tile (1, 2 or 4); AFFINE = codebook a*n+b.
+template <bool UP, bool F16OUT, int MF, bool AFFINE>
+__device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
+                                          const __half* __restrict__ x, void* __restrict__ out, int M,
+                                          int K, float cb_a, float cb_b) {
+  uint8_t* const A0 = smem;
+  uint8_t* const W0 = smem + 2 * A_BYTES;
+  uint8_t* const S0 = W0 + 2 * W_BYTES;
+  const float* cbs = (const float*)(S0 + 2 * S_BYTES);
+  const int* rowidx = (const int*)(cbs + 16);
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int n = lane & 31, h = lane >> 5;
+
+  // LDS row -> global weight row (rows past the matrix are clamped: loaded, never stored)
+  auto wrow_ptrs = [&](int lr, const uint8_t*& cw, const uint8_t*& sw) {
+    size_t grow;
+    const uint8_t *cb0, *sb0;
+    if (UP) {
+      const bool up = lr >= 256;
+      int r = nb * 256 + (lr & 255);
+      r = r < M ? r : M - 1;
+      cb0 = up ? L.w_up : L.w;
+      sb0 = up ? L.sc_up : L.sc;
+      grow = (size_t)e * L.e_rows + (up ? L.up_off : 0) + r;
+    } else {
+      int r = nb * 512 + lr;
+      r = r < M ? r : M - 1;
+      cb0 = L.w;
+      sb0 = L.sc;
+      grow = (size_t)e * L.e_rows + r;
+    }
+    cw = cb0 + grow * (size_t)(K / 2);
+    sw = sb0 + grow * (size_t)L.sstride;
+  };
+
+  // per-lane global sources of the direct-to-LDS loads (wave-load j of a buffer = LDS bytes [1024 j, +1024))
+  // activations: rows 8j..8j+7, lane -> (row 8j + lane/8, slot lane%8 holding chunk slot ^ (row & 7))
+  constexpr int A_LOADS = MF;  // per wave: MF*32 rows / 8 rows per load / 4 waves
+  const __half* a_src[A_LOADS];
+#pragma unroll
+  for (int i = 0; i < A_LOADS; i++) {
+    const int m = 8 * (A_LOADS * wv + i) + (lane >> 3);
+    a_src[i] = x + (size_t)rowidx[m] * K + (((lane & 7) ^ (m & 7)) << 3);
+  }
+  // codes: rows 32j..32j+31, lane -> (row 32j + lane/2, half lane%2); scales: rows 64j.., lane -> row
+  const uint8_t *w_src[4], *s_src[2];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint8_t* sw;
+    wrow_ptrs(32 * (4 * wv + i) + (lane >> 1), w_src[i], sw);
+    w_src[i] += (lane & 1) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const uint8_t* cw;
+    wrow_ptrs(64 * (2 * wv + i) + lane, cw, s_src[i]);
+  }
+  const int nstage = K / BK, ngroups = K / 32;
+  auto issue = [&](int s) {
+    const int b = s & 1;
+#pragma unroll
+    for (int i = 0; i < A_LOADS; i++) g2l16(a_src[i] + (size_t)s * BK, A0 + b * A_BYTES + (A_LOADS * wv + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 4; i++) g2l16(w_src[i] + (size_t)s * 32, W0 + b * W_BYTES + (4 * wv + i) * 1024);
+    if ((s & 3) == 0) {
+      // 8 scales (16 B) per row for stages s..s+3; at the end of K the window is pulled back inside the row
+      int g0 = 2 * s;
+      g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
+      const int sb = (s >> 2) & 1;
+#pragma unroll
+      for (int i = 0; i < 2; i++) g2l16(s_src[i] + (size_t)g0 * 2, S0 + sb * S_BYTES + (2 * wv + i) * 1024);
+    }
+  };
+
+  floatx16 acc[MF][4];
+#pragma unroll
+  for (int mf = 0; mf < MF; mf++)
+#pragma unroll
+    for (int nf = 0; nf < 4; nf++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[mf][nf][i] = 0.f;
+
+  // LDS rows of this wave's four weight fragments (up: 2 gate + the 2 matching up fragments)
+  int wrow[4];
+#pragma unroll
+  for (int nf = 0; nf < 4; nf++) wrow[nf] = UP ? (nf >> 1) * 256 + 64 * wv + 32 * (nf & 1) + n : 128 * wv + 32 * nf + n;
+
+  issue(0);
+  for (int s = 0; s < nstage; s++) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of stage s have landed
+    __syncthreads();                     // ... and everybody else's; stage s-1 is no longer read
+#ifndef EXP_NO_GLOAD
+    if (s + 1 < nstage) issue(s + 1);
+#endif
+    const uint8_t* Ab = A0 + (s & 1) * A_BYTES;
+    const uint8_t* Wb = W0 + (s & 1) * W_BYTES;
+    const uint8_t* Sb = S0 + ((s >> 2) & 1) * S_BYTES;
+    int g0 = 2 * (s & ~3);
+    g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
+    const int sidx = 2 * s + h - g0;  // this lane's scale inside the staged 8
+    uint4 cw[4];
+    _Float16 sc[4];
+#pragma unroll
+    for (int nf = 0; nf < 4; nf++) {
+      cw[nf] = *(const uint4*)(Wb + wrow[nf] * 32 + h * 16);
+      sc[nf] = *(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
+    }
+    half2v as2[4], bs2[4];
+    float scf[4];
+#pragma unroll
+    for (int nf = 0; nf < 4; nf++) {
+      scf[nf] = (float)sc[nf];
+      const _Float16 as = (_Float16)(cb_a * scf[nf]), bs = (_Float16)(cb_b * scf[nf]);
+      as2[nf] = half2v{as, as};
+      bs2[nf] = half2v{bs, bs};
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      half8 a[MF], b[4];
+#pragma unroll
+      for (int mf = 0; mf < MF; mf++) {
+        const int m = 32 * mf + n;
+        a[mf] = *(const half8*)(Ab + m * 128 + (((4 * h + q) ^ (m & 7)) << 4));
+      }
+#pragma unroll
+      for (int nf = 0; nf < 4; nf++) {
+        const uint32_t w = q == 0 ? cw[nf].x : q == 1 ? cw[nf].y : q == 2 ? cw[nf].z : cw[nf].w;
+        b[nf] = AFFINE ? deq8_affine(w, as2[nf], bs2[nf]) : deq8_table(w, scf[nf], cbs);
+      }
+#pragma unroll
+      for (int mf = 0; mf < MF; mf++)
+#pragma unroll
+        for (int nf = 0; nf < 4; nf++)
+          acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+    }
+  }
+
+  // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair)
+#pragma unroll
+  for (int mf = 0; mf < MF; mf++) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int m = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (m >= tile.count) continue;
+      const size_t row = (size_t)(tile.first + m);
+      if (UP) {
+#pragma unroll
+        for (int f = 0; f < 2; f++) {
+          const int col = nb * 256 + 64 * wv + 32 * f + n;
+          if (col < M) {
+            const float g = acc[mf][f][r], u = acc[mf][2 + f][r];
+            const float hv = g / (1.f + __expf(-g)) * u;
+            // hid feeds the down GEMM: interleaved order inside each group of 8 columns
+            ((__half*)out)[row * M + (col & ~7) + ilv_pos(col & 7)] = __float2half(hv);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int nf = 0; nf < 4; nf++) {
+          const int col = nb * 512 + 128 * wv + 32 * nf + n;
+          if (col < M) {
+            if (F16OUT) ((__half*)out)[row * M + col] = __float2half(acc[mf][nf][r]);
+            else ((float*)out)[row * M + col] = acc[mf][nf][r];
+          }
+        }
+      }
+    }
+  }
+}
+
 template <bool UP, bool F16OUT>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(NT, 1)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n) {
-  __shared__ __attribute__((aligned(16))) _Float16 As[BM * A_LD];
-  __shared__ __attribute__((aligned(16))) uint8_t Ws[WROWS * 32];
-  __shared__ __attribute__((aligned(4))) _Float16 Ss[WROWS * 2];
-  __shared__ float cbs[16];
-  __shared__ int rowidx[BM];
-
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  float* cbs = (float*)(smem + 2 * (A_BYTES + W_BYTES + S_BYTES));
+  int* rowidx = (int*)(cbs + 16);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
   const int nt = *ntiles;
@@ -90,7 +273,7 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const bool shared = tile.expert >= n_experts;
   const LutDev& L = shared ? Sh : R;
   const int e = shared ? 0 : tile.expert;
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
 
   // codebook: affine (a*n+b) or table
   const float c0 = L.cb[0], c1 = L.cb[1];
@@ -108,139 +291,16 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
     rowidx[tid] = tokidx ? tokidx[tile.first + m] : tile.first + m;
   }
   __syncthreads();
-
-  // per-thread global sources
-  const int a_c = tid & 7;  // 16-byte chunk of the 128-byte stage row
-  const __half* a_src[4];
-#pragma unroll
-  for (int i = 0; i < 4; i++) a_src[i] = x + (size_t)rowidx[(tid >> 3) + 32 * i] * K + a_c * 8;
-  const uint8_t* w_src[2];
-  const int w_half = tid & 1;
-#pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int lr = (tid >> 1) + 128 * i;
-    size_t grow;
-    const uint8_t* base;
-    if (UP) {
-      base = i == 0 ? L.w : L.w_up;
-      grow = (size_t)e * L.e_rows + (i == 0 ? 0 : L.up_off) + (size_t)nb * 128 + (lr & 127);
-    } else {
-      base = L.w;
-      grow = (size_t)e * L.e_rows + (size_t)nb * 256 + lr;
-    }
-    w_src[i] = base + grow * (size_t)(K / 2) + w_half * 16;
-  }
-  const uint8_t* s_src;
-  {
-    const int lr = tid;
-    size_t grow;
-    const uint8_t* base;
-    if (UP) {
-      base = lr < 128 ? L.sc : L.sc_up;
-      grow = (size_t)e * L.e_rows + (lr < 128 ? 0 : L.up_off) + (size_t)nb * 128 + (lr & 127);
-    } else {
-      base = L.sc;
-      grow = (size_t)e * L.e_rows + (size_t)nb * 256 + lr;
-    }
-    s_src = base + grow * (size_t)L.sstride;
-  }
-
-  floatx16 acc[4][2];
-#pragma unroll
-  for (int mf = 0; mf < 4; mf++)
-#pragma unroll
-    for (int nf = 0; nf < 2; nf++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) acc[mf][nf][i] = 0.f;
-
-  const int nfrag_m = (tile.count + 31) >> 5;  // live 32-row fragments of this tile
-  const int n = lane & 31, h = lane >> 5;
-  // LDS rows of this wave's two weight fragments
-  const int wrow0 = UP ? 32 * wv + n : 64 * wv + n;
-  const int wrow1 = UP ? 128 + 32 * wv + n : 64 * wv + 32 + n;
-
-  uint4 ra[4], rw[2];
-  uint32_t rs;
-  auto gload = [&](int s) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) ra[i] = *(const uint4*)(a_src[i] + (size_t)s * BK);
-#pragma unroll
-    for (int i = 0; i < 2; i++) rw[i] = *(const uint4*)(w_src[i] + (size_t)s * 32);
-    rs = *(const uint32_t*)(s_src + (size_t)s * 4);
-  };
-  const int nstage = K / BK;
-  gload(0);
-  for (int s = 0; s < nstage; s++) {
-    // registers -> LDS (activations re-ordered inside each group of 8: [0,4,1,5,2,6,3,7])
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      uint4 p;
-      p.x = (ra[i].x & 0xffffu) | (ra[i].z << 16);
-      p.y = (ra[i].x >> 16) | (ra[i].z & 0xffff0000u);
-      p.z = (ra[i].y & 0xffffu) | (ra[i].w << 16);
-      p.w = (ra[i].y >> 16) | (ra[i].w & 0xffff0000u);
-      *(uint4*)(As + ((tid >> 3) + 32 * i) * A_LD + a_c * 8) = p;
-    }
-#pragma unroll
-    for (int i = 0; i < 2; i++) *(uint4*)(Ws + ((tid >> 1) + 128 * i) * 32 + w_half * 16) = rw[i];
-    *(uint32_t*)(Ss + tid * 2) = rs;
-    __syncthreads();
-    if (s + 1 < nstage) gload(s + 1);
-
-    // dequantise this wave's 2 x (32 rows x 64 K): lane (n, h) owns K [32h, 32h+32) of row n
-    half8 bfrag[2][4];
-#pragma unroll
-    for (int nf = 0; nf < 2; nf++) {
-      const int wr = nf == 0 ? wrow0 : wrow1;
-      const uint4 cw = *(const uint4*)(Ws + wr * 32 + h * 16);
-      const float sc = (float)Ss[wr * 2 + h];
-      const uint32_t cwv[4] = {cw.x, cw.y, cw.z, cw.w};
-      if (affine) {
-        const _Float16 as = (_Float16)(cb_a * sc), bs = (_Float16)(cb_b * sc);
-        const half2v as2 = {as, as}, bs2 = {bs, bs};
-#pragma unroll
-        for (int q = 0; q < 4; q++) bfrag[nf][q] = deq8_affine(cwv[q], as2, bs2);
-      } else {
-#pragma unroll
-        for (int q = 0; q < 4; q++) bfrag[nf][q] = deq8_table(cwv[q], sc, cbs);
-      }
-    }
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-#pragma unroll
-      for (int mf = 0; mf < 4; mf++) {
-        if (mf < nfrag_m) {
-          const half8 a = *(const half8*)(As + (32 * mf + n) * A_LD + 32 * h + 8 * q);
-          acc[mf][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bfrag[0][q], acc[mf][0], 0, 0, 0);
-          acc[mf][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bfrag[1][q], acc[mf][1], 0, 0, 0);
-        }
-      }
-    }
-    __syncthreads();
-  }
-
-  // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair)
-#pragma unroll
-  for (int mf = 0; mf < 4; mf++) {
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int m = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (m >= tile.count) continue;
-      const size_t row = (size_t)(tile.first + m);
-      if (UP) {
-        const float g = acc[mf][0][r], u = acc[mf][1][r];
-        const float hv = g / (1.f + __expf(-g)) * u;
-        ((__half*)out)[row * M + nb * 128 + 32 * wv + n] = __float2half(hv);
-      } else {
-#pragma unroll
-        for (int nf = 0; nf < 2; nf++) {
-          const size_t col = (size_t)nb * 256 + 64 * wv + 32 * nf + n;
-          if (F16OUT) ((__half*)out)[row * M + col] = __float2half(acc[mf][nf][r]);
-          else ((float*)out)[row * M + col] = acc[mf][nf][r];
-        }
-      }
-    }
-  }
+  const int mfn = (tile.count + 31) >> 5;
+#define GEMM_GO(MF)                                                                                     \
+  do {                                                                                                  \
+    if (affine) gemm_tile<UP, F16OUT, MF, true>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b);        \
+    else gemm_tile<UP, F16OUT, MF, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b);             \
+  } while (0)
+  if (mfn <= 1) GEMM_GO(1);
+  else if (mfn == 2) GEMM_GO(2);
+  else GEMM_GO(4);
+#undef GEMM_GO
 }
 
 LutDev to_dev(const moe_lutw* p) {
@@ -255,7 +315,7 @@ LutDev to_dev(const moe_lutw* p) {
 bool lut_ok(const moe_lutw* p, bool pair, int k) {
   if (!p || !p->w || !p->sc || !p->cb) return false;
   if (pair && (!p->w_up || !p->sc_up)) return false;
-  if (k < 64 || k % 64) return false;
+  if (k < 256 || k % 128) return false;
   if (!moe_aligned(p->w, 16) || !moe_aligned(p->sc, 4) || p->sstride % 4 || p->sstride < k / 32 * 2) return false;
   if (pair && (!moe_aligned(p->w_up, 16) || !moe_aligned(p->sc_up, 4))) return false;
   return true;
@@ -269,19 +329,26 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          int max_tiles, void* out, int m, int k, bool f16out, hipStream_t st) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
   if (!lut_ok(routed, up, k) || (sh && !lut_ok(sh, up, k))) return MOE_E_UNSUPPORTED;
-  if (up ? (m % 128 != 0) : (m % 256 != 0)) return MOE_E_UNSUPPORTED;
+  if (m < 32 || m % 32) return MOE_E_UNSUPPORTED;
   if (!moe_aligned(x, 16) || !moe_aligned(out, 4)) return MOE_E_INVALID;
   if (max_tiles == 0) return MOE_OK;
-  const int nblk_n = up ? m / 128 : m / 256;
+  const int nblk_n = up ? (m + 255) / 256 : (m + 511) / 512;
+  static bool attr_done = false;
+  if (!attr_done) {
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
+    attr_done = true;
+  }
   const int per_xcd = (max_tiles + 7) / 8;
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
   LutDev R = to_dev(routed), S = to_dev(sh ? sh : routed);
   if (up)
-    k_moe_gemm_q4cp<true, true><<<grid, 256, 0, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
+    k_moe_gemm_q4cp<true, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
   else if (f16out)
-    k_moe_gemm_q4cp<false, true><<<grid, 256, 0, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
+    k_moe_gemm_q4cp<false, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
   else
-    k_moe_gemm_q4cp<false, false><<<grid, 256, 0, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
+    k_moe_gemm_q4cp<false, false><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -24,5 +24,5 @@ int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
                       const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
                       hipStream_t st);
-int moe_router_logits_seq(const moe_wview* W, const float* bias, const float* x, int P, float* logits,
-                          hipStream_t st);
+int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
+                          float* logits, float* out_x, hipStream_t st);

@@ -7,30 +7,56 @@
 
 namespace {
 
-__global__ void __launch_bounds__(256) k_f32_to_f16_v4(const float4* __restrict__ x, uint2* __restrict__ y,
-                                                       uint64_t n4) {
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4;
+// 8 floats -> 8 f16 (RNE).  ILV: the order the grouped GEMM keeps its activations in,
+// [e0,e4,e1,e5,e2,e6,e3,e7] inside every group of 8.
+template <bool ILV>
+__global__ void __launch_bounds__(256) k_f32_to_f16_v8(const float4* __restrict__ x, uint4* __restrict__ y,
+                                                       uint64_t n8) {
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
        i += (uint64_t)gridDim.x * blockDim.x) {
-    const float4 v = x[i];
-    const __half2 a = __floats2half2_rn(v.x, v.y), b = __floats2half2_rn(v.z, v.w);
-    uint2 o;
-    o.x = *(const uint32_t*)&a;
-    o.y = *(const uint32_t*)&b;
+    const float4 u = x[2 * i], v = x[2 * i + 1];
+    __half2 a, b, c, d;
+    if (ILV) {
+      a = __floats2half2_rn(u.x, v.x); b = __floats2half2_rn(u.y, v.y);
+      c = __floats2half2_rn(u.z, v.z); d = __floats2half2_rn(u.w, v.w);
+    } else {
+      a = __floats2half2_rn(u.x, u.y); b = __floats2half2_rn(u.z, u.w);
+      c = __floats2half2_rn(v.x, v.y); d = __floats2half2_rn(v.z, v.w);
+    }
+    uint4 o;
+    o.x = *(const uint32_t*)&a; o.y = *(const uint32_t*)&b; o.z = *(const uint32_t*)&c; o.w = *(const uint32_t*)&d;
     y[i] = o;
   }
 }
 
-template <class PT>
-__device__ __forceinline__ float ldp(const PT* p, size_t i);
-template <>
-__device__ __forceinline__ float ldp<float>(const float* p, size_t i) { return p[i]; }
-template <>
-__device__ __forceinline__ float ldp<__half>(const __half* p, size_t i) { return __half2float(p[i]); }
-
 // out[t][c] = sum_{s<K} pw[pid_s] * pairs[pid_s][c]  (pid_s = pairids[t*K+s], ascending expert id)
 //            + sigmoid(sg[t]) * ey[t][c]             (ey f32, or row `sh_first + t` of pairs)
+// One thread per 8 consecutive columns (16-byte loads of f16 pairs); grid (ceil(D/8/256), P).
+template <class PT>
+struct Ld8;
+template <>
+struct Ld8<__half> {
+  static __device__ __forceinline__ void ld(const __half* p, float* v) {
+    const uint4 u = *(const uint4*)p;
+    const __half2* h = (const __half2*)&u;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const float2 f = __half22float2(h[i]);
+      v[2 * i] = f.x;
+      v[2 * i + 1] = f.y;
+    }
+  }
+};
+template <>
+struct Ld8<float> {
+  static __device__ __forceinline__ void ld(const float* p, float* v) {
+    const float4 a = ((const float4*)p)[0], b = ((const float4*)p)[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+};
+
 template <class PT, int KMAX>
-__global__ void __launch_bounds__(256) k_reduce_pw_sg(const PT* __restrict__ pairs,
+__global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pairs,
                                                       const int* __restrict__ pairids,
                                                       const float* __restrict__ pw,
                                                       const float* __restrict__ ey,
@@ -45,18 +71,29 @@ __global__ void __launch_bounds__(256) k_reduce_pw_sg(const PT* __restrict__ pai
     w[threadIdx.x] = pw[id];
   }
   __syncthreads();
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (c >= D) return;
-  float sum = 0.f;
+  float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < KMAX; s++)
-    if (s < K) sum += w[s] * ldp<PT>(pairs, (size_t)ids[s] * D + c);
+    if (s < K) {
+      float v[8];
+      Ld8<PT>::ld(pairs + (size_t)ids[s] * D + c, v);
+      const float ww = w[s];
+#pragma unroll
+      for (int i = 0; i < 8; i++) sum[i] += ww * v[i];
+    }
   if (sg) {
     const float g = sigmoid_f(sg[t]);
-    const float e = ey ? ey[(size_t)t * D + c] : ldp<PT>(pairs, (size_t)(sh_first + t) * D + c);
-    sum += g * e;
+    float v[8];
+    if (ey) Ld8<float>::ld(ey + (size_t)t * D + c, v);
+    else Ld8<PT>::ld(pairs + (size_t)(sh_first + t) * D + c, v);
+#pragma unroll
+    for (int i = 0; i < 8; i++) sum[i] += g * v[i];
   }
-  out[(size_t)t * D + c] = sum;
+  float4* o = (float4*)(out + (size_t)t * D + c);
+  o[0] = make_float4(sum[0], sum[1], sum[2], sum[3]);
+  o[1] = make_float4(sum[4], sum[5], sum[6], sum[7]);
 }
 
 // Tiles of the routed experts (expert order, <= cap pairs each) followed by the shared expert's
@@ -118,24 +155,26 @@ int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, con
                       hipStream_t st) {
   if (!pairs || !pairids || !pw || !out) return MOE_E_INVALID;
   if (P < 0 || D < 1 || K < 1) return MOE_E_INVALID;
-  if (K > 16) return MOE_E_UNSUPPORTED;
+  if (K > 16 || D % 8) return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(pairs, 16) || !moe_aligned(out, 16) || (ey && !moe_aligned(ey, 16))) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
-  dim3 grid((D + 255) / 256, P);
+  dim3 grid((D / 8 + 127) / 128, P);
   if (pairs_f16)
-    k_reduce_pw_sg<__half, 16><<<grid, 256, 0, st>>>((const __half*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K);
+    k_reduce_pw_sg<__half, 16><<<grid, 128, 0, st>>>((const __half*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K);
   else
-    k_reduce_pw_sg<float, 16><<<grid, 256, 0, st>>>((const float*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K);
+    k_reduce_pw_sg<float, 16><<<grid, 128, 0, st>>>((const float*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
 
-MOE_API int moe_f32_to_f16(const float* x, void* x16, uint64_t n, moe_stream_t st) {
+MOE_API int moe_f32_to_f16(const float* x, void* x16, uint64_t n, int layout, moe_stream_t st) {
   if (!x || !x16) return n ? MOE_E_INVALID : MOE_OK;
-  if (n % 4 || !moe_aligned(x, 16) || !moe_aligned(x16, 8)) return MOE_E_INVALID;
+  if (n % 8 || !moe_aligned(x, 16) || !moe_aligned(x16, 16) || (layout != 0 && layout != 1)) return MOE_E_INVALID;
   if (n == 0) return MOE_OK;
-  const uint64_t n4 = n / 4;
-  const unsigned grid = (unsigned)((n4 + 255) / 256 > 1048576 ? 1048576 : (n4 + 255) / 256);
-  k_f32_to_f16_v4<<<grid, 256, 0, moe_s(st)>>>((const float4*)x, (uint2*)x16, n4);
+  const uint64_t n8 = n / 8;
+  const unsigned grid = (unsigned)((n8 + 255) / 256 > 1048576 ? 1048576 : (n8 + 255) / 256);
+  if (layout) k_f32_to_f16_v8<true><<<grid, 256, 0, moe_s(st)>>>((const float4*)x, (uint4*)x16, n8);
+  else k_f32_to_f16_v8<false><<<grid, 256, 0, moe_s(st)>>>((const float4*)x, (uint4*)x16, n8);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -11,58 +11,93 @@ __device__ __forceinline__ float load_w(const void* W, uint64_t i) {
 }
 
 // ---- sequential order: bit-identical to `acc += (double)w*x` for c = 0..d-1 ----
-// Block = 64 tokens x 64 experts, thread = 4 x 4 independent fp64 chains.  The f32*f32 product
-// is exact in fp64, so fma(w, x, acc) equals the reference's multiply-then-add.
-constexpr int RL_T = 64, RL_E = 64, RL_K = 32;
+// Block = 128 tokens x 64 weight rows, thread = 8 x 4 independent fp64 chains; operands are
+// widened to fp64 once, when they are staged in LDS.  The f32*f32 product is exact in fp64, so
+// fma(w, x, acc) equals the reference's multiply-then-add.  Row E (if Wx is given) is the
+// shared-expert gate vector: its logit goes to out_x[t].
+constexpr int RL_T = 128, RL_E = 64, RL_K = 32;
 template <bool BF16>
 __global__ void __launch_bounds__(256) k_router_logits_seq(const void* __restrict__ W,
                                                            const float* __restrict__ bias,
+                                                           const void* __restrict__ Wx, bool wx_bf16,
                                                            const float* __restrict__ x, int P, int E,
-                                                           int d, float* __restrict__ logits) {
-  __shared__ float Xs[RL_K][RL_T + 1];
-  __shared__ float Ws[RL_K][RL_E + 1];
+                                                           int d, float* __restrict__ logits,
+                                                           float* __restrict__ out_x) {
+  __shared__ __attribute__((aligned(16))) double Xs[RL_K][RL_T + 2];
+  __shared__ __attribute__((aligned(16))) double Ws[RL_K][RL_E + 2];
   const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
   const int e0 = blockIdx.x * RL_E, t0 = blockIdx.y * RL_T;
-  double acc[4][4];
+  const int Etot = E + (Wx ? 1 : 0);
+  double acc[8][4];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int j = 0; j < 8; j++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) acc[i][j] = 0.0;
+    for (int i = 0; i < 4; i++) acc[j][i] = 0.0;
+  const bool vec = (d % 4 == 0);
   for (int c0 = 0; c0 < d; c0 += RL_K) {
-    // stage 64 rows x 32 columns of each operand (zero outside the matrix)
+    // stage 128 x 32 activations and 64 x 32 weights (zero outside the matrices)
 #pragma unroll
-    for (int it = 0; it < (RL_T * RL_K) / 256; it++) {
-      const int i = tid + it * 256, r = i / RL_K, c = i % RL_K;
-      const int t = t0 + r, e = e0 + r, cc = c0 + c;
-      Xs[c][r] = (t < P && cc < d) ? x[(size_t)t * d + cc] : 0.f;
-      Ws[c][r] = (e < E && cc < d) ? load_w<BF16>(W, (uint64_t)e * d + cc) : 0.f;
+    for (int it = 0; it < (RL_T * RL_K / 4) / 256; it++) {
+      const int i = tid + it * 256, r = i >> 3, c = (i & 7) * 4;
+      const int t = t0 + r, cc = c0 + c;
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      if (t < P) {
+        if (vec && cc + 3 < d) {
+          const float4 f = *(const float4*)(x + (size_t)t * d + cc);
+          v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+        } else {
+          for (int q = 0; q < 4; q++) if (cc + q < d) v[q] = x[(size_t)t * d + cc + q];
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++) Xs[c + q][r] = (double)v[q];
+    }
+#pragma unroll
+    for (int it = 0; it < (RL_E * RL_K / 4) / 256; it++) {
+      const int i = tid + it * 256, r = i >> 3, c = (i & 7) * 4;
+      const int e = e0 + r, cc = c0 + c;
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      if (e < Etot) {
+        const bool ex = e == E;
+        const void* src = ex ? Wx : W;
+        const uint64_t base = ex ? 0 : (uint64_t)e * d;
+        const bool bf = ex ? wx_bf16 : BF16;
+        for (int q = 0; q < 4; q++)
+          if (cc + q < d) v[q] = bf ? bf16_bits_to_f32(((const uint16_t*)src)[base + cc + q]) : ((const float*)src)[base + cc + q];
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++) Ws[c + q][r] = (double)v[q];
     }
     __syncthreads();
-#pragma unroll 8
+#pragma unroll 4
     for (int c = 0; c < RL_K; c++) {
-      double wv[4], xv[4];
+      double wv[4], xv[8];
 #pragma unroll
-      for (int i = 0; i < 4; i++) wv[i] = (double)Ws[c][tx + 16 * i];
+      for (int i = 0; i < 4; i++) wv[i] = Ws[c][4 * tx + i];
 #pragma unroll
-      for (int j = 0; j < 4; j++) xv[j] = (double)Xs[c][ty + 16 * j];
+      for (int j = 0; j < 8; j++) xv[j] = Xs[c][8 * ty + j];
 #pragma unroll
-      for (int i = 0; i < 4; i++)
+      for (int j = 0; j < 8; j++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = fma(wv[i], xv[j], acc[i][j]);
+        for (int i = 0; i < 4; i++) acc[j][i] = fma(wv[i], xv[j], acc[j][i]);
     }
     __syncthreads();
   }
 #pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const int t = t0 + ty + 16 * j;
+  for (int j = 0; j < 8; j++) {
+    const int t = t0 + 8 * ty + j;
     if (t >= P) continue;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      const int e = e0 + tx + 16 * i;
-      if (e >= E) continue;
-      float v = (float)acc[i][j];
-      if (bias) v += bias[e];
-      logits[(size_t)t * E + e] = v;
+      const int e = e0 + 4 * tx + i;
+      if (e >= Etot) continue;
+      float v = (float)acc[j][i];
+      if (e == E) {
+        out_x[t] = v;
+      } else {
+        if (bias) v += bias[e];
+        logits[(size_t)t * E + e] = v;
+      }
     }
   }
 }
@@ -229,20 +264,22 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
     else k_router_logits_par<false, 4><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
   } else {
     dim3 g((E + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
-    if (bf) k_router_logits_seq<true><<<g, 256, 0, moe_s(st)>>>(W->data, bias, x, P, E, d, logits);
-    else k_router_logits_seq<false><<<g, 256, 0, moe_s(st)>>>(W->data, bias, x, P, E, d, logits);
+    if (bf) k_router_logits_seq<true><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
+    else k_router_logits_seq<false><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
   }
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
 
 // Internal: sequential-order logits for any P (also used for the one-row shared-expert gate).
-int moe_router_logits_seq(const moe_wview* W, const float* bias, const float* x, int P, float* logits,
-                          hipStream_t st) {
+int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
+                          float* logits, float* out_x, hipStream_t st) {
   const int E = (int)W->rows, d = (int)W->cols;
-  dim3 g((E + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
-  if (W->dtype == MOE_DT_BF16) k_router_logits_seq<true><<<g, 256, 0, st>>>(W->data, bias, x, P, E, d, logits);
-  else k_router_logits_seq<false><<<g, 256, 0, st>>>(W->data, bias, x, P, E, d, logits);
+  const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
+  const void* wx = Wx ? Wx->data : nullptr;
+  dim3 g((E + (Wx ? 1 : 0) + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
+  if (W->dtype == MOE_DT_BF16) k_router_logits_seq<true><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x);
+  else k_router_logits_seq<false><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

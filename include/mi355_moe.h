@@ -130,15 +130,19 @@ enum { MOE_LUT_Q4CP = 100 }; /* moelut::kQ4CP (27_kernels_moe_lut.inc:33) */
 /* lut_q4cp_view (27_kernels_moe_lut.inc:811) */
 int moe_lut_q4cp_view(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t scale_stride,
                       int e_rows, int up_off, moe_lutw* out);
-/* k_f32_to_f16_v4 (26_kernels_moe_gguf.inc:389): round-to-nearest-even, n % 4 == 0 */
-int moe_f32_to_f16(const float* x, void* x16, uint64_t n, moe_stream_t st);
+/* k_f32_to_f16_v4 (26_kernels_moe_gguf.inc:389): round-to-nearest-even, n % 8 == 0.
+ * layout 0 = natural order; layout 1 = the order the grouped GEMM reads its f16 activations in:
+ * inside every group of 8 consecutive elements, [e0,e4,e1,e5,e2,e6,e3,e7] (matches the order the
+ * 4-bit unpack produces, so no shuffle is needed on the weight side).  moe_lut_up expects x16 in
+ * layout 1 and writes hid16 in layout 1 for moe_lut_down. */
+int moe_f32_to_f16(const float* x, void* x16, uint64_t n, int layout, moe_stream_t st);
 /* moe_lut_up (27_kernels_moe_lut.inc:660): hid16[pair][m] = f16(silu(gate) * up) for every tile
- * (tiles hold <= 128 pairs); x16: f16 [P][k] gathered through tokidx; m % 128 == 0, k % 64 == 0. */
+ * (tiles hold <= 128 pairs); x16: f16 [P][k] (layout 1) gathered through tokidx; m % 32 == 0, k % 128 == 0, k >= 256. */
 int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* tokidx,
                const moe_tile* tiles, const int* ntiles, int max_tiles, void* hid16, int m, int k,
                moe_stream_t st);
 /* moe_lut_down (27_kernels_moe_lut.inc:765): pairs[pair][m] (unweighted; f32, or f16 if f16 != 0)
- * = W_e[m][k] . hid16[pair]; m % 256 == 0, k % 64 == 0. */
+ * = W_e[m][k] . hid16[pair] (hid16 in layout 1); m % 32 == 0, k % 128 == 0, k >= 256. */
 int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
                  const int* ntiles, int max_tiles, void* pairs, int m, int k, int f16,
                  moe_stream_t st);

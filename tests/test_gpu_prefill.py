@@ -32,7 +32,7 @@ def make_routing(rng, P, E, k, counts=None):
     return ids, ws
 
 
-@pytest.mark.parametrize("d,mid,E,k,P,cb", [(256, 128, 6, 2, 300, "zp8"), (3072, 768, 8, 4, 200, "zp8"),
+@pytest.mark.parametrize("d,mid,E,k,P,cb", [(256, 256, 6, 2, 300, "zp8"), (640, 384, 4, 2, 260, "zp8"), (3072, 768, 8, 4, 200, "zp8"),
                                             (512, 256, 5, 3, 150, "random")])
 def test_grouped_gemm_stages(capi, oracle, d, mid, E, k, P, cb):
     """up -> hid16, down -> pairs, reduce -> y, each against fp64 from the oracle's weights.
@@ -47,7 +47,8 @@ def test_grouped_gemm_stages(capi, oracle, d, mid, E, k, P, cb):
     ids, ws = make_routing(rng, P, E - 1, k)
     ids[:, :k] += 1  # expert 0 empty
     x16 = capi.f32_to_f16(gpu(x))
-    assert (x16.cpu().numpy() == x.astype(np.float16)).all()
+    assert (capi.from_layout1(x16).cpu().numpy() == x.astype(np.float16)).all()
+    assert (capi.f32_to_f16(gpu(x), layout=0).cpu().numpy() == x.astype(np.float16)).all()
     r = capi.Routing(P * k, E)
     tokidx, pw, eoff, pairids = r.run(gpu(ids), gpu(ws), k)
     tiles_t, ntiles = capi.tiles(eoff, 128, P * k)
@@ -57,7 +58,7 @@ def test_grouped_gemm_stages(capi, oracle, d, mid, E, k, P, cb):
     pairs = capi.lut_down(pdn, hid, tiles_t, ntiles, d, f16=False)
     pairs16 = capi.lut_down(pdn, hid, tiles_t, ntiles, d, f16=True)
     y = capi.reduce_pw_sg(pairs, pairids, pw, P, k)
-    hid, pairs, pairs16, y = hid.cpu().numpy(), pairs.cpu().numpy(), pairs16.cpu().numpy(), y.cpu().numpy()
+    hid, pairs, pairs16, y = capi.from_layout1(hid).cpu().numpy(), pairs.cpu().numpy(), pairs16.cpu().numpy(), y.cpu().numpy()
     assert not np.isnan(hid).any() and not np.isnan(pairs).any(), "every pair row must be written"
     tokidx, pw, eoff = tokidx.cpu().numpy(), pw.cpu().numpy(), eoff.cpu().numpy()
     GU = oracle.q4cp_rows(gu, E * 2 * mid, d, 0, E * 2 * mid).astype(np.float64)
