@@ -21,6 +21,12 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+#ifdef EXP_TIMING
+extern __device__ unsigned long long g_dbg[4096];
+#define TSTAMP(i) do { if (threadIdx.x == 0 && blockIdx.x == 800) g_dbg[(UPK ? 2000 : 0) + (i)] = __builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define TSTAMP(i) do {} while (0)
+#endif
 constexpr int NT = 256;        // 4 waves, each 128 pairs x 128 weight rows
 constexpr int BM = 128;        // pairs per tile (4 MFMA row fragments)
 constexpr int BK = 64;         // K per stage
@@ -28,7 +34,8 @@ constexpr int WROWS = 512;     // weight rows per block (up: 256 gate + 256 up)
 constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chunk c of row m at slot c ^ (m & 7)
 constexpr int W_BYTES = WROWS * 32;       // 16 KB  [row][32 B]
 constexpr int S_BYTES = WROWS * 16;       //  8 KB  [row][8 scales], refreshed every 4 stages
-constexpr int SMEM_BYTES = 2 * (A_BYTES + W_BYTES + S_BYTES) + 64 + BM * 4;
+constexpr int NBUF = 3;                   // activation / code buffers in flight (loads run two stages ahead)
+constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES + 64 + BM * 4;
 
 struct LutDev {
   const uint8_t *w, *w_up, *sc, *sc_up;
@@ -89,11 +96,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b) {
   uint8_t* const A0 = smem;
-  uint8_t* const W0 = smem + 2 * A_BYTES;
-  uint8_t* const S0 = W0 + 2 * W_BYTES;
+  uint8_t* const W0 = smem + NBUF * A_BYTES;
+  uint8_t* const S0 = W0 + NBUF * W_BYTES;
   const float* cbs = (const float*)(S0 + 2 * S_BYTES);
   const int* rowidx = (const int*)(cbs + 16);
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  constexpr bool UPK = UP;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, kept scalar
   const int n = lane & 31, h = lane >> 5;
 
   // LDS row -> global weight row (rows past the matrix are clamped: loaded, never stored)
@@ -141,20 +150,36 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     wrow_ptrs(64 * (2 * wv + i) + lane, cw, s_src[i]);
   }
   const int nstage = K / BK, ngroups = K / 32;
-  auto issue = [&](int s) {
-    const int b = s & 1;
-#pragma unroll
-    for (int i = 0; i < A_LOADS; i++) g2l16(a_src[i] + (size_t)s * BK, A0 + b * A_BYTES + (A_LOADS * wv + i) * 1024);
-#pragma unroll
-    for (int i = 0; i < 4; i++) g2l16(w_src[i] + (size_t)s * 32, W0 + b * W_BYTES + (4 * wv + i) * 1024);
-    if ((s & 3) == 0) {
+  constexpr int NLOADS = A_LOADS + 4;  // per stage (+2 scale loads on every fourth stage)
+  // one direct-to-LDS load of stage s: u < A_LOADS activations, then 4 code loads, then 2 scale loads
+  auto issue_unit = [&](int s, int u) {
+    const int b = s % NBUF;
+    if (u < A_LOADS) {
+      g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + (A_LOADS * wv + u) * 1024);
+    } else if (u < NLOADS) {
+      const int i = u - A_LOADS;
+      g2l16(w_src[i] + (size_t)s * 32, W0 + b * W_BYTES + (4 * wv + i) * 1024);
+    } else {
       // 8 scales (16 B) per row for stages s..s+3; at the end of K the window is pulled back inside the row
+      const int i = u - NLOADS;
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
-      const int sb = (s >> 2) & 1;
-#pragma unroll
-      for (int i = 0; i < 2; i++) g2l16(s_src[i] + (size_t)g0 * 2, S0 + sb * S_BYTES + (2 * wv + i) * 1024);
+      g2l16(s_src[i] + (size_t)g0 * 2, S0 + ((s >> 2) & 1) * S_BYTES + (2 * wv + i) * 1024);
     }
+  };
+  auto issue = [&](int s) {
+#pragma unroll
+    for (int u = 0; u < NLOADS; u++) issue_unit(s, u);
+    if ((s & 3) == 0) {
+      issue_unit(s, NLOADS);
+      issue_unit(s, NLOADS + 1);
+    }
+  };
+  // s_waitcnt vmcnt(N), N = loads allowed to stay in flight (loads retire in order)
+  auto wait_loads_except = [&](int s_pending) {  // s_pending: stage whose loads may remain (-1: none)
+    if (s_pending < 0 || s_pending >= nstage) __builtin_amdgcn_s_waitcnt(0x0F70);
+    else if ((s_pending & 3) == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (NLOADS + 2));
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | NLOADS);
   };
 
   floatx16 acc[MF][4];
@@ -170,99 +195,218 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
   for (int nf = 0; nf < 4; nf++) wrow[nf] = UP ? (nf >> 1) * 256 + 64 * wv + 32 * (nf & 1) + n : 128 * wv + 32 * nf + n;
 
-  issue(0);
-  for (int s = 0; s < nstage; s++) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads of stage s have landed
-    __syncthreads();                     // ... and everybody else's; stage s-1 is no longer read
-#ifndef EXP_NO_GLOAD
-    if (s + 1 < nstage) issue(s + 1);
-#endif
-    const uint8_t* Ab = A0 + (s & 1) * A_BYTES;
-    const uint8_t* Wb = W0 + (s & 1) * W_BYTES;
+  // Software pipeline with a hand-placed instruction order.  Inside a stage (four 16-wide K
+  // steps) every MFMA of step q is followed by one "unit" of step q+1's preparation: one
+  // activation fragment read from LDS, or one pair of weights dequantised (3-4 VALU ops), fenced
+  // so the compiler keeps the interleave.  The matrix pipe takes a new MFMA every 32 cycles and a
+  // unit issues in about 20, so the VALU / LDS work hides behind the MFMAs.  Across stages, the
+  // barrier sits in front of the LAST step: by then nobody reads the current LDS buffer any more
+  // (step 3's operands are already in registers), so the loads of stage s+2 can overwrite it, and
+  // step 0 of stage s+1 is prepared from the other buffer while step 3's MFMAs run.
+  half8 a[2][MF];
+  H8 b[2][4];
+  uint4 cw[4];
+  half2v as2[4], bs2[4];
+  float scf[4];
+  const uint8_t* Ab = A0;
+  auto load_a1 = [&](int q, int mf, half8* dst) {
+    const int m = 32 * mf + n;
+    dst[mf] = *(const half8*)(Ab + m * 128 + (((4 * h + q) ^ (m & 7)) << 4));
+  };
+  auto load_codes = [&](int s) {  // raw codes + this lane's scale of stage s (buffers already selected)
+    const uint8_t* Wb = W0 + (s % NBUF) * W_BYTES;
     const uint8_t* Sb = S0 + ((s >> 2) & 1) * S_BYTES;
     int g0 = 2 * (s & ~3);
     g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
     const int sidx = 2 * s + h - g0;  // this lane's scale inside the staged 8
-    uint4 cw[4];
-    _Float16 sc[4];
 #pragma unroll
     for (int nf = 0; nf < 4; nf++) {
       cw[nf] = *(const uint4*)(Wb + wrow[nf] * 32 + h * 16);
-      sc[nf] = *(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
+      scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
     }
-    half2v as2[4], bs2[4];
-    float scf[4];
+  };
+  auto scale_consts = [&]() {
 #pragma unroll
     for (int nf = 0; nf < 4; nf++) {
-      scf[nf] = (float)sc[nf];
       const _Float16 as = (_Float16)(cb_a * scf[nf]), bs = (_Float16)(cb_b * scf[nf]);
       as2[nf] = half2v{as, as};
       bs2[nf] = half2v{bs, bs};
     }
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-      half8 a[MF], b[4];
-#pragma unroll
-      for (int mf = 0; mf < MF; mf++) {
-        const int m = 32 * mf + n;
-        a[mf] = *(const half8*)(Ab + m * 128 + (((4 * h + q) ^ (m & 7)) << 4));
+  };
+  // unit u (0..15) of step q: weight fragment nf = u/4, code pair part = u%4 -> one half2 of b
+  auto deq_unit = [&](int q, int u, H8* dst) {
+    const int nf = u >> 2, part = u & 3;
+    const uint32_t w = q == 0 ? cw[nf].x : q == 1 ? cw[nf].y : q == 2 ? cw[nf].z : cw[nf].w;
+    if (AFFINE) {
+      const uint32_t ws = part >= 2 ? w >> 8 : w;
+      uint32_t t;
+      if ((part & 1) == 0) {
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(ws), "s"(0x000f000fu), "v"(0x64006400u));
+        dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)1024.f, (_Float16)1024.f}) * as2[nf] + bs2[nf];
+      } else {
+        asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(ws), "s"(0x00f000f0u), "v"(0x54005400u));
+        dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)64.f, (_Float16)64.f}) * as2[nf] + bs2[nf];
       }
-#pragma unroll
-      for (int nf = 0; nf < 4; nf++) {
-        const uint32_t w = q == 0 ? cw[nf].x : q == 1 ? cw[nf].y : q == 2 ? cw[nf].z : cw[nf].w;
-        b[nf] = AFFINE ? deq8_affine(w, as2[nf], bs2[nf]) : deq8_table(w, scf[nf], cbs);
-      }
-#pragma unroll
-      for (int mf = 0; mf < MF; mf++)
-#pragma unroll
-        for (int nf = 0; nf < 4; nf++)
-          acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+    } else {
+      half2v hv;
+      hv.x = (_Float16)(cbs[(w >> (4 * part)) & 0xf] * scf[nf]);
+      hv.y = (_Float16)(cbs[(w >> (4 * part + 16)) & 0xf] * scf[nf]);
+      dst[nf].h[part] = hv;
     }
-  }
+  };
+  constexpr int NM = 4 * MF;                      // MFMAs per K step
+  constexpr int UPM = (16 + NM - 1) / NM;         // dequant units behind each MFMA (steps 0-2)
+  constexpr int X0 = NM >= 8 ? NM / 4 : 1;        // step 3: first MFMA slot that dequantises
+  constexpr int XPM = (16 + NM - X0 - 1) / (NM - X0);
 
-  // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair)
+  TSTAMP(1);
+  // loads run two stages ahead of the MFMAs
+  issue(0);
+  if (nstage > 1) issue(1);
+  // stage 0 must have landed; stage 1's loads may still be in flight
+  wait_loads_except(nstage > 1 ? 1 : -1);
+  __syncthreads();
+  load_codes(0);
 #pragma unroll
-  for (int mf = 0; mf < MF; mf++) {
+  for (int mf = 0; mf < MF; mf++) load_a1(0, mf, a[0]);
+  scale_consts();
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int m = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (m >= tile.count) continue;
-      const size_t row = (size_t)(tile.first + m);
-      if (UP) {
+  for (int u = 0; u < 16; u++) deq_unit(0, u, b[0]);
+
+  TSTAMP(2);
+  for (int s = 0; s < nstage; s++) {
+    TSTAMP(10 + 2 * s);
+    Ab = A0 + (s % NBUF) * A_BYTES;
+    const bool pf = s + 2 < nstage;            // stage s+2 exists: its loads go out during step 0
+    const bool pf_s = pf && ((s + 2) & 3) == 0;
 #pragma unroll
-        for (int f = 0; f < 2; f++) {
-          const int col = nb * 256 + 64 * wv + 32 * f + n;
-          if (col < M) {
-            const float g = acc[mf][f][r], u = acc[mf][2 + f][r];
-            const float hv = g / (1.f + __expf(-g)) * u;
-            // hid feeds the down GEMM: interleaved order inside each group of 8 columns
-            ((__half*)out)[row * M + (col & ~7) + ilv_pos(col & 7)] = __float2half(hv);
+    for (int q = 0; q < 3; q++) {
+      const int cur = q & 1, nxt = cur ^ 1;
+#pragma unroll
+      for (int i = 0; i < NM; i++) {
+        const int mf = i >> 2, nf = i & 3;
+        acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][mf], b[cur][nf].v, acc[mf][nf], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i < MF) load_a1(q + 1, i, a[nxt]);
+#pragma unroll
+        for (int k = 0; k < UPM; k++)
+          if (i * UPM + k < 16) deq_unit(q + 1, i * UPM + k, b[nxt]);
+        if (q == 0) {
+          // buffer (s+2)%3 was last read in stage s-1: free since the previous barrier
+          constexpr int LPS = (NLOADS + 2 + NM - 1) / NM;  // loads per MFMA slot
+#pragma unroll
+          for (int k = 0; k < LPS; k++) {
+            const int u = i * LPS + k;
+            if (u < NLOADS) { if (pf) issue_unit(s + 2, u); }
+            else if (u < NLOADS + 2) { if (pf_s) issue_unit(s + 2, u); }
           }
         }
-      } else {
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // last step: a[1], b[1] hold its operands.  Step 0 of stage s+1 is prepared from the next
+    // buffer meanwhile, so that buffer must be complete and visible: loads of stage s+1 done
+    // (stage s+2's may still fly), then the block barrier.
+    TSTAMP(11 + 2 * s);
+#ifndef EXP_NO_VMWAIT
+    wait_loads_except(s + 2);
+#endif
+#ifndef EXP_NO_BARRIER
+    __syncthreads();
+#endif
+    Ab = A0 + ((s + 1) % NBUF) * A_BYTES;
+#pragma unroll
+    for (int i = 0; i < NM; i++) {
+      const int mf = i >> 2, nf = i & 3;
+      acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[1][mf], b[1][nf].v, acc[mf][nf], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // (past the last stage this reads stale LDS and the result is never used)
+#ifndef EXP_NO_PF
+      if (i == 0) load_codes(s + 1);
+      if (i < MF) load_a1(0, i, a[0]);
+      if (i == X0) scale_consts();
+      if (i >= X0) {
+#pragma unroll
+        for (int k = 0; k < XPM; k++)
+          if ((i - X0) * XPM + k < 16) deq_unit(0, (i - X0) * XPM + k, b[0]);
+      }
+#endif
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // no LDS-bound load may outlive the block
+
+  TSTAMP(3);
+  // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair).
+  // f16 results go through a per-wave LDS patch (the stage buffers are dead by now) so that global
+  // stores are 16 bytes per lane and whole rows are contiguous.
+  constexpr int NC = UP ? 64 : 128;          // output columns of this wave
+  constexpr int LDP = NC * 2 + 16;           // padded row pitch of the patch in bytes
+  const int colbase = UP ? nb * 256 + 64 * wv : nb * 512 + 128 * wv;
+  if (UP || F16OUT) {
+    uint8_t* patch = smem + wv * (32 * LDP);
+#pragma unroll
+    for (int mf = 0; mf < MF; mf++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
+        if (UP) {
+#pragma unroll
+          for (int f = 0; f < 2; f++) {
+            const float g = acc[mf][f][r], u = acc[mf][2 + f][r];
+            const float hv = g / (1.f + __expf(-g)) * u;
+            const int c = 32 * f + n;  // hid feeds the down GEMM: interleaved order inside groups of 8
+            *(__half*)(patch + ml * LDP + ((c & ~7) + ilv_pos(c & 7)) * 2) = __float2half(hv);
+          }
+        } else {
+#pragma unroll
+          for (int nf = 0; nf < 4; nf++)
+            *(__half*)(patch + ml * LDP + (32 * nf + n) * 2) = __float2half(acc[mf][nf][r]);
+        }
+      }
+      // 32 rows x NC columns -> NC/8 16-byte chunks per row
+      constexpr int CPR = NC / 8;
+#pragma unroll
+      for (int it = 0; it < (32 * CPR) / 64; it++) {
+        const int c = it * 64 + lane, ml = c / CPR, c8 = c % CPR;
+        const uint4 v = *(const uint4*)(patch + ml * LDP + c8 * 16);
+        const int m = 32 * mf + ml, col = colbase + c8 * 8;
+        if (m < tile.count && col < M) *(uint4*)((__half*)out + (size_t)(tile.first + m) * M + col) = v;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int mf = 0; mf < MF; mf++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int m = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (m >= tile.count) continue;
 #pragma unroll
         for (int nf = 0; nf < 4; nf++) {
-          const int col = nb * 512 + 128 * wv + 32 * nf + n;
-          if (col < M) {
-            if (F16OUT) ((__half*)out)[row * M + col] = __float2half(acc[mf][nf][r]);
-            else ((float*)out)[row * M + col] = acc[mf][nf][r];
-          }
+          const int col = colbase + 32 * nf + n;
+          if (col < M) ((float*)out)[(size_t)(tile.first + m) * M + col] = acc[mf][nf][r];
         }
       }
     }
   }
 }
 
+#ifdef EXP_TIMING
+__device__ unsigned long long g_dbg[4096];
+#endif
+
 template <bool UP, bool F16OUT>
 __global__ void __launch_bounds__(NT, 1)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n) {
+  constexpr bool UPK = UP;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float* cbs = (float*)(smem + 2 * (A_BYTES + W_BYTES + S_BYTES));
+  float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES);
   int* rowidx = (int*)(cbs + 16);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
+  TSTAMP(0);
   const int nt = *ntiles;
   const int wg = blockIdx.x, xcd = wg & 7, j = wg >> 3;
   const int per_xcd = (nt + 7) >> 3;
@@ -301,6 +445,7 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   else if (mfn == 2) GEMM_GO(2);
   else GEMM_GO(4);
 #undef GEMM_GO
+  TSTAMP(4);
 }
 
 LutDev to_dev(const moe_lutw* p) {
@@ -352,6 +497,12 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
+
+#ifdef EXP_TIMING
+MOE_API int moe_dbg_read(unsigned long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg), sizeof(unsigned long long) * 4096);
+}
+#endif
 
 MOE_API int moe_lut_q4cp_view(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t scale_stride,
                               int e_rows, int up_off, moe_lutw* out) {
