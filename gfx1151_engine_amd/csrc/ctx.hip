@@ -119,7 +119,7 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
     if (e == hipSuccess) e = hipMalloc(&c->eoff, (E + 2) * 4);
     if (e == hipSuccess) e = hipMalloc(&c->pairids, T * cfg->topk * 4);
     if (e == hipSuccess) e = hipMalloc(&c->tiles, (size_t)c->max_tiles * sizeof(moe_tile));
-    if (e == hipSuccess) e = hipMalloc(&c->ntiles, 4);
+    if (e == hipSuccess) e = hipMalloc(&c->ntiles, 8);
     if (e == hipSuccess) e = hipMalloc(&c->hid16, k1 * T * mid * 2);
     if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);
   }

@@ -399,7 +399,7 @@ template <bool UP, bool F16OUT>
 __global__ void __launch_bounds__(NT, 1)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
-                const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n) {
+                const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split) {
   constexpr bool UPK = UP;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES);
@@ -407,12 +407,22 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
   TSTAMP(0);
-  const int nt = *ntiles;
+  // Routed tiles and shared-expert tiles (all full) are dealt out separately, or the XCD that
+  // gets the tail of the list would carry every shared tile.
+  const int nt = ntiles[0];
+  const int nr = split ? ntiles[1] : nt;  // routed tiles come first in the list
   const int wg = blockIdx.x, xcd = wg & 7, j = wg >> 3;
-  const int per_xcd = (nt + 7) >> 3;
+  const int per_r = (nr + 7) >> 3, per_s = (nt - nr + 7) >> 3;
   const int tl = j / nblk_n, nb = j - tl * nblk_n;
-  const int ti = xcd * per_xcd + tl;
-  if (tl >= per_xcd || ti >= nt) return;
+  int ti;
+  if (tl < per_r) {
+    ti = xcd * per_r + tl;
+    if (ti >= nr) return;
+  } else {
+    const int k2 = tl - per_r;
+    ti = nr + xcd * per_s + k2;
+    if (k2 >= per_s || ti >= nt) return;
+  }
   const moe_tile tile = tiles[ti];
   const bool shared = tile.expert >= n_experts;
   const LutDev& L = shared ? Sh : R;
@@ -485,15 +495,16 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
     attr_done = true;
   }
-  const int per_xcd = (max_tiles + 7) / 8;
+  // per XCD: ceil(routed/8) + ceil(shared/8) <= max_tiles/8 + 2 tile slots
+  const int per_xcd = (max_tiles + 7) / 8 + 1;
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
   LutDev R = to_dev(routed), S = to_dev(sh ? sh : routed);
   if (up)
-    k_moe_gemm_q4cp<true, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
+    k_moe_gemm_q4cp<true, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, sh ? 1 : 0);
   else if (f16out)
-    k_moe_gemm_q4cp<false, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
+    k_moe_gemm_q4cp<false, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, sh ? 1 : 0);
   else
-    k_moe_gemm_q4cp<false, false><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n);
+    k_moe_gemm_q4cp<false, false><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, sh ? 1 : 0);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -137,7 +137,10 @@ __global__ void __launch_bounds__(1024) k_tiles_shared(const int* __restrict__ e
     t.count = min(cap, P - j * cap);
     tiles[routed_total + j] = t;
   }
-  if (e == 0) *total = routed_total + nsh;
+  if (e == 0) {
+    total[0] = routed_total + nsh;
+    total[1] = routed_total;
+  }
   if (sh_first >= 0)
     for (int i = e; i < P; i += 1024) tokidx[sh_first + i] = i;
 }
