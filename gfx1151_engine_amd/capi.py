@@ -173,6 +173,7 @@ class LutW(C.Structure):
 
 
 LUT_Q4CP = 100
+OPT_INT_DECODE = 1
 
 
 def lut_q4cp_view(blob, rows, cols, e_rows, up_off):
@@ -259,6 +260,9 @@ class Moe:
             y = torch.empty((P, self.cfg.d), dtype=torch.float32, device=x.device)
         check(lib().moe_forward(self.h, layer, ptr(x), P, ptr(y), stream()), "moe_forward")
         return y
+
+    def set_option(self, option, value):
+        check(lib().moe_set_option(self.h, option, value), "moe_set_option")
 
     def profile(self, on=True):
         check(lib().moe_profile_enable(self.h, 1 if on else 0), "moe_profile_enable")

@@ -1,6 +1,7 @@
 // Model-level entry points: a context owns the scratch, layers hold borrowed weight views, and
 // moe_forward picks the path by batch size.
 // (reference: GpuModel::moe / moe_b / moe_gguf / moe_q4w_run, src/gpu/parts/40_model.inc:1664-1861,4018-4157)
+#include <cmath>
 #include <new>
 #include <vector>
 
@@ -15,7 +16,20 @@ struct MoeLayer {
   moe_gg_experts gg{};
   moe_wview sh_gate{}, sh_up{}, sh_down{}, sh_sg{};
   int sh_gguf_type = 0;
+  // every q4cp codebook of the layer is affine (cb[n] = a*n + b): the integer-dot decode kernels apply
+  bool experts_affine = false, shared_affine = false;
 };
+
+// cb[n] == a*n + b for all 16 codes?  Reads the 64-byte codebook back from the device: weight
+// registration is set-up work, not part of the enqueue-only forward path.
+static int codebook_affine(const moe_wview* w, bool* out) {
+  float cb[16];
+  MOE_HIP(hipMemcpy(cb, w->data, sizeof cb, hipMemcpyDeviceToHost));
+  bool ok = true;
+  for (int n = 0; n < 16; n++) ok = ok && cb[n] == fmaf((float)n, cb[1] - cb[0], cb[0]);
+  *out = ok;
+  return MOE_OK;
+}
 
 struct moe_ctx {
   moe_config cfg;
@@ -26,7 +40,10 @@ struct moe_ctx {
   float* ws = nullptr;        // [T][id_stride]
   float* sh_logit = nullptr;  // [T]
   float* hid32 = nullptr;     // [min(T,small_max)][k+1][mid] f32 (small-batch path)
+  uint32_t *xplanes = nullptr, *hplanes = nullptr;  // integer digit planes of x / hid (decode kernels)
+  float2 *xmeta = nullptr, *hmeta = nullptr;
   int small_max = 32;         // batches up to this size take the in-place GEMV path
+  bool int_decode = true;     // small batches: integer-dot kernels where they apply (else f32 kernels)
   // batch path (allocated only when max_tokens > small_max)
   moe_routing* routing = nullptr;
   __half* x16 = nullptr;      // [T][d]
@@ -72,7 +89,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->routing) rc = moe_routing_destroy(c->routing);
   for (hipEvent_t e : c->ev)
     if (e) (void)hipEventDestroy(e);
-  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->hid32, c->x16, c->tokidx, c->pw, c->eoff,
+  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16};
   for (void* b : bufs)
     if (b) {
@@ -102,9 +119,13 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   hipError_t e = hipMalloc(&c->logits, T * E * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ids, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ws, T * S * 4);
-  if (e == hipSuccess) e = hipMalloc(&c->sh_logit, T * 4);
+  if (e == hipSuccess) e = hipMalloc(&c->sh_logit, (T + 1) * 4);  // + one int the decode kernels may flag
   const size_t Ts = T < (size_t)c->small_max ? T : (size_t)c->small_max;
   if (e == hipSuccess) e = hipMalloc(&c->hid32, Ts * (size_t)(cfg->topk + 1) * cfg->mid * 4);
+  if (e == hipSuccess) e = hipMalloc(&c->xplanes, Ts * moe_qvec_plane_bytes(cfg->d));
+  if (e == hipSuccess) e = hipMalloc(&c->xmeta, Ts * moe_qvec_meta_bytes(cfg->d));
+  if (e == hipSuccess) e = hipMalloc(&c->hplanes, Ts * (size_t)(cfg->topk + 1) * moe_qvec_plane_bytes(cfg->mid));
+  if (e == hipSuccess) e = hipMalloc(&c->hmeta, Ts * (size_t)(cfg->topk + 1) * moe_qvec_meta_bytes(cfg->mid));
   if (e == hipSuccess && T > (size_t)c->small_max) {
     const size_t k1 = (size_t)cfg->topk + 1, d = cfg->d, mid = cfg->mid;
     c->max_tiles = (int)((T * cfg->topk + 127) / 128 + E + (T + 127) / 128);
@@ -156,6 +177,10 @@ MOE_API int moe_set_experts_q4cp(moe_ctx* c, int layer, const moe_wview* gu, con
   if (gu->rows != (uint64_t)g.experts * 2 * g.mid || (int)gu->cols != g.d ||
       dn->rows != (uint64_t)g.experts * g.d || (int)dn->cols != g.mid)
     return MOE_E_INVALID;
+  bool a1 = false, a2 = false;
+  int rc;
+  if ((rc = codebook_affine(gu, &a1)) || (rc = codebook_affine(dn, &a2))) return rc;
+  L->experts_affine = a1 && a2;
   L->gate_up = *gu;
   L->down = *dn;
   L->has_q4cp = true;
@@ -188,6 +213,13 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
   } else if (sh_gguf_type != MOE_GGML_Q4_K) {
     return MOE_E_UNSUPPORTED;
   }
+  L->shared_affine = false;
+  if (sh_gguf_type == 0) {
+    bool a1 = false, a2 = false, a3 = false;
+    int rc;
+    if ((rc = codebook_affine(g, &a1)) || (rc = codebook_affine(u, &a2)) || (rc = codebook_affine(dn, &a3))) return rc;
+    L->shared_affine = a1 && a2 && a3;
+  }
   L->sh_gate = *g;
   L->sh_up = *u;
   L->sh_down = *dn;
@@ -195,6 +227,14 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
   L->sh_gguf_type = sh_gguf_type;
   L->has_shared = true;
   return MOE_OK;
+}
+
+MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
+  if (!c) return MOE_E_INVALID;
+  switch (option) {
+    case MOE_OPT_INT_DECODE: c->int_decode = value != 0; return MOE_OK;
+    default: return MOE_E_INVALID;
+  }
 }
 
 MOE_API int moe_profile_enable(moe_ctx* c, int on) {
@@ -234,13 +274,30 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   int rc;
   c->ev_n = 0;
   prof_mark(c, 0, st);
+  const int nslots_d = g.topk + (L.has_shared ? 1 : 0);
+  const bool use_int = L.has_q4cp && c->int_decode && L.experts_affine && (!L.has_shared || L.shared_affine) &&
+                       (!L.has_shared || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
   if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
-                                    c->logits, c->sh_logit, st)))
+                                    c->logits, c->sh_logit, use_int ? c->xplanes : nullptr, c->xmeta, st)))
     return rc;
   if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
   prof_mark(c, MOE_PROF_ROUTER, st);
   if (L.has_q4cp) {
     if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
+    if (use_int) {
+      // integer-dot kernels: activations as digit planes (made by the logits launch above)
+      if ((rc = moe_launch_dec_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
+                                  L.has_shared ? &L.sh_up : nullptr, &L.down,
+                                  L.has_shared ? &L.sh_down : nullptr, (int*)c->sh_logit + c->cfg.max_tokens,
+                                  c->xplanes, c->xmeta, c->ids, g.id_stride,
+                                  g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st)))
+        return rc;
+      prof_mark(c, MOE_PROF_UP, st);
+      rc = moe_launch_dec_dn(&L.down, L.has_shared ? &L.sh_down : nullptr, c->sh_logit, c->hplanes, c->hmeta,
+                             c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, y, (uint64_t)g.d, st);
+      prof_mark(c, MOE_PROF_DOWN, st);
+      return rc;
+    }
     if ((rc = moe_launch_gemv_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
                                  L.has_shared ? &L.sh_up : nullptr, x, (uint64_t)g.d, c->ids, g.id_stride,
                                  g.topk, P, g.mid, c->hid32, st)))

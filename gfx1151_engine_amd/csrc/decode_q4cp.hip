@@ -1,0 +1,366 @@
+// Decode (T <= 32): bandwidth-bound expert GEMV on q4cp weights read in place, integer dot
+// products.  The activation vector is turned once per token into three signed 7-bit digit planes
+// per 32-element group (x ~= q_g * (2^14 p0 + 2^7 p1 + p2), 21 significant bits relative to the
+// group maximum), so that a 16-byte load of 32 weight codes costs 12 unpack + 24 v_dot4_i32_i8
+// instead of ~100 float operations: the VALU then keeps up with HBM.  Weights stay exact (codes are
+// integers; the group scale and q_g are applied in f32 after the integer sum), the zero point is
+// folded in through the group sum of the activations.
+// (reference: src/gpu/parts/20_kernels_gemv.inc:1608-1835 — same contract: per-slot gate/up with
+//  SwiGLU, then the down projection with the top-k weighted combine in slot order, no atomics)
+#include "common.h"
+#include "internal.h"
+#include "qvec.h"
+
+namespace {
+
+
+__device__ __forceinline__ float dpp_max_row(float v) {  // max over each row of 16 lanes
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
+  return v;
+}
+// sum over each half-wave of 32 lanes; every lane of the half gets the result
+__device__ __forceinline__ float sum32(float v) {
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));   // xor 1
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));   // xor 2
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));  // mirror in 8
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));  // mirror in 16
+  v += __shfl_xor(v, 16, 64);
+  return v;
+}
+__device__ __forceinline__ float sum64(float v) {
+  v = sum32(v);
+  return v + __shfl_xor(v, 32, 64);
+}
+
+// Quantise 32 floats held one per lane by lanes [0,32) of a half-wave (j = lane & 31): returns
+// this lane's three digits, q and q*sum(X).
+__device__ __forceinline__ void quant32_lane(float x, int& p0, int& p1, int& p2, float& q, float& qsx) {
+  float m = dpp_max_row(fabsf(x));
+  m = fmaxf(m, __shfl_xor(m, 16, 64));
+  const float inv = m > 0.f ? 1048576.f / m : 0.f;
+  q = m * (1.f / 1048576.f);
+  const int X = (int)rintf(x * inv);
+  p2 = ((X + 64) & 127) - 64;
+  const int X1 = (X - p2) >> 7;
+  p1 = ((X1 + 64) & 127) - 64;
+  p0 = (X1 - p1) >> 7;
+  qsx = q * sum32((float)X);
+}
+
+// One thread per group: x (f32, K elements) -> qvec.  Blocks of 64.
+__global__ void __launch_bounds__(64) k_qvec_from_f32(const float* __restrict__ x, uint64_t x_stride,
+                                                      int G, uint32_t* __restrict__ planes,
+                                                      float2* __restrict__ meta) {
+  const int t = blockIdx.y, g = blockIdx.x * 64 + threadIdx.x;
+  if (g < G) qvec_group_from_f32(x, x_stride, G, t, g, planes, meta);
+}
+
+struct XG {  // one group's activation planes in registers
+  uint32_t p[3][8];
+  float q, qsx;
+};
+__device__ __forceinline__ void load_xg(XG& x, const uint32_t* planes, const float2* meta, size_t gi) {
+  const uint4* s = (const uint4*)(planes + gi * QV_GROUP_DW);
+#pragma unroll
+  for (int p = 0; p < 3; p++) {
+    const uint4 a = s[2 * p], b = s[2 * p + 1];
+    x.p[p][0] = a.x; x.p[p][1] = a.y; x.p[p][2] = a.z; x.p[p][3] = a.w;
+    x.p[p][4] = b.x; x.p[p][5] = b.y; x.p[p][6] = b.z; x.p[p][7] = b.w;
+  }
+  const float2 m = meta[gi];
+  x.q = m.x;
+  x.qsx = m.y;
+}
+
+// sum_k cb[n_k] * x_k over one group, cb = a*n + b:  a * q * (2^14 D0 + 2^7 D1 + D2) + b * q * sum(X)
+__device__ __forceinline__ float chunk_dot(const uint4 cw, const XG& x, float cb_a, float cb_b) {
+  const uint32_t w[4] = {cw.x, cw.y, cw.z, cw.w};
+  int d0 = 0, d1 = 0, d2 = 0;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int lo = (int)(w[i] & 0x0f0f0f0fu), hi = (int)((w[i] >> 4) & 0x0f0f0f0fu);
+    d0 = __builtin_amdgcn_sdot4(lo, (int)x.p[0][2 * i], d0, false);
+    d1 = __builtin_amdgcn_sdot4(lo, (int)x.p[1][2 * i], d1, false);
+    d2 = __builtin_amdgcn_sdot4(lo, (int)x.p[2][2 * i], d2, false);
+    d0 = __builtin_amdgcn_sdot4(hi, (int)x.p[0][2 * i + 1], d0, false);
+    d1 = __builtin_amdgcn_sdot4(hi, (int)x.p[1][2 * i + 1], d1, false);
+    d2 = __builtin_amdgcn_sdot4(hi, (int)x.p[2][2 * i + 1], d2, false);
+  }
+  const float v = fmaf((float)d0, 16384.f, (float)(d1 * 128 + d2));
+  return fmaf(cb_a * x.q, v, cb_b * x.qsx);
+}
+
+struct DecW {  // one q4cp tensor's planes
+  const uint8_t *codes, *scales;
+  const float* cb;
+  uint64_t ss;
+};
+
+struct GuArgs2 {
+  DecW gu;           // fused gate_up [E*2*mid][d]
+  DecW shg, shu;     // shared expert gate / up [mid][d] (codes == nullptr: none)
+  DecW dn, shd;      // down tensors: only touched, so that they sit in L2 / Infinity Cache for k_dec_dn
+  int* sink;         // never written in practice (keeps the touching loads alive)
+};
+
+// grid (mid/32, slots incl. shared, P); block 512.  Wave w: gate rows 4w..4w+3 and the matching up
+// rows of this block's 32; lane L holds activation groups L and 64 + (L & 31).  Rows are taken two
+// at a time with three 16-byte loads per lane: (row0, group L), (row1, group L), and the tail group
+// of row0 (lanes < 32) or row1 (lanes >= 32); all twelve loads of a wave are in flight together.
+constexpr int GU2_ROWS = 32;
+__global__ void __launch_bounds__(512) k_dec_gu(GuArgs2 A, const uint32_t* __restrict__ xplanes,
+                                                const float2* __restrict__ xmeta,
+                                                const int* __restrict__ ids, int id_stride, int kpt, int d,
+                                                int mid, uint32_t* __restrict__ hplanes,
+                                                float2* __restrict__ hmeta, float* __restrict__ hid_f32) {
+  __shared__ float gs[GU2_ROWS], us[GU2_ROWS];
+  __shared__ uint32_t pk[QV_GROUP_DW];
+  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int G = d / 32;
+  const bool shared = s >= kpt;
+  const DecW Wg = shared ? A.shg : A.gu;  // block-uniform choice, by value
+  const DecW Wu = shared ? A.shu : A.gu;
+  const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
+  const uint64_t grow0 = shared ? 0 : (uint64_t)e * 2 * mid;
+  const uint64_t urow0 = shared ? 0 : (uint64_t)e * 2 * mid + mid;
+  const int r0 = blockIdx.x * GU2_ROWS + 4 * wv;  // first of this wave's 4 gate rows
+
+  const int gA = lane, gB = 64 + (lane & 31);
+  const bool vA = gA < G, vB = gB < G;
+  const size_t rb = (size_t)d / 2;
+  // pairs 0,1: gate rows (r0+2p, r0+2p+1); pairs 2,3: the up rows
+  uint4 ca[4], cb[4], ct[4];
+  __half sa[4], sb[4], st[4];
+#pragma unroll
+  for (int p = 0; p < 4; p++) {
+    const DecW W = p >= 2 ? Wu : Wg;
+    const uint64_t row = (p >= 2 ? urow0 : grow0) + r0 + 2 * (p & 1);
+    const uint8_t* c0 = W.codes + row * rb;
+    const uint8_t* s0 = W.scales + row * W.ss;
+    const uint64_t trow = lane < 32 ? 0 : 1;
+    if (vA) {
+      ca[p] = *(const uint4*)(c0 + (size_t)gA * 16);
+      cb[p] = *(const uint4*)(c0 + rb + (size_t)gA * 16);
+      sa[p] = *(const __half*)(s0 + gA * 2);
+      sb[p] = *(const __half*)(s0 + W.ss + gA * 2);
+    }
+    if (vB) {
+      ct[p] = *(const uint4*)(c0 + trow * rb + (size_t)gB * 16);
+      st[p] = *(const __half*)(s0 + trow * W.ss + gB * 2);
+    }
+  }
+  // The down projection only depends on the routing, not on this kernel's result: pull this
+  // block's share (1/gridDim.x) of the slot's down weights towards the chip now, so that the whole
+  // layer's weights stream from HBM in one go and k_dec_dn finds them in L2 / Infinity Cache.
+  uint4 pf[7];
+  {
+    const DecW Wd = shared ? A.shd : A.dn;
+    const size_t cbytes = (size_t)d * (mid / 2), sbytes = (size_t)d * Wd.ss;
+    const uint8_t* cbase = Wd.codes + (shared ? 0 : (size_t)e * cbytes);
+    const uint8_t* sbase = Wd.scales + (shared ? 0 : (size_t)e * sbytes);
+    const size_t cper = cbytes / gridDim.x, sper = sbytes / gridDim.x;  // multiples of 16 for the shapes served
+#pragma unroll
+    for (int i = 0; i < 6; i++) {
+      const size_t off = ((size_t)i * 512 + threadIdx.x) * 16;
+      pf[i] = off + 16 <= cper ? *(const uint4*)(cbase + blockIdx.x * cper + off) : make_uint4(0, 0, 0, 0);
+    }
+    const size_t off = (size_t)threadIdx.x * 16;
+    pf[6] = off + 16 <= sper ? *(const uint4*)(sbase + blockIdx.x * sper + off) : make_uint4(0, 0, 0, 0);
+  }
+  const float ga = Wg.cb[1] - Wg.cb[0], gb = Wg.cb[0], ua = Wu.cb[1] - Wu.cb[0], ub = Wu.cb[0];
+  XG xa, xb;
+  const size_t xbase = (size_t)tok * G;
+  if (vA) load_xg(xa, xplanes, xmeta, xbase + gA);
+  if (vB) load_xg(xb, xplanes, xmeta, xbase + gB);
+
+  float acc[8];
+#pragma unroll
+  for (int p = 0; p < 4; p++) {
+    const float a = p >= 2 ? ua : ga, b = p >= 2 ? ub : gb;
+    float v0 = 0.f, v1 = 0.f;
+    if (vA) {
+      v0 = __half2float(sa[p]) * chunk_dot(ca[p], xa, a, b);
+      v1 = __half2float(sb[p]) * chunk_dot(cb[p], xa, a, b);
+    }
+    if (vB) {
+      const float vt = __half2float(st[p]) * chunk_dot(ct[p], xb, a, b);
+      if (lane < 32) v0 += vt;
+      else v1 += vt;
+    }
+    acc[2 * p] = v0;
+    acc[2 * p + 1] = v1;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = sum64(acc[i]);
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      gs[4 * wv + i] = acc[i];
+      us[4 * wv + i] = acc[4 + i];
+    }
+  }
+  {
+    uint32_t t = 0;
+#pragma unroll
+    for (int i = 0; i < 7; i++) t |= pf[i].x & pf[i].y & pf[i].z & pf[i].w;
+    if (t == 0xffffffffu && A.sink) A.sink[0] = 1;  // 128 one-bits in a row of codes: not in practice
+  }
+  __syncthreads();
+  // SwiGLU on the block's 32 rows = one group of the down projection's input; quantise it
+  if (wv == 0) {
+    const int j = lane & 31;
+    const float g = gs[j], u = us[j];
+    const float hv = g / (1.f + expf(-g)) * u;
+    const size_t slot = (size_t)tok * nslots + s;
+    if (hid_f32 && lane < 32) hid_f32[slot * mid + blockIdx.x * GU2_ROWS + j] = hv;
+    int p0, p1, p2;
+    float q, qsx;
+    quant32_lane(hv, p0, p1, p2, q, qsx);
+    if (lane < QV_GROUP_DW) pk[lane] = 0;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    if (lane < 32) {
+      const int dw = 2 * (j >> 3) + (j & 1), sh = 8 * ((j & 7) >> 1);
+      atomicOr(&pk[dw], (uint32_t)(p0 & 0xff) << sh);
+      atomicOr(&pk[8 + dw], (uint32_t)(p1 & 0xff) << sh);
+      atomicOr(&pk[16 + dw], (uint32_t)(p2 & 0xff) << sh);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_wave_barrier();
+    const size_t gi = slot * (mid / 32) + blockIdx.x;
+    if (lane < QV_GROUP_DW) hplanes[gi * QV_GROUP_DW + lane] = pk[lane];
+    if (lane == 0) hmeta[gi] = make_float2(q, qsx);
+  }
+}
+
+struct DnArgs2 {
+  DecW dn;   // routed down [E*d][mid]
+  DecW shd;  // shared expert down [d][mid] (codes == nullptr: none)
+  const float* sh_logit;
+};
+
+// grid (d/ROWS, P); block = 64 x ceil(slots/2).  Wave = one slot pair, half-wave = one slot: lane
+// (L & 31) holds that slot's activation group (K/32 <= 32 groups) in registers for all the block's
+// rows.  The weighted combine runs afterwards in slot order (descending router probability), then
+// the shared expert: deterministic, no atomics.
+constexpr int DN2_ROWS = 8, DN2_MAXSLOTS = 16;
+__global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __restrict__ hplanes,
+                                                const float2* __restrict__ hmeta,
+                                                const int* __restrict__ ids, const float* __restrict__ ws,
+                                                int id_stride, int kpt, int d, int mid,
+                                                float* __restrict__ out, uint64_t out_stride) {
+  __shared__ float part[DN2_MAXSLOTS][DN2_ROWS];
+  const int tok = blockIdx.y;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const bool has_shared = A.shd.codes != nullptr;
+  const int nslots = kpt + (has_shared ? 1 : 0);
+  const int G = mid / 32, g = lane & 31, half = lane >> 5;
+  const int r0 = blockIdx.x * DN2_ROWS;
+  const size_t rb = (size_t)mid / 2;
+  {
+    const int s = 2 * wv + half;
+    const bool live = s < nslots && g < G;
+    const bool shared = has_shared && s == nslots - 1;
+    // per-lane choice of tensor: pick the members by value (a reference to one of two kernel
+    // arguments would be re-read from memory in front of every load)
+    const uint8_t* wcodes = shared ? A.shd.codes : A.dn.codes;
+    const uint8_t* wscales = shared ? A.shd.scales : A.dn.scales;
+    const float* wcb = shared ? A.shd.cb : A.dn.cb;
+    const uint64_t wss = shared ? A.shd.ss : A.dn.ss;
+    const int e = (live && !shared) ? ids[(size_t)tok * id_stride + s] : 0;
+    const uint64_t row0 = (shared ? 0 : (uint64_t)e * d) + r0;
+    const uint8_t* cp = wcodes + row0 * rb + (size_t)g * 16;
+    const uint8_t* sp = wscales + row0 * wss + g * 2;
+    uint4 cw[DN2_ROWS];
+    __half sc[DN2_ROWS];
+#pragma unroll
+    for (int r = 0; r < DN2_ROWS; r++) {
+      if (live) {
+        cw[r] = *(const uint4*)(cp + r * rb);
+        sc[r] = *(const __half*)(sp + r * wss);
+      }
+    }
+    const float a = wcb[1] - wcb[0], b = wcb[0];
+    XG x;
+    if (live) load_xg(x, hplanes, hmeta, ((size_t)tok * nslots + s) * G + g);
+#pragma unroll
+    for (int r = 0; r < DN2_ROWS; r++) {
+      float v = live ? __half2float(sc[r]) * chunk_dot(cw[r], x, a, b) : 0.f;
+      v = sum32(v);
+      if (g == 0 && s < nslots) part[s][r] = v;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < DN2_ROWS) {
+    const int r = threadIdx.x;
+    float y = 0.f;
+    for (int s = 0; s < kpt; s++) y += ws[(size_t)tok * id_stride + s] * part[s][r];
+    if (has_shared) y += sigmoid_f(A.sh_logit[tok]) * part[kpt][r];
+    out[(size_t)tok * out_stride + r0 + r] = y;
+  }
+}
+
+DecW decw(const moe_wview* w) {
+  DecW o{};
+  if (w) {
+    Q4cpOps q = q4cp_ops(w);
+    o.codes = q.codes; o.scales = q.scales; o.cb = q.cb; o.ss = q.scale_stride;
+  }
+  return o;
+}
+
+}  // namespace
+
+size_t moe_qvec_plane_bytes(int K) { return (size_t)(K / 32) * QV_GROUP_DW * 4; }
+size_t moe_qvec_meta_bytes(int K) { return (size_t)(K / 32) * sizeof(float2); }
+
+// Supported shapes of the integer-dot decode kernels (otherwise the caller uses the f32 kernels).
+bool moe_dec_supported(int d, int mid, int nslots) {
+  return d % 32 == 0 && d / 32 <= 96 && mid % 32 == 0 && mid / 32 <= 32 && nslots <= DN2_MAXSLOTS &&
+         mid % GU2_ROWS == 0 && d % DN2_ROWS == 0;
+}
+
+int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
+                    hipStream_t st) {
+  const int G = K / 32;
+  dim3 grid((G + 63) / 64, P);
+  k_qvec_from_f32<<<grid, 64, 0, st>>>(x, x_stride, G, planes, meta);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
+                      const moe_wview* dn, const moe_wview* sh_down, int* sink, const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
+                      int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
+                      hipStream_t st) {
+  GuArgs2 A{};
+  A.gu = decw(gu);
+  A.shg = decw(sh_gate);
+  A.shu = decw(sh_up);
+  A.dn = decw(dn);
+  A.shd = decw(sh_down);
+  A.sink = sink;
+  dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
+  k_dec_gu<<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,
+                      const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
+                      int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
+                      hipStream_t st) {
+  DnArgs2 A{};
+  A.dn = decw(dn);
+  A.shd = decw(sh_down);
+  A.sh_logit = sh_logit;
+  dim3 grid(d / DN2_ROWS, P);
+  const int nslots = kpt + (sh_down ? 1 : 0);
+  k_dec_dn<<<grid, 64 * ((nslots + 1) / 2), 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}

@@ -3,7 +3,8 @@
 #include "common.h"
 
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
-                            int P, float* logits, float* out_x, hipStream_t st);
+                            int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
+                            hipStream_t st);
 int moe_launch_gemv_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                        const float* x, uint64_t x_stride, const int* ids, int id_stride, int kpt, int P,
                        int mid, float* hid, hipStream_t st);
@@ -26,3 +27,16 @@ int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, con
                       hipStream_t st);
 int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
                           float* logits, float* out_x, hipStream_t st);
+size_t moe_qvec_plane_bytes(int K);
+size_t moe_qvec_meta_bytes(int K);
+bool moe_dec_supported(int d, int mid, int nslots);
+int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
+                    hipStream_t st);
+int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
+                      const moe_wview* dn, const moe_wview* sh_down, int* sink, const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
+                      int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
+                      hipStream_t st);
+int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,
+                      const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
+                      int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
+                      hipStream_t st);

@@ -1,6 +1,7 @@
 // Router: logits with the CPU path's fp64 accumulation, fp64 softmax, top-k, renormalised weights.
 // (reference: src/ref.cpp:68-77,565-594; src/gpu/parts/20_kernels_gemv.inc:1433-1562)
 #include "common.h"
+#include "qvec.h"
 
 namespace {
 
@@ -102,28 +103,39 @@ __global__ void __launch_bounds__(256) k_router_logits_seq(const void* __restric
   }
 }
 
-// ---- lane-parallel order for small P: one wave per weight row, lanes stride the columns,
-// per-lane fp64 chains, fixed butterfly.  The fp64 sum differs from the sequential one only in
-// its last bits, so the f32 logit differs with probability ~1e-8 per value.
-// Row E (if Wx given) is the shared-expert gate vector: out_x[t] = its logit.
+// ---- lane-parallel order for small P: one wave (= one block) per weight row, lanes stride the
+// columns, four independent fp64 chains per lane and token, fixed combination order.  The fp64
+// sum differs from the sequential one only in its last bits, so the f32 logit differs with
+// probability ~1e-8 per value.  Row E (if Wx given) is the shared-expert gate vector: out_x[t] =
+// its logit.  Blocks past the rows (if planes given) turn x into the digit planes of the
+// integer-dot decode kernels, so that work rides along instead of costing a launch.
 template <bool BF16, int TT>
-__global__ void __launch_bounds__(256) k_router_logits_par(const void* __restrict__ W,
-                                                           const float* __restrict__ bias,
-                                                           const void* __restrict__ Wx, bool wx_bf16,
-                                                           const float* __restrict__ x, int P, int E,
-                                                           int d, float* __restrict__ logits,
-                                                           float* __restrict__ out_x) {
-  const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row > E || (row == E && !Wx)) return;
+__global__ void __launch_bounds__(64) k_router_logits_par(const void* __restrict__ W,
+                                                          const float* __restrict__ bias,
+                                                          const void* __restrict__ Wx, bool wx_bf16,
+                                                          const float* __restrict__ x, int P, int E,
+                                                          int d, float* __restrict__ logits,
+                                                          float* __restrict__ out_x, int nrows,
+                                                          uint32_t* __restrict__ planes,
+                                                          float2* __restrict__ meta) {
+  const int lane = threadIdx.x;
+  const int row = blockIdx.x;
+  if (row >= nrows) {
+    const int G = d / 32, gb = (G + 63) / 64;
+    const int q = row - nrows, t = q / gb, g = (q % gb) * 64 + lane;
+    if (t < P && g < G) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
+    return;
+  }
   const bool extra = row == E;
   const void* Wr = extra ? Wx : W;
   const uint64_t base = extra ? 0 : (uint64_t)row * d;
   const bool bf = extra ? wx_bf16 : BF16;
   for (int t0 = 0; t0 < P; t0 += TT) {
-    double acc[TT];
+    double acc[TT][4];
 #pragma unroll
-    for (int i = 0; i < TT; i++) acc[i] = 0.0;
+    for (int i = 0; i < TT; i++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) acc[i][q] = 0.0;
     for (int c = lane * 4; c < d; c += 256) {
       float w[4];
       if (bf) {
@@ -140,16 +152,16 @@ __global__ void __launch_bounds__(256) k_router_logits_par(const void* __restric
       for (int i = 0; i < TT; i++) {
         if (t0 + i < P) {
           const float4 xv = *(const float4*)(x + (size_t)(t0 + i) * d + c);
-          acc[i] = fma((double)w[0], (double)xv.x, acc[i]);
-          acc[i] = fma((double)w[1], (double)xv.y, acc[i]);
-          acc[i] = fma((double)w[2], (double)xv.z, acc[i]);
-          acc[i] = fma((double)w[3], (double)xv.w, acc[i]);
+          acc[i][0] = fma((double)w[0], (double)xv.x, acc[i][0]);
+          acc[i][1] = fma((double)w[1], (double)xv.y, acc[i][1]);
+          acc[i][2] = fma((double)w[2], (double)xv.z, acc[i][2]);
+          acc[i][3] = fma((double)w[3], (double)xv.w, acc[i][3]);
         }
       }
     }
 #pragma unroll
     for (int i = 0; i < TT; i++) {
-      const double s = wave_sum(acc[i]);
+      const double s = wave_sum((acc[i][0] + acc[i][1]) + (acc[i][2] + acc[i][3]));
       if (lane == 0 && t0 + i < P) {
         float v = (float)s;
         if (extra) out_x[t0 + i] = v;
@@ -161,6 +173,8 @@ __global__ void __launch_bounds__(256) k_router_logits_par(const void* __restric
     }
   }
 }
+
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 
 // ---- softmax + top-k, one wave per token (E <= 64*NPL) ----
 template <int NPL>
@@ -207,40 +221,44 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
       for (int e = 0; e < E; e++) s += (double)pbuf[wv][e];
     se = __shfl(s, 0, 64);
   }
-  float sc[NPL];
+  // probabilities are >= 0, so their bit patterns order like unsigned integers; key = bits + 1
+  // (0 = not a candidate: past E, or already selected)
+  uint32_t key[NPL];
 #pragma unroll
   for (int j = 0; j < NPL; j++) {
     const int e = lane + 64 * j;
-    sc[j] = e < E ? (float)((double)p[j] / se) : -1.f;
+    key[j] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
   }
-  // k rounds of arg-max: larger probability first, equal probabilities -> lower index
+  // k rounds of arg-max: larger probability first, equal probabilities -> lower index.  The
+  // maximum goes through DPP row operations + four lane reads (no LDS round trips); the lowest
+  // index holding it is found with ballots: register j holds indices [64j, 64j+63], so the first
+  // register with a hit has the lowest index range and its lowest set lane the lowest index.
   double wsum = 0.0;
   float mine = 0.f;  // lane r keeps the r-th selected probability
   for (int r = 0; r < k; r++) {
-    float bv = -2.f;
-    int bi = 0x7fffffff;
+    uint32_t m = key[0];
 #pragma unroll
-    for (int j = 0; j < NPL; j++)
-      if (sc[j] > bv) {
-        bv = sc[j];
-        bi = lane + 64 * j;
-      }
+    for (int j = 1; j < NPL; j++) m = m > key[j] ? m : key[j];
+    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true));
+    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, true));
+    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x141, 0xf, 0xf, true));
+    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x140, 0xf, 0xf, true));
+    const uint32_t wm = umax(umax((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+                             umax((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+    int bi = -1;
 #pragma unroll
-    for (int o = 32; o; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, 64);
-      const int oi = __shfl_xor(bi, o, 64);
-      if (ov > bv || (ov == bv && oi < bi)) {
-        bv = ov;
-        bi = oi;
-      }
+    for (int j = 0; j < NPL; j++) {
+      const unsigned long long hit = __ballot(key[j] == wm);
+      if (bi < 0 && hit) bi = 64 * j + (__ffsll((long long)hit) - 1);
     }
+    const float bv = __uint_as_float(wm - 1u);
     wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
     if (lane == r) mine = bv;
     if (lane == 0) ids[(size_t)tok * id_stride + r] = bi;
     if ((bi & 63) == lane) {
 #pragma unroll
       for (int j = 0; j < NPL; j++)
-        if (j == (bi >> 6)) sc[j] = -1.f;
+        if (j == (bi >> 6)) key[j] = 0u;
     }
   }
   if (lane < k) ws[(size_t)tok * id_stride + lane] = (float)((double)mine / wsum);
@@ -259,9 +277,9 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool par = mode == 0 && P <= 32 && d % 4 == 0 && moe_aligned(x, 16) && moe_aligned(W->data, 16);
   if (par) {
-    dim3 g((E + 3) / 4);
-    if (bf) k_router_logits_par<true, 4><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
-    else k_router_logits_par<false, 4><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
+    dim3 g(E);
+    if (bf) k_router_logits_par<true, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
+    else k_router_logits_par<false, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
   } else {
     dim3 g((E + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
     if (bf) k_router_logits_seq<true><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
@@ -284,15 +302,19 @@ int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview
   return MOE_OK;
 }
 
-// Internal: small-P logits plus the shared-expert gate row in the same launch.
+// Internal: small-P logits plus the shared-expert gate row (and, if planes != nullptr, the digit
+// planes of x for the integer-dot decode kernels) in the same launch.
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
-                            int P, float* logits, float* out_x, hipStream_t st) {
+                            int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
+                            hipStream_t st) {
   const int E = (int)W->rows, d = (int)W->cols;
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
-  dim3 g((E + 1 + 3) / 4);
-  if (bf) k_router_logits_par<true, 4><<<g, 256, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x);
-  else k_router_logits_par<false, 4><<<g, 256, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x);
+  const int nrows = E + (Wx ? 1 : 0);
+  const int qblocks = planes ? P * ((d / 32 + 63) / 64) : 0;
+  dim3 g(nrows + qblocks);
+  if (bf) k_router_logits_par<true, 4><<<g, 64, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x, nrows, planes, meta);
+  else k_router_logits_par<false, 4><<<g, 64, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x, nrows, planes, meta);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

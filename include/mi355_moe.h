@@ -180,6 +180,12 @@ int moe_set_shared(moe_ctx* ctx, int layer, const moe_wview* gate_proj, const mo
  * batch: y[P][d] = routed experts (top-k, renormalised) + sigmoid-gated shared expert.
  * x, y: f32 [P][d]; y is fully overwritten. */
 int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_stream_t st);
+/* Switches in the spirit of the reference's QWENOX_* opt-outs (src/gpu/parts/40_model.inc:1959-1996):
+ * every fast path is on by default and can be turned off to fall back to the plainer kernel.
+ * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as
+ * three 7-bit digit planes per 32-group, 21 significant bits) instead of the f32 FMA kernels. */
+enum { MOE_OPT_INT_DECODE = 1 };
+int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP
  * events between its stages; moe_profile_read waits for the last one and fills
