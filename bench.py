@@ -1,12 +1,16 @@
 #!/usr/bin/env python3
 """Benchmark of the routed-expert MoE layer on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill|decode|verify|q4k_prefill|q4k_decode|stack]
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+                  [--workload headline|prefill|decode|verify|q4k_prefill|q4k_decode|stack]
 
 One step = one pass of the MoE layer (moe_forward) over one batch of synthetic input that is
 already resident in HBM.  Prints ONE JSON line: whole-layer throughput, the roofline figure of the
 dominant kernel (timed live with HIP events on the launch stream) and the CPU oracle timed on the
 host cores on a bounded sample of the same workload.
+
+`headline` (the default) is the prefill chunk T=16384 as the primary figure, with the decode T=1
+figure of the same layer shape measured in the same run and reported under "decode_T1".
 """
 import argparse
 import json
@@ -17,36 +21,74 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+D, MID, E, K = 3072, 768, 512, 10
+# HBM bytes per launch of the dominant kernel (read + written) at the default shapes, from the
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic.txt (counters
+# cannot be read from inside this process; other shapes report null)
+PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4137.92e6, ("decode", "q4cp", 1): 44.26e6}
+CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="prefill")
-    ap.add_argument("--tokens", type=int, default=0, help="override the batch size of the workload")
-    ap.add_argument("--layers", type=int, default=48, help="stack workload: number of resident layers")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    a = ap.parse_args()
-    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)
-        sys.exit(2)
+def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb):
+    """The CPU restatement of src/ref.cpp Model::moe (OpenMP over rows) on a bounded sample of the
+    same workload, and the GPU result's distance from it on that sample."""
+    import numpy as np
+    import torch
+    from oracle import oracle as O
+    ol = layer.oracle_layer()
+    y = torch.empty((T, D), dtype=torch.float32, device="cuda")
+    if kind == "prefill":
+        # tokens routed to the hottest expert first, then tokens in batch order, in chunks of 256
+        hot = int(np.argmax(cnt))
+        order = np.concatenate([np.where((ids == hot).any(1))[0][:64], np.arange(T)])
+        _, first = np.unique(order, return_index=True)
+        order = order[np.sort(first)]
+        m.forward(0, xs[0], y)
+        yg_all = y.cpu().numpy()
+        xh = xs[0].cpu().numpy()
+        done, cpu_s, err = 0, 0.0, 0.0
+        while cpu_s < CPU_BUDGET_S and done < len(order):
+            toks = order[done:done + 256]
+            t0 = time.perf_counter()
+            yo, _, _ = O.moe_layer(ol, xh[toks])
+            cpu_s += time.perf_counter() - t0
+            err = max(err, float(np.abs(yg_all[toks].astype(np.float64) - yo).max() / np.abs(yo).max()))
+            done += len(toks)
+        out = {"value": round(done / cpu_s, 3), "unit": "tok/s",
+               "sample": f"{done} of the batch's {T} tokens (64 of the hottest expert's first), chunks of 256"}
+    else:
+        done, cpu_s, err, nbytes = 0, 0.0, 0.0, 0
+        while cpu_s < CPU_BUDGET_S and done < 4096:
+            xg = xs[done % len(xs)]
+            xh = xg.cpu().numpy()
+            t0 = time.perf_counter()
+            yo, io, _ = O.moe_layer(ol, xh)
+            cpu_s += time.perf_counter() - t0
+            if done < len(xs):
+                m.forward(0, xg, y)
+                err = max(err, float(np.abs(y.cpu().numpy().astype(np.float64) - yo).max() / np.abs(yo).max()))
+            nbytes += (int(np.unique(io[:, :K]).size) + 1) * eb + E * D * 4 + D * 4 + T * 2 * D * 4
+            done += 1
+        out = {"value": round(nbytes / cpu_s / 1e9, 4), "unit": "GB/s",
+               "sample": f"{done} steps of {T} token(s), same inputs as the GPU steps"}
+    out.update({"cores": O.num_threads(), "kind": "port", "seconds": round(cpu_s, 3),
+                "what": "OpenMP restatement of src/ref.cpp Model::moe (fp64 dot products), weights dequantised row by row",
+                "max_abs_rel_vs_gpu": err})
+    return out
 
+
+def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
     import numpy as np
     import torch
     from gfx1151_engine_amd import capi, workloads as W
     from gfx1151_engine_amd import synth as S
-    capi.lib()
-    assert torch.cuda.is_available(), "bench.py needs the GPU"
-    d, mid, E, k = 3072, 768, 512, 10
-    wl = a.workload
+    d, mid, k = D, MID, K
     fmt = "q4k" if wl.startswith("q4k") else "q4cp"
     kind = wl.replace("q4k_", "")
-    T = a.tokens or {"prefill": 16384 if fmt == "q4cp" else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
-    nlayers = a.layers if kind == "stack" else 1
+    T = tokens or {"prefill": 16384 if fmt == "q4cp" else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
+    nlayers = nlayers_arg if kind == "stack" else 1
 
     layers = [W.DeviceLayer(1000 + l, d, mid, E, k, fmt) for l in range(nlayers)]
     g = torch.Generator(device="cuda")
@@ -75,27 +117,26 @@ def main():
         else:
             m.forward(0, xs[i % len(xs)], y)
 
-    for i in range(a.warmup):
+    for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     # whole-job timing: K steps between two synchronisations, HIP events on the launch stream
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for i in range(a.steps):
-        step(a.warmup + i)
+    for i in range(steps):
+        step(warmup + i)
     e1.record()
     torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
-    ms = e0.elapsed_time(e1) / a.steps
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = e0.elapsed_time(e1) / steps
 
     # per-stage timing (HIP events recorded by the library between its kernels, same stream)
     m.profile(True)
     stage = {}
-    nprof = max(5, min(a.steps, 20))
+    nprof = max(5, min(steps, 20))
     for i in range(nprof):
-        lsel = i % nlayers
-        m.forward(lsel, xs[i % len(xs)], y)
+        m.forward(i % nlayers, xs[i % len(xs)], y)
         for kk, v in m.profile_read().items():
             stage[kk] = stage.get(kk, 0.0) + v / nprof
     m.profile(False)
@@ -107,7 +148,7 @@ def main():
     uniq = int(np.unique(ids).size)
     cnt = np.bincount(ids.reshape(-1), minlength=E)
     pairs = T * k
-    res = {"n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
+    res = {"n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 5),
            "host_ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "data": "synthetic", "stage_ms": {kk: round(v, 5) for kk, v in stage.items()}}
     cfg = {"workload": wl, "tokens": T, "d_model": d, "moe_mid": mid, "experts": E, "topk": k, "shared_experts": 1,
@@ -119,64 +160,73 @@ def main():
         res.update({"metric": "moe_layer_prefill_tokens_per_s", "unit": "tok/s", "value": round(T / (ms * 1e-3), 1),
                     "dtype": "f16",
                     "layer_tflops": round(flop_tok * T / (ms * 1e-3) / 1e12, 2),
+                    "layer_mfma_frac": round(flop_tok * T / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                     "roofline": {"bound": "mfma", "kernel": "k_moe_gemm (gate/up + SwiGLU)",
                                  "achieved": round(up_flop / up_s / 1e12, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": round(up_flop / up_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                                 "traffic": None}})
+                                 "traffic": PMC_TRAFFIC.get((kind, fmt, T))}})
         cfg.update({"hottest_over_mean": round(float(cnt.max() / cnt.mean()), 2), "empty_experts": int((cnt == 0).sum())})
     else:
         # algorithmic bytes of a step: unique experts + shared expert + fp32 router + gate vector + x/y
-        step_bytes = nlayers * ((uniq if kind != "stack" else k) + 1) * eb + nlayers * (E * d * 4 + d * 4 + T * 2 * d * 4)
         if kind == "stack":
             uniq = k
-        gu_bytes = (uniq + 1) * 2 * mid * (eb // (2 * mid + d) if False else 0)  # placeholder, fixed below
-        if fmt == "q4cp":
-            gu_row = d // 2 + S.q4cp_scale_stride(d)
-        else:
-            gu_row = S.q4k_row_bytes(d)
+        step_bytes = nlayers * ((uniq + 1) * eb + E * d * 4 + d * 4 + T * 2 * d * 4)
+        gu_row = d // 2 + S.q4cp_scale_stride(d) if fmt == "q4cp" else S.q4k_row_bytes(d)
         gu_bytes = (uniq + 1) * 2 * mid * gu_row
         up_s = stage["up"] * 1e-3
         res.update({"metric": "moe_layer_decode_hbm_GB_per_s", "unit": "GB/s",
-                    "value": round(step_bytes / (ms * 1e-3) / 1e9, 1), "dtype": "f32",
+                    "value": round(step_bytes / (ms * 1e-3) / 1e9, 1),
+                    "dtype": "i8" if fmt == "q4cp" else "f32",
+                    "hbm_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "tokens_per_s": round(T / (ms * 1e-3), 1),
                     "roofline": {"bound": "hbm", "kernel": "gate/up GEMV + SwiGLU",
                                  "achieved": round(gu_bytes / up_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                 "frac": round(gu_bytes / up_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None}})
+                                 "frac": round(gu_bytes / up_s / 1e9 / HBM_PEAK_GBS, 4),
+                                 "traffic": PMC_TRAFFIC.get((kind, fmt, T))}})
         cfg.update({"unique_experts": uniq, "step_bytes": int(step_bytes)})
     res["config"] = cfg
+    if cpu:
+        res["cpu_baseline"] = cpu_leg(kind, layers[0], xs, ids, cnt, m, T, eb)
+    m.close()
+    return res
 
-    if not a.no_cpu:
-        from oracle import oracle as O
-        ol = layers[0].oracle_layer()
-        if kind == "prefill":
-            nsamp = 32
-            hot = int(np.argmax(cnt))
-            toks = np.concatenate([np.where((ids == hot).any(1))[0][:8], np.arange(nsamp)])[:nsamp]
-            xc = xs[0][torch.from_numpy(toks).cuda()].cpu().numpy()
-        else:
-            nsamp = T
-            xc = xs[0].cpu().numpy()
-        t0 = time.perf_counter()
-        yo, io, wo = O.moe_layer(ol, xc)
-        cpu_s = time.perf_counter() - t0
-        yg = torch.empty((nsamp, d), dtype=torch.float32, device="cuda")
-        m2 = None
-        if kind == "prefill":
-            m.forward(0, xs[0], y)
-            yg = y[torch.from_numpy(toks).cuda()]
-        else:
-            m.forward(0, xs[0], yg)
-        yg = yg.cpu().numpy()
-        err = float(np.abs(yg.astype(np.float64) - yo).max() / np.abs(yo).max())
-        if kind == "prefill":
-            cpu = {"value": round(nsamp / cpu_s, 3), "unit": "tok/s"}
-        else:
-            cb = (int(np.unique(io[:, :k]).size) + 1) * eb + E * d * 4 + d * 4 + T * 2 * d * 4
-            cpu = {"value": round(cb / cpu_s / 1e9, 4), "unit": "GB/s"}
-        cpu.update({"cores": O.num_threads(), "kind": "port", "seconds": round(cpu_s, 3),
-                    "sample": f"{nsamp} tokens of the same batch through the OpenMP restatement of src/ref.cpp Model::moe",
-                    "max_abs_rel_vs_gpu": err})
-        res["cpu_baseline"] = cpu
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="headline")
+    ap.add_argument("--tokens", type=int, default=0, help="override the batch size of the workload")
+    ap.add_argument("--layers", type=int, default=48, help="stack workload: number of resident layers")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 256 MiB device copies (a kernel of known HBM traffic to scale "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from gfx1151_engine_amd import capi
+    capi.lib()  # raises if the HIP library is missing: there is no other path
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    if a.copy_calibration:
+        src = torch.full((1 << 28,), 7, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if a.workload == "headline":
+        res = measure("prefill", a.steps, a.warmup, a.tokens, cpu=not a.no_cpu)
+        torch.cuda.empty_cache()
+        dec = measure("decode", max(a.steps, 64) * 4, max(a.warmup, 8), cpu=not a.no_cpu)
+        res["decode_T1"] = {kk: dec[kk] for kk in ("metric", "value", "unit", "hbm_frac", "ms_per_step", "steps",
+                                                   "stage_ms", "dtype", "roofline", "config", "cpu_baseline")
+                            if kk in dec}
+    else:
+        res = measure(a.workload, a.steps, a.warmup, a.tokens, a.layers, cpu=not a.no_cpu)
     print(json.dumps(res))
 
 

@@ -21,12 +21,6 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-#ifdef EXP_TIMING
-extern __device__ unsigned long long g_dbg[4096];
-#define TSTAMP(i) do { if (threadIdx.x == 0 && blockIdx.x == 800) g_dbg[(UPK ? 2000 : 0) + (i)] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define TSTAMP(i) do {} while (0)
-#endif
 constexpr int NT = 256;        // 4 waves, each 128 pairs x 128 weight rows
 constexpr int BM = 128;        // pairs per tile (4 MFMA row fragments)
 constexpr int BK = 64;         // K per stage
@@ -100,7 +94,6 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
   const float* cbs = (const float*)(S0 + 2 * S_BYTES);
   const int* rowidx = (const int*)(cbs + 16);
-  constexpr bool UPK = UP;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, kept scalar
   const int n = lane & 31, h = lane >> 5;
@@ -258,8 +251,6 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   constexpr int UPM = (16 + NM - 1) / NM;         // dequant units behind each MFMA (steps 0-2)
   constexpr int X0 = NM >= 8 ? NM / 4 : 1;        // step 3: first MFMA slot that dequantises
   constexpr int XPM = (16 + NM - X0 - 1) / (NM - X0);
-
-  TSTAMP(1);
   // loads run two stages ahead of the MFMAs
   issue(0);
   if (nstage > 1) issue(1);
@@ -272,10 +263,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   scale_consts();
 #pragma unroll
   for (int u = 0; u < 16; u++) deq_unit(0, u, b[0]);
-
-  TSTAMP(2);
   for (int s = 0; s < nstage; s++) {
-    TSTAMP(10 + 2 * s);
     Ab = A0 + (s % NBUF) * A_BYTES;
     const bool pf = s + 2 < nstage;            // stage s+2 exists: its loads go out during step 0
     const bool pf_s = pf && ((s + 2) & 3) == 0;
@@ -307,13 +295,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     // last step: a[1], b[1] hold its operands.  Step 0 of stage s+1 is prepared from the next
     // buffer meanwhile, so that buffer must be complete and visible: loads of stage s+1 done
     // (stage s+2's may still fly), then the block barrier.
-    TSTAMP(11 + 2 * s);
-#ifndef EXP_NO_VMWAIT
     wait_loads_except(s + 2);
-#endif
-#ifndef EXP_NO_BARRIER
     __syncthreads();
-#endif
     Ab = A0 + ((s + 1) % NBUF) * A_BYTES;
 #pragma unroll
     for (int i = 0; i < NM; i++) {
@@ -321,7 +304,6 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[1][mf], b[1][nf].v, acc[mf][nf], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
       // (past the last stage this reads stale LDS and the result is never used)
-#ifndef EXP_NO_PF
       if (i == 0) load_codes(s + 1);
       if (i < MF) load_a1(0, i, a[0]);
       if (i == X0) scale_consts();
@@ -330,13 +312,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         for (int k = 0; k < XPM; k++)
           if ((i - X0) * XPM + k < 16) deq_unit(0, (i - X0) * XPM + k, b[0]);
       }
-#endif
       __builtin_amdgcn_sched_barrier(0);
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // no LDS-bound load may outlive the block
-
-  TSTAMP(3);
   // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair).
   // f16 results go through a per-wave LDS patch (the stage buffers are dead by now) so that global
   // stores are 16 bytes per lane and whole rows are contiguous.
@@ -391,22 +370,16 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   }
 }
 
-#ifdef EXP_TIMING
-__device__ unsigned long long g_dbg[4096];
-#endif
-
 template <bool UP, bool F16OUT>
 __global__ void __launch_bounds__(NT, 1)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split) {
-  constexpr bool UPK = UP;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES);
   int* rowidx = (int*)(cbs + 16);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
-  TSTAMP(0);
   // Routed tiles and shared-expert tiles (all full) are dealt out separately, or the XCD that
   // gets the tail of the list would carry every shared tile.
   const int nt = ntiles[0];
@@ -455,7 +428,6 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   else if (mfn == 2) GEMM_GO(2);
   else GEMM_GO(4);
 #undef GEMM_GO
-  TSTAMP(4);
 }
 
 LutDev to_dev(const moe_lutw* p) {
@@ -508,12 +480,6 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
-
-#ifdef EXP_TIMING
-MOE_API int moe_dbg_read(unsigned long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg), sizeof(unsigned long long) * 4096);
-}
-#endif
 
 MOE_API int moe_lut_q4cp_view(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t scale_stride,
                               int e_rows, int up_off, moe_lutw* out) {
