@@ -144,6 +144,19 @@ def test_router_matches_float64_numpy(oracle):
         assert abs(float(ws[t, :k].sum()) - 1.0) < 1e-6 and len(set(ids[t, :k])) == k
 
 
+def test_router_f32_equals_bf16_on_representable_weights(oracle):
+    """f32 router rows (no f32 branch in the reference's matvec) reduce to the bf16 branch, which the
+    reference build pins, when every weight is bf16-representable."""
+    rng = np.random.default_rng(12)
+    T, E, d, k = 3, 24, 96, 5
+    Wb = S.f32_to_bf16_bits((rng.standard_normal((E, d)) * 0.3).astype(np.float32))
+    Wf = (Wb.astype(np.uint32) << 16).view(np.float32)
+    x = rng.standard_normal((T, d)).astype(np.float32)
+    la, ia, wa = oracle.router(oracle.Mat(oracle.F32, Wf, E, d), x, k)
+    lb, ib, wb = oracle.router(oracle.Mat(oracle.BF16, Wb, E, d), x, k)
+    assert (bits(la) == bits(lb)).all() and (ia == ib).all() and (bits(wa) == bits(wb)).all()
+
+
 def test_router_ties_and_special_cases(oracle):
     E, k = 32, 5
     # uniform logits: every probability equal -> lowest indices, equal weights
