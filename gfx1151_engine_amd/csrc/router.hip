@@ -12,95 +12,170 @@ __device__ __forceinline__ float load_w(const void* W, uint64_t i) {
 }
 
 // ---- sequential order: bit-identical to `acc += (double)w*x` for c = 0..d-1 ----
-// Block = 128 tokens x 64 weight rows, thread = 8 x 4 independent fp64 chains; operands are
-// widened to fp64 once, when they are staged in LDS.  The f32*f32 product is exact in fp64, so
-// fma(w, x, acc) equals the reference's multiply-then-add.  Row E (if Wx is given) is the
-// shared-expert gate vector: its logit goes to out_x[t].
-constexpr int RL_T = 128, RL_E = 64, RL_K = 32;
-template <bool BF16>
-__global__ void __launch_bounds__(256) k_router_logits_seq(const void* __restrict__ W,
+// The f32*f32 product is exact in fp64, so a chain of fp64 FMAs over c = 0..d-1 equals the
+// reference's multiply-then-add.  v_mfma_f64_16x16x4_f64 is such a chain: it adds its four k
+// slices to the accumulator one after the other, each with a single FMA rounding (lane group
+// l/16 supplies slice k; checked bit for bit against host fma chains over 3072-long sums with
+// heavy cancellation), so successive MFMAs over ascending c reproduce the CPU sum exactly while
+// the fp64 work runs on the matrix pipe.
+// Block = BT tokens x 128 weight rows, 4 waves as 2 x 2, wave = BT/2 tokens x 64 rows.  Operands
+// are staged in LDS as f32 (k permuted so that one 16-byte read feeds four MFMAs) and widened in
+// registers; the next K slab is fetched into registers while the current one is consumed.
+// D layout: value r of lane l is token 4r + l/16, weight row l%16 of the 16 x 16 tile.
+// The shared-expert gate vector (Wx), if given, is one more plain FMA chain per token in the first
+// column block: its logit goes to out_x[t].  Block ids are dealt so that the column blocks of one
+// token tile run on the same XCD (ids that differ by 8) and share its L2 copy of the activations.
+typedef double double4v __attribute__((ext_vector_type(4)));
+constexpr int RS_E = 128, RS_K = 32, RS_PITCH = 36;
+template <bool BF16, int BT>
+__global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __restrict__ W,
                                                            const float* __restrict__ bias,
                                                            const void* __restrict__ Wx, bool wx_bf16,
                                                            const float* __restrict__ x, int P, int E,
                                                            int d, float* __restrict__ logits,
-                                                           float* __restrict__ out_x) {
-  __shared__ __attribute__((aligned(16))) double Xs[RL_K][RL_T + 2];
-  __shared__ __attribute__((aligned(16))) double Ws[RL_K][RL_E + 2];
-  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
-  const int e0 = blockIdx.x * RL_E, t0 = blockIdx.y * RL_T;
-  const int Etot = E + (Wx ? 1 : 0);
-  double acc[8][4];
-#pragma unroll
-  for (int j = 0; j < 8; j++)
-#pragma unroll
-    for (int i = 0; i < 4; i++) acc[j][i] = 0.0;
+                                                           float* __restrict__ out_x, int ncol, int ntt) {
+  constexpr int MT = BT / 32;                 // 16-token MFMA tiles per wave
+  constexpr int XL = (BT * RS_K / 4) / 256;   // float4 loads per thread and slab (activations)
+  constexpr int WL = (RS_E * RS_K / 4) / 256; // (weights)
+  __shared__ __attribute__((aligned(16))) float Xs[BT][RS_PITCH];
+  __shared__ __attribute__((aligned(16))) float Ws[RS_E][RS_PITCH];
+  __shared__ float Wxs[RS_K];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int li = lane & 15, lg = lane >> 4, wm = wv >> 1, wn = wv & 1;
+  const int b = blockIdx.x, xcd = b & 7, q = b >> 3;
+  const int col = q % ncol, tt = (q / ncol) * 8 + xcd;
+  if (tt >= ntt) return;
+  const int e0 = col * RS_E, t0 = tt * BT;
+  const bool extra = Wx != nullptr && col == 0;
   const bool vec = (d % 4 == 0);
-  for (int c0 = 0; c0 < d; c0 += RL_K) {
-    // stage 128 x 32 activations and 64 x 32 weights (zero outside the matrices)
+
+  auto fetch_x = [&](int c0, float4* v) {
 #pragma unroll
-    for (int it = 0; it < (RL_T * RL_K / 4) / 256; it++) {
-      const int i = tid + it * 256, r = i >> 3, c = (i & 7) * 4;
-      const int t = t0 + r, cc = c0 + c;
-      float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < XL; it++) {
+      const int i = tid + it * 256, r = i >> 3, cc = c0 + (i & 7) * 4;
+      const int t = t0 + r;
+      float4 f = {0.f, 0.f, 0.f, 0.f};
       if (t < P) {
-        if (vec && cc + 3 < d) {
-          const float4 f = *(const float4*)(x + (size_t)t * d + cc);
-          v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
-        } else {
-          for (int q = 0; q < 4; q++) if (cc + q < d) v[q] = x[(size_t)t * d + cc + q];
+        const float* src = x + (size_t)t * d + cc;
+        if (vec && cc + 3 < d) f = *(const float4*)src;
+        else {
+          if (cc < d) f.x = src[0];
+          if (cc + 1 < d) f.y = src[1];
+          if (cc + 2 < d) f.z = src[2];
+          if (cc + 3 < d) f.w = src[3];
         }
       }
-#pragma unroll
-      for (int q = 0; q < 4; q++) Xs[c + q][r] = (double)v[q];
+      v[it] = f;
     }
+  };
+  auto fetch_w = [&](int c0, float4* v) {
 #pragma unroll
-    for (int it = 0; it < (RL_E * RL_K / 4) / 256; it++) {
-      const int i = tid + it * 256, r = i >> 3, c = (i & 7) * 4;
-      const int e = e0 + r, cc = c0 + c;
-      float v[4] = {0.f, 0.f, 0.f, 0.f};
-      if (e < Etot) {
-        const bool ex = e == E;
-        const void* src = ex ? Wx : W;
-        const uint64_t base = ex ? 0 : (uint64_t)e * d;
-        const bool bf = ex ? wx_bf16 : BF16;
-        for (int q = 0; q < 4; q++)
-          if (cc + q < d) v[q] = bf ? bf16_bits_to_f32(((const uint16_t*)src)[base + cc + q]) : ((const float*)src)[base + cc + q];
+    for (int it = 0; it < WL; it++) {
+      const int i = tid + it * 256, r = i >> 3, cc = c0 + (i & 7) * 4;
+      const int e = e0 + r;
+      float4 f = {0.f, 0.f, 0.f, 0.f};
+      if (e < E) {
+        const uint64_t o = (uint64_t)e * d + cc;
+        if (vec && cc + 3 < d) {
+          if (BF16) {
+            const uint2 u = *(const uint2*)((const uint16_t*)W + o);
+            f.x = __uint_as_float(u.x << 16); f.y = __uint_as_float(u.x & 0xffff0000u);
+            f.z = __uint_as_float(u.y << 16); f.w = __uint_as_float(u.y & 0xffff0000u);
+          } else {
+            f = *(const float4*)((const float*)W + o);
+          }
+        } else {
+          if (cc < d) f.x = load_w<BF16>(W, o);
+          if (cc + 1 < d) f.y = load_w<BF16>(W, o + 1);
+          if (cc + 2 < d) f.z = load_w<BF16>(W, o + 2);
+          if (cc + 3 < d) f.w = load_w<BF16>(W, o + 3);
+        }
       }
-#pragma unroll
-      for (int q = 0; q < 4; q++) Ws[c + q][r] = (double)v[q];
+      v[it] = f;
     }
-    __syncthreads();
-#pragma unroll 4
-    for (int c = 0; c < RL_K; c++) {
-      double wv[4], xv[8];
+  };
+  auto fetch_wx = [&](int c0) -> float {
+    const int cc = c0 + tid;
+    if (!extra || tid >= RS_K || cc >= d) return 0.f;
+    return wx_bf16 ? bf16_bits_to_f32(((const uint16_t*)Wx)[cc]) : ((const float*)Wx)[cc];
+  };
+  // slab element k (0..31) of a row sits at [ (k & 3) * 8 + (k >> 2) ]: lane group g reads its
+  // slices k = 4*kk + g for kk = 0..7 as two float4
+  auto stage = [&](float (*dst)[RS_PITCH], const float4* v, int n) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) wv[i] = Ws[c][4 * tx + i];
-#pragma unroll
-      for (int j = 0; j < 8; j++) xv[j] = Xs[c][8 * ty + j];
-#pragma unroll
-      for (int j = 0; j < 8; j++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc[j][i] = fma(wv[i], xv[j], acc[j][i]);
+    for (int it = 0; it < n; it++) {
+      const int i = tid + it * 256, r = i >> 3, m = i & 7;
+      dst[r][m] = v[it].x; dst[r][8 + m] = v[it].y; dst[r][16 + m] = v[it].z; dst[r][24 + m] = v[it].w;
     }
+  };
+
+  double4v acc[MT][4];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = double4v{0.0, 0.0, 0.0, 0.0};
+  double accx = 0.0;
+  const bool do_x = extra && tid < BT;  // this thread also carries token t0 + tid of the gate row
+
+  float4 xr[XL], wr[WL];
+  float wxr;
+  fetch_x(0, xr);
+  fetch_w(0, wr);
+  wxr = fetch_wx(0);
+  for (int c0 = 0; c0 < d; c0 += RS_K) {
+    __syncthreads();  // everybody is done reading the previous slab
+    stage(Xs, xr, XL);
+    stage(Ws, wr, WL);
+    if (tid < RS_K) Wxs[tid] = wxr;
     __syncthreads();
+    if (c0 + RS_K < d) {
+      fetch_x(c0 + RS_K, xr);
+      fetch_w(c0 + RS_K, wr);
+      wxr = fetch_wx(c0 + RS_K);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+      float4 xa[MT], wb[4];
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) xa[mt] = *(const float4*)&Xs[wm * (BT / 2) + 16 * mt + li][lg * 8 + 4 * half];
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++) wb[nt] = *(const float4*)&Ws[wn * 64 + 16 * nt + li][lg * 8 + 4 * half];
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++) {
+        double a[MT], bq[4];
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) a[mt] = (double)(kk == 0 ? xa[mt].x : kk == 1 ? xa[mt].y : kk == 2 ? xa[mt].z : xa[mt].w);
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) bq[nt] = (double)(kk == 0 ? wb[nt].x : kk == 1 ? wb[nt].y : kk == 2 ? wb[nt].z : wb[nt].w);
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+          for (int nt = 0; nt < 4; nt++)
+            acc[mt][nt] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[mt], bq[nt], acc[mt][nt], 0, 0, 0);
+      }
+    }
+    if (do_x) {
+#pragma unroll 8
+      for (int k = 0; k < RS_K; k++) accx = fma((double)Wxs[k], (double)Xs[tid][(k & 3) * 8 + (k >> 2)], accx);
+    }
   }
 #pragma unroll
-  for (int j = 0; j < 8; j++) {
-    const int t = t0 + 8 * ty + j;
-    if (t >= P) continue;
+  for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      const int e = e0 + 4 * tx + i;
-      if (e >= Etot) continue;
-      float v = (float)acc[j][i];
-      if (e == E) {
-        out_x[t] = v;
-      } else {
+    for (int r = 0; r < 4; r++) {
+      const int t = t0 + wm * (BT / 2) + 16 * mt + 4 * r + lg;
+      if (t >= P) continue;
+#pragma unroll
+      for (int nt = 0; nt < 4; nt++) {
+        const int e = e0 + wn * 64 + 16 * nt + li;
+        if (e >= E) continue;
+        float v = (float)acc[mt][nt][r];
         if (bias) v += bias[e];
         logits[(size_t)t * E + e] = v;
       }
     }
   }
+  if (do_x && t0 + tid < P) out_x[t0 + tid] = (float)accx;
 }
 
 // ---- lane-parallel order for small P: one wave (= one block) per weight row, lanes stride the
@@ -264,6 +339,21 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
   if (lane < k) ws[(size_t)tok * id_stride + lane] = (float)((double)mine / wsum);
 }
 
+// Launch of the sequential-order kernel: 128-token tiles when there are enough of them to fill the
+// chip, 64-token tiles otherwise.
+void launch_seq(const void* W, bool bf, const float* bias, const void* wx, bool xbf, const float* x, int P,
+                int E, int d, float* logits, float* out_x, hipStream_t st) {
+  const int ncol = (E + RS_E - 1) / RS_E;
+  const bool big = (int64_t)((P + 127) / 128) * ncol >= 512;
+  const int bt = big ? 128 : 64;
+  const int ntt = (P + bt - 1) / bt;
+  const unsigned grid = (unsigned)(((ntt + 7) / 8) * 8 * ncol);
+#define RS_GO(BF, BT) k_router_logits_seq<BF, BT><<<grid, 256, 0, st>>>(W, bias, wx, xbf, x, P, E, d, logits, out_x, ncol, ntt)
+  if (bf) { if (big) RS_GO(true, 128); else RS_GO(true, 64); }
+  else { if (big) RS_GO(false, 128); else RS_GO(false, 64); }
+#undef RS_GO
+}
+
 }  // namespace
 
 MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float* x, int P,
@@ -281,9 +371,7 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
     if (bf) k_router_logits_par<true, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
     else k_router_logits_par<false, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
   } else {
-    dim3 g((E + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
-    if (bf) k_router_logits_seq<true><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
-    else k_router_logits_seq<false><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr);
+    launch_seq(W->data, bf, bias, nullptr, false, x, P, E, d, logits, nullptr, moe_s(st));
   }
   MOE_LAUNCH_CHECK();
   return MOE_OK;
@@ -295,9 +383,7 @@ int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview
   const int E = (int)W->rows, d = (int)W->cols;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
   const void* wx = Wx ? Wx->data : nullptr;
-  dim3 g((E + (Wx ? 1 : 0) + RL_E - 1) / RL_E, (P + RL_T - 1) / RL_T);
-  if (W->dtype == MOE_DT_BF16) k_router_logits_seq<true><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x);
-  else k_router_logits_seq<false><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x);
+  launch_seq(W->data, W->dtype == MOE_DT_BF16, bias, wx, xbf, x, P, E, d, logits, out_x, st);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
