@@ -200,6 +200,39 @@ def from_layout1(t):
     return t.reshape(*s[:-1], s[-1] // 8, 8)[..., inv].reshape(s)
 
 
+def _q4k_order():
+    o = []
+    for w in range(8):
+        o += [4 * w, 4 * w + 2, 32 + 4 * w, 32 + 4 * w + 2, 4 * w + 1, 4 * w + 3, 32 + 4 * w + 1, 32 + 4 * w + 3]
+    return o
+
+
+Q4K_ORDER = _q4k_order()  # layout 2: position p of a block of 64 holds element Q4K_ORDER[p]
+
+
+def from_layout2(t):
+    """Undo the Q4_K activation order (last dim, blocks of 64) -> natural order."""
+    inv = [Q4K_ORDER.index(e) for e in range(64)]
+    s = t.shape
+    return t.reshape(*s[:-1], s[-1] // 64, 64)[..., inv].reshape(s)
+
+
+def gg_up(gate, up, x16, tokidx, tiles_t, ntiles, mid, npairs):
+    hid = torch.full((npairs, mid), float("nan"), dtype=torch.float16, device=x16.device)
+    check(lib().moe_gg_up(GGML_Q4_K, ptr(gate), ptr(up), ptr(x16), ptr(tokidx), ptr(tiles_t), ptr(ntiles),
+                          tiles_t.shape[0], ptr(hid), mid, x16.shape[1], stream()), "moe_gg_up")
+    return hid
+
+
+def gg_down(down, hid16, tiles_t, ntiles, d, f16=True):
+    npairs = hid16.shape[0]
+    pairs = torch.full((npairs, d), float("nan"), dtype=torch.float16 if f16 else torch.float32,
+                       device=hid16.device)
+    check(lib().moe_gg_down(GGML_Q4_K, ptr(down), ptr(hid16), ptr(tiles_t), ptr(ntiles), tiles_t.shape[0],
+                            ptr(pairs), d, hid16.shape[1], 1 if f16 else 0, stream()), "moe_gg_down")
+    return pairs
+
+
 def lut_up(p, x16, tokidx, tiles_t, ntiles, mid, npairs):
     hid = torch.full((npairs, mid), float("nan"), dtype=torch.float16, device=x16.device)
     check(lib().moe_lut_up(LUT_Q4CP, C.byref(p), ptr(x16), ptr(tokidx), ptr(tiles_t), ptr(ntiles),

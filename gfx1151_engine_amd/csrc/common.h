@@ -57,6 +57,20 @@ __device__ __forceinline__ float wave_max(float v) {
   for (int o = 32; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
   return v;
 }
+// Range guard of the f16 intermediates of the batch path.  hid = silu(g)*u and the down-projection
+// pairs are kept in f16; for weights with large scales (raw Q4_K blocks with big sub-scales) their
+// magnitude, ~ C * mean(x^2) with C a per-layer constant from the weights' row norms, can pass
+// 65504.  The gate/up epilogue multiplies hid by this power of two (<= 1; exactly 1 while the
+// estimate stays below 16), the pairs inherit it and the combine divides it out in f32: exact
+// except for f16 underflow 2^-14 below the typical value.
+__device__ __forceinline__ float moe_hid_scale(float C, float xms) {
+  const float est = C * xms;
+  if (!(est > 16.f)) return 1.f;
+  int e;
+  (void)frexpf(est * 0.0625f, &e);  // est/16 = m * 2^e, m in [0.5, 1)
+  return ldexpf(1.f, -e);
+}
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float silu_f(float x) { return x / (1.f + expf(-x)); }

@@ -18,6 +18,9 @@ struct MoeLayer {
   int sh_gguf_type = 0;
   // every q4cp codebook of the layer is affine (cb[n] = a*n + b): the integer-dot decode kernels apply
   bool experts_affine = false, shared_affine = false;
+  // f16 range guard of the batch path: typical |hid| (and |pair|) per unit mean-square activation,
+  // estimated from sampled weight rows when the weights are registered
+  float c_routed = 0.f, c_shared = 0.f;
 };
 
 // cb[n] == a*n + b for all 16 codes?  Reads the 64-byte codebook back from the device: weight
@@ -31,6 +34,11 @@ static int codebook_affine(const moe_wview* w, bool* out) {
   return MOE_OK;
 }
 
+struct moe_ctx;
+static int magnitude_constant(moe_ctx* c, bool q4k, const moe_wview* gate, uint64_t gate_stride,
+                              const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
+                              float* out);
+
 struct moe_ctx {
   moe_config cfg;
   std::vector<MoeLayer> layers;
@@ -39,6 +47,8 @@ struct moe_ctx {
   int* ids = nullptr;         // [T][id_stride]
   float* ws = nullptr;        // [T][id_stride]
   float* sh_logit = nullptr;  // [T]
+  float* xms = nullptr;       // [T] mean square of each token's activations (batch path)
+  float* sample = nullptr;    // 96 dequantised weight rows (registration-time magnitude estimate)
   float* hid32 = nullptr;     // [min(T,small_max)][k+1][mid] f32 (small-batch path)
   uint32_t *xplanes = nullptr, *hplanes = nullptr;  // integer digit planes of x / hid (decode kernels)
   float2 *xmeta = nullptr, *hmeta = nullptr;
@@ -89,7 +99,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->routing) rc = moe_routing_destroy(c->routing);
   for (hipEvent_t e : c->ev)
     if (e) (void)hipEventDestroy(e);
-  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
+  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16};
   for (void* b : bufs)
     if (b) {
@@ -120,6 +130,8 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   if (e == hipSuccess) e = hipMalloc(&c->ids, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ws, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->sh_logit, (T + 1) * 4);  // + one int the decode kernels may flag
+  if (e == hipSuccess) e = hipMalloc(&c->xms, T * 4);
+  if (e == hipSuccess) e = hipMalloc(&c->sample, (size_t)96 * (cfg->d > cfg->mid ? cfg->d : cfg->mid) * 4);
   const size_t Ts = T < (size_t)c->small_max ? T : (size_t)c->small_max;
   if (e == hipSuccess) e = hipMalloc(&c->hid32, Ts * (size_t)(cfg->topk + 1) * cfg->mid * 4);
   if (e == hipSuccess) e = hipMalloc(&c->xplanes, Ts * moe_qvec_plane_bytes(cfg->d));
@@ -181,6 +193,8 @@ MOE_API int moe_set_experts_q4cp(moe_ctx* c, int layer, const moe_wview* gu, con
   int rc;
   if ((rc = codebook_affine(gu, &a1)) || (rc = codebook_affine(dn, &a2))) return rc;
   L->experts_affine = a1 && a2;
+  if ((rc = magnitude_constant(c, false, gu, (uint64_t)2 * g.mid, gu, (uint64_t)g.mid, dn, g.experts, &L->c_routed)))
+    return rc;
   L->gate_up = *gu;
   L->down = *dn;
   L->has_q4cp = true;
@@ -193,6 +207,14 @@ MOE_API int moe_set_experts_gguf(moe_ctx* c, int layer, const moe_gg_experts* gg
   if (!L || !gg || !gg->gate || !gg->up || !gg->down) return MOE_E_INVALID;
   if (gg->tgu != MOE_GGML_Q4_K || gg->tdn != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
   if (c->cfg.d % 256 || c->cfg.mid % 256) return MOE_E_UNSUPPORTED;
+  {
+    const moe_config& g = c->cfg;
+    moe_wview gv{0, gg->gate, (uint64_t)g.experts * g.mid, (uint64_t)g.d, 0};
+    moe_wview uv{0, gg->up, (uint64_t)g.experts * g.mid, (uint64_t)g.d, 0};
+    moe_wview dv{0, gg->down, (uint64_t)g.experts * g.d, (uint64_t)g.mid, 0};
+    int rc = magnitude_constant(c, true, &gv, (uint64_t)g.mid, &uv, 0, &dv, g.experts, &L->c_routed);
+    if (rc) return rc;
+  }
   L->gg = *gg;
   L->has_gguf = true;
   L->has_q4cp = false;
@@ -220,12 +242,63 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
     if ((rc = codebook_affine(g, &a1)) || (rc = codebook_affine(u, &a2)) || (rc = codebook_affine(dn, &a3))) return rc;
     L->shared_affine = a1 && a2 && a3;
   }
+  {
+    int rc = magnitude_constant(c, sh_gguf_type != 0, g, (uint64_t)cf.mid, u, 0, dn, 1, &L->c_shared);
+    if (rc) return rc;
+  }
   L->sh_gate = *g;
   L->sh_up = *u;
   L->sh_down = *dn;
   L->sh_sg = *sg;
   L->sh_gguf_type = sh_gguf_type;
   L->has_shared = true;
+  return MOE_OK;
+}
+
+// Typical |silu(g)*u| (times the growth through the down projection, if that is > 1) for
+// activations of unit mean square: sigma_gate * sigma_up * max(1, sigma_down), sigma^2 = mean
+// squared row norm over two sampled rows, maximum over up to 16 evenly spaced experts.  Expert e's
+// gate rows start at row e*gate_stride of `gate`, its up rows at e*gate_stride + up_first of `up`
+// (the same fused tensor for hgn, a tensor of its own for GGUF), its down rows at e*down->rows/n.
+// Set-up work: dequantises 6 rows per sampled expert on the device and reads them back.
+static int magnitude_constant(moe_ctx* c, bool q4k, const moe_wview* gate, uint64_t gate_stride,
+                              const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
+                              float* out) {
+  const int ns = n_experts < 16 ? n_experts : 16;
+  const uint64_t d = gate->cols, mid = down->cols, drows = down->rows / (uint64_t)n_experts;
+  const uint64_t pitch = d > mid ? d : mid;
+  auto deq = [&](const moe_wview* w, uint64_t row, float* dst) -> int {
+    if (q4k) return moe_q4k_dequant_rows(w->data + row * (w->cols / 256 * 144), 1, w->cols, dst, nullptr);
+    return moe_q4cp_dequant_rows(w->data, w->rows, w->cols, row, 1, dst, nullptr);
+  };
+  int rc;
+  for (int i = 0; i < ns; i++) {
+    const uint64_t e = (uint64_t)i * n_experts / ns;
+    float* base = c->sample + (size_t)i * 6 * pitch;
+    const uint64_t g0 = e * gate_stride, u0 = e * gate_stride + up_first, d0 = e * drows;
+    if ((rc = deq(gate, g0, base)) || (rc = deq(gate, g0 + mid / 2, base + pitch)) ||
+        (rc = deq(up, u0, base + 2 * pitch)) || (rc = deq(up, u0 + mid / 2, base + 3 * pitch)) ||
+        (rc = deq(down, d0, base + 4 * pitch)) || (rc = deq(down, d0 + drows / 2, base + 5 * pitch)))
+      return rc;
+  }
+  std::vector<float> h((size_t)ns * 6 * pitch);
+  MOE_HIP(hipMemcpy(h.data(), c->sample, h.size() * 4, hipMemcpyDeviceToHost));
+  double best = 0.0;
+  for (int i = 0; i < ns; i++) {
+    double n2[6];
+    for (int r = 0; r < 6; r++) {
+      const float* v = h.data() + ((size_t)i * 6 + r) * pitch;
+      const uint64_t n = r < 4 ? d : mid;
+      double s = 0.0;
+      for (uint64_t j = 0; j < n; j++) s += (double)v[j] * v[j];
+      n2[r] = s;
+    }
+    const double sg = std::sqrt(0.5 * (n2[0] + n2[1])), su = std::sqrt(0.5 * (n2[2] + n2[3])),
+                 sd = std::sqrt(0.5 * (n2[4] + n2[5]));
+    const double cst = sg * su * (sd > 1.0 ? sd : 1.0);
+    if (cst > best) best = cst;
+  }
+  *out = (float)best;
   return MOE_OK;
 }
 
@@ -309,9 +382,15 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     return rc;
   }
   if (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
-  return moe_launch_q4k_gemv(L.gg.gate, L.gg.up, L.gg.down, L.has_shared ? L.sh_gate.data : nullptr,
-                             L.has_shared ? L.sh_up.data : nullptr, L.has_shared ? L.sh_down.data : nullptr,
-                             c->sh_logit, x, c->ids, c->ws, c->hid32, y, P, g.d, g.mid, g.topk, g.id_stride, st);
+  for (int phase = 1; phase <= 2; phase++) {
+    if ((rc = moe_launch_q4k_gemv(phase, L.gg.gate, L.gg.up, L.gg.down, L.has_shared ? L.sh_gate.data : nullptr,
+                                  L.has_shared ? L.sh_up.data : nullptr, L.has_shared ? L.sh_down.data : nullptr,
+                                  c->sh_logit, x, c->ids, c->ws, c->hid32, y, P, g.d, g.mid, g.topk, g.id_stride,
+                                  st)))
+      return rc;
+    prof_mark(c, phase == 1 ? MOE_PROF_UP : MOE_PROF_DOWN, st);
+  }
+  return MOE_OK;
 }
 
 // Batches: expert-sorted permutation, MFMA grouped GEMMs over <=128-pair tiles (the shared expert
@@ -319,13 +398,22 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
 // Returns MOE_E_UNSUPPORTED (before enqueuing anything) for shapes / formats the GEMM does not cover.
 static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
   const moe_config& g = c->cfg;
-  if (!L.has_q4cp) return MOE_E_UNSUPPORTED;
-  if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
-  if (g.d % 128 || g.mid % 128) return MOE_E_UNSUPPORTED;
-  moe_lutw gu, dn, sgu{}, sdn{};
-  moe_lut_q4cp_view(L.gate_up.data, L.gate_up.rows, L.gate_up.cols, L.gate_up.scale_stride, 2 * g.mid, g.mid, &gu);
-  moe_lut_q4cp_view(L.down.data, L.down.rows, L.down.cols, L.down.scale_stride, g.d, 0, &dn);
-  if (L.has_shared) {
+  const bool q4k = L.has_gguf;  // raw GGUF Q4_K blocks (moe_set_experts_gguf admits nothing else)
+  if (L.has_shared && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format per launch
+  if (q4k ? (g.d % 256 || g.mid % 256) : (g.d % 128 || g.mid % 128)) return MOE_E_UNSUPPORTED;
+  moe_lutw gu{}, dn{}, sgu{}, sdn{};
+  if (q4k) {
+    gu.w = L.gg.gate; gu.w_up = L.gg.up; gu.e_rows = g.mid;
+    dn.w = L.gg.down; dn.e_rows = g.d;
+    if (L.has_shared) {
+      sgu.w = L.sh_gate.data; sgu.w_up = L.sh_up.data; sgu.e_rows = g.mid;
+      sdn.w = L.sh_down.data; sdn.e_rows = g.d;
+    }
+  } else {
+    moe_lut_q4cp_view(L.gate_up.data, L.gate_up.rows, L.gate_up.cols, L.gate_up.scale_stride, 2 * g.mid, g.mid, &gu);
+    moe_lut_q4cp_view(L.down.data, L.down.rows, L.down.cols, L.down.scale_stride, g.d, 0, &dn);
+  }
+  if (L.has_shared && !q4k) {
     moe_lutw t;
     moe_lut_q4cp_view(L.sh_gate.data, L.sh_gate.rows, L.sh_gate.cols, L.sh_gate.scale_stride, g.mid, 0, &sgu);
     moe_lut_q4cp_view(L.sh_up.data, L.sh_up.rows, L.sh_up.cols, L.sh_up.scale_stride, g.mid, 0, &t);
@@ -337,8 +425,9 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   int rc;
   c->ev_n = 0;
   prof_mark(c, 0, st);
+  const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
   if ((rc = moe_router_logits_seq(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
-                                  c->sh_logit, st)))
+                                  c->sh_logit, c->xms, st)))
     return rc;
   if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
   prof_mark(c, MOE_PROF_ROUTER, st);
@@ -348,19 +437,19 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const int sh_first = L.has_shared ? P * g.topk : -1;
   if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, sh_first, c->tokidx, st)))
     return rc;
-  if ((rc = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, 1, st))) return rc;
+  if ((rc = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, st))) return rc;
   prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
   if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,
-                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, st)))
+                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, q4k, hs, st)))
     return rc;
   prof_mark(c, MOE_PROF_UP, st);
   if ((rc = moe_launch_gemm_q4cp(false, &dn, L.has_shared ? &sdn : nullptr, g.experts, c->hid16, nullptr,
-                                 c->tiles, c->ntiles, max_tiles, c->pairs16, g.d, g.mid, true, st)))
+                                 c->tiles, c->ntiles, max_tiles, c->pairs16, g.d, g.mid, true, q4k, hs, st)))
     return rc;
   prof_mark(c, MOE_PROF_DOWN, st);
   rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
-                         sh_first, y, P, g.d, g.topk, st);
+                         sh_first, y, P, g.d, g.topk, hs, st);
   prof_mark(c, MOE_PROF_REDUCE, st);
   return rc;
 }

@@ -12,6 +12,15 @@
 // as both sides agree): moe_f32_to_f16(layout 1) and the gate/up epilogue write it.
 // (reference: src/gpu/parts/27_kernels_moe_lut.inc:75-83,110-640,660-821; weights are
 //  w = f16(cb[n] * scale), F32 accumulation over the whole K, as in :16)
+//
+// Q4K = true reads raw GGUF Q4_K super-blocks in place instead (144 B per 256 elements:
+// d, dmin, 12 packed bytes of 6-bit sub-scales / mins, 128 code bytes; src/gguf.h:408-441,
+// src/gpu/parts/26_kernels_moe_gguf.inc:81-485).  One 64-wide K stage is one 32-byte run of code
+// bytes (low nibbles = elements 0..31, high nibbles = elements 32..63 of the stage), so a 32-bit
+// code word unpacks to [4w, 4w+2, 32+4w, 32+4w+2, 4w+1, 4w+3, 32+4w+1, 32+4w+3]: activations are kept
+// in that order (layout 2), and the pairs of one word alternate between the stage's two sub-blocks,
+// each with its own w = (d*sc)*n - dmin*m as one packed f16 FMA.  The 16-byte block header takes
+// the place of q4cp's 8 staged scales (one per row and four stages).
 #include "common.h"
 #include "internal.h"
 
@@ -29,7 +38,7 @@ constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chu
 constexpr int W_BYTES = WROWS * 32;       // 16 KB  [row][32 B]
 constexpr int S_BYTES = WROWS * 16;       //  8 KB  [row][8 scales], refreshed every 4 stages
 constexpr int NBUF = 3;                   // activation / code buffers in flight (loads run two stages ahead)
-constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES + 64 + BM * 4;
+constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES + 64 + BM * 4 + BM * 4;
 
 struct LutDev {
   const uint8_t *w, *w_up, *sc, *sc_up;
@@ -78,6 +87,12 @@ __device__ __forceinline__ half8 deq8_table(uint32_t w, float s, const float* cb
 // position of element e (0..7) inside its interleaved group of 8
 __device__ __forceinline__ int ilv_pos(int e) { return ((e & 3) << 1) | (e >> 2); }
 
+// position of element c (0..63) of a 64-element block in layout 2
+__device__ __forceinline__ int q4k_pos(int c) {
+  const int e = c & 31, w = e >> 2, r = e & 3;
+  return 8 * w + ((r & 1) << 2) + ((c >> 5) << 1) + (r >> 1);
+}
+
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 // 64 lanes x 16 B: global (per-lane address) -> LDS (wave-uniform base, lane l lands at base + 16 l)
 __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
@@ -85,7 +100,7 @@ __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
 }
 
 // MF = live 32-row fragments of the tile (1, 2 or 4); AFFINE = codebook a*n+b.
-template <bool UP, bool F16OUT, int MF, bool AFFINE>
+template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b) {
@@ -94,6 +109,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
   const float* cbs = (const float*)(S0 + 2 * S_BYTES);
   const int* rowidx = (const int*)(cbs + 16);
+  const float* rowscale = (const float*)(rowidx + BM);  // f16 range guard of each pair row (gate/up only)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, kept scalar
   const int n = lane & 31, h = lane >> 5;
@@ -116,8 +132,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       sb0 = L.sc;
       grow = (size_t)e * L.e_rows + r;
     }
-    cw = cb0 + grow * (size_t)(K / 2);
-    sw = sb0 + grow * (size_t)L.sstride;
+    if (Q4K) {
+      cw = cb0 + grow * (size_t)(K / 256 * 144);  // raw row: K/256 super-blocks
+      sw = cw;                                    // block header (d, dmin, packed scales) leads each block
+    } else {
+      cw = cb0 + grow * (size_t)(K / 2);
+      sw = sb0 + grow * (size_t)L.sstride;
+    }
   };
 
   // per-lane global sources of the direct-to-LDS loads (wave-load j of a buffer = LDS bytes [1024 j, +1024))
@@ -151,13 +172,15 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + (A_LOADS * wv + u) * 1024);
     } else if (u < NLOADS) {
       const int i = u - A_LOADS;
-      g2l16(w_src[i] + (size_t)s * 32, W0 + b * W_BYTES + (4 * wv + i) * 1024);
+      const size_t off = Q4K ? (size_t)(s >> 2) * 144 + 16 + (size_t)(s & 3) * 32 : (size_t)s * 32;
+      g2l16(w_src[i] + off, W0 + b * W_BYTES + (4 * wv + i) * 1024);
     } else {
       // 8 scales (16 B) per row for stages s..s+3; at the end of K the window is pulled back inside the row
       const int i = u - NLOADS;
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
-      g2l16(s_src[i] + (size_t)g0 * 2, S0 + ((s >> 2) & 1) * S_BYTES + (2 * wv + i) * 1024);
+      const size_t off = Q4K ? (size_t)(s >> 2) * 144 : (size_t)g0 * 2;
+      g2l16(s_src[i] + off, S0 + ((s >> 2) & 1) * S_BYTES + (2 * wv + i) * 1024);
     }
   };
   auto issue = [&](int s) {
@@ -199,8 +222,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   half8 a[2][MF];
   H8 b[2][4];
   uint4 cw[4];
-  half2v as2[4], bs2[4];
+  constexpr int NS = Q4K ? 2 : 1;  // scale sets per stage (Q4_K: the two sub-blocks of the stage)
+  half2v as2[4][NS], bs2[4][NS];
   float scf[4];
+  uint4 hdr[4];
   const uint8_t* Ab = A0;
   auto load_a1 = [&](int q, int mf, half8* dst) {
     const int m = 32 * mf + n;
@@ -215,15 +240,45 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
     for (int nf = 0; nf < 4; nf++) {
       cw[nf] = *(const uint4*)(Wb + wrow[nf] * 32 + h * 16);
-      scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
+      if (Q4K) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
+      else scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
     }
   };
-  auto scale_consts = [&]() {
+  auto scale_consts = [&](int s) {
+    if (Q4K) {
+      // sub-blocks 2jj and 2jj+1 of the super-block: 6-bit (scale, min) pairs, gguf scale_min_k4
+      const int jj = s & 3;
 #pragma unroll
-    for (int nf = 0; nf < 4; nf++) {
-      const _Float16 as = (_Float16)(cb_a * scf[nf]), bs = (_Float16)(cb_b * scf[nf]);
-      as2[nf] = half2v{as, as};
-      bs2[nf] = half2v{bs, bs};
+      for (int nf = 0; nf < 4; nf++) {
+        const uint4 hd = hdr[nf];
+        union { uint32_t u; half2v h; } dd;
+        dd.u = hd.x;
+        const float d = (float)dd.h.x, dmin = (float)dd.h.y;
+        uint32_t sc0, m0, sc1, m1;
+        if (jj < 2) {
+          const int sh = 16 * jj;
+          sc0 = (hd.y >> sh) & 63; sc1 = (hd.y >> (sh + 8)) & 63;
+          m0 = (hd.z >> sh) & 63; m1 = (hd.z >> (sh + 8)) & 63;
+        } else {
+          const int sh = 16 * (jj - 2);
+          const uint32_t b8 = hd.w >> sh;
+          sc0 = (b8 & 0xf) | (((hd.y >> (sh + 6)) & 3) << 4);
+          m0 = ((b8 >> 4) & 0xf) | (((hd.z >> (sh + 6)) & 3) << 4);
+          sc1 = ((b8 >> 8) & 0xf) | (((hd.y >> (sh + 14)) & 3) << 4);
+          m1 = ((b8 >> 12) & 0xf) | (((hd.z >> (sh + 14)) & 3) << 4);
+        }
+        const _Float16 a0 = (_Float16)(d * (float)sc0), b0 = (_Float16)(-(dmin * (float)m0));
+        const _Float16 a1 = (_Float16)(d * (float)sc1), b1 = (_Float16)(-(dmin * (float)m1));
+        as2[nf][0] = half2v{a0, a0}; bs2[nf][0] = half2v{b0, b0};
+        as2[nf][NS - 1] = half2v{a1, a1}; bs2[nf][NS - 1] = half2v{b1, b1};
+      }
+    } else {
+#pragma unroll
+      for (int nf = 0; nf < 4; nf++) {
+        const _Float16 as = (_Float16)(cb_a * scf[nf]), bs = (_Float16)(cb_b * scf[nf]);
+        as2[nf][0] = half2v{as, as};
+        bs2[nf][0] = half2v{bs, bs};
+      }
     }
   };
   // unit u (0..15) of step q: weight fragment nf = u/4, code pair part = u%4 -> one half2 of b
@@ -232,13 +287,14 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     const uint32_t w = q == 0 ? cw[nf].x : q == 1 ? cw[nf].y : q == 2 ? cw[nf].z : cw[nf].w;
     if (AFFINE) {
       const uint32_t ws = part >= 2 ? w >> 8 : w;
+      const int ss = Q4K ? (part & 1) : 0;  // Q4_K: odd parts are the high nibbles = the stage's second sub-block
       uint32_t t;
       if ((part & 1) == 0) {
         asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(ws), "s"(0x000f000fu), "v"(0x64006400u));
-        dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)1024.f, (_Float16)1024.f}) * as2[nf] + bs2[nf];
+        dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)1024.f, (_Float16)1024.f}) * as2[nf][ss] + bs2[nf][ss];
       } else {
         asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(ws), "s"(0x00f000f0u), "v"(0x54005400u));
-        dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)64.f, (_Float16)64.f}) * as2[nf] + bs2[nf];
+        dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)64.f, (_Float16)64.f}) * as2[nf][ss] + bs2[nf][ss];
       }
     } else {
       half2v hv;
@@ -260,7 +316,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   load_codes(0);
 #pragma unroll
   for (int mf = 0; mf < MF; mf++) load_a1(0, mf, a[0]);
-  scale_consts();
+  scale_consts(0);
 #pragma unroll
   for (int u = 0; u < 16; u++) deq_unit(0, u, b[0]);
   for (int s = 0; s < nstage; s++) {
@@ -306,7 +362,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       // (past the last stage this reads stale LDS and the result is never used)
       if (i == 0) load_codes(s + 1);
       if (i < MF) load_a1(0, i, a[0]);
-      if (i == X0) scale_consts();
+      if (i == X0) scale_consts(s + 1);
       if (i >= X0) {
 #pragma unroll
         for (int k = 0; k < XPM; k++)
@@ -333,9 +389,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
           for (int f = 0; f < 2; f++) {
             const float g = acc[mf][f][r], u = acc[mf][2 + f][r];
-            const float hv = g / (1.f + __expf(-g)) * u;
+            const float hv = g / (1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
             const int c = 32 * f + n;  // hid feeds the down GEMM: interleaved order inside groups of 8
-            *(__half*)(patch + ml * LDP + ((c & ~7) + ilv_pos(c & 7)) * 2) = __float2half(hv);
+            const int pos = Q4K ? q4k_pos(c) : (c & ~7) + ilv_pos(c & 7);
+            *(__half*)(patch + ml * LDP + pos * 2) = __float2half(hv);
           }
         } else {
 #pragma unroll
@@ -370,14 +427,16 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   }
 }
 
-template <bool UP, bool F16OUT>
+template <bool UP, bool F16OUT, bool Q4K>
 __global__ void __launch_bounds__(NT, 1)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
-                const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split) {
+                const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,
+                moe_hscale hs) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES);
   int* rowidx = (int*)(cbs + 16);
+  float* rowscale = (float*)(rowidx + BM);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
   // Routed tiles and shared-expert tiles (all full) are dealt out separately, or the XCD that
@@ -402,27 +461,34 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int e = shared ? 0 : tile.expert;
   const int tid = threadIdx.x, lane = tid & 63;
 
-  // codebook: affine (a*n+b) or table
-  const float c0 = L.cb[0], c1 = L.cb[1];
-  bool aff = true;
-  if (lane < 16) {
-    const float v = L.cb[lane];
-    aff = v == fmaf((float)lane, c1 - c0, c0);
-    if (tid < 16) cbs[lane] = v;
+  // q4cp codebook: affine (a*n+b) or table.  Q4_K has no codebook (w = (d*sc)*n - dmin*m).
+  bool affine = true;
+  float cb_a = 1.f, cb_b = 0.f;
+  if (!Q4K) {
+    const float c0 = L.cb[0], c1 = L.cb[1];
+    bool aff = true;
+    if (lane < 16) {
+      const float v = L.cb[lane];
+      aff = v == fmaf((float)lane, c1 - c0, c0);
+      if (tid < 16) cbs[lane] = v;
+    }
+    affine = __all(aff);
+    cb_a = c1 - c0;
+    cb_b = c0;
   }
-  const bool affine = __all(aff);
-  const float cb_a = c1 - c0, cb_b = c0;
 
   if (tid < BM) {
     const int m = tid < tile.count ? tid : 0;  // rows past the tile read a valid row, never stored
-    rowidx[tid] = tokidx ? tokidx[tile.first + m] : tile.first + m;
+    const int ri = tokidx ? tokidx[tile.first + m] : tile.first + m;
+    rowidx[tid] = ri;
+    if (UP) rowscale[tid] = hs.xms ? moe_hid_scale(shared ? hs.c_shared : hs.c_routed, hs.xms[ri]) : 1.f;
   }
   __syncthreads();
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if (affine) gemm_tile<UP, F16OUT, MF, true>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b);        \
-    else gemm_tile<UP, F16OUT, MF, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b);             \
+    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b); \
+    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b);      \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
@@ -439,7 +505,11 @@ LutDev to_dev(const moe_lutw* p) {
   return d;
 }
 
-bool lut_ok(const moe_lutw* p, bool pair, int k) {
+bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k) {
+  if (q4k) {  // raw Q4_K rows: only the code pointers are used
+    if (!p || !p->w || (pair && !p->w_up) || k < 256 || k % 256) return false;
+    return moe_aligned(p->w, 16) && (!pair || moe_aligned(p->w_up, 16));
+  }
   if (!p || !p->w || !p->sc || !p->cb) return false;
   if (pair && (!p->w_up || !p->sc_up)) return false;
   if (k < 256 || k % 128) return false;
@@ -451,32 +521,44 @@ bool lut_ok(const moe_lutw* p, bool pair, int k) {
 }  // namespace
 
 // Internal: routed + (optional) shared expert in one launch; tile.expert >= n_experts selects Sh.
+// q4k: the views hold raw GGUF Q4_K rows (w / w_up only) instead of q4cp planes.
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
-                         int max_tiles, void* out, int m, int k, bool f16out, hipStream_t st) {
+                         int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
+                         hipStream_t st) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
-  if (!lut_ok(routed, up, k) || (sh && !lut_ok(sh, up, k))) return MOE_E_UNSUPPORTED;
+  if (!lut_ok(routed, up, k, q4k) || (sh && !lut_ok(sh, up, k, q4k))) return MOE_E_UNSUPPORTED;
   if (m < 32 || m % 32) return MOE_E_UNSUPPORTED;
+  if (q4k && up && m % 64) return MOE_E_UNSUPPORTED;  // hid is written in whole 64-element blocks
   if (!moe_aligned(x, 16) || !moe_aligned(out, 4)) return MOE_E_INVALID;
   if (max_tiles == 0) return MOE_OK;
   const int nblk_n = up ? (m + 255) / 256 : (m + 511) / 512;
-  static bool attr_done = false;
-  if (!attr_done) {
-    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
-    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
-    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
-    attr_done = true;
-  }
   // per XCD: ceil(routed/8) + ceil(shared/8) <= max_tiles/8 + 2 tile slots
   const int per_xcd = (max_tiles + 7) / 8 + 1;
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
   LutDev R = to_dev(routed), S = to_dev(sh ? sh : routed);
-  if (up)
-    k_moe_gemm_q4cp<true, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, sh ? 1 : 0);
-  else if (f16out)
-    k_moe_gemm_q4cp<false, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, sh ? 1 : 0);
-  else
-    k_moe_gemm_q4cp<false, false><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, sh ? 1 : 0);
+  const int split = sh ? 1 : 0;
+#define GEMM_LAUNCH(UPK, F16, Q)                                                                              \
+  do {                                                                                                        \
+    static bool attr_done = false;                                                                            \
+    if (!attr_done) {                                                                                         \
+      MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<UPK, F16, Q>,                                  \
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));              \
+      attr_done = true;                                                                                       \
+    }                                                                                                         \
+    k_moe_gemm_q4cp<UPK, F16, Q><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
+                                                               m, k, nblk_n, split, hs);                      \
+  } while (0)
+  if (q4k) {
+    if (up) GEMM_LAUNCH(true, true, true);
+    else if (f16out) GEMM_LAUNCH(false, true, true);
+    else GEMM_LAUNCH(false, false, true);
+  } else {
+    if (up) GEMM_LAUNCH(true, true, false);
+    else if (f16out) GEMM_LAUNCH(false, true, false);
+    else GEMM_LAUNCH(false, false, false);
+  }
+#undef GEMM_LAUNCH
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -499,7 +581,7 @@ MOE_API int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* 
   if (type != MOE_LUT_Q4CP) return MOE_E_UNSUPPORTED;
   if (!tokidx) return MOE_E_INVALID;
   return moe_launch_gemm_q4cp(true, p, nullptr, 1 << 30, (const __half*)x16, tokidx, tiles, ntiles, max_tiles,
-                              hid16, m, k, true, moe_s(st));
+                              hid16, m, k, true, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
 }
 
 MOE_API int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
@@ -507,5 +589,30 @@ MOE_API int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const m
                          moe_stream_t st) {
   if (type != MOE_LUT_Q4CP) return MOE_E_UNSUPPORTED;
   return moe_launch_gemm_q4cp(false, p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
-                              max_tiles, pairs, m, k, f16 != 0, moe_s(st));
+                              max_tiles, pairs, m, k, f16 != 0, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
+}
+
+// moe_gg_up / moe_gg_down: raw GGUF blocks, expert e's rows start at row e * m of each tensor
+MOE_API int moe_gg_up(int type, const uint8_t* gate, const uint8_t* up, const void* x16, const int* tokidx,
+                      const moe_tile* tiles, const int* ntiles, int max_tiles, void* hid16, int m, int k,
+                      moe_stream_t st) {
+  if (type != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
+  if (!tokidx) return MOE_E_INVALID;
+  moe_lutw p{};
+  p.w = gate;
+  p.w_up = up;
+  p.e_rows = m;
+  return moe_launch_gemm_q4cp(true, &p, nullptr, 1 << 30, (const __half*)x16, tokidx, tiles, ntiles, max_tiles,
+                              hid16, m, k, true, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
+}
+
+MOE_API int moe_gg_down(int type, const uint8_t* down, const void* hid16, const moe_tile* tiles,
+                        const int* ntiles, int max_tiles, void* pairs, int m, int k, int f16,
+                        moe_stream_t st) {
+  if (type != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
+  moe_lutw p{};
+  p.w = down;
+  p.e_rows = m;
+  return moe_launch_gemm_q4cp(false, &p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
+                              max_tiles, pairs, m, k, f16 != 0, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
 }

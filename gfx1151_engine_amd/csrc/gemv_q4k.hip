@@ -183,7 +183,8 @@ __global__ void __launch_bounds__(256) k_q4k_gemv_dn(GgArgs A, const float* __re
 }  // namespace
 
 // Internal launcher (shared with the context); shared-expert pointers may be null.
-int moe_launch_q4k_gemv(const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+// phase: 0 = gate/up + down, 1 = gate/up only, 2 = down only (the context times them separately).
+int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
                         const uint8_t* sh_gate, const uint8_t* sh_up, const uint8_t* sh_down,
                         const float* sh_logit, const float* x, const int* ids, const float* ws,
                         float* hid, float* out, int P, int d, int mid, int kpt, int id_stride,
@@ -202,7 +203,7 @@ int moe_launch_q4k_gemv(const uint8_t* gate, const uint8_t* up, const uint8_t* d
   GgArgs A{};
   A.gate = gate; A.up = up; A.down = down;
   A.sh_gate = sh_gate; A.sh_up = sh_up; A.sh_down = sh_down; A.sh_logit = sh_logit;
-  {
+  if (phase != 2) {
     dim3 grid((mid + KG_ROWS - 1) / KG_ROWS, nslots, P);
     const int U = d / 64;
     if (U % 16 == 0) k_q4k_gemv_gu<16><<<grid, 256, (size_t)d * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
@@ -210,7 +211,7 @@ int moe_launch_q4k_gemv(const uint8_t* gate, const uint8_t* up, const uint8_t* d
     else k_q4k_gemv_gu<4><<<grid, 256, (size_t)d * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
     MOE_LAUNCH_CHECK();
   }
-  {
+  if (phase != 1) {
     dim3 grid((d + KD_ROWS - 1) / KD_ROWS, P);
     const size_t lds = (size_t)nslots * mid * 4;
     const int U = mid / 64;
@@ -233,6 +234,6 @@ MOE_API int moe_gg_gemv(int tgu, int tdn, const uint8_t* gate, const uint8_t* up
                         const float* x, const int* ids, const float* ws, float* hid, float* out, int P,
                         int d, int mid, int kpt, int id_stride, moe_stream_t st) {
   if (tgu != MOE_GGML_Q4_K || tdn != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
-  return moe_launch_q4k_gemv(gate, up, down, nullptr, nullptr, nullptr, nullptr, x, ids, ws, hid, out, P, d,
+  return moe_launch_q4k_gemv(0, gate, up, down, nullptr, nullptr, nullptr, nullptr, x, ids, ws, hid, out, P, d,
                              mid, kpt, id_stride, moe_s(st));
 }

@@ -2,6 +2,13 @@
 #pragma once
 #include "common.h"
 
+// f16 range guard of the batch path: per-token mean square of x and the per-class constants
+// (routed experts, shared expert); xms == nullptr switches it off (scale 1).
+struct moe_hscale {
+  const float* xms;
+  float c_routed, c_shared;
+};
+
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             hipStream_t st);
@@ -12,21 +19,23 @@ int moe_launch_gemv_dn(const moe_wview* dn, const moe_wview* sh_down, const floa
                        const float* ey, const float* sg, const float* hid, const int* ids,
                        const float* ws, int id_stride, int kpt, int P, int d, float* out,
                        uint64_t out_stride, hipStream_t st);
-int moe_launch_q4k_gemv(const uint8_t* gate, const uint8_t* up, const uint8_t* down,
+int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
                         const uint8_t* sh_gate, const uint8_t* sh_up, const uint8_t* sh_down,
                         const float* sh_logit, const float* x, const int* ids, const float* ws,
                         float* hid, float* out, int P, int d, int mid, int kpt, int id_stride,
                         hipStream_t st);
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
-                         int max_tiles, void* out, int m, int k, bool f16out, hipStream_t st);
+                         int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
+                         hipStream_t st);
 int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E, int cap, int P,
                             int sh_first, int* tokidx, hipStream_t st);
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
                       const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
-                      hipStream_t st);
+                      moe_hscale hs, hipStream_t st);
 int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
-                          float* logits, float* out_x, hipStream_t st);
+                          float* logits, float* out_x, float* out_xms, hipStream_t st);
+
 size_t moe_qvec_plane_bytes(int K);
 size_t moe_qvec_meta_bytes(int K);
 bool moe_dec_supported(int d, int mid, int nslots);

@@ -29,6 +29,24 @@ __global__ void __launch_bounds__(256) k_f32_to_f16_v8(const float4* __restrict_
   }
 }
 
+// Layout 2 (raw GGUF Q4_K weights): inside every 64 elements, 16-byte chunk w (0..7) holds
+// [4w, 4w+2, 32+4w, 32+4w+2, 4w+1, 4w+3, 32+4w+1, 32+4w+3] - the order in which one 32-bit word of
+// a Q4_K block (bytes 4w..4w+3: low nibbles = elements 4w.., high nibbles = elements 32+4w..)
+// unpacks.
+__global__ void __launch_bounds__(256) k_f32_to_f16_q4k(const float4* __restrict__ x, uint4* __restrict__ y,
+                                                        uint64_t n8) {
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t blk = i >> 3, w = i & 7;
+    const float4 u = x[blk * 16 + w], v = x[blk * 16 + 8 + w];
+    const __half2 a = __floats2half2_rn(u.x, u.z), b = __floats2half2_rn(v.x, v.z);
+    const __half2 c = __floats2half2_rn(u.y, u.w), d = __floats2half2_rn(v.y, v.w);
+    uint4 o;
+    o.x = *(const uint32_t*)&a; o.y = *(const uint32_t*)&b; o.z = *(const uint32_t*)&c; o.w = *(const uint32_t*)&d;
+    y[i] = o;
+  }
+}
+
 // out[t][c] = sum_{s<K} pw[pid_s] * pairs[pid_s][c]  (pid_s = pairids[t*K+s], ascending expert id)
 //            + sigmoid(sg[t]) * ey[t][c]             (ey f32, or row `sh_first + t` of pairs)
 // One thread per 8 consecutive columns (16-byte loads of f16 pairs); grid (ceil(D/8/256), P).
@@ -61,7 +79,8 @@ __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pai
                                                       const float* __restrict__ pw,
                                                       const float* __restrict__ ey,
                                                       const float* __restrict__ sg, int sh_first,
-                                                      float* __restrict__ out, int P, int D, int K) {
+                                                      float* __restrict__ out, int P, int D, int K,
+                                                      moe_hscale hs) {
   __shared__ int ids[KMAX];
   __shared__ float w[KMAX];
   const int t = blockIdx.y;
@@ -83,8 +102,17 @@ __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pai
 #pragma unroll
       for (int i = 0; i < 8; i++) sum[i] += ww * v[i];
     }
+  // pairs of the batch path carry the f16 range-guard factor of their token: divide it out
+  float inv_r = 1.f, inv_s = 1.f;
+  if (hs.xms) {
+    const float ms = hs.xms[t];
+    inv_r = 1.f / moe_hid_scale(hs.c_routed, ms);
+    inv_s = 1.f / moe_hid_scale(hs.c_shared, ms);
+#pragma unroll
+    for (int i = 0; i < 8; i++) sum[i] *= inv_r;
+  }
   if (sg) {
-    const float g = sigmoid_f(sg[t]);
+    const float g = sigmoid_f(sg[t]) * (ey ? 1.f : inv_s);
     float v[8];
     if (ey) Ld8<float>::ld(ey + (size_t)t * D + c, v);
     else Ld8<PT>::ld(pairs + (size_t)(sh_first + t) * D + c, v);
@@ -155,7 +183,7 @@ int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E
 
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
                       const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
-                      hipStream_t st) {
+                      moe_hscale hs, hipStream_t st) {
   if (!pairs || !pairids || !pw || !out) return MOE_E_INVALID;
   if (P < 0 || D < 1 || K < 1) return MOE_E_INVALID;
   if (K > 16 || D % 8) return MOE_E_UNSUPPORTED;
@@ -163,20 +191,22 @@ int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, con
   if (P == 0) return MOE_OK;
   dim3 grid((D / 8 + 127) / 128, P);
   if (pairs_f16)
-    k_reduce_pw_sg<__half, 16><<<grid, 128, 0, st>>>((const __half*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K);
+    k_reduce_pw_sg<__half, 16><<<grid, 128, 0, st>>>((const __half*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs);
   else
-    k_reduce_pw_sg<float, 16><<<grid, 128, 0, st>>>((const float*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K);
+    k_reduce_pw_sg<float, 16><<<grid, 128, 0, st>>>((const float*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
 
 MOE_API int moe_f32_to_f16(const float* x, void* x16, uint64_t n, int layout, moe_stream_t st) {
   if (!x || !x16) return n ? MOE_E_INVALID : MOE_OK;
-  if (n % 8 || !moe_aligned(x, 16) || !moe_aligned(x16, 16) || (layout != 0 && layout != 1)) return MOE_E_INVALID;
+  if (n % 8 || !moe_aligned(x, 16) || !moe_aligned(x16, 16) || layout < 0 || layout > 2) return MOE_E_INVALID;
+  if (layout == 2 && n % 64) return MOE_E_INVALID;
   if (n == 0) return MOE_OK;
   const uint64_t n8 = n / 8;
   const unsigned grid = (unsigned)((n8 + 255) / 256 > 1048576 ? 1048576 : (n8 + 255) / 256);
-  if (layout) k_f32_to_f16_v8<true><<<grid, 256, 0, moe_s(st)>>>((const float4*)x, (uint4*)x16, n8);
+  if (layout == 2) k_f32_to_f16_q4k<<<grid, 256, 0, moe_s(st)>>>((const float4*)x, (uint4*)x16, n8);
+  else if (layout) k_f32_to_f16_v8<true><<<grid, 256, 0, moe_s(st)>>>((const float4*)x, (uint4*)x16, n8);
   else k_f32_to_f16_v8<false><<<grid, 256, 0, moe_s(st)>>>((const float4*)x, (uint4*)x16, n8);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
@@ -186,5 +216,6 @@ MOE_API int moe_reduce_pw_sg(const void* pairs, int pairs_f16, const int* pairid
                              const float* ey, const float* sg, float* out, int P, int D, int K,
                              moe_stream_t st) {
   if ((ey == nullptr) != (sg == nullptr)) return MOE_E_INVALID;
-  return moe_launch_reduce(pairs, pairs_f16 != 0, pairids, pw, ey, sg, -1, out, P, D, K, moe_s(st));
+  return moe_launch_reduce(pairs, pairs_f16 != 0, pairids, pw, ey, sg, -1, out, P, D, K, moe_hscale{nullptr, 0.f, 0.f},
+                           moe_s(st));
 }

@@ -33,7 +33,8 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
                                                            const void* __restrict__ Wx, bool wx_bf16,
                                                            const float* __restrict__ x, int P, int E,
                                                            int d, float* __restrict__ logits,
-                                                           float* __restrict__ out_x, int ncol, int ntt) {
+                                                           float* __restrict__ out_x,
+                                                           float* __restrict__ out_xms, int ncol, int ntt) {
   constexpr int MT = BT / 32;                 // 16-token MFMA tiles per wave
   constexpr int XL = (BT * RS_K / 4) / 256;   // float4 loads per thread and slab (activations)
   constexpr int WL = (RS_E * RS_K / 4) / 256; // (weights)
@@ -47,6 +48,7 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
   if (tt >= ntt) return;
   const int e0 = col * RS_E, t0 = tt * BT;
   const bool extra = Wx != nullptr && col == 0;
+  const bool want_ms = out_xms != nullptr && col == 0;
   const bool vec = (d % 4 == 0);
 
   auto fetch_x = [&](int c0, float4* v) {
@@ -115,7 +117,9 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[i][j] = double4v{0.0, 0.0, 0.0, 0.0};
   double accx = 0.0;
-  const bool do_x = extra && tid < BT;  // this thread also carries token t0 + tid of the gate row
+  float accms = 0.f;
+  const bool do_x = extra && tid < BT;    // this thread also carries token t0 + tid of the gate row
+  const bool do_ms = want_ms && tid < BT;  // ... and that token's sum of squares
 
   float4 xr[XL], wr[WL];
   float wxr;
@@ -158,6 +162,10 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
 #pragma unroll 8
       for (int k = 0; k < RS_K; k++) accx = fma((double)Wxs[k], (double)Xs[tid][(k & 3) * 8 + (k >> 2)], accx);
     }
+    if (do_ms) {
+#pragma unroll 8
+      for (int k = 0; k < RS_K; k++) accms = fmaf(Xs[tid][k], Xs[tid][k], accms);
+    }
   }
 #pragma unroll
   for (int mt = 0; mt < MT; mt++) {
@@ -176,6 +184,7 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
     }
   }
   if (do_x && t0 + tid < P) out_x[t0 + tid] = (float)accx;
+  if (do_ms && t0 + tid < P) out_xms[t0 + tid] = accms / (float)d;
 }
 
 // ---- lane-parallel order for small P: one wave (= one block) per weight row, lanes stride the
@@ -342,13 +351,13 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
 // Launch of the sequential-order kernel: 128-token tiles when there are enough of them to fill the
 // chip, 64-token tiles otherwise.
 void launch_seq(const void* W, bool bf, const float* bias, const void* wx, bool xbf, const float* x, int P,
-                int E, int d, float* logits, float* out_x, hipStream_t st) {
+                int E, int d, float* logits, float* out_x, float* out_xms, hipStream_t st) {
   const int ncol = (E + RS_E - 1) / RS_E;
   const bool big = (int64_t)((P + 127) / 128) * ncol >= 512;
   const int bt = big ? 128 : 64;
   const int ntt = (P + bt - 1) / bt;
   const unsigned grid = (unsigned)(((ntt + 7) / 8) * 8 * ncol);
-#define RS_GO(BF, BT) k_router_logits_seq<BF, BT><<<grid, 256, 0, st>>>(W, bias, wx, xbf, x, P, E, d, logits, out_x, ncol, ntt)
+#define RS_GO(BF, BT) k_router_logits_seq<BF, BT><<<grid, 256, 0, st>>>(W, bias, wx, xbf, x, P, E, d, logits, out_x, out_xms, ncol, ntt)
   if (bf) { if (big) RS_GO(true, 128); else RS_GO(true, 64); }
   else { if (big) RS_GO(false, 128); else RS_GO(false, 64); }
 #undef RS_GO
@@ -371,7 +380,7 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
     if (bf) k_router_logits_par<true, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
     else k_router_logits_par<false, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
   } else {
-    launch_seq(W->data, bf, bias, nullptr, false, x, P, E, d, logits, nullptr, moe_s(st));
+    launch_seq(W->data, bf, bias, nullptr, false, x, P, E, d, logits, nullptr, nullptr, moe_s(st));
   }
   MOE_LAUNCH_CHECK();
   return MOE_OK;
@@ -379,11 +388,11 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
 
 // Internal: sequential-order logits for any P (also used for the one-row shared-expert gate).
 int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
-                          float* logits, float* out_x, hipStream_t st) {
+                          float* logits, float* out_x, float* out_xms, hipStream_t st) {
   const int E = (int)W->rows, d = (int)W->cols;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
   const void* wx = Wx ? Wx->data : nullptr;
-  launch_seq(W->data, W->dtype == MOE_DT_BF16, bias, wx, xbf, x, P, E, d, logits, out_x, st);
+  launch_seq(W->data, W->dtype == MOE_DT_BF16, bias, wx, xbf, x, P, E, d, logits, out_x, out_xms, st);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -134,7 +134,9 @@ int moe_lut_q4cp_view(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_
  * layout 0 = natural order; layout 1 = the order the grouped GEMM reads its f16 activations in:
  * inside every group of 8 consecutive elements, [e0,e4,e1,e5,e2,e6,e3,e7] (matches the order the
  * 4-bit unpack produces, so no shuffle is needed on the weight side).  moe_lut_up expects x16 in
- * layout 1 and writes hid16 in layout 1 for moe_lut_down. */
+ * layout 1 and writes hid16 in layout 1 for moe_lut_down.
+ * layout 2 = the order for raw Q4_K weights (moe_gg_up / moe_gg_down), n % 64 == 0: inside every
+ * 64 elements, 16-byte chunk w = [4w, 4w+2, 32+4w, 32+4w+2, 4w+1, 4w+3, 32+4w+1, 32+4w+3]. */
 int moe_f32_to_f16(const float* x, void* x16, uint64_t n, int layout, moe_stream_t st);
 /* moe_lut_up (27_kernels_moe_lut.inc:660): hid16[pair][m] = f16(silu(gate) * up) for every tile
  * (tiles hold <= 128 pairs); x16: f16 [P][k] (layout 1) gathered through tokidx; m % 32 == 0, k % 128 == 0, k >= 256. */
@@ -146,6 +148,16 @@ int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* tokidx,
 int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
                  const int* ntiles, int max_tiles, void* pairs, int m, int k, int f16,
                  moe_stream_t st);
+/* moe_gg_up / moe_gg_down (src/gpu/parts/26_kernels_moe_gguf.inc:456,473): the same grouped GEMMs
+ * on raw GGUF blocks read in place.  type: ggml type of the tensors (supported: MOE_GGML_Q4_K).
+ * gate / up: ffn_gate_exps / ffn_up_exps [E][m rows][k]; down: ffn_down_exps [E][m rows][k].
+ * x16 / hid16 are f16 in layout 2 (see moe_f32_to_f16); moe_gg_up writes hid16 in layout 2.
+ * k % 256 == 0; m % 64 == 0 (up), m % 32 == 0 (down); tiles hold <= 128 pairs. */
+int moe_gg_up(int type, const uint8_t* gate, const uint8_t* up, const void* x16, const int* tokidx,
+              const moe_tile* tiles, const int* ntiles, int max_tiles, void* hid16, int m, int k,
+              moe_stream_t st);
+int moe_gg_down(int type, const uint8_t* down, const void* hid16, const moe_tile* tiles,
+                const int* ntiles, int max_tiles, void* pairs, int m, int k, int f16, moe_stream_t st);
 /* k_moe_reduce_pw / k_moe_reduce_pw_sg (src/gpu/parts/24_kernels_moe_lt.inc:82,104):
  * out[t] = sum_s pw[pid_s] * pairs[pid_s] in pairids order (+ sigmoid(sg[t]) * ey[t] if given). */
 int moe_reduce_pw_sg(const void* pairs, int pairs_f16, const int* pairids, const float* pw,

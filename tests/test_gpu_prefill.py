@@ -82,6 +82,64 @@ def test_grouped_gemm_stages(capi, oracle, d, mid, E, k, P, cb):
     r.close()
 
 
+@pytest.mark.parametrize("d,mid,E,k,P", [(256, 256, 6, 2, 300), (768, 512, 4, 2, 260), (3072, 768, 6, 3, 200)])
+def test_grouped_gemm_stages_q4k(capi, oracle, d, mid, E, k, P):
+    """moe_gg_up / moe_gg_down on raw Q4_K blocks, against fp64 from the oracle's dequantised weights
+    (f16 weights and activations: per-element error ~2^-11, so 3e-3 of the row maximum is the bound)."""
+    rng = np.random.default_rng(d + P + 1)
+    gate = S.make_q4k(rng, E * mid, d, scale_std=0.0005)
+    up = S.make_q4k(rng, E * mid, d, scale_std=0.0005)
+    dn = S.make_q4k(rng, E * d, mid, scale_std=0.0005)
+    x = rng.standard_normal((P, d), dtype=np.float32)
+    ids, ws = make_routing(rng, P, E - 1, k)
+    ids[:, :k] += 1  # expert 0 empty
+    x16 = capi.f32_to_f16(gpu(x), layout=2)
+    assert (capi.from_layout2(x16).cpu().numpy() == x.astype(np.float16)).all()
+    r = capi.Routing(P * k, E)
+    tokidx, pw, eoff, pairids = r.run(gpu(ids), gpu(ws), k)
+    tiles_t, ntiles = capi.tiles(eoff, 128, P * k)
+    hid = capi.gg_up(gpu(gate), gpu(up), x16, tokidx, tiles_t, ntiles, mid, P * k)
+    pairs = capi.gg_down(gpu(dn), hid, tiles_t, ntiles, d, f16=False)
+    pairs16 = capi.gg_down(gpu(dn), hid, tiles_t, ntiles, d, f16=True)
+    hid, pairs, pairs16 = capi.from_layout2(hid).cpu().numpy(), pairs.cpu().numpy(), pairs16.cpu().numpy()
+    assert not np.isnan(hid).any() and not np.isnan(pairs).any(), "every pair row must be written"
+    tokidx, eoff = tokidx.cpu().numpy(), eoff.cpu().numpy()
+    G = oracle.q4k_rows(gate, E * mid, d).astype(np.float64)
+    U = oracle.q4k_rows(up, E * mid, d).astype(np.float64)
+    DN = oracle.q4k_rows(dn, E * d, mid).astype(np.float64)
+    x64 = x.astype(np.float16).astype(np.float64)
+    for e in range(E):
+        sl = slice(eoff[e], eoff[e + 1])
+        if sl.start == sl.stop:
+            continue
+        xe = x64[tokidx[sl]]
+        g = xe @ G[e * mid:(e + 1) * mid].T
+        u = xe @ U[e * mid:(e + 1) * mid].T
+        h = g / (1 + np.exp(-g)) * u
+        assert np.abs(hid[sl] - h).max() <= 3e-3 * np.abs(h).max(), e
+        pr = hid[sl].astype(np.float64) @ DN[e * d:(e + 1) * d].T
+        assert np.abs(pairs[sl] - pr).max() <= 3e-3 * np.abs(pr).max(), e
+        assert np.abs(pairs16[sl] - pr).max() <= 4e-3 * np.abs(pr).max(), e
+    r.close()
+
+
+@pytest.mark.parametrize("d,mid,E,k,T", [(512, 256, 16, 4, 333), (3072, 768, 32, 10, 300)])
+def test_batch_layer_vs_oracle_q4k(oracle, d, mid, E, k, T):
+    """GGUF Q4_K experts + Q4_K shared expert through the MFMA path."""
+    rng = np.random.default_rng(d * 5 + T)
+    hl = HostLayer(rng, d, mid, E, k, fmt="q4k")
+    x = S.bf16_round(rng.standard_normal((T, d), dtype=np.float32))
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    y = m.forward(0, gpu(x))
+    ids, ws = m.last_routing(T)
+    y, ids = y.cpu().numpy(), ids.cpu().numpy()
+    assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
+    err = max_abs_rel(y, yo)
+    assert err <= TOL_LAYER, err
+    m.close()
+
+
 @pytest.mark.parametrize("d,mid,E,k,T,skew", [(512, 256, 16, 4, 333, False), (3072, 768, 64, 10, 700, True),
                                               (1024, 256, 8, 3, 33, False)])
 def test_batch_layer_vs_oracle(oracle, d, mid, E, k, T, skew):
