@@ -47,6 +47,7 @@ struct moe_ctx {
   int* ids = nullptr;         // [T][id_stride]
   float* ws = nullptr;        // [T][id_stride]
   float* sh_logit = nullptr;  // [T]
+  unsigned* ticket = nullptr; // block counter of the fused small-batch router launch (rests at 0)
   float* xms = nullptr;       // [T] mean square of each token's activations (batch path)
   float* sample = nullptr;    // 96 dequantised weight rows (registration-time magnitude estimate)
   float* hid32 = nullptr;     // [min(T,small_max)][k+1][mid] f32 (small-batch path)
@@ -99,7 +100,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->routing) rc = moe_routing_destroy(c->routing);
   for (hipEvent_t e : c->ev)
     if (e) (void)hipEventDestroy(e);
-  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
+  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16};
   for (void* b : bufs)
     if (b) {
@@ -129,7 +130,9 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   hipError_t e = hipMalloc(&c->logits, T * E * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ids, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ws, T * S * 4);
-  if (e == hipSuccess) e = hipMalloc(&c->sh_logit, (T + 1) * 4);  // + one int the decode kernels may flag
+  if (e == hipSuccess) e = hipMalloc(&c->sh_logit, T * 4);
+  if (e == hipSuccess) e = hipMalloc(&c->ticket, 256);
+  if (e == hipSuccess) e = hipMemset(c->ticket, 0, 256);
   if (e == hipSuccess) e = hipMalloc(&c->xms, T * 4);
   if (e == hipSuccess) e = hipMalloc(&c->sample, (size_t)96 * (cfg->d > cfg->mid ? cfg->d : cfg->mid) * 4);
   const size_t Ts = T < (size_t)c->small_max ? T : (size_t)c->small_max;
@@ -350,19 +353,19 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const int nslots_d = g.topk + (L.has_shared ? 1 : 0);
   const bool use_int = L.has_q4cp && c->int_decode && L.experts_affine && (!L.has_shared || L.shared_affine) &&
                        (!L.has_shared || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
+  bool fused = false;
   if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
-                                    c->logits, c->sh_logit, use_int ? c->xplanes : nullptr, c->xmeta, st)))
+                                    c->logits, c->sh_logit, use_int ? c->xplanes : nullptr, c->xmeta, c->ticket,
+                                    c->ids, c->ws, g.topk, g.id_stride, &fused, st)))
     return rc;
-  if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
+  if (!fused && (rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
   prof_mark(c, MOE_PROF_ROUTER, st);
   if (L.has_q4cp) {
     if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
     if (use_int) {
       // integer-dot kernels: activations as digit planes (made by the logits launch above)
       if ((rc = moe_launch_dec_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
-                                  L.has_shared ? &L.sh_up : nullptr, &L.down,
-                                  L.has_shared ? &L.sh_down : nullptr, (int*)c->sh_logit + c->cfg.max_tokens,
-                                  c->xplanes, c->xmeta, c->ids, g.id_stride,
+                                  L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->ids, g.id_stride,
                                   g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st)))
         return rc;
       prof_mark(c, MOE_PROF_UP, st);

@@ -102,8 +102,6 @@ struct DecW {  // one q4cp tensor's planes
 struct GuArgs2 {
   DecW gu;           // fused gate_up [E*2*mid][d]
   DecW shg, shu;     // shared expert gate / up [mid][d] (codes == nullptr: none)
-  DecW dn, shd;      // down tensors: only touched, so that they sit in L2 / Infinity Cache for k_dec_dn
-  int* sink;         // never written in practice (keeps the touching loads alive)
 };
 
 // grid (mid/32, slots incl. shared, P); block 512.  Wave w: gate rows 4w..4w+3 and the matching up
@@ -111,7 +109,7 @@ struct GuArgs2 {
 // at a time with three 16-byte loads per lane: (row0, group L), (row1, group L), and the tail group
 // of row0 (lanes < 32) or row1 (lanes >= 32); all twelve loads of a wave are in flight together.
 constexpr int GU2_ROWS = 32;
-__global__ void __launch_bounds__(512) k_dec_gu(GuArgs2 A, const uint32_t* __restrict__ xplanes,
+__global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __restrict__ xplanes,
                                                 const float2* __restrict__ xmeta,
                                                 const int* __restrict__ ids, int id_stride, int kpt, int d,
                                                 int mid, uint32_t* __restrict__ hplanes,
@@ -153,24 +151,6 @@ __global__ void __launch_bounds__(512) k_dec_gu(GuArgs2 A, const uint32_t* __res
       st[p] = *(const __half*)(s0 + trow * W.ss + gB * 2);
     }
   }
-  // The down projection only depends on the routing, not on this kernel's result: pull this
-  // block's share (1/gridDim.x) of the slot's down weights towards the chip now, so that the whole
-  // layer's weights stream from HBM in one go and k_dec_dn finds them in L2 / Infinity Cache.
-  uint4 pf[7];
-  {
-    const DecW Wd = shared ? A.shd : A.dn;
-    const size_t cbytes = (size_t)d * (mid / 2), sbytes = (size_t)d * Wd.ss;
-    const uint8_t* cbase = Wd.codes + (shared ? 0 : (size_t)e * cbytes);
-    const uint8_t* sbase = Wd.scales + (shared ? 0 : (size_t)e * sbytes);
-    const size_t cper = cbytes / gridDim.x, sper = sbytes / gridDim.x;  // multiples of 16 for the shapes served
-#pragma unroll
-    for (int i = 0; i < 6; i++) {
-      const size_t off = ((size_t)i * 512 + threadIdx.x) * 16;
-      pf[i] = off + 16 <= cper ? *(const uint4*)(cbase + blockIdx.x * cper + off) : make_uint4(0, 0, 0, 0);
-    }
-    const size_t off = (size_t)threadIdx.x * 16;
-    pf[6] = off + 16 <= sper ? *(const uint4*)(sbase + blockIdx.x * sper + off) : make_uint4(0, 0, 0, 0);
-  }
   const float ga = Wg.cb[1] - Wg.cb[0], gb = Wg.cb[0], ua = Wu.cb[1] - Wu.cb[0], ub = Wu.cb[0];
   XG xa, xb;
   const size_t xbase = (size_t)tok * G;
@@ -202,12 +182,6 @@ __global__ void __launch_bounds__(512) k_dec_gu(GuArgs2 A, const uint32_t* __res
       gs[4 * wv + i] = acc[i];
       us[4 * wv + i] = acc[4 + i];
     }
-  }
-  {
-    uint32_t t = 0;
-#pragma unroll
-    for (int i = 0; i < 7; i++) t |= pf[i].x & pf[i].y & pf[i].z & pf[i].w;
-    if (t == 0xffffffffu && A.sink) A.sink[0] = 1;  // 128 one-bits in a row of codes: not in practice
   }
   __syncthreads();
   // SwiGLU on the block's 32 rows = one group of the down projection's input; quantise it
@@ -334,16 +308,13 @@ int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* p
 }
 
 int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
-                      const moe_wview* dn, const moe_wview* sh_down, int* sink, const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
+                      const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
                       hipStream_t st) {
   GuArgs2 A{};
   A.gu = decw(gu);
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
-  A.dn = decw(dn);
-  A.shd = decw(sh_down);
-  A.sink = sink;
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
   k_dec_gu<<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32);
   MOE_LAUNCH_CHECK();

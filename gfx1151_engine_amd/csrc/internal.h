@@ -11,6 +11,7 @@ struct moe_hscale {
 
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
+                            unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
                             hipStream_t st);
 int moe_launch_gemv_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                        const float* x, uint64_t x_stride, const int* ids, int id_stride, int kpt, int P,
@@ -42,7 +43,7 @@ bool moe_dec_supported(int d, int mid, int nslots);
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
                     hipStream_t st);
 int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
-                      const moe_wview* dn, const moe_wview* sh_down, int* sink, const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
+                      const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
                       hipStream_t st);
 int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,

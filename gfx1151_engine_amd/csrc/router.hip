@@ -4,6 +4,12 @@
 #include "qvec.h"
 
 namespace {
+#ifdef EXP_TS
+__device__ unsigned long long g_ts[16];
+#define TS(i) do { if (threadIdx.x == 0) g_ts[i] = __builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define TS(i) do {} while (0)
+#endif
 
 template <bool BF16>
 __device__ __forceinline__ float load_w(const void* W, uint64_t i) {
@@ -187,78 +193,165 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
   if (do_ms && t0 + tid < P) out_xms[t0 + tid] = accms / (float)d;
 }
 
-// ---- lane-parallel order for small P: one wave (= one block) per weight row, lanes stride the
-// columns, four independent fp64 chains per lane and token, fixed combination order.  The fp64
+// ---- lane-parallel order for small P: one wave per weight row (four rows per block), lanes stride
+// the columns, four independent fp64 chains per lane and token, fixed combination order.  The fp64
 // sum differs from the sequential one only in its last bits, so the f32 logit differs with
 // probability ~1e-8 per value.  Row E (if Wx given) is the shared-expert gate vector: out_x[t] =
 // its logit.  Blocks past the rows (if planes given) turn x into the digit planes of the
 // integer-dot decode kernels, so that work rides along instead of costing a launch.
-template <bool BF16, int TT>
-__global__ void __launch_bounds__(64) k_router_logits_par(const void* __restrict__ W,
-                                                          const float* __restrict__ bias,
-                                                          const void* __restrict__ Wx, bool wx_bf16,
-                                                          const float* __restrict__ x, int P, int E,
-                                                          int d, float* __restrict__ logits,
-                                                          float* __restrict__ out_x, int nrows,
-                                                          uint32_t* __restrict__ planes,
-                                                          float2* __restrict__ meta) {
-  const int lane = threadIdx.x;
-  const int row = blockIdx.x;
-  if (row >= nrows) {
-    const int G = d / 32, gb = (G + 63) / 64;
-    const int q = row - nrows, t = q / gb, g = (q % gb) * 64 + lane;
+// If `counter` is given, the block that finishes last (an atomic ticket per row block, fences at
+// device scope on both sides) runs the softmax / top-k of every token as well and re-arms the
+// counter: one launch instead of two on the latency-bound decode path.
+template <int NPL, bool COH>
+__device__ void topk_block(const float* lg, int* __restrict__ ids_row, float* __restrict__ ws_row, int E, int k);
+
+template <bool BF16, int TT, int NPL>
+__global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W,
+                                                      const float* __restrict__ bias,
+                                                      const void* __restrict__ Wx, bool wx_bf16,
+                                                      const float* __restrict__ x, int P, int E, int d,
+                                                      float* __restrict__ logits, float* __restrict__ out_x,
+                                                      int nrows, uint32_t* __restrict__ planes,
+                                                      float2* __restrict__ meta, unsigned* counter,
+                                                      int* __restrict__ ids, float* __restrict__ ws, int k,
+                                                      int id_stride) {
+  __shared__ int s_last;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int nrb = (nrows + 3) >> 2;
+  if ((int)blockIdx.x >= nrb) {
+    const int G = d / 32, gb = (G + 255) / 256;
+    const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * 256 + threadIdx.x;
     if (t < P && g < G) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
     return;
   }
-  const bool extra = row == E;
-  const void* Wr = extra ? Wx : W;
-  const uint64_t base = extra ? 0 : (uint64_t)row * d;
-  const bool bf = extra ? wx_bf16 : BF16;
-  for (int t0 = 0; t0 < P; t0 += TT) {
-    double acc[TT][4];
+  const int row = blockIdx.x * 4 + wv;
+  if (row < nrows) {
+    const bool extra = row == E;
+    const void* Wr = extra ? Wx : W;
+    const uint64_t base = extra ? 0 : (uint64_t)row * d;
+    const bool bf = extra ? wx_bf16 : BF16;
+    for (int t0 = 0; t0 < P; t0 += TT) {
+      double acc[TT][4];
 #pragma unroll
-    for (int i = 0; i < TT; i++)
+      for (int i = 0; i < TT; i++)
 #pragma unroll
-      for (int q = 0; q < 4; q++) acc[i][q] = 0.0;
-    for (int c = lane * 4; c < d; c += 256) {
-      float w[4];
-      if (bf) {
-        const uint2 u = *(const uint2*)((const uint16_t*)Wr + base + c);
-        w[0] = __uint_as_float(u.x << 16);
-        w[1] = __uint_as_float(u.x & 0xffff0000u);
-        w[2] = __uint_as_float(u.y << 16);
-        w[3] = __uint_as_float(u.y & 0xffff0000u);
-      } else {
-        const float4 f = *(const float4*)((const float*)Wr + base + c);
-        w[0] = f.x; w[1] = f.y; w[2] = f.z; w[3] = f.w;
+        for (int q = 0; q < 4; q++) acc[i][q] = 0.0;
+#pragma unroll 4
+      for (int c = lane * 4; c < d; c += 256) {
+        float w[4];
+        if (bf) {
+          const uint2 u = *(const uint2*)((const uint16_t*)Wr + base + c);
+          w[0] = __uint_as_float(u.x << 16);
+          w[1] = __uint_as_float(u.x & 0xffff0000u);
+          w[2] = __uint_as_float(u.y << 16);
+          w[3] = __uint_as_float(u.y & 0xffff0000u);
+        } else {
+          const float4 f = *(const float4*)((const float*)Wr + base + c);
+          w[0] = f.x; w[1] = f.y; w[2] = f.z; w[3] = f.w;
+        }
+#pragma unroll
+        for (int i = 0; i < TT; i++) {
+          if (t0 + i < P) {
+            const float4 xv = *(const float4*)(x + (size_t)(t0 + i) * d + c);
+            acc[i][0] = fma((double)w[0], (double)xv.x, acc[i][0]);
+            acc[i][1] = fma((double)w[1], (double)xv.y, acc[i][1]);
+            acc[i][2] = fma((double)w[2], (double)xv.z, acc[i][2]);
+            acc[i][3] = fma((double)w[3], (double)xv.w, acc[i][3]);
+          }
+        }
       }
 #pragma unroll
       for (int i = 0; i < TT; i++) {
-        if (t0 + i < P) {
-          const float4 xv = *(const float4*)(x + (size_t)(t0 + i) * d + c);
-          acc[i][0] = fma((double)w[0], (double)xv.x, acc[i][0]);
-          acc[i][1] = fma((double)w[1], (double)xv.y, acc[i][1]);
-          acc[i][2] = fma((double)w[2], (double)xv.z, acc[i][2]);
-          acc[i][3] = fma((double)w[3], (double)xv.w, acc[i][3]);
-        }
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < TT; i++) {
-      const double s = wave_sum((acc[i][0] + acc[i][1]) + (acc[i][2] + acc[i][3]));
-      if (lane == 0 && t0 + i < P) {
-        float v = (float)s;
-        if (extra) out_x[t0 + i] = v;
-        else {
-          if (bias) v += bias[row];
-          logits[(size_t)(t0 + i) * E + row] = v;
+        const double sum = wave_sum((acc[i][0] + acc[i][1]) + (acc[i][2] + acc[i][3]));
+        if (lane == 0 && t0 + i < P) {
+          float v = (float)sum;
+          if (extra) out_x[t0 + i] = v;
+          else {
+            if (bias) v += bias[row];
+            // device-scope store: written through to where every XCD's loads of that scope see it
+            __hip_atomic_store(&logits[(size_t)(t0 + i) * E + row], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
         }
       }
     }
   }
+  if (!counter) return;
+  // the wave's logit stores have completed before its block takes a ticket (no cache-wide
+  // write-back is needed: the stores above and the loads in topk_block are device-scope accesses)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const unsigned ticket = atomicAdd(counter, 1u);
+    s_last = ticket == (unsigned)nrb - 1u;
+  }
+  __syncthreads();
+  if (!s_last) return;
+  TS(0);
+  for (int t = 0; t < P; t++)
+    topk_block<NPL, true>(logits + (size_t)t * E, ids + (size_t)t * id_stride, ws + (size_t)t * id_stride, E, k);
+  if (threadIdx.x == 0) *counter = 0u;  // re-armed for the next launch on the stream
 }
 
 __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+__device__ __forceinline__ uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
+__device__ __forceinline__ uint32_t wave_umax(uint32_t m) {
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true));
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, true));
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x141, 0xf, 0xf, true));
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x140, 0xf, 0xf, true));
+  return umax(umax((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+              umax((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+}
+__device__ __forceinline__ uint32_t wave_umin(uint32_t m) {
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0xB1, 0xf, 0xf, false));
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x4E, 0xf, 0xf, false));
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x141, 0xf, 0xf, false));
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x140, 0xf, 0xf, false));
+  return umin(umin((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+              umin((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+}
+
+// k rounds of arg-max by one wave over keys held NPL per lane (key[j] of lane l = expert l + 64 j;
+// key = probability bits + 1, probabilities are >= 0 so the bit patterns order like unsigned
+// integers; 0 = not a candidate).  Larger probability first, equal probabilities -> lower index.
+// Each lane tracks its own best (value, lowest register holding it); a round is a wave-wide
+// maximum of the values, then a wave-wide minimum of the expert index over the lanes that hold
+// that value, both through DPP row operations and four lane reads.  The selected ids and values
+// stay in registers (lane r keeps round r) and are written once at the end.
+template <int NPL>
+__device__ __forceinline__ void topk_select(uint32_t (&key)[NPL], int lane, int k, int* __restrict__ ids_row,
+                                            float* __restrict__ ws_row) {
+  double wsum = 0.0;
+  float mine = 0.f;
+  int myid = 0;
+  for (int r = 0; r < k; r++) {
+    uint32_t m = key[0];
+    int jm = 0;
+#pragma unroll
+    for (int j = 1; j < NPL; j++) {
+      const bool gt = key[j] > m;  // strict: the lowest register (= lowest expert index) wins a tie
+      m = gt ? key[j] : m;
+      jm = gt ? j : jm;
+    }
+    const uint32_t wm = wave_umax(m);
+    const uint32_t bi = wave_umin(m == wm ? (uint32_t)(64 * jm + lane) : 0xffffffffu);
+    const float bv = __uint_as_float(wm - 1u);
+    wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
+    if (lane == r) {
+      mine = bv;
+      myid = (int)bi;
+    }
+    if ((int)(bi & 63u) == lane) {
+#pragma unroll
+      for (int j = 0; j < NPL; j++)
+        if (j == (int)(bi >> 6)) key[j] = 0u;
+    }
+  }
+  if (lane < k) {
+    ids_row[lane] = myid;
+    ws_row[lane] = (float)((double)mine / wsum);
+  }
+}
 
 // ---- softmax + top-k, one wave per token (E <= 64*NPL) ----
 template <int NPL>
@@ -313,39 +406,85 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
     const int e = lane + 64 * j;
     key[j] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
   }
-  // k rounds of arg-max: larger probability first, equal probabilities -> lower index.  The
-  // maximum goes through DPP row operations + four lane reads (no LDS round trips); the lowest
-  // index holding it is found with ballots: register j holds indices [64j, 64j+63], so the first
-  // register with a hit has the lowest index range and its lowest set lane the lowest index.
-  double wsum = 0.0;
-  float mine = 0.f;  // lane r keeps the r-th selected probability
-  for (int r = 0; r < k; r++) {
-    uint32_t m = key[0];
+  topk_select<NPL>(key, lane, k, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride);
+}
+
+// The same softmax / top-k by one block of 256 threads for one token: the fp64 exps, the costly
+// part, are spread over the block; wave 0 then runs the k selection rounds on the keys in LDS.
+// COH: the logits were written by other blocks of the same launch: read them with device-scope loads.
+template <int NPL, bool COH>
+__device__ void topk_block(const float* lg, int* __restrict__ ids_row, float* __restrict__ ws_row, int E, int k) {
+  constexpr int NPT = NPL / 4;  // values per thread (256 threads, E <= 64*NPL)
+  __shared__ float pb[64 * NPL];
+  __shared__ uint32_t keys[64 * NPL];
+  __shared__ double red[4];
+  __shared__ float redf[4];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  __syncthreads();  // LDS of a previous token is no longer read
+  float v[NPT];
+  float mxf = -INFINITY;
 #pragma unroll
-    for (int j = 1; j < NPL; j++) m = m > key[j] ? m : key[j];
-    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true));
-    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, true));
-    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x141, 0xf, 0xf, true));
-    m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x140, 0xf, 0xf, true));
-    const uint32_t wm = umax(umax((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
-                             umax((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
-    int bi = -1;
-#pragma unroll
-    for (int j = 0; j < NPL; j++) {
-      const unsigned long long hit = __ballot(key[j] == wm);
-      if (bi < 0 && hit) bi = 64 * j + (__ffsll((long long)hit) - 1);
-    }
-    const float bv = __uint_as_float(wm - 1u);
-    wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
-    if (lane == r) mine = bv;
-    if (lane == 0) ids[(size_t)tok * id_stride + r] = bi;
-    if ((bi & 63) == lane) {
-#pragma unroll
-      for (int j = 0; j < NPL; j++)
-        if (j == (bi >> 6)) key[j] = 0u;
-    }
+  for (int j = 0; j < NPT; j++) {
+    const int e = tid + 256 * j;
+    v[j] = -INFINITY;
+    if (e < E) v[j] = COH ? __hip_atomic_load(&lg[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
+    mxf = fmaxf(mxf, v[j]);
   }
-  if (lane < k) ws[(size_t)tok * id_stride + lane] = (float)((double)mine / wsum);
+  TS(1);
+  mxf = wave_max(mxf);
+  if (lane == 0) redf[wv] = mxf;
+  __syncthreads();
+  const double mx = (double)fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
+  TS(2);
+  float p[NPT];
+  bool exact = true;
+  double sloc = 0.0;
+#pragma unroll
+  for (int j = 0; j < NPT; j++) {
+    const int e = tid + 256 * j;
+    p[j] = e < E ? (float)exp((double)v[j] - mx) : 0.f;
+    exact = exact && (p[j] == 0.f || p[j] >= 0x1p-20f);
+    sloc += (double)p[j];
+    pb[e] = p[j];
+  }
+  TS(3);
+  const bool all_exact = __syncthreads_and(exact);
+  double se;
+  if (all_exact) {  // every partial sum is representable: any order gives the reference's fp64 sum
+    sloc = wave_sum(sloc);
+    if (lane == 0) red[wv] = sloc;
+    __syncthreads();
+    se = (red[0] + red[1]) + (red[2] + red[3]);
+  } else {          // very wide logit range: replay the reference's index order on one thread
+    if (tid == 0) {
+      double t = 0.0;
+      for (int e = 0; e < E; e++) t += (double)pb[e];
+      red[0] = t;
+    }
+    __syncthreads();
+    se = red[0];
+  }
+#pragma unroll
+  for (int j = 0; j < NPT; j++) {
+    const int e = tid + 256 * j;
+    keys[e] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
+  }
+  __syncthreads();
+  TS(4);
+  if (wv != 0) return;
+  uint32_t key[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; j++) key[j] = keys[lane + 64 * j];
+  topk_select<NPL>(key, lane, k, ids_row, ws_row);
+  TS(5);
+}
+
+// one block per token (small batches)
+template <int NPL>
+__global__ void __launch_bounds__(256) k_router_topk_block(const float* __restrict__ logits, int* __restrict__ ids,
+                                                           float* __restrict__ ws, int E, int k, int id_stride) {
+  const int t = blockIdx.x;
+  topk_block<NPL, false>(logits + (size_t)t * E, ids + (size_t)t * id_stride, ws + (size_t)t * id_stride, E, k);
 }
 
 // Launch of the sequential-order kernel: 128-token tiles when there are enough of them to fill the
@@ -364,6 +503,9 @@ void launch_seq(const void* W, bool bf, const float* bias, const void* wx, bool 
 }
 
 }  // namespace
+#ifdef EXP_TS
+MOE_API int moe_dbg_ts(unsigned long long* h) { return (int)hipMemcpyFromSymbol(h, HIP_SYMBOL(g_ts), 128); }
+#endif
 
 MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float* x, int P,
                               float* logits, int mode, moe_stream_t st) {
@@ -376,9 +518,9 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool par = mode == 0 && P <= 32 && d % 4 == 0 && moe_aligned(x, 16) && moe_aligned(W->data, 16);
   if (par) {
-    dim3 g(E);
-    if (bf) k_router_logits_par<true, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
-    else k_router_logits_par<false, 4><<<g, 64, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr);
+    dim3 g((E + 3) / 4);
+    if (bf) k_router_small<true, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0);
+    else k_router_small<false, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0);
   } else {
     launch_seq(W->data, bf, bias, nullptr, false, x, P, E, d, logits, nullptr, nullptr, moe_s(st));
   }
@@ -398,18 +540,26 @@ int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview
 }
 
 // Internal: small-P logits plus the shared-expert gate row (and, if planes != nullptr, the digit
-// planes of x for the integer-dot decode kernels) in the same launch.
+// planes of x for the integer-dot decode kernels) in the same launch.  With a counter (device
+// memory holding 0) and P <= 4 the launch also does the softmax / top-k: *fused_topk says so.
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
+                            unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
                             hipStream_t st) {
   const int E = (int)W->rows, d = (int)W->cols;
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
   const int nrows = E + (Wx ? 1 : 0);
-  const int qblocks = planes ? P * ((d / 32 + 63) / 64) : 0;
-  dim3 g(nrows + qblocks);
-  if (bf) k_router_logits_par<true, 4><<<g, 64, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x, nrows, planes, meta);
-  else k_router_logits_par<false, 4><<<g, 64, 0, st>>>(W->data, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x, nrows, planes, meta);
+  const int qblocks = planes ? P * ((d / 32 + 255) / 256) : 0;
+  const bool fuse = counter && ids && ws && P <= 4 && E <= 1024;
+  if (fused_topk) *fused_topk = fuse;
+  unsigned* cn = fuse ? counter : nullptr;
+  dim3 g((nrows + 3) / 4 + qblocks);
+  const void* wx = Wx ? Wx->data : nullptr;
+#define RSM_GO(BF, NPL) k_router_small<BF, 4, NPL><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, cn, ids, ws, k, id_stride)
+  if (E <= 512) { if (bf) RSM_GO(true, 8); else RSM_GO(false, 8); }
+  else { if (bf) RSM_GO(true, 16); else RSM_GO(false, 16); }
+#undef RSM_GO
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -420,6 +570,12 @@ MOE_API int moe_router_topk(const float* logits, int* ids, float* ws, int P, int
   if (P < 0 || E < 1 || k < 1 || k > E || k > 64 || id_stride < k) return MOE_E_INVALID;
   if (E > 1024) return MOE_E_UNSUPPORTED;
   if (P == 0) return MOE_OK;
+  if (P <= 32) {  // few tokens: a block per token, the fp64 exps spread over its threads
+    if (E <= 512) k_router_topk_block<8><<<P, 256, 0, moe_s(st)>>>(logits, ids, ws, E, k, id_stride);
+    else k_router_topk_block<16><<<P, 256, 0, moe_s(st)>>>(logits, ids, ws, E, k, id_stride);
+    MOE_LAUNCH_CHECK();
+    return MOE_OK;
+  }
   dim3 g((P + 3) / 4);
   if (E <= 512) k_router_topk<8><<<g, 256, 0, moe_s(st)>>>(logits, ids, ws, P, E, k, id_stride);
   else k_router_topk<16><<<g, 256, 0, moe_s(st)>>>(logits, ids, ws, P, E, k, id_stride);
