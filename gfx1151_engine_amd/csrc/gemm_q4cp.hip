@@ -30,7 +30,12 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int NT = 256;        // 4 waves, each 128 pairs x 128 weight rows
+#ifndef MOE_GEMM_NF
+#define MOE_GEMM_NF 2
+#endif
+constexpr int NF = MOE_GEMM_NF;          // weight fragments (32 rows) per wave
+constexpr int NW = 16 / NF;               // waves per block
+constexpr int NT = 64 * NW;               // each wave: 128 pairs x 32*NF weight rows
 constexpr int BM = 128;        // pairs per tile (4 MFMA row fragments)
 constexpr int BK = 64;         // K per stage
 constexpr int WROWS = 512;     // weight rows per block (up: 256 gate + 256 up)
@@ -100,10 +105,13 @@ __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
 }
 
 // MF = live 32-row fragments of the tile (1, 2 or 4); AFFINE = codebook a*n+b.
+// NF = weight fragments (32 rows) per wave: the block's 16 fragments are split over NW = 16/NF
+// waves, each wave multiplying all MF pair fragments with its own NF weight fragments.
 template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b) {
+  constexpr int NH = NF / 2;  // gate/up: fragments per half
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
@@ -142,74 +150,87 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   };
 
   // per-lane global sources of the direct-to-LDS loads (wave-load j of a buffer = LDS bytes [1024 j, +1024))
-  // activations: rows 8j..8j+7, lane -> (row 8j + lane/8, slot lane%8 holding chunk slot ^ (row & 7))
-  constexpr int A_LOADS = MF;  // per wave: MF*32 rows / 8 rows per load / 4 waves
+  // activations: rows 8j..8j+7, lane -> (row 8j + lane/8, slot lane%8 holding chunk slot ^ (row & 7)).
+  // The 4*MF row groups are dealt to the waves; with more waves than groups some load a group twice
+  // (same bytes to the same place) so that every wave issues the same number of loads.
+  constexpr int A_GROUPS = 4 * MF;
+  constexpr int A_LOADS = A_GROUPS >= NW ? A_GROUPS / NW : 1;
+  constexpr int W_LOADS = 16 / NW, S_LOADS = 8 / NW;
   const __half* a_src[A_LOADS];
+  int a_grp[A_LOADS];
 #pragma unroll
   for (int i = 0; i < A_LOADS; i++) {
-    const int m = 8 * (A_LOADS * wv + i) + (lane >> 3);
+    a_grp[i] = (A_LOADS * wv + i) % A_GROUPS;
+    const int m = 8 * a_grp[i] + (lane >> 3);
     a_src[i] = x + (size_t)rowidx[m] * K + (((lane & 7) ^ (m & 7)) << 3);
   }
   // codes: rows 32j..32j+31, lane -> (row 32j + lane/2, half lane%2); scales: rows 64j.., lane -> row
-  const uint8_t *w_src[4], *s_src[2];
+  const uint8_t *w_src[W_LOADS], *s_src[S_LOADS];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < W_LOADS; i++) {
     const uint8_t* sw;
-    wrow_ptrs(32 * (4 * wv + i) + (lane >> 1), w_src[i], sw);
+    wrow_ptrs(32 * (W_LOADS * wv + i) + (lane >> 1), w_src[i], sw);
     w_src[i] += (lane & 1) * 16;
   }
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
+  for (int i = 0; i < S_LOADS; i++) {
     const uint8_t* cw;
-    wrow_ptrs(64 * (2 * wv + i) + lane, cw, s_src[i]);
+    wrow_ptrs(64 * (S_LOADS * wv + i) + lane, cw, s_src[i]);
   }
   const int nstage = K / BK, ngroups = K / 32;
-  constexpr int NLOADS = A_LOADS + 4;  // per stage (+2 scale loads on every fourth stage)
-  // one direct-to-LDS load of stage s: u < A_LOADS activations, then 4 code loads, then 2 scale loads
+  constexpr int NLOADS = A_LOADS + W_LOADS;  // per stage (+S_LOADS scale loads on every fourth stage)
+  // one direct-to-LDS load of stage s: u < A_LOADS activations, then the code loads, then the scale loads
   auto issue_unit = [&](int s, int u) {
     const int b = s % NBUF;
     if (u < A_LOADS) {
-      g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + (A_LOADS * wv + u) * 1024);
+      g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + a_grp[u] * 1024);
     } else if (u < NLOADS) {
       const int i = u - A_LOADS;
       const size_t off = Q4K ? (size_t)(s >> 2) * 144 + 16 + (size_t)(s & 3) * 32 : (size_t)s * 32;
-      g2l16(w_src[i] + off, W0 + b * W_BYTES + (4 * wv + i) * 1024);
+      g2l16(w_src[i] + off, W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
     } else {
       // 8 scales (16 B) per row for stages s..s+3; at the end of K the window is pulled back inside the row
       const int i = u - NLOADS;
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
       const size_t off = Q4K ? (size_t)(s >> 2) * 144 : (size_t)g0 * 2;
-      g2l16(s_src[i] + off, S0 + ((s >> 2) & 1) * S_BYTES + (2 * wv + i) * 1024);
+      g2l16(s_src[i] + off, S0 + ((s >> 2) & 1) * S_BYTES + (S_LOADS * wv + i) * 1024);
     }
   };
   auto issue = [&](int s) {
 #pragma unroll
     for (int u = 0; u < NLOADS; u++) issue_unit(s, u);
     if ((s & 3) == 0) {
-      issue_unit(s, NLOADS);
-      issue_unit(s, NLOADS + 1);
+#pragma unroll
+      for (int u = 0; u < S_LOADS; u++) issue_unit(s, NLOADS + u);
     }
   };
   // s_waitcnt vmcnt(N), N = loads allowed to stay in flight (loads retire in order)
   auto wait_loads_except = [&](int s_pending) {  // s_pending: stage whose loads may remain (-1: none)
     if (s_pending < 0 || s_pending >= nstage) __builtin_amdgcn_s_waitcnt(0x0F70);
-    else if ((s_pending & 3) == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (NLOADS + 2));
+    else if ((s_pending & 3) == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (NLOADS + S_LOADS));
     else __builtin_amdgcn_s_waitcnt(0x0F70 | NLOADS);
   };
 
-  floatx16 acc[MF][4];
+  floatx16 acc[MF][NF];
 #pragma unroll
   for (int mf = 0; mf < MF; mf++)
 #pragma unroll
-    for (int nf = 0; nf < 4; nf++)
+    for (int nf = 0; nf < NF; nf++)
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[mf][nf][i] = 0.f;
 
-  // LDS rows of this wave's four weight fragments (up: 2 gate + the 2 matching up fragments)
-  int wrow[4];
+  // LDS rows of this wave's weight fragments (gate/up: NH gate + the NH matching up fragments).
+  // Q4_K gate/up with one fragment per half: hid is written in 64-element blocks whose 16-byte
+  // chunks mix elements c and 32+c, so the fragment takes rows {16q..16q+15} and {32+16q..} of
+  // its 64-row block (q = wave parity): four whole chunks per wave.
+  int wrow[NF];
 #pragma unroll
-  for (int nf = 0; nf < 4; nf++) wrow[nf] = UP ? (nf >> 1) * 256 + 64 * wv + 32 * (nf & 1) + n : 128 * wv + 32 * nf + n;
+  for (int nf = 0; nf < NF; nf++) {
+    if (!UP) wrow[nf] = 32 * NF * wv + 32 * nf + n;
+    else if (Q4K && NH == 1) wrow[nf] = nf * 256 + 64 * (wv >> 1) + 16 * (wv & 1) + (n & 15) + 2 * (n & 16);
+    else wrow[nf] = (nf / NH) * 256 + 32 * NH * wv + 32 * (nf % NH) + n;
+  }
 
   // Software pipeline with a hand-placed instruction order.  Inside a stage (four 16-wide K
   // steps) every MFMA of step q is followed by one "unit" of step q+1's preparation: one
@@ -220,12 +241,12 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // (step 3's operands are already in registers), so the loads of stage s+2 can overwrite it, and
   // step 0 of stage s+1 is prepared from the other buffer while step 3's MFMAs run.
   half8 a[2][MF];
-  H8 b[2][4];
-  uint4 cw[4];
+  H8 b[2][NF];
+  uint4 cw[NF], cw8[NF];  // code words of the stage and the same shifted right by 8 (parts 2, 3)
   constexpr int NS = Q4K ? 2 : 1;  // scale sets per stage (Q4_K: the two sub-blocks of the stage)
-  half2v as2[4][NS], bs2[4][NS];
-  float scf[4];
-  uint4 hdr[4];
+  half2v as2[NF][NS], bs2[NF][NS];
+  float scf[NF];
+  uint4 hdr[NF];
   const uint8_t* Ab = A0;
   auto load_a1 = [&](int q, int mf, half8* dst) {
     const int m = 32 * mf + n;
@@ -238,8 +259,9 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
     const int sidx = 2 * s + h - g0;  // this lane's scale inside the staged 8
 #pragma unroll
-    for (int nf = 0; nf < 4; nf++) {
+    for (int nf = 0; nf < NF; nf++) {
       cw[nf] = *(const uint4*)(Wb + wrow[nf] * 32 + h * 16);
+      if (AFFINE) cw8[nf] = uint4{cw[nf].x >> 8, cw[nf].y >> 8, cw[nf].z >> 8, cw[nf].w >> 8};
       if (Q4K) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
       else scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
     }
@@ -249,7 +271,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       // sub-blocks 2jj and 2jj+1 of the super-block: 6-bit (scale, min) pairs, gguf scale_min_k4
       const int jj = s & 3;
 #pragma unroll
-      for (int nf = 0; nf < 4; nf++) {
+      for (int nf = 0; nf < NF; nf++) {
         const uint4 hd = hdr[nf];
         union { uint32_t u; half2v h; } dd;
         dd.u = hd.x;
@@ -274,19 +296,21 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       }
     } else {
 #pragma unroll
-      for (int nf = 0; nf < 4; nf++) {
+      for (int nf = 0; nf < NF; nf++) {
         const _Float16 as = (_Float16)(cb_a * scf[nf]), bs = (_Float16)(cb_b * scf[nf]);
         as2[nf][0] = half2v{as, as};
         bs2[nf][0] = half2v{bs, bs};
       }
     }
   };
-  // unit u (0..15) of step q: weight fragment nf = u/4, code pair part = u%4 -> one half2 of b
+  // unit u (0..4*NF-1) of step q: weight fragment nf = u/4, code pair part = u%4 -> one half2 of b
+  constexpr int NU = 4 * NF;
   auto deq_unit = [&](int q, int u, H8* dst) {
     const int nf = u >> 2, part = u & 3;
     const uint32_t w = q == 0 ? cw[nf].x : q == 1 ? cw[nf].y : q == 2 ? cw[nf].z : cw[nf].w;
     if (AFFINE) {
-      const uint32_t ws = part >= 2 ? w >> 8 : w;
+      const uint32_t w8 = q == 0 ? cw8[nf].x : q == 1 ? cw8[nf].y : q == 2 ? cw8[nf].z : cw8[nf].w;
+      const uint32_t ws = part >= 2 ? w8 : w;
       const int ss = Q4K ? (part & 1) : 0;  // Q4_K: odd parts are the high nibbles = the stage's second sub-block
       uint32_t t;
       if ((part & 1) == 0) {
@@ -303,10 +327,11 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       dst[nf].h[part] = hv;
     }
   };
-  constexpr int NM = 4 * MF;                      // MFMAs per K step
-  constexpr int UPM = (16 + NM - 1) / NM;         // dequant units behind each MFMA (steps 0-2)
+  constexpr int NM = NF * MF;                     // MFMAs per K step
+  constexpr int UPM = (NU + NM - 1) / NM;         // dequant units behind each MFMA (steps 0-2)
   constexpr int X0 = NM >= 8 ? NM / 4 : 1;        // step 3: first MFMA slot that dequantises
-  constexpr int XPM = (16 + NM - X0 - 1) / (NM - X0);
+  constexpr int XPM = (NU + NM - X0 - 1) / (NM - X0);
+
   // loads run two stages ahead of the MFMAs
   issue(0);
   if (nstage > 1) issue(1);
@@ -318,7 +343,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   for (int mf = 0; mf < MF; mf++) load_a1(0, mf, a[0]);
   scale_consts(0);
 #pragma unroll
-  for (int u = 0; u < 16; u++) deq_unit(0, u, b[0]);
+  for (int u = 0; u < NU; u++) deq_unit(0, u, b[0]);
+
   for (int s = 0; s < nstage; s++) {
     Ab = A0 + (s % NBUF) * A_BYTES;
     const bool pf = s + 2 < nstage;            // stage s+2 exists: its loads go out during step 0
@@ -328,21 +354,21 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       const int cur = q & 1, nxt = cur ^ 1;
 #pragma unroll
       for (int i = 0; i < NM; i++) {
-        const int mf = i >> 2, nf = i & 3;
+        const int mf = i / NF, nf = i % NF;
         acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][mf], b[cur][nf].v, acc[mf][nf], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (i < MF) load_a1(q + 1, i, a[nxt]);
 #pragma unroll
         for (int k = 0; k < UPM; k++)
-          if (i * UPM + k < 16) deq_unit(q + 1, i * UPM + k, b[nxt]);
+          if (i * UPM + k < NU) deq_unit(q + 1, i * UPM + k, b[nxt]);
         if (q == 0) {
           // buffer (s+2)%3 was last read in stage s-1: free since the previous barrier
-          constexpr int LPS = (NLOADS + 2 + NM - 1) / NM;  // loads per MFMA slot
+          constexpr int LPS = (NLOADS + S_LOADS + NM - 1) / NM;  // loads per MFMA slot
 #pragma unroll
           for (int k = 0; k < LPS; k++) {
             const int u = i * LPS + k;
             if (u < NLOADS) { if (pf) issue_unit(s + 2, u); }
-            else if (u < NLOADS + 2) { if (pf_s) issue_unit(s + 2, u); }
+            else if (u < NLOADS + S_LOADS) { if (pf_s) issue_unit(s + 2, u); }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -356,7 +382,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     Ab = A0 + ((s + 1) % NBUF) * A_BYTES;
 #pragma unroll
     for (int i = 0; i < NM; i++) {
-      const int mf = i >> 2, nf = i & 3;
+      const int mf = i / NF, nf = i % NF;
       acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[1][mf], b[1][nf].v, acc[mf][nf], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
       // (past the last stage this reads stale LDS and the result is never used)
@@ -366,18 +392,19 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       if (i >= X0) {
 #pragma unroll
         for (int k = 0; k < XPM; k++)
-          if ((i - X0) * XPM + k < 16) deq_unit(0, (i - X0) * XPM + k, b[0]);
+          if ((i - X0) * XPM + k < NU) deq_unit(0, (i - X0) * XPM + k, b[0]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // no LDS-bound load may outlive the block
+
   // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair).
   // f16 results go through a per-wave LDS patch (the stage buffers are dead by now) so that global
   // stores are 16 bytes per lane and whole rows are contiguous.
-  constexpr int NC = UP ? 64 : 128;          // output columns of this wave
-  constexpr int LDP = NC * 2 + 16;           // padded row pitch of the patch in bytes
-  const int colbase = UP ? nb * 256 + 64 * wv : nb * 512 + 128 * wv;
+  constexpr int NC = UP ? 32 * NH : 32 * NF;  // output columns of this wave
+  constexpr int LDP = NC * 2 + 16;            // padded row pitch of the patch in bytes
+  const int colbase = UP ? nb * 256 + NC * wv : nb * 512 + NC * wv;
   if (UP || F16OUT) {
     uint8_t* patch = smem + wv * (32 * LDP);
 #pragma unroll
@@ -387,27 +414,39 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
         if (UP) {
 #pragma unroll
-          for (int f = 0; f < 2; f++) {
-            const float g = acc[mf][f][r], u = acc[mf][2 + f][r];
+          for (int f = 0; f < NH; f++) {
+            const float g = acc[mf][f][r], u = acc[mf][NH + f][r];
             const float hv = g / (1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
-            const int c = 32 * f + n;  // hid feeds the down GEMM: interleaved order inside groups of 8
-            const int pos = Q4K ? q4k_pos(c) : (c & ~7) + ilv_pos(c & 7);
+            // hid feeds the down GEMM: permuted order inside groups of 8 (q4cp) / blocks of 64 (Q4_K)
+            int pos;
+            if (!Q4K) {
+              const int c = 32 * f + n;
+              pos = (c & ~7) + ilv_pos(c & 7);
+            } else if (NH == 1) {
+              // lane n holds row 16q + (n&15) + 2*(n&16) of the block: chunks 4q..4q+3 -> local 0..31
+              pos = q4k_pos((n & 15) + 2 * (n & 16));
+            } else {
+              pos = q4k_pos(32 * f + n);
+            }
             *(__half*)(patch + ml * LDP + pos * 2) = __float2half(hv);
           }
         } else {
 #pragma unroll
-          for (int nf = 0; nf < 4; nf++)
+          for (int nf = 0; nf < NF; nf++)
             *(__half*)(patch + ml * LDP + (32 * nf + n) * 2) = __float2half(acc[mf][nf][r]);
         }
       }
       // 32 rows x NC columns -> NC/8 16-byte chunks per row
       constexpr int CPR = NC / 8;
+      constexpr int ITS = (32 * CPR + 63) / 64;
 #pragma unroll
-      for (int it = 0; it < (32 * CPR) / 64; it++) {
+      for (int it = 0; it < ITS; it++) {
         const int c = it * 64 + lane, ml = c / CPR, c8 = c % CPR;
-        const uint4 v = *(const uint4*)(patch + ml * LDP + c8 * 16);
-        const int m = 32 * mf + ml, col = colbase + c8 * 8;
-        if (m < tile.count && col < M) *(uint4*)((__half*)out + (size_t)(tile.first + m) * M + col) = v;
+        if (c < 32 * CPR) {
+          const uint4 v = *(const uint4*)(patch + ml * LDP + c8 * 16);
+          const int m = 32 * mf + ml, col = colbase + c8 * 8;
+          if (m < tile.count && col < M) *(uint4*)((__half*)out + (size_t)(tile.first + m) * M + col) = v;
+        }
       }
     }
   } else {
@@ -418,7 +457,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         const int m = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
         if (m >= tile.count) continue;
 #pragma unroll
-        for (int nf = 0; nf < 4; nf++) {
+        for (int nf = 0; nf < NF; nf++) {
           const int col = colbase + 32 * nf + n;
           if (col < M) ((float*)out)[(size_t)(tile.first + m) * M + col] = acc[mf][nf][r];
         }
@@ -428,7 +467,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 }
 
 template <bool UP, bool F16OUT, bool Q4K>
-__global__ void __launch_bounds__(NT, 1)
+__global__ void __launch_bounds__(NT, NW / 4)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,

@@ -4,12 +4,6 @@
 #include "qvec.h"
 
 namespace {
-#ifdef EXP_TS
-__device__ unsigned long long g_ts[16];
-#define TS(i) do { if (threadIdx.x == 0) g_ts[i] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define TS(i) do {} while (0)
-#endif
 
 template <bool BF16>
 __device__ __forceinline__ float load_w(const void* W, uint64_t i) {
@@ -286,7 +280,6 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
   }
   __syncthreads();
   if (!s_last) return;
-  TS(0);
   for (int t = 0; t < P; t++)
     topk_block<NPL, true>(logits + (size_t)t * E, ids + (size_t)t * id_stride, ws + (size_t)t * id_stride, E, k);
   if (threadIdx.x == 0) *counter = 0u;  // re-armed for the next launch on the stream
@@ -430,12 +423,10 @@ __device__ void topk_block(const float* lg, int* __restrict__ ids_row, float* __
     if (e < E) v[j] = COH ? __hip_atomic_load(&lg[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
     mxf = fmaxf(mxf, v[j]);
   }
-  TS(1);
   mxf = wave_max(mxf);
   if (lane == 0) redf[wv] = mxf;
   __syncthreads();
   const double mx = (double)fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
-  TS(2);
   float p[NPT];
   bool exact = true;
   double sloc = 0.0;
@@ -447,7 +438,6 @@ __device__ void topk_block(const float* lg, int* __restrict__ ids_row, float* __
     sloc += (double)p[j];
     pb[e] = p[j];
   }
-  TS(3);
   const bool all_exact = __syncthreads_and(exact);
   double se;
   if (all_exact) {  // every partial sum is representable: any order gives the reference's fp64 sum
@@ -470,13 +460,11 @@ __device__ void topk_block(const float* lg, int* __restrict__ ids_row, float* __
     keys[e] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
   }
   __syncthreads();
-  TS(4);
   if (wv != 0) return;
   uint32_t key[NPL];
 #pragma unroll
   for (int j = 0; j < NPL; j++) key[j] = keys[lane + 64 * j];
   topk_select<NPL>(key, lane, k, ids_row, ws_row);
-  TS(5);
 }
 
 // one block per token (small batches)
@@ -503,9 +491,6 @@ void launch_seq(const void* W, bool bf, const float* bias, const void* wx, bool 
 }
 
 }  // namespace
-#ifdef EXP_TS
-MOE_API int moe_dbg_ts(unsigned long long* h) { return (int)hipMemcpyFromSymbol(h, HIP_SYMBOL(g_ts), 128); }
-#endif
 
 MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float* x, int P,
                               float* logits, int mode, moe_stream_t st) {
