@@ -353,9 +353,12 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const int nslots_d = g.topk + (L.has_shared ? 1 : 0);
   const bool use_int = L.has_q4cp && c->int_decode && L.experts_affine && (!L.has_shared || L.shared_affine) &&
                        (!L.has_shared || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
+  const bool use_int4k = L.has_gguf && c->int_decode && (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K) &&
+                         moe_dec4k_supported(g.d, g.mid, nslots_d);
   bool fused = false;
   if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
-                                    c->logits, c->sh_logit, use_int ? c->xplanes : nullptr, c->xmeta, c->ticket,
+                                    c->logits, c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
+                                    use_int4k, c->ticket,
                                     c->ids, c->ws, g.topk, g.id_stride, &fused, st)))
     return rc;
   if (!fused && (rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
@@ -385,6 +388,17 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     return rc;
   }
   if (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
+  if (use_int4k) {
+    if ((rc = moe_launch_dec4k_gu(L.gg.gate, L.gg.up, L.has_shared ? L.sh_gate.data : nullptr,
+                                  L.has_shared ? L.sh_up.data : nullptr, c->xplanes, c->xmeta, c->ids, g.id_stride,
+                                  g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, st)))
+      return rc;
+    prof_mark(c, MOE_PROF_UP, st);
+    rc = moe_launch_dec4k_dn(L.gg.down, L.has_shared ? L.sh_down.data : nullptr, c->sh_logit, c->hplanes, c->hmeta,
+                             c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, y, (uint64_t)g.d, st);
+    prof_mark(c, MOE_PROF_DOWN, st);
+    return rc;
+  }
   for (int phase = 1; phase <= 2; phase++) {
     if ((rc = moe_launch_q4k_gemv(phase, L.gg.gate, L.gg.up, L.gg.down, L.has_shared ? L.sh_gate.data : nullptr,
                                   L.has_shared ? L.sh_up.data : nullptr, L.has_shared ? L.sh_down.data : nullptr,

@@ -1,0 +1,267 @@
+// Decode (T <= 32) on raw GGUF Q4_K blocks read in place, integer dot products: the Q4_K twin of
+// the q4cp decode kernels.  Unit of work = one 32-byte run of code bytes = 64 weights = two
+// 32-element sub-blocks (low nibbles / high nibbles), each with its own 6-bit scale and min:
+//   sum_k w_k x_k = d * (sc0 * qA * VA + sc1 * qB * VB) - dmin * (m0 * qA * SA + m1 * qB * SB)
+// with V = integer dot product of the codes with the activation group's three 7-bit digit planes
+// (natural element order) and q * S = the group's quantised sum.  A lane owns one unit of a row;
+// rows of 3072 are 48 units (lanes 48..63 idle: the kernels are bandwidth-bound), rows of 768 are
+// 12 units (four slots per wave).
+// (reference: src/gpu/parts/26_kernels_moe_gguf.inc:527-568,693-756,893-939; src/gguf.h:328-336,408-441)
+#include "common.h"
+#include "internal.h"
+#include "qvec.h"
+
+namespace {
+
+__device__ __forceinline__ float dpp_add_row(float v) {  // sum over each row of 16 lanes, in every lane
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));
+  return v;
+}
+__device__ __forceinline__ float dpp_max_row(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true)));
+  return v;
+}
+__device__ __forceinline__ float sum64(float v) {
+  v = dpp_add_row(v);
+  v += __shfl_xor(v, 16, 64);
+  return v + __shfl_xor(v, 32, 64);
+}
+
+// activation planes of one unit: two groups (A = low nibbles, B = high nibbles)
+struct XU {
+  uint32_t a[3][8], b[3][8];
+  float qa, qsa, qb, qsb;
+};
+__device__ __forceinline__ void load_xu(XU& x, const uint32_t* planes, const float2* meta, size_t g0) {
+  const uint4* s = (const uint4*)(planes + g0 * QV_GROUP_DW);
+#pragma unroll
+  for (int p = 0; p < 3; p++) {
+    const uint4 a0 = s[2 * p], a1 = s[2 * p + 1], b0 = s[6 + 2 * p], b1 = s[6 + 2 * p + 1];
+    x.a[p][0] = a0.x; x.a[p][1] = a0.y; x.a[p][2] = a0.z; x.a[p][3] = a0.w;
+    x.a[p][4] = a1.x; x.a[p][5] = a1.y; x.a[p][6] = a1.z; x.a[p][7] = a1.w;
+    x.b[p][0] = b0.x; x.b[p][1] = b0.y; x.b[p][2] = b0.z; x.b[p][3] = b0.w;
+    x.b[p][4] = b1.x; x.b[p][5] = b1.y; x.b[p][6] = b1.z; x.b[p][7] = b1.w;
+  }
+  const float2 ma = meta[g0], mb = meta[g0 + 1];
+  x.qa = ma.x; x.qsa = ma.y; x.qb = mb.x; x.qsb = mb.y;
+}
+
+// gguf scale_min_k4 for sub-blocks 2jj and 2jj+1 of a super-block whose header words are hd
+// (hd.x = d | dmin << 16, hd.y/z/w = the 12 packed bytes); jj differs per lane: both forms, then select
+__device__ __forceinline__ void k4_pair(const uint4 hd, int jj, float& a0, float& b0, float& a1, float& b1) {
+  union { uint32_t u; __half2 h; } dd;
+  dd.u = hd.x;
+  const float d = __low2float(dd.h), dmin = __high2float(dd.h);
+  const int shl = 16 * (jj & 1);
+  const uint32_t ylo = hd.y >> shl, zlo = hd.z >> shl, wlo = hd.w >> shl;
+  // jj < 2
+  const uint32_t sc0a = ylo & 63, sc1a = (ylo >> 8) & 63, m0a = zlo & 63, m1a = (zlo >> 8) & 63;
+  // jj >= 2
+  const uint32_t sc0b = (wlo & 0xf) | (((ylo >> 6) & 3) << 4), m0b = ((wlo >> 4) & 0xf) | (((zlo >> 6) & 3) << 4);
+  const uint32_t sc1b = ((wlo >> 8) & 0xf) | (((ylo >> 14) & 3) << 4), m1b = ((wlo >> 12) & 0xf) | (((zlo >> 14) & 3) << 4);
+  const bool lo = jj < 2;
+  a0 = d * (float)(lo ? sc0a : sc0b);
+  a1 = d * (float)(lo ? sc1a : sc1b);
+  b0 = dmin * (float)(lo ? m0a : m0b);
+  b1 = dmin * (float)(lo ? m1a : m1b);
+}
+
+// one unit of one row: c0, c1 = its 32 code bytes, hd = the super-block header
+__device__ __forceinline__ float unit_dot(const uint4 c0, const uint4 c1, const uint4 hd, int jj, const XU& x) {
+  const uint32_t w[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+  int a0 = 0, a1 = 0, a2 = 0, b0 = 0, b1 = 0, b2 = 0;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int lo = (int)(w[i] & 0x0f0f0f0fu), hi = (int)((w[i] >> 4) & 0x0f0f0f0fu);
+    a0 = __builtin_amdgcn_sdot4(lo, (int)x.a[0][i], a0, false);
+    a1 = __builtin_amdgcn_sdot4(lo, (int)x.a[1][i], a1, false);
+    a2 = __builtin_amdgcn_sdot4(lo, (int)x.a[2][i], a2, false);
+    b0 = __builtin_amdgcn_sdot4(hi, (int)x.b[0][i], b0, false);
+    b1 = __builtin_amdgcn_sdot4(hi, (int)x.b[1][i], b1, false);
+    b2 = __builtin_amdgcn_sdot4(hi, (int)x.b[2][i], b2, false);
+  }
+  const float va = fmaf((float)a0, 16384.f, (float)(a1 * 128 + a2));
+  const float vb = fmaf((float)b0, 16384.f, (float)(b1 * 128 + b2));
+  float sa, ma, sb, mb;
+  k4_pair(hd, jj, sa, ma, sb, mb);
+  return (sa * x.qa * va + sb * x.qb * vb) - (ma * x.qsa + mb * x.qsb);
+}
+
+struct Gu4kArgs {
+  const uint8_t *gate, *up;        // routed experts [E][mid rows][d/256 blocks]
+  const uint8_t *sh_gate, *sh_up;  // shared expert rows (nullptr: none)
+};
+
+// grid (mid/32, slots incl. shared, P); block 512.  Wave w: gate rows 4w..4w+3 and the matching up
+// rows of this block's 32; lane = unit (d/64 <= 64 units per row).  All 24 loads of a lane (8 rows x
+// two code halves + header) are in flight together.
+constexpr int G4_ROWS = 32;
+__global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t* __restrict__ xplanes,
+                                                     const float2* __restrict__ xmeta,
+                                                     const int* __restrict__ ids, int id_stride, int kpt, int d,
+                                                     int mid, uint32_t* __restrict__ hplanes,
+                                                     float2* __restrict__ hmeta) {
+  __shared__ float gs[G4_ROWS], us[G4_ROWS];
+  __shared__ uint32_t pk[QV_GROUP_DW];
+  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int U = d / 64;
+  const bool shared = s >= kpt;
+  const uint64_t rb = (uint64_t)(d / 256) * 144;
+  const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
+  const uint8_t* gbase = shared ? A.sh_gate : A.gate + (uint64_t)e * mid * rb;
+  const uint8_t* ubase = shared ? A.sh_up : A.up + (uint64_t)e * mid * rb;
+  const int r0 = blockIdx.x * G4_ROWS + 4 * wv;
+  const bool live = lane < U;
+  const int jj = lane & 3;
+  const size_t uoff = (size_t)(lane >> 2) * 144;  // this lane's super-block inside a row
+  uint4 c0[8], c1[8], hd[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const uint8_t* row = (i < 4 ? gbase : ubase) + (uint64_t)(r0 + (i & 3)) * rb + uoff;
+    if (live) {
+      hd[i] = *(const uint4*)row;
+      c0[i] = *(const uint4*)(row + 16 + jj * 32);
+      c1[i] = *(const uint4*)(row + 32 + jj * 32);
+    }
+  }
+  XU x;
+  if (live) load_xu(x, xplanes, xmeta, ((size_t)tok * U + lane) * 2);
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = sum64(live ? unit_dot(c0[i], c1[i], hd[i], jj, x) : 0.f);
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      gs[4 * wv + i] = acc[i];
+      us[4 * wv + i] = acc[4 + i];
+    }
+  }
+  __syncthreads();
+  // SwiGLU on the block's 32 rows = one sub-block of the down projection's input; quantise it
+  if (wv == 0) {
+    const int j = lane & 31;
+    const float g = gs[j], u = us[j];
+    const float hv = g / (1.f + expf(-g)) * u;
+    float m = dpp_max_row(fabsf(hv));
+    m = fmaxf(m, __shfl_xor(m, 16, 64));
+    const float inv = m > 0.f ? 1048576.f / m : 0.f;
+    const float q = m * (1.f / 1048576.f);
+    const int X = (int)rintf(hv * inv);
+    const int p2 = ((X + 64) & 127) - 64;
+    const int X1 = (X - p2) >> 7;
+    const int p1 = ((X1 + 64) & 127) - 64;
+    const int p0 = (X1 - p1) >> 7;
+    float sx = dpp_add_row((float)X);
+    sx += __shfl_xor(sx, 16, 64);
+    if (lane < QV_GROUP_DW) pk[lane] = 0;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    if (lane < 32) {
+      const int dw = j >> 2, sh = 8 * (j & 3);  // natural order
+      atomicOr(&pk[dw], (uint32_t)(p0 & 0xff) << sh);
+      atomicOr(&pk[8 + dw], (uint32_t)(p1 & 0xff) << sh);
+      atomicOr(&pk[16 + dw], (uint32_t)(p2 & 0xff) << sh);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_wave_barrier();
+    const size_t gi = ((size_t)tok * nslots + s) * (mid / 32) + blockIdx.x;
+    if (lane < QV_GROUP_DW) hplanes[gi * QV_GROUP_DW + lane] = pk[lane];
+    if (lane == 0) hmeta[gi] = make_float2(q, q * sx);
+  }
+}
+
+struct Dn4kArgs {
+  const uint8_t *down, *sh_down;  // [E][d rows][mid/256 blocks]; shared expert rows (nullptr: none)
+  const float* sh_logit;
+};
+
+// grid (d/ROWS, P); block = 64 x ceil(slots/4).  A row of 16 lanes = one slot (mid/64 <= 16 units),
+// holding that slot's hid planes in registers for all the block's rows.  The weighted combine runs
+// afterwards in slot order (descending router probability), then the shared expert.
+constexpr int D4_ROWS = 8, D4_MAXSLOTS = 16;
+__global__ void __launch_bounds__(256) k_dec4k_dn(Dn4kArgs A, const uint32_t* __restrict__ hplanes,
+                                                  const float2* __restrict__ hmeta, const int* __restrict__ ids,
+                                                  const float* __restrict__ ws, int id_stride, int kpt, int d,
+                                                  int mid, float* __restrict__ out, uint64_t out_stride) {
+  __shared__ float part[D4_MAXSLOTS][D4_ROWS];
+  const int tok = blockIdx.y;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const bool has_shared = A.sh_down != nullptr;
+  const int nslots = kpt + (has_shared ? 1 : 0);
+  const int U = mid / 64, u = lane & 15, s = 4 * wv + (lane >> 4);
+  const int r0 = blockIdx.x * D4_ROWS;
+  const uint64_t rb = (uint64_t)(mid / 256) * 144;
+  {
+    const bool live = s < nslots && u < U;
+    const bool shared = has_shared && s == nslots - 1;
+    const int e = (live && !shared) ? ids[(size_t)tok * id_stride + s] : 0;
+    const uint8_t* base = (shared ? A.sh_down : A.down + (uint64_t)e * d * rb) + (uint64_t)r0 * rb + (size_t)(u >> 2) * 144;
+    const int jj = u & 3;
+    uint4 c0[D4_ROWS], c1[D4_ROWS], hd[D4_ROWS];
+#pragma unroll
+    for (int r = 0; r < D4_ROWS; r++) {
+      if (live) {
+        const uint8_t* row = base + (uint64_t)r * rb;
+        hd[r] = *(const uint4*)row;
+        c0[r] = *(const uint4*)(row + 16 + jj * 32);
+        c1[r] = *(const uint4*)(row + 32 + jj * 32);
+      }
+    }
+    XU x;
+    if (live) load_xu(x, hplanes, hmeta, (((size_t)tok * nslots + s) * U + u) * 2);
+#pragma unroll
+    for (int r = 0; r < D4_ROWS; r++) {
+      const float v = dpp_add_row(live ? unit_dot(c0[r], c1[r], hd[r], jj, x) : 0.f);
+      if (u == 0 && s < nslots) part[s][r] = v;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < D4_ROWS) {
+    const int r = threadIdx.x;
+    float y = 0.f;
+    for (int i = 0; i < kpt; i++) y += ws[(size_t)tok * id_stride + i] * part[i][r];
+    if (has_shared) y += sigmoid_f(A.sh_logit[tok]) * part[kpt][r];
+    out[(size_t)tok * out_stride + r0 + r] = y;
+  }
+}
+
+}  // namespace
+
+bool moe_dec4k_supported(int d, int mid, int nslots) {
+  return d % 256 == 0 && d / 64 <= 64 && mid % 256 == 0 && mid / 64 <= 16 && nslots <= D4_MAXSLOTS &&
+         mid % G4_ROWS == 0 && d % D4_ROWS == 0;
+}
+
+int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
+                        const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
+                        int P, int d, int mid, uint32_t* hplanes, float2* hmeta, hipStream_t st) {
+  if (!gate || !up || !xplanes || !xmeta || !ids || !hplanes || !hmeta) return MOE_E_INVALID;
+  if (!moe_aligned(gate, 16) || !moe_aligned(up, 16) || (sh_gate && (!sh_up || !moe_aligned(sh_gate, 16) || !moe_aligned(sh_up, 16))))
+    return MOE_E_INVALID;
+  Gu4kArgs A{gate, up, sh_gate, sh_up};
+  dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0), P);
+  k_dec4k_gu<<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_dec4k_dn(const uint8_t* down, const uint8_t* sh_down, const float* sh_logit,
+                        const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
+                        int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
+                        hipStream_t st) {
+  if (!down || !hplanes || !hmeta || !ids || !ws || !out || (sh_down && !sh_logit)) return MOE_E_INVALID;
+  if (!moe_aligned(down, 16) || (sh_down && !moe_aligned(sh_down, 16))) return MOE_E_INVALID;
+  Dn4kArgs A{down, sh_down, sh_logit};
+  const int nslots = kpt + (sh_down ? 1 : 0);
+  dim3 grid(d / D4_ROWS, P);
+  k_dec4k_dn<<<grid, 64 * ((nslots + 3) / 4), 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}

@@ -11,7 +11,7 @@ struct moe_hscale {
 
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
-                            unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
+                            bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
                             hipStream_t st);
 int moe_launch_gemv_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                        const float* x, uint64_t x_stride, const int* ids, int id_stride, int kpt, int P,
@@ -46,6 +46,15 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
                       hipStream_t st);
+// the same for raw GGUF Q4_K rows (activation planes in natural order)
+bool moe_dec4k_supported(int d, int mid, int nslots);
+int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
+                        const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
+                        int P, int d, int mid, uint32_t* hplanes, float2* hmeta, hipStream_t st);
+int moe_launch_dec4k_dn(const uint8_t* down, const uint8_t* sh_down, const float* sh_logit,
+                        const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
+                        int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
+                        hipStream_t st);
 int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,
                       const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
                       int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,

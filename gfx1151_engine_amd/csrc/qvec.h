@@ -1,18 +1,27 @@
 // Quantised activation vectors for the integer-dot decode kernels ("qvec"), per group of 32
 // elements:
 //   planes: 3 x 8 dwords of signed 7-bit digits, x ~= q * (2^14 p0 + 2^7 p1 + p2);
-//           dword 2i holds elements 8i+{0,2,4,6}, dword 2i+1 elements 8i+{1,3,5,7}
-//           (the order in which `w & 0x0f0f0f0f` / `(w>>4) & 0x0f0f0f0f` deliver the 4-bit codes)
+//           q4cp order: dword 2i holds elements 8i+{0,2,4,6}, dword 2i+1 elements 8i+{1,3,5,7}
+//           (the order in which `w & 0x0f0f0f0f` / `(w>>4) & 0x0f0f0f0f` deliver the 4-bit codes of
+//           a q4cp row); natural order (Q4_K, where the low nibbles of 32 consecutive bytes are one
+//           32-element sub-block and the high nibbles the next): dword i holds elements 4i..4i+3
 //   meta:   float2 (q, q * sum of the quantised elements)
 #pragma once
 #include "common.h"
 
 constexpr int QV_GROUP_DW = 24;
 
+// digit plane position of element j (0..31) of a group
+__device__ __forceinline__ void qvec_pos(int j, bool natural, int& dw, int& sh) {
+  dw = natural ? j >> 2 : 2 * (j >> 3) + (j & 1);
+  sh = natural ? 8 * (j & 3) : 8 * ((j & 7) >> 1);
+}
+
 // One thread quantises group g of token t.
-__device__ __forceinline__ void qvec_group_from_f32(const float* __restrict__ x, uint64_t x_stride, int G, int t,
-                                                    int g, uint32_t* __restrict__ planes,
-                                                    float2* __restrict__ meta) {
+template <bool NATURAL>
+__device__ __forceinline__ void qvec_group_from_f32_t(const float* __restrict__ x, uint64_t x_stride, int G, int t,
+                                                      int g, uint32_t* __restrict__ planes,
+                                                      float2* __restrict__ meta) {
   const float4* xp = (const float4*)(x + (size_t)t * x_stride + (size_t)g * 32);
   float v[32];
   float m = 0.f;
@@ -38,7 +47,7 @@ __device__ __forceinline__ void qvec_group_from_f32(const float* __restrict__ x,
     const int X1 = (X - p2) >> 7;
     const int p1 = ((X1 + 64) & 127) - 64;
     const int p0 = (X1 - p1) >> 7;
-    const int dw = 2 * (j >> 3) + (j & 1), sh = 8 * ((j & 7) >> 1);
+    const int dw = NATURAL ? j >> 2 : 2 * (j >> 3) + (j & 1), sh = NATURAL ? 8 * (j & 3) : 8 * ((j & 7) >> 1);
     pl[0][dw] |= (uint32_t)(p0 & 0xff) << sh;
     pl[1][dw] |= (uint32_t)(p1 & 0xff) << sh;
     pl[2][dw] |= (uint32_t)(p2 & 0xff) << sh;
@@ -50,4 +59,10 @@ __device__ __forceinline__ void qvec_group_from_f32(const float* __restrict__ x,
     dst[2 * p + 1] = make_uint4(pl[p][4], pl[p][5], pl[p][6], pl[p][7]);
   }
   meta[(size_t)t * G + g] = make_float2(q, q * (float)sx);
+}
+__device__ __forceinline__ void qvec_group_from_f32(const float* __restrict__ x, uint64_t x_stride, int G, int t,
+                                                    int g, uint32_t* __restrict__ planes,
+                                                    float2* __restrict__ meta, bool natural = false) {
+  if (natural) qvec_group_from_f32_t<true>(x, x_stride, G, t, g, planes, meta);
+  else qvec_group_from_f32_t<false>(x, x_stride, G, t, g, planes, meta);
 }

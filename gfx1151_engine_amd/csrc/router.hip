@@ -206,16 +206,16 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
                                                       const float* __restrict__ x, int P, int E, int d,
                                                       float* __restrict__ logits, float* __restrict__ out_x,
                                                       int nrows, uint32_t* __restrict__ planes,
-                                                      float2* __restrict__ meta, unsigned* counter,
-                                                      int* __restrict__ ids, float* __restrict__ ws, int k,
-                                                      int id_stride) {
+                                                      float2* __restrict__ meta, bool planes_natural,
+                                                      unsigned* counter, int* __restrict__ ids,
+                                                      float* __restrict__ ws, int k, int id_stride) {
   __shared__ int s_last;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int nrb = (nrows + 3) >> 2;
   if ((int)blockIdx.x >= nrb) {
     const int G = d / 32, gb = (G + 255) / 256;
     const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * 256 + threadIdx.x;
-    if (t < P && g < G) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
+    if (t < P && g < G) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta, planes_natural);
     return;
   }
   const int row = blockIdx.x * 4 + wv;
@@ -504,8 +504,8 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
   const bool par = mode == 0 && P <= 32 && d % 4 == 0 && moe_aligned(x, 16) && moe_aligned(W->data, 16);
   if (par) {
     dim3 g((E + 3) / 4);
-    if (bf) k_router_small<true, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0);
-    else k_router_small<false, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0);
+    if (bf) k_router_small<true, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, false, nullptr, nullptr, nullptr, 0, 0);
+    else k_router_small<false, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, false, nullptr, nullptr, nullptr, 0, 0);
   } else {
     launch_seq(W->data, bf, bias, nullptr, false, x, P, E, d, logits, nullptr, nullptr, moe_s(st));
   }
@@ -529,7 +529,7 @@ int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview
 // memory holding 0) and P <= 4 the launch also does the softmax / top-k: *fused_topk says so.
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
-                            unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
+                            bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
                             hipStream_t st) {
   const int E = (int)W->rows, d = (int)W->cols;
   const bool bf = W->dtype == MOE_DT_BF16;
@@ -541,9 +541,16 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   unsigned* cn = fuse ? counter : nullptr;
   dim3 g((nrows + 3) / 4 + qblocks);
   const void* wx = Wx ? Wx->data : nullptr;
-#define RSM_GO(BF, NPL) k_router_small<BF, 4, NPL><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, cn, ids, ws, k, id_stride)
-  if (E <= 512) { if (bf) RSM_GO(true, 8); else RSM_GO(false, 8); }
-  else { if (bf) RSM_GO(true, 16); else RSM_GO(false, 16); }
+#define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride)
+  // tokens per pass over a weight row: every row is read ceil(P / TT) times
+  if (P <= 4) {
+    if (E <= 512) { if (bf) RSM_GO(true, 4, 8); else RSM_GO(false, 4, 8); }
+    else { if (bf) RSM_GO(true, 4, 16); else RSM_GO(false, 4, 16); }
+  } else if (P <= 8) {
+    if (bf) RSM_GO(true, 8, 16); else RSM_GO(false, 8, 16);
+  } else {
+    if (bf) RSM_GO(true, 16, 16); else RSM_GO(false, 16, 16);
+  }
 #undef RSM_GO
   MOE_LAUNCH_CHECK();
   return MOE_OK;

@@ -42,6 +42,29 @@ def test_small_batch_layer(oracle, fmt, d, mid, E, k, T, cb):
     assert max_abs_rel(y, yo) <= TOL_GEMV
 
 
+@pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 9), ("q4k", 1), ("q4k", 9)])
+def test_int_decode_switch(oracle, fmt, T):
+    """MOE_OPT_INT_DECODE 1 (integer-dot kernels, default) and 0 (f32 kernels) both meet the GEMV bar
+    and select the same experts."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(77 + T)
+    d, mid, E, k = 3072, 768, 16, 10
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=32)
+    ys = []
+    for opt in (1, 0):
+        m.set_option(capi.OPT_INT_DECODE, opt)
+        y = m.forward(0, gpu(x)).cpu().numpy()
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+        assert max_abs_rel(y, yo) <= TOL_GEMV, (opt, max_abs_rel(y, yo))
+        ys.append(y)
+    assert not (ys[0] == ys[1]).all(), "the two paths are different kernels (digit planes vs f32)"
+    m.close()
+
+
 def test_golden_layers_from_reference(oracle, golden):
     """Inputs and outputs of the reference's own Model::moe (tests/golden/moe_layer.npz)."""
     import torch
