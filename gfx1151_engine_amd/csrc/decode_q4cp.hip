@@ -1,10 +1,11 @@
-// Decode (T <= 32): bandwidth-bound expert GEMV on q4cp weights read in place, integer dot
-// products.  The activation vector is turned once per token into three signed 7-bit digit planes
-// per 32-element group (x ~= q_g * (2^14 p0 + 2^7 p1 + p2), 21 significant bits relative to the
-// group maximum), so that a 16-byte load of 32 weight codes costs 12 unpack + 24 v_dot4_i32_i8
-// instead of ~100 float operations: the VALU then keeps up with HBM.  Weights stay exact (codes are
-// integers; the group scale and q_g are applied in f32 after the integer sum), the zero point is
-// folded in through the group sum of the activations.
+// Decode (T <= 32): bandwidth-bound expert GEMV on q4cp weights read in place, integer dot products.
+// The activation vector is turned once per token into four planes of balanced base-16 digits per
+// 32-element group (x ~= q_g * (4096 p3 + 256 p2 + 16 p1 + p0), 15.9 significant bits relative to the
+// group maximum), stored in the nibble order of a q4cp code word.  A 16-byte load of 32 codes then
+// costs 4 XORs (unsigned code n -> n - 8 in two's complement) and 16 v_dot8_i32_i4 instead of ~100
+// float operations: the VALU keeps up with HBM.  Weights stay exact (codes are integers; the group
+// scale, the codebook slope / offset and q_g are applied in f32 after the integer sum, the offset
+// through the group sum of the activations).
 // (reference: src/gpu/parts/20_kernels_gemv.inc:1608-1835 — same contract: per-slot gate/up with
 //  SwiGLU, then the down projection with the top-k weighted combine in slot order, no atomics)
 #include "common.h"
@@ -35,62 +36,56 @@ __device__ __forceinline__ float sum64(float v) {
   return v + __shfl_xor(v, 32, 64);
 }
 
-// Quantise 32 floats held one per lane by lanes [0,32) of a half-wave (j = lane & 31): returns
-// this lane's three digits, q and q*sum(X).
-__device__ __forceinline__ void quant32_lane(float x, int& p0, int& p1, int& p2, float& q, float& qsx) {
+// Quantise 32 floats held one per lane by lanes [0,32) of a half-wave (j = lane & 31) into the qvec4
+// form: returns this lane's four digits, q and q*sum(X).
+__device__ __forceinline__ void quant32_lane(float x, int& p0, int& p1, int& p2, int& p3, float& q, float& qsx) {
   float m = dpp_max_row(fabsf(x));
   m = fmaxf(m, __shfl_xor(m, 16, 64));
-  const float inv = m > 0.f ? 1048576.f / m : 0.f;
-  q = m * (1.f / 1048576.f);
+  const float inv = m > 0.f ? QV4_XMAX / m : 0.f;
+  q = m * (1.f / QV4_XMAX);
   const int X = (int)rintf(x * inv);
-  p2 = ((X + 64) & 127) - 64;
-  const int X1 = (X - p2) >> 7;
-  p1 = ((X1 + 64) & 127) - 64;
-  p0 = (X1 - p1) >> 7;
+  qv4_digits(X, p0, p1, p2, p3);
   qsx = q * sum32((float)X);
 }
 
-// One thread per group: x (f32, K elements) -> qvec.  Blocks of 64.
+// One thread per group: x (f32, K elements) -> qvec4.  Blocks of 64.
 __global__ void __launch_bounds__(64) k_qvec_from_f32(const float* __restrict__ x, uint64_t x_stride,
                                                       int G, uint32_t* __restrict__ planes,
                                                       float2* __restrict__ meta) {
   const int t = blockIdx.y, g = blockIdx.x * 64 + threadIdx.x;
-  if (g < G) qvec_group_from_f32(x, x_stride, G, t, g, planes, meta);
+  if (g < G) qvec4_group_from_f32(x, x_stride, G, t, g, planes, meta);
 }
 
 struct XG {  // one group's activation planes in registers
-  uint32_t p[3][8];
+  uint32_t p[4][4];
   float q, qsx;
 };
 __device__ __forceinline__ void load_xg(XG& x, const uint32_t* planes, const float2* meta, size_t gi) {
-  const uint4* s = (const uint4*)(planes + gi * QV_GROUP_DW);
+  const uint4* s = (const uint4*)(planes + gi * QV4_GROUP_DW);
 #pragma unroll
-  for (int p = 0; p < 3; p++) {
-    const uint4 a = s[2 * p], b = s[2 * p + 1];
+  for (int p = 0; p < 4; p++) {
+    const uint4 a = s[p];
     x.p[p][0] = a.x; x.p[p][1] = a.y; x.p[p][2] = a.z; x.p[p][3] = a.w;
-    x.p[p][4] = b.x; x.p[p][5] = b.y; x.p[p][6] = b.z; x.p[p][7] = b.w;
   }
   const float2 m = meta[gi];
   x.q = m.x;
   x.qsx = m.y;
 }
 
-// sum_k cb[n_k] * x_k over one group, cb = a*n + b:  a * q * (2^14 D0 + 2^7 D1 + D2) + b * q * sum(X)
-__device__ __forceinline__ float chunk_dot(const uint4 cw, const XG& x, float cb_a, float cb_b) {
-  const uint32_t w[4] = {cw.x, cw.y, cw.z, cw.w};
-  int d0 = 0, d1 = 0, d2 = 0;
+// sum_k cb[n_k] * x_k over one group, cb = a*n + b = a*(n-8) + (8a+b):
+//   a * q * (4096 D3 + 256 D2 + 16 D1 + D0) + (8a + b) * q * sum(X),  D_j = sum_k (n_k - 8) * p_j,k
+__device__ __forceinline__ float chunk_dot(const uint4 cw, const XG& x, float cb_a, float cb_b8) {
+  const uint32_t w[4] = {cw.x ^ 0x88888888u, cw.y ^ 0x88888888u, cw.z ^ 0x88888888u, cw.w ^ 0x88888888u};
+  int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    const int lo = (int)(w[i] & 0x0f0f0f0fu), hi = (int)((w[i] >> 4) & 0x0f0f0f0fu);
-    d0 = __builtin_amdgcn_sdot4(lo, (int)x.p[0][2 * i], d0, false);
-    d1 = __builtin_amdgcn_sdot4(lo, (int)x.p[1][2 * i], d1, false);
-    d2 = __builtin_amdgcn_sdot4(lo, (int)x.p[2][2 * i], d2, false);
-    d0 = __builtin_amdgcn_sdot4(hi, (int)x.p[0][2 * i + 1], d0, false);
-    d1 = __builtin_amdgcn_sdot4(hi, (int)x.p[1][2 * i + 1], d1, false);
-    d2 = __builtin_amdgcn_sdot4(hi, (int)x.p[2][2 * i + 1], d2, false);
+    d0 = __builtin_amdgcn_sdot8((int)w[i], (int)x.p[0][i], d0, false);
+    d1 = __builtin_amdgcn_sdot8((int)w[i], (int)x.p[1][i], d1, false);
+    d2 = __builtin_amdgcn_sdot8((int)w[i], (int)x.p[2][i], d2, false);
+    d3 = __builtin_amdgcn_sdot8((int)w[i], (int)x.p[3][i], d3, false);
   }
-  const float v = fmaf((float)d0, 16384.f, (float)(d1 * 128 + d2));
-  return fmaf(cb_a * x.q, v, cb_b * x.qsx);
+  const int D = ((d3 * 16 + d2) * 16 + d1) * 16 + d0;  // |D| < 2^24: exact as f32
+  return fmaf(cb_a * x.q, (float)D, cb_b8 * x.qsx);
 }
 
 struct DecW {  // one q4cp tensor's planes
@@ -115,7 +110,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
                                                 int mid, uint32_t* __restrict__ hplanes,
                                                 float2* __restrict__ hmeta, float* __restrict__ hid_f32) {
   __shared__ float gs[GU2_ROWS], us[GU2_ROWS];
-  __shared__ uint32_t pk[QV_GROUP_DW];
+  __shared__ uint32_t pk[QV4_GROUP_DW];
   const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int G = d / 32;
@@ -151,7 +146,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
       st[p] = *(const __half*)(s0 + trow * W.ss + gB * 2);
     }
   }
-  const float ga = Wg.cb[1] - Wg.cb[0], gb = Wg.cb[0], ua = Wu.cb[1] - Wu.cb[0], ub = Wu.cb[0];
+  const float ga = Wg.cb[1] - Wg.cb[0], gb = fmaf(8.f, ga, Wg.cb[0]), ua = Wu.cb[1] - Wu.cb[0], ub = fmaf(8.f, ua, Wu.cb[0]);
   XG xa, xb;
   const size_t xbase = (size_t)tok * G;
   if (vA) load_xg(xa, xplanes, xmeta, xbase + gA);
@@ -191,22 +186,23 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     const float hv = g / (1.f + expf(-g)) * u;
     const size_t slot = (size_t)tok * nslots + s;
     if (hid_f32 && lane < 32) hid_f32[slot * mid + blockIdx.x * GU2_ROWS + j] = hv;
-    int p0, p1, p2;
+    int p0, p1, p2, p3;
     float q, qsx;
-    quant32_lane(hv, p0, p1, p2, q, qsx);
-    if (lane < QV_GROUP_DW) pk[lane] = 0;
+    quant32_lane(hv, p0, p1, p2, p3, q, qsx);
+    if (lane < QV4_GROUP_DW) pk[lane] = 0;
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     __builtin_amdgcn_wave_barrier();
     if (lane < 32) {
-      const int dw = 2 * (j >> 3) + (j & 1), sh = 8 * ((j & 7) >> 1);
-      atomicOr(&pk[dw], (uint32_t)(p0 & 0xff) << sh);
-      atomicOr(&pk[8 + dw], (uint32_t)(p1 & 0xff) << sh);
-      atomicOr(&pk[16 + dw], (uint32_t)(p2 & 0xff) << sh);
+      const int dw = j >> 3, sh = 4 * (j & 7);
+      atomicOr(&pk[dw], (uint32_t)(p0 & 15) << sh);
+      atomicOr(&pk[4 + dw], (uint32_t)(p1 & 15) << sh);
+      atomicOr(&pk[8 + dw], (uint32_t)(p2 & 15) << sh);
+      atomicOr(&pk[12 + dw], (uint32_t)(p3 & 15) << sh);
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_wave_barrier();
     const size_t gi = slot * (mid / 32) + blockIdx.x;
-    if (lane < QV_GROUP_DW) hplanes[gi * QV_GROUP_DW + lane] = pk[lane];
+    if (lane < QV4_GROUP_DW) hplanes[gi * QV4_GROUP_DW + lane] = pk[lane];
     if (lane == 0) hmeta[gi] = make_float2(q, qsx);
   }
 }
@@ -258,7 +254,7 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
         sc[r] = *(const __half*)(sp + r * wss);
       }
     }
-    const float a = wcb[1] - wcb[0], b = wcb[0];
+    const float a = wcb[1] - wcb[0], b = fmaf(8.f, a, wcb[0]);
     XG x;
     if (live) load_xg(x, hplanes, hmeta, ((size_t)tok * nslots + s) * G + g);
 #pragma unroll

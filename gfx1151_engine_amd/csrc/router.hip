@@ -215,7 +215,10 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
   if ((int)blockIdx.x >= nrb) {
     const int G = d / 32, gb = (G + 255) / 256;
     const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * 256 + threadIdx.x;
-    if (t < P && g < G) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta, planes_natural);
+    if (t < P && g < G) {
+      if (planes_natural) qvec_group_from_f32_t<true>(x, (uint64_t)d, G, t, g, planes, meta);  // Q4_K kernels
+      else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);                       // q4cp kernels
+    }
     return;
   }
   const int row = blockIdx.x * 4 + wv;
