@@ -42,7 +42,11 @@ constexpr int WROWS = 512;     // weight rows per block (up: 256 gate + 256 up)
 constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chunk c of row m at slot c ^ (m & 7)
 constexpr int W_BYTES = WROWS * 32;       // 16 KB  [row][32 B]
 constexpr int S_BYTES = WROWS * 16;       //  8 KB  [row][8 scales], refreshed every 4 stages
-constexpr int NBUF = 3;                   // activation / code buffers in flight (loads run two stages ahead)
+#ifndef MOE_GEMM_NBUF
+#define MOE_GEMM_NBUF 3
+#endif
+constexpr int NBUF = MOE_GEMM_NBUF;       // activation / code buffers; loads run NBUF-1 stages ahead
+constexpr int AHEAD = NBUF - 1;
 constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES + 64 + BM * 4 + BM * 4;
 
 struct LutDev {
@@ -206,10 +210,25 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     }
   };
   // s_waitcnt vmcnt(N), N = loads allowed to stay in flight (loads retire in order)
-  auto wait_loads_except = [&](int s_pending) {  // s_pending: stage whose loads may remain (-1: none)
-    if (s_pending < 0 || s_pending >= nstage) __builtin_amdgcn_s_waitcnt(0x0F70);
-    else if ((s_pending & 3) == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (NLOADS + S_LOADS));
-    else __builtin_amdgcn_s_waitcnt(0x0F70 | NLOADS);
+  // (the immediate must be a constant: one case per count of outstanding loads)
+  auto wait_vm = [&](int n) {
+    switch (n) {
+#define VM_CASE(N) case N: __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14)); break;
+      VM_CASE(0) VM_CASE(1) VM_CASE(2) VM_CASE(3) VM_CASE(4) VM_CASE(5) VM_CASE(6) VM_CASE(7) VM_CASE(8)
+      VM_CASE(9) VM_CASE(10) VM_CASE(11) VM_CASE(12) VM_CASE(13) VM_CASE(14) VM_CASE(15) VM_CASE(16)
+      VM_CASE(17) VM_CASE(18) VM_CASE(19) VM_CASE(20) VM_CASE(21) VM_CASE(22) VM_CASE(23) VM_CASE(24)
+      VM_CASE(25) VM_CASE(26) VM_CASE(27) VM_CASE(28) VM_CASE(29) VM_CASE(30) VM_CASE(31) VM_CASE(32)
+#undef VM_CASE
+      default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+    }
+  };
+  // wait until the loads of every stage before `first` have landed; stages first .. first+AHEAD-2
+  // (those that exist) may still be in flight
+  auto wait_loads_before = [&](int first) {
+    int n = 0;
+    for (int t = first; t < first + AHEAD - 1; t++)
+      if (t < nstage) n += NLOADS + ((t & 3) == 0 ? S_LOADS : 0);
+    wait_vm(n);
   };
 
   floatx16 acc[MF][NF];
@@ -332,11 +351,12 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   constexpr int X0 = NM >= 8 ? NM / 4 : 1;        // step 3: first MFMA slot that dequantises
   constexpr int XPM = (NU + NM - X0 - 1) / (NM - X0);
 
-  // loads run two stages ahead of the MFMAs
-  issue(0);
-  if (nstage > 1) issue(1);
-  // stage 0 must have landed; stage 1's loads may still be in flight
-  wait_loads_except(nstage > 1 ? 1 : -1);
+  // loads run AHEAD stages ahead of the MFMAs
+#pragma unroll
+  for (int t = 0; t < AHEAD; t++)
+    if (t < nstage) issue(t);
+  // stage 0 must have landed; the later ones may still be in flight
+  wait_loads_before(1);
   __syncthreads();
   load_codes(0);
 #pragma unroll
@@ -347,8 +367,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 
   for (int s = 0; s < nstage; s++) {
     Ab = A0 + (s % NBUF) * A_BYTES;
-    const bool pf = s + 2 < nstage;            // stage s+2 exists: its loads go out during step 0
-    const bool pf_s = pf && ((s + 2) & 3) == 0;
+    const bool pf = s + AHEAD < nstage;        // stage s+AHEAD exists: its loads go out during step 0
+    const bool pf_s = pf && ((s + AHEAD) & 3) == 0;
 #pragma unroll
     for (int q = 0; q < 3; q++) {
       const int cur = q & 1, nxt = cur ^ 1;
@@ -362,13 +382,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         for (int k = 0; k < UPM; k++)
           if (i * UPM + k < NU) deq_unit(q + 1, i * UPM + k, b[nxt]);
         if (q == 0) {
-          // buffer (s+2)%3 was last read in stage s-1: free since the previous barrier
+          // buffer (s+AHEAD)%NBUF was last read in stage s-1: free since the previous barrier
           constexpr int LPS = (NLOADS + S_LOADS + NM - 1) / NM;  // loads per MFMA slot
 #pragma unroll
           for (int k = 0; k < LPS; k++) {
             const int u = i * LPS + k;
-            if (u < NLOADS) { if (pf) issue_unit(s + 2, u); }
-            else if (u < NLOADS + S_LOADS) { if (pf_s) issue_unit(s + 2, u); }
+            if (u < NLOADS) { if (pf) issue_unit(s + AHEAD, u); }
+            else if (u < NLOADS + S_LOADS) { if (pf_s) issue_unit(s + AHEAD, u); }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -377,7 +397,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     // last step: a[1], b[1] hold its operands.  Step 0 of stage s+1 is prepared from the next
     // buffer meanwhile, so that buffer must be complete and visible: loads of stage s+1 done
     // (stage s+2's may still fly), then the block barrier.
-    wait_loads_except(s + 2);
+    wait_loads_before(s + 2);
     __syncthreads();
     Ab = A0 + ((s + 1) % NBUF) * A_BYTES;
 #pragma unroll
