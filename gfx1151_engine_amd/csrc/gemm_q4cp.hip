@@ -39,7 +39,7 @@ constexpr int NT = 64 * NW;               // each wave: 128 pairs x 32*NF weight
 constexpr int BM = 128;        // pairs per tile (4 MFMA row fragments)
 constexpr int BK = 64;         // K per stage
 constexpr int WROWS = 512;     // weight rows per block (up: 256 gate + 256 up)
-constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chunk c of row m at slot c ^ (m & 7)
+constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chunk c of row m at slot c ^ ((m >> 1) & 7): conflict-free for the 128-bit fragment reads
 constexpr int W_BYTES = WROWS * 32;       // 16 KB  [row][32 B]
 constexpr int S_BYTES = WROWS * 16;       //  8 KB  [row][8 scales], refreshed every 4 stages
 #ifndef MOE_GEMM_NBUF
@@ -154,7 +154,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   };
 
   // per-lane global sources of the direct-to-LDS loads (wave-load j of a buffer = LDS bytes [1024 j, +1024))
-  // activations: rows 8j..8j+7, lane -> (row 8j + lane/8, slot lane%8 holding chunk slot ^ (row & 7)).
+  // activations: rows 8j..8j+7, lane -> (row 8j + lane/8, slot lane%8 holding chunk slot ^ ((row >> 1) & 7)).
   // The 4*MF row groups are dealt to the waves; with more waves than groups some load a group twice
   // (same bytes to the same place) so that every wave issues the same number of loads.
   constexpr int A_GROUPS = 4 * MF;
@@ -166,7 +166,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   for (int i = 0; i < A_LOADS; i++) {
     a_grp[i] = (A_LOADS * wv + i) % A_GROUPS;
     const int m = 8 * a_grp[i] + (lane >> 3);
-    a_src[i] = x + (size_t)rowidx[m] * K + (((lane & 7) ^ (m & 7)) << 3);
+    a_src[i] = x + (size_t)rowidx[m] * K + (((lane & 7) ^ ((m >> 1) & 7)) << 3);
   }
   // codes: rows 32j..32j+31, lane -> (row 32j + lane/2, half lane%2); scales: rows 64j.., lane -> row
   const uint8_t *w_src[W_LOADS], *s_src[S_LOADS];
@@ -269,7 +269,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   const uint8_t* Ab = A0;
   auto load_a1 = [&](int q, int mf, half8* dst) {
     const int m = 32 * mf + n;
-    dst[mf] = *(const half8*)(Ab + m * 128 + (((4 * h + q) ^ (m & 7)) << 4));
+    dst[mf] = *(const half8*)(Ab + m * 128 + (((4 * h + q) ^ ((m >> 1) & 7)) << 4));
   };
   auto load_codes = [&](int s) {  // raw codes + this lane's scale of stage s (buffers already selected)
     const uint8_t* Wb = W0 + (s % NBUF) * W_BYTES;
