@@ -1,6 +1,7 @@
 // Router: logits with the CPU path's fp64 accumulation, fp64 softmax, top-k, renormalised weights.
 // (reference: src/ref.cpp:68-77,565-594; src/gpu/parts/20_kernels_gemv.inc:1433-1562)
 #include "common.h"
+#include "internal.h"
 #include "qvec.h"
 
 namespace {
@@ -288,6 +289,98 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
   if (threadIdx.x == 0) *counter = 0u;  // re-armed for the next launch on the stream
 }
 
+// ---- lane-parallel order for 5..32 tokens: four weight rows per block (a wave each); the tokens'
+// activations are widened to fp64 ONCE per block and 128-column slab (in LDS) instead of once per
+// row, and every weight is read once for all tokens.  Lane l owns columns 2l, 2l+1 of each slab:
+// two fp64 chains per token, combined in a fixed order, then the wave sum.  Same accuracy
+// statement as k_router_small.  Blocks past the rows build the digit planes of x.
+constexpr int RM_C = 128;
+template <bool BF16, int PMAX>
+__global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, const float* __restrict__ bias,
+                                                    const void* __restrict__ Wx, bool wx_bf16,
+                                                    const float* __restrict__ x, int P, int E, int d,
+                                                    float* __restrict__ logits, float* __restrict__ out_x,
+                                                    int nrows, uint32_t* __restrict__ planes,
+                                                    float2* __restrict__ meta, bool planes_natural) {
+  __shared__ __attribute__((aligned(16))) double Xd[PMAX][RM_C];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int nrb = (nrows + 3) >> 2;
+  if ((int)blockIdx.x >= nrb) {
+    const int G = d / 32, gb = (G + 255) / 256;
+    const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * 256 + tid;
+    if (t < P && g < G) {
+      if (planes_natural) qvec_group_from_f32_t<true>(x, (uint64_t)d, G, t, g, planes, meta);
+      else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
+    }
+    return;
+  }
+  const int row = blockIdx.x * 4 + wv;
+  const bool live = row < nrows, extra = row == E;
+  const void* Wr = extra ? Wx : W;
+  const uint64_t base = extra ? 0 : (uint64_t)(live ? row : 0) * d;
+  const bool bf = extra ? wx_bf16 : BF16;
+  constexpr int XR = PMAX * RM_C / 256;  // staged activations per thread and slab
+  float xr[XR];
+  float2 wr;
+  auto fetch = [&](int c0) {
+#pragma unroll
+    for (int j = 0; j < XR; j++) {
+      const int e = tid + 256 * j, t = e / RM_C, c = c0 + e % RM_C;
+      xr[j] = (t < P && c < d) ? x[(size_t)t * d + c] : 0.f;
+    }
+    const int c = c0 + 2 * lane;
+    wr = float2{0.f, 0.f};
+    if (live && c + 1 < d) {
+      if (bf) {
+        const uint32_t u = *(const uint32_t*)((const uint16_t*)Wr + base + c);
+        wr.x = __uint_as_float(u << 16);
+        wr.y = __uint_as_float(u & 0xffff0000u);
+      } else {
+        wr = *(const float2*)((const float*)Wr + base + c);
+      }
+    } else if (live && c < d) {
+      wr.x = bf ? bf16_bits_to_f32(((const uint16_t*)Wr)[base + c]) : ((const float*)Wr)[base + c];
+    }
+  };
+  double acc[PMAX][2];
+#pragma unroll
+  for (int t = 0; t < PMAX; t++) acc[t][0] = acc[t][1] = 0.0;
+  fetch(0);
+  for (int c0 = 0; c0 < d; c0 += RM_C) {
+    __syncthreads();  // the previous slab is no longer read
+#pragma unroll
+    for (int j = 0; j < XR; j++) {
+      const int e = tid + 256 * j;
+      Xd[e / RM_C][e % RM_C] = (double)xr[j];
+    }
+    const double w0 = (double)wr.x, w1 = (double)wr.y;
+    __syncthreads();
+    if (c0 + RM_C < d) fetch(c0 + RM_C);
+#pragma unroll
+    for (int t = 0; t < PMAX; t++) {
+      if (t < P) {
+        const double2 xv = *(const double2*)&Xd[t][2 * lane];
+        acc[t][0] = fma(w0, xv.x, acc[t][0]);
+        acc[t][1] = fma(w1, xv.y, acc[t][1]);
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < PMAX; t++) {
+    if (t < P) {
+      const double sum = wave_sum(acc[t][0] + acc[t][1]);
+      if (lane == 0 && live) {
+        float v = (float)sum;
+        if (extra) out_x[t] = v;
+        else {
+          if (bias) v += bias[row];
+          logits[(size_t)t * E + row] = v;
+        }
+      }
+    }
+  }
+}
+
 __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 __device__ __forceinline__ uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
 __device__ __forceinline__ uint32_t wave_umax(uint32_t m) {
@@ -506,9 +599,8 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool par = mode == 0 && P <= 32 && d % 4 == 0 && moe_aligned(x, 16) && moe_aligned(W->data, 16);
   if (par) {
-    dim3 g((E + 3) / 4);
-    if (bf) k_router_small<true, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, false, nullptr, nullptr, nullptr, 0, 0);
-    else k_router_small<false, 4, 8><<<g, 256, 0, moe_s(st)>>>(W->data, bias, nullptr, false, x, P, E, d, logits, nullptr, E, nullptr, nullptr, false, nullptr, nullptr, nullptr, 0, 0);
+    return moe_router_logits_small(W, bias, nullptr, x, P, logits, nullptr, nullptr, nullptr, false, nullptr, nullptr,
+                                   nullptr, 0, 0, nullptr, moe_s(st));
   } else {
     launch_seq(W->data, bf, bias, nullptr, false, x, P, E, d, logits, nullptr, nullptr, moe_s(st));
   }
@@ -545,14 +637,15 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   dim3 g((nrows + 3) / 4 + qblocks);
   const void* wx = Wx ? Wx->data : nullptr;
 #define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride)
-  // tokens per pass over a weight row: every row is read ceil(P / TT) times
   if (P <= 4) {
     if (E <= 512) { if (bf) RSM_GO(true, 4, 8); else RSM_GO(false, 4, 8); }
     else { if (bf) RSM_GO(true, 4, 16); else RSM_GO(false, 4, 16); }
-  } else if (P <= 8) {
-    if (bf) RSM_GO(true, 8, 16); else RSM_GO(false, 8, 16);
   } else {
-    if (bf) RSM_GO(true, 16, 16); else RSM_GO(false, 16, 16);
+#define RMD_GO(BF, PM) k_router_mid<BF, PM><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural)
+    if (P <= 8) { if (bf) RMD_GO(true, 8); else RMD_GO(false, 8); }
+    else if (P <= 16) { if (bf) RMD_GO(true, 16); else RMD_GO(false, 16); }
+    else { if (bf) RMD_GO(true, 32); else RMD_GO(false, 32); }
+#undef RMD_GO
   }
 #undef RSM_GO
   MOE_LAUNCH_CHECK();
