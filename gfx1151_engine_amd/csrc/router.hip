@@ -234,7 +234,7 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
       for (int i = 0; i < TT; i++)
 #pragma unroll
         for (int q = 0; q < 4; q++) acc[i][q] = 0.0;
-#pragma unroll 4
+#pragma unroll 12
       for (int c = lane * 4; c < d; c += 256) {
         float w[4];
         if (bf) {
@@ -637,7 +637,9 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   dim3 g((nrows + 3) / 4 + qblocks);
   const void* wx = Wx ? Wx->data : nullptr;
 #define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride)
-  if (P <= 4) {
+  if (P == 1 && E <= 512) {
+    if (bf) RSM_GO(true, 1, 8); else RSM_GO(false, 1, 8);
+  } else if (P <= 4) {
     if (E <= 512) { if (bf) RSM_GO(true, 4, 8); else RSM_GO(false, 4, 8); }
     else { if (bf) RSM_GO(true, 4, 16); else RSM_GO(false, 4, 16); }
   } else {
