@@ -55,7 +55,7 @@ struct moe_ctx {
   float2 *xmeta = nullptr, *hmeta = nullptr;
   int small_max = 32;         // batches up to this size take the in-place GEMV path
   bool int_decode = true;     // small batches: integer-dot kernels where they apply (else f32 kernels)
-  // batch path (allocated only when max_tokens > small_max)
+  // expert-sorted permutation (batch path; small batches that de-duplicate experts)
   moe_routing* routing = nullptr;
   __half* x16 = nullptr;      // [T][d]
   int* tokidx = nullptr;      // [(k+1)T] routed pairs then the shared expert's P pairs
@@ -67,6 +67,8 @@ struct moe_ctx {
   int max_tiles = 0;
   __half* hid16 = nullptr;    // [(k+1)T][mid]
   __half* pairs16 = nullptr;  // [(k+1)T][d]
+  float* pairs32 = nullptr;   // [(k+1)min(T,small_max)][d] unweighted pair rows of the unique-expert small-batch path
+  int uq_min = 0;             // > 0: small batches of at least this many tokens read every distinct expert once
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
   bool profile = false;
   hipEvent_t ev[MOE_PROF_STAGES + 1] = {};
@@ -101,7 +103,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   for (hipEvent_t e : c->ev)
     if (e) (void)hipEventDestroy(e);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
-                  c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16};
+                  c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16, c->pairs32};
   for (void* b : bufs)
     if (b) {
       hipError_t e = hipFree(b);
@@ -141,21 +143,27 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   if (e == hipSuccess) e = hipMalloc(&c->xmeta, Ts * moe_qvec_meta_bytes(cfg->d));
   if (e == hipSuccess) e = hipMalloc(&c->hplanes, Ts * (size_t)(cfg->topk + 1) * moe_qvec_plane_bytes(cfg->mid));
   if (e == hipSuccess) e = hipMalloc(&c->hmeta, Ts * (size_t)(cfg->topk + 1) * moe_qvec_meta_bytes(cfg->mid));
-  if (e == hipSuccess && T > (size_t)c->small_max) {
-    const size_t k1 = (size_t)cfg->topk + 1, d = cfg->d, mid = cfg->mid;
-    c->max_tiles = (int)((T * cfg->topk + 127) / 128 + E + (T + 127) / 128);
+  const size_t k1 = (size_t)cfg->topk + 1;
+  if (e == hipSuccess) {
+    // expert-sorted permutation: the batch path, and small batches that de-duplicate shared experts
+    const size_t batch_tiles = (T * cfg->topk + 127) / 128 + E + (T + 127) / 128, uq_tiles = Ts * cfg->topk + (Ts + 3) / 4;
+    c->max_tiles = (int)(batch_tiles > uq_tiles ? batch_tiles : uq_tiles);
     int rc = moe_routing_create((int)(T * cfg->topk), cfg->experts, &c->routing);
     if (rc != MOE_OK) {
       moe_destroy(c);
       return rc;
     }
-    e = hipMalloc(&c->x16, T * d * 2);
-    if (e == hipSuccess) e = hipMalloc(&c->tokidx, k1 * T * 4);
+    e = hipMalloc(&c->tokidx, k1 * T * 4);
     if (e == hipSuccess) e = hipMalloc(&c->pw, k1 * T * 4);
     if (e == hipSuccess) e = hipMalloc(&c->eoff, (E + 2) * 4);
     if (e == hipSuccess) e = hipMalloc(&c->pairids, T * cfg->topk * 4);
     if (e == hipSuccess) e = hipMalloc(&c->tiles, (size_t)c->max_tiles * sizeof(moe_tile));
     if (e == hipSuccess) e = hipMalloc(&c->ntiles, 8);
+    if (e == hipSuccess) e = hipMalloc(&c->pairs32, k1 * Ts * (size_t)cfg->d * 4);
+  }
+  if (e == hipSuccess && T > (size_t)c->small_max) {
+    const size_t d = cfg->d, mid = cfg->mid;
+    e = hipMalloc(&c->x16, T * d * 2);
     if (e == hipSuccess) e = hipMalloc(&c->hid16, k1 * T * mid * 2);
     if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);
   }
@@ -309,6 +317,10 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
   if (!c) return MOE_E_INVALID;
   switch (option) {
     case MOE_OPT_INT_DECODE: c->int_decode = value != 0; return MOE_OK;
+    case MOE_OPT_UNIQUE_MIN_TOKENS:
+      if (value < 0) return MOE_E_INVALID;
+      c->uq_min = value;
+      return MOE_OK;
     default: return MOE_E_INVALID;
   }
 }
@@ -365,6 +377,31 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   prof_mark(c, MOE_PROF_ROUTER, st);
   if (L.has_q4cp) {
     if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
+    if (use_int && c->uq_min > 0 && P >= c->uq_min) {
+      // verify-size batches: tokens share experts; walk the expert-sorted pair lists so that every
+      // distinct expert's weights are read once (reference: the _uq kernels, 26_kernels_moe_gguf.inc:758-877)
+      if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
+                                g.experts, g.id_stride, st)))
+        return rc;
+      const int sh_first = L.has_shared ? P * g.topk : -1;
+      if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 4, P, sh_first, c->tokidx, st)))
+        return rc;
+      prof_mark(c, MOE_PROF_ROUTE, st);
+      const int max_tiles = P * g.topk + (L.has_shared ? (P + 3) / 4 : 0);  // tiles of <= 4 pairs
+      if ((rc = moe_launch_dec_gu_uq(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
+                                     L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->tiles, c->ntiles,
+                                     max_tiles, c->tokidx, g.experts, g.d, g.mid, c->hplanes, c->hmeta, st)))
+        return rc;
+      prof_mark(c, MOE_PROF_UP, st);
+      if ((rc = moe_launch_dec_dn_uq(&L.down, L.has_shared ? &L.sh_down : nullptr, c->hplanes, c->hmeta, c->tiles,
+                                     c->ntiles, max_tiles, g.experts, g.d, g.mid, c->pairs32, st)))
+        return rc;
+      prof_mark(c, MOE_PROF_DOWN, st);
+      rc = moe_launch_reduce(c->pairs32, false, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
+                             sh_first, y, P, g.d, g.topk, moe_hscale{nullptr, 0.f, 0.f}, st);
+      prof_mark(c, MOE_PROF_REDUCE, st);
+      return rc;
+    }
     if (use_int) {
       // integer-dot kernels: activations as digit planes (made by the logits launch above)
       if ((rc = moe_launch_dec_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,

@@ -103,21 +103,38 @@ struct GuArgs2 {
 // rows of this block's 32; lane L holds activation groups L and 64 + (L & 31).  Rows are taken two
 // at a time with three 16-byte loads per lane: (row0, group L), (row1, group L), and the tail group
 // of row0 (lanes < 32) or row1 (lanes >= 32); all twelve loads of a wave are in flight together.
+// UQ ("unique experts", verify batches): grid (mid/32, tiles) instead; a tile = one expert with the
+// (token, expert) pairs routed to it (expert-sorted lists of the routing permutation; the shared
+// expert is the tile with expert id >= n_experts over all tokens).  The block reads its weight rows
+// once and walks the tile's pairs; hid planes are then indexed by pair position.
 constexpr int GU2_ROWS = 32;
+template <bool UQ>
 __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __restrict__ xplanes,
                                                 const float2* __restrict__ xmeta,
                                                 const int* __restrict__ ids, int id_stride, int kpt, int d,
                                                 int mid, uint32_t* __restrict__ hplanes,
-                                                float2* __restrict__ hmeta, float* __restrict__ hid_f32) {
+                                                float2* __restrict__ hmeta, float* __restrict__ hid_f32,
+                                                const moe_tile* __restrict__ tiles, const int* __restrict__ ntiles,
+                                                const int* __restrict__ tokidx, int n_experts) {
   __shared__ float gs[GU2_ROWS], us[GU2_ROWS];
   __shared__ uint32_t pk[QV4_GROUP_DW];
-  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int G = d / 32;
-  const bool shared = s >= kpt;
+  int s = blockIdx.y, nslots = gridDim.y, e = 0, first = 0, npairs = 1;
+  bool shared;
+  if (UQ) {
+    if ((int)blockIdx.y >= ntiles[0]) return;
+    const moe_tile tile = tiles[blockIdx.y];
+    shared = tile.expert >= n_experts;
+    e = shared ? 0 : tile.expert;
+    first = tile.first;
+    npairs = tile.count;
+  } else {
+    shared = s >= kpt;
+    e = shared ? 0 : ids[(size_t)blockIdx.z * id_stride + s];
+  }
   const DecW Wg = shared ? A.shg : A.gu;  // block-uniform choice, by value
   const DecW Wu = shared ? A.shu : A.gu;
-  const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
   const uint64_t grow0 = shared ? 0 : (uint64_t)e * 2 * mid;
   const uint64_t urow0 = shared ? 0 : (uint64_t)e * 2 * mid + mid;
   const int r0 = blockIdx.x * GU2_ROWS + 4 * wv;  // first of this wave's 4 gate rows
@@ -147,6 +164,8 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     }
   }
   const float ga = Wg.cb[1] - Wg.cb[0], gb = fmaf(8.f, ga, Wg.cb[0]), ua = Wu.cb[1] - Wu.cb[0], ub = fmaf(8.f, ua, Wu.cb[0]);
+  for (int pi = 0; pi < npairs; pi++) {
+  const int tok = UQ ? tokidx[first + pi] : (int)blockIdx.z;
   XG xa, xb;
   const size_t xbase = (size_t)tok * G;
   if (vA) load_xg(xa, xplanes, xmeta, xbase + gA);
@@ -184,7 +203,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     const int j = lane & 31;
     const float g = gs[j], u = us[j];
     const float hv = g / (1.f + expf(-g)) * u;
-    const size_t slot = (size_t)tok * nslots + s;
+    const size_t slot = UQ ? (size_t)(first + pi) : (size_t)tok * nslots + s;
     if (hid_f32 && lane < 32) hid_f32[slot * mid + blockIdx.x * GU2_ROWS + j] = hv;
     int p0, p1, p2, p3;
     float q, qsx;
@@ -204,6 +223,8 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     const size_t gi = slot * (mid / 32) + blockIdx.x;
     if (lane < QV4_GROUP_DW) hplanes[gi * QV4_GROUP_DW + lane] = pk[lane];
     if (lane == 0) hmeta[gi] = make_float2(q, qsx);
+  }
+  if (UQ) __syncthreads();  // gs / us / pk are reused by the next pair
   }
 }
 
@@ -274,6 +295,49 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
   }
 }
 
+// Down projection of the unique-expert path: grid (d/32, tiles), block 256 = 8 half-waves of 4 rows.
+// Lane g of a half-wave holds group g of its 4 weight rows and walks the tile's pairs; the
+// unweighted row results go to pairs[pair][row] (f32) for the weighted combine that follows.
+constexpr int DU_ROWS = 32;
+__global__ void __launch_bounds__(256) k_dec_dn_uq(DnArgs2 A, const uint32_t* __restrict__ hplanes,
+                                                   const float2* __restrict__ hmeta,
+                                                   const moe_tile* __restrict__ tiles,
+                                                   const int* __restrict__ ntiles, int n_experts, int d, int mid,
+                                                   float* __restrict__ pairs) {
+  if ((int)blockIdx.y >= ntiles[0]) return;
+  const moe_tile tile = tiles[blockIdx.y];
+  const bool shared = tile.expert >= n_experts;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int G = mid / 32, g = lane & 31, hw = 2 * wv + (lane >> 5);
+  const bool live = g < G;
+  const size_t rb = (size_t)mid / 2;
+  const DecW W = shared ? A.shd : A.dn;  // block-uniform, by value
+  const int r0 = blockIdx.x * DU_ROWS + 4 * hw;
+  const uint64_t row0 = (shared ? 0 : (uint64_t)tile.expert * d) + r0;
+  const uint8_t* cp = W.codes + row0 * rb + (size_t)g * 16;
+  const uint8_t* sp = W.scales + row0 * W.ss + g * 2;
+  uint4 cw[4];
+  float sc[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    if (live) {
+      cw[r] = *(const uint4*)(cp + r * rb);
+      sc[r] = __half2float(*(const __half*)(sp + r * W.ss));
+    }
+  }
+  const float a = W.cb[1] - W.cb[0], b = fmaf(8.f, a, W.cb[0]);
+  for (int pi = 0; pi < tile.count; pi++) {
+    const size_t pr = (size_t)tile.first + pi;
+    XG x;
+    if (live) load_xg(x, hplanes, hmeta, pr * G + g);
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+      const float v = sum32(live ? sc[r] * chunk_dot(cw[r], x, a, b) : 0.f);
+      if (g == 0) pairs[pr * d + r0 + r] = v;
+    }
+  }
+}
+
 DecW decw(const moe_wview* w) {
   DecW o{};
   if (w) {
@@ -291,7 +355,7 @@ size_t moe_qvec_meta_bytes(int K) { return (size_t)(K / 32) * sizeof(float2); }
 // Supported shapes of the integer-dot decode kernels (otherwise the caller uses the f32 kernels).
 bool moe_dec_supported(int d, int mid, int nslots) {
   return d % 32 == 0 && d / 32 <= 96 && mid % 32 == 0 && mid / 32 <= 32 && nslots <= DN2_MAXSLOTS &&
-         mid % GU2_ROWS == 0 && d % DN2_ROWS == 0;
+         mid % GU2_ROWS == 0 && d % DN2_ROWS == 0 && d % DU_ROWS == 0;
 }
 
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
@@ -312,7 +376,39 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
-  k_dec_gu<<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32);
+  k_dec_gu<false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
+                                        nullptr, nullptr, nullptr, 0);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// Unique-expert variants: tiles / ntiles / tokidx from the routing permutation (tiles of <= 32 pairs,
+// the shared expert as expert id n_experts); hplanes / hmeta and pairs are indexed by pair position.
+int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
+                         const uint32_t* xplanes, const float2* xmeta, const moe_tile* tiles, const int* ntiles,
+                         int max_tiles, const int* tokidx, int n_experts, int d, int mid, uint32_t* hplanes,
+                         float2* hmeta, hipStream_t st) {
+  GuArgs2 A{};
+  A.gu = decw(gu);
+  A.shg = decw(sh_gate);
+  A.shu = decw(sh_up);
+  if (max_tiles <= 0) return MOE_OK;
+  dim3 grid(mid / GU2_ROWS, max_tiles);
+  k_dec_gu<true><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
+                                       ntiles, tokidx, n_experts);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_dec_dn_uq(const moe_wview* dn, const moe_wview* sh_down, const uint32_t* hplanes,
+                         const float2* hmeta, const moe_tile* tiles, const int* ntiles, int max_tiles,
+                         int n_experts, int d, int mid, float* pairs, hipStream_t st) {
+  DnArgs2 A{};
+  A.dn = decw(dn);
+  A.shd = decw(sh_down);
+  if (max_tiles <= 0) return MOE_OK;
+  dim3 grid(d / DU_ROWS, max_tiles);
+  k_dec_dn_uq<<<grid, 256, 0, st>>>(A, hplanes, hmeta, tiles, ntiles, n_experts, d, mid, pairs);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -46,6 +46,13 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
                       hipStream_t st);
+int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
+                         const uint32_t* xplanes, const float2* xmeta, const moe_tile* tiles, const int* ntiles,
+                         int max_tiles, const int* tokidx, int n_experts, int d, int mid, uint32_t* hplanes,
+                         float2* hmeta, hipStream_t st);
+int moe_launch_dec_dn_uq(const moe_wview* dn, const moe_wview* sh_down, const uint32_t* hplanes,
+                         const float2* hmeta, const moe_tile* tiles, const int* ntiles, int max_tiles,
+                         int n_experts, int d, int mid, float* pairs, hipStream_t st);
 // the same for raw GGUF Q4_K rows (activation planes in natural order)
 bool moe_dec4k_supported(int d, int mid, int nslots);
 int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,

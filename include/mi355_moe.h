@@ -196,7 +196,12 @@ int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_st
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
  * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as
  * three 7-bit digit planes per 32-group, 21 significant bits) instead of the f32 FMA kernels. */
-enum { MOE_OPT_INT_DECODE = 1 };
+/* MOE_OPT_UNIQUE_MIN_TOKENS (default 0 = off): q4cp batches of at least this many tokens (and at most 32) walk
+ * the expert-sorted pair lists, so that an expert shared by several tokens is read once
+ * (the reference's _uq decode kernels, src/gpu/parts/26_kernels_moe_gguf.inc:758-877).  Pays when most
+ * tokens of a speculative-verify batch agree on their experts; off by default because with little sharing the
+ * extra permutation launches cost more than the saved reads. */
+enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP

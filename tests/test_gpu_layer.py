@@ -65,6 +65,32 @@ def test_int_decode_switch(oracle, fmt, T):
     m.close()
 
 
+@pytest.mark.parametrize("share", [0.3, 1.0])
+def test_unique_expert_path(oracle, share):
+    """MOE_OPT_UNIQUE_MIN_TOKENS: a verify-size batch through the expert-sorted pair lists (every distinct
+    expert read once) gives the same experts and, within the GEMV bar, the same output."""
+    import torch
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(91)
+    d, mid, E, k, T = 3072, 768, 24, 10, 20
+    hl = HostLayer(rng, d, mid, E, k)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    n = int(round(share * T))
+    for i in range(1, n):  # drafted tokens that reproduce the template token's routing
+        x[i] = x[0] + 1e-3 * rng.standard_normal(d).astype(np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=32)
+    m.set_option(capi.OPT_UNIQUE_MIN_TOKENS, 8)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    ids, _ = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    assert max_abs_rel(y, yo) <= TOL_GEMV, max_abs_rel(y, yo)
+    m.set_option(capi.OPT_UNIQUE_MIN_TOKENS, 0)
+    y2 = m.forward(0, gpu(x)).cpu().numpy()
+    assert max_abs_rel(y2, yo) <= TOL_GEMV
+    m.close()
+
+
 def test_golden_layers_from_reference(oracle, golden):
     """Inputs and outputs of the reference's own Model::moe (tests/golden/moe_layer.npz)."""
     import torch
