@@ -356,13 +356,12 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
     const double w0 = (double)wr.x, w1 = (double)wr.y;
     __syncthreads();
     if (c0 + RM_C < d) fetch(c0 + RM_C);
+    // rows past P hold zeros: no predicate, so the LDS reads of a slab go out back to back
 #pragma unroll
     for (int t = 0; t < PMAX; t++) {
-      if (t < P) {
-        const double2 xv = *(const double2*)&Xd[t][2 * lane];
-        acc[t][0] = fma(w0, xv.x, acc[t][0]);
-        acc[t][1] = fma(w1, xv.y, acc[t][1]);
-      }
+      const double2 xv = *(const double2*)&Xd[t][2 * lane];
+      acc[t][0] = fma(w0, xv.x, acc[t][0]);
+      acc[t][1] = fma(w1, xv.y, acc[t][1]);
     }
   }
 #pragma unroll
@@ -646,6 +645,7 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
 #define RMD_GO(BF, PM) k_router_mid<BF, PM><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural)
     if (P <= 8) { if (bf) RMD_GO(true, 8); else RMD_GO(false, 8); }
     else if (P <= 16) { if (bf) RMD_GO(true, 16); else RMD_GO(false, 16); }
+    else if (P <= 24) { if (bf) RMD_GO(true, 24); else RMD_GO(false, 24); }
     else { if (bf) RMD_GO(true, 32); else RMD_GO(false, 32); }
 #undef RMD_GO
   }
