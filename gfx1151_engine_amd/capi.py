@@ -324,3 +324,80 @@ class Moe:
             self.close()
         except Exception:
             pass
+
+
+# ---- checkpoint files ----
+
+class TensorInfo(C.Structure):
+    _fields_ = [("dtype", C.c_int), ("ndims", C.c_uint32), ("dims", C.c_uint64 * 4), ("data", C.c_void_p),
+                ("nbytes", C.c_uint64)]
+
+
+FILE_HGN, FILE_GGUF = 1, 2
+
+
+class ModelFile:
+    """moe_file: a .hgn or GGUF file mapped read-only (host only, no GPU needed)."""
+
+    def __init__(self, path):
+        self.h = C.c_void_p()
+        check(lib().moe_file_open(str(path).encode(), C.byref(self.h)), f"moe_file_open({path})")
+
+    @property
+    def format(self):
+        return lib().moe_file_format(self.h)
+
+    def __len__(self):
+        lib().moe_file_tensor_count.restype = C.c_int64
+        return lib().moe_file_tensor_count(self.h)
+
+    def find(self, name):
+        """-> (dtype, dims tuple, bytes as a numpy uint8 copy) or None"""
+        import numpy as np
+        ti = TensorInfo()
+        rc = lib().moe_file_find(self.h, name.encode(), C.byref(ti))
+        if rc == -3:
+            return None
+        check(rc, "moe_file_find")
+        data = np.ctypeslib.as_array(C.cast(ti.data, C.POINTER(C.c_uint8)), shape=(ti.nbytes,)).copy() if ti.nbytes else \
+            np.zeros(0, np.uint8)
+        return ti.dtype, tuple(ti.dims[i] for i in range(ti.ndims)), data
+
+    def config(self, layer=0):
+        cfg = Config()
+        check(lib().moe_file_config(self.h, layer, C.byref(cfg)), "moe_file_config")
+        return cfg
+
+    def load_layers(self, moe, file_layer0, ctx_layer0, n_layers):
+        """-> opaque weights handle (keep it alive as long as the context uses the layers)"""
+        w = C.c_void_p()
+        check(lib().moe_load_layers(moe.h, self.h, file_layer0, ctx_layer0, n_layers, C.byref(w), stream()),
+              "moe_load_layers")
+        return Weights(w)
+
+    def close(self):
+        if self.h:
+            lib().moe_file_close(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class Weights:
+    def __init__(self, h):
+        self.h = h
+
+    @property
+    def nbytes(self):
+        lib().moe_weights_bytes.restype = C.c_uint64
+        return lib().moe_weights_bytes(self.h)
+
+    def free(self):
+        if self.h:
+            check(lib().moe_weights_free(self.h), "moe_weights_free")
+            self.h = None
+

@@ -313,6 +313,13 @@ static int magnitude_constant(moe_ctx* c, bool q4k, const moe_wview* gate, uint6
   return MOE_OK;
 }
 
+MOE_API int moe_clear_layer(moe_ctx* c, int layer) {
+  MoeLayer* L = layer_of(c, layer);
+  if (!L) return MOE_E_INVALID;
+  *L = MoeLayer();
+  return MOE_OK;
+}
+
 MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
   if (!c) return MOE_E_INVALID;
   switch (option) {

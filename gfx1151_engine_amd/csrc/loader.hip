@@ -1,0 +1,461 @@
+// Checkpoint files -> HBM: reads the MoE tensors of a .hgn (HGN1) or GGUF file and registers them in a
+// context.  Host code only: the file is mapped read-only, every tensor of the path is copied to
+// device memory once (one allocation per tensor, bytes unchanged) and handed to moe_set_*.
+// On the reference's APU the experts are read in place from registered host memory; here they
+// are resident in HBM.
+// (reference: src/hgn.h:48-76,295-363 header / record layout and map_file; src/gguf.h:225-314 GGUF
+//  header, key-value section, tensor infos; tensor names src/gpu/parts/40_model.inc:1808-1857,
+//  src/gpu/parts/30_host_util.inc:384-412, src/gguf_map.h:210-214)
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cstring>
+#include <new>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "common.h"
+
+namespace {
+
+struct FTensor {
+  int dtype = 0;  // hgn dtype or ggml type
+  uint32_t nd = 0;
+  uint64_t dims[4] = {1, 1, 1, 1};  // hgn: outermost first (cols last); gguf: ne[] (cols first)
+  const uint8_t* data = nullptr;
+  uint64_t nbytes = 0;
+};
+
+#pragma pack(push, 1)
+struct HgnHeader {  // src/hgn.h:48-54
+  char magic[4];
+  uint32_t version, tensor_count, reserved;
+  uint64_t records_offset, data_offset, file_size;
+  char model_name[64];
+};
+struct HgnRecord {  // src/hgn.h:55-60
+  char name[96];
+  uint32_t dtype, ndims;
+  uint64_t dims[4];
+  uint64_t data_offset, data_size, extra;
+};
+#pragma pack(pop)
+static_assert(sizeof(HgnHeader) == 104 && sizeof(HgnRecord) == 160, "HGN1 on-disk structs");
+
+// ggml block geometry (src/gguf.h:42-64): elements per block, bytes per block
+bool ggml_block(uint32_t t, uint32_t& be, uint32_t& bb) {
+  switch (t) {
+    case 0: be = 1; bb = 4; return true;     // F32
+    case 1: case 30: be = 1; bb = 2; return true;  // F16, BF16
+    case 24: be = 1; bb = 1; return true;    // I8
+    case 25: be = 1; bb = 2; return true;    // I16
+    case 26: be = 1; bb = 4; return true;    // I32
+    case 27: case 28: be = 1; bb = 8; return true;  // I64, F64
+    case 2: be = 32; bb = 18; return true;   // Q4_0
+    case 3: be = 32; bb = 20; return true;   // Q4_1
+    case 6: be = 32; bb = 22; return true;   // Q5_0
+    case 7: be = 32; bb = 24; return true;   // Q5_1
+    case 8: be = 32; bb = 34; return true;   // Q8_0
+    case 20: be = 32; bb = 18; return true;  // IQ4_NL
+    case 10: be = 256; bb = 84; return true;   // Q2_K
+    case 11: be = 256; bb = 110; return true;  // Q3_K
+    case 12: be = 256; bb = 144; return true;  // Q4_K
+    case 13: be = 256; bb = 176; return true;  // Q5_K
+    case 14: be = 256; bb = 210; return true;  // Q6_K
+    case 23: be = 256; bb = 136; return true;  // IQ4_XS
+    default: be = bb = 0; return false;
+  }
+}
+
+struct Cur {  // bounds-checked little-endian reader over the mapped header
+  const uint8_t *p, *end;
+  bool ok = true;
+  template <class T>
+  T get() {
+    T v{};
+    if (!ok || (size_t)(end - p) < sizeof(T)) { ok = false; return v; }
+    memcpy(&v, p, sizeof(T));
+    p += sizeof(T);
+    return v;
+  }
+  std::string str() {
+    const uint64_t n = get<uint64_t>();
+    if (!ok || (uint64_t)(end - p) < n) { ok = false; return {}; }
+    std::string s((const char*)p, (size_t)n);
+    p += n;
+    return s;
+  }
+  void skip(uint64_t n) {
+    if (!ok || (uint64_t)(end - p) < n) { ok = false; return; }
+    p += n;
+  }
+};
+
+// size of a scalar GGUF value type, 0 for string (8) / array (9) / unknown
+uint32_t gguf_scalar_bytes(uint32_t t) {
+  switch (t) {
+    case 0: case 1: case 7: return 1;
+    case 2: case 3: return 2;
+    case 4: case 5: case 6: return 4;
+    case 10: case 11: case 12: return 8;
+    default: return 0;
+  }
+}
+
+}  // namespace
+
+struct moe_file {
+  int format = 0;
+  int fd = -1;
+  const uint8_t* base = nullptr;
+  size_t len = 0;
+  std::unordered_map<std::string, FTensor> idx;
+  std::unordered_map<std::string, int64_t> kv_int;  // GGUF integer metadata
+};
+
+struct moe_weights {
+  std::vector<void*> dev;
+  uint64_t bytes = 0;
+};
+
+static int parse_hgn(moe_file* f) {
+  if (f->len < sizeof(HgnHeader)) return MOE_E_INVALID;
+  HgnHeader h;
+  memcpy(&h, f->base, sizeof h);
+  if (h.file_size != f->len) return MOE_E_INVALID;  // the reference rejects a size mismatch too
+  if (h.records_offset > f->len || (uint64_t)h.tensor_count * sizeof(HgnRecord) > f->len - h.records_offset)
+    return MOE_E_INVALID;
+  for (uint32_t i = 0; i < h.tensor_count; i++) {
+    HgnRecord r;
+    memcpy(&r, f->base + h.records_offset + (uint64_t)i * sizeof r, sizeof r);
+    if (r.data_offset > f->len || r.data_size > f->len - r.data_offset || r.ndims > 4) return MOE_E_INVALID;
+    FTensor t;
+    t.dtype = (int)r.dtype;
+    t.nd = r.ndims;
+    for (int k = 0; k < 4; k++) t.dims[k] = k < (int)r.ndims ? r.dims[k] : 1;
+    t.data = f->base + r.data_offset;
+    t.nbytes = r.data_size;
+    f->idx.emplace(std::string(r.name, strnlen(r.name, sizeof r.name)), t);  // first record of a name wins
+  }
+  return MOE_OK;
+}
+
+static int parse_gguf(moe_file* f) {
+  Cur c{f->base + 4, f->base + f->len};
+  const uint32_t ver = c.get<uint32_t>();
+  if (!c.ok || ver < 2) return MOE_E_UNSUPPORTED;
+  const uint64_t nt = c.get<uint64_t>(), nkv = c.get<uint64_t>();
+  uint64_t align = 32;
+  for (uint64_t i = 0; i < nkv && c.ok; i++) {
+    const std::string key = c.str();
+    uint32_t t = c.get<uint32_t>();
+    if (t == 9) {  // array: element type, count, elements
+      const uint32_t et = c.get<uint32_t>();
+      const uint64_t n = c.get<uint64_t>();
+      if (et == 8) {
+        for (uint64_t j = 0; j < n && c.ok; j++) (void)c.str();
+      } else {
+        const uint32_t sz = gguf_scalar_bytes(et);
+        if (!sz) return MOE_E_INVALID;
+        c.skip(n * sz);
+      }
+    } else if (t == 8) {
+      (void)c.str();
+    } else {
+      const uint32_t sz = gguf_scalar_bytes(t);
+      if (!sz) return MOE_E_INVALID;
+      int64_t v = 0;
+      bool is_int = true;
+      switch (t) {
+        case 0: v = c.get<uint8_t>(); break;
+        case 1: v = c.get<int8_t>(); break;
+        case 2: v = c.get<uint16_t>(); break;
+        case 3: v = c.get<int16_t>(); break;
+        case 4: v = c.get<uint32_t>(); break;
+        case 5: v = c.get<int32_t>(); break;
+        case 7: v = c.get<uint8_t>(); break;
+        case 10: v = (int64_t)c.get<uint64_t>(); break;
+        case 11: v = c.get<int64_t>(); break;
+        default: c.skip(sz); is_int = false; break;  // floats
+      }
+      if (is_int) f->kv_int[key] = v;
+    }
+  }
+  if (!c.ok) return MOE_E_INVALID;
+  if (auto it = f->kv_int.find("general.alignment"); it != f->kv_int.end() && it->second > 0) align = (uint64_t)it->second;
+  struct Pending { std::string name; FTensor t; uint64_t off; };
+  std::vector<Pending> ts;
+  for (uint64_t i = 0; i < nt && c.ok; i++) {
+    Pending p;
+    p.name = c.str();
+    p.t.nd = c.get<uint32_t>();
+    if (p.t.nd > 4) return MOE_E_INVALID;
+    for (uint32_t k = 0; k < p.t.nd; k++) p.t.dims[k] = c.get<uint64_t>();
+    p.t.dtype = (int)c.get<uint32_t>();
+    p.off = c.get<uint64_t>();
+    ts.push_back(std::move(p));
+  }
+  if (!c.ok) return MOE_E_INVALID;
+  const uint64_t hdr = (uint64_t)(c.p - f->base), data0 = (hdr + align - 1) / align * align;
+  for (auto& p : ts) {
+    uint32_t be, bb;
+    if (!ggml_block((uint32_t)p.t.dtype, be, bb)) return MOE_E_UNSUPPORTED;
+    const uint64_t numel = p.t.dims[0] * p.t.dims[1] * p.t.dims[2] * p.t.dims[3];
+    if (p.t.dims[0] % be) return MOE_E_INVALID;
+    p.t.nbytes = numel / be * bb;
+    const uint64_t off = data0 + p.off;
+    if (off > f->len || p.t.nbytes > f->len - off) return MOE_E_INVALID;
+    p.t.data = f->base + off;
+    if (!f->idx.emplace(p.name, p.t).second) return MOE_E_INVALID;  // duplicate name
+  }
+  return MOE_OK;
+}
+
+MOE_API int moe_file_close(moe_file* f) {
+  if (!f) return MOE_OK;
+  if (f->base) munmap((void*)f->base, f->len);
+  if (f->fd >= 0) close(f->fd);
+  delete f;
+  return MOE_OK;
+}
+
+MOE_API int moe_file_open(const char* path, moe_file** out) {
+  if (!path || !out) return MOE_E_INVALID;
+  moe_file* f = new (std::nothrow) moe_file();
+  if (!f) return MOE_E_STATE;
+  f->fd = open(path, O_RDONLY | O_CLOEXEC);
+  struct stat st;
+  if (f->fd < 0 || fstat(f->fd, &st) < 0 || st.st_size < 8) {
+    moe_file_close(f);
+    return MOE_E_INVALID;
+  }
+  f->len = (size_t)st.st_size;
+  void* p = mmap(nullptr, f->len, PROT_READ, MAP_PRIVATE, f->fd, 0);
+  if (p == MAP_FAILED) {
+    f->base = nullptr;
+    moe_file_close(f);
+    return MOE_E_STATE;
+  }
+  f->base = (const uint8_t*)p;
+  int rc;
+  if (memcmp(f->base, "HGN1", 4) == 0) {
+    f->format = MOE_FILE_HGN;
+    rc = parse_hgn(f);
+  } else if (memcmp(f->base, "GGUF", 4) == 0) {
+    f->format = MOE_FILE_GGUF;
+    rc = parse_gguf(f);
+  } else {
+    rc = MOE_E_UNSUPPORTED;
+  }
+  if (rc != MOE_OK) {
+    moe_file_close(f);
+    return rc;
+  }
+  *out = f;
+  return MOE_OK;
+}
+
+MOE_API int moe_file_format(const moe_file* f) { return f ? f->format : 0; }
+MOE_API int64_t moe_file_tensor_count(const moe_file* f) { return f ? (int64_t)f->idx.size() : 0; }
+
+MOE_API int moe_file_find(const moe_file* f, const char* name, moe_tensor_info* out) {
+  if (!f || !name || !out) return MOE_E_INVALID;
+  auto it = f->idx.find(name);
+  if (it == f->idx.end()) return MOE_E_STATE;
+  out->dtype = it->second.dtype;
+  out->ndims = it->second.nd;
+  for (int k = 0; k < 4; k++) out->dims[k] = it->second.dims[k];
+  out->data = it->second.data;
+  out->nbytes = it->second.nbytes;
+  return MOE_OK;
+}
+
+namespace {
+
+const FTensor* find(const moe_file* f, const char* fmt, int layer) {
+  char n[128];
+  snprintf(n, sizeof n, fmt, layer);
+  auto it = f->idx.find(n);
+  return it == f->idx.end() ? nullptr : &it->second;
+}
+
+// rows x cols of a matrix tensor: hgn dims are outermost first (3-D fused experts flatten to
+// [E*rows, cols], src/hgn.h:7-8), gguf ne[] is innermost first
+void matrix_shape(int format, const FTensor& t, uint64_t& rows, uint64_t& cols) {
+  if (format == MOE_FILE_HGN) {
+    cols = t.dims[t.nd ? t.nd - 1 : 0];
+    rows = 1;
+    for (uint32_t k = 0; k + 1 < t.nd; k++) rows *= t.dims[k];
+  } else {
+    cols = t.dims[0];
+    rows = t.dims[1] * t.dims[2] * t.dims[3];
+  }
+}
+
+}  // namespace
+
+// Shapes of the path read off the tensors of layer `layer`: d, mid, experts; layers = the number of
+// consecutive layers from `layer` on that carry the expert tensors.  topk is not stored in a .hgn
+// file; GGUF files carry "<arch>.expert_used_count".  max_tokens / id_stride are left untouched.
+MOE_API int moe_file_config(const moe_file* f, int layer, moe_config* cfg) {
+  if (!f || !cfg || layer < 0) return MOE_E_INVALID;
+  const bool hgn = f->format == MOE_FILE_HGN;
+  const char* dn_name = hgn ? "layers.%d.mlp.experts.down_proj.weight" : "blk.%d.ffn_down_exps.weight";
+  const FTensor* dn = find(f, dn_name, layer);
+  if (!dn) return MOE_E_STATE;
+  if (hgn) {
+    // [E, d, mid] (or flat [E*d, mid] with the router giving E)
+    const FTensor* rt = find(f, "layers.%d.mlp.gate.weight", layer);
+    if (!rt || rt->nd != 2) return MOE_E_STATE;
+    uint64_t rows, cols;
+    matrix_shape(f->format, *dn, rows, cols);
+    cfg->experts = (int)rt->dims[0];
+    cfg->d = (int)rt->dims[1];
+    cfg->mid = (int)cols;
+    if (rows != (uint64_t)cfg->experts * cfg->d) return MOE_E_INVALID;
+  } else {
+    if (dn->nd != 3) return MOE_E_INVALID;
+    cfg->mid = (int)dn->dims[0];
+    cfg->d = (int)dn->dims[1];
+    cfg->experts = (int)dn->dims[2];
+    for (auto& kv : f->kv_int)
+      if (kv.first.size() > 18 && kv.first.compare(kv.first.size() - 18, 18, ".expert_used_count") == 0)
+        cfg->topk = (int)kv.second;
+  }
+  int n = 0;
+  while (find(f, dn_name, layer + n)) n++;
+  cfg->layers = n;
+  return MOE_OK;
+}
+
+namespace {
+
+int upload(moe_weights* w, const FTensor& t, hipStream_t st, const uint8_t** dev) {
+  void* p = nullptr;
+  MOE_HIP(hipMalloc(&p, t.nbytes ? t.nbytes : 1));
+  w->dev.push_back(p);
+  w->bytes += t.nbytes;
+  // pageable source (the file mapping): staged by the runtime; set-up work, so a plain copy
+  (void)st;
+  MOE_HIP(hipMemcpy(p, t.data, t.nbytes, hipMemcpyHostToDevice));
+  *dev = (const uint8_t*)p;
+  return MOE_OK;
+}
+
+int hgn_dtype_ok_dense(int dt) { return dt == MOE_DT_BF16 || dt == MOE_DT_F32; }
+
+int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st) {
+  const FTensor* rt = find(f, "layers.%d.mlp.gate.weight", fl);
+  const FTensor* gu = find(f, "layers.%d.mlp.experts.gate_up_proj.weight", fl);
+  const FTensor* dn = find(f, "layers.%d.mlp.experts.down_proj.weight", fl);
+  if (!rt || !gu || !dn) return MOE_E_STATE;
+  if (!hgn_dtype_ok_dense(rt->dtype) || gu->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP) return MOE_E_UNSUPPORTED;
+  int rc;
+  auto view = [&](const FTensor& t, moe_wview* v) -> int {
+    uint64_t rows, cols;
+    matrix_shape(MOE_FILE_HGN, t, rows, cols);
+    v->dtype = t.dtype;
+    v->rows = rows;
+    v->cols = cols;
+    v->scale_stride = t.dtype == MOE_DT_Q4CP ? (((cols / 32 * 2) + 15) & ~15ULL) : 0;
+    return upload(w, t, st, &v->data);
+  };
+  moe_wview vr{}, vgu{}, vdn{};
+  if ((rc = view(*rt, &vr)) || (rc = view(*gu, &vgu)) || (rc = view(*dn, &vdn))) return rc;
+  if ((rc = moe_set_router(ctx, cl, &vr, nullptr))) return rc;
+  if ((rc = moe_set_experts_q4cp(ctx, cl, &vgu, &vdn))) return rc;
+  const FTensor* sg = find(f, "layers.%d.mlp.shared_expert.gate_proj.weight", fl);
+  if (sg) {
+    const FTensor* su = find(f, "layers.%d.mlp.shared_expert.up_proj.weight", fl);
+    const FTensor* sd = find(f, "layers.%d.mlp.shared_expert.down_proj.weight", fl);
+    const FTensor* sx = find(f, "layers.%d.mlp.shared_expert_gate.weight", fl);
+    if (!su || !sd || !sx) return MOE_E_STATE;
+    // the shared expert of this path is q4cp; bf16 / q8 shared experts stay with the caller's dense kernels
+    if (sg->dtype != MOE_DT_Q4CP || su->dtype != MOE_DT_Q4CP || sd->dtype != MOE_DT_Q4CP || !hgn_dtype_ok_dense(sx->dtype))
+      return MOE_E_UNSUPPORTED;
+    moe_wview a{}, b{}, c2{}, d2{};
+    if ((rc = view(*sg, &a)) || (rc = view(*su, &b)) || (rc = view(*sd, &c2)) || (rc = view(*sx, &d2))) return rc;
+    if ((rc = moe_set_shared(ctx, cl, &a, &b, &c2, &d2, 0))) return rc;
+  }
+  return MOE_OK;
+}
+
+int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st) {
+  const FTensor* rt = find(f, "blk.%d.ffn_gate_inp.weight", fl);
+  const FTensor* g = find(f, "blk.%d.ffn_gate_exps.weight", fl);
+  const FTensor* u = find(f, "blk.%d.ffn_up_exps.weight", fl);
+  const FTensor* dn = find(f, "blk.%d.ffn_down_exps.weight", fl);
+  if (!rt || !g || !u || !dn) return MOE_E_STATE;
+  if (rt->dtype != 0 && rt->dtype != 30) return MOE_E_UNSUPPORTED;  // F32 / BF16 router
+  int rc;
+  moe_wview vr{};
+  vr.dtype = rt->dtype == 0 ? MOE_DT_F32 : MOE_DT_BF16;
+  vr.cols = rt->dims[0];
+  vr.rows = rt->dims[1];
+  if ((rc = upload(w, *rt, st, &vr.data))) return rc;
+  if ((rc = moe_set_router(ctx, cl, &vr, nullptr))) return rc;
+  moe_gg_experts gg{};
+  gg.tgu = g->dtype;
+  gg.tdn = dn->dtype;
+  if (u->dtype != g->dtype) return MOE_E_UNSUPPORTED;
+  if ((rc = upload(w, *g, st, &gg.gate)) || (rc = upload(w, *u, st, &gg.up)) || (rc = upload(w, *dn, st, &gg.down))) return rc;
+  if ((rc = moe_set_experts_gguf(ctx, cl, &gg))) return rc;  // MOE_E_UNSUPPORTED for types other than Q4_K
+  const FTensor* sg = find(f, "blk.%d.ffn_gate_shexp.weight", fl);
+  if (sg) {
+    const FTensor* su = find(f, "blk.%d.ffn_up_shexp.weight", fl);
+    const FTensor* sd = find(f, "blk.%d.ffn_down_shexp.weight", fl);
+    const FTensor* sx = find(f, "blk.%d.ffn_gate_inp_shexp.weight", fl);
+    if (!su || !sd || !sx) return MOE_E_STATE;
+    if (sg->dtype != MOE_GGML_Q4_K || su->dtype != MOE_GGML_Q4_K || sd->dtype != MOE_GGML_Q4_K ||
+        (sx->dtype != 0 && sx->dtype != 30))
+      return MOE_E_UNSUPPORTED;
+    moe_wview a{}, b{}, c2{}, d2{};
+    auto raw = [&](const FTensor& t, moe_wview* v) -> int {
+      v->dtype = 0;
+      v->cols = t.dims[0];
+      v->rows = t.dims[1];
+      return upload(w, t, st, &v->data);
+    };
+    if ((rc = raw(*sg, &a)) || (rc = raw(*su, &b)) || (rc = raw(*sd, &c2)) || (rc = raw(*sx, &d2))) return rc;
+    d2.dtype = sx->dtype == 0 ? MOE_DT_F32 : MOE_DT_BF16;
+    d2.rows = 1;
+    if ((rc = moe_set_shared(ctx, cl, &a, &b, &c2, &d2, MOE_GGML_Q4_K))) return rc;
+  }
+  return MOE_OK;
+}
+
+}  // namespace
+
+MOE_API int moe_weights_free(moe_weights* w) {
+  if (!w) return MOE_OK;
+  int rc = MOE_OK;
+  for (void* p : w->dev) {
+    const hipError_t e = hipFree(p);
+    if (e != hipSuccess && rc == MOE_OK) rc = (int)e;
+  }
+  delete w;
+  return rc;
+}
+
+MOE_API uint64_t moe_weights_bytes(const moe_weights* w) { return w ? w->bytes : 0; }
+
+MOE_API int moe_load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, int ctx_layer0, int n_layers,
+                            moe_weights** out, moe_stream_t st) {
+  if (!ctx || !f || !out || file_layer0 < 0 || ctx_layer0 < 0 || n_layers < 1) return MOE_E_INVALID;
+  moe_weights* w = new (std::nothrow) moe_weights();
+  if (!w) return MOE_E_STATE;
+  for (int i = 0; i < n_layers; i++) {
+    const int rc = f->format == MOE_FILE_HGN ? load_layer_hgn(ctx, f, file_layer0 + i, ctx_layer0 + i, w, moe_s(st))
+                                             : load_layer_gguf(ctx, f, file_layer0 + i, ctx_layer0 + i, w, moe_s(st));
+    if (rc != MOE_OK) {
+      for (int j = 0; j <= i; j++) (void)moe_clear_layer(ctx, ctx_layer0 + j);  // no layer keeps a freed pointer
+      moe_weights_free(w);
+      return rc;
+    }
+  }
+  *out = w;
+  return MOE_OK;
+}

@@ -1,0 +1,113 @@
+"""Writers for small synthetic checkpoint files in the engine's two formats (tests, examples).
+
+  HGN1 (.hgn): 104-byte header, 160-byte tensor records, data  (reference: src/hgn.h:48-76,295-363)
+  GGUF v3:      header, key-value section, tensor infos, aligned data  (reference: src/gguf.h:225-314)
+
+The byte layouts of the tensors themselves are synth.make_q4cp / synth.make_q4k and plain bf16 / f32.
+"""
+import struct
+
+import numpy as np
+
+HGN_BF16, HGN_F32, HGN_Q4CP = 0, 1, 5
+GGML_F32, GGML_BF16, GGML_Q4_K = 0, 30, 12
+_GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144)}
+
+
+def _bytes(a):
+    return np.ascontiguousarray(a).view(np.uint8).reshape(-1).tobytes()
+
+
+def write_hgn(path, tensors, model_name="synthetic", align=64):
+    """tensors: list of (name, dtype, dims, array of raw bytes).  dims are outermost first."""
+    n = len(tensors)
+    rec_off = 104
+    data_off = (rec_off + 160 * n + align - 1) // align * align
+    blobs, recs, off = [], [], data_off
+    for name, dtype, dims, data in tensors:
+        b = _bytes(data)
+        assert len(name) < 96 and len(dims) <= 4
+        d4 = list(dims) + [0] * (4 - len(dims))
+        recs.append(struct.pack("<96sII4QQQQ", name.encode(), dtype, len(dims), *d4, off, len(b), 0))
+        blobs.append((off, b))
+        off = (off + len(b) + align - 1) // align * align
+    size = off
+    with open(path, "wb") as f:
+        f.write(struct.pack("<4sIIIQQQ64s", b"HGN1", 1, n, 0, rec_off, data_off, size, model_name.encode()))
+        for r in recs:
+            f.write(r)
+        for o, b in blobs:
+            f.seek(o)
+            f.write(b)
+        f.truncate(size)
+
+
+def _gguf_str(s):
+    b = s.encode()
+    return struct.pack("<Q", len(b)) + b
+
+
+def write_gguf(path, tensors, kv=None, align=32):
+    """tensors: list of (name, ggml type, ne (innermost first), raw bytes array).
+    kv: dict of str -> int (written as uint32), str, float (float32) or list of str."""
+    kv = dict(kv or {})
+    out = [b"GGUF", struct.pack("<IQQ", 3, len(tensors), len(kv))]
+    for k, v in kv.items():
+        out.append(_gguf_str(k))
+        if isinstance(v, bool):
+            out.append(struct.pack("<IB", 7, int(v)))
+        elif isinstance(v, int):
+            out.append(struct.pack("<II", 4, v))
+        elif isinstance(v, float):
+            out.append(struct.pack("<If", 6, v))
+        elif isinstance(v, str):
+            out.append(struct.pack("<I", 8) + _gguf_str(v))
+        else:  # list of strings
+            out.append(struct.pack("<IIQ", 9, 8, len(v)) + b"".join(_gguf_str(x) for x in v))
+    blobs, off = [], 0
+    for name, typ, ne, data in tensors:
+        b = _bytes(data)
+        be, bb = _GGML_BLOCK[typ]
+        assert int(np.prod(ne)) // be * bb == len(b), name
+        out.append(_gguf_str(name) + struct.pack("<I", len(ne)) + struct.pack(f"<{len(ne)}Q", *ne) +
+                   struct.pack("<IQ", typ, off))
+        blobs.append((off, b))
+        off = (off + len(b) + align - 1) // align * align
+    hdr = b"".join(out)
+    base = (len(hdr) + align - 1) // align * align
+    with open(path, "wb") as f:
+        f.write(hdr)
+        for o, b in blobs:
+            f.seek(base + o)
+            f.write(b)
+        f.truncate(base + off)
+
+
+def hgn_layer_tensors(l, hl):
+    """The MoE tensors of layer l of a tests.helpers.HostLayer-like object (fmt q4cp) as .hgn records."""
+    d, mid, E = hl.d, hl.mid, hl.E
+    rdt = HGN_F32 if hl.router.dtype == np.float32 else HGN_BF16
+    t = [(f"layers.{l}.mlp.gate.weight", rdt, [E, d], hl.router),
+         (f"layers.{l}.mlp.experts.gate_up_proj.weight", HGN_Q4CP, [E, 2 * mid, d], hl.gate_up),
+         (f"layers.{l}.mlp.experts.down_proj.weight", HGN_Q4CP, [E, d, mid], hl.down)]
+    if hl.shared is not None:
+        t += [(f"layers.{l}.mlp.shared_expert.gate_proj.weight", HGN_Q4CP, [mid, d], hl.shared[0]),
+              (f"layers.{l}.mlp.shared_expert.up_proj.weight", HGN_Q4CP, [mid, d], hl.shared[1]),
+              (f"layers.{l}.mlp.shared_expert.down_proj.weight", HGN_Q4CP, [d, mid], hl.shared[2]),
+              (f"layers.{l}.mlp.shared_expert_gate.weight", HGN_F32, [1, d], hl.shared[3])]
+    return t
+
+
+def gguf_layer_tensors(l, hl):
+    """The MoE tensors of layer l of a HostLayer-like object (fmt q4k) as GGUF tensor infos."""
+    d, mid, E = hl.d, hl.mid, hl.E
+    t = [(f"blk.{l}.ffn_gate_inp.weight", GGML_F32, [d, E], hl.router),
+         (f"blk.{l}.ffn_gate_exps.weight", GGML_Q4_K, [d, mid, E], hl.gate),
+         (f"blk.{l}.ffn_up_exps.weight", GGML_Q4_K, [d, mid, E], hl.up),
+         (f"blk.{l}.ffn_down_exps.weight", GGML_Q4_K, [mid, d, E], hl.down)]
+    if hl.shared is not None:
+        t += [(f"blk.{l}.ffn_gate_shexp.weight", GGML_Q4_K, [d, mid], hl.shared[0]),
+              (f"blk.{l}.ffn_up_shexp.weight", GGML_Q4_K, [d, mid], hl.shared[1]),
+              (f"blk.{l}.ffn_down_shexp.weight", GGML_Q4_K, [mid, d], hl.shared[2]),
+              (f"blk.{l}.ffn_gate_inp_shexp.weight", GGML_F32, [d], hl.shared[3])]
+    return t

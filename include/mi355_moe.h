@@ -216,6 +216,47 @@ int moe_profile_read(moe_ctx* ctx, float* ms);
  * 40_model.inc:1811) into caller buffers [P][id_stride] (device memory; async on st). */
 int moe_get_routing(moe_ctx* ctx, int P, int* ids_out, float* ws_out, moe_stream_t st);
 
+/* ---- checkpoint files -> HBM ---- */
+
+/* hgn::Checkpoint (src/hgn.h:48-76,295-363: HGN1 header + 160-byte records) and gguf::File
+ * (src/gguf.h:225-314: GGUF v2/v3 header, key-value section, tensor infos, aligned data) for the tensors
+ * of this path.  The file is mapped read-only; tensor data pointers are host pointers into the mapping,
+ * valid until moe_file_close.  hgn dims are outermost first (cols last); GGUF dims are ggml's ne[]
+ * (cols first).  dtype is the hgn dtype or the ggml type.  Host-only calls: no GPU needed. */
+enum { MOE_FILE_HGN = 1, MOE_FILE_GGUF = 2 };
+typedef struct moe_file moe_file;
+typedef struct moe_tensor_info {
+  int dtype;
+  uint32_t ndims;
+  uint64_t dims[4];
+  const uint8_t* data;
+  uint64_t nbytes;
+} moe_tensor_info;
+int moe_file_open(const char* path, moe_file** out);
+int moe_file_close(moe_file* f);
+int moe_file_format(const moe_file* f);
+int64_t moe_file_tensor_count(const moe_file* f);
+/* MOE_E_STATE if the file has no tensor of that name */
+int moe_file_find(const moe_file* f, const char* name, moe_tensor_info* out);
+/* d, mid, experts read off the expert tensors of layer `layer`, layers = consecutive layers from there
+ * on that carry them; topk only from the standard GGUF
+ * key "<arch>.expert_used_count" (a .hgn file does not store it).  Other fields untouched. */
+int moe_file_config(const moe_file* f, int layer, moe_config* cfg);
+/* Copies the MoE tensors of n_layers file layers (layers.<l>.mlp.{gate,experts.*,shared_expert*} in a .hgn
+ * file, src/gpu/parts/40_model.inc:1808-1857; blk.<l>.ffn_{gate_inp,gate_exps,up_exps,down_exps,*_shexp}
+ * in a GGUF file, src/gpu/parts/30_host_util.inc:384-412, src/gguf_map.h:210-214) to device memory, bytes
+ * unchanged, and registers them as context layers ctx_layer0...  On the reference's APU the experts are
+ * read in place from registered host memory (30_host_util.inc:552-573); here they become resident in HBM.
+ * The returned object owns the device copies: free it after the context (or after moe_clear_layer).
+ * MOE_E_UNSUPPORTED: a tensor type outside this path (the layers registered so far are cleared again). */
+typedef struct moe_weights moe_weights;
+int moe_load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, int ctx_layer0, int n_layers,
+                    moe_weights** out, moe_stream_t st);
+uint64_t moe_weights_bytes(const moe_weights* w);
+int moe_weights_free(moe_weights* w);
+/* Forget the weights registered for a layer (moe_forward on it returns MOE_E_STATE until it is set again). */
+int moe_clear_layer(moe_ctx* ctx, int layer);
+
 #ifdef __cplusplus
 }
 #endif

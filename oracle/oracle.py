@@ -280,3 +280,34 @@ def ref_moe_token(layer, x):
                              _p(sh_down.data), C.c_uint32(sh_sg.dtype), _p(sh_sg.data), _p(x), _p(y))
     assert rc == 0
     return y
+
+
+def _ref_tensor(fn, path, name):
+    """-> (dtype, dims tuple, uint8 array) through one of the reference's file readers, or None."""
+    dt, nd, nb = C.c_uint32(), C.c_uint32(), C.c_uint64()
+    dims = (C.c_uint64 * 4)()
+    rc = fn(str(path).encode(), name.encode(), C.byref(dt), C.byref(nd), dims, C.byref(nb), None, C.c_uint64(0))
+    if rc == 1:
+        return None
+    if rc != 0:
+        raise RuntimeError(f"reference reader failed on {path}")
+    out = np.zeros(nb.value, np.uint8)
+    fn(str(path).encode(), name.encode(), C.byref(dt), C.byref(nd), dims, C.byref(nb),
+       out.ctypes.data_as(C.c_void_p), C.c_uint64(nb.value))
+    return dt.value, tuple(dims[i] for i in range(nd.value)), out
+
+
+def ref_hgn_tensor(path, name):
+    """hgn::Checkpoint(path).find(name)  (src/hgn.h:103-106)"""
+    return _ref_tensor(ref().ref_hgn_tensor, path, name)
+
+
+def ref_gguf_tensor(path, name):
+    """gguf::File(path).find(name)  (src/gguf.h:119-160)"""
+    return _ref_tensor(ref().ref_gguf_tensor, path, name)
+
+
+def ref_gguf_kv_i(path, key, default=-1):
+    f = ref().ref_gguf_kv_i
+    f.restype = C.c_int64
+    return f(str(path).encode(), key.encode(), C.c_int64(default))

@@ -124,4 +124,56 @@ __attribute__((visibility("default"))) int ref_moe_token(
     return -1;
   }
 }
+
+// --- the reference's file readers (checks of the .hgn / GGUF writers and of the library's parser) ---
+// Looks `name` up through hgn::Checkpoint(path) (src/hgn.h:103-106,294-363).  Returns 0, 1 if the file
+// has no such tensor, -1 if the reader throws.  Copies min(nbytes, cap) data bytes to out.
+__attribute__((visibility("default"))) int ref_hgn_tensor(const char* path, const char* name, uint32_t* dtype,
+                                                          uint32_t* ndims, uint64_t* dims, uint64_t* nbytes,
+                                                          uint8_t* out, uint64_t cap) {
+  try {
+    hgn::Checkpoint ck(path);
+    const hgn::Tensor* t = ck.find(name);
+    if (!t) return 1;
+    *dtype = t->dtype;
+    *ndims = t->ndims;
+    for (int k = 0; k < 4; k++) dims[k] = t->dims[k];
+    *nbytes = t->data_size;
+    if (out && cap) memcpy(out, t->data, t->data_size < cap ? t->data_size : cap);
+    return 0;
+  } catch (const std::exception& e) {
+    fprintf(stderr, "ref_hgn_tensor: %s\n", e.what());
+    return -1;
+  }
+}
+
+// Same through gguf::File(path) (src/gguf.h:119-160,225-314); dims are ne[].
+__attribute__((visibility("default"))) int ref_gguf_tensor(const char* path, const char* name, uint32_t* dtype,
+                                                           uint32_t* ndims, uint64_t* dims, uint64_t* nbytes,
+                                                           uint8_t* out, uint64_t cap) {
+  try {
+    gguf::File f(path);
+    const gguf::Tensor* t = f.find(name);
+    if (!t) return 1;
+    *dtype = t->type;
+    *ndims = t->nd;
+    for (int k = 0; k < 4; k++) dims[k] = t->ne[k];
+    *nbytes = t->nbytes;
+    if (out && cap) memcpy(out, t->data, t->nbytes < cap ? t->nbytes : cap);
+    return 0;
+  } catch (const std::exception& e) {
+    fprintf(stderr, "ref_gguf_tensor: %s\n", e.what());
+    return -1;
+  }
+}
+
+__attribute__((visibility("default"))) int64_t ref_gguf_kv_i(const char* path, const char* key, int64_t def) {
+  try {
+    gguf::File f(path);
+    return f.kv_i(key, def);
+  } catch (const std::exception& e) {
+    fprintf(stderr, "ref_gguf_kv_i: %s\n", e.what());
+    return def;
+  }
+}
 }

@@ -1,0 +1,171 @@
+"""Checkpoint files (.hgn / GGUF): the library's parser against the reference's own readers
+(hgn::Checkpoint, gguf::File — built into oracle/_ref) on files written by gfx1151_engine_amd.files,
+and, on the GPU, layers loaded from a file against the same layers registered directly."""
+import ctypes as C
+import os
+import struct
+
+import numpy as np
+import pytest
+
+from gfx1151_engine_amd import capi, files
+from oracle import oracle as O
+from tests.helpers import HostLayer
+
+D, MID, E, K = 256, 256, 8, 3
+
+
+def _layers(fmt, n=2, seed=5, router_dtype="f32"):
+    rng = np.random.default_rng(seed)
+    return [HostLayer(rng, D, MID, E, K, fmt=fmt, router_dtype=router_dtype, shared=(i == 0 or fmt == "q4k"))
+            for i in range(n)]
+
+
+def _hgn(tmp_path, layers, first=3):
+    ts = []
+    for i, hl in enumerate(layers):
+        ts += files.hgn_layer_tensors(first + i, hl)
+    ts.append(("model.norm.weight", files.HGN_BF16, [D], np.arange(D, dtype=np.uint16)))
+    p = tmp_path / "m.hgn"
+    files.write_hgn(p, ts)
+    return p, ts
+
+
+def _gguf(tmp_path, layers, first=0, version_kv=True):
+    ts = []
+    for i, hl in enumerate(layers):
+        ts += files.gguf_layer_tensors(first + i, hl)
+    ts.append(("output_norm.weight", files.GGML_F32, [D], np.arange(D, dtype=np.float32)))
+    kv = {"general.architecture": "synthmoe", "synthmoe.expert_used_count": K, "synthmoe.expert_count": E,
+          "synthmoe.rope.freq_base": 10000.0, "tokenizer.ggml.tokens": ["a", "bc", "def"], "general.alignment": 64}
+    p = tmp_path / "m.gguf"
+    files.write_gguf(p, ts, kv=kv, align=64)
+    return p, ts
+
+
+HAVE_REF = O.ref() is not None   # the reference readers are an extra witness where oracle/_ref is built
+
+
+def test_hgn_parser_matches_reference_reader(tmp_path):
+    p, ts = _hgn(tmp_path, _layers("q4cp", router_dtype="bf16"))
+    f = capi.ModelFile(p)
+    assert f.format == capi.FILE_HGN and len(f) == len(ts)
+    for name, dt, dims, data in ts:
+        raw = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+        for got in [f.find(name)] + ([O.ref_hgn_tensor(p, name)] if HAVE_REF else []):
+            assert got[0] == dt and got[1][:len(dims)] == tuple(dims) and np.array_equal(got[2], raw), name
+    assert f.find("layers.0.mlp.gate.weight") is None
+    assert not HAVE_REF or O.ref_hgn_tensor(p, "layers.0.mlp.gate.weight") is None
+    cfg = f.config(3)
+    assert (cfg.d, cfg.mid, cfg.experts, cfg.layers) == (D, MID, E, 2)
+    assert f.config(4).layers == 1
+    f.close()
+
+
+def test_gguf_parser_matches_reference_reader(tmp_path):
+    p, ts = _gguf(tmp_path, _layers("q4k"))
+    f = capi.ModelFile(p)
+    assert f.format == capi.FILE_GGUF and len(f) == len(ts)
+    for name, dt, ne, data in ts:
+        raw = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+        for got in [f.find(name)] + ([O.ref_gguf_tensor(p, name)] if HAVE_REF else []):
+            assert got[0] == dt and got[1][:len(ne)] == tuple(ne) and np.array_equal(got[2], raw), name
+    cfg = f.config(0)
+    assert (cfg.d, cfg.mid, cfg.experts, cfg.topk, cfg.layers) == (D, MID, E, K, 2)
+    if HAVE_REF:
+        assert O.ref_gguf_kv_i(p, "synthmoe.expert_used_count") == K
+        assert O.ref_gguf_kv_i(p, "general.alignment") == 64
+    f.close()
+
+
+def test_malformed_files_are_rejected(tmp_path):
+    lib = capi.lib()
+
+    def rc_of(path):
+        h = C.c_void_p()
+        rc = lib.moe_file_open(str(path).encode(), C.byref(h))
+        if rc == 0:
+            lib.moe_file_close(h)
+        return rc
+
+    assert rc_of(tmp_path / "absent.hgn") == -2
+    (tmp_path / "tiny").write_bytes(b"HGN1")
+    assert rc_of(tmp_path / "tiny") == -2
+    (tmp_path / "other").write_bytes(b"SAFETENSORS_____")
+    assert rc_of(tmp_path / "other") == -1
+    p, _ = _hgn(tmp_path, _layers("q4cp", n=1))
+    raw = p.read_bytes()
+    (tmp_path / "cut.hgn").write_bytes(raw[:-64])            # file_size field no longer matches
+    assert rc_of(tmp_path / "cut.hgn") == -2
+    bad = bytearray(raw)
+    struct.pack_into("<Q", bad, 104 + 96 + 8 + 32, len(raw) + 1)  # first record: data offset past the end
+    (tmp_path / "off.hgn").write_bytes(bytes(bad))
+    assert rc_of(tmp_path / "off.hgn") == -2
+    g, _ = _gguf(tmp_path, _layers("q4k", n=1))
+    graw = g.read_bytes()
+    (tmp_path / "cut.gguf").write_bytes(graw[:len(graw) // 2])  # tensor data past the end
+    assert rc_of(tmp_path / "cut.gguf") == -2
+    (tmp_path / "hdr.gguf").write_bytes(graw[:40])              # key-value section cut
+    assert rc_of(tmp_path / "hdr.gguf") == -2
+    v1 = bytearray(graw)
+    struct.pack_into("<I", v1, 4, 1)
+    (tmp_path / "v1.gguf").write_bytes(bytes(v1))
+    assert rc_of(tmp_path / "v1.gguf") == -1
+
+
+def _x(T, seed=11):
+    return np.random.default_rng(seed).standard_normal((T, D), dtype=np.float32)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", ["q4cp", "q4k"])
+def test_layers_loaded_from_file_equal_direct_registration(tmp_path, fmt):
+    import torch
+    layers = _layers(fmt, n=2, seed=9)
+    first = 2
+    p, _ = (_hgn if fmt == "q4cp" else _gguf)(tmp_path, layers, first=first)
+    f = capi.ModelFile(p)
+    cfg = f.config(first)
+    m = capi.Moe(cfg.d, cfg.mid, cfg.experts, K, layers=cfg.layers, max_tokens=64)
+    w = f.load_layers(m, first, 0, cfg.layers)
+    f.close()                                  # the device copies do not depend on the mapping
+    assert w.nbytes > 0
+    for T in (1, 7, 48):
+        x = torch.from_numpy(_x(T)).cuda()
+        for l, hl in enumerate(layers):
+            direct, keep = hl.to_gpu(max_tokens=64)
+            y0 = direct.forward(0, x).cpu().numpy()
+            y1 = m.forward(l, x).cpu().numpy()
+            assert np.array_equal(y0, y1), (fmt, T, l)
+            want = O.moe_layer(hl.oracle_layer(), _x(T))[0]
+            assert np.abs(y1 - want).max() <= 2e-3 * np.abs(want).max()
+            del direct, keep
+    # clearing a layer makes forward refuse it; the other layer still runs
+    capi.check(capi.lib().moe_clear_layer(m.h, 0), "moe_clear_layer")
+    x = torch.from_numpy(_x(1)).cuda()
+    y = torch.empty_like(x)
+    assert capi.lib().moe_forward(m.h, 0, capi.ptr(x), 1, capi.ptr(y), capi.stream()) == -3
+    m.forward(1, x)
+    torch.cuda.synchronize()
+    del m
+    w.free()
+
+
+@pytest.mark.gpu
+def test_load_rejects_types_outside_the_path(tmp_path):
+    # a GGUF whose experts are Q8_0: moe_load_layers reports unsupported and leaves no layer registered
+    import torch
+    rng = np.random.default_rng(1)
+    ts = [("blk.0.ffn_gate_inp.weight", files.GGML_F32, [D, E], rng.standard_normal((E, D), dtype=np.float32))]
+    files._GGML_BLOCK[8] = (32, 34)
+    for n, ne in (("gate", [D, MID, E]), ("up", [D, MID, E]), ("down", [MID, D, E])):
+        ts.append((f"blk.0.ffn_{n}_exps.weight", 8, ne, np.zeros(int(np.prod(ne)) // 32 * 34, np.uint8)))
+    p = tmp_path / "q8.gguf"
+    files.write_gguf(p, ts, kv={"general.architecture": "x"})
+    f = capi.ModelFile(p)
+    m = capi.Moe(D, MID, E, K, layers=1, max_tokens=8)
+    w = C.c_void_p()
+    assert capi.lib().moe_load_layers(m.h, f.h, 0, 0, 1, C.byref(w), capi.stream()) == -1
+    x = torch.zeros(1, D, device="cuda")
+    y = torch.empty_like(x)
+    assert capi.lib().moe_forward(m.h, 0, capi.ptr(x), 1, capi.ptr(y), capi.stream()) == -3
