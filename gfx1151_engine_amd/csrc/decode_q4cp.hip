@@ -14,7 +14,6 @@
 
 namespace {
 
-
 __device__ __forceinline__ float dpp_max_row(float v) {  // max over each row of 16 lanes
   v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true)));
   v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true)));
@@ -139,9 +138,22 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   const uint64_t urow0 = shared ? 0 : (uint64_t)e * 2 * mid + mid;
   const int r0 = blockIdx.x * GU2_ROWS + 4 * wv;  // first of this wave's 4 gate rows
 
-  const int gA = lane, gB = 64 + (lane & 31);
-  const bool vA = gA < G, vB = gB < G;
+  // Branch-free loads: a lane whose group lies past the row reads group 0 instead and gets a zero
+  // scale.  (Loads inside divergent branches make the compiler wait for each of them where it is
+  // issued; in straight-line code all of a wave's loads are in flight together.)
+  const bool vA = lane < G, vB = 64 + (lane & 31) < G;
+  const int gA = vA ? lane : 0, gB = vB ? 64 + (lane & 31) : 0;
+  const float mA = vA ? 1.f : 0.f, mB = vB ? 1.f : 0.f;
   const size_t rb = (size_t)d / 2;
+  // the activation planes and codebook constants are requested first: loads return in order, so
+  // the dot products of the first row pair can start while the later rows are still in flight
+  XG xa, xb;
+  if (!UQ) {
+    const size_t xbase = (size_t)blockIdx.z * G;
+    load_xg(xa, xplanes, xmeta, xbase + gA);
+    load_xg(xb, xplanes, xmeta, xbase + gB);
+  }
+  const float ga = Wg.cb[1] - Wg.cb[0], gb = fmaf(8.f, ga, Wg.cb[0]), ua = Wu.cb[1] - Wu.cb[0], ub = fmaf(8.f, ua, Wu.cb[0]);
   // pairs 0,1: gate rows (r0+2p, r0+2p+1); pairs 2,3: the up rows
   uint4 ca[4], cb[4], ct[4];
   __half sa[4], sb[4], st[4];
@@ -152,41 +164,36 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     const uint8_t* c0 = W.codes + row * rb;
     const uint8_t* s0 = W.scales + row * W.ss;
     const uint64_t trow = lane < 32 ? 0 : 1;
-    if (vA) {
-      ca[p] = *(const uint4*)(c0 + (size_t)gA * 16);
-      cb[p] = *(const uint4*)(c0 + rb + (size_t)gA * 16);
-      sa[p] = *(const __half*)(s0 + gA * 2);
-      sb[p] = *(const __half*)(s0 + W.ss + gA * 2);
-    }
-    if (vB) {
-      ct[p] = *(const uint4*)(c0 + trow * rb + (size_t)gB * 16);
-      st[p] = *(const __half*)(s0 + trow * W.ss + gB * 2);
-    }
+    ca[p] = *(const uint4*)(c0 + (size_t)gA * 16);
+    cb[p] = *(const uint4*)(c0 + rb + (size_t)gA * 16);
+    sa[p] = *(const __half*)(s0 + gA * 2);
+    sb[p] = *(const __half*)(s0 + W.ss + gA * 2);
+    ct[p] = *(const uint4*)(c0 + trow * rb + (size_t)gB * 16);
+    st[p] = *(const __half*)(s0 + trow * W.ss + gB * 2);
   }
-  const float ga = Wg.cb[1] - Wg.cb[0], gb = fmaf(8.f, ga, Wg.cb[0]), ua = Wu.cb[1] - Wu.cb[0], ub = fmaf(8.f, ua, Wu.cb[0]);
+  __builtin_amdgcn_sched_barrier(0);  // every load above is issued before the first dot product
   for (int pi = 0; pi < npairs; pi++) {
   const int tok = UQ ? tokidx[first + pi] : (int)blockIdx.z;
-  XG xa, xb;
-  const size_t xbase = (size_t)tok * G;
-  if (vA) load_xg(xa, xplanes, xmeta, xbase + gA);
-  if (vB) load_xg(xb, xplanes, xmeta, xbase + gB);
+  if (UQ) {
+    const size_t xbase = (size_t)tok * G;
+    load_xg(xa, xplanes, xmeta, xbase + gA);
+    load_xg(xb, xplanes, xmeta, xbase + gB);
+  }
 
   float acc[8];
 #pragma unroll
   for (int p = 0; p < 4; p++) {
     const float a = p >= 2 ? ua : ga, b = p >= 2 ? ub : gb;
-    float v0 = 0.f, v1 = 0.f;
-    if (vA) {
-      v0 = __half2float(sa[p]) * chunk_dot(ca[p], xa, a, b);
-      v1 = __half2float(sb[p]) * chunk_dot(cb[p], xa, a, b);
-    }
-    if (vB) {
-      const float vt = __half2float(st[p]) * chunk_dot(ct[p], xb, a, b);
-      if (lane < 32) v0 += vt;
-      else v1 += vt;
-    }
+    // (a multiplication, not a select: a select lets the compiler move the load back under a branch)
+    const float fa = __half2float(sa[p]) * mA, fb = __half2float(sb[p]) * mA, ft = __half2float(st[p]) * mB;
+    float v0 = fa * chunk_dot(ca[p], xa, a, b);
+    float v1 = fb * chunk_dot(cb[p], xa, a, b);
+    const float vt = ft * chunk_dot(ct[p], xb, a, b);
+    if (lane < 32) v0 += vt;
+    else v1 += vt;
     acc[2 * p] = v0;
     acc[2 * p + 1] = v1;
+    __builtin_amdgcn_sched_barrier(0);  // row pair p is finished before the wait for pair p + 1
   }
 #pragma unroll
   for (int i = 0; i < 8; i++) acc[i] = sum64(acc[i]);
@@ -238,23 +245,36 @@ struct DnArgs2 {
 // (L & 31) holds that slot's activation group (K/32 <= 32 groups) in registers for all the block's
 // rows.  The weighted combine runs afterwards in slot order (descending router probability), then
 // the shared expert: deterministic, no atomics.
-constexpr int DN2_ROWS = 8, DN2_MAXSLOTS = 16;
+constexpr int DN2_MAXSLOTS = 16;
+#ifndef MOE_DN_ROWS
+#define MOE_DN_ROWS 6
+#endif
+template <int ROWS>
 __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __restrict__ hplanes,
                                                 const float2* __restrict__ hmeta,
                                                 const int* __restrict__ ids, const float* __restrict__ ws,
                                                 int id_stride, int kpt, int d, int mid,
                                                 float* __restrict__ out, uint64_t out_stride) {
-  __shared__ float part[DN2_MAXSLOTS][DN2_ROWS];
+  __shared__ float part[DN2_MAXSLOTS][ROWS];
+  __shared__ float wsm[DN2_MAXSLOTS];
   const int tok = blockIdx.y;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const bool has_shared = A.shd.codes != nullptr;
   const int nslots = kpt + (has_shared ? 1 : 0);
-  const int G = mid / 32, g = lane & 31, half = lane >> 5;
-  const int r0 = blockIdx.x * DN2_ROWS;
+  const int G = mid / 32, half = lane >> 5;
+  const int r0 = blockIdx.x * ROWS;
   const size_t rb = (size_t)mid / 2;
+  // combine weights of the token, fetched while the weight rows are in flight
+  float wmine = 0.f;
+  if ((int)threadIdx.x < nslots)
+    wmine = (int)threadIdx.x < kpt ? ws[(size_t)tok * id_stride + threadIdx.x] : A.sh_logit[tok];
   {
-    const int s = 2 * wv + half;
-    const bool live = s < nslots && g < G;
+    // Branch-free loads: lanes past the slots or past the row's groups read slot 0 / group 0 and
+    // get a zero factor, so that all of a wave's loads are in flight together.
+    const int s_raw = 2 * wv + half, g_raw = lane & 31;
+    const bool live = s_raw < nslots && g_raw < G;
+    const int s = live ? s_raw : 0, g = live ? g_raw : 0;
+    const float m = live ? 1.f : 0.f;
     const bool shared = has_shared && s == nslots - 1;
     // per-lane choice of tensor: pick the members by value (a reference to one of two kernel
     // arguments would be re-read from memory in front of every load)
@@ -262,35 +282,36 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
     const uint8_t* wscales = shared ? A.shd.scales : A.dn.scales;
     const float* wcb = shared ? A.shd.cb : A.dn.cb;
     const uint64_t wss = shared ? A.shd.ss : A.dn.ss;
-    const int e = (live && !shared) ? ids[(size_t)tok * id_stride + s] : 0;
+    const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
+    XG x;
+    load_xg(x, hplanes, hmeta, ((size_t)tok * nslots + s) * G + g);
+    const float a = wcb[1] - wcb[0], b = fmaf(8.f, a, wcb[0]);
     const uint64_t row0 = (shared ? 0 : (uint64_t)e * d) + r0;
     const uint8_t* cp = wcodes + row0 * rb + (size_t)g * 16;
     const uint8_t* sp = wscales + row0 * wss + g * 2;
-    uint4 cw[DN2_ROWS];
-    __half sc[DN2_ROWS];
+    uint4 cw[ROWS];
+    __half sc[ROWS];
 #pragma unroll
-    for (int r = 0; r < DN2_ROWS; r++) {
-      if (live) {
-        cw[r] = *(const uint4*)(cp + r * rb);
-        sc[r] = *(const __half*)(sp + r * wss);
-      }
+    for (int r = 0; r < ROWS; r++) {
+      cw[r] = *(const uint4*)(cp + r * rb);
+      sc[r] = *(const __half*)(sp + r * wss);
     }
-    const float a = wcb[1] - wcb[0], b = fmaf(8.f, a, wcb[0]);
-    XG x;
-    if (live) load_xg(x, hplanes, hmeta, ((size_t)tok * nslots + s) * G + g);
+    __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first dot product
 #pragma unroll
-    for (int r = 0; r < DN2_ROWS; r++) {
-      float v = live ? __half2float(sc[r]) * chunk_dot(cw[r], x, a, b) : 0.f;
+    for (int r = 0; r < ROWS; r++) {
+      float v = __half2float(sc[r]) * m * chunk_dot(cw[r], x, a, b);
       v = sum32(v);
-      if (g == 0 && s < nslots) part[s][r] = v;
+      if (g_raw == 0 && s_raw < nslots) part[s_raw][r] = v;
+      if ((r & 1) == 1) __builtin_amdgcn_sched_barrier(0);  // rows are consumed in arrival order
     }
   }
+  if ((int)threadIdx.x < nslots) wsm[threadIdx.x] = (int)threadIdx.x < kpt ? wmine : sigmoid_f(wmine);
   __syncthreads();
-  if (threadIdx.x < DN2_ROWS) {
+  if (threadIdx.x < ROWS) {
     const int r = threadIdx.x;
     float y = 0.f;
-    for (int s = 0; s < kpt; s++) y += ws[(size_t)tok * id_stride + s] * part[s][r];
-    if (has_shared) y += sigmoid_f(A.sh_logit[tok]) * part[kpt][r];
+    for (int s = 0; s < kpt; s++) y += wsm[s] * part[s][r];
+    if (has_shared) y += wsm[kpt] * part[kpt][r];
     out[(size_t)tok * out_stride + r0 + r] = y;
   }
 }
@@ -355,7 +376,7 @@ size_t moe_qvec_meta_bytes(int K) { return (size_t)(K / 32) * sizeof(float2); }
 // Supported shapes of the integer-dot decode kernels (otherwise the caller uses the f32 kernels).
 bool moe_dec_supported(int d, int mid, int nslots) {
   return d % 32 == 0 && d / 32 <= 96 && mid % 32 == 0 && mid / 32 <= 32 && nslots <= DN2_MAXSLOTS &&
-         mid % GU2_ROWS == 0 && d % DN2_ROWS == 0 && d % DU_ROWS == 0;
+         mid % GU2_ROWS == 0 && d % DU_ROWS == 0;  // (d % 32 == 0 covers the 8-row down blocks)
 }
 
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
@@ -421,9 +442,12 @@ int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float
   A.dn = decw(dn);
   A.shd = decw(sh_down);
   A.sh_logit = sh_logit;
-  dim3 grid(d / DN2_ROWS, P);
-  const int nslots = kpt + (sh_down ? 1 : 0);
-  k_dec_dn<<<grid, 64 * ((nslots + 1) / 2), 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
+  const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
+  // MOE_DN_ROWS rows per block where that divides d (d = 3072: 512 blocks, two per CU), else 8
+  if (d % MOE_DN_ROWS == 0)
+    k_dec_dn<MOE_DN_ROWS><<<dim3(d / MOE_DN_ROWS, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
+  else
+    k_dec_dn<8><<<dim3(d / 8, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
