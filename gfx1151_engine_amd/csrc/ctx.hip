@@ -374,17 +374,23 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
                        (!L.has_shared || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
   const bool use_int4k = L.has_gguf && c->int_decode && (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K) &&
                          moe_dec4k_supported(g.d, g.mid, nslots_d);
+  const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min;
+  // q4cp integer kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
+  // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
+  const bool gu_topk = use_int && !use_uq && moe_dec_gu_topk_supported(g.experts, g.topk);
   bool fused = false;
   if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
                                     c->logits, c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
-                                    use_int4k, c->ticket,
+                                    use_int4k, gu_topk ? nullptr : c->ticket,
                                     c->ids, c->ws, g.topk, g.id_stride, &fused, st)))
     return rc;
-  if (!fused && (rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
+  if (!fused && !gu_topk &&
+      (rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st)))
+    return rc;
   prof_mark(c, MOE_PROF_ROUTER, st);
   if (L.has_q4cp) {
     if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
-    if (use_int && c->uq_min > 0 && P >= c->uq_min) {
+    if (use_uq) {
       // verify-size batches: tokens share experts; walk the expert-sorted pair lists so that every
       // distinct expert's weights are read once (reference: the _uq kernels, 26_kernels_moe_gguf.inc:758-877)
       if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
@@ -411,10 +417,14 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     }
     if (use_int) {
       // integer-dot kernels: activations as digit planes (made by the logits launch above)
-      if ((rc = moe_launch_dec_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
-                                  L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->ids, g.id_stride,
-                                  g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st)))
-        return rc;
+      rc = gu_topk ? moe_launch_dec_gu_topk(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
+                                            L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->logits,
+                                            g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
+                                            c->hplanes, c->hmeta, nullptr, st)
+                   : moe_launch_dec_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
+                                       L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->ids,
+                                       g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st);
+      if (rc) return rc;
       prof_mark(c, MOE_PROF_UP, st);
       rc = moe_launch_dec_dn(&L.down, L.has_shared ? &L.sh_down : nullptr, c->sh_logit, c->hplanes, c->hmeta,
                              c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, y, (uint64_t)g.d, st);

@@ -11,6 +11,7 @@
 #include "common.h"
 #include "internal.h"
 #include "qvec.h"
+#include "topk.h"
 
 namespace {
 
@@ -106,17 +107,26 @@ struct GuArgs2 {
 // (token, expert) pairs routed to it (expert-sorted lists of the routing permutation; the shared
 // expert is the tile with expert id >= n_experts over all tokens).  The block reads its weight rows
 // once and walks the tile's pairs; hid planes are then indexed by pair position.
+// NPL > 0 (E <= 64*NPL, not with UQ): the router launch only left the logits; every block of a
+// routed slot runs the softmax / top-k of its token itself (the same code and therefore the same
+// ids and weights in every block; cheaper than a last-block ticket in the router launch plus a
+// dependent load of the ids here) and block (0, 0, token) writes ids / weights out for the down
+// kernel.  The shared expert's blocks skip it and have the CU to themselves meanwhile.
 constexpr int GU2_ROWS = 32;
-template <bool UQ>
+template <bool UQ, int NPL>
 __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __restrict__ xplanes,
                                                 const float2* __restrict__ xmeta,
                                                 const int* __restrict__ ids, int id_stride, int kpt, int d,
                                                 int mid, uint32_t* __restrict__ hplanes,
                                                 float2* __restrict__ hmeta, float* __restrict__ hid_f32,
                                                 const moe_tile* __restrict__ tiles, const int* __restrict__ ntiles,
-                                                const int* __restrict__ tokidx, int n_experts) {
+                                                const int* __restrict__ tokidx, int n_experts,
+                                                const float* __restrict__ logits, int* __restrict__ ids_out,
+                                                float* __restrict__ ws_out) {
   __shared__ float gs[GU2_ROWS], us[GU2_ROWS];
   __shared__ uint32_t pk[QV4_GROUP_DW];
+  __shared__ int sel_ids[64];
+  __shared__ float sel_ws[64];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int G = d / 32;
   int s = blockIdx.y, nslots = gridDim.y, e = 0, first = 0, npairs = 1;
@@ -128,6 +138,17 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     e = shared ? 0 : tile.expert;
     first = tile.first;
     npairs = tile.count;
+  } else if (NPL > 0) {
+    shared = s >= kpt;
+    if (!shared) {
+      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)blockIdx.z * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      __syncthreads();
+      e = sel_ids[s];
+      if (blockIdx.x == 0 && s == 0 && (int)threadIdx.x < kpt) {
+        ids_out[(size_t)blockIdx.z * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
+        ws_out[(size_t)blockIdx.z * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+      }
+    }
   } else {
     shared = s >= kpt;
     e = shared ? 0 : ids[(size_t)blockIdx.z * id_stride + s];
@@ -397,8 +418,30 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
-  k_dec_gu<false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
-                                        nullptr, nullptr, nullptr, 0);
+  k_dec_gu<false, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
+                                           nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// The same with the softmax / top-k of every token done inside the launch: logits [P][n_experts] in,
+// ids / ws rows (id_stride wide) out.
+bool moe_dec_gu_topk_supported(int n_experts, int kpt) { return n_experts <= 1024 && kpt <= 64 && kpt <= n_experts; }
+int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
+                           const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
+                           int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
+                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st) {
+  GuArgs2 A{};
+  A.gu = decw(gu);
+  A.shg = decw(sh_gate);
+  A.shu = decw(sh_up);
+  dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
+  if (n_experts <= 512)
+    k_dec_gu<false, 8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
+                                             hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws);
+  else
+    k_dec_gu<false, 16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
+                                              hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -415,8 +458,8 @@ int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const mo
   A.shu = decw(sh_up);
   if (max_tiles <= 0) return MOE_OK;
   dim3 grid(mid / GU2_ROWS, max_tiles);
-  k_dec_gu<true><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
-                                       ntiles, tokidx, n_experts);
+  k_dec_gu<true, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
+                                          ntiles, tokidx, n_experts, nullptr, nullptr, nullptr);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

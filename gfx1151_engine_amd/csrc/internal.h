@@ -42,6 +42,11 @@ size_t moe_qvec_meta_bytes(int K);
 bool moe_dec_supported(int d, int mid, int nslots);
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
                     hipStream_t st);
+bool moe_dec_gu_topk_supported(int n_experts, int kpt);
+int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
+                           const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
+                           int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
+                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st);
 int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,

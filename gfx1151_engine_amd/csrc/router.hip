@@ -3,6 +3,7 @@
 #include "common.h"
 #include "internal.h"
 #include "qvec.h"
+#include "topk.h"
 
 namespace {
 
@@ -197,9 +198,6 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
 // If `counter` is given, the block that finishes last (an atomic ticket per row block, fences at
 // device scope on both sides) runs the softmax / top-k of every token as well and re-arms the
 // counter: one launch instead of two on the latency-bound decode path.
-template <int NPL, bool COH>
-__device__ void topk_block(const float* lg, int* __restrict__ ids_row, float* __restrict__ ws_row, int E, int k);
-
 template <bool BF16, int TT, int NPL>
 __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W,
                                                       const float* __restrict__ bias,
@@ -211,18 +209,21 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
                                                       unsigned* counter, int* __restrict__ ids,
                                                       float* __restrict__ ws, int k, int id_stride) {
   __shared__ int s_last;
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int nrb = (nrows + 3) >> 2;
+  // the wave index as a scalar: row, weight type and base address are then wave-uniform values
+  // and the bf16 / f32 choice below is a scalar branch, not a divergent one around every load
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int rpb = blockDim.x >> 6;  // rows per block: one per wave
+  const int nrb = (nrows + rpb - 1) / rpb;
   if ((int)blockIdx.x >= nrb) {
-    const int G = d / 32, gb = (G + 255) / 256;
-    const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * 256 + threadIdx.x;
+    const int G = d / 32, gb = (G + (int)blockDim.x - 1) / (int)blockDim.x;
+    const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * blockDim.x + threadIdx.x;
     if (t < P && g < G) {
       if (planes_natural) qvec_group_from_f32_t<true>(x, (uint64_t)d, G, t, g, planes, meta);  // Q4_K kernels
       else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);                       // q4cp kernels
     }
     return;
   }
-  const int row = blockIdx.x * 4 + wv;
+  const int row = blockIdx.x * rpb + wv;
   if (row < nrows) {
     const bool extra = row == E;
     const void* Wr = extra ? Wx : W;
@@ -380,67 +381,6 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
   }
 }
 
-__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
-__device__ __forceinline__ uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
-__device__ __forceinline__ uint32_t wave_umax(uint32_t m) {
-  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true));
-  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, true));
-  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x141, 0xf, 0xf, true));
-  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x140, 0xf, 0xf, true));
-  return umax(umax((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
-              umax((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
-}
-__device__ __forceinline__ uint32_t wave_umin(uint32_t m) {
-  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0xB1, 0xf, 0xf, false));
-  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x4E, 0xf, 0xf, false));
-  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x141, 0xf, 0xf, false));
-  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x140, 0xf, 0xf, false));
-  return umin(umin((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
-              umin((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
-}
-
-// k rounds of arg-max by one wave over keys held NPL per lane (key[j] of lane l = expert l + 64 j;
-// key = probability bits + 1, probabilities are >= 0 so the bit patterns order like unsigned
-// integers; 0 = not a candidate).  Larger probability first, equal probabilities -> lower index.
-// Each lane tracks its own best (value, lowest register holding it); a round is a wave-wide
-// maximum of the values, then a wave-wide minimum of the expert index over the lanes that hold
-// that value, both through DPP row operations and four lane reads.  The selected ids and values
-// stay in registers (lane r keeps round r) and are written once at the end.
-template <int NPL>
-__device__ __forceinline__ void topk_select(uint32_t (&key)[NPL], int lane, int k, int* __restrict__ ids_row,
-                                            float* __restrict__ ws_row) {
-  double wsum = 0.0;
-  float mine = 0.f;
-  int myid = 0;
-  for (int r = 0; r < k; r++) {
-    uint32_t m = key[0];
-    int jm = 0;
-#pragma unroll
-    for (int j = 1; j < NPL; j++) {
-      const bool gt = key[j] > m;  // strict: the lowest register (= lowest expert index) wins a tie
-      m = gt ? key[j] : m;
-      jm = gt ? j : jm;
-    }
-    const uint32_t wm = wave_umax(m);
-    const uint32_t bi = wave_umin(m == wm ? (uint32_t)(64 * jm + lane) : 0xffffffffu);
-    const float bv = __uint_as_float(wm - 1u);
-    wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
-    if (lane == r) {
-      mine = bv;
-      myid = (int)bi;
-    }
-    if ((int)(bi & 63u) == lane) {
-#pragma unroll
-      for (int j = 0; j < NPL; j++)
-        if (j == (int)(bi >> 6)) key[j] = 0u;
-    }
-  }
-  if (lane < k) {
-    ids_row[lane] = myid;
-    ws_row[lane] = (float)((double)mine / wsum);
-  }
-}
-
 // ---- softmax + top-k, one wave per token (E <= 64*NPL) ----
 template <int NPL>
 __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ logits,
@@ -497,72 +437,6 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
   topk_select<NPL>(key, lane, k, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride);
 }
 
-// The same softmax / top-k by one block of 256 threads for one token: the fp64 exps, the costly
-// part, are spread over the block; wave 0 then runs the k selection rounds on the keys in LDS.
-// COH: the logits were written by other blocks of the same launch: read them with device-scope loads.
-template <int NPL, bool COH>
-__device__ void topk_block(const float* lg, int* __restrict__ ids_row, float* __restrict__ ws_row, int E, int k) {
-  constexpr int NPT = NPL / 4;  // values per thread (256 threads, E <= 64*NPL)
-  __shared__ float pb[64 * NPL];
-  __shared__ uint32_t keys[64 * NPL];
-  __shared__ double red[4];
-  __shared__ float redf[4];
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  __syncthreads();  // LDS of a previous token is no longer read
-  float v[NPT];
-  float mxf = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < NPT; j++) {
-    const int e = tid + 256 * j;
-    v[j] = -INFINITY;
-    if (e < E) v[j] = COH ? __hip_atomic_load(&lg[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
-    mxf = fmaxf(mxf, v[j]);
-  }
-  mxf = wave_max(mxf);
-  if (lane == 0) redf[wv] = mxf;
-  __syncthreads();
-  const double mx = (double)fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
-  float p[NPT];
-  bool exact = true;
-  double sloc = 0.0;
-#pragma unroll
-  for (int j = 0; j < NPT; j++) {
-    const int e = tid + 256 * j;
-    p[j] = e < E ? (float)exp((double)v[j] - mx) : 0.f;
-    exact = exact && (p[j] == 0.f || p[j] >= 0x1p-20f);
-    sloc += (double)p[j];
-    pb[e] = p[j];
-  }
-  const bool all_exact = __syncthreads_and(exact);
-  double se;
-  if (all_exact) {  // every partial sum is representable: any order gives the reference's fp64 sum
-    sloc = wave_sum(sloc);
-    if (lane == 0) red[wv] = sloc;
-    __syncthreads();
-    se = (red[0] + red[1]) + (red[2] + red[3]);
-  } else {          // very wide logit range: replay the reference's index order on one thread
-    if (tid == 0) {
-      double t = 0.0;
-      for (int e = 0; e < E; e++) t += (double)pb[e];
-      red[0] = t;
-    }
-    __syncthreads();
-    se = red[0];
-  }
-#pragma unroll
-  for (int j = 0; j < NPT; j++) {
-    const int e = tid + 256 * j;
-    keys[e] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
-  }
-  __syncthreads();
-  if (wv != 0) return;
-  uint32_t key[NPL];
-#pragma unroll
-  for (int j = 0; j < NPL; j++) key[j] = keys[lane + 64 * j];
-  topk_select<NPL>(key, lane, k, ids_row, ws_row);
-}
-
-// one block per token (small batches)
 template <int NPL>
 __global__ void __launch_bounds__(256) k_router_topk_block(const float* __restrict__ logits, int* __restrict__ ids,
                                                            float* __restrict__ ws, int E, int k, int id_stride) {
@@ -629,13 +503,16 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
   const int nrows = E + (Wx ? 1 : 0);
-  const int qblocks = planes ? P * ((d / 32 + 255) / 256) : 0;
   const bool fuse = counter && ids && ws && P <= 4 && E <= 1024;
   if (fused_topk) *fused_topk = fuse;
   unsigned* cn = fuse ? counter : nullptr;
-  dim3 g((nrows + 3) / 4 + qblocks);
+  // one token, no top-k in this launch: two rows per block so that the rows cover every CU
+  // (the fused top-k needs its 256 threads)
+  const int bs = (P == 1 && !fuse && E <= 512) ? 128 : 256, rpb = bs / 64;
+  const int qblocks = planes ? P * ((d / 32 + bs - 1) / bs) : 0;
+  dim3 g((nrows + rpb - 1) / rpb + qblocks);
   const void* wx = Wx ? Wx->data : nullptr;
-#define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride)
+#define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, bs, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride)
   if (P == 1 && E <= 512) {
     if (bf) RSM_GO(true, 1, 8); else RSM_GO(false, 1, 8);
   } else if (P <= 4) {

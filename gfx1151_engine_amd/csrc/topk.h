@@ -1,0 +1,138 @@
+// Softmax + top-k selection shared by the router kernels and the decode gate/up kernel.
+// (reference: src/ref.cpp:565-594 — fp64 softmax over f32 logits, k rounds of arg-max with ties to
+//  the lower index, weights renormalised over the selected k)
+#pragma once
+#include "common.h"
+
+__device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
+__device__ __forceinline__ uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
+__device__ __forceinline__ uint32_t wave_umax(uint32_t m) {
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true));
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, true));
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x141, 0xf, 0xf, true));
+  m = umax(m, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x140, 0xf, 0xf, true));
+  return umax(umax((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+              umax((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+}
+__device__ __forceinline__ uint32_t wave_umin(uint32_t m) {
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0xB1, 0xf, 0xf, false));
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x4E, 0xf, 0xf, false));
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x141, 0xf, 0xf, false));
+  m = umin(m, (uint32_t)__builtin_amdgcn_update_dpp(-1, (int)m, 0x140, 0xf, 0xf, false));
+  return umin(umin((uint32_t)__builtin_amdgcn_readlane((int)m, 0), (uint32_t)__builtin_amdgcn_readlane((int)m, 16)),
+              umin((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
+}
+
+// k rounds of arg-max by one wave over keys held NPL per lane (key[j] of lane l = expert l + 64 j;
+// key = probability bits + 1, probabilities are >= 0 so the bit patterns order like unsigned
+// integers; 0 = not a candidate).  Larger probability first, equal probabilities -> lower index.
+// Each lane tracks its own best (value, lowest register holding it); a round is a wave-wide
+// maximum of the values, then a wave-wide minimum of the expert index over the lanes that hold
+// that value, both through DPP row operations and four lane reads.  The selected ids and values
+// stay in registers (lane r keeps round r) and are written once at the end.
+template <int NPL>
+__device__ __forceinline__ void topk_select(uint32_t (&key)[NPL], int lane, int k, int* ids_row,
+                                            float* ws_row) {
+  double wsum = 0.0;
+  float mine = 0.f;
+  int myid = 0;
+  for (int r = 0; r < k; r++) {
+    uint32_t m = key[0];
+    int jm = 0;
+#pragma unroll
+    for (int j = 1; j < NPL; j++) {
+      const bool gt = key[j] > m;  // strict: the lowest register (= lowest expert index) wins a tie
+      m = gt ? key[j] : m;
+      jm = gt ? j : jm;
+    }
+    const uint32_t wm = wave_umax(m);
+    const uint32_t bi = wave_umin(m == wm ? (uint32_t)(64 * jm + lane) : 0xffffffffu);
+    const float bv = __uint_as_float(wm - 1u);
+    wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
+    if (lane == r) {
+      mine = bv;
+      myid = (int)bi;
+    }
+    if ((int)(bi & 63u) == lane) {
+#pragma unroll
+      for (int j = 0; j < NPL; j++)
+        if (j == (int)(bi >> 6)) key[j] = 0u;
+    }
+  }
+  if (lane < k) {
+    ids_row[lane] = myid;
+    ws_row[lane] = (float)((double)mine / wsum);
+  }
+}
+
+// The softmax / top-k of one token by one block of NT threads (E <= 64*NPL): the fp64 exps, the
+// costly part, are spread over the block; wave 0 then runs the k selection rounds on the keys in
+// LDS.  COH: the logits were written by other blocks of the same launch: read them with
+// device-scope loads.  ids_row / ws_row may point to global memory or LDS.
+template <int NPL, bool COH, int NT = 256>
+__device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, int k) {
+  constexpr int NPT = (64 * NPL + NT - 1) / NT;  // values per thread
+  constexpr int NW = NT / 64;
+  __shared__ float pb[64 * NPL];
+  __shared__ uint32_t keys[64 * NPL];
+  __shared__ double red[NW];
+  __shared__ float redf[NW];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  __syncthreads();  // LDS of a previous token is no longer read
+  float v[NPT];
+  float mxf = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NPT; j++) {
+    const int e = tid + NT * j;
+    v[j] = -INFINITY;
+    if (e < E) v[j] = COH ? __hip_atomic_load(&lg[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
+    mxf = fmaxf(mxf, v[j]);
+  }
+  mxf = wave_max(mxf);
+  if (lane == 0) redf[wv] = mxf;
+  __syncthreads();
+  float mxa = redf[0];
+#pragma unroll
+  for (int w = 1; w < NW; w++) mxa = fmaxf(mxa, redf[w]);
+  const double mx = (double)mxa;
+  float p[NPT];
+  bool exact = true;
+  double sloc = 0.0;
+#pragma unroll
+  for (int j = 0; j < NPT; j++) {
+    const int e = tid + NT * j;
+    p[j] = e < E ? (float)exp((double)v[j] - mx) : 0.f;
+    exact = exact && (p[j] == 0.f || p[j] >= 0x1p-20f);
+    sloc += (double)p[j];
+    if (e < 64 * NPL) pb[e] = p[j];
+  }
+  const bool all_exact = __syncthreads_and(exact);
+  double se;
+  if (all_exact) {  // every partial sum is representable: any order gives the reference's fp64 sum
+    sloc = wave_sum(sloc);
+    if (lane == 0) red[wv] = sloc;
+    __syncthreads();
+    se = red[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) se += red[w];
+  } else {          // very wide logit range: replay the reference's index order on one thread
+    if (tid == 0) {
+      double t = 0.0;
+      for (int e = 0; e < E; e++) t += (double)pb[e];
+      red[0] = t;
+    }
+    __syncthreads();
+    se = red[0];
+  }
+#pragma unroll
+  for (int j = 0; j < NPT; j++) {
+    const int e = tid + NT * j;
+    if (e < 64 * NPL) keys[e] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
+  }
+  __syncthreads();
+  if (wv != 0) return;
+  uint32_t key[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; j++) key[j] = keys[lane + 64 * j];
+  topk_select<NPL>(key, lane, k, ids_row, ws_row);
+}
