@@ -295,15 +295,15 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
 // row, and every weight is read once for all tokens.  Lane l owns columns 2l, 2l+1 of each slab:
 // two fp64 chains per token, combined in a fixed order, then the wave sum.  Same accuracy
 // statement as k_router_small.  Blocks past the rows build the digit planes of x.
-constexpr int RM_C = 128;
-template <bool BF16, int PMAX>
+constexpr int RM_C = 128, RM_D = 4;
+template <bool BF16, int PMAX>  // PMAX 8 / 16 / 24
 __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, const float* __restrict__ bias,
                                                     const void* __restrict__ Wx, bool wx_bf16,
                                                     const float* __restrict__ x, int P, int E, int d,
                                                     float* __restrict__ logits, float* __restrict__ out_x,
                                                     int nrows, uint32_t* __restrict__ planes,
                                                     float2* __restrict__ meta, bool planes_natural) {
-  __shared__ __attribute__((aligned(16))) double Xd[PMAX][RM_C];
+  __shared__ __attribute__((aligned(16))) double Xd[2][PMAX][RM_C];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int nrb = (nrows + 3) >> 2;
   if ((int)blockIdx.x >= nrb) {
@@ -315,54 +315,73 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
     }
     return;
   }
-  const int row = blockIdx.x * 4 + wv;
+  // the wave's row as scalar values: the bf16 / f32 choice is then a scalar branch
+  const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(wv);
   const bool live = row < nrows, extra = row == E;
   const void* Wr = extra ? Wx : W;
-  const uint64_t base = extra ? 0 : (uint64_t)(live ? row : 0) * d;
+  const uint64_t base = (extra || !live) ? 0 : (uint64_t)row * d;  // rows past the matrix read row 0, never stored
   const bool bf = extra ? wx_bf16 : BF16;
   constexpr int XR = PMAX * RM_C / 256;  // staged activations per thread and slab
-  float xr[XR];
-  float2 wr;
-  auto fetch = [&](int c0) {
+  // Register ring of RM_D slabs: slot j holds slab s with s % RM_D == j and is refilled for slab
+  // s + RM_D as soon as slab s has gone to LDS, so every load has RM_D slab times to arrive
+  // (one slab ahead left the loop waiting a full memory latency per 128 columns).
+  // All loads are unconditional (clamped address, value times 0 or 1) and weights stay as raw
+  // bits until they are used: a load under a divergent branch, or converted where it is issued,
+  // makes the wave wait for every load in flight.  (d is even: c + 1 < d whenever c < d.)
+  float xr[RM_D][XR];
+  uint2 wr[RM_D];
+  auto fetch = [&](int j, int c0) {
 #pragma unroll
-    for (int j = 0; j < XR; j++) {
-      const int e = tid + 256 * j, t = e / RM_C, c = c0 + e % RM_C;
-      xr[j] = (t < P && c < d) ? x[(size_t)t * d + c] : 0.f;
+    for (int i = 0; i < XR; i++) {
+      const int e = tid + 256 * i, t = e / RM_C, c = c0 + e % RM_C;
+      const bool ok = t < P && c < d;
+      xr[j][i] = x[ok ? (size_t)t * d + c : 0] * (ok ? 1.f : 0.f);
     }
     const int c = c0 + 2 * lane;
-    wr = float2{0.f, 0.f};
-    if (live && c + 1 < d) {
-      if (bf) {
-        const uint32_t u = *(const uint32_t*)((const uint16_t*)Wr + base + c);
-        wr.x = __uint_as_float(u << 16);
-        wr.y = __uint_as_float(u & 0xffff0000u);
-      } else {
-        wr = *(const float2*)((const float*)Wr + base + c);
-      }
-    } else if (live && c < d) {
-      wr.x = bf ? bf16_bits_to_f32(((const uint16_t*)Wr)[base + c]) : ((const float*)Wr)[base + c];
-    }
+    const int cc = c < d ? c : 0;
+    // two 32-bit loads in either format (bf16: the same word twice), so no branch surrounds them
+    const uint8_t* p0 = (const uint8_t*)Wr + (base + cc) * (bf ? 2 : 4);
+    wr[j].x = *(const uint32_t*)p0;
+    wr[j].y = *(const uint32_t*)(p0 + (bf ? 0 : 4));
+  };
+  auto weights = [&](int j, int c0, double& w0, double& w1) {
+    const float m = c0 + 2 * lane < d ? 1.f : 0.f;
+    const float f0 = bf ? __uint_as_float(wr[j].x << 16) : __uint_as_float(wr[j].x);
+    const float f1 = bf ? __uint_as_float(wr[j].x & 0xffff0000u) : __uint_as_float(wr[j].y);
+    w0 = (double)(f0 * m);
+    w1 = (double)(f1 * m);
   };
   double acc[PMAX][2];
 #pragma unroll
   for (int t = 0; t < PMAX; t++) acc[t][0] = acc[t][1] = 0.0;
-  fetch(0);
-  for (int c0 = 0; c0 < d; c0 += RM_C) {
-    __syncthreads();  // the previous slab is no longer read
 #pragma unroll
-    for (int j = 0; j < XR; j++) {
-      const int e = tid + 256 * j;
-      Xd[e / RM_C][e % RM_C] = (double)xr[j];
-    }
-    const double w0 = (double)wr.x, w1 = (double)wr.y;
-    __syncthreads();
-    if (c0 + RM_C < d) fetch(c0 + RM_C);
-    // rows past P hold zeros: no predicate, so the LDS reads of a slab go out back to back
+  for (int j = 0; j < RM_D; j++) fetch(j, j * RM_C);
+  int buf = 0;
+  for (int cg = 0; cg < d; cg += RM_D * RM_C) {
 #pragma unroll
-    for (int t = 0; t < PMAX; t++) {
-      const double2 xv = *(const double2*)&Xd[t][2 * lane];
-      acc[t][0] = fma(w0, xv.x, acc[t][0]);
-      acc[t][1] = fma(w1, xv.y, acc[t][1]);
+    for (int j = 0; j < RM_D; j++) {
+      const int c0 = cg + j * RM_C;
+      if (c0 < d) {  // block-uniform
+        // Xd[buf] was last read two slabs ago; every wave has passed the barrier of the slab in
+        // between, so it is free
+#pragma unroll
+        for (int i = 0; i < XR; i++) {
+          const int e = tid + 256 * i;
+          Xd[buf][e / RM_C][e % RM_C] = (double)xr[j][i];
+        }
+        double w0, w1;
+        weights(j, c0, w0, w1);
+        fetch(j, c0 + RM_D * RM_C);  // slabs past d load column 0 and count as zeros
+        __syncthreads();
+        // rows past P hold zeros: no predicate, so the LDS reads of a slab go out back to back
+#pragma unroll
+        for (int t = 0; t < PMAX; t++) {
+          const double2 xv = *(const double2*)&Xd[buf][t][2 * lane];
+          acc[t][0] = fma(w0, xv.x, acc[t][0]);
+          acc[t][1] = fma(w1, xv.y, acc[t][1]);
+        }
+        buf ^= 1;
+      }
     }
   }
 #pragma unroll
@@ -500,6 +519,20 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
                             hipStream_t st) {
   const int E = (int)W->rows, d = (int)W->cols;
+  if (P > 24) {
+    // more than 24 tokens per block cost the kernel its second wave per SIMD (accumulators):
+    // two launches of at most 16 tokens read the router matrix twice (L2 / MALL) and are faster
+    const int P0 = 16, G = d / 32;
+    const size_t pdw = planes_natural ? QV_GROUP_DW : QV4_GROUP_DW;
+    int rc = moe_router_logits_small(W, bias, Wx, x, P0, logits, out_x, planes, meta, planes_natural, nullptr, nullptr,
+                                     nullptr, k, id_stride, nullptr, st);
+    if (rc) return rc;
+    if (fused_topk) *fused_topk = false;
+    return moe_router_logits_small(W, bias, Wx, x + (size_t)P0 * d, P - P0, logits + (size_t)P0 * E,
+                                   out_x ? out_x + P0 : nullptr, planes ? planes + (size_t)P0 * G * pdw : nullptr,
+                                   meta ? meta + (size_t)P0 * G : nullptr, planes_natural, nullptr, nullptr, nullptr, k,
+                                   id_stride, nullptr, st);
+  }
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
   const int nrows = E + (Wx ? 1 : 0);
@@ -522,8 +555,7 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
 #define RMD_GO(BF, PM) k_router_mid<BF, PM><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural)
     if (P <= 8) { if (bf) RMD_GO(true, 8); else RMD_GO(false, 8); }
     else if (P <= 16) { if (bf) RMD_GO(true, 16); else RMD_GO(false, 16); }
-    else if (P <= 24) { if (bf) RMD_GO(true, 24); else RMD_GO(false, 24); }
-    else { if (bf) RMD_GO(true, 32); else RMD_GO(false, 32); }
+    else { if (bf) RMD_GO(true, 24); else RMD_GO(false, 24); }  // P <= 24 (larger batches were split above)
 #undef RMD_GO
   }
 #undef RSM_GO
