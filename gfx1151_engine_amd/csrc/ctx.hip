@@ -375,9 +375,9 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const bool use_int4k = L.has_gguf && c->int_decode && (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K) &&
                          moe_dec4k_supported(g.d, g.mid, nslots_d);
   const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min;
-  // q4cp integer kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
+  // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
-  const bool gu_topk = use_int && !use_uq && moe_dec_gu_topk_supported(g.experts, g.topk);
+  const bool gu_topk = ((use_int && !use_uq) || use_int4k) && moe_dec_gu_topk_supported(g.experts, g.topk);
   bool fused = false;
   if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
                                     c->logits, c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
@@ -443,10 +443,14 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   }
   if (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
   if (use_int4k) {
-    if ((rc = moe_launch_dec4k_gu(L.gg.gate, L.gg.up, L.has_shared ? L.sh_gate.data : nullptr,
-                                  L.has_shared ? L.sh_up.data : nullptr, c->xplanes, c->xmeta, c->ids, g.id_stride,
-                                  g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, st)))
-      return rc;
+    rc = gu_topk ? moe_launch_dec4k_gu_topk(L.gg.gate, L.gg.up, L.has_shared ? L.sh_gate.data : nullptr,
+                                            L.has_shared ? L.sh_up.data : nullptr, c->xplanes, c->xmeta, c->logits,
+                                            g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
+                                            c->hplanes, c->hmeta, st)
+                 : moe_launch_dec4k_gu(L.gg.gate, L.gg.up, L.has_shared ? L.sh_gate.data : nullptr,
+                                       L.has_shared ? L.sh_up.data : nullptr, c->xplanes, c->xmeta, c->ids,
+                                       g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, st);
+    if (rc) return rc;
     prof_mark(c, MOE_PROF_UP, st);
     rc = moe_launch_dec4k_dn(L.gg.down, L.has_shared ? L.sh_down.data : nullptr, c->sh_logit, c->hplanes, c->hmeta,
                              c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, y, (uint64_t)g.d, st);

@@ -10,6 +10,7 @@
 #include "common.h"
 #include "internal.h"
 #include "qvec.h"
+#include "topk.h"
 
 namespace {
 
@@ -101,41 +102,67 @@ struct Gu4kArgs {
 // grid (mid/32, slots incl. shared, P); block 512.  Wave w: gate rows 4w..4w+3 and the matching up
 // rows of this block's 32; lane = unit (d/64 <= 64 units per row).  All 24 loads of a lane (8 rows x
 // two code halves + header) are in flight together.
+// NPL > 0 (E <= 64*NPL): only the logits are given; the blocks of the routed slots run the softmax /
+// top-k of their token themselves and block (0, 0, token) writes ids / weights out for the down
+// kernel (as in the q4cp gate/up kernel).
 constexpr int G4_ROWS = 32;
+template <int NPL>
 __global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t* __restrict__ xplanes,
                                                      const float2* __restrict__ xmeta,
                                                      const int* __restrict__ ids, int id_stride, int kpt, int d,
                                                      int mid, uint32_t* __restrict__ hplanes,
-                                                     float2* __restrict__ hmeta) {
+                                                     float2* __restrict__ hmeta, const float* __restrict__ logits,
+                                                     int n_experts, int* __restrict__ ids_out,
+                                                     float* __restrict__ ws_out) {
   __shared__ float gs[G4_ROWS], us[G4_ROWS];
   __shared__ uint32_t pk[QV_GROUP_DW];
+  __shared__ int sel_ids[64];
+  __shared__ float sel_ws[64];
   const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int U = d / 64;
   const bool shared = s >= kpt;
   const uint64_t rb = (uint64_t)(d / 256) * 144;
-  const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
+  int e = 0;
+  if (NPL > 0) {
+    if (!shared) {
+      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      __syncthreads();
+      e = sel_ids[s];
+      if (blockIdx.x == 0 && s == 0 && (int)threadIdx.x < kpt) {
+        ids_out[(size_t)tok * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
+        ws_out[(size_t)tok * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+      }
+    }
+  } else if (!shared) {
+    e = ids[(size_t)tok * id_stride + s];
+  }
   const uint8_t* gbase = shared ? A.sh_gate : A.gate + (uint64_t)e * mid * rb;
   const uint8_t* ubase = shared ? A.sh_up : A.up + (uint64_t)e * mid * rb;
   const int r0 = blockIdx.x * G4_ROWS + 4 * wv;
+  // branch-free loads: lanes past the row's units read unit 0 and count as zero
   const bool live = lane < U;
-  const int jj = lane & 3;
-  const size_t uoff = (size_t)(lane >> 2) * 144;  // this lane's super-block inside a row
+  const int ul = live ? lane : 0;
+  const float mlive = live ? 1.f : 0.f;
+  const int jj = ul & 3;
+  const size_t uoff = (size_t)(ul >> 2) * 144;  // this lane's super-block inside a row
+  XU x;
+  load_xu(x, xplanes, xmeta, ((size_t)tok * U + ul) * 2);
   uint4 c0[8], c1[8], hd[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     const uint8_t* row = (i < 4 ? gbase : ubase) + (uint64_t)(r0 + (i & 3)) * rb + uoff;
-    if (live) {
-      hd[i] = *(const uint4*)row;
-      c0[i] = *(const uint4*)(row + 16 + jj * 32);
-      c1[i] = *(const uint4*)(row + 32 + jj * 32);
-    }
+    hd[i] = *(const uint4*)row;
+    c0[i] = *(const uint4*)(row + 16 + jj * 32);
+    c1[i] = *(const uint4*)(row + 32 + jj * 32);
   }
-  XU x;
-  if (live) load_xu(x, xplanes, xmeta, ((size_t)tok * U + lane) * 2);
+  __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first dot product
   float acc[8];
 #pragma unroll
-  for (int i = 0; i < 8; i++) acc[i] = sum64(live ? unit_dot(c0[i], c1[i], hd[i], jj, x) : 0.f);
+  for (int i = 0; i < 8; i++) {
+    acc[i] = sum64(unit_dot(c0[i], c1[i], hd[i], jj, x) * mlive);
+    if (i & 1) __builtin_amdgcn_sched_barrier(0);  // rows are consumed in arrival order
+  }
   if (lane == 0) {
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -191,43 +218,52 @@ __global__ void __launch_bounds__(256) k_dec4k_dn(Dn4kArgs A, const uint32_t* __
                                                   const float* __restrict__ ws, int id_stride, int kpt, int d,
                                                   int mid, float* __restrict__ out, uint64_t out_stride) {
   __shared__ float part[D4_MAXSLOTS][D4_ROWS];
+  __shared__ float wsm[D4_MAXSLOTS];
   const int tok = blockIdx.y;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const bool has_shared = A.sh_down != nullptr;
   const int nslots = kpt + (has_shared ? 1 : 0);
-  const int U = mid / 64, u = lane & 15, s = 4 * wv + (lane >> 4);
+  const int U = mid / 64, u_raw = lane & 15, s_raw = 4 * wv + (lane >> 4);
   const int r0 = blockIdx.x * D4_ROWS;
   const uint64_t rb = (uint64_t)(mid / 256) * 144;
+  // combine weights of the token, fetched while the weight rows are in flight
+  float wmine = 0.f;
+  if ((int)threadIdx.x < nslots)
+    wmine = (int)threadIdx.x < kpt ? ws[(size_t)tok * id_stride + threadIdx.x] : A.sh_logit[tok];
   {
-    const bool live = s < nslots && u < U;
+    // branch-free loads: lanes past the slots or the row's units read slot 0 / unit 0 and count as zero
+    const bool live = s_raw < nslots && u_raw < U;
+    const int s = live ? s_raw : 0, u = live ? u_raw : 0;
+    const float mlive = live ? 1.f : 0.f;
     const bool shared = has_shared && s == nslots - 1;
-    const int e = (live && !shared) ? ids[(size_t)tok * id_stride + s] : 0;
+    const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
     const uint8_t* base = (shared ? A.sh_down : A.down + (uint64_t)e * d * rb) + (uint64_t)r0 * rb + (size_t)(u >> 2) * 144;
     const int jj = u & 3;
+    XU x;
+    load_xu(x, hplanes, hmeta, (((size_t)tok * nslots + s) * U + u) * 2);
     uint4 c0[D4_ROWS], c1[D4_ROWS], hd[D4_ROWS];
 #pragma unroll
     for (int r = 0; r < D4_ROWS; r++) {
-      if (live) {
-        const uint8_t* row = base + (uint64_t)r * rb;
-        hd[r] = *(const uint4*)row;
-        c0[r] = *(const uint4*)(row + 16 + jj * 32);
-        c1[r] = *(const uint4*)(row + 32 + jj * 32);
-      }
+      const uint8_t* row = base + (uint64_t)r * rb;
+      hd[r] = *(const uint4*)row;
+      c0[r] = *(const uint4*)(row + 16 + jj * 32);
+      c1[r] = *(const uint4*)(row + 32 + jj * 32);
     }
-    XU x;
-    if (live) load_xu(x, hplanes, hmeta, (((size_t)tok * nslots + s) * U + u) * 2);
+    __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first dot product
 #pragma unroll
     for (int r = 0; r < D4_ROWS; r++) {
-      const float v = dpp_add_row(live ? unit_dot(c0[r], c1[r], hd[r], jj, x) : 0.f);
-      if (u == 0 && s < nslots) part[s][r] = v;
+      const float v = dpp_add_row(unit_dot(c0[r], c1[r], hd[r], jj, x) * mlive);
+      if (u_raw == 0 && s_raw < nslots) part[s_raw][r] = v;
+      if (r & 1) __builtin_amdgcn_sched_barrier(0);  // rows are consumed in arrival order
     }
   }
+  if ((int)threadIdx.x < nslots) wsm[threadIdx.x] = (int)threadIdx.x < kpt ? wmine : sigmoid_f(wmine);
   __syncthreads();
   if (threadIdx.x < D4_ROWS) {
     const int r = threadIdx.x;
     float y = 0.f;
-    for (int i = 0; i < kpt; i++) y += ws[(size_t)tok * id_stride + i] * part[i][r];
-    if (has_shared) y += sigmoid_f(A.sh_logit[tok]) * part[kpt][r];
+    for (int i = 0; i < kpt; i++) y += wsm[i] * part[i][r];
+    if (has_shared) y += wsm[kpt] * part[kpt][r];
     out[(size_t)tok * out_stride + r0 + r] = y;
   }
 }
@@ -247,7 +283,30 @@ int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* s
     return MOE_E_INVALID;
   Gu4kArgs A{gate, up, sh_gate, sh_up};
   dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0), P);
-  k_dec4k_gu<<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta);
+  k_dec4k_gu<0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, nullptr, 0,
+                                      nullptr, nullptr);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// The same with the softmax / top-k of every token done inside the launch: logits [P][n_experts] in,
+// ids / ws rows (id_stride wide) out.
+int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
+                             const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
+                             int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st) {
+  if (!gate || !up || !xplanes || !xmeta || !logits || !ids || !ws || !hplanes || !hmeta || (!sh_gate != !sh_up))
+    return MOE_E_INVALID;
+  if (!moe_aligned(gate, 16) || !moe_aligned(up, 16) || (sh_gate && (!moe_aligned(sh_gate, 16) || !moe_aligned(sh_up, 16))))
+    return MOE_E_INVALID;
+  Gu4kArgs A{gate, up, sh_gate, sh_up};
+  dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0), P);
+  if (n_experts <= 512)
+    k_dec4k_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta, logits,
+                                        n_experts, ids, ws);
+  else
+    k_dec4k_gu<16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta, logits,
+                                         n_experts, ids, ws);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

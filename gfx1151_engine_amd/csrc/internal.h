@@ -60,6 +60,10 @@ int moe_launch_dec_dn_uq(const moe_wview* dn, const moe_wview* sh_down, const ui
                          int n_experts, int d, int mid, float* pairs, hipStream_t st);
 // the same for raw GGUF Q4_K rows (activation planes in natural order)
 bool moe_dec4k_supported(int d, int mid, int nslots);
+int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
+                             const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
+                             int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st);
 int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
                         const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                         int P, int d, int mid, uint32_t* hplanes, float2* hmeta, hipStream_t st);
