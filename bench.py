@@ -191,6 +191,68 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
     return res
 
 
+def measure_load(fmt, steps, nlayers):
+    """Checkpoint file -> HBM: writes `nlayers` synthetic full-size layers to a temporary .hgn / GGUF file,
+    then times moe_load_layers (file mapping -> one H2D copy per tensor -> registration).  Host-side,
+    PCIe-bound set-up work: reported beside the hot path, never as its throughput."""
+    import tempfile
+    import torch
+    from gfx1151_engine_amd import capi, files, workloads as W
+    d, mid, k = D, MID, K
+    tmp = tempfile.mkdtemp(prefix="moe_load_")
+    path = os.path.join(tmp, "layers.hgn" if fmt == "q4cp" else "layers.gguf")
+    tens = []
+    for l in range(nlayers):
+        L = W.DeviceLayer(2000 + l, d, mid, E, k, fmt)
+        h = lambda t: t.cpu().numpy()
+
+        class HL:  # the attribute names files.*_layer_tensors read
+            pass
+        hl = HL()
+        hl.d, hl.mid, hl.E = d, mid, E
+        hl.router = h(L.router)
+        hl.shared = [h(L.sh[0]), h(L.sh[1]), h(L.sh[2]), h(L.sh_sg)]
+        hl.down = h(L.down)
+        if fmt == "q4cp":
+            hl.gate_up = h(L.gate_up)
+            tens += files.hgn_layer_tensors(l, hl)
+        else:
+            hl.gate, hl.up = h(L.gate), h(L.up)
+            hl.shared[3] = hl.shared[3].reshape(-1)
+            tens += files.gguf_layer_tensors(l, hl)
+        del L
+        torch.cuda.empty_cache()
+    (files.write_hgn if fmt == "q4cp" else files.write_gguf)(path, tens)
+    del tens
+    nbytes = os.path.getsize(path)
+    times = []
+    try:
+        for i in range(steps + 1):  # the first pass also pages the file in: not timed
+            f = capi.ModelFile(path)
+            cfg = f.config(0)
+            m = capi.Moe(cfg.d, cfg.mid, cfg.experts, k, layers=cfg.layers, max_tokens=1)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            w = f.load_layers(m, 0, 0, cfg.layers)
+            torch.cuda.synchronize()
+            if i:
+                times.append(time.perf_counter() - t0)
+            wb = w.nbytes
+            f.close()
+            m.close()
+            w.free()
+    finally:
+        os.remove(path)
+        os.rmdir(tmp)
+    ms = 1e3 * sum(times) / len(times)
+    return {"metric": "moe_file_load_GB_per_s", "value": round(wb / (ms * 1e-3) / 1e9, 2), "unit": "GB/s", "n_gpus": 1,
+            "steps": steps, "warmup": 1, "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+            "config": {"workload": "load_" + fmt, "layers": nlayers, "file_bytes": nbytes, "device_bytes": int(wb),
+                       "format": ".hgn (HGN1)" if fmt == "q4cp" else "GGUF v3", "path": "page cache -> pageable H2D copy"},
+            "roofline": None, "cpu_baseline": None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -225,6 +287,8 @@ def main():
         res["decode_T1"] = {kk: dec[kk] for kk in ("metric", "value", "unit", "hbm_frac", "ms_per_step", "steps",
                                                    "stage_ms", "dtype", "roofline", "config", "cpu_baseline")
                             if kk in dec}
+    elif a.workload in ("load", "q4k_load"):
+        res = measure_load("q4k" if a.workload.startswith("q4k") else "q4cp", min(a.steps, 5), min(a.layers, 2))
     else:
         res = measure(a.workload, a.steps, a.warmup, a.tokens, a.layers, cpu=not a.no_cpu)
     print(json.dumps(res))

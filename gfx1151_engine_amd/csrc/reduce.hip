@@ -73,7 +73,7 @@ struct Ld8<float> {
   }
 };
 
-template <class PT, int KMAX>
+template <class PT, int KMAX, int KC>  // KC = K when it is one of the instantiated values, else 0
 __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pairs,
                                                       const int* __restrict__ pairids,
                                                       const float* __restrict__ pw,
@@ -93,15 +93,30 @@ __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pai
   const int c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
   if (c >= D) return;
   float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (KC > 0) {
+    // K known at compile time: all pair rows are requested before the first is used (a load under
+    // the run-time `s < K` test is waited for where it is issued), summed in the same slot order
+    float v[KC > 0 ? KC : 1][8];
 #pragma unroll
-  for (int s = 0; s < KMAX; s++)
-    if (s < K) {
-      float v[8];
-      Ld8<PT>::ld(pairs + (size_t)ids[s] * D + c, v);
+    for (int s = 0; s < KC; s++) Ld8<PT>::ld(pairs + (size_t)ids[s] * D + c, v[s]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < KC; s++) {
       const float ww = w[s];
 #pragma unroll
-      for (int i = 0; i < 8; i++) sum[i] += ww * v[i];
+      for (int i = 0; i < 8; i++) sum[i] += ww * v[s][i];
     }
+  } else {
+#pragma unroll
+    for (int s = 0; s < KMAX; s++)
+      if (s < K) {
+        float v[8];
+        Ld8<PT>::ld(pairs + (size_t)ids[s] * D + c, v);
+        const float ww = w[s];
+#pragma unroll
+        for (int i = 0; i < 8; i++) sum[i] += ww * v[i];
+      }
+  }
   // pairs of the batch path carry the f16 range-guard factor of their token: divide it out
   float inv_r = 1.f, inv_s = 1.f;
   if (hs.xms) {
@@ -190,10 +205,13 @@ int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, con
   if (!moe_aligned(pairs, 16) || !moe_aligned(out, 16) || (ey && !moe_aligned(ey, 16))) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
   dim3 grid((D / 8 + 127) / 128, P);
-  if (pairs_f16)
-    k_reduce_pw_sg<__half, 16><<<grid, 128, 0, st>>>((const __half*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs);
-  else
-    k_reduce_pw_sg<float, 16><<<grid, 128, 0, st>>>((const float*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs);
+#define RED_GO(PT, KC) k_reduce_pw_sg<PT, 16, KC><<<grid, 128, 0, st>>>((const PT*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs)
+  if (pairs_f16) {
+    if (K == 10) RED_GO(__half, 10); else if (K == 8) RED_GO(__half, 8); else RED_GO(__half, 0);
+  } else {
+    if (K == 10) RED_GO(float, 10); else if (K == 8) RED_GO(float, 8); else RED_GO(float, 0);
+  }
+#undef RED_GO
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
