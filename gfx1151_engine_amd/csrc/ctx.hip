@@ -213,6 +213,12 @@ MOE_API int moe_set_experts_q4cp(moe_ctx* c, int layer, const moe_wview* gu, con
   return MOE_OK;
 }
 
+MOE_API int moe_get_config(const moe_ctx* c, moe_config* out) {
+  if (!c || !out) return MOE_E_INVALID;
+  *out = c->cfg;
+  return MOE_OK;
+}
+
 MOE_API int moe_set_experts_gguf(moe_ctx* c, int layer, const moe_gg_experts* gg) {
   MoeLayer* L = layer_of(c, layer);
   if (!L || !gg || !gg->gate || !gg->up || !gg->down) return MOE_E_INVALID;

@@ -203,9 +203,12 @@ static int parse_gguf(moe_file* f) {
   for (auto& p : ts) {
     uint32_t be, bb;
     if (!ggml_block((uint32_t)p.t.dtype, be, bb)) return MOE_E_UNSUPPORTED;
-    const uint64_t numel = p.t.dims[0] * p.t.dims[1] * p.t.dims[2] * p.t.dims[3];
+    // element count without wrap-around: a crafted file must not get a small byte size for huge dims
+    uint64_t numel = 1;
+    for (int k = 0; k < 4; k++)
+      if (__builtin_mul_overflow(numel, p.t.dims[k], &numel)) return MOE_E_INVALID;
     if (p.t.dims[0] % be) return MOE_E_INVALID;
-    p.t.nbytes = numel / be * bb;
+    if (__builtin_mul_overflow(numel / be, (uint64_t)bb, &p.t.nbytes)) return MOE_E_INVALID;
     const uint64_t off = data0 + p.off;
     if (off > f->len || p.t.nbytes > f->len - off) return MOE_E_INVALID;
     p.t.data = f->base + off;
@@ -284,15 +287,18 @@ const FTensor* find(const moe_file* f, const char* fmt, int layer) {
 
 // rows x cols of a matrix tensor: hgn dims are outermost first (3-D fused experts flatten to
 // [E*rows, cols], src/hgn.h:7-8), gguf ne[] is innermost first
-void matrix_shape(int format, const FTensor& t, uint64_t& rows, uint64_t& cols) {
+bool matrix_shape(int format, const FTensor& t, uint64_t& rows, uint64_t& cols) {
+  rows = 1;
   if (format == MOE_FILE_HGN) {
     cols = t.dims[t.nd ? t.nd - 1 : 0];
-    rows = 1;
-    for (uint32_t k = 0; k + 1 < t.nd; k++) rows *= t.dims[k];
+    for (uint32_t k = 0; k + 1 < t.nd; k++)
+      if (__builtin_mul_overflow(rows, t.dims[k], &rows)) return false;
   } else {
     cols = t.dims[0];
-    rows = t.dims[1] * t.dims[2] * t.dims[3];
+    for (int k = 1; k < 4; k++)
+      if (__builtin_mul_overflow(rows, t.dims[k], &rows)) return false;
   }
+  return true;
 }
 
 }  // namespace
@@ -311,13 +317,16 @@ MOE_API int moe_file_config(const moe_file* f, int layer, moe_config* cfg) {
     const FTensor* rt = find(f, "layers.%d.mlp.gate.weight", layer);
     if (!rt || rt->nd != 2) return MOE_E_STATE;
     uint64_t rows, cols;
-    matrix_shape(f->format, *dn, rows, cols);
+    if (!matrix_shape(f->format, *dn, rows, cols) || rt->dims[0] > (1u << 20) || rt->dims[1] > (1u << 24) ||
+        cols > (1u << 24))
+      return MOE_E_INVALID;
     cfg->experts = (int)rt->dims[0];
     cfg->d = (int)rt->dims[1];
     cfg->mid = (int)cols;
     if (rows != (uint64_t)cfg->experts * cfg->d) return MOE_E_INVALID;
   } else {
-    if (dn->nd != 3) return MOE_E_INVALID;
+    if (dn->nd != 3 || dn->dims[0] > (1u << 24) || dn->dims[1] > (1u << 24) || dn->dims[2] > (1u << 20))
+      return MOE_E_INVALID;
     cfg->mid = (int)dn->dims[0];
     cfg->d = (int)dn->dims[1];
     cfg->experts = (int)dn->dims[2];
@@ -356,11 +365,23 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
   int rc;
   auto view = [&](const FTensor& t, moe_wview* v) -> int {
     uint64_t rows, cols;
-    matrix_shape(MOE_FILE_HGN, t, rows, cols);
+    if (!matrix_shape(MOE_FILE_HGN, t, rows, cols)) return MOE_E_INVALID;
     v->dtype = t.dtype;
     v->rows = rows;
     v->cols = cols;
     v->scale_stride = t.dtype == MOE_DT_Q4CP ? (((cols / 32 * 2) + 15) & ~15ULL) : 0;
+    // the record's byte count must be what the kernels will read for these dims (src/hgn.h:225-233)
+    uint64_t want, cells;
+    if (__builtin_mul_overflow(rows, cols, &cells)) return MOE_E_INVALID;
+    if (t.dtype == MOE_DT_Q4CP) {
+      uint64_t sc;
+      if (cols % 32 || __builtin_mul_overflow(rows, (uint64_t)v->scale_stride, &sc) ||
+          __builtin_add_overflow(64 + cells / 2, sc, &want))
+        return MOE_E_INVALID;
+    } else if (__builtin_mul_overflow(cells, (uint64_t)(t.dtype == MOE_DT_F32 ? 4 : 2), &want)) {
+      return MOE_E_INVALID;
+    }
+    if (t.nbytes != want) return MOE_E_INVALID;
     return upload(w, t, st, &v->data);
   };
   moe_wview vr{}, vgu{}, vdn{};
@@ -385,12 +406,21 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
 
 int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st) {
   const FTensor* rt = find(f, "blk.%d.ffn_gate_inp.weight", fl);
-  const FTensor* g = find(f, "blk.%d.ffn_gate_exps.weight", fl);
+  const FTensor* g_ = find(f, "blk.%d.ffn_gate_exps.weight", fl);
   const FTensor* u = find(f, "blk.%d.ffn_up_exps.weight", fl);
   const FTensor* dn = find(f, "blk.%d.ffn_down_exps.weight", fl);
-  if (!rt || !g || !u || !dn) return MOE_E_STATE;
+  if (!rt || !g_ || !u || !dn) return MOE_E_STATE;
   if (rt->dtype != 0 && rt->dtype != 30) return MOE_E_UNSUPPORTED;  // F32 / BF16 router
   int rc;
+  // raw GGUF blocks are registered by pointer only: the shapes the kernels will read are the
+  // context's, so the file's must be exactly those
+  moe_config g{};
+  if ((rc = moe_get_config(ctx, &g))) return rc;
+  auto is = [](const FTensor& t, uint64_t a, uint64_t b, uint64_t c) {
+    return t.dims[0] == a && t.dims[1] == b && t.dims[2] == c && t.dims[3] == 1;
+  };
+  const uint64_t D = (uint64_t)g.d, M = (uint64_t)g.mid, NE = (uint64_t)g.experts;
+  if (!is(*rt, D, NE, 1) || !is(*g_, D, M, NE) || !is(*u, D, M, NE) || !is(*dn, M, D, NE)) return MOE_E_INVALID;
   moe_wview vr{};
   vr.dtype = rt->dtype == 0 ? MOE_DT_F32 : MOE_DT_BF16;
   vr.cols = rt->dims[0];
@@ -398,10 +428,10 @@ int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights
   if ((rc = upload(w, *rt, st, &vr.data))) return rc;
   if ((rc = moe_set_router(ctx, cl, &vr, nullptr))) return rc;
   moe_gg_experts gg{};
-  gg.tgu = g->dtype;
+  gg.tgu = g_->dtype;
   gg.tdn = dn->dtype;
-  if (u->dtype != g->dtype) return MOE_E_UNSUPPORTED;
-  if ((rc = upload(w, *g, st, &gg.gate)) || (rc = upload(w, *u, st, &gg.up)) || (rc = upload(w, *dn, st, &gg.down))) return rc;
+  if (u->dtype != g_->dtype) return MOE_E_UNSUPPORTED;
+  if ((rc = upload(w, *g_, st, &gg.gate)) || (rc = upload(w, *u, st, &gg.up)) || (rc = upload(w, *dn, st, &gg.down))) return rc;
   if ((rc = moe_set_experts_gguf(ctx, cl, &gg))) return rc;  // MOE_E_UNSUPPORTED for types other than Q4_K
   const FTensor* sg = find(f, "blk.%d.ffn_gate_shexp.weight", fl);
   if (sg) {
@@ -412,6 +442,7 @@ int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights
     if (sg->dtype != MOE_GGML_Q4_K || su->dtype != MOE_GGML_Q4_K || sd->dtype != MOE_GGML_Q4_K ||
         (sx->dtype != 0 && sx->dtype != 30))
       return MOE_E_UNSUPPORTED;
+    if (!is(*sg, D, M, 1) || !is(*su, D, M, 1) || !is(*sd, M, D, 1) || !is(*sx, D, 1, 1)) return MOE_E_INVALID;
     moe_wview a{}, b{}, c2{}, d2{};
     auto raw = [&](const FTensor& t, moe_wview* v) -> int {
       v->dtype = 0;

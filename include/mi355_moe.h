@@ -175,6 +175,8 @@ typedef struct moe_config {
 
 typedef struct moe_ctx moe_ctx;
 int moe_create(const moe_config* cfg, moe_ctx** out);
+/* The configuration the context was created with (no counterpart in the reference: its g_cfg is a global). */
+int moe_get_config(const moe_ctx* ctx, moe_config* out);
 int moe_destroy(moe_ctx* ctx);
 /* weights of one layer; all pointers are device memory owned by the caller.
  * router: mlp.gate.weight [E][d] (f32 / bf16); router_bias optional (synthetic skew).

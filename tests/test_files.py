@@ -113,6 +113,19 @@ def test_malformed_files_are_rejected(tmp_path):
     assert rc_of(tmp_path / "v1.gguf") == -1
 
 
+def test_gguf_dims_that_wrap_around_are_rejected(tmp_path):
+    # ne = [2^33, 2^33, 1]: the element count wraps to 4 in 64 bits; the parser must not accept 16 bytes for it
+    name = b"blk.0.ffn_down_exps.weight"
+    hdr = b"GGUF" + struct.pack("<IQQ", 3, 1, 0)
+    hdr += struct.pack("<Q", len(name)) + name + struct.pack("<I", 3) + struct.pack("<3Q", 1 << 33, 1 << 33, 1)
+    hdr += struct.pack("<IQ", files.GGML_F32, 0)
+    pad = (-len(hdr)) % 32
+    p = tmp_path / "wrap.gguf"
+    p.write_bytes(hdr + b"\0" * pad + b"\0" * 64)
+    h = C.c_void_p()
+    assert capi.lib().moe_file_open(str(p).encode(), C.byref(h)) == -2
+
+
 def _x(T, seed=11):
     return np.random.default_rng(seed).standard_normal((T, D), dtype=np.float32)
 
@@ -169,3 +182,42 @@ def test_load_rejects_types_outside_the_path(tmp_path):
     x = torch.zeros(1, D, device="cuda")
     y = torch.empty_like(x)
     assert capi.lib().moe_forward(m.h, 0, capi.ptr(x), 1, capi.ptr(y), capi.stream()) == -3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt", ["q4cp", "q4k"])
+def test_load_rejects_shapes_that_differ_from_the_context(tmp_path, fmt):
+    # the kernels read what the context's shapes say: a file whose tensors are smaller must not be registered
+    import torch
+    layers = _layers(fmt, n=1, seed=4)
+    p, _ = (_hgn if fmt == "q4cp" else _gguf)(tmp_path, layers, first=0)
+    f = capi.ModelFile(p)
+    for d, mid, e in ((D, 2 * MID, E), (2 * D, MID, E), (D, MID, 2 * E)):
+        m = capi.Moe(d, mid, e, K, layers=1, max_tokens=8)
+        w = C.c_void_p()
+        assert capi.lib().moe_load_layers(m.h, f.h, 0, 0, 1, C.byref(w), capi.stream()) == -2, (d, mid, e)
+        x = torch.zeros(1, d, device="cuda")
+        y = torch.empty_like(x)
+        assert capi.lib().moe_forward(m.h, 0, capi.ptr(x), 1, capi.ptr(y), capi.stream()) == -3
+        cfg = capi.Config()
+        assert capi.lib().moe_get_config(m.h, C.byref(cfg)) == 0 and (cfg.d, cfg.mid, cfg.experts) == (d, mid, e)
+        m.close()
+    f.close()
+
+
+@pytest.mark.gpu
+def test_hgn_record_size_must_match_its_dims(tmp_path):
+    # a q4cp record that claims more rows than its bytes hold
+    layers = _layers("q4cp", n=1, seed=6)
+    ts = files.hgn_layer_tensors(0, layers[0])
+    name, dt, dims, data = ts[1]
+    ts[1] = (name, dt, [dims[0] * 2, dims[1], dims[2]], data)   # experts doubled, bytes unchanged
+    p = tmp_path / "short.hgn"
+    files.write_hgn(p, ts)
+    f = capi.ModelFile(p)
+    m = capi.Moe(D, MID, 2 * E, K, layers=1, max_tokens=8)
+    w = C.c_void_p()
+    assert capi.lib().moe_load_layers(m.h, f.h, 0, 0, 1, C.byref(w), capi.stream()) == -2
+    m.close()
+    f.close()
+
