@@ -65,6 +65,42 @@ __device__ __forceinline__ void topk_select(uint32_t (&key)[NPL], int lane, int 
   }
 }
 
+// The same with the keys held lane-major (key[j] of lane l = expert NPL*l + j): among equal keys
+// the lowest expert is then in the lowest lane, so the second wave-wide reduction becomes a ballot
+// and a find-first-one, and the winner's register index is one lane read.
+template <int NPL>
+__device__ __forceinline__ void topk_select_lm(uint32_t (&key)[NPL], int lane, int k, int* ids_row, float* ws_row) {
+  double wsum = 0.0;
+  float mine = 0.f;
+  int myid = 0;
+  for (int r = 0; r < k; r++) {
+    uint32_t m = key[0];
+    int jm = 0;
+#pragma unroll
+    for (int j = 1; j < NPL; j++) {
+      const bool gt = key[j] > m;  // strict: the lowest register (= lowest expert index) wins a tie
+      m = gt ? key[j] : m;
+      jm = gt ? j : jm;
+    }
+    const uint32_t wm = wave_umax(m);
+    const int wl = __builtin_ctzll(__ballot(m == wm));          // lowest lane holding the maximum
+    const int wj = __builtin_amdgcn_readlane(jm, wl);           // its register
+    const float bv = __uint_as_float(wm - 1u);
+    wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
+    if (lane == r) {
+      mine = bv;
+      myid = NPL * wl + wj;
+    }
+    const bool me = lane == wl;
+#pragma unroll
+    for (int j = 0; j < NPL; j++) key[j] = (me && j == wj) ? 0u : key[j];
+  }
+  if (lane < k) {
+    ids_row[lane] = myid;
+    ws_row[lane] = (float)((double)mine / wsum);
+  }
+}
+
 // The softmax / top-k of one token by one block of NT threads (E <= 64*NPL): the fp64 exps, the
 // costly part, are spread over the block; wave 0 then runs the k selection rounds on the keys in
 // LDS.  COH: the logits were written by other blocks of the same launch: read them with
@@ -133,6 +169,6 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
   if (wv != 0) return;
   uint32_t key[NPL];
 #pragma unroll
-  for (int j = 0; j < NPL; j++) key[j] = keys[lane + 64 * j];
-  topk_select<NPL>(key, lane, k, ids_row, ws_row);
+  for (int j = 0; j < NPL; j++) key[j] = keys[NPL * lane + j];
+  topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
 }
