@@ -42,6 +42,23 @@ def test_small_batch_layer(oracle, fmt, d, mid, E, k, T, cb):
     assert max_abs_rel(y, yo) <= TOL_GEMV
 
 
+@pytest.mark.parametrize("fmt,T,rdt", [("q4cp", 3, "f32"), ("q4cp", 32, "f32"), ("q4k", 27, "f32"), ("q4k", 2, "f32"),
+                                        ("q4cp", 1, "bf16"), ("q4cp", 4, "bf16"), ("q4cp", 12, "bf16"),
+                                        ("q4k", 30, "bf16")])
+def test_small_batch_sizes_and_router_dtypes(oracle, fmt, T, rdt):
+    """The token counts at which the small path changes kernels (1 / 2-4 / 5-24 / 25-32: the logits
+    launch differs, above 24 tokens it is split in two) with f32 and bf16 router matrices."""
+    rng = np.random.default_rng(4242 + 7 * T + (rdt == "bf16"))
+    d, mid, E, k = 3072, 768, 24, 10
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt, router_dtype=rdt)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    y, ids, ws = run_layer(hl, x)
+    assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
+    assert np.abs(ws[:, :k] - wo[:, :k]).max() <= 1e-6
+    assert max_abs_rel(y, yo) <= TOL_GEMV
+
+
 @pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 9), ("q4k", 1), ("q4k", 9)])
 def test_int_decode_switch(oracle, fmt, T):
     """MOE_OPT_INT_DECODE 1 (integer-dot kernels, default) and 0 (f32 kernels) both meet the GEMV bar
