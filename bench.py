@@ -173,9 +173,9 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
                                  "unit": "TFLOP/s", "frac": round(up_flop / up_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                                  "traffic": PMC_TRAFFIC.get((kind, fmt, T))}})
         # rows the grouped GEMM computes for the routed pairs: tiles of 128, the last tile of an expert padded
-        # to 32 / 64 / 128 rows
+        # to a multiple of 32 rows
         rem = cnt % 128
-        padded = (cnt // 128) * 128 + np.where(rem == 0, 0, np.where(rem <= 32, 32, np.where(rem <= 64, 64, 128)))
+        padded = (cnt // 128) * 128 + (rem + 31) // 32 * 32
         cfg.update({"hottest_over_mean": round(float(cnt.max() / cnt.mean()), 2), "empty_experts": int((cnt == 0).sum()),
                     "tile_row_fill": round(float(cnt.sum() / max(1, padded.sum())), 4)})
     else:

@@ -108,7 +108,7 @@ __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, LDS_PTR(lds_base), 16, 0, 0);
 }
 
-// MF = live 32-row fragments of the tile (1, 2 or 4); AFFINE = codebook a*n+b.
+// MF = live 32-row fragments of the tile (1 .. 4); AFFINE = codebook a*n+b.
 // NF = weight fragments (32 rows) per wave: the block's 16 fragments are split over NW = 16/NF
 // waves, each wave multiplying all MF pair fragments with its own NF weight fragments.
 template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K>
@@ -158,7 +158,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // The 4*MF row groups are dealt to the waves; with more waves than groups some load a group twice
   // (same bytes to the same place) so that every wave issues the same number of loads.
   constexpr int A_GROUPS = 4 * MF;
-  constexpr int A_LOADS = A_GROUPS >= NW ? A_GROUPS / NW : 1;
+  constexpr int A_LOADS = (A_GROUPS + NW - 1) / NW;
   constexpr int W_LOADS = 16 / NW, S_LOADS = 8 / NW;
   const __half* a_src[A_LOADS];
   int a_grp[A_LOADS];
@@ -551,6 +551,7 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
+  else if (mfn == 3) GEMM_GO(3);
   else GEMM_GO(4);
 #undef GEMM_GO
 }
