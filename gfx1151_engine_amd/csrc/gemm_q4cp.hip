@@ -114,14 +114,15 @@ __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
 template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
-                                          int K, float cb_a, float cb_b) {
+                                          int K, float cb_a, float cb_b, int ri, const float* __restrict__ xms,
+                                          float cmag) {
   constexpr int NH = NF / 2;  // gate/up: fragments per half
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
   const float* cbs = (const float*)(S0 + 2 * S_BYTES);
-  const int* rowidx = (const int*)(cbs + 16);
-  const float* rowscale = (const float*)(rowidx + BM);  // f16 range guard of each pair row (gate/up only)
+  int* rowidx = (int*)(cbs + 16);
+  float* rowscale = (float*)(rowidx + BM);  // f16 range guard of each pair row (gate/up only)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, kept scalar
   const int n = lane & 31, h = lane >> 5;
@@ -163,11 +164,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   const __half* a_src[A_LOADS];
   int a_grp[A_LOADS];
 #pragma unroll
-  for (int i = 0; i < A_LOADS; i++) {
-    a_grp[i] = (A_LOADS * wv + i) % A_GROUPS;
-    const int m = 8 * a_grp[i] + (lane >> 3);
-    a_src[i] = x + (size_t)rowidx[m] * K + (((lane & 7) ^ ((m >> 1) & 7)) << 3);
-  }
+  for (int i = 0; i < A_LOADS; i++) a_grp[i] = (A_LOADS * wv + i) % A_GROUPS;  // a_src: once the row indices are in LDS
   // codes: rows 32j..32j+31, lane -> (row 32j + lane/2, half lane%2); scales: rows 64j.., lane -> row
   const uint8_t *w_src[W_LOADS], *s_src[S_LOADS];
 #pragma unroll
@@ -201,9 +198,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       g2l16(s_src[i] + off, S0 + ((s >> 2) & 1) * S_BYTES + (S_LOADS * wv + i) * 1024);
     }
   };
-  auto issue = [&](int s) {
+  auto issue_a = [&](int s) {
 #pragma unroll
-    for (int u = 0; u < NLOADS; u++) issue_unit(s, u);
+    for (int u = 0; u < A_LOADS; u++) issue_unit(s, u);
+  };
+  auto issue_w = [&](int s) {  // codes, and the scales on every fourth stage
+#pragma unroll
+    for (int u = A_LOADS; u < NLOADS; u++) issue_unit(s, u);
     if ((s & 3) == 0) {
 #pragma unroll
       for (int u = 0; u < S_LOADS; u++) issue_unit(s, NLOADS + u);
@@ -351,12 +352,28 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   constexpr int X0 = NM >= 8 ? NM / 4 : 1;        // step 3: first MFMA slot that dequantises
   constexpr int XPM = (NU + NM - X0 - 1) / (NM - X0);
 
-  // loads run AHEAD stages ahead of the MFMAs
+  // Loads run AHEAD stages ahead of the MFMAs.  The first stages' weight loads go out before the
+  // tile's row indices (a dependent global load made by the caller, `ri`) are needed: the weights'
+  // trip to HBM then overlaps the index fetch instead of following it.
 #pragma unroll
   for (int t = 0; t < AHEAD; t++)
-    if (t < nstage) issue(t);
-  // stage 0 must have landed; the later ones may still be in flight
-  wait_loads_before(1);
+    if (t < nstage) issue_w(t);
+  float xms_v = 1.f;
+  if (tid < BM) {
+    rowidx[tid] = ri;
+    if (UP && xms) xms_v = xms[ri];  // for the epilogue; the wait for it comes after the K loop
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < A_LOADS; i++) {
+    const int m = 8 * a_grp[i] + (lane >> 3);
+    a_src[i] = x + (size_t)rowidx[m] * K + (((lane & 7) ^ ((m >> 1) & 7)) << 3);
+  }
+#pragma unroll
+  for (int t = 0; t < AHEAD; t++)
+    if (t < nstage) issue_a(t);
+  // stage 0 must have landed; only the activation loads of the later stages may still be in flight
+  wait_vm(nstage > 1 ? A_LOADS * (AHEAD - 1) : 0);
   __syncthreads();
   load_codes(0);
 #pragma unroll
@@ -418,6 +435,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // no LDS-bound load may outlive the block
+  if (UP) {
+    if (tid < BM) rowscale[tid] = xms ? moe_hid_scale(cmag, xms_v) : 1.f;
+    __syncthreads();
+  }
 
   // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair).
   // f16 results go through a per-wave LDS patch (the stage buffers are dead by now) so that global
@@ -436,7 +457,9 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
           for (int f = 0; f < NH; f++) {
             const float g = acc[mf][f][r], u = acc[mf][NH + f][r];
-            const float hv = g / (1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
+            // hardware reciprocal (1 ulp) instead of the IEEE division sequence: the result is rounded
+            // to f16 below, and this epilogue is VALU time during which the matrix pipe idles
+            const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
             // hid feeds the down GEMM: permuted order inside groups of 8 (q4cp) / blocks of 64 (Q4_K)
             int pos;
             if (!Q4K) {
@@ -494,8 +517,6 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
                 moe_hscale hs) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES);
-  int* rowidx = (int*)(cbs + 16);
-  float* rowscale = (float*)(rowidx + BM);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
   // Routed tiles and shared-expert tiles (all full) are dealt out separately, or the XCD that
@@ -536,18 +557,18 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
     cb_b = c0;
   }
 
+  int ri = 0;
   if (tid < BM) {
     const int m = tid < tile.count ? tid : 0;  // rows past the tile read a valid row, never stored
-    const int ri = tokidx ? tokidx[tile.first + m] : tile.first + m;
-    rowidx[tid] = ri;
-    if (UP) rowscale[tid] = hs.xms ? moe_hid_scale(shared ? hs.c_shared : hs.c_routed, hs.xms[ri]) : 1.f;
+    ri = tokidx ? tokidx[tile.first + m] : tile.first + m;  // used inside gemm_tile, after its first weight loads
   }
-  __syncthreads();
+  const float cmag = shared ? hs.c_shared : hs.c_routed;
+  __syncthreads();  // cbs
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b); \
-    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b);      \
+    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag); \
+    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag);      \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
