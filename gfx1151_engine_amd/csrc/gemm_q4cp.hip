@@ -363,7 +363,12 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     rowidx[tid] = ri;
     if (UP && xms) xms_v = xms[ri];  // for the epilogue; the wait for it comes after the K loop
   }
-  __syncthreads();
+  // barrier for the LDS row indices only: __syncthreads() would also wait for the weight loads
+  // just issued (its fence drains the vector memory counter), a full trip to HBM
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
 #pragma unroll
   for (int i = 0; i < A_LOADS; i++) {
     const int m = 8 * a_grp[i] + (lane >> 3);
@@ -541,6 +546,14 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int e = shared ? 0 : tile.expert;
   const int tid = threadIdx.x, lane = tid & 63;
 
+  // the tile's row indices: requested before the codebook is looked at, so that the two round trips
+  // overlap; used inside gemm_tile, after its first weight loads
+  int ri = 0;
+  if (tid < BM) {
+    const int m = tid < tile.count ? tid : 0;  // rows past the tile read a valid row, never stored
+    ri = tokidx ? tokidx[tile.first + m] : tile.first + m;
+  }
+
   // q4cp codebook: affine (a*n+b) or table.  Q4_K has no codebook (w = (d*sc)*n - dmin*m).
   bool affine = true;
   float cb_a = 1.f, cb_b = 0.f;
@@ -557,11 +570,6 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
     cb_b = c0;
   }
 
-  int ri = 0;
-  if (tid < BM) {
-    const int m = tid < tile.count ? tid : 0;  // rows past the tile read a valid row, never stored
-    ri = tokidx ? tokidx[tile.first + m] : tile.first + m;  // used inside gemm_tile, after its first weight loads
-  }
   const float cmag = shared ? hs.c_shared : hs.c_routed;
   __syncthreads();  // cbs
   const int mfn = (tile.count + 31) >> 5;
