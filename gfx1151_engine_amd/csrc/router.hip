@@ -478,6 +478,117 @@ void launch_seq(const void* W, bool bf, const float* bias, const void* wx, bool 
 #undef RS_GO
 }
 
+
+// ---- 25..32 tokens on the f64 matrix pipe: a block = 16 weight rows x all tokens, its eight waves
+// each take one eighth of the columns and the partial 16 x 16 tiles are added in wave order (fixed,
+// so the result does not depend on timing; same accuracy statement as k_router_small).
+// v_mfma_f64_16x16x4_f64: lane l supplies A[row l%16][k l/16] and B[k l/16][token l%16]; a 16-byte load
+// per lane (4 consecutive columns 4*(l/16)..+3 of its row / token) therefore feeds four MFMAs.
+// Every weight is read once, activations come from L2; loads run through a register ring of
+// RX_D 16-column steps.  Needs d % 128 == 0.  Blocks past the rows build the digit planes of x.
+constexpr int RX_D = 12;
+template <bool BF16, int NTT>  // NTT = token tiles of 16 (1 or 2)
+__global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__ W, const float* __restrict__ bias,
+                                                        const void* __restrict__ Wx, bool wx_bf16,
+                                                        const float* __restrict__ x, int P, int E, int d,
+                                                        float* __restrict__ logits, float* __restrict__ out_x,
+                                                        int nrows, uint32_t* __restrict__ planes,
+                                                        float2* __restrict__ meta, bool planes_natural) {
+  __shared__ double part[8][NTT][64][4];
+  const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nrt = (nrows + 15) >> 4;
+  if ((int)blockIdx.x >= nrt) {
+    const int G = d / 32, gb = (G + 511) / 512;
+    const int q = blockIdx.x - nrt, t = q / gb, g = (q % gb) * 512 + tid;
+    if (t < P && g < G) {
+      if (planes_natural) qvec_group_from_f32_t<true>(x, (uint64_t)d, G, t, g, planes, meta);
+      else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
+    }
+    return;
+  }
+  const int li = lane & 15, lg = lane >> 4;
+  const int row = blockIdx.x * 16 + li;
+  const bool rlive = row < nrows, extra = Wx != nullptr && row == E;
+  // per-lane weight row (rows past the end read row 0 and are never stored); all loads unconditional
+  const bool wbf = extra ? wx_bf16 : BF16;
+  const uint8_t* wrow = extra ? (const uint8_t*)Wx : (const uint8_t*)W + (rlive ? (uint64_t)row : 0) * d * (BF16 ? 2 : 4);
+  const float* xrow[NTT];
+  float xm[NTT];
+#pragma unroll
+  for (int tt = 0; tt < NTT; tt++) {
+    const int t = 16 * tt + li;
+    xrow[tt] = x + (size_t)(t < P ? t : 0) * d;
+    xm[tt] = t < P ? 1.f : 0.f;
+  }
+  const int kper = d / 8, k0 = wv * kper + 4 * lg;  // this lane's first column
+  const int nit = kper / 16;
+  uint4 wr[RX_D];
+  float4 xr[RX_D][NTT];
+  auto fetch = [&](int j, int it) {
+    const int c = k0 + 16 * (it < nit ? it : nit - 1);  // past the end: a repeat that is never used
+    // 16 bytes in either format (bf16: 8 bytes twice), so no branch surrounds the load
+    const uint8_t* p = wrow + (size_t)c * (wbf ? 2 : 4);
+    const uint2 lo = *(const uint2*)p, hi = *(const uint2*)(p + (wbf ? 0 : 8));
+    wr[j] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+#pragma unroll
+    for (int tt = 0; tt < NTT; tt++) xr[j][tt] = *(const float4*)(xrow[tt] + c);
+  };
+  double4v acc[NTT];
+#pragma unroll
+  for (int tt = 0; tt < NTT; tt++) acc[tt] = double4v{0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+  for (int j = 0; j < RX_D; j++) fetch(j, j);
+  for (int ib = 0; ib < nit; ib += RX_D) {
+#pragma unroll
+    for (int j = 0; j < RX_D; j++) {
+      if (ib + j < nit) {  // block-uniform
+        float w[4];
+        if (wbf) {
+          w[0] = __uint_as_float(wr[j].x << 16); w[1] = __uint_as_float(wr[j].x & 0xffff0000u);
+          w[2] = __uint_as_float(wr[j].y << 16); w[3] = __uint_as_float(wr[j].y & 0xffff0000u);
+        } else {
+          w[0] = __uint_as_float(wr[j].x); w[1] = __uint_as_float(wr[j].y);
+          w[2] = __uint_as_float(wr[j].z); w[3] = __uint_as_float(wr[j].w);
+        }
+        float4 xv[NTT];
+#pragma unroll
+        for (int tt = 0; tt < NTT; tt++) xv[tt] = xr[j][tt];
+        fetch(j, ib + j + RX_D);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const double a = (double)w[q];
+#pragma unroll
+          for (int tt = 0; tt < NTT; tt++) {
+            const float xq = q == 0 ? xv[tt].x : q == 1 ? xv[tt].y : q == 2 ? xv[tt].z : xv[tt].w;
+            acc[tt] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, (double)(xq * xm[tt]), acc[tt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < NTT; tt++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) part[wv][tt][lane][r] = acc[tt][r];
+  __syncthreads();
+  // D value r of lane l = [row 4r + l/16][token l%16]; one thread per (tile, lane, r) adds the eight partials
+  for (int i = tid; i < NTT * 256; i += 512) {
+    const int tt = i >> 8, l = (i >> 2) & 63, r = i & 3;
+    double sum = part[0][tt][l][r];
+#pragma unroll
+    for (int w = 1; w < 8; w++) sum += part[w][tt][l][r];
+    const int orow = blockIdx.x * 16 + 4 * r + (l >> 4), t = 16 * tt + (l & 15);
+    if (orow < nrows && t < P) {
+      float v = (float)sum;
+      if (orow == E) out_x[t] = v;
+      else {
+        if (bias) v += bias[orow];
+        logits[(size_t)t * E + orow] = v;
+      }
+    }
+  }
+}
+
 }  // namespace
 
 MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float* x, int P,
@@ -519,7 +630,11 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
                             hipStream_t st) {
   const int E = (int)W->rows, d = (int)W->cols;
-  if (P > 24) {
+  // 25..32 tokens with d a multiple of 128 (and one weight format): the f64 matrix pipe kernel.
+  // (Below that k_router_mid is as fast or faster: one block per 16 rows leaves most CUs idle, the
+  // matrix pipe of the busy ones is the limit: 38 us at 32 tokens against 2 x 38 for the split.)
+  const bool mfma_ok = P > 24 && d % 128 == 0 && (!Wx || (Wx->dtype == MOE_DT_BF16) == (W->dtype == MOE_DT_BF16));
+  if (P > 24 && !mfma_ok) {
     // more than 24 tokens per block cost the kernel its second wave per SIMD (accumulators):
     // two launches of at most 16 tokens read the router matrix twice (L2 / MALL) and are faster
     const int P0 = 16, G = d / 32;
@@ -552,6 +667,16 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
     if (E <= 512) { if (bf) RSM_GO(true, 4, 8); else RSM_GO(false, 4, 8); }
     else { if (bf) RSM_GO(true, 4, 16); else RSM_GO(false, 4, 16); }
   } else {
+    if (mfma_ok) {
+      // the f64 matrix pipe: 16 rows per block, columns split over its eight waves
+      const int qb = planes ? P * ((d / 32 + 511) / 512) : 0;
+      dim3 gx((nrows + 15) / 16 + qb);
+#define RX_GO(BF, NTT) k_router_mfma<BF, NTT><<<gx, 512, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural)
+      if (bf) RX_GO(true, 2); else RX_GO(false, 2);
+#undef RX_GO
+      MOE_LAUNCH_CHECK();
+      return MOE_OK;
+    }
 #define RMD_GO(BF, PM) k_router_mid<BF, PM><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural)
     if (P <= 8) { if (bf) RMD_GO(true, 8); else RMD_GO(false, 8); }
     else if (P <= 16) { if (bf) RMD_GO(true, 16); else RMD_GO(false, 16); }
