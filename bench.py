@@ -262,7 +262,7 @@ def measure_load(fmt, steps, nlayers):
             "steps": steps, "warmup": 1, "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "u8", "data": "synthetic",
             "config": {"workload": "load_" + fmt, "layers": nlayers, "file_bytes": nbytes, "device_bytes": int(wb),
-                       "format": ".hgn (HGN1)" if fmt == "q4cp" else "GGUF v3", "path": "page cache -> pageable H2D copy"},
+                       "format": ".hgn (HGN1)" if fmt == "q4cp" else "GGUF v3", "path": "page cache -> pinned staging (2 x 32 MiB, 6 threads) -> H2D"},
             "roofline": None, "cpu_baseline": None}
 
 

@@ -12,7 +12,9 @@
 #include <unistd.h>
 
 #include <cstring>
+#include <memory>
 #include <new>
+#include <thread>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -116,9 +118,13 @@ struct moe_file {
   std::unordered_map<std::string, int64_t> kv_int;  // GGUF integer metadata
 };
 
+namespace {
+struct Stager;
+}
 struct moe_weights {
   std::vector<void*> dev;
   uint64_t bytes = 0;
+  std::shared_ptr<Stager> stager;  // pinned staging buffers, kept for the duration of one moe_load_layers call
 };
 
 static int parse_hgn(moe_file* f) {
@@ -342,13 +348,74 @@ MOE_API int moe_file_config(const moe_file* f, int layer, moe_config* cfg) {
 
 namespace {
 
+// Host -> device through two pinned staging buffers: worker threads copy the next chunk out of the file
+// mapping (page cache) while the previous one is on its way over PCIe.  A plain hipMemcpy from the
+// pageable mapping measures 28 GB/s here; the staged path is used for tensors of at least 64 MiB.
+constexpr size_t STAGE_BYTES = (size_t)32 << 20;
+constexpr int STAGE_THREADS = 6;
+
+struct Stager {
+  void* pin[2] = {nullptr, nullptr};
+  hipEvent_t done[2] = {nullptr, nullptr};
+  hipStream_t stream = nullptr;
+  bool ok = false;
+  Stager() {
+    ok = hipHostMalloc(&pin[0], STAGE_BYTES, hipHostMallocDefault) == hipSuccess &&
+         hipHostMalloc(&pin[1], STAGE_BYTES, hipHostMallocDefault) == hipSuccess &&
+         hipEventCreateWithFlags(&done[0], hipEventDisableTiming) == hipSuccess &&
+         hipEventCreateWithFlags(&done[1], hipEventDisableTiming) == hipSuccess &&
+         hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) == hipSuccess;  // default priority
+  }
+  ~Stager() {
+    if (stream) (void)hipStreamSynchronize(stream);
+    for (int i = 0; i < 2; i++) {
+      if (done[i]) (void)hipEventDestroy(done[i]);
+      if (pin[i]) (void)hipHostFree(pin[i]);
+    }
+    if (stream) (void)hipStreamDestroy(stream);
+  }
+  static void fill(uint8_t* dst, const uint8_t* src, size_t n) {
+    const size_t per = (n / STAGE_THREADS + 4095) & ~(size_t)4095;
+    std::thread th[STAGE_THREADS];
+    int nt = 0;
+    for (size_t o = 0; o < n; o += per) {
+      const size_t m = n - o < per ? n - o : per;
+      th[nt++] = std::thread([=] { memcpy(dst + o, src + o, m); });
+    }
+    for (int i = 0; i < nt; i++) th[i].join();
+  }
+  int copy(void* dev, const uint8_t* src, size_t n) {
+    bool used[2] = {false, false};
+    int b = 0;
+    for (size_t o = 0; o < n; o += STAGE_BYTES, b ^= 1) {
+      const size_t m = n - o < STAGE_BYTES ? n - o : STAGE_BYTES;
+      if (used[b]) MOE_HIP(hipEventSynchronize(done[b]));  // the buffer's previous chunk has left
+      fill((uint8_t*)pin[b], src + o, m);
+      MOE_HIP(hipMemcpyAsync((uint8_t*)dev + o, pin[b], m, hipMemcpyHostToDevice, stream));
+      MOE_HIP(hipEventRecord(done[b], stream));
+      used[b] = true;
+    }
+    MOE_HIP(hipStreamSynchronize(stream));
+    return MOE_OK;
+  }
+};
+
 int upload(moe_weights* w, const FTensor& t, hipStream_t st, const uint8_t** dev) {
   void* p = nullptr;
   MOE_HIP(hipMalloc(&p, t.nbytes ? t.nbytes : 1));
   w->dev.push_back(p);
   w->bytes += t.nbytes;
-  // pageable source (the file mapping): staged by the runtime; set-up work, so a plain copy
-  (void)st;
+  (void)st;  // set-up work: the copy is complete when this returns
+  if (t.nbytes >= ((size_t)64 << 20)) {
+    if (!w->stager) w->stager.reset(new (std::nothrow) Stager());
+    if (w->stager && w->stager->ok) {
+      const int rc = w->stager->copy(p, t.data, t.nbytes);
+      if (rc != MOE_OK) return rc;
+      *dev = (const uint8_t*)p;
+      return MOE_OK;
+    }
+  }
+  // small tensors, or no pinned memory to be had: pageable source, staged by the runtime
   MOE_HIP(hipMemcpy(p, t.data, t.nbytes, hipMemcpyHostToDevice));
   *dev = (const uint8_t*)p;
   return MOE_OK;
@@ -487,6 +554,7 @@ MOE_API int moe_load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, in
       return rc;
     }
   }
+  w->stager.reset();  // the staging buffers are not needed once the layers are resident
   *out = w;
   return MOE_OK;
 }

@@ -221,3 +221,26 @@ def test_hgn_record_size_must_match_its_dims(tmp_path):
     m.close()
     f.close()
 
+
+@pytest.mark.gpu
+def test_large_tensor_takes_the_staged_copy_and_arrives_intact(tmp_path):
+    # tensors of 64 MiB and more go through the pinned double-buffered staging (several chunks, worker
+    # threads); the layer must still equal the directly registered one bit for bit
+    import torch
+    d, mid, e, k = 1024, 1024, 72, 4
+    rng = np.random.default_rng(31)
+    hl = HostLayer(rng, d, mid, e, k, fmt="q4cp", shared=False)
+    assert hl.gate_up.nbytes > (64 << 20) > hl.down.nbytes
+    p = tmp_path / "big.hgn"
+    files.write_hgn(p, files.hgn_layer_tensors(0, hl))
+    f = capi.ModelFile(p)
+    m = capi.Moe(d, mid, e, k, layers=1, max_tokens=8)
+    w = f.load_layers(m, 0, 0, 1)
+    f.close()
+    x = torch.from_numpy(np.random.default_rng(2).standard_normal((5, d), dtype=np.float32)).cuda()
+    direct, keep = hl.to_gpu(max_tokens=8)
+    assert torch.equal(direct.forward(0, x), m.forward(0, x))
+    torch.cuda.synchronize()
+    del m, direct, keep
+    w.free()
+
