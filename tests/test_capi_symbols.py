@@ -44,3 +44,44 @@ def test_null_and_shape_validation_without_gpu(lib):
     assert lib.moe_routing_create(0, 8, None) == -2
     assert lib.moe_tiles(None, None, None, 8, 64, None) == -2
     assert lib.moe_gg_gemv(2, 12, None, None, None, None, None, None, None, None, 1, 256, 256, 10, 16, None) == -1
+
+
+def _cc_example(out):
+    import subprocess
+    pkg = os.path.join(ROOT, "gfx1151_engine_amd")
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-O1", "-D__HIP_PLATFORM_AMD__", "-I/opt/rocm/include",
+           "-I" + os.path.join(ROOT, "include"), os.path.join(ROOT, "examples", "forward.c"), "-L" + pkg, "-lmi355moe",
+           "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath," + pkg, "-Wl,-rpath,/opt/rocm/lib", "-o", str(out)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    return out
+
+
+def test_header_is_c99_and_the_c_example_links(lib, tmp_path):
+    """The boundary is a C ABI: the header must compile as plain C (not only as C++) and a C program
+    must link against the library with nothing but the HIP runtime beside it."""
+    import subprocess
+    src = tmp_path / "hdr.c"
+    src.write_text('#include "mi355_moe.h"\nint main(void) { return moe_status_string(0) ? 0 : 1; }\n')
+    r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only",
+                        "-I" + os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    _cc_example(tmp_path / "forward")
+
+
+@pytest.mark.gpu
+def test_c_example_runs_a_token_through_a_file(tmp_path):
+    import subprocess
+    import numpy as np
+    from gfx1151_engine_amd import files
+    from tests.helpers import HostLayer
+    exe = _cc_example(tmp_path / "forward")
+    hl = HostLayer(np.random.default_rng(3), 256, 256, 8, 3, fmt="q4cp")
+    p = tmp_path / "m.hgn"
+    files.write_hgn(p, files.hgn_layer_tensors(0, hl))
+    r = subprocess.run([str(exe), str(p), "3"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "experts=8 topk=3 layers=1" in r.stdout and "y[0..3]" in r.stdout
+    vals = [float(v) for v in r.stdout.strip().splitlines()[-1].split("=")[1].split()]
+    assert all(np.isfinite(vals)) and any(v != 0 for v in vals)
+
