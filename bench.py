@@ -37,7 +37,7 @@ def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb):
     import numpy as np
     import torch
     from oracle import oracle as O
-    ol = layer.oracle_layer()
+    ol = O.layer_from_device(layer)
     y = torch.empty((T, D), dtype=torch.float32, device="cuda")
     if kind == "prefill":
         # tokens routed to the hottest expert first, then tokens in batch order, in chunks of 256

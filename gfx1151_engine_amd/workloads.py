@@ -1,6 +1,6 @@
 """Full-size synthetic MoE layers generated directly in HBM (torch is only the allocator / RNG).
 
-Byte layouts are the engine's: hgn q4cp blobs and GGUF Q4_K raw blocks.  The CPU oracle is fed the
+Byte layouts are the engine's: hgn q4cp blobs and GGUF Q4_K raw blocks.  The checker (tests, benchmark baseline) is fed the
 very same bytes, read back from the device, so both sides see identical weights.
 """
 import numpy as np
@@ -96,23 +96,6 @@ class DeviceLayer:
             wt, gt = 0, capi.GGML_Q4_K
         m.set_shared(layer, capi.wview(self.sh[0], wt, mid, d), capi.wview(self.sh[1], wt, mid, d),
                      capi.wview(self.sh[2], wt, d, mid), capi.wview(self.sh_sg, capi.F32, 1, d), gt)
-
-    def oracle_layer(self):
-        """The same bytes, copied to the host, as an oracle layer (test / cpu_baseline use only)."""
-        from oracle import oracle as O
-        d, mid, E, k = self.d, self.mid, self.E, self.k
-        wt = O.Q4CP if self.fmt == "q4cp" else O.Q4K
-        h = lambda t: t.cpu().numpy()
-        sh = [O.Mat(wt, h(self.sh[0]), mid, d), O.Mat(wt, h(self.sh[1]), mid, d), O.Mat(wt, h(self.sh[2]), d, mid),
-              O.Mat(O.F32, h(self.sh_sg), 1, d)]
-        router = O.Mat(O.F32, h(self.router), E, d)
-        bias = h(self.bias) if self.bias is not None else None
-        if self.fmt == "q4cp":
-            return O.Layer(d, mid, E, k, router, O.Mat(wt, h(self.down), E * d, mid),
-                           gate_up=O.Mat(wt, h(self.gate_up), E * 2 * mid, d), shared=sh, router_bias=bias)
-        return O.Layer(d, mid, E, k, router, O.Mat(wt, h(self.down), E * d, mid),
-                       gate=O.Mat(wt, h(self.gate), E * mid, d), up=O.Mat(wt, h(self.up), E * mid, d),
-                       shared=sh, router_bias=bias)
 
 
 def calibrate_zipf(router, x, k, s=1.1, target=12.0, seed=3):

@@ -311,3 +311,21 @@ def ref_gguf_kv_i(path, key, default=-1):
     f = ref().ref_gguf_kv_i
     f.restype = C.c_int64
     return f(str(path).encode(), key.encode(), C.c_int64(default))
+
+
+def layer_from_device(dl):
+    """An oracle Layer over the very bytes of a synthetic device layer (an object with the attributes of
+    gfx1151_engine_amd.workloads.DeviceLayer), copied to the host.  Checker side only."""
+    d, mid, E, k = dl.d, dl.mid, dl.E, dl.k
+    wt = Q4CP if dl.fmt == "q4cp" else Q4K
+    h = lambda t: t.cpu().numpy()
+    sh = [Mat(wt, h(dl.sh[0]), mid, d), Mat(wt, h(dl.sh[1]), mid, d), Mat(wt, h(dl.sh[2]), d, mid),
+          Mat(F32, h(dl.sh_sg), 1, d)]
+    router = Mat(F32, h(dl.router), E, d)
+    bias = h(dl.bias) if dl.bias is not None else None
+    if dl.fmt == "q4cp":
+        return Layer(d, mid, E, k, router, Mat(wt, h(dl.down), E * d, mid),
+                     gate_up=Mat(wt, h(dl.gate_up), E * 2 * mid, d), shared=sh, router_bias=bias)
+    return Layer(d, mid, E, k, router, Mat(wt, h(dl.down), E * d, mid),
+                 gate=Mat(wt, h(dl.gate), E * mid, d), up=Mat(wt, h(dl.up), E * mid, d),
+                 shared=sh, router_bias=bias)

@@ -85,3 +85,13 @@ def test_c_example_runs_a_token_through_a_file(tmp_path):
     vals = [float(v) for v in r.stdout.strip().splitlines()[-1].split("=")[1].split()]
     assert all(np.isfinite(vals)) and any(v != 0 for v in vals)
 
+
+
+def test_product_never_refers_to_the_checker():
+    """The CPU restatement is test infrastructure: nothing in the package may import, link or name it."""
+    import pathlib
+    import re
+    pkg = pathlib.Path(__file__).resolve().parents[1] / "gfx1151_engine_amd"
+    hits = [str(p) for p in pkg.rglob("*") if p.suffix in (".py", ".hip", ".h", ".cpp", ".c")
+            and re.search(r"\boracle\b", p.read_text(errors="replace"))]
+    assert not hits, hits

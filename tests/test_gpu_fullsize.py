@@ -41,7 +41,7 @@ def test_full_size_layer(oracle, fmt, T):
     sample = np.unique(np.concatenate([np.where((ids == hot).any(1))[0][:8], np.where((ids == rare).any(1))[0][:4],
                                        np.arange(12)]))
     xs = x[torch.from_numpy(sample).cuda()].contiguous()
-    yo, io, wo = oracle.moe_layer(L.oracle_layer(), xs.cpu().numpy())
+    yo, io, wo = oracle.moe_layer(oracle.layer_from_device(L), xs.cpu().numpy())
     assert (ids[sample] == io[:, :K]).all(), "router ids bit-exact with the CPU path"
     assert (ws[sample].view(np.uint32) == wo[:, :K].view(np.uint32)).all(), "router weights bit-exact (sequential order)"
     err = _max_abs_rel(y[sample], yo)
@@ -62,7 +62,7 @@ def test_full_size_decode_rotating_tokens(oracle):
     L = W.DeviceLayer(777, D, MID, E, K, "q4cp")
     m = capi.Moe(D, MID, E, K, layers=1, max_tokens=1)
     L.register(m, 0)
-    ol = L.oracle_layer()
+    ol = oracle.layer_from_device(L)
     g = torch.Generator(device="cuda")
     g.manual_seed(11)
     for i in range(6):
