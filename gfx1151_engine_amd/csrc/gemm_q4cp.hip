@@ -1,11 +1,13 @@
 // Prefill: grouped expert GEMM on q4cp weights with CDNA4 MFMA (v_mfma_f32_32x32x16_f16).
 //
-// One block (4 waves) = one tile of up to 128 (token, expert) pairs of ONE expert x 512 weight rows
-// (gate/up: 256 gate + the matching 256 up rows, SwiGLU on the accumulators).  Each wave owns
-// 128 pairs x 128 weight rows, so one activation fragment read from LDS feeds four MFMAs: LDS
-// bandwidth, not the matrix pipe, is what a narrower wave tile runs out of first.
+// One block (4 waves) = one tile of up to 128 (token, expert) pairs of ONE expert x 256 weight rows
+// (gate/up: 128 gate + the matching 128 up rows, SwiGLU on the accumulators).  Each wave owns
+// 128 pairs x 64 weight rows = 8 accumulators.  Two such blocks share a CU (2 x 77 KB of LDS, one
+// wave of each per SIMD): they pass their barriers, prologues and epilogues independently, so the
+// matrix pipe has the other block's MFMAs to run meanwhile (8-wave blocks of 512 rows, one per
+// CU, measured 4 % (q4cp) to 10 % (Q4_K) slower).
 // Activations (f16), raw 4-bit codes and fp16 scales go global -> LDS directly (no registers),
-// double-buffered, one barrier per 64-wide K stage.  Codes are dequantised in registers straight
+// three stage buffers, one barrier per 64-wide K stage.  Codes are dequantised in registers straight
 // into the MFMA B-operand layout: one 32-bit code word = 8 consecutive K of one weight row = one
 // lane's operand.  The unpack yields the K order [0,4,1,5,2,6,3,7] inside each group of 8, so
 // f16 activations are kept in that same "interleaved" order (a dot product does not care as long
@@ -33,21 +35,29 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #ifndef MOE_GEMM_NF
 #define MOE_GEMM_NF 2
 #endif
+#ifndef MOE_GEMM_WROWS
+#define MOE_GEMM_WROWS 256
+#endif
 constexpr int NF = MOE_GEMM_NF;          // weight fragments (32 rows) per wave
-constexpr int NW = 16 / NF;               // waves per block
+constexpr int WROWS = MOE_GEMM_WROWS;    // weight rows per block (up: WROWS/2 gate + the matching WROWS/2 up rows)
+constexpr int HALF = WROWS / 2;
+constexpr int NW = WROWS / 32 / NF;       // waves per block
 constexpr int NT = 64 * NW;               // each wave: 128 pairs x 32*NF weight rows
+constexpr int WPE = NT * (WROWS == 512 ? 1 : 2) / 256;  // waves per SIMD: 256-row blocks run two to a CU
 constexpr int BM = 128;        // pairs per tile (4 MFMA row fragments)
 constexpr int BK = 64;         // K per stage
-constexpr int WROWS = 512;     // weight rows per block (up: 256 gate + 256 up)
 constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chunk c of row m at slot c ^ ((m >> 1) & 7): conflict-free for the 128-bit fragment reads
-constexpr int W_BYTES = WROWS * 32;       // 16 KB  [row][32 B]
-constexpr int S_BYTES = WROWS * 16;       //  8 KB  [row][8 scales], refreshed every 4 stages
+constexpr int W_BYTES = WROWS * 32;       // [row][32 B]
+constexpr int S_BYTES = WROWS * 16;       // [row][8 scales], refreshed every 4 stages
+// scale buffers: two, or one whose four stages' worth a lane keeps in registers (two 256-row
+// blocks then fit the CU's 160 KB)
+constexpr int NSB = WROWS == 512 ? 2 : 1;
 #ifndef MOE_GEMM_NBUF
 #define MOE_GEMM_NBUF 3
 #endif
 constexpr int NBUF = MOE_GEMM_NBUF;       // activation / code buffers; loads run NBUF-1 stages ahead
 constexpr int AHEAD = NBUF - 1;
-constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES + 64 + BM * 4 + BM * 4;
+constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES + 64 + BM * 4 + BM * 4;
 
 struct LutDev {
   const uint8_t *w, *w_up, *sc, *sc_up;
@@ -120,7 +130,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
-  const float* cbs = (const float*)(S0 + 2 * S_BYTES);
+  const float* cbs = (const float*)(S0 + NSB * S_BYTES);
   int* rowidx = (int*)(cbs + 16);
   float* rowscale = (float*)(rowidx + BM);  // f16 range guard of each pair row (gate/up only)
   const int tid = threadIdx.x, lane = tid & 63;
@@ -132,14 +142,14 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     size_t grow;
     const uint8_t *cb0, *sb0;
     if (UP) {
-      const bool up = lr >= 256;
-      int r = nb * 256 + (lr & 255);
+      const bool up = lr >= HALF;
+      int r = nb * HALF + (lr & (HALF - 1));
       r = r < M ? r : M - 1;
       cb0 = up ? L.w_up : L.w;
       sb0 = up ? L.sc_up : L.sc;
       grow = (size_t)e * L.e_rows + (up ? L.up_off : 0) + r;
     } else {
-      int r = nb * 512 + lr;
+      int r = nb * WROWS + lr;
       r = r < M ? r : M - 1;
       cb0 = L.w;
       sb0 = L.sc;
@@ -160,7 +170,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // (same bytes to the same place) so that every wave issues the same number of loads.
   constexpr int A_GROUPS = 4 * MF;
   constexpr int A_LOADS = (A_GROUPS + NW - 1) / NW;
-  constexpr int W_LOADS = 16 / NW, S_LOADS = 8 / NW;
+  constexpr int W_LOADS = WROWS / 32 / NW, S_LOADS = (WROWS / 64 + NW - 1) / NW;
   const __half* a_src[A_LOADS];
   int a_grp[A_LOADS];
 #pragma unroll
@@ -195,7 +205,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
       const size_t off = Q4K ? (size_t)(s >> 2) * 144 : (size_t)g0 * 2;
-      g2l16(s_src[i] + off, S0 + ((s >> 2) & 1) * S_BYTES + (S_LOADS * wv + i) * 1024);
+      g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + (S_LOADS * wv + i) * 1024);
     }
   };
   auto issue_a = [&](int s) {
@@ -248,8 +258,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
   for (int nf = 0; nf < NF; nf++) {
     if (!UP) wrow[nf] = 32 * NF * wv + 32 * nf + n;
-    else if (Q4K && NH == 1) wrow[nf] = nf * 256 + 64 * (wv >> 1) + 16 * (wv & 1) + (n & 15) + 2 * (n & 16);
-    else wrow[nf] = (nf / NH) * 256 + 32 * NH * wv + 32 * (nf % NH) + n;
+    else if (Q4K && NH == 1) wrow[nf] = nf * HALF + 64 * (wv >> 1) + 16 * (wv & 1) + (n & 15) + 2 * (n & 16);
+    else wrow[nf] = (nf / NH) * HALF + 32 * NH * wv + 32 * (nf % NH) + n;
   }
 
   // Software pipeline with a hand-placed instruction order.  Inside a stage (four 16-wide K
@@ -272,9 +282,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     const int m = 32 * mf + n;
     dst[mf] = *(const half8*)(Ab + m * 128 + (((4 * h + q) ^ ((m >> 1) & 7)) << 4));
   };
+  uint32_t sc4[NSB == 1 ? NF : 1][4];  // single scale buffer: this lane's scales of four stages (f16 bits)
   auto load_codes = [&](int s) {  // raw codes + this lane's scale of stage s (buffers already selected)
     const uint8_t* Wb = W0 + (s % NBUF) * W_BYTES;
-    const uint8_t* Sb = S0 + ((s >> 2) & 1) * S_BYTES;
+    const uint8_t* Sb = S0 + ((s >> 2) & (NSB - 1)) * S_BYTES;
     int g0 = 2 * (s & ~3);
     g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
     const int sidx = 2 * s + h - g0;  // this lane's scale inside the staged 8
@@ -282,8 +293,30 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     for (int nf = 0; nf < NF; nf++) {
       cw[nf] = *(const uint4*)(Wb + wrow[nf] * 32 + h * 16);
       if (AFFINE) cw8[nf] = uint4{cw[nf].x >> 8, cw[nf].y >> 8, cw[nf].z >> 8, cw[nf].w >> 8};
-      if (Q4K) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
-      else scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
+      if (NSB == 1) {
+        // the buffer is rewritten while its stages are still being worked on: take all four
+        // stages' values when the first of them is prepared (every wave has by the next barrier;
+        // the loads that overwrite it are issued two barriers later)
+        if (Q4K) {
+          if ((s & 3) == 0) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
+        } else {
+          if ((s & 3) == 0) {
+            const uint4 w = *(const uint4*)(Sb + wrow[nf] * 16);
+            sc4[nf][0] = h ? w.x >> 16 : w.x & 0xffffu;
+            sc4[nf][1] = h ? w.y >> 16 : w.y & 0xffffu;
+            sc4[nf][2] = h ? w.z >> 16 : w.z & 0xffffu;
+            sc4[nf][3] = h ? w.w >> 16 : w.w & 0xffffu;
+          }
+          const int wi = (sidx - h) >> 1;  // wave-uniform
+          const uint32_t bits = wi == 0 ? sc4[nf][0] : wi == 1 ? sc4[nf][1] : wi == 2 ? sc4[nf][2] : sc4[nf][3];
+          union { uint16_t u; _Float16 f; } cv;
+          cv.u = (uint16_t)bits;
+          scf[nf] = (float)cv.f;
+        }
+      } else {
+        if (Q4K) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
+        else scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
+      }
     }
   };
   auto scale_consts = [&](int s) {
@@ -450,7 +483,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // stores are 16 bytes per lane and whole rows are contiguous.
   constexpr int NC = UP ? 32 * NH : 32 * NF;  // output columns of this wave
   constexpr int LDP = NC * 2 + 16;            // padded row pitch of the patch in bytes
-  const int colbase = UP ? nb * 256 + NC * wv : nb * 512 + NC * wv;
+  const int colbase = UP ? nb * HALF + NC * wv : nb * WROWS + NC * wv;
   if (UP || F16OUT) {
     uint8_t* patch = smem + wv * (32 * LDP);
 #pragma unroll
@@ -515,13 +548,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 }
 
 template <bool UP, bool F16OUT, bool Q4K>
-__global__ void __launch_bounds__(NT, NW / 4)
+__global__ void __launch_bounds__(NT, WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,
                 moe_hscale hs) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + 2 * S_BYTES);
+  float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
   // Routed tiles and shared-expert tiles (all full) are dealt out separately, or the XCD that
@@ -621,7 +654,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   if (q4k && up && m % 64) return MOE_E_UNSUPPORTED;  // hid is written in whole 64-element blocks
   if (!moe_aligned(x, 16) || !moe_aligned(out, 4)) return MOE_E_INVALID;
   if (max_tiles == 0) return MOE_OK;
-  const int nblk_n = up ? (m + 255) / 256 : (m + 511) / 512;
+  const int nblk_n = up ? (m + HALF - 1) / HALF : (m + WROWS - 1) / WROWS;
   // per XCD: ceil(routed/8) + ceil(shared/8) <= max_tiles/8 + 2 tile slots
   const int per_xcd = (max_tiles + 7) / 8 + 1;
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
