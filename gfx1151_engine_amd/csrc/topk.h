@@ -101,6 +101,63 @@ __device__ __forceinline__ void topk_select_lm(uint32_t (&key)[NPL], int lane, i
   }
 }
 
+// Lane-major keys again, each lane's keys sorted first (descending, equal keys keep their index
+// order: an odd-even transposition sort with strict compares never lets equal keys pass each other).
+// A round is then the wave-wide maximum of the lanes' heads and a pop in the winning lane — the
+// per-lane scan over NPL registers, a chain of dependent compares and selects, leaves the
+// rounds.  The keys' original register indices travel in 4-bit fields of one word.
+template <int NPL>
+__device__ __forceinline__ void topk_select_sorted(uint32_t (&key)[NPL], int lane, int k, int* ids_row,
+                                                   float* ws_row) {
+  static_assert(NPL <= 8, "4-bit index fields in one 32-bit word");
+  uint32_t jj[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; j++) jj[j] = (uint32_t)j;
+#pragma unroll
+  for (int pass = 0; pass < NPL; pass++) {
+#pragma unroll
+    for (int i = pass & 1; i + 1 < NPL; i += 2) {
+      const uint32_t ka = key[i], kb = key[i + 1], ia = jj[i], ib = jj[i + 1];  // values, not lvalues:
+      const bool sw = kb > ka;                                                   // see the note below
+      key[i] = umax(ka, kb); key[i + 1] = umin(ka, kb);
+      jj[i] = sw ? ib : ia; jj[i + 1] = sw ? ia : ib;
+    }
+  }
+  // (a conditional between two array elements, `c ? key[j + 1] : key[j]`, is compiled as a load
+  //  through a selected address, i.e. a computed index into the register array, which costs a
+  //  chain of selects per access: the operands are copied to plain values first)
+  uint32_t jw = 0;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) jw |= jj[j] << (4 * j);
+  double wsum = 0.0;
+  float mine = 0.f;
+  int myid = 0;
+  for (int r = 0; r < k; r++) {
+    const uint32_t wm = wave_umax(key[0]);
+    const int wl = __builtin_ctzll(__ballot(key[0] == wm));        // lowest lane whose head is the maximum
+    const int wj = __builtin_amdgcn_readlane((int)jw, wl) & 15;    // the head's register before the sort
+    const float bv = __uint_as_float(wm - 1u);
+    wsum += (double)bv;  // selection order, as the reference's loop over idx[0..k)
+    if (lane == r) {
+      mine = bv;
+      myid = NPL * wl + wj;
+    }
+    const bool me = lane == wl;
+#pragma unroll
+    for (int j = 0; j + 1 < NPL; j++) {
+      const uint32_t cur = key[j], nxt = key[j + 1];
+      key[j] = me ? nxt : cur;
+    }
+    const uint32_t last = key[NPL - 1], jsh = jw >> 4;
+    key[NPL - 1] = me ? 0u : last;
+    jw = me ? jsh : jw;
+  }
+  if (lane < k) {
+    ids_row[lane] = myid;
+    ws_row[lane] = (float)((double)mine / wsum);
+  }
+}
+
 // The softmax / top-k of one token by one block of NT threads (E <= 64*NPL): the fp64 exps, the
 // costly part, are spread over the block; wave 0 then runs the k selection rounds on the keys in
 // LDS.  COH: the logits were written by other blocks of the same launch: read them with
@@ -170,5 +227,10 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
   uint32_t key[NPL];
 #pragma unroll
   for (int j = 0; j < NPL; j++) key[j] = keys[NPL * lane + j];
+#ifdef MOE_TOPK_SCAN
   topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
+#else
+  if constexpr (NPL <= 8) topk_select_sorted<NPL>(key, lane, k, ids_row, ws_row);
+  else topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
+#endif
 }
