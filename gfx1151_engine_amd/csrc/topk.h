@@ -23,6 +23,44 @@ __device__ __forceinline__ uint32_t wave_umin(uint32_t m) {
               umin((uint32_t)__builtin_amdgcn_readlane((int)m, 32), (uint32_t)__builtin_amdgcn_readlane((int)m, 48)));
 }
 
+// Wave-wide maximum / fp64 sum through DPP row operations and four lane reads: a butterfly of
+// __shfl_xor steps goes through the LDS crossbar six times, each a dependent round trip.
+__device__ __forceinline__ float wave_fmax_dpp(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false)));
+  const int b = __float_as_int(v);
+  return fmaxf(fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 0)), __int_as_float(__builtin_amdgcn_readlane(b, 16))),
+               fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 32)), __int_as_float(__builtin_amdgcn_readlane(b, 48))));
+}
+__device__ __forceinline__ double dpp_f64(double v, int ctrl_sel) {
+  union { double d; int i[2]; } a, r;
+  a.d = v;
+  switch (ctrl_sel) {
+    case 0: r.i[0] = __builtin_amdgcn_update_dpp(0, a.i[0], 0xB1, 0xf, 0xf, false); r.i[1] = __builtin_amdgcn_update_dpp(0, a.i[1], 0xB1, 0xf, 0xf, false); break;
+    case 1: r.i[0] = __builtin_amdgcn_update_dpp(0, a.i[0], 0x4E, 0xf, 0xf, false); r.i[1] = __builtin_amdgcn_update_dpp(0, a.i[1], 0x4E, 0xf, 0xf, false); break;
+    case 2: r.i[0] = __builtin_amdgcn_update_dpp(0, a.i[0], 0x141, 0xf, 0xf, false); r.i[1] = __builtin_amdgcn_update_dpp(0, a.i[1], 0x141, 0xf, 0xf, false); break;
+    default: r.i[0] = __builtin_amdgcn_update_dpp(0, a.i[0], 0x140, 0xf, 0xf, false); r.i[1] = __builtin_amdgcn_update_dpp(0, a.i[1], 0x140, 0xf, 0xf, false); break;
+  }
+  return r.d;
+}
+__device__ __forceinline__ double readlane_f64(double v, int l) {
+  union { double d; int i[2]; } a, r;
+  a.d = v;
+  r.i[0] = __builtin_amdgcn_readlane(a.i[0], l);
+  r.i[1] = __builtin_amdgcn_readlane(a.i[1], l);
+  return r.d;
+}
+// (the order of the additions differs from a plain loop: callers use it where every partial sum is exact)
+__device__ __forceinline__ double wave_dsum_dpp(double v) {
+  v += dpp_f64(v, 0);
+  v += dpp_f64(v, 1);
+  v += dpp_f64(v, 2);
+  v += dpp_f64(v, 3);
+  return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
+}
+
 // k rounds of arg-max by one wave over keys held NPL per lane (key[j] of lane l = expert l + 64 j;
 // key = probability bits + 1, probabilities are >= 0 so the bit patterns order like unsigned
 // integers; 0 = not a candidate).  Larger probability first, equal probabilities -> lower index.
@@ -170,6 +208,7 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
   __shared__ uint32_t keys[64 * NPL];
   __shared__ double red[NW];
   __shared__ float redf[NW];
+  __shared__ int redx[NW];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   __syncthreads();  // LDS of a previous token is no longer read
   float v[NPT];
@@ -181,12 +220,29 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
     if (e < E) v[j] = COH ? __hip_atomic_load(&lg[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
     mxf = fmaxf(mxf, v[j]);
   }
-  mxf = wave_max(mxf);
-  if (lane == 0) redf[wv] = mxf;
-  __syncthreads();
-  float mxa = redf[0];
+  // The maximum: every wave reads the whole row itself (NPL values per lane, 16-byte loads; rows
+  // past the end re-read the last four values) and needs no exchange with the other waves.
+  // Otherwise (unaligned rows, logits written by this launch) it goes through LDS and a barrier.
+  const bool wide = !COH && NPL % 4 == 0 && E % 4 == 0 && E >= 4 && ((uintptr_t)lg & 15) == 0;
+  float mxa;
+  if (wide) {
+    float m = -INFINITY;
 #pragma unroll
-  for (int w = 1; w < NW; w++) mxa = fmaxf(mxa, redf[w]);
+    for (int q = 0; q < NPL / 4; q++) {
+      int idx = NPL * lane + 4 * q;
+      idx = idx < E ? idx : E - 4;
+      const float4 f = *(const float4*)(lg + idx);
+      m = fmaxf(fmaxf(m, fmaxf(f.x, f.y)), fmaxf(f.z, f.w));
+    }
+    mxa = wave_fmax_dpp(m);
+  } else {
+    mxf = wave_fmax_dpp(mxf);
+    if (lane == 0) redf[wv] = mxf;
+    __syncthreads();
+    mxa = redf[0];
+#pragma unroll
+    for (int w = 1; w < NW; w++) mxa = fmaxf(mxa, redf[w]);
+  }
   const double mx = (double)mxa;
   float p[NPT];
   bool exact = true;
@@ -199,16 +255,24 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
     sloc += (double)p[j];
     if (e < 64 * NPL) pb[e] = p[j];
   }
-  const bool all_exact = __syncthreads_and(exact);
+  // wave sums and "every term exact" flags cross the block together, behind one barrier
+  sloc = wave_dsum_dpp(sloc);
+  const int wex = __all(exact);
+  if (lane == 0) {
+    red[wv] = sloc;
+    redx[wv] = wex;
+  }
+  __syncthreads();
+  bool all_exact = true;
+#pragma unroll
+  for (int w = 0; w < NW; w++) all_exact = all_exact && redx[w] != 0;
   double se;
   if (all_exact) {  // every partial sum is representable: any order gives the reference's fp64 sum
-    sloc = wave_sum(sloc);
-    if (lane == 0) red[wv] = sloc;
-    __syncthreads();
     se = red[0];
 #pragma unroll
     for (int w = 1; w < NW; w++) se += red[w];
   } else {          // very wide logit range: replay the reference's index order on one thread
+    __syncthreads();  // red[] has been read
     if (tid == 0) {
       double t = 0.0;
       for (int e = 0; e < E; e++) t += (double)pb[e];
