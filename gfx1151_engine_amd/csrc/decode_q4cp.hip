@@ -28,19 +28,21 @@ __device__ __forceinline__ float sum32(float v) {
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));   // xor 2
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));  // mirror in 8
   v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));  // mirror in 16
-  v += __shfl_xor(v, 16, 64);
-  return v;
+  return rows_half_add(v);
 }
 __device__ __forceinline__ float sum64(float v) {
-  v = sum32(v);
-  return v + __shfl_xor(v, 32, 64);
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, true));
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, true));
+  return rows_total_add(v);
 }
 
 // Quantise 32 floats held one per lane by lanes [0,32) of a half-wave (j = lane & 31) into the qvec4
 // form: returns this lane's four digits, q and q*sum(X).
 __device__ __forceinline__ void quant32_lane(float x, int& p0, int& p1, int& p2, int& p3, float& q, float& qsx) {
   float m = dpp_max_row(fabsf(x));
-  m = fmaxf(m, __shfl_xor(m, 16, 64));
+  m = rows_half_max(m);
   const float inv = m > 0.f ? QV4_XMAX / m : 0.f;
   q = m * (1.f / QV4_XMAX);
   const int X = (int)rintf(x * inv);

@@ -2,7 +2,7 @@
 // the q4cp decode kernels.  Unit of work = one 32-byte run of code bytes = 64 weights = two
 // 32-element sub-blocks (low nibbles / high nibbles), each with its own 6-bit scale and min:
 //   sum_k w_k x_k = d * (sc0 * qA * VA + sc1 * qB * VB) - dmin * (m0 * qA * SA + m1 * qB * SB)
-// with V = integer dot product of the codes with the activation group's three 7-bit digit planes
+// with V = integer dot product of the codes with the activation group's two 8-bit digit planes
 // (natural element order) and q * S = the group's quantised sum.  A lane owns one unit of a row;
 // rows of 3072 are 48 units (lanes 48..63 idle: the kernels are bandwidth-bound), rows of 768 are
 // 12 units (four slots per wave).
@@ -29,21 +29,19 @@ __device__ __forceinline__ float dpp_max_row(float v) {
   return v;
 }
 __device__ __forceinline__ float sum64(float v) {
-  v = dpp_add_row(v);
-  v += __shfl_xor(v, 16, 64);
-  return v + __shfl_xor(v, 32, 64);
+  return rows_total_add(dpp_add_row(v));
 }
 
 // activation planes of one unit: two groups (A = low nibbles, B = high nibbles)
 struct XU {
-  uint32_t a[3][8], b[3][8];
+  uint32_t a[2][8], b[2][8];
   float qa, qsa, qb, qsb;
 };
 __device__ __forceinline__ void load_xu(XU& x, const uint32_t* planes, const float2* meta, size_t g0) {
   const uint4* s = (const uint4*)(planes + g0 * QV_GROUP_DW);
 #pragma unroll
-  for (int p = 0; p < 3; p++) {
-    const uint4 a0 = s[2 * p], a1 = s[2 * p + 1], b0 = s[6 + 2 * p], b1 = s[6 + 2 * p + 1];
+  for (int p = 0; p < 2; p++) {
+    const uint4 a0 = s[2 * p], a1 = s[2 * p + 1], b0 = s[4 + 2 * p], b1 = s[4 + 2 * p + 1];
     x.a[p][0] = a0.x; x.a[p][1] = a0.y; x.a[p][2] = a0.z; x.a[p][3] = a0.w;
     x.a[p][4] = a1.x; x.a[p][5] = a1.y; x.a[p][6] = a1.z; x.a[p][7] = a1.w;
     x.b[p][0] = b0.x; x.b[p][1] = b0.y; x.b[p][2] = b0.z; x.b[p][3] = b0.w;
@@ -76,19 +74,18 @@ __device__ __forceinline__ void k4_pair(const uint4 hd, int jj, float& a0, float
 // one unit of one row: c0, c1 = its 32 code bytes, hd = the super-block header
 __device__ __forceinline__ float unit_dot(const uint4 c0, const uint4 c1, const uint4 hd, int jj, const XU& x) {
   const uint32_t w[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
-  int a0 = 0, a1 = 0, a2 = 0, b0 = 0, b1 = 0, b2 = 0;
+  int a0 = 0, a1 = 0, b0 = 0, b1 = 0;
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     const int lo = (int)(w[i] & 0x0f0f0f0fu), hi = (int)((w[i] >> 4) & 0x0f0f0f0fu);
     a0 = __builtin_amdgcn_sdot4(lo, (int)x.a[0][i], a0, false);
     a1 = __builtin_amdgcn_sdot4(lo, (int)x.a[1][i], a1, false);
-    a2 = __builtin_amdgcn_sdot4(lo, (int)x.a[2][i], a2, false);
     b0 = __builtin_amdgcn_sdot4(hi, (int)x.b[0][i], b0, false);
     b1 = __builtin_amdgcn_sdot4(hi, (int)x.b[1][i], b1, false);
-    b2 = __builtin_amdgcn_sdot4(hi, (int)x.b[2][i], b2, false);
   }
-  const float va = fmaf((float)a0, 16384.f, (float)(a1 * 128 + a2));
-  const float vb = fmaf((float)b0, 16384.f, (float)(b1 * 128 + b2));
+  // |a0| <= 32 * 15 * 128: the integer sum stays below 2^24 and converts exactly
+  const float va = (float)(a0 * 256 + a1);
+  const float vb = (float)(b0 * 256 + b1);
   float sa, ma, sb, mb;
   k4_pair(hd, jj, sa, ma, sb, mb);
   return (sa * x.qa * va + sb * x.qb * vb) - (ma * x.qsa + mb * x.qsb);
@@ -177,16 +174,14 @@ __global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t*
     const float g = gs[j], u = us[j];
     const float hv = g / (1.f + expf(-g)) * u;
     float m = dpp_max_row(fabsf(hv));
-    m = fmaxf(m, __shfl_xor(m, 16, 64));
-    const float inv = m > 0.f ? 1048576.f / m : 0.f;
-    const float q = m * (1.f / 1048576.f);
+    m = rows_half_max(m);
+    const float inv = m > 0.f ? QV_XMAX / m : 0.f;
+    const float q = m * (1.f / QV_XMAX);
     const int X = (int)rintf(hv * inv);
-    const int p2 = ((X + 64) & 127) - 64;
-    const int X1 = (X - p2) >> 7;
-    const int p1 = ((X1 + 64) & 127) - 64;
-    const int p0 = (X1 - p1) >> 7;
+    int p0, p1;
+    qv_digits(X, p0, p1);
     float sx = dpp_add_row((float)X);
-    sx += __shfl_xor(sx, 16, 64);
+    sx = rows_half_add(sx);
     if (lane < QV_GROUP_DW) pk[lane] = 0;
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     __builtin_amdgcn_wave_barrier();
@@ -194,7 +189,6 @@ __global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t*
       const int dw = j >> 2, sh = 8 * (j & 3);  // natural order
       atomicOr(&pk[dw], (uint32_t)(p0 & 0xff) << sh);
       atomicOr(&pk[8 + dw], (uint32_t)(p1 & 0xff) << sh);
-      atomicOr(&pk[16 + dw], (uint32_t)(p2 & 0xff) << sh);
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);
     __builtin_amdgcn_wave_barrier();

@@ -9,30 +9,51 @@
 //   meta: float2 (q, q * sum of the quantised elements).
 //
 // qvec (GGUF Q4_K weights, v_dot4_i32_i8):
-//   planes: 3 x 8 dwords of signed 7-bit digits, x ~= q * (2^14 p0 + 2^7 p1 + p2);
-//           q4cp order: dword 2i holds elements 8i+{0,2,4,6}, dword 2i+1 elements 8i+{1,3,5,7}
-//           (the order in which `w & 0x0f0f0f0f` / `(w>>4) & 0x0f0f0f0f` deliver the 4-bit codes of
-//           a q4cp row); natural order (Q4_K, where the low nibbles of 32 consecutive bytes are one
-//           32-element sub-block and the high nibbles the next): dword i holds elements 4i..4i+3
+//   planes: 2 x 8 dwords of signed 8-bit digits, x ~= q * (256 p0 + p1), |X| <= 32639 (15.99 bits
+//           relative to the group maximum, the same resolution as qvec4); natural order: dword i
+//           holds elements 4i..4i+3 (in Q4_K the low nibbles of 32 consecutive bytes are one
+//           32-element sub-block and the high nibbles the next, so `w & 0x0f0f0f0f` and
+//           `(w >> 4) & 0x0f0f0f0f` deliver four consecutive codes of one sub-block each)
 //   meta:   float2 (q, q * sum of the quantised elements)
 #pragma once
 #include "common.h"
 
-constexpr int QV_GROUP_DW = 24;
+constexpr int QV_GROUP_DW = 16;
 constexpr int QV4_GROUP_DW = 16;
+constexpr float QV_XMAX = 32639.f;   // 0x7f7f: both balanced digits at +127
 constexpr float QV4_XMAX = 30583.f;  // 0x7777: every balanced digit at +7
 
-// digit plane position of element j (0..31) of a group
-__device__ __forceinline__ void qvec_pos(int j, bool natural, int& dw, int& sh) {
-  dw = natural ? j >> 2 : 2 * (j >> 3) + (j & 1);
-  sh = natural ? 8 * (j & 3) : 8 * ((j & 7) >> 1);
+// Cross-row steps of the wave reductions of the decode kernels.  v holds its row's (16 lanes) result
+// in every lane; lane reads + scalar operands instead of shuffles through the LDS crossbar.  The
+// additions pair the rows as the xor-16 / xor-32 butterfly does: (r0 + r1) + (r2 + r3).
+__device__ __forceinline__ float rows_total_add(float v) {
+  const int b = __float_as_int(v);
+  return (__int_as_float(__builtin_amdgcn_readlane(b, 0)) + __int_as_float(__builtin_amdgcn_readlane(b, 16))) +
+         (__int_as_float(__builtin_amdgcn_readlane(b, 32)) + __int_as_float(__builtin_amdgcn_readlane(b, 48)));
+}
+__device__ __forceinline__ float rows_half_add(float v) {  // lanes < 32: r0 + r1, the others: r2 + r3
+  const int b = __float_as_int(v);
+  const float lo = __int_as_float(__builtin_amdgcn_readlane(b, 0)) + __int_as_float(__builtin_amdgcn_readlane(b, 16));
+  const float hi = __int_as_float(__builtin_amdgcn_readlane(b, 32)) + __int_as_float(__builtin_amdgcn_readlane(b, 48));
+  return (threadIdx.x & 32) ? hi : lo;
+}
+__device__ __forceinline__ float rows_half_max(float v) {
+  const int b = __float_as_int(v);
+  const float lo = fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 0)), __int_as_float(__builtin_amdgcn_readlane(b, 16)));
+  const float hi = fmaxf(__int_as_float(__builtin_amdgcn_readlane(b, 32)), __int_as_float(__builtin_amdgcn_readlane(b, 48)));
+  return (threadIdx.x & 32) ? hi : lo;
 }
 
-// One thread quantises group g of token t.
-template <bool NATURAL>
-__device__ __forceinline__ void qvec_group_from_f32_t(const float* __restrict__ x, uint64_t x_stride, int G, int t,
-                                                      int g, uint32_t* __restrict__ planes,
-                                                      float2* __restrict__ meta) {
+// balanced base-256 digits of X (|X| <= 32639): X = 256 p0 + p1
+__device__ __forceinline__ void qv_digits(int X, int& p0, int& p1) {
+  p1 = ((X + 128) & 255) - 128;
+  p0 = (X - p1) >> 8;
+}
+
+// One thread quantises group g of token t into the qvec form.
+__device__ __forceinline__ void qvec_group_from_f32(const float* __restrict__ x, uint64_t x_stride, int G, int t,
+                                                    int g, uint32_t* __restrict__ planes,
+                                                    float2* __restrict__ meta) {
   const float4* xp = (const float4*)(x + (size_t)t * x_stride + (size_t)g * 32);
   float v[32];
   float m = 0.f;
@@ -42,11 +63,11 @@ __device__ __forceinline__ void qvec_group_from_f32_t(const float* __restrict__ 
     v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
     m = fmaxf(m, fmaxf(fmaxf(fabsf(f.x), fabsf(f.y)), fmaxf(fabsf(f.z), fabsf(f.w))));
   }
-  const float inv = m > 0.f ? 1048576.f / m : 0.f;
-  const float q = m * (1.f / 1048576.f);
-  uint32_t pl[3][8];
+  const float inv = m > 0.f ? QV_XMAX / m : 0.f;
+  const float q = m * (1.f / QV_XMAX);
+  uint32_t pl[2][8];
 #pragma unroll
-  for (int p = 0; p < 3; p++)
+  for (int p = 0; p < 2; p++)
 #pragma unroll
     for (int i = 0; i < 8; i++) pl[p][i] = 0;
   int sx = 0;
@@ -54,28 +75,19 @@ __device__ __forceinline__ void qvec_group_from_f32_t(const float* __restrict__ 
   for (int j = 0; j < 32; j++) {
     const int X = (int)rintf(v[j] * inv);
     sx += X;
-    const int p2 = ((X + 64) & 127) - 64;
-    const int X1 = (X - p2) >> 7;
-    const int p1 = ((X1 + 64) & 127) - 64;
-    const int p0 = (X1 - p1) >> 7;
-    const int dw = NATURAL ? j >> 2 : 2 * (j >> 3) + (j & 1), sh = NATURAL ? 8 * (j & 3) : 8 * ((j & 7) >> 1);
+    int p0, p1;
+    qv_digits(X, p0, p1);
+    const int dw = j >> 2, sh = 8 * (j & 3);
     pl[0][dw] |= (uint32_t)(p0 & 0xff) << sh;
     pl[1][dw] |= (uint32_t)(p1 & 0xff) << sh;
-    pl[2][dw] |= (uint32_t)(p2 & 0xff) << sh;
   }
   uint4* dst = (uint4*)(planes + ((size_t)t * G + g) * QV_GROUP_DW);
 #pragma unroll
-  for (int p = 0; p < 3; p++) {
+  for (int p = 0; p < 2; p++) {
     dst[2 * p] = make_uint4(pl[p][0], pl[p][1], pl[p][2], pl[p][3]);
     dst[2 * p + 1] = make_uint4(pl[p][4], pl[p][5], pl[p][6], pl[p][7]);
   }
   meta[(size_t)t * G + g] = make_float2(q, q * (float)sx);
-}
-__device__ __forceinline__ void qvec_group_from_f32(const float* __restrict__ x, uint64_t x_stride, int G, int t,
-                                                    int g, uint32_t* __restrict__ planes,
-                                                    float2* __restrict__ meta, bool natural = false) {
-  if (natural) qvec_group_from_f32_t<true>(x, x_stride, G, t, g, planes, meta);
-  else qvec_group_from_f32_t<false>(x, x_stride, G, t, g, planes, meta);
 }
 
 // balanced base-16 digits of X (|X| <= 30583), least significant first

@@ -218,7 +218,7 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
     const int G = d / 32, gb = (G + (int)blockDim.x - 1) / (int)blockDim.x;
     const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * blockDim.x + threadIdx.x;
     if (t < P && g < G) {
-      if (planes_natural) qvec_group_from_f32_t<true>(x, (uint64_t)d, G, t, g, planes, meta);  // Q4_K kernels
+      if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);  // Q4_K kernels
       else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);                       // q4cp kernels
     }
     return;
@@ -310,7 +310,7 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
     const int G = d / 32, gb = (G + 255) / 256;
     const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * 256 + tid;
     if (t < P && g < G) {
-      if (planes_natural) qvec_group_from_f32_t<true>(x, (uint64_t)d, G, t, g, planes, meta);
+      if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
       else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
     }
     return;
@@ -501,7 +501,7 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
     const int G = d / 32, gb = (G + 511) / 512;
     const int q = blockIdx.x - nrt, t = q / gb, g = (q % gb) * 512 + tid;
     if (t < P && g < G) {
-      if (planes_natural) qvec_group_from_f32_t<true>(x, (uint64_t)d, G, t, g, planes, meta);
+      if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
       else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
     }
     return;

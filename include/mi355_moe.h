@@ -197,7 +197,7 @@ int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_st
 /* Switches in the spirit of the reference's QWENOX_* opt-outs (src/gpu/parts/40_model.inc:1959-1996):
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
  * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as
- * three 7-bit digit planes per 32-group, 21 significant bits) instead of the f32 FMA kernels. */
+ * digit planes per 32-group, 16 significant bits relative to the group maximum) instead of the f32 FMA kernels. */
 /* MOE_OPT_UNIQUE_MIN_TOKENS (default 0 = off): q4cp batches of at least this many tokens (and at most 32) walk
  * the expert-sorted pair lists, so that an expert shared by several tokens is read once
  * (the reference's _uq decode kernels, src/gpu/parts/26_kernels_moe_gguf.inc:758-877).  Pays when most

@@ -1,6 +1,8 @@
 """GPU parity of the whole layer through moe_forward against the oracle (the restated
 src/ref.cpp Model::moe): router ids bit-exact, y within max-abs-rel 2e-3 (the small-batch f32
-path is held to 1e-4)."""
+kernels are held to 1e-4, the integer-dot kernels to 2e-4 (q4cp) and 5e-4 (Q4_K))."""
+import zlib
+
 import numpy as np
 import pytest
 
@@ -9,7 +11,16 @@ from helpers import HostLayer, bits, max_abs_rel
 pytestmark = pytest.mark.gpu
 
 TOL_LAYER = 2e-3   # stated tolerance for the layer (f16/bf16 MFMA path)
-TOL_GEMV = 1e-4    # f32 in-place GEMV path
+TOL_GEMV = 1e-4    # small-batch GEMV path, f32 kernels
+TOL_INT_Q4CP = 2e-4  # integer-dot kernels, q4cp: activations as four 4-bit digit planes per 32-group (worst of
+                     # 60 seeds at one token: 7.8e-5)
+TOL_INT_Q4K = 5e-4  # integer-dot kernels on raw Q4_K blocks: activations as two 8-bit digit planes per
+                    # 32-group; the unsigned codes (w = d*sc*n - dmin*m, n in 0..15) double the weight of
+                    # the activations' rounding against the zero-centred q4cp codes (worst of 80 seeds: 2.4e-4)
+
+
+def tol_small(fmt):
+    return TOL_INT_Q4K if fmt == "q4k" else TOL_INT_Q4CP
 
 
 def gpu(a):
@@ -31,7 +42,7 @@ def run_layer(hl, x, max_tokens=None):
     ("q4cp", 640, 160, 16, 4, 7, "random"), ("q4k", 3072, 768, 24, 10, 1, None),
     ("q4k", 3072, 768, 24, 10, 20, None), ("q4k", 256, 256, 8, 3, 5, None)])
 def test_small_batch_layer(oracle, fmt, d, mid, E, k, T, cb):
-    rng = np.random.default_rng(hash((fmt, d, T)) % 2**31)
+    rng = np.random.default_rng(zlib.crc32(f"{fmt}-{d}-{T}".encode()))  # (hash() of a str changes per process)
     codebook = rng.uniform(-2, 2, 16).astype(np.float32) if cb == "random" else None
     hl = HostLayer(rng, d, mid, E, k, fmt=fmt, codebook=codebook)
     x = rng.standard_normal((T, d), dtype=np.float32)
@@ -39,7 +50,7 @@ def test_small_batch_layer(oracle, fmt, d, mid, E, k, T, cb):
     y, ids, ws = run_layer(hl, x)
     assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
     assert np.abs(ws[:, :k] - wo[:, :k]).max() <= 1e-6
-    assert max_abs_rel(y, yo) <= TOL_GEMV
+    assert max_abs_rel(y, yo) <= tol_small(fmt), max_abs_rel(y, yo)
 
 
 @pytest.mark.parametrize("fmt,T,rdt", [("q4cp", 3, "f32"), ("q4cp", 32, "f32"), ("q4k", 27, "f32"), ("q4k", 2, "f32"),
@@ -56,7 +67,7 @@ def test_small_batch_sizes_and_router_dtypes(oracle, fmt, T, rdt):
     y, ids, ws = run_layer(hl, x)
     assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
     assert np.abs(ws[:, :k] - wo[:, :k]).max() <= 1e-6
-    assert max_abs_rel(y, yo) <= TOL_GEMV
+    assert max_abs_rel(y, yo) <= tol_small(fmt), max_abs_rel(y, yo)
 
 
 @pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 9), ("q4k", 1), ("q4k", 9)])
@@ -76,7 +87,7 @@ def test_int_decode_switch(oracle, fmt, T):
         y = m.forward(0, gpu(x)).cpu().numpy()
         ids, _ = m.last_routing(T)
         assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
-        assert max_abs_rel(y, yo) <= TOL_GEMV, (opt, max_abs_rel(y, yo))
+        assert max_abs_rel(y, yo) <= (tol_small(fmt) if opt else TOL_GEMV), (opt, max_abs_rel(y, yo))
         ys.append(y)
     assert not (ys[0] == ys[1]).all(), "the two paths are different kernels (digit planes vs f32)"
     m.close()
@@ -101,10 +112,10 @@ def test_unique_expert_path(oracle, share):
     y = m.forward(0, gpu(x)).cpu().numpy()
     ids, _ = m.last_routing(T)
     assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
-    assert max_abs_rel(y, yo) <= TOL_GEMV, max_abs_rel(y, yo)
+    assert max_abs_rel(y, yo) <= TOL_INT_Q4CP, max_abs_rel(y, yo)
     m.set_option(capi.OPT_UNIQUE_MIN_TOKENS, 0)
     y2 = m.forward(0, gpu(x)).cpu().numpy()
-    assert max_abs_rel(y2, yo) <= TOL_GEMV
+    assert max_abs_rel(y2, yo) <= TOL_INT_Q4CP
     m.close()
 
 
