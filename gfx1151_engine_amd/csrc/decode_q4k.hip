@@ -52,23 +52,26 @@ __device__ __forceinline__ void load_xu(XU& x, const uint32_t* planes, const flo
 }
 
 // gguf scale_min_k4 for sub-blocks 2jj and 2jj+1 of a super-block whose header words are hd
-// (hd.x = d | dmin << 16, hd.y/z/w = the 12 packed bytes); jj differs per lane: both forms, then select
+// (hd.x = d | dmin << 16, hd.y/z/w = the 12 packed bytes q[0..11]).  Sub-blocks j < 4 keep their
+// 6-bit scale in q[j] and min in q[4+j]; j >= 4 keep 4 bits of each in q[4+j] and the top 2 bits in
+// the upper bits of q[j-4] / q[j].  jj differs per lane, so both forms are one sequence of
+// bit-field extracts whose source word and widths are per-lane values (a width of 0 extracts 0).
 __device__ __forceinline__ void k4_pair(const uint4 hd, int jj, float& a0, float& b0, float& a1, float& b1) {
   union { uint32_t u; __half2 h; } dd;
   dd.u = hd.x;
   const float d = __low2float(dd.h), dmin = __high2float(dd.h);
-  const int shl = 16 * (jj & 1);
-  const uint32_t ylo = hd.y >> shl, zlo = hd.z >> shl, wlo = hd.w >> shl;
-  // jj < 2
-  const uint32_t sc0a = ylo & 63, sc1a = (ylo >> 8) & 63, m0a = zlo & 63, m1a = (zlo >> 8) & 63;
-  // jj >= 2
-  const uint32_t sc0b = (wlo & 0xf) | (((ylo >> 6) & 3) << 4), m0b = ((wlo >> 4) & 0xf) | (((zlo >> 6) & 3) << 4);
-  const uint32_t sc1b = ((wlo >> 8) & 0xf) | (((ylo >> 14) & 3) << 4), m1b = ((wlo >> 12) & 0xf) | (((zlo >> 14) & 3) << 4);
   const bool lo = jj < 2;
-  a0 = d * (float)(lo ? sc0a : sc0b);
-  a1 = d * (float)(lo ? sc1a : sc1b);
-  b0 = dmin * (float)(lo ? m0a : m0b);
-  b1 = dmin * (float)(lo ? m1a : m1b);
+  const uint32_t sh = 16u * (jj & 1), wid = lo ? 6u : 4u, wid2 = lo ? 0u : 2u;
+  const uint32_t y = hd.y, z = hd.z, w = hd.w;
+  const uint32_t A = lo ? y : w, B = lo ? z : w >> 4;
+  const uint32_t sc0 = __builtin_amdgcn_ubfe(A, sh, wid) | (__builtin_amdgcn_ubfe(y, sh + 6, wid2) << 4);
+  const uint32_t sc1 = __builtin_amdgcn_ubfe(A, sh + 8, wid) | (__builtin_amdgcn_ubfe(y, sh + 14, wid2) << 4);
+  const uint32_t m0 = __builtin_amdgcn_ubfe(B, sh, wid) | (__builtin_amdgcn_ubfe(z, sh + 6, wid2) << 4);
+  const uint32_t m1 = __builtin_amdgcn_ubfe(B, sh + 8, wid) | (__builtin_amdgcn_ubfe(z, sh + 14, wid2) << 4);
+  a0 = d * (float)sc0;
+  a1 = d * (float)sc1;
+  b0 = dmin * (float)m0;
+  b1 = dmin * (float)m1;
 }
 
 // one unit of one row: c0, c1 = its 32 code bytes, hd = the super-block header
