@@ -74,6 +74,10 @@ struct moe_ctx {
   hipEvent_t ev[MOE_PROF_STAGES + 1] = {};
   int ev_n = 0;            // events recorded by the last call
   int ev_stage[MOE_PROF_STAGES] = {};
+  // batch path: the f32 -> f16 copy of x runs on a side stream next to the latency-bound top-k and
+  // permutation launches (forked after the logits launch, joined in front of the gate/up GEMM)
+  hipStream_t side = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
 };
 
 static void prof_mark(moe_ctx* c, int stage_done, hipStream_t st) {
@@ -102,6 +106,9 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->routing) rc = moe_routing_destroy(c->routing);
   for (hipEvent_t e : c->ev)
     if (e) (void)hipEventDestroy(e);
+  if (c->ev_fork) (void)hipEventDestroy(c->ev_fork);
+  if (c->ev_join) (void)hipEventDestroy(c->ev_join);
+  if (c->side) (void)hipStreamDestroy(c->side);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16, c->pairs32};
   for (void* b : bufs)
@@ -168,6 +175,11 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
     if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);
   }
   for (int i = 0; i <= MOE_PROF_STAGES && e == hipSuccess; i++) e = hipEventCreate(&c->ev[i]);
+  if (e == hipSuccess && c->x16) {
+    e = hipStreamCreateWithFlags(&c->side, hipStreamNonBlocking);  // default priority
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_join, hipEventDisableTiming);
+  }
   if (e != hipSuccess) {
     moe_destroy(c);
     return (int)e;
@@ -510,15 +522,28 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   if ((rc = moe_router_logits_seq(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
                                   c->sh_logit, c->xms, st)))
     return rc;
-  if ((rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st))) return rc;
-  prof_mark(c, MOE_PROF_ROUTER, st);
-  if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
-                            g.experts, g.id_stride, st)))
-    return rc;
+  // x -> f16 (HBM-bound) on the side stream while top-k, counting, scan and scatter (small dependent
+  // launches that leave the memory system idle) run on the caller's stream
+  MOE_HIP(hipEventRecord(c->ev_fork, st));
+  MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
+  const int rc16 = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
+  // the side stream is joined on every path out of here (a capture on `st` must not end with it forked)
+  auto join = [&]() -> int {
+    hipError_t e = hipEventRecord(c->ev_join, c->side);
+    if (e == hipSuccess) e = hipStreamWaitEvent(st, c->ev_join, 0);
+    return (int)e;
+  };
   const int sh_first = L.has_shared ? P * g.topk : -1;
-  if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, sh_first, c->tokidx, st)))
-    return rc;
-  if ((rc = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, st))) return rc;
+  rc = rc16;
+  if (!rc) rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
+  prof_mark(c, MOE_PROF_ROUTER, st);
+  if (!rc)
+    rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
+                         g.id_stride, st);
+  if (!rc) rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, sh_first, c->tokidx, st);
+  const int jrc = join();
+  if (rc) return rc;
+  if (jrc) return jrc;
   prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
   if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,
