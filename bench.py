@@ -27,7 +27,7 @@ D, MID, E, K = 3072, 768, 512, 10
 # HBM bytes per launch of the dominant kernel (read + written) at the default shapes, from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic.txt (counters
 # cannot be read from inside this process; other shapes report null)
-PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4878.16e6, ("decode", "q4cp", 1): 29.58e6}
+PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4852.10e6, ("decode", "q4cp", 1): 29.60e6}
 CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
 
 
