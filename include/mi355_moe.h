@@ -192,7 +192,11 @@ int moe_set_shared(moe_ctx* ctx, int layer, const moe_wview* gate_proj, const mo
                    const moe_wview* down_proj, const moe_wview* shared_gate, int sh_gguf_type);
 /* GpuModel::moe (40_model.inc:1806) for P == 1 and GpuModel::moe_b (40_model.inc:4018) for a
  * batch: y[P][d] = routed experts (top-k, renormalised) + sigmoid-gated shared expert.
- * x, y: f32 [P][d]; y is fully overwritten. */
+ * x, y: f32 [P][d]; y is fully overwritten.
+ * Everything is enqueued, nothing waits on the host and nothing is allocated.  Batches above 32 tokens also
+ * use one stream that the context owns (default priority): it is forked from st and joined back into st by
+ * events inside the call, so work queued on st after the call is ordered after all of it, and a stream
+ * capture on st takes that stream in and closes it again. */
 int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_stream_t st);
 /* Switches in the spirit of the reference's QWENOX_* opt-outs (src/gpu/parts/40_model.inc:1959-1996):
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
