@@ -277,6 +277,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   half2v as2[NF][NS], bs2[NF][NS];
   float scf[NF];
   uint4 hdr[NF];
+  uint32_t k4w[Q4K ? NF : 1][6];  // Q4_K: the current super-block's scale / min fields and (d, d), (-dmin, -dmin)
   const uint8_t* Ab = A0;
   auto load_a1 = [&](int q, int mf, half8* dst) {
     const int m = 32 * mf + n;
@@ -314,38 +315,47 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
           scf[nf] = (float)cv.f;
         }
       } else {
-        if (Q4K) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
-        else scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
+        if (Q4K) {
+          if ((s & 3) == 0) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
+        } else {
+          scf[nf] = (float)*(const _Float16*)(Sb + wrow[nf] * 16 + sidx * 2);
+        }
       }
     }
   };
   auto scale_consts = [&](int s) {
     if (Q4K) {
-      // sub-blocks 2jj and 2jj+1 of the super-block: 6-bit (scale, min) pairs, gguf scale_min_k4
+      // sub-blocks 2jj and 2jj+1 of the super-block: 6-bit (scale, min) pairs, gguf scale_min_k4.
+      // At the first stage of a super-block its 12 packed bytes are spread into four words of byte
+      // fields (scales 0-3, scales 4-7, mins 0-3, mins 4-7: nine bit operations for all sixteen)
+      // and (d, d), (-dmin, -dmin) are kept as packed halves.  A stage then takes its two bytes of
+      // each word straight into the f16 "1024 + n" form with one byte permute, and d * sc, dmin * m
+      // are packed f16 products: exact integers times an f16, one rounding, the same values as
+      // f16(f32(d) * sc).
       const int jj = s & 3;
+      const uint32_t selb = (jj & 1) ? 0x04030402u : 0x04010400u;  // bytes 2,3 or 0,1 of the word | 0x64 above each
 #pragma unroll
       for (int nf = 0; nf < NF; nf++) {
-        const uint4 hd = hdr[nf];
-        union { uint32_t u; half2v h; } dd;
-        dd.u = hd.x;
-        const float d = (float)dd.h.x, dmin = (float)dd.h.y;
-        uint32_t sc0, m0, sc1, m1;
-        if (jj < 2) {
-          const int sh = 16 * jj;
-          sc0 = (hd.y >> sh) & 63; sc1 = (hd.y >> (sh + 8)) & 63;
-          m0 = (hd.z >> sh) & 63; m1 = (hd.z >> (sh + 8)) & 63;
-        } else {
-          const int sh = 16 * (jj - 2);
-          const uint32_t b8 = hd.w >> sh;
-          sc0 = (b8 & 0xf) | (((hd.y >> (sh + 6)) & 3) << 4);
-          m0 = ((b8 >> 4) & 0xf) | (((hd.z >> (sh + 6)) & 3) << 4);
-          sc1 = ((b8 >> 8) & 0xf) | (((hd.y >> (sh + 14)) & 3) << 4);
-          m1 = ((b8 >> 12) & 0xf) | (((hd.z >> (sh + 14)) & 3) << 4);
+        if (jj == 0) {
+          const uint4 hd = hdr[nf];
+          k4w[nf][0] = hd.y & 0x3f3f3f3fu;
+          k4w[nf][1] = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
+          k4w[nf][2] = hd.z & 0x3f3f3f3fu;
+          k4w[nf][3] = ((hd.w >> 4) & 0x0f0f0f0fu) | ((hd.z >> 2) & 0x30303030u);
+          k4w[nf][4] = __builtin_amdgcn_perm(hd.x, hd.x, 0x01000100u);                 // (d, d)
+          k4w[nf][5] = __builtin_amdgcn_perm(hd.x, hd.x, 0x03020302u) ^ 0x80008000u;  // (-dmin, -dmin)
         }
-        const _Float16 a0 = (_Float16)(d * (float)sc0), b0 = (_Float16)(-(dmin * (float)m0));
-        const _Float16 a1 = (_Float16)(d * (float)sc1), b1 = (_Float16)(-(dmin * (float)m1));
-        as2[nf][0] = half2v{a0, a0}; bs2[nf][0] = half2v{b0, b0};
-        as2[nf][NS - 1] = half2v{a1, a1}; bs2[nf][NS - 1] = half2v{b1, b1};
+        const uint32_t wsc = jj < 2 ? k4w[nf][0] : k4w[nf][1], wmn = jj < 2 ? k4w[nf][2] : k4w[nf][3];
+        const half2v k1024 = half2v{(_Float16)1024.f, (_Float16)1024.f};
+        const half2v sc = as_h2(__builtin_amdgcn_perm(0x64646464u, wsc, selb)) - k1024;
+        const half2v mn = as_h2(__builtin_amdgcn_perm(0x64646464u, wmn, selb)) - k1024;
+        union { half2v h; uint32_t u; } a, b;
+        a.h = sc * as_h2(k4w[nf][4]);
+        b.h = mn * as_h2(k4w[nf][5]);
+        as2[nf][0] = as_h2(__builtin_amdgcn_perm(a.u, a.u, 0x01000100u));
+        bs2[nf][0] = as_h2(__builtin_amdgcn_perm(b.u, b.u, 0x01000100u));
+        as2[nf][NS - 1] = as_h2(__builtin_amdgcn_perm(a.u, a.u, 0x03020302u));
+        bs2[nf][NS - 1] = as_h2(__builtin_amdgcn_perm(b.u, b.u, 0x03020302u));
       }
     } else {
 #pragma unroll
