@@ -55,11 +55,13 @@ def test_full_size_layer(oracle, fmt, T):
     m.close()
 
 
-def test_full_size_decode_rotating_tokens(oracle):
-    """T=1 over several tokens of one full-size q4cp layer: ids bit-exact, output within 1e-4."""
+@pytest.mark.parametrize("fmt,tol", [("q4cp", 2e-4), ("q4k", 5e-4)])
+def test_full_size_decode_rotating_tokens(oracle, fmt, tol):
+    """T=1 over several tokens of one full-size layer (E = 512: the top-k inside the gate/up launch at its
+    real width): ids and router weights bit-exact, output within the integer-dot kernels' tolerance."""
     import torch
     from gfx1151_engine_amd import capi, workloads as W
-    L = W.DeviceLayer(777, D, MID, E, K, "q4cp")
+    L = W.DeviceLayer(777, D, MID, E, K, fmt)
     m = capi.Moe(D, MID, E, K, layers=1, max_tokens=1)
     L.register(m, 0)
     ol = oracle.layer_from_device(L)
@@ -71,5 +73,6 @@ def test_full_size_decode_rotating_tokens(oracle):
         ids, ws = m.last_routing(1)
         yo, io, wo = oracle.moe_layer(ol, x.cpu().numpy())
         assert (ids.cpu().numpy()[:, :K] == io[:, :K]).all(), i
-        assert _max_abs_rel(y, yo) <= 1e-4, i
+        assert np.abs(ws.cpu().numpy()[:, :K] - wo[:, :K]).max() <= 1e-6, i
+        assert _max_abs_rel(y, yo) <= tol, (i, _max_abs_rel(y, yo))
     m.close()
