@@ -57,12 +57,25 @@ __global__ void __launch_bounds__(RT_MAXE) k_route_scan(const int* __restrict__ 
   __shared__ int wsum[RT_MAXE / 64];
   const int e = threadIdx.x, lane = e & 63, w = e >> 6;
   int run = 0;
-  if (e < E)
-    for (int b = 0; b < nblk; b++) {
+  if (e < E) {
+    // eight block counts are requested together: one at a time the loop is a chain of L2 round trips
+    int b = 0;
+    for (; b + 8 <= nblk; b += 8) {
+      int c[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) c[i] = blockcnt[(size_t)(b + i) * E + e];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        blockoff[(size_t)(b + i) * E + e] = run;
+        run += c[i];
+      }
+    }
+    for (; b < nblk; b++) {
       const int c = blockcnt[(size_t)b * E + e];
       blockoff[(size_t)b * E + e] = run;
       run += c;
     }
+  }
   // inclusive scan inside the wave
   int inc = run;
 #pragma unroll
@@ -91,18 +104,35 @@ __global__ void __launch_bounds__(256) k_route_scatter(const int* __restrict__ i
   const int tok = blockIdx.x * RT_TOK + threadIdx.x;
   if (tok >= P) return;
   const unsigned long long below = lane ? (~0ull >> (64 - lane)) : 0ull;
-  for (int s = 0; s < k; s++) {
-    const int key = ids[(size_t)tok * id_stride + s];
-    if (key < 0 || key >= E) continue;
-    int pos = eoff[key] + blockoff[(size_t)blockIdx.x * E + key];
-    for (int i = 0; i < w; i++) pos += __popcll(masks[i][key]);
-    pos += __popcll(masks[w][key] & below);
-    tokidx[pos] = tok;
-    pw[pos] = ws[(size_t)tok * id_stride + s];
-    if (pairids) {
-      int rank = 0;
-      for (int j = 0; j < k; j++) rank += ids[(size_t)tok * id_stride + j] < key;
-      pairids[(size_t)tok * k + rank] = pos;
+  // the token's slots four at a time: ids and weights first, then the offsets they index, so that
+  // each step of the dependent chain ids -> eoff / blockoff is one round trip for four slots
+  for (int s0 = 0; s0 < k; s0 += 4) {
+    int key[4], base[4];
+    float wv[4];
+    bool ok[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int s = s0 + i < k ? s0 + i : k - 1;
+      key[i] = ids[(size_t)tok * id_stride + s];
+      wv[i] = ws[(size_t)tok * id_stride + s];
+      ok[i] = s0 + i < k && key[i] >= 0 && key[i] < E;
+      key[i] = ok[i] ? key[i] : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) base[i] = eoff[key[i]] + blockoff[(size_t)blockIdx.x * E + key[i]];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      if (!ok[i]) continue;
+      int pos = base[i];
+      for (int j = 0; j < w; j++) pos += __popcll(masks[j][key[i]]);
+      pos += __popcll(masks[w][key[i]] & below);
+      tokidx[pos] = tok;
+      pw[pos] = wv[i];
+      if (pairids) {
+        int rank = 0;
+        for (int j = 0; j < k; j++) rank += ids[(size_t)tok * id_stride + j] < key[i];
+        pairids[(size_t)tok * k + rank] = pos;
+      }
     }
   }
 }
