@@ -68,7 +68,7 @@ struct moe_ctx {
   __half* hid16 = nullptr;    // [(k+1)T][mid]
   __half* pairs16 = nullptr;  // [(k+1)T][d]
   float* pairs32 = nullptr;   // [(k+1)min(T,small_max)][d] unweighted pair rows of the unique-expert small-batch path
-  int uq_min = 0;             // > 0: small batches of at least this many tokens read every distinct expert once
+  int uq_min = 20;            // > 0: small batches of at least this many tokens read every distinct expert once
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
   bool profile = false;
   hipEvent_t ev[MOE_PROF_STAGES + 1] = {};
@@ -411,12 +411,18 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     if (use_uq) {
       // verify-size batches: tokens share experts; walk the expert-sorted pair lists so that every
       // distinct expert's weights are read once (reference: the _uq kernels, 26_kernels_moe_gguf.inc:758-877)
-      if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
-                                g.experts, g.id_stride, st)))
-        return rc;
       const int sh_first = L.has_shared ? P * g.topk : -1;
-      if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 4, P, sh_first, c->tokidx, st)))
-        return rc;
+      if (moe_route_small_supported(P, g.topk, g.experts)) {  // permutation and tiles in one launch
+        if ((rc = moe_launch_route_small(c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
+                                         g.id_stride, c->tiles, c->ntiles, 4, sh_first, st)))
+          return rc;
+      } else {
+        if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
+                                  g.experts, g.id_stride, st)))
+          return rc;
+        if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 4, P, sh_first, c->tokidx, st)))
+          return rc;
+      }
       prof_mark(c, MOE_PROF_ROUTE, st);
       const int max_tiles = P * g.topk + (L.has_shared ? (P + 3) / 4 : 0);  // tiles of <= 4 pairs
       if ((rc = moe_launch_dec_gu_uq(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,

@@ -29,6 +29,11 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
                          hipStream_t st);
+// permutation (+ tile list with tiles != nullptr) of a batch of at most 32 tokens in one launch
+bool moe_route_small_supported(int P, int k, int experts);
+int moe_launch_route_small(const int* ids, const float* ws, int* tokidx, float* pw, int* eoff, int* pairids,
+                           int P, int k, int experts, int id_stride, moe_tile* tiles, int* ntiles, int cap,
+                           int sh_first, hipStream_t st);
 int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E, int cap, int P,
                             int sh_first, int* tokidx, hipStream_t st);
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,

@@ -4,6 +4,7 @@
 // ascending token order, exactly what the reference's stable radix sort yields.
 // (reference: src/gpu/parts/10_ple_io.inc:784-861)
 #include "common.h"
+#include "internal.h"
 
 struct moe_routing {
   int capacity_pairs, experts, max_blocks;
@@ -166,7 +167,116 @@ __global__ void __launch_bounds__(RT_MAXE) k_tiles(const int* __restrict__ eoff,
     tiles[begin + j] = t;
   }
 }
+// Batches of at most 32 tokens: the whole permutation in one block and one launch.  An expert's
+// members are a 32-bit token mask in LDS (a token picks an expert at most once), so a pair's slot
+// is its expert's offset plus the count of lower tokens in the mask: the same stable order as the
+// general kernels.  With `tiles` the tile list (routed experts in runs of `cap`, then the shared
+// expert's runs over all tokens, whose tokidx entries are the identity) comes out of the same launch.
+__global__ void __launch_bounds__(RT_MAXE) k_route_small(const int* __restrict__ ids, const float* __restrict__ ws,
+                                                         int P, int k, int E, int id_stride,
+                                                         int* __restrict__ tokidx, float* __restrict__ pw,
+                                                         int* __restrict__ eoff, int* __restrict__ pairids,
+                                                         moe_tile* __restrict__ tiles, int* __restrict__ total,
+                                                         int cap, int sh_first) {
+  __shared__ uint32_t mask[RT_MAXE];
+  __shared__ int eo[RT_MAXE];
+  __shared__ int wsum[RT_MAXE / 64], tsum[RT_MAXE / 64];
+  __shared__ int routed_total;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  mask[tid] = 0u;
+  __syncthreads();
+  const int n = P * k;
+  int tok = 0, key = -1;
+  float wt = 0.f;
+  if (tid < n) {
+    tok = tid / k;
+    const int s = tid - tok * k;
+    key = ids[(size_t)tok * id_stride + s];
+    wt = ws[(size_t)tok * id_stride + s];
+    if (key < 0 || key >= E) key = -1;
+    else atomicOr(&mask[key], 1u << tok);
+  }
+  __syncthreads();
+  const int e = tid;
+  const int ne = e < E ? __popc(mask[e]) : 0;
+  const int nt = tiles ? (ne + cap - 1) / cap : 0;
+  int incE = ne, incT = nt;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(incE, o, 64), u = __shfl_up(incT, o, 64);
+    if (lane >= o) {
+      incE += v;
+      incT += u;
+    }
+  }
+  if (lane == 63) {
+    wsum[w] = incE;
+    tsum[w] = incT;
+  }
+  __syncthreads();
+  int baseE = 0, baseT = 0;
+  for (int i = 0; i < w; i++) {
+    baseE += wsum[i];
+    baseT += tsum[i];
+  }
+  const int first = baseE + incE - ne, begin = baseT + incT - nt;
+  eo[e] = first;
+  if (e < E) eoff[e] = first;
+  if (e == E - 1) eoff[E] = first + ne;
+  if (e == RT_MAXE - 1) routed_total = begin + nt;
+  for (int j = 0; j < nt; j++) {
+    moe_tile t;
+    t.expert = e;
+    t.first = first + j * cap;
+    t.count = min(cap, ne - j * cap);
+    tiles[begin + j] = t;
+  }
+  __syncthreads();
+  if (key >= 0) {
+    const int pos = eo[key] + __popc(mask[key] & ((1u << tok) - 1u));
+    tokidx[pos] = tok;
+    pw[pos] = wt;
+    if (pairids) {
+      int rank = 0;
+      for (int j = 0; j < k; j++) rank += ids[(size_t)tok * id_stride + j] < key;
+      pairids[(size_t)tok * k + rank] = pos;
+    }
+  }
+  if (tiles) {
+    const int nsh = sh_first >= 0 ? (P + cap - 1) / cap : 0;
+    for (int j = tid; j < nsh; j += RT_MAXE) {
+      moe_tile t;
+      t.expert = E;
+      t.first = sh_first + j * cap;
+      t.count = min(cap, P - j * cap);
+      tiles[routed_total + j] = t;
+    }
+    if (tid == 0) {
+      total[0] = routed_total + nsh;
+      total[1] = routed_total;
+    }
+    if (sh_first >= 0)
+      for (int i = tid; i < P; i += RT_MAXE) tokidx[sh_first + i] = i;
+  }
+}
 }  // namespace
+
+bool moe_route_small_supported(int P, int k, int experts) {
+  return P >= 1 && P <= 32 && k >= 1 && P * k <= RT_MAXE && experts >= 1 && experts <= RT_MAXE;
+}
+
+// Internal: permutation (and, with tiles != nullptr, the tile list incl. the shared expert's) of a
+// batch of at most 32 tokens in one launch.
+int moe_launch_route_small(const int* ids, const float* ws, int* tokidx, float* pw, int* eoff, int* pairids,
+                           int P, int k, int experts, int id_stride, moe_tile* tiles, int* ntiles, int cap,
+                           int sh_first, hipStream_t st) {
+  if (!ids || !ws || !tokidx || !pw || !eoff || (tiles && (!ntiles || cap < 1))) return MOE_E_INVALID;
+  if (!moe_route_small_supported(P, k, experts) || id_stride < k) return MOE_E_UNSUPPORTED;
+  k_route_small<<<1, RT_MAXE, 0, st>>>(ids, ws, P, k, experts, id_stride, tokidx, pw, eoff, pairids, tiles, ntiles,
+                                       cap, sh_first);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
 
 MOE_API int moe_routing_create(int capacity_pairs, int experts, moe_routing** out) {
   if (!out || capacity_pairs < 1 || experts < 1) return MOE_E_INVALID;
@@ -202,6 +312,9 @@ MOE_API int moe_routing_run(moe_routing* r, const int* ids, const float* ws, int
   if (!r || !eoff || (P > 0 && (!ids || !ws || !tokidx || !pw))) return MOE_E_INVALID;
   if (P < 0 || k < 1 || id_stride < k || experts != r->experts) return MOE_E_INVALID;
   if ((int64_t)P * k > r->capacity_pairs) return MOE_E_STATE;
+  if (moe_route_small_supported(P, k, experts))
+    return moe_launch_route_small(ids, ws, tokidx, pw, eoff, pairids, P, k, experts, id_stride, nullptr, nullptr, 0,
+                                  -1, moe_s(st));
   int nbits = 0;
   for (int v = experts - 1; v; v >>= 1) nbits++;
   const int nblk = (P + RT_TOK - 1) / RT_TOK;

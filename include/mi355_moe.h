@@ -202,11 +202,12 @@ int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_st
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
  * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as
  * digit planes per 32-group, 16 significant bits relative to the group maximum) instead of the f32 FMA kernels. */
-/* MOE_OPT_UNIQUE_MIN_TOKENS (default 0 = off): q4cp batches of at least this many tokens (and at most 32) walk
- * the expert-sorted pair lists, so that an expert shared by several tokens is read once
- * (the reference's _uq decode kernels, src/gpu/parts/26_kernels_moe_gguf.inc:758-877).  Pays when most
- * tokens of a speculative-verify batch agree on their experts; off by default because with little sharing the
- * extra permutation launches cost more than the saved reads. */
+/* MOE_OPT_UNIQUE_MIN_TOKENS (default 20; 0 = off): q4cp batches of at least this many tokens (and at most 32)
+ * walk the expert-sorted pair lists, so that an expert shared by several tokens is read once
+ * (the reference's _uq decode kernels, src/gpu/parts/26_kernels_moe_gguf.inc:758-877).  One extra launch
+ * builds the permutation and the tile list; from about 20 tokens on the saved reads outweigh it even when
+ * the tokens route independently (measured break-even at 20 tokens with 166 distinct experts of 200 slots).
+ * The pairs are then combined in ascending expert order, as on the batch path. */
 enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags

@@ -120,7 +120,7 @@ def test_router_topk_ties_and_wide_range(capi, oracle):
 
 
 # ---------- permutation: exact ----------
-@pytest.mark.parametrize("P,E,k", [(1, 512, 10), (20, 512, 10), (255, 512, 10), (257, 40, 6), (5000, 512, 10), (3, 7, 7)])
+@pytest.mark.parametrize("P,E,k", [(1, 512, 10), (20, 512, 10), (32, 512, 10), (33, 512, 10), (32, 20, 16), (255, 512, 10), (257, 40, 6), (5000, 512, 10), (3, 7, 7)])
 def test_routing_exact(capi, oracle, P, E, k):
     rng = np.random.default_rng(P * 7 + E)
     ids = np.zeros((P, 16), np.int32)
