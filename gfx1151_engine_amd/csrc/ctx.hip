@@ -48,6 +48,8 @@ struct moe_ctx {
   float* ws = nullptr;        // [T][id_stride]
   float* sh_logit = nullptr;  // [T]
   unsigned* ticket = nullptr; // block counter of the fused small-batch router launch (rests at 0)
+  double* kpart = nullptr;    // partial tiles and per-row-group tickets (resting at 0) of the column-split router launch
+  unsigned* ktickets = nullptr;
   float* xms = nullptr;       // [T] mean square of each token's activations (batch path)
   float* sample = nullptr;    // 96 dequantised weight rows (registration-time magnitude estimate)
   float* hid32 = nullptr;     // [min(T,small_max)][k+1][mid] f32 (small-batch path)
@@ -109,7 +111,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->ev_fork) (void)hipEventDestroy(c->ev_fork);
   if (c->ev_join) (void)hipEventDestroy(c->ev_join);
   if (c->side) (void)hipStreamDestroy(c->side);
-  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
+  void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->kpart, c->ktickets, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16, c->pairs32};
   for (void* b : bufs)
     if (b) {
@@ -142,6 +144,9 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   if (e == hipSuccess) e = hipMalloc(&c->sh_logit, T * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ticket, 256);
   if (e == hipSuccess) e = hipMemset(c->ticket, 0, 256);
+  if (e == hipSuccess) e = hipMalloc(&c->kpart, MOE_ROUTER_KPART_BYTES);
+  if (e == hipSuccess) e = hipMalloc(&c->ktickets, MOE_ROUTER_KTICKET_BYTES);
+  if (e == hipSuccess) e = hipMemset(c->ktickets, 0, MOE_ROUTER_KTICKET_BYTES);
   if (e == hipSuccess) e = hipMalloc(&c->xms, T * 4);
   if (e == hipSuccess) e = hipMalloc(&c->sample, (size_t)96 * (cfg->d > cfg->mid ? cfg->d : cfg->mid) * 4);
   const size_t Ts = T < (size_t)c->small_max ? T : (size_t)c->small_max;
@@ -400,7 +405,7 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
                                     c->logits, c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
                                     use_int4k, gu_topk ? nullptr : c->ticket,
-                                    c->ids, c->ws, g.topk, g.id_stride, &fused, st)))
+                                    c->ids, c->ws, g.topk, g.id_stride, &fused, st, c->kpart, c->ktickets)))
     return rc;
   if (!fused && !gu_topk &&
       (rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st)))

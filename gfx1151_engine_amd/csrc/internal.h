@@ -12,7 +12,12 @@ struct moe_hscale {
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
-                            hipStream_t st);
+                            hipStream_t st, double* kpart, unsigned* ktickets);
+// scratch of the column-split router launch (5..32 tokens): fp64 partial tiles of up to 8 splits x 32 tokens
+// for at most MOE_ROUTER_KSPLIT_ROWS rows, and one ticket counter (resting at 0) per 16 rows
+constexpr int MOE_ROUTER_KSPLIT_ROWS = 1040;
+constexpr size_t MOE_ROUTER_KPART_BYTES = (size_t)8 * (MOE_ROUTER_KSPLIT_ROWS / 16) * 512 * sizeof(double);
+constexpr size_t MOE_ROUTER_KTICKET_BYTES = (MOE_ROUTER_KSPLIT_ROWS / 16) * sizeof(unsigned);
 int moe_launch_gemv_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                        const float* x, uint64_t x_stride, const int* ids, int id_stride, int kpt, int P,
                        int mid, float* hid, hipStream_t st);

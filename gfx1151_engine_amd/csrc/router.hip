@@ -479,35 +479,42 @@ void launch_seq(const void* W, bool bf, const float* bias, const void* wx, bool 
 }
 
 
-// ---- 25..32 tokens on the f64 matrix pipe: a block = 16 weight rows x all tokens, its eight waves
-// each take one eighth of the columns and the partial 16 x 16 tiles are added in wave order (fixed,
-// so the result does not depend on timing; same accuracy statement as k_router_small).
+// ---- 5..32 tokens on the f64 matrix pipe: a block = 16 weight rows x all tokens x one column split,
+// its eight waves each take one eighth of the block's columns and the partial 16 x 16 tiles are added in
+// wave order (fixed, so the result does not depend on timing; same accuracy statement as k_router_small).
 // v_mfma_f64_16x16x4_f64: lane l supplies A[row l%16][k l/16] and B[k l/16][token l%16]; a 16-byte load
 // per lane (4 consecutive columns 4*(l/16)..+3 of its row / token) therefore feeds four MFMAs.
 // Every weight is read once, activations come from L2; loads run through a register ring of
-// RX_D 16-column steps.  Needs d % 128 == 0.  Blocks past the rows build the digit planes of x.
-constexpr int RX_D = 12;
-template <bool BF16, int NTT>  // NTT = token tiles of 16 (1 or 2)
+// RD 16-column steps.  Needs d % (128 * KS) == 0.  Blocks past the rows build the digit planes of x.
+// KS > 1 (needs gpart and tickets): the columns are split over KS blocks per row group as well, so that
+// 16 rows x d columns, one block's work with KS = 1 and the whole time of the launch, become KS blocks on KS
+// CUs.  Each block leaves its fp64 partial tile in gpart and takes a ticket of its row group; the block that
+// draws the last one adds the KS partial tiles in split order (fixed again) and writes the logits.  Partial
+// tiles go out and come back as device-scope accesses, the ticket counters rest at 0 between launches.
+template <bool BF16, int NTT, int RD>  // NTT = token tiles of 16 (1 or 2)
 __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__ W, const float* __restrict__ bias,
                                                         const void* __restrict__ Wx, bool wx_bf16,
                                                         const float* __restrict__ x, int P, int E, int d,
                                                         float* __restrict__ logits, float* __restrict__ out_x,
                                                         int nrows, uint32_t* __restrict__ planes,
-                                                        float2* __restrict__ meta, bool planes_natural) {
+                                                        float2* __restrict__ meta, bool planes_natural, int KS,
+                                                        double* gpart, unsigned* tickets) {
   __shared__ double part[8][NTT][64][4];
+  __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nrt = (nrows + 15) >> 4;
-  if ((int)blockIdx.x >= nrt) {
+  if ((int)blockIdx.x >= nrt * KS) {
     const int G = d / 32, gb = (G + 511) / 512;
-    const int q = blockIdx.x - nrt, t = q / gb, g = (q % gb) * 512 + tid;
+    const int q = blockIdx.x - nrt * KS, t = q / gb, g = (q % gb) * 512 + tid;
     if (t < P && g < G) {
       if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
       else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
     }
     return;
   }
+  const int rg = (int)blockIdx.x % nrt, ks = (int)blockIdx.x / nrt;  // row group, column split
   const int li = lane & 15, lg = lane >> 4;
-  const int row = blockIdx.x * 16 + li;
+  const int row = rg * 16 + li;
   const bool rlive = row < nrows, extra = Wx != nullptr && row == E;
   // per-lane weight row (rows past the end read row 0 and are never stored); all loads unconditional
   const bool wbf = extra ? wx_bf16 : BF16;
@@ -520,10 +527,10 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
     xrow[tt] = x + (size_t)(t < P ? t : 0) * d;
     xm[tt] = t < P ? 1.f : 0.f;
   }
-  const int kper = d / 8, k0 = wv * kper + 4 * lg;  // this lane's first column
+  const int kper = d / (8 * KS), k0 = (ks * 8 + wv) * kper + 4 * lg;  // this lane's first column
   const int nit = kper / 16;
-  uint4 wr[RX_D];
-  float4 xr[RX_D][NTT];
+  uint4 wr[RD];
+  float4 xr[RD][NTT];
   auto fetch = [&](int j, int it) {
     const int c = k0 + 16 * (it < nit ? it : nit - 1);  // past the end: a repeat that is never used
     // 16 bytes in either format (bf16: 8 bytes twice), so no branch surrounds the load
@@ -537,10 +544,10 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
 #pragma unroll
   for (int tt = 0; tt < NTT; tt++) acc[tt] = double4v{0.0, 0.0, 0.0, 0.0};
 #pragma unroll
-  for (int j = 0; j < RX_D; j++) fetch(j, j);
-  for (int ib = 0; ib < nit; ib += RX_D) {
+  for (int j = 0; j < RD; j++) fetch(j, j);
+  for (int ib = 0; ib < nit; ib += RD) {
 #pragma unroll
-    for (int j = 0; j < RX_D; j++) {
+    for (int j = 0; j < RD; j++) {
       if (ib + j < nit) {  // block-uniform
         float w[4];
         if (wbf) {
@@ -553,7 +560,7 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
         float4 xv[NTT];
 #pragma unroll
         for (int tt = 0; tt < NTT; tt++) xv[tt] = xr[j][tt];
-        fetch(j, ib + j + RX_D);
+        fetch(j, ib + j + RD);
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const double a = (double)w[q];
@@ -572,12 +579,9 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
     for (int r = 0; r < 4; r++) part[wv][tt][lane][r] = acc[tt][r];
   __syncthreads();
   // D value r of lane l = [row 4r + l/16][token l%16]; one thread per (tile, lane, r) adds the eight partials
-  for (int i = tid; i < NTT * 256; i += 512) {
+  auto emit = [&](int i, double sum) {
     const int tt = i >> 8, l = (i >> 2) & 63, r = i & 3;
-    double sum = part[0][tt][l][r];
-#pragma unroll
-    for (int w = 1; w < 8; w++) sum += part[w][tt][l][r];
-    const int orow = blockIdx.x * 16 + 4 * r + (l >> 4), t = 16 * tt + (l & 15);
+    const int orow = rg * 16 + 4 * r + (l >> 4), t = 16 * tt + (l & 15);
     if (orow < nrows && t < P) {
       float v = (float)sum;
       if (orow == E) out_x[t] = v;
@@ -586,6 +590,39 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
         logits[(size_t)t * E + orow] = v;
       }
     }
+  };
+  constexpr int NV = NTT * 256;
+  for (int i = tid; i < NV; i += 512) {
+    const int tt = i >> 8, l = (i >> 2) & 63, r = i & 3;
+    double sum = part[0][tt][l][r];
+#pragma unroll
+    for (int w = 1; w < 8; w++) sum += part[w][tt][l][r];
+    if (KS == 1) emit(i, sum);
+    else __hip_atomic_store(&gpart[((size_t)ks * nrt + rg) * NV + i], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  if (KS == 1) return;
+  // the block's partial-tile stores have completed before it takes its ticket
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+  if (tid == 0) {
+    const unsigned ticket = __hip_atomic_fetch_add(&tickets[rg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = ticket == (unsigned)KS - 1u;
+    if (s_last) __hip_atomic_store(&tickets[rg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-armed
+  }
+  __syncthreads();
+  if (!s_last) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  for (int i = tid; i < NV; i += 512) {
+    double v[8];  // KS <= 8: all partials requested before the first is used
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+      v[q] = __hip_atomic_load(&gpart[((size_t)(q < KS ? q : 0) * nrt + rg) * NV + i], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+    double sum = v[0];
+#pragma unroll
+    for (int q = 1; q < 8; q++)
+      if (q < KS) sum += v[q];
+    emit(i, sum);
   }
 }
 
@@ -603,7 +640,7 @@ MOE_API int moe_router_logits(const moe_wview* W, const float* bias, const float
   const bool par = mode == 0 && P <= 32 && d % 4 == 0 && moe_aligned(x, 16) && moe_aligned(W->data, 16);
   if (par) {
     return moe_router_logits_small(W, bias, nullptr, x, P, logits, nullptr, nullptr, nullptr, false, nullptr, nullptr,
-                                   nullptr, 0, 0, nullptr, moe_s(st));
+                                   nullptr, 0, 0, nullptr, moe_s(st), nullptr, nullptr);
   } else {
     launch_seq(W->data, bf, bias, nullptr, false, x, P, E, d, logits, nullptr, nullptr, moe_s(st));
   }
@@ -628,25 +665,34 @@ int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
-                            hipStream_t st) {
+                            hipStream_t st, double* kpart, unsigned* ktickets) {
   const int E = (int)W->rows, d = (int)W->cols;
-  // 25..32 tokens with d a multiple of 128 (and one weight format): the f64 matrix pipe kernel.
-  // (Below that k_router_mid is as fast or faster: one block per 16 rows leaves most CUs idle, the
-  // matrix pipe of the busy ones is the limit: 38 us at 32 tokens against 2 x 38 for the split.)
-  const bool mfma_ok = P > 24 && d % 128 == 0 && (!Wx || (Wx->dtype == MOE_DT_BF16) == (W->dtype == MOE_DT_BF16));
+  // The f64 matrix pipe kernel (d a multiple of 128, one weight format).  With the caller's scratch for
+  // partial tiles the columns are split over up to eight blocks per 16 rows and it serves 5..32 tokens;
+  // without it one block per 16 rows leaves most CUs idle (38 us at 32 tokens), which only beats
+  // k_router_mid above 24 tokens.
+  const bool one_fmt = !Wx || (Wx->dtype == MOE_DT_BF16) == (W->dtype == MOE_DT_BF16);
+  int KS = 1;
+  if (kpart && ktickets && one_fmt && P > 4 && E + 1 <= MOE_ROUTER_KSPLIT_ROWS)
+    for (int s = 8; s > 1; s >>= 1)
+      if (d % (128 * s) == 0) {
+        KS = s;
+        break;
+      }
+  const bool mfma_ok = (P > 24 || KS > 1) && d % 128 == 0 && one_fmt;
   if (P > 24 && !mfma_ok) {
     // more than 24 tokens per block cost the kernel its second wave per SIMD (accumulators):
     // two launches of at most 16 tokens read the router matrix twice (L2 / MALL) and are faster
     const int P0 = 16, G = d / 32;
     const size_t pdw = planes_natural ? QV_GROUP_DW : QV4_GROUP_DW;
     int rc = moe_router_logits_small(W, bias, Wx, x, P0, logits, out_x, planes, meta, planes_natural, nullptr, nullptr,
-                                     nullptr, k, id_stride, nullptr, st);
+                                     nullptr, k, id_stride, nullptr, st, nullptr, nullptr);
     if (rc) return rc;
     if (fused_topk) *fused_topk = false;
     return moe_router_logits_small(W, bias, Wx, x + (size_t)P0 * d, P - P0, logits + (size_t)P0 * E,
                                    out_x ? out_x + P0 : nullptr, planes ? planes + (size_t)P0 * G * pdw : nullptr,
                                    meta ? meta + (size_t)P0 * G : nullptr, planes_natural, nullptr, nullptr, nullptr, k,
-                                   id_stride, nullptr, st);
+                                   id_stride, nullptr, st, nullptr, nullptr);
   }
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
@@ -668,11 +714,18 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
     else { if (bf) RSM_GO(true, 4, 16); else RSM_GO(false, 4, 16); }
   } else {
     if (mfma_ok) {
-      // the f64 matrix pipe: 16 rows per block, columns split over its eight waves
+      // the f64 matrix pipe: 16 rows per block, columns split over KS blocks and their eight waves
       const int qb = planes ? P * ((d / 32 + 511) / 512) : 0;
-      dim3 gx((nrows + 15) / 16 + qb);
-#define RX_GO(BF, NTT) k_router_mfma<BF, NTT><<<gx, 512, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural)
-      if (bf) RX_GO(true, 2); else RX_GO(false, 2);
+      dim3 gx((nrows + 15) / 16 * KS + qb);
+#define RX_GO(BF, NTT, RD) k_router_mfma<BF, NTT, RD><<<gx, 512, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, KS, kpart, ktickets)
+      const int nit = d / (8 * KS) / 16;  // ring steps a wave walks
+      if (nit <= 3) {
+        if (P <= 16) { if (bf) RX_GO(true, 1, 3); else RX_GO(false, 1, 3); }
+        else { if (bf) RX_GO(true, 2, 3); else RX_GO(false, 2, 3); }
+      } else {
+        if (P <= 16) { if (bf) RX_GO(true, 1, 12); else RX_GO(false, 1, 12); }
+        else { if (bf) RX_GO(true, 2, 12); else RX_GO(false, 2, 12); }
+      }
 #undef RX_GO
       MOE_LAUNCH_CHECK();
       return MOE_OK;
