@@ -27,6 +27,7 @@ D, MID, E, K = 3072, 768, 512, 10
 # HBM bytes per launch of the dominant kernel (read + written) at the default shapes, from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic.txt (counters
 # cannot be read from inside this process; other shapes report null)
+LIB_OPTIONS = []              # (option id, value) pairs of --opt, applied to every context
 PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4852.10e6, ("decode", "q4cp", 1): 29.60e6}
 CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
 
@@ -108,6 +109,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
     m = capi.Moe(d, mid, E, k, layers=nlayers, max_tokens=T)
     for l, L in enumerate(layers):
         L.register(m, l)
+    for o, v in LIB_OPTIONS:
+        m.set_option(o, v)
     y = torch.empty((T, d), dtype=torch.float32, device="cuda")
 
     def step(i):
@@ -273,12 +276,15 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="headline")
     ap.add_argument("--tokens", type=int, default=0, help="override the batch size of the workload")
+    ap.add_argument("--opt", action="append", default=[], metavar="ID=VALUE",
+                    help="moe_set_option(ID, VALUE) on the context before the run (A/B runs of the library's switches)")
     ap.add_argument("--layers", type=int, default=48, help="stack workload: number of resident layers")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (a kernel of known HBM traffic to scale "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
     a = ap.parse_args()
+    LIB_OPTIONS.extend(tuple(int(v) for v in o.split("=")) for o in a.opt)
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)
         sys.exit(2)

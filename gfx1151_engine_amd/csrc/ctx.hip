@@ -70,6 +70,7 @@ struct moe_ctx {
   __half* hid16 = nullptr;    // [(k+1)T][mid]
   __half* pairs16 = nullptr;  // [(k+1)T][d]
   float* pairs32 = nullptr;   // [(k+1)min(T,small_max)][d] unweighted pair rows of the unique-expert small-batch path
+  bool fused_combine = false; // batch path: the down GEMM adds its weighted rows into y with f32 atomics (no pairs buffer, no reduce launch)
   int uq_min = 20;            // > 0: small batches of at least this many tokens read every distinct expert once
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
   bool profile = false;
@@ -351,6 +352,7 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
       if (value < 0) return MOE_E_INVALID;
       c->uq_min = value;
       return MOE_OK;
+    case MOE_OPT_FUSED_COMBINE: c->fused_combine = value != 0; return MOE_OK;
     default: return MOE_E_INVALID;
   }
 }
@@ -537,7 +539,9 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   // launches that leave the memory system idle) run on the caller's stream
   MOE_HIP(hipEventRecord(c->ev_fork, st));
   MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
-  const int rc16 = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
+  int rc16 = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
+  const bool fused = c->fused_combine;
+  if (fused && !rc16) rc16 = moe_launch_zero_f32(y, (uint64_t)P * g.d, c->side);  // after the last read of x
   // the side stream is joined on every path out of here (a capture on `st` must not end with it forked)
   auto join = [&]() -> int {
     hipError_t e = hipEventRecord(c->ev_join, c->side);
@@ -558,11 +562,18 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
   if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,
-                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, q4k, hs, st)))
+                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr)))
     return rc;
   prof_mark(c, MOE_PROF_UP, st);
+  if (fused) {
+    const moe_comb cmb{y, c->tokidx, c->pw, L.has_shared ? c->sh_logit : nullptr};
+    rc = moe_launch_gemm_q4cp(false, &dn, L.has_shared ? &sdn : nullptr, g.experts, c->hid16, nullptr, c->tiles,
+                              c->ntiles, max_tiles, y, g.d, g.mid, false, q4k, hs, st, &cmb);
+    prof_mark(c, MOE_PROF_DOWN, st);
+    return rc;
+  }
   if ((rc = moe_launch_gemm_q4cp(false, &dn, L.has_shared ? &sdn : nullptr, g.experts, c->hid16, nullptr,
-                                 c->tiles, c->ntiles, max_tiles, c->pairs16, g.d, g.mid, true, q4k, hs, st)))
+                                 c->tiles, c->ntiles, max_tiles, c->pairs16, g.d, g.mid, true, q4k, hs, st, nullptr)))
     return rc;
   prof_mark(c, MOE_PROF_DOWN, st);
   rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,

@@ -125,7 +125,7 @@ template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, int ri, const float* __restrict__ xms,
-                                          float cmag) {
+                                          float cmag, const moe_comb& cmb, bool shared) {
   constexpr int NH = NF / 2;  // gate/up: fragments per half
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
@@ -540,6 +540,36 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         }
       }
     }
+  } else if (cmb.y) {
+    // fused weighted combine: the tile's rows are added straight into their tokens' output rows
+    // (f32 atomics executed in L2, no value returned), weight = the pair's routing weight (the
+    // shared expert's: sigmoid of its gate logit) over the f16 range-guard factor of the token.
+    // A half-wave covers 32 consecutive floats of one output row per instruction.
+    __syncthreads();  // every wave is past its last use of rowidx
+    if (tid < BM) {
+      const int p = tile.first + (tid < tile.count ? tid : 0);
+      const int t = cmb.tokidx[p];
+      float w = shared ? sigmoid_f(cmb.sg[t]) : cmb.pw[p];
+      if (xms) w /= moe_hid_scale(cmag, xms[t]);
+      rowidx[tid] = t;
+      rowscale[tid] = w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int mf = 0; mf < MF; mf++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int m = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
+        if (m >= tile.count) continue;
+        float* yrow = cmb.y + (size_t)rowidx[m] * M;
+        const float w = rowscale[m];
+#pragma unroll
+        for (int nf = 0; nf < NF; nf++) {
+          const int col = colbase + 32 * nf + n;
+          if (col < M) unsafeAtomicAdd(yrow + col, w * acc[mf][nf][r]);
+        }
+      }
+    }
   } else {
 #pragma unroll
     for (int mf = 0; mf < MF; mf++) {
@@ -562,7 +592,7 @@ __global__ void __launch_bounds__(NT, WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,
-                moe_hscale hs) {
+                moe_hscale hs, moe_comb cmb) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
@@ -618,8 +648,8 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag); \
-    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag);      \
+    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag, cmb, shared); \
+    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag, cmb, shared); \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
@@ -657,8 +687,13 @@ bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k) {
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st) {
+                         hipStream_t st, const moe_comb* comb) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
+  moe_comb cmb{};
+  if (comb) {  // fused combine: down launch with f32 results, out = the (zeroed) token rows
+    if (up || f16out || !comb->tokidx || !comb->pw || (sh && !comb->sg) || comb->y != out) return MOE_E_INVALID;
+    cmb = *comb;
+  }
   if (!lut_ok(routed, up, k, q4k) || (sh && !lut_ok(sh, up, k, q4k))) return MOE_E_UNSUPPORTED;
   if (m < 32 || m % 32) return MOE_E_UNSUPPORTED;
   if (q4k && up && m % 64) return MOE_E_UNSUPPORTED;  // hid is written in whole 64-element blocks
@@ -679,7 +714,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
       attr_done = true;                                                                                       \
     }                                                                                                         \
     k_moe_gemm_q4cp<UPK, F16, Q><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
-                                                               m, k, nblk_n, split, hs);                      \
+                                                               m, k, nblk_n, split, hs, cmb);                 \
   } while (0)
   if (q4k) {
     if (up) GEMM_LAUNCH(true, true, true);
@@ -713,7 +748,7 @@ MOE_API int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* 
   if (type != MOE_LUT_Q4CP) return MOE_E_UNSUPPORTED;
   if (!tokidx) return MOE_E_INVALID;
   return moe_launch_gemm_q4cp(true, p, nullptr, 1 << 30, (const __half*)x16, tokidx, tiles, ntiles, max_tiles,
-                              hid16, m, k, true, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
+                              hid16, m, k, true, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
 }
 
 MOE_API int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
@@ -721,7 +756,7 @@ MOE_API int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const m
                          moe_stream_t st) {
   if (type != MOE_LUT_Q4CP) return MOE_E_UNSUPPORTED;
   return moe_launch_gemm_q4cp(false, p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
-                              max_tiles, pairs, m, k, f16 != 0, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
+                              max_tiles, pairs, m, k, f16 != 0, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
 }
 
 // moe_gg_up / moe_gg_down: raw GGUF blocks, expert e's rows start at row e * m of each tensor
@@ -735,7 +770,7 @@ MOE_API int moe_gg_up(int type, const uint8_t* gate, const uint8_t* up, const vo
   p.w_up = up;
   p.e_rows = m;
   return moe_launch_gemm_q4cp(true, &p, nullptr, 1 << 30, (const __half*)x16, tokidx, tiles, ntiles, max_tiles,
-                              hid16, m, k, true, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
+                              hid16, m, k, true, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
 }
 
 MOE_API int moe_gg_down(int type, const uint8_t* down, const void* hid16, const moe_tile* tiles,
@@ -746,5 +781,5 @@ MOE_API int moe_gg_down(int type, const uint8_t* down, const void* hid16, const 
   p.w = down;
   p.e_rows = m;
   return moe_launch_gemm_q4cp(false, &p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
-                              max_tiles, pairs, m, k, f16 != 0, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st));
+                              max_tiles, pairs, m, k, f16 != 0, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
 }

@@ -9,6 +9,15 @@ struct moe_hscale {
   float c_routed, c_shared;
 };
 
+// Fused weighted combine of the down launch (f32 results): rows are added into y[tokidx[pair]] with the
+// weight pw[pair] (shared expert: sigmoid(sg[token])); y holds zeros when the launch starts.
+struct moe_comb {
+  float* y;
+  const int* tokidx;
+  const float* pw;
+  const float* sg;
+};
+
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
@@ -33,7 +42,8 @@ int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st);
+                         hipStream_t st, const moe_comb* comb);
+int moe_launch_zero_f32(float* p, uint64_t n, hipStream_t st);
 // permutation (+ tile list with tiles != nullptr) of a batch of at most 32 tokens in one launch
 bool moe_route_small_supported(int P, int k, int experts);
 int moe_launch_route_small(const int* ids, const float* ws, int* tokidx, float* pw, int* eoff, int* pairids,

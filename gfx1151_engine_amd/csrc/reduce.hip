@@ -73,6 +73,11 @@ struct Ld8<float> {
   }
 };
 
+__global__ void __launch_bounds__(256) k_zero_f32(float4* __restrict__ p, uint64_t n4) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += (uint64_t)gridDim.x * 256)
+    p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 template <class PT, int KMAX, int KC>  // KC = K when it is one of the instantiated values, else 0
 __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pairs,
                                                       const int* __restrict__ pairids,
@@ -212,6 +217,17 @@ int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, con
     if (K == 10) RED_GO(float, 10); else if (K == 8) RED_GO(float, 8); else RED_GO(float, 0);
   }
 #undef RED_GO
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// Zero fill by a kernel (a memset node in a captured graph is avoided on purpose).
+int moe_launch_zero_f32(float* p, uint64_t n, hipStream_t st) {
+  if (!p || n % 4 || !moe_aligned(p, 16)) return MOE_E_INVALID;
+  if (n == 0) return MOE_OK;
+  const uint64_t n4 = n / 4;
+  const unsigned grid = (unsigned)((n4 + 255) / 256 > 65536 ? 65536 : (n4 + 255) / 256);
+  k_zero_f32<<<grid, 256, 0, st>>>((float4*)p, n4);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

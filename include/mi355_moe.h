@@ -208,7 +208,12 @@ int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_st
  * builds the permutation and the tile list; from about 20 tokens on the saved reads outweigh it even when
  * the tokens route independently (measured break-even at 20 tokens with 166 distinct experts of 200 slots).
  * The pairs are then combined in ascending expert order, as on the batch path. */
-enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2 };
+/* MOE_OPT_FUSED_COMBINE (default 0): batches over 32 tokens fold the top-k weighted combine into the epilogue of
+ * the down GEMM (the reference keeps pairs + k_moe_reduce_pw_sg, src/gpu/parts/24_kernels_moe_lt.inc:104): a tile's
+ * weighted rows are added into y with f32 atomics, y is zeroed on the context's side stream, no pairs buffer is
+ * written and no reduce launch follows.  The order of the k+1 additions per element then depends on timing, so
+ * results can differ in their last bits from run to run; 0 keeps the ordered two-step form. */
+enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2, MOE_OPT_FUSED_COMBINE = 3 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP

@@ -123,6 +123,20 @@ def test_grouped_gemm_stages_q4k(capi, oracle, d, mid, E, k, P):
     r.close()
 
 
+def check_fused_combine(m, x, y_ordered, yo):
+    """MOE_OPT_FUSED_COMBINE: the down GEMM adds its weighted rows into y (f32 atomics).  Same layer bar; against
+    the ordered two-step result only the f16 rounding of the pair rows and the order of the additions differ.
+    Run twice: y is zeroed inside every call, so what an earlier call left there must not matter."""
+    from gfx1151_engine_amd import capi
+    m.set_option(capi.OPT_FUSED_COMBINE, 1)
+    for _ in range(2):
+        yf = m.forward(0, gpu(x)).cpu().numpy()
+        assert max_abs_rel(yf, yo) <= TOL_LAYER, max_abs_rel(yf, yo)
+        assert max_abs_rel(yf, y_ordered) <= 1e-3, max_abs_rel(yf, y_ordered)
+    m.set_option(capi.OPT_FUSED_COMBINE, 0)
+    assert (m.forward(0, gpu(x)).cpu().numpy() == y_ordered).all(), "the ordered form is deterministic"
+
+
 @pytest.mark.parametrize("d,mid,E,k,T", [(512, 256, 16, 4, 333), (3072, 768, 32, 10, 300)])
 def test_batch_layer_vs_oracle_q4k(oracle, d, mid, E, k, T):
     """GGUF Q4_K experts + Q4_K shared expert through the MFMA path."""
@@ -137,6 +151,7 @@ def test_batch_layer_vs_oracle_q4k(oracle, d, mid, E, k, T):
     assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
     err = max_abs_rel(y, yo)
     assert err <= TOL_LAYER, err
+    check_fused_combine(m, x, y, yo)
     m.close()
 
 
@@ -156,6 +171,7 @@ def test_batch_layer_vs_oracle(oracle, d, mid, E, k, T, skew):
     assert (ws[:, :k].view(np.uint32) == wo[:, :k].view(np.uint32)).all(), "sequential-order router weights are bit-exact"
     err = max_abs_rel(y, yo)
     assert err <= TOL_LAYER, err
+    check_fused_combine(m, x, y, yo)
     m.close()
 
 
