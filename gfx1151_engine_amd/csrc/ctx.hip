@@ -399,7 +399,7 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
                        (!L.has_shared || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
   const bool use_int4k = L.has_gguf && c->int_decode && (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K) &&
                          moe_dec4k_supported(g.d, g.mid, nslots_d);
-  const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min;
+  const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min && moe_dec_uq_supported(g.d);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
   const bool gu_topk = ((use_int && !use_uq) || use_int4k) && moe_dec_gu_topk_supported(g.experts, g.topk);

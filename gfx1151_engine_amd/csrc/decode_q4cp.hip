@@ -339,10 +339,12 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
   }
 }
 
-// Down projection of the unique-expert path: grid (d/32, tiles), block 256 = 8 half-waves of 4 rows.
-// Lane g of a half-wave holds group g of its 4 weight rows and walks the tile's pairs; the
+// Down projection of the unique-expert path: grid (d/DU_ROWS, tiles), block 256 = 8 half-waves of
+// DU_HW rows.  Lane g of a half-wave holds group g of its weight rows and walks the tile's pairs; the
 // unweighted row results go to pairs[pair][row] (f32) for the weighted combine that follows.
-constexpr int DU_ROWS = 32;
+// All loads are unconditional (a lane past the last group reads group 0 and contributes 0) and are
+// requested before the first is used: activation planes of the first pair, then the rows.
+constexpr int DU_HW = 8, DU_ROWS = 8 * DU_HW;
 __global__ void __launch_bounds__(256) k_dec_dn_uq(DnArgs2 A, const uint32_t* __restrict__ hplanes,
                                                    const float2* __restrict__ hmeta,
                                                    const moe_tile* __restrict__ tiles,
@@ -352,33 +354,41 @@ __global__ void __launch_bounds__(256) k_dec_dn_uq(DnArgs2 A, const uint32_t* __
   const moe_tile tile = tiles[blockIdx.y];
   const bool shared = tile.expert >= n_experts;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int G = mid / 32, g = lane & 31, hw = 2 * wv + (lane >> 5);
-  const bool live = g < G;
+  const int G = mid / 32, g_raw = lane & 31, hw = 2 * wv + (lane >> 5);
+  const int g = g_raw < G ? g_raw : 0;
+  const float live = g_raw < G ? 1.f : 0.f;
   const size_t rb = (size_t)mid / 2;
   const DecW W = shared ? A.shd : A.dn;  // block-uniform, by value
-  const int r0 = blockIdx.x * DU_ROWS + 4 * hw;
+  const int r0 = blockIdx.x * DU_ROWS + DU_HW * hw;
   const uint64_t row0 = (shared ? 0 : (uint64_t)tile.expert * d) + r0;
   const uint8_t* cp = W.codes + row0 * rb + (size_t)g * 16;
   const uint8_t* sp = W.scales + row0 * W.ss + g * 2;
-  uint4 cw[4];
-  float sc[4];
+  XG x;
+  load_xg(x, hplanes, hmeta, (size_t)tile.first * G + g);
+  const float c0 = W.cb[0], c1 = W.cb[1];
+  uint4 cw[DU_HW];
+  uint16_t sr[DU_HW];
 #pragma unroll
-  for (int r = 0; r < 4; r++) {
-    if (live) {
-      cw[r] = *(const uint4*)(cp + r * rb);
-      sc[r] = __half2float(*(const __half*)(sp + r * W.ss));
-    }
+  for (int r = 0; r < DU_HW; r++) {
+    cw[r] = *(const uint4*)(cp + r * rb);
+    sr[r] = *(const uint16_t*)(sp + r * W.ss);
   }
-  const float a = W.cb[1] - W.cb[0], b = fmaf(8.f, a, W.cb[0]);
+  __builtin_amdgcn_sched_barrier(0);
+  const float a = c1 - c0, b = fmaf(8.f, a, c0);
   for (int pi = 0; pi < tile.count; pi++) {
     const size_t pr = (size_t)tile.first + pi;
-    XG x;
-    if (live) load_xg(x, hplanes, hmeta, pr * G + g);
+    XG xn;  // the next pair's planes are requested before this pair's dot products (the last pair repeats itself)
+    load_xg(xn, hplanes, hmeta, (pr + (pi + 1 < tile.count ? 1 : 0)) * G + g);
+    float v[DU_HW];
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      const float v = sum32(live ? sc[r] * chunk_dot(cw[r], x, a, b) : 0.f);
-      if (g == 0) pairs[pr * d + r0 + r] = v;
+    for (int r = 0; r < DU_HW; r++)
+      v[r] = sum32(live * __half2float(__ushort_as_half(sr[r])) * chunk_dot(cw[r], x, a, b));
+    if (g_raw == 0) {
+      float4* o = (float4*)(pairs + pr * d + r0);
+#pragma unroll
+      for (int r = 0; r < DU_HW; r += 4) o[r / 4] = make_float4(v[r], v[r + 1], v[r + 2], v[r + 3]);
     }
+    x = xn;
   }
 }
 
@@ -399,8 +409,10 @@ size_t moe_qvec_meta_bytes(int K) { return (size_t)(K / 32) * sizeof(float2); }
 // Supported shapes of the integer-dot decode kernels (otherwise the caller uses the f32 kernels).
 bool moe_dec_supported(int d, int mid, int nslots) {
   return d % 32 == 0 && d / 32 <= 96 && mid % 32 == 0 && mid / 32 <= 32 && nslots <= DN2_MAXSLOTS &&
-         mid % GU2_ROWS == 0 && d % DU_ROWS == 0;  // (d % 32 == 0 covers the 8-row down blocks)
+         mid % GU2_ROWS == 0;  // (d % 32 == 0 covers the 8-row down blocks)
 }
+// the unique-expert kernels on top of that: whole row blocks of the down kernel
+bool moe_dec_uq_supported(int d) { return d % DU_ROWS == 0; }
 
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
                     hipStream_t st) {

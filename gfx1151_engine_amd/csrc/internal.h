@@ -60,6 +60,7 @@ int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview
 size_t moe_qvec_plane_bytes(int K);
 size_t moe_qvec_meta_bytes(int K);
 bool moe_dec_supported(int d, int mid, int nslots);
+bool moe_dec_uq_supported(int d);
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
                     hipStream_t st);
 bool moe_dec_gu_topk_supported(int n_experts, int kpt);
