@@ -71,7 +71,7 @@ struct moe_ctx {
   __half* pairs16 = nullptr;  // [(k+1)T][d]
   float* pairs32 = nullptr;   // [(k+1)min(T,small_max)][d] unweighted pair rows of the unique-expert small-batch path
   bool fused_combine = false; // batch path: the down GEMM adds its weighted rows into y with f32 atomics (no pairs buffer, no reduce launch)
-  int uq_min = 20;            // > 0: small batches of at least this many tokens read every distinct expert once
+  int uq_min = 12;            // > 0: small batches of at least this many tokens read every distinct expert once
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
   bool profile = false;
   hipEvent_t ev[MOE_PROF_STAGES + 1] = {};

@@ -202,11 +202,12 @@ int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_st
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
  * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as
  * digit planes per 32-group, 16 significant bits relative to the group maximum) instead of the f32 FMA kernels. */
-/* MOE_OPT_UNIQUE_MIN_TOKENS (default 20; 0 = off): q4cp batches of at least this many tokens (and at most 32)
+/* MOE_OPT_UNIQUE_MIN_TOKENS (default 12; 0 = off): q4cp batches of at least this many tokens (and at most 32)
  * walk the expert-sorted pair lists, so that an expert shared by several tokens is read once
  * (the reference's _uq decode kernels, src/gpu/parts/26_kernels_moe_gguf.inc:758-877).  One extra launch
- * builds the permutation and the tile list; from about 20 tokens on the saved reads outweigh it even when
- * the tokens route independently (measured break-even at 20 tokens with 166 distinct experts of 200 slots).
+ * builds the permutation and the tile list and a reduce launch follows; from about 12 tokens on the saved reads
+ * outweigh them even when the tokens route independently (measured: 117 against 120 us at 12 tokens with 109
+ * distinct experts for 120 slots, 141 against 153 us at 16, 227 against 296 us at 32).
  * The pairs are then combined in ascending expert order, as on the batch path. */
 /* MOE_OPT_FUSED_COMBINE (default 0): batches over 32 tokens fold the top-k weighted combine into the epilogue of
  * the down GEMM (the reference keeps pairs + k_moe_reduce_pw_sg, src/gpu/parts/24_kernels_moe_lt.inc:104): a tile's

@@ -54,7 +54,7 @@ def test_small_batch_layer(oracle, fmt, d, mid, E, k, T, cb):
 
 
 @pytest.mark.parametrize("fmt,T,rdt", [("q4cp", 3, "f32"), ("q4cp", 32, "f32"), ("q4k", 27, "f32"), ("q4k", 2, "f32"),
-                                        ("q4cp", 1, "bf16"), ("q4cp", 4, "bf16"), ("q4cp", 12, "bf16"),
+                                        ("q4cp", 1, "bf16"), ("q4cp", 4, "bf16"), ("q4cp", 5, "f32"), ("q4cp", 11, "f32"), ("q4cp", 12, "bf16"), ("q4cp", 17, "f32"),
                                         ("q4k", 30, "bf16")])
 def test_small_batch_sizes_and_router_dtypes(oracle, fmt, T, rdt):
     """The token counts at which the small path changes kernels (1 / 2-4 / 5-24 / 25-32: the logits
