@@ -131,7 +131,20 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   __shared__ float sel_ws[64];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int G = d / 32;
-  int s = blockIdx.y, nslots = gridDim.y, e = 0, first = 0, npairs = 1;
+  int s = blockIdx.y, nslots = gridDim.y - (NPL > 0 ? 1 : 0), e = 0, first = 0, npairs = 1;
+  if (NPL > 0 && s == nslots) {
+    // one block of the extra grid row: the exact softmax / top-k (ids, renormalised weights) for the down
+    // launch, next to the blocks that stream the weights and only need the ids
+    if (blockIdx.x == 0) {
+      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)blockIdx.z * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      __syncthreads();
+      if ((int)threadIdx.x < kpt) {
+        ids_out[(size_t)blockIdx.z * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
+        ws_out[(size_t)blockIdx.z * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+      }
+    }
+    return;
+  }
   bool shared;
   if (UQ) {
     if ((int)blockIdx.y >= ntiles[0]) return;
@@ -143,13 +156,14 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   } else if (NPL > 0) {
     shared = s >= kpt;
     if (!shared) {
-      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)blockIdx.z * n_experts, sel_ids, sel_ws, n_experts, kpt);
-      __syncthreads();
-      e = sel_ids[s];
-      if (blockIdx.x == 0 && s == 0 && (int)threadIdx.x < kpt) {
-        ids_out[(size_t)blockIdx.z * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
-        ws_out[(size_t)blockIdx.z * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+      // the ids by logit order (no exps, no sums); the exact selection only when two of the best logits
+      // are too close for that to be certain
+      const float* lg = logits + (size_t)blockIdx.z * n_experts;
+      if (!topk_ids_by_logit<NPL ? NPL : 8>(lg, sel_ids, n_experts, kpt)) {
+        topk_block<NPL ? NPL : 8, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
+        __syncthreads();
       }
+      e = sel_ids[s];
     }
   } else {
     shared = s >= kpt;
@@ -449,7 +463,7 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
   A.gu = decw(gu);
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
-  dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
+  dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);  // + the row of the exact top-k block
   if (n_experts <= 512)
     k_dec_gu<false, 8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
                                              hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws);

@@ -118,7 +118,20 @@ __global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t*
   __shared__ uint32_t pk[QV_GROUP_DW];
   __shared__ int sel_ids[64];
   __shared__ float sel_ws[64];
-  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y;
+  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y - (NPL > 0 ? 1 : 0);
+  if (NPL > 0 && s == nslots) {
+    // one block of the extra grid row: the exact softmax / top-k (ids, renormalised weights) for the down
+    // launch, next to the blocks that stream the weights and only need the ids
+    if (blockIdx.x == 0) {
+      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      __syncthreads();
+      if ((int)threadIdx.x < kpt) {
+        ids_out[(size_t)tok * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
+        ws_out[(size_t)tok * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+      }
+    }
+    return;
+  }
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int U = d / 64;
   const bool shared = s >= kpt;
@@ -126,13 +139,13 @@ __global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t*
   int e = 0;
   if (NPL > 0) {
     if (!shared) {
-      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
-      __syncthreads();
-      e = sel_ids[s];
-      if (blockIdx.x == 0 && s == 0 && (int)threadIdx.x < kpt) {
-        ids_out[(size_t)tok * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
-        ws_out[(size_t)tok * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+      // the ids by logit order; the exact selection only when two of the best logits are too close
+      const float* lg = logits + (size_t)tok * n_experts;
+      if (!topk_ids_by_logit<NPL ? NPL : 8>(lg, sel_ids, n_experts, kpt)) {
+        topk_block<NPL ? NPL : 8, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
+        __syncthreads();
       }
+      e = sel_ids[s];
     }
   } else if (!shared) {
     e = ids[(size_t)tok * id_stride + s];
@@ -297,7 +310,7 @@ int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8
   if (!moe_aligned(gate, 16) || !moe_aligned(up, 16) || (sh_gate && (!moe_aligned(sh_gate, 16) || !moe_aligned(sh_up, 16))))
     return MOE_E_INVALID;
   Gu4kArgs A{gate, up, sh_gate, sh_up};
-  dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0), P);
+  dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);  // + the row of the exact top-k block
   if (n_experts <= 512)
     k_dec4k_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta, logits,
                                         n_experts, ids, ws);

@@ -298,3 +298,85 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
   else topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
 #endif
 }
+
+// The k best experts of one token by their LOGITS, without the softmax: wave 0 of the block selects,
+// all threads return the verdict (the call contains block barriers).  The probabilities of the
+// reference, p = (float)((float)exp(l - max) / sum), are a non-decreasing function of the logit l, so
+// the order by logit is the order by probability unless two probabilities round to the same float,
+// where the reference order falls back to the expert index.  Two logits more than 1e-6 apart give
+// probabilities whose ratio exceeds 1 + 2^-23 after both roundings, i.e. different floats in the same
+// order.  The function therefore checks the k + 1 best logits: every gap between neighbours above
+// 1e-6 -> ids_row[0..k) (LDS) holds the reference's ranking and true is returned; otherwise (also:
+// rows it does not handle, NaNs) false, and the caller runs the exact selection.
+template <int NPL>
+__device__ bool topk_ids_by_logit(const float* lg, int* ids_row, int E, int k) {
+  __shared__ int fast_ok;
+  const int tid = threadIdx.x, lane = tid & 63;
+  bool handled = false;
+  if constexpr (NPL == 8) handled = E % 4 == 0 && E >= 4 && k < E && k < 63 && ((uintptr_t)lg & 15) == 0;
+  if (!handled) return false;  // block-uniform
+  if constexpr (NPL == 8) {
+    if (tid < 64) {
+      // lane-major keys: key[j] of lane l = expert 8 l + j; unsigned keys that order like the floats
+      uint32_t key[8], jj[8];
+#pragma unroll
+      for (int q = 0; q < 2; q++) {
+        const int idx = 8 * lane + 4 * q;
+        const float4 f = *(const float4*)(lg + (idx < E ? idx : 0));
+        const float fv[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const uint32_t u = __float_as_uint(fv[i]);
+          const uint32_t o = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+          key[4 * q + i] = idx < E ? o : 0u;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; j++) jj[j] = (uint32_t)j;
+#pragma unroll
+      for (int pass = 0; pass < 8; pass++) {
+#pragma unroll
+        for (int i = pass & 1; i + 1 < 8; i += 2) {
+          const uint32_t ka = key[i], kb = key[i + 1], ia = jj[i], ib = jj[i + 1];
+          const bool sw = kb > ka;
+          key[i] = umax(ka, kb); key[i + 1] = umin(ka, kb);
+          jj[i] = sw ? ib : ia; jj[i + 1] = sw ? ia : ib;
+        }
+      }
+      uint32_t jw = 0;
+#pragma unroll
+      for (int j = 0; j < 8; j++) jw |= jj[j] << (4 * j);
+      uint32_t mykey = 0;
+      int myid = 0;
+      for (int r = 0; r <= k; r++) {  // k + 1 rounds: the runner-up is needed for the gap test
+        const uint32_t wm = wave_umax(key[0]);
+        const int wl = __builtin_ctzll(__ballot(key[0] == wm));
+        const int wj = __builtin_amdgcn_readlane((int)jw, wl) & 15;
+        if (lane == r) {
+          mykey = wm;
+          myid = 8 * wl + wj;
+        }
+        const bool me = lane == wl;
+#pragma unroll
+        for (int j = 0; j + 1 < 8; j++) {
+          const uint32_t cur = key[j], nxt = key[j + 1];
+          key[j] = me ? nxt : cur;
+        }
+        const uint32_t last = key[7], jsh = jw >> 4;
+        key[7] = me ? 0u : last;
+        jw = me ? jsh : jw;
+      }
+      // lane r holds rank r: its logit against the next rank's (the subtraction of close floats is exact)
+      const uint32_t nk = (uint32_t)__shfl_down((int)mykey, 1, 64);
+      const float la = __uint_as_float((mykey & 0x80000000u) ? (mykey ^ 0x80000000u) : ~mykey);
+      const float lb = __uint_as_float((nk & 0x80000000u) ? (nk ^ 0x80000000u) : ~nk);
+      const bool good = lane >= k || (mykey != 0u && nk != 0u && la - lb > 1e-6f);  // false for NaNs
+      const int ok = __all(good);
+      if (lane < k) ids_row[lane] = myid;
+      if (lane == 0) fast_ok = ok;
+    }
+    __syncthreads();
+    return fast_ok != 0;
+  }
+  return false;
+}

@@ -93,6 +93,33 @@ def test_int_decode_switch(oracle, fmt, T):
     m.close()
 
 
+@pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 6), ("q4k", 1), ("q4k", 3)])
+def test_decode_topk_near_ties(oracle, fmt, T):
+    """The decode gate/up kernels rank the experts by logit and fall back to the exact softmax selection when two
+    of the k + 1 best logits are closer than 1e-6.  Router rows repeated (equal logits: the lower index must come
+    first, and a copy may sit on the rank k / k + 1 boundary) and rows that differ in the last bits force that
+    fallback; ids and order must still be the oracle's."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(17 + T)
+    d, mid, E, k = (3072, 768, 24, 10) if fmt == "q4cp" else (512, 256, 24, 10)
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt)
+    hl.router[7] = hl.router[3]
+    hl.router[20] = hl.router[3]
+    hl.router[11] = hl.router[5]
+    hl.router[16] = hl.router[5] * np.float32(1 + 2 ** -22)
+    hl.router[2] = hl.router[9]
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=8)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    ids, ws = m.last_routing(T)
+    ids, ws = ids.cpu().numpy(), ws.cpu().numpy()
+    assert (ids[:, :k] == io[:, :k]).all(), (ids[:, :k], io[:, :k])
+    assert np.abs(ws[:, :k] - wo[:, :k]).max() <= 1e-6
+    assert max_abs_rel(y, yo) <= tol_small(fmt), max_abs_rel(y, yo)
+    m.close()
+
+
 @pytest.mark.parametrize("share", [0.3, 1.0])
 def test_unique_expert_path(oracle, share):
     """MOE_OPT_UNIQUE_MIN_TOKENS: a verify-size batch through the expert-sorted pair lists (every distinct
