@@ -10,7 +10,7 @@ from helpers import HostLayer
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 48), ("q4k", 1)])
+@pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 7), ("q4cp", 20), ("q4cp", 48), ("q4k", 1), ("q4k", 9)])
 def test_forward_under_graph_capture(oracle, fmt, T):
     import torch
     rng = np.random.default_rng(5 + T)
