@@ -12,6 +12,7 @@ from .build import LIB
 
 F32, BF16, Q4CP = 1, 0, 5
 GGML_Q4_K = 12
+GGML_Q5_K, GGML_Q5_1, GGML_Q8_0 = 13, 7, 8
 
 
 class MoeError(RuntimeError):
@@ -89,6 +90,13 @@ def q4k_dequant_rows(raw, nrows, cols):
     out = torch.empty((nrows, cols), dtype=torch.float32, device=raw.device)
     check(lib().moe_q4k_dequant_rows(ptr(raw), u64(nrows), u64(cols), ptr(out), stream()),
           "moe_q4k_dequant_rows")
+    return out
+
+
+def gg_dequant_rows(gtype, raw, nrows, cols):
+    out = torch.empty((nrows, cols), dtype=torch.float32, device=raw.device)
+    check(lib().moe_gg_dequant_rows(gtype, ptr(raw), u64(nrows), u64(cols), ptr(out), stream()),
+          "moe_gg_dequant_rows")
     return out
 
 

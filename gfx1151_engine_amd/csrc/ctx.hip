@@ -240,9 +240,9 @@ MOE_API int moe_get_config(const moe_ctx* c, moe_config* out) {
 MOE_API int moe_set_experts_gguf(moe_ctx* c, int layer, const moe_gg_experts* gg) {
   MoeLayer* L = layer_of(c, layer);
   if (!L || !gg || !gg->gate || !gg->up || !gg->down) return MOE_E_INVALID;
-  if (gg->tgu != MOE_GGML_Q4_K || gg->tdn != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
-  if (c->cfg.d % 256 || c->cfg.mid % 256) return MOE_E_UNSUPPORTED;
-  {
+  if (!moe_gg_types_supported(gg->tgu, gg->tdn, c->cfg.d, c->cfg.mid)) return MOE_E_UNSUPPORTED;
+  L->c_routed = 0.f;  // the f16 range guard belongs to the grouped GEMM, which reads Q4_K only
+  if (gg->tgu == MOE_GGML_Q4_K && gg->tdn == MOE_GGML_Q4_K) {
     const moe_config& g = c->cfg;
     moe_wview gv{0, gg->gate, (uint64_t)g.experts * g.mid, (uint64_t)g.d, 0};
     moe_wview uv{0, gg->up, (uint64_t)g.experts * g.mid, (uint64_t)g.d, 0};
@@ -267,7 +267,7 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
   if (sg->dtype != MOE_DT_F32 && sg->dtype != MOE_DT_BF16) return MOE_E_UNSUPPORTED;
   if (sh_gguf_type == 0) {
     if (g->dtype != MOE_DT_Q4CP || u->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP) return MOE_E_UNSUPPORTED;
-  } else if (sh_gguf_type != MOE_GGML_Q4_K) {
+  } else if (!moe_gg_types_supported(sh_gguf_type, sh_gguf_type, cf.d, cf.mid)) {
     return MOE_E_UNSUPPORTED;
   }
   L->shared_affine = false;
@@ -277,7 +277,8 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
     if ((rc = codebook_affine(g, &a1)) || (rc = codebook_affine(u, &a2)) || (rc = codebook_affine(dn, &a3))) return rc;
     L->shared_affine = a1 && a2 && a3;
   }
-  {
+  L->c_shared = 0.f;
+  if (sh_gguf_type == 0 || sh_gguf_type == MOE_GGML_Q4_K) {
     int rc = magnitude_constant(c, sh_gguf_type != 0, g, (uint64_t)cf.mid, u, 0, dn, 1, &L->c_shared);
     if (rc) return rc;
   }
@@ -397,7 +398,8 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const int nslots_d = g.topk + (L.has_shared ? 1 : 0);
   const bool use_int = L.has_q4cp && c->int_decode && L.experts_affine && (!L.has_shared || L.shared_affine) &&
                        (!L.has_shared || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
-  const bool use_int4k = L.has_gguf && c->int_decode && (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K) &&
+  const bool use_int4k = L.has_gguf && c->int_decode && L.gg.tgu == MOE_GGML_Q4_K && L.gg.tdn == MOE_GGML_Q4_K &&
+                         (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K) &&
                          moe_dec4k_supported(g.d, g.mid, nslots_d);
   const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min && moe_dec_uq_supported(g.d);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
@@ -472,7 +474,19 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     prof_mark(c, MOE_PROF_DOWN, st);
     return rc;
   }
-  if (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
+  if (L.has_shared && L.sh_gguf_type == 0) return MOE_E_UNSUPPORTED;
+  if (L.gg.tgu != MOE_GGML_Q4_K || L.gg.tdn != MOE_GGML_Q4_K || (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K)) {
+    // Q5_K gate/up, Q5_1 / Q8_0 down (or such a shared expert): the general kernels
+    for (int phase = 1; phase <= 2; phase++) {
+      if ((rc = moe_launch_ggx_gemv(phase, L.gg.tgu, L.gg.tdn, L.sh_gguf_type, L.gg.gate, L.gg.up, L.gg.down,
+                                    L.has_shared ? L.sh_gate.data : nullptr, L.has_shared ? L.sh_up.data : nullptr,
+                                    L.has_shared ? L.sh_down.data : nullptr, c->sh_logit, x, c->ids, c->ws, c->hid32,
+                                    y, P, g.d, g.mid, g.topk, g.id_stride, st)))
+        return rc;
+      prof_mark(c, phase == 1 ? MOE_PROF_UP : MOE_PROF_DOWN, st);
+    }
+    return MOE_OK;
+  }
   if (use_int4k) {
     rc = gu_topk ? moe_launch_dec4k_gu_topk(L.gg.gate, L.gg.up, L.has_shared ? L.sh_gate.data : nullptr,
                                             L.has_shared ? L.sh_up.data : nullptr, c->xplanes, c->xmeta, c->logits,
@@ -504,7 +518,10 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
 // Returns MOE_E_UNSUPPORTED (before enqueuing anything) for shapes / formats the GEMM does not cover.
 static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
   const moe_config& g = c->cfg;
-  const bool q4k = L.has_gguf;  // raw GGUF Q4_K blocks (moe_set_experts_gguf admits nothing else)
+  const bool q4k = L.has_gguf;  // raw GGUF blocks: the grouped GEMM reads Q4_K only
+  if (q4k && (L.gg.tgu != MOE_GGML_Q4_K || L.gg.tdn != MOE_GGML_Q4_K ||
+              (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K)))
+    return MOE_E_UNSUPPORTED;  // the caller walks the batch through the small path
   if (L.has_shared && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format per launch
   if (q4k ? (g.d % 256 || g.mid % 256) : (g.d % 128 || g.mid % 128)) return MOE_E_UNSUPPORTED;
   moe_lutw gu{}, dn{}, sgu{}, sdn{};

@@ -3,6 +3,7 @@
 //   d*(s0*sum(q_lo*x_lo) + s1*sum(q_hi*x_hi)) - dmin*(m0*sum(x_lo) + m1*sum(x_hi))
 // (reference: src/gpu/parts/26_kernels_moe_gguf.inc:527-568,693-756,893-939; src/gguf.h:408-441)
 #include "common.h"
+#include "internal.h"
 
 namespace {
 
@@ -233,7 +234,10 @@ int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const
 MOE_API int moe_gg_gemv(int tgu, int tdn, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
                         const float* x, const int* ids, const float* ws, float* hid, float* out, int P,
                         int d, int mid, int kpt, int id_stride, moe_stream_t st) {
-  if (tgu != MOE_GGML_Q4_K || tdn != MOE_GGML_Q4_K) return MOE_E_UNSUPPORTED;
+  if (!moe_gg_types_supported(tgu, tdn, d, mid)) return MOE_E_UNSUPPORTED;
+  if (tgu != MOE_GGML_Q4_K || tdn != MOE_GGML_Q4_K)  // Q5_K gate/up, Q5_1 / Q8_0 down: the general kernels
+    return moe_launch_ggx_gemv(0, tgu, tdn, 0, gate, up, down, nullptr, nullptr, nullptr, nullptr, x, ids, ws, hid, out,
+                               P, d, mid, kpt, id_stride, moe_s(st));
   return moe_launch_q4k_gemv(0, gate, up, down, nullptr, nullptr, nullptr, nullptr, x, ids, ws, hid, out, P, d,
                              mid, kpt, id_stride, moe_s(st));
 }

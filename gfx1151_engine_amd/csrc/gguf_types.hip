@@ -1,0 +1,239 @@
+// The further ggml block types of GGUF expert tensors, read in place: Q5_K (gate/up), Q5_1 and Q8_0 (down)
+// next to Q4_K — the mix of the reference's GGUF checkpoints (src/gpu/parts/30_host_util.inc:399-405,
+// src/gpu/parts/26_kernels_moe_gguf.inc:32-48).  Dequantisation (bit-exact with gguf::dequant_row,
+// src/gguf.h:339-445) and plain f32 GEMV kernels for any mix of the four types: one wave per weight row,
+// one lane per 32-element block.  These are the general kernels; Q4_K alone has the tuned ones
+// (gemv_q4k.hip, decode_q4k.hip, the Q4_K instantiation of the grouped GEMM).
+#include "common.h"
+#include "internal.h"
+
+namespace {
+
+__device__ __host__ __forceinline__ uint64_t gg_row_bytes(int t, uint64_t k) {
+  switch (t) {
+    case MOE_GGML_Q4_K: return k / 256 * 144;
+    case MOE_GGML_Q5_K: return k / 256 * 176;
+    case MOE_GGML_Q8_0: return k / 32 * 34;
+    case MOE_GGML_Q5_1: return k / 32 * 24;
+    default: return 0;
+  }
+}
+__host__ bool gg_type_ok(int t, int k) {
+  if (t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K) return k >= 256 && k % 256 == 0;
+  if (t == MOE_GGML_Q8_0 || t == MOE_GGML_Q5_1) return k >= 32 && k % 32 == 0;
+  return false;
+}
+
+__device__ __forceinline__ void k4_sm(int j, const uint8_t* q, int& sc, int& mn) {  // gguf.h:328-336
+  if (j < 4) {
+    sc = q[j] & 63;
+    mn = q[j + 4] & 63;
+  } else {
+    sc = (q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4);
+    mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+  }
+}
+__device__ __forceinline__ float h2f(const uint8_t* p) {
+  const uint16_t h = (uint16_t)(p[0] | (p[1] << 8));
+  return __half2float(__ushort_as_half(h));
+}
+
+// Block b (32 consecutive elements) of a row: the 32 integer codes q[] in element order and the two
+// constants of w = a*q + c (a, c and a*q are exact in f32: fp16 fields times integers of at most 8 bits).
+__device__ __forceinline__ void gg_block(int t, const uint8_t* row, int b, int (&q)[32], float& a, float& c) {
+  if (t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K) {
+    const bool k5 = t == MOE_GGML_Q5_K;
+    const uint8_t* sb = row + (size_t)(b >> 3) * (k5 ? 176 : 144);
+    const int j = b & 7;  // sub-block: pair j/2, low nibbles if j even
+    int sc, mn;
+    k4_sm(j, sb + 4, sc, mn);
+    a = h2f(sb) * (float)sc;
+    c = -(h2f(sb + 2) * (float)mn);
+    const uint8_t* ql = sb + (k5 ? 48 : 16) + 32 * (j >> 1);
+    const uint8_t* qh = sb + 16;
+#pragma unroll
+    for (int l = 0; l < 32; l++) {
+      int v = (j & 1) ? ql[l] >> 4 : ql[l] & 0xF;
+      if (k5) v += ((qh[l] >> j) & 1) << 4;
+      q[l] = v;
+    }
+  } else if (t == MOE_GGML_Q8_0) {
+    const uint8_t* p = row + (size_t)b * 34;
+    a = h2f(p);
+    c = 0.f;
+#pragma unroll
+    for (int l = 0; l < 32; l++) q[l] = (int)(int8_t)p[2 + l];
+  } else {  // Q5_1
+    const uint8_t* p = row + (size_t)b * 24;
+    a = h2f(p);
+    c = h2f(p + 2);
+    const uint32_t qh = (uint32_t)p[4] | ((uint32_t)p[5] << 8) | ((uint32_t)p[6] << 16) | ((uint32_t)p[7] << 24);
+#pragma unroll
+    for (int l = 0; l < 16; l++) {
+      q[l] = (p[8 + l] & 0xF) | (((qh >> l) & 1) << 4);
+      q[l + 16] = (p[8 + l] >> 4) | (((qh >> (l + 16)) & 1) << 4);
+    }
+  }
+}
+
+// one thread per 32-element block
+__global__ void __launch_bounds__(256) k_gg_dequant(int t, const uint8_t* __restrict__ raw, uint64_t cols,
+                                                    uint64_t nblocks, float* __restrict__ out) {
+  const uint64_t bpr = cols / 32, rbytes = gg_row_bytes(t, cols);
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nblocks; i += (uint64_t)gridDim.x * blockDim.x) {
+    const uint64_t r = i / bpr;
+    const int b = (int)(i % bpr);
+    int q[32];
+    float a, c;
+    gg_block(t, raw + r * rbytes, b, q, a, c);
+    float* y = out + r * cols + (uint64_t)b * 32;
+#pragma unroll
+    for (int l = 0; l < 32; l++) {
+      const float prod = __fmul_rn(a, (float)q[l]);  // exact
+      y[l] = t == MOE_GGML_Q8_0 ? prod : __fadd_rn(prod, c);  // Q8_0 has no constant term (keeps -0.0); else one rounded add
+    }
+  }
+}
+
+__device__ __forceinline__ float wave_sum_f(float v) {
+#pragma unroll
+  for (int o = 32; o; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// dot product of one row with x (K floats in LDS): lanes take the 32-element blocks in turn
+__device__ __forceinline__ float gg_row_dot(int t, const uint8_t* row, const float* x, int K, int lane) {
+  float acc = 0.f;
+  for (int b = lane; b < K / 32; b += 64) {
+    int q[32];
+    float a, c;
+    gg_block(t, row, b, q, a, c);
+    const float* xb = x + 32 * b;
+    float sq = 0.f, sx = 0.f;
+#pragma unroll
+    for (int l = 0; l < 32; l++) {
+      const float xv = xb[l];
+      sq = fmaf((float)q[l], xv, sq);
+      sx += xv;
+    }
+    acc += a * sq + c * sx;
+  }
+  return wave_sum_f(acc);
+}
+
+struct GgxArgs {
+  const uint8_t *gate, *up, *down;           // routed experts [E][rows][row bytes]
+  const uint8_t *sh_gate, *sh_up, *sh_down;  // optional shared expert (raw rows of type tsh)
+  int tgu, tdn, tsh;
+  const float* sh_logit;
+};
+
+constexpr int GX_ROWS = 16;
+// grid (ceil(mid/GX_ROWS), slots incl. shared, P), block 256: hid[token][slot][row] = silu(gate.x) * (up.x)
+__global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restrict__ x, const int* __restrict__ ids,
+                                                int id_stride, int kpt, int d, int mid, float* __restrict__ hid) {
+  extern __shared__ float xs[];
+  const int s = blockIdx.y, tok = blockIdx.z;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) xs[i] = x[(size_t)tok * d + i];
+  __syncthreads();
+  const bool shared = s >= kpt;
+  const int t = shared ? A.tsh : A.tgu;
+  const uint64_t rb = gg_row_bytes(t, d);
+  const uint64_t e = shared ? 0 : (uint64_t)ids[(size_t)tok * id_stride + s];
+  const uint8_t* gbase = shared ? A.sh_gate : A.gate + e * mid * rb;
+  const uint8_t* ubase = shared ? A.sh_up : A.up + e * mid * rb;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  float* ho = hid + ((size_t)tok * gridDim.y + s) * mid;
+  for (int rr = wv; rr < GX_ROWS; rr += 4) {
+    const int r = blockIdx.x * GX_ROWS + rr;
+    if (r >= mid) break;  // wave-uniform
+    const float g = gg_row_dot(t, gbase + (uint64_t)r * rb, xs, d, lane);
+    const float u = gg_row_dot(t, ubase + (uint64_t)r * rb, xs, d, lane);
+    if (lane == 0) ho[r] = silu_f(g) * u;
+  }
+}
+
+// grid (ceil(d/GX_ROWS), P), block 256: y[token][row] = sum over slots (selection order) of w_s * (down_s . hid_s)
+// + sigmoid(shared gate logit) * (shared down . hid_shared)
+__global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restrict__ hid, const int* __restrict__ ids,
+                                                const float* __restrict__ ws, int id_stride, int kpt, int d, int mid,
+                                                float* __restrict__ out) {
+  extern __shared__ float hs[];  // [slot][mid]
+  __shared__ int eid[17];
+  __shared__ float wgt[17];
+  const int tok = blockIdx.y;
+  const bool has_shared = A.sh_down != nullptr;
+  const int nslots = kpt + (has_shared ? 1 : 0);
+  for (int i = threadIdx.x; i < nslots * mid; i += blockDim.x) hs[i] = hid[(size_t)tok * nslots * mid + i];
+  if ((int)threadIdx.x < nslots) {
+    const int s = threadIdx.x;
+    eid[s] = s < kpt ? ids[(size_t)tok * id_stride + s] : 0;
+    wgt[s] = s < kpt ? ws[(size_t)tok * id_stride + s] : sigmoid_f(A.sh_logit[tok]);
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  for (int rr = wv; rr < GX_ROWS; rr += 4) {
+    const int r = blockIdx.x * GX_ROWS + rr;
+    if (r >= d) break;
+    float y = 0.f;
+    for (int s = 0; s < nslots; s++) {
+      const bool sh = has_shared && s == nslots - 1;
+      const int t = sh ? A.tsh : A.tdn;
+      const uint64_t rb = gg_row_bytes(t, mid);
+      const uint8_t* row = sh ? A.sh_down + (uint64_t)r * rb : A.down + ((uint64_t)eid[s] * d + r) * rb;
+      y += wgt[s] * gg_row_dot(t, row, hs + (size_t)s * mid, mid, lane);
+    }
+    if (lane == 0) out[(size_t)tok * d + r] = y;
+  }
+}
+
+}  // namespace
+
+bool moe_gg_types_supported(int tgu, int tdn, int d, int mid) { return gg_type_ok(tgu, d) && gg_type_ok(tdn, mid); }
+uint64_t moe_gg_row_bytes(int type, uint64_t k) { return gg_row_bytes(type, k); }
+
+MOE_API int moe_gg_dequant_rows(int type, const uint8_t* raw, uint64_t nrows, uint64_t cols, float* out,
+                                moe_stream_t st) {
+  if (!raw || (!out && nrows)) return MOE_E_INVALID;
+  if (cols == 0 || cols > (1ull << 31)) return MOE_E_INVALID;
+  if (!gg_type_ok(type, (int)cols)) return MOE_E_UNSUPPORTED;
+  if (nrows == 0) return MOE_OK;
+  const uint64_t nblocks = nrows * (cols / 32);
+  const unsigned grid = (unsigned)((nblocks + 255) / 256 > 65535 * 16 ? 65535 * 16 : (nblocks + 255) / 256);
+  k_gg_dequant<<<grid, 256, 0, moe_s(st)>>>(type, raw, cols, nblocks, out);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// Internal launcher (shared with the context); shared-expert pointers may be null, tsh is their ggml type.
+// phase: 0 = gate/up + down, 1 = gate/up only, 2 = down only.
+int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gate, const uint8_t* up,
+                        const uint8_t* down, const uint8_t* sh_gate, const uint8_t* sh_up, const uint8_t* sh_down,
+                        const float* sh_logit, const float* x, const int* ids, const float* ws, float* hid,
+                        float* out, int P, int d, int mid, int kpt, int id_stride, hipStream_t st) {
+  if (!gate || !up || !down || !x || !ids || !ws || !hid || !out) return MOE_E_INVALID;
+  if (P < 0 || kpt < 1 || id_stride < kpt) return MOE_E_INVALID;
+  if (!moe_gg_types_supported(tgu, tdn, d, mid)) return MOE_E_UNSUPPORTED;
+  const bool sh = sh_gate != nullptr;
+  if (sh && (!sh_up || !sh_down || !sh_logit)) return MOE_E_INVALID;
+  if (sh && !(gg_type_ok(tsh, d) && gg_type_ok(tsh, mid))) return MOE_E_UNSUPPORTED;
+  const int nslots = kpt + (sh ? 1 : 0);
+  if (nslots > 16 || (size_t)d * 4 > 60 * 1024 || (size_t)nslots * mid * 4 > 60 * 1024) return MOE_E_UNSUPPORTED;
+  if (P == 0) return MOE_OK;
+  GgxArgs A{};
+  A.gate = gate; A.up = up; A.down = down;
+  A.sh_gate = sh_gate; A.sh_up = sh_up; A.sh_down = sh_down;
+  A.tgu = tgu; A.tdn = tdn; A.tsh = tsh;
+  A.sh_logit = sh_logit;
+  if (phase != 2) {
+    dim3 grid((mid + GX_ROWS - 1) / GX_ROWS, nslots, P);
+    k_ggx_gu<<<grid, 256, (size_t)d * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
+    MOE_LAUNCH_CHECK();
+  }
+  if (phase != 1) {
+    dim3 grid((d + GX_ROWS - 1) / GX_ROWS, P);
+    k_ggx_dn<<<grid, 256, (size_t)nslots * mid * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
+    MOE_LAUNCH_CHECK();
+  }
+  return MOE_OK;
+}

@@ -96,3 +96,10 @@ int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float
                       const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
                       int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
                       hipStream_t st);
+// general GEMV kernels for any supported mix of ggml block types (gguf_types.hip)
+bool moe_gg_types_supported(int tgu, int tdn, int d, int mid);
+uint64_t moe_gg_row_bytes(int type, uint64_t k);
+int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gate, const uint8_t* up,
+                        const uint8_t* down, const uint8_t* sh_gate, const uint8_t* sh_up, const uint8_t* sh_down,
+                        const float* sh_logit, const float* x, const int* ids, const float* ws, float* hid,
+                        float* out, int P, int d, int mid, int kpt, int id_stride, hipStream_t st);

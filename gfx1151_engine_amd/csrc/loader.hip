@@ -499,15 +499,15 @@ int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights
   gg.tdn = dn->dtype;
   if (u->dtype != g_->dtype) return MOE_E_UNSUPPORTED;
   if ((rc = upload(w, *g_, st, &gg.gate)) || (rc = upload(w, *u, st, &gg.up)) || (rc = upload(w, *dn, st, &gg.down))) return rc;
-  if ((rc = moe_set_experts_gguf(ctx, cl, &gg))) return rc;  // MOE_E_UNSUPPORTED for types other than Q4_K
+  if ((rc = moe_set_experts_gguf(ctx, cl, &gg))) return rc;  // MOE_E_UNSUPPORTED for types outside Q4_K / Q5_K / Q5_1 / Q8_0
   const FTensor* sg = find(f, "blk.%d.ffn_gate_shexp.weight", fl);
   if (sg) {
     const FTensor* su = find(f, "blk.%d.ffn_up_shexp.weight", fl);
     const FTensor* sd = find(f, "blk.%d.ffn_down_shexp.weight", fl);
     const FTensor* sx = find(f, "blk.%d.ffn_gate_inp_shexp.weight", fl);
     if (!su || !sd || !sx) return MOE_E_STATE;
-    if (sg->dtype != MOE_GGML_Q4_K || su->dtype != MOE_GGML_Q4_K || sd->dtype != MOE_GGML_Q4_K ||
-        (sx->dtype != 0 && sx->dtype != 30))
+    // one ggml type for the three shared tensors (moe_set_shared checks that it is a supported one)
+    if (su->dtype != sg->dtype || sd->dtype != sg->dtype || (sx->dtype != 0 && sx->dtype != 30))
       return MOE_E_UNSUPPORTED;
     if (!is(*sg, D, M, 1) || !is(*su, D, M, 1) || !is(*sd, M, D, 1) || !is(*sx, D, 1, 1)) return MOE_E_INVALID;
     moe_wview a{}, b{}, c2{}, d2{};
@@ -520,7 +520,7 @@ int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights
     if ((rc = raw(*sg, &a)) || (rc = raw(*su, &b)) || (rc = raw(*sd, &c2)) || (rc = raw(*sx, &d2))) return rc;
     d2.dtype = sx->dtype == 0 ? MOE_DT_F32 : MOE_DT_BF16;
     d2.rows = 1;
-    if ((rc = moe_set_shared(ctx, cl, &a, &b, &c2, &d2, MOE_GGML_Q4_K))) return rc;
+    if ((rc = moe_set_shared(ctx, cl, &a, &b, &c2, &d2, sg->dtype))) return rc;
   }
   return MOE_OK;
 }

@@ -11,7 +11,7 @@ import numpy as np
 
 HGN_BF16, HGN_F32, HGN_Q4CP = 0, 1, 5
 GGML_F32, GGML_BF16, GGML_Q4_K = 0, 30, 12
-_GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144)}
+_GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24)}
 
 
 def _bytes(a):
@@ -99,15 +99,17 @@ def hgn_layer_tensors(l, hl):
 
 
 def gguf_layer_tensors(l, hl):
-    """The MoE tensors of layer l of a HostLayer-like object (fmt q4k) as GGUF tensor infos."""
+    """The MoE tensors of layer l of a HostLayer-like object (fmt q4k; ggml types hl.tgu / hl.tdn / hl.tsh where
+    it has them, else Q4_K) as GGUF tensor infos."""
     d, mid, E = hl.d, hl.mid, hl.E
+    tgu, tdn, tsh = (getattr(hl, a, GGML_Q4_K) for a in ("tgu", "tdn", "tsh"))
     t = [(f"blk.{l}.ffn_gate_inp.weight", GGML_F32, [d, E], hl.router),
-         (f"blk.{l}.ffn_gate_exps.weight", GGML_Q4_K, [d, mid, E], hl.gate),
-         (f"blk.{l}.ffn_up_exps.weight", GGML_Q4_K, [d, mid, E], hl.up),
-         (f"blk.{l}.ffn_down_exps.weight", GGML_Q4_K, [mid, d, E], hl.down)]
+         (f"blk.{l}.ffn_gate_exps.weight", tgu, [d, mid, E], hl.gate),
+         (f"blk.{l}.ffn_up_exps.weight", tgu, [d, mid, E], hl.up),
+         (f"blk.{l}.ffn_down_exps.weight", tdn, [mid, d, E], hl.down)]
     if hl.shared is not None:
-        t += [(f"blk.{l}.ffn_gate_shexp.weight", GGML_Q4_K, [d, mid], hl.shared[0]),
-              (f"blk.{l}.ffn_up_shexp.weight", GGML_Q4_K, [d, mid], hl.shared[1]),
-              (f"blk.{l}.ffn_down_shexp.weight", GGML_Q4_K, [mid, d], hl.shared[2]),
+        t += [(f"blk.{l}.ffn_gate_shexp.weight", tsh, [d, mid], hl.shared[0]),
+              (f"blk.{l}.ffn_up_shexp.weight", tsh, [d, mid], hl.shared[1]),
+              (f"blk.{l}.ffn_down_shexp.weight", tsh, [mid, d], hl.shared[2]),
               (f"blk.{l}.ffn_gate_inp_shexp.weight", GGML_F32, [d], hl.shared[3])]
     return t

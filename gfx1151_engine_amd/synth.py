@@ -68,6 +68,50 @@ def make_q4k(rng, rows, cols, scale_std=0.01):
     return blk.reshape(-1)
 
 
+def make_q5k(rng, rows, cols, scale_std=0.01):
+    """Random Q5_K rows (176-byte super-blocks: d, dmin, scales[12], qh[32], ql[128]; src/gguf.h:408-441)."""
+    assert cols % 256 == 0
+    nb = rows * cols // 256
+    blk = np.zeros((nb, 176), np.uint8)
+    dd = (np.abs(rng.standard_normal((nb, 2), dtype=np.float32)) * scale_std).astype(np.float16)
+    blk[:, 0:4] = dd.view(np.uint8)
+    sc = rng.integers(0, 64, (nb, 8), dtype=np.uint8)
+    mn = rng.integers(0, 64, (nb, 8), dtype=np.uint8)
+    blk[:, 4:16] = pack_scale_min_k4(sc, mn)
+    blk[:, 16:] = rng.integers(0, 256, (nb, 160), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+def make_q8_0(rng, rows, cols, scale_std=0.01):
+    """Random Q8_0 rows (34-byte blocks: d fp16, 32 x int8; src/gguf.h:352-359)."""
+    assert cols % 32 == 0
+    nb = rows * cols // 32
+    blk = np.zeros((nb, 34), np.uint8)
+    blk[:, 0:2] = (np.abs(rng.standard_normal((nb, 1), dtype=np.float32)) * scale_std / 8).astype(np.float16).view(np.uint8)
+    blk[:, 2:] = rng.integers(0, 256, (nb, 32), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+def make_q5_1(rng, rows, cols, scale_std=0.01):
+    """Random Q5_1 rows (24-byte blocks: d, m fp16, qh u32, qs[16]; src/gguf.h:360-375); m = -16 d so that
+    the 5-bit codes are centred like the other formats' weights."""
+    assert cols % 32 == 0
+    nb = rows * cols // 32
+    blk = np.zeros((nb, 24), np.uint8)
+    d = (np.abs(rng.standard_normal((nb, 1), dtype=np.float32)) * scale_std / 2).astype(np.float16)
+    blk[:, 0:2] = d.view(np.uint8)
+    blk[:, 2:4] = (d.astype(np.float32) * -16).astype(np.float16).view(np.uint8)
+    blk[:, 4:] = rng.integers(0, 256, (nb, 20), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+GG_Q4_K, GG_Q5_K, GG_Q5_1, GG_Q8_0 = 12, 13, 7, 8  # ggml type ids
+
+
+def make_gg(rng, t, rows, cols, scale_std=0.01):
+    return {GG_Q4_K: make_q4k, GG_Q5_K: make_q5k, GG_Q5_1: make_q5_1, GG_Q8_0: make_q8_0}[t](rng, rows, cols, scale_std)
+
+
 def f32_to_bf16_bits(a):
     """Round-to-nearest-even f32 -> bf16 bit patterns (uint16)."""
     u = np.ascontiguousarray(a, np.float32).view(np.uint32)

@@ -33,7 +33,9 @@ enum moe_status {
 
 /* hgn tensor dtypes (src/hgn.h:2-23) and ggml types (src/gguf.h:42-64) used on this path */
 enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5 };
-enum { MOE_GGML_Q4_K = 12 };
+/* Q4_K: every kernel of the path.  Q5_K (gate/up), Q5_1 and Q8_0 (down) — the mix of the reference's GGUF
+ * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — : dequantisation and the general GEMV kernels. */
+enum { MOE_GGML_Q5_1 = 7, MOE_GGML_Q8_0 = 8, MOE_GGML_Q4_K = 12, MOE_GGML_Q5_K = 13 };
 
 /* WView (src/gpu/parts/30_host_util.inc:772-780): a weight tensor as it lies in memory.
  * q4cp: data = [64 B codebook][rows*cols/2 codes][rows x scale_stride]. */
@@ -66,6 +68,10 @@ int moe_q4cp_dequant_rows(const uint8_t* blob, uint64_t rows, uint64_t cols, uin
 /* gguf::dequant_row, Q4_K branch (src/gguf.h:408-441) for nrows raw rows of `cols` elements. */
 int moe_q4k_dequant_rows(const uint8_t* raw, uint64_t nrows, uint64_t cols, float* out,
                          moe_stream_t st);
+/* gguf::dequant_row (src/gguf.h:339-445) for nrows raw rows of `cols` elements of ggml type
+ * MOE_GGML_Q4_K / Q5_K (cols % 256 == 0) / Q5_1 / Q8_0 (cols % 32 == 0); bit-exact. */
+int moe_gg_dequant_rows(int type, const uint8_t* raw, uint64_t nrows, uint64_t cols, float* out,
+                        moe_stream_t st);
 
 /* ---- router ---- */
 

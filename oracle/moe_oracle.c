@@ -10,7 +10,8 @@
  *   src/hgn.h:77-84      fp16 -> f32
  *   src/hgn.h:219-261    q4cp blob layout, q4cp_parse / q4cp_row
  *   src/gguf.h:328-336   scale_min_k4
- *   src/gguf.h:408-441   Q4_K dequant_row
+ *   src/gguf.h:408-441   Q4_K / Q5_K dequant_row
+ *   src/gguf.h:352-375   Q8_0 / Q5_1 dequant_row
  *   src/ref.cpp:55-56    sigmoid / silu
  *   src/ref.cpp:68-77    matvec: fp64 sequential accumulate, f32 result
  *   src/ref.cpp:563-637  Model::moe (router, top-k, experts, shared expert)
@@ -36,7 +37,7 @@
 #define ORC_API __attribute__((visibility("default")))
 
 /* ---- weight format tags (shared with the library header by value) ---- */
-enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12 };
+enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q5_1 = 7, ORC_Q8_0 = 8 };
 
 /* src/hgn.h:77-84 and src/gguf.h:318-325 (same function twice in the reference) */
 ORC_API float orc_fp16_to_f32(uint16_t h) {
@@ -127,9 +128,82 @@ ORC_API void orc_q4k_row(const uint8_t* src, float* y, uint64_t k) {
 }
 ORC_API uint64_t orc_q4k_row_bytes(uint64_t k) { return k / 256 * 144; } /* gguf.h:79-84 */
 
+/* src/gguf.h:408-441, Q5_K branch: 176-byte super-blocks {d, dmin, scales[12], qh[32], ql[128]}; bit 2j of
+ * qh[l] is the fifth bit of the low-nibble element l of pair j, bit 2j+1 that of the high-nibble element.
+ * (d*sc)*q with q <= 31 is still exact in f32 (11 + 6 + 5 bits): one rounded subtraction. */
+static void orc_q5k_row(const uint8_t* src, float* y, uint64_t k) {
+  for (uint64_t b = 0; b < k / 256; b++, src += 176) {
+    uint16_t dh, mh;
+    memcpy(&dh, src, 2);
+    memcpy(&mh, src + 2, 2);
+    const float d = orc_fp16_to_f32(dh), dmin = orc_fp16_to_f32(mh);
+    const uint8_t* sc = src + 4;
+    const uint8_t* qh = src + 16;
+    const uint8_t* ql = src + 48;
+    float* yy = y + b * 256;
+    for (int j = 0; j < 4; j++) {
+      uint8_t s0, m0, s1, m1;
+      orc_scale_min_k4(2 * j, sc, &s0, &m0);
+      orc_scale_min_k4(2 * j + 1, sc, &s1, &m1);
+      const float d1 = d * s0, dm1 = dmin * m0, d2 = d * s1, dm2 = dmin * m1;
+      for (int l = 0; l < 32; l++) *yy++ = d1 * (float)((ql[l] & 0xF) + (((qh[l] >> (2 * j)) & 1) << 4)) - dm1;
+      for (int l = 0; l < 32; l++) *yy++ = d2 * (float)((ql[l] >> 4) + (((qh[l] >> (2 * j + 1)) & 1) << 4)) - dm2;
+      ql += 32;
+    }
+  }
+}
+/* src/gguf.h:352-359: 34-byte blocks {d fp16, 32 x int8}; d*q is exact (11 + 8 bits) */
+static void orc_q8_0_row(const uint8_t* src, float* y, uint64_t k) {
+  for (uint64_t b = 0; b < k / 32; b++, src += 34) {
+    uint16_t dh;
+    memcpy(&dh, src, 2);
+    const float d = orc_fp16_to_f32(dh);
+    for (int j = 0; j < 32; j++) y[b * 32 + j] = d * (float)(int8_t)src[2 + j];
+  }
+}
+/* src/gguf.h:360-375: 24-byte blocks {d, m fp16, qh u32, qs[16]}; element j = low nibble of qs[j] + bit j of
+ * qh, element j + 16 = high nibble + bit j + 16; x*d is exact (5 + 11 bits), so x*d + m is one rounded add
+ * with or without contraction. */
+static void orc_q5_1_row(const uint8_t* src, float* y, uint64_t k) {
+  for (uint64_t b = 0; b < k / 32; b++, src += 24) {
+    uint16_t dh, mh;
+    uint32_t qh;
+    memcpy(&dh, src, 2);
+    memcpy(&mh, src + 2, 2);
+    memcpy(&qh, src + 4, 4);
+    const float d = orc_fp16_to_f32(dh), mn = orc_fp16_to_f32(mh);
+    const uint8_t* qs = src + 8;
+    for (int j = 0; j < 16; j++) {
+      const int x0 = (qs[j] & 0xF) | (((qh >> j) & 1) << 4);
+      const int x1 = (qs[j] >> 4) | (((qh >> (j + 16)) & 1) << 4);
+      y[b * 32 + j] = (float)x0 * d + mn;
+      y[b * 32 + j + 16] = (float)x1 * d + mn;
+    }
+  }
+}
+/* src/gguf.h:42-84: bytes of one row of k elements */
+ORC_API uint64_t orc_gg_row_bytes(int type, uint64_t k) {
+  switch (type) {
+    case ORC_Q4K: return k / 256 * 144;
+    case ORC_Q5K: return k / 256 * 176;
+    case ORC_Q8_0: return k / 32 * 34;
+    case ORC_Q5_1: return k / 32 * 24;
+    default: return 0;
+  }
+}
+ORC_API int orc_gg_row(int type, const uint8_t* src, float* y, uint64_t k) {
+  switch (type) {
+    case ORC_Q4K: orc_q4k_row(src, y, k); return 0;
+    case ORC_Q5K: orc_q5k_row(src, y, k); return 0;
+    case ORC_Q8_0: orc_q8_0_row(src, y, k); return 0;
+    case ORC_Q5_1: orc_q5_1_row(src, y, k); return 0;
+    default: return -1;
+  }
+}
+
 /* ---- generic "row r of a weight matrix" in any supported storage ---- */
 typedef struct {
-  int dtype;            /* ORC_F32 / ORC_BF16 / ORC_Q4CP / ORC_Q4K */
+  int dtype;            /* ORC_F32 / ORC_BF16 / ORC_Q4CP / ORC_Q4K / ORC_Q5K / ORC_Q8_0 / ORC_Q5_1 */
   const uint8_t* data;  /* f32/bf16: row-major; q4cp: whole blob; q4k: row-major raw blocks */
   uint64_t rows, cols;  /* logical matrix (q4cp: rows of the whole blob) */
 } orc_mat;
@@ -144,6 +218,9 @@ static void mat_row(const orc_mat* W, uint64_t r, float* out) {
     }
     case ORC_Q4CP: orc_q4cp_row(W->data, W->rows, W->cols, r, out); break;
     case ORC_Q4K: orc_q4k_row(W->data + r * orc_q4k_row_bytes(W->cols), out, W->cols); break;
+    case ORC_Q5K: case ORC_Q8_0: case ORC_Q5_1:
+      orc_gg_row(W->dtype, W->data + r * orc_gg_row_bytes(W->dtype, W->cols), out, W->cols);
+      break;
     default: memset(out, 0, W->cols * 4);
   }
 }

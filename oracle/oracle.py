@@ -11,6 +11,8 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 F32, BF16, Q4CP, Q4K = 1, 0, 5, 12
+Q5K, Q5_1, Q8_0 = 13, 7, 8          # further ggml block types of the expert tensors (ids as in GGUF)
+GG_TYPES = (Q4K, Q5K, Q5_1, Q8_0)
 
 
 def build(force=False):
@@ -51,6 +53,8 @@ def lib():
         _lib.orc_q4k_row_bytes.restype = C.c_uint64
         _lib.orc_q4k_row_bytes.argtypes = [C.c_uint64]
         _lib.orc_num_threads.restype = C.c_int
+        _lib.orc_gg_row_bytes.restype = C.c_uint64
+        _lib.orc_gg_row_bytes.argtypes = [C.c_int, C.c_uint64]
     return _lib
 
 
@@ -66,6 +70,8 @@ def ref():
         _ref.ref_fp16_to_f32.argtypes = [C.c_uint16]
         _ref.ref_q4k_row_bytes.restype = C.c_uint64
         _ref.ref_q4k_row_bytes.argtypes = [C.c_uint64]
+        _ref.ref_gg_row_bytes.restype = C.c_uint64
+        _ref.ref_gg_row_bytes.argtypes = [C.c_uint32, C.c_uint64]
     return _ref
 
 
@@ -88,6 +94,8 @@ class Mat:
             assert self.data.dtype == np.uint8 and self.data.size == lib().orc_q4cp_blob_bytes(rows, cols)
         elif dtype == Q4K:
             assert self.data.dtype == np.uint8 and self.data.size == rows * lib().orc_q4k_row_bytes(cols)
+        elif dtype in GG_TYPES:
+            assert self.data.dtype == np.uint8 and self.data.size == rows * lib().orc_gg_row_bytes(dtype, cols)
         elif dtype == F32:
             assert self.data.dtype == np.float32 and self.data.size == rows * cols
         elif dtype == BF16:
@@ -103,6 +111,9 @@ class Mat:
         if self.dtype == Q4K:
             rb = lib().orc_q4k_row_bytes(self.cols)
             return q4k_rows(self.data[row0 * rb:(row0 + nrows) * rb], nrows, self.cols)
+        if self.dtype in GG_TYPES:
+            rb = lib().orc_gg_row_bytes(self.dtype, self.cols)
+            return gg_rows(self.dtype, self.data[row0 * rb:(row0 + nrows) * rb], nrows, self.cols)
         if self.dtype == F32:
             return self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].copy()
         u = self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].astype(np.uint32) << 16
@@ -121,6 +132,36 @@ def q4cp_rows(blob, rows, cols, row0, nrows):
     out = np.empty((nrows, cols), np.float32)
     lib().orc_q4cp_rows(_p(blob), C.c_uint64(rows), C.c_uint64(cols), C.c_uint64(row0),
                         C.c_uint64(nrows), _p(out))
+    return out
+
+
+def gg_row_bytes(t, k):
+    return int(lib().orc_gg_row_bytes(int(t), C.c_uint64(k)))
+
+
+def gg_rows(t, raw, nrows, k):
+    """Dequantised rows of a ggml block type (Q4_K, Q5_K, Q5_1, Q8_0), src/gguf.h:339-445."""
+    raw = _c(raw, np.uint8)
+    rb = gg_row_bytes(t, k)
+    assert rb and raw.size == nrows * rb
+    out = np.empty((nrows, k), np.float32)
+    for r in range(nrows):
+        rc = lib().orc_gg_row(int(t), C.c_void_p(raw.ctypes.data + r * rb), C.c_void_p(out.ctypes.data + r * k * 4),
+                              C.c_uint64(k))
+        assert rc == 0
+    return out
+
+
+def ref_gg_rows(t, raw, nrows, k):
+    """The same through the reference's own gguf::dequant_row (oracle/_ref)."""
+    raw = _c(raw, np.uint8)
+    rb = int(ref().ref_gg_row_bytes(C.c_uint32(t), C.c_uint64(k)))
+    assert raw.size == nrows * rb
+    out = np.empty((nrows, k), np.float32)
+    for r in range(nrows):
+        rc = ref().ref_gg_row(C.c_uint32(t), C.c_void_p(raw.ctypes.data + r * rb),
+                              C.c_void_p(out.ctypes.data + r * k * 4), C.c_uint64(k))
+        assert rc == 0
     return out
 
 

@@ -71,6 +71,18 @@ __attribute__((visibility("default"))) int ref_q4k_row(const uint8_t* src, float
     return -1;
   }
 }
+// gguf::dequant_row / gguf::row_bytes for any ggml type id
+__attribute__((visibility("default"))) int ref_gg_row(uint32_t type, const uint8_t* src, float* y, uint64_t k) {
+  try {
+    gguf::dequant_row(type, src, y, k);
+    return 0;
+  } catch (...) {
+    return -1;
+  }
+}
+__attribute__((visibility("default"))) uint64_t ref_gg_row_bytes(uint32_t type, uint64_t k) {
+  return gguf::row_bytes(type, k);
+}
 __attribute__((visibility("default"))) uint64_t ref_q4k_row_bytes(uint64_t k) {
   return gguf::row_bytes(gguf::Q4_K, k);
 }

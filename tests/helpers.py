@@ -19,8 +19,10 @@ class HostLayer:
     """One synthetic MoE layer as host bytes (the 'file' side)."""
 
     def __init__(self, rng, d, mid, E, k, fmt="q4cp", router_dtype="f32", codebook=None, scale_std=0.01,
-                 router_std=0.02, shared=True, bias=None):
+                 router_std=0.02, shared=True, bias=None, gg_types=(12, 12, 12)):
+        """fmt "q4k": raw GGUF blocks; gg_types = ggml types of (gate/up, down, shared expert)."""
         self.d, self.mid, self.E, self.k, self.fmt = d, mid, E, k, fmt
+        self.tgu, self.tdn, self.tsh = gg_types
         rw = (rng.standard_normal((E, d), dtype=np.float32) * router_std)
         if router_dtype == "bf16":
             self.router = S.f32_to_bf16_bits(rw)
@@ -33,13 +35,13 @@ class HostLayer:
             self.gate_up = S.make_q4cp(rng, E * 2 * mid, d, codebook=codebook, scale_std=scale_std)
             self.down = S.make_q4cp(rng, E * d, mid, codebook=codebook, scale_std=scale_std)
         else:
-            self.gate = S.make_q4k(rng, E * mid, d, scale_std=scale_std)
-            self.up = S.make_q4k(rng, E * mid, d, scale_std=scale_std)
-            self.down = S.make_q4k(rng, E * d, mid, scale_std=scale_std)
+            self.gate = S.make_gg(rng, self.tgu, E * mid, d, scale_std=scale_std)
+            self.up = S.make_gg(rng, self.tgu, E * mid, d, scale_std=scale_std)
+            self.down = S.make_gg(rng, self.tdn, E * d, mid, scale_std=scale_std)
         self.shared = None
         if shared:
             mk = (lambda r, c: S.make_q4cp(rng, r, c, codebook=codebook, scale_std=scale_std)) if fmt == "q4cp" \
-                else (lambda r, c: S.make_q4k(rng, r, c, scale_std=scale_std))
+                else (lambda r, c: S.make_gg(rng, self.tsh, r, c, scale_std=scale_std))
             self.shared = [mk(mid, d), mk(mid, d), mk(d, mid),
                            rng.standard_normal((1, d), dtype=np.float32) * router_std]
 
@@ -48,14 +50,15 @@ class HostLayer:
         wt = O.Q4CP if self.fmt == "q4cp" else O.Q4K
         sh = None
         if self.shared is not None:
-            sh = [O.Mat(wt, self.shared[0], mid, d), O.Mat(wt, self.shared[1], mid, d),
-                  O.Mat(wt, self.shared[2], d, mid), O.Mat(O.F32, self.shared[3], 1, d)]
+            st = O.Q4CP if self.fmt == "q4cp" else self.tsh
+            sh = [O.Mat(st, self.shared[0], mid, d), O.Mat(st, self.shared[1], mid, d),
+                  O.Mat(st, self.shared[2], d, mid), O.Mat(O.F32, self.shared[3], 1, d)]
         router = O.Mat(self.router_dt, self.router, E, d)
         if self.fmt == "q4cp":
             return O.Layer(d, mid, E, k, router, O.Mat(wt, self.down, E * d, mid),
                            gate_up=O.Mat(wt, self.gate_up, E * 2 * mid, d), shared=sh, router_bias=self.bias)
-        return O.Layer(d, mid, E, k, router, O.Mat(wt, self.down, E * d, mid),
-                       gate=O.Mat(wt, self.gate, E * mid, d), up=O.Mat(wt, self.up, E * mid, d), shared=sh,
+        return O.Layer(d, mid, E, k, router, O.Mat(self.tdn, self.down, E * d, mid),
+                       gate=O.Mat(self.tgu, self.gate, E * mid, d), up=O.Mat(self.tgu, self.up, E * mid, d), shared=sh,
                        router_bias=self.bias)
 
     def to_gpu(self, max_tokens=32):
@@ -77,12 +80,12 @@ class HostLayer:
             m.set_experts_q4cp(0, capi.wview(up("gate_up", self.gate_up), capi.Q4CP, E * 2 * mid, d),
                                capi.wview(up("down", self.down), capi.Q4CP, E * d, mid))
         else:
-            m.set_experts_gguf(0, up("gate", self.gate), up("up", self.up), up("down", self.down))
+            m.set_experts_gguf(0, up("gate", self.gate), up("up", self.up), up("down", self.down), self.tgu, self.tdn)
         if self.shared is not None:
             wt = capi.Q4CP if self.fmt == "q4cp" else 0
             m.set_shared(0, capi.wview(up("shg", self.shared[0]), wt, mid, d),
                          capi.wview(up("shu", self.shared[1]), wt, mid, d),
                          capi.wview(up("shd", self.shared[2]), wt, d, mid),
                          capi.wview(up("shsg", self.shared[3]), capi.F32, 1, d),
-                         0 if self.fmt == "q4cp" else capi.GGML_Q4_K)
+                         0 if self.fmt == "q4cp" else self.tsh)
         return m, dev

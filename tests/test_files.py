@@ -166,14 +166,14 @@ def test_layers_loaded_from_file_equal_direct_registration(tmp_path, fmt):
 
 @pytest.mark.gpu
 def test_load_rejects_types_outside_the_path(tmp_path):
-    # a GGUF whose experts are Q8_0: moe_load_layers reports unsupported and leaves no layer registered
+    # a GGUF whose experts are Q6_K: moe_load_layers reports unsupported and leaves no layer registered
     import torch
     rng = np.random.default_rng(1)
     ts = [("blk.0.ffn_gate_inp.weight", files.GGML_F32, [D, E], rng.standard_normal((E, D), dtype=np.float32))]
-    files._GGML_BLOCK[8] = (32, 34)
+    files._GGML_BLOCK[14] = (256, 210)
     for n, ne in (("gate", [D, MID, E]), ("up", [D, MID, E]), ("down", [MID, D, E])):
-        ts.append((f"blk.0.ffn_{n}_exps.weight", 8, ne, np.zeros(int(np.prod(ne)) // 32 * 34, np.uint8)))
-    p = tmp_path / "q8.gguf"
+        ts.append((f"blk.0.ffn_{n}_exps.weight", 14, ne, np.zeros(int(np.prod(ne)) // 256 * 210, np.uint8)))
+    p = tmp_path / "q6.gguf"
     files.write_gguf(p, ts, kv={"general.architecture": "x"})
     f = capi.ModelFile(p)
     m = capi.Moe(D, MID, E, K, layers=1, max_tokens=8)
@@ -244,3 +244,31 @@ def test_large_tensor_takes_the_staged_copy_and_arrives_intact(tmp_path):
     del m, direct, keep
     w.free()
 
+
+@pytest.mark.gpu
+def test_load_gguf_mixed_types(tmp_path):
+    """A GGUF layer in the reference checkpoints' type mix (Q5_K gate/up, Q8_0 down, Q4_K shared expert):
+    loaded from the file it gives the same output, bit for bit, as the same bytes registered directly, and
+    stays within the GEMV bar of the oracle."""
+    import torch
+    from helpers import HostLayer, max_abs_rel
+    rng = np.random.default_rng(23)
+    d, mid, E, k = 512, 256, 8, 3
+    hl = HostLayer(rng, d, mid, E, k, fmt="q4k", gg_types=(13, 8, 12))
+    ts = files.gguf_layer_tensors(0, hl)
+    p = tmp_path / "mixed.gguf"
+    files.write_gguf(p, ts, kv={"general.architecture": "x"})
+    f = capi.ModelFile(p)
+    m = capi.Moe(d, mid, E, k, layers=1, max_tokens=8)
+    w = f.load_layers(m, 0, 0, 1)
+    x = rng.standard_normal((5, d), dtype=np.float32)
+    xt = torch.from_numpy(x).cuda()
+    y = m.forward(0, xt).cpu().numpy()
+    m2, dev = hl.to_gpu(max_tokens=8)
+    y2 = m2.forward(0, xt).cpu().numpy()
+    assert (y == y2).all()
+    yo, io, wo = O.moe_layer(hl.oracle_layer(), x)
+    assert max_abs_rel(y, yo) <= 1e-4
+    m.close()
+    m2.close()
+    w.free()

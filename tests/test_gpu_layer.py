@@ -120,6 +120,25 @@ def test_decode_topk_near_ties(oracle, fmt, T):
     m.close()
 
 
+@pytest.mark.parametrize("tgu,tdn,tsh,T", [(13, 8, 12, 1), (12, 7, 12, 5), (13, 7, 8, 3), (12, 8, 13, 40)])
+def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
+    """GGUF layers in the type mix of the reference's checkpoints (Q4_K / Q5_K gate and up, Q5_1 / Q8_0 down,
+    src/gpu/parts/30_host_util.inc:399-405): the general f32 GEMV kernels, ids bit-exact, output within the GEMV
+    bar; T = 40 walks a batch the grouped GEMM cannot take through the small path 32 rows at a time."""
+    rng = np.random.default_rng(tgu * 100 + tdn * 10 + T)
+    d, mid, E, k = 512, 256, 12, 4
+    hl = HostLayer(rng, d, mid, E, k, fmt="q4k", gg_types=(tgu, tdn, tsh))
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=64)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    ids, _ = m.last_routing(min(T, 32))
+    if T <= 32:
+        assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    assert max_abs_rel(y, yo) <= TOL_GEMV, max_abs_rel(y, yo)
+    m.close()
+
+
 @pytest.mark.parametrize("share", [0.3, 1.0])
 def test_unique_expert_path(oracle, share):
     """MOE_OPT_UNIQUE_MIN_TOKENS: a verify-size batch through the expert-sorted pair lists (every distinct

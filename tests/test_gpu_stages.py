@@ -72,6 +72,22 @@ def test_q4k_all_scale_min_codes(capi, oracle):
     assert same_bits(capi.q4k_dequant_rows(gpu(raw), n, 256).cpu().numpy(), oracle.q4k_rows(raw, n, 256))
 
 
+@pytest.mark.parametrize("t,cols", [(13, 768), (8, 96), (7, 96), (8, 3072), (7, 768), (12, 512)])
+def test_gg_dequant_other_types(capi, oracle, t, cols):
+    """Q5_K / Q8_0 / Q5_1 (and Q4_K through the same entry point): bit-exact with the oracle's rows, which the
+    CPU tests pin against the reference's gguf::dequant_row; random bytes in the integer fields, so every code
+    value occurs."""
+    rng = np.random.default_rng(t * 1000 + cols)
+    rows = 37
+    raw = S.make_gg(rng, t, rows, cols)
+    got = capi.gg_dequant_rows(t, gpu(raw), rows, cols).cpu().numpy()
+    assert same_bits(got, oracle.gg_rows(t, raw, rows, cols))
+    with pytest.raises(capi.MoeError):
+        capi.gg_dequant_rows(t, gpu(raw), 1, 48)  # not a whole number of blocks
+    with pytest.raises(capi.MoeError):
+        capi.gg_dequant_rows(14, gpu(raw), 1, 256)  # Q6_K: outside the path
+
+
 # ---------- router: bit-exact ----------
 @pytest.mark.parametrize("P,E,d,k,dt,mode", [
     (1, 512, 3072, 10, "f32", 0), (20, 512, 3072, 10, "f32", 0), (20, 512, 3072, 10, "f32", 1),

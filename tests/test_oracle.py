@@ -297,3 +297,36 @@ def test_layer_matches_float64_numpy_q4k(oracle):
         ey = shd @ (g / (1 + np.exp(-g)) * u)
         want = acc + ey / (1 + np.exp(-(sg @ xt)))
         assert np.abs(y[t] - want).max() <= 2e-5 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("t,name", [(13, "Q5_K"), (8, "Q8_0"), (7, "Q5_1"), (12, "Q4_K")])
+def test_gg_rows_against_reference(oracle, t, name):
+    """The further ggml block types of the expert tensors: the oracle's rows against the reference's own
+    gguf::dequant_row (oracle/_ref) on random block bytes, bit for bit, and against a numpy evaluation of the
+    published block layout for one type with every code value present (Q8_0: d * int8)."""
+    O = oracle
+    rng = np.random.default_rng(t)
+    rows, cols = 5, 768
+    raw = S.make_gg(rng, t, rows, cols)
+    got = O.gg_rows(t, raw, rows, cols)
+    assert np.isfinite(got).all()
+    if O.ref() is not None:
+        assert O.gg_row_bytes(t, cols) == int(O.ref().ref_gg_row_bytes(t, cols))
+        want = O.ref_gg_rows(t, raw, rows, cols)
+        assert (got.view(np.uint32) == want.view(np.uint32)).all(), name
+    if t == 8:
+        blk = raw.reshape(-1, 34)
+        d = blk[:, :2].copy().view(np.float16).astype(np.float32)
+        q = blk[:, 2:].copy().view(np.int8).astype(np.float32)
+        assert ((d * q).reshape(rows, cols).view(np.uint32) == got.view(np.uint32)).all()
+    if t == 7:
+        blk = raw.reshape(-1, 24)
+        d = blk[:, :2].copy().view(np.float16).astype(np.float32)
+        m = blk[:, 2:4].copy().view(np.float16).astype(np.float32)
+        qh = blk[:, 4:8].copy().view(np.uint32)
+        qs = blk[:, 8:]
+        j = np.arange(16)
+        x0 = (qs & 15) | (((qh >> j) & 1) << 4)
+        x1 = (qs >> 4) | (((qh >> (j + 16)) & 1) << 4)
+        y = np.concatenate([x0, x1], 1).astype(np.float32) * d + m
+        assert (y.reshape(rows, cols).view(np.uint32) == got.view(np.uint32)).all()
