@@ -117,7 +117,9 @@ int moe_q4cp_gemv_down_topk(const moe_wview* dn, const float* hid, const int* id
                             int id_stride, int kpt, int P, int d, const float* ey, const float* sg,
                             float* out, uint64_t out_stride, moe_stream_t st);
 /* moe_gg_gemv (src/gpu/parts/26_kernels_moe_gguf.inc:893): GGUF raw-block experts, small P.
- * Supported: tgu = tdn = Q4_K, d % 256 == 0, mid % 256 == 0. */
+ * Supported: tgu and tdn each one of Q4_K, Q5_K (row length % 256 == 0), Q5_1, Q8_0 (row length % 32 == 0);
+ * tgu = tdn = Q4_K with d % 256 == 0 and mid % 256 == 0 takes the tuned kernels, any other mix the general ones.
+ * MOE_E_UNSUPPORTED for other types, as the reference's wrapper returns false. */
 int moe_gg_gemv(int tgu, int tdn, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
                 const float* x, const int* ids, const float* ws, float* hid, float* out, int P,
                 int d, int mid, int kpt, int id_stride, moe_stream_t st);
