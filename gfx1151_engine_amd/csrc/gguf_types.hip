@@ -18,6 +18,7 @@ __device__ __host__ __forceinline__ uint64_t gg_row_bytes(int t, uint64_t k) {
     default: return 0;
   }
 }
+__host__ size_t gg_align(int t) { return t == MOE_GGML_Q8_0 ? 2 : t == MOE_GGML_Q5_1 ? 8 : 16; }  // widest load used
 __host__ bool gg_type_ok(int t, int k) {
   if (t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K) return k >= 256 && k % 256 == 0;
   if (t == MOE_GGML_Q8_0 || t == MOE_GGML_Q5_1) return k >= 32 && k % 32 == 0;
@@ -33,45 +34,66 @@ __device__ __forceinline__ void k4_sm(int j, const uint8_t* q, int& sc, int& mn)
     mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
   }
 }
-__device__ __forceinline__ float h2f(const uint8_t* p) {
-  const uint16_t h = (uint16_t)(p[0] | (p[1] << 8));
-  return __half2float(__ushort_as_half(h));
-}
+__device__ __forceinline__ float h2f_bits(uint32_t h) { return __half2float(__ushort_as_half((uint16_t)h)); }
 
 // Block b (32 consecutive elements) of a row: the 32 integer codes q[] in element order and the two
 // constants of w = a*q + c (a, c and a*q are exact in f32: fp16 fields times integers of at most 8 bits).
+// Loads are as wide as the block layouts allow: K-quant super-blocks (144 / 176 bytes) keep their fields
+// 16-byte aligned, Q5_1 blocks (24 bytes) 8-byte aligned, Q8_0 blocks (34 bytes) 2-byte aligned; rows
+// start on 32-byte boundaries in a GGUF file and on allocation boundaries in device memory.
 __device__ __forceinline__ void gg_block(int t, const uint8_t* row, int b, int (&q)[32], float& a, float& c) {
   if (t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K) {
     const bool k5 = t == MOE_GGML_Q5_K;
     const uint8_t* sb = row + (size_t)(b >> 3) * (k5 ? 176 : 144);
     const int j = b & 7;  // sub-block: pair j/2, low nibbles if j even
+    const uint4 hd = *(const uint4*)sb;  // d, dmin, scales[12]
+    const uint8_t sc12[12] = {(uint8_t)hd.y, (uint8_t)(hd.y >> 8), (uint8_t)(hd.y >> 16), (uint8_t)(hd.y >> 24),
+                              (uint8_t)hd.z, (uint8_t)(hd.z >> 8), (uint8_t)(hd.z >> 16), (uint8_t)(hd.z >> 24),
+                              (uint8_t)hd.w, (uint8_t)(hd.w >> 8), (uint8_t)(hd.w >> 16), (uint8_t)(hd.w >> 24)};
     int sc, mn;
-    k4_sm(j, sb + 4, sc, mn);
-    a = h2f(sb) * (float)sc;
-    c = -(h2f(sb + 2) * (float)mn);
-    const uint8_t* ql = sb + (k5 ? 48 : 16) + 32 * (j >> 1);
-    const uint8_t* qh = sb + 16;
+    k4_sm(j, sc12, sc, mn);
+    a = h2f_bits(hd.x & 0xffffu) * (float)sc;
+    c = -(h2f_bits(hd.x >> 16) * (float)mn);
+    const uint4* ql = (const uint4*)(sb + (k5 ? 48 : 16) + 32 * (j >> 1));
+    const uint4 l0 = ql[0], l1 = ql[1];
+    const uint32_t lw[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+    uint32_t hw[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (k5) {
+      const uint4* qh = (const uint4*)(sb + 16);
+      const uint4 h0 = qh[0], h1 = qh[1];
+      hw[0] = h0.x; hw[1] = h0.y; hw[2] = h0.z; hw[3] = h0.w;
+      hw[4] = h1.x; hw[5] = h1.y; hw[6] = h1.z; hw[7] = h1.w;
+    }
+    const int nsh = (j & 1) ? 4 : 0;
 #pragma unroll
     for (int l = 0; l < 32; l++) {
-      int v = (j & 1) ? ql[l] >> 4 : ql[l] & 0xF;
-      if (k5) v += ((qh[l] >> j) & 1) << 4;
-      q[l] = v;
+      const uint32_t byte = (lw[l >> 2] >> (8 * (l & 3))) & 0xffu, hb = (hw[l >> 2] >> (8 * (l & 3))) & 0xffu;
+      q[l] = (int)(((byte >> nsh) & 0xFu) | (((hb >> j) & 1u) << 4));
     }
   } else if (t == MOE_GGML_Q8_0) {
-    const uint8_t* p = row + (size_t)b * 34;
-    a = h2f(p);
+    const uint16_t* p = (const uint16_t*)(row + (size_t)b * 34);
+    uint16_t w[17];
+#pragma unroll
+    for (int i = 0; i < 17; i++) w[i] = p[i];
+    a = h2f_bits(w[0]);
     c = 0.f;
 #pragma unroll
-    for (int l = 0; l < 32; l++) q[l] = (int)(int8_t)p[2 + l];
+    for (int l = 0; l < 16; l++) {
+      q[2 * l] = (int)(int8_t)(w[1 + l] & 0xff);
+      q[2 * l + 1] = (int)(int8_t)(w[1 + l] >> 8);
+    }
   } else {  // Q5_1
-    const uint8_t* p = row + (size_t)b * 24;
-    a = h2f(p);
-    c = h2f(p + 2);
-    const uint32_t qh = (uint32_t)p[4] | ((uint32_t)p[5] << 8) | ((uint32_t)p[6] << 16) | ((uint32_t)p[7] << 24);
+    const uint2* p = (const uint2*)(row + (size_t)b * 24);
+    const uint2 p0 = p[0], p1 = p[1], p2 = p[2];
+    a = h2f_bits(p0.x & 0xffffu);
+    c = h2f_bits(p0.x >> 16);
+    const uint32_t qh = p0.y;
+    const uint32_t qs[4] = {p1.x, p1.y, p2.x, p2.y};
 #pragma unroll
     for (int l = 0; l < 16; l++) {
-      q[l] = (p[8 + l] & 0xF) | (((qh >> l) & 1) << 4);
-      q[l + 16] = (p[8 + l] >> 4) | (((qh >> (l + 16)) & 1) << 4);
+      const uint32_t byte = (qs[l >> 2] >> (8 * (l & 3))) & 0xffu;
+      q[l] = (int)((byte & 0xFu) | (((qh >> l) & 1u) << 4));
+      q[l + 16] = (int)((byte >> 4) | (((qh >> (l + 16)) & 1u) << 4));
     }
   }
 }
@@ -101,14 +123,18 @@ __device__ __forceinline__ float wave_sum_f(float v) {
   return v;
 }
 
-// dot product of one row with x (K floats in LDS): lanes take the 32-element blocks in turn
+// Activations sit in LDS with one float of padding per 32 (element i at GX_PAD(i)): lanes work on different
+// 32-element blocks at the same offset, which without the padding is the same bank for every lane.
+#define GX_PAD(i) ((i) + ((i) >> 5))
+
+// dot product of one row with x (K floats in LDS, padded): lanes take the 32-element blocks in turn
 __device__ __forceinline__ float gg_row_dot(int t, const uint8_t* row, const float* x, int K, int lane) {
   float acc = 0.f;
   for (int b = lane; b < K / 32; b += 64) {
     int q[32];
     float a, c;
     gg_block(t, row, b, q, a, c);
-    const float* xb = x + 32 * b;
+    const float* xb = x + 33 * b;
     float sq = 0.f, sx = 0.f;
 #pragma unroll
     for (int l = 0; l < 32; l++) {
@@ -134,7 +160,7 @@ __global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restri
                                                 int id_stride, int kpt, int d, int mid, float* __restrict__ hid) {
   extern __shared__ float xs[];
   const int s = blockIdx.y, tok = blockIdx.z;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) xs[i] = x[(size_t)tok * d + i];
+  for (int i = threadIdx.x; i < d; i += blockDim.x) xs[GX_PAD(i)] = x[(size_t)tok * d + i];
   __syncthreads();
   const bool shared = s >= kpt;
   const int t = shared ? A.tsh : A.tgu;
@@ -153,18 +179,18 @@ __global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restri
   }
 }
 
-// grid (ceil(d/GX_ROWS), P), block 256: y[token][row] = sum over slots (selection order) of w_s * (down_s . hid_s)
+// grid (ceil(d/GX_ROWS), P), block 256: y[token][row] = sum over slots of w_s * (down_s . hid_s)
 // + sigmoid(shared gate logit) * (shared down . hid_shared)
 __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restrict__ hid, const int* __restrict__ ids,
                                                 const float* __restrict__ ws, int id_stride, int kpt, int d, int mid,
                                                 float* __restrict__ out) {
-  extern __shared__ float hs[];  // [slot][mid]
+  extern __shared__ float hs[];  // [slot][mid], padded
   __shared__ int eid[17];
   __shared__ float wgt[17];
   const int tok = blockIdx.y;
   const bool has_shared = A.sh_down != nullptr;
   const int nslots = kpt + (has_shared ? 1 : 0);
-  for (int i = threadIdx.x; i < nslots * mid; i += blockDim.x) hs[i] = hid[(size_t)tok * nslots * mid + i];
+  for (int i = threadIdx.x; i < nslots * mid; i += blockDim.x) hs[GX_PAD(i)] = hid[(size_t)tok * nslots * mid + i];
   if ((int)threadIdx.x < nslots) {
     const int s = threadIdx.x;
     eid[s] = s < kpt ? ids[(size_t)tok * id_stride + s] : 0;
@@ -172,18 +198,34 @@ __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restri
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  // a wave per row; its lanes take the (slot, 32-element block) units in turn, each weighted by the slot's
+  // combine weight, so a row needs one wave-wide sum (a fixed order: the result does not depend on timing)
+  const int nb = mid / 32;
   for (int rr = wv; rr < GX_ROWS; rr += 4) {
     const int r = blockIdx.x * GX_ROWS + rr;
     if (r >= d) break;
-    float y = 0.f;
-    for (int s = 0; s < nslots; s++) {
+    float acc = 0.f;
+    for (int u = lane; u < nslots * nb; u += 64) {
+      const int s = u / nb, b = u - s * nb;
       const bool sh = has_shared && s == nslots - 1;
       const int t = sh ? A.tsh : A.tdn;
       const uint64_t rb = gg_row_bytes(t, mid);
       const uint8_t* row = sh ? A.sh_down + (uint64_t)r * rb : A.down + ((uint64_t)eid[s] * d + r) * rb;
-      y += wgt[s] * gg_row_dot(t, row, hs + (size_t)s * mid, mid, lane);
+      int q[32];
+      float a, c;
+      gg_block(t, row, b, q, a, c);
+      const float* xb = hs + 33 * (s * nb + b);
+      float sq = 0.f, sx = 0.f;
+#pragma unroll
+      for (int l = 0; l < 32; l++) {
+        const float xv = xb[l];
+        sq = fmaf((float)q[l], xv, sq);
+        sx += xv;
+      }
+      acc += wgt[s] * (a * sq + c * sx);
     }
-    if (lane == 0) out[(size_t)tok * d + r] = y;
+    acc = wave_sum_f(acc);
+    if (lane == 0) out[(size_t)tok * d + r] = acc;
   }
 }
 
@@ -198,6 +240,7 @@ MOE_API int moe_gg_dequant_rows(int type, const uint8_t* raw, uint64_t nrows, ui
   if (cols == 0 || cols > (1ull << 31)) return MOE_E_INVALID;
   if (!gg_type_ok(type, (int)cols)) return MOE_E_UNSUPPORTED;
   if (nrows == 0) return MOE_OK;
+  if (!moe_aligned(raw, gg_align(type)) || !moe_aligned(out, 4)) return MOE_E_INVALID;
   const uint64_t nblocks = nrows * (cols / 32);
   const unsigned grid = (unsigned)((nblocks + 255) / 256 > 65535 * 16 ? 65535 * 16 : (nblocks + 255) / 256);
   k_gg_dequant<<<grid, 256, 0, moe_s(st)>>>(type, raw, cols, nblocks, out);
@@ -217,6 +260,10 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
   const bool sh = sh_gate != nullptr;
   if (sh && (!sh_up || !sh_down || !sh_logit)) return MOE_E_INVALID;
   if (sh && !(gg_type_ok(tsh, d) && gg_type_ok(tsh, mid))) return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(gate, gg_align(tgu)) || !moe_aligned(up, gg_align(tgu)) || !moe_aligned(down, gg_align(tdn)) ||
+      (sh && (!moe_aligned(sh_gate, gg_align(tsh)) || !moe_aligned(sh_up, gg_align(tsh)) ||
+              !moe_aligned(sh_down, gg_align(tsh)))))
+    return MOE_E_INVALID;
   const int nslots = kpt + (sh ? 1 : 0);
   if (nslots > 16 || (size_t)d * 4 > 60 * 1024 || (size_t)nslots * mid * 4 > 60 * 1024) return MOE_E_UNSUPPORTED;
   if (P == 0) return MOE_OK;
@@ -227,12 +274,12 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
   A.sh_logit = sh_logit;
   if (phase != 2) {
     dim3 grid((mid + GX_ROWS - 1) / GX_ROWS, nslots, P);
-    k_ggx_gu<<<grid, 256, (size_t)d * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
+    k_ggx_gu<<<grid, 256, (size_t)d / 32 * 33 * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
     MOE_LAUNCH_CHECK();
   }
   if (phase != 1) {
     dim3 grid((d + GX_ROWS - 1) / GX_ROWS, P);
-    k_ggx_dn<<<grid, 256, (size_t)nslots * mid * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
+    k_ggx_dn<<<grid, 256, (size_t)nslots * mid / 32 * 33 * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
     MOE_LAUNCH_CHECK();
   }
   return MOE_OK;
