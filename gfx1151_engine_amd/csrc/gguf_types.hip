@@ -1,7 +1,7 @@
-// The further ggml block types of GGUF expert tensors, read in place: Q5_K (gate/up), Q5_1 and Q8_0 (down)
-// next to Q4_K — the mix of the reference's GGUF checkpoints (src/gpu/parts/30_host_util.inc:399-405,
+// The further ggml block types of GGUF expert tensors, read in place: Q5_K (gate/up), Q5_1 and Q8_0 (down),
+// IQ4_NL and IQ4_XS next to Q4_K — the mix of the reference's GGUF checkpoints (src/gpu/parts/30_host_util.inc:399-405,
 // src/gpu/parts/26_kernels_moe_gguf.inc:32-48).  Dequantisation (bit-exact with gguf::dequant_row,
-// src/gguf.h:339-445) and plain f32 GEMV kernels for any mix of the four types: one wave per weight row,
+// src/gguf.h:339-445) and plain f32 GEMV kernels for any mix of these types: one wave per weight row,
 // one lane per 32-element block.  These are the general kernels; Q4_K alone has the tuned ones
 // (gemv_q4k.hip, decode_q4k.hip, the Q4_K instantiation of the grouped GEMM).
 #include "common.h"
@@ -15,13 +15,17 @@ __device__ __host__ __forceinline__ uint64_t gg_row_bytes(int t, uint64_t k) {
     case MOE_GGML_Q5_K: return k / 256 * 176;
     case MOE_GGML_Q8_0: return k / 32 * 34;
     case MOE_GGML_Q5_1: return k / 32 * 24;
+    case MOE_GGML_IQ4_NL: return k / 32 * 18;
+    case MOE_GGML_IQ4_XS: return k / 256 * 136;
     default: return 0;
   }
 }
-__host__ size_t gg_align(int t) { return t == MOE_GGML_Q8_0 ? 2 : t == MOE_GGML_Q5_1 ? 8 : 16; }  // widest load used
+__host__ size_t gg_align(int t) {  // widest load used
+  return (t == MOE_GGML_Q8_0 || t == MOE_GGML_IQ4_NL) ? 2 : (t == MOE_GGML_Q5_1 || t == MOE_GGML_IQ4_XS) ? 8 : 16;
+}
 __host__ bool gg_type_ok(int t, int k) {
-  if (t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K) return k >= 256 && k % 256 == 0;
-  if (t == MOE_GGML_Q8_0 || t == MOE_GGML_Q5_1) return k >= 32 && k % 32 == 0;
+  if (t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K || t == MOE_GGML_IQ4_XS) return k >= 256 && k % 256 == 0;
+  if (t == MOE_GGML_Q8_0 || t == MOE_GGML_Q5_1 || t == MOE_GGML_IQ4_NL) return k >= 32 && k % 32 == 0;
   return false;
 }
 
@@ -82,6 +86,35 @@ __device__ __forceinline__ void gg_block(int t, const uint8_t* row, int b, int (
       q[2 * l] = (int)(int8_t)(w[1 + l] & 0xff);
       q[2 * l + 1] = (int)(int8_t)(w[1 + l] >> 8);
     }
+  } else if (t == MOE_GGML_IQ4_NL || t == MOE_GGML_IQ4_XS) {
+    // non-linear 4-bit codes (src/gguf.h:376-407): q = kv[nibble]; IQ4_XS adds a 6-bit scale per 32 elements
+    uint16_t w[8];
+    if (t == MOE_GGML_IQ4_NL) {
+      const uint16_t* p = (const uint16_t*)(row + (size_t)b * 18);
+      a = h2f_bits(p[0]);
+#pragma unroll
+      for (int i = 0; i < 8; i++) w[i] = p[1 + i];
+    } else {
+      const uint8_t* sb = row + (size_t)(b >> 3) * 136;
+      const int ib = b & 7;
+      const uint2 hd = *(const uint2*)sb;  // d, scales_h, scales_l[4]
+      const uint32_t sh = hd.x >> 16, sl = (hd.y >> (8 * (ib >> 1))) & 0xffu;
+      const int ls = (int)(((sl >> (4 * (ib & 1))) & 0xFu) | (((sh >> (2 * ib)) & 3u) << 4));
+      a = h2f_bits(hd.x & 0xffffu) * (float)(ls - 32);
+      const uint2* qs = (const uint2*)(sb + 8 + 16 * ib);
+      const uint2 q0 = qs[0], q1 = qs[1];
+      w[0] = (uint16_t)q0.x; w[1] = (uint16_t)(q0.x >> 16); w[2] = (uint16_t)q0.y; w[3] = (uint16_t)(q0.y >> 16);
+      w[4] = (uint16_t)q1.x; w[5] = (uint16_t)(q1.x >> 16); w[6] = (uint16_t)q1.y; w[7] = (uint16_t)(q1.y >> 16);
+    }
+    c = 0.f;
+    // kv = {-127,-104,-83,-65,-49,-35,-22,-10,1,13,25,38,53,69,89,113} as bytes of four words
+    const uint32_t kv[4] = {0xbfad9881u, 0xf6eaddcfu, 0x26190d01u, 0x71594535u};
+#pragma unroll
+    for (int l = 0; l < 16; l++) {
+      const uint32_t byte = (w[l >> 1] >> (8 * (l & 1))) & 0xffu, lo = byte & 0xFu, hi = byte >> 4;
+      q[l] = (int)(int8_t)(kv[lo >> 2] >> (8 * (lo & 3)));
+      q[l + 16] = (int)(int8_t)(kv[hi >> 2] >> (8 * (hi & 3)));
+    }
   } else {  // Q5_1
     const uint2* p = (const uint2*)(row + (size_t)b * 24);
     const uint2 p0 = p[0], p1 = p[1], p2 = p[2];
@@ -112,7 +145,8 @@ __global__ void __launch_bounds__(256) k_gg_dequant(int t, const uint8_t* __rest
 #pragma unroll
     for (int l = 0; l < 32; l++) {
       const float prod = __fmul_rn(a, (float)q[l]);  // exact
-      y[l] = t == MOE_GGML_Q8_0 ? prod : __fadd_rn(prod, c);  // Q8_0 has no constant term (keeps -0.0); else one rounded add
+      // Q8_0 / IQ4 have no constant term (keeps -0.0); else one rounded add
+      y[l] = (t == MOE_GGML_Q8_0 || t == MOE_GGML_IQ4_NL || t == MOE_GGML_IQ4_XS) ? prod : __fadd_rn(prod, c);
     }
   }
 }

@@ -11,7 +11,8 @@ import numpy as np
 
 HGN_BF16, HGN_F32, HGN_Q4CP = 0, 1, 5
 GGML_F32, GGML_BF16, GGML_Q4_K = 0, 30, 12
-_GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24)}
+_GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24),
+               20: (32, 18), 23: (256, 136)}
 
 
 def _bytes(a):

@@ -105,11 +105,32 @@ def make_q5_1(rng, rows, cols, scale_std=0.01):
     return blk.reshape(-1)
 
 
-GG_Q4_K, GG_Q5_K, GG_Q5_1, GG_Q8_0 = 12, 13, 7, 8  # ggml type ids
+def make_iq4_nl(rng, rows, cols, scale_std=0.01):
+    """Random IQ4_NL rows (18-byte blocks: d fp16, qs[16]; codes index a 16-entry table of int8; src/gguf.h:376-388)."""
+    assert cols % 32 == 0
+    nb = rows * cols // 32
+    blk = np.zeros((nb, 18), np.uint8)
+    blk[:, 0:2] = (np.abs(rng.standard_normal((nb, 1), dtype=np.float32)) * scale_std / 16).astype(np.float16).view(np.uint8)
+    blk[:, 2:] = rng.integers(0, 256, (nb, 16), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+def make_iq4_xs(rng, rows, cols, scale_std=0.01):
+    """Random IQ4_XS rows (136-byte super-blocks: d fp16, scales_h u16, scales_l[4], qs[128]; src/gguf.h:389-407)."""
+    assert cols % 256 == 0
+    nb = rows * cols // 256
+    blk = np.zeros((nb, 136), np.uint8)
+    blk[:, 0:2] = (np.abs(rng.standard_normal((nb, 1), dtype=np.float32)) * scale_std / 256).astype(np.float16).view(np.uint8)
+    blk[:, 2:] = rng.integers(0, 256, (nb, 134), dtype=np.uint8)
+    return blk.reshape(-1)
+
+
+GG_Q4_K, GG_Q5_K, GG_Q5_1, GG_Q8_0, GG_IQ4_NL, GG_IQ4_XS = 12, 13, 7, 8, 20, 23  # ggml type ids
 
 
 def make_gg(rng, t, rows, cols, scale_std=0.01):
-    return {GG_Q4_K: make_q4k, GG_Q5_K: make_q5k, GG_Q5_1: make_q5_1, GG_Q8_0: make_q8_0}[t](rng, rows, cols, scale_std)
+    return {GG_Q4_K: make_q4k, GG_Q5_K: make_q5k, GG_Q5_1: make_q5_1, GG_Q8_0: make_q8_0, GG_IQ4_NL: make_iq4_nl,
+            GG_IQ4_XS: make_iq4_xs}[t](rng, rows, cols, scale_std)
 
 
 def f32_to_bf16_bits(a):

@@ -34,8 +34,10 @@ enum moe_status {
 /* hgn tensor dtypes (src/hgn.h:2-23) and ggml types (src/gguf.h:42-64) used on this path */
 enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5 };
 /* Q4_K: every kernel of the path.  Q5_K (gate/up), Q5_1 and Q8_0 (down) — the mix of the reference's GGUF
- * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — : dequantisation and the general GEMV kernels. */
-enum { MOE_GGML_Q5_1 = 7, MOE_GGML_Q8_0 = 8, MOE_GGML_Q4_K = 12, MOE_GGML_Q5_K = 13 };
+ * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — and IQ4_NL / IQ4_XS (src/gguf.h:376-407):
+ * dequantisation and the general GEMV kernels. */
+enum { MOE_GGML_Q5_1 = 7, MOE_GGML_Q8_0 = 8, MOE_GGML_Q4_K = 12, MOE_GGML_Q5_K = 13, MOE_GGML_IQ4_NL = 20,
+       MOE_GGML_IQ4_XS = 23 };
 
 /* WView (src/gpu/parts/30_host_util.inc:772-780): a weight tensor as it lies in memory.
  * q4cp: data = [64 B codebook][rows*cols/2 codes][rows x scale_stride]. */
@@ -69,7 +71,7 @@ int moe_q4cp_dequant_rows(const uint8_t* blob, uint64_t rows, uint64_t cols, uin
 int moe_q4k_dequant_rows(const uint8_t* raw, uint64_t nrows, uint64_t cols, float* out,
                          moe_stream_t st);
 /* gguf::dequant_row (src/gguf.h:339-445) for nrows raw rows of `cols` elements of ggml type
- * MOE_GGML_Q4_K / Q5_K (cols % 256 == 0) / Q5_1 / Q8_0 (cols % 32 == 0); bit-exact. */
+ * MOE_GGML_Q4_K / Q5_K / IQ4_XS (cols % 256 == 0) or Q5_1 / Q8_0 / IQ4_NL (cols % 32 == 0); bit-exact. */
 int moe_gg_dequant_rows(int type, const uint8_t* raw, uint64_t nrows, uint64_t cols, float* out,
                         moe_stream_t st);
 
@@ -117,7 +119,7 @@ int moe_q4cp_gemv_down_topk(const moe_wview* dn, const float* hid, const int* id
                             int id_stride, int kpt, int P, int d, const float* ey, const float* sg,
                             float* out, uint64_t out_stride, moe_stream_t st);
 /* moe_gg_gemv (src/gpu/parts/26_kernels_moe_gguf.inc:893): GGUF raw-block experts, small P.
- * Supported: tgu and tdn each one of Q4_K, Q5_K (row length % 256 == 0), Q5_1, Q8_0 (row length % 32 == 0);
+ * Supported: tgu and tdn each one of Q4_K, Q5_K, IQ4_XS (row length % 256 == 0), Q5_1, Q8_0, IQ4_NL (% 32 == 0);
  * tgu = tdn = Q4_K with d % 256 == 0 and mid % 256 == 0 takes the tuned kernels, any other mix the general ones.
  * MOE_E_UNSUPPORTED for other types, as the reference's wrapper returns false. */
 int moe_gg_gemv(int tgu, int tdn, const uint8_t* gate, const uint8_t* up, const uint8_t* down,

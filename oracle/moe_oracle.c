@@ -12,6 +12,7 @@
  *   src/gguf.h:328-336   scale_min_k4
  *   src/gguf.h:408-441   Q4_K / Q5_K dequant_row
  *   src/gguf.h:352-375   Q8_0 / Q5_1 dequant_row
+ *   src/gguf.h:376-407   IQ4_NL / IQ4_XS dequant_row
  *   src/ref.cpp:55-56    sigmoid / silu
  *   src/ref.cpp:68-77    matvec: fp64 sequential accumulate, f32 result
  *   src/ref.cpp:563-637  Model::moe (router, top-k, experts, shared expert)
@@ -37,7 +38,8 @@
 #define ORC_API __attribute__((visibility("default")))
 
 /* ---- weight format tags (shared with the library header by value) ---- */
-enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q5_1 = 7, ORC_Q8_0 = 8 };
+enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q5_1 = 7, ORC_Q8_0 = 8,
+       ORC_IQ4_NL = 20, ORC_IQ4_XS = 23 };
 
 /* src/hgn.h:77-84 and src/gguf.h:318-325 (same function twice in the reference) */
 ORC_API float orc_fp16_to_f32(uint16_t h) {
@@ -181,6 +183,42 @@ static void orc_q5_1_row(const uint8_t* src, float* y, uint64_t k) {
     }
   }
 }
+/* src/gguf.h:376-407: the non-linear 4-bit codebook of IQ4_NL / IQ4_XS */
+static const int8_t orc_iq4_kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+/* IQ4_NL: 18-byte blocks {d fp16, qs[16]}; element j = kv[low nibble of qs[j]], element j + 16 = kv[high] */
+static void orc_iq4_nl_row(const uint8_t* src, float* y, uint64_t k) {
+  for (uint64_t b = 0; b < k / 32; b++, src += 18) {
+    uint16_t dh;
+    memcpy(&dh, src, 2);
+    const float d = orc_fp16_to_f32(dh);
+    for (int j = 0; j < 16; j++) {
+      y[b * 32 + j] = d * orc_iq4_kv[src[2 + j] & 0xF];
+      y[b * 32 + j + 16] = d * orc_iq4_kv[src[2 + j] >> 4];
+    }
+  }
+}
+/* IQ4_XS: 136-byte super-blocks {d fp16, scales_h u16, scales_l[4], qs[128]}: eight 32-element sub-blocks with
+ * 6-bit scales ls (low 4 bits in scales_l, high 2 in scales_h), dl = d*(ls - 32), elements as IQ4_NL.
+ * d*(ls-32) and dl*kv are exact in f32 (11 + 6 + 7 bits). */
+static void orc_iq4_xs_row(const uint8_t* src, float* y, uint64_t k) {
+  for (uint64_t b = 0; b < k / 256; b++, src += 136) {
+    uint16_t dh, sh;
+    memcpy(&dh, src, 2);
+    memcpy(&sh, src + 2, 2);
+    const float d = orc_fp16_to_f32(dh);
+    const uint8_t* sl = src + 4;
+    const uint8_t* qs = src + 8;
+    for (int ib = 0; ib < 8; ib++, qs += 16) {
+      const int ls = ((sl[ib / 2] >> (4 * (ib % 2))) & 0xF) | (((sh >> (2 * ib)) & 3) << 4);
+      const float dl = d * (float)(ls - 32);
+      float* yy = y + b * 256 + ib * 32;
+      for (int j = 0; j < 16; j++) {
+        yy[j] = dl * orc_iq4_kv[qs[j] & 0xF];
+        yy[j + 16] = dl * orc_iq4_kv[qs[j] >> 4];
+      }
+    }
+  }
+}
 /* src/gguf.h:42-84: bytes of one row of k elements */
 ORC_API uint64_t orc_gg_row_bytes(int type, uint64_t k) {
   switch (type) {
@@ -188,6 +226,8 @@ ORC_API uint64_t orc_gg_row_bytes(int type, uint64_t k) {
     case ORC_Q5K: return k / 256 * 176;
     case ORC_Q8_0: return k / 32 * 34;
     case ORC_Q5_1: return k / 32 * 24;
+    case ORC_IQ4_NL: return k / 32 * 18;
+    case ORC_IQ4_XS: return k / 256 * 136;
     default: return 0;
   }
 }
@@ -197,6 +237,8 @@ ORC_API int orc_gg_row(int type, const uint8_t* src, float* y, uint64_t k) {
     case ORC_Q5K: orc_q5k_row(src, y, k); return 0;
     case ORC_Q8_0: orc_q8_0_row(src, y, k); return 0;
     case ORC_Q5_1: orc_q5_1_row(src, y, k); return 0;
+    case ORC_IQ4_NL: orc_iq4_nl_row(src, y, k); return 0;
+    case ORC_IQ4_XS: orc_iq4_xs_row(src, y, k); return 0;
     default: return -1;
   }
 }
@@ -218,7 +260,7 @@ static void mat_row(const orc_mat* W, uint64_t r, float* out) {
     }
     case ORC_Q4CP: orc_q4cp_row(W->data, W->rows, W->cols, r, out); break;
     case ORC_Q4K: orc_q4k_row(W->data + r * orc_q4k_row_bytes(W->cols), out, W->cols); break;
-    case ORC_Q5K: case ORC_Q8_0: case ORC_Q5_1:
+    case ORC_Q5K: case ORC_Q8_0: case ORC_Q5_1: case ORC_IQ4_NL: case ORC_IQ4_XS:
       orc_gg_row(W->dtype, W->data + r * orc_gg_row_bytes(W->dtype, W->cols), out, W->cols);
       break;
     default: memset(out, 0, W->cols * 4);

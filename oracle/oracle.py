@@ -11,8 +11,8 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 F32, BF16, Q4CP, Q4K = 1, 0, 5, 12
-Q5K, Q5_1, Q8_0 = 13, 7, 8          # further ggml block types of the expert tensors (ids as in GGUF)
-GG_TYPES = (Q4K, Q5K, Q5_1, Q8_0)
+Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS = 13, 7, 8, 20, 23   # further ggml block types of the expert tensors (ids as in GGUF)
+GG_TYPES = (Q4K, Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS)
 
 
 def build(force=False):

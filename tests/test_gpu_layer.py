@@ -120,7 +120,8 @@ def test_decode_topk_near_ties(oracle, fmt, T):
     m.close()
 
 
-@pytest.mark.parametrize("tgu,tdn,tsh,T", [(13, 8, 12, 1), (12, 7, 12, 5), (13, 7, 8, 3), (12, 8, 13, 40)])
+@pytest.mark.parametrize("tgu,tdn,tsh,T", [(13, 8, 12, 1), (12, 7, 12, 5), (13, 7, 8, 3), (12, 8, 13, 40), (23, 20, 12, 2),
+                                            (20, 23, 23, 7)])
 def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
     """GGUF layers in the type mix of the reference's checkpoints (Q4_K / Q5_K gate and up, Q5_1 / Q8_0 down,
     src/gpu/parts/30_host_util.inc:399-405): the general f32 GEMV kernels, ids bit-exact, output within the GEMV

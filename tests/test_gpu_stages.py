@@ -72,7 +72,7 @@ def test_q4k_all_scale_min_codes(capi, oracle):
     assert same_bits(capi.q4k_dequant_rows(gpu(raw), n, 256).cpu().numpy(), oracle.q4k_rows(raw, n, 256))
 
 
-@pytest.mark.parametrize("t,cols", [(13, 768), (8, 96), (7, 96), (8, 3072), (7, 768), (12, 512)])
+@pytest.mark.parametrize("t,cols", [(13, 768), (8, 96), (7, 96), (8, 3072), (7, 768), (12, 512), (20, 96), (20, 768), (23, 768)])
 def test_gg_dequant_other_types(capi, oracle, t, cols):
     """Q5_K / Q8_0 / Q5_1 (and Q4_K through the same entry point): bit-exact with the oracle's rows, which the
     CPU tests pin against the reference's gguf::dequant_row; random bytes in the integer fields, so every code

@@ -299,7 +299,7 @@ def test_layer_matches_float64_numpy_q4k(oracle):
         assert np.abs(y[t] - want).max() <= 2e-5 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("t,name", [(13, "Q5_K"), (8, "Q8_0"), (7, "Q5_1"), (12, "Q4_K")])
+@pytest.mark.parametrize("t,name", [(13, "Q5_K"), (8, "Q8_0"), (7, "Q5_1"), (12, "Q4_K"), (20, "IQ4_NL"), (23, "IQ4_XS")])
 def test_gg_rows_against_reference(oracle, t, name):
     """The further ggml block types of the expert tensors: the oracle's rows against the reference's own
     gguf::dequant_row (oracle/_ref) on random block bytes, bit for bit, and against a numpy evaluation of the
