@@ -24,11 +24,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 D, MID, E, K = 3072, 768, 512, 10
+LIB_OPTIONS = []              # (option id, value) pairs of --opt, applied to every context
 # HBM bytes per launch of the dominant kernel (read + written) at the default shapes, from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic.txt (counters
 # cannot be read from inside this process; other shapes report null)
-LIB_OPTIONS = []              # (option id, value) pairs of --opt, applied to every context
-PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4852.10e6, ("decode", "q4cp", 1): 29.60e6}
+PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4885.30e6, ("decode", "q4cp", 1): 29.60e6}
 CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
 
 
