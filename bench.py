@@ -28,7 +28,7 @@ LIB_OPTIONS = []              # (option id, value) pairs of --opt, applied to ev
 # HBM bytes per launch of the dominant kernel (read + written) at the default shapes, from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic.txt (counters
 # cannot be read from inside this process; other shapes report null)
-PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4885.30e6, ("decode", "q4cp", 1): 29.60e6}
+PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4543.03e6, ("decode", "q4cp", 1): 29.60e6}
 CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
 
 
@@ -166,16 +166,22 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
            "format": "q4cp g32 zero-point 8" if fmt == "q4cp" else "GGUF Q4_K", "layers": nlayers, **extra}
     if kind == "prefill":
         flop_tok = k * 6 * d * mid + 6 * d * mid + 2 * d * E + 2 * d
-        up_flop = (pairs + T) * 2 * (2 * mid) * d  # gate+up GEMM incl. shared expert, one launch
+        # the timed gate/up launch: the routed experts' pairs; the shared expert's tiles are in the same launch only
+        # with MOE_OPT_SHARED_ASIDE = 0 or MOE_OPT_FUSED_COMBINE = 1 (by default its GEMMs run on the library's side
+        # stream next to the router launch and are over before this launch starts)
+        opts = dict(LIB_OPTIONS)
+        shared_in_launch = opts.get(4, 1) == 0 or opts.get(3, 0) != 0
+        up_flop = (pairs + (T if shared_in_launch else 0)) * 2 * (2 * mid) * d
         up_s = stage["up"] * 1e-3
         res.update({"metric": "moe_layer_prefill_tokens_per_s", "unit": "tok/s", "value": round(T / (ms * 1e-3), 1),
                     "dtype": "f16",
                     "layer_tflops": round(flop_tok * T / (ms * 1e-3) / 1e12, 2),
                     "layer_mfma_frac": round(flop_tok * T / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                    "roofline": {"bound": "mfma", "kernel": "k_moe_gemm (gate/up + SwiGLU)",
+                    "roofline": {"bound": "mfma", "kernel": "k_moe_gemm (gate/up + SwiGLU), " +
+                                 ("routed + shared expert tiles" if shared_in_launch else "routed experts' tiles"),
                                  "achieved": round(up_flop / up_s / 1e12, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": round(up_flop / up_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                                 "traffic": PMC_TRAFFIC.get((kind, fmt, T))}})
+                                 "traffic": None if shared_in_launch else PMC_TRAFFIC.get((kind, fmt, T))}})
         # rows the grouped GEMM computes for the routed pairs: tiles of 128, the last tile of an expert padded
         # to a multiple of 32 rows
         rem = cnt % 128

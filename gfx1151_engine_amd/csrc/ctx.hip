@@ -80,7 +80,11 @@ struct moe_ctx {
   // batch path: the f32 -> f16 copy of x runs on a side stream next to the latency-bound top-k and
   // permutation launches (forked after the logits launch, joined in front of the gate/up GEMM)
   hipStream_t side = nullptr;
-  hipEvent_t ev_fork = nullptr, ev_join = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_join = nullptr, ev_x16 = nullptr;
+  // batch path, shared expert on the side stream: its tile list and the switch
+  moe_tile* tiles_sh = nullptr;
+  int* ntiles_sh = nullptr;
+  bool shared_aside = true;
 };
 
 static void prof_mark(moe_ctx* c, int stage_done, hipStream_t st) {
@@ -111,9 +115,10 @@ MOE_API int moe_destroy(moe_ctx* c) {
     if (e) (void)hipEventDestroy(e);
   if (c->ev_fork) (void)hipEventDestroy(c->ev_fork);
   if (c->ev_join) (void)hipEventDestroy(c->ev_join);
+  if (c->ev_x16) (void)hipEventDestroy(c->ev_x16);
   if (c->side) (void)hipStreamDestroy(c->side);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->kpart, c->ktickets, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
-                  c->pairids, c->tiles, c->ntiles, c->hid16, c->pairs16, c->pairs32};
+                  c->pairids, c->tiles, c->ntiles, c->tiles_sh, c->ntiles_sh, c->hid16, c->pairs16, c->pairs32};
   for (void* b : bufs)
     if (b) {
       hipError_t e = hipFree(b);
@@ -172,6 +177,8 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
     if (e == hipSuccess) e = hipMalloc(&c->pairids, T * cfg->topk * 4);
     if (e == hipSuccess) e = hipMalloc(&c->tiles, (size_t)c->max_tiles * sizeof(moe_tile));
     if (e == hipSuccess) e = hipMalloc(&c->ntiles, 8);
+    if (e == hipSuccess) e = hipMalloc(&c->tiles_sh, ((T + 127) / 128 + 1) * sizeof(moe_tile));
+    if (e == hipSuccess) e = hipMalloc(&c->ntiles_sh, 8);
     if (e == hipSuccess) e = hipMalloc(&c->pairs32, k1 * Ts * (size_t)cfg->d * 4);
   }
   if (e == hipSuccess && T > (size_t)c->small_max) {
@@ -185,6 +192,7 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
     e = hipStreamCreateWithFlags(&c->side, hipStreamNonBlocking);  // default priority
     if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_fork, hipEventDisableTiming);
     if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_join, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&c->ev_x16, hipEventDisableTiming);
   }
   if (e != hipSuccess) {
     moe_destroy(c);
@@ -354,6 +362,7 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
       c->uq_min = value;
       return MOE_OK;
     case MOE_OPT_FUSED_COMBINE: c->fused_combine = value != 0; return MOE_OK;
+    case MOE_OPT_SHARED_ASIDE: c->shared_aside = value != 0; return MOE_OK;
     default: return MOE_E_INVALID;
   }
 }
@@ -549,6 +558,57 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   c->ev_n = 0;
   prof_mark(c, 0, st);
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
+  if (L.has_shared && c->shared_aside && !c->fused_combine) {
+    // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
+    // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
+    // side stream also makes what both streams need first: the per-token mean square of x (range guard) and
+    // the f16 copy of x.  Joins: in front of the routed gate/up GEMM (x16, xms) and in front of the combine.
+    const int sh_first = P * g.topk;
+    const int max_tiles_sh = (P + 127) / 128;
+    const int max_tiles = (P * g.topk + 127) / 128 + g.experts;
+    MOE_HIP(hipEventRecord(c->ev_fork, st));
+    MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
+    int rs = moe_launch_row_meansq(x, P, g.d, c->xms, c->side);
+    if (!rs) rs = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
+    hipError_t ee = hipEventRecord(c->ev_x16, c->side);
+    if (!rs && ee != hipSuccess) rs = (int)ee;
+    if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, 128, P, sh_first, c->tokidx, c->side);
+    if (!rs)
+      rs = moe_launch_gemm_q4cp(true, &gu, &sgu, g.experts, c->x16, c->tokidx, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
+                                c->hid16, g.mid, g.d, true, q4k, hs, c->side, nullptr);
+    if (!rs)
+      rs = moe_launch_gemm_q4cp(false, &dn, &sdn, g.experts, c->hid16, nullptr, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
+                                c->pairs16, g.d, g.mid, true, q4k, hs, c->side, nullptr);
+    // caller's stream: router, top-k, permutation, the routed experts' GEMMs
+    rc = moe_router_logits_seq(&L.router, L.router_bias, &L.sh_sg, x, P, c->logits, c->sh_logit, nullptr, st);
+    if (!rc) rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
+    prof_mark(c, MOE_PROF_ROUTER, st);
+    if (!rc)
+      rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
+                           g.id_stride, st);
+    if (!rc) rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, -1, c->tokidx, st);
+    ee = hipStreamWaitEvent(st, c->ev_x16, 0);
+    if (!rc && ee != hipSuccess) rc = (int)ee;
+    prof_mark(c, MOE_PROF_ROUTE, st);
+    if (!rc && !rs)
+      rc = moe_launch_gemm_q4cp(true, &gu, nullptr, g.experts, c->x16, c->tokidx, c->tiles, c->ntiles, max_tiles,
+                                c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr);
+    prof_mark(c, MOE_PROF_UP, st);
+    if (!rc && !rs)
+      rc = moe_launch_gemm_q4cp(false, &dn, nullptr, g.experts, c->hid16, nullptr, c->tiles, c->ntiles, max_tiles,
+                                c->pairs16, g.d, g.mid, true, q4k, hs, st, nullptr);
+    // the side stream is joined on every path out of here (a capture on `st` must not end with it forked)
+    ee = hipEventRecord(c->ev_join, c->side);
+    if (ee == hipSuccess) ee = hipStreamWaitEvent(st, c->ev_join, 0);
+    prof_mark(c, MOE_PROF_DOWN, st);
+    if (rc) return rc;
+    if (rs) return rs;
+    if (ee != hipSuccess) return (int)ee;
+    rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, c->sh_logit, sh_first, y, P, g.d, g.topk, hs,
+                           st);
+    prof_mark(c, MOE_PROF_REDUCE, st);
+    return rc;
+  }
   if ((rc = moe_router_logits_seq(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
                                   c->sh_logit, c->xms, st)))
     return rc;

@@ -192,7 +192,59 @@ __global__ void __launch_bounds__(1024) k_tiles_shared(const int* __restrict__ e
   if (sh_first >= 0)
     for (int i = e; i < P; i += 1024) tokidx[sh_first + i] = i;
 }
+// The shared expert's tile list on its own (it does not depend on the routing): tiles over pairs
+// [sh_first, sh_first + P) in runs of cap, expert id = n_experts, total = {tiles, 0 routed}; also the
+// identity tokidx entries of those pairs.
+__global__ void __launch_bounds__(256) k_tiles_only_shared(moe_tile* __restrict__ tiles, int* __restrict__ total,
+                                                           int E, int cap, int P, int sh_first,
+                                                           int* __restrict__ tokidx) {
+  const int nsh = (P + cap - 1) / cap;
+  const int i0 = blockIdx.x * 256 + threadIdx.x, stride = gridDim.x * 256;
+  for (int j = i0; j < nsh; j += stride) {
+    moe_tile t;
+    t.expert = E;
+    t.first = sh_first + j * cap;
+    t.count = min(cap, P - j * cap);
+    tiles[j] = t;
+  }
+  if (i0 == 0) {
+    total[0] = nsh;
+    total[1] = 0;
+  }
+  for (int i = i0; i < P; i += stride) tokidx[sh_first + i] = i;
+}
+
+// Mean square of each token's activations (input of the f16 range guard): one wave per token.
+__global__ void __launch_bounds__(256) k_row_meansq(const float* __restrict__ x, int P, int d, float* __restrict__ out) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= P) return;
+  const float4* row = (const float4*)(x + (size_t)t * d);
+  float acc = 0.f;
+  for (int i = lane; i < d / 4; i += 64) {
+    const float4 v = row[i];
+    acc += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (lane == 0) out[t] = acc / (float)d;
+}
 }  // namespace
+
+int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, int P, int sh_first, int* tokidx,
+                                 hipStream_t st) {
+  const int n = P > (P + cap - 1) / cap ? P : (P + cap - 1) / cap;
+  k_tiles_only_shared<<<(n + 255) / 256 > 64 ? 64 : (n + 255) / 256, 256, 0, st>>>(tiles, ntiles, E, cap, P, sh_first, tokidx);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_row_meansq(const float* x, int P, int d, float* out, hipStream_t st) {
+  if (!x || !out || d % 4 || !moe_aligned(x, 16)) return MOE_E_INVALID;
+  if (P == 0) return MOE_OK;
+  k_row_meansq<<<(P + 3) / 4, 256, 0, st>>>(x, P, d, out);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
 
 int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E, int cap, int P,
                             int sh_first, int* tokidx, hipStream_t st) {

@@ -224,7 +224,10 @@ int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_st
  * weighted rows are added into y with f32 atomics, y is zeroed on the context's side stream, no pairs buffer is
  * written and no reduce launch follows.  The order of the k+1 additions per element then depends on timing, so
  * results can differ in their last bits from run to run; 0 keeps the ordered two-step form. */
-enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2, MOE_OPT_FUSED_COMBINE = 3 };
+/* MOE_OPT_SHARED_ASIDE (default 1): batches over 32 tokens run the shared expert's two GEMMs (which do not depend
+ * on the routing) on the context's side stream from the start of the call, next to the router launch; 0 = the shared
+ * expert's tiles ride in the routed experts' launches.  Same arithmetic either way. */
+enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2, MOE_OPT_FUSED_COMBINE = 3, MOE_OPT_SHARED_ASIDE = 4 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP
