@@ -401,6 +401,8 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
 }
 
 // ---- softmax + top-k, one wave per token (E <= 64*NPL) ----
+// Lane l holds experts NPL*l .. NPL*l + NPL - 1 (lane-major), so that among equal keys the lowest expert
+// sits in the lowest lane and register, and the selection can pre-sort each lane's keys.
 template <int NPL>
 __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ logits,
                                                      int* __restrict__ ids, float* __restrict__ ws,
@@ -414,7 +416,7 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
   float mxf = -INFINITY;
 #pragma unroll
   for (int j = 0; j < NPL; j++) {
-    const int e = lane + 64 * j;
+    const int e = NPL * lane + j;
     v[j] = e < E ? lg[e] : -INFINITY;
     mxf = fmaxf(mxf, v[j]);
   }
@@ -424,7 +426,7 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
   bool exact = true;  // all partial sums representable -> any summation order gives the same fp64
 #pragma unroll
   for (int j = 0; j < NPL; j++) {
-    const int e = lane + 64 * j;
+    const int e = NPL * lane + j;
     p[j] = e < E ? (float)exp((double)v[j] - mx) : 0.f;
     exact = exact && (p[j] == 0.f || p[j] >= 0x1p-20f);
   }
@@ -437,7 +439,7 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
   } else {
     // very wide logit range: replay the reference's index order on one lane
 #pragma unroll
-    for (int j = 0; j < NPL; j++) pbuf[wv][lane + 64 * j] = p[j];
+    for (int j = 0; j < NPL; j++) pbuf[wv][NPL * lane + j] = p[j];
     __builtin_amdgcn_s_waitcnt(0);
     __builtin_amdgcn_wave_barrier();
     double s = 0.0;
@@ -450,10 +452,11 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
   uint32_t key[NPL];
 #pragma unroll
   for (int j = 0; j < NPL; j++) {
-    const int e = lane + 64 * j;
+    const int e = NPL * lane + j;
     key[j] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
   }
-  topk_select<NPL>(key, lane, k, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride);
+  if constexpr (NPL <= 8) topk_select_sorted<NPL>(key, lane, k, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride);
+  else topk_select_lm<NPL>(key, lane, k, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride);
 }
 
 template <int NPL>
