@@ -28,7 +28,7 @@ LIB_OPTIONS = []              # (option id, value) pairs of --opt, applied to ev
 # HBM bytes per launch of the dominant kernel (read + written) at the default shapes, from the
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic.txt (counters
 # cannot be read from inside this process; other shapes report null)
-PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4543.03e6, ("decode", "q4cp", 1): 29.60e6}
+PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4569.79e6, ("decode", "q4cp", 1): 29.60e6}
 CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
 
 

@@ -568,8 +568,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     const int max_tiles = (P * g.topk + 127) / 128 + g.experts;
     MOE_HIP(hipEventRecord(c->ev_fork, st));
     MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
-    int rs = moe_launch_row_meansq(x, P, g.d, c->xms, c->side);
-    if (!rs) rs = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
+    int rs = moe_launch_f16_rows_meansq(x, c->x16, P, g.d, q4k ? 2 : 1, c->xms, c->side);
     hipError_t ee = hipEventRecord(c->ev_x16, c->side);
     if (!rs && ee != hipSuccess) rs = (int)ee;
     if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, 128, P, sh_first, c->tokidx, c->side);

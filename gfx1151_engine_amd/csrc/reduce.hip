@@ -47,6 +47,41 @@ __global__ void __launch_bounds__(256) k_f32_to_f16_q4k(const float4* __restrict
   }
 }
 
+// The f16 copy of whole rows in layout 1 or 2 plus each row's mean square (the f16 range guard's input) in
+// one pass over x: a wave per row, lanes take the row's 8-element chunks in turn.
+template <int LAYOUT>
+__global__ void __launch_bounds__(256) k_f32_to_f16_rows(const float* __restrict__ x, uint4* __restrict__ y, int P,
+                                                         int d, float* __restrict__ xms) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= P) return;
+  const float4* xr = (const float4*)(x + (size_t)t * d);
+  uint4* yr = y + (size_t)t * (d / 8);
+  float acc = 0.f;
+  for (int i = lane; i < d / 8; i += 64) {
+    float4 u, v;
+    __half2 a, b, c, e;
+    if (LAYOUT == 2) {
+      const int blk = i >> 3, w = i & 7;
+      u = xr[blk * 16 + w];
+      v = xr[blk * 16 + 8 + w];
+      a = __floats2half2_rn(u.x, u.z); b = __floats2half2_rn(v.x, v.z);
+      c = __floats2half2_rn(u.y, u.w); e = __floats2half2_rn(v.y, v.w);
+    } else {
+      u = xr[2 * i];
+      v = xr[2 * i + 1];
+      a = __floats2half2_rn(u.x, v.x); b = __floats2half2_rn(u.y, v.y);
+      c = __floats2half2_rn(u.z, v.z); e = __floats2half2_rn(u.w, v.w);
+    }
+    acc += ((u.x * u.x + u.y * u.y) + (u.z * u.z + u.w * u.w)) + ((v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w));
+    uint4 o;
+    o.x = *(const uint32_t*)&a; o.y = *(const uint32_t*)&b; o.z = *(const uint32_t*)&c; o.w = *(const uint32_t*)&e;
+    yr[i] = o;
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (lane == 0) xms[t] = acc / (float)d;
+}
+
 // out[t][c] = sum_{s<K} pw[pid_s] * pairs[pid_s][c]  (pid_s = pairids[t*K+s], ascending expert id)
 //            + sigmoid(sg[t]) * ey[t][c]             (ey f32, or row `sh_first + t` of pairs)
 // One thread per 8 consecutive columns (16-byte loads of f16 pairs); grid (ceil(D/8/256), P).
@@ -214,20 +249,6 @@ __global__ void __launch_bounds__(256) k_tiles_only_shared(moe_tile* __restrict_
   for (int i = i0; i < P; i += stride) tokidx[sh_first + i] = i;
 }
 
-// Mean square of each token's activations (input of the f16 range guard): one wave per token.
-__global__ void __launch_bounds__(256) k_row_meansq(const float* __restrict__ x, int P, int d, float* __restrict__ out) {
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (t >= P) return;
-  const float4* row = (const float4*)(x + (size_t)t * d);
-  float acc = 0.f;
-  for (int i = lane; i < d / 4; i += 64) {
-    const float4 v = row[i];
-    acc += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
-  }
-#pragma unroll
-  for (int o = 32; o; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (lane == 0) out[t] = acc / (float)d;
-}
 }  // namespace
 
 int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, int P, int sh_first, int* tokidx,
@@ -238,10 +259,13 @@ int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, i
   return MOE_OK;
 }
 
-int moe_launch_row_meansq(const float* x, int P, int d, float* out, hipStream_t st) {
-  if (!x || !out || d % 4 || !moe_aligned(x, 16)) return MOE_E_INVALID;
+// x16 (layout 1 or 2) and the mean square of every row in one launch
+int moe_launch_f16_rows_meansq(const float* x, void* x16, int P, int d, int layout, float* xms, hipStream_t st) {
+  if (!x || !x16 || !xms || (layout != 1 && layout != 2)) return MOE_E_INVALID;
+  if (d % 8 || (layout == 2 && d % 64) || !moe_aligned(x, 16) || !moe_aligned(x16, 16)) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
-  k_row_meansq<<<(P + 3) / 4, 256, 0, st>>>(x, P, d, out);
+  if (layout == 2) k_f32_to_f16_rows<2><<<(P + 3) / 4, 256, 0, st>>>(x, (uint4*)x16, P, d, xms);
+  else k_f32_to_f16_rows<1><<<(P + 3) / 4, 256, 0, st>>>(x, (uint4*)x16, P, d, xms);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
