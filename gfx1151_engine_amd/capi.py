@@ -268,6 +268,13 @@ def reduce_pw_sg(pairs, pairids, pw, P, K, ey=None, sg=None):
     return out
 
 
+def reduce_pw_sg_hc(pairs, pairids, pw, P, K, w4, R, ey=None, sg=None):
+    D = pairs.shape[1]
+    check(lib().moe_reduce_pw_sg_hc(ptr(pairs), 1 if pairs.dtype == torch.float16 else 0, ptr(pairids), ptr(pw),
+                                    ptr(ey), ptr(sg), ptr(w4), ptr(R), P, D, K, stream()), "moe_reduce_pw_sg_hc")
+    return R
+
+
 # ---- model level ----
 
 class Moe:
@@ -304,6 +311,11 @@ class Moe:
             y = torch.empty((P, self.cfg.d), dtype=torch.float32, device=x.device)
         check(lib().moe_forward(self.h, layer, ptr(x), P, ptr(y), stream()), "moe_forward")
         return y
+
+    def forward_hc(self, layer, x, w4, R):
+        """moe_b(try_hcw): the combine writes into the bf16 HC state R [P][4][d] (int16 tensor of bf16 bits)."""
+        check(lib().moe_forward_hc(self.h, layer, ptr(x), x.shape[0], ptr(w4), ptr(R), stream()), "moe_forward_hc")
+        return R
 
     def set_option(self, option, value):
         check(lib().moe_set_option(self.h, option, value), "moe_set_option")

@@ -84,6 +84,7 @@ struct moe_ctx {
   // batch path, shared expert on the side stream: its tile list and the switch
   moe_tile* tiles_sh = nullptr;
   int* ntiles_sh = nullptr;
+  const moe_hc* hc = nullptr;  // set for the duration of moe_forward_hc: the combine writes into the HC state
   bool shared_aside = true;
 };
 
@@ -453,7 +454,7 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
         return rc;
       prof_mark(c, MOE_PROF_DOWN, st);
       rc = moe_launch_reduce(c->pairs32, false, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
-                             sh_first, y, P, g.d, g.topk, moe_hscale{nullptr, 0.f, 0.f}, st);
+                             sh_first, y, P, g.d, g.topk, moe_hscale{nullptr, 0.f, 0.f}, st, nullptr);
       prof_mark(c, MOE_PROF_REDUCE, st);
       return rc;
     }
@@ -558,7 +559,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   c->ev_n = 0;
   prof_mark(c, 0, st);
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
-  if (L.has_shared && c->shared_aside && !c->fused_combine) {
+  if (L.has_shared && c->shared_aside && (!c->fused_combine || c->hc)) {
     // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
     // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
     // side stream also makes what both streams need first: the per-token mean square of x (range guard) and
@@ -604,7 +605,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     if (rs) return rs;
     if (ee != hipSuccess) return (int)ee;
     rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, c->sh_logit, sh_first, y, P, g.d, g.topk, hs,
-                           st);
+                           st, c->hc);
     prof_mark(c, MOE_PROF_REDUCE, st);
     return rc;
   }
@@ -616,7 +617,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   MOE_HIP(hipEventRecord(c->ev_fork, st));
   MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
   int rc16 = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
-  const bool fused = c->fused_combine;
+  const bool fused = c->fused_combine && !c->hc;  // the HC write-back belongs to the ordered combine
   if (fused && !rc16) rc16 = moe_launch_zero_f32(y, (uint64_t)P * g.d, c->side);  // after the last read of x
   // the side stream is joined on every path out of here (a capture on `st` must not end with it forked)
   auto join = [&]() -> int {
@@ -653,7 +654,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     return rc;
   prof_mark(c, MOE_PROF_DOWN, st);
   rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
-                         sh_first, y, P, g.d, g.topk, hs, st);
+                         sh_first, y, P, g.d, g.topk, hs, st, c->hc);
   prof_mark(c, MOE_PROF_REDUCE, st);
   return rc;
 }
@@ -675,4 +676,23 @@ MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, 
     if (r2) return r2;
   }
   return MOE_OK;
+}
+
+// GpuModel::moe_b(l, P, try_hcw = true) (src/gpu/parts/40_model.inc:4018,4082-4094): the batch call with the HC
+// write-back fused into the combine.  MOE_E_UNSUPPORTED (nothing enqueued) where the reference returns false:
+// batches of at most 32 tokens and formats outside the grouped GEMM; the caller then runs moe_forward and its own
+// write-back.
+MOE_API int moe_forward_hc(moe_ctx* c, int layer, const float* x, int P, const float* w4, uint16_t* R,
+                           moe_stream_t st) {
+  MoeLayer* L = layer_of(c, layer);
+  if (!L || !x || !w4 || !R || P < 0) return MOE_E_INVALID;
+  if (!L->has_router || !(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
+  if (P > c->cfg.max_tokens) return MOE_E_STATE;
+  if (!moe_aligned(x, 16) || !moe_aligned(R, 16)) return MOE_E_INVALID;
+  if (P <= c->small_max) return MOE_E_UNSUPPORTED;
+  const moe_hc hc{w4, R};
+  c->hc = &hc;
+  const int rc = forward_batch(c, *L, x, P, nullptr, moe_s(st));
+  c->hc = nullptr;
+  return rc;
 }

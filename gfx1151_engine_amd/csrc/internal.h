@@ -18,6 +18,12 @@ struct moe_comb {
   const float* sg;
 };
 
+// HC write-back fused into the combine: w4 = inject gate logits [P][4], R = bf16 state [P][4][d]
+struct moe_hc {
+  const float* w4;
+  uint16_t* R;
+};
+
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
@@ -56,7 +62,7 @@ int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E
                             int sh_first, int* tokidx, hipStream_t st);
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
                       const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
-                      moe_hscale hs, hipStream_t st);
+                      moe_hscale hs, hipStream_t st, const moe_hc* hc);
 int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
                           float* logits, float* out_x, float* out_xms, hipStream_t st);
 

@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pai
                                                       const float* __restrict__ ey,
                                                       const float* __restrict__ sg, int sh_first,
                                                       float* __restrict__ out, int P, int D, int K,
-                                                      moe_hscale hs) {
+                                                      moe_hscale hs, moe_hc hc) {
   __shared__ int ids[KMAX];
   __shared__ float w[KMAX];
   const int t = blockIdx.y;
@@ -173,6 +173,32 @@ __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pai
     else Ld8<PT>::ld(pairs + (size_t)(sh_first + t) * D + c, v);
 #pragma unroll
     for (int i = 0; i < 8; i++) sum[i] += g * v[i];
+  }
+  if (hc.R) {
+    // HC write-back fused into the combine (reference: k_moe_reduce_pw_sg_hc, 24_kernels_moe_lt.inc:126-161):
+    // the four branches of the bf16 state R[t][b][:] take inj_b * sum, inj_b = 2 * sigmoid(w4[t][b] / 4);
+    // bf16 <-> f32 as the reference's bf2f / f2bf (22_kernels_prefill.inc:4-9: round to nearest even)
+    float inj[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++) inj[b] = 2.f / (1.f + expf(-hc.w4[(size_t)t * 4 + b] * 0.25f));
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+      uint4* Rp = (uint4*)(hc.R + ((size_t)t * 4 + b) * D + c);
+      const uint4 rv = *Rp;
+      const uint32_t w[4] = {rv.x, rv.y, rv.z, rv.w};
+      uint32_t o[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float lo = __uint_as_float(w[i] << 16) + inj[b] * sum[2 * i];
+        const float hi = __uint_as_float(w[i] & 0xffff0000u) + inj[b] * sum[2 * i + 1];
+        uint32_t ul = __float_as_uint(lo), uh = __float_as_uint(hi);
+        ul += 0x7FFFu + ((ul >> 16) & 1u);
+        uh += 0x7FFFu + ((uh >> 16) & 1u);
+        o[i] = (ul >> 16) | (uh & 0xffff0000u);
+      }
+      *Rp = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    return;
   }
   float4* o = (float4*)(out + (size_t)t * D + c);
   o[0] = make_float4(sum[0], sum[1], sum[2], sum[3]);
@@ -279,14 +305,19 @@ int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E
 
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
                       const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
-                      moe_hscale hs, hipStream_t st) {
-  if (!pairs || !pairids || !pw || !out) return MOE_E_INVALID;
+                      moe_hscale hs, hipStream_t st, const moe_hc* hcp) {
+  moe_hc hc{nullptr, nullptr};
+  if (hcp) {  // results go into the bf16 HC state instead of out
+    if (!hcp->w4 || !hcp->R || !moe_aligned(hcp->R, 16)) return MOE_E_INVALID;
+    hc = *hcp;
+  }
+  if (!pairs || !pairids || !pw || (!out && !hc.R)) return MOE_E_INVALID;
   if (P < 0 || D < 1 || K < 1) return MOE_E_INVALID;
   if (K > 16 || D % 8) return MOE_E_UNSUPPORTED;
-  if (!moe_aligned(pairs, 16) || !moe_aligned(out, 16) || (ey && !moe_aligned(ey, 16))) return MOE_E_INVALID;
+  if (!moe_aligned(pairs, 16) || (out && !moe_aligned(out, 16)) || (ey && !moe_aligned(ey, 16))) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
   dim3 grid((D / 8 + 127) / 128, P);
-#define RED_GO(PT, KC) k_reduce_pw_sg<PT, 16, KC><<<grid, 128, 0, st>>>((const PT*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs)
+#define RED_GO(PT, KC) k_reduce_pw_sg<PT, 16, KC><<<grid, 128, 0, st>>>((const PT*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs, hc)
   if (pairs_f16) {
     if (K == 10) RED_GO(__half, 10); else if (K == 8) RED_GO(__half, 8); else RED_GO(__half, 0);
   } else {
@@ -327,5 +358,14 @@ MOE_API int moe_reduce_pw_sg(const void* pairs, int pairs_f16, const int* pairid
                              moe_stream_t st) {
   if ((ey == nullptr) != (sg == nullptr)) return MOE_E_INVALID;
   return moe_launch_reduce(pairs, pairs_f16 != 0, pairids, pw, ey, sg, -1, out, P, D, K, moe_hscale{nullptr, 0.f, 0.f},
-                           moe_s(st));
+                           moe_s(st), nullptr);
+}
+
+MOE_API int moe_reduce_pw_sg_hc(const void* pairs, int pairs_f16, const int* pairids, const float* pw,
+                                const float* ey, const float* sg, const float* w4, uint16_t* R, int P, int D, int K,
+                                moe_stream_t st) {
+  if ((ey == nullptr) != (sg == nullptr) || !w4 || !R) return MOE_E_INVALID;
+  const moe_hc hc{w4, R};
+  return moe_launch_reduce(pairs, pairs_f16 != 0, pairids, pw, ey, sg, -1, nullptr, P, D, K,
+                           moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), &hc);
 }

@@ -173,6 +173,13 @@ int moe_gg_down(int type, const uint8_t* down, const void* hid16, const moe_tile
 int moe_reduce_pw_sg(const void* pairs, int pairs_f16, const int* pairids, const float* pw,
                      const float* ey, const float* sg, float* out, int P, int D, int K,
                      moe_stream_t st);
+/* k_moe_reduce_pw_sg_hc (src/gpu/parts/24_kernels_moe_lt.inc:126-161): the same combine with the HC write-back
+ * folded in - instead of storing the f32 result, the four branches of the bf16 state take it:
+ * R[t][b][c] = bf16(f32(R[t][b][c]) + inj_b * sum), inj_b = 2 / (1 + exp(-w4[t][b] / 4)), b = 0..3.
+ * w4: f32 [P][4] (inject gate logits), R: bf16 [P][4][D] (16-byte aligned), D % 8 == 0. */
+int moe_reduce_pw_sg_hc(const void* pairs, int pairs_f16, const int* pairids, const float* pw,
+                        const float* ey, const float* sg, const float* w4, uint16_t* R, int P, int D, int K,
+                        moe_stream_t st);
 
 /* ---- model level ---- */
 
@@ -208,6 +215,11 @@ int moe_set_shared(moe_ctx* ctx, int layer, const moe_wview* gate_proj, const mo
  * events inside the call, so work queued on st after the call is ordered after all of it, and a stream
  * capture on st takes that stream in and closes it again. */
 int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_stream_t st);
+/* GpuModel::moe_b(l, P, try_hcw = true) (40_model.inc:4018,4082-4094): the batch call with the HC write-back fused
+ * into the combine (moe_reduce_pw_sg_hc above); no f32 output is written.  Returns MOE_E_UNSUPPORTED, with nothing
+ * enqueued, where the reference's call returns false (P <= 32, formats outside the grouped GEMM): the caller then
+ * runs moe_forward and its own write-back. */
+int moe_forward_hc(moe_ctx* ctx, int layer, const float* x, int P, const float* w4, uint16_t* R, moe_stream_t st);
 /* Switches in the spirit of the reference's QWENOX_* opt-outs (src/gpu/parts/40_model.inc:1959-1996):
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
  * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as

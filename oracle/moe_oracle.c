@@ -17,6 +17,7 @@
  *   src/ref.cpp:68-77    matvec: fp64 sequential accumulate, f32 result
  *   src/ref.cpp:563-637  Model::moe (router, top-k, experts, shared expert)
  *   src/gpu/parts/10_ple_io.inc:784-825  expert-sorted permutation + tiles
+ *   src/gpu/parts/24_kernels_moe_lt.inc:126-161  HC write-back folded into the combine
  *
  * Pinning status of every function is listed in oracle/README.md; each one is
  * checked in tests/ against the reference's own code built under oracle/_ref
@@ -553,4 +554,23 @@ ORC_API void orc_set_threads(int n) {
 #else
   (void)n;
 #endif
+}
+
+/* ---- HC write-back of the combine: src/gpu/parts/24_kernels_moe_lt.inc:126-161 ----
+ * R[t][b][c] = f2bf(bf2f(R[t][b][c]) + inj_b * y[t][c]), inj_b = 2 / (1 + expf(-w4[t][b] * 0.25f)), b = 0..3;
+ * f2bf = round to nearest even by the bit trick of src/gpu/parts/22_kernels_prefill.inc:4-9.  The reference
+ * expression is compiled for the GPU with contraction on, i.e. as one fused multiply-add: fmaf here. */
+static inline uint16_t f2bf_ref(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  u += 0x7FFF + ((u >> 16) & 1);
+  return (uint16_t)(u >> 16);
+}
+ORC_API void orc_hc_writeback(const float* y, const float* w4, uint16_t* R, int P, int D) {
+  for (int t = 0; t < P; t++)
+    for (int b = 0; b < 4; b++) {
+      const float inj = 2.f / (1.f + expf(-w4[(size_t)t * 4 + b] * 0.25f));
+      uint16_t* Rt = R + ((size_t)t * 4 + b) * D;
+      for (int c = 0; c < D; c++) Rt[c] = f2bf_ref(fmaf(inj, y[(size_t)t * D + c], bf16_to_f32(Rt[c])));
+    }
 }

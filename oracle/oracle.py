@@ -370,3 +370,15 @@ def layer_from_device(dl):
     return Layer(d, mid, E, k, router, Mat(wt, h(dl.down), E * d, mid),
                  gate=Mat(wt, h(dl.gate), E * mid, d), up=Mat(wt, h(dl.up), E * mid, d),
                  shared=sh, router_bias=bias)
+
+
+def hc_writeback(y, w4, R):
+    """R (uint16 bf16 bits [P][4][D]) after the HC write-back of y (f32 [P][D]) with inject gate logits w4 [P][4]
+    (src/gpu/parts/24_kernels_moe_lt.inc:126-161); returns a new array."""
+    y = _c(y, np.float32)
+    w4 = _c(w4, np.float32)
+    out = np.ascontiguousarray(R, np.uint16).copy()
+    P, D = y.shape
+    assert w4.shape == (P, 4) and out.shape == (P, 4, D)
+    lib().orc_hc_writeback(_p(y), _p(w4), _p(out), C.c_int(P), C.c_int(D))
+    return out

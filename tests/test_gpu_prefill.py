@@ -186,3 +186,46 @@ def test_batch_equals_small_path_statistically(oracle):
     ys = np.concatenate([m.forward(0, xb[:20].contiguous()).cpu().numpy(), m.forward(0, xb[20:].contiguous()).cpu().numpy()])
     assert max_abs_rel(yb, ys) <= TOL_LAYER
     m.close()
+
+
+@pytest.mark.parametrize("fmt", ["q4cp", "q4k"])
+def test_forward_hc_writeback(oracle, fmt):
+    """moe_forward_hc (the reference's moe_b with try_hcw): the combine adds into the bf16 HC state instead of
+    writing f32.  Against the oracle's write-back applied to moe_forward's own output: identical where the gate
+    logit is 0 (inj = 1 exactly); elsewhere device and host expf may differ in the last bit of inj, which can move
+    a result across a bf16 rounding boundary: at most one bf16 step at the operands' size, in well under 1 % of the
+    elements.  Batches
+    of at most 32 tokens are refused, as the reference's call returns false there."""
+    import torch
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(77)
+    d, mid, E, k, T = 512, 256, 12, 4, 150
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt)
+    x = S.bf16_round(rng.standard_normal((T, d), dtype=np.float32))
+    m, dev = hl.to_gpu(max_tokens=T)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    w4 = rng.standard_normal((T, 4)).astype(np.float32) * 2
+    w4[:, 0] = 0.0
+    R0 = (rng.standard_normal((T, 4, d)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    want = oracle.hc_writeback(y, w4, R0)
+    R = torch.from_numpy(R0.view(np.int16).copy()).cuda()
+    m.forward_hc(0, gpu(x), gpu(w4), R)
+    got = R.cpu().numpy().view(np.uint16)
+    assert (got[:, 0] == want[:, 0]).all()
+    gv, wv = ((a.astype(np.uint32) << 16).view(np.float32) for a in (got, want))
+    r0 = (R0.astype(np.uint32) << 16).view(np.float32)
+    step = 2.0 ** -7 * (np.abs(r0) + 2 * np.abs(y)[:, None, :])  # a bf16 step at the operands' size (sums may cancel)
+    assert (np.abs(gv - wv) <= step).all() and (got != want).mean() < 0.01, (got != want).mean()
+    with pytest.raises(capi.MoeError):
+        m.forward_hc(0, gpu(x[:8]), gpu(w4[:8]), R)
+    # stage level: the same kernel behind moe_reduce_pw_sg_hc, no shared expert, f32 pairs
+    P2, K2 = 40, 3
+    pairs = rng.standard_normal((P2 * K2, d)).astype(np.float32)
+    pairids = rng.permutation(P2 * K2).astype(np.int32).reshape(P2, K2)
+    pw = rng.random(P2 * K2).astype(np.float32)
+    y2 = capi.reduce_pw_sg(gpu(pairs), gpu(pairids), gpu(pw), P2, K2).cpu().numpy()
+    R2 = torch.from_numpy(R0[:P2].view(np.int16).copy()).cuda()
+    z4 = np.zeros((P2, 4), np.float32)
+    capi.reduce_pw_sg_hc(gpu(pairs), gpu(pairids), gpu(pw), P2, K2, gpu(z4), R2)
+    assert (R2.cpu().numpy().view(np.uint16) == oracle.hc_writeback(y2, z4, R0[:P2])).all()
+    m.close()

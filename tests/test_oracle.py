@@ -330,3 +330,40 @@ def test_gg_rows_against_reference(oracle, t, name):
         x1 = (qs >> 4) | (((qh >> (j + 16)) & 1) << 4)
         y = np.concatenate([x0, x1], 1).astype(np.float32) * d + m
         assert (y.reshape(rows, cols).view(np.uint32) == got.view(np.uint32)).all()
+
+
+def test_hc_writeback_closed_forms(oracle):
+    """HC write-back of the combine (src/gpu/parts/24_kernels_moe_lt.inc:126-161).  Cases that the formula fixes
+    without retyping it: gate logit 0 gives inj = 1 exactly, so R' = bf16(R + y) (checked against an independent
+    round-to-nearest-even through float64 arithmetic on values where the sum is exact in f32); a very negative logit
+    gives inj = 0 and leaves R as it is; a very positive one gives inj = 2; halfway cases round to even."""
+    O = oracle
+    rng = np.random.default_rng(4)
+    P, D = 3, 64
+    # small integers: every R + y below is exact in f32 and in f64
+    y = rng.integers(-200, 200, (P, D)).astype(np.float32)
+    Rf = rng.integers(-100, 100, (P, 4, D)).astype(np.float32)
+    R = (Rf.view(np.uint32) >> 16).astype(np.uint16)  # small integers are exact in bf16
+    w4 = np.zeros((P, 4), np.float32)
+    w4[:, 1] = -1e4   # inj = 2 / (1 + inf) = 0
+    w4[:, 2] = 1e4    # inj = 2 / (1 + 0) = 2
+    got = O.hc_writeback(y, w4, R)
+
+    def bf16_rne(a64):  # independent: nearest bf16 of exactly representable reals, ties to even
+        a = a64.astype(np.float32)
+        u = a.view(np.uint32).astype(np.uint64)
+        low = u & 0xFFFF
+        up = u >> 16
+        rnd = (low > 0x8000) | ((low == 0x8000) & ((up & 1) == 1))
+        return (up + rnd).astype(np.uint16)
+    assert (got[:, 0] == bf16_rne(Rf[:, 0].astype(np.float64) + y)).all()
+    assert (got[:, 3] == bf16_rne(Rf[:, 3].astype(np.float64) + y)).all()
+    assert (got[:, 1] == R[:, 1]).all()
+    assert (got[:, 2] == bf16_rne(Rf[:, 2].astype(np.float64) + 2.0 * y)).all()
+    # ties: 257 = 0x1.01p8 lies halfway between the bf16 neighbours 256 and 258 -> 256 (even); 259 -> 260
+    y2 = np.array([[1.0, 3.0]], np.float32)
+    R2 = np.zeros((1, 4, 2), np.uint16)
+    R2[:] = (np.float32(256.0).view(np.uint32) >> 16).astype(np.uint16)
+    out = O.hc_writeback(y2, np.zeros((1, 4), np.float32), R2)
+    vals = (out.astype(np.uint32) << 16).view(np.float32)
+    assert (vals[0, :, 0] == 256.0).all() and (vals[0, :, 1] == 260.0).all()
