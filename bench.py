@@ -2,7 +2,7 @@
 """Benchmark of the routed-expert MoE layer on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
-                  [--workload headline|prefill|decode|verify|q4k_prefill|q4k_decode|stack]
+                  [--workload headline|prefill|decode|verify|q4k_prefill|q4k_decode|stack|ggmix_decode|ggmix_verify]
 
 One step = one pass of the MoE layer (moe_forward) over one batch of synthetic input that is
 already resident in HBM.  Prints ONE JSON line: whole-layer throughput, the roofline figure of the
@@ -86,12 +86,16 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
     from gfx1151_engine_amd import capi, workloads as W
     from gfx1151_engine_amd import synth as S
     d, mid, k = D, MID, K
-    fmt = "q4k" if wl.startswith("q4k") else "q4cp"
-    kind = wl.replace("q4k_", "")
+    # ggmix_*: GGUF layer in the reference checkpoints' type mix (Q5_K gate/up, Q8_0 down, Q4_K shared expert) on the
+    # general GEMV kernels
+    ggmix = wl.startswith("ggmix_")
+    fmt = "q4k" if wl.startswith("q4k") or ggmix else "q4cp"
+    gg_types = (13, 8, 12) if ggmix else (12, 12, 12)
+    kind = wl.replace("q4k_", "").replace("ggmix_", "")
     T = tokens or {"prefill": 16384 if fmt == "q4cp" else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
     nlayers = nlayers_arg if kind == "stack" else 1
 
-    layers = [W.DeviceLayer(1000 + l, d, mid, E, k, fmt) for l in range(nlayers)]
+    layers = [W.DeviceLayer(1000 + l, d, mid, E, k, fmt, gg_types=gg_types) for l in range(nlayers)]
     g = torch.Generator(device="cuda")
     g.manual_seed(99)
     extra = {}
@@ -163,7 +167,9 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
            "vs_baseline": None, "data": "synthetic", "stage_ms": {kk: round(v, 5) for kk, v in stage.items()},
            "stage_event_overhead_ms": round(stage_overhead, 5)}
     cfg = {"workload": wl, "tokens": T, "d_model": d, "moe_mid": mid, "experts": E, "topk": k, "shared_experts": 1,
-           "format": "q4cp g32 zero-point 8" if fmt == "q4cp" else "GGUF Q4_K", "layers": nlayers, **extra}
+           "format": "q4cp g32 zero-point 8" if fmt == "q4cp" else
+           ("GGUF Q5_K gate/up, Q8_0 down, Q4_K shared expert (general f32 kernels)" if ggmix else "GGUF Q4_K"),
+           "layers": nlayers, **extra}
     if kind == "prefill":
         flop_tok = k * 6 * d * mid + 6 * d * mid + 2 * d * E + 2 * d
         # the timed gate/up launch: the routed experts' pairs; the shared expert's tiles are in the same launch only
@@ -192,13 +198,15 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
         # algorithmic bytes of a step: unique experts + shared expert + fp32 router + gate vector + x/y
         if kind == "stack":
             uniq = k
-        step_bytes = nlayers * ((uniq + 1) * eb + E * d * 4 + d * 4 + T * 2 * d * 4)
-        gu_row = d // 2 + S.q4cp_scale_stride(d) if fmt == "q4cp" else S.q4k_row_bytes(d)
-        gu_bytes = (uniq + 1) * 2 * mid * gu_row
+        step_bytes = nlayers * (uniq * eb + layers[0].shared_bytes() + E * d * 4 + d * 4 + T * 2 * d * 4)
+        if fmt == "q4cp":
+            gu_bytes = (uniq + 1) * 2 * mid * (d // 2 + S.q4cp_scale_stride(d))
+        else:
+            gu_bytes = 2 * mid * (uniq * W.gg_row_bytes(gg_types[0], d) + W.gg_row_bytes(gg_types[2], d))
         up_s = stage["up"] * 1e-3
         res.update({"metric": "moe_layer_decode_hbm_GB_per_s", "unit": "GB/s",
                     "value": round(step_bytes / (ms * 1e-3) / 1e9, 1),
-                    "dtype": "i8" if fmt == "q4cp" else "f32",
+                    "dtype": "f32" if ggmix else "i8",
                     "hbm_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "tokens_per_s": round(T / (ms * 1e-3), 1),
                     "roofline": {"bound": "hbm", "kernel": "gate/up GEMV + SwiGLU",

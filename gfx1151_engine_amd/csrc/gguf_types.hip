@@ -188,7 +188,8 @@ struct GgxArgs {
   const float* sh_logit;
 };
 
-constexpr int GX_ROWS = 16;
+constexpr int GX_ROWS = 8;      // gate rows per block of k_ggx_gu (a wave takes every fourth)
+constexpr int GX_DN_ROWS = 4;   // output rows per block of k_ggx_dn: one per wave, d / 4 blocks fill the chip
 // grid (ceil(mid/GX_ROWS), slots incl. shared, P), block 256: hid[token][slot][row] = silu(gate.x) * (up.x)
 __global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restrict__ x, const int* __restrict__ ids,
                                                 int id_stride, int kpt, int d, int mid, float* __restrict__ hid) {
@@ -213,7 +214,7 @@ __global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restri
   }
 }
 
-// grid (ceil(d/GX_ROWS), P), block 256: y[token][row] = sum over slots of w_s * (down_s . hid_s)
+// grid (ceil(d/GX_DN_ROWS), P), block 256: y[token][row] = sum over slots of w_s * (down_s . hid_s)
 // + sigmoid(shared gate logit) * (shared down . hid_shared)
 __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restrict__ hid, const int* __restrict__ ids,
                                                 const float* __restrict__ ws, int id_stride, int kpt, int d, int mid,
@@ -235,8 +236,8 @@ __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restri
   // a wave per row; its lanes take the (slot, 32-element block) units in turn, each weighted by the slot's
   // combine weight, so a row needs one wave-wide sum (a fixed order: the result does not depend on timing)
   const int nb = mid / 32;
-  for (int rr = wv; rr < GX_ROWS; rr += 4) {
-    const int r = blockIdx.x * GX_ROWS + rr;
+  for (int rr = wv; rr < GX_DN_ROWS; rr += 4) {
+    const int r = blockIdx.x * GX_DN_ROWS + rr;
     if (r >= d) break;
     float acc = 0.f;
     for (int u = lane; u < nslots * nb; u += 64) {
@@ -312,7 +313,7 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
     MOE_LAUNCH_CHECK();
   }
   if (phase != 1) {
-    dim3 grid((d + GX_ROWS - 1) / GX_ROWS, P);
+    dim3 grid((d + GX_DN_ROWS - 1) / GX_DN_ROWS, P);
     k_ggx_dn<<<grid, 256, (size_t)nslots * mid / 32 * 33 * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
     MOE_LAUNCH_CHECK();
   }

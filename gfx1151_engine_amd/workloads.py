@@ -59,12 +59,47 @@ def q4k_rows(g, rows, cols, scale_std=0.01):
     return blk.view(-1)
 
 
-class DeviceLayer:
-    """One layer's weights in HBM + registration into a capi.Moe context."""
+GG_ROW_BYTES = {12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24)}  # ggml type -> (block elements, bytes)
 
-    def __init__(self, seed, d=3072, mid=768, E=512, k=10, fmt="q4cp", bias=None):
+
+def gg_row_bytes(t, cols):
+    be, bb = GG_ROW_BYTES[t]
+    return cols // be * bb
+
+
+def gg_rows(g, t, rows, cols, scale_std=0.01):
+    """uint8 tensor of raw rows of ggml type t: Q4_K (12), Q5_K (13), Q8_0 (8) or Q5_1 (7); integer fields uniform,
+    fp16 fields |N|*std scaled so that weights have the size of the Q4_K ones."""
+    if t == 12:
+        return q4k_rows(g, rows, cols, scale_std)
+    be, bb = GG_ROW_BYTES[t]
+    nb = rows * cols // be
+    blk = torch.empty((nb, bb), dtype=torch.uint8, device="cuda")
+    step = max(1, (1 << 28) // bb)
+    for i in range(0, nb, step):
+        n = min(step, nb - i)
+        blk[i:i + n] = torch.randint(0, 256, (n, bb), dtype=torch.uint8, device="cuda", generator=g)
+    if t == 13:    # d, dmin, packed 6-bit scales (any bytes are valid), qh, ql
+        dd = (torch.randn((nb, 2), device="cuda", generator=g).abs() * scale_std / 2).to(torch.float16)
+        blk[:, 0:4] = dd.view(torch.uint8)
+    elif t == 8:   # d, 32 x int8
+        dd = (torch.randn((nb, 1), device="cuda", generator=g).abs() * scale_std / 8).to(torch.float16)
+        blk[:, 0:2] = dd.view(torch.uint8)
+    else:          # Q5_1: d, m = -16 d, qh, qs
+        dd = (torch.randn((nb, 1), device="cuda", generator=g).abs() * scale_std / 2).to(torch.float16)
+        blk[:, 0:2] = dd.view(torch.uint8)
+        blk[:, 2:4] = (dd.float() * -16).to(torch.float16).view(torch.uint8)
+    return blk.view(-1)
+
+
+class DeviceLayer:
+    """One layer's weights in HBM + registration into a capi.Moe context.
+    fmt "q4k": raw GGUF blocks, gg_types = ggml types of (gate/up, down, shared expert)."""
+
+    def __init__(self, seed, d=3072, mid=768, E=512, k=10, fmt="q4cp", bias=None, gg_types=(12, 12, 12)):
         g = _gen(seed)
         self.d, self.mid, self.E, self.k, self.fmt = d, mid, E, k, fmt
+        self.tgu, self.tdn, self.tsh = gg_types
         self.router = torch.randn((E, d), device="cuda", generator=g) * 0.02
         self.sh_sg = torch.randn((1, d), device="cuda", generator=g) * 0.02
         self.bias = bias
@@ -73,16 +108,22 @@ class DeviceLayer:
             self.down = q4cp_blob(g, E * d, mid)
             self.sh = [q4cp_blob(g, mid, d), q4cp_blob(g, mid, d), q4cp_blob(g, d, mid)]
         else:
-            self.gate = q4k_rows(g, E * mid, d)
-            self.up = q4k_rows(g, E * mid, d)
-            self.down = q4k_rows(g, E * d, mid)
-            self.sh = [q4k_rows(g, mid, d), q4k_rows(g, mid, d), q4k_rows(g, d, mid)]
+            self.gate = gg_rows(g, self.tgu, E * mid, d)
+            self.up = gg_rows(g, self.tgu, E * mid, d)
+            self.down = gg_rows(g, self.tdn, E * d, mid)
+            self.sh = [gg_rows(g, self.tsh, mid, d), gg_rows(g, self.tsh, mid, d), gg_rows(g, self.tsh, d, mid)]
 
     def expert_bytes(self):
         d, mid = self.d, self.mid
         if self.fmt == "q4cp":
             return 2 * mid * (d // 2 + S.q4cp_scale_stride(d)) + d * (mid // 2 + S.q4cp_scale_stride(mid))
-        return 2 * mid * S.q4k_row_bytes(d) + d * S.q4k_row_bytes(mid)
+        return 2 * mid * gg_row_bytes(self.tgu, d) + d * gg_row_bytes(self.tdn, mid)
+
+    def shared_bytes(self):
+        d, mid = self.d, self.mid
+        if self.fmt == "q4cp":
+            return self.expert_bytes()
+        return 2 * mid * gg_row_bytes(self.tsh, d) + d * gg_row_bytes(self.tsh, mid)
 
     def register(self, m, layer=0):
         d, mid, E = self.d, self.mid, self.E
@@ -92,8 +133,8 @@ class DeviceLayer:
                                capi.wview(self.down, capi.Q4CP, E * d, mid))
             wt, gt = capi.Q4CP, 0
         else:
-            m.set_experts_gguf(layer, self.gate, self.up, self.down)
-            wt, gt = 0, capi.GGML_Q4_K
+            m.set_experts_gguf(layer, self.gate, self.up, self.down, self.tgu, self.tdn)
+            wt, gt = 0, self.tsh
         m.set_shared(layer, capi.wview(self.sh[0], wt, mid, d), capi.wview(self.sh[1], wt, mid, d),
                      capi.wview(self.sh[2], wt, d, mid), capi.wview(self.sh_sg, capi.F32, 1, d), gt)
 

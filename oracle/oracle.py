@@ -359,16 +359,18 @@ def layer_from_device(dl):
     gfx1151_engine_amd.workloads.DeviceLayer), copied to the host.  Checker side only."""
     d, mid, E, k = dl.d, dl.mid, dl.E, dl.k
     wt = Q4CP if dl.fmt == "q4cp" else Q4K
+    tgu, tdn, tsh = (getattr(dl, a, Q4K) for a in ("tgu", "tdn", "tsh"))  # ggml types of a raw-block layer
+    st = wt if dl.fmt == "q4cp" else tsh
     h = lambda t: t.cpu().numpy()
-    sh = [Mat(wt, h(dl.sh[0]), mid, d), Mat(wt, h(dl.sh[1]), mid, d), Mat(wt, h(dl.sh[2]), d, mid),
+    sh = [Mat(st, h(dl.sh[0]), mid, d), Mat(st, h(dl.sh[1]), mid, d), Mat(st, h(dl.sh[2]), d, mid),
           Mat(F32, h(dl.sh_sg), 1, d)]
     router = Mat(F32, h(dl.router), E, d)
     bias = h(dl.bias) if dl.bias is not None else None
     if dl.fmt == "q4cp":
         return Layer(d, mid, E, k, router, Mat(wt, h(dl.down), E * d, mid),
                      gate_up=Mat(wt, h(dl.gate_up), E * 2 * mid, d), shared=sh, router_bias=bias)
-    return Layer(d, mid, E, k, router, Mat(wt, h(dl.down), E * d, mid),
-                 gate=Mat(wt, h(dl.gate), E * mid, d), up=Mat(wt, h(dl.up), E * mid, d),
+    return Layer(d, mid, E, k, router, Mat(tdn, h(dl.down), E * d, mid),
+                 gate=Mat(tgu, h(dl.gate), E * mid, d), up=Mat(tgu, h(dl.up), E * mid, d),
                  shared=sh, router_bias=bias)
 
 
