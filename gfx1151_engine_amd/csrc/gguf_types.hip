@@ -161,23 +161,88 @@ __device__ __forceinline__ float wave_sum_f(float v) {
 // 32-element blocks at the same offset, which without the padding is the same bank for every lane.
 #define GX_PAD(i) ((i) + ((i) >> 5))
 
-// dot product of one row with x (K floats in LDS, padded): lanes take the 32-element blocks in turn
-__device__ __forceinline__ float gg_row_dot(int t, const uint8_t* row, const float* x, int K, int lane) {
-  float acc = 0.f;
-  for (int b = lane; b < K / 32; b += 64) {
-    int q[32];
-    float a, c;
-    gg_block(t, row, b, q, a, c);
-    const float* xb = x + 33 * b;
-    float sq = 0.f, sx = 0.f;
-#pragma unroll
-    for (int l = 0; l < 32; l++) {
-      const float xv = xb[l];
-      sq = fmaf((float)q[l], xv, sq);
-      sx += xv;
+// four bits b0..b3 of x to bit 0 of bytes 0..3
+__device__ __forceinline__ uint32_t spread4(uint32_t x) { return ((x & 0xFu) * 0x00204081u) & 0x01010101u; }
+
+// The same block for the dot products: the codes as unsigned bytes, four to a word (byte i of word w = element
+// 4w + i), so that unpacking is a few word operations and a byte-to-float conversion per element; w = a*q + c
+// with the constants adjusted where the stored codes are signed (Q8_0: q + 128).  Q4_K, Q5_K, Q8_0, Q5_1.
+__device__ __forceinline__ void gg_block_packed(int t, const uint8_t* row, int b, uint32_t (&qp)[8], float& a, float& c) {
+  if (t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K) {
+    const bool k5 = t == MOE_GGML_Q5_K;
+    const uint8_t* sb = row + (size_t)(b >> 3) * (k5 ? 176 : 144);
+    const int j = b & 7;
+    const uint4 hd = *(const uint4*)sb;
+    const uint8_t sc12[12] = {(uint8_t)hd.y, (uint8_t)(hd.y >> 8), (uint8_t)(hd.y >> 16), (uint8_t)(hd.y >> 24),
+                              (uint8_t)hd.z, (uint8_t)(hd.z >> 8), (uint8_t)(hd.z >> 16), (uint8_t)(hd.z >> 24),
+                              (uint8_t)hd.w, (uint8_t)(hd.w >> 8), (uint8_t)(hd.w >> 16), (uint8_t)(hd.w >> 24)};
+    int sc, mn;
+    k4_sm(j, sc12, sc, mn);
+    a = h2f_bits(hd.x & 0xffffu) * (float)sc;
+    c = -(h2f_bits(hd.x >> 16) * (float)mn);
+    const uint4* ql = (const uint4*)(sb + (k5 ? 48 : 16) + 32 * (j >> 1));
+    const uint4 l0 = ql[0], l1 = ql[1];
+    const uint32_t lw[8] = {l0.x, l0.y, l0.z, l0.w, l1.x, l1.y, l1.z, l1.w};
+    uint32_t hw[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (k5) {
+      const uint4* qh = (const uint4*)(sb + 16);
+      const uint4 h0 = qh[0], h1 = qh[1];
+      hw[0] = h0.x; hw[1] = h0.y; hw[2] = h0.z; hw[3] = h0.w;
+      hw[4] = h1.x; hw[5] = h1.y; hw[6] = h1.z; hw[7] = h1.w;
     }
-    acc += a * sq + c * sx;
+    const int nsh = (j & 1) ? 4 : 0;
+#pragma unroll
+    for (int w = 0; w < 8; w++) qp[w] = ((lw[w] >> nsh) & 0x0f0f0f0fu) | (((hw[w] >> j) & 0x01010101u) << 4);
+  } else if (t == MOE_GGML_Q8_0) {
+    const uint16_t* p = (const uint16_t*)(row + (size_t)b * 34);
+    uint16_t w16[17];
+#pragma unroll
+    for (int i = 0; i < 17; i++) w16[i] = p[i];
+    a = h2f_bits(w16[0]);
+    c = -128.f * a;
+#pragma unroll
+    for (int w = 0; w < 8; w++) qp[w] = ((uint32_t)w16[1 + 2 * w] | ((uint32_t)w16[2 + 2 * w] << 16)) ^ 0x80808080u;
+  } else {  // Q5_1
+    const uint2* p = (const uint2*)(row + (size_t)b * 24);
+    const uint2 p0 = p[0], p1 = p[1], p2 = p[2];
+    a = h2f_bits(p0.x & 0xffffu);
+    c = h2f_bits(p0.x >> 16);
+    const uint32_t qh = p0.y;
+    const uint32_t qs[4] = {p1.x, p1.y, p2.x, p2.y};
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      qp[w] = (qs[w] & 0x0f0f0f0fu) | (spread4(qh >> (4 * w)) << 4);
+      qp[4 + w] = ((qs[w] >> 4) & 0x0f0f0f0fu) | (spread4(qh >> (16 + 4 * w)) << 4);
+    }
   }
+}
+
+// dot product of one row with x (K floats in LDS, padded; xsum[b] = sum of block b's activations): lanes take the
+// 32-element blocks in turn
+__device__ __forceinline__ float gg_unit_dot(int t, const uint8_t* row, int b, const float* xb, float sx) {
+  float a, c, sq = 0.f;
+  if (t == MOE_GGML_IQ4_NL || t == MOE_GGML_IQ4_XS) {
+    int q[32];
+    gg_block(t, row, b, q, a, c);
+#pragma unroll
+    for (int l = 0; l < 32; l++) sq = fmaf((float)q[l], xb[l], sq);
+  } else {
+    uint32_t qp[8];
+    gg_block_packed(t, row, b, qp, a, c);
+#pragma unroll
+    for (int w = 0; w < 8; w++) {
+      sq = fmaf((float)(qp[w] & 0xffu), xb[4 * w], sq);
+      sq = fmaf((float)((qp[w] >> 8) & 0xffu), xb[4 * w + 1], sq);
+      sq = fmaf((float)((qp[w] >> 16) & 0xffu), xb[4 * w + 2], sq);
+      sq = fmaf((float)(qp[w] >> 24), xb[4 * w + 3], sq);
+    }
+  }
+  return a * sq + c * sx;
+}
+__device__ __forceinline__ float gg_row_dot(int t, const uint8_t* row, const float* x, const float* xsum, int K,
+                                            int lane) {
+  float acc = 0.f;
+  for (int b = lane; b < K / 32; b += 64) acc += gg_unit_dot(t, row, b, x + 33 * b, xsum[b]);
   return wave_sum_f(acc);
 }
 
@@ -197,6 +262,13 @@ __global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restri
   const int s = blockIdx.y, tok = blockIdx.z;
   for (int i = threadIdx.x; i < d; i += blockDim.x) xs[GX_PAD(i)] = x[(size_t)tok * d + i];
   __syncthreads();
+  float* xsum = xs + d / 32 * 33;  // per-block sums of the activations, behind the padded activations
+  for (int b = threadIdx.x; b < d / 32; b += blockDim.x) {
+    float sx = 0.f;
+    for (int l = 0; l < 32; l++) sx += xs[33 * b + l];
+    xsum[b] = sx;
+  }
+  __syncthreads();
   const bool shared = s >= kpt;
   const int t = shared ? A.tsh : A.tgu;
   const uint64_t rb = gg_row_bytes(t, d);
@@ -208,8 +280,8 @@ __global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restri
   for (int rr = wv; rr < GX_ROWS; rr += 4) {
     const int r = blockIdx.x * GX_ROWS + rr;
     if (r >= mid) break;  // wave-uniform
-    const float g = gg_row_dot(t, gbase + (uint64_t)r * rb, xs, d, lane);
-    const float u = gg_row_dot(t, ubase + (uint64_t)r * rb, xs, d, lane);
+    const float g = gg_row_dot(t, gbase + (uint64_t)r * rb, xs, xsum, d, lane);
+    const float u = gg_row_dot(t, ubase + (uint64_t)r * rb, xs, xsum, d, lane);
     if (lane == 0) ho[r] = silu_f(g) * u;
   }
 }
@@ -232,6 +304,13 @@ __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restri
     wgt[s] = s < kpt ? ws[(size_t)tok * id_stride + s] : sigmoid_f(A.sh_logit[tok]);
   }
   __syncthreads();
+  float* hsum = hs + nslots * mid / 32 * 33;  // per-block sums, behind the padded activations
+  for (int b = threadIdx.x; b < nslots * mid / 32; b += blockDim.x) {
+    float sx = 0.f;
+    for (int l = 0; l < 32; l++) sx += hs[33 * b + l];
+    hsum[b] = sx;
+  }
+  __syncthreads();
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   // a wave per row; its lanes take the (slot, 32-element block) units in turn, each weighted by the slot's
   // combine weight, so a row needs one wave-wide sum (a fixed order: the result does not depend on timing)
@@ -246,18 +325,7 @@ __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restri
       const int t = sh ? A.tsh : A.tdn;
       const uint64_t rb = gg_row_bytes(t, mid);
       const uint8_t* row = sh ? A.sh_down + (uint64_t)r * rb : A.down + ((uint64_t)eid[s] * d + r) * rb;
-      int q[32];
-      float a, c;
-      gg_block(t, row, b, q, a, c);
-      const float* xb = hs + 33 * (s * nb + b);
-      float sq = 0.f, sx = 0.f;
-#pragma unroll
-      for (int l = 0; l < 32; l++) {
-        const float xv = xb[l];
-        sq = fmaf((float)q[l], xv, sq);
-        sx += xv;
-      }
-      acc += wgt[s] * (a * sq + c * sx);
+      acc += wgt[s] * gg_unit_dot(t, row, b, hs + 33 * (s * nb + b), hsum[s * nb + b]);
     }
     acc = wave_sum_f(acc);
     if (lane == 0) out[(size_t)tok * d + r] = acc;
@@ -300,7 +368,9 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
               !moe_aligned(sh_down, gg_align(tsh)))))
     return MOE_E_INVALID;
   const int nslots = kpt + (sh ? 1 : 0);
-  if (nslots > 16 || (size_t)d * 4 > 60 * 1024 || (size_t)nslots * mid * 4 > 60 * 1024) return MOE_E_UNSUPPORTED;
+  // LDS: the activations with one float of padding and one block sum per 32
+  if (nslots > 16 || (size_t)d / 32 * 34 * 4 > 60 * 1024 || (size_t)nslots * mid / 32 * 34 * 4 > 60 * 1024)
+    return MOE_E_UNSUPPORTED;
   if (P == 0) return MOE_OK;
   GgxArgs A{};
   A.gate = gate; A.up = up; A.down = down;
@@ -309,12 +379,12 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
   A.sh_logit = sh_logit;
   if (phase != 2) {
     dim3 grid((mid + GX_ROWS - 1) / GX_ROWS, nslots, P);
-    k_ggx_gu<<<grid, 256, (size_t)d / 32 * 33 * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
+    k_ggx_gu<<<grid, 256, (size_t)d / 32 * 34 * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
     MOE_LAUNCH_CHECK();
   }
   if (phase != 1) {
     dim3 grid((d + GX_DN_ROWS - 1) / GX_DN_ROWS, P);
-    k_ggx_dn<<<grid, 256, (size_t)nslots * mid / 32 * 33 * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
+    k_ggx_dn<<<grid, 256, (size_t)nslots * mid / 32 * 34 * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
     MOE_LAUNCH_CHECK();
   }
   return MOE_OK;
