@@ -149,6 +149,20 @@ class Routing:
             pass
 
 
+def routing_run_static(ids, ws, k, experts, want_pairids=True):
+    """moe_routing_run_static: the permutation on the library's fixed scratch (the outputs are the caller's)."""
+    P, stride = ids.shape
+    dev = ids.device
+    n = P * k
+    tokidx = torch.full((max(n, 1),), -1, dtype=torch.int32, device=dev)
+    pw = torch.zeros((max(n, 1),), dtype=torch.float32, device=dev)
+    eoff = torch.full((experts + 1,), -1, dtype=torch.int32, device=dev)
+    pairids = torch.full((max(n, 1),), -1, dtype=torch.int32, device=dev) if want_pairids else None
+    check(lib().moe_routing_run_static(ptr(ids), ptr(ws), ptr(tokidx), ptr(pw), ptr(eoff), ptr(pairids), P, k,
+                                       experts, stride, stream()), "moe_routing_run_static")
+    return tokidx[:n], pw[:n], eoff, (pairids[:n] if want_pairids else None)
+
+
 def tiles(eoff, cap, pairs):
     E = eoff.numel() - 1
     max_tiles = (pairs + cap - 1) // cap + E
@@ -181,6 +195,7 @@ class LutW(C.Structure):
 
 
 LUT_Q4CP = 100
+ROUTING_STATIC_MAX_TOKENS = 32768
 OPT_INT_DECODE = 1
 OPT_UNIQUE_MIN_TOKENS = 2
 OPT_FUSED_COMBINE = 3

@@ -3,6 +3,9 @@
 // waves / blocks / experts give every pair its slot.  Stable: inside an expert pairs are in
 // ascending token order, exactly what the reference's stable radix sort yields.
 // (reference: src/gpu/parts/10_ple_io.inc:784-861)
+#include <mutex>
+#include <new>
+
 #include "common.h"
 #include "internal.h"
 
@@ -306,6 +309,27 @@ MOE_API int moe_routing_destroy(moe_routing* r) {
   return e1 != hipSuccess ? (int)e1 : (int)e2;
 }
 
+// Counting, scan and scatter launches of a batch of more than 32 tokens; blockcnt / blockoff hold
+// [ceil(P/256)][experts] ints each.
+static int routing_launch(int* blockcnt, int* blockoff, const int* ids, const float* ws, int* tokidx, float* pw,
+                          int* eoff, int* pairids, int P, int k, int experts, int id_stride, hipStream_t st) {
+  int nbits = 0;
+  for (int v = experts - 1; v; v >>= 1) nbits++;
+  const int nblk = (P + RT_TOK - 1) / RT_TOK;
+  if (nblk > 0) {
+    k_route_count<<<nblk, 256, 0, st>>>(ids, P, k, experts, id_stride, nbits, blockcnt);
+    MOE_LAUNCH_CHECK();
+  }
+  k_route_scan<<<1, RT_MAXE, 0, st>>>(blockcnt, blockoff, eoff, nblk, experts);
+  MOE_LAUNCH_CHECK();
+  if (nblk > 0) {
+    k_route_scatter<<<nblk, 256, 0, st>>>(ids, ws, P, k, experts, id_stride, nbits, blockoff, eoff, tokidx, pw,
+                                          pairids);
+    MOE_LAUNCH_CHECK();
+  }
+  return MOE_OK;
+}
+
 MOE_API int moe_routing_run(moe_routing* r, const int* ids, const float* ws, int* tokidx, float* pw,
                             int* eoff, int* pairids, int P, int k, int experts, int id_stride,
                             moe_stream_t st) {
@@ -315,21 +339,54 @@ MOE_API int moe_routing_run(moe_routing* r, const int* ids, const float* ws, int
   if (moe_route_small_supported(P, k, experts))
     return moe_launch_route_small(ids, ws, tokidx, pw, eoff, pairids, P, k, experts, id_stride, nullptr, nullptr, 0,
                                   -1, moe_s(st));
-  int nbits = 0;
-  for (int v = experts - 1; v; v >>= 1) nbits++;
-  const int nblk = (P + RT_TOK - 1) / RT_TOK;
-  if (nblk > 0) {
-    k_route_count<<<nblk, 256, 0, moe_s(st)>>>(ids, P, k, experts, id_stride, nbits, r->blockcnt);
-    MOE_LAUNCH_CHECK();
+  return routing_launch(r->blockcnt, r->blockoff, ids, ws, tokidx, pw, eoff, pairids, P, k, experts, id_stride,
+                        moe_s(st));
+}
+
+// ---- the permutation for callers that cannot allocate ----
+// The per-block histograms and their prefix sums live in a file-scope device array instead of a
+// moe_routing object's allocations: MOE_ROUTING_STATIC_MAX_TOKENS / 256 blocks x 1024 experts x 2 arrays
+// of ints = 1 MiB per GPU, held until the process ends.  Every kernel of a call writes the part of the
+// array it later reads (nothing has to start at zero), and every call on a GPU uses the same array:
+// calls that overlap on one GPU (two streams, two threads) race.
+namespace {
+constexpr int RT_STATIC_BLOCKS = MOE_ROUTING_STATIC_MAX_TOKENS / RT_TOK;
+constexpr int RT_MAX_DEVICES = 64;
+}  // namespace
+static __device__ __align__(256) int scratch[2 * RT_STATIC_BLOCKS * RT_MAXE];
+static int* g_scratch_ptr[RT_MAX_DEVICES];  // device address of `scratch` on each GPU (its name is no address on the host)
+static std::mutex g_scratch_mu;
+
+// The address of this GPU's copy of `scratch`, looked up once per device with that device current.
+static int scratch_of_current_device(int** out) {
+  int dev = -1;
+  MOE_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= RT_MAX_DEVICES) return MOE_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    int* p = nullptr;
+    MOE_HIP(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+    if (!p) return (int)hipErrorInvalidSymbol;
+    g_scratch_ptr[dev] = p;
   }
-  k_route_scan<<<1, RT_MAXE, 0, moe_s(st)>>>(r->blockcnt, r->blockoff, eoff, nblk, experts);
-  MOE_LAUNCH_CHECK();
-  if (nblk > 0) {
-    k_route_scatter<<<nblk, 256, 0, moe_s(st)>>>(ids, ws, P, k, experts, id_stride, nbits,
-                                                 r->blockoff, eoff, tokidx, pw, pairids);
-    MOE_LAUNCH_CHECK();
-  }
+  *out = g_scratch_ptr[dev];
   return MOE_OK;
+}
+
+MOE_API int moe_routing_run_static(const int* ids, const float* ws, int* tokidx, float* pw, int* eoff, int* pairids,
+                                   int P, int k, int experts, int id_stride, moe_stream_t st) {
+  if (!eoff || (P > 0 && (!ids || !ws || !tokidx || !pw))) return MOE_E_INVALID;
+  if (P < 0 || k < 1 || id_stride < k || experts < 1) return MOE_E_INVALID;
+  if (experts > RT_MAXE) return MOE_E_UNSUPPORTED;
+  if (P > MOE_ROUTING_STATIC_MAX_TOKENS) return MOE_E_STATE;  // beyond the fixed scratch: use moe_routing_create / run
+  if (moe_route_small_supported(P, k, experts))
+    return moe_launch_route_small(ids, ws, tokidx, pw, eoff, pairids, P, k, experts, id_stride, nullptr, nullptr, 0,
+                                  -1, moe_s(st));
+  int* base = nullptr;
+  const int rc = scratch_of_current_device(&base);
+  if (rc) return rc;
+  return routing_launch(base, base + (size_t)RT_STATIC_BLOCKS * RT_MAXE, ids, ws, tokidx, pw, eoff, pairids, P, k,
+                        experts, id_stride, moe_s(st));
 }
 
 MOE_API int moe_tiles(const int* eoff, moe_tile* tiles, int* ntiles, int experts, int cap,

@@ -101,6 +101,16 @@ int moe_routing_destroy(moe_routing* r);
 int moe_routing_run(moe_routing* r, const int* ids, const float* ws, int* tokidx, float* pw,
                     int* eoff, int* pairids, int P, int k, int experts, int id_stride,
                     moe_stream_t st);
+/* moe_routing_run for callers that cannot allocate and hold no moe_routing object (code under HIP graph
+ * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * GpuMoeRouting::init allocates.  Same arguments, results and launches as moe_routing_run; the per-block
+ * histograms live in a fixed 1 MiB array inside the library's device image (one copy per GPU, kept until the
+ * process ends), so nothing is allocated or freed, at the first call or later.  P <= MOE_ROUTING_STATIC_MAX_TOKENS
+ * (MOE_E_STATE beyond it), experts <= 1024.  Every call on a GPU uses that GPU's one array: calls that
+ * overlap on the same GPU (two streams or two host threads) race; calls on one stream are ordered. */
+enum { MOE_ROUTING_STATIC_MAX_TOKENS = 32768 };
+int moe_routing_run_static(const int* ids, const float* ws, int* tokidx, float* pw, int* eoff, int* pairids,
+                           int P, int k, int experts, int id_stride, moe_stream_t st);
 /* k_moe_tiles (10_ple_io.inc:815): split each expert's run into <= cap pair tiles, expert order.
  * tiles must hold (pairs+cap-1)/cap + experts entries. */
 int moe_tiles(const int* eoff, moe_tile* tiles, int* ntiles, int experts, int cap, moe_stream_t st);

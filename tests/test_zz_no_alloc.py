@@ -1,0 +1,55 @@
+"""moe_routing_run_static (the permutation on the library's fixed device scratch, for callers that cannot
+allocate) against moe_routing_run, through the C ABI: bit-exact on two calls in a row, the second smaller."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def _ids(rng, P, E, k):
+    ids = np.zeros((P, 16), np.int32)
+    ws = np.zeros((P, 16), np.float32)
+    pr = 1.0 / (np.arange(E) + 1.0) ** 1.1
+    pr[-3:] = 0
+    pr /= pr.sum()
+    for t in range(P):
+        ids[t, :k] = rng.choice(E, k, replace=False, p=pr)
+        ws[t, :k] = rng.random(k)
+    return ids, ws
+
+
+def test_static_scratch_routing_equals_routing_run():
+    import torch
+    from gfx1151_engine_amd import capi
+    L = capi.lib()
+    assert torch.cuda.is_available()
+    E, k = 512, 10
+    rng = np.random.default_rng(77)
+    r = capi.Routing(6000 * k, E)
+    # larger first, then smaller (the scratch keeps the first call's histograms), then a batch of the one-launch size
+    for P in (6000, 700, 20):
+        ids, ws = _ids(rng, P, E, k)
+        gi, gw = torch.from_numpy(ids).cuda(), torch.from_numpy(ws).cuda()
+        want = [a.cpu().numpy() for a in r.run(gi, gw, k)]
+        n = P * k
+        tokidx = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+        pw = torch.zeros((n,), dtype=torch.float32, device="cuda")
+        eoff = torch.full((E + 1,), -1, dtype=torch.int32, device="cuda")
+        pairids = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        capi.check(L.moe_routing_run_static(capi.ptr(gi), capi.ptr(gw), capi.ptr(tokidx), capi.ptr(pw), capi.ptr(eoff),
+                                            capi.ptr(pairids), P, k, E, 16, capi.stream()), "moe_routing_run_static")
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0, "the call must not change the device's free memory"
+        for name, a, b in zip(("tokidx", "pw", "eoff", "pairids"), (tokidx, pw, eoff, pairids), want):
+            assert (a.cpu().numpy().view(np.int32) == b.view(np.int32)).all(), (P, name)
+    # the wrapper in capi.py gives the same
+    got = capi.routing_run_static(gi, gw, k, E)
+    for a, b in zip(got, want):
+        assert (a.cpu().numpy().view(np.int32) == b.view(np.int32)).all()
+    # beyond the fixed scratch: refused, nothing enqueued
+    big = torch.zeros((capi.ROUTING_STATIC_MAX_TOKENS + 1, 16), dtype=torch.int32, device="cuda")
+    with pytest.raises(capi.MoeError):
+        capi.routing_run_static(big, big.float(), k, E)
+    r.close()
