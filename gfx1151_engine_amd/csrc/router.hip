@@ -195,9 +195,10 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
 // probability ~1e-8 per value.  Row E (if Wx given) is the shared-expert gate vector: out_x[t] =
 // its logit.  Blocks past the rows (if planes given) turn x into the digit planes of the
 // integer-dot decode kernels, so that work rides along instead of costing a launch.
-// If `counter` is given, the block that finishes last (an atomic ticket per row block, fences at
-// device scope on both sides) runs the softmax / top-k of every token as well and re-arms the
-// counter: one launch instead of two on the latency-bound decode path.
+// If `counter` is given, the block that finishes last (an atomic ticket per row block; the logits
+// cross as device-scope stores that have completed before the ticket, and device-scope loads after
+// it) runs the softmax / top-k of every token as well and re-arms the counter: one launch instead
+// of two on the latency-bound decode path.
 template <bool BF16, int TT, int NPL>
 __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W,
                                                       const float* __restrict__ bias,
@@ -275,8 +276,13 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
     }
   }
   if (!counter) return;
-  // the wave's logit stores have completed before its block takes a ticket (no cache-wide
-  // write-back is needed: the stores above and the loads in topk_block are device-scope accesses)
+  // Hand-over to the block that draws the last ticket (possibly on another XCD).  The logits above are
+  // device-scope atomic stores (written through to the device's coherence point, not left in this XCD's
+  // L2), and every storing wave waits here until the memory system has acknowledged all of them
+  // (vmcnt = 0) before it reaches the barrier; only then does thread 0 take the ticket.  The reader
+  // (topk_block<.., true>) uses device-scope atomic loads issued after its own ticket came back, which
+  // read at that same point.  No cache-wide write-back or invalidate is involved on either side.
+  __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -604,7 +610,12 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
     else __hip_atomic_store(&gpart[((size_t)ks * nrt + rg) * NV + i], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   if (KS == 1) return;
-  // the block's partial-tile stores have completed before it takes its ticket
+  // Hand-over of the partial tiles to the block that draws the row group's last ticket (possibly on another
+  // XCD): the tiles are device-scope atomic stores, every storing thread waits until all of its stores have
+  // been acknowledged (vmcnt = 0) before the barrier, thread 0 takes the device-scope ticket after the
+  // barrier, and the last block reads the tiles back with device-scope atomic loads issued after its own
+  // ticket returned.  Both sides go to the device's coherence point; no cache-wide write-back / invalidate.
+  __builtin_amdgcn_s_waitcnt(0);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
   __syncthreads();
   if (tid == 0) {
