@@ -196,6 +196,7 @@ class LutW(C.Structure):
 
 LUT_Q4CP = 100
 ROUTING_STATIC_MAX_TOKENS = 32768
+DENSE_SHARED = False  # moe_set_shared with bf16 / f32 matrices
 OPT_INT_DECODE = 1
 OPT_UNIQUE_MIN_TOKENS = 2
 OPT_FUSED_COMBINE = 3
@@ -371,6 +372,7 @@ class TensorInfo(C.Structure):
 
 
 FILE_HGN, FILE_GGUF = 1, 2
+FILE_OPT_GGUF_F32_ROUTER = 1
 
 
 class ModelFile:
@@ -399,6 +401,9 @@ class ModelFile:
         data = np.ctypeslib.as_array(C.cast(ti.data, C.POINTER(C.c_uint8)), shape=(ti.nbytes,)).copy() if ti.nbytes else \
             np.zeros(0, np.uint8)
         return ti.dtype, tuple(ti.dims[i] for i in range(ti.ndims)), data
+
+    def set_option(self, option, value):
+        check(lib().moe_file_set_option(self.h, option, value), "moe_file_set_option")
 
     def config(self, layer=0):
         cfg = Config()

@@ -535,6 +535,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   if (L.has_shared && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format per launch
   if (q4k ? (g.d % 256 || g.mid % 256) : (g.d % 128 || g.mid % 128)) return MOE_E_UNSUPPORTED;
   moe_lutw gu{}, dn{}, sgu{}, sdn{};
+  const float* sh_cb_up = nullptr;
   if (q4k) {
     gu.w = L.gg.gate; gu.w_up = L.gg.up; gu.e_rows = g.mid;
     dn.w = L.gg.down; dn.e_rows = g.d;
@@ -552,7 +553,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     moe_lut_q4cp_view(L.sh_up.data, L.sh_up.rows, L.sh_up.cols, L.sh_up.scale_stride, g.mid, 0, &t);
     sgu.w_up = t.w;
     sgu.sc_up = t.sc;
-    // one codebook per LutW: gate and up of the shared expert must agree (they come from one quantiser)
+    sh_cb_up = t.cb;  // up_proj is a tensor of its own, with its own codebook (the converter trains one per tensor)
     moe_lut_q4cp_view(L.sh_down.data, L.sh_down.rows, L.sh_down.cols, L.sh_down.scale_stride, g.d, 0, &sdn);
   }
   int rc;
@@ -575,7 +576,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, 128, P, sh_first, c->tokidx, c->side);
     if (!rs)
       rs = moe_launch_gemm_q4cp(true, &gu, &sgu, g.experts, c->x16, c->tokidx, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
-                                c->hid16, g.mid, g.d, true, q4k, hs, c->side, nullptr);
+                                c->hid16, g.mid, g.d, true, q4k, hs, c->side, nullptr, sh_cb_up);
     if (!rs)
       rs = moe_launch_gemm_q4cp(false, &dn, &sdn, g.experts, c->hid16, nullptr, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
                                 c->pairs16, g.d, g.mid, true, q4k, hs, c->side, nullptr);
@@ -639,7 +640,8 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
   if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,
-                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr)))
+                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr,
+                                 sh_cb_up)))
     return rc;
   prof_mark(c, MOE_PROF_UP, st);
   if (fused) {

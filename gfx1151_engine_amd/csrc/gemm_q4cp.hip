@@ -57,11 +57,11 @@ constexpr int NSB = WROWS == 512 ? 2 : 1;
 #endif
 constexpr int NBUF = MOE_GEMM_NBUF;       // activation / code buffers; loads run NBUF-1 stages ahead
 constexpr int AHEAD = NBUF - 1;
-constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES + 64 + BM * 4 + BM * 4;
+constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES + 128 + BM * 4 + BM * 4;  // + two 16-entry codebooks, row indices, row scales
 
 struct LutDev {
   const uint8_t *w, *w_up, *sc, *sc_up;
-  const float* cb;
+  const float *cb, *cb_up;  // codebook of the (gate) rows and of the up rows (the same for a fused gate_up tensor)
   int sstride, e_rows, up_off;
 };
 
@@ -124,14 +124,15 @@ __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
 template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
-                                          int K, float cb_a, float cb_b, int ri, const float* __restrict__ xms,
+                                          int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
+                                          const float* __restrict__ xms,
                                           float cmag, const moe_comb& cmb, bool shared) {
   constexpr int NH = NF / 2;  // gate/up: fragments per half
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
   const float* cbs = (const float*)(S0 + NSB * S_BYTES);
-  int* rowidx = (int*)(cbs + 16);
+  int* rowidx = (int*)(cbs + 32);  // cbs[16..31]: the up rows' codebook
   float* rowscale = (float*)(rowidx + BM);  // f16 range guard of each pair row (gate/up only)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, kept scalar
@@ -360,7 +361,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     } else {
 #pragma unroll
       for (int nf = 0; nf < NF; nf++) {
-        const _Float16 as = (_Float16)(cb_a * scf[nf]), bs = (_Float16)(cb_b * scf[nf]);
+        const bool upf = UP && nf >= NH;  // the up half may come from a tensor with a codebook of its own
+        const _Float16 as = (_Float16)((upf ? cb_a_up : cb_a) * scf[nf]), bs = (_Float16)((upf ? cb_b_up : cb_b) * scf[nf]);
         as2[nf][0] = half2v{as, as};
         bs2[nf][0] = half2v{bs, bs};
       }
@@ -385,8 +387,9 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       }
     } else {
       half2v hv;
-      hv.x = (_Float16)(cbs[(w >> (4 * part)) & 0xf] * scf[nf]);
-      hv.y = (_Float16)(cbs[(w >> (4 * part + 16)) & 0xf] * scf[nf]);
+      const float* tb = (UP && nf >= NH) ? cbs + 16 : cbs;
+      hv.x = (_Float16)(tb[(w >> (4 * part)) & 0xf] * scf[nf]);
+      hv.y = (_Float16)(tb[(w >> (4 * part + 16)) & 0xf] * scf[nf]);
       dst[nf].h[part] = hv;
     }
   };
@@ -629,18 +632,25 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
 
   // q4cp codebook: affine (a*n+b) or table.  Q4_K has no codebook (w = (d*sc)*n - dmin*m).
   bool affine = true;
-  float cb_a = 1.f, cb_b = 0.f;
+  float cb_a = 1.f, cb_b = 0.f, cb_a_up = 1.f, cb_b_up = 0.f;
   if (!Q4K) {
-    const float c0 = L.cb[0], c1 = L.cb[1];
+    // lanes 0..15: the (gate) rows' codebook, lanes 16..31: the up rows' (the same table unless the two
+    // halves come from separately quantised tensors, as a shared expert's gate_proj / up_proj do)
+    const float* cbu = UP ? L.cb_up : L.cb;
+    const float c0 = L.cb[0], c1 = L.cb[1], u0 = cbu[0], u1 = cbu[1];
     bool aff = true;
-    if (lane < 16) {
-      const float v = L.cb[lane];
-      aff = v == fmaf((float)lane, c1 - c0, c0);
-      if (tid < 16) cbs[lane] = v;
+    if (lane < 32) {
+      const int nn = lane & 15;
+      const bool upl = lane >= 16;
+      const float v = upl ? cbu[nn] : L.cb[nn];
+      aff = v == fmaf((float)nn, upl ? u1 - u0 : c1 - c0, upl ? u0 : c0);
+      if (tid < 32) cbs[lane] = v;
     }
     affine = __all(aff);
     cb_a = c1 - c0;
     cb_b = c0;
+    cb_a_up = u1 - u0;
+    cb_b_up = u0;
   }
 
   const float cmag = shared ? hs.c_shared : hs.c_routed;
@@ -648,8 +658,8 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag, cmb, shared); \
-    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, ri, hs.xms, cmag, cmb, shared); \
+    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
@@ -658,10 +668,11 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
 #undef GEMM_GO
 }
 
-LutDev to_dev(const moe_lutw* p) {
+LutDev to_dev(const moe_lutw* p, const float* cb_up) {
   LutDev d{};
   if (p) {
     d.w = p->w; d.w_up = p->w_up; d.sc = p->sc; d.sc_up = p->sc_up; d.cb = p->cb;
+    d.cb_up = cb_up ? cb_up : p->cb;
     d.sstride = p->sstride; d.e_rows = p->e_rows; d.up_off = p->up_off;
   }
   return d;
@@ -683,11 +694,12 @@ bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k) {
 }  // namespace
 
 // Internal: routed + (optional) shared expert in one launch; tile.expert >= n_experts selects Sh.
+// sh_cb_up: codebook of the shared expert's up rows when they are a tensor of their own (nullptr: sh->cb).
 // q4k: the views hold raw GGUF Q4_K rows (w / w_up only) instead of q4cp planes.
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st, const moe_comb* comb) {
+                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
   moe_comb cmb{};
   if (comb) {  // fused combine: down launch with f32 results, out = the (zeroed) token rows
@@ -703,7 +715,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   // per XCD: ceil(routed/8) + ceil(shared/8) <= max_tiles/8 + 2 tile slots
   const int per_xcd = (max_tiles + 7) / 8 + 1;
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
-  LutDev R = to_dev(routed), S = to_dev(sh ? sh : routed);
+  LutDev R = to_dev(routed, nullptr), S = to_dev(sh ? sh : routed, sh ? sh_cb_up : nullptr);
   const int split = sh ? 1 : 0;
 #define GEMM_LAUNCH(UPK, F16, Q)                                                                              \
   do {                                                                                                        \
@@ -748,7 +760,7 @@ MOE_API int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* 
   if (type != MOE_LUT_Q4CP) return MOE_E_UNSUPPORTED;
   if (!tokidx) return MOE_E_INVALID;
   return moe_launch_gemm_q4cp(true, p, nullptr, 1 << 30, (const __half*)x16, tokidx, tiles, ntiles, max_tiles,
-                              hid16, m, k, true, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
+                              hid16, m, k, true, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr);
 }
 
 MOE_API int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
@@ -756,7 +768,7 @@ MOE_API int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const m
                          moe_stream_t st) {
   if (type != MOE_LUT_Q4CP) return MOE_E_UNSUPPORTED;
   return moe_launch_gemm_q4cp(false, p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
-                              max_tiles, pairs, m, k, f16 != 0, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
+                              max_tiles, pairs, m, k, f16 != 0, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr);
 }
 
 // moe_gg_up / moe_gg_down: raw GGUF blocks, expert e's rows start at row e * m of each tensor
@@ -770,7 +782,7 @@ MOE_API int moe_gg_up(int type, const uint8_t* gate, const uint8_t* up, const vo
   p.w_up = up;
   p.e_rows = m;
   return moe_launch_gemm_q4cp(true, &p, nullptr, 1 << 30, (const __half*)x16, tokidx, tiles, ntiles, max_tiles,
-                              hid16, m, k, true, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
+                              hid16, m, k, true, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr);
 }
 
 MOE_API int moe_gg_down(int type, const uint8_t* down, const void* hid16, const moe_tile* tiles,
@@ -781,5 +793,5 @@ MOE_API int moe_gg_down(int type, const uint8_t* down, const void* hid16, const 
   p.w = down;
   p.e_rows = m;
   return moe_launch_gemm_q4cp(false, &p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
-                              max_tiles, pairs, m, k, f16 != 0, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr);
+                              max_tiles, pairs, m, k, f16 != 0, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr);
 }

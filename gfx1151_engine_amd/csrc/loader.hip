@@ -47,29 +47,22 @@ struct HgnRecord {  // src/hgn.h:55-60
 #pragma pack(pop)
 static_assert(sizeof(HgnHeader) == 104 && sizeof(HgnRecord) == 160, "HGN1 on-disk structs");
 
-// ggml block geometry (src/gguf.h:42-64): elements per block, bytes per block
+// ggml tensor types this reader can size: {type id, elements per block, bytes per block}, ordered by id
+// (the constants are ggml's on-disk format; src/gguf.h:42-64 lists the same ones)
+struct GgmlGeom { uint16_t type, elems, bytes; };
+constexpr GgmlGeom kGgmlGeom[] = {
+    {0, 1, 4},      {1, 1, 2},      {2, 32, 18},    {3, 32, 20},    {6, 32, 22},    {7, 32, 24},   {8, 32, 34},
+    {10, 256, 84},  {11, 256, 110}, {12, 256, 144}, {13, 256, 176}, {14, 256, 210}, {20, 32, 18},  {23, 256, 136},
+    {24, 1, 1},     {25, 1, 2},     {26, 1, 4},     {27, 1, 8},     {28, 1, 8},     {30, 1, 2}};
 bool ggml_block(uint32_t t, uint32_t& be, uint32_t& bb) {
-  switch (t) {
-    case 0: be = 1; bb = 4; return true;     // F32
-    case 1: case 30: be = 1; bb = 2; return true;  // F16, BF16
-    case 24: be = 1; bb = 1; return true;    // I8
-    case 25: be = 1; bb = 2; return true;    // I16
-    case 26: be = 1; bb = 4; return true;    // I32
-    case 27: case 28: be = 1; bb = 8; return true;  // I64, F64
-    case 2: be = 32; bb = 18; return true;   // Q4_0
-    case 3: be = 32; bb = 20; return true;   // Q4_1
-    case 6: be = 32; bb = 22; return true;   // Q5_0
-    case 7: be = 32; bb = 24; return true;   // Q5_1
-    case 8: be = 32; bb = 34; return true;   // Q8_0
-    case 20: be = 32; bb = 18; return true;  // IQ4_NL
-    case 10: be = 256; bb = 84; return true;   // Q2_K
-    case 11: be = 256; bb = 110; return true;  // Q3_K
-    case 12: be = 256; bb = 144; return true;  // Q4_K
-    case 13: be = 256; bb = 176; return true;  // Q5_K
-    case 14: be = 256; bb = 210; return true;  // Q6_K
-    case 23: be = 256; bb = 136; return true;  // IQ4_XS
-    default: be = bb = 0; return false;
-  }
+  for (const GgmlGeom& g : kGgmlGeom)
+    if (g.type == t) {
+      be = g.elems;
+      bb = g.bytes;
+      return true;
+    }
+  be = bb = 0;
+  return false;
 }
 
 struct Cur {  // bounds-checked little-endian reader over the mapped header
@@ -116,6 +109,7 @@ struct moe_file {
   size_t len = 0;
   std::unordered_map<std::string, FTensor> idx;
   std::unordered_map<std::string, int64_t> kv_int;  // GGUF integer metadata
+  bool gguf_keep_f32 = false;  // MOE_FILE_OPT_GGUF_F32_ROUTER
 };
 
 namespace {
@@ -165,8 +159,9 @@ static int parse_gguf(moe_file* f) {
         for (uint64_t j = 0; j < n && c.ok; j++) (void)c.str();
       } else {
         const uint32_t sz = gguf_scalar_bytes(et);
-        if (!sz) return MOE_E_INVALID;
-        c.skip(n * sz);
+        uint64_t bytes;
+        if (!sz || __builtin_mul_overflow(n, (uint64_t)sz, &bytes)) return MOE_E_INVALID;
+        c.skip(bytes);
       }
     } else if (t == 8) {
       (void)c.str();
@@ -191,7 +186,12 @@ static int parse_gguf(moe_file* f) {
     }
   }
   if (!c.ok) return MOE_E_INVALID;
-  if (auto it = f->kv_int.find("general.alignment"); it != f->kv_int.end() && it->second > 0) align = (uint64_t)it->second;
+  if (auto it = f->kv_int.find("general.alignment"); it != f->kv_int.end()) {
+    // a power of two of at most 4096 (ggml's default is 32): anything else is a corrupt or crafted header
+    const int64_t a = it->second;
+    if (a < 1 || a > 4096 || (a & (a - 1))) return MOE_E_INVALID;
+    align = (uint64_t)a;
+  }
   struct Pending { std::string name; FTensor t; uint64_t off; };
   std::vector<Pending> ts;
   for (uint64_t i = 0; i < nt && c.ok; i++) {
@@ -205,7 +205,8 @@ static int parse_gguf(moe_file* f) {
     ts.push_back(std::move(p));
   }
   if (!c.ok) return MOE_E_INVALID;
-  const uint64_t hdr = (uint64_t)(c.p - f->base), data0 = (hdr + align - 1) / align * align;
+  const uint64_t hdr = (uint64_t)(c.p - f->base);  // <= file length; align <= 4096: no wrap-around below
+  const uint64_t data0 = (hdr + align - 1) & ~(align - 1);
   for (auto& p : ts) {
     uint32_t be, bb;
     if (!ggml_block((uint32_t)p.t.dtype, be, bb)) return MOE_E_UNSUPPORTED;
@@ -215,7 +216,8 @@ static int parse_gguf(moe_file* f) {
       if (__builtin_mul_overflow(numel, p.t.dims[k], &numel)) return MOE_E_INVALID;
     if (p.t.dims[0] % be) return MOE_E_INVALID;
     if (__builtin_mul_overflow(numel / be, (uint64_t)bb, &p.t.nbytes)) return MOE_E_INVALID;
-    const uint64_t off = data0 + p.off;
+    uint64_t off;
+    if (__builtin_add_overflow(data0, p.off, &off)) return MOE_E_INVALID;  // an offset that wraps around to the header
     if (off > f->len || p.t.nbytes > f->len - off) return MOE_E_INVALID;
     p.t.data = f->base + off;
     if (!f->idx.emplace(p.name, p.t).second) return MOE_E_INVALID;  // duplicate name
@@ -423,6 +425,34 @@ int upload(moe_weights* w, const FTensor& t, hipStream_t st, const uint8_t** dev
 
 int hgn_dtype_ok_dense(int dt) { return dt == MOE_DT_BF16 || dt == MOE_DT_F32; }
 
+// f32 -> bf16, round to nearest even, NaN -> 0x7fc0: the rounding the reference applies to the F32 router and
+// shared-expert gate tensors of a GGUF file when it builds its bf16 tensors from them (src/gguf_map.h:66-72,145-157)
+uint16_t bf16_rne(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// An F32 tensor of the file as bf16 in device memory (host-side rounding, then one copy).
+int upload_f32_as_bf16(moe_weights* w, const FTensor& t, const uint8_t** dev) {
+  const size_t n = t.nbytes / 4;
+  std::vector<uint16_t> h(n);
+  for (size_t i = 0; i < n; i++) {
+    float v;
+    memcpy(&v, t.data + 4 * i, 4);
+    h[i] = bf16_rne(v);
+  }
+  void* p = nullptr;
+  MOE_HIP(hipMalloc(&p, n ? n * 2 : 1));
+  w->dev.push_back(p);
+  w->bytes += n * 2;
+  MOE_HIP(hipMemcpy(p, h.data(), n * 2, hipMemcpyHostToDevice));
+  *dev = (const uint8_t*)p;
+  return MOE_OK;
+}
+
 int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st) {
   const FTensor* rt = find(f, "layers.%d.mlp.gate.weight", fl);
   const FTensor* gu = find(f, "layers.%d.mlp.experts.gate_up_proj.weight", fl);
@@ -488,11 +518,15 @@ int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights
   };
   const uint64_t D = (uint64_t)g.d, M = (uint64_t)g.mid, NE = (uint64_t)g.experts;
   if (!is(*rt, D, NE, 1) || !is(*g_, D, M, NE) || !is(*u, D, M, NE) || !is(*dn, M, D, NE)) return MOE_E_INVALID;
+  // The reference turns the F32 ffn_gate_inp / ffn_gate_inp_shexp tensors into bf16 when it maps a GGUF file
+  // (src/gguf_map.h:9,210-211): its router sees the rounded values, so this loader rounds the same way
+  // unless the file object was told to keep F32 (MOE_FILE_OPT_GGUF_F32_ROUTER).
   moe_wview vr{};
-  vr.dtype = rt->dtype == 0 ? MOE_DT_F32 : MOE_DT_BF16;
+  const bool round_rt = rt->dtype == 0 && !f->gguf_keep_f32;
+  vr.dtype = (rt->dtype == 0 && !round_rt) ? MOE_DT_F32 : MOE_DT_BF16;
   vr.cols = rt->dims[0];
   vr.rows = rt->dims[1];
-  if ((rc = upload(w, *rt, st, &vr.data))) return rc;
+  if ((rc = round_rt ? upload_f32_as_bf16(w, *rt, &vr.data) : upload(w, *rt, st, &vr.data))) return rc;
   if ((rc = moe_set_router(ctx, cl, &vr, nullptr))) return rc;
   moe_gg_experts gg{};
   gg.tgu = g_->dtype;
@@ -517,8 +551,11 @@ int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights
       v->rows = t.dims[1];
       return upload(w, t, st, &v->data);
     };
-    if ((rc = raw(*sg, &a)) || (rc = raw(*su, &b)) || (rc = raw(*sd, &c2)) || (rc = raw(*sx, &d2))) return rc;
-    d2.dtype = sx->dtype == 0 ? MOE_DT_F32 : MOE_DT_BF16;
+    if ((rc = raw(*sg, &a)) || (rc = raw(*su, &b)) || (rc = raw(*sd, &c2))) return rc;
+    const bool round_sx = sx->dtype == 0 && !f->gguf_keep_f32;
+    d2.cols = sx->dims[0];
+    if ((rc = round_sx ? upload_f32_as_bf16(w, *sx, &d2.data) : upload(w, *sx, st, &d2.data))) return rc;
+    d2.dtype = (sx->dtype == 0 && !round_sx) ? MOE_DT_F32 : MOE_DT_BF16;
     d2.rows = 1;
     if ((rc = moe_set_shared(ctx, cl, &a, &b, &c2, &d2, sg->dtype))) return rc;
   }
@@ -526,6 +563,14 @@ int load_layer_gguf(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights
 }
 
 }  // namespace
+
+MOE_API int moe_file_set_option(moe_file* f, int option, int value) {
+  if (!f) return MOE_E_INVALID;
+  switch (option) {
+    case MOE_FILE_OPT_GGUF_F32_ROUTER: f->gguf_keep_f32 = value != 0; return MOE_OK;
+    default: return MOE_E_INVALID;
+  }
+}
 
 MOE_API int moe_weights_free(moe_weights* w) {
   if (!w) return MOE_OK;

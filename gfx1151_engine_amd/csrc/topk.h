@@ -306,8 +306,9 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
 // where the reference order falls back to the expert index.  Two logits more than 1e-6 apart give
 // probabilities whose ratio exceeds 1 + 2^-23 after both roundings, i.e. different floats in the same
 // order.  The function therefore checks the k + 1 best logits: every gap between neighbours above
-// 1e-6 -> ids_row[0..k) (LDS) holds the reference's ranking and true is returned; otherwise (also:
-// rows it does not handle, NaNs) false, and the caller runs the exact selection.
+// 1e-6 and all of them within 70 of the maximum (probabilities that are normal floats) -> ids_row[0..k) (LDS)
+// holds the reference's ranking and true is returned; otherwise (also: rows it does not handle, NaNs) false,
+// and the caller runs the exact selection.
 template <int NPL>
 __device__ bool topk_ids_by_logit(const float* lg, int* ids_row, int E, int k) {
   __shared__ int fast_ok;
@@ -370,7 +371,12 @@ __device__ bool topk_ids_by_logit(const float* lg, int* ids_row, int E, int k) {
       const uint32_t nk = (uint32_t)__shfl_down((int)mykey, 1, 64);
       const float la = __uint_as_float((mykey & 0x80000000u) ? (mykey ^ 0x80000000u) : ~mykey);
       const float lb = __uint_as_float((nk & 0x80000000u) ? (nk ^ 0x80000000u) : ~nk);
-      const bool good = lane >= k || (mykey != 0u && nk != 0u && la - lb > 1e-6f);  // false for NaNs
+      // The gap argument needs normal floats: a probability keeps 24 significant bits while exp(l - max) / sum
+      // stays above the smallest normal float, i.e. while l - max > -70 (exp(-70) / 1024 = 4e-34).  Further down
+      // the probabilities go subnormal or to zero, the reference sees ties there and orders them by index, so
+      // such rows take the exact selection as well.
+      const float lmax = __shfl(la, 0, 64);
+      const bool good = lane >= k || (mykey != 0u && nk != 0u && la - lb > 1e-6f && lmax - lb < 70.f);  // false for NaNs
       const int ok = __all(good);
       if (lane < k) ids_row[lane] = myid;
       if (lane == 0) fast_ok = ok;

@@ -210,8 +210,9 @@ int moe_destroy(moe_ctx* ctx);
  * hgn: gate_up [E*2*mid][d] and down [E*d][mid] q4cp views (40_model.inc:1826-1829).
  * gguf: GgExperts (40_model.inc:1823).  Exactly one of hgn / gguf per layer.
  * shared expert: gate_proj/up_proj [mid][d], down_proj [d][mid], shared_expert_gate [1][d]
- * (40_model.inc:1848-1857); dtype q4cp, f32 or bf16; sh_gguf_type != 0 means gate/up/down are
- * raw GGUF rows of that ggml type. */
+ * (40_model.inc:1848-1857).  gate_proj / up_proj / down_proj: q4cp (each tensor with its own codebook), or,
+ * with sh_gguf_type != 0, raw GGUF rows of that one ggml type; shared_expert_gate: f32 or bf16.
+ * MOE_E_UNSUPPORTED for other matrix dtypes. */
 int moe_set_router(moe_ctx* ctx, int layer, const moe_wview* gate_w, const float* router_bias);
 int moe_set_experts_q4cp(moe_ctx* ctx, int layer, const moe_wview* gate_up, const moe_wview* down);
 int moe_set_experts_gguf(moe_ctx* ctx, int layer, const moe_gg_experts* gg);
@@ -286,6 +287,12 @@ int moe_file_format(const moe_file* f);
 int64_t moe_file_tensor_count(const moe_file* f);
 /* MOE_E_STATE if the file has no tensor of that name */
 int moe_file_find(const moe_file* f, const char* name, moe_tensor_info* out);
+/* MOE_FILE_OPT_GGUF_F32_ROUTER (default 0): moe_load_layers registers the F32 tensors ffn_gate_inp and
+ * ffn_gate_inp_shexp of a GGUF file rounded to bf16 (nearest even), as the reference does when it maps a GGUF
+ * file (src/gguf_map.h:9,66-72,145-157,210-211), so that a layer routes exactly like the engine it drops into;
+ * 1 keeps them F32.  No effect on .hgn files (their tensors are registered in the dtype they are stored in). */
+enum { MOE_FILE_OPT_GGUF_F32_ROUTER = 1 };
+int moe_file_set_option(moe_file* f, int option, int value);
 /* d, mid, experts read off the expert tensors of layer `layer`, layers = consecutive layers from there
  * on that carry them; topk only from the standard GGUF
  * key "<arch>.expert_used_count" (a .hgn file does not store it).  Other fields untouched. */

@@ -19,8 +19,10 @@ class HostLayer:
     """One synthetic MoE layer as host bytes (the 'file' side)."""
 
     def __init__(self, rng, d, mid, E, k, fmt="q4cp", router_dtype="f32", codebook=None, scale_std=0.01,
-                 router_std=0.02, shared=True, bias=None, gg_types=(12, 12, 12)):
-        """fmt "q4k": raw GGUF blocks; gg_types = ggml types of (gate/up, down, shared expert)."""
+                 router_std=0.02, shared=True, bias=None, gg_types=(12, 12, 12), shared_codebooks=None):
+        """fmt "q4k": raw GGUF blocks; gg_types = ggml types of (gate/up, down, shared expert).
+        shared_codebooks: three 16-entry tables for the shared expert's gate_proj / up_proj / down_proj (q4cp; the
+        reference's converter trains one codebook per dense tensor, tools/flashnext2hgn.py:164-187)."""
         self.d, self.mid, self.E, self.k, self.fmt = d, mid, E, k, fmt
         self.tgu, self.tdn, self.tsh = gg_types
         rw = (rng.standard_normal((E, d), dtype=np.float32) * router_std)
@@ -40,9 +42,10 @@ class HostLayer:
             self.down = S.make_gg(rng, self.tdn, E * d, mid, scale_std=scale_std)
         self.shared = None
         if shared:
-            mk = (lambda r, c: S.make_q4cp(rng, r, c, codebook=codebook, scale_std=scale_std)) if fmt == "q4cp" \
-                else (lambda r, c: S.make_gg(rng, self.tsh, r, c, scale_std=scale_std))
-            self.shared = [mk(mid, d), mk(mid, d), mk(d, mid),
+            scb = shared_codebooks if shared_codebooks is not None else [codebook] * 3
+            mk = (lambda r, c, i: S.make_q4cp(rng, r, c, codebook=scb[i], scale_std=scale_std)) if fmt == "q4cp" \
+                else (lambda r, c, i: S.make_gg(rng, self.tsh, r, c, scale_std=scale_std))
+            self.shared = [mk(mid, d, 0), mk(mid, d, 1), mk(d, mid, 2),
                            rng.standard_normal((1, d), dtype=np.float32) * router_std]
 
     def oracle_layer(self):

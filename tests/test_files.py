@@ -126,6 +126,47 @@ def test_gguf_dims_that_wrap_around_are_rejected(tmp_path):
     assert capi.lib().moe_file_open(str(p).encode(), C.byref(h)) == -2
 
 
+def test_gguf_offsets_alignment_and_array_sizes_that_wrap_are_rejected(tmp_path):
+    """Crafted headers: a tensor offset near 2^64 (data start + offset wraps to a small number that points into
+    the header), general.alignment that is no power of two or is huge, and an array whose byte count wraps."""
+    lib = capi.lib()
+
+    def rc_of(blob, name):
+        p = tmp_path / name
+        p.write_bytes(blob)
+        h = C.c_void_p()
+        rc = lib.moe_file_open(str(p).encode(), C.byref(h))
+        if rc == 0:
+            lib.moe_file_close(h)
+        return rc
+
+    def s(b):
+        return struct.pack("<Q", len(b)) + b
+
+    def tensor(name, off):
+        return s(name) + struct.pack("<I", 1) + struct.pack("<Q", 8) + struct.pack("<IQ", files.GGML_F32, off)
+
+    def kv_u32(key, v):
+        return s(key) + struct.pack("<II", 4, v)
+
+    def pad32(b):
+        return b + b"\0" * ((-len(b)) % 32)
+
+    good = pad32(b"GGUF" + struct.pack("<IQQ", 3, 1, 0) + tensor(b"t", 0)) + b"\0" * 64
+    assert rc_of(good, "good.gguf") == 0
+    hdr = b"GGUF" + struct.pack("<IQQ", 3, 1, 0) + tensor(b"t", (1 << 64) - 32)
+    assert rc_of(pad32(hdr) + b"\0" * 64, "wrapoff.gguf") == -2
+    for i, al in enumerate((48, 0, 1 << 20)):
+        hdr = b"GGUF" + struct.pack("<IQQ", 3, 1, 1) + kv_u32(b"general.alignment", al) + tensor(b"t", 0)
+        assert rc_of(hdr + b"\0" * 4096, f"align{i}.gguf") == -2, al
+    # array of 2^61 + 1 u64 values: the byte count wraps to 8
+    arr = s(b"a") + struct.pack("<IIQ", 9, 10, (1 << 61) + 1)
+    hdr = b"GGUF" + struct.pack("<IQQ", 3, 1, 1) + arr + b"\0" * 8 + tensor(b"t", 0)
+    assert rc_of(pad32(hdr) + b"\0" * 64, "wraparr.gguf") == -2
+    # a GGUF cut in the middle of a tensor-info record
+    assert rc_of(good[:len(b"GGUF") + 20 + 12], "cutinfo.gguf") == -2
+
+
 def _x(T, seed=11):
     return np.random.default_rng(seed).standard_normal((T, D), dtype=np.float32)
 
@@ -140,6 +181,7 @@ def test_layers_loaded_from_file_equal_direct_registration(tmp_path, fmt):
     f = capi.ModelFile(p)
     cfg = f.config(first)
     m = capi.Moe(cfg.d, cfg.mid, cfg.experts, K, layers=cfg.layers, max_tokens=64)
+    f.set_option(capi.FILE_OPT_GGUF_F32_ROUTER, 1)  # bytes unchanged (by default a GGUF's F32 router goes to bf16)
     w = f.load_layers(m, first, 0, cfg.layers)
     f.close()                                  # the device copies do not depend on the mapping
     assert w.nbytes > 0
@@ -162,6 +204,71 @@ def test_layers_loaded_from_file_equal_direct_registration(tmp_path, fmt):
     torch.cuda.synchronize()
     del m
     w.free()
+
+
+@pytest.mark.gpu
+def test_hgn_file_with_a_codebook_per_shared_tensor(tmp_path):
+    """A standard .hgn file: the routed experts share one codebook, gate_proj / up_proj / down_proj of the shared
+    expert each carry their own (tools/flashnext2hgn.py:164-187).  Decode, small batch and grouped-GEMM batch."""
+    import torch
+    rng = np.random.default_rng(21)
+    cbs = [np.sort(rng.standard_normal(16)).astype(np.float32) * (i + 1) for i in range(3)]
+    hl = HostLayer(rng, D, MID, E, K, codebook=np.sort(rng.uniform(-2, 2, 16)).astype(np.float32), shared_codebooks=cbs)
+    p, _ = _hgn(tmp_path, [hl], first=0)
+    f = capi.ModelFile(p)
+    cfg = f.config(0)
+    m = capi.Moe(cfg.d, cfg.mid, cfg.experts, K, layers=1, max_tokens=80)
+    w = f.load_layers(m, 0, 0, 1)
+    f.close()
+    for T in (1, 9, 80):
+        x = _x(T, seed=T)
+        want, io, _ = O.moe_layer(hl.oracle_layer(), x)
+        y = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :K] == io[:, :K]).all()
+        assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max(), T
+    del m
+    w.free()
+
+
+@pytest.mark.gpu
+def test_gguf_router_tensors_are_rounded_to_bf16_like_the_reference(tmp_path):
+    """The reference maps a GGUF's F32 ffn_gate_inp / ffn_gate_inp_shexp to bf16 tensors (src/gguf_map.h:210-211), so
+    its router multiplies the rounded values.  A loaded layer must route like the oracle fed those bf16 values, and
+    like the oracle fed the F32 values only when the file object is told to keep them."""
+    import torch
+    from gfx1151_engine_amd import synth as S
+    rng = np.random.default_rng(33)
+    hl = HostLayer(rng, D, MID, E, K, fmt="q4k", router_std=1.0)
+    # two pairs of rows that differ by less than a bf16 step: the rounding decides their order for many tokens
+    hl.router[1] = hl.router[0] * (1 + 1e-4 * rng.standard_normal(D).astype(np.float32))
+    hl.router[5] = hl.router[4] * (1 + 1e-4 * rng.standard_normal(D).astype(np.float32))
+    p, _ = _gguf(tmp_path, [hl], first=0)
+    T = 64
+    x = _x(T, seed=3)
+    l32 = hl.oracle_layer()
+    y32, i32, w32 = O.moe_layer(l32, x)
+    rb = S.f32_to_bf16_bits(hl.router)
+    sgb = S.f32_to_bf16_bits(hl.shared[3])
+    assert (S.bf16_round(hl.router) != hl.router).any()
+    l16 = O.Layer(D, MID, E, K, O.Mat(O.BF16, rb, E, D), O.Mat(hl.tdn, hl.down, E * D, MID),
+                  gate=O.Mat(hl.tgu, hl.gate, E * MID, D), up=O.Mat(hl.tgu, hl.up, E * MID, D),
+                  shared=[O.Mat(hl.tsh, hl.shared[0], MID, D), O.Mat(hl.tsh, hl.shared[1], MID, D),
+                          O.Mat(hl.tsh, hl.shared[2], D, MID), O.Mat(O.BF16, sgb, 1, D)])
+    y16, i16, w16 = O.moe_layer(l16, x)
+    assert (i16[:, :K] != i32[:, :K]).any(), "the test needs tokens whose routing the rounding changes"
+    for keep_f32, (yo, io) in ((0, (y16, i16)), (1, (y32, i32))):
+        f = capi.ModelFile(p)
+        f.set_option(capi.FILE_OPT_GGUF_F32_ROUTER, keep_f32)
+        m = capi.Moe(D, MID, E, K, layers=1, max_tokens=T)
+        w = f.load_layers(m, 0, 0, 1)
+        f.close()
+        y = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :K] == io[:, :K]).all(), keep_f32
+        assert np.abs(y - yo).max() <= 2e-3 * np.abs(yo).max(), keep_f32
+        del m
+        w.free()
 
 
 @pytest.mark.gpu
@@ -259,6 +366,7 @@ def test_load_gguf_mixed_types(tmp_path):
     p = tmp_path / "mixed.gguf"
     files.write_gguf(p, ts, kv={"general.architecture": "x"})
     f = capi.ModelFile(p)
+    f.set_option(capi.FILE_OPT_GGUF_F32_ROUTER, 1)  # the comparison below is with the F32 router registered directly
     m = capi.Moe(d, mid, E, k, layers=1, max_tokens=8)
     w = f.load_layers(m, 0, 0, 1)
     x = rng.standard_normal((5, d), dtype=np.float32)

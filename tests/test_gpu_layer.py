@@ -120,6 +120,36 @@ def test_decode_topk_near_ties(oracle, fmt, T):
     m.close()
 
 
+@pytest.mark.parametrize("fmt", ["q4cp", "q4k"])
+def test_decode_topk_wide_logit_range(oracle, fmt):
+    """Router rows scaled so that the logits span hundreds: below the best few, the reference's f32 probabilities
+    go subnormal or to zero and tie, and ties are ordered by expert index.  The gate/up launch of the decode path
+    (which ranks by logit) and the down launch (which takes the ids of the exact selection) must still agree with
+    each other and with the oracle: a slot that ran gate/up for one expert and down for another shows in y."""
+    rng = np.random.default_rng(29)
+    d, mid, E, k = (3072, 768, 24, 10) if fmt == "q4cp" else (512, 256, 24, 10)
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt)
+    # rows in descending-logit order that runs AGAINST the index order: ties between underflowed probabilities
+    # then come out by index, i.e. opposite to the logits
+    x = rng.standard_normal((3, d), dtype=np.float32)
+    u = x[0] / np.linalg.norm(x[0])
+    hl.router[:] = 1e-3 * rng.standard_normal((E, d), dtype=np.float32)
+    hl.router += np.outer(np.linspace(-9.0, 3.0, E), u).astype(np.float32)  # token 0: logits ~ 55 * (-9 .. 3)
+    x[2] = 0.0                                                                # token 2: all logits equal
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    lg = oracle.router(hl.oracle_layer().router, x, k)[0]
+    assert lg[0].max() - np.sort(lg[0])[-k] > 90, "the k-th logit of token 0 must lie in the underflow range"
+    m, dev = hl.to_gpu(max_tokens=8)
+    for T in (1, 3):
+        y = m.forward(0, gpu(x[:T])).cpu().numpy()
+        ids, ws = m.last_routing(T)
+        ids, ws = ids.cpu().numpy(), ws.cpu().numpy()
+        assert (ids[:, :k] == io[:T, :k]).all(), (T, ids[:, :k], io[:T, :k])
+        assert np.abs(ws[:, :k] - wo[:T, :k]).max() <= 1e-6
+        assert max_abs_rel(y, yo[:T]) <= tol_small(fmt), (T, max_abs_rel(y, yo[:T]))
+    m.close()
+
+
 @pytest.mark.parametrize("tgu,tdn,tsh,T", [(13, 8, 12, 1), (12, 7, 12, 5), (13, 7, 8, 3), (12, 8, 13, 40), (23, 20, 12, 2),
                                             (20, 23, 23, 7)])
 def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
@@ -166,27 +196,32 @@ def test_unique_expert_path(oracle, share):
     m.close()
 
 
-def test_golden_layers_from_reference(oracle, golden):
-    """Inputs and outputs of the reference's own Model::moe (tests/golden/moe_layer.npz)."""
+@pytest.mark.parametrize("i", [0, 1, 2])
+def test_golden_layers_from_reference(oracle, golden, i):
+    """Inputs and outputs of the reference's own Model::moe (tests/golden/moe_layer.npz): three layers, two of them
+    with a bf16 shared expert."""
     import torch
     from gfx1151_engine_amd import capi
     g = golden("moe_layer.npz")
-    for i in range(int(g["n"])):
-        d, mid, E, k, sh_dt = (int(v) for v in g[f"cfg{i}"])
-        if sh_dt != oracle.Q4CP:
-            continue  # bf16 shared-expert matrices are outside this path's formats
-        m = capi.Moe(d, mid, E, k)
-        keep = [gpu(g[f"router{i}"].view(np.int16)), gpu(g[f"gu{i}"]), gpu(g[f"dn{i}"]), gpu(g[f"shg{i}"]),
-                gpu(g[f"shu{i}"]), gpu(g[f"shd{i}"]), gpu(g[f"sg{i}"].view(np.int16))]
-        m.set_router(0, capi.wview(keep[0], capi.BF16, E, d))
-        m.set_experts_q4cp(0, capi.wview(keep[1], capi.Q4CP, E * 2 * mid, d), capi.wview(keep[2], capi.Q4CP, E * d, mid))
-        m.set_shared(0, capi.wview(keep[3], capi.Q4CP, mid, d), capi.wview(keep[4], capi.Q4CP, mid, d),
-                     capi.wview(keep[5], capi.Q4CP, d, mid), capi.wview(keep[6], capi.BF16, 1, d))
-        x = g[f"x{i}"]
-        y = m.forward(0, gpu(x)).cpu().numpy()
-        want = g[f"ybits{i}"].view(np.float32)
-        assert max_abs_rel(y, want) <= TOL_GEMV, i
-        m.close()
+    assert int(g["n"]) == 3
+    d, mid, E, k, sh_dt = (int(v) for v in g[f"cfg{i}"])
+    m = capi.Moe(d, mid, E, k)
+    sh16 = sh_dt != oracle.Q4CP  # bf16 matrices are stored as uint16 bit patterns
+    if sh16 and not capi.DENSE_SHARED:
+        pytest.skip("bf16 shared-expert matrices: moe_set_shared takes q4cp or raw GGUF rows only")
+    shv = [g[f"shg{i}"], g[f"shu{i}"], g[f"shd{i}"]]
+    keep = [gpu(g[f"router{i}"].view(np.int16)), gpu(g[f"gu{i}"]), gpu(g[f"dn{i}"])] + \
+           [gpu(a.view(np.int16) if sh16 else a) for a in shv] + [gpu(g[f"sg{i}"].view(np.int16))]
+    wt = capi.BF16 if sh16 else capi.Q4CP
+    m.set_router(0, capi.wview(keep[0], capi.BF16, E, d))
+    m.set_experts_q4cp(0, capi.wview(keep[1], capi.Q4CP, E * 2 * mid, d), capi.wview(keep[2], capi.Q4CP, E * d, mid))
+    m.set_shared(0, capi.wview(keep[3], wt, mid, d), capi.wview(keep[4], wt, mid, d),
+                 capi.wview(keep[5], wt, d, mid), capi.wview(keep[6], capi.BF16, 1, d))
+    x = g[f"x{i}"]
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    want = g[f"ybits{i}"].view(np.float32)
+    assert max_abs_rel(y, want) <= TOL_GEMV, i
+    m.close()
 
 
 def test_forward_errors(oracle):

@@ -175,6 +175,33 @@ def test_batch_layer_vs_oracle(oracle, d, mid, E, k, T, skew):
     m.close()
 
 
+@pytest.mark.parametrize("kind", ["affine", "table", "mixed"])
+@pytest.mark.parametrize("T", [70, 20])
+def test_shared_expert_with_a_codebook_per_tensor(oracle, kind, T):
+    """gate_proj, up_proj and down_proj of the shared expert are separately quantised tensors: each carries its own
+    codebook (the reference's converter trains one per dense tensor; only routed experts share one).  Batch path
+    (grouped GEMM: gate and up rows in one launch) and small path against the oracle."""
+    rng = np.random.default_rng(len(kind) * 100 + T)
+    n = np.arange(16, dtype=np.float32)
+    if kind == "affine":     # three different uniform grids
+        cbs = [n - 8, 0.5 * n - 3.0, -0.25 * n + 1.0]
+    elif kind == "table":    # three different non-uniform tables
+        cbs = [np.sort(rng.uniform(-2, 2, 16)).astype(np.float32) for _ in range(3)]
+    else:                    # gate uniform, up a table, down another grid
+        cbs = [n - 8, np.sort(rng.standard_normal(16)).astype(np.float32) * 3, 2 * n - 15]
+    d, mid, E, k = 512, 256, 8, 3
+    hl = HostLayer(rng, d, mid, E, k, shared_codebooks=[c.astype(np.float32) for c in cbs])
+    x = S.bf16_round(rng.standard_normal((T, d), dtype=np.float32))
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    y = m.forward(0, gpu(x))
+    ids, _ = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    err = max_abs_rel(y.cpu().numpy(), yo)
+    assert err <= TOL_LAYER, err
+    m.close()
+
+
 def test_batch_equals_small_path_statistically(oracle):
     """Same layer through the MFMA path (T=40) and the f32 in-place path (two calls of 20)."""
     rng = np.random.default_rng(5)

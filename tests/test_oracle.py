@@ -367,3 +367,13 @@ def test_hc_writeback_closed_forms(oracle):
     out = O.hc_writeback(y2, np.zeros((1, 4), np.float32), R2)
     vals = (out.astype(np.uint32) << 16).view(np.float32)
     assert (vals[0, :, 0] == 256.0).all() and (vals[0, :, 1] == 260.0).all()
+    # a gate strictly between the saturated ends: w4 = 4 ln 3 gives inj = 2 / (1 + 1/3) = 1.5 (to within an ulp of
+    # the f32 exp), w4 = -4 ln 3 gives 2 / (1 + 3) = 0.5.  With R = 0 and y = 2^j the results 1.5 * 2^j and 0.5 * 2^j
+    # are bf16 numbers that an ulp of inj cannot move; a wrong divisor in inj (w4 / 2, w4 / 8) or a missing factor 2
+    # gives 1.8 / 1.27 / 0.75 times y instead and fails.
+    y3 = np.array([[2.0, -4.0, 0.5, 64.0]], np.float32)
+    w3 = np.array([[4 * np.log(3.0), -4 * np.log(3.0), 4 * np.log(7.0), 0.0]], np.float32)  # inj 1.5, 0.5, 1.75, 1
+    out3 = O.hc_writeback(y3, w3, np.zeros((1, 4, 4), np.uint16))
+    v3 = (out3.astype(np.uint32) << 16).view(np.float32)
+    for b, inj in enumerate((1.5, 0.5, 1.75, 1.0)):
+        assert (v3[0, b] == inj * y3[0]).all(), (b, v3[0, b])
