@@ -25,14 +25,31 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 D, MID, E, K = 3072, 768, 512, 10
 LIB_OPTIONS = []              # (option id, value) pairs of --opt, applied to every context
-# HBM bytes per launch of the dominant kernel (read + written) at the default shapes, from the
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised in profiles/*_hbm_traffic.txt (counters
-# cannot be read from inside this process; other shapes report null)
-PMC_TRAFFIC = {("prefill", "q4cp", 16384): 4569.79e6, ("decode", "q4cp", 1): 29.60e6}
 CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
+# Counters cannot be read from inside this process: the HBM bytes per launch of the dominant kernel (read + written)
+# come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (the table's "total MB" column of
+# the named kernel's line); a workload or shape without such a summary reports null.
+PMC_TRAFFIC = {("prefill", "q4cp", 16384): ("prefill_q4cp_T16384_hbm_traffic.txt", "k_moe_gemm_q4cp<true", "max"),
+               ("decode", "q4cp", 1): ("decode_q4cp_T1_hbm_traffic.txt", "k_dec_gu", "max"),
+               ("verify", "q4cp", 20): ("verify_q4cp_T20_hbm_traffic.txt", "k_dec_gu", "max"),
+               ("decode", "q4k", 1): ("decode_q4k_T1_hbm_traffic.txt", "k_dec4k_gu", "max"),
+               ("prefill", "q4k", 8192): ("prefill_q4k_T8192_hbm_traffic.txt", "k_moe_gemm_q4cp<true", "max")}
 
 
-def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb):
+def pmc_traffic(kind, fmt, T):
+    """HBM bytes per launch of the workload's dominant kernel from its committed counter summary, or None."""
+    ent = PMC_TRAFFIC.get((kind, fmt, T))
+    if not ent:
+        return None
+    path = os.path.join(ROOT, "profiles", ent[0])
+    try:
+        vals = [float(ln.split()[-1]) for ln in open(path) if ln.startswith(ent[1]) and len(ln.split()) >= 7]
+    except (OSError, ValueError):
+        return None
+    return max(vals) * 1e6 if vals else None  # routed and shared-expert launches of one kernel: the larger grid
+
+
+def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb, budget=CPU_BUDGET_S):
     """The CPU restatement of src/ref.cpp Model::moe (OpenMP over rows) on a bounded sample of the
     same workload, and the GPU result's distance from it on that sample."""
     import numpy as np
@@ -50,7 +67,7 @@ def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb):
         yg_all = y.cpu().numpy()
         xh = xs[0].cpu().numpy()
         done, cpu_s, err = 0, 0.0, 0.0
-        while cpu_s < CPU_BUDGET_S and done < len(order):
+        while cpu_s < budget and done < len(order):
             toks = order[done:done + 256]
             t0 = time.perf_counter()
             yo, _, _ = O.moe_layer(ol, xh[toks])
@@ -61,7 +78,7 @@ def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb):
                "sample": f"{done} of the batch's {T} tokens (64 of the hottest expert's first), chunks of 256"}
     else:
         done, cpu_s, err, nbytes = 0, 0.0, 0.0, 0
-        while cpu_s < CPU_BUDGET_S and done < 4096:
+        while cpu_s < budget and done < 4096:
             xg = xs[done % len(xs)]
             xh = xg.cpu().numpy()
             t0 = time.perf_counter()
@@ -80,7 +97,7 @@ def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb):
     return out
 
 
-def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
+def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_budget=CPU_BUDGET_S):
     import numpy as np
     import torch
     from gfx1151_engine_amd import capi, workloads as W
@@ -113,7 +130,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
     m = capi.Moe(d, mid, E, k, layers=nlayers, max_tokens=T)
     for l, L in enumerate(layers):
         L.register(m, l)
-    for o, v in LIB_OPTIONS:
+    for o, v in list(LIB_OPTIONS) + list(opts):
         m.set_option(o, v)
     y = torch.empty((T, d), dtype=torch.float32, device="cuda")
 
@@ -147,6 +164,28 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
         for kk, v in m.profile_read().items():
             stage[kk] = stage.get(kk, 0.0) + v / nprof
     m.profile(False)
+    # Batches of at most 32 tokens: a kernel takes about as long as an event pair's own dispatch latency, so the
+    # dominant kernel (gate/up) is timed as the difference between the step loop above and the same loop with that
+    # stage's launch left out (MOE_OPT_TIMING_SKIP_STAGE): its cost inside the pipelined stream, on the same
+    # rotating inputs (so no cache level holds the experts).  Three alternations, median.
+    up_marginal_ms = None
+    if T <= 32:
+        def loop_ms():
+            f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            f0.record()
+            for i in range(steps):
+                step(warmup + i)
+            f1.record()
+            torch.cuda.synchronize()
+            return f0.elapsed_time(f1) / steps
+        diffs = []
+        for _ in range(3):
+            full = loop_ms()
+            m.set_option(5, 3)   # MOE_OPT_TIMING_SKIP_STAGE = 1 + MOE_PROF_UP
+            part = loop_ms()
+            m.set_option(5, 0)
+            diffs.append(full - part)
+        up_marginal_ms = sorted(diffs)[1] / nlayers
 
     # A pair of stage events costs a few microseconds more than the kernels between them take when they run
     # back to back (the event makes the next dispatch wait).  The mean surplus per stage is reported for
@@ -175,8 +214,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
         # the timed gate/up launch: the routed experts' pairs; the shared expert's tiles are in the same launch only
         # with MOE_OPT_SHARED_ASIDE = 0 or MOE_OPT_FUSED_COMBINE = 1 (by default its GEMMs run on the library's side
         # stream next to the router launch and are over before this launch starts)
-        opts = dict(LIB_OPTIONS)
-        shared_in_launch = opts.get(4, 1) == 0 or opts.get(3, 0) != 0
+        od = dict(list(LIB_OPTIONS) + list(opts))
+        shared_in_launch = od.get(4, 1) == 0 or od.get(3, 0) != 0
         up_flop = (pairs + (T if shared_in_launch else 0)) * 2 * (2 * mid) * d
         up_s = stage["up"] * 1e-3
         res.update({"metric": "moe_layer_prefill_tokens_per_s", "unit": "tok/s", "value": round(T / (ms * 1e-3), 1),
@@ -187,7 +226,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
                                  ("routed + shared expert tiles" if shared_in_launch else "routed experts' tiles"),
                                  "achieved": round(up_flop / up_s / 1e12, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": round(up_flop / up_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                                 "traffic": None if shared_in_launch else PMC_TRAFFIC.get((kind, fmt, T))}})
+                                 "timing": "HIP events around the launch (moe_profile_enable), same stream",
+                                 "traffic": None if shared_in_launch else pmc_traffic(kind, fmt, T)}})
         # rows the grouped GEMM computes for the routed pairs: tiles of 128, the last tile of an expert padded
         # to a multiple of 32 rows
         rem = cnt % 128
@@ -203,20 +243,29 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True):
             gu_bytes = (uniq + 1) * 2 * mid * (d // 2 + S.q4cp_scale_stride(d))
         else:
             gu_bytes = 2 * mid * (uniq * W.gg_row_bytes(gg_types[0], d) + W.gg_row_bytes(gg_types[2], d))
-        up_s = stage["up"] * 1e-3
+        up_s = up_marginal_ms * 1e-3
+        od = dict(list(LIB_OPTIONS) + list(opts))
+        int_dec = od.get(1, 1) != 0 and not ggmix
+        # the arithmetic of the GEMV kernels: integer dot products of the 4-bit codes with the activations' 4-bit
+        # (q4cp: v_dot8_i32_i4, four planes) or 8-bit (Q4_K: v_dot4_i32_i8, two planes) digit planes, f32 scales;
+        # or plain f32 FMAs (MOE_OPT_INT_DECODE = 0, and the general GGUF kernels)
         res.update({"metric": "moe_layer_decode_hbm_GB_per_s", "unit": "GB/s",
                     "value": round(step_bytes / (ms * 1e-3) / 1e9, 1),
-                    "dtype": "f32" if ggmix else "i8",
+                    "dtype": "f32" if not int_dec else ("i4" if fmt == "q4cp" else "i8"),
+                    "up_kernel_ms": round(up_marginal_ms, 5),
                     "hbm_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "tokens_per_s": round(T / (ms * 1e-3), 1),
                     "roofline": {"bound": "hbm", "kernel": "gate/up GEMV + SwiGLU",
                                  "achieved": round(gu_bytes / up_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                  "frac": round(gu_bytes / up_s / 1e9 / HBM_PEAK_GBS, 4),
-                                 "traffic": PMC_TRAFFIC.get((kind, fmt, T))}})
+                                 "timing": "step loop minus the same loop without this launch, HIP events around the "
+                                           "loops (an event pair around the single launch reads %.2f us: the pair's "
+                                           "dispatch latency is of the kernel's size)" % (stage["up"] * 1e3),
+                                 "traffic": pmc_traffic(kind, fmt, T) if int_dec else None}})
         cfg.update({"unique_experts": uniq, "step_bytes": int(step_bytes)})
     res["config"] = cfg
     if cpu:
-        res["cpu_baseline"] = cpu_leg(kind, layers[0], xs, ids, cnt, m, T, eb)
+        res["cpu_baseline"] = cpu_leg(kind, layers[0], xs, ids, cnt, m, T, eb, cpu_budget)
     m.close()
     return res
 
@@ -316,10 +365,21 @@ def main():
     if a.workload == "headline":
         res = measure("prefill", a.steps, a.warmup, a.tokens, cpu=not a.no_cpu)
         torch.cuda.empty_cache()
-        dec = measure("decode", max(a.steps, 64) * 4, max(a.warmup, 8), cpu=not a.no_cpu)
-        res["decode_T1"] = {kk: dec[kk] for kk in ("metric", "value", "unit", "hbm_frac", "ms_per_step", "steps",
-                                                   "stage_ms", "dtype", "roofline", "config", "cpu_baseline")
-                            if kk in dec}
+        # the other configurations of the benchmark, measured in the same run and reported as sub-records
+        keys = ("metric", "value", "unit", "hbm_frac", "layer_mfma_frac", "ms_per_step", "steps", "stage_ms",
+                "up_kernel_ms", "dtype", "roofline", "config", "cpu_baseline")
+        nd, wd = max(a.steps, 64) * 4, max(a.warmup, 8)
+
+        def sub(name, wl, steps, warmup, **kw):
+            torch.cuda.empty_cache()
+            r = measure(wl, steps, warmup, cpu=not a.no_cpu, cpu_budget=5.0, **kw)
+            res[name] = {kk: r[kk] for kk in keys if kk in r}
+        sub("decode_T1", "decode", nd, wd)
+        sub("decode_T1_f32_kernels", "decode", nd, wd, opts=((1, 0),))   # MOE_OPT_INT_DECODE = 0
+        sub("verify_T20", "verify", 128, wd)
+        sub("stack48_T1", "stack", 16, 2)
+        sub("q4k_prefill_T8192", "q4k_prefill", a.steps, a.warmup)
+        sub("q4k_decode_T1", "q4k_decode", nd, wd)
     elif a.workload in ("load", "q4k_load"):
         res = measure_load("q4k" if a.workload.startswith("q4k") else "q4cp", min(a.steps, 5), min(a.layers, 2))
     else:

@@ -201,6 +201,7 @@ OPT_INT_DECODE = 1
 OPT_UNIQUE_MIN_TOKENS = 2
 OPT_FUSED_COMBINE = 3
 OPT_SHARED_ASIDE = 4
+OPT_TIMING_SKIP_STAGE = 5
 
 
 def lut_q4cp_view(blob, rows, cols, e_rows, up_off):

@@ -74,6 +74,7 @@ struct moe_ctx {
   int uq_min = 12;            // > 0: small batches of at least this many tokens read every distinct expert once
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
   bool profile = false;
+  int skip_stage = 0;      // MOE_OPT_TIMING_SKIP_STAGE: 1 + the stage whose launches are left out (0 = none)
   hipEvent_t ev[MOE_PROF_STAGES + 1] = {};
   int ev_n = 0;            // events recorded by the last call
   int ev_stage[MOE_PROF_STAGES] = {};
@@ -364,6 +365,10 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
       return MOE_OK;
     case MOE_OPT_FUSED_COMBINE: c->fused_combine = value != 0; return MOE_OK;
     case MOE_OPT_SHARED_ASIDE: c->shared_aside = value != 0; return MOE_OK;
+    case MOE_OPT_TIMING_SKIP_STAGE:
+      if (value < 0 || value > MOE_PROF_STAGES) return MOE_E_INVALID;
+      c->skip_stage = value;
+      return MOE_OK;
     default: return MOE_E_INVALID;
   }
 }
@@ -405,121 +410,127 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   int rc;
   c->ev_n = 0;
   prof_mark(c, 0, st);
-  const int nslots_d = g.topk + (L.has_shared ? 1 : 0);
-  const bool use_int = L.has_q4cp && c->int_decode && L.experts_affine && (!L.has_shared || L.shared_affine) &&
-                       (!L.has_shared || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
+  // A stage = the launches between two profile events.  MOE_OPT_TIMING_SKIP_STAGE leaves one stage's launches
+  // out (timing experiments only: the output is then meaningless).
+  auto stage = [&](int tag, auto&& launch) -> int {
+    if (c->skip_stage != tag + 1) {
+      const int e = launch();
+      if (e) return e;
+    }
+    prof_mark(c, tag, st);
+    return MOE_OK;
+  };
+  const bool sh = L.has_shared;
+  const int nslots_d = g.topk + (sh ? 1 : 0);
+  const bool use_int = L.has_q4cp && c->int_decode && L.experts_affine && (!sh || L.shared_affine) &&
+                       (!sh || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
   const bool use_int4k = L.has_gguf && c->int_decode && L.gg.tgu == MOE_GGML_Q4_K && L.gg.tdn == MOE_GGML_Q4_K &&
-                         (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K) &&
-                         moe_dec4k_supported(g.d, g.mid, nslots_d);
+                         (!sh || L.sh_gguf_type == MOE_GGML_Q4_K) && moe_dec4k_supported(g.d, g.mid, nslots_d);
   const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min && moe_dec_uq_supported(g.d);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
   const bool gu_topk = ((use_int && !use_uq) || use_int4k) && moe_dec_gu_topk_supported(g.experts, g.topk);
-  bool fused = false;
-  if ((rc = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P,
-                                    c->logits, c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
-                                    use_int4k, gu_topk ? nullptr : c->ticket,
-                                    c->ids, c->ws, g.topk, g.id_stride, &fused, st, c->kpart, c->ktickets)))
+  if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
+         bool fused = false;
+         int e = moe_router_logits_small(&L.router, L.router_bias, sh ? &L.sh_sg : nullptr, x, P, c->logits,
+                                         c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
+                                         use_int4k, gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk,
+                                         g.id_stride, &fused, st, c->kpart, c->ktickets);
+         if (!e && !fused && !gu_topk)
+           e = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
+         return e;
+       })))
     return rc;
-  if (!fused && !gu_topk &&
-      (rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st)))
-    return rc;
-  prof_mark(c, MOE_PROF_ROUTER, st);
+  const moe_wview *shg = sh ? &L.sh_gate : nullptr, *shu = sh ? &L.sh_up : nullptr, *shd = sh ? &L.sh_down : nullptr;
+  const uint8_t *rg = sh ? L.sh_gate.data : nullptr, *ru = sh ? L.sh_up.data : nullptr, *rd = sh ? L.sh_down.data : nullptr;
   if (L.has_q4cp) {
-    if (L.has_shared && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
+    if (sh && L.sh_gguf_type != 0) return MOE_E_UNSUPPORTED;
     if (use_uq) {
       // verify-size batches: tokens share experts; walk the expert-sorted pair lists so that every
       // distinct expert's weights are read once (reference: the _uq kernels, 26_kernels_moe_gguf.inc:758-877)
-      const int sh_first = L.has_shared ? P * g.topk : -1;
-      if (moe_route_small_supported(P, g.topk, g.experts)) {  // permutation and tiles in one launch
-        if ((rc = moe_launch_route_small(c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
-                                         g.id_stride, c->tiles, c->ntiles, 4, sh_first, st)))
-          return rc;
-      } else {
-        if ((rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
-                                  g.experts, g.id_stride, st)))
-          return rc;
-        if ((rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 4, P, sh_first, c->tokidx, st)))
-          return rc;
-      }
-      prof_mark(c, MOE_PROF_ROUTE, st);
-      const int max_tiles = P * g.topk + (L.has_shared ? (P + 3) / 4 : 0);  // tiles of <= 4 pairs
-      if ((rc = moe_launch_dec_gu_uq(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
-                                     L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->tiles, c->ntiles,
-                                     max_tiles, c->tokidx, g.experts, g.d, g.mid, c->hplanes, c->hmeta, st)))
+      const int sh_first = sh ? P * g.topk : -1;
+      const int max_tiles = P * g.topk + (sh ? (P + 3) / 4 : 0);  // tiles of <= 4 pairs
+      if ((rc = stage(MOE_PROF_ROUTE, [&]() -> int {
+             if (moe_route_small_supported(P, g.topk, g.experts))  // permutation and tiles in one launch
+               return moe_launch_route_small(c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
+                                             g.experts, g.id_stride, c->tiles, c->ntiles, 4, sh_first, st);
+             const int e = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P,
+                                           g.topk, g.experts, g.id_stride, st);
+             return e ? e : moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 4, P, sh_first, c->tokidx, st);
+           })))
         return rc;
-      prof_mark(c, MOE_PROF_UP, st);
-      if ((rc = moe_launch_dec_dn_uq(&L.down, L.has_shared ? &L.sh_down : nullptr, c->hplanes, c->hmeta, c->tiles,
-                                     c->ntiles, max_tiles, g.experts, g.d, g.mid, c->pairs32, st)))
+      if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+             return moe_launch_dec_gu_uq(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->tiles, c->ntiles, max_tiles,
+                                         c->tokidx, g.experts, g.d, g.mid, c->hplanes, c->hmeta, st);
+           })))
         return rc;
-      prof_mark(c, MOE_PROF_DOWN, st);
-      rc = moe_launch_reduce(c->pairs32, false, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
-                             sh_first, y, P, g.d, g.topk, moe_hscale{nullptr, 0.f, 0.f}, st, nullptr);
-      prof_mark(c, MOE_PROF_REDUCE, st);
-      return rc;
+      if ((rc = stage(MOE_PROF_DOWN, [&]() -> int {
+             return moe_launch_dec_dn_uq(&L.down, shd, c->hplanes, c->hmeta, c->tiles, c->ntiles, max_tiles, g.experts,
+                                         g.d, g.mid, c->pairs32, st);
+           })))
+        return rc;
+      return stage(MOE_PROF_REDUCE, [&]() -> int {
+        return moe_launch_reduce(c->pairs32, false, c->pairids, c->pw, nullptr, sh ? c->sh_logit : nullptr, sh_first, y,
+                                 P, g.d, g.topk, moe_hscale{nullptr, 0.f, 0.f}, st, nullptr);
+      });
     }
     if (use_int) {
       // integer-dot kernels: activations as digit planes (made by the logits launch above)
-      rc = gu_topk ? moe_launch_dec_gu_topk(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
-                                            L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->logits,
-                                            g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
-                                            c->hplanes, c->hmeta, nullptr, st)
-                   : moe_launch_dec_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
-                                       L.has_shared ? &L.sh_up : nullptr, c->xplanes, c->xmeta, c->ids,
-                                       g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st);
-      if (rc) return rc;
-      prof_mark(c, MOE_PROF_UP, st);
-      rc = moe_launch_dec_dn(&L.down, L.has_shared ? &L.sh_down : nullptr, c->sh_logit, c->hplanes, c->hmeta,
-                             c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, y, (uint64_t)g.d, st);
-      prof_mark(c, MOE_PROF_DOWN, st);
-      return rc;
-    }
-    if ((rc = moe_launch_gemv_gu(&L.gate_up, L.has_shared ? &L.sh_gate : nullptr,
-                                 L.has_shared ? &L.sh_up : nullptr, x, (uint64_t)g.d, c->ids, g.id_stride,
-                                 g.topk, P, g.mid, c->hid32, st)))
-      return rc;
-    prof_mark(c, MOE_PROF_UP, st);
-    rc = moe_launch_gemv_dn(&L.down, L.has_shared ? &L.sh_down : nullptr, c->sh_logit, nullptr, nullptr,
-                            c->hid32, c->ids, c->ws, g.id_stride, g.topk, P, g.d, y, (uint64_t)g.d, st);
-    prof_mark(c, MOE_PROF_DOWN, st);
-    return rc;
-  }
-  if (L.has_shared && L.sh_gguf_type == 0) return MOE_E_UNSUPPORTED;
-  if (L.gg.tgu != MOE_GGML_Q4_K || L.gg.tdn != MOE_GGML_Q4_K || (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K)) {
-    // Q5_K gate/up, Q5_1 / Q8_0 down (or such a shared expert): the general kernels
-    for (int phase = 1; phase <= 2; phase++) {
-      if ((rc = moe_launch_ggx_gemv(phase, L.gg.tgu, L.gg.tdn, L.sh_gguf_type, L.gg.gate, L.gg.up, L.gg.down,
-                                    L.has_shared ? L.sh_gate.data : nullptr, L.has_shared ? L.sh_up.data : nullptr,
-                                    L.has_shared ? L.sh_down.data : nullptr, c->sh_logit, x, c->ids, c->ws, c->hid32,
-                                    y, P, g.d, g.mid, g.topk, g.id_stride, st)))
+      if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+             return gu_topk ? moe_launch_dec_gu_topk(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->logits, g.experts,
+                                                     c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes,
+                                                     c->hmeta, nullptr, st)
+                            : moe_launch_dec_gu(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->ids, g.id_stride, g.topk,
+                                                P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st);
+           })))
         return rc;
-      prof_mark(c, phase == 1 ? MOE_PROF_UP : MOE_PROF_DOWN, st);
+      return stage(MOE_PROF_DOWN, [&]() -> int {
+        return moe_launch_dec_dn(&L.down, shd, c->sh_logit, c->hplanes, c->hmeta, c->ids, c->ws, g.id_stride, g.topk, P,
+                                 g.d, g.mid, y, (uint64_t)g.d, st);
+      });
     }
+    if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+           return moe_launch_gemv_gu(&L.gate_up, shg, shu, x, (uint64_t)g.d, c->ids, g.id_stride, g.topk, P, g.mid,
+                                     c->hid32, st);
+         })))
+      return rc;
+    return stage(MOE_PROF_DOWN, [&]() -> int {
+      return moe_launch_gemv_dn(&L.down, shd, c->sh_logit, nullptr, nullptr, c->hid32, c->ids, c->ws, g.id_stride,
+                                g.topk, P, g.d, y, (uint64_t)g.d, st);
+    });
+  }
+  if (sh && L.sh_gguf_type == 0) return MOE_E_UNSUPPORTED;
+  if (L.gg.tgu != MOE_GGML_Q4_K || L.gg.tdn != MOE_GGML_Q4_K || (sh && L.sh_gguf_type != MOE_GGML_Q4_K)) {
+    // Q5_K gate/up, Q5_1 / Q8_0 down (or such a shared expert): the general kernels
+    for (int phase = 1; phase <= 2; phase++)
+      if ((rc = stage(phase == 1 ? MOE_PROF_UP : MOE_PROF_DOWN, [&]() -> int {
+             return moe_launch_ggx_gemv(phase, L.gg.tgu, L.gg.tdn, L.sh_gguf_type, L.gg.gate, L.gg.up, L.gg.down, rg, ru,
+                                        rd, c->sh_logit, x, c->ids, c->ws, c->hid32, y, P, g.d, g.mid, g.topk,
+                                        g.id_stride, st);
+           })))
+        return rc;
     return MOE_OK;
   }
   if (use_int4k) {
-    rc = gu_topk ? moe_launch_dec4k_gu_topk(L.gg.gate, L.gg.up, L.has_shared ? L.sh_gate.data : nullptr,
-                                            L.has_shared ? L.sh_up.data : nullptr, c->xplanes, c->xmeta, c->logits,
-                                            g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
-                                            c->hplanes, c->hmeta, st)
-                 : moe_launch_dec4k_gu(L.gg.gate, L.gg.up, L.has_shared ? L.sh_gate.data : nullptr,
-                                       L.has_shared ? L.sh_up.data : nullptr, c->xplanes, c->xmeta, c->ids,
-                                       g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, st);
-    if (rc) return rc;
-    prof_mark(c, MOE_PROF_UP, st);
-    rc = moe_launch_dec4k_dn(L.gg.down, L.has_shared ? L.sh_down.data : nullptr, c->sh_logit, c->hplanes, c->hmeta,
-                             c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, y, (uint64_t)g.d, st);
-    prof_mark(c, MOE_PROF_DOWN, st);
-    return rc;
-  }
-  for (int phase = 1; phase <= 2; phase++) {
-    if ((rc = moe_launch_q4k_gemv(phase, L.gg.gate, L.gg.up, L.gg.down, L.has_shared ? L.sh_gate.data : nullptr,
-                                  L.has_shared ? L.sh_up.data : nullptr, L.has_shared ? L.sh_down.data : nullptr,
-                                  c->sh_logit, x, c->ids, c->ws, c->hid32, y, P, g.d, g.mid, g.topk, g.id_stride,
-                                  st)))
+    if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+           return gu_topk ? moe_launch_dec4k_gu_topk(L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta, c->logits,
+                                                     g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
+                                                     c->hplanes, c->hmeta, st)
+                          : moe_launch_dec4k_gu(L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta, c->ids, g.id_stride,
+                                                g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, st);
+         })))
       return rc;
-    prof_mark(c, phase == 1 ? MOE_PROF_UP : MOE_PROF_DOWN, st);
+    return stage(MOE_PROF_DOWN, [&]() -> int {
+      return moe_launch_dec4k_dn(L.gg.down, rd, c->sh_logit, c->hplanes, c->hmeta, c->ids, c->ws, g.id_stride, g.topk, P,
+                                 g.d, g.mid, y, (uint64_t)g.d, st);
+    });
   }
+  for (int phase = 1; phase <= 2; phase++)
+    if ((rc = stage(phase == 1 ? MOE_PROF_UP : MOE_PROF_DOWN, [&]() -> int {
+           return moe_launch_q4k_gemv(phase, L.gg.gate, L.gg.up, L.gg.down, rg, ru, rd, c->sh_logit, x, c->ids, c->ws,
+                                      c->hid32, y, P, g.d, g.mid, g.topk, g.id_stride, st);
+         })))
+      return rc;
   return MOE_OK;
 }
 
