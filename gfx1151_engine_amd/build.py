@@ -10,10 +10,11 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvi
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
 
 
-def build(verbose=False):
-    """Compile every HIP source of the package into one shared library (always recompiles)."""
+def build(verbose=False, out=LIB, extra=()):
+    """Compile every HIP source of the package into one shared library (always recompiles).
+    out / extra: another output path and additional compiler flags (-D switches of experimental variants)."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + ["-o", LIB] + SOURCES
+    cmd = [hipcc] + FLAGS + list(extra) + ["-o", out] + SOURCES
     if verbose:
         print(" ".join(cmd))
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -22,7 +23,7 @@ def build(verbose=False):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
-    return LIB
+    return out
 
 
 if __name__ == "__main__":

@@ -40,9 +40,10 @@ _lib = None
 def lib():
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB):
-            raise MoeError(f"{LIB} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
-        _lib = C.CDLL(LIB)
+        path = os.environ.get("MI355MOE_LIB", LIB)  # another build of the same library (A/B timing runs)
+        if not os.path.exists(path):
+            raise MoeError(f"{path} is missing: run `python -c 'import __graft_entry__ as g; g.build()'`")
+        _lib = C.CDLL(path)
         _lib.moe_version.restype = C.c_char_p
         _lib.moe_status_string.restype = C.c_char_p
     return _lib
@@ -202,6 +203,7 @@ OPT_UNIQUE_MIN_TOKENS = 2
 OPT_FUSED_COMBINE = 3
 OPT_SHARED_ASIDE = 4
 OPT_TIMING_SKIP_STAGE = 5
+OPT_ROUTER_CANDIDATES = 6
 
 
 def lut_q4cp_view(blob, rows, cols, e_rows, up_off):

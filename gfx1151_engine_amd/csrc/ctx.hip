@@ -87,6 +87,9 @@ struct moe_ctx {
   int* ntiles_sh = nullptr;
   const moe_hc* hc = nullptr;  // set for the duration of moe_forward_hc: the combine writes into the HC state
   bool shared_aside = true;
+  // batch router through candidate selection (exact ids at a fraction of the fp64 work); its scratch
+  bool router_cand = true;
+  void* rc_scratch = nullptr;
 };
 
 static void prof_mark(moe_ctx* c, int stage_done, hipStream_t st) {
@@ -120,7 +123,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->ev_x16) (void)hipEventDestroy(c->ev_x16);
   if (c->side) (void)hipStreamDestroy(c->side);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->kpart, c->ktickets, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
-                  c->pairids, c->tiles, c->ntiles, c->tiles_sh, c->ntiles_sh, c->hid16, c->pairs16, c->pairs32};
+                  c->pairids, c->tiles, c->ntiles, c->tiles_sh, c->ntiles_sh, c->hid16, c->pairs16, c->pairs32, c->rc_scratch};
   for (void* b : bufs)
     if (b) {
       hipError_t e = hipFree(b);
@@ -185,7 +188,8 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   }
   if (e == hipSuccess && T > (size_t)c->small_max) {
     const size_t d = cfg->d, mid = cfg->mid;
-    e = hipMalloc(&c->x16, T * d * 2);
+    e = hipMalloc(&c->rc_scratch, moe_router_cand_scratch_bytes(cfg->max_tokens, cfg->experts));
+    if (e == hipSuccess) e = hipMalloc(&c->x16, T * d * 2);
     if (e == hipSuccess) e = hipMalloc(&c->hid16, k1 * T * mid * 2);
     if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);
   }
@@ -365,6 +369,7 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
       return MOE_OK;
     case MOE_OPT_FUSED_COMBINE: c->fused_combine = value != 0; return MOE_OK;
     case MOE_OPT_SHARED_ASIDE: c->shared_aside = value != 0; return MOE_OK;
+    case MOE_OPT_ROUTER_CANDIDATES: c->router_cand = value != 0; return MOE_OK;
     case MOE_OPT_TIMING_SKIP_STAGE:
       if (value < 0 || value > MOE_PROF_STAGES) return MOE_E_INVALID;
       c->skip_stage = value;
@@ -534,6 +539,20 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   return MOE_OK;
 }
 
+// Router of a batch: ids / ws, the shared-expert gate logit and (if asked) the per-token mean square of x.
+// By default through candidate selection (router_cand.hip); MOE_OPT_ROUTER_CANDIDATES = 0, or a shape it does not
+// take, runs the dense fp64 launch and the exact softmax / top-k over all experts.
+static int router_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* out_xms, hipStream_t st) {
+  const moe_config& g = c->cfg;
+  const moe_wview* wx = L.has_shared ? &L.sh_sg : nullptr;
+  if (c->router_cand && c->rc_scratch && moe_router_cand_supported(&L.router, wx, P, g.topk))
+    return moe_router_batch_cand(&L.router, L.router_bias, wx, x, P, c->logits, c->sh_logit, out_xms, c->ids, c->ws,
+                                 g.topk, g.id_stride, c->rc_scratch, st);
+  int rc = moe_router_logits_seq(&L.router, L.router_bias, wx, x, P, c->logits, c->sh_logit, out_xms, st);
+  if (!rc) rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
+  return rc;
+}
+
 // Batches: expert-sorted permutation, MFMA grouped GEMMs over <=128-pair tiles (the shared expert
 // rides along as expert index E over all tokens), f16 pair buffer, deterministic weighted combine.
 // Returns MOE_E_UNSUPPORTED (before enqueuing anything) for shapes / formats the GEMM does not cover.
@@ -592,8 +611,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
       rs = moe_launch_gemm_q4cp(false, &dn, &sdn, g.experts, c->hid16, nullptr, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
                                 c->pairs16, g.d, g.mid, true, q4k, hs, c->side, nullptr);
     // caller's stream: router, top-k, permutation, the routed experts' GEMMs
-    rc = moe_router_logits_seq(&L.router, L.router_bias, &L.sh_sg, x, P, c->logits, c->sh_logit, nullptr, st);
-    if (!rc) rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
+    rc = router_batch(c, L, x, P, nullptr, st);
     prof_mark(c, MOE_PROF_ROUTER, st);
     if (!rc)
       rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
@@ -621,9 +639,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     prof_mark(c, MOE_PROF_REDUCE, st);
     return rc;
   }
-  if ((rc = moe_router_logits_seq(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
-                                  c->sh_logit, c->xms, st)))
-    return rc;
+  if ((rc = router_batch(c, L, x, P, c->xms, st))) return rc;
   // x -> f16 (HBM-bound) on the side stream while top-k, counting, scan and scatter (small dependent
   // launches that leave the memory system idle) run on the caller's stream
   MOE_HIP(hipEventRecord(c->ev_fork, st));
@@ -639,7 +655,6 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   };
   const int sh_first = L.has_shared ? P * g.topk : -1;
   rc = rc16;
-  if (!rc) rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
   prof_mark(c, MOE_PROF_ROUTER, st);
   if (!rc)
     rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,

@@ -66,6 +66,16 @@ int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, con
 int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
                           float* logits, float* out_x, float* out_xms, hipStream_t st);
 
+int moe_router_logits_seq_if(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
+                             float* logits, float* out_x, float* out_xms, const int* run_if_above, int run_thr,
+                             hipStream_t st);
+// batch router through candidate selection (router_cand.hip): bit-exact ids, weights within an ulp or two
+bool moe_router_cand_supported(const moe_wview* W, const moe_wview* Wx, int P, int k);
+size_t moe_router_cand_scratch_bytes(int max_tokens, int experts);
+int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
+                          float* logits, float* out_x, float* out_xms, int* ids, float* ws, int k, int id_stride,
+                          void* scratch, hipStream_t st);
+
 size_t moe_qvec_plane_bytes(int K);
 size_t moe_qvec_meta_bytes(int K);
 bool moe_dec_supported(int d, int mid, int nslots);

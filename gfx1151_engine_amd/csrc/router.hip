@@ -36,7 +36,10 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
                                                            const float* __restrict__ x, int P, int E,
                                                            int d, float* __restrict__ logits,
                                                            float* __restrict__ out_x,
-                                                           float* __restrict__ out_xms, int ncol, int ntt) {
+                                                           float* __restrict__ out_xms, int ncol, int ntt,
+                                                           const int* __restrict__ run_if_above, int run_thr) {
+  // (a launch that is only needed when many tokens were listed for an exact redo returns at once otherwise)
+  if (run_if_above && *run_if_above <= run_thr) return;
   constexpr int MT = BT / 32;                 // 16-token MFMA tiles per wave
   constexpr int XL = (BT * RS_K / 4) / 256;   // float4 loads per thread and slab (activations)
   constexpr int WL = (RS_E * RS_K / 4) / 256; // (weights)
@@ -406,63 +409,16 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
   }
 }
 
-// ---- softmax + top-k, one wave per token (E <= 64*NPL) ----
-// Lane l holds experts NPL*l .. NPL*l + NPL - 1 (lane-major), so that among equal keys the lowest expert
-// sits in the lowest lane and register, and the selection can pre-sort each lane's keys.
+// ---- softmax + top-k, one wave per token (E <= 64*NPL): topk_wave in topk.h ----
 template <int NPL>
 __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ logits,
                                                      int* __restrict__ ids, float* __restrict__ ws,
                                                      int P, int E, int k, int id_stride) {
   __shared__ float pbuf[4][64 * NPL];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int wv = threadIdx.x >> 6;
   const int tok = blockIdx.x * 4 + wv;
   if (tok >= P) return;
-  const float* lg = logits + (size_t)tok * E;
-  float v[NPL];
-  float mxf = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < NPL; j++) {
-    const int e = NPL * lane + j;
-    v[j] = e < E ? lg[e] : -INFINITY;
-    mxf = fmaxf(mxf, v[j]);
-  }
-  const double mx = (double)wave_max(mxf);
-  // p = (float)exp((double)logit - mx)
-  float p[NPL];
-  bool exact = true;  // all partial sums representable -> any summation order gives the same fp64
-#pragma unroll
-  for (int j = 0; j < NPL; j++) {
-    const int e = NPL * lane + j;
-    p[j] = e < E ? (float)exp((double)v[j] - mx) : 0.f;
-    exact = exact && (p[j] == 0.f || p[j] >= 0x1p-20f);
-  }
-  double se;
-  if (__all(exact)) {
-    double s = 0.0;
-#pragma unroll
-    for (int j = 0; j < NPL; j++) s += (double)p[j];
-    se = wave_sum(s);
-  } else {
-    // very wide logit range: replay the reference's index order on one lane
-#pragma unroll
-    for (int j = 0; j < NPL; j++) pbuf[wv][NPL * lane + j] = p[j];
-    __builtin_amdgcn_s_waitcnt(0);
-    __builtin_amdgcn_wave_barrier();
-    double s = 0.0;
-    if (lane == 0)
-      for (int e = 0; e < E; e++) s += (double)pbuf[wv][e];
-    se = __shfl(s, 0, 64);
-  }
-  // probabilities are >= 0, so their bit patterns order like unsigned integers; key = bits + 1
-  // (0 = not a candidate: past E, or already selected)
-  uint32_t key[NPL];
-#pragma unroll
-  for (int j = 0; j < NPL; j++) {
-    const int e = NPL * lane + j;
-    key[j] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
-  }
-  if constexpr (NPL <= 8) topk_select_sorted<NPL>(key, lane, k, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride);
-  else topk_select_lm<NPL>(key, lane, k, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride);
+  topk_wave<NPL>(logits + (size_t)tok * E, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride, E, k, pbuf[wv]);
 }
 
 template <int NPL>
@@ -475,13 +431,14 @@ __global__ void __launch_bounds__(256) k_router_topk_block(const float* __restri
 // Launch of the sequential-order kernel: 128-token tiles when there are enough of them to fill the
 // chip, 64-token tiles otherwise.
 void launch_seq(const void* W, bool bf, const float* bias, const void* wx, bool xbf, const float* x, int P,
-                int E, int d, float* logits, float* out_x, float* out_xms, hipStream_t st) {
+                int E, int d, float* logits, float* out_x, float* out_xms, hipStream_t st,
+                const int* run_if_above = nullptr, int run_thr = 0) {
   const int ncol = (E + RS_E - 1) / RS_E;
   const bool big = (int64_t)((P + 127) / 128) * ncol >= 512;
   const int bt = big ? 128 : 64;
   const int ntt = (P + bt - 1) / bt;
   const unsigned grid = (unsigned)(((ntt + 7) / 8) * 8 * ncol);
-#define RS_GO(BF, BT) k_router_logits_seq<BF, BT><<<grid, 256, 0, st>>>(W, bias, wx, xbf, x, P, E, d, logits, out_x, out_xms, ncol, ntt)
+#define RS_GO(BF, BT) k_router_logits_seq<BF, BT><<<grid, 256, 0, st>>>(W, bias, wx, xbf, x, P, E, d, logits, out_x, out_xms, ncol, ntt, run_if_above, run_thr)
   if (bf) { if (big) RS_GO(true, 128); else RS_GO(true, 64); }
   else { if (big) RS_GO(false, 128); else RS_GO(false, 64); }
 #undef RS_GO
@@ -669,6 +626,18 @@ int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
   const void* wx = Wx ? Wx->data : nullptr;
   launch_seq(W->data, W->dtype == MOE_DT_BF16, bias, wx, xbf, x, P, E, d, logits, out_x, out_xms, st);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// Internal: the same launch, doing its work only if *run_if_above > run_thr when it starts (device memory).
+int moe_router_logits_seq_if(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
+                             float* logits, float* out_x, float* out_xms, const int* run_if_above, int run_thr,
+                             hipStream_t st) {
+  const int E = (int)W->rows, d = (int)W->cols;
+  const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
+  launch_seq(W->data, W->dtype == MOE_DT_BF16, bias, Wx ? Wx->data : nullptr, xbf, x, P, E, d, logits, out_x, out_xms, st,
+             run_if_above, run_thr);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -1,0 +1,555 @@
+// Batch router without the dense fp64 pass: bit-exact expert ids at a fraction of the fp64 work.
+//
+// The reference's router (src/ref.cpp:565-594) needs every logit as a sequential fp64 sum, but only the k
+// best logits of a token decide its experts and weights; the other ~500 enter through the softmax
+// normaliser alone, which cancels in the renormalised weights up to rounding.  So:
+//   1. k_router_approx   all T x E logits on the f16 matrix pipe (f32 accumulation), with the row norms of x and W;
+//   2. k_router_cand     per token a RIGOROUS error bound B_e on each approximate logit (below) gives an interval
+//                        [a_e - B_e, a_e + B_e] that holds the exact logit; tau = the k-th largest lower end; every
+//                        expert whose upper end reaches tau - 1e-5 is a candidate (the true top k are among them:
+//                        at least k exact logits are >= tau, and a true top-k logit is >= the k-th largest exact one);
+//   3. k_router_exact_pairs the candidates' logits (typically 12-18 of 512) as the reference's sequential fp64
+//                        chains, one lane per (token, candidate), written over the approximate values;
+//   4. k_router_topk_mixed  ranks the k + 1 best logits; if every gap between neighbours exceeds 1e-6 and all lie
+//                        within 70 of the maximum, the order by logit is the reference's order by f32 probability
+//                        (no two of them can round to one float) and the ids are final; the weights use the exact
+//                        logits of the selected experts and a normaliser in which the non-candidates' terms are
+//                        approximate, which moves a renormalised weight by an ulp or two at most;
+//   5. tokens that fail any test (near ties, a logit range where probabilities underflow, more candidates than
+//      lanes, non-finite values) are listed and redone exactly: all E logits as fp64 chains and the exact softmax /
+//      top-k; when more than T/16 tokens are listed the dense fp64 kernel runs for the whole batch instead.
+// Error bound.  a~ = fl32(sum of f16(x_c) * f16(w_c)): |f16(v) - v| <= 2^-11 |v| + 2^-25 (the second term covers
+// f16 subnormals), so sum |x~ w~ - x w| <= 1.001 (2^-10 |x||w| + 2^-25 sqrt(d) (|x| + |w|)) by Cauchy-Schwarz, and
+// the accumulation adds at most d * 2^-22 * 1.001 |x||w| however the matrix pipe orders and rounds its partial sums
+// (twice the IEEE bound per addition, one addition charged per product).  Non-finite approximations (overflow of
+// the f16 conversions) send the token to step 5.
+#include "common.h"
+#include "internal.h"
+#include "topk.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int RA_BT = 128, RA_BE = 128, RA_K = 32;
+constexpr int RA_PITCH = 80;  // bytes per LDS row: 32 f16 + 16 B of padding (the 16-byte fragment reads of 8 rows then cover all banks)
+constexpr int RC_SLOTS = 32;  // lanes per token in the exact pass: up to 31 candidates + the shared-expert gate row
+
+// ---- 1. approximate logits: block = 128 tokens x 128 experts, 4 waves as 2 x 2, wave = 64 x 64 (2 x 2 MFMA tiles) ----
+template <bool BF16>
+__global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict__ W, const float* __restrict__ bias,
+                                                         const float* __restrict__ x, int P, int E, int d,
+                                                         float* __restrict__ alog, float* __restrict__ wnorm,
+                                                         float* __restrict__ xnorm, float* __restrict__ out_xms,
+                                                         int* __restrict__ counters, int ncol, int ntt) {
+  __shared__ __attribute__((aligned(16))) uint8_t Xs[RA_BT * RA_PITCH];
+  __shared__ __attribute__((aligned(16))) uint8_t Ws[RA_BE * RA_PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int n = lane & 31, h = lane >> 5, wm = wv >> 1, wn = wv & 1;
+  const int b = blockIdx.x, xcd = b & 7, q = b >> 3;
+  const int col = q % ncol, tt = (q / ncol) * 8 + xcd;  // the column blocks of a token tile share an XCD (and its L2 copy of x)
+  if (b == 0 && tid == 0) {
+    counters[0] = 0;  // tokens listed for the exact redo
+    counters[1] = 0;  // (token, row) pairs of the exact pass      (both are first used by later launches)
+  }
+  if (tt >= ntt) return;
+  const int e0 = col * RA_BE, t0 = tt * RA_BT;
+
+  float4 xr[4], wr[4];
+  auto fetch = [&](int c0) {
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+      const int i = tid + it * 256, r = i >> 3, cc = c0 + (i & 7) * 4;
+      const int t = t0 + r, e = e0 + r;
+      xr[it] = t < P ? *(const float4*)(x + (size_t)t * d + cc) : float4{0.f, 0.f, 0.f, 0.f};
+      if (e < E) {
+        if (BF16) {
+          const uint2 u = *(const uint2*)((const uint16_t*)W + (size_t)e * d + cc);
+          wr[it] = float4{__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                          __uint_as_float(u.y & 0xffff0000u)};
+        } else {
+          wr[it] = *(const float4*)((const float*)W + (size_t)e * d + cc);
+        }
+      } else {
+        wr[it] = float4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+  };
+  float xs2[4] = {0.f, 0.f, 0.f, 0.f}, ws2[4] = {0.f, 0.f, 0.f, 0.f};
+  auto stage = [&]() {
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+      const int i = tid + it * 256, r = i >> 3, m = i & 7;
+      const float4 a = xr[it], w = wr[it];
+      xs2[it] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+      ws2[it] += w.x * w.x + w.y * w.y + w.z * w.z + w.w * w.w;
+      *(half4v*)(Xs + r * RA_PITCH + m * 8) = half4v{(_Float16)a.x, (_Float16)a.y, (_Float16)a.z, (_Float16)a.w};
+      *(half4v*)(Ws + r * RA_PITCH + m * 8) = half4v{(_Float16)w.x, (_Float16)w.y, (_Float16)w.z, (_Float16)w.w};
+    }
+  };
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  fetch(0);
+  for (int c0 = 0; c0 < d; c0 += RA_K) {
+    __syncthreads();  // the previous slab has been read
+    stage();
+    __syncthreads();
+    if (c0 + RA_K < d) fetch(c0 + RA_K);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      half8 a[2], bq[2];
+#pragma unroll
+      for (int mf = 0; mf < 2; mf++) a[mf] = *(const half8*)(Xs + (wm * 64 + 32 * mf + n) * RA_PITCH + ks * 32 + h * 16);
+#pragma unroll
+      for (int nf = 0; nf < 2; nf++) bq[nf] = *(const half8*)(Ws + (wn * 64 + 32 * nf + n) * RA_PITCH + ks * 32 + h * 16);
+#pragma unroll
+      for (int mf = 0; mf < 2; mf++)
+#pragma unroll
+        for (int nf = 0; nf < 2; nf++)
+          acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], bq[nf], acc[mf][nf], 0, 0, 0);
+    }
+  }
+  // D[i][j]: j = lane % 32 (expert), i = 8 * (r / 4) + 4 * (lane / 32) + r % 4 (token)
+#pragma unroll
+  for (int mf = 0; mf < 2; mf++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int t = t0 + wm * 64 + 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (t >= P) continue;
+#pragma unroll
+      for (int nf = 0; nf < 2; nf++) {
+        const int e = e0 + wn * 64 + 32 * nf + n;
+        if (e < E) alog[(size_t)t * E + e] = acc[mf][nf][r] + (bias ? bias[e] : 0.f);
+      }
+    }
+  // row norms: the 8 threads that share a row are 8 consecutive lanes
+#pragma unroll
+  for (int it = 0; it < 4; it++) {
+    float sx = xs2[it], sw = ws2[it];
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) {
+      sx += __shfl_xor(sx, o, 64);
+      sw += __shfl_xor(sw, o, 64);
+    }
+    const int r = (tid + it * 256) >> 3;
+    if ((tid & 7) == 0) {
+      if (col == 0 && t0 + r < P) {
+        xnorm[t0 + r] = sqrtf(sx);
+        if (out_xms) out_xms[t0 + r] = sx / (float)d;
+      }
+      if (tt == 0 && e0 + r < E) wnorm[e0 + r] = sqrtf(sw);
+    }
+  }
+}
+
+// ---- 2. candidates: one wave per token, lane l holds experts NPL*l .. NPL*l + NPL - 1 ----
+template <int NPL>
+__global__ void __launch_bounds__(1024) k_router_cand(const float* __restrict__ alog, const float* __restrict__ wnorm,
+                                                     const float* __restrict__ xnorm, int P, int E, int k, float eps,
+                                                     float dterm, uint32_t* __restrict__ pairs, int* __restrict__ nc,
+                                                     int* __restrict__ fb_list, int* __restrict__ counters, int gate_row) {
+  __shared__ int s_want[16], s_base;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int t = blockIdx.x * 16 + wv;
+  const bool tok = t < P;
+  const float xn = xnorm[tok ? t : 0];
+  float U[NPL], L[NPL];
+  bool fin = isfinite(xn);
+  float maxU = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = NPL * lane + j;
+    if (e < E && tok) {
+      const float a = alog[(size_t)t * E + e], wn = wnorm[e];
+      const float B = eps * xn * wn + dterm * (xn + wn) + 1e-6f * (1.f + fabsf(a));
+      fin = fin && isfinite(a) && isfinite(B);
+      U[j] = a + B;
+      L[j] = a - B;
+    } else {
+      U[j] = L[j] = -INFINITY;
+    }
+    maxU = fmaxf(maxU, U[j]);
+  }
+  maxU = wave_fmax_dpp(maxU);
+  // tau = the k-th largest lower end
+  float tau = -INFINITY;
+  for (int r = 0; r < k; r++) {
+    float m = L[0];
+#pragma unroll
+    for (int j = 1; j < NPL; j++) m = fmaxf(m, L[j]);
+    const float wmx = wave_fmax_dpp(m);
+    const int owner = __builtin_ctzll(__ballot(m == wmx) | (1ull << 63));
+    tau = wmx;
+    if (lane == owner) {  // drop one instance
+      bool done = false;
+#pragma unroll
+      for (int j = 0; j < NPL; j++) {
+        const bool hit = !done && L[j] == wmx;
+        L[j] = hit ? -INFINITY : L[j];
+        done = done || hit;
+      }
+    }
+  }
+  const float thr = tau - 1e-5f;
+  int mine = 0;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) mine += (U[j] >= thr) ? 1 : 0;
+  int inc = mine;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int v = __shfl_up(inc, o, 64);
+    if (lane >= o) inc += v;
+  }
+  const int total = __shfl(inc, 63, 64);
+  const bool ok = __all(fin) && total <= RC_SLOTS - 1 && total >= 1 && (maxU - thr) < 60.f && isfinite(tau);
+  // The (token, row) pairs of the exact pass go into one dense list (token << 10 | row; row E = the shared-expert
+  // gate vector, which every token needs).  A token's pairs are contiguous; the order of the tokens in the list
+  // depends on timing, the result of a pair does not.
+  // (one atomic per block of 16 tokens: thousands of atomics on one address would serialise for longer than the
+  // rest of the kernel takes)
+  const int want = tok ? (ok ? total : 0) + gate_row : 0;
+  if (lane == 0) s_want[wv] = want;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sum = 0;
+    for (int i = 0; i < 16; i++) sum += s_want[i];
+    s_base = sum ? atomicAdd(&counters[1], sum) : 0;
+  }
+  __syncthreads();
+  if (!tok) return;
+  int base = s_base;
+  for (int i = 0; i < wv; i++) base += s_want[i];
+  if (gate_row && lane == 0) pairs[base] = ((uint32_t)t << 10) | (uint32_t)E;
+  if (!ok) {
+    if (lane == 0) {
+      nc[t] = -1;
+      fb_list[atomicAdd(&counters[0], 1)] = t;
+    }
+    return;
+  }
+  int pos = base + gate_row + inc - mine;
+#pragma unroll
+  for (int j = 0; j < NPL; j++)
+    if (U[j] >= thr) pairs[pos++] = ((uint32_t)t << 10) | (uint32_t)(NPL * lane + j);
+  if (lane == 0) nc[t] = total;
+}
+
+// One sequential fp64 chain over c = 0..d-1 per lane: acc = fma((double)w[c], (double)x[c], acc); the f32 x f32
+// product is exact in fp64, so this is the reference's `acc += (double)w * x` bit for bit.  Every lane streams its
+// own weight row, 128 bytes (a cache line) at a time, the next 32 columns in flight while the current ones are used.
+template <bool BF16>
+__device__ __forceinline__ double chain_row(const void* wrow, const float* xrow, int d) {
+  double acc = 0.0;
+  float4 wq[8], xq[8];
+  auto load = [&](int c) {
+    if (BF16) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint4 u = *(const uint4*)((const uint16_t*)wrow + c + 8 * i);
+        wq[2 * i] = float4{__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                           __uint_as_float(u.y & 0xffff0000u)};
+        wq[2 * i + 1] = float4{__uint_as_float(u.z << 16), __uint_as_float(u.z & 0xffff0000u),
+                               __uint_as_float(u.w << 16), __uint_as_float(u.w & 0xffff0000u)};
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) wq[i] = *(const float4*)((const float*)wrow + c + 4 * i);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) xq[i] = *(const float4*)(xrow + c + 4 * i);
+  };
+  load(0);
+  for (int c = 0; c < d; c += 32) {
+    float4 w[8], xv[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      w[i] = wq[i];
+      xv[i] = xq[i];
+    }
+    if (c + 32 < d) load(c + 32);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      acc = fma((double)w[i].x, (double)xv[i].x, acc);
+      acc = fma((double)w[i].y, (double)xv[i].y, acc);
+      acc = fma((double)w[i].z, (double)xv[i].z, acc);
+      acc = fma((double)w[i].w, (double)xv[i].w, acc);
+    }
+  }
+  return acc;
+}
+
+// ---- 3. exact logits of the listed (token, row) pairs: a lane per pair, 64 pairs per wave ----
+// f32 weights: a wave stages the 64 weight-row pieces of an iteration (32 columns = one 128-byte line per row)
+// through LDS, so that a load instruction fetches 8 whole lines (8 lanes per row) instead of 16 bytes of 64
+// different lines; lane l of instruction i takes row 8i + l/8, piece (l%8 + l/8) % 8, which lands at byte 16 l of
+// the instruction's 1 KB image, and a lane reads its own row's piece j from slot 8a + (j - a) % 8, a = row % 8:
+// the 8 lanes of an LDS phase then hit 8 different 16-byte bank groups.  Two images per wave (next iteration in
+// flight), waves are independent (no block barrier).  Activations come straight from global memory: the pairs of
+// a token are neighbours in the list, so a wave touches a handful of rows.
+template <bool BF16>
+__global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restrict__ W, const float* __restrict__ bias,
+                                                            const void* __restrict__ Wx, const float* __restrict__ x,
+                                                            int E, int d, const uint32_t* __restrict__ pairs,
+                                                            const int* __restrict__ counters,
+                                                            float* __restrict__ logits, float* __restrict__ out_x) {
+  __shared__ __attribute__((aligned(16))) uint8_t img[4][2][8192];
+  const int np = counters[1];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int p0 = (blockIdx.x * 4 + wv) * 64;
+  if (p0 >= np) return;
+  const bool live = p0 + lane < np;
+  const uint32_t pr = pairs[live ? p0 + lane : p0];  // idle lanes repeat the wave's first pair (no extra traffic)
+  const int t = (int)(pr >> 10), e = (int)(pr & 1023u);
+  const bool gate = e == E;
+  const uint8_t* wrow = gate ? (const uint8_t*)Wx : (const uint8_t*)W + (size_t)e * d * (BF16 ? 2 : 4);
+  const float* xrow = x + (size_t)t * d;
+  double acc = 0.0;
+  if constexpr (BF16) {
+    acc = chain_row<true>(wrow, xrow, d);
+  } else {
+    // row pointers of the 8 rows this lane fetches pieces of
+    const uint8_t* src[8];
+    const int a = lane >> 3, piece = ((lane & 7) + a) & 7;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const uint64_t pw = (uint64_t)wrow;
+      const int from = 8 * i + a;
+      const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)pw, from, 64), hi = (uint32_t)__shfl((int)(uint32_t)(pw >> 32), from, 64);
+      src[i] = (const uint8_t*)(((uint64_t)hi << 32) | lo) + piece * 16;
+    }
+    uint8_t* const my = &img[wv][0][0];
+    auto issue = [&](int c, int buf) {
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[i] + (size_t)c * 4),
+                                         (__attribute__((address_space(3))) void*)(my + buf * 8192 + i * 1024), 16, 0, 0);
+    };
+    float4 xq[8];
+    auto loadx = [&](int c) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) xq[i] = *(const float4*)(xrow + c + 4 * i);
+    };
+    const int ar = lane & 7;
+    const uint8_t* rd = my + (lane >> 3) * 1024 + ar * 128;  // this lane's row inside an image
+    issue(0, 0);
+    loadx(0);
+    int buf = 0;
+    for (int c = 0; c < d; c += 32) {
+      float4 xv[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) xv[i] = xq[i];
+      const bool more = c + 32 < d;
+      if (more) {
+        issue(c + 32, buf ^ 1);
+        loadx(c + 32);
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // all but the 16 loads just issued have landed (LDS image of this iteration)
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      float4 w[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) w[j] = *(const float4*)(rd + buf * 8192 + (((j - ar) & 7) << 4));
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        acc = fma((double)w[i].x, (double)xv[i].x, acc);
+        acc = fma((double)w[i].y, (double)xv[i].y, acc);
+        acc = fma((double)w[i].z, (double)xv[i].z, acc);
+        acc = fma((double)w[i].w, (double)xv[i].w, acc);
+      }
+      buf ^= 1;
+    }
+  }
+  if (!live) return;
+  if (gate) out_x[t] = (float)acc;
+  else {
+    float v = (float)acc;
+    if (bias) v += bias[e];
+    logits[(size_t)t * E + e] = v;
+  }
+}
+
+// ---- 4. ids and weights from the mixed logits (exact for the candidates) ----
+template <int NPL>
+__global__ void __launch_bounds__(256) k_router_topk_mixed(const float* __restrict__ lg, int* __restrict__ ids,
+                                                           float* __restrict__ ws, int P, int E, int k, int id_stride,
+                                                           const int* __restrict__ nc, int* __restrict__ fb_list,
+                                                           int* __restrict__ counters) {
+  static_assert(NPL <= 8, "4-bit index fields in one 32-bit word");
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + wv;
+  if (t >= P || nc[t] < 0) return;  // listed already
+  float v[NPL];
+  uint32_t key[NPL], jj[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = NPL * lane + j;
+    v[j] = e < E ? lg[(size_t)t * E + e] : -INFINITY;
+    const uint32_t u = __float_as_uint(v[j]);
+    key[j] = e < E ? ((u & 0x80000000u) ? ~u : (u | 0x80000000u)) : 0u;  // unsigned keys that order like the floats
+    jj[j] = (uint32_t)j;
+  }
+#pragma unroll
+  for (int pass = 0; pass < NPL; pass++) {
+#pragma unroll
+    for (int i = pass & 1; i + 1 < NPL; i += 2) {
+      const uint32_t ka = key[i], kb = key[i + 1], ia = jj[i], ib = jj[i + 1];
+      const bool sw = kb > ka;
+      key[i] = umax(ka, kb); key[i + 1] = umin(ka, kb);
+      jj[i] = sw ? ib : ia; jj[i + 1] = sw ? ia : ib;
+    }
+  }
+  uint32_t jw = 0;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) jw |= jj[j] << (4 * j);
+  uint32_t mykey = 0;
+  int myid = 0;
+  for (int r = 0; r <= k; r++) {  // k + 1 rounds: the runner-up is needed for the gap test
+    const uint32_t wmx = wave_umax(key[0]);
+    const int wl = __builtin_ctzll(__ballot(key[0] == wmx) | (1ull << 63));
+    const int wj = __builtin_amdgcn_readlane((int)jw, wl) & 15;
+    if (lane == r) {
+      mykey = wmx;
+      myid = NPL * wl + wj;
+    }
+    const bool me = lane == wl;
+#pragma unroll
+    for (int j = 0; j + 1 < NPL; j++) {
+      const uint32_t cur = key[j], nxt = key[j + 1];
+      key[j] = me ? nxt : cur;
+    }
+    const uint32_t last = key[NPL - 1], jsh = jw >> 4;
+    key[NPL - 1] = me ? 0u : last;
+    jw = me ? jsh : jw;
+  }
+  const uint32_t nk = (uint32_t)__shfl_down((int)mykey, 1, 64);
+  const float la = __uint_as_float((mykey & 0x80000000u) ? (mykey ^ 0x80000000u) : ~mykey);
+  const float lb = __uint_as_float((nk & 0x80000000u) ? (nk ^ 0x80000000u) : ~nk);
+  const float lmax = __shfl(la, 0, 64);
+  const bool good = lane >= k || (mykey != 0u && nk != 0u && la - lb > 1e-6f && lmax - lb < 70.f);  // false for NaNs
+  if (!__all(good)) {
+    if (lane == 0) fb_list[atomicAdd(&counters[0], 1)] = t;
+    return;
+  }
+  // softmax terms of every expert (the non-candidates' are approximate: they only enter the normaliser)
+  const double mx = (double)lmax;
+  double s = 0.0;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) s += (double)(NPL * lane + j < E ? (float)exp((double)v[j] - mx) : 0.f);
+  const double se = wave_dsum_dpp(s);
+  const float sc = lane < k ? (float)((double)(float)exp((double)la - mx) / se) : 0.f;
+  double wsum = 0.0;
+  for (int r = 0; r < k; r++) wsum += (double)__shfl(sc, r, 64);  // selection order, as the reference's loop
+  if (lane < k) {
+    ids[(size_t)t * id_stride + lane] = myid;
+    ws[(size_t)t * id_stride + lane] = (float)((double)sc / wsum);
+  }
+}
+
+// ---- 5. listed tokens: every logit as an fp64 chain (a lane per expert), unless the dense kernel takes over ----
+template <bool BF16>
+__global__ void __launch_bounds__(256) k_router_exact_listed(const void* __restrict__ W, const float* __restrict__ bias,
+                                                             const float* __restrict__ x, int E, int d,
+                                                             const int* __restrict__ fb_list,
+                                                             const int* __restrict__ counters, int dense_above,
+                                                             float* __restrict__ logits) {
+  const int nl = counters[0];
+  if (nl == 0 || nl > dense_above) return;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int ne64 = (E + 63) >> 6, total = nl * ne64;
+  for (int item = blockIdx.x * 4 + wv; item < total; item += gridDim.x * 4) {
+    const int t = fb_list[item / ne64], e = 64 * (item % ne64) + lane;
+    const int er = e < E ? e : 0;
+    const double acc = chain_row<BF16>((const uint8_t*)W + (size_t)er * d * (BF16 ? 2 : 4), x + (size_t)t * d, d);
+    if (e < E) logits[(size_t)t * E + e] = (float)acc + (bias ? bias[e] : 0.f);
+  }
+}
+
+// exact softmax / top-k of the listed tokens (of every token when the dense kernel ran)
+template <int NPL>
+__global__ void __launch_bounds__(256) k_router_topk_listed(const float* __restrict__ logits, int* __restrict__ ids,
+                                                            float* __restrict__ ws, int P, int E, int k, int id_stride,
+                                                            const int* __restrict__ fb_list,
+                                                            const int* __restrict__ counters, int dense_above) {
+  __shared__ float pbuf[4][64 * NPL];
+  const int nl = counters[0];
+  if (nl == 0) return;
+  const int wv = threadIdx.x >> 6;
+  const int w = blockIdx.x * 4 + wv;
+  int tok;
+  if (nl > dense_above) {
+    if (w >= P) return;
+    tok = w;
+  } else {
+    if (w >= nl) return;
+    tok = fb_list[w];
+  }
+  topk_wave<NPL>(logits + (size_t)tok * E, ids + (size_t)tok * id_stride, ws + (size_t)tok * id_stride, E, k, pbuf[wv]);
+}
+
+}  // namespace
+
+bool moe_router_cand_supported(const moe_wview* W, const moe_wview* Wx, int P, int k) {
+  const int E = (int)W->rows, d = (int)W->cols;
+  if (P < 1 || d % 32 || d < 32 || E > 512 || k + 1 > RC_SLOTS - 1 || k >= E) return false;
+  if (Wx && (Wx->dtype == MOE_DT_BF16) != (W->dtype == MOE_DT_BF16)) return false;
+  return moe_aligned(W->data, 16) && (!Wx || moe_aligned(Wx->data, 16));
+}
+
+size_t moe_router_cand_scratch_bytes(int max_tokens, int experts) {
+  // counters [16], pairs [T][32] u32, nc [T], fb_list [T], xnorm [T], wnorm [E]
+  return (size_t)max_tokens * (RC_SLOTS * 4 + 4 + 4 + 4) + (size_t)experts * 4 + 64 + 256;
+}
+
+// Internal: ids / ws (and the shared-expert gate logit, the per-token mean square of x) of a batch; `logits` ends
+// up holding exact values for each token's candidates and approximate ones elsewhere.
+int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
+                          float* logits, float* out_x, float* out_xms, int* ids, float* ws, int k, int id_stride,
+                          void* scratch, hipStream_t st) {
+  const int E = (int)W->rows, d = (int)W->cols;
+  if (!moe_router_cand_supported(W, Wx, P, k) || !moe_aligned(x, 16)) return MOE_E_UNSUPPORTED;
+  uint8_t* sp = (uint8_t*)scratch;
+  int* counters = (int*)sp; sp += 64;
+  uint32_t* pairs = (uint32_t*)sp; sp += (size_t)P * RC_SLOTS * 4;
+  int* nc = (int*)sp; sp += (size_t)P * 4;
+  int* fb_list = (int*)sp; sp += (size_t)P * 4;
+  float* xnorm = (float*)sp; sp += (size_t)P * 4;
+  float* wnorm = (float*)sp;
+  const bool bf = W->dtype == MOE_DT_BF16;
+  const int ncol = (E + RA_BE - 1) / RA_BE, ntt = (P + RA_BT - 1) / RA_BT;
+  const unsigned grid_a = (unsigned)(((ntt + 7) / 8) * 8 * ncol);
+  const float eps = (0x1p-10f + (float)d * 0x1p-22f) * 1.002f * 1.01f;  // 1.01: the f32 norms' own rounding
+  const float dterm = 0x1p-25f * 1.01f * sqrtf((float)d);
+  const int dense_above = P / 16;
+  const void* wx = Wx ? Wx->data : nullptr;
+  const unsigned gtok = (unsigned)((P + 3) / 4), gtok16 = (unsigned)((P + 15) / 16);
+  if (bf) k_router_approx<true><<<grid_a, 256, 0, st>>>(W->data, bias, x, P, E, d, logits, wnorm, xnorm, out_xms, counters, ncol, ntt);
+  else k_router_approx<false><<<grid_a, 256, 0, st>>>(W->data, bias, x, P, E, d, logits, wnorm, xnorm, out_xms, counters, ncol, ntt);
+  MOE_LAUNCH_CHECK();
+  k_router_cand<8><<<gtok16, 1024, 0, st>>>(logits, wnorm, xnorm, P, E, k, eps, dterm, pairs, nc, fb_list, counters,
+                                         wx ? 1 : 0);
+  MOE_LAUNCH_CHECK();
+  // at most 32 pairs per token (31 candidates + the gate row); surplus blocks return at once
+  const unsigned gpair = (unsigned)(((size_t)P * RC_SLOTS + 255) / 256);
+  if (bf) k_router_exact_pairs<true><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x);
+  else k_router_exact_pairs<false><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x);
+  MOE_LAUNCH_CHECK();
+  k_router_topk_mixed<8><<<gtok, 256, 0, st>>>(logits, ids, ws, P, E, k, id_stride, nc, fb_list, counters);
+  MOE_LAUNCH_CHECK();
+  // the exact redo of the listed tokens: three launches that return at once when nothing is listed
+  if (bf) k_router_exact_listed<true><<<512, 256, 0, st>>>(W->data, bias, x, E, d, fb_list, counters, dense_above, logits);
+  else k_router_exact_listed<false><<<512, 256, 0, st>>>(W->data, bias, x, E, d, fb_list, counters, dense_above, logits);
+  MOE_LAUNCH_CHECK();
+  int rc = moe_router_logits_seq_if(W, bias, nullptr, x, P, logits, nullptr, nullptr, counters, dense_above, st);
+  if (rc) return rc;
+  k_router_topk_listed<8><<<gtok, 256, 0, st>>>(logits, ids, ws, P, E, k, id_stride, fb_list, counters, dense_above);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}

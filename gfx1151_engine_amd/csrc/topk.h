@@ -196,6 +196,60 @@ __device__ __forceinline__ void topk_select_sorted(uint32_t (&key)[NPL], int lan
   }
 }
 
+// The softmax / top-k of one token by one wave (E <= 64 * NPL): lane l holds experts NPL*l .. NPL*l + NPL - 1
+// (lane-major), so that among equal keys the lowest expert sits in the lowest lane and register, and the
+// selection can pre-sort each lane's keys.  pbuf: 64 * NPL floats of LDS owned by this wave.
+template <int NPL>
+__device__ __forceinline__ void topk_wave(const float* __restrict__ lg, int* __restrict__ ids_row,
+                                          float* __restrict__ ws_row, int E, int k, float* pbuf) {
+  const int lane = threadIdx.x & 63;
+  float v[NPL];
+  float mxf = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = NPL * lane + j;
+    v[j] = e < E ? lg[e] : -INFINITY;
+    mxf = fmaxf(mxf, v[j]);
+  }
+  const double mx = (double)wave_max(mxf);
+  // p = (float)exp((double)logit - mx)
+  float p[NPL];
+  bool exact = true;  // all partial sums representable -> any summation order gives the same fp64
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = NPL * lane + j;
+    p[j] = e < E ? (float)exp((double)v[j] - mx) : 0.f;
+    exact = exact && (p[j] == 0.f || p[j] >= 0x1p-20f);
+  }
+  double se;
+  if (__all(exact)) {
+    double s = 0.0;
+#pragma unroll
+    for (int j = 0; j < NPL; j++) s += (double)p[j];
+    se = wave_sum(s);
+  } else {
+    // very wide logit range: replay the reference's index order on one lane
+#pragma unroll
+    for (int j = 0; j < NPL; j++) pbuf[NPL * lane + j] = p[j];
+    __builtin_amdgcn_s_waitcnt(0);
+    __builtin_amdgcn_wave_barrier();
+    double s = 0.0;
+    if (lane == 0)
+      for (int e = 0; e < E; e++) s += (double)pbuf[e];
+    se = __shfl(s, 0, 64);
+  }
+  // probabilities are >= 0, so their bit patterns order like unsigned integers; key = bits + 1
+  // (0 = not a candidate: past E, or already selected)
+  uint32_t key[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; j++) {
+    const int e = NPL * lane + j;
+    key[j] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
+  }
+  if constexpr (NPL <= 8) topk_select_sorted<NPL>(key, lane, k, ids_row, ws_row);
+  else topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
+}
+
 // The softmax / top-k of one token by one block of NT threads (E <= 64*NPL): the fp64 exps, the
 // costly part, are spread over the block; wave 0 then runs the k selection rounds on the keys in
 // LDS.  COH: the logits were written by other blocks of the same launch: read them with

@@ -250,12 +250,19 @@ int moe_forward_hc(moe_ctx* ctx, int layer, const float* x, int P, const float* 
 /* MOE_OPT_SHARED_ASIDE (default 1): batches over 32 tokens run the shared expert's two GEMMs (which do not depend
  * on the routing) on the context's side stream from the start of the call, next to the router launch; 0 = the shared
  * expert's tiles ride in the routed experts' launches.  Same arithmetic either way. */
+/* MOE_OPT_ROUTER_CANDIDATES (default 1): batches over 32 tokens find each token's experts without the dense fp64
+ * pass over all experts: approximate logits on the f16 matrix pipe with a rigorous error bound select the experts
+ * that can be among the k best, whose logits are then computed as the reference's sequential fp64 sums
+ * (src/ref.cpp:70-77); tokens with near ties or a logit range in which probabilities underflow are redone with the
+ * exact arithmetic over all experts.  Expert ids and their order are the reference's bit for bit; the renormalised
+ * weights can differ from it in the last bit or two (the softmax normaliser, which cancels in them up to rounding,
+ * contains approximate terms for the experts that were not candidates).  0 = dense fp64 logits and exact weights. */
 /* MOE_OPT_TIMING_SKIP_STAGE (default 0): timing experiments only.  value = 1 + MOE_PROF_* stage: calls with at most 32
  * tokens leave that stage's launches out (the later stages then work on stale scratch and the output is meaningless).
  * The difference between the times of a loop of calls without and with the skip is that stage's cost inside the
  * pipelined stream, without the dispatch latency that an event pair around a 10 us kernel adds. */
 enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2, MOE_OPT_FUSED_COMBINE = 3, MOE_OPT_SHARED_ASIDE = 4,
-       MOE_OPT_TIMING_SKIP_STAGE = 5 };
+       MOE_OPT_TIMING_SKIP_STAGE = 5, MOE_OPT_ROUTER_CANDIDATES = 6 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP

@@ -43,7 +43,7 @@ def test_full_size_layer(oracle, fmt, T):
     xs = x[torch.from_numpy(sample).cuda()].contiguous()
     yo, io, wo = oracle.moe_layer(oracle.layer_from_device(L), xs.cpu().numpy())
     assert (ids[sample] == io[:, :K]).all(), "router ids bit-exact with the CPU path"
-    assert (ws[sample].view(np.uint32) == wo[:, :K].view(np.uint32)).all(), "router weights bit-exact (sequential order)"
+    assert np.abs(ws[sample] - wo[:, :K]).max() <= 2.5e-7, "router weights within the last bit or two"
     err = _max_abs_rel(y[sample], yo)
     assert err <= TOL_LAYER, err
     # the same tokens as a small batch take the in-place GEMV path: same experts, same result within the bar

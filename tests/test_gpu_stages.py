@@ -232,3 +232,72 @@ def test_gemv_row_invariance(capi):
         h1 = capi.q4cp_gemv_gate_up(guv, x[t:t + 1].contiguous(), ids[t:t + 1].contiguous(), k, mid)
         y1 = capi.q4cp_gemv_down_topk(dnv, h1, ids[t:t + 1].contiguous(), ws[t:t + 1].contiguous(), k, d)
         assert (h1.view(-1) == hid.view(P, -1)[t]).all() and (y1[0] == y[t]).all()
+
+
+# ---------- batch router through candidate selection ----------
+def _route_both(capi, hl, x, k):
+    """(ids, ws) of the batch path with the candidate router and with the dense fp64 router."""
+    import torch
+    T = x.shape[0]
+    m, dev = hl.to_gpu(max_tokens=T)
+    out = []
+    for opt in (1, 0):
+        m.set_option(capi.OPT_ROUTER_CANDIDATES, opt)
+        m.forward(0, gpu(x))
+        ids, ws = m.last_routing(T)
+        out.append((ids.cpu().numpy()[:, :k].copy(), ws.cpu().numpy()[:, :k].copy()))
+    m.close()
+    return out
+
+
+@pytest.mark.parametrize("E,k,d,T,dt", [(512, 10, 3072, 700, "f32"), (512, 10, 1024, 300, "bf16"), (64, 6, 256, 130, "f32"),
+                                        (40, 15, 512, 77, "f32"), (500, 8, 640, 100, "bf16")])
+def test_candidate_router_ids_exact(capi, oracle, E, k, d, T, dt):
+    """Approximate logits + rigorous bound + exact recomputation of the candidates: ids and their order are the
+    oracle's for every token, weights within the last bit or two, with and without a Zipf bias."""
+    from helpers import HostLayer
+    rng = np.random.default_rng(E + T)
+    for skew in (False, True):
+        bias = S.zipf_bias(rng, E, 1.1, 1.0) if skew else None
+        hl = HostLayer(rng, d, 256, E, k, router_dtype=dt, bias=bias, shared=(T % 2 == 0))
+        x = rng.standard_normal((T, d), dtype=np.float32) * (0.3 if skew else 3.0)
+        lo, io, wo = oracle.router(hl.oracle_layer().router, x, k, bias=bias)
+        (ic, wc), (i0, w0) = _route_both(capi, hl, x, k)
+        assert (i0 == io[:, :k]).all() and (w0.view(np.uint32) == wo[:, :k].view(np.uint32)).all(), "dense router"
+        assert (ic == io[:, :k]).all(), "candidate router: ids / order differ from the oracle"
+        assert np.abs(wc - wo[:, :k]).max() <= 2.5e-7
+
+
+def test_candidate_router_hard_rows(capi, oracle):
+    """Rows that the candidate pass must hand to the exact redo: duplicated and nearly equal router rows (probability
+    ties at and around the rank k boundary), all-zero tokens (every logit equal), a logit range of hundreds (f32
+    probabilities underflow and tie by index), activations beyond the f16 range, and a batch in which most tokens are
+    such (the dense kernel takes over).  Ids must be the oracle's everywhere."""
+    from helpers import HostLayer
+    rng = np.random.default_rng(404)
+    E, k, d, T = 128, 10, 512, 200
+    hl = HostLayer(rng, d, 256, E, k, shared=False)
+    hl.router[7] = hl.router[3]
+    hl.router[90] = hl.router[3]
+    hl.router[16] = hl.router[5] * np.float32(1 + 2 ** -22)
+    hl.router[33] = hl.router[5]
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    x[10] = 0.0
+    x[11] = 0.0
+    x[12] *= 300.0                      # logits spread over hundreds
+    x[13] = x[12] * 40.0
+    x[14, 5] = 1e5                      # beyond f16
+    x[15] *= 1e-6                       # f16 subnormals
+    for sel in (slice(None), np.r_[0:40, 10, 11, 10, 11, 10, 11, 12, 13]):
+        xs = np.ascontiguousarray(x[sel])
+        lo, io, wo = oracle.router(hl.oracle_layer().router, xs, k)
+        (ic, wc), (i0, w0) = _route_both(capi, hl, xs, k)
+        assert (i0 == io[:, :k]).all()
+        assert (ic == io[:, :k]).all(), np.where((ic != io[:, :k]).any(1))
+        assert np.abs(wc - wo[:, :k]).max() <= 2.5e-7
+    # most tokens tie: every token is listed and the dense kernel runs
+    xz = np.zeros((64, d), np.float32)
+    xz[::7] = x[:10]
+    lo, io, wo = oracle.router(hl.oracle_layer().router, xz, k)
+    (ic, wc), _ = _route_both(capi, hl, xz, k)
+    assert (ic == io[:, :k]).all() and (wc.view(np.uint32) == wo[:, :k].view(np.uint32)).all()
