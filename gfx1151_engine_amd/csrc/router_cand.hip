@@ -20,9 +20,10 @@
 //      top-k; when more than T/16 tokens are listed the dense fp64 kernel runs for the whole batch instead.
 // Error bound.  a~ = fl32(sum of f16(x_c) * f16(w_c)): |f16(v) - v| <= 2^-11 |v| + 2^-25 (the second term covers
 // f16 subnormals), so sum |x~ w~ - x w| <= 1.001 (2^-10 |x||w| + 2^-25 sqrt(d) (|x| + |w|)) by Cauchy-Schwarz, and
-// the accumulation adds at most d * 2^-22 * 1.001 |x||w| however the matrix pipe orders and rounds its partial sums
-// (twice the IEEE bound per addition, one addition charged per product).  Non-finite approximations (overflow of
-// the f16 conversions) send the token to step 5.
+// the accumulation adds at most (RA_CHUNK * 2^-22 + (d / RA_CHUNK) * 2^-23) * 1.001 |x||w|: inside a chunk of RA_CHUNK
+// columns however the matrix pipe orders and rounds its partial sums (twice the IEEE bound per addition, one addition
+// charged per product), plus one IEEE f32 addition per chunk for the running sum.  Non-finite approximations
+// (overflow of the f16 conversions) send the token to step 5.
 #include "common.h"
 #include "internal.h"
 #include "topk.h"
@@ -34,10 +35,13 @@ typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int RA_BT = 128, RA_BE = 128, RA_K = 32;
-constexpr int RA_PITCH = 80;  // bytes per LDS row: 32 f16 + 16 B of padding (the 16-byte fragment reads of 8 rows then cover all banks)
-constexpr int RC_SLOTS = 32;  // lanes per token in the exact pass: up to 31 candidates + the shared-expert gate row
+constexpr int RA_PITCH = 80;   // bytes per LDS row: 32 f16 + 16 B of padding (the 16-byte fragment reads of 8 rows then cover all banks)
+constexpr int RA_CHUNK = 128;  // columns summed in the matrix pipe's f32 accumulators before they are added to the running sums
+constexpr int RC_SLOTS = 32;   // at most 31 candidates per token (+ the shared-expert gate row) in the exact pass
 
 // ---- 1. approximate logits: block = 128 tokens x 128 experts, 4 waves as 2 x 2, wave = 64 x 64 (2 x 2 MFMA tiles) ----
+// The accumulators of the matrix pipe are flushed into running f32 sums every RA_CHUNK columns, which bounds the
+// rounding of the accumulation by the chunk length instead of d (see the error bound in moe_router_batch_cand).
 template <bool BF16>
 __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict__ W, const float* __restrict__ bias,
                                                          const float* __restrict__ x, int P, int E, int d,
@@ -56,12 +60,14 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
   }
   if (tt >= ntt) return;
   const int e0 = col * RA_BE, t0 = tt * RA_BT;
+  constexpr int NL = RA_BT * RA_K / 4 / 256;  // float4 loads per thread, slab and operand (8)
+  constexpr int TPR = RA_K / 4;               // threads per row (16)
 
-  float4 xr[4], wr[4];
+  float4 xr[NL], wr[NL];
   auto fetch = [&](int c0) {
 #pragma unroll
-    for (int it = 0; it < 4; it++) {
-      const int i = tid + it * 256, r = i >> 3, cc = c0 + (i & 7) * 4;
+    for (int it = 0; it < NL; it++) {
+      const int i = tid + it * 256, r = i / TPR, cc = c0 + (i % TPR) * 4;
       const int t = t0 + r, e = e0 + r;
       xr[it] = t < P ? *(const float4*)(x + (size_t)t * d + cc) : float4{0.f, 0.f, 0.f, 0.f};
       if (e < E) {
@@ -77,11 +83,13 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
       }
     }
   };
-  float xs2[4] = {0.f, 0.f, 0.f, 0.f}, ws2[4] = {0.f, 0.f, 0.f, 0.f};
+  float xs2[NL], ws2[NL];
+#pragma unroll
+  for (int it = 0; it < NL; it++) xs2[it] = ws2[it] = 0.f;
   auto stage = [&]() {
 #pragma unroll
-    for (int it = 0; it < 4; it++) {
-      const int i = tid + it * 256, r = i >> 3, m = i & 7;
+    for (int it = 0; it < NL; it++) {
+      const int i = tid + it * 256, r = i / TPR, m = i % TPR;
       const float4 a = xr[it], w = wr[it];
       xs2[it] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
       ws2[it] += w.x * w.x + w.y * w.y + w.z * w.z + w.w * w.w;
@@ -89,13 +97,13 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
       *(half4v*)(Ws + r * RA_PITCH + m * 8) = half4v{(_Float16)w.x, (_Float16)w.y, (_Float16)w.z, (_Float16)w.w};
     }
   };
-  floatx16 acc[2][2];
+  floatx16 acc[2][2], run[2][2];
 #pragma unroll
   for (int i = 0; i < 2; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 16; r++) acc[i][j][r] = run[i][j][r] = 0.f;
 
   fetch(0);
   for (int c0 = 0; c0 < d; c0 += RA_K) {
@@ -104,7 +112,7 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
     __syncthreads();
     if (c0 + RA_K < d) fetch(c0 + RA_K);
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
+    for (int ks = 0; ks < RA_K / 16; ks++) {
       half8 a[2], bq[2];
 #pragma unroll
       for (int mf = 0; mf < 2; mf++) a[mf] = *(const half8*)(Xs + (wm * 64 + 32 * mf + n) * RA_PITCH + ks * 32 + h * 16);
@@ -115,6 +123,17 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
 #pragma unroll
         for (int nf = 0; nf < 2; nf++)
           acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], bq[nf], acc[mf][nf], 0, 0, 0);
+    }
+    if ((c0 + RA_K) % RA_CHUNK == 0 || c0 + RA_K >= d) {
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            run[i][j][r] += acc[i][j][r];
+            acc[i][j][r] = 0.f;
+          }
     }
   }
   // D[i][j]: j = lane % 32 (expert), i = 8 * (r / 4) + 4 * (lane / 32) + r % 4 (token)
@@ -127,20 +146,20 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
 #pragma unroll
       for (int nf = 0; nf < 2; nf++) {
         const int e = e0 + wn * 64 + 32 * nf + n;
-        if (e < E) alog[(size_t)t * E + e] = acc[mf][nf][r] + (bias ? bias[e] : 0.f);
+        if (e < E) alog[(size_t)t * E + e] = run[mf][nf][r] + (bias ? bias[e] : 0.f);
       }
     }
-  // row norms: the 8 threads that share a row are 8 consecutive lanes
+  // row norms: the TPR threads that share a row are consecutive lanes
 #pragma unroll
-  for (int it = 0; it < 4; it++) {
+  for (int it = 0; it < NL; it++) {
     float sx = xs2[it], sw = ws2[it];
 #pragma unroll
-    for (int o = 1; o < 8; o <<= 1) {
+    for (int o = 1; o < TPR; o <<= 1) {
       sx += __shfl_xor(sx, o, 64);
       sw += __shfl_xor(sw, o, 64);
     }
-    const int r = (tid + it * 256) >> 3;
-    if ((tid & 7) == 0) {
+    const int r = (tid + it * 256) / TPR;
+    if (tid % TPR == 0) {
       if (col == 0 && t0 + r < P) {
         xnorm[t0 + r] = sqrtf(sx);
         if (out_xms) out_xms[t0 + r] = sx / (float)d;
@@ -498,7 +517,7 @@ __global__ void __launch_bounds__(256) k_router_topk_listed(const float* __restr
 
 bool moe_router_cand_supported(const moe_wview* W, const moe_wview* Wx, int P, int k) {
   const int E = (int)W->rows, d = (int)W->cols;
-  if (P < 1 || d % 32 || d < 32 || E > 512 || k + 1 > RC_SLOTS - 1 || k >= E) return false;
+  if (P < 1 || d % RA_K || d < RA_K || E > 512 || k + 1 > RC_SLOTS - 1 || k >= E) return false;
   if (Wx && (Wx->dtype == MOE_DT_BF16) != (W->dtype == MOE_DT_BF16)) return false;
   return moe_aligned(W->data, 16) && (!Wx || moe_aligned(Wx->data, 16));
 }
@@ -525,7 +544,8 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
   const bool bf = W->dtype == MOE_DT_BF16;
   const int ncol = (E + RA_BE - 1) / RA_BE, ntt = (P + RA_BT - 1) / RA_BT;
   const unsigned grid_a = (unsigned)(((ntt + 7) / 8) * 8 * ncol);
-  const float eps = (0x1p-10f + (float)d * 0x1p-22f) * 1.002f * 1.01f;  // 1.01: the f32 norms' own rounding
+  // 1.002: second-order terms; 1.01: the f32 norms' own rounding
+  const float eps = (0x1p-10f + (float)RA_CHUNK * 0x1p-22f + (float)(d / RA_CHUNK + 1) * 0x1p-23f) * 1.002f * 1.01f;
   const float dterm = 0x1p-25f * 1.01f * sqrtf((float)d);
   const int dense_above = P / 16;
   const void* wx = Wx ? Wx->data : nullptr;
