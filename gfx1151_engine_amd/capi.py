@@ -331,6 +331,20 @@ class Moe:
         check(lib().moe_forward(self.h, layer, ptr(x), P, ptr(y), stream()), "moe_forward")
         return y
 
+    def forward_x16(self, layer, x, x16, y=None):
+        """moe_forward_x16: the caller's f16 copy of x (capi.f32_to_f16(x, layout=self.x16_layout(layer)))."""
+        P = x.shape[0]
+        if y is None:
+            y = torch.empty((P, self.cfg.d), dtype=torch.float32, device=x.device)
+        check(lib().moe_forward_x16(self.h, layer, ptr(x), ptr(x16), P, ptr(y), stream()), "moe_forward_x16")
+        return y
+
+    def x16_layout(self, layer):
+        rc = lib().moe_x16_layout(self.h, layer)
+        if rc < 0:
+            check(rc, "moe_x16_layout")
+        return rc
+
     def forward_hc(self, layer, x, w4, R):
         """moe_b(try_hcw): the combine writes into the bf16 HC state R [P][4][d] (int16 tensor of bf16 bits)."""
         check(lib().moe_forward_hc(self.h, layer, ptr(x), x.shape[0], ptr(w4), ptr(R), stream()), "moe_forward_hc")
@@ -412,6 +426,12 @@ class ModelFile:
         cfg = Config()
         check(lib().moe_file_config(self.h, layer, C.byref(cfg)), "moe_file_config")
         return cfg
+
+    def load_mtp_layers(self, moe, mtp_layer0, ctx_layer0, n_layers):
+        w = C.c_void_p()
+        check(lib().moe_load_mtp_layers(moe.h, self.h, mtp_layer0, ctx_layer0, n_layers, C.byref(w), stream()),
+              "moe_load_mtp_layers")
+        return Weights(w)
 
     def load_layers(self, moe, file_layer0, ctx_layer0, n_layers):
         """-> opaque weights handle (keep it alive as long as the context uses the layers)"""

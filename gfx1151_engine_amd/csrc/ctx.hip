@@ -86,6 +86,7 @@ struct moe_ctx {
   moe_tile* tiles_sh = nullptr;
   int* ntiles_sh = nullptr;
   const moe_hc* hc = nullptr;  // set for the duration of moe_forward_hc: the combine writes into the HC state
+  const __half* x16_ext = nullptr;  // set for the duration of moe_forward_x16: the caller's f16 copy of x
   bool shared_aside = true;
   // batch router through candidate selection (exact ids at a fraction of the fp64 work); its scratch
   bool router_cand = true;
@@ -590,6 +591,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   c->ev_n = 0;
   prof_mark(c, 0, st);
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
+  const __half* xh = c->x16_ext ? c->x16_ext : c->x16;  // f16 activations in the GEMM's order
   if (L.has_shared && c->shared_aside && (!c->fused_combine || c->hc)) {
     // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
     // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
@@ -600,12 +602,13 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     const int max_tiles = (P * g.topk + 127) / 128 + g.experts;
     MOE_HIP(hipEventRecord(c->ev_fork, st));
     MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
-    int rs = moe_launch_f16_rows_meansq(x, c->x16, P, g.d, q4k ? 2 : 1, c->xms, c->side);
+    int rs = c->x16_ext ? moe_launch_meansq_f16(xh, P, g.d, c->xms, c->side)
+                        : moe_launch_f16_rows_meansq(x, c->x16, P, g.d, q4k ? 2 : 1, c->xms, c->side);
     hipError_t ee = hipEventRecord(c->ev_x16, c->side);
     if (!rs && ee != hipSuccess) rs = (int)ee;
     if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, 128, P, sh_first, c->tokidx, c->side);
     if (!rs)
-      rs = moe_launch_gemm_q4cp(true, &gu, &sgu, g.experts, c->x16, c->tokidx, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
+      rs = moe_launch_gemm_q4cp(true, &gu, &sgu, g.experts, xh, c->tokidx, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
                                 c->hid16, g.mid, g.d, true, q4k, hs, c->side, nullptr, sh_cb_up);
     if (!rs)
       rs = moe_launch_gemm_q4cp(false, &dn, &sdn, g.experts, c->hid16, nullptr, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
@@ -621,7 +624,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     if (!rc && ee != hipSuccess) rc = (int)ee;
     prof_mark(c, MOE_PROF_ROUTE, st);
     if (!rc && !rs)
-      rc = moe_launch_gemm_q4cp(true, &gu, nullptr, g.experts, c->x16, c->tokidx, c->tiles, c->ntiles, max_tiles,
+      rc = moe_launch_gemm_q4cp(true, &gu, nullptr, g.experts, xh, c->tokidx, c->tiles, c->ntiles, max_tiles,
                                 c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr);
     prof_mark(c, MOE_PROF_UP, st);
     if (!rc && !rs)
@@ -644,7 +647,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   // launches that leave the memory system idle) run on the caller's stream
   MOE_HIP(hipEventRecord(c->ev_fork, st));
   MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
-  int rc16 = moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
+  int rc16 = c->x16_ext ? MOE_OK : moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
   const bool fused = c->fused_combine && !c->hc;  // the HC write-back belongs to the ordered combine
   if (fused && !rc16) rc16 = moe_launch_zero_f32(y, (uint64_t)P * g.d, c->side);  // after the last read of x
   // the side stream is joined on every path out of here (a capture on `st` must not end with it forked)
@@ -665,7 +668,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   if (jrc) return jrc;
   prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
-  if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, c->x16, c->tokidx,
+  if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, xh, c->tokidx,
                                  c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr,
                                  sh_cb_up)))
     return rc;
@@ -722,5 +725,29 @@ MOE_API int moe_forward_hc(moe_ctx* c, int layer, const float* x, int P, const f
   c->hc = &hc;
   const int rc = forward_batch(c, *L, x, P, nullptr, moe_s(st));
   c->hc = nullptr;
+  return rc;
+}
+
+// The layout of the f16 activations the grouped GEMM of a layer reads (moe_f32_to_f16's `layout`): 1 for q4cp
+// experts, 2 for raw GGUF blocks; MOE_E_STATE without expert weights.
+MOE_API int moe_x16_layout(moe_ctx* c, int layer) {
+  MoeLayer* L = layer_of(c, layer);
+  if (!L) return MOE_E_INVALID;
+  if (!(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
+  return L->has_gguf ? 2 : 1;
+}
+
+// moe_forward for a batch whose f16 copy the caller has already made (its HC-read epilogue can write it next to
+// the f32 rows, src/gpu/parts/40_model.inc:2556-2565,4817): the library's own conversion pass is left out.
+MOE_API int moe_forward_x16(moe_ctx* c, int layer, const float* x, const void* x16, int P, float* y, moe_stream_t st) {
+  MoeLayer* L = layer_of(c, layer);
+  if (!L || !x || !x16 || !y || P < 0) return MOE_E_INVALID;
+  if (!L->has_router || !(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
+  if (P > c->cfg.max_tokens) return MOE_E_STATE;
+  if (!moe_aligned(x, 16) || !moe_aligned(y, 16) || !moe_aligned(x16, 16)) return MOE_E_INVALID;
+  if (P <= c->small_max) return MOE_E_UNSUPPORTED;  // small batches never use an f16 copy
+  c->x16_ext = (const __half*)x16;
+  const int rc = forward_batch(c, *L, x, P, y, moe_s(st));
+  c->x16_ext = nullptr;
   return rc;
 }

@@ -52,6 +52,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
 int moe_launch_zero_f32(float* p, uint64_t n, hipStream_t st);
 int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, int P, int sh_first, int* tokidx,
                                  hipStream_t st);
+int moe_launch_meansq_f16(const void* x16, int P, int d, float* xms, hipStream_t st);
 int moe_launch_f16_rows_meansq(const float* x, void* x16, int P, int d, int layout, float* xms, hipStream_t st);
 // permutation (+ tile list with tiles != nullptr) of a batch of at most 32 tokens in one launch
 bool moe_route_small_supported(int P, int k, int experts);

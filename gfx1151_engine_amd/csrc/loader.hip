@@ -453,10 +453,17 @@ int upload_f32_as_bf16(moe_weights* w, const FTensor& t, const uint8_t** dev) {
   return MOE_OK;
 }
 
-int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st) {
-  const FTensor* rt = find(f, "layers.%d.mlp.gate.weight", fl);
-  const FTensor* gu = find(f, "layers.%d.mlp.experts.gate_up_proj.weight", fl);
-  const FTensor* dn = find(f, "layers.%d.mlp.experts.down_proj.weight", fl);
+// mtp: the MTP draft layer's MoE, stored as mtp.layers.<i>.mlp.* (src/gpu/parts/40_model.inc:5546-5548,5893)
+int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st, bool mtp) {
+  auto findp = [&](const char* leaf) -> const FTensor* {
+    char n[160];
+    snprintf(n, sizeof n, "%slayers.%d.mlp.%s", mtp ? "mtp." : "", fl, leaf);
+    auto it = f->idx.find(n);
+    return it == f->idx.end() ? nullptr : &it->second;
+  };
+  const FTensor* rt = findp("gate.weight");
+  const FTensor* gu = findp("experts.gate_up_proj.weight");
+  const FTensor* dn = findp("experts.down_proj.weight");
   if (!rt || !gu || !dn) return MOE_E_STATE;
   if (!hgn_dtype_ok_dense(rt->dtype) || gu->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP) return MOE_E_UNSUPPORTED;
   int rc;
@@ -485,11 +492,11 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
   if ((rc = view(*rt, &vr)) || (rc = view(*gu, &vgu)) || (rc = view(*dn, &vdn))) return rc;
   if ((rc = moe_set_router(ctx, cl, &vr, nullptr))) return rc;
   if ((rc = moe_set_experts_q4cp(ctx, cl, &vgu, &vdn))) return rc;
-  const FTensor* sg = find(f, "layers.%d.mlp.shared_expert.gate_proj.weight", fl);
+  const FTensor* sg = findp("shared_expert.gate_proj.weight");
   if (sg) {
-    const FTensor* su = find(f, "layers.%d.mlp.shared_expert.up_proj.weight", fl);
-    const FTensor* sd = find(f, "layers.%d.mlp.shared_expert.down_proj.weight", fl);
-    const FTensor* sx = find(f, "layers.%d.mlp.shared_expert_gate.weight", fl);
+    const FTensor* su = findp("shared_expert.up_proj.weight");
+    const FTensor* sd = findp("shared_expert.down_proj.weight");
+    const FTensor* sx = findp("shared_expert_gate.weight");
     if (!su || !sd || !sx) return MOE_E_STATE;
     // the shared expert of this path is q4cp; bf16 / q8 shared experts stay with the caller's dense kernels
     if (sg->dtype != MOE_DT_Q4CP || su->dtype != MOE_DT_Q4CP || sd->dtype != MOE_DT_Q4CP || !hgn_dtype_ok_dense(sx->dtype))
@@ -585,13 +592,13 @@ MOE_API int moe_weights_free(moe_weights* w) {
 
 MOE_API uint64_t moe_weights_bytes(const moe_weights* w) { return w ? w->bytes : 0; }
 
-MOE_API int moe_load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, int ctx_layer0, int n_layers,
-                            moe_weights** out, moe_stream_t st) {
+static int load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, int ctx_layer0, int n_layers,
+                       moe_weights** out, moe_stream_t st, bool mtp) {
   if (!ctx || !f || !out || file_layer0 < 0 || ctx_layer0 < 0 || n_layers < 1) return MOE_E_INVALID;
   moe_weights* w = new (std::nothrow) moe_weights();
   if (!w) return MOE_E_STATE;
   for (int i = 0; i < n_layers; i++) {
-    const int rc = f->format == MOE_FILE_HGN ? load_layer_hgn(ctx, f, file_layer0 + i, ctx_layer0 + i, w, moe_s(st))
+    const int rc = f->format == MOE_FILE_HGN ? load_layer_hgn(ctx, f, file_layer0 + i, ctx_layer0 + i, w, moe_s(st), mtp)
                                              : load_layer_gguf(ctx, f, file_layer0 + i, ctx_layer0 + i, w, moe_s(st));
     if (rc != MOE_OK) {
       for (int j = 0; j <= i; j++) (void)moe_clear_layer(ctx, ctx_layer0 + j);  // no layer keeps a freed pointer
@@ -602,4 +609,14 @@ MOE_API int moe_load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, in
   w->stager.reset();  // the staging buffers are not needed once the layers are resident
   *out = w;
   return MOE_OK;
+}
+
+MOE_API int moe_load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, int ctx_layer0, int n_layers,
+                            moe_weights** out, moe_stream_t st) {
+  return load_layers(ctx, f, file_layer0, ctx_layer0, n_layers, out, st, false);
+}
+
+MOE_API int moe_load_mtp_layers(moe_ctx* ctx, const moe_file* f, int mtp_layer0, int ctx_layer0, int n_layers,
+                                moe_weights** out, moe_stream_t st) {
+  return load_layers(ctx, f, mtp_layer0, ctx_layer0, n_layers, out, st, true);
 }

@@ -296,6 +296,35 @@ int moe_launch_f16_rows_meansq(const float* x, void* x16, int P, int d, int layo
   return MOE_OK;
 }
 
+// per-token mean square from an f16 copy of x (any element order): one wave per token
+__global__ void __launch_bounds__(256) k_meansq_f16_rows(const uint4* __restrict__ x16, int P, int d,
+                                                         float* __restrict__ xms) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= P) return;
+  const uint4* xr = x16 + (size_t)t * (d / 8);
+  float acc = 0.f;
+  for (int i = lane; i < d / 8; i += 64) {
+    const uint4 u = xr[i];
+    const __half2* h = (const __half2*)&u;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const float2 f = __half22float2(h[q]);
+      acc += f.x * f.x + f.y * f.y;
+    }
+  }
+#pragma unroll
+  for (int o = 32; o; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if (lane == 0) xms[t] = acc / (float)d;
+}
+
+int moe_launch_meansq_f16(const void* x16, int P, int d, float* xms, hipStream_t st) {
+  if (!x16 || !xms || d % 8 || !moe_aligned(x16, 16)) return MOE_E_INVALID;
+  if (P <= 0) return MOE_OK;
+  k_meansq_f16_rows<<<(P + 3) / 4, 256, 0, st>>>((const uint4*)x16, P, d, xms);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
 int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E, int cap, int P,
                             int sh_first, int* tokidx, hipStream_t st) {
   k_tiles_shared<<<1, 1024, 0, st>>>(eoff, tiles, ntiles, E, cap, P, sh_first, tokidx);

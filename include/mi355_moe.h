@@ -231,6 +231,14 @@ int moe_forward(moe_ctx* ctx, int layer, const float* x, int P, float* y, moe_st
  * enqueued, where the reference's call returns false (P <= 32, formats outside the grouped GEMM): the caller then
  * runs moe_forward and its own write-back. */
 int moe_forward_hc(moe_ctx* ctx, int layer, const float* x, int P, const float* w4, uint16_t* R, moe_stream_t st);
+/* moe_forward for a caller that already holds the batch as f16 in the order the grouped GEMM reads (the reference's
+ * callers write a 16-bit copy of x in the epilogue that produces x, src/gpu/parts/40_model.inc:2556-2565; its
+ * moe_q4w_run / moe_gguf convert once more, :1762, :1703).  x16: f16 [P][d] as moe_f32_to_f16(x, ., layout) makes it,
+ * layout = moe_x16_layout(ctx, layer) (1: q4cp experts, 2: raw GGUF blocks).  x (f32) is still read by the router.
+ * The library's own conversion pass is left out.  P > 32 only (MOE_E_UNSUPPORTED below: the small-batch kernels do
+ * not use an f16 copy; call moe_forward there), and a format outside the grouped GEMM returns MOE_E_UNSUPPORTED. */
+int moe_x16_layout(moe_ctx* ctx, int layer);
+int moe_forward_x16(moe_ctx* ctx, int layer, const float* x, const void* x16, int P, float* y, moe_stream_t st);
 /* Switches in the spirit of the reference's QWENOX_* opt-outs (src/gpu/parts/40_model.inc:1959-1996):
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
  * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as
@@ -319,6 +327,13 @@ int moe_file_config(const moe_file* f, int layer, moe_config* cfg);
 typedef struct moe_weights moe_weights;
 int moe_load_layers(moe_ctx* ctx, const moe_file* f, int file_layer0, int ctx_layer0, int n_layers,
                     moe_weights** out, moe_stream_t st);
+/* The MoE of the MTP draft layer(s) (GpuModel::mtp_moe / mtp_moe_b, src/gpu/parts/40_model.inc:5546,5892): the same
+ * computation on the tensors mtp.layers.<i>.mlp.* of a .hgn file, registered as context layer ctx_layer0 + i (create
+ * the context with one layer slot more per MTP layer and call moe_forward on that slot).  In a GGUF file the MTP
+ * layer is an ordinary block (blk.<n_layers>.*, the sidecar of src/gguf_map.h:3): use moe_load_layers for it; this
+ * call does the same there. */
+int moe_load_mtp_layers(moe_ctx* ctx, const moe_file* f, int mtp_layer0, int ctx_layer0, int n_layers,
+                        moe_weights** out, moe_stream_t st);
 uint64_t moe_weights_bytes(const moe_weights* w);
 int moe_weights_free(moe_weights* w);
 /* Forget the weights registered for a layer (moe_forward on it returns MOE_E_STATE until it is set again). */

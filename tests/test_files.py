@@ -272,6 +272,46 @@ def test_gguf_router_tensors_are_rounded_to_bf16_like_the_reference(tmp_path):
 
 
 @pytest.mark.gpu
+def test_mtp_layer_from_a_file(tmp_path):
+    """The MTP draft layer's MoE (mtp_moe / mtp_moe_b in the reference): the tensors mtp.layers.0.mlp.* of a .hgn file
+    go into one more layer slot behind the trunk's layers; one token, a verify-size batch and a prefill-size batch
+    through that slot against the oracle, and the trunk layer next to it is untouched."""
+    import torch
+    rng = np.random.default_rng(58)
+    trunk = HostLayer(rng, D, MID, E, K)
+    mtp = HostLayer(rng, D, MID, E, K, router_dtype="bf16")
+    ts = files.hgn_layer_tensors(0, trunk)
+    ts += [("mtp." + n, dt, dims, a) for n, dt, dims, a in files.hgn_layer_tensors(0, mtp)]
+    p = tmp_path / "with_mtp.hgn"
+    files.write_hgn(p, ts)
+    f = capi.ModelFile(p)
+    cfg = f.config(0)
+    assert cfg.layers == 1
+    m = capi.Moe(cfg.d, cfg.mid, cfg.experts, K, layers=2, max_tokens=70)
+    w0 = f.load_layers(m, 0, 0, 1)
+    w1 = f.load_mtp_layers(m, 0, 1, 1)
+    f.close()
+    for T in (1, 5, 70):
+        x = _x(T, seed=40 + T)
+        xt = torch.from_numpy(x).cuda()
+        for slot, hl in ((1, mtp), (0, trunk)):
+            want, io, _ = O.moe_layer(hl.oracle_layer(), x)
+            y = m.forward(slot, xt).cpu().numpy()
+            ids, _ = m.last_routing(T)
+            assert (ids.cpu().numpy()[:, :K] == io[:, :K]).all(), (T, slot)
+            assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max(), (T, slot)
+    # a file without MTP tensors: nothing to load
+    p2, _ = _hgn(tmp_path, [trunk], first=0)
+    f2 = capi.ModelFile(p2)
+    wv = C.c_void_p()
+    assert capi.lib().moe_load_mtp_layers(m.h, f2.h, 0, 1, 1, C.byref(wv), capi.stream()) == -3
+    f2.close()
+    del m
+    w0.free()
+    w1.free()
+
+
+@pytest.mark.gpu
 def test_load_rejects_types_outside_the_path(tmp_path):
     # a GGUF whose experts are Q6_K: moe_load_layers reports unsupported and leaves no layer registered
     import torch

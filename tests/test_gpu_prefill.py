@@ -264,3 +264,29 @@ def test_forward_hc_writeback(oracle, fmt):
     capi.reduce_pw_sg_hc(gpu(pairs), gpu(pairids), gpu(pw), P2, K2, gpu(z4), R2)
     assert (R2.cpu().numpy().view(np.uint16) == oracle.hc_writeback(y2, z4, R0[:P2])).all()
     m.close()
+
+
+@pytest.mark.parametrize("fmt", ["q4cp", "q4k"])
+def test_forward_with_the_callers_f16_copy(oracle, fmt):
+    """moe_forward_x16: the caller hands over the f16 copy of the batch in the grouped GEMM's order (its own epilogue
+    wrote it), the library skips its conversion pass.  Same bits as moe_forward; small batches are refused."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(61)
+    d, mid, E, k, T = 512, 256, 12, 4, 130
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    m, dev = hl.to_gpu(max_tokens=T)
+    xg = gpu(x)
+    layout = m.x16_layout(0)
+    assert layout == (1 if fmt == "q4cp" else 2)
+    y0 = m.forward(0, xg).cpu().numpy()
+    x16 = capi.f32_to_f16(xg, layout=layout)
+    for aside in (1, 0):
+        m.set_option(capi.OPT_SHARED_ASIDE, aside)
+        y1 = m.forward_x16(0, xg, x16).cpu().numpy()
+        assert (y1 == y0).all(), aside
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    assert max_abs_rel(y0, yo) <= TOL_LAYER
+    with pytest.raises(capi.MoeError):
+        m.forward_x16(0, xg[:8].contiguous(), x16[:8].contiguous())
+    m.close()
