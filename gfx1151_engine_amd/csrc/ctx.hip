@@ -35,7 +35,7 @@ static int codebook_affine(const moe_wview* w, bool* out) {
 }
 
 struct moe_ctx;
-static int magnitude_constant(moe_ctx* c, bool q4k, const moe_wview* gate, uint64_t gate_stride,
+static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gate, uint64_t gate_stride,
                               const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
                               float* out);
 
@@ -237,7 +237,7 @@ MOE_API int moe_set_experts_q4cp(moe_ctx* c, int layer, const moe_wview* gu, con
   int rc;
   if ((rc = codebook_affine(gu, &a1)) || (rc = codebook_affine(dn, &a2))) return rc;
   L->experts_affine = a1 && a2;
-  if ((rc = magnitude_constant(c, false, gu, (uint64_t)2 * g.mid, gu, (uint64_t)g.mid, dn, g.experts, &L->c_routed)))
+  if ((rc = magnitude_constant(c, 0, 0, gu, (uint64_t)2 * g.mid, gu, (uint64_t)g.mid, dn, g.experts, &L->c_routed)))
     return rc;
   L->gate_up = *gu;
   L->down = *dn;
@@ -256,13 +256,13 @@ MOE_API int moe_set_experts_gguf(moe_ctx* c, int layer, const moe_gg_experts* gg
   MoeLayer* L = layer_of(c, layer);
   if (!L || !gg || !gg->gate || !gg->up || !gg->down) return MOE_E_INVALID;
   if (!moe_gg_types_supported(gg->tgu, gg->tdn, c->cfg.d, c->cfg.mid)) return MOE_E_UNSUPPORTED;
-  L->c_routed = 0.f;  // the f16 range guard belongs to the grouped GEMM, which reads Q4_K only
-  if (gg->tgu == MOE_GGML_Q4_K && gg->tdn == MOE_GGML_Q4_K) {
+  L->c_routed = 0.f;
+  {  // constant of the f16 range guard of the grouped GEMMs
     const moe_config& g = c->cfg;
     moe_wview gv{0, gg->gate, (uint64_t)g.experts * g.mid, (uint64_t)g.d, 0};
     moe_wview uv{0, gg->up, (uint64_t)g.experts * g.mid, (uint64_t)g.d, 0};
     moe_wview dv{0, gg->down, (uint64_t)g.experts * g.d, (uint64_t)g.mid, 0};
-    int rc = magnitude_constant(c, true, &gv, (uint64_t)g.mid, &uv, 0, &dv, g.experts, &L->c_routed);
+    int rc = magnitude_constant(c, gg->tgu, gg->tdn, &gv, (uint64_t)g.mid, &uv, 0, &dv, g.experts, &L->c_routed);
     if (rc) return rc;
   }
   L->gg = *gg;
@@ -293,8 +293,8 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
     L->shared_affine = a1 && a2 && a3;
   }
   L->c_shared = 0.f;
-  if (sh_gguf_type == 0 || sh_gguf_type == MOE_GGML_Q4_K) {
-    int rc = magnitude_constant(c, sh_gguf_type != 0, g, (uint64_t)cf.mid, u, 0, dn, 1, &L->c_shared);
+  {
+    int rc = magnitude_constant(c, sh_gguf_type, sh_gguf_type, g, (uint64_t)cf.mid, u, 0, dn, 1, &L->c_shared);
     if (rc) return rc;
   }
   L->sh_gate = *g;
@@ -312,14 +312,16 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
 // gate rows start at row e*gate_stride of `gate`, its up rows at e*gate_stride + up_first of `up`
 // (the same fused tensor for hgn, a tensor of its own for GGUF), its down rows at e*down->rows/n.
 // Set-up work: dequantises 6 rows per sampled expert on the device and reads them back.
-static int magnitude_constant(moe_ctx* c, bool q4k, const moe_wview* gate, uint64_t gate_stride,
+// tgu / tdn: ggml block types of raw GGUF rows (gate and up; down), 0 = q4cp views.
+static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gate, uint64_t gate_stride,
                               const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
                               float* out) {
   const int ns = n_experts < 16 ? n_experts : 16;
   const uint64_t d = gate->cols, mid = down->cols, drows = down->rows / (uint64_t)n_experts;
   const uint64_t pitch = d > mid ? d : mid;
   auto deq = [&](const moe_wview* w, uint64_t row, float* dst) -> int {
-    if (q4k) return moe_q4k_dequant_rows(w->data + row * (w->cols / 256 * 144), 1, w->cols, dst, nullptr);
+    const int t = w == down ? tdn : tgu;
+    if (t) return moe_gg_dequant_rows(t, w->data + row * moe_gg_row_bytes(t, w->cols), 1, w->cols, dst, nullptr);
     return moe_q4cp_dequant_rows(w->data, w->rows, w->cols, row, 1, dst, nullptr);
   };
   int rc;
@@ -540,6 +542,15 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   return MOE_OK;
 }
 
+// Which grouped GEMM a layer's batches take: 0 = q4cp (tuned), 1 = raw GGUF Q4_K throughout (tuned), 2 = raw GGUF
+// blocks of any supported type (general kernel, f16 operands in natural order).
+static int batch_gemm_kind(const MoeLayer& L) {
+  if (!L.has_gguf) return 0;
+  const bool all4k = L.gg.tgu == MOE_GGML_Q4_K && L.gg.tdn == MOE_GGML_Q4_K &&
+                     (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K);
+  return all4k ? 1 : 2;
+}
+
 // Router of a batch: ids / ws, the shared-expert gate logit and (if asked) the per-token mean square of x.
 // By default through candidate selection (router_cand.hip); MOE_OPT_ROUTER_CANDIDATES = 0, or a shape it does not
 // take, runs the dense fp64 launch and the exact softmax / top-k over all experts.
@@ -559,12 +570,13 @@ static int router_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* o
 // Returns MOE_E_UNSUPPORTED (before enqueuing anything) for shapes / formats the GEMM does not cover.
 static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
   const moe_config& g = c->cfg;
-  const bool q4k = L.has_gguf;  // raw GGUF blocks: the grouped GEMM reads Q4_K only
-  if (q4k && (L.gg.tgu != MOE_GGML_Q4_K || L.gg.tdn != MOE_GGML_Q4_K ||
-              (L.has_shared && L.sh_gguf_type != MOE_GGML_Q4_K)))
+  const bool q4k = L.has_gguf;  // raw GGUF blocks
+  // gen: a GGUF layer that is not Q4_K throughout takes the general grouped GEMM (any supported block type,
+  // dequantised into f16 tiles in LDS); Q4_K-only and q4cp layers take the tuned kernel
+  const bool gen = batch_gemm_kind(L) == 2;
+  if (L.has_shared && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format family per layer
+  if (gen ? (g.d % 64 || g.mid % 64) : q4k ? (g.d % 256 || g.mid % 256) : (g.d % 128 || g.mid % 128 || g.mid < 256 || g.d < 256))
     return MOE_E_UNSUPPORTED;  // the caller walks the batch through the small path
-  if (L.has_shared && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format per launch
-  if (q4k ? (g.d % 256 || g.mid % 256) : (g.d % 128 || g.mid % 128)) return MOE_E_UNSUPPORTED;
   moe_lutw gu{}, dn{}, sgu{}, sdn{};
   const float* sh_cb_up = nullptr;
   if (q4k) {
@@ -592,7 +604,26 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   prof_mark(c, 0, st);
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
   const __half* xh = c->x16_ext ? c->x16_ext : c->x16;  // f16 activations in the GEMM's order
-  if (L.has_shared && c->shared_aside && (!c->fused_combine || c->hc)) {
+  const int xl = gen ? 0 : q4k ? 2 : 1;                 // that order (moe_f32_to_f16's layout)
+  // gate/up (+ SwiGLU) and down launches over a tile list: routed experts, with_sh: the shared expert as well
+  // (tiles whose expert index is >= n_experts)
+  auto gemm_up = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2) -> int {
+    if (gen)
+      return moe_launch_gemm_gg(true, L.gg.tgu, L.gg.gate, L.gg.up, L.sh_gguf_type, with_sh ? L.sh_gate.data : nullptr,
+                                with_sh ? L.sh_up.data : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid,
+                                g.d, hs, s2);
+    return moe_launch_gemm_q4cp(true, &gu, with_sh ? &sgu : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16,
+                                g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up);
+  };
+  auto gemm_dn = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2, const moe_comb* cmb) -> int {
+    if (gen)
+      return moe_launch_gemm_gg(false, L.gg.tdn, L.gg.down, nullptr, L.sh_gguf_type, with_sh ? L.sh_down.data : nullptr,
+                                nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2);
+    return moe_launch_gemm_q4cp(false, &dn, with_sh ? &sdn : nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt,
+                                cmb ? (void*)cmb->y : (void*)c->pairs16, g.d, g.mid, cmb == nullptr, q4k, hs, s2, cmb);
+  };
+  const bool fused = c->fused_combine && !c->hc && !gen;  // the HC write-back belongs to the ordered combine
+  if (L.has_shared && c->shared_aside && !fused) {
     // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
     // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
     // side stream also makes what both streams need first: the per-token mean square of x (range guard) and
@@ -603,33 +634,25 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     MOE_HIP(hipEventRecord(c->ev_fork, st));
     MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
     int rs = c->x16_ext ? moe_launch_meansq_f16(xh, P, g.d, c->xms, c->side)
-                        : moe_launch_f16_rows_meansq(x, c->x16, P, g.d, q4k ? 2 : 1, c->xms, c->side);
+                        : moe_launch_f16_rows_meansq(x, c->x16, P, g.d, xl, c->xms, c->side);
     hipError_t ee = hipEventRecord(c->ev_x16, c->side);
     if (!rs && ee != hipSuccess) rs = (int)ee;
-    if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, 128, P, sh_first, c->tokidx, c->side);
-    if (!rs)
-      rs = moe_launch_gemm_q4cp(true, &gu, &sgu, g.experts, xh, c->tokidx, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
-                                c->hid16, g.mid, g.d, true, q4k, hs, c->side, nullptr, sh_cb_up);
-    if (!rs)
-      rs = moe_launch_gemm_q4cp(false, &dn, &sdn, g.experts, c->hid16, nullptr, c->tiles_sh, c->ntiles_sh, max_tiles_sh,
-                                c->pairs16, g.d, g.mid, true, q4k, hs, c->side, nullptr);
+    if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, moe_gemm_tile_cap(), P, sh_first, c->tokidx, c->side);
+    if (!rs) rs = gemm_up(true, c->tiles_sh, c->ntiles_sh, max_tiles_sh, c->side);
+    if (!rs) rs = gemm_dn(true, c->tiles_sh, c->ntiles_sh, max_tiles_sh, c->side, nullptr);
     // caller's stream: router, top-k, permutation, the routed experts' GEMMs
     rc = router_batch(c, L, x, P, nullptr, st);
     prof_mark(c, MOE_PROF_ROUTER, st);
     if (!rc)
       rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
                            g.id_stride, st);
-    if (!rc) rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, -1, c->tokidx, st);
+    if (!rc) rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, moe_gemm_tile_cap(), P, -1, c->tokidx, st);
     ee = hipStreamWaitEvent(st, c->ev_x16, 0);
     if (!rc && ee != hipSuccess) rc = (int)ee;
     prof_mark(c, MOE_PROF_ROUTE, st);
-    if (!rc && !rs)
-      rc = moe_launch_gemm_q4cp(true, &gu, nullptr, g.experts, xh, c->tokidx, c->tiles, c->ntiles, max_tiles,
-                                c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr);
+    if (!rc && !rs) rc = gemm_up(false, c->tiles, c->ntiles, max_tiles, st);
     prof_mark(c, MOE_PROF_UP, st);
-    if (!rc && !rs)
-      rc = moe_launch_gemm_q4cp(false, &dn, nullptr, g.experts, c->hid16, nullptr, c->tiles, c->ntiles, max_tiles,
-                                c->pairs16, g.d, g.mid, true, q4k, hs, st, nullptr);
+    if (!rc && !rs) rc = gemm_dn(false, c->tiles, c->ntiles, max_tiles, st, nullptr);
     // the side stream is joined on every path out of here (a capture on `st` must not end with it forked)
     ee = hipEventRecord(c->ev_join, c->side);
     if (ee == hipSuccess) ee = hipStreamWaitEvent(st, c->ev_join, 0);
@@ -647,8 +670,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   // launches that leave the memory system idle) run on the caller's stream
   MOE_HIP(hipEventRecord(c->ev_fork, st));
   MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
-  int rc16 = c->x16_ext ? MOE_OK : moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, q4k ? 2 : 1, c->side);
-  const bool fused = c->fused_combine && !c->hc;  // the HC write-back belongs to the ordered combine
+  int rc16 = c->x16_ext ? MOE_OK : moe_f32_to_f16(x, c->x16, (uint64_t)P * g.d, xl, c->side);
   if (fused && !rc16) rc16 = moe_launch_zero_f32(y, (uint64_t)P * g.d, c->side);  // after the last read of x
   // the side stream is joined on every path out of here (a capture on `st` must not end with it forked)
   auto join = [&]() -> int {
@@ -662,27 +684,21 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   if (!rc)
     rc = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
                          g.id_stride, st);
-  if (!rc) rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, 128, P, sh_first, c->tokidx, st);
+  if (!rc) rc = moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, moe_gemm_tile_cap(), P, sh_first, c->tokidx, st);
   const int jrc = join();
   if (rc) return rc;
   if (jrc) return jrc;
   prof_mark(c, MOE_PROF_ROUTE, st);
   const int max_tiles = (P * g.topk + 127) / 128 + g.experts + (L.has_shared ? (P + 127) / 128 : 0);
-  if ((rc = moe_launch_gemm_q4cp(true, &gu, L.has_shared ? &sgu : nullptr, g.experts, xh, c->tokidx,
-                                 c->tiles, c->ntiles, max_tiles, c->hid16, g.mid, g.d, true, q4k, hs, st, nullptr,
-                                 sh_cb_up)))
-    return rc;
+  if ((rc = gemm_up(L.has_shared, c->tiles, c->ntiles, max_tiles, st))) return rc;
   prof_mark(c, MOE_PROF_UP, st);
   if (fused) {
     const moe_comb cmb{y, c->tokidx, c->pw, L.has_shared ? c->sh_logit : nullptr};
-    rc = moe_launch_gemm_q4cp(false, &dn, L.has_shared ? &sdn : nullptr, g.experts, c->hid16, nullptr, c->tiles,
-                              c->ntiles, max_tiles, y, g.d, g.mid, false, q4k, hs, st, &cmb);
+    rc = gemm_dn(L.has_shared, c->tiles, c->ntiles, max_tiles, st, &cmb);
     prof_mark(c, MOE_PROF_DOWN, st);
     return rc;
   }
-  if ((rc = moe_launch_gemm_q4cp(false, &dn, L.has_shared ? &sdn : nullptr, g.experts, c->hid16, nullptr,
-                                 c->tiles, c->ntiles, max_tiles, c->pairs16, g.d, g.mid, true, q4k, hs, st, nullptr)))
-    return rc;
+  if ((rc = gemm_dn(L.has_shared, c->tiles, c->ntiles, max_tiles, st, nullptr))) return rc;
   prof_mark(c, MOE_PROF_DOWN, st);
   rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
                          sh_first, y, P, g.d, g.topk, hs, st, c->hc);
@@ -729,12 +745,14 @@ MOE_API int moe_forward_hc(moe_ctx* c, int layer, const float* x, int P, const f
 }
 
 // The layout of the f16 activations the grouped GEMM of a layer reads (moe_f32_to_f16's `layout`): 1 for q4cp
-// experts, 2 for raw GGUF blocks; MOE_E_STATE without expert weights.
+// experts, 2 for raw GGUF Q4_K blocks, 0 (natural order) for GGUF layers with other block types; MOE_E_STATE
+// without expert weights.
 MOE_API int moe_x16_layout(moe_ctx* c, int layer) {
   MoeLayer* L = layer_of(c, layer);
   if (!L) return MOE_E_INVALID;
   if (!(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
-  return L->has_gguf ? 2 : 1;
+  const int kind = batch_gemm_kind(*L);
+  return kind == 0 ? 1 : kind == 1 ? 2 : 0;
 }
 
 // moe_forward for a batch whose f16 copy the caller has already made (its HC-read epilogue can write it next to

@@ -43,8 +43,11 @@ constexpr int WROWS = MOE_GEMM_WROWS;    // weight rows per block (up: WROWS/2 g
 constexpr int HALF = WROWS / 2;
 constexpr int NW = WROWS / 32 / NF;       // waves per block
 constexpr int NT = 64 * NW;               // each wave: 128 pairs x 32*NF weight rows
-constexpr int WPE = NT * (WROWS == 512 ? 1 : 2) / 256;  // waves per SIMD: 256-row blocks run two to a CU
-constexpr int BM = 128;        // pairs per tile (4 MFMA row fragments)
+#ifndef MOE_GEMM_BM
+#define MOE_GEMM_BM 128
+#endif
+constexpr int BM = MOE_GEMM_BM;  // pairs per tile (32-row MFMA fragments: 4, or 8 with one block per CU and accumulators in AGPRs)
+constexpr int WPE = BM > 128 ? 1 : NT * (WROWS == 512 ? 1 : 2) / 256;  // waves per SIMD: 256-row blocks of 128 pairs run two to a CU
 constexpr int BK = 64;         // K per stage
 constexpr int A_BYTES = BM * BK * 2;      // 16 KB  [row][8 chunks of 16 B], chunk c of row m at slot c ^ ((m >> 1) & 7): conflict-free for the 128-bit fragment reads
 constexpr int W_BYTES = WROWS * 32;       // [row][32 B]
@@ -664,7 +667,11 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
   else if (mfn == 3) GEMM_GO(3);
-  else GEMM_GO(4);
+  else if (BM <= 128 || mfn == 4) GEMM_GO(4);
+  else if constexpr (BM > 128) {
+    if (mfn <= 6) GEMM_GO(6);
+    else GEMM_GO(8);
+  }
 #undef GEMM_GO
 }
 
@@ -795,3 +802,6 @@ MOE_API int moe_gg_down(int type, const uint8_t* down, const void* hid16, const 
   return moe_launch_gemm_q4cp(false, &p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
                               max_tiles, pairs, m, k, f16 != 0, true, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr);
 }
+
+// pairs per tile of the grouped GEMM launches (the cap of the tile lists that moe_forward builds)
+int moe_gemm_tile_cap() { return BM; }

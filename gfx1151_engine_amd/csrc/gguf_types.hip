@@ -332,6 +332,143 @@ __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restri
   }
 }
 
+
+// ---- grouped GEMM on MFMA for any of these block types (batches; src/gpu/parts/26_kernels_moe_gguf.inc:81-386) ----
+// The general form of the batch path: a block = one tile of up to 128 (token, expert) pairs x 128 weight rows
+// (gate/up: 64 gate rows and the matching 64 up rows, SwiGLU on the accumulators).  Per 64-wide K stage every
+// thread dequantises one 32-element block of one weight row (gg_block: the ggml formula in f32, rounded to f16)
+// into an f16 tile in LDS and copies four 16-byte pieces of the activation tile; the four waves (2 x 2, each
+// 64 pairs x 64 rows = 2 x 2 tiles of v_mfma_f32_32x32x16_f16) read both operands from LDS.  Two stage buffers;
+// the next stage is dequantised behind the current stage's MFMAs.  Activations and hid are f16 in natural element
+// order.  The Q4_K-only layers keep the tuned kernel (gemm_q4cp.hip), which dequantises in registers.
+typedef _Float16 gg_half8 __attribute__((ext_vector_type(8)));
+typedef float gg_floatx16 __attribute__((ext_vector_type(16)));
+constexpr int GG_BM = 128, GG_BN = 128, GG_BK = 64, GG_PITCH = 144;  // bytes per LDS row: 64 f16 + 16 (bank spread)
+constexpr int GG_TILE_BYTES = GG_BM * GG_PITCH;                       // 18 KB per operand and stage
+constexpr int GG_SMEM = 4 * GG_TILE_BYTES + GG_BM * 8;                // A, B x 2 stages + row indices + row scales
+
+struct GgGemmW {
+  const uint8_t *w, *w_up;  // expert tensors [E][M rows][row bytes] (gate / down, and up for the gate/up launch)
+  int type;
+};
+
+template <bool UP>
+__global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, int n_experts,
+                                                       const __half* __restrict__ x16, const int* __restrict__ tokidx,
+                                                       const moe_tile* __restrict__ tiles,
+                                                       const int* __restrict__ ntiles, __half* __restrict__ out, int M,
+                                                       int K, moe_hscale hs) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t gsm[];
+  uint8_t* const As = gsm;
+  uint8_t* const Bs = gsm + 2 * GG_TILE_BYTES;
+  int* rowidx = (int*)(gsm + 4 * GG_TILE_BYTES);
+  float* rowscale = (float*)(rowidx + GG_BM);
+  const int ti = blockIdx.y;
+  if (ti >= ntiles[0]) return;
+  const moe_tile tile = tiles[ti];
+  const bool shared = tile.expert >= n_experts;
+  const GgGemmW& G = shared ? Sh : R;
+  const int e = shared ? 0 : tile.expert, nb = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int n = lane & 31, h = lane >> 5, wm = wv >> 1, wn = wv & 1;
+  if (tid < GG_BM) {
+    const int m = tid < tile.count ? tid : 0;  // rows past the tile repeat row 0, never stored
+    const int ri = tokidx ? tokidx[tile.first + m] : tile.first + m;
+    rowidx[tid] = ri;
+    rowscale[tid] = (UP && hs.xms) ? moe_hid_scale(shared ? hs.c_shared : hs.c_routed, hs.xms[ri]) : 1.f;
+  }
+  // this thread's weight row (half of each 64-wide stage of it)
+  const int brow = tid >> 1, half = tid & 1;
+  const uint64_t rb = gg_row_bytes(G.type, (uint64_t)K);
+  int wr;
+  const uint8_t* wbase;
+  if (UP) {
+    wr = nb * 64 + (brow & 63);
+    wbase = brow < 64 ? G.w : G.w_up;
+  } else {
+    wr = nb * GG_BN + brow;
+    wbase = G.w;
+  }
+  wr = wr < M ? wr : M - 1;  // clamped rows are computed and never stored
+  const uint8_t* wrow = wbase + ((uint64_t)e * M + wr) * rb;
+  __syncthreads();
+  const __half* arow[4];
+#pragma unroll
+  for (int it = 0; it < 4; it++) arow[it] = x16 + (size_t)rowidx[(tid + 256 * it) >> 3] * K + ((tid + 256 * it) & 7) * 8;
+
+  auto fill = [&](int s, int buf) {
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+      const int i = tid + 256 * it;
+      *(uint4*)(As + buf * GG_TILE_BYTES + (i >> 3) * GG_PITCH + (i & 7) * 16) = *(const uint4*)(arow[it] + (size_t)s * GG_BK);
+    }
+    int q[32];
+    float a, c;
+    gg_block(G.type, wrow, 2 * s + half, q, a, c);
+    uint8_t* dst = Bs + buf * GG_TILE_BYTES + brow * GG_PITCH + half * 64;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      gg_half8 v;
+#pragma unroll
+      for (int l = 0; l < 8; l++) v[l] = (_Float16)fmaf(a, (float)q[8 * j + l], c);
+      *(gg_half8*)(dst + 16 * j) = v;
+    }
+  };
+  gg_floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  const int nstage = K / GG_BK;
+  fill(0, 0);
+  __syncthreads();
+  for (int s = 0; s < nstage; s++) {
+    const int buf = s & 1;
+    const uint8_t* Ab = As + buf * GG_TILE_BYTES;
+    const uint8_t* Bb = Bs + buf * GG_TILE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      gg_half8 a[2], b[2];
+#pragma unroll
+      for (int mf = 0; mf < 2; mf++) a[mf] = *(const gg_half8*)(Ab + (wm * 64 + 32 * mf + n) * GG_PITCH + ks * 32 + h * 16);
+#pragma unroll
+      for (int nf = 0; nf < 2; nf++) {
+        const int br = UP ? 64 * nf + 32 * wn + n : 64 * wn + 32 * nf + n;
+        b[nf] = *(const gg_half8*)(Bb + br * GG_PITCH + ks * 32 + h * 16);
+      }
+#pragma unroll
+      for (int mf = 0; mf < 2; mf++)
+#pragma unroll
+        for (int nf = 0; nf < 2; nf++)
+          acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+    }
+    if (s + 1 < nstage) fill(s + 1, buf ^ 1);  // behind the MFMAs just issued; the other buffer was read a stage ago
+    __syncthreads();
+  }
+  // D[i][j]: j = lane % 32 (weight row), i = 8 * (r / 4) + 4 * (lane / 32) + r % 4 (pair)
+#pragma unroll
+  for (int mf = 0; mf < 2; mf++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int m = wm * 64 + 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (m >= tile.count) continue;
+      __half* orow = out + (size_t)(tile.first + m) * M;
+      if (UP) {
+        const int col = nb * 64 + 32 * wn + n;
+        const float g = acc[mf][0][r], u = acc[mf][1][r];
+        if (col < M) orow[col] = __float2half(g / (1.f + __expf(-g)) * u * rowscale[m]);
+      } else {
+#pragma unroll
+        for (int nf = 0; nf < 2; nf++) {
+          const int col = nb * GG_BN + 64 * wn + 32 * nf + n;
+          if (col < M) orow[col] = __float2half(acc[mf][nf][r]);
+        }
+      }
+    }
+}
+
 }  // namespace
 
 bool moe_gg_types_supported(int tgu, int tdn, int d, int mid) { return gg_type_ok(tgu, d) && gg_type_ok(tdn, mid); }
@@ -387,5 +524,32 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
     k_ggx_dn<<<grid, 256, (size_t)nslots * mid / 32 * 34 * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
     MOE_LAUNCH_CHECK();
   }
+  return MOE_OK;
+}
+
+// Internal: grouped GEMM over tiles of <= 128 pairs for raw GGUF expert tensors of any supported block type
+// (routed experts of type `type`, optional shared expert of type `tsh`; tile.expert >= n_experts selects it).
+// up: gate/up + SwiGLU -> hid f16 [pairs][m]; else down -> pairs f16 [pairs][m].  x / hid: f16, natural order.
+int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up, int tsh, const uint8_t* sh_w,
+                       const uint8_t* sh_w_up, int n_experts, const __half* x16, const int* tokidx,
+                       const moe_tile* tiles, const int* ntiles, int max_tiles, __half* out, int m, int k,
+                       moe_hscale hs, hipStream_t st) {
+  if (!w || (up && !w_up) || !x16 || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
+  if (!gg_type_ok(type, k) || (sh_w && !gg_type_ok(tsh, k)) || k % GG_BK || m < 1) return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(w, gg_align(type)) || (up && !moe_aligned(w_up, gg_align(type))) || !moe_aligned(x16, 16) ||
+      (sh_w && (!moe_aligned(sh_w, gg_align(tsh)) || (up && (!sh_w_up || !moe_aligned(sh_w_up, gg_align(tsh)))))))
+    return MOE_E_INVALID;
+  if (max_tiles == 0) return MOE_OK;
+  GgGemmW R{w, w_up, type}, S{sh_w ? sh_w : w, sh_w ? sh_w_up : w_up, sh_w ? tsh : type};
+  const dim3 grid((unsigned)(up ? (m + 63) / 64 : (m + GG_BN - 1) / GG_BN), (unsigned)max_tiles);
+  static bool attr_done = false;
+  if (!attr_done) {
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    attr_done = true;
+  }
+  if (up) k_moe_gemm_gg<true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs);
+  else k_moe_gemm_gg<false><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs);
+  MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -49,6 +49,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
                          hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr);
+int moe_gemm_tile_cap();
 int moe_launch_zero_f32(float* p, uint64_t n, hipStream_t st);
 int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, int P, int sh_first, int* tokidx,
                                  hipStream_t st);
@@ -117,6 +118,10 @@ int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float
                       int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
                       hipStream_t st);
 // general GEMV kernels for any supported mix of ggml block types (gguf_types.hip)
+int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up, int tsh, const uint8_t* sh_w,
+                       const uint8_t* sh_w_up, int n_experts, const __half* x16, const int* tokidx,
+                       const moe_tile* tiles, const int* ntiles, int max_tiles, __half* out, int m, int k,
+                       moe_hscale hs, hipStream_t st);
 bool moe_gg_types_supported(int tgu, int tdn, int d, int mid);
 uint64_t moe_gg_row_bytes(int type, uint64_t k);
 int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gate, const uint8_t* up,

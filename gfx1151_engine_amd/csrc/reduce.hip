@@ -66,6 +66,11 @@ __global__ void __launch_bounds__(256) k_f32_to_f16_rows(const float* __restrict
       v = xr[blk * 16 + 8 + w];
       a = __floats2half2_rn(u.x, u.z); b = __floats2half2_rn(v.x, v.z);
       c = __floats2half2_rn(u.y, u.w); e = __floats2half2_rn(v.y, v.w);
+    } else if (LAYOUT == 0) {
+      u = xr[2 * i];
+      v = xr[2 * i + 1];
+      a = __floats2half2_rn(u.x, u.y); b = __floats2half2_rn(u.z, u.w);
+      c = __floats2half2_rn(v.x, v.y); e = __floats2half2_rn(v.z, v.w);
     } else {
       u = xr[2 * i];
       v = xr[2 * i + 1];
@@ -287,10 +292,11 @@ int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, i
 
 // x16 (layout 1 or 2) and the mean square of every row in one launch
 int moe_launch_f16_rows_meansq(const float* x, void* x16, int P, int d, int layout, float* xms, hipStream_t st) {
-  if (!x || !x16 || !xms || (layout != 1 && layout != 2)) return MOE_E_INVALID;
+  if (!x || !x16 || !xms || layout < 0 || layout > 2) return MOE_E_INVALID;
   if (d % 8 || (layout == 2 && d % 64) || !moe_aligned(x, 16) || !moe_aligned(x16, 16)) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
-  if (layout == 2) k_f32_to_f16_rows<2><<<(P + 3) / 4, 256, 0, st>>>(x, (uint4*)x16, P, d, xms);
+  if (layout == 0) k_f32_to_f16_rows<0><<<(P + 3) / 4, 256, 0, st>>>(x, (uint4*)x16, P, d, xms);
+  else if (layout == 2) k_f32_to_f16_rows<2><<<(P + 3) / 4, 256, 0, st>>>(x, (uint4*)x16, P, d, xms);
   else k_f32_to_f16_rows<1><<<(P + 3) / 4, 256, 0, st>>>(x, (uint4*)x16, P, d, xms);
   MOE_LAUNCH_CHECK();
   return MOE_OK;

@@ -155,7 +155,7 @@ def test_decode_topk_wide_logit_range(oracle, fmt):
 def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
     """GGUF layers in the type mix of the reference's checkpoints (Q4_K / Q5_K gate and up, Q5_1 / Q8_0 down,
     src/gpu/parts/30_host_util.inc:399-405): the general f32 GEMV kernels, ids bit-exact, output within the GEMV
-    bar; T = 40 walks a batch the grouped GEMM cannot take through the small path 32 rows at a time."""
+    bar; T = 40 is a batch for the general grouped GEMM."""
     rng = np.random.default_rng(tgu * 100 + tdn * 10 + T)
     d, mid, E, k = 512, 256, 12, 4
     hl = HostLayer(rng, d, mid, E, k, fmt="q4k", gg_types=(tgu, tdn, tsh))
@@ -163,10 +163,10 @@ def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
     yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
     m, dev = hl.to_gpu(max_tokens=64)
     y = m.forward(0, gpu(x)).cpu().numpy()
-    ids, _ = m.last_routing(min(T, 32))
-    if T <= 32:
-        assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
-    assert max_abs_rel(y, yo) <= TOL_GEMV, max_abs_rel(y, yo)
+    ids, _ = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    # batches over 32 tokens take the general grouped GEMM (f16 MFMA operands): the batch tolerance
+    assert max_abs_rel(y, yo) <= (TOL_GEMV if T <= 32 else 2e-3), max_abs_rel(y, yo)
     m.close()
 
 

@@ -290,3 +290,33 @@ def test_forward_with_the_callers_f16_copy(oracle, fmt):
     with pytest.raises(capi.MoeError):
         m.forward_x16(0, xg[:8].contiguous(), x16[:8].contiguous())
     m.close()
+
+
+@pytest.mark.parametrize("tgu,tdn,tsh,d,mid,T", [(13, 8, 12, 512, 256, 150), (12, 7, 12, 512, 256, 70), (13, 7, 8, 768, 256, 333),
+                                                  (23, 20, 12, 512, 256, 90), (20, 23, 23, 256, 256, 40), (8, 8, 8, 512, 64, 100),
+                                                  (13, 8, 12, 3072, 768, 200)])
+def test_batch_layer_other_gguf_types(oracle, tgu, tdn, tsh, d, mid, T):
+    """GGUF layers whose tensors are not Q4_K throughout (the reference checkpoints' Q5_K gate/up with Q5_1 / Q8_0
+    down, IQ4 types, a Q8_0 MTP sidecar) through the general grouped GEMM (src/gpu/parts/26_kernels_moe_gguf.inc:81-386):
+    ids bit-exact, output within the batch tolerance; the HC write-back variant and the caller's f16 copy as well."""
+    import torch
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(tgu * 100 + tdn + T)
+    E, k = 8, 3
+    hl = HostLayer(rng, d, mid, E, k, fmt="q4k", gg_types=(tgu, tdn, tsh))
+    x = S.bf16_round(rng.standard_normal((T, d), dtype=np.float32))
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    xg = gpu(x)
+    y = m.forward(0, xg).cpu().numpy()
+    ids, _ = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    err = max_abs_rel(y, yo)
+    assert err <= TOL_LAYER, err
+    assert m.x16_layout(0) == 0
+    y2 = m.forward_x16(0, xg, capi.f32_to_f16(xg, layout=0)).cpu().numpy()
+    assert (y2 == y).all()
+    m.set_option(capi.OPT_SHARED_ASIDE, 0)
+    y3 = m.forward(0, xg).cpu().numpy()
+    assert max_abs_rel(y3, yo) <= TOL_LAYER
+    m.close()
