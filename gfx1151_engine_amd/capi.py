@@ -10,7 +10,7 @@ import torch
 
 from .build import LIB
 
-F32, BF16, Q4CP = 1, 0, 5
+F32, BF16, Q4CP, Q8G64 = 1, 0, 5, 7
 GGML_Q4_K = 12
 GGML_Q5_K, GGML_Q5_1, GGML_Q8_0 = 13, 7, 8
 
@@ -197,7 +197,7 @@ class LutW(C.Structure):
 
 LUT_Q4CP = 100
 ROUTING_STATIC_MAX_TOKENS = 32768
-DENSE_SHARED = False  # moe_set_shared with bf16 / f32 matrices
+DENSE_SHARED = True  # moe_set_shared takes bf16 / f32 / q8g64 matrices
 OPT_INT_DECODE = 1
 OPT_UNIQUE_MIN_TOKENS = 2
 OPT_FUSED_COMBINE = 3

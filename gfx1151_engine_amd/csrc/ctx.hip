@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "common.h"
+#include "dense.h"
 #include "internal.h"
 
 struct MoeLayer {
@@ -16,6 +17,7 @@ struct MoeLayer {
   moe_gg_experts gg{};
   moe_wview sh_gate{}, sh_up{}, sh_down{}, sh_sg{};
   int sh_gguf_type = 0;
+  int sh_dense = 0;  // != 0: gate/up/down of the shared expert are dense rows of this kind (dense.h), in launches of their own
   // every q4cp codebook of the layer is affine (cb[n] = a*n + b): the integer-dot decode kernels apply
   bool experts_affine = false, shared_affine = false;
   // f16 range guard of the batch path: typical |hid| (and |pair|) per unit mean-square activation,
@@ -280,13 +282,18 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
       (int)dn->rows != cf.d || (int)dn->cols != cf.mid || (int)sg->rows != 1 || (int)sg->cols != cf.d)
     return MOE_E_INVALID;
   if (sg->dtype != MOE_DT_F32 && sg->dtype != MOE_DT_BF16) return MOE_E_UNSUPPORTED;
+  int dense = 0;
   if (sh_gguf_type == 0) {
-    if (g->dtype != MOE_DT_Q4CP || u->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP) return MOE_E_UNSUPPORTED;
+    if (g->dtype != u->dtype || g->dtype != dn->dtype) return MOE_E_UNSUPPORTED;
+    if (g->dtype != MOE_DT_Q4CP) {
+      dense = moe_dense_type_of_hgn(g->dtype);
+      if (!dense || !moe_dense_shared_supported(dense, cf.d, cf.mid)) return MOE_E_UNSUPPORTED;
+    }
   } else if (!moe_gg_types_supported(sh_gguf_type, sh_gguf_type, cf.d, cf.mid)) {
     return MOE_E_UNSUPPORTED;
   }
   L->shared_affine = false;
-  if (sh_gguf_type == 0) {
+  if (sh_gguf_type == 0 && !dense) {
     bool a1 = false, a2 = false, a3 = false;
     int rc;
     if ((rc = codebook_affine(g, &a1)) || (rc = codebook_affine(u, &a2)) || (rc = codebook_affine(dn, &a3))) return rc;
@@ -294,9 +301,11 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
   }
   L->c_shared = 0.f;
   {
-    int rc = magnitude_constant(c, sh_gguf_type, sh_gguf_type, g, (uint64_t)cf.mid, u, 0, dn, 1, &L->c_shared);
+    const int t = dense ? dense : sh_gguf_type;
+    int rc = magnitude_constant(c, t, t, g, (uint64_t)cf.mid, u, 0, dn, 1, &L->c_shared);
     if (rc) return rc;
   }
+  L->sh_dense = dense;
   L->sh_gate = *g;
   L->sh_up = *u;
   L->sh_down = *dn;
@@ -312,7 +321,7 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
 // gate rows start at row e*gate_stride of `gate`, its up rows at e*gate_stride + up_first of `up`
 // (the same fused tensor for hgn, a tensor of its own for GGUF), its down rows at e*down->rows/n.
 // Set-up work: dequantises 6 rows per sampled expert on the device and reads them back.
-// tgu / tdn: ggml block types of raw GGUF rows (gate and up; down), 0 = q4cp views.
+// tgu / tdn: ggml block types of raw GGUF rows (gate and up; down), a dense code of dense.h, or 0 = q4cp views.
 static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gate, uint64_t gate_stride,
                               const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
                               float* out) {
@@ -321,6 +330,8 @@ static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gat
   const uint64_t pitch = d > mid ? d : mid;
   auto deq = [&](const moe_wview* w, uint64_t row, float* dst) -> int {
     const int t = w == down ? tdn : tgu;
+    if (moe_is_dense_type(t))
+      return moe_dense_dequant_row(t, w->data + row * moe_dense_row_bytes(t, w->cols), (int)w->cols, dst, nullptr);
     if (t) return moe_gg_dequant_rows(t, w->data + row * moe_gg_row_bytes(t, w->cols), 1, w->cols, dst, nullptr);
     return moe_q4cp_dequant_rows(w->data, w->rows, w->cols, row, 1, dst, nullptr);
   };
@@ -413,7 +424,21 @@ MOE_API int moe_get_routing(moe_ctx* c, int P, int* ids_out, float* ws_out, moe_
 // Small batches: every (token, expert) slot reads its expert in place.  Four launches:
 // logits (+ shared-gate logit), top-k, gate/up/SwiGLU (shared expert as one more slot),
 // down + weighted combine + shared expert.
+static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st);
+
 static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
+  const int rc = forward_small_routed(c, L, x, P, y, st);
+  if (rc || !L.has_shared || !L.sh_dense) return rc;
+  // a densely stored shared expert: added to y behind the routed experts' kernels (its gate logit is in
+  // sh_logit since the router launch); scratch: the shared slot's part of hid32
+  const moe_config& g = c->cfg;
+  return moe_launch_dense_shared_small(L.sh_dense, L.sh_gate.data, L.sh_up.data, L.sh_down.data, c->sh_logit, x, P, g.d,
+                                       g.mid, c->hid32 + (size_t)(g.max_tokens < c->small_max ? g.max_tokens : c->small_max) * g.topk * g.mid,
+                                       y, st);
+}
+
+// the router and the routed experts (and the shared expert where the kernels take it along as one more slot)
+static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
   const moe_config& g = c->cfg;
   int rc;
   c->ev_n = 0;
@@ -428,7 +453,7 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     prof_mark(c, tag, st);
     return MOE_OK;
   };
-  const bool sh = L.has_shared;
+  const bool sh = L.has_shared && !L.sh_dense;  // the shared expert rides in these kernels as one more slot
   const int nslots_d = g.topk + (sh ? 1 : 0);
   const bool use_int = L.has_q4cp && c->int_decode && L.experts_affine && (!sh || L.shared_affine) &&
                        (!sh || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
@@ -440,7 +465,7 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const bool gu_topk = ((use_int && !use_uq) || use_int4k) && moe_dec_gu_topk_supported(g.experts, g.topk);
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
-         int e = moe_router_logits_small(&L.router, L.router_bias, sh ? &L.sh_sg : nullptr, x, P, c->logits,
+         int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
                                          c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
                                          use_int4k, gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk,
                                          g.id_stride, &fused, st, c->kpart, c->ktickets);
@@ -546,6 +571,7 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
 // blocks of any supported type (general kernel, f16 operands in natural order).
 static int batch_gemm_kind(const MoeLayer& L) {
   if (!L.has_gguf) return 0;
+  if (L.has_shared && L.sh_dense) return 2;  // (the dense shared expert reads activations in natural order)
   const bool all4k = L.gg.tgu == MOE_GGML_Q4_K && L.gg.tdn == MOE_GGML_Q4_K &&
                      (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K);
   return all4k ? 1 : 2;
@@ -574,7 +600,8 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   // gen: a GGUF layer that is not Q4_K throughout takes the general grouped GEMM (any supported block type,
   // dequantised into f16 tiles in LDS); Q4_K-only and q4cp layers take the tuned kernel
   const bool gen = batch_gemm_kind(L) == 2;
-  if (L.has_shared && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format family per layer
+  const bool shd = L.has_shared && L.sh_dense;  // shared expert stored densely: the general GEMM, launches of its own
+  if (L.has_shared && !shd && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format family per layer
   if (gen ? (g.d % 64 || g.mid % 64) : q4k ? (g.d % 256 || g.mid % 256) : (g.d % 128 || g.mid % 128 || g.mid < 256 || g.d < 256))
     return MOE_E_UNSUPPORTED;  // the caller walks the batch through the small path
   moe_lutw gu{}, dn{}, sgu{}, sdn{};
@@ -582,7 +609,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   if (q4k) {
     gu.w = L.gg.gate; gu.w_up = L.gg.up; gu.e_rows = g.mid;
     dn.w = L.gg.down; dn.e_rows = g.d;
-    if (L.has_shared) {
+    if (L.has_shared && !shd) {
       sgu.w = L.sh_gate.data; sgu.w_up = L.sh_up.data; sgu.e_rows = g.mid;
       sdn.w = L.sh_down.data; sdn.e_rows = g.d;
     }
@@ -590,7 +617,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     moe_lut_q4cp_view(L.gate_up.data, L.gate_up.rows, L.gate_up.cols, L.gate_up.scale_stride, 2 * g.mid, g.mid, &gu);
     moe_lut_q4cp_view(L.down.data, L.down.rows, L.down.cols, L.down.scale_stride, g.d, 0, &dn);
   }
-  if (L.has_shared && !q4k) {
+  if (L.has_shared && !q4k && !shd) {
     moe_lutw t;
     moe_lut_q4cp_view(L.sh_gate.data, L.sh_gate.rows, L.sh_gate.cols, L.sh_gate.scale_stride, g.mid, 0, &sgu);
     moe_lut_q4cp_view(L.sh_up.data, L.sh_up.rows, L.sh_up.cols, L.sh_up.scale_stride, g.mid, 0, &t);
@@ -608,6 +635,9 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   // gate/up (+ SwiGLU) and down launches over a tile list: routed experts, with_sh: the shared expert as well
   // (tiles whose expert index is >= n_experts)
   auto gemm_up = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2) -> int {
+    if (shd && with_sh)  // the shared expert's own tile list
+      return moe_launch_gemm_gg(true, L.sh_dense, L.sh_gate.data, L.sh_up.data, 0, nullptr, nullptr, g.experts, xh,
+                                c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, hs, s2, xl == 1 ? 1 : 0);
     if (gen)
       return moe_launch_gemm_gg(true, L.gg.tgu, L.gg.gate, L.gg.up, L.sh_gguf_type, with_sh ? L.sh_gate.data : nullptr,
                                 with_sh ? L.sh_up.data : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid,
@@ -616,14 +646,17 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
                                 g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up);
   };
   auto gemm_dn = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2, const moe_comb* cmb) -> int {
+    if (shd && with_sh)  // (hid rows of the shared tiles were written in natural order by the launch above)
+      return moe_launch_gemm_gg(false, L.sh_dense, L.sh_down.data, nullptr, 0, nullptr, nullptr, g.experts, c->hid16,
+                                nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2, 0);
     if (gen)
       return moe_launch_gemm_gg(false, L.gg.tdn, L.gg.down, nullptr, L.sh_gguf_type, with_sh ? L.sh_down.data : nullptr,
                                 nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2);
     return moe_launch_gemm_q4cp(false, &dn, with_sh ? &sdn : nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt,
                                 cmb ? (void*)cmb->y : (void*)c->pairs16, g.d, g.mid, cmb == nullptr, q4k, hs, s2, cmb);
   };
-  const bool fused = c->fused_combine && !c->hc && !gen;  // the HC write-back belongs to the ordered combine
-  if (L.has_shared && c->shared_aside && !fused) {
+  const bool fused = c->fused_combine && !c->hc && !gen && !shd;  // the HC write-back belongs to the ordered combine
+  if (L.has_shared && (shd || (c->shared_aside && !fused))) {
     // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
     // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
     // side stream also makes what both streams need first: the per-token mean square of x (range guard) and

@@ -5,11 +5,13 @@
 // one lane per 32-element block.  These are the general kernels; Q4_K alone has the tuned ones
 // (gemv_q4k.hip, decode_q4k.hip, the Q4_K instantiation of the grouped GEMM).
 #include "common.h"
+#include "dense.h"
 #include "internal.h"
 
 namespace {
 
 __device__ __host__ __forceinline__ uint64_t gg_row_bytes(int t, uint64_t k) {
+  if (moe_is_dense_type(t)) return moe_dense_row_bytes(t, k);
   switch (t) {
     case MOE_GGML_Q4_K: return k / 256 * 144;
     case MOE_GGML_Q5_K: return k / 256 * 176;
@@ -357,7 +359,7 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
                                                        const __half* __restrict__ x16, const int* __restrict__ tokidx,
                                                        const moe_tile* __restrict__ tiles,
                                                        const int* __restrict__ ntiles, __half* __restrict__ out, int M,
-                                                       int K, moe_hscale hs) {
+                                                       int K, moe_hscale hs, int a_layout) {
   extern __shared__ __attribute__((aligned(16))) uint8_t gsm[];
   uint8_t* const As = gsm;
   uint8_t* const Bs = gsm + 2 * GG_TILE_BYTES;
@@ -400,18 +402,39 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
 #pragma unroll
     for (int it = 0; it < 4; it++) {
       const int i = tid + 256 * it;
-      *(uint4*)(As + buf * GG_TILE_BYTES + (i >> 3) * GG_PITCH + (i & 7) * 16) = *(const uint4*)(arow[it] + (size_t)s * GG_BK);
+      uint4 v = *(const uint4*)(arow[it] + (size_t)s * GG_BK);
+      if (a_layout == 1) {
+        // the q4cp GEMM's order inside a group of 8, [e0,e4,e1,e5,e2,e6,e3,e7], back to natural order
+        const uint4 w = v;
+        v.x = __builtin_amdgcn_perm(w.y, w.x, 0x05040100u);
+        v.y = __builtin_amdgcn_perm(w.w, w.z, 0x05040100u);
+        v.z = __builtin_amdgcn_perm(w.y, w.x, 0x07060302u);
+        v.w = __builtin_amdgcn_perm(w.w, w.z, 0x07060302u);
+      }
+      *(uint4*)(As + buf * GG_TILE_BYTES + (i >> 3) * GG_PITCH + (i & 7) * 16) = v;
     }
-    int q[32];
-    float a, c;
-    gg_block(G.type, wrow, 2 * s + half, q, a, c);
     uint8_t* dst = Bs + buf * GG_TILE_BYTES + brow * GG_PITCH + half * 64;
+    if (moe_is_dense_type(G.type)) {
+      float w[32];
+      moe_dense_block(G.type, wrow, K, 2 * s + half, w);
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      gg_half8 v;
+      for (int j = 0; j < 4; j++) {
+        gg_half8 v;
 #pragma unroll
-      for (int l = 0; l < 8; l++) v[l] = (_Float16)fmaf(a, (float)q[8 * j + l], c);
-      *(gg_half8*)(dst + 16 * j) = v;
+        for (int l = 0; l < 8; l++) v[l] = (_Float16)w[8 * j + l];
+        *(gg_half8*)(dst + 16 * j) = v;
+      }
+    } else {
+      int q[32];
+      float a, c;
+      gg_block(G.type, wrow, 2 * s + half, q, a, c);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        gg_half8 v;
+#pragma unroll
+        for (int l = 0; l < 8; l++) v[l] = (_Float16)fmaf(a, (float)q[8 * j + l], c);
+        *(gg_half8*)(dst + 16 * j) = v;
+      }
     }
   };
   gg_floatx16 acc[2][2];
@@ -529,15 +552,20 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
 
 // Internal: grouped GEMM over tiles of <= 128 pairs for raw GGUF expert tensors of any supported block type
 // (routed experts of type `type`, optional shared expert of type `tsh`; tile.expert >= n_experts selects it).
-// up: gate/up + SwiGLU -> hid f16 [pairs][m]; else down -> pairs f16 [pairs][m].  x / hid: f16, natural order.
+// `type` / `tsh` may also be a dense code of dense.h (bf16 / f32 / q8g64 rows).
+// up: gate/up + SwiGLU -> hid f16 [pairs][m]; else down -> pairs f16 [pairs][m].  x / hid: f16, natural order
+// (a_layout = 1: x is in the q4cp GEMM's order and is put back in natural order on its way into LDS).
 int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up, int tsh, const uint8_t* sh_w,
                        const uint8_t* sh_w_up, int n_experts, const __half* x16, const int* tokidx,
                        const moe_tile* tiles, const int* ntiles, int max_tiles, __half* out, int m, int k,
-                       moe_hscale hs, hipStream_t st) {
+                       moe_hscale hs, hipStream_t st, int a_layout) {
   if (!w || (up && !w_up) || !x16 || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
-  if (!gg_type_ok(type, k) || (sh_w && !gg_type_ok(tsh, k)) || k % GG_BK || m < 1) return MOE_E_UNSUPPORTED;
-  if (!moe_aligned(w, gg_align(type)) || (up && !moe_aligned(w_up, gg_align(type))) || !moe_aligned(x16, 16) ||
-      (sh_w && (!moe_aligned(sh_w, gg_align(tsh)) || (up && (!sh_w_up || !moe_aligned(sh_w_up, gg_align(tsh)))))))
+  auto type_ok = [&](int t) { return moe_is_dense_type(t) ? k % 64 == 0 : gg_type_ok(t, k); };
+  auto align_of = [&](int t) -> size_t { return moe_is_dense_type(t) ? 16 : gg_align(t); };
+  if (!type_ok(type) || (sh_w && !type_ok(tsh)) || k % GG_BK || m < 1 || a_layout < 0 || a_layout > 1)
+    return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(w, align_of(type)) || (up && !moe_aligned(w_up, align_of(type))) || !moe_aligned(x16, 16) ||
+      (sh_w && (!moe_aligned(sh_w, align_of(tsh)) || (up && (!sh_w_up || !moe_aligned(sh_w_up, align_of(tsh)))))))
     return MOE_E_INVALID;
   if (max_tiles == 0) return MOE_OK;
   GgGemmW R{w, w_up, type}, S{sh_w ? sh_w : w, sh_w ? sh_w_up : w_up, sh_w ? tsh : type};
@@ -548,8 +576,8 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     attr_done = true;
   }
-  if (up) k_moe_gemm_gg<true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs);
-  else k_moe_gemm_gg<false><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs);
+  if (up) k_moe_gemm_gg<true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+  else k_moe_gemm_gg<false><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -121,7 +121,12 @@ int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float
 int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up, int tsh, const uint8_t* sh_w,
                        const uint8_t* sh_w_up, int n_experts, const __half* x16, const int* tokidx,
                        const moe_tile* tiles, const int* ntiles, int max_tiles, __half* out, int m, int k,
-                       moe_hscale hs, hipStream_t st);
+                       moe_hscale hs, hipStream_t st, int a_layout = 0);
+// shared expert stored densely (bf16 / f32 / q8g64; type codes of dense.h)
+bool moe_dense_shared_supported(int type, int d, int mid);
+int moe_launch_dense_shared_small(int type, const uint8_t* g, const uint8_t* u, const uint8_t* dn, const float* sh_logit,
+                                  const float* x, int P, int d, int mid, float* hid, float* y, hipStream_t st);
+int moe_dense_dequant_row(int type, const uint8_t* row, int K, float* out, hipStream_t st);
 bool moe_gg_types_supported(int tgu, int tdn, int d, int mid);
 uint64_t moe_gg_row_bytes(int type, uint64_t k);
 int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gate, const uint8_t* up,

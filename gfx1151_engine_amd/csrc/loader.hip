@@ -482,6 +482,10 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
       if (cols % 32 || __builtin_mul_overflow(rows, (uint64_t)v->scale_stride, &sc) ||
           __builtin_add_overflow(64 + cells / 2, sc, &want))
         return MOE_E_INVALID;
+    } else if (t.dtype == MOE_DT_Q8G64) {  // per row: cols codes + cols/64 x (fp16 scale, fp16 min) (src/hgn.h:189-196)
+      uint64_t stride;
+      if (cols % 64 || __builtin_add_overflow(cols, cols / 64 * 4, &stride) || __builtin_mul_overflow(rows, stride, &want))
+        return MOE_E_INVALID;
     } else if (__builtin_mul_overflow(cells, (uint64_t)(t.dtype == MOE_DT_F32 ? 4 : 2), &want)) {
       return MOE_E_INVALID;
     }
@@ -498,8 +502,10 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
     const FTensor* sd = findp("shared_expert.down_proj.weight");
     const FTensor* sx = findp("shared_expert_gate.weight");
     if (!su || !sd || !sx) return MOE_E_STATE;
-    // the shared expert of this path is q4cp; bf16 / q8 shared experts stay with the caller's dense kernels
-    if (sg->dtype != MOE_DT_Q4CP || su->dtype != MOE_DT_Q4CP || sd->dtype != MOE_DT_Q4CP || !hgn_dtype_ok_dense(sx->dtype))
+    // q4cp, or one of the dense dtypes of the reference's generic matvec (bf16, f32, the overlay files' q8g64);
+    // moe_set_shared checks that the three agree
+    auto sh_ok = [](int dt) { return dt == MOE_DT_Q4CP || dt == MOE_DT_BF16 || dt == MOE_DT_F32 || dt == MOE_DT_Q8G64; };
+    if (!sh_ok(sg->dtype) || !sh_ok(su->dtype) || !sh_ok(sd->dtype) || !hgn_dtype_ok_dense(sx->dtype))
       return MOE_E_UNSUPPORTED;
     moe_wview a{}, b{}, c2{}, d2{};
     if ((rc = view(*sg, &a)) || (rc = view(*su, &b)) || (rc = view(*sd, &c2)) || (rc = view(*sx, &d2))) return rc;

@@ -133,6 +133,33 @@ def make_gg(rng, t, rows, cols, scale_std=0.01):
             GG_IQ4_XS: make_iq4_xs}[t](rng, rows, cols, scale_std)
 
 
+def quantize_q8g64(w):
+    """f32 [rows][cols] -> the reference checkpoint format's q8g64 bytes (src/hgn.h:189-196): per row cols uint8
+    codes, then cols/64 pairs of fp16 (scale, min), w ~ code * scale + min.  uint8 [rows][cols + cols/64*4]."""
+    w = np.ascontiguousarray(w, np.float32)
+    rows, cols = w.shape
+    assert cols % 64 == 0
+    g = w.reshape(rows, cols // 64, 64)
+    mn = g.min(axis=2).astype(np.float16)
+    sc = ((g.max(axis=2) - mn.astype(np.float32)) / 255.0).astype(np.float16)
+    scf = np.where(sc == 0, np.float16(1), sc).astype(np.float32)
+    codes = np.clip(np.rint((g - mn.astype(np.float32)[..., None]) / scf[..., None]), 0, 255).astype(np.uint8)
+    sm = np.stack([sc, mn], axis=2).reshape(rows, cols // 64 * 2).view(np.uint8)
+    return np.ascontiguousarray(np.concatenate([codes.reshape(rows, cols), sm], axis=1))
+
+
+def make_q8g64(rng, rows, cols, std=0.05):
+    return quantize_q8g64(rng.standard_normal((rows, cols), dtype=np.float32) * std)
+
+
+def make_dense(rng, kind, rows, cols, std=0.05):
+    """A dense weight matrix as stored bytes: kind "bf16" (uint16 bit patterns), "f32" or "q8g64"."""
+    if kind == "q8g64":
+        return make_q8g64(rng, rows, cols, std)
+    w = rng.standard_normal((rows, cols), dtype=np.float32) * std
+    return f32_to_bf16_bits(w) if kind == "bf16" else w
+
+
 def f32_to_bf16_bits(a):
     """Round-to-nearest-even f32 -> bf16 bit patterns (uint16)."""
     u = np.ascontiguousarray(a, np.float32).view(np.uint32)

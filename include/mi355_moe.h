@@ -32,7 +32,7 @@ enum moe_status {
 };
 
 /* hgn tensor dtypes (src/hgn.h:2-23) and ggml types (src/gguf.h:42-64) used on this path */
-enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5 };
+enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5, MOE_DT_Q8G64 = 7 };
 /* Q4_K: every kernel of the path.  Q5_K (gate/up), Q5_1 and Q8_0 (down) — the mix of the reference's GGUF
  * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — and IQ4_NL / IQ4_XS (src/gguf.h:376-407):
  * dequantisation and the general GEMV kernels. */
@@ -210,9 +210,12 @@ int moe_destroy(moe_ctx* ctx);
  * hgn: gate_up [E*2*mid][d] and down [E*d][mid] q4cp views (40_model.inc:1826-1829).
  * gguf: GgExperts (40_model.inc:1823).  Exactly one of hgn / gguf per layer.
  * shared expert: gate_proj/up_proj [mid][d], down_proj [d][mid], shared_expert_gate [1][d]
- * (40_model.inc:1848-1857).  gate_proj / up_proj / down_proj: q4cp (each tensor with its own codebook), or,
- * with sh_gguf_type != 0, raw GGUF rows of that one ggml type; shared_expert_gate: f32 or bf16.
- * MOE_E_UNSUPPORTED for other matrix dtypes. */
+ * (40_model.inc:1848-1857).  gate_proj / up_proj / down_proj: q4cp (each tensor with its own codebook); or one of
+ * the dense dtypes of the reference's generic matvec (src/ref.cpp:68-109) for all three: bf16, f32, q8g64 (dtype 7,
+ * the overlay files' tensors: per row cols uint8 codes then cols/64 x (fp16 scale, fp16 min)); or, with
+ * sh_gguf_type != 0, raw GGUF rows of that one ggml type.  shared_expert_gate: f32 or bf16.
+ * MOE_E_UNSUPPORTED for other matrix dtypes.  A densely stored shared expert of a q4cp layer runs in launches of its
+ * own next to the routed experts' kernels. */
 int moe_set_router(moe_ctx* ctx, int layer, const moe_wview* gate_w, const float* router_bias);
 int moe_set_experts_q4cp(moe_ctx* ctx, int layer, const moe_wview* gate_up, const moe_wview* down);
 int moe_set_experts_gguf(moe_ctx* ctx, int layer, const moe_gg_experts* gg);

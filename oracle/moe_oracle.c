@@ -40,7 +40,8 @@
 
 /* ---- weight format tags (shared with the library header by value) ---- */
 enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q5_1 = 7, ORC_Q8_0 = 8,
-       ORC_IQ4_NL = 20, ORC_IQ4_XS = 23 };
+       ORC_IQ4_NL = 20, ORC_IQ4_XS = 23,
+       ORC_Q8G64 = 107 /* hgn dtype 7; the tag is moved off ggml's Q5_1 = 7 */ };
 
 /* src/hgn.h:77-84 and src/gguf.h:318-325 (same function twice in the reference) */
 ORC_API float orc_fp16_to_f32(uint16_t h) {
@@ -264,14 +265,46 @@ static void mat_row(const orc_mat* W, uint64_t r, float* out) {
     case ORC_Q5K: case ORC_Q8_0: case ORC_Q5_1: case ORC_IQ4_NL: case ORC_IQ4_XS:
       orc_gg_row(W->dtype, W->data + r * orc_gg_row_bytes(W->dtype, W->cols), out, W->cols);
       break;
+    case ORC_Q8G64: { /* src/hgn.h:189-202: per row [cols uint8][cols/64 x (fp16 scale, fp16 min)], w = code * s + m */
+      const uint8_t* rp = W->data + r * (W->cols + W->cols / 64 * 4);
+      const uint16_t* sm = (const uint16_t*)(rp + W->cols);
+      for (uint64_t g = 0; g < W->cols / 64; g++) {
+        const float s = orc_fp16_to_f32(sm[g * 2]), m = orc_fp16_to_f32(sm[g * 2 + 1]);
+        for (uint64_t j = 0; j < 64; j++) out[g * 64 + j] = rp[g * 64 + j] * s + m;
+      }
+      break;
+    }
     default: memset(out, 0, W->cols * 4);
   }
+}
+ORC_API void orc_mat_rows(const orc_mat* W, uint64_t row0, uint64_t nrows, float* out) {
+  for (uint64_t r = 0; r < nrows; r++) mat_row(W, row0 + r, out + r * W->cols);
 }
 
 /* src/ref.cpp:75-77,85-87: acc (double) += (double)w * x, c ascending, then (float) */
 static inline float dot_f64(const float* w, const float* x, uint64_t n) {
   double acc = 0;
   for (uint64_t c = 0; c < n; c++) acc += (double)w[c] * x[c];
+  return (float)acc;
+}
+
+/* One output of the reference's matvec (src/ref.cpp:68-109) for row r of W, whose dequantised row is wr.  q8g64 does
+ * not go through the dequantised row: per 64-group it sums code * x and x in fp64 and adds a2 * s + mn * csum
+ * (ref.cpp:91-106). */
+static inline float mat_dot(const orc_mat* W, uint64_t r, const float* wr, const float* x) {
+  if (W->dtype != ORC_Q8G64) return dot_f64(wr, x, W->cols);
+  const uint8_t* codes = W->data + r * (W->cols + W->cols / 64 * 4);
+  const uint16_t* sm = (const uint16_t*)(codes + W->cols);
+  double acc = 0;
+  for (uint64_t g = 0; g < W->cols / 64; g++) {
+    const float s = orc_fp16_to_f32(sm[g * 2]), mn = orc_fp16_to_f32(sm[g * 2 + 1]);
+    double a2 = 0, csum = 0;
+    for (int j = 0; j < 64; j++) {
+      a2 += (double)codes[g * 64 + j] * x[g * 64 + j];
+      csum += x[g * 64 + j];
+    }
+    acc += a2 * s + mn * csum;
+  }
   return (float)acc;
 }
 
@@ -507,12 +540,12 @@ ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int*
       mat_row(&L->sh_gate, (uint64_t)r, wr);
       for (int i = 0; i < n; i++) {
         const int t = tok_list ? tok_list[i] : i;
-        g1[(size_t)i * mid + r] = dot_f64(wr, x + (size_t)t * d, d);
+        g1[(size_t)i * mid + r] = mat_dot(&L->sh_gate, (uint64_t)r, wr, x + (size_t)t * d);
       }
       mat_row(&L->sh_up, (uint64_t)r, wr);
       for (int i = 0; i < n; i++) {
         const int t = tok_list ? tok_list[i] : i;
-        u1[(size_t)i * mid + r] = dot_f64(wr, x + (size_t)t * d, d);
+        u1[(size_t)i * mid + r] = mat_dot(&L->sh_up, (uint64_t)r, wr, x + (size_t)t * d);
       }
     }
 #pragma omp single
@@ -520,7 +553,7 @@ ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int*
       mat_row(&L->sh_sg, 0, wr);
       for (int i = 0; i < n; i++) {
         const int t = tok_list ? tok_list[i] : i;
-        sg[i] = sigmoidf_ref(dot_f64(wr, x + (size_t)t * d, d));
+        sg[i] = sigmoidf_ref(mat_dot(&L->sh_sg, 0, wr, x + (size_t)t * d));
       }
     }
 #pragma omp for schedule(static)
@@ -530,7 +563,7 @@ ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int*
       mat_row(&L->sh_down, (uint64_t)r, wr);
       for (int i = 0; i < n; i++) {
         const int t = tok_list ? tok_list[i] : i;
-        const float ey = dot_f64(wr, g1 + (size_t)i * mid, mid);
+        const float ey = mat_dot(&L->sh_down, (uint64_t)r, wr, g1 + (size_t)i * mid);
         y[(size_t)t * d + r] = y[(size_t)t * d + r] + sg[i] * ey; /* ref.cpp:636 */
       }
     }

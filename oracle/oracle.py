@@ -12,6 +12,8 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 F32, BF16, Q4CP, Q4K = 1, 0, 5, 12
 Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS = 13, 7, 8, 20, 23   # further ggml block types of the expert tensors (ids as in GGUF)
+Q8G64 = 107  # hgn dtype 7 (the oracle's tag is moved off ggml's Q5_1 = 7)
+HGN_DTYPE = {BF16: 0, F32: 1, Q4CP: 5, Q8G64: 7}  # oracle tag -> dtype field of the reference's checkpoint format
 GG_TYPES = (Q4K, Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS)
 
 
@@ -46,6 +48,8 @@ def lib():
         _lib = C.CDLL(path)
         _lib.orc_fp16_to_f32.restype = C.c_float
         _lib.orc_fp16_to_f32.argtypes = [C.c_uint16]
+        _lib.orc_mat_rows.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_void_p]
+        _lib.orc_mat_rows.restype = None
         _lib.orc_q4cp_scale_stride.restype = C.c_uint64
         _lib.orc_q4cp_scale_stride.argtypes = [C.c_uint64]
         _lib.orc_q4cp_blob_bytes.restype = C.c_uint64
@@ -100,6 +104,8 @@ class Mat:
             assert self.data.dtype == np.float32 and self.data.size == rows * cols
         elif dtype == BF16:
             assert self.data.dtype == np.uint16 and self.data.size == rows * cols
+        elif dtype == Q8G64:
+            assert self.data.dtype == np.uint8 and cols % 64 == 0 and self.data.size == rows * (cols + cols // 64 * 4)
 
     def c(self):
         return _Mat(self.dtype, self.data.ctypes.data, self.rows, self.cols)
@@ -116,6 +122,11 @@ class Mat:
             return gg_rows(self.dtype, self.data[row0 * rb:(row0 + nrows) * rb], nrows, self.cols)
         if self.dtype == F32:
             return self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].copy()
+        if self.dtype == Q8G64:
+            out = np.empty((nrows, self.cols), np.float32)
+            m = self.c()
+            lib().orc_mat_rows(C.byref(m), row0, nrows, _p(out))
+            return out
         u = self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].astype(np.uint32) << 16
         return u.view(np.float32)
 
@@ -290,6 +301,15 @@ def ref_q4cp_rows(blob, rows, cols, row0, nrows):
     return out
 
 
+def ref_dequant_tensor(mat):
+    """Checkpoint::dequant of the reference on a BF16 / Q8G64 Mat."""
+    out = np.empty((mat.rows, mat.cols), np.float32)
+    rc = ref().ref_dequant_tensor(C.c_uint32(HGN_DTYPE[mat.dtype]), C.c_uint64(mat.rows), C.c_uint64(mat.cols),
+                                  _p(mat.data), _p(out))
+    assert rc == 0
+    return out
+
+
 def ref_q4k_rows(raw, nrows, k):
     raw = _c(raw, np.uint8)
     rb = ref().ref_q4k_row_bytes(C.c_uint64(k))
@@ -315,10 +335,10 @@ def ref_moe_token(layer, x):
     y = np.empty(layer.d, np.float32)
     sh_gate, sh_up, sh_down, sh_sg = layer.shared
     assert sh_gate.dtype == sh_up.dtype == sh_down.dtype
-    rc = ref().ref_moe_token(layer.d, layer.mid, layer.E, layer.k, C.c_uint32(layer.router.dtype),
+    rc = ref().ref_moe_token(layer.d, layer.mid, layer.E, layer.k, C.c_uint32(HGN_DTYPE[layer.router.dtype]),
                              _p(layer.router.data), _p(layer.gate_up.data), _p(layer.down.data),
-                             C.c_uint32(sh_gate.dtype), _p(sh_gate.data), _p(sh_up.data),
-                             _p(sh_down.data), C.c_uint32(sh_sg.dtype), _p(sh_sg.data), _p(x), _p(y))
+                             C.c_uint32(HGN_DTYPE[sh_gate.dtype]), _p(sh_gate.data), _p(sh_up.data),
+                             _p(sh_down.data), C.c_uint32(HGN_DTYPE[sh_sg.dtype]), _p(sh_sg.data), _p(x), _p(y))
     assert rc == 0
     return y
 

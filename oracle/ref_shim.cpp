@@ -33,6 +33,7 @@ hgn::Tensor mk(const char* name, uint32_t dtype, uint64_t rows, uint64_t cols,
 uint64_t dense_bytes(uint32_t dtype, uint64_t rows, uint64_t cols) {
   if (dtype == 0) return rows * cols * 2;  // bf16
   if (dtype == 5) return 64 + rows * cols / 2 + rows * (((cols / 32 * 2) + 15) & ~15ULL);
+  if (dtype == 7) return rows * (cols + cols / 64 * 4);  // q8g64
   return 0;
 }
 }  // namespace
@@ -51,6 +52,18 @@ __attribute__((visibility("default"))) int ref_q4cp_rows(const uint8_t* blob, ui
     hgn::Tensor t = mk("w", 5, rows, cols, blob, dense_bytes(5, rows, cols));
     auto q = hgn::Checkpoint::q4cp_parse(t);
     for (uint64_t r = 0; r < nrows; r++) hgn::Checkpoint::q4cp_row(q, row0 + r, out + r * cols);
+    return 0;
+  } catch (...) {
+    return -1;
+  }
+}
+
+// hgn::Checkpoint::dequant (src/hgn.h:165-207) of a whole tensor of `rows` x `cols` stored as `dtype` (0 bf16, 7 q8g64)
+__attribute__((visibility("default"))) int ref_dequant_tensor(uint32_t dtype, uint64_t rows, uint64_t cols,
+                                                              const uint8_t* data, float* out) {
+  try {
+    hgn::Checkpoint ck;
+    ck.dequant(mk("w", dtype, rows, cols, data, dense_bytes(dtype, rows, cols)), out);
     return 0;
   } catch (...) {
     return -1;
@@ -88,7 +101,7 @@ __attribute__((visibility("default"))) uint64_t ref_q4k_row_bytes(uint64_t k) {
 }
 
 // The reference's Model::moe for ONE token on a one-layer synthetic checkpoint.
-// router / shared-expert tensors: dtype 0 (bf16) or 5 (q4cp) as the reference's
+// router / shared-expert tensors: dtype 0 (bf16), 5 (q4cp) or 7 (q8g64) as the reference's
 // matvec supports; routed experts: q4cp blobs [E*2*mid, d] and [E*d, mid].
 __attribute__((visibility("default"))) int ref_moe_token(
     int d, int mid, int E, int k, uint32_t router_dtype, const uint8_t* router,

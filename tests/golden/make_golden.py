@@ -67,7 +67,8 @@ def q4k_cases():
 def layer_cases():
     """Model::moe on tiny layers: (d, mid, E, k, router/shared dtype)."""
     out = {}
-    cases = [(64, 32, 8, 3, "bf16"), (128, 64, 8, 4, "q4cp"), (96, 64, 12, 10, "bf16")]
+    cases = [(64, 32, 8, 3, "bf16"), (128, 64, 8, 4, "q4cp"), (96, 64, 12, 10, "bf16"),
+             (128, 64, 8, 3, "q8g64")]
     for i, (d, mid, E, k, kind) in enumerate(cases):
         rng = np.random.default_rng(777 + i)
         cb = rng.uniform(-2, 2, 16).astype(np.float32) if i == 2 else None
@@ -79,6 +80,9 @@ def layer_cases():
             shg, shu, shd = (S.make_q4cp(rng, mid, d, scale_std=0.05), S.make_q4cp(rng, mid, d, scale_std=0.05),
                              S.make_q4cp(rng, d, mid, scale_std=0.05))
             sh_dt = O.Q4CP
+        elif kind == "q8g64":  # the overlay files' storage of the shared expert (src/hgn.h:10, src/ref.cpp:91-106)
+            shg, shu, shd = (S.make_q8g64(rng, mid, d, 0.1), S.make_q8g64(rng, mid, d, 0.1), S.make_q8g64(rng, d, mid, 0.1))
+            sh_dt = O.Q8G64
         else:
             shg = S.f32_to_bf16_bits(rng.standard_normal((mid, d)).astype(np.float32) * 0.1)
             shu = S.f32_to_bf16_bits(rng.standard_normal((mid, d)).astype(np.float32) * 0.1)
@@ -97,6 +101,11 @@ def layer_cases():
                     f"sg{i}": sg, f"shg{i}": np.asarray(shg), f"shu{i}": np.asarray(shu), f"shd{i}": np.asarray(shd),
                     f"x{i}": x, f"ybits{i}": y.view(np.uint32)})
     out["n"] = np.array(len(cases))
+    # Checkpoint::dequant of one q8g64 tensor (src/hgn.h:189-202)
+    rng = np.random.default_rng(790)
+    q8 = S.make_q8g64(rng, 5, 192, 0.3)
+    out["q8g64_raw"] = q8
+    out["q8g64_bits"] = O.ref_dequant_tensor(O.Mat(O.Q8G64, q8, 5, 192)).view(np.uint32)
     np.savez_compressed(os.path.join(OUT, "moe_layer.npz"), **out)
 
 

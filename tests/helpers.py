@@ -19,10 +19,13 @@ class HostLayer:
     """One synthetic MoE layer as host bytes (the 'file' side)."""
 
     def __init__(self, rng, d, mid, E, k, fmt="q4cp", router_dtype="f32", codebook=None, scale_std=0.01,
-                 router_std=0.02, shared=True, bias=None, gg_types=(12, 12, 12), shared_codebooks=None):
+                 router_std=0.02, shared=True, bias=None, gg_types=(12, 12, 12), shared_codebooks=None,
+                 shared_dense=None):
         """fmt "q4k": raw GGUF blocks; gg_types = ggml types of (gate/up, down, shared expert).
         shared_codebooks: three 16-entry tables for the shared expert's gate_proj / up_proj / down_proj (q4cp; the
-        reference's converter trains one codebook per dense tensor, tools/flashnext2hgn.py:164-187)."""
+        reference's converter trains one codebook per dense tensor, tools/flashnext2hgn.py:164-187).
+        shared_dense: "bf16" / "f32" / "q8g64": the shared expert's matrices in that dense storage instead."""
+        self.shared_dense = shared_dense
         self.d, self.mid, self.E, self.k, self.fmt = d, mid, E, k, fmt
         self.tgu, self.tdn, self.tsh = gg_types
         rw = (rng.standard_normal((E, d), dtype=np.float32) * router_std)
@@ -45,6 +48,8 @@ class HostLayer:
             scb = shared_codebooks if shared_codebooks is not None else [codebook] * 3
             mk = (lambda r, c, i: S.make_q4cp(rng, r, c, codebook=scb[i], scale_std=scale_std)) if fmt == "q4cp" \
                 else (lambda r, c, i: S.make_gg(rng, self.tsh, r, c, scale_std=scale_std))
+            if shared_dense:
+                mk = lambda r, c, i: S.make_dense(rng, shared_dense, r, c, std=0.05)
             self.shared = [mk(mid, d, 0), mk(mid, d, 1), mk(d, mid, 2),
                            rng.standard_normal((1, d), dtype=np.float32) * router_std]
 
@@ -54,6 +59,8 @@ class HostLayer:
         sh = None
         if self.shared is not None:
             st = O.Q4CP if self.fmt == "q4cp" else self.tsh
+            if self.shared_dense:
+                st = {"bf16": O.BF16, "f32": O.F32, "q8g64": O.Q8G64}[self.shared_dense]
             sh = [O.Mat(st, self.shared[0], mid, d), O.Mat(st, self.shared[1], mid, d),
                   O.Mat(st, self.shared[2], d, mid), O.Mat(O.F32, self.shared[3], 1, d)]
         router = O.Mat(self.router_dt, self.router, E, d)
@@ -86,9 +93,14 @@ class HostLayer:
             m.set_experts_gguf(0, up("gate", self.gate), up("up", self.up), up("down", self.down), self.tgu, self.tdn)
         if self.shared is not None:
             wt = capi.Q4CP if self.fmt == "q4cp" else 0
-            m.set_shared(0, capi.wview(up("shg", self.shared[0]), wt, mid, d),
-                         capi.wview(up("shu", self.shared[1]), wt, mid, d),
-                         capi.wview(up("shd", self.shared[2]), wt, d, mid),
+            shw = self.shared[:3]
+            if self.shared_dense:
+                wt = {"bf16": capi.BF16, "f32": capi.F32, "q8g64": capi.Q8G64}[self.shared_dense]
+                if self.shared_dense == "bf16":
+                    shw = [a.view(np.int16) for a in shw]
+            m.set_shared(0, capi.wview(up("shg", shw[0]), wt, mid, d),
+                         capi.wview(up("shu", shw[1]), wt, mid, d),
+                         capi.wview(up("shd", shw[2]), wt, d, mid),
                          capi.wview(up("shsg", self.shared[3]), capi.F32, 1, d),
-                         0 if self.fmt == "q4cp" else self.tsh)
+                         0 if self.fmt == "q4cp" or self.shared_dense else self.tsh)
         return m, dev

@@ -232,6 +232,28 @@ def test_hgn_file_with_a_codebook_per_shared_tensor(tmp_path):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["bf16", "q8g64"])
+def test_hgn_file_with_a_densely_stored_shared_expert(tmp_path, kind):
+    """The shared expert as bf16 (an unquantised checkpoint) or q8g64 (the overlay files' storage, src/hgn.h:10):
+    the reference runs these through its generic matvec (src/ref.cpp:68-109,623-636)."""
+    import torch
+    rng = np.random.default_rng(23)
+    hl = HostLayer(rng, D, MID, E, K, shared_dense=kind)
+    p, _ = _hgn(tmp_path, [hl], first=0)
+    f = capi.ModelFile(p)
+    m = capi.Moe(D, MID, E, K, layers=1, max_tokens=80)
+    w = f.load_layers(m, 0, 0, 1)
+    f.close()
+    for T in (1, 9, 80):
+        x = _x(T, seed=T)
+        want, io, _ = O.moe_layer(hl.oracle_layer(), x)
+        y = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max(), T
+    del m
+    w.free()
+
+
+@pytest.mark.gpu
 def test_gguf_router_tensors_are_rounded_to_bf16_like_the_reference(tmp_path):
     """The reference maps a GGUF's F32 ffn_gate_inp / ffn_gate_inp_shexp to bf16 tensors (src/gguf_map.h:210-211), so
     its router multiplies the rounded values.  A loaded layer must route like the oracle fed those bf16 values, and

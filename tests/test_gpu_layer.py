@@ -196,31 +196,32 @@ def test_unique_expert_path(oracle, share):
     m.close()
 
 
-@pytest.mark.parametrize("i", [0, 1, 2])
+@pytest.mark.parametrize("i", [0, 1, 2, 3])
 def test_golden_layers_from_reference(oracle, golden, i):
-    """Inputs and outputs of the reference's own Model::moe (tests/golden/moe_layer.npz): three layers, two of them
-    with a bf16 shared expert."""
+    """Inputs and outputs of the reference's own Model::moe (tests/golden/moe_layer.npz): four layers, two of them
+    with a bf16 shared expert, one with a q8g64 one."""
     import torch
     from gfx1151_engine_amd import capi
     g = golden("moe_layer.npz")
-    assert int(g["n"]) == 3
+    assert int(g["n"]) == 4
     d, mid, E, k, sh_dt = (int(v) for v in g[f"cfg{i}"])
     m = capi.Moe(d, mid, E, k)
-    sh16 = sh_dt != oracle.Q4CP  # bf16 matrices are stored as uint16 bit patterns
-    if sh16 and not capi.DENSE_SHARED:
-        pytest.skip("bf16 shared-expert matrices: moe_set_shared takes q4cp or raw GGUF rows only")
+    sh16 = sh_dt == oracle.BF16  # bf16 matrices are stored as uint16 bit patterns
     shv = [g[f"shg{i}"], g[f"shu{i}"], g[f"shd{i}"]]
     keep = [gpu(g[f"router{i}"].view(np.int16)), gpu(g[f"gu{i}"]), gpu(g[f"dn{i}"])] + \
            [gpu(a.view(np.int16) if sh16 else a) for a in shv] + [gpu(g[f"sg{i}"].view(np.int16))]
-    wt = capi.BF16 if sh16 else capi.Q4CP
+    wt = {oracle.BF16: capi.BF16, oracle.Q4CP: capi.Q4CP, oracle.Q8G64: capi.Q8G64}[sh_dt]
     m.set_router(0, capi.wview(keep[0], capi.BF16, E, d))
     m.set_experts_q4cp(0, capi.wview(keep[1], capi.Q4CP, E * 2 * mid, d), capi.wview(keep[2], capi.Q4CP, E * d, mid))
     m.set_shared(0, capi.wview(keep[3], wt, mid, d), capi.wview(keep[4], wt, mid, d),
                  capi.wview(keep[5], wt, d, mid), capi.wview(keep[6], capi.BF16, 1, d))
     x = g[f"x{i}"]
-    y = m.forward(0, gpu(x)).cpu().numpy()
     want = g[f"ybits{i}"].view(np.float32)
-    assert max_abs_rel(y, want) <= TOL_GEMV, i
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    assert max_abs_rel(y, want) <= TOL_INT_Q4CP, i  # integer-dot decode kernels where the codebook is affine
+    m.set_option(capi.OPT_INT_DECODE, 0)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    assert max_abs_rel(y, want) <= 5e-6, i          # f32 kernels: f32 against the reference's fp64 sums
     m.close()
 
 

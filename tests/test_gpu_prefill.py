@@ -320,3 +320,27 @@ def test_batch_layer_other_gguf_types(oracle, tgu, tdn, tsh, d, mid, T):
     y3 = m.forward(0, xg).cpu().numpy()
     assert max_abs_rel(y3, yo) <= TOL_LAYER
     m.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fmt,kind", [("q4cp", "bf16"), ("q4cp", "q8g64"), ("q4cp", "f32"), ("q4k", "bf16"), ("gg", "q8g64")])
+def test_batch_layer_with_a_densely_stored_shared_expert(oracle, fmt, kind):
+    """bf16 / f32 / q8g64 shared-expert matrices beside q4cp, all-Q4_K and mixed-GGUF routed experts: decode, a small
+    batch and a grouped-GEMM batch against the oracle (which follows the reference's matvec per storage,
+    src/ref.cpp:68-109)."""
+    import torch
+    rng = np.random.default_rng(77)
+    d, mid, E, k = 512, 256, 16, 4
+    gg = (13, 8, 12) if fmt == "gg" else (12, 12, 12)
+    hl = HostLayer(rng, d, mid, E, k, fmt="q4cp" if fmt == "q4cp" else "q4k", gg_types=gg, scale_std=0.02,
+                   router_std=0.3, shared_dense=kind)
+    m, dev = hl.to_gpu(max_tokens=300)
+    L = hl.oracle_layer()
+    for T in (1, 7, 32, 300):
+        x = rng.standard_normal((T, d)).astype(np.float32)
+        want, io, _ = oracle.moe_layer(L, x)
+        y = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+        assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max(), (T, np.abs(y - want).max() / np.abs(want).max())
+    m.close()

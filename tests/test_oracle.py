@@ -222,6 +222,36 @@ def test_layer_golden_from_reference_moe(oracle, golden):
         assert (bits(y2[[1, 4]]) == g[f"ybits{i}"][[1, 4]]).all() and np.isnan(y2[0]).all()
 
 
+def test_q8g64_dequant_golden(oracle, golden):
+    """Checkpoint::dequant of the reference on a q8g64 tensor (src/hgn.h:189-202): bit-identical rows."""
+    g = golden("moe_layer.npz")
+    m = oracle.Mat(oracle.Q8G64, g["q8g64_raw"], 5, 192)
+    assert (bits(m.dequant()) == g["q8g64_bits"]).all()
+    assert (bits(m.dequant(2, 2)) == g["q8g64_bits"][2:4]).all()
+    # closed form on hand-made bytes: code * scale + min
+    raw = np.zeros((1, 64 + 4), np.uint8)
+    raw[0, :64] = np.arange(64) * 4
+    raw[0, 64:].view(np.float16)[:] = [0.5, -3.0]
+    w = oracle.Mat(oracle.Q8G64, raw, 1, 64).dequant()
+    assert (w[0] == np.arange(64, dtype=np.float32) * 4 * 0.5 - 3.0).all()
+
+
+def test_q8g64_shared_expert_vs_reference_build(oracle):
+    """The reference's q8g64 matvec sums per 64-group (code . x) * scale + min * sum(x) (src/ref.cpp:91-106), not the
+    dot with the dequantised row: the oracle follows it to the bit."""
+    if oracle.ref() is None:
+        pytest.skip("oracle/_ref not built here")
+    rng = np.random.default_rng(43)
+    d, mid, E, k = 192, 128, 6, 2
+    hl = HostLayer(rng, d, mid, E, k, router_dtype="bf16", scale_std=0.05, router_std=0.3, shared_dense="q8g64")
+    L = hl.oracle_layer()
+    L.shared[3] = oracle.Mat(oracle.BF16, S.f32_to_bf16_bits(hl.shared[3]), 1, d)
+    x = rng.standard_normal((3, d)).astype(np.float32)
+    y, ids, ws = oracle.moe_layer(L, x)
+    for t in range(3):
+        assert (bits(oracle.ref_moe_token(L, x[t])) == bits(y[t])).all()
+
+
 def test_layer_vs_reference_build_random(oracle):
     if oracle.ref() is None:
         pytest.skip("oracle/_ref not built here")
