@@ -97,7 +97,7 @@ def cpu_leg(kind, layer, xs, ids, cnt, m, T, eb, budget=CPU_BUDGET_S):
     return out
 
 
-def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_budget=CPU_BUDGET_S):
+def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_budget=CPU_BUDGET_S, codebook="zp8"):
     import numpy as np
     import torch
     from gfx1151_engine_amd import capi, workloads as W
@@ -112,7 +112,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     T = tokens or {"prefill": 16384 if fmt == "q4cp" else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
     nlayers = nlayers_arg if kind == "stack" else 1
 
-    layers = [W.DeviceLayer(1000 + l, d, mid, E, k, fmt, gg_types=gg_types) for l in range(nlayers)]
+    layers = [W.DeviceLayer(1000 + l, d, mid, E, k, fmt, gg_types=gg_types, codebook=codebook) for l in range(nlayers)]
+    universal = fmt == "q4cp" and codebook == "universal"
     g = torch.Generator(device="cuda")
     g.manual_seed(99)
     extra = {}
@@ -206,7 +207,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
            "vs_baseline": None, "data": "synthetic", "stage_ms": {kk: round(v, 5) for kk, v in stage.items()},
            "stage_event_overhead_ms": round(stage_overhead, 5)}
     cfg = {"workload": wl, "tokens": T, "d_model": d, "moe_mid": mid, "experts": E, "topk": k, "shared_experts": 1,
-           "format": "q4cp g32 zero-point 8" if fmt == "q4cp" else
+           "format": ("q4cp g32, the reference converter's universal expert codebook (table look-up, f32 GEMV kernels)"
+                      if universal else "q4cp g32 zero-point 8") if fmt == "q4cp" else
            ("GGUF Q5_K gate/up, Q8_0 down, Q4_K shared expert (general f32 kernels)" if ggmix else "GGUF Q4_K"),
            "layers": nlayers, **extra}
     if kind == "prefill":
@@ -227,7 +229,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
                                  "achieved": round(up_flop / up_s / 1e12, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": round(up_flop / up_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                                  "timing": "HIP events around the launch (moe_profile_enable), same stream",
-                                 "traffic": None if shared_in_launch else pmc_traffic(kind, fmt, T)}})
+                                 "traffic": None if shared_in_launch or universal else pmc_traffic(kind, fmt, T)}})
         # rows the grouped GEMM computes for the routed pairs: tiles of 128, the last tile of an expert padded
         # to a multiple of 32 rows
         rem = cnt % 128
@@ -245,7 +247,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
             gu_bytes = 2 * mid * (uniq * W.gg_row_bytes(gg_types[0], d) + W.gg_row_bytes(gg_types[2], d))
         up_s = up_marginal_ms * 1e-3
         od = dict(list(LIB_OPTIONS) + list(opts))
-        int_dec = od.get(1, 1) != 0 and not ggmix
+        int_dec = od.get(1, 1) != 0 and not ggmix and not universal  # (a table codebook takes the f32 kernels)
         # the arithmetic of the GEMV kernels: integer dot products of the 4-bit codes with the activations' 4-bit
         # (q4cp: v_dot8_i32_i4, four planes) or 8-bit (Q4_K: v_dot4_i32_i8, two planes) digit planes, f32 scales;
         # or plain f32 FMAs (MOE_OPT_INT_DECODE = 0, and the general GGUF kernels)
@@ -342,6 +344,9 @@ def main():
     ap.add_argument("--opt", action="append", default=[], metavar="ID=VALUE",
                     help="moe_set_option(ID, VALUE) on the context before the run (A/B runs of the library's switches)")
     ap.add_argument("--layers", type=int, default=48, help="stack workload: number of resident layers")
+    ap.add_argument("--codebook", default="zp8", choices=("zp8", "universal"),
+                    help="q4cp workloads: the benchmark's zero-point-8 grid, or the non-uniform 16-entry table that the "
+                         "reference's converter writes into its checkpoints")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (a kernel of known HBM traffic to scale "
@@ -383,7 +388,7 @@ def main():
     elif a.workload in ("load", "q4k_load"):
         res = measure_load("q4k" if a.workload.startswith("q4k") else "q4cp", min(a.steps, 5), min(a.layers, 2))
     else:
-        res = measure(a.workload, a.steps, a.warmup, a.tokens, a.layers, cpu=not a.no_cpu)
+        res = measure(a.workload, a.steps, a.warmup, a.tokens, a.layers, cpu=not a.no_cpu, codebook=a.codebook)
     print(json.dumps(res))
 
 

@@ -459,10 +459,14 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
                        (!sh || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d);
   const bool use_int4k = L.has_gguf && c->int_decode && L.gg.tgu == MOE_GGML_Q4_K && L.gg.tdn == MOE_GGML_Q4_K &&
                          (!sh || L.sh_gguf_type == MOE_GGML_Q4_K) && moe_dec4k_supported(g.d, g.mid, nslots_d);
+  // q4cp codebooks that are not affine (the reference converter's fixed table, trained tables): the same launch
+  // structure with look-up arithmetic
+  const bool use_lut = L.has_q4cp && c->int_decode && !use_int && (!sh || L.sh_gguf_type == 0) &&
+                       moe_dec_supported(g.d, g.mid, nslots_d) && moe_dec_gu_topk_supported(g.experts, g.topk);
   const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min && moe_dec_uq_supported(g.d);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
-  const bool gu_topk = ((use_int && !use_uq) || use_int4k) && moe_dec_gu_topk_supported(g.experts, g.topk);
+  const bool gu_topk = ((use_int && !use_uq) || use_int4k || use_lut) && moe_dec_gu_topk_supported(g.experts, g.topk);
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
          int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
@@ -520,6 +524,17 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
       return stage(MOE_PROF_DOWN, [&]() -> int {
         return moe_launch_dec_dn(&L.down, shd, c->sh_logit, c->hplanes, c->hmeta, c->ids, c->ws, g.id_stride, g.topk, P,
                                  g.d, g.mid, y, (uint64_t)g.d, st);
+      });
+    }
+    if (use_lut) {
+      if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+             return moe_launch_dec_gu_lut(&L.gate_up, shg, shu, x, c->logits, g.experts, c->ids, c->ws, g.id_stride,
+                                          g.topk, P, g.d, g.mid, c->hid32, st);
+           })))
+        return rc;
+      return stage(MOE_PROF_DOWN, [&]() -> int {
+        return moe_launch_dec_dn_lut(&L.down, shd, c->sh_logit, c->hid32, c->ids, c->ws, g.id_stride, g.topk, P, g.d,
+                                     g.mid, y, (uint64_t)g.d, st);
       });
     }
     if ((rc = stage(MOE_PROF_UP, [&]() -> int {

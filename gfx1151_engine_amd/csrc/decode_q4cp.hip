@@ -96,6 +96,58 @@ struct DecW {  // one q4cp tensor's planes
   uint64_t ss;
 };
 
+// ---- codebooks that are not a*n + b (the reference converter's fixed non-uniform table, trained tables): the same
+// kernels with a look-up instead of the integer dots, all in f32 (no quantised activations: the result differs
+// from the f32 GEMV kernels only by the order of the additions).  The 16 codebook entries lie in LDS 32 times
+// side by side (entry n, copy c at dword 32 n + c), so that lane l always reads bank l % 32: no conflicts,
+// whatever the codes are.  A weight costs one bit-field extract, one address operation, one LDS read and one
+// FMA; a lane keeps the 32 activations of the group it is working on in registers.
+constexpr int LUT_DW = 16 * 32;  // dwords per table (2 KB)
+
+struct XF {  // one group's activations
+  float v[32];
+};
+__device__ __forceinline__ void load_xf(XF& x, const float* src) {  // src: global or LDS, 16-byte aligned
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const float4 f = ((const float4*)src)[i];
+    x.v[4 * i] = f.x; x.v[4 * i + 1] = f.y; x.v[4 * i + 2] = f.z; x.v[4 * i + 3] = f.w;
+  }
+}
+// the block fills one table
+__device__ __forceinline__ void build_lut(float* lut, const float* __restrict__ cb) {
+  for (int i = threadIdx.x; i < LUT_DW; i += blockDim.x) lut[i] = cb[i >> 5];
+}
+// sum_k cb[n_k] * x_k over one group (16 code bytes, low nibble = the earlier element); lut_lane = table + (lane & 31)
+__device__ __forceinline__ float lut_dot(const uint4 cw, const XF& x, const float* lut_lane) {
+  const uint32_t w[4] = {cw.x, cw.y, cw.z, cw.w};
+  const uint32_t base = (uint32_t)(uintptr_t)lut_lane;  // LDS byte address of this lane's copy of entry 0
+  float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    // (an opaque copy of the word, pinned between this step's neighbours: otherwise the compiler works out the
+    // addresses of a whole launch's look-ups ahead of the first one and spills hundreds of registers)
+    uint32_t wi = w[i];
+    asm volatile("" : "+v"(wi));
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      // entry n of this lane's copy: base + 128 n, two instructions (left to itself the compiler takes three:
+      // shift, mask, add)
+      uint32_t n_lo, n_hi, a_lo, a_hi;
+      asm("v_bfe_u32 %0, %1, %2, 4" : "=v"(n_lo) : "v"(wi), "n"(4 * j));
+      asm("v_bfe_u32 %0, %1, %2, 4" : "=v"(n_hi) : "v"(wi), "n"(4 * j + 4));
+      asm("v_lshl_add_u32 %0, %1, 7, %2" : "=v"(a_lo) : "v"(n_lo), "v"(base));
+      asm("v_lshl_add_u32 %0, %1, 7, %2" : "=v"(a_hi) : "v"(n_hi), "v"(base));
+      const float t0 = *(const __attribute__((address_space(3))) float*)(uintptr_t)a_lo;
+      const float t1 = *(const __attribute__((address_space(3))) float*)(uintptr_t)a_hi;
+      a0 = fmaf(t0, x.v[8 * i + j], a0);
+      a1 = fmaf(t1, x.v[8 * i + j + 1], a1);
+    }
+    if (i & 1) __builtin_amdgcn_sched_barrier(0);  // sixteen look-ups in flight at a time, not a whole row's
+  }
+  return a0 + a1;
+}
+
 struct GuArgs2 {
   DecW gu;           // fused gate_up [E*2*mid][d]
   DecW shg, shu;     // shared expert gate / up [mid][d] (codes == nullptr: none)
@@ -114,8 +166,10 @@ struct GuArgs2 {
 // ids and weights in every block; cheaper than a last-block ticket in the router launch plus a
 // dependent load of the ids here) and block (0, 0, token) writes ids / weights out for the down
 // kernel.  The shared expert's blocks skip it and have the CU to themselves meanwhile.
+// LUT (not with UQ): table look-up arithmetic (above) for any codebook; xf32 = the tokens' activations [P][d],
+// dynamic LDS = two tables (gate rows', up rows') and the token's d activations, hid goes out as f32 only.
 constexpr int GU2_ROWS = 32;
-template <bool UQ, int NPL>
+template <bool UQ, int NPL, bool LUT>
 __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __restrict__ xplanes,
                                                 const float2* __restrict__ xmeta,
                                                 const int* __restrict__ ids, int id_stride, int kpt, int d,
@@ -124,7 +178,8 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
                                                 const moe_tile* __restrict__ tiles, const int* __restrict__ ntiles,
                                                 const int* __restrict__ tokidx, int n_experts,
                                                 const float* __restrict__ logits, int* __restrict__ ids_out,
-                                                float* __restrict__ ws_out) {
+                                                float* __restrict__ ws_out, const float* __restrict__ xf32) {
+  extern __shared__ float lutmem[];
   __shared__ float gs[GU2_ROWS], us[GU2_ROWS];
   __shared__ uint32_t pk[QV4_GROUP_DW];
   __shared__ int sel_ids[64];
@@ -171,6 +226,19 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   }
   const DecW Wg = shared ? A.shg : A.gu;  // block-uniform choice, by value
   const DecW Wu = shared ? A.shu : A.gu;
+  const float *lutg = lutmem + (lane & 31), *lutu = lutg;
+  if (LUT) {
+    build_lut(lutmem, Wg.cb);
+    if (Wu.cb != Wg.cb) {  // (block-uniform) the shared expert's up_proj is a tensor with a codebook of its own
+      build_lut(lutmem + LUT_DW, Wu.cb);
+      lutu += LUT_DW;
+    }
+    // the token's activations, staged once per block: a lane fetches a group's 32 values when it starts on it
+    const float4* xr = (const float4*)(xf32 + (size_t)blockIdx.z * d);
+    for (int i = threadIdx.x; i < d / 4; i += blockDim.x) ((float4*)(lutmem + 2 * LUT_DW))[i] = xr[i];
+    __syncthreads();
+  }
+  const float* xs = lutmem + 2 * LUT_DW;
   const uint64_t grow0 = shared ? 0 : (uint64_t)e * 2 * mid;
   const uint64_t urow0 = shared ? 0 : (uint64_t)e * 2 * mid + mid;
   const int r0 = blockIdx.x * GU2_ROWS + 4 * wv;  // first of this wave's 4 gate rows
@@ -185,7 +253,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   // the activation planes and codebook constants are requested first: loads return in order, so
   // the dot products of the first row pair can start while the later rows are still in flight
   XG xa, xb;
-  if (!UQ) {
+  if (!LUT && !UQ) {
     const size_t xbase = (size_t)blockIdx.z * G;
     load_xg(xa, xplanes, xmeta, xbase + gA);
     load_xg(xb, xplanes, xmeta, xbase + gB);
@@ -218,6 +286,24 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   }
 
   float acc[8];
+  if (LUT) {
+    // group gA of all eight rows first, then the tail group: one group's activations in registers at a time
+    XF xf;
+    load_xf(xf, xs + (size_t)gA * 32);
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const float* lt = p >= 2 ? lutu : lutg;
+      acc[2 * p] = __half2float(sa[p]) * mA * lut_dot(ca[p], xf, lt);
+      acc[2 * p + 1] = __half2float(sb[p]) * mA * lut_dot(cb[p], xf, lt);
+    }
+    load_xf(xf, xs + (size_t)gB * 32);
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+      const float vt = __half2float(st[p]) * mB * lut_dot(ct[p], xf, p >= 2 ? lutu : lutg);
+      if (lane < 32) acc[2 * p] += vt;
+      else acc[2 * p + 1] += vt;
+    }
+  } else {
 #pragma unroll
   for (int p = 0; p < 4; p++) {
     const float a = p >= 2 ? ua : ga, b = p >= 2 ? ub : gb;
@@ -231,6 +317,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     acc[2 * p] = v0;
     acc[2 * p + 1] = v1;
     __builtin_amdgcn_sched_barrier(0);  // row pair p is finished before the wait for pair p + 1
+  }
   }
 #pragma unroll
   for (int i = 0; i < 8; i++) acc[i] = sum64(acc[i]);
@@ -249,6 +336,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     const float hv = g / (1.f + expf(-g)) * u;
     const size_t slot = UQ ? (size_t)(first + pi) : (size_t)tok * nslots + s;
     if (hid_f32 && lane < 32) hid_f32[slot * mid + blockIdx.x * GU2_ROWS + j] = hv;
+    if (LUT) return;  // (the down kernel of this arithmetic reads hid as f32)
     int p0, p1, p2, p3;
     float q, qsx;
     quant32_lane(hv, p0, p1, p2, p3, q, qsx);
@@ -286,12 +374,16 @@ constexpr int DN2_MAXSLOTS = 16;
 #ifndef MOE_DN_ROWS
 #define MOE_DN_ROWS 6
 #endif
-template <int ROWS>
+// LUT: table look-up arithmetic for any codebook; hid_f32 = [P][slots][mid], dynamic LDS = two tables (the routed
+// experts' tensor, the shared expert's).
+template <int ROWS, bool LUT>
 __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __restrict__ hplanes,
                                                 const float2* __restrict__ hmeta,
                                                 const int* __restrict__ ids, const float* __restrict__ ws,
                                                 int id_stride, int kpt, int d, int mid,
-                                                float* __restrict__ out, uint64_t out_stride) {
+                                                float* __restrict__ out, uint64_t out_stride,
+                                                const float* __restrict__ hid_f32) {
+  extern __shared__ float lutmem[];
   __shared__ float part[DN2_MAXSLOTS][ROWS];
   __shared__ float wsm[DN2_MAXSLOTS];
   const int tok = blockIdx.y;
@@ -301,6 +393,11 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
   const int G = mid / 32, half = lane >> 5;
   const int r0 = blockIdx.x * ROWS;
   const size_t rb = (size_t)mid / 2;
+  if (LUT) {
+    build_lut(lutmem, A.dn.cb);
+    if (has_shared) build_lut(lutmem + LUT_DW, A.shd.cb);
+    __syncthreads();
+  }
   // combine weights of the token, fetched while the weight rows are in flight
   float wmine = 0.f;
   if ((int)threadIdx.x < nslots)
@@ -321,7 +418,10 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
     const uint64_t wss = shared ? A.shd.ss : A.dn.ss;
     const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
     XG x;
-    load_xg(x, hplanes, hmeta, ((size_t)tok * nslots + s) * G + g);
+    XF xh;
+    if (LUT) load_xf(xh, hid_f32 + ((size_t)tok * nslots + s) * mid + (size_t)g * 32);
+    else load_xg(x, hplanes, hmeta, ((size_t)tok * nslots + s) * G + g);
+    const float* lt = lutmem + (shared ? LUT_DW : 0) + (lane & 31);
     const float a = wcb[1] - wcb[0], b = fmaf(8.f, a, wcb[0]);
     const uint64_t row0 = (shared ? 0 : (uint64_t)e * d) + r0;
     const uint8_t* cp = wcodes + row0 * rb + (size_t)g * 16;
@@ -336,7 +436,7 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
     __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first dot product
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
-      float v = __half2float(sc[r]) * m * chunk_dot(cw[r], x, a, b);
+      float v = __half2float(sc[r]) * m * (LUT ? lut_dot(cw[r], xh, lt) : chunk_dot(cw[r], x, a, b));
       v = sum32(v);
       if (g_raw == 0 && s_raw < nslots) part[s_raw][r] = v;
       if ((r & 1) == 1) __builtin_amdgcn_sched_barrier(0);  // rows are consumed in arrival order
@@ -446,8 +546,8 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
-  k_dec_gu<false, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
-                                           nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr);
+  k_dec_gu<false, 0, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
+                                                  nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -465,11 +565,53 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
   A.shu = decw(sh_up);
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);  // + the row of the exact top-k block
   if (n_experts <= 512)
-    k_dec_gu<false, 8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
-                                             hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws);
+    k_dec_gu<false, 8, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
+                                                    hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr);
   else
-    k_dec_gu<false, 16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
-                                              hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws);
+    k_dec_gu<false, 16, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
+                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// The look-up kernels (any codebook): x f32 [P][d] in, hid f32 [P][kpt + shared][mid] out; softmax / top-k inside
+// the launch as above.
+int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up, const float* x,
+                          const float* logits, int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d,
+                          int mid, float* hid_f32, hipStream_t st) {
+  if (!x || !hid_f32 || !logits || !moe_dec_gu_topk_supported(n_experts, kpt)) return MOE_E_INVALID;
+  GuArgs2 A{};
+  A.gu = decw(gu);
+  A.shg = decw(sh_gate);
+  A.shu = decw(sh_up);
+  dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);
+  const int lds = 2 * LUT_DW * 4 + d * 4;
+  if (lds > 64 * 1024) return MOE_E_UNSUPPORTED;
+  if (n_experts <= 512)
+    k_dec_gu<false, 8, true><<<grid, 512, lds, st>>>(A, nullptr, nullptr, nullptr, id_stride, kpt, d, mid, nullptr, nullptr,
+                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x);
+  else
+    k_dec_gu<false, 16, true><<<grid, 512, lds, st>>>(A, nullptr, nullptr, nullptr, id_stride, kpt, d, mid, nullptr, nullptr,
+                                                      hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_dec_dn_lut(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit, const float* hid_f32,
+                          const int* ids, const float* ws, int id_stride, int kpt, int P, int d, int mid, float* out,
+                          uint64_t out_stride, hipStream_t st) {
+  DnArgs2 A{};
+  A.dn = decw(dn);
+  A.shd = decw(sh_down);
+  A.sh_logit = sh_logit;
+  const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
+  constexpr int lds = 2 * LUT_DW * 4;
+  if (d % MOE_DN_ROWS == 0)
+    k_dec_dn<MOE_DN_ROWS, true><<<dim3(d / MOE_DN_ROWS, P), bs, lds, st>>>(A, nullptr, nullptr, ids, ws, id_stride, kpt, d,
+                                                                           mid, out, out_stride, hid_f32);
+  else
+    k_dec_dn<8, true><<<dim3(d / 8, P), bs, lds, st>>>(A, nullptr, nullptr, ids, ws, id_stride, kpt, d, mid, out,
+                                                       out_stride, hid_f32);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -486,8 +628,8 @@ int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const mo
   A.shu = decw(sh_up);
   if (max_tiles <= 0) return MOE_OK;
   dim3 grid(mid / GU2_ROWS, max_tiles);
-  k_dec_gu<true, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
-                                          ntiles, tokidx, n_experts, nullptr, nullptr, nullptr);
+  k_dec_gu<true, 0, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
+                                                 ntiles, tokidx, n_experts, nullptr, nullptr, nullptr, nullptr);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -516,9 +658,9 @@ int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float
   const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
   // MOE_DN_ROWS rows per block where that divides d (d = 3072: 512 blocks, two per CU), else 8
   if (d % MOE_DN_ROWS == 0)
-    k_dec_dn<MOE_DN_ROWS><<<dim3(d / MOE_DN_ROWS, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
+    k_dec_dn<MOE_DN_ROWS, false><<<dim3(d / MOE_DN_ROWS, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride, nullptr);
   else
-    k_dec_dn<8><<<dim3(d / 8, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
+    k_dec_dn<8, false><<<dim3(d / 8, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride, nullptr);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -115,6 +115,10 @@ __device__ __forceinline__ int q4k_pos(int c) {
   return 8 * w + ((r & 1) << 2) + ((c >> 5) << 1) + (r >> 1);
 }
 
+__device__ __forceinline__ void mfma16(floatx16& acc, const half8& a, const half8& b) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc, 0, 0, 0);
+}
+
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 // 64 lanes x 16 B: global (per-lane address) -> LDS (wave-uniform base, lane l lands at base + 16 l)
 __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
@@ -446,7 +450,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
       for (int i = 0; i < NM; i++) {
         const int mf = i / NF, nf = i % NF;
-        acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[cur][mf], b[cur][nf].v, acc[mf][nf], 0, 0, 0);
+        mfma16(acc[mf][nf], a[cur][mf], b[cur][nf].v);
         __builtin_amdgcn_sched_barrier(0);
         if (i < MF) load_a1(q + 1, i, a[nxt]);
 #pragma unroll
@@ -474,7 +478,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
     for (int i = 0; i < NM; i++) {
       const int mf = i / NF, nf = i % NF;
-      acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[1][mf], b[1][nf].v, acc[mf][nf], 0, 0, 0);
+      mfma16(acc[mf][nf], a[1][mf], b[1][nf].v);
       __builtin_amdgcn_sched_barrier(0);
       // (past the last stage this reads stale LDS and the result is never used)
       if (i == 0) load_codes(s + 1);

@@ -93,6 +93,12 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
                       hipStream_t st);
+int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up, const float* x,
+                          const float* logits, int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d,
+                          int mid, float* hid_f32, hipStream_t st);
+int moe_launch_dec_dn_lut(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit, const float* hid_f32,
+                          const int* ids, const float* ws, int id_stride, int kpt, int P, int d, int mid, float* out,
+                          uint64_t out_stride, hipStream_t st);
 int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                          const uint32_t* xplanes, const float2* xmeta, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, const int* tokidx, int n_experts, int d, int mid, uint32_t* hplanes,

@@ -19,6 +19,12 @@ def q4cp_blob_bytes(rows, cols):
     return 64 + rows * cols // 2 + rows * q4cp_scale_stride(cols)
 
 
+# The 16-entry table the reference's converter writes into every routed-expert tensor unless told otherwise
+# (tools/flashnext2hgn.py:530-531, UNIVERSAL_EXPERT_CB): sorted, symmetric, not an affine function of the code.
+_UCB_HALF = (0.042080, 0.128362, 0.220943, 0.324402, 0.444132, 0.587296, 0.765293, 1.0)
+UNIVERSAL_CODEBOOK = np.array([-v for v in _UCB_HALF[::-1]] + list(_UCB_HALF), np.float32)
+
+
 def make_q4cp(rng, rows, cols, codebook=None, scale_std=0.01, scales=None, codes=None):
     """Random q4cp blob. scales: fp16 |N(0,1)|*scale_std unless given ([rows][cols/32] float16)."""
     assert cols % 32 == 0

@@ -16,12 +16,14 @@ def _gen(seed):
     return g
 
 
-def q4cp_blob(g, rows, cols, scale_std=0.01):
-    """uint8 tensor [64 + rows*cols/2 + rows*ss]: zero-point-8 codebook, uniform codes, fp16 |N|*std scales."""
+def q4cp_blob(g, rows, cols, scale_std=0.01, codebook=None):
+    """uint8 tensor [64 + rows*cols/2 + rows*ss]: zero-point-8 codebook (or the 16 floats given), uniform codes,
+    fp16 |N|*std scales."""
     ss = S.q4cp_scale_stride(cols)
     nb = rows * cols // 2
     blob = torch.empty(64 + nb + rows * ss, dtype=torch.uint8, device="cuda")
-    blob[:64] = torch.from_numpy(S.ZP8_CODEBOOK.view(np.uint8).copy()).cuda()
+    cb = S.ZP8_CODEBOOK if codebook is None else np.ascontiguousarray(codebook, np.float32)
+    blob[:64] = torch.from_numpy(cb.view(np.uint8).copy()).cuda()
     step = 1 << 28
     for i in range(0, nb, step):
         n = min(step, nb - i)
@@ -94,9 +96,12 @@ def gg_rows(g, t, rows, cols, scale_std=0.01):
 
 class DeviceLayer:
     """One layer's weights in HBM + registration into a capi.Moe context.
-    fmt "q4k": raw GGUF blocks, gg_types = ggml types of (gate/up, down, shared expert)."""
+    fmt "q4k": raw GGUF blocks, gg_types = ggml types of (gate/up, down, shared expert).
+    codebook (q4cp): "zp8" = the zero-point-8 grid cb[n] = n - 8; "universal" = the fixed non-uniform table of the
+    reference's converter (scales 8.4 times larger, so that the weights keep their size)."""
 
-    def __init__(self, seed, d=3072, mid=768, E=512, k=10, fmt="q4cp", bias=None, gg_types=(12, 12, 12)):
+    def __init__(self, seed, d=3072, mid=768, E=512, k=10, fmt="q4cp", bias=None, gg_types=(12, 12, 12),
+                 codebook="zp8"):
         g = _gen(seed)
         self.d, self.mid, self.E, self.k, self.fmt = d, mid, E, k, fmt
         self.tgu, self.tdn, self.tsh = gg_types
@@ -104,9 +109,10 @@ class DeviceLayer:
         self.sh_sg = torch.randn((1, d), device="cuda", generator=g) * 0.02
         self.bias = bias
         if fmt == "q4cp":
-            self.gate_up = q4cp_blob(g, E * 2 * mid, d)
-            self.down = q4cp_blob(g, E * d, mid)
-            self.sh = [q4cp_blob(g, mid, d), q4cp_blob(g, mid, d), q4cp_blob(g, d, mid)]
+            cb, sd = (S.UNIVERSAL_CODEBOOK, 0.084) if codebook == "universal" else (None, 0.01)
+            self.gate_up = q4cp_blob(g, E * 2 * mid, d, sd, cb)
+            self.down = q4cp_blob(g, E * d, mid, sd, cb)
+            self.sh = [q4cp_blob(g, mid, d, sd, cb), q4cp_blob(g, mid, d, sd, cb), q4cp_blob(g, d, mid, sd, cb)]
         else:
             self.gate = gg_rows(g, self.tgu, E * mid, d)
             self.up = gg_rows(g, self.tgu, E * mid, d)

@@ -6,6 +6,8 @@ import zlib
 import numpy as np
 import pytest
 
+from gfx1151_engine_amd import synth as S
+
 from helpers import HostLayer, bits, max_abs_rel
 
 pytestmark = pytest.mark.gpu
@@ -51,6 +53,39 @@ def test_small_batch_layer(oracle, fmt, d, mid, E, k, T, cb):
     assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
     assert np.abs(ws[:, :k] - wo[:, :k]).max() <= 1e-6
     assert max_abs_rel(y, yo) <= tol_small(fmt), max_abs_rel(y, yo)
+
+
+TOL_LUT = 2e-5  # look-up kernels for codebooks that are not a*n + b: f32 throughout (f32 sums against the
+                # reference's fp64 ones; the order of the additions is the only difference from the f32 GEMV kernels)
+
+
+@pytest.mark.parametrize("T", [1, 2, 11, 20, 32])
+@pytest.mark.parametrize("kind", ["universal", "random"])
+def test_small_batch_table_codebooks(oracle, T, kind):
+    """The reference converter's fixed non-uniform table (tools/flashnext2hgn.py:530-531) in every routed-expert
+    tensor, and a table of its own in each of the shared expert's tensors (:164-187): the look-up decode kernels
+    against the oracle, and the plain f32 kernels (MOE_OPT_INT_DECODE = 0) as a second opinion."""
+    import torch
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(500 + T)
+    d, mid, E, k = 3072, 768, 24, 10
+    cb = S.UNIVERSAL_CODEBOOK if kind == "universal" else np.sort(rng.standard_normal(16)).astype(np.float32)
+    scb = [np.sort(rng.standard_normal(16)).astype(np.float32) * (0.5 + i) for i in range(3)]
+    hl = HostLayer(rng, d, mid, E, k, codebook=cb, shared_codebooks=scb, scale_std=0.05)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    x[0] *= 300.0  # (each 32-group of activations is rescaled by a power of two on its way to f16)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=32)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    ids, ws = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    assert np.abs(ws.cpu().numpy()[:, :k] - wo[:, :k]).max() <= 1e-6
+    err = max(max_abs_rel(y[t], yo[t]) for t in range(T))  # per token: token 0 is 300 times larger
+    assert err <= TOL_LUT, err
+    m.set_option(capi.OPT_INT_DECODE, 0)
+    y2 = m.forward(0, gpu(x)).cpu().numpy()
+    assert max(max_abs_rel(y2[t], yo[t]) for t in range(T)) <= TOL_GEMV
+    m.close()
 
 
 @pytest.mark.parametrize("fmt,T,rdt", [("q4cp", 3, "f32"), ("q4cp", 32, "f32"), ("q4k", 27, "f32"), ("q4k", 2, "f32"),
