@@ -385,6 +385,10 @@ def main():
         sub("stack48_T1", "stack", 16, 2)
         sub("q4k_prefill_T8192", "q4k_prefill", a.steps, a.warmup)
         sub("q4k_decode_T1", "q4k_decode", nd, wd)
+        # the same q4cp shapes with the 16-entry table of the reference's converter (not affine: the grouped GEMM
+        # dequantises through a table, the decode kernels look codes up instead of taking integer dots)
+        sub("universal_codebook_prefill_T16384", "prefill", a.steps, a.warmup, codebook="universal")
+        sub("universal_codebook_decode_T1", "decode", nd, wd, codebook="universal")
     elif a.workload in ("load", "q4k_load"):
         res = measure_load("q4k" if a.workload.startswith("q4k") else "q4cp", min(a.steps, 5), min(a.layers, 2))
     else:
