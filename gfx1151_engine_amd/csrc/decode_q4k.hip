@@ -74,6 +74,17 @@ __device__ __forceinline__ void k4_pair(const uint4 hd, int jj, float& a0, float
   b1 = dmin * (float)m1;
 }
 
+// The four lanes that work on one super-block (a quad: units 4b .. 4b+3) each load one dword of its 16-byte
+// header and hand the others theirs when the row is computed: 1 register per row in flight instead of 4.
+__device__ __forceinline__ uint4 quad_header(uint32_t mine) {
+  uint4 hd;
+  hd.x = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0x00, 0xf, 0xf, true);  // quad_perm [0,0,0,0]
+  hd.y = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0x55, 0xf, 0xf, true);  // [1,1,1,1]
+  hd.z = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xAA, 0xf, 0xf, true);  // [2,2,2,2]
+  hd.w = (uint32_t)__builtin_amdgcn_mov_dpp((int)mine, 0xFF, 0xf, 0xf, true);  // [3,3,3,3]
+  return hd;
+}
+
 // one unit of one row: c0, c1 = its 32 code bytes, hd = the super-block header
 __device__ __forceinline__ float unit_dot(const uint4 c0, const uint4 c1, const uint4 hd, int jj, const XU& x) {
   const uint32_t w[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
@@ -101,13 +112,15 @@ struct Gu4kArgs {
 
 // grid (mid/32, slots incl. shared, P); block 512.  Wave w: gate rows 4w..4w+3 and the matching up
 // rows of this block's 32; lane = unit (d/64 <= 64 units per row).  All 24 loads of a lane (8 rows x
-// two code halves + header) are in flight together.
+// two code halves + its dword of the header) are in flight together, in under 128 registers: two blocks fit
+// a CU, so the grid's 265 blocks are all resident at once (with one block per CU the last nine waited for a
+// second round).
 // NPL > 0 (E <= 64*NPL): only the logits are given; the blocks of the routed slots run the softmax /
 // top-k of their token themselves and block (0, 0, token) writes ids / weights out for the down
 // kernel (as in the q4cp gate/up kernel).
 constexpr int G4_ROWS = 32;
 template <int NPL>
-__global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t* __restrict__ xplanes,
+__global__ void __launch_bounds__(512, 4) k_dec4k_gu(Gu4kArgs A, const uint32_t* __restrict__ xplanes,
                                                      const float2* __restrict__ xmeta,
                                                      const int* __restrict__ ids, int id_stride, int kpt, int d,
                                                      int mid, uint32_t* __restrict__ hplanes,
@@ -153,19 +166,21 @@ __global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t*
   const uint8_t* gbase = shared ? A.sh_gate : A.gate + (uint64_t)e * mid * rb;
   const uint8_t* ubase = shared ? A.sh_up : A.up + (uint64_t)e * mid * rb;
   const int r0 = blockIdx.x * G4_ROWS + 4 * wv;
-  // branch-free loads: lanes past the row's units read unit 0 and count as zero
+  // branch-free loads: lanes past the row's units read a unit of the first super-block (their quad then still
+  // assembles a real header) and count as zero
   const bool live = lane < U;
-  const int ul = live ? lane : 0;
+  const int ul = live ? lane : (lane & 3);
   const float mlive = live ? 1.f : 0.f;
   const int jj = ul & 3;
   const size_t uoff = (size_t)(ul >> 2) * 144;  // this lane's super-block inside a row
   XU x;
   load_xu(x, xplanes, xmeta, ((size_t)tok * U + ul) * 2);
-  uint4 c0[8], c1[8], hd[8];
+  uint4 c0[8], c1[8];
+  uint32_t hw[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
     const uint8_t* row = (i < 4 ? gbase : ubase) + (uint64_t)(r0 + (i & 3)) * rb + uoff;
-    hd[i] = *(const uint4*)row;
+    hw[i] = *(const uint32_t*)(row + 4 * jj);
     c0[i] = *(const uint4*)(row + 16 + jj * 32);
     c1[i] = *(const uint4*)(row + 32 + jj * 32);
   }
@@ -173,7 +188,7 @@ __global__ void __launch_bounds__(512, 2) k_dec4k_gu(Gu4kArgs A, const uint32_t*
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; i++) {
-    acc[i] = sum64(unit_dot(c0[i], c1[i], hd[i], jj, x) * mlive);
+    acc[i] = sum64(unit_dot(c0[i], c1[i], quad_header(hw[i]), jj, x) * mlive);
     if (i & 1) __builtin_amdgcn_sched_barrier(0);  // rows are consumed in arrival order
   }
   if (lane == 0) {
