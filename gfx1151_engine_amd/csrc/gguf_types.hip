@@ -162,6 +162,8 @@ __device__ __forceinline__ float wave_sum_f(float v) {
 // Activations sit in LDS with one float of padding per 32 (element i at GX_PAD(i)): lanes work on different
 // 32-element blocks at the same offset, which without the padding is the same bank for every lane.
 #define GX_PAD(i) ((i) + ((i) >> 5))
+constexpr int GX_PITCH = 33;  // floats per 32-element block in LDS
+                              // (128-bit reads at a pitch of 36 floats were measured: no faster, and the 32 extra registers cost occupancy)
 
 // four bits b0..b3 of x to bit 0 of bytes 0..3
 __device__ __forceinline__ uint32_t spread4(uint32_t x) { return ((x & 0xFu) * 0x00204081u) & 0x01010101u; }
@@ -241,12 +243,57 @@ __device__ __forceinline__ float gg_unit_dot(int t, const uint8_t* row, int b, c
   }
   return a * sq + c * sx;
 }
-__device__ __forceinline__ float gg_row_dot(int t, const uint8_t* row, const float* x, const float* xsum, int K,
-                                            int lane) {
-  float acc = 0.f;
-  for (int b = lane; b < K / 32; b += 64) acc += gg_unit_dot(t, row, b, x + 33 * b, xsum[b]);
-  return wave_sum_f(acc);
+// Gate and up row of one wave against x: the block type is a compile-time constant here and the loop body is
+// straight-line code over two blocks per lane and row (lanes past the row work on block 0 and count as zero: no
+// load sits under a branch), so the compiler issues the four blocks' loads together instead of one memory
+// round trip after the other.
+template <int T>
+__device__ __forceinline__ void gg_rowpair_dot(const uint8_t* grow, const uint8_t* urow, const float* x,
+                                               const float* xsum, int K, int lane, float& g, float& u) {
+  const int nb = K / 32;
+  float ag = 0.f, au = 0.f;
+  for (int base = 0; base < nb; base += 128) {
+    const int r0 = base + lane, r1 = base + 64 + lane;
+    const int b0 = r0 < nb ? r0 : 0, b1 = r1 < nb ? r1 : 0;
+    const float m0 = r0 < nb ? 1.f : 0.f, m1 = r1 < nb ? 1.f : 0.f;
+    const float g0 = gg_unit_dot(T, grow, b0, x + GX_PITCH * b0, xsum[b0]);
+    const float u0 = gg_unit_dot(T, urow, b0, x + GX_PITCH * b0, xsum[b0]);
+    const float g1 = gg_unit_dot(T, grow, b1, x + GX_PITCH * b1, xsum[b1]);
+    const float u1 = gg_unit_dot(T, urow, b1, x + GX_PITCH * b1, xsum[b1]);
+    ag += m0 * g0 + m1 * g1;
+    au += m0 * u0 + m1 * u1;
+  }
+  g = wave_sum_f(ag);
+  u = wave_sum_f(au);
 }
+// the same for GG_DN_UNITS (slot, block) units of one output row of the down projection; unit = base + lane + 64 i
+constexpr int GG_DN_UNITS = 2;  // (four at a time need more than 170 registers: fewer waves per CU, slower)
+template <int T>
+__device__ __forceinline__ float gg_down_units(const uint8_t* down, uint64_t rb, const int* eid, const float* wgt,
+                                               int d, int r, int nb, int nunits, int base, int lane, const float* hs,
+                                               const float* hsum) {
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < GG_DN_UNITS; i++) {
+    const int uraw = base + lane + 64 * i;
+    const bool ok = uraw < nunits;
+    const int un = ok ? uraw : 0;
+    const int s = un / nb, b = un - s * nb;
+    const uint8_t* row = down + ((uint64_t)eid[s] * d + r) * rb;
+    acc += (ok ? wgt[s] : 0.f) * gg_unit_dot(T, row, b, hs + GX_PITCH * un, hsum[un]);
+  }
+  return acc;
+}
+// dispatch on a block-uniform type: one scalar branch outside the loads
+#define GG_TYPE_SWITCH(t, CALL)                                   \
+  switch (t) {                                                    \
+    case MOE_GGML_Q4_K: { constexpr int T = MOE_GGML_Q4_K; CALL; } break;   \
+    case MOE_GGML_Q5_K: { constexpr int T = MOE_GGML_Q5_K; CALL; } break;   \
+    case MOE_GGML_Q8_0: { constexpr int T = MOE_GGML_Q8_0; CALL; } break;   \
+    case MOE_GGML_Q5_1: { constexpr int T = MOE_GGML_Q5_1; CALL; } break;   \
+    case MOE_GGML_IQ4_NL: { constexpr int T = MOE_GGML_IQ4_NL; CALL; } break; \
+    default: { constexpr int T = MOE_GGML_IQ4_XS; CALL; } break;            \
+  }
 
 struct GgxArgs {
   const uint8_t *gate, *up, *down;           // routed experts [E][rows][row bytes]
@@ -255,19 +302,27 @@ struct GgxArgs {
   const float* sh_logit;
 };
 
-constexpr int GX_ROWS = 8;      // gate rows per block of k_ggx_gu (a wave takes every fourth)
+#ifndef MOE_GX_ROWS
+#define MOE_GX_ROWS 8
+#endif
+#ifndef MOE_GX_THREADS
+#define MOE_GX_THREADS 256
+#endif
+constexpr int GX_ROWS = MOE_GX_ROWS;        // gate rows per block of k_ggx_gu (16 measured the same; 32 rows in 256 or 512 threads 1.5x slower:
+                                            // a wave's row pairs are sequential memory round trips)
+constexpr int GX_THREADS = MOE_GX_THREADS;  // its block size (a wave takes every GX_THREADS/64-th row)
 constexpr int GX_DN_ROWS = 4;   // output rows per block of k_ggx_dn: one per wave, d / 4 blocks fill the chip
-// grid (ceil(mid/GX_ROWS), slots incl. shared, P), block 256: hid[token][slot][row] = silu(gate.x) * (up.x)
-__global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restrict__ x, const int* __restrict__ ids,
+// grid (ceil(mid/GX_ROWS), slots incl. shared, P), block GX_THREADS: hid[token][slot][row] = silu(gate.x) * (up.x)
+__global__ void __launch_bounds__(GX_THREADS) k_ggx_gu(GgxArgs A, const float* __restrict__ x, const int* __restrict__ ids,
                                                 int id_stride, int kpt, int d, int mid, float* __restrict__ hid) {
   extern __shared__ float xs[];
   const int s = blockIdx.y, tok = blockIdx.z;
   for (int i = threadIdx.x; i < d; i += blockDim.x) xs[GX_PAD(i)] = x[(size_t)tok * d + i];
   __syncthreads();
-  float* xsum = xs + d / 32 * 33;  // per-block sums of the activations, behind the padded activations
+  float* xsum = xs + d / 32 * GX_PITCH;  // per-block sums of the activations, behind the padded activations
   for (int b = threadIdx.x; b < d / 32; b += blockDim.x) {
     float sx = 0.f;
-    for (int l = 0; l < 32; l++) sx += xs[33 * b + l];
+    for (int l = 0; l < 32; l++) sx += xs[GX_PITCH * b + l];
     xsum[b] = sx;
   }
   __syncthreads();
@@ -279,11 +334,11 @@ __global__ void __launch_bounds__(256) k_ggx_gu(GgxArgs A, const float* __restri
   const uint8_t* ubase = shared ? A.sh_up : A.up + e * mid * rb;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   float* ho = hid + ((size_t)tok * gridDim.y + s) * mid;
-  for (int rr = wv; rr < GX_ROWS; rr += 4) {
+  for (int rr = wv; rr < GX_ROWS; rr += GX_THREADS / 64) {
     const int r = blockIdx.x * GX_ROWS + rr;
     if (r >= mid) break;  // wave-uniform
-    const float g = gg_row_dot(t, gbase + (uint64_t)r * rb, xs, xsum, d, lane);
-    const float u = gg_row_dot(t, ubase + (uint64_t)r * rb, xs, xsum, d, lane);
+    float g, u;
+    GG_TYPE_SWITCH(t, gg_rowpair_dot<T>(gbase + (uint64_t)r * rb, ubase + (uint64_t)r * rb, xs, xsum, d, lane, g, u));
     if (lane == 0) ho[r] = silu_f(g) * u;
   }
 }
@@ -306,10 +361,10 @@ __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restri
     wgt[s] = s < kpt ? ws[(size_t)tok * id_stride + s] : sigmoid_f(A.sh_logit[tok]);
   }
   __syncthreads();
-  float* hsum = hs + nslots * mid / 32 * 33;  // per-block sums, behind the padded activations
+  float* hsum = hs + nslots * mid / 32 * GX_PITCH;  // per-block sums, behind the padded activations
   for (int b = threadIdx.x; b < nslots * mid / 32; b += blockDim.x) {
     float sx = 0.f;
-    for (int l = 0; l < 32; l++) sx += hs[33 * b + l];
+    for (int l = 0; l < 32; l++) sx += hs[GX_PITCH * b + l];
     hsum[b] = sx;
   }
   __syncthreads();
@@ -321,13 +376,19 @@ __global__ void __launch_bounds__(256) k_ggx_dn(GgxArgs A, const float* __restri
     const int r = blockIdx.x * GX_DN_ROWS + rr;
     if (r >= d) break;
     float acc = 0.f;
-    for (int u = lane; u < nslots * nb; u += 64) {
-      const int s = u / nb, b = u - s * nb;
-      const bool sh = has_shared && s == nslots - 1;
-      const int t = sh ? A.tsh : A.tdn;
-      const uint64_t rb = gg_row_bytes(t, mid);
-      const uint8_t* row = sh ? A.sh_down + (uint64_t)r * rb : A.down + ((uint64_t)eid[s] * d + r) * rb;
-      acc += wgt[s] * gg_unit_dot(t, row, b, hs + 33 * (s * nb + b), hsum[s * nb + b]);
+    {  // routed slots: one block type, GG_DN_UNITS units per lane and pass with all their loads in flight together
+      const uint64_t rb = gg_row_bytes(A.tdn, mid);
+      for (int base = 0; base < kpt * nb; base += 64 * GG_DN_UNITS)
+        GG_TYPE_SWITCH(A.tdn, acc += gg_down_units<T>(A.down, rb, eid, wgt, d, r, nb, kpt * nb, base, lane, hs, hsum));
+    }
+    if (has_shared) {  // the shared expert's row: its own type; eid[kpt] = 0 and its rows start at sh_down
+      const uint64_t rb = gg_row_bytes(A.tsh, mid);
+      for (int base = 0; base < nb; base += 64 * GG_DN_UNITS) {
+        float v = 0.f;
+        GG_TYPE_SWITCH(A.tsh, v = gg_down_units<T>(A.sh_down, rb, eid + kpt, wgt + kpt, d, r, nb, nb, base, lane,
+                                                   hs + GX_PITCH * (kpt * nb), hsum + kpt * nb));
+        acc += v;
+      }
     }
     acc = wave_sum_f(acc);
     if (lane == 0) out[(size_t)tok * d + r] = acc;
@@ -529,7 +590,7 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
     return MOE_E_INVALID;
   const int nslots = kpt + (sh ? 1 : 0);
   // LDS: the activations with one float of padding and one block sum per 32
-  if (nslots > 16 || (size_t)d / 32 * 34 * 4 > 60 * 1024 || (size_t)nslots * mid / 32 * 34 * 4 > 60 * 1024)
+  if (nslots > 16 || (size_t)d / 32 * (GX_PITCH + 1) * 4 > 60 * 1024 || (size_t)nslots * mid / 32 * (GX_PITCH + 1) * 4 > 60 * 1024)
     return MOE_E_UNSUPPORTED;
   if (P == 0) return MOE_OK;
   GgxArgs A{};
@@ -539,12 +600,12 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
   A.sh_logit = sh_logit;
   if (phase != 2) {
     dim3 grid((mid + GX_ROWS - 1) / GX_ROWS, nslots, P);
-    k_ggx_gu<<<grid, 256, (size_t)d / 32 * 34 * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
+    k_ggx_gu<<<grid, GX_THREADS, (size_t)d / 32 * (GX_PITCH + 1) * 4, st>>>(A, x, ids, id_stride, kpt, d, mid, hid);
     MOE_LAUNCH_CHECK();
   }
   if (phase != 1) {
     dim3 grid((d + GX_DN_ROWS - 1) / GX_DN_ROWS, P);
-    k_ggx_dn<<<grid, 256, (size_t)nslots * mid / 32 * 34 * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
+    k_ggx_dn<<<grid, 256, (size_t)nslots * mid / 32 * (GX_PITCH + 1) * 4, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out);
     MOE_LAUNCH_CHECK();
   }
   return MOE_OK;
