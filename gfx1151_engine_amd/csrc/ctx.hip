@@ -461,7 +461,9 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
                          (!sh || L.sh_gguf_type == MOE_GGML_Q4_K) && moe_dec4k_supported(g.d, g.mid, nslots_d);
   // q4cp codebooks that are not affine (the reference converter's fixed table, trained tables): the same launch
   // structure with look-up arithmetic
-  const bool use_lut = L.has_q4cp && c->int_decode && !use_int && (!sh || L.sh_gguf_type == 0) &&
+  // (up to 5 tokens: 65 / 107 us against 78 / 119 for the plain f32 kernels at 2 / 4 tokens, but 163 against 141 at 8 --
+  // the look-up kernels win on latency, not on throughput)
+  const bool use_lut = L.has_q4cp && c->int_decode && !use_int && P <= 5 && (!sh || L.sh_gguf_type == 0) &&
                        moe_dec_supported(g.d, g.mid, nslots_d) && moe_dec_gu_topk_supported(g.experts, g.topk);
   const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min && moe_dec_uq_supported(g.d);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the

@@ -59,7 +59,7 @@ TOL_LUT = 2e-5  # look-up kernels for codebooks that are not a*n + b: f32 throug
                 # reference's fp64 ones; the order of the additions is the only difference from the f32 GEMV kernels)
 
 
-@pytest.mark.parametrize("T", [1, 2, 11, 20, 32])
+@pytest.mark.parametrize("T", [1, 2, 5, 6, 20, 32])
 @pytest.mark.parametrize("kind", ["universal", "random"])
 def test_small_batch_table_codebooks(oracle, T, kind):
     """The reference converter's fixed non-uniform table (tools/flashnext2hgn.py:530-531) in every routed-expert
@@ -81,7 +81,7 @@ def test_small_batch_table_codebooks(oracle, T, kind):
     assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
     assert np.abs(ws.cpu().numpy()[:, :k] - wo[:, :k]).max() <= 1e-6
     err = max(max_abs_rel(y[t], yo[t]) for t in range(T))  # per token: token 0 is 300 times larger
-    assert err <= TOL_LUT, err
+    assert err <= TOL_LUT, err  # (up to 5 tokens the look-up kernels, beyond that the plain f32 kernels)
     m.set_option(capi.OPT_INT_DECODE, 0)
     y2 = m.forward(0, gpu(x)).cpu().numpy()
     assert max(max_abs_rel(y2[t], yo[t]) for t in range(T)) <= TOL_GEMV
