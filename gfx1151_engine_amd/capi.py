@@ -10,7 +10,7 @@ import torch
 
 from .build import LIB
 
-F32, BF16, Q4CP, Q8G64 = 1, 0, 5, 7
+F32, BF16, Q4CP, Q8G64, Q8G32 = 1, 0, 5, 7, 8
 GGML_Q4_K = 12
 GGML_Q5_K, GGML_Q5_1, GGML_Q8_0 = 13, 7, 8
 
@@ -421,6 +421,14 @@ class ModelFile:
 
     def set_option(self, option, value):
         check(lib().moe_file_set_option(self.h, option, value), "moe_file_set_option")
+
+    def add_overlay(self, path):
+        """True if the overlay file was applied, False if it was left out (already mapped / would replace v2 tensors)."""
+        rc = lib().moe_file_add_overlay(self.h, str(path).encode())
+        if rc == -3:
+            return False
+        check(rc, f"moe_file_add_overlay({path})")
+        return True
 
     def config(self, layer=0):
         cfg = Config()

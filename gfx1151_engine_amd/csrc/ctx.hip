@@ -331,7 +331,7 @@ static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gat
   auto deq = [&](const moe_wview* w, uint64_t row, float* dst) -> int {
     const int t = w == down ? tdn : tgu;
     if (moe_is_dense_type(t))
-      return moe_dense_dequant_row(t, w->data + row * moe_dense_row_bytes(t, w->cols), (int)w->cols, dst, nullptr);
+      return moe_dense_dequant_row(t, w->data, w->rows, (int)w->cols, row, dst, nullptr);
     if (t) return moe_gg_dequant_rows(t, w->data + row * moe_gg_row_bytes(t, w->cols), 1, w->cols, dst, nullptr);
     return moe_q4cp_dequant_rows(w->data, w->rows, w->cols, row, 1, dst, nullptr);
   };

@@ -477,7 +477,8 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
     uint8_t* dst = Bs + buf * GG_TILE_BYTES + brow * GG_PITCH + half * 64;
     if (moe_is_dense_type(G.type)) {
       float w[32];
-      moe_dense_block(G.type, wrow, K, 2 * s + half, w);
+      // (dense storage is the shared expert's: one matrix of M rows, e = 0; the planar q8g32 form needs the row count)
+      moe_dense_block(G.type, wbase, (uint64_t)M, K, (uint64_t)e * M + wr, 2 * s + half, w);
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         gg_half8 v;

@@ -132,7 +132,7 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
 bool moe_dense_shared_supported(int type, int d, int mid);
 int moe_launch_dense_shared_small(int type, const uint8_t* g, const uint8_t* u, const uint8_t* dn, const float* sh_logit,
                                   const float* x, int P, int d, int mid, float* hid, float* y, hipStream_t st);
-int moe_dense_dequant_row(int type, const uint8_t* row, int K, float* out, hipStream_t st);
+int moe_dense_dequant_row(int type, const uint8_t* base, uint64_t nrows, int K, uint64_t r, float* out, hipStream_t st);
 bool moe_gg_types_supported(int tgu, int tdn, int d, int mid);
 uint64_t moe_gg_row_bytes(int type, uint64_t k);
 int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gate, const uint8_t* up,

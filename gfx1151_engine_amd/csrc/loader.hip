@@ -102,11 +102,17 @@ uint32_t gguf_scalar_bytes(uint32_t t) {
 
 }  // namespace
 
-struct moe_file {
-  int format = 0;
+struct FMap {  // one mapped file: the base file, a GGUF shard or an .hgn overlay
   int fd = -1;
   const uint8_t* base = nullptr;
   size_t len = 0;
+  dev_t dev = 0;
+  ino_t ino = 0;
+};
+
+struct moe_file {
+  int format = 0;
+  std::vector<FMap> maps;
   std::unordered_map<std::string, FTensor> idx;
   std::unordered_map<std::string, int64_t> kv_int;  // GGUF integer metadata
   bool gguf_keep_f32 = false;  // MOE_FILE_OPT_GGUF_F32_ROUTER
@@ -121,30 +127,54 @@ struct moe_weights {
   std::shared_ptr<Stager> stager;  // pinned staging buffers, kept for the duration of one moe_load_layers call
 };
 
-static int parse_hgn(moe_file* f) {
-  if (f->len < sizeof(HgnHeader)) return MOE_E_INVALID;
+// hgn v2 dtypes (ht, i4r, q6g64): an overlay must not replace tensors stored that way (src/hgn.h:292)
+static bool hgn_v2_dtype(int dt) { return dt == 16 || dt == 23 || dt == 24; }
+
+// Indexes the tensors of one mapped HGN1 file.  Base file: the first record of a name wins.  Overlay
+// (hgn::Checkpoint::add_overlay, src/hgn.h:108-121,348-362): its tensors replace those of the same name, unless
+// one of them would replace an hgn v2 tensor -- then the whole file is left out (*skipped = true).
+static int parse_hgn(moe_file* f, const FMap& m, bool overlay, bool* skipped) {
+  if (m.len < sizeof(HgnHeader)) return MOE_E_INVALID;
   HgnHeader h;
-  memcpy(&h, f->base, sizeof h);
-  if (h.file_size != f->len) return MOE_E_INVALID;  // the reference rejects a size mismatch too
-  if (h.records_offset > f->len || (uint64_t)h.tensor_count * sizeof(HgnRecord) > f->len - h.records_offset)
+  memcpy(&h, m.base, sizeof h);
+  if (memcmp(h.magic, "HGN1", 4) != 0) return MOE_E_UNSUPPORTED;
+  if (h.file_size != m.len) return MOE_E_INVALID;  // the reference rejects a size mismatch too
+  if (h.records_offset > m.len || (uint64_t)h.tensor_count * sizeof(HgnRecord) > m.len - h.records_offset)
     return MOE_E_INVALID;
+  std::vector<std::pair<std::string, FTensor>> ts;
+  ts.reserve(h.tensor_count);
   for (uint32_t i = 0; i < h.tensor_count; i++) {
     HgnRecord r;
-    memcpy(&r, f->base + h.records_offset + (uint64_t)i * sizeof r, sizeof r);
-    if (r.data_offset > f->len || r.data_size > f->len - r.data_offset || r.ndims > 4) return MOE_E_INVALID;
+    memcpy(&r, m.base + h.records_offset + (uint64_t)i * sizeof r, sizeof r);
+    if (r.data_offset > m.len || r.data_size > m.len - r.data_offset || r.ndims > 4) return MOE_E_INVALID;
     FTensor t;
     t.dtype = (int)r.dtype;
     t.nd = r.ndims;
     for (int k = 0; k < 4; k++) t.dims[k] = k < (int)r.ndims ? r.dims[k] : 1;
-    t.data = f->base + r.data_offset;
+    t.data = m.base + r.data_offset;
     t.nbytes = r.data_size;
-    f->idx.emplace(std::string(r.name, strnlen(r.name, sizeof r.name)), t);  // first record of a name wins
+    std::string name(r.name, strnlen(r.name, sizeof r.name));
+    if (overlay) {
+      auto it = f->idx.find(name);
+      if (it != f->idx.end() && hgn_v2_dtype(it->second.dtype)) {
+        *skipped = true;
+        return MOE_OK;
+      }
+    }
+    ts.emplace_back(std::move(name), t);
+  }
+  for (auto& nt : ts) {
+    if (overlay) f->idx[nt.first] = nt.second;
+    else f->idx.emplace(nt.first, nt.second);  // first record of a name wins
   }
   return MOE_OK;
 }
 
-static int parse_gguf(moe_file* f) {
-  Cur c{f->base + 4, f->base + f->len};
+// Indexes one GGUF file or shard (src/gguf.h:230-314): metadata of the first shard wins, later shards only add
+// keys it does not have; general.alignment is read from the merged metadata.
+static int parse_gguf(moe_file* f, const FMap& m, int shard) {
+  if (m.len < 8 || memcmp(m.base, "GGUF", 4) != 0) return MOE_E_UNSUPPORTED;
+  Cur c{m.base + 4, m.base + m.len};
   const uint32_t ver = c.get<uint32_t>();
   if (!c.ok || ver < 2) return MOE_E_UNSUPPORTED;
   const uint64_t nt = c.get<uint64_t>(), nkv = c.get<uint64_t>();
@@ -182,7 +212,7 @@ static int parse_gguf(moe_file* f) {
         case 11: v = c.get<int64_t>(); break;
         default: c.skip(sz); is_int = false; break;  // floats
       }
-      if (is_int) f->kv_int[key] = v;
+      if (is_int && (shard == 0 || !f->kv_int.count(key))) f->kv_int[key] = v;
     }
   }
   if (!c.ok) return MOE_E_INVALID;
@@ -205,7 +235,7 @@ static int parse_gguf(moe_file* f) {
     ts.push_back(std::move(p));
   }
   if (!c.ok) return MOE_E_INVALID;
-  const uint64_t hdr = (uint64_t)(c.p - f->base);  // <= file length; align <= 4096: no wrap-around below
+  const uint64_t hdr = (uint64_t)(c.p - m.base);  // <= file length; align <= 4096: no wrap-around below
   const uint64_t data0 = (hdr + align - 1) & ~(align - 1);
   for (auto& p : ts) {
     uint32_t be, bb;
@@ -218,8 +248,8 @@ static int parse_gguf(moe_file* f) {
     if (__builtin_mul_overflow(numel / be, (uint64_t)bb, &p.t.nbytes)) return MOE_E_INVALID;
     uint64_t off;
     if (__builtin_add_overflow(data0, p.off, &off)) return MOE_E_INVALID;  // an offset that wraps around to the header
-    if (off > f->len || p.t.nbytes > f->len - off) return MOE_E_INVALID;
-    p.t.data = f->base + off;
+    if (off > m.len || p.t.nbytes > m.len - off) return MOE_E_INVALID;
+    p.t.data = m.base + off;
     if (!f->idx.emplace(p.name, p.t).second) return MOE_E_INVALID;  // duplicate name
   }
   return MOE_OK;
@@ -227,45 +257,117 @@ static int parse_gguf(moe_file* f) {
 
 MOE_API int moe_file_close(moe_file* f) {
   if (!f) return MOE_OK;
-  if (f->base) munmap((void*)f->base, f->len);
-  if (f->fd >= 0) close(f->fd);
+  for (FMap& m : f->maps) {
+    if (m.base) munmap((void*)m.base, m.len);
+    if (m.fd >= 0) close(m.fd);
+  }
   delete f;
   return MOE_OK;
+}
+
+// maps `path` read-only and appends it to f->maps
+static int map_one(moe_file* f, const char* path) {
+  FMap m;
+  m.fd = open(path, O_RDONLY | O_CLOEXEC);
+  struct stat st;
+  if (m.fd < 0 || fstat(m.fd, &st) < 0 || st.st_size < 8) {
+    if (m.fd >= 0) close(m.fd);
+    return MOE_E_INVALID;
+  }
+  m.len = (size_t)st.st_size;
+  m.dev = st.st_dev;
+  m.ino = st.st_ino;
+  void* p = mmap(nullptr, m.len, PROT_READ, MAP_PRIVATE, m.fd, 0);
+  if (p == MAP_FAILED) {
+    close(m.fd);
+    return MOE_E_STATE;
+  }
+  m.base = (const uint8_t*)p;
+  f->maps.push_back(m);
+  return MOE_OK;
+}
+
+// "<stem>-<5 digits>-of-<5 digits>.gguf": the reference opens all n shards when it is given any one of them
+// (src/gguf.h:133-150).  Returns n (0: not a shard name) and the stem with its trailing '-'.
+static int gguf_shard_count(const std::string& path, std::string* stem) {
+  const size_t p = path.rfind("-of-");
+  if (p == std::string::npos || p < 6 || path.size() != p + 4 + 5 + 5 || path.compare(path.size() - 5, 5, ".gguf") != 0)
+    return 0;
+  for (size_t i = p - 5; i < p; i++)
+    if (path[i] < '0' || path[i] > '9') return 0;
+  if (path[p - 6] != '-') return 0;
+  int n = 0;
+  for (size_t i = p + 4; i < p + 9; i++) {
+    if (path[i] < '0' || path[i] > '9') return 0;
+    n = n * 10 + (path[i] - '0');
+  }
+  *stem = path.substr(0, p - 5);
+  return n;
 }
 
 MOE_API int moe_file_open(const char* path, moe_file** out) {
   if (!path || !out) return MOE_E_INVALID;
   moe_file* f = new (std::nothrow) moe_file();
   if (!f) return MOE_E_STATE;
-  f->fd = open(path, O_RDONLY | O_CLOEXEC);
-  struct stat st;
-  if (f->fd < 0 || fstat(f->fd, &st) < 0 || st.st_size < 8) {
-    moe_file_close(f);
-    return MOE_E_INVALID;
-  }
-  f->len = (size_t)st.st_size;
-  void* p = mmap(nullptr, f->len, PROT_READ, MAP_PRIVATE, f->fd, 0);
-  if (p == MAP_FAILED) {
-    f->base = nullptr;
-    moe_file_close(f);
-    return MOE_E_STATE;
-  }
-  f->base = (const uint8_t*)p;
-  int rc;
-  if (memcmp(f->base, "HGN1", 4) == 0) {
-    f->format = MOE_FILE_HGN;
-    rc = parse_hgn(f);
-  } else if (memcmp(f->base, "GGUF", 4) == 0) {
-    f->format = MOE_FILE_GGUF;
-    rc = parse_gguf(f);
-  } else {
-    rc = MOE_E_UNSUPPORTED;
+  int rc = map_one(f, path);
+  if (rc == MOE_OK) {
+    const FMap& m0 = f->maps[0];
+    if (memcmp(m0.base, "HGN1", 4) == 0) {
+      f->format = MOE_FILE_HGN;
+      bool skipped = false;
+      rc = parse_hgn(f, m0, false, &skipped);
+    } else if (memcmp(m0.base, "GGUF", 4) == 0) {
+      f->format = MOE_FILE_GGUF;
+      std::string stem;
+      const int n = gguf_shard_count(path, &stem);
+      if (n > 0) {  // a sharded model: every shard, in order (the mapping made above is dropped for shard 1's)
+        munmap((void*)m0.base, m0.len);
+        close(m0.fd);
+        f->maps.clear();
+        for (int i = 1; i <= n && rc == MOE_OK; i++) {
+          char buf[32];
+          snprintf(buf, sizeof buf, "%05d-of-%05d.gguf", i, n);
+          rc = map_one(f, (stem + buf).c_str());
+          if (rc == MOE_OK) rc = parse_gguf(f, f->maps.back(), i - 1);
+        }
+      } else {
+        rc = parse_gguf(f, m0, 0);
+      }
+    } else {
+      rc = MOE_E_UNSUPPORTED;
+    }
   }
   if (rc != MOE_OK) {
     moe_file_close(f);
     return rc;
   }
   *out = f;
+  return MOE_OK;
+}
+
+MOE_API int moe_file_add_overlay(moe_file* f, const char* path) {
+  if (!f || !path) return MOE_E_INVALID;
+  if (f->format != MOE_FILE_HGN) return MOE_E_UNSUPPORTED;
+  int rc = map_one(f, path);
+  if (rc != MOE_OK) return rc;
+  auto drop_last = [&]() {
+    FMap& m = f->maps.back();
+    munmap((void*)m.base, m.len);
+    close(m.fd);
+    f->maps.pop_back();
+  };
+  const FMap& m = f->maps.back();
+  for (size_t i = 0; i + 1 < f->maps.size(); i++)
+    if (f->maps[i].dev == m.dev && f->maps[i].ino == m.ino) {  // already mapped (the reference compares paths)
+      drop_last();
+      return MOE_E_STATE;
+    }
+  bool skipped = false;
+  rc = parse_hgn(f, m, true, &skipped);
+  if (rc != MOE_OK || skipped) {
+    drop_last();
+    return rc != MOE_OK ? rc : MOE_E_STATE;
+  }
   return MOE_OK;
 }
 
@@ -482,6 +584,8 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
       if (cols % 32 || __builtin_mul_overflow(rows, (uint64_t)v->scale_stride, &sc) ||
           __builtin_add_overflow(64 + cells / 2, sc, &want))
         return MOE_E_INVALID;
+    } else if (t.dtype == MOE_DT_Q8G32) {  // planar: rows*cols int8 codes, then rows*cols/32 fp16 scales (src/hgn.h:176-183)
+      if (cols % 32 || __builtin_add_overflow(cells, cells / 32 * 2, &want)) return MOE_E_INVALID;
     } else if (t.dtype == MOE_DT_Q8G64) {  // per row: cols codes + cols/64 x (fp16 scale, fp16 min) (src/hgn.h:189-196)
       uint64_t stride;
       if (cols % 64 || __builtin_add_overflow(cols, cols / 64 * 4, &stride) || __builtin_mul_overflow(rows, stride, &want))
@@ -504,7 +608,9 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
     if (!su || !sd || !sx) return MOE_E_STATE;
     // q4cp, or one of the dense dtypes of the reference's generic matvec (bf16, f32, the overlay files' q8g64);
     // moe_set_shared checks that the three agree
-    auto sh_ok = [](int dt) { return dt == MOE_DT_Q4CP || dt == MOE_DT_BF16 || dt == MOE_DT_F32 || dt == MOE_DT_Q8G64; };
+    auto sh_ok = [](int dt) {
+      return dt == MOE_DT_Q4CP || dt == MOE_DT_BF16 || dt == MOE_DT_F32 || dt == MOE_DT_Q8G64 || dt == MOE_DT_Q8G32;
+    };
     if (!sh_ok(sg->dtype) || !sh_ok(su->dtype) || !sh_ok(sd->dtype) || !hgn_dtype_ok_dense(sx->dtype))
       return MOE_E_UNSUPPORTED;
     moe_wview a{}, b{}, c2{}, d2{};

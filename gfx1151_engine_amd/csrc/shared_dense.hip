@@ -17,14 +17,13 @@ __global__ void __launch_bounds__(256) k_shd_gu(int type, const uint8_t* __restr
                                                 float* __restrict__ hid) {
   const int lane = threadIdx.x & 63, r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= mid) return;
-  const uint64_t rb = moe_dense_row_bytes(type, (uint64_t)d);
   float ag[SD_MAXP], au[SD_MAXP];
 #pragma unroll
   for (int t = 0; t < SD_MAXP; t++) ag[t] = au[t] = 0.f;
   for (int b = lane; b < d / 32; b += 64) {
     float wg[32], wu[32];
-    moe_dense_block(type, Wg + (uint64_t)r * rb, d, b, wg);
-    moe_dense_block(type, Wu + (uint64_t)r * rb, d, b, wu);
+    moe_dense_block(type, Wg, (uint64_t)mid, d, (uint64_t)r, b, wg);
+    moe_dense_block(type, Wu, (uint64_t)mid, d, (uint64_t)r, b, wu);
 #pragma unroll
     for (int t = 0; t < SD_MAXP; t++) {
       if (t < P) {
@@ -58,13 +57,12 @@ __global__ void __launch_bounds__(256) k_shd_dn_axpy(int type, const uint8_t* __
                                                      int P, int d, int mid, float* __restrict__ y) {
   const int lane = threadIdx.x & 63, r = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= d) return;
-  const uint64_t rb = moe_dense_row_bytes(type, (uint64_t)mid);
   float acc[SD_MAXP];
 #pragma unroll
   for (int t = 0; t < SD_MAXP; t++) acc[t] = 0.f;
   for (int b = lane; b < mid / 32; b += 64) {
     float w[32];
-    moe_dense_block(type, Wd + (uint64_t)r * rb, mid, b, w);
+    moe_dense_block(type, Wd, (uint64_t)d, mid, (uint64_t)r, b, w);
 #pragma unroll
     for (int t = 0; t < SD_MAXP; t++) {
       if (t < P) {
@@ -90,10 +88,11 @@ __global__ void __launch_bounds__(256) k_shd_dn_axpy(int type, const uint8_t* __
 }
 
 // one row as f32 (registration-time sampling for the f16 range guard)
-__global__ void __launch_bounds__(64) k_dense_row(int type, const uint8_t* __restrict__ row, int K, float* __restrict__ out) {
+__global__ void __launch_bounds__(64) k_dense_row(int type, const uint8_t* __restrict__ base, uint64_t nrows, int K,
+                                                  uint64_t r, float* __restrict__ out) {
   for (int b = threadIdx.x; b < K / 32; b += 64) {
     float w[32];
-    moe_dense_block(type, row, K, b, w);
+    moe_dense_block(type, base, nrows, K, r, b, w);
 #pragma unroll
     for (int l = 0; l < 32; l++) out[32 * b + l] = w[l];
   }
@@ -103,7 +102,7 @@ __global__ void __launch_bounds__(64) k_dense_row(int type, const uint8_t* __res
 
 bool moe_dense_shared_supported(int type, int d, int mid) {
   if (!moe_is_dense_type(type)) return false;
-  if (type == MOE_T_Q8G64) return d % 64 == 0 && mid % 64 == 0;
+  if (type == MOE_T_Q8G64) return d % 64 == 0 && mid % 64 == 0;  // (whole 64-groups per row)
   return d % 32 == 0 && mid % 32 == 0;
 }
 
@@ -120,9 +119,9 @@ int moe_launch_dense_shared_small(int type, const uint8_t* g, const uint8_t* u, 
   return MOE_OK;
 }
 
-int moe_dense_dequant_row(int type, const uint8_t* row, int K, float* out, hipStream_t st) {
-  if (!row || !out || !moe_is_dense_type(type) || K % 32) return MOE_E_INVALID;
-  k_dense_row<<<1, 64, 0, st>>>(type, row, K, out);
+int moe_dense_dequant_row(int type, const uint8_t* base, uint64_t nrows, int K, uint64_t r, float* out, hipStream_t st) {
+  if (!base || !out || !moe_is_dense_type(type) || K % 32 || r >= nrows) return MOE_E_INVALID;
+  k_dense_row<<<1, 64, 0, st>>>(type, base, nrows, K, r, out);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -9,7 +9,7 @@ import struct
 
 import numpy as np
 
-HGN_BF16, HGN_F32, HGN_Q4CP, HGN_Q8G64 = 0, 1, 5, 7
+HGN_BF16, HGN_F32, HGN_Q4CP, HGN_Q8G64, HGN_Q8G32 = 0, 1, 5, 7, 8
 GGML_F32, GGML_BF16, GGML_Q4_K = 0, 30, 12
 _GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24),
                20: (32, 18), 23: (256, 136)}
@@ -92,7 +92,7 @@ def hgn_layer_tensors(l, hl):
          (f"layers.{l}.mlp.experts.gate_up_proj.weight", HGN_Q4CP, [E, 2 * mid, d], hl.gate_up),
          (f"layers.{l}.mlp.experts.down_proj.weight", HGN_Q4CP, [E, d, mid], hl.down)]
     if hl.shared is not None:
-        sdt = {None: HGN_Q4CP, "bf16": HGN_BF16, "f32": HGN_F32, "q8g64": HGN_Q8G64}[getattr(hl, "shared_dense", None)]
+        sdt = {None: HGN_Q4CP, "bf16": HGN_BF16, "f32": HGN_F32, "q8g64": HGN_Q8G64, "q8g32": HGN_Q8G32}[getattr(hl, "shared_dense", None)]
         t += [(f"layers.{l}.mlp.shared_expert.gate_proj.weight", sdt, [mid, d], hl.shared[0]),
               (f"layers.{l}.mlp.shared_expert.up_proj.weight", sdt, [mid, d], hl.shared[1]),
               (f"layers.{l}.mlp.shared_expert.down_proj.weight", sdt, [d, mid], hl.shared[2]),

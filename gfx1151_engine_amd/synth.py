@@ -158,10 +158,25 @@ def make_q8g64(rng, rows, cols, std=0.05):
     return quantize_q8g64(rng.standard_normal((rows, cols), dtype=np.float32) * std)
 
 
+def quantize_q8g32(w):
+    """f32 [rows][cols] -> the reference checkpoint format's planar q8g32 bytes (src/hgn.h:18,176-183): rows*cols int8
+    codes, then rows*cols/32 fp16 scales, w ~ code * scale (llama.cpp's Q8_0 arithmetic)."""
+    w = np.ascontiguousarray(w, np.float32)
+    rows, cols = w.shape
+    assert cols % 32 == 0
+    g = w.reshape(-1, 32)
+    sc = (np.abs(g).max(axis=1) / 127.0).astype(np.float16)
+    scf = np.where(sc == 0, np.float16(1), sc).astype(np.float32)
+    codes = np.clip(np.rint(g / scf[:, None]), -127, 127).astype(np.int8)
+    return np.ascontiguousarray(np.concatenate([codes.reshape(-1).view(np.uint8), sc.view(np.uint8)]))
+
+
 def make_dense(rng, kind, rows, cols, std=0.05):
-    """A dense weight matrix as stored bytes: kind "bf16" (uint16 bit patterns), "f32" or "q8g64"."""
+    """A dense weight matrix as stored bytes: kind "bf16" (uint16 bit patterns), "f32", "q8g64" or "q8g32"."""
     if kind == "q8g64":
         return make_q8g64(rng, rows, cols, std)
+    if kind == "q8g32":
+        return quantize_q8g32(rng.standard_normal((rows, cols), dtype=np.float32) * std)
     w = rng.standard_normal((rows, cols), dtype=np.float32) * std
     return f32_to_bf16_bits(w) if kind == "bf16" else w
 

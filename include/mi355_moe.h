@@ -32,7 +32,7 @@ enum moe_status {
 };
 
 /* hgn tensor dtypes (src/hgn.h:2-23) and ggml types (src/gguf.h:42-64) used on this path */
-enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5, MOE_DT_Q8G64 = 7 };
+enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5, MOE_DT_Q8G64 = 7, MOE_DT_Q8G32 = 8 };
 /* Q4_K: every kernel of the path.  Q5_K (gate/up), Q5_1 and Q8_0 (down) — the mix of the reference's GGUF
  * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — and IQ4_NL / IQ4_XS (src/gguf.h:376-407):
  * dequantisation and the general GEMV kernels. */
@@ -211,8 +211,9 @@ int moe_destroy(moe_ctx* ctx);
  * gguf: GgExperts (40_model.inc:1823).  Exactly one of hgn / gguf per layer.
  * shared expert: gate_proj/up_proj [mid][d], down_proj [d][mid], shared_expert_gate [1][d]
  * (40_model.inc:1848-1857).  gate_proj / up_proj / down_proj: q4cp (each tensor with its own codebook); or one of
- * the dense dtypes of the reference's generic matvec (src/ref.cpp:68-109) for all three: bf16, f32, q8g64 (dtype 7,
- * the overlay files' tensors: per row cols uint8 codes then cols/64 x (fp16 scale, fp16 min)); or, with
+ * the dense dtypes of the reference's generic matvec (src/ref.cpp:68-109) for all three: bf16, f32, q8g64 (dtype 7:
+ * per row cols uint8 codes then cols/64 x (fp16 scale, fp16 min)), and q8g32 (dtype 8, the quality overlay's dense
+ * tensors: rows*cols int8 codes then rows*cols/32 fp16 scales over the whole tensor, src/hgn.h:18,176-183); or, with
  * sh_gguf_type != 0, raw GGUF rows of that one ggml type.  shared_expert_gate: f32 or bf16.
  * MOE_E_UNSUPPORTED for other matrix dtypes.  A densely stored shared expert of a q4cp layer runs in launches of its
  * own next to the routed experts' kernels. */
@@ -304,8 +305,17 @@ typedef struct moe_tensor_info {
   const uint8_t* data;
   uint64_t nbytes;
 } moe_tensor_info;
+/* A GGUF path of the form <stem>-<5 digits>-of-<5 digits>.gguf opens every shard of that model, whichever shard is
+ * named (gguf::File::open, src/gguf.h:133-150): tensors of all shards are indexed, integer metadata of the first
+ * shard wins. */
 int moe_file_open(const char* path, moe_file** out);
 int moe_file_close(moe_file* f);
+/* Maps a second .hgn file whose tensors replace those of the same name (hgn::Checkpoint::add_overlay,
+ * src/hgn.h:108-121: the "quality overlay" that stores dense tensors, the shared expert among them, in another
+ * dtype).  MOE_OK: applied.  MOE_E_STATE: the file was left out as a whole, as the reference leaves it out -- it is
+ * already mapped, or one of its tensors would replace an hgn v2 tensor (dtype 16 / 23 / 24).  The overlay stays
+ * mapped until moe_file_close. */
+int moe_file_add_overlay(moe_file* f, const char* path);
 int moe_file_format(const moe_file* f);
 int64_t moe_file_tensor_count(const moe_file* f);
 /* MOE_E_STATE if the file has no tensor of that name */

@@ -21,7 +21,12 @@
  *
  * Pinning status of every function is listed in oracle/README.md; each one is
  * checked in tests/ against the reference's own code built under oracle/_ref
- * and against closed forms / brute force.  None is "parity unpinned".
+ * and against closed forms / brute force.  One form is "parity unpinned": a shared
+ * expert stored as planar q8g32 (hgn dtype 8).  Its dequantisation (mat_row) is pinned
+ * against the reference's Checkpoint::dequant, but the reference's CPU matvec has no
+ * branch for that dtype (src/ref.cpp:68-109 throws), so the layer form used here -- the
+ * dequantised row in the generic fp64 dot product -- is confirmed by no run of the
+ * reference.  Everything else is pinned.
  *
  * One deliberate addition: std::partial_sort in src/ref.cpp:587 leaves the
  * order of equal probabilities unspecified.  The oracle fixes it to "lowest
@@ -41,7 +46,8 @@
 /* ---- weight format tags (shared with the library header by value) ---- */
 enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q5_1 = 7, ORC_Q8_0 = 8,
        ORC_IQ4_NL = 20, ORC_IQ4_XS = 23,
-       ORC_Q8G64 = 107 /* hgn dtype 7; the tag is moved off ggml's Q5_1 = 7 */ };
+       ORC_Q8G64 = 107 /* hgn dtype 7; the tag is moved off ggml's Q5_1 = 7 */,
+       ORC_Q8G32 = 108 /* hgn dtype 8 (moved off ggml's Q8_0 = 8) */ };
 
 /* src/hgn.h:77-84 and src/gguf.h:318-325 (same function twice in the reference) */
 ORC_API float orc_fp16_to_f32(uint16_t h) {
@@ -271,6 +277,15 @@ static void mat_row(const orc_mat* W, uint64_t r, float* out) {
       for (uint64_t g = 0; g < W->cols / 64; g++) {
         const float s = orc_fp16_to_f32(sm[g * 2]), m = orc_fp16_to_f32(sm[g * 2 + 1]);
         for (uint64_t j = 0; j < 64; j++) out[g * 64 + j] = rp[g * 64 + j] * s + m;
+      }
+      break;
+    }
+    case ORC_Q8G32: { /* src/hgn.h:176-183: planar [rows*cols int8][rows*cols/32 fp16 scales], w = q[i] * s[i / 32] */
+      const int8_t* q = (const int8_t*)W->data;
+      const uint16_t* sc = (const uint16_t*)(W->data + W->rows * W->cols);
+      for (uint64_t c = 0; c < W->cols; c++) {
+        const uint64_t i = r * W->cols + c;
+        out[c] = q[i] * orc_fp16_to_f32(sc[i / 32]);
       }
       break;
     }

@@ -13,7 +13,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 F32, BF16, Q4CP, Q4K = 1, 0, 5, 12
 Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS = 13, 7, 8, 20, 23   # further ggml block types of the expert tensors (ids as in GGUF)
 Q8G64 = 107  # hgn dtype 7 (the oracle's tag is moved off ggml's Q5_1 = 7)
-HGN_DTYPE = {BF16: 0, F32: 1, Q4CP: 5, Q8G64: 7}  # oracle tag -> dtype field of the reference's checkpoint format
+Q8G32 = 108  # hgn dtype 8 (moved off ggml's Q8_0 = 8)
+HGN_DTYPE = {BF16: 0, F32: 1, Q4CP: 5, Q8G64: 7, Q8G32: 8}  # oracle tag -> dtype field of the reference's checkpoint format
 GG_TYPES = (Q4K, Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS)
 
 
@@ -106,6 +107,8 @@ class Mat:
             assert self.data.dtype == np.uint16 and self.data.size == rows * cols
         elif dtype == Q8G64:
             assert self.data.dtype == np.uint8 and cols % 64 == 0 and self.data.size == rows * (cols + cols // 64 * 4)
+        elif dtype == Q8G32:
+            assert self.data.dtype == np.uint8 and cols % 32 == 0 and self.data.size == rows * cols + rows * cols // 32 * 2
 
     def c(self):
         return _Mat(self.dtype, self.data.ctypes.data, self.rows, self.cols)
@@ -122,7 +125,7 @@ class Mat:
             return gg_rows(self.dtype, self.data[row0 * rb:(row0 + nrows) * rb], nrows, self.cols)
         if self.dtype == F32:
             return self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].copy()
-        if self.dtype == Q8G64:
+        if self.dtype in (Q8G64, Q8G32):
             out = np.empty((nrows, self.cols), np.float32)
             m = self.c()
             lib().orc_mat_rows(C.byref(m), row0, nrows, _p(out))

@@ -34,6 +34,7 @@ uint64_t dense_bytes(uint32_t dtype, uint64_t rows, uint64_t cols) {
   if (dtype == 0) return rows * cols * 2;  // bf16
   if (dtype == 5) return 64 + rows * cols / 2 + rows * (((cols / 32 * 2) + 15) & ~15ULL);
   if (dtype == 7) return rows * (cols + cols / 64 * 4);  // q8g64
+  if (dtype == 8) return rows * cols + rows * cols / 32 * 2;  // q8g32 planar
   return 0;
 }
 }  // namespace

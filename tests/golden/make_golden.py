@@ -106,6 +106,10 @@ def layer_cases():
     q8 = S.make_q8g64(rng, 5, 192, 0.3)
     out["q8g64_raw"] = q8
     out["q8g64_bits"] = O.ref_dequant_tensor(O.Mat(O.Q8G64, q8, 5, 192)).view(np.uint32)
+    # Checkpoint::dequant of one planar q8g32 tensor (src/hgn.h:176-183)
+    q8p = S.quantize_q8g32(rng.standard_normal((6, 96)).astype(np.float32) * 0.3)
+    out["q8g32_raw"] = q8p
+    out["q8g32_bits"] = O.ref_dequant_tensor(O.Mat(O.Q8G32, q8p, 6, 96)).view(np.uint32)
     np.savez_compressed(os.path.join(OUT, "moe_layer.npz"), **out)
 
 

@@ -60,7 +60,7 @@ class HostLayer:
         if self.shared is not None:
             st = O.Q4CP if self.fmt == "q4cp" else self.tsh
             if self.shared_dense:
-                st = {"bf16": O.BF16, "f32": O.F32, "q8g64": O.Q8G64}[self.shared_dense]
+                st = {"bf16": O.BF16, "f32": O.F32, "q8g64": O.Q8G64, "q8g32": O.Q8G32}[self.shared_dense]
             sh = [O.Mat(st, self.shared[0], mid, d), O.Mat(st, self.shared[1], mid, d),
                   O.Mat(st, self.shared[2], d, mid), O.Mat(O.F32, self.shared[3], 1, d)]
         router = O.Mat(self.router_dt, self.router, E, d)
@@ -95,7 +95,7 @@ class HostLayer:
             wt = capi.Q4CP if self.fmt == "q4cp" else 0
             shw = self.shared[:3]
             if self.shared_dense:
-                wt = {"bf16": capi.BF16, "f32": capi.F32, "q8g64": capi.Q8G64}[self.shared_dense]
+                wt = {"bf16": capi.BF16, "f32": capi.F32, "q8g64": capi.Q8G64, "q8g32": capi.Q8G32}[self.shared_dense]
                 if self.shared_dense == "bf16":
                     shw = [a.view(np.int16) for a in shw]
             m.set_shared(0, capi.wview(up("shg", shw[0]), wt, mid, d),

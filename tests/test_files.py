@@ -78,6 +78,110 @@ def test_gguf_parser_matches_reference_reader(tmp_path):
     f.close()
 
 
+def test_split_gguf_opens_every_shard(tmp_path):
+    """<stem>-0000i-of-0000n.gguf: naming any shard opens all of them (src/gguf.h:133-150); metadata of the first
+    shard wins.  Checked against the reference's own reader where it is built."""
+    layers = _layers("q4k")
+    ts = []
+    for i, hl in enumerate(layers):
+        ts += files.gguf_layer_tensors(i, hl)
+    kv0 = {"general.architecture": "synthmoe", "synthmoe.expert_used_count": K, "general.alignment": 64}
+    kv1 = {"general.architecture": "synthmoe", "synthmoe.expert_used_count": K + 1, "synthmoe.only_in_shard_2": 7}
+    cut = len(ts) // 2 + 1
+    p1, p2 = tmp_path / "m-00001-of-00002.gguf", tmp_path / "m-00002-of-00002.gguf"
+    files.write_gguf(p1, ts[:cut], kv=kv0, align=64)
+    files.write_gguf(p2, ts[cut:], kv=kv1, align=32)
+    for path in (p2, p1):
+        f = capi.ModelFile(path)
+        assert len(f) == len(ts)
+        for name, dt, ne, data in ts:
+            raw = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+            for got in [f.find(name)] + ([O.ref_gguf_tensor(path, name)] if HAVE_REF else []):
+                assert got[0] == dt and got[1][:len(ne)] == tuple(ne) and np.array_equal(got[2], raw), name
+        assert f.config(0).topk == K  # the first shard's value, not the second's
+        f.close()
+    if HAVE_REF:
+        assert O.ref_gguf_kv_i(p2, "synthmoe.expert_used_count") == K
+        assert O.ref_gguf_kv_i(p2, "synthmoe.only_in_shard_2") == 7
+    # a missing shard is an error, and so is a tensor name that two shards both carry
+    os.rename(p2, tmp_path / "gone.gguf")
+    with pytest.raises(capi.MoeError):
+        capi.ModelFile(p1)
+    files.write_gguf(p2, ts[cut - 1:], kv=kv1, align=32)
+    with pytest.raises(capi.MoeError):
+        capi.ModelFile(p1)
+
+
+def test_hgn_overlay_replaces_tensors_by_name(tmp_path):
+    """hgn::Checkpoint::add_overlay (src/hgn.h:108-121,348-362): tensors of the overlay file replace the base file's;
+    the file is left out as a whole if it is already mapped or would replace an hgn v2 tensor."""
+    rng = np.random.default_rng(31)
+    base_l = HostLayer(rng, D, MID, E, K)
+    p, _ = _hgn(tmp_path, [base_l], first=0)
+    over = HostLayer(rng, D, MID, E, K, shared_dense="bf16")
+    ots = [t for t in files.hgn_layer_tensors(0, over) if "shared_expert." in t[0]]
+    po = tmp_path / "overlay.hgn"
+    files.write_hgn(po, ots + [("extra.tensor", files.HGN_F32, [4], np.arange(4, dtype=np.float32))])
+    f = capi.ModelFile(p)
+    n0 = len(f)
+    assert f.find("layers.0.mlp.shared_expert.up_proj.weight")[0] == files.HGN_Q4CP
+    assert f.add_overlay(po) is True
+    assert len(f) == n0 + 1
+    got = f.find("layers.0.mlp.shared_expert.up_proj.weight")
+    assert got[0] == files.HGN_BF16 and np.array_equal(got[2], np.ascontiguousarray(over.shared[1]).view(np.uint8).reshape(-1))
+    assert f.find("layers.0.mlp.gate.weight")[0] in (files.HGN_F32, files.HGN_BF16)  # untouched
+    assert f.add_overlay(po) is False and f.add_overlay(p) is False  # already mapped
+    f.close()
+    # an overlay that would replace an hgn v2 tensor (dtype 23) is left out as a whole
+    pv2 = tmp_path / "v2.hgn"
+    files.write_hgn(pv2, [("a", 23, [2, 64], np.zeros(64, np.uint8)), ("b", files.HGN_F32, [4], np.zeros(4, np.float32))])
+    pov = tmp_path / "ov2.hgn"
+    files.write_hgn(pov, [("b", files.HGN_F32, [4], np.ones(4, np.float32)), ("a", files.HGN_F32, [4], np.ones(4, np.float32))])
+    f = capi.ModelFile(pv2)
+    assert f.add_overlay(pov) is False
+    assert f.find("a")[0] == 23 and not f.find("b")[2].any()
+    f.close()
+    # GGUF files take no overlay; a file that is not HGN1 is refused
+    pg, _ = _gguf(tmp_path, _layers("q4k"))
+    f = capi.ModelFile(pg)
+    with pytest.raises(capi.MoeError):
+        f.add_overlay(po)
+    f.close()
+    f = capi.ModelFile(p)
+    with pytest.raises(capi.MoeError):
+        f.add_overlay(pg)
+    f.close()
+
+
+@pytest.mark.gpu
+def test_layer_loaded_through_an_overlay(tmp_path):
+    """Base file with a q4cp shared expert, overlay file with the same tensors in q8g32: the loaded layer computes
+    with the overlay's."""
+    import torch
+    rng = np.random.default_rng(33)
+    base_l = HostLayer(rng, D, MID, E, K)
+    p, _ = _hgn(tmp_path, [base_l], first=0)
+    over = HostLayer(rng, D, MID, E, K, shared_dense="q8g32")  # (the quality overlay's dtype for dense tensors)
+    po = tmp_path / "overlay.hgn"
+    files.write_hgn(po, [t for t in files.hgn_layer_tensors(0, over) if "shared_expert." in t[0]])
+    f = capi.ModelFile(p)
+    assert f.add_overlay(po)
+    m = capi.Moe(D, MID, E, K, layers=1, max_tokens=64)
+    w = f.load_layers(m, 0, 0, 1)
+    f.close()
+    base_l.shared[:3] = over.shared[:3]
+    base_l.shared_dense = "q8g32"
+    for T in (1, 7, 64):
+        x = _x(T, seed=T)
+        want, io, _ = O.moe_layer(base_l.oracle_layer(), x)
+        y = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :K] == io[:, :K]).all()
+        assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max(), T
+    del m
+    w.free()
+
+
 def test_malformed_files_are_rejected(tmp_path):
     lib = capi.lib()
 
@@ -232,7 +336,7 @@ def test_hgn_file_with_a_codebook_per_shared_tensor(tmp_path):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("kind", ["bf16", "q8g64"])
+@pytest.mark.parametrize("kind", ["bf16", "q8g64", "q8g32"])
 def test_hgn_file_with_a_densely_stored_shared_expert(tmp_path, kind):
     """The shared expert as bf16 (an unquantised checkpoint) or q8g64 (the overlay files' storage, src/hgn.h:10):
     the reference runs these through its generic matvec (src/ref.cpp:68-109,623-636)."""

@@ -323,9 +323,10 @@ def test_batch_layer_other_gguf_types(oracle, tgu, tdn, tsh, d, mid, T):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("fmt,kind", [("q4cp", "bf16"), ("q4cp", "q8g64"), ("q4cp", "f32"), ("q4k", "bf16"), ("gg", "q8g64")])
+@pytest.mark.parametrize("fmt,kind", [("q4cp", "bf16"), ("q4cp", "q8g64"), ("q4cp", "f32"), ("q4cp", "q8g32"), ("q4k", "bf16"),
+                                      ("gg", "q8g64"), ("q4k", "q8g32")])
 def test_batch_layer_with_a_densely_stored_shared_expert(oracle, fmt, kind):
-    """bf16 / f32 / q8g64 shared-expert matrices beside q4cp, all-Q4_K and mixed-GGUF routed experts: decode, a small
+    """bf16 / f32 / q8g64 / q8g32 shared-expert matrices beside q4cp, all-Q4_K and mixed-GGUF routed experts: decode, a small
     batch and a grouped-GEMM batch against the oracle (which follows the reference's matvec per storage,
     src/ref.cpp:68-109)."""
     import torch

@@ -236,6 +236,27 @@ def test_q8g64_dequant_golden(oracle, golden):
     assert (w[0] == np.arange(64, dtype=np.float32) * 4 * 0.5 - 3.0).all()
 
 
+def test_q8g32_dequant_golden(oracle, golden):
+    """Checkpoint::dequant of the reference on a planar q8g32 tensor (src/hgn.h:176-183): bit-identical rows, from
+    the committed vector and (where the reference build is present) live on another tensor.  The reference's CPU
+    matvec has no q8g32 branch (src/ref.cpp:68-109 throws for it), so a layer with such a shared expert is the
+    dequantised row in the generic fp64 dot product: that form is not pinned by a run of the reference."""
+    g = golden("moe_layer.npz")
+    m = oracle.Mat(oracle.Q8G32, g["q8g32_raw"], 6, 96)
+    assert (bits(m.dequant()) == g["q8g32_bits"]).all()
+    assert (bits(m.dequant(4, 2)) == g["q8g32_bits"][4:6]).all()
+    raw = np.zeros(64 + 4, np.uint8)  # two rows of 32: codes -128..127 step 4, scales 0.25 and -2
+    raw[:64] = (np.arange(64) * 4 - 128).astype(np.int8).view(np.uint8)
+    raw[64:].view(np.float16)[:] = [0.25, -2.0]
+    w = oracle.Mat(oracle.Q8G32, raw, 2, 32).dequant()
+    assert (w[0] == (np.arange(32) * 4 - 128) * 0.25).all() and (w[1] == (np.arange(32, 64) * 4 - 128) * -2.0).all()
+    if oracle.ref() is not None:
+        rng = np.random.default_rng(9)
+        q = S.quantize_q8g32(rng.standard_normal((8, 160)).astype(np.float32))
+        mm = oracle.Mat(oracle.Q8G32, q, 8, 160)
+        assert (bits(mm.dequant()) == bits(oracle.ref_dequant_tensor(mm))).all()
+
+
 def test_q8g64_shared_expert_vs_reference_build(oracle):
     """The reference's q8g64 matvec sums per 64-group (code . x) * scale + min * sum(x) (src/ref.cpp:91-106), not the
     dot with the dequantised row: the oracle follows it to the bit."""
