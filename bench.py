@@ -103,11 +103,11 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     from gfx1151_engine_amd import capi, workloads as W
     from gfx1151_engine_amd import synth as S
     d, mid, k = D, MID, K
-    # ggmix_*: GGUF layer in the reference checkpoints' type mix (Q5_K gate/up, Q8_0 down, Q4_K shared expert) on the
+    # ggmix_*: GGUF layer in the reference checkpoints' type mix (Q5_K gate/up, Q8_0 down, Q8_0 shared expert) on the
     # general GEMV kernels
     ggmix = wl.startswith("ggmix_")
     fmt = "q4k" if wl.startswith("q4k") or ggmix else "q4cp"
-    gg_types = (13, 8, 12) if ggmix else (12, 12, 12)
+    gg_types = (13, 8, 8) if ggmix else (12, 12, 12)
     kind = wl.replace("q4k_", "").replace("ggmix_", "")
     T = tokens or {"prefill": 16384 if fmt == "q4cp" else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
     nlayers = nlayers_arg if kind == "stack" else 1
@@ -209,7 +209,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     cfg = {"workload": wl, "tokens": T, "d_model": d, "moe_mid": mid, "experts": E, "topk": k, "shared_experts": 1,
            "format": ("q4cp g32, the reference converter's universal expert codebook (table look-up, f32 GEMV kernels)"
                       if universal else "q4cp g32 zero-point 8") if fmt == "q4cp" else
-           ("GGUF Q5_K gate/up, Q8_0 down, Q4_K shared expert (general f32 kernels)" if ggmix else "GGUF Q4_K"),
+           ("GGUF Q5_K gate/up, Q8_0 down, Q8_0 shared expert" if ggmix else "GGUF Q4_K"),
            "layers": nlayers, **extra}
     if kind == "prefill":
         flop_tok = k * 6 * d * mid + 6 * d * mid + 2 * d * E + 2 * d
@@ -247,7 +247,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
             gu_bytes = 2 * mid * (uniq * W.gg_row_bytes(gg_types[0], d) + W.gg_row_bytes(gg_types[2], d))
         up_s = up_marginal_ms * 1e-3
         od = dict(list(LIB_OPTIONS) + list(opts))
-        int_dec = od.get(1, 1) != 0 and not ggmix and not universal  # (a table codebook takes the f32 kernels)
+        int_dec = od.get(1, 1) != 0 and not universal  # (a table codebook takes look-up / f32 kernels)
         # the arithmetic of the GEMV kernels: integer dot products of the 4-bit codes with the activations' 4-bit
         # (q4cp: v_dot8_i32_i4, four planes) or 8-bit (Q4_K: v_dot4_i32_i8, two planes) digit planes, f32 scales;
         # or plain f32 FMAs (MOE_OPT_INT_DECODE = 0, and the general GGUF kernels)

@@ -465,15 +465,20 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
   // the look-up kernels win on latency, not on throughput)
   const bool use_lut = L.has_q4cp && c->int_decode && !use_int && P <= 5 && (!sh || L.sh_gguf_type == 0) &&
                        moe_dec_supported(g.d, g.mid, nslots_d) && moe_dec_gu_topk_supported(g.experts, g.topk);
+  // GGUF layers in other mixes of Q4_K / Q5_K / Q8_0 / Q5_1 (the reference checkpoints' types): the same integer-dot
+  // launches, generalised over the block type
+  const bool use_intgg = L.has_gguf && c->int_decode && !use_int4k &&
+                         moe_decgg_supported(L.gg.tgu, L.gg.tdn, L.sh_gguf_type, sh, g.d, g.mid, g.topk, g.experts) &&
+                         (!sh || L.sh_gguf_type != 0);
   const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min && moe_dec_uq_supported(g.d);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
-  const bool gu_topk = ((use_int && !use_uq) || use_int4k || use_lut) && moe_dec_gu_topk_supported(g.experts, g.topk);
+  const bool gu_topk = ((use_int && !use_uq) || use_int4k || use_intgg || use_lut) && moe_dec_gu_topk_supported(g.experts, g.topk);
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
          int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
-                                         c->sh_logit, (use_int || use_int4k) ? c->xplanes : nullptr, c->xmeta,
-                                         use_int4k, gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk,
+                                         c->sh_logit, (use_int || use_int4k || use_intgg) ? c->xplanes : nullptr, c->xmeta,
+                                         use_int4k || use_intgg, gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk,
                                          g.id_stride, &fused, st, c->kpart, c->ktickets);
          if (!e && !fused && !gu_topk)
            e = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
@@ -550,6 +555,18 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
     });
   }
   if (sh && L.sh_gguf_type == 0) return MOE_E_UNSUPPORTED;
+  if (use_intgg) {
+    if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+           return moe_launch_decgg_gu_topk(L.gg.tgu, L.sh_gguf_type, L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta,
+                                           c->logits, g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
+                                           c->hplanes, c->hmeta, st);
+         })))
+      return rc;
+    return stage(MOE_PROF_DOWN, [&]() -> int {
+      return moe_launch_decgg_dn(L.gg.tdn, L.sh_gguf_type, L.gg.down, rd, c->sh_logit, c->hplanes, c->hmeta, c->ids, c->ws,
+                                 g.id_stride, g.topk, P, g.d, g.mid, y, (uint64_t)g.d, st);
+    });
+  }
   if (L.gg.tgu != MOE_GGML_Q4_K || L.gg.tdn != MOE_GGML_Q4_K || (sh && L.sh_gguf_type != MOE_GGML_Q4_K)) {
     // Q5_K gate/up, Q5_1 / Q8_0 down (or such a shared expert): the general kernels
     for (int phase = 1; phase <= 2; phase++)

@@ -293,6 +293,332 @@ __global__ void __launch_bounds__(256) k_dec4k_dn(Dn4kArgs A, const uint32_t* __
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same launches for the other block types of the reference's GGUF checkpoints (Q5_K gate/up, Q5_1 / Q8_0 down,
+// a Q8_0 shared expert; src/gpu/parts/30_host_util.inc:399-405, src/gguf_map.h:212-214), any mix of them with Q4_K.
+// A lane still owns one unit of 64 weights = two activation groups with their two 8-bit digit planes; what differs
+// per type is what a unit's bytes are and how its integer sums are scaled:
+//   Q5_K  (176 B / 256): Q4_K plus a fifth bit per code; unit jj of a super-block takes bits 2jj and 2jj+1 of the 32
+//         qh bytes; the four lanes of the super-block load 8 qh bytes each and hand them round by DPP
+//   Q8_0  (34 B / 32):   two blocks = 68 bytes starting on a 4-byte boundary: fp16 d, 32 int8 codes (2 bytes off the
+//         dword grid in the first block: one v_alignbit per word), d, 32 codes; w = d q
+//   Q5_1  (24 B / 32):   two blocks = 48 bytes: fp16 d, m, 32 fifth bits, 16 code bytes (low nibbles = elements
+//         0..15, high nibbles = 16..31); w = d q + m
+// The type of a block (gate/up launch: one slot) or of a wave (down launch: the shared expert has a wave of its
+// own) is uniform, so it is one scalar branch outside the loads.  Types with more than 9 registers per row in
+// flight take the wave's eight rows in two batches of four.
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int T> struct GgU;
+template <> struct GgU<MOE_GGML_Q4_K> { uint4 c0, c1; uint32_t hw; };
+template <> struct GgU<MOE_GGML_Q5_K> { uint4 c0, c1; uint2 qh; uint32_t hw; };
+template <> struct GgU<MOE_GGML_Q8_0> { uint32_t w[17]; };
+template <> struct GgU<MOE_GGML_Q5_1> { uint4 a, b, c; };
+
+__host__ __device__ constexpr uint64_t ggu_row_bytes(int t, uint64_t k) {
+  return t == MOE_GGML_Q4_K ? k / 256 * 144 : t == MOE_GGML_Q5_K ? k / 256 * 176 : t == MOE_GGML_Q8_0 ? k / 32 * 34 : k / 32 * 24;
+}
+template <int T> constexpr int ggu_batch() { return T == MOE_GGML_Q4_K ? 8 : 4; }  // rows in flight together
+
+template <int T>
+__device__ __forceinline__ void ggu_fetch(const uint8_t* row, int ul, GgU<T>& o) {
+  const int jj = ul & 3;
+  if constexpr (T == MOE_GGML_Q4_K) {
+    const uint8_t* sb = row + (size_t)(ul >> 2) * 144;
+    o.hw = *(const uint32_t*)(sb + 4 * jj);
+    o.c0 = *(const uint4*)(sb + 16 + jj * 32);
+    o.c1 = *(const uint4*)(sb + 32 + jj * 32);
+  } else if constexpr (T == MOE_GGML_Q5_K) {
+    const uint8_t* sb = row + (size_t)(ul >> 2) * 176;
+    o.hw = *(const uint32_t*)(sb + 4 * jj);
+    o.qh = *(const uint2*)(sb + 16 + 8 * jj);
+    o.c0 = *(const uint4*)(sb + 48 + jj * 32);
+    o.c1 = *(const uint4*)(sb + 64 + jj * 32);
+  } else if constexpr (T == MOE_GGML_Q8_0) {
+    const uint8_t* p = row + (size_t)ul * 68;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const u32x4_a4 v = *(const u32x4_a4*)(p + 16 * i);
+      o.w[4 * i] = v.x; o.w[4 * i + 1] = v.y; o.w[4 * i + 2] = v.z; o.w[4 * i + 3] = v.w;
+    }
+    o.w[16] = *(const uint32_t*)(p + 64);
+  } else {
+    const uint4* p = (const uint4*)(row + (size_t)ul * 48);
+    o.a = p[0]; o.b = p[1]; o.c = p[2];
+  }
+}
+
+// integer sum of a group against both digit planes -> float (the sums can exceed 2^24 for 5- and 8-bit codes: two
+// exact conversions and one rounded fma instead of an integer combine)
+__device__ __forceinline__ float planes_val(int hi, int lo) { return fmaf((float)hi, 256.f, (float)lo); }
+
+template <int T>
+__device__ __forceinline__ float ggu_dot(const GgU<T>& o, int jj, const XU& x) {
+  if constexpr (T == MOE_GGML_Q4_K) {
+    return unit_dot(o.c0, o.c1, quad_header(o.hw), jj, x);
+  } else if constexpr (T == MOE_GGML_Q5_K) {
+    const uint4 hd = quad_header(o.hw);
+    const uint32_t w[8] = {o.c0.x, o.c0.y, o.c0.z, o.c0.w, o.c1.x, o.c1.y, o.c1.z, o.c1.w};
+    // qh word i (bytes 4i..4i+3) sits in lane i/2 of the quad, register i%2
+    uint32_t qh[8];
+    qh[0] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.x, 0x00, 0xf, 0xf, true);
+    qh[1] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.y, 0x00, 0xf, 0xf, true);
+    qh[2] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.x, 0x55, 0xf, 0xf, true);
+    qh[3] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.y, 0x55, 0xf, 0xf, true);
+    qh[4] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.x, 0xAA, 0xf, 0xf, true);
+    qh[5] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.y, 0xAA, 0xf, 0xf, true);
+    qh[6] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.x, 0xFF, 0xf, 0xf, true);
+    qh[7] = (uint32_t)__builtin_amdgcn_mov_dpp((int)o.qh.y, 0xFF, 0xf, 0xf, true);
+    int a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const uint32_t hb = qh[i] >> (2 * jj);
+      const int lo = (int)((w[i] & 0x0f0f0f0fu) | ((hb & 0x01010101u) << 4));
+      const int hi = (int)(((w[i] >> 4) & 0x0f0f0f0fu) | (((hb >> 1) & 0x01010101u) << 4));
+      a0 = __builtin_amdgcn_sdot4(lo, (int)x.a[0][i], a0, false);
+      a1 = __builtin_amdgcn_sdot4(lo, (int)x.a[1][i], a1, false);
+      b0 = __builtin_amdgcn_sdot4(hi, (int)x.b[0][i], b0, false);
+      b1 = __builtin_amdgcn_sdot4(hi, (int)x.b[1][i], b1, false);
+    }
+    float sa, ma, sb, mb;
+    k4_pair(hd, jj, sa, ma, sb, mb);
+    return (sa * x.qa * planes_val(a0, a1) + sb * x.qb * planes_val(b0, b1)) - (ma * x.qsa + mb * x.qsb);
+  } else if constexpr (T == MOE_GGML_Q8_0) {
+    int a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const int ca = (int)__builtin_amdgcn_alignbit(o.w[i + 1], o.w[i], 16);  // the first block's codes: 2 bytes off the dword grid
+      const int cb = (int)o.w[9 + i];
+      a0 = __builtin_amdgcn_sdot4(ca, (int)x.a[0][i], a0, false);
+      a1 = __builtin_amdgcn_sdot4(ca, (int)x.a[1][i], a1, false);
+      b0 = __builtin_amdgcn_sdot4(cb, (int)x.b[0][i], b0, false);
+      b1 = __builtin_amdgcn_sdot4(cb, (int)x.b[1][i], b1, false);
+    }
+    union { uint16_t u; __half h; } d0, d1;
+    d0.u = (uint16_t)(o.w[0] & 0xffffu);
+    d1.u = (uint16_t)(o.w[8] >> 16);
+    return __half2float(d0.h) * x.qa * planes_val(a0, a1) + __half2float(d1.h) * x.qb * planes_val(b0, b1);
+  } else {  // Q5_1
+    const uint32_t dw[12] = {o.a.x, o.a.y, o.a.z, o.a.w, o.b.x, o.b.y, o.b.z, o.b.w, o.c.x, o.c.y, o.c.z, o.c.w};
+    float r = 0.f;
+#pragma unroll
+    for (int blk = 0; blk < 2; blk++) {
+      const uint32_t dm = dw[6 * blk], qh = dw[6 * blk + 1];
+      int v0 = 0, v1 = 0;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t q = dw[6 * blk + 2 + i];
+        // four bits of qh -> bit 4 of four bytes
+        const uint32_t hl = ((((qh >> (4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+        const uint32_t hh = ((((qh >> (16 + 4 * i)) & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+        const int lo = (int)((q & 0x0f0f0f0fu) | hl), hi = (int)(((q >> 4) & 0x0f0f0f0fu) | hh);
+        const uint32_t* p0 = blk ? x.b[0] : x.a[0];
+        const uint32_t* p1 = blk ? x.b[1] : x.a[1];
+        v0 = __builtin_amdgcn_sdot4(lo, (int)p0[i], v0, false);
+        v1 = __builtin_amdgcn_sdot4(lo, (int)p1[i], v1, false);
+        v0 = __builtin_amdgcn_sdot4(hi, (int)p0[4 + i], v0, false);
+        v1 = __builtin_amdgcn_sdot4(hi, (int)p1[4 + i], v1, false);
+      }
+      union { uint32_t u; __half2 h; } cv;
+      cv.u = dm;
+      r += __low2float(cv.h) * (blk ? x.qb : x.qa) * planes_val(v0, v1) + __high2float(cv.h) * (blk ? x.qsb : x.qsa);
+    }
+    return r;
+  }
+}
+
+// eight rows of one wave (gate/up launch: four gate rows and the matching up rows): acc[i] = wave sum of row i
+template <int T>
+__device__ __forceinline__ void ggu_gu_rows(const uint8_t* gbase, const uint8_t* ubase, int r0, int d, int ul,
+                                            float mlive, const XU& x, float (&acc)[8]) {
+  constexpr int RB = ggu_batch<T>();
+  const uint64_t rb = ggu_row_bytes(T, (uint64_t)d);
+  const int jj = ul & 3;
+#pragma unroll
+  for (int h = 0; h < 8; h += RB) {
+    GgU<T> u[RB];
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+      ggu_fetch<T>(((i + h) < 4 ? gbase : ubase) + (uint64_t)(r0 + ((i + h) & 3)) * rb, ul, u[i]);
+    __builtin_amdgcn_sched_barrier(0);  // every load of the batch is issued before the first dot product
+#pragma unroll
+    for (int i = 0; i < RB; i++) {
+      acc[i + h] = sum64(ggu_dot<T>(u[i], jj, x) * mlive);
+      if (i & 1) __builtin_amdgcn_sched_barrier(0);  // rows are consumed in arrival order
+    }
+  }
+}
+
+#define GGU_SWITCH(t, CALL)                                                       \
+  switch (t) {                                                                    \
+    case MOE_GGML_Q4_K: { constexpr int T = MOE_GGML_Q4_K; CALL; } break;          \
+    case MOE_GGML_Q5_K: { constexpr int T = MOE_GGML_Q5_K; CALL; } break;          \
+    case MOE_GGML_Q8_0: { constexpr int T = MOE_GGML_Q8_0; CALL; } break;          \
+    default: { constexpr int T = MOE_GGML_Q5_1; CALL; } break;                    \
+  }
+
+struct GuGgArgs {
+  const uint8_t *gate, *up, *sh_gate, *sh_up;
+  int tgu, tsh;
+};
+
+// grid (mid/32, slots incl. shared + the exact top-k row, P); block 512: k_dec4k_gu<NPL> for any of the four types
+template <int NPL>
+__global__ void __launch_bounds__(512, 4) k_decgg_gu(GuGgArgs A, const uint32_t* __restrict__ xplanes,
+                                                     const float2* __restrict__ xmeta, int id_stride, int kpt, int d,
+                                                     int mid, uint32_t* __restrict__ hplanes,
+                                                     float2* __restrict__ hmeta, const float* __restrict__ logits,
+                                                     int n_experts, int* __restrict__ ids_out,
+                                                     float* __restrict__ ws_out) {
+  __shared__ float gs[G4_ROWS], us[G4_ROWS];
+  __shared__ uint32_t pk[QV_GROUP_DW];
+  __shared__ int sel_ids[64];
+  __shared__ float sel_ws[64];
+  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y - 1;
+  if (s == nslots) {  // the extra grid row: exact softmax / top-k for the down launch
+    if (blockIdx.x == 0) {
+      topk_block<NPL, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      __syncthreads();
+      if ((int)threadIdx.x < kpt) {
+        ids_out[(size_t)tok * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
+        ws_out[(size_t)tok * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+      }
+    }
+    return;
+  }
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int U = d / 64;
+  const bool shared = s >= kpt;
+  int e = 0;
+  if (!shared) {
+    const float* lg = logits + (size_t)tok * n_experts;
+    if (!topk_ids_by_logit<NPL>(lg, sel_ids, n_experts, kpt)) {
+      topk_block<NPL, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
+      __syncthreads();
+    }
+    e = sel_ids[s];
+  }
+  const int t = shared ? A.tsh : A.tgu;
+  const uint64_t rb = ggu_row_bytes(t, (uint64_t)d);
+  const uint8_t* gbase = shared ? A.sh_gate : A.gate + (uint64_t)e * mid * rb;
+  const uint8_t* ubase = shared ? A.sh_up : A.up + (uint64_t)e * mid * rb;
+  const int r0 = blockIdx.x * G4_ROWS + 4 * wv;
+  const bool live = lane < U;
+  const int ul = live ? lane : (lane & 3);
+  const float mlive = live ? 1.f : 0.f;
+  XU x;
+  load_xu(x, xplanes, xmeta, ((size_t)tok * U + ul) * 2);
+  float acc[8];
+  GGU_SWITCH(t, ggu_gu_rows<T>(gbase, ubase, r0, d, ul, mlive, x, acc));
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      gs[4 * wv + i] = acc[i];
+      us[4 * wv + i] = acc[4 + i];
+    }
+  }
+  __syncthreads();
+  if (wv == 0) {  // SwiGLU on the block's 32 rows = one activation group of the down projection; quantise it
+    const int j = lane & 31;
+    const float g = gs[j], u = us[j];
+    const float hv = g / (1.f + expf(-g)) * u;
+    float m = dpp_max_row(fabsf(hv));
+    m = rows_half_max(m);
+    const float inv = m > 0.f ? QV_XMAX / m : 0.f;
+    const float q = m * (1.f / QV_XMAX);
+    const int X = (int)rintf(hv * inv);
+    int p0, p1;
+    qv_digits(X, p0, p1);
+    float sx = dpp_add_row((float)X);
+    sx = rows_half_add(sx);
+    if (lane < QV_GROUP_DW) pk[lane] = 0;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    if (lane < 32) {
+      const int dw = j >> 2, sh = 8 * (j & 3);
+      atomicOr(&pk[dw], (uint32_t)(p0 & 0xff) << sh);
+      atomicOr(&pk[8 + dw], (uint32_t)(p1 & 0xff) << sh);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_wave_barrier();
+    const size_t gi = ((size_t)tok * nslots + s) * (mid / 32) + blockIdx.x;
+    if (lane < QV_GROUP_DW) hplanes[gi * QV_GROUP_DW + lane] = pk[lane];
+    if (lane == 0) hmeta[gi] = make_float2(q, q * sx);
+  }
+}
+
+struct DnGgArgs {
+  const uint8_t *down, *sh_down;
+  const float* sh_logit;
+  int tdn, tsh;
+};
+
+// D4_ROWS output rows of one wave's slots: a row of 16 lanes = one slot
+template <int T>
+__device__ __forceinline__ void ggu_dn_rows(const uint8_t* base, int mid, int ul, float mlive, const XU& x, bool store,
+                                            float* part_s) {
+  constexpr int RB = ggu_batch<T>();
+  const uint64_t rb = ggu_row_bytes(T, (uint64_t)mid);
+  const int jj = ul & 3;
+#pragma unroll
+  for (int h = 0; h < D4_ROWS; h += RB) {
+    GgU<T> u[RB];
+#pragma unroll
+    for (int r = 0; r < RB; r++) ggu_fetch<T>(base + (uint64_t)(h + r) * rb, ul, u[r]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int r = 0; r < RB; r++) {
+      const float v = dpp_add_row(ggu_dot<T>(u[r], jj, x) * mlive);
+      if (store) part_s[h + r] = v;
+      if (r & 1) __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+// grid (d/D4_ROWS, P); block = 64 x (ceil(kpt/4) + 1 with a shared expert): waves 0.. hold four routed slots each (a row
+// of 16 lanes per slot), the last wave the shared expert alone, so that a wave's block type is uniform.
+__global__ void __launch_bounds__(320) k_decgg_dn(DnGgArgs A, const uint32_t* __restrict__ hplanes,
+                                                  const float2* __restrict__ hmeta, const int* __restrict__ ids,
+                                                  const float* __restrict__ ws, int id_stride, int kpt, int d, int mid,
+                                                  float* __restrict__ out, uint64_t out_stride) {
+  __shared__ float part[D4_MAXSLOTS + 1][D4_ROWS];
+  __shared__ float wsm[D4_MAXSLOTS + 1];
+  const int tok = blockIdx.y;
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const bool has_shared = A.sh_down != nullptr;
+  const int nslots = kpt + (has_shared ? 1 : 0), rw = (kpt + 3) >> 2;  // rw: waves of routed slots
+  const int U = mid / 64, u_raw = lane & 15;
+  const int r0 = blockIdx.x * D4_ROWS;
+  float wmine = 0.f;
+  if ((int)threadIdx.x < nslots)
+    wmine = (int)threadIdx.x < kpt ? ws[(size_t)tok * id_stride + threadIdx.x] : A.sh_logit[tok];
+  {
+    const bool shw = wv >= rw;  // the shared expert's wave (its slot in lanes 0..15)
+    const int s_raw = shw ? kpt + (lane >> 4) * D4_MAXSLOTS : 4 * wv + (lane >> 4);  // lanes 16.. of that wave: no slot
+    const bool okslot = shw ? (lane >> 4) == 0 : s_raw < kpt;
+    const bool live = okslot && u_raw < U;
+    const int s = okslot ? s_raw : (shw ? kpt : 0);
+    const int ul = u_raw < U ? u_raw : (u_raw & 3);
+    const float mlive = live ? 1.f : 0.f;
+    const int t = shw ? A.tsh : A.tdn;
+    const uint64_t rb = ggu_row_bytes(t, (uint64_t)mid);
+    const int e = shw ? 0 : ids[(size_t)tok * id_stride + s];
+    const uint8_t* base = (shw ? A.sh_down : A.down + (uint64_t)e * d * rb) + (uint64_t)r0 * rb;
+    XU x;
+    load_xu(x, hplanes, hmeta, (((size_t)tok * nslots + s) * U + ul) * 2);
+    GGU_SWITCH(t, ggu_dn_rows<T>(base, mid, ul, mlive, x, u_raw == 0 && okslot, part[s]));
+  }
+  if ((int)threadIdx.x < nslots) wsm[threadIdx.x] = (int)threadIdx.x < kpt ? wmine : sigmoid_f(wmine);
+  __syncthreads();
+  if (threadIdx.x < D4_ROWS) {
+    const int r = threadIdx.x;
+    float y = 0.f;
+    for (int i = 0; i < kpt; i++) y += wsm[i] * part[i][r];
+    if (has_shared) y += wsm[kpt] * part[kpt][r];
+    out[(size_t)tok * out_stride + r0 + r] = y;
+  }
+}
+
 }  // namespace
 
 bool moe_dec4k_supported(int d, int mid, int nslots) {
@@ -346,6 +672,50 @@ int moe_launch_dec4k_dn(const uint8_t* down, const uint8_t* sh_down, const float
   const int nslots = kpt + (sh_down ? 1 : 0);
   dim3 grid(d / D4_ROWS, P);
   k_dec4k_dn<<<grid, 64 * ((nslots + 3) / 4), 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// ---- any mix of Q4_K / Q5_K / Q8_0 / Q5_1 (integer-dot kernels above) ----
+static bool ggu_type(int t) { return t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K || t == MOE_GGML_Q8_0 || t == MOE_GGML_Q5_1; }
+bool moe_decgg_supported(int tgu, int tdn, int tsh, bool has_shared, int d, int mid, int kpt, int n_experts) {
+  if (!ggu_type(tgu) || !ggu_type(tdn) || (has_shared && !ggu_type(tsh))) return false;
+  // (whole 256-element super-blocks in both directions also cover the 64-weight units of the 32-element types)
+  return d % 256 == 0 && d / 64 <= 64 && mid % 256 == 0 && mid / 64 <= 16 && kpt + 1 <= D4_MAXSLOTS &&
+         mid % G4_ROWS == 0 && d % D4_ROWS == 0 && ((kpt + 3) / 4 + 1) * 64 <= 320 && n_experts <= 1024 && kpt <= 64 &&
+         kpt <= n_experts;
+}
+static size_t ggu_align(int t) { return t == MOE_GGML_Q8_0 ? 4 : 16; }
+
+int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
+                             const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const float* logits,
+                             int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st) {
+  if (!gate || !up || !xplanes || !xmeta || !logits || !ids || !ws || !hplanes || !hmeta || (!sh_gate != !sh_up))
+    return MOE_E_INVALID;
+  if (!moe_decgg_supported(tgu, tgu, tsh, sh_gate != nullptr, d, mid, kpt, n_experts)) return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(gate, ggu_align(tgu)) || !moe_aligned(up, ggu_align(tgu)) ||
+      (sh_gate && (!moe_aligned(sh_gate, ggu_align(tsh)) || !moe_aligned(sh_up, ggu_align(tsh)))))
+    return MOE_E_INVALID;
+  GuGgArgs A{gate, up, sh_gate, sh_up, tgu, tsh};
+  dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);
+  if (n_experts <= 512)
+    k_decgg_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws);
+  else
+    k_decgg_gu<16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_decgg_dn(int tdn, int tsh, const uint8_t* down, const uint8_t* sh_down, const float* sh_logit,
+                        const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws, int id_stride,
+                        int kpt, int P, int d, int mid, float* out, uint64_t out_stride, hipStream_t st) {
+  if (!down || !hplanes || !hmeta || !ids || !ws || !out || (sh_down && !sh_logit)) return MOE_E_INVALID;
+  if (!moe_aligned(down, ggu_align(tdn)) || (sh_down && !moe_aligned(sh_down, ggu_align(tsh)))) return MOE_E_INVALID;
+  DnGgArgs A{down, sh_down, sh_logit, tdn, tsh};
+  dim3 grid(d / D4_ROWS, P);
+  k_decgg_dn<<<grid, 64 * ((kpt + 3) / 4 + (sh_down ? 1 : 0)), 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid,
+                                                                        out, out_stride);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -108,6 +108,14 @@ int moe_launch_dec_dn_uq(const moe_wview* dn, const moe_wview* sh_down, const ui
                          int n_experts, int d, int mid, float* pairs, hipStream_t st);
 // the same for raw GGUF Q4_K rows (activation planes in natural order)
 bool moe_dec4k_supported(int d, int mid, int nslots);
+bool moe_decgg_supported(int tgu, int tdn, int tsh, bool has_shared, int d, int mid, int kpt, int n_experts);
+int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
+                             const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const float* logits,
+                             int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st);
+int moe_launch_decgg_dn(int tdn, int tsh, const uint8_t* down, const uint8_t* sh_down, const float* sh_logit,
+                        const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws, int id_stride,
+                        int kpt, int P, int d, int mid, float* out, uint64_t out_stride, hipStream_t st);
 int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
                              const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                              int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,

@@ -186,11 +186,13 @@ def test_decode_topk_wide_logit_range(oracle, fmt):
 
 
 @pytest.mark.parametrize("tgu,tdn,tsh,T", [(13, 8, 12, 1), (12, 7, 12, 5), (13, 7, 8, 3), (12, 8, 13, 40), (23, 20, 12, 2),
-                                            (20, 23, 23, 7)])
+                                            (20, 23, 23, 7), (13, 8, 8, 1), (13, 8, 8, 20), (12, 7, 7, 32), (8, 13, 7, 2)])
 def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
-    """GGUF layers in the type mix of the reference's checkpoints (Q4_K / Q5_K gate and up, Q5_1 / Q8_0 down,
-    src/gpu/parts/30_host_util.inc:399-405): the general f32 GEMV kernels, ids bit-exact, output within the GEMV
-    bar; T = 40 is a batch for the general grouped GEMM."""
+    """GGUF layers in the type mix of the reference's checkpoints (Q4_K / Q5_K gate and up, Q5_1 / Q8_0 down, a Q8_0
+    shared expert; src/gpu/parts/30_host_util.inc:399-405, src/gguf_map.h:212-214): mixes of Q4_K / Q5_K / Q8_0 /
+    Q5_1 take the integer-dot decode kernels (and, with MOE_OPT_INT_DECODE = 0, like the IQ4 types, the general f32
+    GEMV kernels); ids bit-exact; T = 40 is a batch for the general grouped GEMM."""
+    from gfx1151_engine_amd import capi
     rng = np.random.default_rng(tgu * 100 + tdn * 10 + T)
     d, mid, E, k = 512, 256, 12, 4
     hl = HostLayer(rng, d, mid, E, k, fmt="q4k", gg_types=(tgu, tdn, tsh))
@@ -198,10 +200,17 @@ def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
     yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
     m, dev = hl.to_gpu(max_tokens=64)
     y = m.forward(0, gpu(x)).cpu().numpy()
-    ids, _ = m.last_routing(T)
+    ids, ws = m.last_routing(T)
     assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    assert np.abs(ws.cpu().numpy()[:, :k] - wo[:, :k]).max() <= 1e-6
+    int_types = all(t in (12, 13, 8, 7) for t in (tgu, tdn, tsh))
     # batches over 32 tokens take the general grouped GEMM (f16 MFMA operands): the batch tolerance
-    assert max_abs_rel(y, yo) <= (TOL_GEMV if T <= 32 else 2e-3), max_abs_rel(y, yo)
+    tol = 2e-3 if T > 32 else (TOL_INT_Q4K if int_types else TOL_GEMV)
+    assert max_abs_rel(y, yo) <= tol, max_abs_rel(y, yo)
+    if T <= 32:
+        m.set_option(capi.OPT_INT_DECODE, 0)
+        y2 = m.forward(0, gpu(x)).cpu().numpy()
+        assert max_abs_rel(y2, yo) <= TOL_GEMV, max_abs_rel(y2, yo)
     m.close()
 
 
