@@ -11,6 +11,7 @@ import torch
 from .build import LIB
 
 F32, BF16, Q4CP, Q8G64, Q8G32 = 1, 0, 5, 7, 8
+I4R = 23  # hgn v2 routed experts
 GGML_Q4_K = 12
 GGML_Q5_K, GGML_Q5_1, GGML_Q8_0 = 13, 7, 8
 
@@ -196,6 +197,7 @@ class LutW(C.Structure):
 
 
 LUT_Q4CP = 100
+LUT_I4R = 101
 ROUTING_STATIC_MAX_TOKENS = 32768
 DENSE_SHARED = True  # moe_set_shared takes bf16 / f32 / q8g64 matrices
 OPT_INT_DECODE = 1
@@ -212,6 +214,53 @@ def lut_q4cp_view(blob, rows, cols, e_rows, up_off):
           "moe_lut_q4cp_view")
     p._keep = blob
     return p
+
+
+def lut_i4r_view(blob, rows, cols, e_rows, up_off=0):
+    p = LutW()
+    check(lib().moe_lut_i4r_view(ptr(blob), u64(rows), u64(cols), e_rows, up_off, C.byref(p)), "moe_lut_i4r_view")
+    p._keep = blob
+    return p
+
+
+def i4r_dequant_rows(blob, rows, cols, row0, nrows):
+    out = torch.empty((nrows, cols), dtype=torch.float32, device=blob.device)
+    check(lib().moe_i4r_dequant_rows(ptr(blob), u64(rows), u64(cols), u64(row0), u64(nrows), ptr(out), stream()),
+          "moe_i4r_dequant_rows")
+    return out
+
+
+def v2_rot(x, pre=None, post=None, out_f16=False):
+    """post * H(pre * x) / sqrt(128) per 128 block of every row; f32 rows, or f16 rows in layout 1."""
+    P, n = x.shape
+    y = torch.empty((P, n), dtype=torch.float16 if out_f16 else torch.float32, device=x.device)
+    check(lib().moe_v2_rot(ptr(x), u64(n), ptr(y), u64(n), ptr(pre), ptr(post), n, P, 1 if out_f16 else 0, stream()),
+          "moe_v2_rot")
+    return y
+
+
+def i4r_mid(guv, svh_gu, suh_dn, mid, out_f16=False):
+    """guv [nslots][2 mid] (f32 or f16) -> the rotated down-projection input [nslots][mid] (f32, or f16 in layout 1)."""
+    n = guv.shape[0]
+    out = torch.empty((n, mid), dtype=torch.float16 if out_f16 else torch.float32, device=guv.device)
+    check(lib().moe_i4r_mid(ptr(guv), 1 if guv.dtype == torch.float16 else 0, u64(guv.shape[1]), ptr(out),
+                            1 if out_f16 else 0, u64(mid), ptr(svh_gu), ptr(suh_dn), mid, n, stream()), "moe_i4r_mid")
+    return out
+
+
+def lut_up_raw(p, x16, tokidx, tiles_t, ntiles, mid, npairs):
+    guv = torch.full((npairs, 2 * mid), float("nan"), dtype=torch.float16, device=x16.device)
+    check(lib().moe_lut_up_raw(LUT_I4R, C.byref(p), ptr(x16), ptr(tokidx), ptr(tiles_t), ptr(ntiles), tiles_t.shape[0],
+                               ptr(guv), mid, x16.shape[1], stream()), "moe_lut_up_raw")
+    return guv
+
+
+def v2_reduce_rot(pairs, pairids, pw, svh, P, K, ey=None, sg=None):
+    D = pairs.shape[1]
+    out = torch.empty((P, D), dtype=torch.float32, device=pairs.device)
+    check(lib().moe_v2_reduce_rot(ptr(pairs), 1 if pairs.dtype == torch.float16 else 0, ptr(pairids), ptr(pw), ptr(svh),
+                                  ptr(ey), ptr(sg), ptr(out), P, D, K, stream()), "moe_v2_reduce_rot")
+    return out
 
 
 def f32_to_f16(x, layout=1):
@@ -270,11 +319,11 @@ def lut_up(p, x16, tokidx, tiles_t, ntiles, mid, npairs):
     return hid
 
 
-def lut_down(p, hid16, tiles_t, ntiles, d, f16=True):
+def lut_down(p, hid16, tiles_t, ntiles, d, f16=True, lut_type=LUT_Q4CP):
     npairs = hid16.shape[0]
     pairs = torch.full((npairs, d), float("nan"), dtype=torch.float16 if f16 else torch.float32,
                        device=hid16.device)
-    check(lib().moe_lut_down(LUT_Q4CP, C.byref(p), ptr(hid16), ptr(tiles_t), ptr(ntiles), tiles_t.shape[0],
+    check(lib().moe_lut_down(lut_type, C.byref(p), ptr(hid16), ptr(tiles_t), ptr(ntiles), tiles_t.shape[0],
                              ptr(pairs), d, hid16.shape[1], 1 if f16 else 0, stream()), "moe_lut_down")
     return pairs
 
@@ -313,6 +362,12 @@ class Moe:
         self._keep += [gate_up, down]
         check(lib().moe_set_experts_q4cp(self.h, layer, C.byref(gate_up), C.byref(down)),
               "moe_set_experts_q4cp")
+
+    def set_experts_i4r(self, layer, gate_up, down, su, svh_gu, suh_dn, svh_dn):
+        """hgn v2 routed experts: I4R views and the four sign-scale planes as f32 device tensors."""
+        self._keep += [gate_up, down, su, svh_gu, suh_dn, svh_dn]
+        check(lib().moe_set_experts_i4r(self.h, layer, C.byref(gate_up), C.byref(down), ptr(su), ptr(svh_gu),
+                                        ptr(suh_dn), ptr(svh_dn)), "moe_set_experts_i4r")
 
     def set_experts_gguf(self, layer, gate, up, down, tgu=GGML_Q4_K, tdn=GGML_Q4_K):
         self._keep += [gate, up, down]

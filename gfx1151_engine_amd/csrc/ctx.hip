@@ -23,6 +23,9 @@ struct MoeLayer {
   // f16 range guard of the batch path: typical |hid| (and |pair|) per unit mean-square activation,
   // estimated from sampled weight rows when the weights are registered
   float c_routed = 0.f, c_shared = 0.f;
+  // hgn v2 rotated experts (gate_up / down are MOE_DT_I4R views): the sign-scale planes of the two tensors, f32
+  bool has_i4r = false;
+  const float *v2_su = nullptr, *v2_svh_gu = nullptr, *v2_suh_dn = nullptr, *v2_svh_dn = nullptr;
 };
 
 // cb[n] == a*n + b for all 16 codes?  Reads the 64-byte codebook back from the device: weight
@@ -93,6 +96,15 @@ struct moe_ctx {
   // batch router through candidate selection (exact ids at a fraction of the fp64 work); its scratch
   bool router_cand = true;
   void* rc_scratch = nullptr;
+  // hgn v2 layers (allocated when the first one is registered): unfused gate | up sums and the rotated activations'
+  // planes of the small-batch path, the routed sum and the shared expert's rows ahead of the last rotation; the
+  // rotated f16 activations and the unfused f16 gate | up rows of the batch path
+  float* v2_zraw = nullptr;      // [min(T,small_max)][k][2 mid]
+  uint32_t* v2_xplanes = nullptr;
+  float2* v2_xmeta = nullptr;
+  float *v2_acc = nullptr, *v2_ey = nullptr;  // [min(T,small_max)][d] each
+  __half* v2_x16 = nullptr;      // [T][d]
+  __half* v2_z16 = nullptr;      // [kT][2 mid]
 };
 
 static void prof_mark(moe_ctx* c, int stage_done, hipStream_t st) {
@@ -126,7 +138,8 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->ev_x16) (void)hipEventDestroy(c->ev_x16);
   if (c->side) (void)hipStreamDestroy(c->side);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->kpart, c->ktickets, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
-                  c->pairids, c->tiles, c->ntiles, c->tiles_sh, c->ntiles_sh, c->hid16, c->pairs16, c->pairs32, c->rc_scratch};
+                  c->pairids, c->tiles, c->ntiles, c->tiles_sh, c->ntiles_sh, c->hid16, c->pairs16, c->pairs32, c->rc_scratch,
+                  c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16};
   for (void* b : bufs)
     if (b) {
       hipError_t e = hipFree(b);
@@ -245,6 +258,56 @@ MOE_API int moe_set_experts_q4cp(moe_ctx* c, int layer, const moe_wview* gu, con
   L->down = *dn;
   L->has_q4cp = true;
   L->has_gguf = false;
+  L->has_i4r = false;
+  return MOE_OK;
+}
+
+// hgn v2 routed experts (reference: v2_init, src/gpu/parts/30_host_util.inc:818-870; moe_b_v2's shape checks,
+// 40_model.inc:4574-4576)
+MOE_API int moe_set_experts_i4r(moe_ctx* c, int layer, const moe_wview* gu, const moe_wview* dn, const float* su,
+                                const float* svh_gu, const float* suh_dn, const float* svh_dn) {
+  MoeLayer* L = layer_of(c, layer);
+  if (!L || !gu || !dn || !gu->data || !dn->data || !su || !svh_gu || !suh_dn || !svh_dn) return MOE_E_INVALID;
+  if (gu->dtype != MOE_DT_I4R || dn->dtype != MOE_DT_I4R) return MOE_E_UNSUPPORTED;
+  const moe_config& g = c->cfg;
+  if (gu->rows != (uint64_t)g.experts * 2 * g.mid || (int)gu->cols != g.d || dn->rows != (uint64_t)g.experts * g.d ||
+      (int)dn->cols != g.mid)
+    return MOE_E_INVALID;
+  if (!moe_v2_shapes_ok(g.d, g.mid) || !moe_dec_supported(g.d, g.mid, g.topk + 1) ||
+      !moe_dec_gu_topk_supported(g.experts, g.topk))
+    return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(gu->data, 16) || !moe_aligned(dn->data, 16) || !moe_aligned(su, 16) || !moe_aligned(svh_gu, 16) ||
+      !moe_aligned(suh_dn, 16) || !moe_aligned(svh_dn, 16))
+    return MOE_E_INVALID;
+  if (!moe_i4r_codebook()) return MOE_E_STATE;
+  if (!c->v2_zraw) {  // set-up work: the scratch of these layers
+    const size_t T = (size_t)g.max_tokens, Ts = T < (size_t)c->small_max ? T : (size_t)c->small_max;
+    hipError_t e = hipMalloc(&c->v2_zraw, Ts * g.topk * 2 * g.mid * 4);
+    if (e == hipSuccess) e = hipMalloc(&c->v2_xplanes, Ts * moe_qvec_plane_bytes(g.d));
+    if (e == hipSuccess) e = hipMalloc(&c->v2_xmeta, Ts * moe_qvec_meta_bytes(g.d));
+    if (e == hipSuccess) e = hipMalloc(&c->v2_acc, Ts * (size_t)g.d * 4);
+    if (e == hipSuccess) e = hipMalloc(&c->v2_ey, Ts * (size_t)g.d * 4);
+    if (e == hipSuccess && c->x16) {
+      e = hipMalloc(&c->v2_x16, T * (size_t)g.d * 2);
+      if (e == hipSuccess) e = hipMalloc(&c->v2_z16, T * g.topk * 2 * (size_t)g.mid * 2);
+    }
+    if (e != hipSuccess) {
+      void* bufs[] = {c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16};
+      for (void* b : bufs)
+        if (b) (void)hipFree(b);
+      c->v2_zraw = nullptr; c->v2_xplanes = nullptr; c->v2_xmeta = nullptr; c->v2_acc = c->v2_ey = nullptr;
+      c->v2_x16 = c->v2_z16 = nullptr;
+      return (int)e;
+    }
+  }
+  L->gate_up = *gu;
+  L->down = *dn;
+  L->v2_su = su; L->v2_svh_gu = svh_gu; L->v2_suh_dn = suh_dn; L->v2_svh_dn = svh_dn;
+  L->c_routed = 0.f;  // (no f16 range guard on these launches: the reference's have none either)
+  L->experts_affine = true;
+  L->has_i4r = true;
+  L->has_q4cp = false;
+  L->has_gguf = false;
   return MOE_OK;
 }
 
@@ -270,6 +333,7 @@ MOE_API int moe_set_experts_gguf(moe_ctx* c, int layer, const moe_gg_experts* gg
   L->gg = *gg;
   L->has_gguf = true;
   L->has_q4cp = false;
+  L->has_i4r = false;
   return MOE_OK;
 }
 
@@ -426,8 +490,10 @@ MOE_API int moe_get_routing(moe_ctx* c, int P, int* ids_out, float* ws_out, moe_
 // down + weighted combine + shared expert.
 static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st);
 
+static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st);
+
 static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
-  const int rc = forward_small_routed(c, L, x, P, y, st);
+  const int rc = L.has_i4r ? forward_small_v2(c, L, x, P, y, st) : forward_small_routed(c, L, x, P, y, st);
   if (rc || !L.has_shared || !L.sh_dense) return rc;
   // a densely stored shared expert: added to y behind the routed experts' kernels (its gate logit is in
   // sh_logit since the router launch); scratch: the shared slot's part of hid32
@@ -601,6 +667,55 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
   return MOE_OK;
 }
 
+// hgn v2 rotated experts, small batches (reference: moe_v2_1, 40_model.inc:1638-1656): the integer-dot launches of
+// the q4cp path with the rotations in between --
+//   router logits (+ planes of x for the shared expert's slot) -> planes of rot_in(x, su)
+//   -> gate | up sums of the routed slots, unfused (the shared expert's slot as usual)
+//   -> per slot rot_out(svh_gu), SwiGLU, rot_in(suh_dn) -> planes
+//   -> down + weighted sum (the shared expert's rows aside) -> rot_out(svh_dn) + shared expert.
+static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
+  const moe_config& g = c->cfg;
+  int rc;
+  c->ev_n = 0;
+  prof_mark(c, 0, st);
+  auto stage = [&](int tag, auto&& launch) -> int {
+    if (c->skip_stage != tag + 1) {
+      const int e = launch();
+      if (e) return e;
+    }
+    prof_mark(c, tag, st);
+    return MOE_OK;
+  };
+  const bool sh = L.has_shared && !L.sh_dense;  // a q4cp shared expert rides in these kernels as one more slot
+  if (sh && (L.sh_gguf_type != 0 || !L.shared_affine)) return MOE_E_UNSUPPORTED;
+  const int nslots_d = g.topk + (sh ? 1 : 0);
+  if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
+         bool fused = false;
+         const int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
+                                               c->sh_logit, sh ? c->xplanes : nullptr, c->xmeta, false, nullptr, c->ids,
+                                               c->ws, g.topk, g.id_stride, &fused, st, c->kpart, c->ktickets);
+         return e ? e : moe_launch_v2_rot(x, (uint64_t)g.d, P, g.d, L.v2_su, nullptr, 2, nullptr, 0, nullptr, 0,
+                                          c->v2_xplanes, c->v2_xmeta, st);
+       })))
+    return rc;
+  const moe_wview *shg = sh ? &L.sh_gate : nullptr, *shu = sh ? &L.sh_up : nullptr, *shd = sh ? &L.sh_down : nullptr;
+  if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+         const moe_dec_v2 v2{c->v2_zraw, c->v2_xplanes, c->v2_xmeta};
+         const int e = moe_launch_dec_gu_topk(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->logits, g.experts, c->ids,
+                                              c->ws, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st,
+                                              &v2);
+         return e ? e : moe_launch_i4r_mid(c->v2_zraw, false, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu,
+                                           L.v2_suh_dn, 2, nullptr, 0, g.topk, nslots_d, c->hplanes, c->hmeta, st);
+       })))
+    return rc;
+  return stage(MOE_PROF_DOWN, [&]() -> int {
+    const int e = moe_launch_dec_dn(&L.down, shd, c->sh_logit, c->hplanes, c->hmeta, c->ids, c->ws, g.id_stride, g.topk, P,
+                                    g.d, g.mid, c->v2_acc, (uint64_t)g.d, st, sh ? c->v2_ey : nullptr);
+    return e ? e : moe_launch_v2_rot(c->v2_acc, (uint64_t)g.d, P, g.d, nullptr, L.v2_svh_dn, 0, y, (uint64_t)g.d,
+                                     sh ? c->v2_ey : nullptr, (uint64_t)g.d, nullptr, nullptr, st);
+  });
+}
+
 // Which grouped GEMM a layer's batches take: 0 = q4cp (tuned), 1 = raw GGUF Q4_K throughout (tuned), 2 = raw GGUF
 // blocks of any supported type (general kernel, f16 operands in natural order).
 static int batch_gemm_kind(const MoeLayer& L) {
@@ -631,6 +746,10 @@ static int router_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* o
 static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
   const moe_config& g = c->cfg;
   const bool q4k = L.has_gguf;  // raw GGUF blocks
+  // hgn v2 rotated experts (reference: moe_b_v2, 40_model.inc:4570-4686): the routed launches read rot_in(x, su),
+  // leave gate | up unfused for the rotations around SwiGLU, and the combine rotates the weighted sum
+  const bool v2 = L.has_i4r;
+  if (v2 && (!c->v2_x16 || g.d % 256 || g.mid % 256)) return MOE_E_UNSUPPORTED;
   // gen: a GGUF layer that is not Q4_K throughout takes the general grouped GEMM (any supported block type,
   // dequantised into f16 tiles in LDS); Q4_K-only and q4cp layers take the tuned kernel
   const bool gen = batch_gemm_kind(L) == 2;
@@ -647,6 +766,10 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
       sgu.w = L.sh_gate.data; sgu.w_up = L.sh_up.data; sgu.e_rows = g.mid;
       sdn.w = L.sh_down.data; sdn.e_rows = g.d;
     }
+  } else if (v2) {
+    int e = moe_lut_i4r_view(L.gate_up.data, L.gate_up.rows, L.gate_up.cols, 2 * g.mid, 0, &gu);
+    if (!e) e = moe_lut_i4r_view(L.down.data, L.down.rows, L.down.cols, g.d, 0, &dn);
+    if (e) return e;
   } else {
     moe_lut_q4cp_view(L.gate_up.data, L.gate_up.rows, L.gate_up.cols, L.gate_up.scale_stride, 2 * g.mid, g.mid, &gu);
     moe_lut_q4cp_view(L.down.data, L.down.rows, L.down.cols, L.down.scale_stride, g.d, 0, &dn);
@@ -676,6 +799,15 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
       return moe_launch_gemm_gg(true, L.gg.tgu, L.gg.gate, L.gg.up, L.sh_gguf_type, with_sh ? L.sh_gate.data : nullptr,
                                 with_sh ? L.sh_up.data : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid,
                                 g.d, hs, s2);
+    if (v2 && !with_sh) {  // the routed experts' tiles: plain rows of the fused tensor, then the slot-wise middle
+      const int e = moe_launch_gemm_q4cp(false, &gu, nullptr, g.experts, c->v2_x16, c->tokidx, tl, ntl, mt, c->v2_z16,
+                                         2 * g.mid, g.d, true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
+      return e ? e : moe_launch_i4r_mid(c->v2_z16, true, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu, L.v2_suh_dn,
+                                        1, c->hid16, (uint64_t)g.mid, 1, 1, nullptr, nullptr, s2);
+    }
+    if (v2)  // the shared expert's own tile list (q4cp, not rotated; every tile's expert index is >= n_experts)
+      return moe_launch_gemm_q4cp(true, &sgu, &sgu, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, true,
+                                  false, hs, s2, nullptr, sh_cb_up);
     return moe_launch_gemm_q4cp(true, &gu, with_sh ? &sgu : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16,
                                 g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up);
   };
@@ -686,11 +818,17 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     if (gen)
       return moe_launch_gemm_gg(false, L.gg.tdn, L.gg.down, nullptr, L.sh_gguf_type, with_sh ? L.sh_down.data : nullptr,
                                 nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2);
+    if (v2 && !with_sh)
+      return moe_launch_gemm_q4cp(false, &dn, nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid,
+                                  true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
+    if (v2)
+      return moe_launch_gemm_q4cp(false, &sdn, &sdn, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid,
+                                  true, false, hs, s2, nullptr);
     return moe_launch_gemm_q4cp(false, &dn, with_sh ? &sdn : nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt,
                                 cmb ? (void*)cmb->y : (void*)c->pairs16, g.d, g.mid, cmb == nullptr, q4k, hs, s2, cmb);
   };
-  const bool fused = c->fused_combine && !c->hc && !gen && !shd;  // the HC write-back belongs to the ordered combine
-  if (L.has_shared && (shd || (c->shared_aside && !fused))) {
+  const bool fused = c->fused_combine && !c->hc && !gen && !shd && !v2;  // the HC write-back belongs to the ordered combine
+  if (v2 || (L.has_shared && (shd || (c->shared_aside && !fused)))) {
     // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
     // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
     // side stream also makes what both streams need first: the per-token mean square of x (range guard) and
@@ -700,13 +838,18 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     const int max_tiles = (P * g.topk + 127) / 128 + g.experts;
     MOE_HIP(hipEventRecord(c->ev_fork, st));
     MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
-    int rs = c->x16_ext ? moe_launch_meansq_f16(xh, P, g.d, c->xms, c->side)
-                        : moe_launch_f16_rows_meansq(x, c->x16, P, g.d, xl, c->xms, c->side);
+    int rs = MOE_OK;
+    if (v2) rs = moe_launch_v2_rot(x, (uint64_t)g.d, P, g.d, L.v2_su, nullptr, 1, c->v2_x16, (uint64_t)g.d, nullptr, 0, nullptr, nullptr, c->side);
+    if (!rs && (!v2 || L.has_shared))
+      rs = c->x16_ext ? moe_launch_meansq_f16(xh, P, g.d, c->xms, c->side)
+                      : moe_launch_f16_rows_meansq(x, c->x16, P, g.d, xl, c->xms, c->side);
     hipError_t ee = hipEventRecord(c->ev_x16, c->side);
     if (!rs && ee != hipSuccess) rs = (int)ee;
-    if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, moe_gemm_tile_cap(), P, sh_first, c->tokidx, c->side);
-    if (!rs) rs = gemm_up(true, c->tiles_sh, c->ntiles_sh, max_tiles_sh, c->side);
-    if (!rs) rs = gemm_dn(true, c->tiles_sh, c->ntiles_sh, max_tiles_sh, c->side, nullptr);
+    if (L.has_shared) {
+      if (!rs) rs = moe_launch_tiles_only_shared(c->tiles_sh, c->ntiles_sh, g.experts, moe_gemm_tile_cap(), P, sh_first, c->tokidx, c->side);
+      if (!rs) rs = gemm_up(true, c->tiles_sh, c->ntiles_sh, max_tiles_sh, c->side);
+      if (!rs) rs = gemm_dn(true, c->tiles_sh, c->ntiles_sh, max_tiles_sh, c->side, nullptr);
+    }
     // caller's stream: router, top-k, permutation, the routed experts' GEMMs
     rc = router_batch(c, L, x, P, nullptr, st);
     prof_mark(c, MOE_PROF_ROUTER, st);
@@ -727,8 +870,10 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     if (rc) return rc;
     if (rs) return rs;
     if (ee != hipSuccess) return (int)ee;
-    rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, c->sh_logit, sh_first, y, P, g.d, g.topk, hs,
-                           st, c->hc);
+    rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
+                           L.has_shared ? sh_first : -1, y, P, g.d, g.topk,
+                           v2 ? moe_hscale{L.has_shared ? c->xms : nullptr, 0.f, L.c_shared} : hs, st, c->hc,
+                           v2 ? L.v2_svh_dn : nullptr);
     prof_mark(c, MOE_PROF_REDUCE, st);
     return rc;
   }
@@ -776,7 +921,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
 MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, moe_stream_t st) {
   MoeLayer* L = layer_of(c, layer);
   if (!L || !x || !y || P < 0) return MOE_E_INVALID;
-  if (!L->has_router || !(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
+  if (!L->has_router || !(L->has_q4cp || L->has_gguf || L->has_i4r)) return MOE_E_STATE;
   if (P > c->cfg.max_tokens) return MOE_E_STATE;
   if (!moe_aligned(x, 16) || !moe_aligned(y, 16)) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
@@ -800,7 +945,7 @@ MOE_API int moe_forward_hc(moe_ctx* c, int layer, const float* x, int P, const f
                            moe_stream_t st) {
   MoeLayer* L = layer_of(c, layer);
   if (!L || !x || !w4 || !R || P < 0) return MOE_E_INVALID;
-  if (!L->has_router || !(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
+  if (!L->has_router || !(L->has_q4cp || L->has_gguf || L->has_i4r)) return MOE_E_STATE;
   if (P > c->cfg.max_tokens) return MOE_E_STATE;
   if (!moe_aligned(x, 16) || !moe_aligned(R, 16)) return MOE_E_INVALID;
   if (P <= c->small_max) return MOE_E_UNSUPPORTED;
@@ -817,7 +962,7 @@ MOE_API int moe_forward_hc(moe_ctx* c, int layer, const float* x, int P, const f
 MOE_API int moe_x16_layout(moe_ctx* c, int layer) {
   MoeLayer* L = layer_of(c, layer);
   if (!L) return MOE_E_INVALID;
-  if (!(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
+  if (!(L->has_q4cp || L->has_gguf || L->has_i4r)) return MOE_E_STATE;
   const int kind = batch_gemm_kind(*L);
   return kind == 0 ? 1 : kind == 1 ? 2 : 0;
 }
@@ -827,10 +972,11 @@ MOE_API int moe_x16_layout(moe_ctx* c, int layer) {
 MOE_API int moe_forward_x16(moe_ctx* c, int layer, const float* x, const void* x16, int P, float* y, moe_stream_t st) {
   MoeLayer* L = layer_of(c, layer);
   if (!L || !x || !x16 || !y || P < 0) return MOE_E_INVALID;
-  if (!L->has_router || !(L->has_q4cp || L->has_gguf)) return MOE_E_STATE;
+  if (!L->has_router || !(L->has_q4cp || L->has_gguf || L->has_i4r)) return MOE_E_STATE;
   if (P > c->cfg.max_tokens) return MOE_E_STATE;
   if (!moe_aligned(x, 16) || !moe_aligned(y, 16) || !moe_aligned(x16, 16)) return MOE_E_INVALID;
   if (P <= c->small_max) return MOE_E_UNSUPPORTED;  // small batches never use an f16 copy
+  if (L->has_i4r) return MOE_E_UNSUPPORTED;  // (these layers read the rotated activations, made from the f32 rows)
   c->x16_ext = (const __half*)x16;
   const int rc = forward_batch(c, *L, x, P, y, moe_s(st));
   c->x16_ext = nullptr;

@@ -94,6 +94,7 @@ struct DecW {  // one q4cp tensor's planes
   const uint8_t *codes, *scales;
   const float* cb;
   uint64_t ss;
+  int gsh;  // 32-element groups per scale = 1 << gsh (q4cp: 0; hgn v2 i4r, one scale per 128 columns: 2)
 };
 
 // ---- codebooks that are not a*n + b (the reference converter's fixed non-uniform table, trained tables): the same
@@ -151,6 +152,12 @@ __device__ __forceinline__ float lut_dot(const uint4 cw, const XF& x, const floa
 struct GuArgs2 {
   DecW gu;           // fused gate_up [E*2*mid][d]
   DecW shg, shu;     // shared expert gate / up [mid][d] (codes == nullptr: none)
+  // hgn v2 rotated experts (not with UQ / LUT): the routed slots read the rotated activations' planes and write
+  // their gate | up sums as they are, zraw[token][slot][2 mid] (the rotation back comes before SwiGLU); the shared
+  // expert's slot is untouched by this
+  float* zraw;
+  const uint32_t* xplanes_rot;
+  const float2* xmeta_rot;
 };
 
 // grid (mid/32, slots incl. shared, P); block 512.  Wave w: gate rows 4w..4w+3 and the matching up
@@ -253,10 +260,13 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   // the activation planes and codebook constants are requested first: loads return in order, so
   // the dot products of the first row pair can start while the later rows are still in flight
   XG xa, xb;
+  const bool raw = !UQ && !LUT && A.zraw && !shared;  // (block-uniform)
   if (!LUT && !UQ) {
     const size_t xbase = (size_t)blockIdx.z * G;
-    load_xg(xa, xplanes, xmeta, xbase + gA);
-    load_xg(xb, xplanes, xmeta, xbase + gB);
+    const uint32_t* xp = raw ? A.xplanes_rot : xplanes;
+    const float2* xm = raw ? A.xmeta_rot : xmeta;
+    load_xg(xa, xp, xm, xbase + gA);
+    load_xg(xb, xp, xm, xbase + gB);
   }
   const float ga = Wg.cb[1] - Wg.cb[0], gb = fmaf(8.f, ga, Wg.cb[0]), ua = Wu.cb[1] - Wu.cb[0], ub = fmaf(8.f, ua, Wu.cb[0]);
   // pairs 0,1: gate rows (r0+2p, r0+2p+1); pairs 2,3: the up rows
@@ -271,10 +281,10 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     const uint64_t trow = lane < 32 ? 0 : 1;
     ca[p] = *(const uint4*)(c0 + (size_t)gA * 16);
     cb[p] = *(const uint4*)(c0 + rb + (size_t)gA * 16);
-    sa[p] = *(const __half*)(s0 + gA * 2);
-    sb[p] = *(const __half*)(s0 + W.ss + gA * 2);
+    sa[p] = *(const __half*)(s0 + (gA >> W.gsh) * 2);
+    sb[p] = *(const __half*)(s0 + W.ss + (gA >> W.gsh) * 2);
     ct[p] = *(const uint4*)(c0 + trow * rb + (size_t)gB * 16);
-    st[p] = *(const __half*)(s0 + trow * W.ss + gB * 2);
+    st[p] = *(const __half*)(s0 + trow * W.ss + (gB >> W.gsh) * 2);
   }
   __builtin_amdgcn_sched_barrier(0);  // every load above is issued before the first dot product
   for (int pi = 0; pi < npairs; pi++) {
@@ -329,6 +339,14 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     }
   }
   __syncthreads();
+  if (raw) {
+    if (threadIdx.x < 32) {
+      float* zr = A.zraw + ((size_t)tok * kpt + s) * 2 * mid + blockIdx.x * GU2_ROWS + threadIdx.x;
+      zr[0] = gs[threadIdx.x];
+      zr[mid] = us[threadIdx.x];
+    }
+    return;
+  }
   // SwiGLU on the block's 32 rows = one group of the down projection's input; quantise it
   if (wv == 0) {
     const int j = lane & 31;
@@ -364,6 +382,7 @@ struct DnArgs2 {
   DecW dn;   // routed down [E*d][mid]
   DecW shd;  // shared expert down [d][mid] (codes == nullptr: none)
   const float* sh_logit;
+  float* out_sh;  // != nullptr: the shared expert's gated rows go here instead of into the sum (same strides as out)
 };
 
 // grid (d/ROWS, P); block = 64 x ceil(slots/2).  Wave = one slot pair, half-wave = one slot: lane
@@ -416,6 +435,7 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
     const uint8_t* wscales = shared ? A.shd.scales : A.dn.scales;
     const float* wcb = shared ? A.shd.cb : A.dn.cb;
     const uint64_t wss = shared ? A.shd.ss : A.dn.ss;
+    const int wgsh = shared ? A.shd.gsh : A.dn.gsh;
     const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
     XG x;
     XF xh;
@@ -425,7 +445,7 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
     const float a = wcb[1] - wcb[0], b = fmaf(8.f, a, wcb[0]);
     const uint64_t row0 = (shared ? 0 : (uint64_t)e * d) + r0;
     const uint8_t* cp = wcodes + row0 * rb + (size_t)g * 16;
-    const uint8_t* sp = wscales + row0 * wss + g * 2;
+    const uint8_t* sp = wscales + row0 * wss + (g >> wgsh) * 2;
     uint4 cw[ROWS];
     __half sc[ROWS];
 #pragma unroll
@@ -448,7 +468,11 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
     const int r = threadIdx.x;
     float y = 0.f;
     for (int s = 0; s < kpt; s++) y += wsm[s] * part[s][r];
-    if (has_shared) y += wsm[kpt] * part[kpt][r];
+    if (has_shared) {
+      const float shv = wsm[kpt] * part[kpt][r];
+      if (A.out_sh) A.out_sh[(size_t)tok * out_stride + r0 + r] = shv;
+      else y += shv;
+    }
     out[(size_t)tok * out_stride + r0 + r] = y;
   }
 }
@@ -476,7 +500,7 @@ __global__ void __launch_bounds__(256) k_dec_dn_uq(DnArgs2 A, const uint32_t* __
   const int r0 = blockIdx.x * DU_ROWS + DU_HW * hw;
   const uint64_t row0 = (shared ? 0 : (uint64_t)tile.expert * d) + r0;
   const uint8_t* cp = W.codes + row0 * rb + (size_t)g * 16;
-  const uint8_t* sp = W.scales + row0 * W.ss + g * 2;
+  const uint8_t* sp = W.scales + row0 * W.ss + (g >> W.gsh) * 2;
   XG x;
   load_xg(x, hplanes, hmeta, (size_t)tile.first * G + g);
   const float c0 = W.cb[0], c1 = W.cb[1];
@@ -508,7 +532,13 @@ __global__ void __launch_bounds__(256) k_dec_dn_uq(DnArgs2 A, const uint32_t* __
 
 DecW decw(const moe_wview* w) {
   DecW o{};
-  if (w) {
+  if (w && w->dtype == MOE_DT_I4R) {  // codes, then one fp16 scale per 128 columns, rows unpadded; codebook n - 8
+    o.codes = w->data;
+    o.scales = w->data + w->rows * w->cols / 2;
+    o.cb = moe_i4r_codebook();
+    o.ss = w->cols / 128 * 2;
+    o.gsh = 2;
+  } else if (w) {
     Q4cpOps q = q4cp_ops(w);
     o.codes = q.codes; o.scales = q.scales; o.cb = q.cb; o.ss = q.scale_stride;
   }
@@ -558,11 +588,18 @@ bool moe_dec_gu_topk_supported(int n_experts, int kpt) { return n_experts <= 102
 int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                            const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                            int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
-                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st) {
+                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st, const moe_dec_v2* v2) {
   GuArgs2 A{};
   A.gu = decw(gu);
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
+  if (v2) {
+    if (!v2->zraw || !v2->xplanes_rot || !v2->xmeta_rot) return MOE_E_INVALID;
+    A.zraw = v2->zraw;
+    A.xplanes_rot = v2->xplanes_rot;
+    A.xmeta_rot = v2->xmeta_rot;
+  }
+  if (!A.gu.cb) return MOE_E_STATE;
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);  // + the row of the exact top-k block
   if (n_experts <= 512)
     k_dec_gu<false, 8, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
@@ -650,11 +687,13 @@ int moe_launch_dec_dn_uq(const moe_wview* dn, const moe_wview* sh_down, const ui
 int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,
                       const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
                       int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
-                      hipStream_t st) {
+                      hipStream_t st, float* out_sh) {
   DnArgs2 A{};
   A.dn = decw(dn);
   A.shd = decw(sh_down);
   A.sh_logit = sh_logit;
+  A.out_sh = out_sh;
+  if (!A.dn.cb) return MOE_E_STATE;
   const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
   // MOE_DN_ROWS rows per block where that divides d (d = 3072: 512 blocks, two per CU), else 8
   if (d % MOE_DN_ROWS == 0)

@@ -23,6 +23,10 @@
 // in that order (layout 2), and the pairs of one word alternate between the stage's two sub-blocks,
 // each with its own w = (d*sc)*n - dmin*m as one packed f16 FMA.  The 16-byte block header takes
 // the place of q4cp's 8 staged scales (one per row and four stages).
+//
+// GS = 2: one scale per 128 columns instead of 32 (hgn v2 i4r experts, reference kI4R,
+// src/gpu/parts/27_kernels_moe_lut.inc:23-29): the four stages between two scale refreshes span exactly two scales,
+// fetched as one 4-byte load per row.
 #include "common.h"
 #include "internal.h"
 
@@ -124,17 +128,22 @@ __device__ __forceinline__ void mfma16(floatx16& acc, const half8& a, const half
 __device__ __forceinline__ void g2l16(const void* g, uint8_t* lds_base) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, LDS_PTR(lds_base), 16, 0, 0);
 }
+// 64 lanes x 4 B: lane l lands at base + 4 l
+__device__ __forceinline__ void g2l4(const void* g, uint8_t* lds_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g, LDS_PTR(lds_base), 4, 0, 0);
+}
 
 // MF = live 32-row fragments of the tile (1 .. 4); AFFINE = codebook a*n+b.
 // NF = weight fragments (32 rows) per wave: the block's 16 fragments are split over NW = 16/NF
 // waves, each wave multiplying all MF pair fragments with its own NF weight fragments.
-template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K>
+template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
                                           const float* __restrict__ xms,
                                           float cmag, const moe_comb& cmb, bool shared) {
   constexpr int NH = NF / 2;  // gate/up: fragments per half
+  static_assert(GS == 0 || (GS == 2 && !Q4K && NSB == 1), "one scale per 128 columns: q4cp-style planes, single scale buffer");
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
@@ -213,7 +222,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
       const size_t off = Q4K ? (size_t)(s >> 2) * 144 : (size_t)g0 * 2;
-      g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + (S_LOADS * wv + i) * 1024);
+      if (GS == 2)  // the two scales of stages s..s+3 (s % 4 == 0: columns 64 s .. 64 s + 255), [row][4 B]
+        g2l4(s_src[i] + (size_t)s, S0 + (S_LOADS * wv + i) * 256);
+      else
+        g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + (S_LOADS * wv + i) * 1024);
     }
   };
   auto issue_a = [&](int s) {
@@ -309,14 +321,20 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         if (Q4K) {
           if ((s & 3) == 0) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
         } else {
-          if ((s & 3) == 0) {
+          if (GS == 2) {
+            if ((s & 3) == 0) {
+              const uint32_t w = *(const uint32_t*)(Sb + wrow[nf] * 4);
+              sc4[nf][0] = sc4[nf][1] = w & 0xffffu;
+              sc4[nf][2] = sc4[nf][3] = w >> 16;
+            }
+          } else if ((s & 3) == 0) {
             const uint4 w = *(const uint4*)(Sb + wrow[nf] * 16);
             sc4[nf][0] = h ? w.x >> 16 : w.x & 0xffffu;
             sc4[nf][1] = h ? w.y >> 16 : w.y & 0xffffu;
             sc4[nf][2] = h ? w.z >> 16 : w.z & 0xffffu;
             sc4[nf][3] = h ? w.w >> 16 : w.w & 0xffffu;
           }
-          const int wi = (sidx - h) >> 1;  // wave-uniform
+          const int wi = GS == 2 ? (s & 3) : (sidx - h) >> 1;  // wave-uniform
           const uint32_t bits = wi == 0 ? sc4[nf][0] : wi == 1 ? sc4[nf][1] : wi == 2 ? sc4[nf][2] : sc4[nf][3];
           union { uint16_t u; _Float16 f; } cv;
           cv.u = (uint16_t)bits;
@@ -597,7 +615,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   }
 }
 
-template <bool UP, bool F16OUT, bool Q4K>
+template <bool UP, bool F16OUT, bool Q4K, int GS>
 __global__ void __launch_bounds__(NT, WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
@@ -665,8 +683,8 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
-    else gemm_tile<UP, F16OUT, MF, false, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    else gemm_tile<UP, F16OUT, MF, false, false, GS>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
@@ -689,7 +707,11 @@ LutDev to_dev(const moe_lutw* p, const float* cb_up) {
   return d;
 }
 
-bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k) {
+bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k, int gs = 0) {
+  if (gs == 2) {  // one scale per 128 columns, unpadded scale rows; whole 256-column scale windows
+    if (q4k || pair || !p || !p->w || !p->sc || !p->cb || k < 256 || k % 256) return false;
+    return moe_aligned(p->w, 16) && moe_aligned(p->sc, 4) && p->sstride % 4 == 0 && p->sstride >= k / 128 * 2;
+  }
   if (q4k) {  // raw Q4_K rows: only the code pointers are used
     if (!p || !p->w || (pair && !p->w_up) || k < 256 || k % 256) return false;
     return moe_aligned(p->w, 16) && (!pair || moe_aligned(p->w_up, 16));
@@ -710,14 +732,15 @@ bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k) {
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up) {
+                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
+  if (gs != 0 && (gs != 2 || up || !f16out || q4k || sh || comb)) return MOE_E_UNSUPPORTED;
   moe_comb cmb{};
   if (comb) {  // fused combine: down launch with f32 results, out = the (zeroed) token rows
     if (up || f16out || !comb->tokidx || !comb->pw || (sh && !comb->sg) || comb->y != out) return MOE_E_INVALID;
     cmb = *comb;
   }
-  if (!lut_ok(routed, up, k, q4k) || (sh && !lut_ok(sh, up, k, q4k))) return MOE_E_UNSUPPORTED;
+  if (!lut_ok(routed, up, k, q4k, gs) || (sh && !lut_ok(sh, up, k, q4k))) return MOE_E_UNSUPPORTED;
   if (m < 32 || m % 32) return MOE_E_UNSUPPORTED;
   if (q4k && up && m % 64) return MOE_E_UNSUPPORTED;  // hid is written in whole 64-element blocks
   if (!moe_aligned(x, 16) || !moe_aligned(out, 4)) return MOE_E_INVALID;
@@ -728,25 +751,27 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
   LutDev R = to_dev(routed, nullptr), S = to_dev(sh ? sh : routed, sh ? sh_cb_up : nullptr);
   const int split = sh ? 1 : 0;
-#define GEMM_LAUNCH(UPK, F16, Q)                                                                              \
-  do {                                                                                                        \
-    static bool attr_done = false;                                                                            \
-    if (!attr_done) {                                                                                         \
-      MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<UPK, F16, Q>,                                  \
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));              \
-      attr_done = true;                                                                                       \
-    }                                                                                                         \
-    k_moe_gemm_q4cp<UPK, F16, Q><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
-                                                               m, k, nblk_n, split, hs, cmb);                 \
+#define GEMM_LAUNCH(UPK, F16, Q, G)                                                                              \
+  do {                                                                                                           \
+    static bool attr_done = false;                                                                               \
+    if (!attr_done) {                                                                                            \
+      MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<UPK, F16, Q, G>,                                  \
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));                 \
+      attr_done = true;                                                                                          \
+    }                                                                                                            \
+    k_moe_gemm_q4cp<UPK, F16, Q, G><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
+                                                                  m, k, nblk_n, split, hs, cmb);                 \
   } while (0)
-  if (q4k) {
-    if (up) GEMM_LAUNCH(true, true, true);
-    else if (f16out) GEMM_LAUNCH(false, true, true);
-    else GEMM_LAUNCH(false, false, true);
+  if (gs == 2) {
+    GEMM_LAUNCH(false, true, false, 2);
+  } else if (q4k) {
+    if (up) GEMM_LAUNCH(true, true, true, 0);
+    else if (f16out) GEMM_LAUNCH(false, true, true, 0);
+    else GEMM_LAUNCH(false, false, true, 0);
   } else {
-    if (up) GEMM_LAUNCH(true, true, false);
-    else if (f16out) GEMM_LAUNCH(false, true, false);
-    else GEMM_LAUNCH(false, false, false);
+    if (up) GEMM_LAUNCH(true, true, false, 0);
+    else if (f16out) GEMM_LAUNCH(false, true, false, 0);
+    else GEMM_LAUNCH(false, false, false, 0);
   }
 #undef GEMM_LAUNCH
   MOE_LAUNCH_CHECK();
@@ -765,6 +790,31 @@ MOE_API int moe_lut_q4cp_view(const uint8_t* data, uint64_t rows, uint64_t cols,
   return MOE_OK;
 }
 
+// hgn v2 i4r tensor [codes][scales], no header: the reference's lut_i4r_view (27_kernels_moe_lut.inc:823-834)
+MOE_API int moe_lut_i4r_view(const uint8_t* data, uint64_t rows, uint64_t cols, int e_rows, int up_off, moe_lutw* out) {
+  if (!data || !out || cols == 0 || cols % 128) return MOE_E_INVALID;
+  out->cb = moe_i4r_codebook();
+  if (!out->cb) return MOE_E_STATE;
+  out->w = out->w_up = data;
+  out->sc = out->sc_up = data + rows * cols / 2;
+  out->sstride = (int)(cols / 128 * 2);
+  out->e_rows = e_rows;
+  out->up_off = up_off;
+  return MOE_OK;
+}
+
+// gate | up unfused, f16 [slot][2 m] (the rotation back comes before SwiGLU): the reference's moe_lut_up_raw
+// (27_kernels_moe_lut.inc:677-685).  x16 in the grouped GEMM's activation order, as for moe_lut_up.
+MOE_API int moe_lut_up_raw(int type, const moe_lutw* p, const void* x16, const int* tokidx, const moe_tile* tiles,
+                           const int* ntiles, int max_tiles, void* guv16, int m, int k, moe_stream_t st) {
+  if (type != MOE_LUT_I4R) return MOE_E_UNSUPPORTED;
+  if (!tokidx || !p) return MOE_E_INVALID;
+  moe_lutw q = *p;
+  q.e_rows = 2 * m;  // the fused tensor's rows of one expert, walked as plain rows
+  return moe_launch_gemm_q4cp(false, &q, nullptr, 1 << 30, (const __half*)x16, tokidx, tiles, ntiles, max_tiles, guv16,
+                              2 * m, k, true, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr, 2);
+}
+
 MOE_API int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* tokidx,
                        const moe_tile* tiles, const int* ntiles, int max_tiles, void* hid16, int m, int k,
                        moe_stream_t st) {
@@ -777,6 +827,11 @@ MOE_API int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* 
 MOE_API int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
                          const int* ntiles, int max_tiles, void* pairs, int m, int k, int f16,
                          moe_stream_t st) {
+  if (type == MOE_LUT_I4R) {  // (f16 pairs only, the reference's default for hgn v2: 40_model.inc:4619-4631)
+    if (!f16) return MOE_E_UNSUPPORTED;
+    return moe_launch_gemm_q4cp(false, p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles, max_tiles, pairs,
+                                m, k, true, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr, 2);
+  }
   if (type != MOE_LUT_Q4CP) return MOE_E_UNSUPPORTED;
   return moe_launch_gemm_q4cp(false, p, nullptr, 1 << 30, (const __half*)hid16, nullptr, tiles, ntiles,
                               max_tiles, pairs, m, k, f16 != 0, false, moe_hscale{nullptr, 0.f, 0.f}, moe_s(st), nullptr, nullptr);

@@ -1,0 +1,299 @@
+// hgn v2 routed experts (dtype 23 "i4r"): 4-bit codes n with w = (n - 8) * fp16 scale per 128 columns, stored in the
+// rotated domain G of W = diag(svh) . H . G . H . diag(suh) / 128 (H = 128-block Hadamard).  The rotation moves onto
+// the activations:
+//   rot_in   x^ = H(suh . x) / sqrt(128)          per 128 block of the input
+//   GEMV     z  = G . x^
+//   rot_out  y  = svh . H(z) / sqrt(128)          per 128 block of the output
+// so a layer is rot_in(x, su) -> gate_up -> [rot_out(svh_gu), SwiGLU, rot_in(suh_dn)] -> down -> weighted sum over the
+// experts -> rot_out(svh_dn) (svh_dn is shared by all experts of a layer, so the last rotation runs once on the sum).
+// (reference: src/gpu/parts/28_kernels_hgn_v2.inc:1-15 format notes, :62-98 k_v2_rot, :105-150 k_i4r_mid;
+//  src/gpu/parts/40_model.inc:1638-1656 moe_v2_1, :4570-4686 moe_b_v2; CPU dequantisation tools/moe_lut_test.cu:936-948)
+// The kernels here are the pieces around the projections; the projections themselves run on the q4cp kernels with
+// one scale per 128 columns (decode_q4cp.hip, gemm_q4cp.hip).  A lane holds 8 consecutive elements, 16 lanes one
+// 128-block: 16-byte accesses, and the f16 / digit-plane outputs need no exchange beyond a quad.
+#include <mutex>
+
+#include "common.h"
+#include "hv2.h"
+#include "internal.h"
+#include "qvec.h"
+
+namespace {
+
+__device__ __forceinline__ float quad_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float quad_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ void ld8(const float* p, float (&v)[8]) {
+  const float4 a = ((const float4*)p)[0], b = ((const float4*)p)[1];
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void ld8(const __half* p, float (&v)[8]) {
+  const uint4 u = *(const uint4*)p;
+  const __half2* h = (const __half2*)&u;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const float2 f = __half22float2(h[i]);
+    v[2 * i] = f.x;
+    v[2 * i + 1] = f.y;
+  }
+}
+__device__ __forceinline__ void st8(float* p, const float (&v)[8]) {
+  ((float4*)p)[0] = make_float4(v[0], v[1], v[2], v[3]);
+  ((float4*)p)[1] = make_float4(v[4], v[5], v[6], v[7]);
+}
+// 8 values as f16 in the order the grouped GEMM keeps its activations in: [e0,e4,e1,e5,e2,e6,e3,e7]
+__device__ __forceinline__ void st8_f16_ilv(__half* p, const float (&v)[8]) {
+  const __half2 a = __floats2half2_rn(v[0], v[4]), b = __floats2half2_rn(v[1], v[5]);
+  const __half2 c = __floats2half2_rn(v[2], v[6]), d = __floats2half2_rn(v[3], v[7]);
+  uint4 o;
+  o.x = *(const uint32_t*)&a; o.y = *(const uint32_t*)&b; o.z = *(const uint32_t*)&c; o.w = *(const uint32_t*)&d;
+  *(uint4*)p = o;
+}
+// 8 values per lane, the four lanes of a quad = one 32-element group -> the group's four digit planes and (q, q*sum)
+// in the form the integer-dot decode kernels read (qvec.h, qvec4): lane j of the quad holds dword j of every plane.
+__device__ __forceinline__ void st8_planes(const float (&v)[8], int lane, uint32_t* __restrict__ planes,
+                                           float2* __restrict__ meta, size_t gi, bool live) {
+  float m = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+  m = fmaxf(m, quad_xor1(m));
+  m = fmaxf(m, quad_xor2(m));
+  const float inv = m > 0.f ? QV4_XMAX / m : 0.f;
+  const float q = m * (1.f / QV4_XMAX);
+  uint32_t pl[4] = {0u, 0u, 0u, 0u};
+  int sx = 0;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int X = (int)rintf(v[i] * inv);
+    sx += X;
+    int p0, p1, p2, p3;
+    qv4_digits(X, p0, p1, p2, p3);
+    pl[0] |= (uint32_t)(p0 & 15) << (4 * i);
+    pl[1] |= (uint32_t)(p1 & 15) << (4 * i);
+    pl[2] |= (uint32_t)(p2 & 15) << (4 * i);
+    pl[3] |= (uint32_t)(p3 & 15) << (4 * i);
+  }
+  sx += __builtin_amdgcn_update_dpp(0, sx, 0xB1, 0xf, 0xf, true);
+  sx += __builtin_amdgcn_update_dpp(0, sx, 0x4E, 0xf, 0xf, true);
+  if (live) {
+    uint32_t* dst = planes + gi * QV4_GROUP_DW + (lane & 3);
+#pragma unroll
+    for (int p = 0; p < 4; p++) dst[4 * p] = pl[p];
+    if ((lane & 3) == 0) meta[gi] = make_float2(q, q * (float)sx);
+  }
+}
+
+// y[p][i] = post[i] * H(pre . x[p])[i] / sqrt(128) (+ add[p][i]) per 128 block; pre / post / add optional.
+// P rows of n values (n % 128 == 0), n/8 lanes per row.  MODE 0: f32 rows; 1: f16 rows in the grouped GEMM's order;
+// 2: digit planes of the decode kernels (planes / meta indexed [p][n/32]).  In place (MODE 0, y == x) is fine.
+template <int MODE>
+__global__ void __launch_bounds__(256) k_v2_rot(const float* x, uint64_t xs, void* y, uint64_t ys,
+                                                const float* __restrict__ pre, const float* __restrict__ post,
+                                                const float* add, uint64_t adds, int n, int P,
+                                                uint32_t* __restrict__ planes, float2* __restrict__ meta) {
+  const int lane = threadIdx.x & 63;
+  const int per_row = n >> 3;
+  const int64_t gl = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int p = (int)(gl / per_row), c = (int)(gl - (int64_t)p * per_row) * 8;
+  const bool live = p < P;  // (whole groups of 16 lanes are live or not: n % 128 == 0)
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = 0.f;
+  if (live) {
+    ld8(x + (size_t)p * xs + c, v);
+    if (pre) {
+      float s[8];
+      ld8(pre + c, s);
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] *= s[i];
+    }
+  }
+  moe_fwht128_r8(v, lane);
+  float s[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) s[i] = 1.f;
+  if (live && post) ld8(post + c, s);
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = v[i] * MOE_RS128 * s[i];
+  if (MODE == 0) {
+    if (!live) return;
+    if (add) {
+      float a[8];
+      ld8(add + (size_t)p * adds + c, a);
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] += a[i];
+    }
+    st8((float*)y + (size_t)p * ys + c, v);
+  } else if (MODE == 1) {
+    if (live) st8_f16_ilv((__half*)y + (size_t)p * ys + c, v);
+  } else {
+    st8_planes(v, lane, planes, meta, (size_t)p * (n >> 5) + (c >> 5), live);
+  }
+}
+
+// The middle of an i4r expert, one block per (token, expert) slot, ceil(2 mid / 512) waves:
+//   g | u = svh_gu . H(z) / sqrt(128)      z = the slot's rotated gate_up output [2 mid]
+//   h     = silu(g) * u
+//   out   = H(suh_dn . h) / sqrt(128)      the rotated input of down_proj [mid]
+// MODE 0: f32 rows, 1: f16 rows in the grouped GEMM's order, 2: digit planes; slot s of the launch goes to output
+// row (s / k) * row_slots + s % k (the decode path keeps a token's slots next to its shared-expert slot).
+template <class TG, int MODE>
+__global__ void __launch_bounds__(256) k_i4r_mid(const TG* __restrict__ z, uint64_t zs, void* out, uint64_t os,
+                                                 const float* __restrict__ svh_gu, const float* __restrict__ suh_dn,
+                                                 int mid, int k, int row_slots, uint32_t* __restrict__ planes,
+                                                 float2* __restrict__ meta) {
+  __shared__ float s[2048];
+  const int slot = blockIdx.x, lane = threadIdx.x & 63;
+  const int c = threadIdx.x * 8;
+  {
+    const bool live = c < 2 * mid;
+    float v[8], f[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = 0.f, f[i] = 0.f;
+    if (live) {
+      ld8(z + (size_t)slot * zs + c, v);
+      ld8(svh_gu + c, f);
+    }
+    moe_fwht128_r8(v, lane);
+    if (live) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) s[c + i] = v[i] * MOE_RS128 * f[i];
+    }
+  }
+  __syncthreads();
+  const bool live = c < mid;
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = 0.f;
+  if (live) {
+    float f[8];
+    ld8(suh_dn + c, f);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      const float g = s[c + i], u = s[mid + c + i];
+      v[i] = g / (1.f + expf(-g)) * u * f[i];
+    }
+  }
+  moe_fwht128_r8(v, lane);
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] *= MOE_RS128;
+  const size_t row = (size_t)(slot / k) * row_slots + slot % k;
+  if (MODE == 0) {
+    if (live) st8((float*)out + row * os + c, v);
+  } else if (MODE == 1) {
+    if (live) st8_f16_ilv((__half*)out + row * os + c, v);
+  } else {
+    st8_planes(v, lane, planes, meta, row * (mid >> 5) + (c >> 5), live);
+  }
+}
+
+// rows [row0, row0 + nrows) of an i4r tensor as f32 (bit-exact: (n - 8) * fp16 scale, one rounding);
+// a thread per 8 elements
+__global__ void __launch_bounds__(256) k_i4r_rows(const uint8_t* __restrict__ data, uint64_t rows, uint64_t cols,
+                                                  uint64_t row0, uint64_t nrows, float* __restrict__ out) {
+  const uint64_t per_row = cols / 8;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < nrows * per_row; i += (uint64_t)gridDim.x * 256) {
+    const uint64_t r = i / per_row, c = (i - r * per_row) * 8, gr = row0 + r;
+    const uint32_t w = *(const uint32_t*)(data + gr * (cols / 2) + c / 2);
+    const __half sc = *(const __half*)(data + rows * (cols / 2) + gr * (cols / 128 * 2) + (c >> 7) * 2);
+    const float sf = __half2float(sc);
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = (float)((int)((w >> (4 * j)) & 15u) - 8) * sf;
+    st8(out + r * cols + c, v);
+  }
+}
+
+}  // namespace
+
+// (not const and not in the unnamed namespace: a device variable that no kernel names must survive into the code
+// object for the host to look its address up)
+static __device__ __align__(64) float g_i4r_cb[16] = {-8.f, -7.f, -6.f, -5.f, -4.f, -3.f, -2.f, -1.f,
+                                                       0.f,  1.f,  2.f,  3.f,  4.f,  5.f,  6.f,  7.f};
+static std::mutex g_i4r_cb_mu;
+
+// The linear codebook -8..7 of the i4r codes as a device array (the q4cp-style kernels read their codebook from
+// memory; reference: g_i4r_cb, src/gpu/parts/30_host_util.inc:790,863-866).  One copy per device, looked up once.
+const float* moe_i4r_codebook() {
+  static const float* ptr[64] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(g_i4r_cb_mu);
+  if (!ptr[dev]) {
+    float* p = nullptr;
+    if (hipGetSymbolAddress((void**)&p, HIP_SYMBOL(g_i4r_cb)) != hipSuccess) return nullptr;
+    ptr[dev] = p;
+  }
+  return ptr[dev];
+}
+
+bool moe_v2_shapes_ok(int d, int mid) { return d % 128 == 0 && mid % 128 == 0 && 2 * mid <= 2048; }
+
+// mode 0: f32 rows (y, ys; + add), 1: f16 rows in the grouped GEMM's order (y, ys), 2: digit planes (planes, meta)
+int moe_launch_v2_rot(const float* x, uint64_t xs, int P, int n, const float* pre, const float* post, int mode, void* y,
+                      uint64_t ys, const float* add, uint64_t adds, uint32_t* planes, float2* meta, hipStream_t st) {
+  if (!x || P < 0 || n < 128 || n % 128 || mode < 0 || mode > 2) return MOE_E_INVALID;
+  if (mode == 2 ? (!planes || !meta) : !y) return MOE_E_INVALID;
+  if (!moe_aligned(x, 16) || xs % 4 || (y && !moe_aligned(y, 16)) || ys % 8 || (add && (!moe_aligned(add, 16) || adds % 4)) ||
+      (pre && !moe_aligned(pre, 16)) || (post && !moe_aligned(post, 16)))
+    return MOE_E_INVALID;
+  if (P == 0) return MOE_OK;
+  const int64_t lanes = (int64_t)P * (n / 8);
+  const unsigned grid = (unsigned)((lanes + 255) / 256);
+  if (mode == 0) k_v2_rot<0><<<grid, 256, 0, st>>>(x, xs, y, ys, pre, post, add, adds, n, P, nullptr, nullptr);
+  else if (mode == 1) k_v2_rot<1><<<grid, 256, 0, st>>>(x, xs, y, ys, pre, post, nullptr, 0, n, P, nullptr, nullptr);
+  else k_v2_rot<2><<<grid, 256, 0, st>>>(x, xs, nullptr, 0, pre, post, nullptr, 0, n, P, planes, meta);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// z: [nslots][zs] f32 or f16; output row of slot s: (s / k) * row_slots + s % k (k = row_slots = 1: row s)
+int moe_launch_i4r_mid(const void* z, bool z_f16, uint64_t zs, int nslots, int mid, const float* svh_gu,
+                       const float* suh_dn, int mode, void* out, uint64_t os, int k, int row_slots, uint32_t* planes,
+                       float2* meta, hipStream_t st) {
+  if (!z || !svh_gu || !suh_dn || nslots < 0 || mode < 0 || mode > 2 || k < 1 || row_slots < k) return MOE_E_INVALID;
+  if (mode == 2 ? (!planes || !meta) : !out) return MOE_E_INVALID;
+  if (mid < 128 || mid % 128 || 2 * mid > 2048) return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(z, 16) || zs % 8 || (out && !moe_aligned(out, 16)) || os % 8 || !moe_aligned(svh_gu, 16) ||
+      !moe_aligned(suh_dn, 16))
+    return MOE_E_INVALID;
+  if (nslots == 0) return MOE_OK;
+  const int bs = 64 * ((2 * mid / 8 + 63) / 64);
+#define MID_GO(TG, M) \
+  k_i4r_mid<TG, M><<<nslots, bs, 0, st>>>((const TG*)z, zs, out, os, svh_gu, suh_dn, mid, k, row_slots, planes, meta)
+  if (z_f16) {
+    if (mode == 0) MID_GO(__half, 0); else if (mode == 1) MID_GO(__half, 1); else MID_GO(__half, 2);
+  } else {
+    if (mode == 0) MID_GO(float, 0); else if (mode == 1) MID_GO(float, 1); else MID_GO(float, 2);
+  }
+#undef MID_GO
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+MOE_API int moe_i4r_dequant_rows(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t row0, uint64_t nrows,
+                                 float* out, moe_stream_t st) {
+  if (!data || !out || cols == 0 || cols % 128 || row0 + nrows > rows) return MOE_E_INVALID;
+  if (!moe_aligned(data, 4) || !moe_aligned(out, 16)) return MOE_E_INVALID;
+  if (nrows == 0) return MOE_OK;
+  const uint64_t n = nrows * (cols / 8);
+  const unsigned grid = (unsigned)((n + 255) / 256 > 65536 ? 65536 : (n + 255) / 256);
+  k_i4r_rows<<<grid, 256, 0, moe_s(st)>>>(data, rows, cols, row0, nrows, out);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+MOE_API int moe_v2_rot(const float* x, uint64_t xs, void* y, uint64_t ys, const float* pre, const float* post, int n,
+                       int P, int out_f16, moe_stream_t st) {
+  return moe_launch_v2_rot(x, xs, P, n, pre, post, out_f16 ? 1 : 0, y, ys, nullptr, 0, nullptr, nullptr, moe_s(st));
+}
+
+MOE_API int moe_i4r_mid(const void* guv, int guv_f16, uint64_t gs, void* out, int out_f16, uint64_t os,
+                        const float* svh_gu, const float* suh_dn, int mid, int nslots, moe_stream_t st) {
+  return moe_launch_i4r_mid(guv, guv_f16 != 0, gs, nslots, mid, svh_gu, suh_dn, out_f16 ? 1 : 0, out, os, 1, 1, nullptr,
+                            nullptr, moe_s(st));
+}

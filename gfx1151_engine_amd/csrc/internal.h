@@ -48,7 +48,7 @@ int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr);
+                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr, int gs = 0);
 int moe_gemm_tile_cap();
 int moe_launch_zero_f32(float* p, uint64_t n, hipStream_t st);
 int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, int P, int sh_first, int* tokidx,
@@ -64,7 +64,7 @@ int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E
                             int sh_first, int* tokidx, hipStream_t st);
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
                       const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
-                      moe_hscale hs, hipStream_t st, const moe_hc* hc);
+                      moe_hscale hs, hipStream_t st, const moe_hc* hc, const float* rot_svh = nullptr);
 int moe_router_logits_seq(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
                           float* logits, float* out_x, float* out_xms, hipStream_t st);
 
@@ -85,10 +85,18 @@ bool moe_dec_uq_supported(int d);
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
                     hipStream_t st);
 bool moe_dec_gu_topk_supported(int n_experts, int kpt);
+// hgn v2 rotated experts in the gate/up launch: the routed slots read the rotated activations' planes and leave
+// their gate | up sums unfused in zraw [P][kpt][2 mid]
+struct moe_dec_v2 {
+  float* zraw;
+  const uint32_t* xplanes_rot;
+  const float2* xmeta_rot;
+};
 int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                            const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                            int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
-                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st);
+                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st,
+                           const moe_dec_v2* v2 = nullptr);
 int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
@@ -130,7 +138,15 @@ int moe_launch_dec4k_dn(const uint8_t* down, const uint8_t* sh_down, const float
 int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,
                       const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws,
                       int id_stride, int kpt, int P, int d, int mid, float* out, uint64_t out_stride,
-                      hipStream_t st);
+                      hipStream_t st, float* out_sh = nullptr);
+// hgn v2 (hgn_v2.hip)
+const float* moe_i4r_codebook();
+bool moe_v2_shapes_ok(int d, int mid);
+int moe_launch_v2_rot(const float* x, uint64_t xs, int P, int n, const float* pre, const float* post, int mode, void* y,
+                      uint64_t ys, const float* add, uint64_t adds, uint32_t* planes, float2* meta, hipStream_t st);
+int moe_launch_i4r_mid(const void* z, bool z_f16, uint64_t zs, int nslots, int mid, const float* svh_gu,
+                       const float* suh_dn, int mode, void* out, uint64_t os, int k, int row_slots, uint32_t* planes,
+                       float2* meta, hipStream_t st);
 // general GEMV kernels for any supported mix of ggml block types (gguf_types.hip)
 int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up, int tsh, const uint8_t* sh_w,
                        const uint8_t* sh_w_up, int n_experts, const __half* x16, const int* tokidx,

@@ -3,6 +3,7 @@
 // (reference: src/gpu/parts/26_kernels_moe_gguf.inc:389; src/gpu/parts/24_kernels_moe_lt.inc:82-124;
 //  src/gpu/parts/40_model.inc:8897)
 #include "common.h"
+#include "hv2.h"
 #include "internal.h"
 
 namespace {
@@ -125,7 +126,7 @@ __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pai
                                                       const float* __restrict__ ey,
                                                       const float* __restrict__ sg, int sh_first,
                                                       float* __restrict__ out, int P, int D, int K,
-                                                      moe_hscale hs, moe_hc hc) {
+                                                      moe_hscale hs, moe_hc hc, const float* __restrict__ rot_svh) {
   __shared__ int ids[KMAX];
   __shared__ float w[KMAX];
   const int t = blockIdx.y;
@@ -170,6 +171,16 @@ __global__ void __launch_bounds__(128) k_reduce_pw_sg(const PT* __restrict__ pai
     inv_s = 1.f / moe_hid_scale(hs.c_shared, ms);
 #pragma unroll
     for (int i = 0; i < 8; i++) sum[i] *= inv_r;
+  }
+  if (rot_svh) {
+    // hgn v2 rotated experts: the weighted sum is still in the rotated domain; svh . H(sum) / sqrt(128) per 128 block
+    // before the shared expert is added (reference: k_v2_reduce_rot, src/gpu/parts/28_kernels_hgn_v2.inc:153-187).
+    // D % 128 == 0: the 16 lanes of a block are all here.
+    moe_fwht128_r8(sum, threadIdx.x);
+    const float4 a = ((const float4*)(rot_svh + c))[0], b = ((const float4*)(rot_svh + c))[1];
+    const float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int i = 0; i < 8; i++) sum[i] = sum[i] * MOE_RS128 * f[i];
   }
   if (sg) {
     const float g = sigmoid_f(sg[t]) * (ey ? 1.f : inv_s);
@@ -340,7 +351,7 @@ int moe_launch_tiles_shared(const int* eoff, moe_tile* tiles, int* ntiles, int E
 
 int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, const float* pw,
                       const float* ey, const float* sg, int sh_first, float* out, int P, int D, int K,
-                      moe_hscale hs, hipStream_t st, const moe_hc* hcp) {
+                      moe_hscale hs, hipStream_t st, const moe_hc* hcp, const float* rot_svh) {
   moe_hc hc{nullptr, nullptr};
   if (hcp) {  // results go into the bf16 HC state instead of out
     if (!hcp->w4 || !hcp->R || !moe_aligned(hcp->R, 16)) return MOE_E_INVALID;
@@ -349,10 +360,11 @@ int moe_launch_reduce(const void* pairs, bool pairs_f16, const int* pairids, con
   if (!pairs || !pairids || !pw || (!out && !hc.R)) return MOE_E_INVALID;
   if (P < 0 || D < 1 || K < 1) return MOE_E_INVALID;
   if (K > 16 || D % 8) return MOE_E_UNSUPPORTED;
+  if (rot_svh && (D % 128 || !moe_aligned(rot_svh, 16))) return MOE_E_INVALID;
   if (!moe_aligned(pairs, 16) || (out && !moe_aligned(out, 16)) || (ey && !moe_aligned(ey, 16))) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
   dim3 grid((D / 8 + 127) / 128, P);
-#define RED_GO(PT, KC) k_reduce_pw_sg<PT, 16, KC><<<grid, 128, 0, st>>>((const PT*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs, hc)
+#define RED_GO(PT, KC) k_reduce_pw_sg<PT, 16, KC><<<grid, 128, 0, st>>>((const PT*)pairs, pairids, pw, ey, sg, sh_first, out, P, D, K, hs, hc, rot_svh)
   if (pairs_f16) {
     if (K == 10) RED_GO(__half, 10); else if (K == 8) RED_GO(__half, 8); else RED_GO(__half, 0);
   } else {
@@ -394,6 +406,13 @@ MOE_API int moe_reduce_pw_sg(const void* pairs, int pairs_f16, const int* pairid
   if ((ey == nullptr) != (sg == nullptr)) return MOE_E_INVALID;
   return moe_launch_reduce(pairs, pairs_f16 != 0, pairids, pw, ey, sg, -1, out, P, D, K, moe_hscale{nullptr, 0.f, 0.f},
                            moe_s(st), nullptr);
+}
+
+MOE_API int moe_v2_reduce_rot(const void* pairs, int pairs_f16, const int* pairids, const float* pw, const float* svh,
+                              const float* ey, const float* sg, float* out, int P, int D, int K, moe_stream_t st) {
+  if ((ey == nullptr) != (sg == nullptr) || !svh) return MOE_E_INVALID;
+  return moe_launch_reduce(pairs, pairs_f16 != 0, pairids, pw, ey, sg, -1, out, P, D, K, moe_hscale{nullptr, 0.f, 0.f},
+                           moe_s(st), nullptr, svh);
 }
 
 MOE_API int moe_reduce_pw_sg_hc(const void* pairs, int pairs_f16, const int* pairids, const float* pw,

@@ -181,6 +181,25 @@ def make_dense(rng, kind, rows, cols, std=0.05):
     return f32_to_bf16_bits(w) if kind == "bf16" else w
 
 
+def make_i4r(rng, rows, cols, scale_std=0.01):
+    """hgn v2 i4r tensor (dtype 23): [rows*cols/2 code bytes (byte b = elements 2b | 2b+1 << 4)][rows x cols/128 fp16
+    scales], w = (nibble - 8) * scale.  Scales of either sign (the reference's encoder stores signed scales,
+    tools/v2repro/v2enc.py:103-106)."""
+    assert cols % 128 == 0
+    codes = rng.integers(0, 256, size=rows * cols // 2, dtype=np.uint8)
+    sc = (rng.standard_normal((rows, cols // 128)) * scale_std).astype(np.float16)
+    return np.concatenate([codes, sc.reshape(-1).view(np.uint8)])
+
+
+def make_v2_planes(rng, d, mid):
+    """The four sign-scale planes of an hgn v2 layer's expert tensors as f16-representable f32 values (the files hold
+    them as f16): su [d], svh_gu [2 mid], suh_dn [mid], svh_dn [d]; magnitudes around 1, random signs."""
+    def plane(n):
+        v = (0.5 + rng.random(n)) * rng.choice([-1.0, 1.0], size=n)
+        return v.astype(np.float16).astype(np.float32)
+    return plane(d), plane(2 * mid), plane(mid), plane(d)
+
+
 def f32_to_bf16_bits(a):
     """Round-to-nearest-even f32 -> bf16 bit patterns (uint16)."""
     u = np.ascontiguousarray(a, np.float32).view(np.uint32)

@@ -32,7 +32,10 @@ enum moe_status {
 };
 
 /* hgn tensor dtypes (src/hgn.h:2-23) and ggml types (src/gguf.h:42-64) used on this path */
-enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_Q4CP = 5, MOE_DT_Q8G64 = 7, MOE_DT_Q8G32 = 8 };
+enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_F16 = 2, MOE_DT_Q4CP = 5, MOE_DT_Q8G64 = 7, MOE_DT_Q8G32 = 8,
+       /* hgn v2 routed experts (src/gpu/parts/28_kernels_hgn_v2.inc:1-15): data = [rows*cols/2 codes][rows x cols/128
+        * fp16 scales], no header, w = (nibble - 8) * scale, stored in the Hadamard-rotated domain */
+       MOE_DT_I4R = 23 };
 /* Q4_K: every kernel of the path.  Q5_K (gate/up), Q5_1 and Q8_0 (down) — the mix of the reference's GGUF
  * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — and IQ4_NL / IQ4_XS (src/gguf.h:376-407):
  * dequantisation and the general GEMV kernels. */
@@ -146,10 +149,19 @@ typedef struct moe_lutw {
   const float* cb;
   int sstride, e_rows, up_off;
 } moe_lutw;
-enum { MOE_LUT_Q4CP = 100 }; /* moelut::kQ4CP (27_kernels_moe_lut.inc:33) */
+enum { MOE_LUT_Q4CP = 100,  /* moelut::kQ4CP (27_kernels_moe_lut.inc:33) */
+       MOE_LUT_I4R = 101 }; /* moelut::kI4R (27_kernels_moe_lut.inc:34): one scale per 128 columns, codebook n - 8 */
 /* lut_q4cp_view (27_kernels_moe_lut.inc:811) */
 int moe_lut_q4cp_view(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t scale_stride,
                       int e_rows, int up_off, moe_lutw* out);
+/* lut_i4r_view (27_kernels_moe_lut.inc:823-834): the planes of an hgn v2 i4r tensor (MOE_DT_I4R layout); the linear
+ * codebook is a device array the library owns */
+int moe_lut_i4r_view(const uint8_t* data, uint64_t rows, uint64_t cols, int e_rows, int up_off, moe_lutw* out);
+/* moe_lut_up_raw (27_kernels_moe_lut.inc:677-685), type MOE_LUT_I4R: guv16[pair][2 m] = gate | up rows of the fused
+ * tensor times x16[tokidx[pair]], unfused (hgn v2: the rotation back comes before SwiGLU, moe_i4r_mid), f16 in natural
+ * order; x16 in layout 1 (moe_v2_rot writes it so); m % 16 == 0, k % 256 == 0 */
+int moe_lut_up_raw(int type, const moe_lutw* p, const void* x16, const int* tokidx, const moe_tile* tiles,
+                   const int* ntiles, int max_tiles, void* guv16, int m, int k, moe_stream_t st);
 /* k_f32_to_f16_v4 (26_kernels_moe_gguf.inc:389): round-to-nearest-even, n % 8 == 0.
  * layout 0 = natural order; layout 1 = the order the grouped GEMM reads its f16 activations in:
  * inside every group of 8 consecutive elements, [e0,e4,e1,e5,e2,e6,e3,e7] (matches the order the
@@ -164,7 +176,8 @@ int moe_lut_up(int type, const moe_lutw* p, const void* x16, const int* tokidx,
                const moe_tile* tiles, const int* ntiles, int max_tiles, void* hid16, int m, int k,
                moe_stream_t st);
 /* moe_lut_down (27_kernels_moe_lut.inc:765): pairs[pair][m] (unweighted; f32, or f16 if f16 != 0)
- * = W_e[m][k] . hid16[pair] (hid16 in layout 1); m % 32 == 0, k % 128 == 0, k >= 256. */
+ * = W_e[m][k] . hid16[pair] (hid16 in layout 1); m % 32 == 0, k % 128 == 0, k >= 256.
+ * type MOE_LUT_I4R: f16 pairs only, k % 256 == 0. */
 int moe_lut_down(int type, const moe_lutw* p, const void* hid16, const moe_tile* tiles,
                  const int* ntiles, int max_tiles, void* pairs, int m, int k, int f16,
                  moe_stream_t st);
@@ -222,6 +235,16 @@ int moe_set_experts_q4cp(moe_ctx* ctx, int layer, const moe_wview* gate_up, cons
 int moe_set_experts_gguf(moe_ctx* ctx, int layer, const moe_gg_experts* gg);
 int moe_set_shared(moe_ctx* ctx, int layer, const moe_wview* gate_proj, const moe_wview* up_proj,
                    const moe_wview* down_proj, const moe_wview* shared_gate, int sh_gguf_type);
+/* hgn v2 routed experts of a layer (GpuModel::moe_v2_1 / moe_b_v2, 40_model.inc:1638-1656,4570-4686): gate_up
+ * [E*2*mid][d] and down [E*d][mid] as MOE_DT_I4R views, and the four sign-scale planes of the two tensors as f32
+ * device arrays (the reference uploads the f16 sidecars .su / .svh / .suh as f32, 30_host_util.inc:818-861):
+ * su [d] (input plane of gate_up, "experts.su"), svh_gu [2*mid], suh_dn [mid], svh_dn [d].
+ * d % 128 == 0, mid % 128 == 0, 2*mid <= 2048 (as the reference); batches above 32 tokens also need d % 256 == 0 and
+ * mid % 256 == 0 (else they are walked through the small-batch path).  The shared expert of such a layer is not
+ * rotated: moe_set_shared as usual (q4cp with affine codebooks, or dense).  The first call allocates the scratch
+ * these layers need on top of the context's. */
+int moe_set_experts_i4r(moe_ctx* ctx, int layer, const moe_wview* gate_up, const moe_wview* down, const float* su,
+                        const float* svh_gu, const float* suh_dn, const float* svh_dn);
 /* GpuModel::moe (40_model.inc:1806) for P == 1 and GpuModel::moe_b (40_model.inc:4018) for a
  * batch: y[P][d] = routed experts (top-k, renormalised) + sigmoid-gated shared expert.
  * x, y: f32 [P][d]; y is fully overwritten.
@@ -288,6 +311,26 @@ int moe_profile_read(moe_ctx* ctx, float* ms);
 /* Copy the last call's router output (the reference keeps it in d_topids / d_topw,
  * 40_model.inc:1811) into caller buffers [P][id_stride] (device memory; async on st). */
 int moe_get_routing(moe_ctx* ctx, int P, int* ids_out, float* ws_out, moe_stream_t st);
+
+/* ---- hgn v2 rotated experts: the stages around the projections ---- */
+/* rows [row0, row0 + nrows) of an i4r tensor as f32, bit-exact (tools/moe_lut_test.cu:936-948) */
+int moe_i4r_dequant_rows(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t row0, uint64_t nrows, float* out,
+                         moe_stream_t st);
+/* k_v2_rot (28_kernels_hgn_v2.inc:62-98): y[p][i] = post[i] * H(pre . x[p])[i] / sqrt(128) per block of 128, H the
+ * Sylvester Hadamard matrix in natural order; pre / post may be NULL (= 1).  P rows of n values (n % 128 == 0), row
+ * strides xs / ys in elements.  out_f16 = 0: f32 rows (in place is fine); 1: f16 rows in layout 1 of moe_f32_to_f16
+ * (what moe_lut_up_raw reads). */
+int moe_v2_rot(const float* x, uint64_t xs, void* y, uint64_t ys, const float* pre, const float* post, int n, int P,
+               int out_f16, moe_stream_t st);
+/* k_i4r_mid (28_kernels_hgn_v2.inc:105-150): per slot, g | u = svh_gu . H(guv) / sqrt(128), h = silu(g) * u,
+ * out = H(suh_dn . h) / sqrt(128).  guv: [nslots][gs] f32 or f16 (2*mid used), out: [nslots][os] f32, or f16 in
+ * layout 1 (what moe_lut_down reads).  mid % 128 == 0, 2*mid <= 2048. */
+int moe_i4r_mid(const void* guv, int guv_f16, uint64_t gs, void* out, int out_f16, uint64_t os, const float* svh_gu,
+                const float* suh_dn, int mid, int nslots, moe_stream_t st);
+/* k_v2_reduce_rot (28_kernels_hgn_v2.inc:153-187): moe_reduce_pw_sg with svh . H(sum) / sqrt(128) applied to the
+ * weighted sum before the shared expert's rows are added; D % 128 == 0. */
+int moe_v2_reduce_rot(const void* pairs, int pairs_f16, const int* pairids, const float* pw, const float* svh,
+                      const float* ey, const float* sg, float* out, int P, int D, int K, moe_stream_t st);
 
 /* ---- checkpoint files -> HBM ---- */
 

@@ -18,6 +18,9 @@
  *   src/ref.cpp:563-637  Model::moe (router, top-k, experts, shared expert)
  *   src/gpu/parts/10_ple_io.inc:784-825  expert-sorted permutation + tiles
  *   src/gpu/parts/24_kernels_moe_lt.inc:126-161  HC write-back folded into the combine
+ *   tools/moe_lut_test.cu:936-948, tools/v2repro/v2enc.py:87-101  hgn v2 i4r rows: (nibble - 8) * fp16 scale per 128
+ *   src/gpu/parts/27_kernels_moe_lut.inc:44-65, 28_kernels_hgn_v2.inc:62-150, 40_model.inc:1638-1656
+ *                        hgn v2 rotated experts: 128-block Hadamard on the activations around each projection
  *
  * Pinning status of every function is listed in oracle/README.md; each one is
  * checked in tests/ against the reference's own code built under oracle/_ref
@@ -47,7 +50,8 @@
 enum { ORC_F32 = 1, ORC_BF16 = 0, ORC_Q4CP = 5, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q5_1 = 7, ORC_Q8_0 = 8,
        ORC_IQ4_NL = 20, ORC_IQ4_XS = 23,
        ORC_Q8G64 = 107 /* hgn dtype 7; the tag is moved off ggml's Q5_1 = 7 */,
-       ORC_Q8G32 = 108 /* hgn dtype 8 (moved off ggml's Q8_0 = 8) */ };
+       ORC_Q8G32 = 108 /* hgn dtype 8 (moved off ggml's Q8_0 = 8) */,
+       ORC_I4R = 123 /* hgn v2 dtype 23 (moved off ggml's IQ4_XS = 23) */ };
 
 /* src/hgn.h:77-84 and src/gguf.h:318-325 (same function twice in the reference) */
 ORC_API float orc_fp16_to_f32(uint16_t h) {
@@ -289,7 +293,41 @@ static void mat_row(const orc_mat* W, uint64_t r, float* out) {
       }
       break;
     }
+    case ORC_I4R: { /* tools/moe_lut_test.cu:936-948: [rows][cols/2] codes (byte b = element 2b | 2b+1 << 4), then
+                       [rows][cols/128] fp16 scales, rows unpadded; w = (nibble - 8) * scale */
+      const uint8_t* codes = W->data + r * (W->cols / 2);
+      const uint16_t* sc = (const uint16_t*)(W->data + W->rows * (W->cols / 2) + r * (W->cols / 128 * 2));
+      for (uint64_t c = 0; c < W->cols; c++) {
+        const uint8_t b = codes[c >> 1];
+        const int nib = (c & 1) ? b >> 4 : b & 15;
+        out[c] = (float)(nib - 8) * orc_fp16_to_f32(sc[c >> 7]);
+      }
+      break;
+    }
     default: memset(out, 0, W->cols * 4);
+  }
+}
+
+/* ---- hgn v2 rotation (src/gpu/parts/27_kernels_moe_lut.inc:44-65, 28_kernels_hgn_v2.inc:62-98) ----
+ * y[i] = post[i] * H(pre . x)[i] / sqrt(128) per block of 128, H the Sylvester Hadamard matrix in natural order;
+ * the butterflies run over strides 1, 2, ..., 64 with (lo + hi, lo - hi) in f32, the order of the reference's fwht128.
+ * pre / post may be NULL (= 1).  In place is fine. */
+static const float kRs128 = 0.0883883476483184405f;
+static void fwht128(float* v) {
+  for (int h = 1; h < 128; h <<= 1)
+    for (int i = 0; i < 128; i += 2 * h)
+      for (int j = i; j < i + h; j++) {
+        const float a = v[j], b = v[j + h];
+        v[j] = a + b;
+        v[j + h] = a - b;
+      }
+}
+ORC_API void orc_v2_rot(const float* x, float* y, const float* pre, const float* post, int n) {
+  float v[128];
+  for (int b = 0; b < n / 128; b++) {
+    for (int i = 0; i < 128; i++) v[i] = x[b * 128 + i] * (pre ? pre[b * 128 + i] : 1.f);
+    fwht128(v);
+    for (int i = 0; i < 128; i++) y[b * 128 + i] = v[i] * kRs128 * (post ? post[b * 128 + i] : 1.f);
   }
 }
 ORC_API void orc_mat_rows(const orc_mat* W, uint64_t row0, uint64_t nrows, float* out) {
@@ -443,6 +481,9 @@ typedef struct {
   orc_mat sh_gate, sh_up, sh_down; /* [mid][d],[mid][d],[d][mid] */
   orc_mat sh_sg;           /* [1][d] */
   int has_shared;
+  /* hgn v2 rotated routed experts (all four NULL otherwise): input / output sign-scale planes of the two expert
+   * tensors, f32: su_gu [d], svh_gu [2*mid], suh_dn [mid], svh_dn [d] */
+  const float *su_gu, *svh_gu, *suh_dn, *svh_dn;
 } orc_layer;
 
 static void expert_rows_gate_up(const orc_layer* L, int e, int r, float* out) {
@@ -459,6 +500,10 @@ static void expert_rows_gate_up(const orc_layer* L, int e, int r, float* out) {
  * routed to it) which changes no value: every dot product is an independent
  * fp64 chain, and each token's f32 accumulation still runs in rank order.
  * ids/ws are outputs ([T][id_stride]); hid_out (optional) is [T][k][mid].
+ * hgn v2 layers (rotation planes set; 40_model.inc:1638-1656): the routed experts see rot_in(x, su_gu); their
+ * gate|up outputs go through rot_out(svh_gu) before SwiGLU and the result through rot_in(suh_dn)
+ * (k_i4r_mid, 28_kernels_hgn_v2.inc:105-150); the weighted sum over the experts through rot_out(svh_dn); the
+ * shared expert reads the plain x.  hid_out then holds the rotated down-projection inputs.
  */
 ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int* tok_list,
                            int n_list, int id_stride, int* ids, float* ws, float* hid_out,
@@ -466,6 +511,17 @@ ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int*
   const int d = L->d, mid = L->mid, E = L->E, k = L->k;
   orc_router(&L->router, L->router_bias, x, T, k, id_stride, NULL, ids, ws);
   const int n = tok_list ? n_list : T;
+  const int v2 = L->su_gu != NULL;
+  const float* xe = x; /* what the routed experts read */
+  float* xrot = NULL;
+  if (v2) {
+    xrot = (float*)malloc((size_t)T * d * 4);
+    for (int i = 0; i < n; i++) {
+      const int t = tok_list ? tok_list[i] : i;
+      orc_v2_rot(x + (size_t)t * d, xrot + (size_t)t * d, L->su_gu, NULL, d);
+    }
+    xe = xrot;
+  }
   /* pair list grouped by expert (only tokens in the list) */
   int* cnt = (int*)calloc((size_t)E + 1, sizeof(int));
   for (int i = 0; i < n; i++) {
@@ -500,14 +556,16 @@ ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int*
         expert_rows_gate_up(L, e, r, wr);
         for (int q = cnt[e]; q < cnt[e + 1]; q++) {
           const int i = pair_i[q], t = tok_list ? tok_list[i] : i;
-          guv[((size_t)i * k + pair_s[q]) * 2 * mid + r] = dot_f64(wr, x + (size_t)t * d, d);
+          guv[((size_t)i * k + pair_s[q]) * 2 * mid + r] = dot_f64(wr, xe + (size_t)t * d, d);
         }
       }
 #pragma omp for schedule(static)
-    for (int i = 0; i < n * k; i++)
-      for (int r = 0; r < mid; r++)
-        hid[(size_t)i * mid + r] =
-            siluf_ref(guv[(size_t)i * 2 * mid + r]) * guv[(size_t)i * 2 * mid + mid + r];
+    for (int i = 0; i < n * k; i++) {
+      float* z = guv + (size_t)i * 2 * mid;
+      if (v2) orc_v2_rot(z, z, NULL, L->svh_gu, 2 * mid);
+      for (int r = 0; r < mid; r++) hid[(size_t)i * mid + r] = siluf_ref(z[r]) * z[mid + r];
+      if (v2) orc_v2_rot(hid + (size_t)i * mid, hid + (size_t)i * mid, L->suh_dn, NULL, mid);
+    }
 #pragma omp for schedule(dynamic, 16) collapse(2)
     for (int e = 0; e < E; e++)
       for (int r = 0; r < d; r++) {
@@ -530,7 +588,9 @@ ORC_API void orc_moe_layer(const orc_layer* L, const float* x, int T, const int*
       for (int s = 0; s < k; s++) acc += ws[t * id_stride + s] * dn[((size_t)i * k + s) * d + r];
       yt[r] = acc;
     }
+    if (v2) orc_v2_rot(yt, yt, NULL, L->svh_dn, d);
   }
+  free(xrot);
   if (hid_out)
     for (int i = 0; i < n; i++) {
       const int t = tok_list ? tok_list[i] : i;

@@ -14,7 +14,8 @@ F32, BF16, Q4CP, Q4K = 1, 0, 5, 12
 Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS = 13, 7, 8, 20, 23   # further ggml block types of the expert tensors (ids as in GGUF)
 Q8G64 = 107  # hgn dtype 7 (the oracle's tag is moved off ggml's Q5_1 = 7)
 Q8G32 = 108  # hgn dtype 8 (moved off ggml's Q8_0 = 8)
-HGN_DTYPE = {BF16: 0, F32: 1, Q4CP: 5, Q8G64: 7, Q8G32: 8}  # oracle tag -> dtype field of the reference's checkpoint format
+I4R = 123    # hgn v2 dtype 23 (moved off ggml's IQ4_XS = 23)
+HGN_DTYPE = {BF16: 0, F32: 1, Q4CP: 5, Q8G64: 7, Q8G32: 8, I4R: 23}  # oracle tag -> dtype field of the reference's checkpoint format
 GG_TYPES = (Q4K, Q5K, Q5_1, Q8_0, IQ4_NL, IQ4_XS)
 
 
@@ -33,7 +34,8 @@ class _Layer(C.Structure):
                 ("router", _Mat), ("router_bias", C.c_void_p),
                 ("gate_up", _Mat), ("gate", _Mat), ("up", _Mat), ("down", _Mat),
                 ("sh_gate", _Mat), ("sh_up", _Mat), ("sh_down", _Mat), ("sh_sg", _Mat),
-                ("has_shared", C.c_int)]
+                ("has_shared", C.c_int),
+                ("su_gu", C.c_void_p), ("svh_gu", C.c_void_p), ("suh_dn", C.c_void_p), ("svh_dn", C.c_void_p)]
 
 
 _lib = None
@@ -109,6 +111,8 @@ class Mat:
             assert self.data.dtype == np.uint8 and cols % 64 == 0 and self.data.size == rows * (cols + cols // 64 * 4)
         elif dtype == Q8G32:
             assert self.data.dtype == np.uint8 and cols % 32 == 0 and self.data.size == rows * cols + rows * cols // 32 * 2
+        elif dtype == I4R:
+            assert self.data.dtype == np.uint8 and cols % 128 == 0 and self.data.size == rows * cols // 2 + rows * cols // 128 * 2
 
     def c(self):
         return _Mat(self.dtype, self.data.ctypes.data, self.rows, self.cols)
@@ -125,7 +129,7 @@ class Mat:
             return gg_rows(self.dtype, self.data[row0 * rb:(row0 + nrows) * rb], nrows, self.cols)
         if self.dtype == F32:
             return self.data.reshape(self.rows, self.cols)[row0:row0 + nrows].copy()
-        if self.dtype in (Q8G64, Q8G32):
+        if self.dtype in (Q8G64, Q8G32, I4R):
             out = np.empty((nrows, self.cols), np.float32)
             m = self.c()
             lib().orc_mat_rows(C.byref(m), row0, nrows, _p(out))
@@ -246,8 +250,10 @@ class Layer:
     """One MoE layer's weights for the oracle (numpy-backed)."""
 
     def __init__(self, d, mid, E, k, router, down, gate_up=None, gate=None, up=None,
-                 shared=None, router_bias=None):
+                 shared=None, router_bias=None, rot=None):
         self.d, self.mid, self.E, self.k = d, mid, E, k
+        # hgn v2 rotated experts: (su_gu [d], svh_gu [2 mid], suh_dn [mid], svh_dn [d]) as f32, else None
+        self.rot = tuple(_c(a, np.float32) for a in rot) if rot is not None else None
         self.router, self.down, self.gate_up, self.gate, self.up = router, down, gate_up, gate, up
         self.shared = shared  # (sh_gate, sh_up, sh_down, sh_sg) or None
         self.router_bias = _c(router_bias, np.float32) if router_bias is not None else None
@@ -267,6 +273,8 @@ class Layer:
         else:
             L.sh_gate = L.sh_up = L.sh_down = L.sh_sg = _NULL
             L.has_shared = 0
+        if self.rot is not None:
+            L.su_gu, L.svh_gu, L.suh_dn, L.svh_dn = (a.ctypes.data for a in self.rot)
         return L
 
 
@@ -283,6 +291,19 @@ def moe_layer(layer, x, tok_list=None, id_stride=16, want_hid=False):
     lib().orc_moe_layer(C.byref(L), _p(x), T, _p(tl), 0 if tl is None else tl.size, id_stride,
                         _p(ids), _p(ws), _p(hid), _p(y))
     return (y, ids, ws, hid) if want_hid else (y, ids, ws)
+
+
+def v2_rot(x, pre=None, post=None):
+    """post * H(pre * x) / sqrt(128) per block of 128 of every row (hgn v2 rotation)."""
+    x = _c(x, np.float32)
+    n = x.shape[-1]
+    pre = _c(pre, np.float32) if pre is not None else None
+    post = _c(post, np.float32) if post is not None else None
+    out = np.empty_like(x)
+    xr, orr = x.reshape(-1, n), out.reshape(-1, n)
+    for i in range(xr.shape[0]):
+        lib().orc_v2_rot(_p(xr[i]), _p(orr[i]), _p(pre), _p(post), n)
+    return out
 
 
 def num_threads():

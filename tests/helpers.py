@@ -36,9 +36,14 @@ class HostLayer:
             self.router = rw
             self.router_dt = O.F32
         self.bias = bias
+        self.planes = None
         if fmt == "q4cp":
             self.gate_up = S.make_q4cp(rng, E * 2 * mid, d, codebook=codebook, scale_std=scale_std)
             self.down = S.make_q4cp(rng, E * d, mid, codebook=codebook, scale_std=scale_std)
+        elif fmt == "i4r":  # hgn v2 rotated experts (the shared expert as in a q4cp layer)
+            self.gate_up = S.make_i4r(rng, E * 2 * mid, d, scale_std=scale_std)
+            self.down = S.make_i4r(rng, E * d, mid, scale_std=scale_std)
+            self.planes = S.make_v2_planes(rng, d, mid)
         else:
             self.gate = S.make_gg(rng, self.tgu, E * mid, d, scale_std=scale_std)
             self.up = S.make_gg(rng, self.tgu, E * mid, d, scale_std=scale_std)
@@ -46,7 +51,7 @@ class HostLayer:
         self.shared = None
         if shared:
             scb = shared_codebooks if shared_codebooks is not None else [codebook] * 3
-            mk = (lambda r, c, i: S.make_q4cp(rng, r, c, codebook=scb[i], scale_std=scale_std)) if fmt == "q4cp" \
+            mk = (lambda r, c, i: S.make_q4cp(rng, r, c, codebook=scb[i], scale_std=scale_std)) if fmt in ("q4cp", "i4r") \
                 else (lambda r, c, i: S.make_gg(rng, self.tsh, r, c, scale_std=scale_std))
             if shared_dense:
                 mk = lambda r, c, i: S.make_dense(rng, shared_dense, r, c, std=0.05)
@@ -55,18 +60,19 @@ class HostLayer:
 
     def oracle_layer(self):
         d, mid, E, k = self.d, self.mid, self.E, self.k
-        wt = O.Q4CP if self.fmt == "q4cp" else O.Q4K
+        wt = O.Q4CP if self.fmt == "q4cp" else O.I4R if self.fmt == "i4r" else O.Q4K
         sh = None
         if self.shared is not None:
-            st = O.Q4CP if self.fmt == "q4cp" else self.tsh
+            st = O.Q4CP if self.fmt in ("q4cp", "i4r") else self.tsh
             if self.shared_dense:
                 st = {"bf16": O.BF16, "f32": O.F32, "q8g64": O.Q8G64, "q8g32": O.Q8G32}[self.shared_dense]
             sh = [O.Mat(st, self.shared[0], mid, d), O.Mat(st, self.shared[1], mid, d),
                   O.Mat(st, self.shared[2], d, mid), O.Mat(O.F32, self.shared[3], 1, d)]
         router = O.Mat(self.router_dt, self.router, E, d)
-        if self.fmt == "q4cp":
+        if self.fmt in ("q4cp", "i4r"):
             return O.Layer(d, mid, E, k, router, O.Mat(wt, self.down, E * d, mid),
-                           gate_up=O.Mat(wt, self.gate_up, E * 2 * mid, d), shared=sh, router_bias=self.bias)
+                           gate_up=O.Mat(wt, self.gate_up, E * 2 * mid, d), shared=sh, router_bias=self.bias,
+                           rot=self.planes)
         return O.Layer(d, mid, E, k, router, O.Mat(self.tdn, self.down, E * d, mid),
                        gate=O.Mat(self.tgu, self.gate, E * mid, d), up=O.Mat(self.tgu, self.up, E * mid, d), shared=sh,
                        router_bias=self.bias)
@@ -89,10 +95,14 @@ class HostLayer:
         if self.fmt == "q4cp":
             m.set_experts_q4cp(0, capi.wview(up("gate_up", self.gate_up), capi.Q4CP, E * 2 * mid, d),
                                capi.wview(up("down", self.down), capi.Q4CP, E * d, mid))
+        elif self.fmt == "i4r":
+            m.set_experts_i4r(0, capi.wview(up("gate_up", self.gate_up), capi.I4R, E * 2 * mid, d),
+                              capi.wview(up("down", self.down), capi.I4R, E * d, mid),
+                              *(up("plane%d" % i, a) for i, a in enumerate(self.planes)))
         else:
             m.set_experts_gguf(0, up("gate", self.gate), up("up", self.up), up("down", self.down), self.tgu, self.tdn)
         if self.shared is not None:
-            wt = capi.Q4CP if self.fmt == "q4cp" else 0
+            wt = capi.Q4CP if self.fmt in ("q4cp", "i4r") else 0
             shw = self.shared[:3]
             if self.shared_dense:
                 wt = {"bf16": capi.BF16, "f32": capi.F32, "q8g64": capi.Q8G64, "q8g32": capi.Q8G32}[self.shared_dense]
@@ -102,5 +112,5 @@ class HostLayer:
                          capi.wview(up("shu", shw[1]), wt, mid, d),
                          capi.wview(up("shd", shw[2]), wt, d, mid),
                          capi.wview(up("shsg", self.shared[3]), capi.F32, 1, d),
-                         0 if self.fmt == "q4cp" or self.shared_dense else self.tsh)
+                         0 if self.fmt in ("q4cp", "i4r") or self.shared_dense else self.tsh)
         return m, dev

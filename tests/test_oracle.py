@@ -350,6 +350,86 @@ def test_layer_matches_float64_numpy_q4k(oracle):
         assert np.abs(y[t] - want).max() <= 2e-5 * np.abs(want).max()
 
 
+def test_i4r_rows_closed_form(oracle):
+    """hgn v2 i4r rows: every code value times positive, negative, subnormal and zero scales against the published
+    layout evaluated element-wise in numpy (codes plane, low nibble first, then one fp16 scale per 128 columns, rows
+    unpadded; w = (n - 8) * scale, exact in f32)."""
+    O = oracle
+    rows, cols = 6, 384
+    rng = np.random.default_rng(23)
+    codes = rng.integers(0, 256, size=(rows, cols // 2), dtype=np.uint8)
+    codes[0, :8] = [0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE]  # elements 0..15 of row 0 hold the codes 0..15
+    sc = (rng.standard_normal((rows, cols // 128)) * 0.02).astype(np.float16)
+    sc[1, 0], sc[2, 1], sc[3, 2] = np.float16(6e-8), np.float16(0.0), np.float16(-1.5)
+    blob = np.concatenate([codes.reshape(-1), sc.reshape(-1).view(np.uint8)])
+    got = O.Mat(O.I4R, blob, rows, cols).dequant()
+    q = np.stack([codes & 15, codes >> 4], -1).reshape(rows, cols).astype(np.float32) - 8
+    want = (q.reshape(rows, -1, 128) * sc.astype(np.float32)[..., None]).reshape(rows, cols)
+    assert same_bits(got, bits(want))
+    assert (got[0, :16] == (np.arange(16, dtype=np.float32) - 8) * np.float32(sc[0, 0])).all()
+
+
+def test_v2_rotation_against_the_hadamard_matrix(oracle):
+    """rot(x) = post * H(pre * x) / sqrt(128) per 128 block against scipy's Sylvester matrix in float64; H / sqrt(128) is
+    its own inverse; a unit vector gives a column of +-1 / sqrt(128) with the sign pattern popcount(i & j)."""
+    from scipy.linalg import hadamard
+    O = oracle
+    rng = np.random.default_rng(24)
+    n = 384
+    x = rng.standard_normal((5, n)).astype(np.float32)
+    pre, post = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    Hn = hadamard(128).astype(np.float64) / np.sqrt(128.0)
+    want = np.stack([np.concatenate([Hn @ (x[t, b:b + 128].astype(np.float64) * pre[b:b + 128]) for b in range(0, n, 128)])
+                     for t in range(5)]) * post
+    got = O.v2_rot(x, pre, post)
+    assert np.abs(got - want).max() <= 2e-6 * np.abs(want).max()
+    back = O.v2_rot(O.v2_rot(x))
+    assert np.abs(back - x).max() <= 2e-6 * np.abs(x).max()
+    e = np.zeros((1, 128), np.float32)
+    e[0, 77] = 1.0
+    col = O.v2_rot(e)[0]
+    sign = np.array([(-1) ** bin(i & 77).count("1") for i in range(128)], np.float32)
+    assert (col == sign * np.float32(0.0883883476483184405)).all()
+
+
+def test_v2_layer_equals_the_unrotated_layer_in_float64(oracle):
+    """An hgn v2 layer (rotated i4r experts) against an independent float64 evaluation of the ordinary layer on the
+    un-rotated weights W = diag(svh) . Hn . G . Hn . diag(suh) (Hn = block-diagonal H / sqrt(128)): a wrong plane, a
+    swapped input / output side or a missing rotation would change the result by O(1)."""
+    from scipy.linalg import hadamard
+    O = oracle
+    rng = np.random.default_rng(25)
+    d, mid, E, k = 256, 128, 6, 3
+    hl = HostLayer(rng, d, mid, E, k, fmt="i4r", scale_std=0.02, router_std=0.2)
+    L = hl.oracle_layer()
+    x = rng.standard_normal((4, d)).astype(np.float32)
+    y, ids, ws = O.moe_layer(L, x)
+    su, svh_gu, suh_dn, svh_dn = (p.astype(np.float64) for p in hl.planes)
+    Hn = hadamard(128).astype(np.float64) / np.sqrt(128.0)
+
+    def unrot(G, sv, su_):  # G [O][K] in the rotated domain -> W
+        O_, K = G.shape
+        W = G.reshape(O_, K // 128, 128) @ Hn           # . Hn on the input side (Hn symmetric)
+        W = W.reshape(O_, K)
+        W = (Hn @ W.reshape(O_ // 128, 128, K)).reshape(O_, K)
+        return sv[:, None] * W * su_[None, :]
+    GU = L.gate_up.dequant().astype(np.float64)
+    DN = L.down.dequant().astype(np.float64)
+    shg, shu, shd, sg = (m.dequant().astype(np.float64) for m in L.shared)
+    for t in range(4):
+        xt = x[t].astype(np.float64)
+        acc = np.zeros(d)
+        for s in range(k):
+            e = ids[t, s]
+            W = unrot(GU[e * 2 * mid:(e + 1) * 2 * mid], svh_gu, su)
+            g, u = W[:mid] @ xt, W[mid:] @ xt
+            h = g / (1 + np.exp(-g)) * u
+            acc += float(ws[t, s]) * (unrot(DN[e * d:(e + 1) * d], svh_dn, suh_dn) @ h)
+        g, u = shg @ xt, shu @ xt
+        want = acc + (shd @ (g / (1 + np.exp(-g)) * u)) / (1 + np.exp(-(sg @ xt)))
+        assert np.abs(y[t] - want).max() <= 2e-5 * np.abs(want).max()
+
+
 @pytest.mark.parametrize("t,name", [(13, "Q5_K"), (8, "Q8_0"), (7, "Q5_1"), (12, "Q4_K"), (20, "IQ4_NL"), (23, "IQ4_XS")])
 def test_gg_rows_against_reference(oracle, t, name):
     """The further ggml block types of the expert tensors: the oracle's rows against the reference's own
