@@ -2,7 +2,8 @@
 """Benchmark of the routed-expert MoE layer on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
-                  [--workload headline|prefill|decode|verify|q4k_prefill|q4k_decode|stack|ggmix_decode|ggmix_verify]
+                  [--workload headline|prefill|decode|verify|q4k_prefill|q4k_decode|stack|ggmix_decode|ggmix_verify|
+                              v2_prefill|v2_decode|v2_verify]
 
 One step = one pass of the MoE layer (moe_forward) over one batch of synthetic input that is
 already resident in HBM.  Prints ONE JSON line: whole-layer throughput, the roofline figure of the
@@ -105,11 +106,12 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     d, mid, k = D, MID, K
     # ggmix_*: GGUF layer in the reference checkpoints' type mix (Q5_K gate/up, Q8_0 down, Q8_0 shared expert) on the
     # general GEMV kernels
+    # v2_*: hgn v2 layer (Hadamard-rotated i4r routed experts, q4cp shared expert)
     ggmix = wl.startswith("ggmix_")
-    fmt = "q4k" if wl.startswith("q4k") or ggmix else "q4cp"
+    fmt = "q4k" if wl.startswith("q4k") or ggmix else "i4r" if wl.startswith("v2_") else "q4cp"
     gg_types = (13, 8, 8) if ggmix else (12, 12, 12)
-    kind = wl.replace("q4k_", "").replace("ggmix_", "")
-    T = tokens or {"prefill": 16384 if fmt == "q4cp" else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
+    kind = wl.replace("q4k_", "").replace("ggmix_", "").replace("v2_", "")
+    T = tokens or {"prefill": 16384 if fmt in ("q4cp", "i4r") else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
     nlayers = nlayers_arg if kind == "stack" else 1
 
     layers = [W.DeviceLayer(1000 + l, d, mid, E, k, fmt, gg_types=gg_types, codebook=codebook) for l in range(nlayers)]
@@ -209,6 +211,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     cfg = {"workload": wl, "tokens": T, "d_model": d, "moe_mid": mid, "experts": E, "topk": k, "shared_experts": 1,
            "format": ("q4cp g32, the reference converter's universal expert codebook (table look-up, f32 GEMV kernels)"
                       if universal else "q4cp g32 zero-point 8") if fmt == "q4cp" else
+           "hgn v2 i4r g128, Hadamard-rotated (q4cp shared expert)" if fmt == "i4r" else
            ("GGUF Q5_K gate/up, Q8_0 down, Q8_0 shared expert" if ggmix else "GGUF Q4_K"),
            "layers": nlayers, **extra}
     if kind == "prefill":
@@ -224,7 +227,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
                     "dtype": "f16",
                     "layer_tflops": round(flop_tok * T / (ms * 1e-3) / 1e12, 2),
                     "layer_mfma_frac": round(flop_tok * T / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                    "roofline": {"bound": "mfma", "kernel": "k_moe_gemm (gate/up + SwiGLU), " +
+                    "roofline": {"bound": "mfma", "kernel": ("k_moe_gemm (gate | up unfused) + the slot-wise rotations and SwiGLU, "
+                                                              if fmt == "i4r" else "k_moe_gemm (gate/up + SwiGLU), ") +
                                  ("routed + shared expert tiles" if shared_in_launch else "routed experts' tiles"),
                                  "achieved": round(up_flop / up_s / 1e12, 2), "peak": MFMA_F16_PEAK_TFLOPS,
                                  "unit": "TFLOP/s", "frac": round(up_flop / up_s / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
@@ -243,6 +247,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
         step_bytes = nlayers * (uniq * eb + layers[0].shared_bytes() + E * d * 4 + d * 4 + T * 2 * d * 4)
         if fmt == "q4cp":
             gu_bytes = (uniq + 1) * 2 * mid * (d // 2 + S.q4cp_scale_stride(d))
+        elif fmt == "i4r":
+            gu_bytes = uniq * 2 * mid * (d // 2 + d // 128 * 2) + 2 * mid * (d // 2 + S.q4cp_scale_stride(d))
         else:
             gu_bytes = 2 * mid * (uniq * W.gg_row_bytes(gg_types[0], d) + W.gg_row_bytes(gg_types[2], d))
         up_s = up_marginal_ms * 1e-3
@@ -253,7 +259,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
         # or plain f32 FMAs (MOE_OPT_INT_DECODE = 0, and the general GGUF kernels)
         res.update({"metric": "moe_layer_decode_hbm_GB_per_s", "unit": "GB/s",
                     "value": round(step_bytes / (ms * 1e-3) / 1e9, 1),
-                    "dtype": "f32" if not int_dec else ("i4" if fmt == "q4cp" else "i8"),
+                    "dtype": "f32" if not int_dec else ("i4" if fmt in ("q4cp", "i4r") else "i8"),
                     "up_kernel_ms": round(up_marginal_ms, 5),
                     "hbm_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "tokens_per_s": round(T / (ms * 1e-3), 1),

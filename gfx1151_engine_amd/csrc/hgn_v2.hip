@@ -135,59 +135,56 @@ __global__ void __launch_bounds__(256) k_v2_rot(const float* x, uint64_t xs, voi
   }
 }
 
-// The middle of an i4r expert, one block per (token, expert) slot, ceil(2 mid / 512) waves:
+// The middle of an i4r expert, per (token, expert) slot:
 //   g | u = svh_gu . H(z) / sqrt(128)      z = the slot's rotated gate_up output [2 mid]
 //   h     = silu(g) * u
 //   out   = H(suh_dn . h) / sqrt(128)      the rotated input of down_proj [mid]
+// Sixteen lanes per 128-block b of the slot: they rotate block b of the gate half and block b of the up half (each
+// lane then holds g and u of its 8 columns), apply SwiGLU and rotate the result.  No LDS, no block barrier.
 // MODE 0: f32 rows, 1: f16 rows in the grouped GEMM's order, 2: digit planes; slot s of the launch goes to output
 // row (s / k) * row_slots + s % k (the decode path keeps a token's slots next to its shared-expert slot).
+// MODE 1 (batches: the result is rounded to f16) takes the hardware's exp2 / reciprocal approximations (1 ulp) in
+// SwiGLU, as the grouped GEMM's fused epilogue does; the other modes the exact expf and division.
 template <class TG, int MODE>
 __global__ void __launch_bounds__(256) k_i4r_mid(const TG* __restrict__ z, uint64_t zs, void* out, uint64_t os,
                                                  const float* __restrict__ svh_gu, const float* __restrict__ suh_dn,
-                                                 int mid, int k, int row_slots, uint32_t* __restrict__ planes,
-                                                 float2* __restrict__ meta) {
-  __shared__ float s[2048];
-  const int slot = blockIdx.x, lane = threadIdx.x & 63;
-  const int c = threadIdx.x * 8;
-  {
-    const bool live = c < 2 * mid;
-    float v[8], f[8];
+                                                 int mid, int nslots, int k, int row_slots,
+                                                 uint32_t* __restrict__ planes, float2* __restrict__ meta) {
+  const int lane = threadIdx.x & 63;
+  const int nb = mid >> 7;
+  const int64_t grp = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  const int slot = (int)(grp / nb), b = (int)(grp - (int64_t)slot * nb);
+  const bool live = slot < nslots;
+  const int c = b * 128 + (lane & 15) * 8;  // this lane's 8 columns of each half
+  float g[8], u[8], fg[8], fu[8], sd[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) v[i] = 0.f, f[i] = 0.f;
-    if (live) {
-      ld8(z + (size_t)slot * zs + c, v);
-      ld8(svh_gu + c, f);
-    }
-    moe_fwht128_r8(v, lane);
-    if (live) {
-#pragma unroll
-      for (int i = 0; i < 8; i++) s[c + i] = v[i] * MOE_RS128 * f[i];
-    }
-  }
-  __syncthreads();
-  const bool live = c < mid;
-  float v[8];
-#pragma unroll
-  for (int i = 0; i < 8; i++) v[i] = 0.f;
+  for (int i = 0; i < 8; i++) g[i] = u[i] = fg[i] = fu[i] = sd[i] = 0.f;
   if (live) {
-    float f[8];
-    ld8(suh_dn + c, f);
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const float g = s[c + i], u = s[mid + c + i];
-      v[i] = g / (1.f + expf(-g)) * u * f[i];
-    }
+    ld8(z + (size_t)slot * zs + c, g);
+    ld8(z + (size_t)slot * zs + mid + c, u);
+    ld8(svh_gu + c, fg);
+    ld8(svh_gu + mid + c, fu);
+    ld8(suh_dn + c, sd);
   }
-  moe_fwht128_r8(v, lane);
+  moe_fwht128_r8(g, lane);
+  moe_fwht128_r8(u, lane);
+  float h[8];
 #pragma unroll
-  for (int i = 0; i < 8; i++) v[i] *= MOE_RS128;
-  const size_t row = (size_t)(slot / k) * row_slots + slot % k;
+  for (int i = 0; i < 8; i++) {
+    const float gv = g[i] * MOE_RS128 * fg[i], uv = u[i] * MOE_RS128 * fu[i];
+    if (MODE == 1) h[i] = gv * __builtin_amdgcn_rcpf(1.f + __expf(-gv)) * uv * sd[i];
+    else h[i] = gv / (1.f + expf(-gv)) * uv * sd[i];
+  }
+  moe_fwht128_r8(h, lane);
+#pragma unroll
+  for (int i = 0; i < 8; i++) h[i] *= MOE_RS128;
+  const size_t row = live ? (size_t)(slot / k) * row_slots + slot % k : 0;
   if (MODE == 0) {
-    if (live) st8((float*)out + row * os + c, v);
+    if (live) st8((float*)out + row * os + c, h);
   } else if (MODE == 1) {
-    if (live) st8_f16_ilv((__half*)out + row * os + c, v);
+    if (live) st8_f16_ilv((__half*)out + row * os + c, h);
   } else {
-    st8_planes(v, lane, planes, meta, row * (mid >> 5) + (c >> 5), live);
+    st8_planes(h, lane, planes, meta, row * (mid >> 5) + (c >> 5), live);
   }
 }
 
@@ -262,9 +259,10 @@ int moe_launch_i4r_mid(const void* z, bool z_f16, uint64_t zs, int nslots, int m
       !moe_aligned(suh_dn, 16))
     return MOE_E_INVALID;
   if (nslots == 0) return MOE_OK;
-  const int bs = 64 * ((2 * mid / 8 + 63) / 64);
+  const int64_t threads = (int64_t)nslots * (mid / 128) * 16;
+  const unsigned grid = (unsigned)((threads + 255) / 256);
 #define MID_GO(TG, M) \
-  k_i4r_mid<TG, M><<<nslots, bs, 0, st>>>((const TG*)z, zs, out, os, svh_gu, suh_dn, mid, k, row_slots, planes, meta)
+  k_i4r_mid<TG, M><<<grid, 256, 0, st>>>((const TG*)z, zs, out, os, svh_gu, suh_dn, mid, nslots, k, row_slots, planes, meta)
   if (z_f16) {
     if (mode == 0) MID_GO(__half, 0); else if (mode == 1) MID_GO(__half, 1); else MID_GO(__half, 2);
   } else {

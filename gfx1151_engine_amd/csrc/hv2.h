@@ -7,6 +7,18 @@
 
 constexpr float MOE_RS128 = 0.0883883476483184405f;  // 1 / sqrt(128)
 
+// the value of lane (l ^ S) of the same row of 16 lanes, S = 1, 2, 4, 8: data-parallel-primitive moves (no trip
+// through the LDS crossbar).  l ^ 4 = half-row mirror followed by a quad reversal; l ^ 8 = rotation of the row by 8.
+template <int S>
+__device__ __forceinline__ float moe_row_xor(float v) {
+  const int b = __float_as_int(v);
+  if (S == 1) return __int_as_float(__builtin_amdgcn_update_dpp(0, b, 0xB1, 0xf, 0xf, true));
+  if (S == 2) return __int_as_float(__builtin_amdgcn_update_dpp(0, b, 0x4E, 0xf, 0xf, true));
+  if (S == 8) return __int_as_float(__builtin_amdgcn_update_dpp(0, b, 0x128, 0xf, 0xf, true));
+  const int m = __builtin_amdgcn_update_dpp(0, b, 0x141, 0xf, 0xf, true);
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, m, 0x1B, 0xf, 0xf, true));
+}
+
 // Unnormalised Hadamard transform of 128 values spread over 16 consecutive lanes (an aligned group of 16), lane j of
 // the group holding elements 8j .. 8j+7.  The butterflies (lo + hi, lo - hi) run over strides 1, 2, 4 inside the
 // lane and 8 .. 64 across lanes, i.e. in ascending stride order whatever the distribution: the same f32 additions
@@ -21,13 +33,17 @@ __device__ __forceinline__ void moe_fwht128_r8(float (&v)[8], int lane) {
         v[i] = a + b;
         v[i | h] = a - b;
       }
-#pragma unroll
-  for (int s = 1; s < 16; s <<= 1) {
-    const bool hi = (lane & s) != 0;
-#pragma unroll
-    for (int i = 0; i < 8; i++) {
-      const float p = __shfl_xor(v[i], s, 64);
-      v[i] = hi ? p - v[i] : v[i] + p;
-    }
+#define MOE_FWHT_STEP(S)                                  \
+  {                                                       \
+    const bool hi = (lane & S) != 0;                      \
+    _Pragma("unroll") for (int i = 0; i < 8; i++) {       \
+      const float p = moe_row_xor<S>(v[i]);               \
+      v[i] = hi ? p - v[i] : v[i] + p;                    \
+    }                                                     \
   }
+  MOE_FWHT_STEP(1)
+  MOE_FWHT_STEP(2)
+  MOE_FWHT_STEP(4)
+  MOE_FWHT_STEP(8)
+#undef MOE_FWHT_STEP
 }

@@ -555,6 +555,25 @@ int upload_f32_as_bf16(moe_weights* w, const FTensor& t, const uint8_t** dev) {
   return MOE_OK;
 }
 
+// An f16 vector of the file (an hgn v2 sign-scale plane, dtype 2) as f32 in device memory, as the reference uploads
+// its sidecars (src/gpu/parts/30_host_util.inc:824-838)
+int upload_f16_as_f32(moe_weights* w, const FTensor& t, uint64_t want_n, const float** dev) {
+  if (t.dtype != MOE_DT_F16 || t.nbytes != want_n * 2) return MOE_E_INVALID;
+  std::vector<float> h(want_n);
+  for (uint64_t i = 0; i < want_n; i++) {
+    _Float16 v;
+    memcpy(&v, t.data + 2 * i, 2);
+    h[i] = (float)v;
+  }
+  void* p = nullptr;
+  MOE_HIP(hipMalloc(&p, want_n ? want_n * 4 : 1));
+  w->dev.push_back(p);
+  w->bytes += want_n * 4;
+  MOE_HIP(hipMemcpy(p, h.data(), want_n * 4, hipMemcpyHostToDevice));
+  *dev = (const float*)p;
+  return MOE_OK;
+}
+
 // mtp: the MTP draft layer's MoE, stored as mtp.layers.<i>.mlp.* (src/gpu/parts/40_model.inc:5546-5548,5893)
 int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st, bool mtp) {
   auto findp = [&](const char* leaf) -> const FTensor* {
@@ -567,7 +586,10 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
   const FTensor* gu = findp("experts.gate_up_proj.weight");
   const FTensor* dn = findp("experts.down_proj.weight");
   if (!rt || !gu || !dn) return MOE_E_STATE;
-  if (!hgn_dtype_ok_dense(rt->dtype) || gu->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP) return MOE_E_UNSUPPORTED;
+  // routed experts: q4cp, or hgn v2 i4r (both tensors) with its four sign-scale planes
+  const bool v2 = gu->dtype == MOE_DT_I4R && dn->dtype == MOE_DT_I4R;
+  if (!hgn_dtype_ok_dense(rt->dtype) || (!v2 && (gu->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP)))
+    return MOE_E_UNSUPPORTED;  // (an hgn v2 file's hashed-trellis tensors, dtype 16, among them)
   int rc;
   auto view = [&](const FTensor& t, moe_wview* v) -> int {
     uint64_t rows, cols;
@@ -584,6 +606,8 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
       if (cols % 32 || __builtin_mul_overflow(rows, (uint64_t)v->scale_stride, &sc) ||
           __builtin_add_overflow(64 + cells / 2, sc, &want))
         return MOE_E_INVALID;
+    } else if (t.dtype == MOE_DT_I4R) {  // codes, then one fp16 scale per 128 columns, rows unpadded
+      if (cols % 128 || __builtin_add_overflow(cells / 2, cells / 128 * 2, &want)) return MOE_E_INVALID;
     } else if (t.dtype == MOE_DT_Q8G32) {  // planar: rows*cols int8 codes, then rows*cols/32 fp16 scales (src/hgn.h:176-183)
       if (cols % 32 || __builtin_add_overflow(cells, cells / 32 * 2, &want)) return MOE_E_INVALID;
     } else if (t.dtype == MOE_DT_Q8G64) {  // per row: cols codes + cols/64 x (fp16 scale, fp16 min) (src/hgn.h:189-196)
@@ -599,7 +623,24 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
   moe_wview vr{}, vgu{}, vdn{};
   if ((rc = view(*rt, &vr)) || (rc = view(*gu, &vgu)) || (rc = view(*dn, &vdn))) return rc;
   if ((rc = moe_set_router(ctx, cl, &vr, nullptr))) return rc;
-  if ((rc = moe_set_experts_q4cp(ctx, cl, &vgu, &vdn))) return rc;
+  if (v2) {
+    // the planes' names (src/gpu/parts/30_host_util.inc:840-852): <tensor>.suh / <tensor>.svh without the ".weight";
+    // the input plane of gate_up_proj is shared by the layer's experts as "experts.su"
+    const FTensor* su = findp("experts.gate_up_proj.suh");
+    if (!su) su = findp("experts.su");
+    const FTensor* svg = findp("experts.gate_up_proj.svh");
+    const FTensor* sud = findp("experts.down_proj.suh");
+    const FTensor* svd = findp("experts.down_proj.svh");
+    if (!su || !svg || !sud || !svd) return MOE_E_STATE;
+    const uint64_t d = vgu.cols, mid = vdn.cols;
+    const float *p_su, *p_svg, *p_sud, *p_svd;
+    if ((rc = upload_f16_as_f32(w, *su, d, &p_su)) || (rc = upload_f16_as_f32(w, *svg, 2 * mid, &p_svg)) ||
+        (rc = upload_f16_as_f32(w, *sud, mid, &p_sud)) || (rc = upload_f16_as_f32(w, *svd, d, &p_svd)))
+      return rc;
+    if ((rc = moe_set_experts_i4r(ctx, cl, &vgu, &vdn, p_su, p_svg, p_sud, p_svd))) return rc;
+  } else if ((rc = moe_set_experts_q4cp(ctx, cl, &vgu, &vdn))) {
+    return rc;
+  }
   const FTensor* sg = findp("shared_expert.gate_proj.weight");
   if (sg) {
     const FTensor* su = findp("shared_expert.up_proj.weight");

@@ -10,6 +10,7 @@ import struct
 import numpy as np
 
 HGN_BF16, HGN_F32, HGN_Q4CP, HGN_Q8G64, HGN_Q8G32 = 0, 1, 5, 7, 8
+HGN_F16, HGN_I4R = 2, 23  # hgn v2: f16 sign-scale planes, rotated routed experts
 GGML_F32, GGML_BF16, GGML_Q4_K = 0, 30, 12
 _GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24),
                20: (32, 18), 23: (256, 136)}
@@ -85,12 +86,20 @@ def write_gguf(path, tensors, kv=None, align=32):
 
 
 def hgn_layer_tensors(l, hl):
-    """The MoE tensors of layer l of a tests.helpers.HostLayer-like object (fmt q4cp) as .hgn records."""
+    """The MoE tensors of layer l of a tests.helpers.HostLayer-like object (fmt q4cp, or i4r = hgn v2 rotated experts
+    with their four f16 planes under the reference's names, tools/v2repro/v2_encode.py:84-90) as .hgn records."""
     d, mid, E = hl.d, hl.mid, hl.E
     rdt = HGN_F32 if hl.router.dtype == np.float32 else HGN_BF16
+    edt = HGN_I4R if getattr(hl, "fmt", "q4cp") == "i4r" else HGN_Q4CP
     t = [(f"layers.{l}.mlp.gate.weight", rdt, [E, d], hl.router),
-         (f"layers.{l}.mlp.experts.gate_up_proj.weight", HGN_Q4CP, [E, 2 * mid, d], hl.gate_up),
-         (f"layers.{l}.mlp.experts.down_proj.weight", HGN_Q4CP, [E, d, mid], hl.down)]
+         (f"layers.{l}.mlp.experts.gate_up_proj.weight", edt, [E, 2 * mid, d], hl.gate_up),
+         (f"layers.{l}.mlp.experts.down_proj.weight", edt, [E, d, mid], hl.down)]
+    if edt == HGN_I4R:
+        su, svh_gu, suh_dn, svh_dn = (np.asarray(p, np.float32).astype(np.float16) for p in hl.planes)
+        t += [(f"layers.{l}.mlp.experts.su", HGN_F16, [d], su),
+              (f"layers.{l}.mlp.experts.gate_up_proj.svh", HGN_F16, [2 * mid], svh_gu),
+              (f"layers.{l}.mlp.experts.down_proj.suh", HGN_F16, [mid], suh_dn),
+              (f"layers.{l}.mlp.experts.down_proj.svh", HGN_F16, [d], svh_dn)]
     if hl.shared is not None:
         sdt = {None: HGN_Q4CP, "bf16": HGN_BF16, "f32": HGN_F32, "q8g64": HGN_Q8G64, "q8g32": HGN_Q8G32}[getattr(hl, "shared_dense", None)]
         t += [(f"layers.{l}.mlp.shared_expert.gate_proj.weight", sdt, [mid, d], hl.shared[0]),

@@ -39,6 +39,26 @@ def q4cp_blob(g, rows, cols, scale_std=0.01, codebook=None):
     return blob
 
 
+def i4r_blob(g, rows, cols, scale_std=0.01):
+    """uint8 tensor [rows*cols/2 codes][rows x cols/128 fp16 scales] (hgn v2 dtype 23): uniform codes, N*std scales
+    of either sign."""
+    nb = rows * cols // 2
+    blob = torch.empty(nb + rows * (cols // 128) * 2, dtype=torch.uint8, device="cuda")
+    step = 1 << 28
+    for i in range(0, nb, step):
+        n = min(step, nb - i)
+        blob[i:i + n] = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    sc = (torch.randn((rows * (cols // 128),), device="cuda", generator=g) * scale_std).to(torch.float16)
+    blob[nb:] = sc.view(torch.uint8)
+    return blob
+
+
+def v2_plane(g, n):
+    """A sign-scale plane of an hgn v2 tensor: f16-representable values of magnitude 0.5 .. 1.5, random signs, as f32."""
+    v = (0.5 + torch.rand((n,), device="cuda", generator=g)) * (torch.randint(0, 2, (n,), device="cuda", generator=g) * 2 - 1)
+    return v.to(torch.float16).to(torch.float32)
+
+
 def q4k_rows(g, rows, cols, scale_std=0.01):
     """uint8 tensor of rows*cols/256 Q4_K super-blocks (144 B): d,dmin fp16 |N|*std; 6-bit sub-scales/mins
     uniform [0,63]; codes uniform."""
@@ -97,6 +117,7 @@ def gg_rows(g, t, rows, cols, scale_std=0.01):
 class DeviceLayer:
     """One layer's weights in HBM + registration into a capi.Moe context.
     fmt "q4k": raw GGUF blocks, gg_types = ggml types of (gate/up, down, shared expert).
+    fmt "i4r": hgn v2 rotated routed experts with their four planes; the shared expert as in a q4cp layer.
     codebook (q4cp): "zp8" = the zero-point-8 grid cb[n] = n - 8; "universal" = the fixed non-uniform table of the
     reference's converter (scales 8.4 times larger, so that the weights keep their size)."""
 
@@ -113,6 +134,11 @@ class DeviceLayer:
             self.gate_up = q4cp_blob(g, E * 2 * mid, d, sd, cb)
             self.down = q4cp_blob(g, E * d, mid, sd, cb)
             self.sh = [q4cp_blob(g, mid, d, sd, cb), q4cp_blob(g, mid, d, sd, cb), q4cp_blob(g, d, mid, sd, cb)]
+        elif fmt == "i4r":
+            self.gate_up = i4r_blob(g, E * 2 * mid, d)
+            self.down = i4r_blob(g, E * d, mid)
+            self.planes = [v2_plane(g, d), v2_plane(g, 2 * mid), v2_plane(g, mid), v2_plane(g, d)]
+            self.sh = [q4cp_blob(g, mid, d), q4cp_blob(g, mid, d), q4cp_blob(g, d, mid)]
         else:
             self.gate = gg_rows(g, self.tgu, E * mid, d)
             self.up = gg_rows(g, self.tgu, E * mid, d)
@@ -123,12 +149,16 @@ class DeviceLayer:
         d, mid = self.d, self.mid
         if self.fmt == "q4cp":
             return 2 * mid * (d // 2 + S.q4cp_scale_stride(d)) + d * (mid // 2 + S.q4cp_scale_stride(mid))
+        if self.fmt == "i4r":
+            return 2 * mid * (d // 2 + d // 128 * 2) + d * (mid // 2 + mid // 128 * 2)
         return 2 * mid * gg_row_bytes(self.tgu, d) + d * gg_row_bytes(self.tdn, mid)
 
     def shared_bytes(self):
         d, mid = self.d, self.mid
         if self.fmt == "q4cp":
             return self.expert_bytes()
+        if self.fmt == "i4r":
+            return 2 * mid * (d // 2 + S.q4cp_scale_stride(d)) + d * (mid // 2 + S.q4cp_scale_stride(mid))
         return 2 * mid * gg_row_bytes(self.tsh, d) + d * gg_row_bytes(self.tsh, mid)
 
     def register(self, m, layer=0):
@@ -137,6 +167,10 @@ class DeviceLayer:
         if self.fmt == "q4cp":
             m.set_experts_q4cp(layer, capi.wview(self.gate_up, capi.Q4CP, E * 2 * mid, d),
                                capi.wview(self.down, capi.Q4CP, E * d, mid))
+            wt, gt = capi.Q4CP, 0
+        elif self.fmt == "i4r":
+            m.set_experts_i4r(layer, capi.wview(self.gate_up, capi.I4R, E * 2 * mid, d),
+                              capi.wview(self.down, capi.I4R, E * d, mid), *self.planes)
             wt, gt = capi.Q4CP, 0
         else:
             m.set_experts_gguf(layer, self.gate, self.up, self.down, self.tgu, self.tdn)

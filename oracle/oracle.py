@@ -402,17 +402,18 @@ def layer_from_device(dl):
     """An oracle Layer over the very bytes of a synthetic device layer (an object with the attributes of
     gfx1151_engine_amd.workloads.DeviceLayer), copied to the host.  Checker side only."""
     d, mid, E, k = dl.d, dl.mid, dl.E, dl.k
-    wt = Q4CP if dl.fmt == "q4cp" else Q4K
+    wt = Q4CP if dl.fmt == "q4cp" else I4R if dl.fmt == "i4r" else Q4K
     tgu, tdn, tsh = (getattr(dl, a, Q4K) for a in ("tgu", "tdn", "tsh"))  # ggml types of a raw-block layer
-    st = wt if dl.fmt == "q4cp" else tsh
+    st = Q4CP if dl.fmt in ("q4cp", "i4r") else tsh
     h = lambda t: t.cpu().numpy()
     sh = [Mat(st, h(dl.sh[0]), mid, d), Mat(st, h(dl.sh[1]), mid, d), Mat(st, h(dl.sh[2]), d, mid),
           Mat(F32, h(dl.sh_sg), 1, d)]
     router = Mat(F32, h(dl.router), E, d)
     bias = h(dl.bias) if dl.bias is not None else None
-    if dl.fmt == "q4cp":
+    if dl.fmt in ("q4cp", "i4r"):
         return Layer(d, mid, E, k, router, Mat(wt, h(dl.down), E * d, mid),
-                     gate_up=Mat(wt, h(dl.gate_up), E * 2 * mid, d), shared=sh, router_bias=bias)
+                     gate_up=Mat(wt, h(dl.gate_up), E * 2 * mid, d), shared=sh, router_bias=bias,
+                     rot=[h(p) for p in dl.planes] if dl.fmt == "i4r" else None)
     return Layer(d, mid, E, k, router, Mat(tdn, h(dl.down), E * d, mid),
                  gate=Mat(tgu, h(dl.gate), E * mid, d), up=Mat(tgu, h(dl.up), E * mid, d),
                  shared=sh, router_bias=bias)

@@ -437,6 +437,56 @@ def test_mtp_layer_from_a_file(tmp_path):
     w1.free()
 
 
+def test_hgn_v2_records_match_reference_reader(tmp_path):
+    """An hgn v2 layer's records (dtype 23 expert tensors, dtype 2 planes under the reference's names): the library's
+    parser and the reference's own Checkpoint reader agree on dtype, dims and bytes."""
+    rng = np.random.default_rng(31)
+    hl = HostLayer(rng, D, MID, E, K, fmt="i4r")
+    p, ts = _hgn(tmp_path, [hl], first=0)
+    f = capi.ModelFile(p)
+    names = {t[0] for t in ts}
+    assert {"layers.0.mlp.experts.su", "layers.0.mlp.experts.gate_up_proj.svh", "layers.0.mlp.experts.down_proj.suh",
+            "layers.0.mlp.experts.down_proj.svh"} <= names
+    for name, dt, dims, data in ts:
+        raw = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+        for got in [f.find(name)] + ([O.ref_hgn_tensor(p, name)] if HAVE_REF else []):
+            assert got[0] == dt and got[1][:len(dims)] == tuple(dims) and np.array_equal(got[2], raw), name
+    cfg = f.config(0)
+    assert (cfg.d, cfg.mid, cfg.experts, cfg.layers) == (D, MID, E, 1)
+    f.close()
+
+
+@pytest.mark.gpu
+def test_hgn_v2_layer_loaded_from_a_file(tmp_path):
+    """moe_load_layers on an hgn v2 layer: i4r expert tensors copied as they are, the four f16 planes uploaded as f32
+    (src/gpu/parts/30_host_util.inc:818-861); decode, small batch and grouped-GEMM batch against the oracle.  A
+    file without one of the planes is refused."""
+    import torch
+    rng = np.random.default_rng(32)
+    hl = HostLayer(rng, D, MID, E, K, fmt="i4r")
+    p, ts = _hgn(tmp_path, [hl], first=0)
+    f = capi.ModelFile(p)
+    m = capi.Moe(D, MID, E, K, layers=1, max_tokens=80)
+    w = f.load_layers(m, 0, 0, 1)
+    f.close()
+    for T in (1, 9, 80):
+        x = _x(T, seed=T)
+        want, io, _ = O.moe_layer(hl.oracle_layer(), x)
+        y = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :K] == io[:, :K]).all()
+        assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max(), T
+    del m
+    w.free()
+    p2 = tmp_path / "noplane.hgn"
+    files.write_hgn(p2, [t for t in ts if not t[0].endswith("down_proj.suh")])
+    f = capi.ModelFile(p2)
+    m = capi.Moe(D, MID, E, K, layers=1, max_tokens=8)
+    wh = C.c_void_p()
+    assert capi.lib().moe_load_layers(m.h, f.h, 0, 0, 1, C.byref(wh), capi.stream()) == -3
+    f.close()
+
+
 @pytest.mark.gpu
 def test_load_rejects_types_outside_the_path(tmp_path):
     # a GGUF whose experts are Q6_K: moe_load_layers reports unsupported and leaves no layer registered
