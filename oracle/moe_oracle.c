@@ -29,7 +29,9 @@
  * against the reference's Checkpoint::dequant, but the reference's CPU matvec has no
  * branch for that dtype (src/ref.cpp:68-109 throws), so the layer form used here -- the
  * dequantised row in the generic fp64 dot product -- is confirmed by no run of the
- * reference.  Everything else is pinned.
+ * reference.  Everything else is pinned; the hgn v2 functions (i4r rows, the 128-block
+ * rotation, the rotated layer) by closed forms and by a float64 evaluation of the same
+ * layer on the un-rotated weights, because the reference has no CPU code for that format.
  *
  * One deliberate addition: std::partial_sort in src/ref.cpp:587 leaves the
  * order of equal probabilities unspecified.  The oracle fixes it to "lowest
