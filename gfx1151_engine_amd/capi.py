@@ -206,6 +206,8 @@ OPT_FUSED_COMBINE = 3
 OPT_SHARED_ASIDE = 4
 OPT_TIMING_SKIP_STAGE = 5
 OPT_ROUTER_CANDIDATES = 6
+OPT_UNIQUE_GGUF = 7
+OPT_GU_TOPK_MAX_TOKENS = 8
 
 
 def lut_q4cp_view(blob, rows, cols, e_rows, up_off):

@@ -76,7 +76,9 @@ struct moe_ctx {
   __half* pairs16 = nullptr;  // [(k+1)T][d]
   float* pairs32 = nullptr;   // [(k+1)min(T,small_max)][d] unweighted pair rows of the unique-expert small-batch path
   bool fused_combine = false; // batch path: the down GEMM adds its weighted rows into y with f32 atomics (no pairs buffer, no reduce launch)
-  int uq_min = 12;            // > 0: small batches of at least this many tokens read every distinct expert once
+  int uq_min = 24;            // > 0: small batches of at least this many tokens read every distinct expert once
+  int gu_topk_max = 4;        // batches up to this size run the softmax / top-k inside the gate/up launch (else in the router's launches)
+  bool uq_gguf = false;       // the same for GGUF layers (off: their per-token kernels measure faster unless most tokens share experts)
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
   bool profile = false;
   int skip_stage = 0;      // MOE_OPT_TIMING_SKIP_STAGE: 1 + the stage whose launches are left out (0 = none)
@@ -448,6 +450,11 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
     case MOE_OPT_FUSED_COMBINE: c->fused_combine = value != 0; return MOE_OK;
     case MOE_OPT_SHARED_ASIDE: c->shared_aside = value != 0; return MOE_OK;
     case MOE_OPT_ROUTER_CANDIDATES: c->router_cand = value != 0; return MOE_OK;
+    case MOE_OPT_UNIQUE_GGUF: c->uq_gguf = value != 0; return MOE_OK;
+    case MOE_OPT_GU_TOPK_MAX_TOKENS:
+      if (value < 0) return MOE_E_INVALID;
+      c->gu_topk_max = value;
+      return MOE_OK;
     case MOE_OPT_TIMING_SKIP_STAGE:
       if (value < 0 || value > MOE_PROF_STAGES) return MOE_E_INVALID;
       c->skip_stage = value;
@@ -537,9 +544,14 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
                          moe_decgg_supported(L.gg.tgu, L.gg.tdn, L.sh_gguf_type, sh, g.d, g.mid, g.topk, g.experts) &&
                          (!sh || L.sh_gguf_type != 0);
   const bool use_uq = use_int && c->uq_min > 0 && P >= c->uq_min && moe_dec_uq_supported(g.d);
+  // the same for GGUF layers on the integer-dot kernels (any mix of their four block types)
+  const bool use_uq_gg = (use_int4k || use_intgg) && c->uq_gguf && c->uq_min > 0 && P >= c->uq_min && moe_decgg_uq_supported(g.d) &&
+                         moe_decgg_supported(L.gg.tgu, L.gg.tdn, L.sh_gguf_type, sh, g.d, g.mid, g.topk, g.experts) &&
+                         (!sh || L.sh_gguf_type != 0);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
-  const bool gu_topk = ((use_int && !use_uq) || use_int4k || use_intgg || use_lut) && moe_dec_gu_topk_supported(g.experts, g.topk);
+  const bool gu_topk = ((((use_int && !use_uq) || ((use_int4k || use_intgg) && !use_uq_gg)) && P <= c->gu_topk_max) || use_lut) &&
+                       moe_dec_gu_topk_supported(g.experts, g.topk);
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
          int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
@@ -621,11 +633,44 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
     });
   }
   if (sh && L.sh_gguf_type == 0) return MOE_E_UNSUPPORTED;
+  if (use_uq_gg) {
+    // verify-size batches of a GGUF layer: every distinct expert's rows read once (reference: the _uq kernels,
+    // 26_kernels_moe_gguf.inc:758-886)
+    const int cap = moe_decgg_uq_tile_cap();
+    const int sh_first = sh ? P * g.topk : -1;
+    const int max_tiles = P * g.topk + (sh ? (P + cap - 1) / cap : 0);
+    if ((rc = stage(MOE_PROF_ROUTE, [&]() -> int {
+           if (moe_route_small_supported(P, g.topk, g.experts))
+             return moe_launch_route_small(c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk, g.experts,
+                                           g.id_stride, c->tiles, c->ntiles, cap, sh_first, st);
+           const int e = moe_routing_run(c->routing, c->ids, c->ws, c->tokidx, c->pw, c->eoff, c->pairids, P, g.topk,
+                                         g.experts, g.id_stride, st);
+           return e ? e : moe_launch_tiles_shared(c->eoff, c->tiles, c->ntiles, g.experts, cap, P, sh_first, c->tokidx, st);
+         })))
+      return rc;
+    if ((rc = stage(MOE_PROF_UP, [&]() -> int {
+           return moe_launch_decgg_gu_uq(L.gg.tgu, L.sh_gguf_type, L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta, c->tiles,
+                                         c->ntiles, max_tiles, c->tokidx, g.experts, g.d, g.mid, c->hplanes, c->hmeta, st);
+         })))
+      return rc;
+    if ((rc = stage(MOE_PROF_DOWN, [&]() -> int {
+           return moe_launch_decgg_dn_uq(L.gg.tdn, L.sh_gguf_type, L.gg.down, rd, c->hplanes, c->hmeta, c->tiles, c->ntiles,
+                                         max_tiles, g.experts, g.d, g.mid, c->pairs32, st);
+         })))
+      return rc;
+    return stage(MOE_PROF_REDUCE, [&]() -> int {
+      return moe_launch_reduce(c->pairs32, false, c->pairids, c->pw, nullptr, sh ? c->sh_logit : nullptr, sh_first, y, P,
+                               g.d, g.topk, moe_hscale{nullptr, 0.f, 0.f}, st, nullptr);
+    });
+  }
   if (use_intgg) {
     if ((rc = stage(MOE_PROF_UP, [&]() -> int {
-           return moe_launch_decgg_gu_topk(L.gg.tgu, L.sh_gguf_type, L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta,
-                                           c->logits, g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
-                                           c->hplanes, c->hmeta, st);
+           return gu_topk ? moe_launch_decgg_gu_topk(L.gg.tgu, L.sh_gguf_type, L.gg.gate, L.gg.up, rg, ru, c->xplanes,
+                                                     c->xmeta, c->logits, g.experts, c->ids, c->ws, g.id_stride, g.topk,
+                                                     P, g.d, g.mid, c->hplanes, c->hmeta, st)
+                          : moe_launch_decgg_gu(L.gg.tgu, L.sh_gguf_type, L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta,
+                                                c->ids, g.experts, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta,
+                                                st);
          })))
       return rc;
     return stage(MOE_PROF_DOWN, [&]() -> int {
@@ -689,11 +734,14 @@ static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, floa
   const bool sh = L.has_shared && !L.sh_dense;  // a q4cp shared expert rides in these kernels as one more slot
   if (sh && (L.sh_gguf_type != 0 || !L.shared_affine)) return MOE_E_UNSUPPORTED;
   const int nslots_d = g.topk + (sh ? 1 : 0);
+  const bool gu_topk = P <= c->gu_topk_max;
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
-         const int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
-                                               c->sh_logit, sh ? c->xplanes : nullptr, c->xmeta, false, nullptr, c->ids,
-                                               c->ws, g.topk, g.id_stride, &fused, st, c->kpart, c->ktickets);
+         int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
+                                         c->sh_logit, sh ? c->xplanes : nullptr, c->xmeta, false,
+                                         gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk, g.id_stride, &fused, st,
+                                         c->kpart, c->ktickets);
+         if (!e && !fused && !gu_topk) e = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
          return e ? e : moe_launch_v2_rot(x, (uint64_t)g.d, P, g.d, L.v2_su, nullptr, 2, nullptr, 0, nullptr, 0,
                                           c->v2_xplanes, c->v2_xmeta, st);
        })))
@@ -701,9 +749,11 @@ static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, floa
   const moe_wview *shg = sh ? &L.sh_gate : nullptr, *shu = sh ? &L.sh_up : nullptr, *shd = sh ? &L.sh_down : nullptr;
   if ((rc = stage(MOE_PROF_UP, [&]() -> int {
          const moe_dec_v2 v2{c->v2_zraw, c->v2_xplanes, c->v2_xmeta};
-         const int e = moe_launch_dec_gu_topk(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->logits, g.experts, c->ids,
-                                              c->ws, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st,
-                                              &v2);
+         const int e = gu_topk ? moe_launch_dec_gu_topk(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->logits, g.experts,
+                                                        c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes,
+                                                        c->hmeta, nullptr, st, &v2)
+                               : moe_launch_dec_gu(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->ids, g.id_stride, g.topk,
+                                                   P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st, &v2);
          return e ? e : moe_launch_i4r_mid(c->v2_zraw, false, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu,
                                            L.v2_suh_dn, 2, nullptr, 0, g.topk, nslots_d, c->hplanes, c->hmeta, st);
        })))

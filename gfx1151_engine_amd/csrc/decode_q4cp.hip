@@ -570,11 +570,18 @@ int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* p
 int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
-                      hipStream_t st) {
+                      hipStream_t st, const moe_dec_v2* v2) {
   GuArgs2 A{};
   A.gu = decw(gu);
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
+  if (v2) {
+    if (!v2->zraw || !v2->xplanes_rot || !v2->xmeta_rot) return MOE_E_INVALID;
+    A.zraw = v2->zraw;
+    A.xplanes_rot = v2->xplanes_rot;
+    A.xmeta_rot = v2->xmeta_rot;
+  }
+  if (!A.gu.cb) return MOE_E_STATE;
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
   k_dec_gu<false, 0, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
                                                   nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr);

@@ -469,15 +469,15 @@ __global__ void __launch_bounds__(512, 4) k_decgg_gu(GuGgArgs A, const uint32_t*
                                                      int mid, uint32_t* __restrict__ hplanes,
                                                      float2* __restrict__ hmeta, const float* __restrict__ logits,
                                                      int n_experts, int* __restrict__ ids_out,
-                                                     float* __restrict__ ws_out) {
+                                                     float* __restrict__ ws_out, const int* __restrict__ ids_in) {
   __shared__ float gs[G4_ROWS], us[G4_ROWS];
   __shared__ uint32_t pk[QV_GROUP_DW];
   __shared__ int sel_ids[64];
   __shared__ float sel_ws[64];
-  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y - 1;
-  if (s == nslots) {  // the extra grid row: exact softmax / top-k for the down launch
+  const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y - (NPL > 0 ? 1 : 0);
+  if (NPL > 0 && s == nslots) {  // the extra grid row: exact softmax / top-k for the down launch
     if (blockIdx.x == 0) {
-      topk_block<NPL, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
       __syncthreads();
       if ((int)threadIdx.x < kpt) {
         ids_out[(size_t)tok * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
@@ -491,12 +491,16 @@ __global__ void __launch_bounds__(512, 4) k_decgg_gu(GuGgArgs A, const uint32_t*
   const bool shared = s >= kpt;
   int e = 0;
   if (!shared) {
-    const float* lg = logits + (size_t)tok * n_experts;
-    if (!topk_ids_by_logit<NPL>(lg, sel_ids, n_experts, kpt)) {
-      topk_block<NPL, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
-      __syncthreads();
+    if (NPL > 0) {
+      const float* lg = logits + (size_t)tok * n_experts;
+      if (!topk_ids_by_logit<NPL ? NPL : 8>(lg, sel_ids, n_experts, kpt)) {
+        topk_block<NPL ? NPL : 8, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
+        __syncthreads();
+      }
+      e = sel_ids[s];
+    } else {
+      e = ids_in[(size_t)tok * id_stride + s];  // (NPL == 0: the ids come from the router's launches)
     }
-    e = sel_ids[s];
   }
   const int t = shared ? A.tsh : A.tgu;
   const uint64_t rb = ggu_row_bytes(t, (uint64_t)d);
@@ -619,6 +623,165 @@ __global__ void __launch_bounds__(320) k_decgg_dn(DnGgArgs A, const uint32_t* __
   }
 }
 
+// ---- distinct experts of a small batch (verify-size batches: tokens share experts) ----
+// The expert-sorted pair lists of the routing permutation, cut into tiles of at most GGQ_PAIRS pairs of one expert
+// (the shared expert: expert id >= n_experts, over all tokens): a block fetches its weight rows once and walks the
+// tile's pairs, so every distinct expert's bytes are read once per batch instead of once per token
+// (reference: the _uq kernels, src/gpu/parts/26_kernels_moe_gguf.inc:758-886).
+constexpr int GGQ_PAIRS = 4;  // pairs per tile (the tile lists are built with this cap)
+// rows fetched together: two (with a pair's activation planes next to them the kernels stay under 128 registers,
+// two blocks per CU; four rows spill)
+template <int T>
+__device__ __host__ constexpr int ggq_batch() { return T == MOE_GGML_Q8_0 ? 4 : 8; }
+template <int T>
+__device__ __host__ constexpr int ggq_dn_batch() { return T == MOE_GGML_Q8_0 ? 2 : 4; }
+constexpr int GGQ_DR = 4, GGQ_DROWS = 16 * GGQ_DR;  // down: output rows per row of 16 lanes, per block
+
+// eight rows of one wave in batches of GGQ_RB, each batch against every pair of the tile; gs / us: [pair][32] rows of
+// the block in LDS, already offset to this wave's four
+template <int T>
+__device__ __forceinline__ void ggq_gu_rows(const uint8_t* gbase, const uint8_t* ubase, int r0, uint64_t rb, int ul, int jj,
+                                            float mlive, const uint32_t* __restrict__ xplanes,
+                                            const float2* __restrict__ xmeta, const int (&toks)[GGQ_PAIRS], int npairs,
+                                            int U, bool writer, float* gs, float* us) {
+  constexpr int RB = ggq_batch<T>();
+#pragma unroll
+  for (int h = 0; h < 8; h += RB) {
+    GgU<T> u[RB];
+#pragma unroll
+    for (int i = 0; i < RB; i++)
+      ggu_fetch<T>(((i + h) < 4 ? gbase : ubase) + (uint64_t)(r0 + ((i + h) & 3)) * rb, ul, u[i]);
+    __builtin_amdgcn_sched_barrier(0);  // every load of the batch is issued before the first dot product
+#pragma unroll 1
+    for (int pi = 0; pi < npairs; pi++) {
+      XU x;
+      load_xu(x, xplanes, xmeta, ((size_t)toks[pi] * U + ul) * 2);
+#pragma unroll
+      for (int i = 0; i < RB; i++) {
+        const float v = sum64(ggu_dot<T>(u[i], jj, x) * mlive);
+        if (writer) {
+          if (i + h < 4) gs[pi * G4_ROWS + i + h] = v;
+          else us[pi * G4_ROWS + i + h - 4] = v;
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);  // the next batch's loads stay behind this batch's pairs
+  }
+}
+
+// GGQ_DR output rows of one row of 16 lanes against every pair of the tile; out: pairs + first pair's row + r0
+template <int T>
+__device__ __forceinline__ void ggq_dn_rows(const uint8_t* base, uint64_t rb, int ul, int jj, float mlive,
+                                            const uint32_t* __restrict__ hplanes, const float2* __restrict__ hmeta,
+                                            size_t first, int npairs, int U, bool writer, float* out, int d);
+
+// gate/up: grid (mid/32, tiles), block 512 (wave w: gate rows 4w..4w+3 and the matching up rows of the block's 32);
+// hid planes go out by pair position, [pair][mid/32 groups]
+__global__ void __launch_bounds__(512, 2) k_decgg_gu_uq(GuGgArgs A, const uint32_t* __restrict__ xplanes,
+                                                        const float2* __restrict__ xmeta,
+                                                        const moe_tile* __restrict__ tiles,
+                                                        const int* __restrict__ ntiles, const int* __restrict__ tokidx,
+                                                        int n_experts, int d, int mid, uint32_t* __restrict__ hplanes,
+                                                        float2* __restrict__ hmeta) {
+  __shared__ float gs[GGQ_PAIRS][G4_ROWS], us[GGQ_PAIRS][G4_ROWS];
+  __shared__ uint32_t pk[GGQ_PAIRS][QV_GROUP_DW];
+  if ((int)blockIdx.y >= ntiles[0]) return;
+  const moe_tile tile = tiles[blockIdx.y];
+  const bool shared = tile.expert >= n_experts;
+  const int npairs = tile.count < GGQ_PAIRS ? tile.count : GGQ_PAIRS;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int U = d / 64;
+  const int t = shared ? A.tsh : A.tgu;
+  const uint64_t rb = ggu_row_bytes(t, (uint64_t)d);
+  const uint8_t* gbase = shared ? A.sh_gate : A.gate + (uint64_t)tile.expert * mid * rb;
+  const uint8_t* ubase = shared ? A.sh_up : A.up + (uint64_t)tile.expert * mid * rb;
+  const int r0 = blockIdx.x * G4_ROWS + 4 * wv;
+  const bool live = lane < U;
+  const int ul = live ? lane : (lane & 3);
+  const float mlive = live ? 1.f : 0.f;
+  const int jj = ul & 3;
+  int toks[GGQ_PAIRS];
+#pragma unroll
+  for (int pi = 0; pi < GGQ_PAIRS; pi++) toks[pi] = tokidx[tile.first + (pi < npairs ? pi : 0)];
+  GGU_SWITCH(t, ggq_gu_rows<T>(gbase, ubase, r0, rb, ul, jj, mlive, xplanes, xmeta, toks, npairs, U, lane == 0,
+                               &gs[0][4 * wv], &us[0][4 * wv]));
+  __syncthreads();
+  if (wv < npairs) {  // wave pi: SwiGLU on pair pi's 32 rows = one activation group of the down projection; quantise it
+    const int j = lane & 31;
+    const float g = gs[wv][j], u = us[wv][j];
+    const float hv = g / (1.f + expf(-g)) * u;
+    float m = dpp_max_row(fabsf(hv));
+    m = rows_half_max(m);
+    const float inv = m > 0.f ? QV_XMAX / m : 0.f;
+    const float q = m * (1.f / QV_XMAX);
+    const int X = (int)rintf(hv * inv);
+    int p0, p1;
+    qv_digits(X, p0, p1);
+    float sx = dpp_add_row((float)X);
+    sx = rows_half_add(sx);
+    if (lane < QV_GROUP_DW) pk[wv][lane] = 0;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_wave_barrier();
+    if (lane < 32) {
+      const int dw = j >> 2, sh = 8 * (j & 3);
+      atomicOr(&pk[wv][dw], (uint32_t)(p0 & 0xff) << sh);
+      atomicOr(&pk[wv][8 + dw], (uint32_t)(p1 & 0xff) << sh);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_wave_barrier();
+    const size_t gi = (size_t)(tile.first + wv) * (mid / 32) + blockIdx.x;
+    if (lane < QV_GROUP_DW) hplanes[gi * QV_GROUP_DW + lane] = pk[wv][lane];
+    if (lane == 0) hmeta[gi] = make_float2(q, q * sx);
+  }
+}
+
+// down: grid (d/GGQ_DROWS, tiles), block 256 = 16 rows of 16 lanes, each with GGQ_DR output rows; the unweighted row
+// results go to pairs[pair][row] (f32) for the weighted combine that follows
+template <int T>
+__device__ __forceinline__ void ggq_dn_rows(const uint8_t* base, uint64_t rb, int ul, int jj, float mlive,
+                                            const uint32_t* __restrict__ hplanes, const float2* __restrict__ hmeta,
+                                            size_t first, int npairs, int U, bool writer, float* out, int d) {
+  constexpr int RB = ggq_dn_batch<T>();
+#pragma unroll
+  for (int h = 0; h < GGQ_DR; h += RB) {
+    GgU<T> u[RB];
+#pragma unroll
+    for (int r = 0; r < RB; r++) ggu_fetch<T>(base + (uint64_t)(h + r) * rb, ul, u[r]);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int pi = 0; pi < npairs; pi++) {
+      XU x;
+      load_xu(x, hplanes, hmeta, ((first + pi) * U + ul) * 2);
+#pragma unroll
+      for (int r = 0; r < RB; r++) {
+        const float v = dpp_add_row(ggu_dot<T>(u[r], jj, x) * mlive);
+        if (writer) out[(size_t)pi * d + h + r] = v;
+      }
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256) k_decgg_dn_uq(DnGgArgs A, const uint32_t* __restrict__ hplanes,
+                                                     const float2* __restrict__ hmeta,
+                                                     const moe_tile* __restrict__ tiles, const int* __restrict__ ntiles,
+                                                     int n_experts, int d, int mid, float* __restrict__ pairs) {
+  if ((int)blockIdx.y >= ntiles[0]) return;
+  const moe_tile tile = tiles[blockIdx.y];
+  const bool shared = tile.expert >= n_experts;
+  const int npairs = tile.count < GGQ_PAIRS ? tile.count : GGQ_PAIRS;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int U = mid / 64, u_raw = lane & 15;
+  const bool live = u_raw < U;
+  const int ul = live ? u_raw : (u_raw & 3);
+  const float mlive = live ? 1.f : 0.f;
+  const int jj = ul & 3;
+  const int t = shared ? A.tsh : A.tdn;
+  const uint64_t rb = ggu_row_bytes(t, (uint64_t)mid);
+  const int r0 = blockIdx.x * GGQ_DROWS + (4 * wv + (lane >> 4)) * GGQ_DR;
+  const uint8_t* base = (shared ? A.sh_down : A.down + (uint64_t)tile.expert * d * rb) + (uint64_t)r0 * rb;
+  GGU_SWITCH(t, ggq_dn_rows<T>(base, rb, ul, jj, mlive, hplanes, hmeta, (size_t)tile.first, npairs, U, u_raw == 0,
+                               pairs + (size_t)tile.first * d + r0, d));
+}
+
 }  // namespace
 
 bool moe_dec4k_supported(int d, int mid, int nslots) {
@@ -700,9 +863,26 @@ int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_
   GuGgArgs A{gate, up, sh_gate, sh_up, tgu, tsh};
   dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);
   if (n_experts <= 512)
-    k_decgg_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws);
+    k_decgg_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws, nullptr);
   else
-    k_decgg_gu<16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws);
+    k_decgg_gu<16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws, nullptr);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// the same with the ids already there (the router's launches made them)
+int moe_launch_decgg_gu(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
+                        const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const int* ids, int n_experts,
+                        int id_stride, int kpt, int P, int d, int mid, uint32_t* hplanes, float2* hmeta, hipStream_t st) {
+  if (!gate || !up || !xplanes || !xmeta || !ids || !hplanes || !hmeta || (!sh_gate != !sh_up)) return MOE_E_INVALID;
+  if (!moe_decgg_supported(tgu, tgu, tsh, sh_gate != nullptr, d, mid, kpt, n_experts)) return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(gate, ggu_align(tgu)) || !moe_aligned(up, ggu_align(tgu)) ||
+      (sh_gate && (!moe_aligned(sh_gate, ggu_align(tsh)) || !moe_aligned(sh_up, ggu_align(tsh)))))
+    return MOE_E_INVALID;
+  GuGgArgs A{gate, up, sh_gate, sh_up, tgu, tsh};
+  dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0), P);
+  k_decgg_gu<0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, nullptr, n_experts, nullptr,
+                                      nullptr, ids);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -716,6 +896,44 @@ int moe_launch_decgg_dn(int tdn, int tsh, const uint8_t* down, const uint8_t* sh
   dim3 grid(d / D4_ROWS, P);
   k_decgg_dn<<<grid, 64 * ((kpt + 3) / 4 + (sh_down ? 1 : 0)), 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid,
                                                                         out, out_stride);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// Distinct-expert variants: tiles (at most 4 pairs each; the shared expert as expert id n_experts) / ntiles / tokidx
+// from the routing permutation; hplanes / hmeta and pairs are indexed by pair position.
+bool moe_decgg_uq_supported(int d) { return d % GGQ_DROWS == 0; }
+int moe_decgg_uq_tile_cap() { return GGQ_PAIRS; }
+
+int moe_launch_decgg_gu_uq(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
+                           const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const moe_tile* tiles,
+                           const int* ntiles, int max_tiles, const int* tokidx, int n_experts, int d, int mid,
+                           uint32_t* hplanes, float2* hmeta, hipStream_t st) {
+  if (!gate || !up || !xplanes || !xmeta || !tiles || !ntiles || !tokidx || !hplanes || !hmeta || (!sh_gate != !sh_up))
+    return MOE_E_INVALID;
+  if (!moe_decgg_supported(tgu, tgu, tsh, sh_gate != nullptr, d, mid, 1, n_experts < 1024 ? n_experts : 1024))
+    return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(gate, ggu_align(tgu)) || !moe_aligned(up, ggu_align(tgu)) ||
+      (sh_gate && (!moe_aligned(sh_gate, ggu_align(tsh)) || !moe_aligned(sh_up, ggu_align(tsh)))))
+    return MOE_E_INVALID;
+  if (max_tiles <= 0) return MOE_OK;
+  GuGgArgs A{gate, up, sh_gate, sh_up, tgu, tsh};
+  k_decgg_gu_uq<<<dim3(mid / G4_ROWS, max_tiles), 512, 0, st>>>(A, xplanes, xmeta, tiles, ntiles, tokidx, n_experts, d, mid,
+                                                                hplanes, hmeta);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_launch_decgg_dn_uq(int tdn, int tsh, const uint8_t* down, const uint8_t* sh_down, const uint32_t* hplanes,
+                           const float2* hmeta, const moe_tile* tiles, const int* ntiles, int max_tiles, int n_experts,
+                           int d, int mid, float* pairs, hipStream_t st) {
+  if (!down || !hplanes || !hmeta || !tiles || !ntiles || !pairs) return MOE_E_INVALID;
+  if (!moe_decgg_uq_supported(d) || mid % 256 || mid / 64 > 16) return MOE_E_UNSUPPORTED;
+  if (!moe_aligned(down, ggu_align(tdn)) || (sh_down && !moe_aligned(sh_down, ggu_align(tsh))) || !moe_aligned(pairs, 16))
+    return MOE_E_INVALID;
+  if (max_tiles <= 0) return MOE_OK;
+  DnGgArgs A{down, sh_down, nullptr, tdn, tsh};
+  k_decgg_dn_uq<<<dim3(d / GGQ_DROWS, max_tiles), 256, 0, st>>>(A, hplanes, hmeta, tiles, ntiles, n_experts, d, mid, pairs);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

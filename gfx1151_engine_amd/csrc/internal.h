@@ -84,7 +84,6 @@ bool moe_dec_supported(int d, int mid, int nslots);
 bool moe_dec_uq_supported(int d);
 int moe_launch_qvec(const float* x, uint64_t x_stride, int P, int K, uint32_t* planes, float2* meta,
                     hipStream_t st);
-bool moe_dec_gu_topk_supported(int n_experts, int kpt);
 // hgn v2 rotated experts in the gate/up launch: the routed slots read the rotated activations' planes and leave
 // their gate | up sums unfused in zraw [P][kpt][2 mid]
 struct moe_dec_v2 {
@@ -92,6 +91,7 @@ struct moe_dec_v2 {
   const uint32_t* xplanes_rot;
   const float2* xmeta_rot;
 };
+bool moe_dec_gu_topk_supported(int n_experts, int kpt);
 int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                            const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                            int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
@@ -100,7 +100,7 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
 int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
-                      hipStream_t st);
+                      hipStream_t st, const moe_dec_v2* v2 = nullptr);
 int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up, const float* x,
                           const float* logits, int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d,
                           int mid, float* hid_f32, hipStream_t st);
@@ -121,9 +121,21 @@ int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_
                              const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const float* logits,
                              int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
                              uint32_t* hplanes, float2* hmeta, hipStream_t st);
+int moe_launch_decgg_gu(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
+                        const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const int* ids, int n_experts,
+                        int id_stride, int kpt, int P, int d, int mid, uint32_t* hplanes, float2* hmeta, hipStream_t st);
 int moe_launch_decgg_dn(int tdn, int tsh, const uint8_t* down, const uint8_t* sh_down, const float* sh_logit,
                         const uint32_t* hplanes, const float2* hmeta, const int* ids, const float* ws, int id_stride,
                         int kpt, int P, int d, int mid, float* out, uint64_t out_stride, hipStream_t st);
+bool moe_decgg_uq_supported(int d);
+int moe_decgg_uq_tile_cap();
+int moe_launch_decgg_gu_uq(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
+                           const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const moe_tile* tiles,
+                           const int* ntiles, int max_tiles, const int* tokidx, int n_experts, int d, int mid,
+                           uint32_t* hplanes, float2* hmeta, hipStream_t st);
+int moe_launch_decgg_dn_uq(int tdn, int tsh, const uint8_t* down, const uint8_t* sh_down, const uint32_t* hplanes,
+                           const float2* hmeta, const moe_tile* tiles, const int* ntiles, int max_tiles, int n_experts,
+                           int d, int mid, float* pairs, hipStream_t st);
 int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
                              const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                              int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,

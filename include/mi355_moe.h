@@ -270,13 +270,13 @@ int moe_forward_x16(moe_ctx* ctx, int layer, const float* x, const void* x16, in
  * every fast path is on by default and can be turned off to fall back to the plainer kernel.
  * MOE_OPT_INT_DECODE (default 1): small batches use the integer-dot GEMV kernels (activations as
  * digit planes per 32-group, 16 significant bits relative to the group maximum) instead of the f32 FMA kernels. */
-/* MOE_OPT_UNIQUE_MIN_TOKENS (default 12; 0 = off): q4cp batches of at least this many tokens (and at most 32)
+/* MOE_OPT_UNIQUE_MIN_TOKENS (default 24; 0 = off): q4cp batches of at least this many tokens (and at most 32)
  * walk the expert-sorted pair lists, so that an expert shared by several tokens is read once
  * (the reference's _uq decode kernels, src/gpu/parts/26_kernels_moe_gguf.inc:758-877).  One extra launch
- * builds the permutation and the tile list and a reduce launch follows; from about 12 tokens on the saved reads
- * outweigh them even when the tokens route independently (measured: 117 against 120 us at 12 tokens with 109
- * distinct experts for 120 slots, 141 against 153 us at 16, 227 against 296 us at 32).
- * The pairs are then combined in ascending expert order, as on the batch path. */
+ * builds the permutation and the tile list and a reduce launch follows; measured on verify batches with 30 % of the
+ * expert picks shared, against the per-token kernels: 163 against 160 us at 20 tokens, 223 against 234 us at 32 (the
+ * per-token kernels find shared experts in L2).  The pairs are then combined in ascending expert order, as on the
+ * batch path. */
 /* MOE_OPT_FUSED_COMBINE (default 0): batches over 32 tokens fold the top-k weighted combine into the epilogue of
  * the down GEMM (the reference keeps pairs + k_moe_reduce_pw_sg, src/gpu/parts/24_kernels_moe_lt.inc:104): a tile's
  * weighted rows are added into y with f32 atomics, y is zeroed on the context's side stream, no pairs buffer is
@@ -296,8 +296,17 @@ int moe_forward_x16(moe_ctx* ctx, int layer, const float* x, const void* x16, in
  * tokens leave that stage's launches out (the later stages then work on stale scratch and the output is meaningless).
  * The difference between the times of a loop of calls without and with the skip is that stage's cost inside the
  * pipelined stream, without the dispatch latency that an event pair around a 10 us kernel adds. */
+/* MOE_OPT_GU_TOPK_MAX_TOKENS (default 4: the measured crossover on every weight format): batches of at most this many tokens run the softmax / top-k inside the gate/up launch
+ * (every block of a routed slot selects its token's experts itself: one launch less on the latency-bound path);
+ * larger batches of the integer-dot kernels take the ids from the router's launches, so that the thousands of blocks
+ * of such a launch do not each repeat the selection. */
+/* MOE_OPT_UNIQUE_GGUF (default 0): 1 = GGUF layers on the integer-dot kernels also take the distinct-expert path for
+ * batches of MOE_OPT_UNIQUE_MIN_TOKENS .. 32 tokens (the reference's _uq kernels, 26_kernels_moe_gguf.inc:758-886:
+ * every distinct expert's rows are read once per batch).  Off by default: at the benchmark's verify batch (20 tokens,
+ * 30 % of the expert picks shared) the per-token kernels measure faster; it pays when most tokens share their experts. */
 enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2, MOE_OPT_FUSED_COMBINE = 3, MOE_OPT_SHARED_ASIDE = 4,
-       MOE_OPT_TIMING_SKIP_STAGE = 5, MOE_OPT_ROUTER_CANDIDATES = 6 };
+       MOE_OPT_TIMING_SKIP_STAGE = 5, MOE_OPT_ROUTER_CANDIDATES = 6, MOE_OPT_UNIQUE_GGUF = 7,
+       MOE_OPT_GU_TOPK_MAX_TOKENS = 8 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP

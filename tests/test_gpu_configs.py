@@ -117,11 +117,11 @@ def test_prefill_chunk_at_full_token_count(oracle, fmt, T):
     m.close()
 
 
-@pytest.mark.parametrize("uq", [12, 0])
+@pytest.mark.parametrize("uq", [12, 0])  # (12: the distinct-expert path at this size; the default threshold is 24)
 def test_verify_batch_of_20_tokens_at_512_experts(oracle, uq):
     """Speculative-verify batch: 4 requests x (4 drafted + 1) = 20 tokens, about 30 % of them reproducing one token's
-    top-10 set.  Ids bit-exact, output within the decode tolerance, on the distinct-expert path (default) and with every
-    token reading its own experts (MOE_OPT_UNIQUE_MIN_TOKENS = 0)."""
+    top-10 set.  Ids bit-exact, output within the decode tolerance, on the distinct-expert path and with every
+    token reading its own experts (MOE_OPT_UNIQUE_MIN_TOKENS = 0, the default at 20 tokens)."""
     import torch
     from gfx1151_engine_amd import capi, workloads as W
     T = 20

@@ -240,6 +240,39 @@ def test_unique_expert_path(oracle, share):
     m.close()
 
 
+@pytest.mark.parametrize("types,T,share,shared", [((12, 12, 12), 20, 0.3, True), ((13, 8, 8), 20, 1.0, True),
+                                                  ((12, 7, 13), 12, 0.3, True), ((13, 8, 8), 32, 0.5, False),
+                                                  ((8, 13, 7), 17, 0.0, True)])
+def test_unique_expert_path_gguf(oracle, types, T, share, shared):
+    """The distinct-expert kernels for GGUF layers (any mix of Q4_K / Q5_K / Q8_0 / Q5_1): a verify-size batch through
+    the expert-sorted pair lists, tiles of at most four pairs, against the oracle and against the per-token kernels."""
+    import torch
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(92 + T)
+    d, mid, E, k = 3072, 768, 24, 10
+    hl = HostLayer(rng, d, mid, E, k, fmt="q4k", gg_types=types, shared=shared)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    for i in range(1, int(round(share * T))):
+        x[i] = x[0] + 1e-3 * rng.standard_normal(d).astype(np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=32)
+    m.set_option(capi.OPT_UNIQUE_MIN_TOKENS, 8)
+    m.set_option(capi.OPT_UNIQUE_GGUF, 1)
+    m.profile(True)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    assert m.profile_read()["reduce"] > 0, "the distinct-expert path ends in a combine launch"
+    m.profile(False)
+    ids, ws = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    assert np.abs(ws.cpu().numpy()[:, :k] - wo[:, :k]).max() <= 1e-6
+    assert max_abs_rel(y, yo) <= TOL_INT_Q4K, max_abs_rel(y, yo)
+    m.set_option(capi.OPT_UNIQUE_GGUF, 0)
+    y2 = m.forward(0, gpu(x)).cpu().numpy()
+    assert max_abs_rel(y2, yo) <= TOL_INT_Q4K
+    assert max_abs_rel(y, y2) <= 1e-5, "the same integer sums per pair: only the order of the combine's additions differs"
+    m.close()
+
+
 @pytest.mark.parametrize("i", [0, 1, 2, 3])
 def test_golden_layers_from_reference(oracle, golden, i):
     """Inputs and outputs of the reference's own Model::moe (tests/golden/moe_layer.npz): four layers, two of them
