@@ -766,14 +766,38 @@ static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, floa
   });
 }
 
-// Which grouped GEMM a layer's batches take: 0 = q4cp (tuned), 1 = raw GGUF Q4_K throughout (tuned), 2 = raw GGUF
-// blocks of any supported type (general kernel, f16 operands in natural order).
-static int batch_gemm_kind(const MoeLayer& L) {
-  if (!L.has_gguf) return 0;
-  if (L.has_shared && L.sh_dense) return 2;  // (the dense shared expert reads activations in natural order)
-  const bool all4k = L.gg.tgu == MOE_GGML_Q4_K && L.gg.tdn == MOE_GGML_Q4_K &&
-                     (!L.has_shared || L.sh_gguf_type == MOE_GGML_Q4_K);
-  return all4k ? 1 : 2;
+// Which grouped GEMM each of a GGUF layer's four launches takes.  The tuned kernel (gemm_q4cp.hip: raw K-quant blocks
+// dequantised in registers, activations in the order the unpack produces) has gate/up forms for Q4_K and Q5_K and a
+// down form for Q4_K, which reads the hid rows its own gate/up form wrote; everything else (Q8_0, Q5_1, IQ4 types,
+// densely stored shared experts) goes through the general kernel (gguf_types.hip), which puts activations of either
+// order back into natural order on their way into LDS.
+struct GgKinds {
+  bool r_gu, r_dn, s_gu, s_dn;  // tuned? (routed gate/up, routed down, shared gate/up, shared down)
+  bool any_tuned() const { return r_gu || s_gu; }
+  // routed and shared tiles can share a launch when they take the same kernel with the same block type
+  bool uniform(const MoeLayer& L) const {
+    if (!L.has_shared) return true;
+    if (L.sh_dense) return false;
+    return r_gu == s_gu && r_dn == s_dn && (!r_gu || L.gg.tgu == L.sh_gguf_type);
+  }
+};
+static GgKinds gg_kinds(const MoeLayer& L, int d, int mid) {
+  GgKinds k{false, false, false, false};
+  if (!L.has_gguf) return k;
+  auto gu_ok = [](int t) { return t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K; };
+  const bool shapes = d % 256 == 0 && mid % 256 == 0;
+  k.r_gu = shapes && gu_ok(L.gg.tgu);
+  k.r_dn = k.r_gu && L.gg.tdn == MOE_GGML_Q4_K;
+  if (L.has_shared && !L.sh_dense) {
+    k.s_gu = shapes && gu_ok(L.sh_gguf_type);
+    k.s_dn = k.s_gu && L.sh_gguf_type == MOE_GGML_Q4_K;
+  }
+  return k;
+}
+// the order of the f16 activations a layer's grouped GEMMs read (moe_f32_to_f16's layout)
+static int batch_x16_layout(const MoeLayer& L, int d, int mid) {
+  if (!L.has_gguf) return 1;
+  return gg_kinds(L, d, mid).any_tuned() ? 2 : 0;
 }
 
 // Router of a batch: ids / ws, the shared-expert gate logit and (if asked) the per-token mean square of x.
@@ -800,12 +824,12 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   // leave gate | up unfused for the rotations around SwiGLU, and the combine rotates the weighted sum
   const bool v2 = L.has_i4r;
   if (v2 && (!c->v2_x16 || g.d % 256 || g.mid % 256)) return MOE_E_UNSUPPORTED;
-  // gen: a GGUF layer that is not Q4_K throughout takes the general grouped GEMM (any supported block type,
-  // dequantised into f16 tiles in LDS); Q4_K-only and q4cp layers take the tuned kernel
-  const bool gen = batch_gemm_kind(L) == 2;
+  // GGUF layers: each launch on the tuned kernel where it has a form for the block type, else on the general one
+  const GgKinds kd = gg_kinds(L, g.d, g.mid);
   const bool shd = L.has_shared && L.sh_dense;  // shared expert stored densely: the general GEMM, launches of its own
+  const bool split = shd || (q4k && !kd.uniform(L));  // routed and shared experts in launches of their own
   if (L.has_shared && !shd && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format family per layer
-  if (gen ? (g.d % 64 || g.mid % 64) : q4k ? (g.d % 256 || g.mid % 256) : (g.d % 128 || g.mid % 128 || g.mid < 256 || g.d < 256))
+  if (q4k ? (g.d % 64 || g.mid % 64) : (g.d % 128 || g.mid % 128 || g.mid < 256 || g.d < 256))
     return MOE_E_UNSUPPORTED;  // the caller walks the batch through the small path
   moe_lutw gu{}, dn{}, sgu{}, sdn{};
   const float* sh_cb_up = nullptr;
@@ -838,17 +862,28 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   prof_mark(c, 0, st);
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
   const __half* xh = c->x16_ext ? c->x16_ext : c->x16;  // f16 activations in the GEMM's order
-  const int xl = gen ? 0 : q4k ? 2 : 1;                 // that order (moe_f32_to_f16's layout)
+  const int xl = batch_x16_layout(L, g.d, g.mid);       // that order (moe_f32_to_f16's layout)
   // gate/up (+ SwiGLU) and down launches over a tile list: routed experts, with_sh: the shared expert as well
   // (tiles whose expert index is >= n_experts)
   auto gemm_up = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2) -> int {
     if (shd && with_sh)  // the shared expert's own tile list
       return moe_launch_gemm_gg(true, L.sh_dense, L.sh_gate.data, L.sh_up.data, 0, nullptr, nullptr, g.experts, xh,
-                                c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, hs, s2, xl == 1 ? 1 : 0);
-    if (gen)
+                                c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, hs, s2, xl);
+    if (q4k && split) {  // one class per launch: the shared expert's tiles (with_sh) or the routed experts'
+      if (with_sh ? kd.s_gu : kd.r_gu)
+        return moe_launch_gemm_q4cp(true, with_sh ? &sgu : &gu, with_sh ? &sgu : nullptr, g.experts, xh, c->tokidx, tl, ntl,
+                                    mt, c->hid16, g.mid, g.d, true, true, hs, s2, nullptr, nullptr, 0,
+                                    (with_sh ? L.sh_gguf_type : L.gg.tgu) == MOE_GGML_Q5_K);
+      return with_sh ? moe_launch_gemm_gg(true, L.sh_gguf_type, L.sh_gate.data, L.sh_up.data, L.sh_gguf_type,
+                                          L.sh_gate.data, L.sh_up.data, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16,
+                                          g.mid, g.d, hs, s2, xl)
+                     : moe_launch_gemm_gg(true, L.gg.tgu, L.gg.gate, L.gg.up, 0, nullptr, nullptr, g.experts, xh,
+                                          c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, hs, s2, xl);
+    }
+    if (q4k && !kd.r_gu)
       return moe_launch_gemm_gg(true, L.gg.tgu, L.gg.gate, L.gg.up, L.sh_gguf_type, with_sh ? L.sh_gate.data : nullptr,
                                 with_sh ? L.sh_up.data : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid,
-                                g.d, hs, s2);
+                                g.d, hs, s2, xl);
     if (v2 && !with_sh) {  // the routed experts' tiles: plain rows of the fused tensor, then the slot-wise middle
       const int e = moe_launch_gemm_q4cp(false, &gu, nullptr, g.experts, c->v2_x16, c->tokidx, tl, ntl, mt, c->v2_z16,
                                          2 * g.mid, g.d, true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
@@ -859,15 +894,27 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
       return moe_launch_gemm_q4cp(true, &sgu, &sgu, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, true,
                                   false, hs, s2, nullptr, sh_cb_up);
     return moe_launch_gemm_q4cp(true, &gu, with_sh ? &sgu : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16,
-                                g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up);
+                                g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up, 0, q4k && L.gg.tgu == MOE_GGML_Q5_K);
   };
   auto gemm_dn = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2, const moe_comb* cmb) -> int {
     if (shd && with_sh)  // (hid rows of the shared tiles were written in natural order by the launch above)
       return moe_launch_gemm_gg(false, L.sh_dense, L.sh_down.data, nullptr, 0, nullptr, nullptr, g.experts, c->hid16,
                                 nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2, 0);
-    if (gen)
+    if (q4k && split) {
+      // (hid rows are in the tuned kernel's order where its gate/up form wrote them, else in natural order)
+      if (with_sh ? kd.s_dn : kd.r_dn)
+        return moe_launch_gemm_q4cp(false, with_sh ? &sdn : &dn, with_sh ? &sdn : nullptr, g.experts, c->hid16, nullptr, tl,
+                                    ntl, mt, c->pairs16, g.d, g.mid, true, true, hs, s2, nullptr);
+      return with_sh ? moe_launch_gemm_gg(false, L.sh_gguf_type, L.sh_down.data, nullptr, L.sh_gguf_type, L.sh_down.data,
+                                          nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2,
+                                          kd.s_gu ? 2 : 0)
+                     : moe_launch_gemm_gg(false, L.gg.tdn, L.gg.down, nullptr, 0, nullptr, nullptr, g.experts, c->hid16,
+                                          nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2, kd.r_gu ? 2 : 0);
+    }
+    if (q4k && !kd.r_dn)
       return moe_launch_gemm_gg(false, L.gg.tdn, L.gg.down, nullptr, L.sh_gguf_type, with_sh ? L.sh_down.data : nullptr,
-                                nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2);
+                                nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2,
+                                kd.r_gu ? 2 : 0);
     if (v2 && !with_sh)
       return moe_launch_gemm_q4cp(false, &dn, nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid,
                                   true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
@@ -877,8 +924,8 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     return moe_launch_gemm_q4cp(false, &dn, with_sh ? &sdn : nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt,
                                 cmb ? (void*)cmb->y : (void*)c->pairs16, g.d, g.mid, cmb == nullptr, q4k, hs, s2, cmb);
   };
-  const bool fused = c->fused_combine && !c->hc && !gen && !shd && !v2;  // the HC write-back belongs to the ordered combine
-  if (v2 || (L.has_shared && (shd || (c->shared_aside && !fused)))) {
+  const bool fused = c->fused_combine && !c->hc && !(q4k && !kd.r_dn) && !split && !v2;  // the HC write-back belongs to the ordered combine
+  if (v2 || (L.has_shared && (split || (c->shared_aside && !fused)))) {
     // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
     // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
     // side stream also makes what both streams need first: the per-token mean square of x (range guard) and
@@ -1013,8 +1060,7 @@ MOE_API int moe_x16_layout(moe_ctx* c, int layer) {
   MoeLayer* L = layer_of(c, layer);
   if (!L) return MOE_E_INVALID;
   if (!(L->has_q4cp || L->has_gguf || L->has_i4r)) return MOE_E_STATE;
-  const int kind = batch_gemm_kind(*L);
-  return kind == 0 ? 1 : kind == 1 ? 2 : 0;
+  return batch_x16_layout(*L, c->cfg.d, c->cfg.mid);
 }
 
 // moe_forward for a batch whose f16 copy the caller has already made (its HC-read epilogue can write it next to

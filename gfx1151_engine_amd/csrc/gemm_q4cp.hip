@@ -24,6 +24,13 @@
 // each with its own w = (d*sc)*n - dmin*m as one packed f16 FMA.  The 16-byte block header takes
 // the place of q4cp's 8 staged scales (one per row and four stages).
 //
+// Q5 (with Q4K): raw GGUF Q5_K super-blocks (176 B: the Q4_K header, 32 bytes qh, 128 code bytes; src/gguf.h:421-441):
+// the same stages with a fifth bit per code -- bit 2jj of qh byte l for the low nibble of code byte l in stage jj of the
+// super-block, bit 2jj+1 for the high nibble.  The 32 qh bytes travel with the header (48 bytes per row and super-block
+// in the scale buffer); a lane keeps its 16 of them in registers for the four stages and ORs the bit into the
+// magic-number form of each code pair (1024 + n and 64 + n stay exact for n < 32).  The larger scale buffer leaves room
+// for one block per CU instead of two.
+//
 // GS = 2: one scale per 128 columns instead of 32 (hgn v2 i4r experts, reference kI4R,
 // src/gpu/parts/27_kernels_moe_lut.inc:23-29): the four stages between two scale refreshes span exactly two scales,
 // fetched as one 4-byte load per row.
@@ -136,7 +143,7 @@ __device__ __forceinline__ void g2l4(const void* g, uint8_t* lds_base) {
 // MF = live 32-row fragments of the tile (1 .. 4); AFFINE = codebook a*n+b.
 // NF = weight fragments (32 rows) per wave: the block's 16 fragments are split over NW = 16/NF
 // waves, each wave multiplying all MF pair fragments with its own NF weight fragments.
-template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS>
+template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS, bool Q5>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
@@ -144,10 +151,14 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
                                           float cmag, const moe_comb& cmb, bool shared) {
   constexpr int NH = NF / 2;  // gate/up: fragments per half
   static_assert(GS == 0 || (GS == 2 && !Q4K && NSB == 1), "one scale per 128 columns: q4cp-style planes, single scale buffer");
+  static_assert(!Q5 || (Q4K && NSB == 1), "Q5_K: the Q4_K stages plus a fifth bit");
+  constexpr int KBLK = Q5 ? 176 : 144;   // bytes per super-block
+  constexpr int KQS = Q5 ? 48 : 16;      // offset of the code bytes in it
+  constexpr int SP = Q5 ? 3 : 1;         // 16-byte pieces per row in the scale buffer (header; Q5_K: + 32 bytes qh)
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
-  const float* cbs = (const float*)(S0 + NSB * S_BYTES);
+  const float* cbs = (const float*)(S0 + NSB * S_BYTES * SP);
   int* rowidx = (int*)(cbs + 32);  // cbs[16..31]: the up rows' codebook
   float* rowscale = (float*)(rowidx + BM);  // f16 range guard of each pair row (gate/up only)
   const int tid = threadIdx.x, lane = tid & 63;
@@ -173,7 +184,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       grow = (size_t)e * L.e_rows + r;
     }
     if (Q4K) {
-      cw = cb0 + grow * (size_t)(K / 256 * 144);  // raw row: K/256 super-blocks
+      cw = cb0 + grow * (size_t)(K / 256 * KBLK);  // raw row: K/256 super-blocks
       sw = cw;                                    // block header (d, dmin, packed scales) leads each block
     } else {
       cw = cb0 + grow * (size_t)(K / 2);
@@ -187,13 +198,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // (same bytes to the same place) so that every wave issues the same number of loads.
   constexpr int A_GROUPS = 4 * MF;
   constexpr int A_LOADS = (A_GROUPS + NW - 1) / NW;
-  constexpr int W_LOADS = WROWS / 32 / NW, S_LOADS = (WROWS / 64 + NW - 1) / NW;
+  constexpr int W_LOADS = WROWS / 32 / NW, S_ROWG = (WROWS / 64 + NW - 1) / NW, S_LOADS = S_ROWG * SP;
   const __half* a_src[A_LOADS];
   int a_grp[A_LOADS];
 #pragma unroll
   for (int i = 0; i < A_LOADS; i++) a_grp[i] = (A_LOADS * wv + i) % A_GROUPS;  // a_src: once the row indices are in LDS
   // codes: rows 32j..32j+31, lane -> (row 32j + lane/2, half lane%2); scales: rows 64j.., lane -> row
-  const uint8_t *w_src[W_LOADS], *s_src[S_LOADS];
+  const uint8_t *w_src[W_LOADS], *s_src[S_ROWG];
 #pragma unroll
   for (int i = 0; i < W_LOADS; i++) {
     const uint8_t* sw;
@@ -201,9 +212,9 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     w_src[i] += (lane & 1) * 16;
   }
 #pragma unroll
-  for (int i = 0; i < S_LOADS; i++) {
+  for (int i = 0; i < S_ROWG; i++) {
     const uint8_t* cw;
-    wrow_ptrs(64 * (S_LOADS * wv + i) + lane, cw, s_src[i]);
+    wrow_ptrs(64 * (S_ROWG * wv + i) + lane, cw, s_src[i]);
   }
   const int nstage = K / BK, ngroups = K / 32;
   constexpr int NLOADS = A_LOADS + W_LOADS;  // per stage (+S_LOADS scale loads on every fourth stage)
@@ -214,18 +225,18 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + a_grp[u] * 1024);
     } else if (u < NLOADS) {
       const int i = u - A_LOADS;
-      const size_t off = Q4K ? (size_t)(s >> 2) * 144 + 16 + (size_t)(s & 3) * 32 : (size_t)s * 32;
+      const size_t off = Q4K ? (size_t)(s >> 2) * KBLK + KQS + (size_t)(s & 3) * 32 : (size_t)s * 32;
       g2l16(w_src[i] + off, W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
     } else {
       // 8 scales (16 B) per row for stages s..s+3; at the end of K the window is pulled back inside the row
-      const int i = u - NLOADS;
+      const int i = (u - NLOADS) / SP, pc = (u - NLOADS) % SP;  // row group, 16-byte piece of the row's record
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
-      const size_t off = Q4K ? (size_t)(s >> 2) * 144 : (size_t)g0 * 2;
+      const size_t off = Q4K ? (size_t)(s >> 2) * KBLK + 16 * pc : (size_t)g0 * 2;
       if (GS == 2)  // the two scales of stages s..s+3 (s % 4 == 0: columns 64 s .. 64 s + 255), [row][4 B]
-        g2l4(s_src[i] + (size_t)s, S0 + (S_LOADS * wv + i) * 256);
-      else
-        g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + (S_LOADS * wv + i) * 1024);
+        g2l4(s_src[i] + (size_t)s, S0 + (S_ROWG * wv + i) * 256);
+      else  // piece pc of every row: a region of its own, [row][16 B]
+        g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + pc * S_BYTES + (S_ROWG * wv + i) * 1024);
     }
   };
   auto issue_a = [&](int s) {
@@ -297,6 +308,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   half2v as2[NF][NS], bs2[NF][NS];
   float scf[NF];
   uint4 hdr[NF];
+  uint4 qh4[Q5 ? NF : 1];  // Q5_K: this lane's 16 qh bytes of the current super-block (code bytes 16 h .. 16 h + 15)
+  int q5sh = 0;            // Q5_K: 2 * (stage within the super-block) = the bit of a qh byte that belongs to the stage's low nibbles
   uint32_t k4w[Q4K ? NF : 1][6];  // Q4_K: the current super-block's scale / min fields and (d, d), (-dmin, -dmin)
   const uint8_t* Ab = A0;
   auto load_a1 = [&](int q, int mf, half8* dst) {
@@ -305,6 +318,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   };
   uint32_t sc4[NSB == 1 ? NF : 1][4];  // single scale buffer: this lane's scales of four stages (f16 bits)
   auto load_codes = [&](int s) {  // raw codes + this lane's scale of stage s (buffers already selected)
+    if (Q5) q5sh = 2 * (s & 3);
     const uint8_t* Wb = W0 + (s % NBUF) * W_BYTES;
     const uint8_t* Sb = S0 + ((s >> 2) & (NSB - 1)) * S_BYTES;
     int g0 = 2 * (s & ~3);
@@ -319,7 +333,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         // stages' values when the first of them is prepared (every wave has by the next barrier;
         // the loads that overwrite it are issued two barriers later)
         if (Q4K) {
-          if ((s & 3) == 0) hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
+          if ((s & 3) == 0) {
+            hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
+            if (Q5) qh4[nf] = *(const uint4*)(Sb + (1 + h) * S_BYTES + wrow[nf] * 16);
+          }
         } else {
           if (GS == 2) {
             if ((s & 3) == 0) {
@@ -403,11 +420,22 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       const uint32_t ws = part >= 2 ? w8 : w;
       const int ss = Q4K ? (part & 1) : 0;  // Q4_K: odd parts are the high nibbles = the stage's second sub-block
       uint32_t t;
+      // Q5_K: the qh word of these four code bytes; the pair's two fifth bits go to bit 4 / 20 (low nibbles: value 16
+      // on top of 1024 + n) or bit 8 / 24 (high nibbles: 16 on top of 64 + n, whose unit is bit 4)
+      uint32_t q5 = 0;
+      if (Q5) {
+        const uint32_t qw = q == 0 ? qh4[nf].x : q == 1 ? qh4[nf].y : q == 2 ? qh4[nf].z : qh4[nf].w;
+        // bytes 0, 2 (parts 0, 1) or 1, 3 (parts 2, 3); bit 2 jj (low nibbles) or 2 jj + 1 (high nibbles) of each
+        const int from = (part >= 2 ? 8 : 0) + q5sh + (part & 1), to = (part & 1) ? 8 : 4;
+        q5 = __builtin_amdgcn_alignbit(qw, qw, (uint32_t)(from - to) & 31u);  // rotate: the mask below drops the rest
+      }
       if ((part & 1) == 0) {
         asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(ws), "s"(0x000f000fu), "v"(0x64006400u));
+        if (Q5) asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(q5), "s"(0x00100010u), "v"(t));
         dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)1024.f, (_Float16)1024.f}) * as2[nf][ss] + bs2[nf][ss];
       } else {
         asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(ws), "s"(0x00f000f0u), "v"(0x54005400u));
+        if (Q5) asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(t) : "v"(q5), "s"(0x01000100u), "v"(t));
         dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)64.f, (_Float16)64.f}) * as2[nf][ss] + bs2[nf][ss];
       }
     } else {
@@ -615,14 +643,14 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   }
 }
 
-template <bool UP, bool F16OUT, bool Q4K, int GS>
-__global__ void __launch_bounds__(NT, WPE)
+template <bool UP, bool F16OUT, bool Q4K, int GS, bool Q5 = false>
+__global__ void __launch_bounds__(NT, Q5 ? 1 : WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,
                 moe_hscale hs, moe_comb cmb) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES);
+  float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES * (Q5 ? 3 : 1));
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
   // Routed tiles and shared-expert tiles (all full) are dealt out separately, or the XCD that
@@ -683,8 +711,8 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
-    else gemm_tile<UP, F16OUT, MF, false, false, GS>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS, Q5>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    else gemm_tile<UP, F16OUT, MF, false, false, GS, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
@@ -732,8 +760,9 @@ bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k, int gs = 0) {
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs) {
+                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs, bool q5k) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
+  if (q5k && (!q4k || !up || comb)) return MOE_E_UNSUPPORTED;  // (Q5_K: gate/up tensors, the reference checkpoints' use of it)
   if (gs != 0 && (gs != 2 || up || !f16out || q4k || sh || comb)) return MOE_E_UNSUPPORTED;
   moe_comb cmb{};
   if (comb) {  // fused combine: down launch with f32 results, out = the (zeroed) token rows
@@ -762,7 +791,17 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
     k_moe_gemm_q4cp<UPK, F16, Q, G><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
                                                                   m, k, nblk_n, split, hs, cmb);                 \
   } while (0)
-  if (gs == 2) {
+  if (q5k) {
+    constexpr int SMEM5 = SMEM_BYTES + 2 * S_BYTES;  // header + 32 qh bytes per row: one block per CU
+    static bool attr5 = false;
+    if (!attr5) {
+      MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<true, true, true, 0, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, SMEM5));
+      attr5 = true;
+    }
+    k_moe_gemm_q4cp<true, true, true, 0, true><<<grid, NT, SMEM5, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k,
+                                                                        nblk_n, split, hs, cmb);
+  } else if (gs == 2) {
     GEMM_LAUNCH(false, true, false, 2);
   } else if (q4k) {
     if (up) GEMM_LAUNCH(true, true, true, 0);

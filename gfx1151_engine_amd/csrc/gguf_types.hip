@@ -472,6 +472,20 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
         v.z = __builtin_amdgcn_perm(w.y, w.x, 0x07060302u);
         v.w = __builtin_amdgcn_perm(w.w, w.z, 0x07060302u);
       }
+      if (a_layout == 2) {
+        // the Q4_K / Q5_K GEMM's order inside a block of 64: chunk w = [4w, 4w+2, 32+4w, 32+4w+2, 4w+1, 4w+3, 32+4w+1,
+        // 32+4w+3] -> elements 4w..4w+3 and 32+4w..32+4w+3 in natural order, two 8-byte pieces
+        const int w = i & 7;
+        uint8_t* rowp = As + buf * GG_TILE_BYTES + (i >> 3) * GG_PITCH;
+        uint2 lo, hi;
+        lo.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (e4w, e4w+1)
+        lo.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (e4w+2, e4w+3)
+        hi.x = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+        hi.y = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+        *(uint2*)(rowp + 8 * w) = lo;
+        *(uint2*)(rowp + 64 + 8 * w) = hi;
+        continue;
+      }
       *(uint4*)(As + buf * GG_TILE_BYTES + (i >> 3) * GG_PITCH + (i & 7) * 16) = v;
     }
     uint8_t* dst = Bs + buf * GG_TILE_BYTES + brow * GG_PITCH + half * 64;
@@ -616,7 +630,7 @@ int moe_launch_ggx_gemv(int phase, int tgu, int tdn, int tsh, const uint8_t* gat
 // (routed experts of type `type`, optional shared expert of type `tsh`; tile.expert >= n_experts selects it).
 // `type` / `tsh` may also be a dense code of dense.h (bf16 / f32 / q8g64 rows).
 // up: gate/up + SwiGLU -> hid f16 [pairs][m]; else down -> pairs f16 [pairs][m].  x / hid: f16, natural order
-// (a_layout = 1: x is in the q4cp GEMM's order and is put back in natural order on its way into LDS).
+// (a_layout = 1 / 2: x is in the q4cp / Q4_K GEMM's order and is put back in natural order on its way into LDS).
 int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up, int tsh, const uint8_t* sh_w,
                        const uint8_t* sh_w_up, int n_experts, const __half* x16, const int* tokidx,
                        const moe_tile* tiles, const int* ntiles, int max_tiles, __half* out, int m, int k,
@@ -624,7 +638,7 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
   if (!w || (up && !w_up) || !x16 || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
   auto type_ok = [&](int t) { return moe_is_dense_type(t) ? k % 64 == 0 : gg_type_ok(t, k); };
   auto align_of = [&](int t) -> size_t { return moe_is_dense_type(t) ? 16 : gg_align(t); };
-  if (!type_ok(type) || (sh_w && !type_ok(tsh)) || k % GG_BK || m < 1 || a_layout < 0 || a_layout > 1)
+  if (!type_ok(type) || (sh_w && !type_ok(tsh)) || k % GG_BK || m < 1 || a_layout < 0 || a_layout > 2)
     return MOE_E_UNSUPPORTED;
   if (!moe_aligned(w, align_of(type)) || (up && !moe_aligned(w_up, align_of(type))) || !moe_aligned(x16, 16) ||
       (sh_w && (!moe_aligned(sh_w, align_of(tsh)) || (up && (!sh_w_up || !moe_aligned(sh_w_up, align_of(tsh)))))))

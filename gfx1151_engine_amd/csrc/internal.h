@@ -48,7 +48,8 @@ int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr, int gs = 0);
+                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr, int gs = 0,
+                         bool q5k = false);
 int moe_gemm_tile_cap();
 int moe_launch_zero_f32(float* p, uint64_t n, hipStream_t st);
 int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, int P, int sh_first, int* tokidx,
