@@ -415,7 +415,16 @@ struct GgGemmW {
   int type;
 };
 
-template <bool UP>
+// Q8 = true: every tensor of the launch is Q8_0 (the reference checkpoints' down tensors and MTP sidecar).  Those launches
+// keep the raw bytes of three stages in flight in registers (a thread's 34-byte block as nine dwords from the 4-byte
+// boundary at or below it, its four activation pieces) and turn the int8 codes into f16 with byte permutes into the
+// 1024 + u form and two packed operations per pair: the plain form below waits for a trip to memory in every stage.
+constexpr int GQ_D = 3;
+struct GgRawQ8 {
+  uint32_t w[9];
+};
+
+template <bool UP, bool Q8 = false>
 __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, int n_experts,
                                                        const __half* __restrict__ x16, const int* __restrict__ tokidx,
                                                        const moe_tile* __restrict__ tiles,
@@ -521,10 +530,7 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
   const int nstage = K / GG_BK;
-  fill(0, 0);
-  __syncthreads();
-  for (int s = 0; s < nstage; s++) {
-    const int buf = s & 1;
+  auto mfmas = [&](int buf) {
     const uint8_t* Ab = As + buf * GG_TILE_BYTES;
     const uint8_t* Bb = Bs + buf * GG_TILE_BYTES;
 #pragma unroll
@@ -543,8 +549,97 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
         for (int nf = 0; nf < 2; nf++)
           acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
     }
-    if (s + 1 < nstage) fill(s + 1, buf ^ 1);  // behind the MFMAs just issued; the other buffer was read a stage ago
+  };
+  if constexpr (Q8) {
+    GgRawQ8 rw[GQ_D];
+    uint4 ra[GQ_D][4];
+    // block 2 s + half of the row: 34 bytes; odd blocks start 2 bytes past a 4-byte boundary (rows are whole pairs of
+    // blocks), so nine dwords from the boundary at or below cover the block and never pass the row's end
+    auto fetch = [&](int st, GgRawQ8& r, uint4 (&a4)[4]) {
+      const int sc = st < nstage ? st : nstage - 1;  // (past the end: a repeat that is never used)
+      const uint32_t* b4 = (const uint32_t*)(wrow + (size_t)(2 * sc + half) * 34 - 2 * half);
+#pragma unroll
+      for (int i = 0; i < 9; i++) r.w[i] = b4[i];
+#pragma unroll
+      for (int it = 0; it < 4; it++) a4[it] = *(const uint4*)(arow[it] + (size_t)sc * GG_BK);
+    };
+    auto decode = [&](const GgRawQ8& r, const uint4 (&a4)[4], int buf) {
+#pragma unroll
+      for (int it = 0; it < 4; it++) {
+        const int i = tid + 256 * it;
+        uint4 v = a4[it];
+        uint8_t* rowp = As + buf * GG_TILE_BYTES + (i >> 3) * GG_PITCH;
+        if (a_layout == 2) {
+          const int w = i & 7;
+          uint2 lo, hi;
+          lo.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+          lo.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+          hi.x = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+          hi.y = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+          *(uint2*)(rowp + 8 * w) = lo;
+          *(uint2*)(rowp + 64 + 8 * w) = hi;
+          continue;
+        }
+        if (a_layout == 1) {
+          const uint4 w = v;
+          v.x = __builtin_amdgcn_perm(w.y, w.x, 0x05040100u);
+          v.y = __builtin_amdgcn_perm(w.w, w.z, 0x05040100u);
+          v.z = __builtin_amdgcn_perm(w.y, w.x, 0x07060302u);
+          v.w = __builtin_amdgcn_perm(w.w, w.z, 0x07060302u);
+        }
+        *(uint4*)(rowp + (i & 7) * 16) = v;
+      }
+      // d and the 32 codes: at byte 0 / 2 of the dwords (even block) or at byte 2 / 4 (odd block)
+      union { uint16_t u; _Float16 f; } dv;
+      dv.u = (uint16_t)(half ? r.w[0] >> 16 : r.w[0] & 0xffffu);
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      const h2 d2 = {dv.f, dv.f}, k1152 = {(_Float16)1152.f, (_Float16)1152.f};
+      uint8_t* dst = Bs + buf * GG_TILE_BYTES + brow * GG_PITCH + half * 64;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        uint32_t o[4];
+#pragma unroll
+        for (int l = 0; l < 2; l++) {
+          const int i = 2 * j + l;
+          const uint32_t cd = (half ? r.w[i + 1] : __builtin_amdgcn_alignbit(r.w[i + 1], r.w[i], 16)) ^ 0x80808080u;
+          union { uint32_t u; h2 v; } p0, p1;
+          p0.u = __builtin_amdgcn_perm(0x64646464u, cd, 0x05010400u);  // (1024 + u0, 1024 + u1), u = code + 128
+          p1.u = __builtin_amdgcn_perm(0x64646464u, cd, 0x05030402u);
+          p0.v = (p0.v - k1152) * d2;  // code * d, one rounding: the f16 of the exact product
+          p1.v = (p1.v - k1152) * d2;
+          o[2 * l] = p0.u;
+          o[2 * l + 1] = p1.u;
+        }
+        *(uint4*)(dst + 16 * j) = make_uint4(o[0], o[1], o[2], o[3]);
+      }
+    };
+#pragma unroll
+    for (int i = 0; i < GQ_D; i++) fetch(i, rw[i], ra[i]);
+    decode(rw[0], ra[0], 0);
     __syncthreads();
+    for (int s0 = 0; s0 < nstage; s0 += GQ_D) {
+#pragma unroll
+      for (int u = 0; u < GQ_D; u++) {
+        const int s = s0 + u;
+        if (s < nstage) {
+          const int buf = s & 1;
+          // stage s is in LDS; the registers hold stages s + 1 and s + 2; slot u takes stage s + 3
+          fetch(s + GQ_D, rw[u], ra[u]);
+          mfmas(buf);
+          if (s + 1 < nstage) decode(rw[(u + 1) % GQ_D], ra[(u + 1) % GQ_D], buf ^ 1);
+          __syncthreads();
+        }
+      }
+    }
+  } else {
+    fill(0, 0);
+    __syncthreads();
+    for (int s = 0; s < nstage; s++) {
+      const int buf = s & 1;
+      mfmas(buf);
+      if (s + 1 < nstage) fill(s + 1, buf ^ 1);  // behind the MFMAs just issued; the other buffer was read a stage ago
+      __syncthreads();
+    }
   }
   // D[i][j]: j = lane % 32 (weight row), i = 8 * (r / 4) + 4 * (lane / 32) + r % 4 (pair)
 #pragma unroll
@@ -650,9 +745,17 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
   if (!attr_done) {
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     attr_done = true;
   }
-  if (up) k_moe_gemm_gg<true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+  // all-Q8_0 launches (4-byte aligned rows: whole pairs of 34-byte blocks from a 4-byte aligned base)
+  const bool q8 = type == MOE_GGML_Q8_0 && (!sh_w || tsh == MOE_GGML_Q8_0) && moe_aligned(w, 4) &&
+                  (!up || moe_aligned(w_up, 4)) && (!sh_w || (moe_aligned(sh_w, 4) && (!up || moe_aligned(sh_w_up, 4))));
+  if (q8) {
+    if (up) k_moe_gemm_gg<true, true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+    else k_moe_gemm_gg<false, true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+  } else if (up) k_moe_gemm_gg<true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   else k_moe_gemm_gg<false><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
