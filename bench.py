@@ -395,6 +395,11 @@ def main():
         # dequantises through a table, the decode kernels look codes up instead of taking integer dots)
         sub("universal_codebook_prefill_T16384", "prefill", a.steps, a.warmup, codebook="universal")
         sub("universal_codebook_decode_T1", "decode", nd, wd, codebook="universal")
+        # a GGUF layer in the type mix of the reference's checkpoints, and an hgn v2 layer (rotated i4r experts)
+        sub("gguf_q5k_q8_0_prefill_T8192", "ggmix_prefill", a.steps, a.warmup)
+        sub("gguf_q5k_q8_0_decode_T1", "ggmix_decode", nd, wd)
+        sub("hgn_v2_prefill_T16384", "v2_prefill", a.steps, a.warmup)
+        sub("hgn_v2_decode_T1", "v2_decode", nd, wd)
     elif a.workload in ("load", "q4k_load"):
         res = measure_load("q4k" if a.workload.startswith("q4k") else "q4cp", min(a.steps, 5), min(a.layers, 2))
     else:

@@ -737,13 +737,14 @@ static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, floa
   const bool gu_topk = P <= c->gu_topk_max;
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
+         // (the planes of rot_in(x, su) ride in the router launch's spare blocks)
+         const moe_rot_planes rot{L.v2_su, c->v2_xplanes, c->v2_xmeta};
          int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
                                          c->sh_logit, sh ? c->xplanes : nullptr, c->xmeta, false,
                                          gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk, g.id_stride, &fused, st,
-                                         c->kpart, c->ktickets);
+                                         c->kpart, c->ktickets, &rot);
          if (!e && !fused && !gu_topk) e = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
-         return e ? e : moe_launch_v2_rot(x, (uint64_t)g.d, P, g.d, L.v2_su, nullptr, 2, nullptr, 0, nullptr, 0,
-                                          c->v2_xplanes, c->v2_xmeta, st);
+         return e;
        })))
     return rc;
   const moe_wview *shg = sh ? &L.sh_gate : nullptr, *shu = sh ? &L.sh_up : nullptr, *shd = sh ? &L.sh_down : nullptr;

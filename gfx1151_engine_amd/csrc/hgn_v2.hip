@@ -20,13 +20,6 @@
 
 namespace {
 
-__device__ __forceinline__ float quad_xor1(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float quad_xor2(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));
-}
-
 __device__ __forceinline__ void ld8(const float* p, float (&v)[8]) {
   const float4 a = ((const float4*)p)[0], b = ((const float4*)p)[1];
   v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
@@ -53,40 +46,6 @@ __device__ __forceinline__ void st8_f16_ilv(__half* p, const float (&v)[8]) {
   o.x = *(const uint32_t*)&a; o.y = *(const uint32_t*)&b; o.z = *(const uint32_t*)&c; o.w = *(const uint32_t*)&d;
   *(uint4*)p = o;
 }
-// 8 values per lane, the four lanes of a quad = one 32-element group -> the group's four digit planes and (q, q*sum)
-// in the form the integer-dot decode kernels read (qvec.h, qvec4): lane j of the quad holds dword j of every plane.
-__device__ __forceinline__ void st8_planes(const float (&v)[8], int lane, uint32_t* __restrict__ planes,
-                                           float2* __restrict__ meta, size_t gi, bool live) {
-  float m = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
-  m = fmaxf(m, quad_xor1(m));
-  m = fmaxf(m, quad_xor2(m));
-  const float inv = m > 0.f ? QV4_XMAX / m : 0.f;
-  const float q = m * (1.f / QV4_XMAX);
-  uint32_t pl[4] = {0u, 0u, 0u, 0u};
-  int sx = 0;
-#pragma unroll
-  for (int i = 0; i < 8; i++) {
-    const int X = (int)rintf(v[i] * inv);
-    sx += X;
-    int p0, p1, p2, p3;
-    qv4_digits(X, p0, p1, p2, p3);
-    pl[0] |= (uint32_t)(p0 & 15) << (4 * i);
-    pl[1] |= (uint32_t)(p1 & 15) << (4 * i);
-    pl[2] |= (uint32_t)(p2 & 15) << (4 * i);
-    pl[3] |= (uint32_t)(p3 & 15) << (4 * i);
-  }
-  sx += __builtin_amdgcn_update_dpp(0, sx, 0xB1, 0xf, 0xf, true);
-  sx += __builtin_amdgcn_update_dpp(0, sx, 0x4E, 0xf, 0xf, true);
-  if (live) {
-    uint32_t* dst = planes + gi * QV4_GROUP_DW + (lane & 3);
-#pragma unroll
-    for (int p = 0; p < 4; p++) dst[4 * p] = pl[p];
-    if ((lane & 3) == 0) meta[gi] = make_float2(q, q * (float)sx);
-  }
-}
-
 // y[p][i] = post[i] * H(pre . x[p])[i] / sqrt(128) (+ add[p][i]) per 128 block; pre / post / add optional.
 // P rows of n values (n % 128 == 0), n/8 lanes per row.  MODE 0: f32 rows; 1: f16 rows in the grouped GEMM's order;
 // 2: digit planes of the decode kernels (planes / meta indexed [p][n/32]).  In place (MODE 0, y == x) is fine.
@@ -131,7 +90,7 @@ __global__ void __launch_bounds__(256) k_v2_rot(const float* x, uint64_t xs, voi
   } else if (MODE == 1) {
     if (live) st8_f16_ilv((__half*)y + (size_t)p * ys + c, v);
   } else {
-    st8_planes(v, lane, planes, meta, (size_t)p * (n >> 5) + (c >> 5), live);
+    moe_st8_planes(v, lane, planes, meta, (size_t)p * (n >> 5) + (c >> 5), live);
   }
 }
 
@@ -184,7 +143,7 @@ __global__ void __launch_bounds__(256) k_i4r_mid(const TG* __restrict__ z, uint6
   } else if (MODE == 1) {
     if (live) st8_f16_ilv((__half*)out + row * os + c, h);
   } else {
-    st8_planes(h, lane, planes, meta, row * (mid >> 5) + (c >> 5), live);
+    moe_st8_planes(h, lane, planes, meta, row * (mid >> 5) + (c >> 5), live);
   }
 }
 

@@ -4,6 +4,7 @@
 // src/gpu/parts/27_kernels_moe_lut.inc:44-65).
 #pragma once
 #include "common.h"
+#include "qvec.h"
 
 constexpr float MOE_RS128 = 0.0883883476483184405f;  // 1 / sqrt(128)
 
@@ -47,3 +48,45 @@ __device__ __forceinline__ void moe_fwht128_r8(float (&v)[8], int lane) {
   MOE_FWHT_STEP(8)
 #undef MOE_FWHT_STEP
 }
+
+__device__ __forceinline__ float moe_quad_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float moe_quad_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, true));
+}
+
+// 8 values per lane, the four lanes of a quad = one 32-element group -> the group's four digit planes and (q, q*sum)
+// in the form the integer-dot decode kernels read (qvec.h, qvec4): lane j of the quad holds dword j of every plane.
+__device__ __forceinline__ void moe_st8_planes(const float (&v)[8], int lane, uint32_t* __restrict__ planes,
+                                           float2* __restrict__ meta, size_t gi, bool live) {
+  float m = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+  m = fmaxf(m, moe_quad_xor1(m));
+  m = fmaxf(m, moe_quad_xor2(m));
+  const float inv = m > 0.f ? QV4_XMAX / m : 0.f;
+  const float q = m * (1.f / QV4_XMAX);
+  uint32_t pl[4] = {0u, 0u, 0u, 0u};
+  int sx = 0;
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int X = (int)rintf(v[i] * inv);
+    sx += X;
+    int p0, p1, p2, p3;
+    qv4_digits(X, p0, p1, p2, p3);
+    pl[0] |= (uint32_t)(p0 & 15) << (4 * i);
+    pl[1] |= (uint32_t)(p1 & 15) << (4 * i);
+    pl[2] |= (uint32_t)(p2 & 15) << (4 * i);
+    pl[3] |= (uint32_t)(p3 & 15) << (4 * i);
+  }
+  sx += __builtin_amdgcn_update_dpp(0, sx, 0xB1, 0xf, 0xf, true);
+  sx += __builtin_amdgcn_update_dpp(0, sx, 0x4E, 0xf, 0xf, true);
+  if (live) {
+    uint32_t* dst = planes + gi * QV4_GROUP_DW + (lane & 3);
+#pragma unroll
+    for (int p = 0; p < 4; p++) dst[4 * p] = pl[p];
+    if ((lane & 3) == 0) meta[gi] = make_float2(q, q * (float)sx);
+  }
+}
+

@@ -24,10 +24,16 @@ struct moe_hc {
   uint16_t* R;
 };
 
+// hgn v2 layers: the small-batch router launch also leaves the digit planes of rot_in(x, pre) (planes / meta [P][d/32])
+struct moe_rot_planes {
+  const float* pre;
+  uint32_t* planes;
+  float2* meta;
+};
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
-                            hipStream_t st, double* kpart, unsigned* ktickets);
+                            hipStream_t st, double* kpart, unsigned* ktickets, const moe_rot_planes* rot = nullptr);
 // scratch of the column-split router launch (5..32 tokens): fp64 partial tiles of up to 8 splits x 32 tokens
 // for at most MOE_ROUTER_KSPLIT_ROWS rows, and one ticket counter (resting at 0) per 16 rows
 constexpr int MOE_ROUTER_KSPLIT_ROWS = 1040;

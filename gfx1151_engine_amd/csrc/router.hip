@@ -1,6 +1,7 @@
 // Router: logits with the CPU path's fp64 accumulation, fp64 softmax, top-k, renormalised weights.
 // (reference: src/ref.cpp:68-77,565-594; src/gpu/parts/20_kernels_gemv.inc:1433-1562)
 #include "common.h"
+#include "hv2.h"
 #include "internal.h"
 #include "qvec.h"
 #include "topk.h"
@@ -192,6 +193,44 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
   if (do_ms && t0 + tid < P) out_xms[t0 + tid] = accms / (float)d;
 }
 
+// The blocks past the rows of the small-batch router launches: the digit planes of x for the integer-dot decode
+// kernels (a thread per 32-element group) and, for hgn v2 layers, the planes of rot_in(x, pre) = H(pre . x) / sqrt(128)
+// (a thread per 8 elements, 16 lanes per 128-block) -- work that rides along instead of costing a launch.
+// q = index among these blocks, bs = block size.
+__device__ __forceinline__ void router_plane_blocks(int q, int bs, int tid, const float* __restrict__ x, int P, int d,
+                                                    uint32_t* __restrict__ planes, float2* __restrict__ meta,
+                                                    bool planes_natural, const moe_rot_planes& R) {
+  const int G = d / 32, gb = (G + bs - 1) / bs;
+  const int nq = planes ? P * gb : 0;
+  if (q < nq) {
+    const int t = q / gb, g = (q % gb) * bs + tid;
+    if (t < P && g < G) {
+      if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);  // Q4_K kernels
+      else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);                       // q4cp kernels
+    }
+    return;
+  }
+  if (!R.planes) return;
+  q -= nq;
+  const int per_row = d / 8, rb = (per_row + bs - 1) / bs;
+  const int t = q / rb, c8 = (q % rb) * bs + tid;
+  const bool live = t < P && c8 < per_row;  // (whole groups of 16 lanes: d % 128 == 0)
+  float v[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] = 0.f;
+  if (live) {
+    const float4* xp = (const float4*)(x + (size_t)t * d + 8 * c8);
+    const float4* pp = (const float4*)(R.pre + 8 * c8);
+    const float4 a = xp[0], b = xp[1], e = pp[0], f = pp[1];
+    v[0] = a.x * e.x; v[1] = a.y * e.y; v[2] = a.z * e.z; v[3] = a.w * e.w;
+    v[4] = b.x * f.x; v[5] = b.y * f.y; v[6] = b.z * f.z; v[7] = b.w * f.w;
+  }
+  moe_fwht128_r8(v, tid);
+#pragma unroll
+  for (int i = 0; i < 8; i++) v[i] *= MOE_RS128;
+  moe_st8_planes(v, tid, R.planes, R.meta, (size_t)t * G + (c8 >> 2), live);
+}
+
 // ---- lane-parallel order for small P: one wave per weight row (four rows per block), lanes stride
 // the columns, four independent fp64 chains per lane and token, fixed combination order.  The fp64
 // sum differs from the sequential one only in its last bits, so the f32 logit differs with
@@ -211,7 +250,7 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
                                                       int nrows, uint32_t* __restrict__ planes,
                                                       float2* __restrict__ meta, bool planes_natural,
                                                       unsigned* counter, int* __restrict__ ids,
-                                                      float* __restrict__ ws, int k, int id_stride) {
+                                                      float* __restrict__ ws, int k, int id_stride, moe_rot_planes rot) {
   __shared__ int s_last;
   // the wave index as a scalar: row, weight type and base address are then wave-uniform values
   // and the bf16 / f32 choice below is a scalar branch, not a divergent one around every load
@@ -219,12 +258,7 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
   const int rpb = blockDim.x >> 6;  // rows per block: one per wave
   const int nrb = (nrows + rpb - 1) / rpb;
   if ((int)blockIdx.x >= nrb) {
-    const int G = d / 32, gb = (G + (int)blockDim.x - 1) / (int)blockDim.x;
-    const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * blockDim.x + threadIdx.x;
-    if (t < P && g < G) {
-      if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);  // Q4_K kernels
-      else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);                       // q4cp kernels
-    }
+    router_plane_blocks((int)blockIdx.x - nrb, (int)blockDim.x, (int)threadIdx.x, x, P, d, planes, meta, planes_natural, rot);
     return;
   }
   const int row = blockIdx.x * rpb + wv;
@@ -311,17 +345,12 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
                                                     const float* __restrict__ x, int P, int E, int d,
                                                     float* __restrict__ logits, float* __restrict__ out_x,
                                                     int nrows, uint32_t* __restrict__ planes,
-                                                    float2* __restrict__ meta, bool planes_natural) {
+                                                    float2* __restrict__ meta, bool planes_natural, moe_rot_planes rot) {
   __shared__ __attribute__((aligned(16))) double Xd[2][PMAX][RM_C];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int nrb = (nrows + 3) >> 2;
   if ((int)blockIdx.x >= nrb) {
-    const int G = d / 32, gb = (G + 255) / 256;
-    const int q = blockIdx.x - nrb, t = q / gb, g = (q % gb) * 256 + tid;
-    if (t < P && g < G) {
-      if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
-      else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
-    }
+    router_plane_blocks((int)blockIdx.x - nrb, 256, tid, x, P, d, planes, meta, planes_natural, rot);
     return;
   }
   // the wave's row as scalar values: the bf16 / f32 choice is then a scalar branch
@@ -464,18 +493,13 @@ __global__ void __launch_bounds__(512, 2) k_router_mfma(const void* __restrict__
                                                         float* __restrict__ logits, float* __restrict__ out_x,
                                                         int nrows, uint32_t* __restrict__ planes,
                                                         float2* __restrict__ meta, bool planes_natural, int KS,
-                                                        double* gpart, unsigned* tickets) {
+                                                        double* gpart, unsigned* tickets, moe_rot_planes rot) {
   __shared__ double part[8][NTT][64][4];
   __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int nrt = (nrows + 15) >> 4;
   if ((int)blockIdx.x >= nrt * KS) {
-    const int G = d / 32, gb = (G + 511) / 512;
-    const int q = blockIdx.x - nrt * KS, t = q / gb, g = (q % gb) * 512 + tid;
-    if (t < P && g < G) {
-      if (planes_natural) qvec_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
-      else qvec4_group_from_f32(x, (uint64_t)d, G, t, g, planes, meta);
-    }
+    router_plane_blocks((int)blockIdx.x - nrt * KS, 512, tid, x, P, d, planes, meta, planes_natural, rot);
     return;
   }
   const int rg = (int)blockIdx.x % nrt, ks = (int)blockIdx.x / nrt;  // row group, column split
@@ -648,8 +672,13 @@ int moe_router_logits_seq_if(const moe_wview* W, const float* bias, const moe_wv
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
-                            hipStream_t st, double* kpart, unsigned* ktickets) {
+                            hipStream_t st, double* kpart, unsigned* ktickets, const moe_rot_planes* rotp) {
   const int E = (int)W->rows, d = (int)W->cols;
+  moe_rot_planes rot{nullptr, nullptr, nullptr};
+  if (rotp) {  // hgn v2: the planes of rot_in(x, pre) in the same launch
+    if (!rotp->pre || !rotp->planes || !rotp->meta || d % 128 || !moe_aligned(rotp->pre, 16) || !moe_aligned(x, 16)) return MOE_E_INVALID;
+    rot = *rotp;
+  }
   // The f64 matrix pipe kernel (d a multiple of 128, one weight format).  With the caller's scratch for
   // partial tiles the columns are split over up to eight blocks per 16 rows and it serves 5..32 tokens;
   // without it one block per 16 rows leaves most CUs idle (38 us at 32 tokens), which only beats
@@ -669,13 +698,18 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
     const int P0 = 16, G = d / 32;
     const size_t pdw = planes_natural ? QV_GROUP_DW : QV4_GROUP_DW;
     int rc = moe_router_logits_small(W, bias, Wx, x, P0, logits, out_x, planes, meta, planes_natural, nullptr, nullptr,
-                                     nullptr, k, id_stride, nullptr, st, nullptr, nullptr);
+                                     nullptr, k, id_stride, nullptr, st, nullptr, nullptr, rotp);
     if (rc) return rc;
     if (fused_topk) *fused_topk = false;
+    moe_rot_planes rot2 = rot;
+    if (rotp) {
+      rot2.planes += (size_t)P0 * G * QV4_GROUP_DW;
+      rot2.meta += (size_t)P0 * G;
+    }
     return moe_router_logits_small(W, bias, Wx, x + (size_t)P0 * d, P - P0, logits + (size_t)P0 * E,
                                    out_x ? out_x + P0 : nullptr, planes ? planes + (size_t)P0 * G * pdw : nullptr,
                                    meta ? meta + (size_t)P0 * G : nullptr, planes_natural, nullptr, nullptr, nullptr, k,
-                                   id_stride, nullptr, st, nullptr, nullptr);
+                                   id_stride, nullptr, st, nullptr, nullptr, rotp ? &rot2 : nullptr);
   }
   const bool bf = W->dtype == MOE_DT_BF16;
   const bool xbf = Wx && Wx->dtype == MOE_DT_BF16;
@@ -686,10 +720,10 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   // one token, no top-k in this launch: two rows per block so that the rows cover every CU
   // (the fused top-k needs its 256 threads)
   const int bs = (P == 1 && !fuse && E <= 512) ? 128 : 256, rpb = bs / 64;
-  const int qblocks = planes ? P * ((d / 32 + bs - 1) / bs) : 0;
+  const int qblocks = (planes ? P * ((d / 32 + bs - 1) / bs) : 0) + (rot.planes ? P * ((d / 8 + bs - 1) / bs) : 0);
   dim3 g((nrows + rpb - 1) / rpb + qblocks);
   const void* wx = Wx ? Wx->data : nullptr;
-#define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, bs, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride)
+#define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, bs, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride, rot)
   if (P == 1 && E <= 512) {
     if (bf) RSM_GO(true, 1, 8); else RSM_GO(false, 1, 8);
   } else if (P <= 4) {
@@ -698,9 +732,9 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   } else {
     if (mfma_ok) {
       // the f64 matrix pipe: 16 rows per block, columns split over KS blocks and their eight waves
-      const int qb = planes ? P * ((d / 32 + 511) / 512) : 0;
+      const int qb = (planes ? P * ((d / 32 + 511) / 512) : 0) + (rot.planes ? P * ((d / 8 + 511) / 512) : 0);
       dim3 gx((nrows + 15) / 16 * KS + qb);
-#define RX_GO(BF, NTT, RD) k_router_mfma<BF, NTT, RD><<<gx, 512, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, KS, kpart, ktickets)
+#define RX_GO(BF, NTT, RD) k_router_mfma<BF, NTT, RD><<<gx, 512, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, KS, kpart, ktickets, rot)
       const int nit = d / (8 * KS) / 16;  // ring steps a wave walks
       if (nit <= 3) {
         if (P <= 16) { if (bf) RX_GO(true, 1, 3); else RX_GO(false, 1, 3); }
@@ -713,7 +747,7 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
       MOE_LAUNCH_CHECK();
       return MOE_OK;
     }
-#define RMD_GO(BF, PM) k_router_mid<BF, PM><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural)
+#define RMD_GO(BF, PM) k_router_mid<BF, PM><<<g, 256, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, rot)
     if (P <= 8) { if (bf) RMD_GO(true, 8); else RMD_GO(false, 8); }
     else if (P <= 16) { if (bf) RMD_GO(true, 16); else RMD_GO(false, 16); }
     else { if (bf) RMD_GO(true, 24); else RMD_GO(false, 24); }  // P <= 24 (larger batches were split above)
