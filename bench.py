@@ -263,7 +263,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
                     "up_kernel_ms": round(up_marginal_ms, 5),
                     "hbm_frac": round(step_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                     "tokens_per_s": round(T / (ms * 1e-3), 1),
-                    "roofline": {"bound": "hbm", "kernel": "gate/up GEMV + SwiGLU",
+                    "roofline": {"bound": "hbm", "kernel": ("gate | up GEMV in the rotated domain (sums left unfused)"
+                                                             if fmt == "i4r" else "gate/up GEMV + SwiGLU"),
                                  "achieved": round(gu_bytes / up_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                  "frac": round(gu_bytes / up_s / 1e9 / HBM_PEAK_GBS, 4),
                                  "timing": "step loop minus the same loop without this launch, HIP events around the "
