@@ -69,15 +69,26 @@ def test_resident_stack_of_48_layers_one_token(oracle):
     m.close()
 
 
-@pytest.mark.parametrize("fmt,T", [("q4cp", 16384), ("q4k", 8192), ("q4cp", 3001)])
+# "ggmix": the GGUF type mix of the reference's checkpoints (Q5_K gate/up, Q8_0 down, Q8_0 shared expert);
+# "i4r": hgn v2 rotated experts with a q4cp shared expert
+GG_MIX = (13, 8, 8)
+
+
+def _device_layer(W, seed, fmt):
+    if fmt == "ggmix":
+        return W.DeviceLayer(seed, D, MID, E, K, "q4k", gg_types=GG_MIX)
+    return W.DeviceLayer(seed, D, MID, E, K, fmt)
+
+
+@pytest.mark.parametrize("fmt,T", [("q4cp", 16384), ("q4k", 8192), ("q4cp", 3001), ("ggmix", 8192), ("i4r", 16384)])
 def test_prefill_chunk_at_full_token_count(oracle, fmt, T):
-    """The prefill configurations themselves (T = 16384 q4cp, T = 8192 Q4_K; 3001 for a ragged batch), Zipf-skewed
-    routing.  Whole batch: ids distinct and in range, weights descending with sum 1, the skew is there, every output
+    """The prefill configurations themselves (T = 16384 q4cp, T = 8192 Q4_K; 3001 for a ragged batch; the same
+    chunks for the Q5_K / Q8_0 mix and for hgn v2 rotated experts), Zipf-skewed routing.  Whole batch: ids distinct and in range, weights descending with sum 1, the skew is there, every output
     finite, and each token's result is independent of its position in the batch (the reversed batch gives the
     reversed output bit for bit).  Oracle on a sample: ids and weights bit-exact, output within 2e-3."""
     import torch
     from gfx1151_engine_amd import capi, workloads as W
-    L = W.DeviceLayer(5151 + T, D, MID, E, K, fmt)
+    L = _device_layer(W, 5151 + T, fmt)
     g = torch.Generator(device="cuda")
     g.manual_seed(T)
     x = torch.randn((T, D), device="cuda", generator=g).to(torch.bfloat16).to(torch.float32)

@@ -55,13 +55,15 @@ def test_full_size_layer(oracle, fmt, T):
     m.close()
 
 
-@pytest.mark.parametrize("fmt,tol", [("q4cp", 2e-4), ("q4k", 5e-4)])
+@pytest.mark.parametrize("fmt,tol", [("q4cp", 2e-4), ("q4k", 5e-4), ("ggmix", 5e-4), ("i4r", 2e-4)])
 def test_full_size_decode_rotating_tokens(oracle, fmt, tol):
     """T=1 over several tokens of one full-size layer (E = 512: the top-k inside the gate/up launch at its
     real width): ids and router weights bit-exact, output within the integer-dot kernels' tolerance."""
     import torch
     from gfx1151_engine_amd import capi, workloads as W
-    L = W.DeviceLayer(777, D, MID, E, K, fmt)
+    # "ggmix": Q5_K gate/up, Q8_0 down, Q8_0 shared expert (the reference checkpoints' mix); "i4r": hgn v2 experts
+    L = W.DeviceLayer(777, D, MID, E, K, "q4k", gg_types=(13, 8, 8)) if fmt == "ggmix" else \
+        W.DeviceLayer(777, D, MID, E, K, fmt)
     m = capi.Moe(D, MID, E, K, layers=1, max_tokens=1)
     L.register(m, 0)
     ol = oracle.layer_from_device(L)
