@@ -26,6 +26,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 D, MID, E, K = 3072, 768, 512, 10
 LIB_OPTIONS = []              # (option id, value) pairs of --opt, applied to every context
+GG_MIX_TYPES = None           # --gg-types: ggml types (gate/up, down, shared expert) of the ggmix_* workloads
 CPU_BUDGET_S = 12.0            # the cpu_baseline leg stops starting new work after this long
 # Counters cannot be read from inside this process: the HBM bytes per launch of the dominant kernel (read + written)
 # come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries under profiles/ (the table's "total MB" column of
@@ -109,7 +110,7 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     # v2_*: hgn v2 layer (Hadamard-rotated i4r routed experts, q4cp shared expert)
     ggmix = wl.startswith("ggmix_")
     fmt = "q4k" if wl.startswith("q4k") or ggmix else "i4r" if wl.startswith("v2_") else "q4cp"
-    gg_types = (13, 8, 8) if ggmix else (12, 12, 12)
+    gg_types = (GG_MIX_TYPES or (13, 8, 8)) if ggmix else (12, 12, 12)
     kind = wl.replace("q4k_", "").replace("ggmix_", "").replace("v2_", "")
     T = tokens or {"prefill": 16384 if fmt in ("q4cp", "i4r") else 8192, "decode": 1, "verify": 20, "stack": 1}[kind]
     nlayers = nlayers_arg if kind == "stack" else 1
@@ -212,7 +213,8 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
            "format": ("q4cp g32, the reference converter's universal expert codebook (table look-up, f32 GEMV kernels)"
                       if universal else "q4cp g32 zero-point 8") if fmt == "q4cp" else
            "hgn v2 i4r g128, Hadamard-rotated (q4cp shared expert)" if fmt == "i4r" else
-           ("GGUF Q5_K gate/up, Q8_0 down, Q8_0 shared expert" if ggmix else "GGUF Q4_K"),
+           (("GGUF ggml types %d gate/up, %d down, %d shared expert" % gg_types if GG_MIX_TYPES else
+             "GGUF Q5_K gate/up, Q8_0 down, Q8_0 shared expert") if ggmix else "GGUF Q4_K"),
            "layers": nlayers, **extra}
     if kind == "prefill":
         flop_tok = k * 6 * d * mid + 6 * d * mid + 2 * d * E + 2 * d
@@ -355,10 +357,17 @@ def main():
                     help="q4cp workloads: the benchmark's zero-point-8 grid, or the non-uniform 16-entry table that the "
                          "reference's converter writes into its checkpoints")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--gg-types", default="", metavar="GU,DN,SH",
+                    help="ggmix_* workloads: ggml types of gate/up, down and the shared expert (default 13,8,8)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies (a kernel of known HBM traffic to scale "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters by)")
     a = ap.parse_args()
+    if a.gg_types:
+        global GG_MIX_TYPES
+        GG_MIX_TYPES = tuple(int(v) for v in a.gg_types.split(","))
+        if len(GG_MIX_TYPES) != 3:
+            ap.error("--gg-types takes three ggml type numbers")
     LIB_OPTIONS.extend(tuple(int(v) for v in o.split("=")) for o in a.opt)
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (the path has no multi-GPU part); use --gpus 1", file=sys.stderr)

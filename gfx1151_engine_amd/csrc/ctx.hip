@@ -775,11 +775,12 @@ static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, floa
 struct GgKinds {
   bool r_gu, r_dn, s_gu, s_dn;  // tuned? (routed gate/up, routed down, shared gate/up, shared down)
   bool any_tuned() const { return r_gu || s_gu; }
-  // routed and shared tiles can share a launch when they take the same kernel with the same block type
+  // routed and shared tiles can share a launch when they take the same kernel with the same block type (the general
+  // kernel reads any two types in one launch, but its pipelined Q8_0 / Q5_1 forms want one type per launch)
   bool uniform(const MoeLayer& L) const {
     if (!L.has_shared) return true;
     if (L.sh_dense) return false;
-    return r_gu == s_gu && r_dn == s_dn && (!r_gu || L.gg.tgu == L.sh_gguf_type);
+    return r_gu == s_gu && r_dn == s_dn && L.gg.tgu == L.sh_gguf_type && L.gg.tdn == L.sh_gguf_type;
   }
 };
 static GgKinds gg_kinds(const MoeLayer& L, int d, int mid) {

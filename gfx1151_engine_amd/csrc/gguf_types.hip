@@ -415,16 +415,18 @@ struct GgGemmW {
   int type;
 };
 
-// Q8 = true: every tensor of the launch is Q8_0 (the reference checkpoints' down tensors and MTP sidecar).  Those launches
-// keep the raw bytes of three stages in flight in registers (a thread's 34-byte block as nine dwords from the 4-byte
-// boundary at or below it, its four activation pieces) and turn the int8 codes into f16 with byte permutes into the
-// 1024 + u form and two packed operations per pair: the plain form below waits for a trip to memory in every stage.
+// PK != 0: every tensor of the launch is Q8_0 (PK = 1) or Q5_1 (PK = 2): the reference checkpoints' down tensors and MTP
+// sidecar.  Those launches keep the raw bytes of three stages in flight in registers (a thread's block as dwords -- nine
+// from the 4-byte boundary at or below a 34-byte Q8_0 block, the six of a 24-byte Q5_1 block -- and its four activation
+// pieces) and turn the codes into f16 with byte permutes into the 1024 + u form and two packed operations per pair:
+// the plain form below waits for a trip to memory in every stage.
 constexpr int GQ_D = 3;
+constexpr int GG_PK_Q8_0 = 1, GG_PK_Q5_1 = 2;
 struct GgRawQ8 {
   uint32_t w[9];
 };
 
-template <bool UP, bool Q8 = false>
+template <bool UP, int PK = 0>
 __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, int n_experts,
                                                        const __half* __restrict__ x16, const int* __restrict__ tokidx,
                                                        const moe_tile* __restrict__ tiles,
@@ -550,16 +552,22 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
           acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
     }
   };
-  if constexpr (Q8) {
+  if constexpr (PK != 0) {
     GgRawQ8 rw[GQ_D];
     uint4 ra[GQ_D][4];
     // block 2 s + half of the row: 34 bytes; odd blocks start 2 bytes past a 4-byte boundary (rows are whole pairs of
     // blocks), so nine dwords from the boundary at or below cover the block and never pass the row's end
     auto fetch = [&](int st, GgRawQ8& r, uint4 (&a4)[4]) {
       const int sc = st < nstage ? st : nstage - 1;  // (past the end: a repeat that is never used)
-      const uint32_t* b4 = (const uint32_t*)(wrow + (size_t)(2 * sc + half) * 34 - 2 * half);
+      if constexpr (PK == GG_PK_Q8_0) {
+        const uint32_t* b4 = (const uint32_t*)(wrow + (size_t)(2 * sc + half) * 34 - 2 * half);
 #pragma unroll
-      for (int i = 0; i < 9; i++) r.w[i] = b4[i];
+        for (int i = 0; i < 9; i++) r.w[i] = b4[i];
+      } else {  // Q5_1: d | m, qh, 16 bytes of nibbles
+        const uint32_t* b4 = (const uint32_t*)(wrow + (size_t)(2 * sc + half) * 24);
+#pragma unroll
+        for (int i = 0; i < 6; i++) r.w[i] = b4[i];
+      }
 #pragma unroll
       for (int it = 0; it < 4; it++) a4[it] = *(const uint4*)(arow[it] + (size_t)sc * GG_BK);
     };
@@ -589,12 +597,48 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
         }
         *(uint4*)(rowp + (i & 7) * 16) = v;
       }
-      // d and the 32 codes: at byte 0 / 2 of the dwords (even block) or at byte 2 / 4 (odd block)
+      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+      uint8_t* dst = Bs + buf * GG_TILE_BYTES + brow * GG_PITCH + half * 64;
+      if constexpr (PK == GG_PK_Q5_1) {
+        // w = d * q + m, q = nibble | fifth bit << 4 (element j: low nibble of byte j, bit j of qh; element 16 + j: high
+        // nibble, bit 16 + j).  Four codes per dword as bytes; their fifth bits come out of qh with one multiply:
+        // (u << 4) * (1 + 2^7 + 2^14 + 2^21) puts bit i of the 4-bit field u on bit 4 of byte i (all partial products
+        // fall on distinct bits).  The f16 of d * q + m is one fused packed operation on the exact integer q.
+        union { uint16_t u; _Float16 f; } dv, mv;
+        dv.u = (uint16_t)(r.w[0] & 0xffffu);
+        mv.u = (uint16_t)(r.w[0] >> 16);
+        const h2 d2 = {dv.f, dv.f}, m2 = {mv.f, mv.f}, k1024 = {(_Float16)1024.f, (_Float16)1024.f};
+        const uint32_t qh = r.w[1];
+        uint32_t o[16];
+#pragma unroll
+        for (int cq = 0; cq < 4; cq++) {
+          const uint32_t w = r.w[2 + cq];
+          const uint32_t f_lo = (cq == 0 ? qh << 4 : qh >> (4 * cq - 4)) & 0xf0u;
+          const uint32_t f_hi = (qh >> (12 + 4 * cq)) & 0xf0u;
+          const uint32_t lo = ((f_lo * 0x204081u) & 0x10101010u) | (w & 0x0f0f0f0fu);
+          const uint32_t hi = ((f_hi * 0x204081u) & 0x10101010u) | ((w >> 4) & 0x0f0f0f0fu);
+          union { uint32_t u; h2 v; } p;
+          p.u = __builtin_amdgcn_perm(0x64646464u, lo, 0x05010400u);  // (1024 + q0, 1024 + q1)
+          p.v = (p.v - k1024) * d2 + m2;
+          o[2 * cq] = p.u;
+          p.u = __builtin_amdgcn_perm(0x64646464u, lo, 0x05030402u);
+          p.v = (p.v - k1024) * d2 + m2;
+          o[2 * cq + 1] = p.u;
+          p.u = __builtin_amdgcn_perm(0x64646464u, hi, 0x05010400u);
+          p.v = (p.v - k1024) * d2 + m2;
+          o[8 + 2 * cq] = p.u;
+          p.u = __builtin_amdgcn_perm(0x64646464u, hi, 0x05030402u);
+          p.v = (p.v - k1024) * d2 + m2;
+          o[8 + 2 * cq + 1] = p.u;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) *(uint4*)(dst + 16 * j) = make_uint4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
+        return;
+      }
+      // Q8_0: d and the 32 codes, at byte 0 / 2 of the dwords (even block) or at byte 2 / 4 (odd block)
       union { uint16_t u; _Float16 f; } dv;
       dv.u = (uint16_t)(half ? r.w[0] >> 16 : r.w[0] & 0xffffu);
-      typedef _Float16 h2 __attribute__((ext_vector_type(2)));
       const h2 d2 = {dv.f, dv.f}, k1152 = {(_Float16)1152.f, (_Float16)1152.f};
-      uint8_t* dst = Bs + buf * GG_TILE_BYTES + brow * GG_PITCH + half * 64;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         uint32_t o[4];
@@ -745,16 +789,23 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
   if (!attr_done) {
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
-    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
-    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, GG_PK_Q8_0>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_Q8_0>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, GG_PK_Q5_1>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_Q5_1>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     attr_done = true;
   }
-  // all-Q8_0 launches (4-byte aligned rows: whole pairs of 34-byte blocks from a 4-byte aligned base)
-  const bool q8 = type == MOE_GGML_Q8_0 && (!sh_w || tsh == MOE_GGML_Q8_0) && moe_aligned(w, 4) &&
-                  (!up || moe_aligned(w_up, 4)) && (!sh_w || (moe_aligned(sh_w, 4) && (!up || moe_aligned(sh_w_up, 4))));
-  if (q8) {
-    if (up) k_moe_gemm_gg<true, true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
-    else k_moe_gemm_gg<false, true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+  // all-Q8_0 / all-Q5_1 launches (4-byte aligned rows: whole pairs of 34-byte blocks, or 24-byte blocks, from a 4-byte
+  // aligned base)
+  const bool al4 = moe_aligned(w, 4) && (!up || moe_aligned(w_up, 4)) &&
+                   (!sh_w || (moe_aligned(sh_w, 4) && (!up || moe_aligned(sh_w_up, 4))));
+  const bool one_type = !sh_w || tsh == type;
+  if (type == MOE_GGML_Q8_0 && one_type && al4) {
+    if (up) k_moe_gemm_gg<true, GG_PK_Q8_0><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+    else k_moe_gemm_gg<false, GG_PK_Q8_0><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+  } else if (type == MOE_GGML_Q5_1 && one_type && al4) {
+    if (up) k_moe_gemm_gg<true, GG_PK_Q5_1><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+    else k_moe_gemm_gg<false, GG_PK_Q5_1><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   } else if (up) k_moe_gemm_gg<true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   else k_moe_gemm_gg<false><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   MOE_LAUNCH_CHECK();
