@@ -783,23 +783,27 @@ struct GgKinds {
     return r_gu == s_gu && r_dn == s_dn && L.gg.tgu == L.sh_gguf_type && L.gg.tdn == L.sh_gguf_type;
   }
 };
-static GgKinds gg_kinds(const MoeLayer& L, int d, int mid) {
+static GgKinds gg_kinds(const MoeLayer& L, const moe_config& g) {
+  const int d = g.d, mid = g.mid;
   GgKinds k{false, false, false, false};
   if (!L.has_gguf) return k;
-  auto gu_ok = [](int t) { return t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K; };
+  // (the Q5_K form wants tensors and activation rows below 4 GB: 32-bit byte offsets)
+  auto gu_ok = [&](int t, uint64_t rows) {
+    return t == MOE_GGML_Q4_K || (t == MOE_GGML_Q5_K && moe_gemm_q5k_fits(rows, (uint64_t)g.max_tokens, d));
+  };
   const bool shapes = d % 256 == 0 && mid % 256 == 0;
-  k.r_gu = shapes && gu_ok(L.gg.tgu);
+  k.r_gu = shapes && gu_ok(L.gg.tgu, (uint64_t)g.experts * mid);
   k.r_dn = k.r_gu && L.gg.tdn == MOE_GGML_Q4_K;
   if (L.has_shared && !L.sh_dense) {
-    k.s_gu = shapes && gu_ok(L.sh_gguf_type);
+    k.s_gu = shapes && gu_ok(L.sh_gguf_type, (uint64_t)mid);
     k.s_dn = k.s_gu && L.sh_gguf_type == MOE_GGML_Q4_K;
   }
   return k;
 }
 // the order of the f16 activations a layer's grouped GEMMs read (moe_f32_to_f16's layout)
-static int batch_x16_layout(const MoeLayer& L, int d, int mid) {
+static int batch_x16_layout(const MoeLayer& L, const moe_config& g) {
   if (!L.has_gguf) return 1;
-  return gg_kinds(L, d, mid).any_tuned() ? 2 : 0;
+  return gg_kinds(L, g).any_tuned() ? 2 : 0;
 }
 
 // Router of a batch: ids / ws, the shared-expert gate logit and (if asked) the per-token mean square of x.
@@ -827,7 +831,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const bool v2 = L.has_i4r;
   if (v2 && (!c->v2_x16 || g.d % 256 || g.mid % 256)) return MOE_E_UNSUPPORTED;
   // GGUF layers: each launch on the tuned kernel where it has a form for the block type, else on the general one
-  const GgKinds kd = gg_kinds(L, g.d, g.mid);
+  const GgKinds kd = gg_kinds(L, g);
   const bool shd = L.has_shared && L.sh_dense;  // shared expert stored densely: the general GEMM, launches of its own
   const bool split = shd || (q4k && !kd.uniform(L));  // routed and shared experts in launches of their own
   if (L.has_shared && !shd && (L.sh_gguf_type != 0) != q4k) return MOE_E_UNSUPPORTED;  // one format family per layer
@@ -864,7 +868,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   prof_mark(c, 0, st);
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
   const __half* xh = c->x16_ext ? c->x16_ext : c->x16;  // f16 activations in the GEMM's order
-  const int xl = batch_x16_layout(L, g.d, g.mid);       // that order (moe_f32_to_f16's layout)
+  const int xl = batch_x16_layout(L, g);       // that order (moe_f32_to_f16's layout)
   // gate/up (+ SwiGLU) and down launches over a tile list: routed experts, with_sh: the shared expert as well
   // (tiles whose expert index is >= n_experts)
   auto gemm_up = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2) -> int {
@@ -1062,7 +1066,7 @@ MOE_API int moe_x16_layout(moe_ctx* c, int layer) {
   MoeLayer* L = layer_of(c, layer);
   if (!L) return MOE_E_INVALID;
   if (!(L->has_q4cp || L->has_gguf || L->has_i4r)) return MOE_E_STATE;
-  return batch_x16_layout(*L, c->cfg.d, c->cfg.mid);
+  return batch_x16_layout(*L, c->cfg);
 }
 
 // moe_forward for a batch whose f16 copy the caller has already made (its HC-read epilogue can write it next to

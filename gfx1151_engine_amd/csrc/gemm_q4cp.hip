@@ -26,10 +26,10 @@
 //
 // Q5 (with Q4K): raw GGUF Q5_K super-blocks (176 B: the Q4_K header, 32 bytes qh, 128 code bytes; src/gguf.h:421-441):
 // the same stages with a fifth bit per code -- bit 2jj of qh byte l for the low nibble of code byte l in stage jj of the
-// super-block, bit 2jj+1 for the high nibble.  The 32 qh bytes travel with the header (48 bytes per row and super-block
-// in the scale buffer); a lane keeps its 16 of them in registers for the four stages and ORs the bit into the
-// magic-number form of each code pair (1024 + n and 64 + n stay exact for n < 32).  The larger scale buffer leaves room
-// for one block per CU instead of two.
+// super-block, bit 2jj+1 for the high nibble.  A lane fetches the 16 qh bytes of its half of each fragment row straight
+// into registers, together with the header's load one super-block ahead (through LDS they would take 8 KB more, one
+// block per CU instead of two), keeps them for the four stages and ORs the bit into the magic-number form of each code
+// pair (1024 + n and 64 + n stay exact for n < 32).
 //
 // GS = 2: one scale per 128 columns instead of 32 (hgn v2 i4r experts, reference kI4R,
 // src/gpu/parts/27_kernels_moe_lut.inc:23-29): the four stages between two scale refreshes span exactly two scales,
@@ -154,11 +154,16 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   static_assert(!Q5 || (Q4K && NSB == 1), "Q5_K: the Q4_K stages plus a fifth bit");
   constexpr int KBLK = Q5 ? 176 : 144;   // bytes per super-block
   constexpr int KQS = Q5 ? 48 : 16;      // offset of the code bytes in it
-  constexpr int SP = Q5 ? 3 : 1;         // 16-byte pieces per row in the scale buffer (header; Q5_K: + 32 bytes qh)
+  // loads per row group behind the scale buffer's: the header's 16 bytes go to LDS; Q5_K adds two 8-byte register loads
+  // per weight fragment of the lane (its half of the row's 32 qh bytes; pairs of registers are easier to place than
+  // quadruples in a kernel this close to the register limit), issued in the same place so that the count of outstanding
+  // loads the waits rely on is the same for every wave
+  constexpr int SP = Q5 ? 1 + 2 * NF : 1;
+  static_assert(!Q5 || (WROWS / 64 + NW - 1) / NW == 1, "Q5_K: one row group per wave in the scale buffer");
   uint8_t* const A0 = smem;
   uint8_t* const W0 = smem + NBUF * A_BYTES;
   uint8_t* const S0 = W0 + NBUF * W_BYTES;
-  const float* cbs = (const float*)(S0 + NSB * S_BYTES * SP);
+  const float* cbs = (const float*)(S0 + NSB * S_BYTES);
   int* rowidx = (int*)(cbs + 32);  // cbs[16..31]: the up rows' codebook
   float* rowscale = (float*)(rowidx + BM);  // f16 range guard of each pair row (gate/up only)
   const int tid = threadIdx.x, lane = tid & 63;
@@ -205,16 +210,54 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   for (int i = 0; i < A_LOADS; i++) a_grp[i] = (A_LOADS * wv + i) % A_GROUPS;  // a_src: once the row indices are in LDS
   // codes: rows 32j..32j+31, lane -> (row 32j + lane/2, half lane%2); scales: rows 64j.., lane -> row
   const uint8_t *w_src[W_LOADS], *s_src[S_ROWG];
+  // Q5_K keeps 32-bit byte offsets from wave-uniform bases instead of per-lane pointers (the launcher checks that the
+  // tensors and the activation rows stay below 4 GB): the registers that saves are what lets two blocks share a CU.
+  // A wave's code and header rows lie in one half of the block's rows: gate rows for the first NW / 2 waves, up rows
+  // for the others.
+  uint32_t a_off[Q5 ? A_LOADS : 1], w_off[Q5 ? W_LOADS : 1], s_off = 0, qh_off0 = 0, qh_off1 = 0;
+  const uint8_t* const wave_w = Q5 ? (wv >= NW / 2 ? L.w_up : L.w) : nullptr;
+  auto wrow_off = [&](int lr) -> uint32_t {  // Q5_K gate/up: byte offset of LDS row lr's weight row in its tensor
+    int r = nb * HALF + (lr & (HALF - 1));
+    r = r < M ? r : M - 1;
+    const uint32_t grow = (uint32_t)e * (uint32_t)L.e_rows + (lr >= HALF ? (uint32_t)L.up_off : 0u) + (uint32_t)r;
+    return grow * (uint32_t)(K / 256 * KBLK);
+  };
+  if (Q5) {
 #pragma unroll
-  for (int i = 0; i < W_LOADS; i++) {
-    const uint8_t* sw;
-    wrow_ptrs(32 * (W_LOADS * wv + i) + (lane >> 1), w_src[i], sw);
-    w_src[i] += (lane & 1) * 16;
+    for (int i = 0; i < W_LOADS; i++) w_off[i] = wrow_off(32 * (W_LOADS * wv + i) + (lane >> 1)) + (lane & 1) * 16;
+    s_off = wrow_off(64 * wv + lane);
+  } else {
+#pragma unroll
+    for (int i = 0; i < W_LOADS; i++) {
+      const uint8_t* sw;
+      wrow_ptrs(32 * (W_LOADS * wv + i) + (lane >> 1), w_src[i], sw);
+      w_src[i] += (lane & 1) * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < S_ROWG; i++) {
+      const uint8_t* cw;
+      wrow_ptrs(64 * (S_ROWG * wv + i) + lane, cw, s_src[i]);
+    }
   }
+  // LDS rows of this wave's weight fragments (gate/up: NH gate + the NH matching up fragments).
+  // Q4_K gate/up with one fragment per half: hid is written in 64-element blocks whose 16-byte
+  // chunks mix elements c and 32+c, so the fragment takes rows {16q..16q+15} and {32+16q..} of
+  // its 64-row block (q = wave parity): four whole chunks per wave.
+  int wrow[NF];
 #pragma unroll
-  for (int i = 0; i < S_ROWG; i++) {
-    const uint8_t* cw;
-    wrow_ptrs(64 * (S_ROWG * wv + i) + lane, cw, s_src[i]);
+  for (int nf = 0; nf < NF; nf++) {
+    if (!UP) wrow[nf] = 32 * NF * wv + 32 * nf + n;
+    else if (Q4K && NH == 1) wrow[nf] = nf * HALF + 64 * (wv >> 1) + 16 * (wv & 1) + (n & 15) + 2 * (n & 16);
+    else wrow[nf] = (nf / NH) * HALF + 32 * NH * wv + 32 * (nf % NH) + n;
+  }
+
+  // Q5_K: the lane's half (code bytes 16 h .. 16 h + 15) of its fragment rows' 32 qh bytes, fetched into registers one
+  // super-block ahead
+  static_assert(!Q5 || (UP && NF == 2 && W_LOADS * 32 * (NW / 2) == HALF), "Q5_K: gate/up, a gate and an up fragment per wave");
+  uint2 qhn[4] = {{0u, 0u}, {0u, 0u}, {0u, 0u}, {0u, 0u}};
+  if (Q5) {
+    qh_off0 = wrow_off(wrow[0]) + 16 + 16 * h;        // fragment 0: a gate row (base L.w)
+    qh_off1 = wrow_off(wrow[NF - 1]) + 16 + 16 * h;   // fragment 1: the matching up row (base L.w_up)
   }
   const int nstage = K / BK, ngroups = K / 32;
   constexpr int NLOADS = A_LOADS + W_LOADS;  // per stage (+S_LOADS scale loads on every fourth stage)
@@ -222,21 +265,33 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   auto issue_unit = [&](int s, int u) {
     const int b = s % NBUF;
     if (u < A_LOADS) {
-      g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + a_grp[u] * 1024);
+      if (Q5) g2l16((const uint8_t*)x + (a_off[Q5 ? u : 0] + (uint32_t)s * (BK * 2)), A0 + b * A_BYTES + a_grp[u] * 1024);
+      else g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + a_grp[u] * 1024);
     } else if (u < NLOADS) {
       const int i = u - A_LOADS;
       const size_t off = Q4K ? (size_t)(s >> 2) * KBLK + KQS + (size_t)(s & 3) * 32 : (size_t)s * 32;
-      g2l16(w_src[i] + off, W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
+      if (Q5) g2l16(wave_w + (w_off[Q5 ? i : 0] + (uint32_t)off), W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
+      else g2l16(w_src[i] + off, W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
     } else {
       // 8 scales (16 B) per row for stages s..s+3; at the end of K the window is pulled back inside the row
       const int i = (u - NLOADS) / SP, pc = (u - NLOADS) % SP;  // row group, 16-byte piece of the row's record
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
-      const size_t off = Q4K ? (size_t)(s >> 2) * KBLK + 16 * pc : (size_t)g0 * 2;
-      if (GS == 2)  // the two scales of stages s..s+3 (s % 4 == 0: columns 64 s .. 64 s + 255), [row][4 B]
+      const size_t off = Q4K ? (size_t)(s >> 2) * KBLK : (size_t)g0 * 2;
+      if (Q5 && pc == 1)  // this lane's 16 qh bytes of each fragment, into registers
+        qhn[0] = *(const uint2*)(L.w + (qh_off0 + (uint32_t)off));
+      else if (Q5 && pc == 2)
+        qhn[1] = *(const uint2*)(L.w + (qh_off0 + (uint32_t)off + 8u));
+      else if (Q5 && pc == 3)
+        qhn[2] = *(const uint2*)(L.w_up + (qh_off1 + (uint32_t)off));
+      else if (Q5 && pc == 4)
+        qhn[3] = *(const uint2*)(L.w_up + (qh_off1 + (uint32_t)off + 8u));
+      else if (Q5)
+        g2l16(wave_w + (s_off + (uint32_t)off), S0 + wv * 1024);
+      else if (GS == 2)  // the two scales of stages s..s+3 (s % 4 == 0: columns 64 s .. 64 s + 255), [row][4 B]
         g2l4(s_src[i] + (size_t)s, S0 + (S_ROWG * wv + i) * 256);
       else  // piece pc of every row: a region of its own, [row][16 B]
-        g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + pc * S_BYTES + (S_ROWG * wv + i) * 1024);
+        g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + (S_ROWG * wv + i) * 1024);
     }
   };
   auto issue_a = [&](int s) {
@@ -281,18 +336,6 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
       for (int i = 0; i < 16; i++) acc[mf][nf][i] = 0.f;
 
-  // LDS rows of this wave's weight fragments (gate/up: NH gate + the NH matching up fragments).
-  // Q4_K gate/up with one fragment per half: hid is written in 64-element blocks whose 16-byte
-  // chunks mix elements c and 32+c, so the fragment takes rows {16q..16q+15} and {32+16q..} of
-  // its 64-row block (q = wave parity): four whole chunks per wave.
-  int wrow[NF];
-#pragma unroll
-  for (int nf = 0; nf < NF; nf++) {
-    if (!UP) wrow[nf] = 32 * NF * wv + 32 * nf + n;
-    else if (Q4K && NH == 1) wrow[nf] = nf * HALF + 64 * (wv >> 1) + 16 * (wv & 1) + (n & 15) + 2 * (n & 16);
-    else wrow[nf] = (nf / NH) * HALF + 32 * NH * wv + 32 * (nf % NH) + n;
-  }
-
   // Software pipeline with a hand-placed instruction order.  Inside a stage (four 16-wide K
   // steps) every MFMA of step q is followed by one "unit" of step q+1's preparation: one
   // activation fragment read from LDS, or one pair of weights dequantised (3-4 VALU ops), fenced
@@ -327,7 +370,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
     for (int nf = 0; nf < NF; nf++) {
       cw[nf] = *(const uint4*)(Wb + wrow[nf] * 32 + h * 16);
-      if (AFFINE) cw8[nf] = uint4{cw[nf].x >> 8, cw[nf].y >> 8, cw[nf].z >> 8, cw[nf].w >> 8};
+      if (AFFINE && !Q5) cw8[nf] = uint4{cw[nf].x >> 8, cw[nf].y >> 8, cw[nf].z >> 8, cw[nf].w >> 8};
       if (NSB == 1) {
         // the buffer is rewritten while its stages are still being worked on: take all four
         // stages' values when the first of them is prepared (every wave has by the next barrier;
@@ -335,7 +378,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         if (Q4K) {
           if ((s & 3) == 0) {
             hdr[nf] = *(const uint4*)(Sb + wrow[nf] * 16);
-            if (Q5) qh4[nf] = *(const uint4*)(Sb + (1 + h) * S_BYTES + wrow[nf] * 16);
+            if (Q5) qh4[nf] = uint4{qhn[2 * nf].x, qhn[2 * nf].y, qhn[2 * nf + 1].x, qhn[2 * nf + 1].y};  // (requested with the header's load, two stages ago)
           }
         } else {
           if (GS == 2) {
@@ -416,7 +459,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     const int nf = u >> 2, part = u & 3;
     const uint32_t w = q == 0 ? cw[nf].x : q == 1 ? cw[nf].y : q == 2 ? cw[nf].z : cw[nf].w;
     if (AFFINE) {
-      const uint32_t w8 = q == 0 ? cw8[nf].x : q == 1 ? cw8[nf].y : q == 2 ? cw8[nf].z : cw8[nf].w;
+      // (Q5_K shifts on the spot: it has no registers to spare for the shifted copies)
+      const uint32_t w8 = Q5 ? w >> 8 : q == 0 ? cw8[nf].x : q == 1 ? cw8[nf].y : q == 2 ? cw8[nf].z : cw8[nf].w;
       const uint32_t ws = part >= 2 ? w8 : w;
       const int ss = Q4K ? (part & 1) : 0;  // Q4_K: odd parts are the high nibbles = the stage's second sub-block
       uint32_t t;
@@ -472,6 +516,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   for (int i = 0; i < A_LOADS; i++) {
     const int m = 8 * a_grp[i] + (lane >> 3);
     a_src[i] = x + (size_t)rowidx[m] * K + (((lane & 7) ^ ((m >> 1) & 7)) << 3);
+    if (Q5) a_off[Q5 ? i : 0] = ((uint32_t)rowidx[m] * (uint32_t)K + (((lane & 7) ^ ((m >> 1) & 7)) << 3)) * 2u;
   }
 #pragma unroll
   for (int t = 0; t < AHEAD; t++)
@@ -644,13 +689,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 }
 
 template <bool UP, bool F16OUT, bool Q4K, int GS, bool Q5 = false>
-__global__ void __launch_bounds__(NT, Q5 ? 1 : WPE)
+__global__ void __launch_bounds__(NT, WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,
                 moe_hscale hs, moe_comb cmb) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES * (Q5 ? 3 : 1));
+  float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
   // contiguous run of tiles so that tiles of one expert share that XCD's L2.
   // Routed tiles and shared-expert tiles (all full) are dealt out separately, or the XCD that
@@ -754,6 +799,11 @@ bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k, int gs = 0) {
 
 }  // namespace
 
+bool moe_gemm_q5k_fits(uint64_t rows, uint64_t x_rows, int k) {
+  const uint64_t lim = (1ull << 32) - (1ull << 16);
+  return k > 0 && k % 256 == 0 && rows * (uint64_t)(k / 256 * 176) < lim && x_rows * (uint64_t)k * 2 < lim;
+}
+
 // Internal: routed + (optional) shared expert in one launch; tile.expert >= n_experts selects Sh.
 // sh_cb_up: codebook of the shared expert's up rows when they are a tensor of their own (nullptr: sh->cb).
 // q4k: the views hold raw GGUF Q4_K rows (w / w_up only) instead of q4cp planes.
@@ -763,6 +813,11 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs, bool q5k) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
   if (q5k && (!q4k || !up || comb)) return MOE_E_UNSUPPORTED;  // (Q5_K: gate/up tensors, the reference checkpoints' use of it)
+  // (Q5_K: 32-bit byte offsets into the tensors; the caller vouches for the activation rows, moe_gemm_q5k_fits)
+  if (q5k && routed && !moe_gemm_q5k_fits((uint64_t)(sh == routed ? 1 : n_experts) * (uint64_t)routed->e_rows + (uint64_t)routed->up_off + (uint64_t)m, 0, k))
+    return MOE_E_UNSUPPORTED;
+  if (q5k && sh && sh != routed && !moe_gemm_q5k_fits((uint64_t)sh->e_rows + (uint64_t)sh->up_off + (uint64_t)m, 0, k))
+    return MOE_E_UNSUPPORTED;
   if (gs != 0 && (gs != 2 || up || !f16out || q4k || sh || comb)) return MOE_E_UNSUPPORTED;
   moe_comb cmb{};
   if (comb) {  // fused combine: down launch with f32 results, out = the (zeroed) token rows
@@ -792,15 +847,14 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                                                                   m, k, nblk_n, split, hs, cmb);                 \
   } while (0)
   if (q5k) {
-    constexpr int SMEM5 = SMEM_BYTES + 2 * S_BYTES;  // header + 32 qh bytes per row: one block per CU
     static bool attr5 = false;
     if (!attr5) {
       MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<true, true, true, 0, true>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, SMEM5));
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
       attr5 = true;
     }
-    k_moe_gemm_q4cp<true, true, true, 0, true><<<grid, NT, SMEM5, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k,
-                                                                        nblk_n, split, hs, cmb);
+    k_moe_gemm_q4cp<true, true, true, 0, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out,
+                                                                             m, k, nblk_n, split, hs, cmb);
   } else if (gs == 2) {
     GEMM_LAUNCH(false, true, false, 2);
   } else if (q4k) {

@@ -56,6 +56,10 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
                          hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr, int gs = 0,
                          bool q5k = false);
+// The Q5_K form addresses weights and activations with 32-bit byte offsets: true when a tensor of `rows` rows of k
+// columns and an activation buffer of `x_rows` rows of k f16 values both stay below 4 GB (the caller of
+// moe_launch_gemm_q4cp(q5k = true) checks it; other layers take the general kernel)
+bool moe_gemm_q5k_fits(uint64_t rows, uint64_t x_rows, int k);
 int moe_gemm_tile_cap();
 int moe_launch_zero_f32(float* p, uint64_t n, hipStream_t st);
 int moe_launch_tiles_only_shared(moe_tile* tiles, int* ntiles, int E, int cap, int P, int sh_first, int* tokidx,
