@@ -716,7 +716,17 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   }
   const moe_tile tile = tiles[ti];
   const bool shared = tile.expert >= n_experts;
-  const LutDev& L = shared ? Sh : R;
+  // (field by field: a reference to one of the two argument structs would put both on the stack)
+  LutDev L;
+  L.w = shared ? Sh.w : R.w;
+  L.w_up = shared ? Sh.w_up : R.w_up;
+  L.sc = shared ? Sh.sc : R.sc;
+  L.sc_up = shared ? Sh.sc_up : R.sc_up;
+  L.cb = shared ? Sh.cb : R.cb;
+  L.cb_up = shared ? Sh.cb_up : R.cb_up;
+  L.sstride = shared ? Sh.sstride : R.sstride;
+  L.e_rows = shared ? Sh.e_rows : R.e_rows;
+  L.up_off = shared ? Sh.up_off : R.up_off;
   const int e = shared ? 0 : tile.expert;
   const int tid = threadIdx.x, lane = tid & 63;
 
