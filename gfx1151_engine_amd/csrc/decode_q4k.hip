@@ -304,6 +304,11 @@ __global__ void __launch_bounds__(256) k_dec4k_dn(Dn4kArgs A, const uint32_t* __
 //         dword grid in the first block: one v_alignbit per word), d, 32 codes; w = d q
 //   Q5_1  (24 B / 32):   two blocks = 48 bytes: fp16 d, m, 32 fifth bits, 16 code bytes (low nibbles = elements
 //         0..15, high nibbles = 16..31); w = d q + m
+//   IQ4_NL (18 B / 32):  two blocks = 36 bytes from a 4-byte boundary: fp16 d, 16 code bytes (2 bytes off the dword
+//         grid in the first block), d, 16 code bytes; w = d kv[n] with the 16-entry int8 table of src/gguf.h:376-379,
+//         looked up four codes at a time with byte permutes (iq4_lookup4): the table is four registers of constants
+//   IQ4_XS (136 B / 256): fp16 d, 8 x 6-bit sub-block scales (scales_h, scales_l), 128 code bytes; a unit = the
+//         8-byte header + the 32 code bytes of sub-blocks 2jj, 2jj+1; w = d (ls - 32) kv[n]
 // The type of a block (gate/up launch: one slot) or of a wave (down launch: the shared expert has a wave of its
 // own) is uniform, so it is one scalar branch outside the loads.  Types with more than 9 registers per row in
 // flight take the wave's eight rows in two batches of four.
@@ -314,9 +319,27 @@ template <> struct GgU<MOE_GGML_Q4_K> { uint4 c0, c1; uint32_t hw; };
 template <> struct GgU<MOE_GGML_Q5_K> { uint4 c0, c1; uint2 qh; uint32_t hw; };
 template <> struct GgU<MOE_GGML_Q8_0> { uint32_t w[17]; };
 template <> struct GgU<MOE_GGML_Q5_1> { uint4 a, b, c; };
+template <> struct GgU<MOE_GGML_IQ4_NL> { uint32_t w[9]; };
+template <> struct GgU<MOE_GGML_IQ4_XS> { uint2 hd; uint4 c0, c1; };
 
 __host__ __device__ constexpr uint64_t ggu_row_bytes(int t, uint64_t k) {
-  return t == MOE_GGML_Q4_K ? k / 256 * 144 : t == MOE_GGML_Q5_K ? k / 256 * 176 : t == MOE_GGML_Q8_0 ? k / 32 * 34 : k / 32 * 24;
+  return t == MOE_GGML_Q4_K   ? k / 256 * 144
+         : t == MOE_GGML_Q5_K ? k / 256 * 176
+         : t == MOE_GGML_Q8_0 ? k / 32 * 34
+         : t == MOE_GGML_IQ4_NL ? k / 32 * 18
+         : t == MOE_GGML_IQ4_XS ? k / 256 * 136
+                                : k / 32 * 24;
+}
+
+// kv[n] for the four 4-bit codes in the low nibbles of q's bytes (shift = 0) or in the high nibbles (shift = 4), as four
+// int8 bytes: entries 0-7 and 8-15 of the table through one byte permute each (selector = the code's low three bits),
+// then a third permute takes byte j from the first or the second result by the code's bit 3
+__device__ __forceinline__ int iq4_lookup4(uint32_t q, int shift) {
+  const uint32_t i7 = (q >> shift) & 0x07070707u;
+  const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, i7);  // -127 -104 -83 -65 | -49 -35 -22 -10
+  const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, i7);  // 1 13 25 38 | 53 69 89 113
+  const uint32_t sel = ((q >> (shift + 1)) & 0x04040404u) | 0x03020100u;
+  return (int)__builtin_amdgcn_perm(hi, lo, sel);
 }
 template <int T> constexpr int ggu_batch() { return T == MOE_GGML_Q4_K ? 8 : 4; }  // rows in flight together
 
@@ -342,6 +365,18 @@ __device__ __forceinline__ void ggu_fetch(const uint8_t* row, int ul, GgU<T>& o)
       o.w[4 * i] = v.x; o.w[4 * i + 1] = v.y; o.w[4 * i + 2] = v.z; o.w[4 * i + 3] = v.w;
     }
     o.w[16] = *(const uint32_t*)(p + 64);
+  } else if constexpr (T == MOE_GGML_IQ4_NL) {
+    const uint32_t* p = (const uint32_t*)(row + (size_t)ul * 36);
+    const u32x4_a4 v0 = *(const u32x4_a4*)p, v1 = *(const u32x4_a4*)(p + 4);
+    o.w[0] = v0.x; o.w[1] = v0.y; o.w[2] = v0.z; o.w[3] = v0.w;
+    o.w[4] = v1.x; o.w[5] = v1.y; o.w[6] = v1.z; o.w[7] = v1.w;
+    o.w[8] = p[8];
+  } else if constexpr (T == MOE_GGML_IQ4_XS) {
+    const uint8_t* sb = row + (size_t)(ul >> 2) * 136;
+    o.hd = *(const uint2*)sb;
+    const u32x4_a4 v0 = *(const u32x4_a4*)(sb + 8 + jj * 32), v1 = *(const u32x4_a4*)(sb + 24 + jj * 32);
+    o.c0 = uint4{v0.x, v0.y, v0.z, v0.w};
+    o.c1 = uint4{v1.x, v1.y, v1.z, v1.w};
   } else {
     const uint4* p = (const uint4*)(row + (size_t)ul * 48);
     o.a = p[0]; o.b = p[1]; o.c = p[2];
@@ -398,6 +433,48 @@ __device__ __forceinline__ float ggu_dot(const GgU<T>& o, int jj, const XU& x) {
     d0.u = (uint16_t)(o.w[0] & 0xffffu);
     d1.u = (uint16_t)(o.w[8] >> 16);
     return __half2float(d0.h) * x.qa * planes_val(a0, a1) + __half2float(d1.h) * x.qb * planes_val(b0, b1);
+  } else if constexpr (T == MOE_GGML_IQ4_NL || T == MOE_GGML_IQ4_XS) {
+    uint32_t qa[4], qb[4];  // the 16 code bytes of the unit's two 32-element blocks
+    float da, db;           // their scales
+    if constexpr (T == MOE_GGML_IQ4_NL) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        qa[i] = __builtin_amdgcn_alignbit(o.w[i + 1], o.w[i], 16);  // the first block's codes: 2 bytes off the dword grid
+        qb[i] = o.w[5 + i];
+      }
+      union { uint16_t u; __half h; } d0, d1;
+      d0.u = (uint16_t)(o.w[0] & 0xffffu);
+      d1.u = (uint16_t)(o.w[4] >> 16);
+      da = __half2float(d0.h);
+      db = __half2float(d1.h);
+    } else {
+      qa[0] = o.c0.x; qa[1] = o.c0.y; qa[2] = o.c0.z; qa[3] = o.c0.w;
+      qb[0] = o.c1.x; qb[1] = o.c1.y; qb[2] = o.c1.z; qb[3] = o.c1.w;
+      // sub-blocks 2jj, 2jj+1: 6-bit scales = a nibble of scales_l[jj] | two bits of scales_h << 4, minus 32
+      union { uint16_t u; __half h; } dv;
+      dv.u = (uint16_t)(o.hd.x & 0xffffu);
+      const uint32_t sh = o.hd.x >> 16, sl = (o.hd.y >> (8 * jj)) & 0xffu;
+      const int la = (int)((sl & 0xfu) | (((sh >> (4 * jj)) & 3u) << 4)) - 32;
+      const int lb = (int)((sl >> 4) | (((sh >> (4 * jj + 2)) & 3u) << 4)) - 32;
+      const float dd = __half2float(dv.h);
+      da = dd * (float)la;
+      db = dd * (float)lb;
+    }
+    int a0 = 0, a1 = 0, b0 = 0, b1 = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int al = iq4_lookup4(qa[i], 0), ah = iq4_lookup4(qa[i], 4);
+      const int bl = iq4_lookup4(qb[i], 0), bh = iq4_lookup4(qb[i], 4);
+      a0 = __builtin_amdgcn_sdot4(al, (int)x.a[0][i], a0, false);
+      a1 = __builtin_amdgcn_sdot4(al, (int)x.a[1][i], a1, false);
+      a0 = __builtin_amdgcn_sdot4(ah, (int)x.a[0][4 + i], a0, false);
+      a1 = __builtin_amdgcn_sdot4(ah, (int)x.a[1][4 + i], a1, false);
+      b0 = __builtin_amdgcn_sdot4(bl, (int)x.b[0][i], b0, false);
+      b1 = __builtin_amdgcn_sdot4(bl, (int)x.b[1][i], b1, false);
+      b0 = __builtin_amdgcn_sdot4(bh, (int)x.b[0][4 + i], b0, false);
+      b1 = __builtin_amdgcn_sdot4(bh, (int)x.b[1][4 + i], b1, false);
+    }
+    return da * x.qa * planes_val(a0, a1) + db * x.qb * planes_val(b0, b1);
   } else {  // Q5_1
     const uint32_t dw[12] = {o.a.x, o.a.y, o.a.z, o.a.w, o.b.x, o.b.y, o.b.z, o.b.w, o.c.x, o.c.y, o.c.z, o.c.w};
     float r = 0.f;
@@ -454,6 +531,8 @@ __device__ __forceinline__ void ggu_gu_rows(const uint8_t* gbase, const uint8_t*
     case MOE_GGML_Q4_K: { constexpr int T = MOE_GGML_Q4_K; CALL; } break;          \
     case MOE_GGML_Q5_K: { constexpr int T = MOE_GGML_Q5_K; CALL; } break;          \
     case MOE_GGML_Q8_0: { constexpr int T = MOE_GGML_Q8_0; CALL; } break;          \
+    case MOE_GGML_IQ4_NL: { constexpr int T = MOE_GGML_IQ4_NL; CALL; } break;      \
+    case MOE_GGML_IQ4_XS: { constexpr int T = MOE_GGML_IQ4_XS; CALL; } break;      \
     default: { constexpr int T = MOE_GGML_Q5_1; CALL; } break;                    \
   }
 
@@ -839,8 +918,11 @@ int moe_launch_dec4k_dn(const uint8_t* down, const uint8_t* sh_down, const float
   return MOE_OK;
 }
 
-// ---- any mix of Q4_K / Q5_K / Q8_0 / Q5_1 (integer-dot kernels above) ----
-static bool ggu_type(int t) { return t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K || t == MOE_GGML_Q8_0 || t == MOE_GGML_Q5_1; }
+// ---- any mix of Q4_K / Q5_K / Q8_0 / Q5_1 / IQ4_NL / IQ4_XS (integer-dot kernels above) ----
+static bool ggu_type(int t) {
+  return t == MOE_GGML_Q4_K || t == MOE_GGML_Q5_K || t == MOE_GGML_Q8_0 || t == MOE_GGML_Q5_1 || t == MOE_GGML_IQ4_NL ||
+         t == MOE_GGML_IQ4_XS;
+}
 bool moe_decgg_supported(int tgu, int tdn, int tsh, bool has_shared, int d, int mid, int kpt, int n_experts) {
   if (!ggu_type(tgu) || !ggu_type(tdn) || (has_shared && !ggu_type(tsh))) return false;
   // (whole 256-element super-blocks in both directions also cover the 64-weight units of the 32-element types)
@@ -848,7 +930,7 @@ bool moe_decgg_supported(int tgu, int tdn, int tsh, bool has_shared, int d, int 
          mid % G4_ROWS == 0 && d % D4_ROWS == 0 && ((kpt + 3) / 4 + 1) * 64 <= 320 && n_experts <= 1024 && kpt <= 64 &&
          kpt <= n_experts;
 }
-static size_t ggu_align(int t) { return t == MOE_GGML_Q8_0 ? 4 : 16; }
+static size_t ggu_align(int t) { return t == MOE_GGML_Q8_0 || t == MOE_GGML_IQ4_NL ? 4 : 16; }
 
 int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
                              const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const float* logits,

@@ -81,7 +81,8 @@ def q4k_rows(g, rows, cols, scale_std=0.01):
     return blk.view(-1)
 
 
-GG_ROW_BYTES = {12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24)}  # ggml type -> (block elements, bytes)
+GG_ROW_BYTES = {12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24),  # ggml type -> (block elements, bytes)
+                20: (32, 18), 23: (256, 136)}
 
 
 def gg_row_bytes(t, cols):
@@ -90,8 +91,8 @@ def gg_row_bytes(t, cols):
 
 
 def gg_rows(g, t, rows, cols, scale_std=0.01):
-    """uint8 tensor of raw rows of ggml type t: Q4_K (12), Q5_K (13), Q8_0 (8) or Q5_1 (7); integer fields uniform,
-    fp16 fields |N|*std scaled so that weights have the size of the Q4_K ones."""
+    """uint8 tensor of raw rows of ggml type t: Q4_K (12), Q5_K (13), Q8_0 (8), Q5_1 (7), IQ4_NL (20) or IQ4_XS (23);
+    integer fields uniform, fp16 fields |N|*std scaled so that weights have the size of the Q4_K ones."""
     if t == 12:
         return q4k_rows(g, rows, cols, scale_std)
     be, bb = GG_ROW_BYTES[t]
@@ -106,6 +107,12 @@ def gg_rows(g, t, rows, cols, scale_std=0.01):
         blk[:, 0:4] = dd.view(torch.uint8)
     elif t == 8:   # d, 32 x int8
         dd = (torch.randn((nb, 1), device="cuda", generator=g).abs() * scale_std / 8).to(torch.float16)
+        blk[:, 0:2] = dd.view(torch.uint8)
+    elif t == 20:  # IQ4_NL: d, 16 code bytes into a table of int8 values up to 127 in size
+        dd = (torch.randn((nb, 1), device="cuda", generator=g).abs() * scale_std / 8).to(torch.float16)
+        blk[:, 0:2] = dd.view(torch.uint8)
+    elif t == 23:  # IQ4_XS: d, 6-bit sub-block scales (minus 32) in scales_h / scales_l, 128 code bytes
+        dd = (torch.randn((nb, 1), device="cuda", generator=g).abs() * scale_std / 128).to(torch.float16)
         blk[:, 0:2] = dd.view(torch.uint8)
     else:          # Q5_1: d, m = -16 d, qh, qs
         dd = (torch.randn((nb, 1), device="cuda", generator=g).abs() * scale_std / 2).to(torch.float16)

@@ -186,12 +186,13 @@ def test_decode_topk_wide_logit_range(oracle, fmt):
 
 
 @pytest.mark.parametrize("tgu,tdn,tsh,T", [(13, 8, 12, 1), (12, 7, 12, 5), (13, 7, 8, 3), (12, 8, 13, 40), (23, 20, 12, 2),
-                                            (20, 23, 23, 7), (13, 8, 8, 1), (13, 8, 8, 20), (12, 7, 7, 32), (8, 13, 7, 2)])
+                                            (20, 23, 23, 7), (13, 8, 8, 1), (13, 8, 8, 20), (12, 7, 7, 32), (8, 13, 7, 2),
+                                            (20, 20, 20, 1), (23, 23, 23, 4), (23, 20, 8, 19), (12, 23, 20, 30)])
 def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
     """GGUF layers in the type mix of the reference's checkpoints (Q4_K / Q5_K gate and up, Q5_1 / Q8_0 down, a Q8_0
-    shared expert; src/gpu/parts/30_host_util.inc:399-405, src/gguf_map.h:212-214): mixes of Q4_K / Q5_K / Q8_0 /
-    Q5_1 take the integer-dot decode kernels (and, with MOE_OPT_INT_DECODE = 0, like the IQ4 types, the general f32
-    GEMV kernels); ids bit-exact; T = 40 is a batch for the general grouped GEMM."""
+    shared expert; src/gpu/parts/30_host_util.inc:399-405, src/gguf_map.h:212-214) and in the IQ4_NL / IQ4_XS types
+    (src/gguf.h:376-407): every mix takes the integer-dot decode kernels (and, with MOE_OPT_INT_DECODE = 0, the general
+    f32 GEMV kernels); ids bit-exact; T = 40 is a batch for the general grouped GEMM."""
     from gfx1151_engine_amd import capi
     rng = np.random.default_rng(tgu * 100 + tdn * 10 + T)
     d, mid, E, k = 512, 256, 12, 4
@@ -203,9 +204,8 @@ def test_gguf_mixed_types(oracle, tgu, tdn, tsh, T):
     ids, ws = m.last_routing(T)
     assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
     assert np.abs(ws.cpu().numpy()[:, :k] - wo[:, :k]).max() <= 1e-6
-    int_types = all(t in (12, 13, 8, 7) for t in (tgu, tdn, tsh))
     # batches over 32 tokens take the general grouped GEMM (f16 MFMA operands): the batch tolerance
-    tol = 2e-3 if T > 32 else (TOL_INT_Q4K if int_types else TOL_GEMV)
+    tol = 2e-3 if T > 32 else TOL_INT_Q4K
     assert max_abs_rel(y, yo) <= tol, max_abs_rel(y, yo)
     if T <= 32:
         m.set_option(capi.OPT_INT_DECODE, 0)
