@@ -9,6 +9,7 @@
 // (reference: src/gpu/parts/26_kernels_moe_gguf.inc:527-568,693-756,893-939; src/gguf.h:328-336,408-441)
 #include "common.h"
 #include "internal.h"
+#include "iq4.h"
 #include "qvec.h"
 #include "topk.h"
 
@@ -306,7 +307,7 @@ __global__ void __launch_bounds__(256) k_dec4k_dn(Dn4kArgs A, const uint32_t* __
 //         0..15, high nibbles = 16..31); w = d q + m
 //   IQ4_NL (18 B / 32):  two blocks = 36 bytes from a 4-byte boundary: fp16 d, 16 code bytes (2 bytes off the dword
 //         grid in the first block), d, 16 code bytes; w = d kv[n] with the 16-entry int8 table of src/gguf.h:376-379,
-//         looked up four codes at a time with byte permutes (iq4_lookup4): the table is four registers of constants
+//         looked up four codes at a time with byte permutes (iq4.h): the table is four registers of constants
 //   IQ4_XS (136 B / 256): fp16 d, 8 x 6-bit sub-block scales (scales_h, scales_l), 128 code bytes; a unit = the
 //         8-byte header + the 32 code bytes of sub-blocks 2jj, 2jj+1; w = d (ls - 32) kv[n]
 // The type of a block (gate/up launch: one slot) or of a wave (down launch: the shared expert has a wave of its
@@ -331,16 +332,7 @@ __host__ __device__ constexpr uint64_t ggu_row_bytes(int t, uint64_t k) {
                                 : k / 32 * 24;
 }
 
-// kv[n] for the four 4-bit codes in the low nibbles of q's bytes (shift = 0) or in the high nibbles (shift = 4), as four
-// int8 bytes: entries 0-7 and 8-15 of the table through one byte permute each (selector = the code's low three bits),
-// then a third permute takes byte j from the first or the second result by the code's bit 3
-__device__ __forceinline__ int iq4_lookup4(uint32_t q, int shift) {
-  const uint32_t i7 = (q >> shift) & 0x07070707u;
-  const uint32_t lo = __builtin_amdgcn_perm(0xF6EADDCFu, 0xBFAD9881u, i7);  // -127 -104 -83 -65 | -49 -35 -22 -10
-  const uint32_t hi = __builtin_amdgcn_perm(0x71594535u, 0x26190D01u, i7);  // 1 13 25 38 | 53 69 89 113
-  const uint32_t sel = ((q >> (shift + 1)) & 0x04040404u) | 0x03020100u;
-  return (int)__builtin_amdgcn_perm(hi, lo, sel);
-}
+__device__ __forceinline__ int iq4_lookup4(uint32_t q, int shift) { return (int)moe_iq4_lookup4<0>(q, shift); }
 template <int T> constexpr int ggu_batch() { return T == MOE_GGML_Q4_K ? 8 : 4; }  // rows in flight together
 
 template <int T>

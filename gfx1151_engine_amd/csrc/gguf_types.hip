@@ -7,6 +7,7 @@
 #include "common.h"
 #include "dense.h"
 #include "internal.h"
+#include "iq4.h"
 
 namespace {
 
@@ -415,13 +416,14 @@ struct GgGemmW {
   int type;
 };
 
-// PK != 0: every tensor of the launch is Q8_0 (PK = 1) or Q5_1 (PK = 2): the reference checkpoints' down tensors and MTP
-// sidecar.  Those launches keep the raw bytes of three stages in flight in registers (a thread's block as dwords -- nine
-// from the 4-byte boundary at or below a 34-byte Q8_0 block, the six of a 24-byte Q5_1 block -- and its four activation
-// pieces) and turn the codes into f16 with byte permutes into the 1024 + u form and two packed operations per pair:
-// the plain form below waits for a trip to memory in every stage.
+// PK != 0: every tensor of the launch is Q8_0 (PK = 1), Q5_1 (PK = 2) -- the reference checkpoints' down tensors and MTP
+// sidecar --, IQ4_NL (PK = 3) or IQ4_XS (PK = 4).  Those launches keep the raw bytes of three stages in flight in
+// registers (a thread's block as dwords -- nine from the 4-byte boundary at or below a 34-byte Q8_0 block, the six of a
+// 24-byte Q5_1 block, five around an 18-byte IQ4_NL block, an IQ4_XS super-block's header and the block's 16 code bytes
+// -- and its four activation pieces) and turn the codes into f16 with byte permutes into the 1024 + u form and two or
+// three packed operations per pair: the plain form below waits for a trip to memory in every stage.
 constexpr int GQ_D = 3;
-constexpr int GG_PK_Q8_0 = 1, GG_PK_Q5_1 = 2;
+constexpr int GG_PK_Q8_0 = 1, GG_PK_Q5_1 = 2, GG_PK_IQ4_NL = 3, GG_PK_IQ4_XS = 4;
 struct GgRawQ8 {
   uint32_t w[9];
 };
@@ -563,15 +565,26 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
         const uint32_t* b4 = (const uint32_t*)(wrow + (size_t)(2 * sc + half) * 34 - 2 * half);
 #pragma unroll
         for (int i = 0; i < 9; i++) r.w[i] = b4[i];
-      } else {  // Q5_1: d | m, qh, 16 bytes of nibbles
+      } else if constexpr (PK == GG_PK_Q5_1) {  // d | m, qh, 16 bytes of nibbles
         const uint32_t* b4 = (const uint32_t*)(wrow + (size_t)(2 * sc + half) * 24);
 #pragma unroll
         for (int i = 0; i < 6; i++) r.w[i] = b4[i];
+      } else if constexpr (PK == GG_PK_IQ4_NL) {  // 18 bytes: d, 16 bytes of nibbles; odd blocks start 2 bytes past a boundary
+        const uint32_t* b4 = (const uint32_t*)(wrow + (size_t)(2 * sc + half) * 18 - 2 * half);
+#pragma unroll
+        for (int i = 0; i < 5; i++) r.w[i] = b4[i];
+      } else {  // IQ4_XS: the super-block's d | scales_h, scales_l and sub-block (2 sc + half) % 8's 16 bytes of nibbles
+        const uint32_t* sb = (const uint32_t*)(wrow + (size_t)(sc >> 2) * 136);
+        r.w[0] = sb[0];
+        r.w[1] = sb[1];
+        const uint32_t* q4 = sb + 2 + 4 * ((2 * sc + half) & 7);
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.w[2 + i] = q4[i];
       }
 #pragma unroll
       for (int it = 0; it < 4; it++) a4[it] = *(const uint4*)(arow[it] + (size_t)sc * GG_BK);
     };
-    auto decode = [&](const GgRawQ8& r, const uint4 (&a4)[4], int buf) {
+    auto decode = [&](const GgRawQ8& r, const uint4 (&a4)[4], int buf, int stg) {
 #pragma unroll
       for (int it = 0; it < 4; it++) {
         const int i = tid + 256 * it;
@@ -635,6 +648,57 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
         for (int j = 0; j < 4; j++) *(uint4*)(dst + 16 * j) = make_uint4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
         return;
       }
+      if constexpr (PK == GG_PK_IQ4_NL || PK == GG_PK_IQ4_XS) {
+        // w = dl * kv[n] (element j: low nibble of code byte j, element 16 + j: its high nibble), dl = d (IQ4_NL) or
+        // d * (ls - 32) with the sub-block's 6-bit scale ls (IQ4_XS).  kv + 128 comes out of the register table as
+        // bytes, becomes the f16 1024 + u by a byte permute, and (u - 128) * dl is a packed f16 product: the f16 of the
+        // exact product for IQ4_NL; for IQ4_XS dl (17 significant bits) goes in as an f16 pair hi + lo with
+        // fma(kv, hi, kv * lo), whose only early rounding is in the 2^-11 times smaller term.
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        uint32_t qd[4];
+        h2 dh, dlo = {(_Float16)0.f, (_Float16)0.f};
+        if constexpr (PK == GG_PK_IQ4_NL) {
+          union { uint16_t u; _Float16 f; } dv;
+          dv.u = (uint16_t)(half ? r.w[0] >> 16 : r.w[0] & 0xffffu);
+          dh = h2{dv.f, dv.f};
+#pragma unroll
+          for (int i = 0; i < 4; i++) qd[i] = half ? r.w[i + 1] : __builtin_amdgcn_alignbit(r.w[i + 1], r.w[i], 16);
+        } else {
+          union { uint16_t u; _Float16 f; } dv;
+          dv.u = (uint16_t)(r.w[0] & 0xffffu);
+          const uint32_t sh = r.w[0] >> 16;
+          const int sub = (2 * stg + half) & 7;  // sub-block within the super-block
+          const uint32_t slb = (r.w[1] >> (8 * (sub >> 1))) & 0xffu;
+          const int ls = (int)(((sub & 1) ? slb >> 4 : slb & 0xfu) | (((sh >> (2 * sub)) & 3u) << 4)) - 32;
+          const float dl = (float)dv.f * (float)ls;  // exact in f32
+          const _Float16 hi = (_Float16)dl, lo = (_Float16)(dl - (float)hi);
+          dh = h2{hi, hi};
+          dlo = h2{lo, lo};
+#pragma unroll
+          for (int i = 0; i < 4; i++) qd[i] = r.w[2 + i];
+        }
+        const h2 k1152 = {(_Float16)1152.f, (_Float16)1152.f};
+        uint32_t o[16];
+#pragma unroll
+        for (int cq = 0; cq < 4; cq++) {
+#pragma unroll
+          for (int hn = 0; hn < 2; hn++) {  // low nibbles: elements 4 cq .. 4 cq + 3; high nibbles: 16 + the same
+            const uint32_t ub = moe_iq4_lookup4<128>(qd[cq], 4 * hn);
+#pragma unroll
+            for (int l = 0; l < 2; l++) {
+              union { uint32_t u; h2 v; } p;
+              p.u = __builtin_amdgcn_perm(0x64646464u, ub, l ? 0x05030402u : 0x05010400u);
+              const h2 kv = p.v - k1152;
+              if constexpr (PK == GG_PK_IQ4_NL) p.v = kv * dh;
+              else p.v = kv * dh + kv * dlo;
+              o[8 * hn + 2 * cq + l] = p.u;
+            }
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) *(uint4*)(dst + 16 * j) = make_uint4(o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]);
+        return;
+      }
       // Q8_0: d and the 32 codes, at byte 0 / 2 of the dwords (even block) or at byte 2 / 4 (odd block)
       union { uint16_t u; _Float16 f; } dv;
       dv.u = (uint16_t)(half ? r.w[0] >> 16 : r.w[0] & 0xffffu);
@@ -659,7 +723,7 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
     };
 #pragma unroll
     for (int i = 0; i < GQ_D; i++) fetch(i, rw[i], ra[i]);
-    decode(rw[0], ra[0], 0);
+    decode(rw[0], ra[0], 0, 0);
     __syncthreads();
     for (int s0 = 0; s0 < nstage; s0 += GQ_D) {
 #pragma unroll
@@ -670,7 +734,7 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
           // stage s is in LDS; the registers hold stages s + 1 and s + 2; slot u takes stage s + 3
           fetch(s + GQ_D, rw[u], ra[u]);
           mfmas(buf);
-          if (s + 1 < nstage) decode(rw[(u + 1) % GQ_D], ra[(u + 1) % GQ_D], buf ^ 1);
+          if (s + 1 < nstage) decode(rw[(u + 1) % GQ_D], ra[(u + 1) % GQ_D], buf ^ 1, s + 1);
           __syncthreads();
         }
       }
@@ -793,6 +857,10 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_Q8_0>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, GG_PK_Q5_1>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_Q5_1>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, GG_PK_IQ4_NL>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_IQ4_NL>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, GG_PK_IQ4_XS>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
+    MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_IQ4_XS>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     attr_done = true;
   }
   // all-Q8_0 / all-Q5_1 launches (4-byte aligned rows: whole pairs of 34-byte blocks, or 24-byte blocks, from a 4-byte
@@ -806,6 +874,12 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
   } else if (type == MOE_GGML_Q5_1 && one_type && al4) {
     if (up) k_moe_gemm_gg<true, GG_PK_Q5_1><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
     else k_moe_gemm_gg<false, GG_PK_Q5_1><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+  } else if (type == MOE_GGML_IQ4_NL && one_type && al4) {
+    if (up) k_moe_gemm_gg<true, GG_PK_IQ4_NL><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+    else k_moe_gemm_gg<false, GG_PK_IQ4_NL><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+  } else if (type == MOE_GGML_IQ4_XS && one_type && al4) {
+    if (up) k_moe_gemm_gg<true, GG_PK_IQ4_XS><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
+    else k_moe_gemm_gg<false, GG_PK_IQ4_XS><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   } else if (up) k_moe_gemm_gg<true><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   else k_moe_gemm_gg<false><<<grid, 256, GG_SMEM, st>>>(R, S, n_experts, x16, tokidx, tiles, ntiles, out, m, k, hs, a_layout);
   MOE_LAUNCH_CHECK();

@@ -296,7 +296,8 @@ def test_forward_with_the_callers_f16_copy(oracle, fmt):
                                                   (23, 20, 12, 512, 256, 90), (20, 23, 23, 256, 256, 40), (8, 8, 8, 512, 64, 100),
                                                   (13, 8, 12, 3072, 768, 200), (13, 8, 8, 3072, 768, 300), (13, 13, 13, 512, 256, 130),
                                                   (13, 12, 13, 768, 512, 260), (8, 12, 13, 512, 256, 97), (8, 7, 8, 320, 64, 50),
-                                                  (7, 7, 7, 512, 256, 140), (13, 7, 7, 3072, 768, 300)])
+                                                  (7, 7, 7, 512, 256, 140), (13, 7, 7, 3072, 768, 300),
+                                                  (20, 20, 20, 768, 256, 170), (23, 23, 23, 3072, 768, 200), (23, 20, 23, 512, 512, 77)])
 def test_batch_layer_other_gguf_types(oracle, tgu, tdn, tsh, d, mid, T):
     """GGUF layers whose tensors are not Q4_K throughout (the reference checkpoints' Q5_K gate/up with Q5_1 / Q8_0
     down, IQ4 types, a Q8_0 MTP sidecar; src/gpu/parts/26_kernels_moe_gguf.inc:81-386): Q4_K / Q5_K gate/up and Q4_K down
