@@ -38,7 +38,8 @@ enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_F16 = 2, MOE_DT_Q4CP = 5, MOE_DT_
        MOE_DT_I4R = 23 };
 /* Q4_K: every kernel of the path.  Q5_K (gate/up), Q5_1 and Q8_0 (down) — the mix of the reference's GGUF
  * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — and IQ4_NL / IQ4_XS (src/gguf.h:376-407):
- * dequantisation and the general GEMV kernels. */
+ * bit-exact dequantisation, the stateless general GEMV kernels (moe_gg_gemv), and inside moe_forward integer-dot
+ * decode kernels and grouped GEMMs for any mix of the six. */
 enum { MOE_GGML_Q5_1 = 7, MOE_GGML_Q8_0 = 8, MOE_GGML_Q4_K = 12, MOE_GGML_Q5_K = 13, MOE_GGML_IQ4_NL = 20,
        MOE_GGML_IQ4_XS = 23 };
 
