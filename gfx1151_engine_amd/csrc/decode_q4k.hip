@@ -311,8 +311,8 @@ __global__ void __launch_bounds__(256) k_dec4k_dn(Dn4kArgs A, const uint32_t* __
 //   IQ4_XS (136 B / 256): fp16 d, 8 x 6-bit sub-block scales (scales_h, scales_l), 128 code bytes; a unit = the
 //         8-byte header + the 32 code bytes of sub-blocks 2jj, 2jj+1; w = d (ls - 32) kv[n]
 // The type of a block (gate/up launch: one slot) or of a wave (down launch: the shared expert has a wave of its
-// own) is uniform, so it is one scalar branch outside the loads.  Types with more than 9 registers per row in
-// flight take the wave's eight rows in two batches of four.
+// own) is uniform, so it is one scalar branch outside the loads.  A wave's eight rows are fetched in two batches of
+// four.
 typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 template <int T> struct GgU;
@@ -333,7 +333,9 @@ __host__ __device__ constexpr uint64_t ggu_row_bytes(int t, uint64_t k) {
 }
 
 __device__ __forceinline__ int iq4_lookup4(uint32_t q, int shift) { return (int)moe_iq4_lookup4<0>(q, shift); }
-template <int T> constexpr int ggu_batch() { return T == MOE_GGML_Q4_K ? 8 : 4; }  // rows in flight together
+// rows in flight together: four (eight Q4_K rows of nine registers spill next to the kernel's other state and measured
+// 1.4 us slower per token than two batches of four)
+template <int T> constexpr int ggu_batch() { return 4; }
 
 template <int T>
 __device__ __forceinline__ void ggu_fetch(const uint8_t* row, int ul, GgU<T>& o) {
