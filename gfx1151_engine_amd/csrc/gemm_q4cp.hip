@@ -595,38 +595,61 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   constexpr int NC = UP ? 32 * NH : 32 * NF;  // output columns of this wave
   constexpr int LDP = NC * 2 + 16;            // padded row pitch of the patch in bytes
   const int colbase = UP ? nb * HALF + NC * wv : nb * WROWS + NC * wv;
-  if (UP || F16OUT) {
+  if (UP) {
+    // gate/up: a wave holds 32 of the block's HALF hid columns, 64 bytes of a row -- stored per wave, the two halves of
+    // a 128-byte line reach memory separately (measured: 2.3 times the payload written).  So the block's waves put
+    // their columns into one patch of whole rows and every store instruction writes complete lines.
+    constexpr int BP = HALF * 2 + 16;  // row pitch of the block-wide patch in bytes
+    uint8_t* patch = smem;
+#pragma unroll
+    for (int mf = 0; mf < MF; mf++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
+#pragma unroll
+        for (int f = 0; f < NH; f++) {
+          const float g = acc[mf][f][r], u = acc[mf][NH + f][r];
+          // hardware reciprocal (1 ulp) instead of the IEEE division sequence: the result is rounded
+          // to f16 below, and this epilogue is VALU time during which the matrix pipe idles
+          const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
+          // hid feeds the down GEMM: permuted order inside groups of 8 (q4cp) / blocks of 64 (Q4_K)
+          int pos;
+          if (!Q4K) {
+            const int c = 32 * f + n;
+            pos = (c & ~7) + ilv_pos(c & 7);
+          } else if (NH == 1) {
+            // lane n holds row 16q + (n&15) + 2*(n&16) of the block: chunks 4q..4q+3 -> local 0..31
+            pos = q4k_pos((n & 15) + 2 * (n & 16));
+          } else {
+            pos = q4k_pos(32 * f + n);
+          }
+          *(__half*)(patch + (32 * mf + ml) * BP + (NC * wv + pos) * 2) = __float2half(hv);
+        }
+      }
+    }
+    __syncthreads();
+    constexpr int CH = HALF / 8;  // 16-byte chunks per row
+#pragma unroll
+    for (int it = 0; it < (32 * MF * CH + NT - 1) / NT; it++) {
+      const int c = it * NT + tid, m = c / CH, c8 = c % CH;
+      if (c < 32 * MF * CH) {
+        const uint4 v = *(const uint4*)(patch + m * BP + c8 * 16);
+        const int col = nb * HALF + c8 * 8;
+        if (m < tile.count && col < M) *(uint4*)((__half*)out + (size_t)(tile.first + m) * M + col) = v;
+      }
+    }
+  } else if (F16OUT) {
+    // down: a wave's 64 columns are whole 128-byte lines of a row; a per-wave patch turns the accumulators' layout into
+    // 16-byte stores
     uint8_t* patch = smem + wv * (32 * LDP);
 #pragma unroll
     for (int mf = 0; mf < MF; mf++) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
-        if (UP) {
 #pragma unroll
-          for (int f = 0; f < NH; f++) {
-            const float g = acc[mf][f][r], u = acc[mf][NH + f][r];
-            // hardware reciprocal (1 ulp) instead of the IEEE division sequence: the result is rounded
-            // to f16 below, and this epilogue is VALU time during which the matrix pipe idles
-            const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
-            // hid feeds the down GEMM: permuted order inside groups of 8 (q4cp) / blocks of 64 (Q4_K)
-            int pos;
-            if (!Q4K) {
-              const int c = 32 * f + n;
-              pos = (c & ~7) + ilv_pos(c & 7);
-            } else if (NH == 1) {
-              // lane n holds row 16q + (n&15) + 2*(n&16) of the block: chunks 4q..4q+3 -> local 0..31
-              pos = q4k_pos((n & 15) + 2 * (n & 16));
-            } else {
-              pos = q4k_pos(32 * f + n);
-            }
-            *(__half*)(patch + ml * LDP + pos * 2) = __float2half(hv);
-          }
-        } else {
-#pragma unroll
-          for (int nf = 0; nf < NF; nf++)
-            *(__half*)(patch + ml * LDP + (32 * nf + n) * 2) = __float2half(acc[mf][nf][r]);
-        }
+        for (int nf = 0; nf < NF; nf++)
+          *(__half*)(patch + ml * LDP + (32 * nf + n) * 2) = __float2half(acc[mf][nf][r]);
       }
       // 32 rows x NC columns -> NC/8 16-byte chunks per row
       constexpr int CPR = NC / 8;
