@@ -313,19 +313,30 @@ __device__ __forceinline__ double chain_row(const void* wrow, const float* xrow,
 // the 8 lanes of an LDS phase then hit 8 different 16-byte bank groups.  Two images per wave (next iteration in
 // flight), waves are independent (no block barrier).  Activations come straight from global memory: the pairs of
 // a token are neighbours in the list, so a wave touches a handful of rows.
-template <bool BF16>
+// LISTED = true is step 5: the pairs are (listed token, expert) for every expert, taken from the list of tokens
+// (fb_list, counters[0] entries; nothing to do when the dense kernel takes over) instead of from the pair list.
+template <bool BF16, bool LISTED = false>
 __global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restrict__ W, const float* __restrict__ bias,
                                                             const void* __restrict__ Wx, const float* __restrict__ x,
                                                             int E, int d, const uint32_t* __restrict__ pairs,
                                                             const int* __restrict__ counters,
-                                                            float* __restrict__ logits, float* __restrict__ out_x) {
+                                                            float* __restrict__ logits, float* __restrict__ out_x,
+                                                            const int* __restrict__ fb_list = nullptr, int dense_above = 0) {
   __shared__ __attribute__((aligned(16))) uint8_t img[4][2][8192];
-  const int np = counters[1];
+  int np;
+  if (LISTED) {
+    const int nl = counters[0];
+    if (nl == 0 || nl > dense_above) return;
+    np = nl * E;
+  } else {
+    np = counters[1];
+  }
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int p0 = (blockIdx.x * 4 + wv) * 64;
   if (p0 >= np) return;
   const bool live = p0 + lane < np;
-  const uint32_t pr = pairs[live ? p0 + lane : p0];  // idle lanes repeat the wave's first pair (no extra traffic)
+  const int pi = live ? p0 + lane : p0;  // idle lanes repeat the wave's first pair (no extra traffic)
+  const uint32_t pr = LISTED ? ((uint32_t)fb_list[pi / E] << 10) | (uint32_t)(pi % E) : pairs[pi];
   const int t = (int)(pr >> 10), e = (int)(pr & 1023u);
   const bool gate = e == E;
   const uint8_t* wrow = gate ? (const uint8_t*)Wx : (const uint8_t*)W + (size_t)e * d * (BF16 ? 2 : 4);
@@ -472,25 +483,7 @@ __global__ void __launch_bounds__(256) k_router_topk_mixed(const float* __restri
   }
 }
 
-// ---- 5. listed tokens: every logit as an fp64 chain (a lane per expert), unless the dense kernel takes over ----
-template <bool BF16>
-__global__ void __launch_bounds__(256) k_router_exact_listed(const void* __restrict__ W, const float* __restrict__ bias,
-                                                             const float* __restrict__ x, int E, int d,
-                                                             const int* __restrict__ fb_list,
-                                                             const int* __restrict__ counters, int dense_above,
-                                                             float* __restrict__ logits) {
-  const int nl = counters[0];
-  if (nl == 0 || nl > dense_above) return;
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int ne64 = (E + 63) >> 6, total = nl * ne64;
-  for (int item = blockIdx.x * 4 + wv; item < total; item += gridDim.x * 4) {
-    const int t = fb_list[item / ne64], e = 64 * (item % ne64) + lane;
-    const int er = e < E ? e : 0;
-    const double acc = chain_row<BF16>((const uint8_t*)W + (size_t)er * d * (BF16 ? 2 : 4), x + (size_t)t * d, d);
-    if (e < E) logits[(size_t)t * E + e] = (float)acc + (bias ? bias[e] : 0.f);
-  }
-}
-
+// ---- 5. listed tokens: every logit as an fp64 chain = k_router_exact_pairs<., true> above, unless the dense kernel takes over ----
 // exact softmax / top-k of the listed tokens (of every token when the dense kernel ran)
 template <int NPL>
 __global__ void __launch_bounds__(256) k_router_topk_listed(const float* __restrict__ logits, int* __restrict__ ids,
@@ -564,8 +557,10 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
   k_router_topk_mixed<8><<<gtok, 256, 0, st>>>(logits, ids, ws, P, E, k, id_stride, nc, fb_list, counters);
   MOE_LAUNCH_CHECK();
   // the exact redo of the listed tokens: three launches that return at once when nothing is listed
-  if (bf) k_router_exact_listed<true><<<512, 256, 0, st>>>(W->data, bias, x, E, d, fb_list, counters, dense_above, logits);
-  else k_router_exact_listed<false><<<512, 256, 0, st>>>(W->data, bias, x, E, d, fb_list, counters, dense_above, logits);
+  // (sized for the most tokens the listed path takes, dense_above of them; surplus blocks return at once)
+  const unsigned glist = (unsigned)(((size_t)(dense_above > 0 ? dense_above : 1) * E + 255) / 256);
+  if (bf) k_router_exact_pairs<true, true><<<glist, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, fb_list, dense_above);
+  else k_router_exact_pairs<false, true><<<glist, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, fb_list, dense_above);
   MOE_LAUNCH_CHECK();
   int rc = moe_router_logits_seq_if(W, bias, nullptr, x, P, logits, nullptr, nullptr, counters, dense_above, st);
   if (rc) return rc;
