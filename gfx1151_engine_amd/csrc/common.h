@@ -42,6 +42,17 @@ static inline Q4cpOps q4cp_ops(const moe_wview* w) {
   return o;
 }
 
+// Block barrier for data exchanged through LDS only.  __syncthreads() carries a workgroup fence that the compiler
+// lowers to s_waitcnt vmcnt(0) as well: a kernel that keeps global loads in flight across its barriers (prefetch into
+// registers or straight into LDS) would wait for all of them at every barrier.  This one waits for the wave's own LDS
+// accesses and synchronises; global memory written before it is NOT made visible to the other waves by it.
+__device__ __forceinline__ void moe_lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o; o >>= 1) v += __shfl_xor(v, o, 64);

@@ -523,10 +523,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     if (t < nstage) issue_a(t);
   // stage 0 must have landed; only the activation loads of the later stages may still be in flight
   wait_vm(nstage > 1 ? A_LOADS * (AHEAD - 1) : 0);
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0); a bare barrier again: the later stages' loads stay in flight
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
+  moe_lds_barrier();  // the later stages' loads stay in flight
   load_codes(0);
 #pragma unroll
   for (int mf = 0; mf < MF; mf++) load_a1(0, mf, a[0]);
@@ -567,12 +564,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     // buffer meanwhile, so that buffer must be complete and visible: loads of stage s+1 done
     // (stage s+2's may still fly), then the block barrier.
     wait_loads_before(s + 2);
-    // a bare barrier: __syncthreads() carries a fence that the compiler turns into s_waitcnt vmcnt(0), which would
-    // make every stage wait for the loads just issued two stages ahead
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
+    moe_lds_barrier();  // (not __syncthreads(): its fence would wait for the loads just issued two stages ahead)
     Ab = A0 + ((s + 1) % NBUF) * A_BYTES;
 #pragma unroll
     for (int i = 0; i < NM; i++) {

@@ -724,7 +724,7 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
 #pragma unroll
     for (int i = 0; i < GQ_D; i++) fetch(i, rw[i], ra[i]);
     decode(rw[0], ra[0], 0, 0);
-    __syncthreads();
+    moe_lds_barrier();  // (every barrier of this loop: the raw blocks of the next stages stay in flight across it)
     for (int s0 = 0; s0 < nstage; s0 += GQ_D) {
 #pragma unroll
       for (int u = 0; u < GQ_D; u++) {
@@ -735,7 +735,7 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
           fetch(s + GQ_D, rw[u], ra[u]);
           mfmas(buf);
           if (s + 1 < nstage) decode(rw[(u + 1) % GQ_D], ra[(u + 1) % GQ_D], buf ^ 1, s + 1);
-          __syncthreads();
+          moe_lds_barrier();
         }
       }
     }

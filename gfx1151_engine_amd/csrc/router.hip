@@ -133,11 +133,11 @@ __global__ void __launch_bounds__(256, 2) k_router_logits_seq(const void* __rest
   fetch_w(0, wr);
   wxr = fetch_wx(0);
   for (int c0 = 0; c0 < d; c0 += RS_K) {
-    __syncthreads();  // everybody is done reading the previous slab
+    moe_lds_barrier();  // everybody is done reading the previous slab (LDS-only barriers: the next slab's loads stay in flight)
     stage(Xs, xr, XL);
     stage(Ws, wr, WL);
     if (tid < RS_K) Wxs[tid] = wxr;
-    __syncthreads();
+    moe_lds_barrier();
     if (c0 + RS_K < d) {
       fetch_x(c0 + RS_K, xr);
       fetch_w(c0 + RS_K, wr);

@@ -107,9 +107,9 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
 
   fetch(0);
   for (int c0 = 0; c0 < d; c0 += RA_K) {
-    __syncthreads();  // the previous slab has been read
+    moe_lds_barrier();  // the previous slab has been read (LDS-only barriers: the next slab's loads stay in flight)
     stage();
-    __syncthreads();
+    moe_lds_barrier();
     if (c0 + RA_K < d) fetch(c0 + RA_K);
 #pragma unroll
     for (int ks = 0; ks < RA_K / 16; ks++) {
