@@ -206,7 +206,7 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   }
   if (e == hipSuccess && T > (size_t)c->small_max) {
     const size_t d = cfg->d, mid = cfg->mid;
-    e = hipMalloc(&c->rc_scratch, moe_router_cand_scratch_bytes(cfg->max_tokens, cfg->experts));
+    e = hipMalloc(&c->rc_scratch, moe_router_cand_scratch_bytes(cfg->max_tokens, cfg->experts, cfg->d));
     if (e == hipSuccess) e = hipMalloc(&c->x16, T * d * 2);
     if (e == hipSuccess) e = hipMalloc(&c->hid16, k1 * T * mid * 2);
     if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);

@@ -84,7 +84,7 @@ int moe_router_logits_seq_if(const moe_wview* W, const float* bias, const moe_wv
                              hipStream_t st);
 // batch router through candidate selection (router_cand.hip): bit-exact ids, weights within an ulp or two
 bool moe_router_cand_supported(const moe_wview* W, const moe_wview* Wx, int P, int k);
-size_t moe_router_cand_scratch_bytes(int max_tokens, int experts);
+size_t moe_router_cand_scratch_bytes(int max_tokens, int experts, int d);
 int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
                           float* logits, float* out_x, float* out_xms, int* ids, float* ws, int k, int id_stride,
                           void* scratch, hipStream_t st);

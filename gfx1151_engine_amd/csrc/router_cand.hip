@@ -3,7 +3,9 @@
 // The reference's router (src/ref.cpp:565-594) needs every logit as a sequential fp64 sum, but only the k
 // best logits of a token decide its experts and weights; the other ~500 enter through the softmax
 // normaliser alone, which cancels in the renormalised weights up to rounding.  So:
-//   1. k_router_approx   all T x E logits on the f16 matrix pipe (f32 accumulation), with the row norms of x and W;
+//   1. k_router_approx   all T x E logits on the f16 matrix pipe (f32 accumulation), with the row norms of x and W
+//                        (for d a multiple of 128: k_router_w16 + k_router_approx2, the same arithmetic with the
+//                        router matrix converted to f16 once per call and a token tile's activations read once);
 //   2. k_router_cand     per token a RIGOROUS error bound B_e on each approximate logit (below) gives an interval
 //                        [a_e - B_e, a_e + B_e] that holds the exact logit; tau = the k-th largest lower end; every
 //                        expert whose upper end reaches tau - 1e-5 is a candidate (the true top k are among them:
@@ -165,6 +167,217 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
         if (out_xms) out_xms[t0 + r] = sx / (float)d;
       }
       if (tt == 0 && e0 + r < E) wnorm[e0 + r] = sqrtf(sw);
+    }
+  }
+}
+
+// ---- 1'. the same approximate logits with the router matrix converted once per call ----
+// k_router_w16: W -> f16 (round to nearest even, the conversion the error bound charges) in scratch, rows padded with
+// zeros to a multiple of R2_BE, and the row norms of W (from the unrounded values).  A wave per row.
+constexpr int R2_BT = 64, R2_BE = 512, R2_K = 32, R2_NBUF = 4;
+constexpr int R2_WBYTES = R2_BE * R2_K * 2, R2_XBYTES = R2_BT * R2_K * 2;  // per slab: 32 KB of W16, 4 KB of x as f16
+constexpr int R2_SMEM = R2_NBUF * R2_WBYTES + 2 * R2_XBYTES;
+
+template <bool BF16>
+__global__ void __launch_bounds__(256) k_router_w16(const void* __restrict__ W, int E, int Epad, int d,
+                                                    __half* __restrict__ W16, float* __restrict__ wnorm,
+                                                    int* __restrict__ counters) {
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int row = blockIdx.x * 4 + wv;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    counters[0] = 0;  // tokens listed for the exact redo
+    counters[1] = 0;  // (token, row) pairs of the exact pass      (both are first used by later launches)
+  }
+  if (row >= Epad) return;
+  float s2 = 0.f;
+  for (int c = 4 * lane; c < d; c += 256) {
+    float4 w = float4{0.f, 0.f, 0.f, 0.f};
+    if (row < E) {
+      if (BF16) {
+        const uint2 u = *(const uint2*)((const uint16_t*)W + (size_t)row * d + c);
+        w = float4{__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                   __uint_as_float(u.y & 0xffff0000u)};
+      } else {
+        w = *(const float4*)((const float*)W + (size_t)row * d + c);
+      }
+    }
+    s2 += w.x * w.x + w.y * w.y + w.z * w.z + w.w * w.w;
+    // slab-major tiles [column group of R2_BE rows][32-column slab][row][four 16-byte chunks, chunk q in slot
+    // q ^ ((row >> 2) & 3)]: a slab of a column group is 32 KB of consecutive bytes in the order the LDS image has
+    const int rl = row % R2_BE, sl = c / R2_K, q = (c % R2_K) >> 3;
+    __half* dst = W16 + ((size_t)(row / R2_BE) * (d / R2_K) + sl) * (R2_BE * R2_K) + (size_t)rl * R2_K +
+                  ((q ^ ((rl >> 2) & 3)) << 3) + (c & 7);
+    *(half4v*)dst = half4v{(_Float16)w.x, (_Float16)w.y, (_Float16)w.z, (_Float16)w.w};
+  }
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) s2 += __shfl_xor(s2, o, 64);
+  if (lane == 0 && row < E) wnorm[row] = sqrtf(s2);
+}
+
+// k_router_approx2: block = 64 tokens x 512 experts, 8 waves of 64 x 64 (2 x 2 MFMA tiles); a token tile's activations
+// are read and converted once (the first kernel's four column blocks each did it again).  Per 32-column slab the f16
+// rows of W go global -> LDS directly (64-byte rows, the 16-byte chunk c of row r in slot c ^ ((r >> 2) & 3): the
+// fragment reads of 16 rows then cover all banks), four slab buffers; x is converted by its loader threads into a
+// double-buffered tile.  The two operands come from different distances -- W out of L2 (every block reads the same
+// 3 MB), x out of HBM -- and a wave's loads retire in order, so the loading is split between the waves: waves 0-3
+// fetch x eight slabs ahead (registers), waves 4-7 fetch W three slabs ahead (LDS), each half with a wait count of
+// its own.  One block barrier per slab.  Accumulators are flushed into running sums every RA_CHUNK columns, as in
+// k_router_approx: the error bound is the same.
+constexpr int R2_XD = 8;  // slabs of x in flight
+typedef float f32x4_nt __attribute__((ext_vector_type(4)));
+// 16 bytes that this kernel reads exactly once: loaded as streaming data, so that they do not push the f16 router
+// matrix (read by every block) out of L2
+__device__ __forceinline__ float4 ld_stream4(const float* p) {
+  const f32x4_nt v = __builtin_nontemporal_load((const f32x4_nt*)p);
+  return float4{v.x, v.y, v.z, v.w};
+}
+__global__ void __launch_bounds__(512, 1) k_router_approx2(const __half* __restrict__ W16, const float* __restrict__ bias,
+                                                         const float* __restrict__ x, int P, int E, int d,
+                                                         float* __restrict__ alog, float* __restrict__ xnorm,
+                                                         float* __restrict__ out_xms) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t r2sm[];
+  uint8_t* const Wl = r2sm;
+  uint8_t* const Xl = r2sm + R2_NBUF * R2_WBYTES;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool xwave = wv < 4;
+  const int n = lane & 31, h = lane >> 5;
+  const int t0 = blockIdx.x * R2_BT, e0 = blockIdx.y * R2_BE;
+  const int nslab = d / R2_K;
+  // W16 (waves 4-7): a slab of this column group is 32 KB of consecutive bytes in LDS order (k_router_w16); wave
+  // instruction j = 8 (wv - 4) + i copies bytes [1024 j, 1024 j + 1024)
+  const int wj0 = 8 * (wv & 3);
+  const uint8_t* const wsrc = (const uint8_t*)W16 + (size_t)blockIdx.y * nslab * R2_WBYTES + wj0 * 1024 + lane * 16;
+  auto issue_w = [&](int s) {
+    uint8_t* dst = Wl + (s % R2_NBUF) * R2_WBYTES + wj0 * 1024;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wsrc + (size_t)s * R2_WBYTES + i * 1024),
+                                       (__attribute__((address_space(3))) void*)(dst + i * 1024), 16, 0, 0);
+  };
+  // x (waves 0-3): thread -> float4 f = tid + 256 j (j = 0, 1) of the slab: token row f / 8, columns 4 (f % 8) .. + 3
+  const float* xsrc[2];
+  uint8_t* xdst[2];
+  bool xlive[2];
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int f = (tid & 255) + 256 * j, row = f >> 3, p = f & 7;
+    xlive[j] = t0 + row < P;
+    xsrc[j] = x + (size_t)(xlive[j] ? t0 + row : 0) * d + 4 * p;
+    xdst[j] = Xl + row * 64 + (((p >> 1) ^ ((row >> 2) & 3)) << 4) + (p & 1) * 8;
+  }
+  float4 xq[R2_XD][2];
+  float xs2[2] = {0.f, 0.f};
+  floatx16 acc[2][2], run[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = run[i][j][r] = 0.f;
+  if (xwave) {
+#pragma unroll
+    for (int s = 0; s < R2_XD; s++)
+      if (s < nslab) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) xq[s][j] = ld_stream4(xsrc[j] + (size_t)s * R2_K);
+      }
+  } else {
+#pragma unroll
+    for (int s = 0; s < 3; s++)
+      if (s < nslab) issue_w(s);
+  }
+  for (int s0 = 0; s0 < nslab; s0 += R2_XD) {
+#pragma unroll
+    for (int u = 0; u < R2_XD; u++) {
+      const int s = s0 + u;
+      if (s >= nslab) break;
+      if (xwave) {
+        // (the compiler waits for xq[u]: the seven later slabs' loads stay in flight)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+          const float4 a = xlive[j] ? xq[u][j] : float4{0.f, 0.f, 0.f, 0.f};
+          xs2[j] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+          *(half4v*)(xdst[j] + (s & 1) * R2_XBYTES) = half4v{(_Float16)a.x, (_Float16)a.y, (_Float16)a.z, (_Float16)a.w};
+        }
+      } else {
+        // slab s has landed when at most the loads of the (up to two) later slabs in flight are outstanding
+        const int later = nslab - 1 - s < 2 ? nslab - 1 - s : 2;
+        if (later == 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        else if (later == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      // slab s of W (its loaders waited for it) and of x is in LDS; slab s - 1 has been read by all.  An LDS-only
+      // barrier: __syncthreads() would wait for every load in flight
+      moe_lds_barrier();
+      if (xwave) {
+        if (s + R2_XD < nslab) {
+#pragma unroll
+          for (int j = 0; j < 2; j++) xq[u][j] = ld_stream4(xsrc[j] + (size_t)(s + R2_XD) * R2_K);
+        }
+      } else if (s + 3 < nslab) {
+        issue_w(s + 3);
+      }
+      const uint8_t* Wb = Wl + (s % R2_NBUF) * R2_WBYTES;
+      const uint8_t* Xb = Xl + (s & 1) * R2_XBYTES;
+#pragma unroll
+      for (int ks = 0; ks < R2_K / 16; ks++) {
+        half8 a[2], b[2];
+#pragma unroll
+        for (int mf = 0; mf < 2; mf++) {
+          const int row = 32 * mf + n;
+          a[mf] = *(const half8*)(Xb + row * 64 + (((2 * ks + h) ^ ((row >> 2) & 3)) << 4));
+        }
+#pragma unroll
+        for (int nf = 0; nf < 2; nf++) {
+          const int row = 64 * wv + 32 * nf + n;
+          b[nf] = *(const half8*)(Wb + row * 64 + (((2 * ks + h) ^ ((row >> 2) & 3)) << 4));
+        }
+#pragma unroll
+        for (int mf = 0; mf < 2; mf++)
+#pragma unroll
+          for (int nf = 0; nf < 2; nf++)
+            acc[mf][nf] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mf], b[nf], acc[mf][nf], 0, 0, 0);
+      }
+      if (((s + 1) * R2_K) % RA_CHUNK == 0 || s + 1 == nslab) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+          for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              run[i][j][r] += acc[i][j][r];
+              acc[i][j][r] = 0.f;
+            }
+      }
+    }
+  }
+  // D[i][j]: j = lane % 32 (expert), i = 8 * (r / 4) + 4 * (lane / 32) + r % 4 (token)
+#pragma unroll
+  for (int mf = 0; mf < 2; mf++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int t = t0 + 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (t >= P) continue;
+#pragma unroll
+      for (int nf = 0; nf < 2; nf++) {
+        const int e = e0 + 64 * wv + 32 * nf + n;
+        if (e < E) alog[(size_t)t * E + e] = run[mf][nf][r] + (bias ? bias[e] : 0.f);
+      }
+    }
+  // row norms of x: the 8 threads of a row are consecutive lanes of the loading waves
+  if (xwave) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      float v = xs2[j];
+      v += __shfl_xor(v, 1, 64);
+      v += __shfl_xor(v, 2, 64);
+      v += __shfl_xor(v, 4, 64);
+      const int f = (tid & 255) + 256 * j, row = f >> 3;
+      if (blockIdx.y == 0 && (f & 7) == 0 && xlive[j]) {
+        xnorm[t0 + row] = sqrtf(v);
+        if (out_xms) out_xms[t0 + row] = v / (float)d;
+      }
     }
   }
 }
@@ -515,9 +728,10 @@ bool moe_router_cand_supported(const moe_wview* W, const moe_wview* Wx, int P, i
   return moe_aligned(W->data, 16) && (!Wx || moe_aligned(Wx->data, 16));
 }
 
-size_t moe_router_cand_scratch_bytes(int max_tokens, int experts) {
-  // counters [16], pairs [T][32] u32, nc [T], fb_list [T], xnorm [T], wnorm [E]
-  return (size_t)max_tokens * (RC_SLOTS * 4 + 4 + 4 + 4) + (size_t)experts * 4 + 64 + 256;
+static size_t rc_epad(int experts) { return ((size_t)experts + R2_BE - 1) / R2_BE * R2_BE; }
+size_t moe_router_cand_scratch_bytes(int max_tokens, int experts, int d) {
+  // counters [16], pairs [T][32] u32, nc [T], fb_list [T], xnorm [T], wnorm [E], the router matrix as f16 (rows padded)
+  return (size_t)max_tokens * (RC_SLOTS * 4 + 4 + 4 + 4) + rc_epad(experts) * 4 + 64 + 256 + 256 + rc_epad(experts) * (size_t)d * 2;
 }
 
 // Internal: ids / ws (and the shared-expert gate logit, the per-token mean square of x) of a batch; `logits` ends
@@ -533,7 +747,8 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
   int* nc = (int*)sp; sp += (size_t)P * 4;
   int* fb_list = (int*)sp; sp += (size_t)P * 4;
   float* xnorm = (float*)sp; sp += (size_t)P * 4;
-  float* wnorm = (float*)sp;
+  float* wnorm = (float*)sp; sp += rc_epad(E) * 4;
+  __half* W16 = (__half*)(((uintptr_t)sp + 255) & ~(uintptr_t)255);
   const bool bf = W->dtype == MOE_DT_BF16;
   const int ncol = (E + RA_BE - 1) / RA_BE, ntt = (P + RA_BT - 1) / RA_BT;
   const unsigned grid_a = (unsigned)(((ntt + 7) / 8) * 8 * ncol);
@@ -543,8 +758,25 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
   const int dense_above = P / 16;
   const void* wx = Wx ? Wx->data : nullptr;
   const unsigned gtok = (unsigned)((P + 3) / 4), gtok16 = (unsigned)((P + 15) / 16);
-  if (bf) k_router_approx<true><<<grid_a, 256, 0, st>>>(W->data, bias, x, P, E, d, logits, wnorm, xnorm, out_xms, counters, ncol, ntt);
-  else k_router_approx<false><<<grid_a, 256, 0, st>>>(W->data, bias, x, P, E, d, logits, wnorm, xnorm, out_xms, counters, ncol, ntt);
+  if (d % RA_CHUNK == 0) {
+    // the router matrix as f16 once per call (a few microseconds), then the approximate logits with a token tile's
+    // activations read and converted once
+    const int Epad = (int)rc_epad(E);
+    if (bf) k_router_w16<true><<<(Epad + 3) / 4, 256, 0, st>>>(W->data, E, Epad, d, W16, wnorm, counters);
+    else k_router_w16<false><<<(Epad + 3) / 4, 256, 0, st>>>(W->data, E, Epad, d, W16, wnorm, counters);
+    MOE_LAUNCH_CHECK();
+    static bool attr_done = false;
+    if (!attr_done) {
+      MOE_HIP(hipFuncSetAttribute((const void*)k_router_approx2, hipFuncAttributeMaxDynamicSharedMemorySize, R2_SMEM));
+      attr_done = true;
+    }
+    const dim3 g2((unsigned)((P + R2_BT - 1) / R2_BT), (unsigned)(Epad / R2_BE));
+    k_router_approx2<<<g2, 512, R2_SMEM, st>>>(W16, bias, x, P, E, d, logits, xnorm, out_xms);
+  } else if (bf) {
+    k_router_approx<true><<<grid_a, 256, 0, st>>>(W->data, bias, x, P, E, d, logits, wnorm, xnorm, out_xms, counters, ncol, ntt);
+  } else {
+    k_router_approx<false><<<grid_a, 256, 0, st>>>(W->data, bias, x, P, E, d, logits, wnorm, xnorm, out_xms, counters, ncol, ntt);
+  }
   MOE_LAUNCH_CHECK();
   k_router_cand<8><<<gtok16, 1024, 0, st>>>(logits, wnorm, xnorm, P, E, k, eps, dterm, pairs, nc, fb_list, counters,
                                          wx ? 1 : 0);
