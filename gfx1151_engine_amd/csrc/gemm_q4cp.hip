@@ -322,6 +322,14 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // wait until the loads of every stage before `first` have landed; stages first .. first+AHEAD-2
   // (those that exist) may still be in flight
   auto wait_loads_before = [&](int first) {
+    if (AHEAD == 2) {
+      // one later stage can be in flight: none, its NLOADS loads, or those and the scale loads -- three immediates
+      // (the general count below compiles to a search tree of scalar branches in every stage)
+      if (first >= nstage) __builtin_amdgcn_s_waitcnt(0x0F70);
+      else if ((first & 3) == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | ((NLOADS + S_LOADS) & 15) | (((NLOADS + S_LOADS) >> 4) << 14));
+      else __builtin_amdgcn_s_waitcnt(0x0F70 | (NLOADS & 15) | ((NLOADS >> 4) << 14));
+      return;
+    }
     int n = 0;
     for (int t = first; t < first + AHEAD - 1; t++)
       if (t < nstage) n += NLOADS + ((t & 3) == 0 ? S_LOADS : 0);
