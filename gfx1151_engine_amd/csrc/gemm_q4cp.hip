@@ -367,7 +367,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     const int m = 32 * mf + n;
     dst[mf] = *(const half8*)(Ab + m * 128 + (((4 * h + q) ^ ((m >> 1) & 7)) << 4));
   };
-  uint32_t sc4[NSB == 1 ? NF : 1][4];  // single scale buffer: this lane's scales of four stages (f16 bits)
+  // single scale buffer: this lane's scales of four stages, f16 bits packed two to a word (stages 0 | 1, 2 | 3); a
+  // stage takes its own with one 64-bit shift (a choice between four registers by the wave-uniform stage index
+  // compiles to a tree of scalar branches in every stage)
+  uint32_t scp[NSB == 1 ? NF : 1][2];
   auto load_codes = [&](int s) {  // raw codes + this lane's scale of stage s (buffers already selected)
     if (Q5) q5sh = 2 * (s & 3);
     const uint8_t* Wb = W0 + (s % NBUF) * W_BYTES;
@@ -392,20 +395,19 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
           if (GS == 2) {
             if ((s & 3) == 0) {
               const uint32_t w = *(const uint32_t*)(Sb + wrow[nf] * 4);
-              sc4[nf][0] = sc4[nf][1] = w & 0xffffu;
-              sc4[nf][2] = sc4[nf][3] = w >> 16;
+              scp[nf][0] = __builtin_amdgcn_perm(w, w, 0x01000100u);  // (lo, lo)
+              scp[nf][1] = __builtin_amdgcn_perm(w, w, 0x03020302u);  // (hi, hi)
             }
           } else if ((s & 3) == 0) {
             const uint4 w = *(const uint4*)(Sb + wrow[nf] * 16);
-            sc4[nf][0] = h ? w.x >> 16 : w.x & 0xffffu;
-            sc4[nf][1] = h ? w.y >> 16 : w.y & 0xffffu;
-            sc4[nf][2] = h ? w.z >> 16 : w.z & 0xffffu;
-            sc4[nf][3] = h ? w.w >> 16 : w.w & 0xffffu;
+            const uint32_t sel = h ? 0x07060302u : 0x05040100u;  // this lane's half of each word
+            scp[nf][0] = __builtin_amdgcn_perm(w.y, w.x, sel);
+            scp[nf][1] = __builtin_amdgcn_perm(w.w, w.z, sel);
           }
           const int wi = GS == 2 ? (s & 3) : (sidx - h) >> 1;  // wave-uniform
-          const uint32_t bits = wi == 0 ? sc4[nf][0] : wi == 1 ? sc4[nf][1] : wi == 2 ? sc4[nf][2] : sc4[nf][3];
+          const uint64_t both = ((uint64_t)scp[nf][1] << 32) | scp[nf][0];
           union { uint16_t u; _Float16 f; } cv;
-          cv.u = (uint16_t)bits;
+          cv.u = (uint16_t)(both >> (16 * wi));
           scf[nf] = (float)cv.f;
         }
       } else {
