@@ -410,7 +410,7 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
         double w0, w1;
         weights(j, c0, w0, w1);
         fetch(j, c0 + RM_D * RM_C);  // slabs past d load column 0 and count as zeros
-        __syncthreads();
+        moe_lds_barrier();  // (LDS only: the ring's loads stay in flight across it)
         // rows past P hold zeros: no predicate, so the LDS reads of a slab go out back to back
 #pragma unroll
         for (int t = 0; t < PMAX; t++) {
