@@ -801,8 +801,11 @@ static GgKinds gg_kinds(const MoeLayer& L, const moe_config& g) {
   return k;
 }
 // the order of the f16 activations a layer's grouped GEMMs read (moe_f32_to_f16's layout)
+// q4cp experts whose codebook is a table (not a*n + b): the grouped GEMMs of the whole layer then run in natural K
+// order and dequantise through pair tables (gemm_q4cp.hip, NAT); affine experts keep the interleaved order
+static bool batch_nat(const MoeLayer& L) { return L.has_q4cp && !L.has_i4r && !L.experts_affine; }
 static int batch_x16_layout(const MoeLayer& L, const moe_config& g) {
-  if (!L.has_gguf) return 1;
+  if (!L.has_gguf) return batch_nat(L) ? 0 : 1;
   return gg_kinds(L, g).any_tuned() ? 2 : 0;
 }
 
@@ -869,6 +872,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
   const __half* xh = c->x16_ext ? c->x16_ext : c->x16;  // f16 activations in the GEMM's order
   const int xl = batch_x16_layout(L, g);       // that order (moe_f32_to_f16's layout)
+  const bool nat = batch_nat(L);               // table codebooks: natural K order, pair tables
   // gate/up (+ SwiGLU) and down launches over a tile list: routed experts, with_sh: the shared expert as well
   // (tiles whose expert index is >= n_experts)
   auto gemm_up = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2) -> int {
@@ -900,7 +904,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
       return moe_launch_gemm_q4cp(true, &sgu, &sgu, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, true,
                                   false, hs, s2, nullptr, sh_cb_up);
     return moe_launch_gemm_q4cp(true, &gu, with_sh ? &sgu : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16,
-                                g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up, 0, q4k && L.gg.tgu == MOE_GGML_Q5_K);
+                                g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up, 0, q4k && L.gg.tgu == MOE_GGML_Q5_K, nat);
   };
   auto gemm_dn = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2, const moe_comb* cmb) -> int {
     if (shd && with_sh)  // (hid rows of the shared tiles were written in natural order by the launch above)
@@ -928,7 +932,8 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
       return moe_launch_gemm_q4cp(false, &sdn, &sdn, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid,
                                   true, false, hs, s2, nullptr);
     return moe_launch_gemm_q4cp(false, &dn, with_sh ? &sdn : nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt,
-                                cmb ? (void*)cmb->y : (void*)c->pairs16, g.d, g.mid, cmb == nullptr, q4k, hs, s2, cmb);
+                                cmb ? (void*)cmb->y : (void*)c->pairs16, g.d, g.mid, cmb == nullptr, q4k, hs, s2, cmb, nullptr,
+                                0, false, nat);
   };
   const bool fused = c->fused_combine && !c->hc && !(q4k && !kd.r_dn) && !split && !v2;  // the HC write-back belongs to the ordered combine
   if (v2 || (L.has_shared && (split || (c->shared_aside && !fused)))) {

@@ -72,6 +72,9 @@ constexpr int NSB = WROWS == 512 ? 2 : 1;
 constexpr int NBUF = MOE_GEMM_NBUF;       // activation / code buffers; loads run NBUF-1 stages ahead
 constexpr int AHEAD = NBUF - 1;
 constexpr int SMEM_BYTES = NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES + 128 + BM * 4 + BM * 4;  // + two 16-entry codebooks, row indices, row scales
+// NAT (table codebooks in natural K order): two 256-entry tables of f16 pairs behind the rest, indexed by a whole code
+// byte = two neighbouring weights (the (gate) rows' codebook and the up rows')
+constexpr int PT_BYTES = 2 * 256 * 4;
 
 struct LutDev {
   const uint8_t *w, *w_up, *sc, *sc_up;
@@ -143,7 +146,7 @@ __device__ __forceinline__ void g2l4(const void* g, uint8_t* lds_base) {
 // MF = live 32-row fragments of the tile (1 .. 4); AFFINE = codebook a*n+b.
 // NF = weight fragments (32 rows) per wave: the block's 16 fragments are split over NW = 16/NF
 // waves, each wave multiplying all MF pair fragments with its own NF weight fragments.
-template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS, bool Q5>
+template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS, bool Q5, bool NAT = false>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
@@ -152,6 +155,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   constexpr int NH = NF / 2;  // gate/up: fragments per half
   static_assert(GS == 0 || (GS == 2 && !Q4K && NSB == 1), "one scale per 128 columns: q4cp-style planes, single scale buffer");
   static_assert(!Q5 || (Q4K && NSB == 1), "Q5_K: the Q4_K stages plus a fifth bit");
+  static_assert(!NAT || (!AFFINE && !Q4K && GS == 0), "pair tables: q4cp planes with a table codebook");
+  const uint32_t* const ptab = (const uint32_t*)(smem + SMEM_BYTES);
   constexpr int KBLK = Q5 ? 176 : 144;   // bytes per super-block
   constexpr int KQS = Q5 ? 48 : 16;      // offset of the code bytes in it
   // loads per row group behind the scale buffer's: the header's 16 bytes go to LDS; Q5_K adds two 8-byte register loads
@@ -457,6 +462,11 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
       for (int nf = 0; nf < NF; nf++) {
         const bool upf = UP && nf >= NH;  // the up half may come from a tensor with a codebook of its own
+        if (NAT) {
+          const _Float16 sh = (_Float16)scf[nf];  // (exact: the scale is an f16)
+          as2[nf][0] = half2v{sh, sh};
+          continue;
+        }
         const _Float16 as = (_Float16)((upf ? cb_a_up : cb_a) * scf[nf]), bs = (_Float16)((upf ? cb_b_up : cb_b) * scf[nf]);
         as2[nf][0] = half2v{as, as};
         bs2[nf][0] = half2v{bs, bs};
@@ -493,11 +503,19 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         dst[nf].h[part] = (as_h2(t) - half2v{(_Float16)64.f, (_Float16)64.f}) * as2[nf][ss] + bs2[nf][ss];
       }
     } else {
-      half2v hv;
-      const float* tb = (UP && nf >= NH) ? cbs + 16 : cbs;
-      hv.x = (_Float16)(tb[(w >> (4 * part)) & 0xf] * scf[nf]);
-      hv.y = (_Float16)(tb[(w >> (4 * part + 16)) & 0xf] * scf[nf]);
-      dst[nf].h[part] = hv;
+      if (NAT) {
+        // byte `part` of the word = weights 2 part, 2 part + 1 of the step in natural order: one look-up gives both as
+        // f16(cb), one packed product applies the scale: w = f16(f16(cb[n]) * scale), the reference kernel's contract
+        // (src/gpu/parts/27_kernels_moe_lut.inc:16)
+        const uint32_t* pt = (UP && nf >= NH) ? ptab + 256 : ptab;
+        dst[nf].h[part] = as_h2(pt[(w >> (8 * part)) & 0xffu]) * as2[nf][0];
+      } else {
+        half2v hv;
+        const float* tb = (UP && nf >= NH) ? cbs + 16 : cbs;
+        hv.x = (_Float16)(tb[(w >> (4 * part)) & 0xf] * scf[nf]);
+        hv.y = (_Float16)(tb[(w >> (4 * part + 16)) & 0xf] * scf[nf]);
+        dst[nf].h[part] = hv;
+      }
     }
   };
   constexpr int NM = NF * MF;                     // MFMAs per K step
@@ -624,7 +642,9 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
           const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
           // hid feeds the down GEMM: permuted order inside groups of 8 (q4cp) / blocks of 64 (Q4_K)
           int pos;
-          if (!Q4K) {
+          if (NAT) {
+            pos = 32 * f + n;  // natural order
+          } else if (!Q4K) {
             const int c = 32 * f + n;
             pos = (c & ~7) + ilv_pos(c & 7);
           } else if (NH == 1) {
@@ -721,7 +741,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   }
 }
 
-template <bool UP, bool F16OUT, bool Q4K, int GS, bool Q5 = false>
+template <bool UP, bool F16OUT, bool Q4K, int GS, bool Q5 = false, bool NAT = false>
 __global__ void __launch_bounds__(NT, WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
@@ -774,7 +794,19 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   // q4cp codebook: affine (a*n+b) or table.  Q4_K has no codebook (w = (d*sc)*n - dmin*m).
   bool affine = true;
   float cb_a = 1.f, cb_b = 0.f, cb_a_up = 1.f, cb_b_up = 0.f;
-  if (!Q4K) {
+  if (NAT) {
+    // pair tables: entry b = (f16(cb[b & 15]), f16(cb[b >> 4])) = the two weights of code byte b before scaling
+    uint32_t* pt = (uint32_t*)(smem + SMEM_BYTES);
+    const float* cbu = UP ? L.cb_up : L.cb;
+    for (int i = tid; i < 256; i += NT) {
+      union { half2v h; uint32_t u; } g, u;
+      g.h = half2v{(_Float16)L.cb[i & 15], (_Float16)L.cb[i >> 4]};
+      u.h = half2v{(_Float16)cbu[i & 15], (_Float16)cbu[i >> 4]};
+      pt[i] = g.u;
+      pt[256 + i] = u.u;
+    }
+    affine = false;
+  } else if (!Q4K) {
     // lanes 0..15: the (gate) rows' codebook, lanes 16..31: the up rows' (the same table unless the two
     // halves come from separately quantised tensors, as a shared expert's gate_proj / up_proj do)
     const float* cbu = UP ? L.cb_up : L.cb;
@@ -799,7 +831,8 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS, Q5>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    if constexpr (NAT) gemm_tile<UP, F16OUT, MF, false, false, 0, false, true>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    else if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS, Q5>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
     else gemm_tile<UP, F16OUT, MF, false, false, GS, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
@@ -853,8 +886,9 @@ bool moe_gemm_q5k_fits(uint64_t rows, uint64_t x_rows, int k) {
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs, bool q5k) {
+                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs, bool q5k, bool nat) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
+  if (nat && (q4k || q5k || gs != 0)) return MOE_E_UNSUPPORTED;  // (natural K order: q4cp planes through pair tables)
   if (q5k && (!q4k || !up || comb)) return MOE_E_UNSUPPORTED;  // (Q5_K: gate/up tensors, the reference checkpoints' use of it)
   // (Q5_K: 32-bit byte offsets into the tensors; the caller vouches for the activation rows, moe_gemm_q5k_fits)
   if (q5k && routed && !moe_gemm_q5k_fits((uint64_t)(sh == routed ? 1 : n_experts) * (uint64_t)routed->e_rows + (uint64_t)routed->up_off + (uint64_t)m, 0, k))
@@ -889,7 +923,22 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
     k_moe_gemm_q4cp<UPK, F16, Q, G><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
                                                                   m, k, nblk_n, split, hs, cmb);                 \
   } while (0)
-  if (q5k) {
+#define GEMM_LAUNCH_NAT(UPK, F16)                                                                                \
+  do {                                                                                                           \
+    static bool attr_done = false;                                                                               \
+    if (!attr_done) {                                                                                            \
+      MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<UPK, F16, false, 0, false, true>,                 \
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SMEM_BYTES + PT_BYTES)));    \
+      attr_done = true;                                                                                          \
+    }                                                                                                            \
+    k_moe_gemm_q4cp<UPK, F16, false, 0, false, true><<<grid, NT, SMEM_BYTES + PT_BYTES, st>>>(                    \
+        R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, split, hs, cmb);                           \
+  } while (0)
+  if (nat) {
+    if (up) GEMM_LAUNCH_NAT(true, true);
+    else if (f16out) GEMM_LAUNCH_NAT(false, true);
+    else GEMM_LAUNCH_NAT(false, false);
+  } else if (q5k) {
     static bool attr5 = false;
     if (!attr5) {
       MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<true, true, true, 0, true>,
@@ -910,6 +959,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
     else GEMM_LAUNCH(false, false, false, 0);
   }
 #undef GEMM_LAUNCH
+#undef GEMM_LAUNCH_NAT
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -55,7 +55,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
                          hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr, int gs = 0,
-                         bool q5k = false);
+                         bool q5k = false, bool nat = false);
 // The Q5_K form addresses weights and activations with 32-bit byte offsets: true when a tensor of `rows` rows of k
 // columns and an activation buffer of `x_rows` rows of k f16 values both stay below 4 GB (the caller of
 // moe_launch_gemm_q4cp(q5k = true) checks it; other layers take the general kernel)

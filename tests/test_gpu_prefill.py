@@ -266,6 +266,47 @@ def test_forward_hc_writeback(oracle, fmt):
     m.close()
 
 
+@pytest.mark.parametrize("shared", ["same", "per_tensor", "affine", "bf16", "none"])
+@pytest.mark.parametrize("d,mid,E,k,T", [(512, 256, 8, 3, 70), (768, 512, 6, 2, 300), (3072, 768, 12, 4, 161)])
+def test_batch_layer_with_a_table_codebook(oracle, shared, d, mid, E, k, T):
+    """Routed experts with a codebook that is not a*n + b (what the reference's converter writes by default: its
+    universal expert codebook): the grouped GEMMs of the layer run in natural K order through pair tables.  The shared
+    expert with the same table, a table per tensor, uniform grids, dense bf16 rows, or absent; the shared expert aside
+    or in the routed launches, the ordered and the fused combine.  ids bit-exact, output within the batch bar."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(d + T + len(shared))
+    n = np.arange(16, dtype=np.float32)
+    cb = np.sort(rng.uniform(-2, 2, 16)).astype(np.float32)
+    kw = {}
+    if shared == "per_tensor":
+        kw["shared_codebooks"] = [np.sort(rng.uniform(-2, 2, 16)).astype(np.float32) for _ in range(3)]
+    elif shared == "affine":
+        kw["shared_codebooks"] = [n - 8, 0.5 * n - 3.0, -0.25 * n + 1.0]
+    elif shared == "bf16":
+        kw["shared_dense"] = "bf16"
+    elif shared == "none":
+        kw["shared"] = False
+    hl = HostLayer(rng, d, mid, E, k, codebook=cb, **kw)
+    x = S.bf16_round(rng.standard_normal((T, d), dtype=np.float32))
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    assert m.x16_layout(0) == 0, "table codebooks: activations in natural order"
+    for aside, fused in ((1, 0), (0, 0), (0, 1)):
+        m.set_option(capi.OPT_SHARED_ASIDE, aside)
+        m.set_option(capi.OPT_FUSED_COMBINE, fused)
+        y = m.forward(0, gpu(x))
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+        err = max_abs_rel(y.cpu().numpy(), yo)
+        assert err <= TOL_LAYER, (aside, fused, err)
+    m.set_option(capi.OPT_SHARED_ASIDE, 1)
+    m.set_option(capi.OPT_FUSED_COMBINE, 0)
+    y0 = m.forward(0, gpu(x)).cpu().numpy()
+    y1 = m.forward_x16(0, gpu(x), capi.f32_to_f16(gpu(x), layout=0)).cpu().numpy()
+    assert (y1 == y0).all(), "the caller's natural-order f16 copy gives the same bits"
+    m.close()
+
+
 @pytest.mark.parametrize("fmt", ["q4cp", "q4k"])
 def test_forward_with_the_callers_f16_copy(oracle, fmt):
     """moe_forward_x16: the caller hands over the f16 copy of the batch in the grouped GEMM's order (its own epilogue
