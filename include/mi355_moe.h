@@ -262,8 +262,8 @@ int moe_forward_hc(moe_ctx* ctx, int layer, const float* x, int P, const float* 
 /* moe_forward for a caller that already holds the batch as f16 in the order the grouped GEMM reads (the reference's
  * callers write a 16-bit copy of x in the epilogue that produces x, src/gpu/parts/40_model.inc:2556-2565; its
  * moe_q4w_run / moe_gguf convert once more, :1762, :1703).  x16: f16 [P][d] as moe_f32_to_f16(x, ., layout) makes it,
- * layout = moe_x16_layout(ctx, layer) (1: q4cp experts; GGUF layers: 2 when the launches that read x run Q4_K / Q5_K
- * tensors on the tuned kernel, else 0 = natural order).  x (f32) is still read by the router.
+ * layout = moe_x16_layout(ctx, layer) (q4cp experts: 1, or 0 = natural order when their codebook is a table rather than
+ * a*n + b; GGUF layers: 2 when the launches that read x run Q4_K / Q5_K tensors on the tuned kernel, else 0).  x (f32) is still read by the router.
  * The library's own conversion pass is left out.  P > 32 only (MOE_E_UNSUPPORTED below: the small-batch kernels do
  * not use an f16 copy; call moe_forward there), and a format outside the grouped GEMM returns MOE_E_UNSUPPORTED. */
 int moe_x16_layout(moe_ctx* ctx, int layer);
