@@ -193,7 +193,7 @@ def make_i4r(rng, rows, cols, scale_std=0.01):
 
 def make_v2_planes(rng, d, mid):
     """The four sign-scale planes of an hgn v2 layer's expert tensors as f16-representable f32 values (the files hold
-    them as f16): su [d], svh_gu [2 mid], suh_dn [mid], svh_dn [d]; magnitudes around 1, random signs."""
+    them as f16): su [d], svh_gu [2 mid], suh_dn [mid], svh_dn [d]; magnitudes near 1, random signs."""
     def plane(n):
         v = (0.5 + rng.random(n)) * rng.choice([-1.0, 1.0], size=n)
         return v.astype(np.float16).astype(np.float32)
