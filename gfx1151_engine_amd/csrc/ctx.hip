@@ -1036,11 +1036,18 @@ MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, 
   if (P <= c->small_max) return forward_small(c, *L, x, P, y, moe_s(st));
   const int rc = forward_batch(c, *L, x, P, y, moe_s(st));
   if (rc != MOE_E_UNSUPPORTED) return rc;
-  // formats the grouped GEMM does not cover yet: the in-place path, 32 rows at a time
-  for (int t0 = 0; t0 < P; t0 += c->small_max) {
+  // formats the grouped GEMM does not cover yet: the in-place path, 32 rows at a time.  Every chunk leaves its
+  // router output in the first rows of ids / ws; the walk runs from the last chunk to the first and moves each
+  // chunk's rows to their place, so that moe_get_routing sees the whole batch afterwards.
+  const size_t stride = (size_t)c->cfg.id_stride;
+  for (int t0 = (P - 1) / c->small_max * c->small_max; t0 >= 0; t0 -= c->small_max) {
     const int n = P - t0 < c->small_max ? P - t0 : c->small_max;
     const int r2 = forward_small(c, *L, x + (size_t)t0 * c->cfg.d, n, y + (size_t)t0 * c->cfg.d, moe_s(st));
     if (r2) return r2;
+    if (t0 > 0) {
+      MOE_HIP(hipMemcpyAsync(c->ids + t0 * stride, c->ids, n * stride * 4, hipMemcpyDeviceToDevice, moe_s(st)));
+      MOE_HIP(hipMemcpyAsync(c->ws + t0 * stride, c->ws, n * stride * 4, hipMemcpyDeviceToDevice, moe_s(st)));
+    }
   }
   return MOE_OK;
 }
