@@ -12,6 +12,7 @@ from .build import LIB
 
 F32, BF16, Q4CP, Q8G64, Q8G32 = 1, 0, 5, 7, 8
 I4R = 23  # hgn v2 routed experts
+HT, Q6G64 = 16, 24  # hgn v2 dense tensors (converted to bf16 by v2_dense_to_bf16 / the file loader)
 GGML_Q4_K = 12
 GGML_Q5_K, GGML_Q5_1, GGML_Q8_0 = 13, 7, 8
 
@@ -229,6 +230,14 @@ def i4r_dequant_rows(blob, rows, cols, row0, nrows):
     out = torch.empty((nrows, cols), dtype=torch.float32, device=blob.device)
     check(lib().moe_i4r_dequant_rows(ptr(blob), u64(rows), u64(cols), u64(row0), u64(nrows), ptr(out), stream()),
           "moe_i4r_dequant_rows")
+    return out
+
+
+def v2_dense_to_bf16(dtype, blob, rows, cols, suh=None, svh=None):
+    """An hgn v2 dense tensor (HT with its planes as f32, or Q6G64) -> the bf16 bits [rows][cols] of the matrix."""
+    out = torch.empty((rows, cols), dtype=torch.int16, device=blob.device)
+    check(lib().moe_v2_dense_to_bf16(dtype, ptr(blob), ptr(suh), ptr(svh), u64(rows), u64(cols), ptr(out), stream()),
+          "moe_v2_dense_to_bf16")
     return out
 
 

@@ -232,6 +232,115 @@ int moe_launch_i4r_mid(const void* z, bool z_f16, uint64_t zs, int nslots, int m
   return MOE_OK;
 }
 
+// ---- hgn v2 dense tensors ("ht", dtype 16; q6g64, dtype 24) -> bf16 W[rows][cols] ----
+// The matrix the reference's prefill GEMM reads for such a tensor (v2_deq_bf16, src/gpu/parts/30_host_util.inc:1019-1031).
+// The loader runs this once per tensor; the router and shared-expert kernels then see a bf16 matrix.
+
+// ht value of a 16-bit window (28_kernels_hgn_v2.inc:19-25): byte sum of w16 * 0x83dcd12d, f32 fma, rounded to f16
+__device__ __forceinline__ float ht_val(uint32_t w16) {
+  const uint32_t s = __builtin_amdgcn_sad_u8(w16 * 0x83dcd12du, 0u, 0u);
+  return (float)(_Float16)fmaf((float)(1024u + s), 1.732421875f / 256.f, -10.3828125f);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {  // the reference's f2bf bit trick
+  const uint32_t u = __float_as_uint(f);
+  return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+// One block per 128 x 128 tile (k_ht_deq_bf16, 28_kernels_hgn_v2.inc:386-440): 8 granules of 1 KiB (tile columns
+// 16g .. 16g+15), each of 8 blocks of 128 bytes (tile rows 16q .. 16q+15); word L of a block belongs to row L % 16,
+// column half L / 16, and carries 8 values, windows over the words L-1 (mod 32) : L.  The tile goes to LDS as f32
+// (element (r, c) at r * 128 + (c ^ (r >> 3)): the column pass reads rows 8 apart), is transformed down the columns,
+// then along the rows -- W = diag(svh) . H . G . H . diag(suh) / 128 with the butterflies in ascending stride order,
+// as the reference's fwht128 -- and leaves as bf16(v * (svh[R] / 128) * suh[C]).
+__global__ void __launch_bounds__(256) k_ht_to_bf16(const uint8_t* __restrict__ codes, const float* __restrict__ suh,
+                                                    const float* __restrict__ svh, uint16_t* __restrict__ out, int K) {
+  __shared__ float t[128 * 128];
+  const int ntx = K >> 7;
+  const int tile = blockIdx.x, ty = tile / ntx, tx = tile - ty * ntx;
+  const uint32_t* tb = (const uint32_t*)(codes + (size_t)tile * 8192);
+  const int tid = threadIdx.x, L = tid & 31;
+  for (int it = 0; it < 8; it++) {
+    const int blk = it * 8 + (tid >> 5), g = blk >> 3, q = blk & 7;
+    const uint32_t* bw = tb + g * 256 + q * 32;
+    const uint64_t V = ((uint64_t)bw[(L + 31) & 31] << 32) | bw[L];
+    const int r = q * 16 + (L & 15), c0 = g * 16 + (L >> 4) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; e++) t[r * 128 + ((c0 + e) ^ (r >> 3))] = ht_val((uint32_t)(V >> (28 - 4 * e)) & 0xffffu);
+  }
+  __syncthreads();
+  const int j = tid & 15, vec = tid >> 4;  // 16 lanes per 128-vector, 8 elements each
+  float v[8];
+  for (int pass = 0; pass < 8; pass++) {  // H down the columns
+    const int c = pass * 16 + vec;
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = t[(8 * j + i) * 128 + (c ^ j)];
+    moe_fwht128_r8(v, tid);
+#pragma unroll
+    for (int i = 0; i < 8; i++) t[(8 * j + i) * 128 + (c ^ j)] = v[i];
+  }
+  __syncthreads();
+  for (int pass = 0; pass < 8; pass++) {  // H along the rows, the planes, bf16
+    const int r = pass * 16 + vec;
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = t[r * 128 + ((8 * j + i) ^ (r >> 3))];
+    moe_fwht128_r8(v, tid);
+    const size_t R = (size_t)ty * 128 + r;
+    const float sv = svh[R] * (1.f / 128.f);
+    const int C = tx * 128 + 8 * j;
+    uint32_t pk[4];
+#pragma unroll
+    for (int i = 0; i < 8; i += 2)
+      pk[i / 2] = (uint32_t)f32_to_bf16_rne(v[i] * sv * suh[C + i]) | ((uint32_t)f32_to_bf16_rne(v[i + 1] * sv * suh[C + i + 1]) << 16);
+    *(uint4*)(out + R * K + C) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+  }
+}
+
+// q6g64 (k_q6g64_deq_bf16, 28_kernels_hgn_v2.inc:442-447,604-634): row r at r * align16(13 C / 16) = C/2 bytes of low
+// nibbles (even column = low nibble), C/4 bytes of the codes' two high bits (column k: byte k/4, bits 2 (k % 4)),
+// C/64 x (f16 scale, f16 bias); W = bf16(fma(code, scale, bias)).  One thread per eight columns.
+__global__ void __launch_bounds__(256) k_q6g64_to_bf16(const uint8_t* __restrict__ wq, uint16_t* __restrict__ out, uint64_t R,
+                                                       int C, uint64_t st) {
+  const uint64_t n8 = R * (uint64_t)(C >> 3);
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (uint64_t)gridDim.x * 256) {
+    const uint64_t r = i / (C >> 3);
+    const int c = (int)(i - r * (C >> 3)) * 8;
+    const uint8_t* row = wq + r * st;
+    const uint32_t lo = *(const uint32_t*)(row + (c >> 1));
+    const uint32_t hi = *(const uint16_t*)(row + C / 2 + (c >> 2));
+    const uint32_t sb = *(const uint32_t*)(row + 3 * (C / 4) + (c >> 6) * 4);
+    const float sc = (float)__builtin_bit_cast(_Float16, (uint16_t)(sb & 0xffffu));
+    const float bi = (float)__builtin_bit_cast(_Float16, (uint16_t)(sb >> 16));
+    uint32_t pk[4];
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      const uint32_t c0 = ((lo >> (4 * e)) & 15u) | (((hi >> (2 * e)) & 3u) << 4);
+      const uint32_t c1 = ((lo >> (4 * e + 4)) & 15u) | (((hi >> (2 * e + 2)) & 3u) << 4);
+      pk[e / 2] = (uint32_t)f32_to_bf16_rne(fmaf((float)c0, sc, bi)) | ((uint32_t)f32_to_bf16_rne(fmaf((float)c1, sc, bi)) << 16);
+    }
+    *(uint4*)(out + r * C + c) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+  }
+}
+
+MOE_API int moe_v2_dense_to_bf16(int dtype, const uint8_t* data, const float* suh, const float* svh, uint64_t rows,
+                                 uint64_t cols, uint16_t* out, moe_stream_t st) {
+  if (!data || !out || rows == 0 || cols == 0 || cols > (1u << 30)) return MOE_E_INVALID;
+  if (!moe_aligned(data, 16) || !moe_aligned(out, 16)) return MOE_E_INVALID;
+  if (dtype == MOE_DT_HT) {
+    if (rows % 128 || cols % 128 || !suh || !svh) return MOE_E_INVALID;
+    const uint64_t tiles = (rows / 128) * (cols / 128);
+    if (tiles > 0x7fffffffu) return MOE_E_INVALID;
+    k_ht_to_bf16<<<(unsigned)tiles, 256, 0, moe_s(st)>>>(data, suh, svh, out, (int)cols);
+  } else if (dtype == MOE_DT_Q6G64) {
+    if (cols % 64) return MOE_E_INVALID;
+    const uint64_t stride = ((13 * cols / 16) + 15) & ~15ull, n = (rows * (cols / 8) + 255) / 256;
+    k_q6g64_to_bf16<<<(unsigned)(n > 65536 ? 65536 : n), 256, 0, moe_s(st)>>>(data, out, rows, (int)cols, stride);
+  } else {
+    return MOE_E_UNSUPPORTED;
+  }
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
 MOE_API int moe_i4r_dequant_rows(const uint8_t* data, uint64_t rows, uint64_t cols, uint64_t row0, uint64_t nrows,
                                  float* out, moe_stream_t st) {
   if (!data || !out || cols == 0 || cols % 128 || row0 + nrows > rows) return MOE_E_INVALID;

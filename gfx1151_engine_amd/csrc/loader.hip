@@ -574,6 +574,50 @@ int upload_f16_as_f32(moe_weights* w, const FTensor& t, uint64_t want_n, const f
   return MOE_OK;
 }
 
+// An hgn v2 dense tensor (ht with its two f16 planes, or q6g64) -> a bf16 matrix in device memory.  The raw bytes and
+// the planes are staged in device memory for the conversion kernel and freed again; only the bf16 matrix stays.
+int upload_v2_dense(moe_weights* w, const FTensor& t, const FTensor* su, const FTensor* sv, uint64_t rows, uint64_t cols,
+                    hipStream_t st, const uint8_t** dev) {
+  uint64_t cells, want;
+  if (__builtin_mul_overflow(rows, cols, &cells) || cells > (UINT64_MAX >> 2)) return MOE_E_INVALID;
+  if (t.dtype == MOE_DT_HT) {
+    if (rows % 128 || cols % 128) return MOE_E_INVALID;
+    want = cells / 2;
+    if (su->dtype != MOE_DT_F16 || su->nbytes != cols * 2 || sv->dtype != MOE_DT_F16 || sv->nbytes != rows * 2) return MOE_E_INVALID;
+  } else {
+    if (cols % 64 || __builtin_mul_overflow(rows, ((13 * cols / 16) + 15) & ~15ULL, &want)) return MOE_E_INVALID;
+  }
+  if (t.nbytes != want) return MOE_E_INVALID;
+  void *raw = nullptr, *planes = nullptr, *out = nullptr;
+  auto done = [&](int rc) {
+    if (raw) (void)hipFree(raw);
+    if (planes) (void)hipFree(planes);
+    return rc;
+  };
+  MOE_HIP(hipMalloc(&out, cells * 2));
+  w->dev.push_back(out);
+  w->bytes += cells * 2;
+  if (hipMalloc(&raw, want) != hipSuccess) return done(MOE_E_STATE);
+  if (hipMemcpy(raw, t.data, want, hipMemcpyHostToDevice) != hipSuccess) return done(MOE_E_STATE);
+  const float *p_su = nullptr, *p_sv = nullptr;
+  if (t.dtype == MOE_DT_HT) {
+    std::vector<float> h(cols + rows);
+    for (uint64_t i = 0; i < cols + rows; i++) {
+      _Float16 v;
+      memcpy(&v, i < cols ? su->data + 2 * i : sv->data + 2 * (i - cols), 2);
+      h[i] = (float)v;
+    }
+    if (hipMalloc(&planes, h.size() * 4) != hipSuccess) return done(MOE_E_STATE);
+    if (hipMemcpy(planes, h.data(), h.size() * 4, hipMemcpyHostToDevice) != hipSuccess) return done(MOE_E_STATE);
+    p_su = (const float*)planes;
+    p_sv = p_su + cols;
+  }
+  int rc = moe_v2_dense_to_bf16(t.dtype, (const uint8_t*)raw, p_su, p_sv, rows, cols, (uint16_t*)out, (moe_stream_t)st);
+  if (rc == MOE_OK && hipStreamSynchronize(st) != hipSuccess) rc = MOE_E_STATE;
+  *dev = (const uint8_t*)out;
+  return done(rc);
+}
+
 // mtp: the MTP draft layer's MoE, stored as mtp.layers.<i>.mlp.* (src/gpu/parts/40_model.inc:5546-5548,5893)
 int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights* w, hipStream_t st, bool mtp) {
   auto findp = [&](const char* leaf) -> const FTensor* {
@@ -588,12 +632,33 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
   if (!rt || !gu || !dn) return MOE_E_STATE;
   // routed experts: q4cp, or hgn v2 i4r (both tensors) with its four sign-scale planes
   const bool v2 = gu->dtype == MOE_DT_I4R && dn->dtype == MOE_DT_I4R;
-  if (!hgn_dtype_ok_dense(rt->dtype) || (!v2 && (gu->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP)))
-    return MOE_E_UNSUPPORTED;  // (an hgn v2 file's hashed-trellis tensors, dtype 16, among them)
+  const auto v2_dense = [](int dt) { return dt == MOE_DT_HT || dt == MOE_DT_Q6G64; };
+  if (!(hgn_dtype_ok_dense(rt->dtype) || v2_dense(rt->dtype)) || (!v2 && (gu->dtype != MOE_DT_Q4CP || dn->dtype != MOE_DT_Q4CP)))
+    return MOE_E_UNSUPPORTED;
   int rc;
-  auto view = [&](const FTensor& t, moe_wview* v) -> int {
+  auto view = [&](const FTensor& t, moe_wview* v, const char* leaf) -> int {
     uint64_t rows, cols;
     if (!matrix_shape(MOE_FILE_HGN, t, rows, cols)) return MOE_E_INVALID;
+    if (t.dtype == MOE_DT_HT || t.dtype == MOE_DT_Q6G64) {
+      // an hgn v2 dense tensor: converted here, once, to the bf16 matrix the reference's prefill GEMM reads
+      // (v2_deq_bf16, src/gpu/parts/30_host_util.inc:1019-1031); planes: <tensor without ".weight">.suh / .svh
+      // (30_host_util.inc:840-858)
+      const FTensor *su = nullptr, *sv = nullptr;
+      if (t.dtype == MOE_DT_HT) {
+        std::string base(leaf);
+        const std::string sfx = ".weight";
+        if (base.size() > sfx.size() && base.compare(base.size() - sfx.size(), sfx.size(), sfx) == 0)
+          base.resize(base.size() - sfx.size());
+        su = findp((base + ".suh").c_str());
+        sv = findp((base + ".svh").c_str());
+        if (!su || !sv) return MOE_E_STATE;
+      }
+      v->dtype = MOE_DT_BF16;
+      v->rows = rows;
+      v->cols = cols;
+      v->scale_stride = 0;
+      return upload_v2_dense(w, t, su, sv, rows, cols, st, &v->data);
+    }
     v->dtype = t.dtype;
     v->rows = rows;
     v->cols = cols;
@@ -621,7 +686,7 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
     return upload(w, t, st, &v->data);
   };
   moe_wview vr{}, vgu{}, vdn{};
-  if ((rc = view(*rt, &vr)) || (rc = view(*gu, &vgu)) || (rc = view(*dn, &vdn))) return rc;
+  if ((rc = view(*rt, &vr, "gate.weight")) || (rc = view(*gu, &vgu, "")) || (rc = view(*dn, &vdn, ""))) return rc;
   if ((rc = moe_set_router(ctx, cl, &vr, nullptr))) return rc;
   if (v2) {
     // the planes' names (src/gpu/parts/30_host_util.inc:840-852): <tensor>.suh / <tensor>.svh without the ".weight";
@@ -649,13 +714,19 @@ int load_layer_hgn(moe_ctx* ctx, const moe_file* f, int fl, int cl, moe_weights*
     if (!su || !sd || !sx) return MOE_E_STATE;
     // q4cp, or one of the dense dtypes of the reference's generic matvec (bf16, f32, the overlay files' q8g64);
     // moe_set_shared checks that the three agree
-    auto sh_ok = [](int dt) {
-      return dt == MOE_DT_Q4CP || dt == MOE_DT_BF16 || dt == MOE_DT_F32 || dt == MOE_DT_Q8G64 || dt == MOE_DT_Q8G32;
+    // (an hgn v2 file's ht / q6g64 tensors become bf16 on their way in)
+    auto sh_ok = [&](int dt) {
+      return dt == MOE_DT_Q4CP || dt == MOE_DT_BF16 || dt == MOE_DT_F32 || dt == MOE_DT_Q8G64 || dt == MOE_DT_Q8G32 || v2_dense(dt);
     };
-    if (!sh_ok(sg->dtype) || !sh_ok(su->dtype) || !sh_ok(sd->dtype) || !hgn_dtype_ok_dense(sx->dtype))
+    if (!sh_ok(sg->dtype) || !sh_ok(su->dtype) || !sh_ok(sd->dtype) || !(hgn_dtype_ok_dense(sx->dtype) || sx->dtype == MOE_DT_Q6G64))
       return MOE_E_UNSUPPORTED;
+    // one storage for the three matrices; ht and q6g64 both arrive as bf16 and may be mixed
+    const bool all_v2 = v2_dense(sg->dtype) && v2_dense(su->dtype) && v2_dense(sd->dtype);
+    if (!all_v2 && (v2_dense(sg->dtype) || v2_dense(su->dtype) || v2_dense(sd->dtype))) return MOE_E_UNSUPPORTED;
     moe_wview a{}, b{}, c2{}, d2{};
-    if ((rc = view(*sg, &a)) || (rc = view(*su, &b)) || (rc = view(*sd, &c2)) || (rc = view(*sx, &d2))) return rc;
+    if ((rc = view(*sg, &a, "shared_expert.gate_proj.weight")) || (rc = view(*su, &b, "shared_expert.up_proj.weight")) ||
+        (rc = view(*sd, &c2, "shared_expert.down_proj.weight")) || (rc = view(*sx, &d2, "shared_expert_gate.weight")))
+      return rc;
     if ((rc = moe_set_shared(ctx, cl, &a, &b, &c2, &d2, 0))) return rc;
   }
   return MOE_OK;

@@ -11,6 +11,7 @@ import numpy as np
 
 HGN_BF16, HGN_F32, HGN_Q4CP, HGN_Q8G64, HGN_Q8G32 = 0, 1, 5, 7, 8
 HGN_F16, HGN_I4R = 2, 23  # hgn v2: f16 sign-scale planes, rotated routed experts
+HGN_HT, HGN_Q6G64 = 16, 24  # hgn v2 dense tensors: hashed-trellis codes (with .suh / .svh planes), 6-bit groups of 64
 GGML_F32, GGML_BF16, GGML_Q4_K = 0, 30, 12
 _GGML_BLOCK = {0: (1, 4), 30: (1, 2), 1: (1, 2), 12: (256, 144), 13: (256, 176), 8: (32, 34), 7: (32, 24),
                20: (32, 18), 23: (256, 136)}

@@ -35,7 +35,12 @@ enum moe_status {
 enum { MOE_DT_BF16 = 0, MOE_DT_F32 = 1, MOE_DT_F16 = 2, MOE_DT_Q4CP = 5, MOE_DT_Q8G64 = 7, MOE_DT_Q8G32 = 8,
        /* hgn v2 routed experts (src/gpu/parts/28_kernels_hgn_v2.inc:1-15): data = [rows*cols/2 codes][rows x cols/128
         * fp16 scales], no header, w = (nibble - 8) * scale, stored in the Hadamard-rotated domain */
-       MOE_DT_I4R = 23 };
+       MOE_DT_I4R = 23,
+       /* hgn v2 dense tensors (28_kernels_hgn_v2.inc:1-15,226-231,442-447): "ht" = 4-bit hashed-trellis codes in
+        * 128 x 128 tiles, Hadamard-rotated domain, with f16 planes <name>.suh [cols] / <name>.svh [rows]; q6g64 = 6-bit
+        * codes with (fp16 scale, fp16 bias) per 64 columns.  Accepted by moe_v2_dense_to_bf16 and by the file loader
+        * (which converts them), not by moe_set_router / moe_set_shared. */
+       MOE_DT_HT = 16, MOE_DT_Q6G64 = 24 };
 /* Q4_K: every kernel of the path.  Q5_K (gate/up), Q5_1 and Q8_0 (down) — the mix of the reference's GGUF
  * checkpoints (src/gpu/parts/30_host_util.inc:399-405) — and IQ4_NL / IQ4_XS (src/gguf.h:376-407):
  * bit-exact dequantisation, the stateless general GEMV kernels (moe_gg_gemv), and inside moe_forward integer-dot
@@ -333,6 +338,12 @@ int moe_i4r_dequant_rows(const uint8_t* data, uint64_t rows, uint64_t cols, uint
  * (what moe_lut_up_raw reads). */
 int moe_v2_rot(const float* x, uint64_t xs, void* y, uint64_t ys, const float* pre, const float* post, int n, int P,
                int out_f16, moe_stream_t st);
+/* v2_deq_bf16 (src/gpu/parts/30_host_util.inc:1019-1031; k_ht_deq_bf16 / k_q6g64_deq_bf16, 28_kernels_hgn_v2.inc:386-440,
+ * 604-634): an hgn v2 dense tensor (MOE_DT_HT or MOE_DT_Q6G64) as the bf16 matrix out[rows][cols] the reference's prefill
+ * GEMM reads, bit for bit.  ht: rows % 128 == 0, cols % 128 == 0, suh [cols] / svh [rows] = the tensor's f16 planes as
+ * f32; q6g64: cols % 64 == 0, planes unused (may be NULL).  data and out 16-byte aligned. */
+int moe_v2_dense_to_bf16(int dtype, const uint8_t* data, const float* suh, const float* svh, uint64_t rows,
+                         uint64_t cols, uint16_t* out, moe_stream_t st);
 /* k_i4r_mid (28_kernels_hgn_v2.inc:105-150): per slot, g | u = svh_gu . H(guv) / sqrt(128), h = silu(g) * u,
  * out = H(suh_dn . h) / sqrt(128).  guv: [nslots][gs] f32 or f16 (2*mid used), out: [nslots][os] f32, or f16 in
  * layout 1 (what moe_lut_down reads).  mid % 128 == 0, 2*mid <= 2048. */

@@ -21,6 +21,9 @@
  *   tools/moe_lut_test.cu:936-948, tools/v2repro/v2enc.py:87-101  hgn v2 i4r rows: (nibble - 8) * fp16 scale per 128
  *   src/gpu/parts/27_kernels_moe_lut.inc:44-65, 28_kernels_hgn_v2.inc:62-150, 40_model.inc:1638-1656
  *                        hgn v2 rotated experts: 128-block Hadamard on the activations around each projection
+ *   src/gpu/parts/28_kernels_hgn_v2.inc:19-25,226-231,386-440,442-447,604-634, 30_host_util.inc:1019-1031,
+ *   tools/v2repro/v2enc.py:48-84  hgn v2 dense tensors: ht (hashed-trellis) values, tile layout and un-rotation
+ *                        to bf16; q6g64 rows to bf16
  *
  * Pinning status of every function is listed in oracle/README.md; each one is
  * checked in tests/ against the reference's own code built under oracle/_ref
@@ -332,6 +335,104 @@ ORC_API void orc_v2_rot(const float* x, float* y, const float* pre, const float*
     for (int i = 0; i < 128; i++) y[b * 128 + i] = v[i] * kRs128 * (post ? post[b * 128 + i] : 1.f);
   }
 }
+static inline uint16_t f2bf_ref(float f);
+/* ---- hgn v2 dense tensors: "ht" (dtype 16) and q6g64 (dtype 24) -> the bf16 matrix the reference's prefill GEMM
+ * reads (v2_deq_bf16, src/gpu/parts/30_host_util.inc:1019-1031) ----
+ *
+ * ht value of a 16-bit trellis window (28_kernels_hgn_v2.inc:19-25; tools/v2repro/v2enc.py:48-61): the byte sum s of
+ * w16 * 0x83dcd12d (mod 2^32), then f16(fma(1024 + s, 1.732421875 / 256, -10.3828125)) with the fma in f32. */
+static inline uint16_t f32_to_fp16_rne(float f) { /* round to nearest even; finite |f| < 65520 */
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+  const uint32_t a = u & 0x7fffffffu;
+  if (a < 0x38800000u) { /* below the smallest normal f16: a subnormal, in units of 2^-24 */
+    float m;
+    memcpy(&m, &a, 4);
+    return sign | (uint16_t)lrintf(m * 16777216.f); /* lrintf: nearest even in the default rounding mode */
+  }
+  const uint32_t r = a + 0xfffu + ((a >> 13) & 1u); /* drop 13 mantissa bits */
+  return sign | (uint16_t)((r - 0x38000000u) >> 13);
+}
+ORC_API float orc_ht_value(uint32_t w16) {
+  const uint32_t t = (w16 & 0xffffu) * 0x83dcd12du;
+  const uint32_t s = (t & 0xff) + ((t >> 8) & 0xff) + ((t >> 16) & 0xff) + (t >> 24);
+  const float v = fmaf((float)(1024u + s), 1.732421875f / 256.f, -10.3828125f);
+  return orc_fp16_to_f32(f32_to_fp16_rne(v));
+}
+/* The code stream of an ht tensor [O][K] -> its values G[O][K] in the rotated domain.  Layout
+ * (28_kernels_hgn_v2.inc:226-231,386-412; v2enc.py:67-84): tiles of 128 x 128, tile (ty, tx) = 8 granules of 1 KiB at
+ * ((ty * K/128 + tx) * 8 + g) * 1024; granule g = tile columns 16g .. 16g+15; its 128-byte block q = tile rows
+ * 16q .. 16q+15; in a block, 32-bit word L (little endian) belongs to row L % 16 and column half L / 16 and carries 8
+ * values: value e = the 16 bits of (word L-1 mod 32 : word L) that start 28 - 4e bits above the low end of word L. */
+ORC_API void orc_ht_decode(const uint8_t* codes, uint64_t O, uint64_t K, float* G) {
+  const uint64_t ntx = K / 128;
+  for (uint64_t ty = 0; ty < O / 128; ty++)
+    for (uint64_t tx = 0; tx < ntx; tx++)
+      for (int g = 0; g < 8; g++)
+        for (int q = 0; q < 8; q++) {
+          const uint8_t* blk = codes + ((ty * ntx + tx) * 8 + g) * 1024 + q * 128;
+          uint32_t w[32];
+          memcpy(w, blk, 128);
+          for (int L = 0; L < 32; L++) {
+            const uint64_t V = ((uint64_t)w[(L + 31) & 31] << 32) | w[L];
+            const uint64_t r = ty * 128 + q * 16 + (L & 15), c0 = tx * 128 + g * 16 + (L >> 4) * 8;
+            for (int e = 0; e < 8; e++) G[r * K + c0 + e] = orc_ht_value((uint32_t)(V >> (28 - 4 * e)) & 0xffffu);
+          }
+        }
+}
+/* k_ht_deq_bf16 (28_kernels_hgn_v2.inc:386-440): per tile, the unnormalised Hadamard transform down the columns, then
+ * along the rows, then bf16(v * (svh[R] / 128) * suh[C]) -- W = diag(svh) . H . G . H . diag(suh) / 128.
+ * k_q6g64_deq_bf16 (28_kernels_hgn_v2.inc:442-447,604-634): row r at r * align16(13 C / 16): C/2 bytes of low
+ * nibbles (even column = low nibble), C/4 bytes of the codes' two high bits (column k: byte k/4, bits 2(k%4)),
+ * C/64 x (f16 scale, f16 bias); W = bf16(fma(code, scale, bias)).
+ * suh [cols] / svh [rows]: the f16 planes as f32 (ht only).  Returns 0, or -1 for a dtype / shape outside the two. */
+ORC_API int orc_v2_dense_bf16(int dtype, const uint8_t* data, const float* suh, const float* svh, uint64_t rows,
+                              uint64_t cols, uint16_t* out) {
+  if (dtype == 16) {
+    if (rows % 128 || cols % 128 || !suh || !svh) return -1;
+    float* G = (float*)malloc(rows * cols * 4);
+    orc_ht_decode(data, rows, cols, G);
+    float v[128];
+    for (uint64_t ty = 0; ty < rows / 128; ty++)
+      for (uint64_t tx = 0; tx < cols / 128; tx++) {
+        float* t = G + ty * 128 * cols + tx * 128;
+        for (int c = 0; c < 128; c++) {
+          for (int r = 0; r < 128; r++) v[r] = t[(uint64_t)r * cols + c];
+          fwht128(v);
+          for (int r = 0; r < 128; r++) t[(uint64_t)r * cols + c] = v[r];
+        }
+        for (int r = 0; r < 128; r++) {
+          fwht128(t + (uint64_t)r * cols);
+          const uint64_t R = ty * 128 + r;
+          const float sv = svh[R] * (1.f / 128.f);
+          for (int c = 0; c < 128; c++) {
+            const uint64_t C = tx * 128 + c;
+            out[R * cols + C] = f2bf_ref(t[(uint64_t)r * cols + c] * sv * suh[C]);
+          }
+        }
+      }
+    free(G);
+    return 0;
+  }
+  if (dtype == 24) {
+    if (cols % 64) return -1;
+    const uint64_t st = ((13 * cols / 16) + 15) & ~15ull;
+    for (uint64_t r = 0; r < rows; r++) {
+      const uint8_t* row = data + r * st;
+      for (uint64_t c = 0; c < cols; c++) {
+        const uint32_t lo = (row[c >> 1] >> (4 * (c & 1))) & 15u;
+        const uint32_t hi = (row[cols / 2 + (c >> 2)] >> (2 * (c & 3))) & 3u;
+        uint16_t sb[2];
+        memcpy(sb, row + 3 * cols / 4 + (c >> 6) * 4, 4);
+        out[r * cols + c] = f2bf_ref(fmaf((float)(lo | (hi << 4)), orc_fp16_to_f32(sb[0]), orc_fp16_to_f32(sb[1])));
+      }
+    }
+    return 0;
+  }
+  return -1;
+}
+
 ORC_API void orc_mat_rows(const orc_mat* W, uint64_t row0, uint64_t nrows, float* out) {
   for (uint64_t r = 0; r < nrows; r++) mat_row(W, row0 + r, out + r * W->cols);
 }

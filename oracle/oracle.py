@@ -306,6 +306,31 @@ def v2_rot(x, pre=None, post=None):
     return out
 
 
+def ht_value(w16):
+    lib().orc_ht_value.restype = C.c_float
+    return lib().orc_ht_value(C.c_uint32(int(w16)))
+
+
+def ht_decode(codes, rows, cols):
+    """ht code stream -> its values G [rows][cols] in the rotated domain."""
+    codes = _c(codes, np.uint8)
+    assert codes.size == rows * cols // 2
+    out = np.empty((rows, cols), np.float32)
+    lib().orc_ht_decode(_p(codes), C.c_uint64(rows), C.c_uint64(cols), _p(out))
+    return out
+
+
+def v2_dense_bf16(dtype, data, rows, cols, suh=None, svh=None):
+    """hgn v2 dense tensor (16 = ht with its planes as f32, 24 = q6g64) -> bf16 bits [rows][cols] (uint16)."""
+    data = _c(data, np.uint8)
+    out = np.empty((rows, cols), np.uint16)
+    suh = _c(suh, np.float32) if suh is not None else None
+    svh = _c(svh, np.float32) if svh is not None else None
+    rc = lib().orc_v2_dense_bf16(int(dtype), _p(data), _p(suh), _p(svh), C.c_uint64(rows), C.c_uint64(cols), _p(out))
+    assert rc == 0, rc
+    return out
+
+
 def num_threads():
     return lib().orc_num_threads()
 

@@ -596,3 +596,62 @@ def test_load_gguf_mixed_types(tmp_path):
     m.close()
     m2.close()
     w.free()
+
+
+@pytest.mark.gpu
+def test_hgn_v2_file_with_ht_and_q6g64_dense_tensors(tmp_path):
+    """An hgn v2 file whose router and shared expert are "ht" tensors (dtype 16, with their .suh / .svh planes) and whose
+    shared-expert gate is q6g64 (dtype 24): moe_load_layers turns them into the bf16 matrices of the reference's
+    v2_deq_bf16 (src/gpu/parts/30_host_util.inc:1019-1031), so the loaded layer equals, bit for bit, the same layer
+    registered with those bf16 matrices, and stays within the layer tolerance of the oracle.  A file without one of the
+    planes is refused."""
+    import torch
+    d, mid, ne, k = 256, 128, 128, 3
+    rng = np.random.default_rng(52)
+    hl = HostLayer(rng, d, mid, ne, k, fmt="i4r", router_dtype="bf16", shared_dense="bf16")
+    raw, extra = {}, []
+
+    def ht(leaf, rows, cols, scale):
+        codes = rng.integers(0, 256, rows * cols // 2, dtype=np.uint8)
+        pl = [(rng.uniform(0.5, 1.5, n) * rng.choice([-1, 1], n) * s).astype(np.float16) for n, s in ((cols, scale), (rows, 1.0))]
+        raw[f"layers.0.mlp.{leaf}.weight"] = (files.HGN_HT, codes)
+        extra.extend([(f"layers.0.mlp.{leaf}.suh", files.HGN_F16, [cols], pl[0]), (f"layers.0.mlp.{leaf}.svh", files.HGN_F16, [rows], pl[1])])
+        return O.v2_dense_bf16(16, codes, rows, cols, pl[0].astype(np.float32), pl[1].astype(np.float32))
+
+    hl.router = ht("gate", ne, d, 0.02)
+    hl.shared[0] = ht("shared_expert.gate_proj", mid, d, 0.05)
+    hl.shared[1] = ht("shared_expert.up_proj", mid, d, 0.05)
+    hl.shared[2] = ht("shared_expert.down_proj", d, mid, 0.05)
+    st = (13 * d // 16 + 15) & ~15
+    q6 = rng.integers(0, 256, (1, st), dtype=np.uint8)
+    q6[0, 3 * d // 4: 3 * d // 4 + d // 64 * 4] = np.stack([rng.uniform(5e-4, 2e-3, d // 64), rng.uniform(-0.03, -0.01, d // 64)],
+                                                          -1).astype(np.float16).view(np.uint8).reshape(-1)
+    raw["layers.0.mlp.shared_expert_gate.weight"] = (files.HGN_Q6G64, q6)
+    sx_bits = O.v2_dense_bf16(24, q6, 1, d)
+    hl.shared[3] = (sx_bits.astype(np.uint32) << 16).view(np.float32)  # the gate as exact f32 for the direct registration
+    ts = [(n, raw[n][0], dims, raw[n][1]) if n in raw else (n, dt, dims, a) for n, dt, dims, a in files.hgn_layer_tensors(0, hl)] + extra
+    p = tmp_path / "v2dense.hgn"
+    files.write_hgn(p, ts)
+    f = capi.ModelFile(p)
+    m = capi.Moe(d, mid, ne, k, layers=1, max_tokens=80)
+    w = f.load_layers(m, 0, 0, 1)
+    f.close()
+    m2, keep = hl.to_gpu(max_tokens=80)
+    for T in (1, 9, 80):
+        x = np.random.default_rng(T).standard_normal((T, d), dtype=np.float32)
+        want, io, _ = O.moe_layer(hl.oracle_layer(), x)
+        xg = torch.from_numpy(x).cuda()
+        y = m.forward(0, xg).cpu().numpy()
+        ids, _ = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+        assert np.abs(y - want).max() <= 2e-3 * np.abs(want).max(), T
+        assert (y == m2.forward(0, xg).cpu().numpy()).all(), T
+    del m, m2
+    w.free()
+    p2 = tmp_path / "noplane.hgn"
+    files.write_hgn(p2, [t for t in ts if not t[0].endswith("mlp.gate.svh")])
+    f = capi.ModelFile(p2)
+    m = capi.Moe(d, mid, ne, k, layers=1, max_tokens=8)
+    wh = C.c_void_p()
+    assert capi.lib().moe_load_layers(m.h, f.h, 0, 0, 1, C.byref(wh), capi.stream()) == -3
+    f.close()

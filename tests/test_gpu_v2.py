@@ -218,3 +218,44 @@ def test_v2_layer_under_graph_capture(oracle, T):
             torch.cuda.synchronize()
             assert torch.equal(y, eager[(i + 1) % 3])
     m.close()
+
+
+def _q6g64_blob(rng, rows, cols):
+    """random q6g64 rows: codes, then (f16 scale, f16 bias) per 64 columns, row stride align16(13 cols / 16)"""
+    st = (13 * cols // 16 + 15) & ~15
+    blob = rng.integers(0, 256, (rows, st), dtype=np.uint8)
+    sb = np.stack([rng.uniform(0.005, 0.03, (rows, cols // 64)), rng.uniform(-1, 1, (rows, cols // 64))], -1).astype(np.float16)
+    blob[:, 3 * cols // 4: 3 * cols // 4 + cols // 64 * 4] = sb.view(np.uint8).reshape(rows, -1)
+    return blob
+
+
+def _planes(rng, n):
+    return (rng.uniform(0.5, 1.5, n) * rng.choice([-1, 1], n)).astype(np.float16).astype(np.float32)
+
+
+def test_v2_dense_tensors_to_bf16_bit_exact(capi, oracle):
+    """ht (dtype 16) and q6g64 (dtype 24) -> the bf16 matrix of the reference's v2_deq_bf16, bit for bit against the
+    oracle (ht: random code streams -- every stream is a valid tensor --, several tiles both ways, signed planes)."""
+    rng = np.random.default_rng(71)
+    for rows, cols in ((128, 128), (256, 384), (384, 1024)):
+        codes = rng.integers(0, 256, rows * cols // 2, dtype=np.uint8)
+        suh, svh = _planes(rng, cols), _planes(rng, rows)
+        want = oracle.v2_dense_bf16(16, codes, rows, cols, suh, svh)
+        got = capi.v2_dense_to_bf16(capi.HT, gpu(codes), rows, cols, gpu(suh), gpu(svh)).cpu().numpy().view(np.uint16)
+        assert (got == want).all(), (rows, cols)
+    for rows, cols in ((1, 256), (5, 192), (130, 3072)):
+        blob = _q6g64_blob(rng, rows, cols)
+        want = oracle.v2_dense_bf16(24, blob, rows, cols)
+        got = capi.v2_dense_to_bf16(capi.Q6G64, gpu(blob), rows, cols).cpu().numpy().view(np.uint16)
+        assert (got == want).all(), (rows, cols)
+    # shapes off the grid, a missing plane, another dtype
+    import torch
+    out = torch.empty(128 * 128, dtype=torch.int16, device="cuda")
+    c = gpu(np.zeros(128 * 128, np.uint8))
+    f = gpu(np.ones(128, np.float32))
+    L = capi.lib()
+    u64 = capi.u64
+    assert L.moe_v2_dense_to_bf16(16, capi.ptr(c), capi.ptr(f), capi.ptr(f), u64(64), u64(128), capi.ptr(out), capi.stream()) == -2
+    assert L.moe_v2_dense_to_bf16(16, capi.ptr(c), None, capi.ptr(f), u64(128), u64(128), capi.ptr(out), capi.stream()) == -2
+    assert L.moe_v2_dense_to_bf16(24, capi.ptr(c), None, None, u64(4), u64(96), capi.ptr(out), capi.stream()) == -2
+    assert L.moe_v2_dense_to_bf16(5, capi.ptr(c), None, None, u64(128), u64(128), capi.ptr(out), capi.stream()) == -1

@@ -508,3 +508,104 @@ def test_hc_writeback_closed_forms(oracle):
     v3 = (out3.astype(np.uint32) << 16).view(np.float32)
     for b, inj in enumerate((1.5, 0.5, 1.75, 1.0)):
         assert (v3[0, b] == inj * y3[0]).all(), (b, v3[0, b])
+
+
+# ---------- hgn v2 dense tensors: ht (dtype 16), q6g64 (dtype 24) ----------
+def _bf16_to_f64(b):
+    return (np.asarray(b, np.uint16).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+def test_ht_alphabet(oracle):
+    """The 65536 values of the hashed alphabet.  w16 = 0 hashes to byte sum 0: 1024 * 1.732421875 / 256 - 10.3828125 =
+    -3.453125, exact in f16.  The byte sum of a well-mixed 32-bit word is the sum of four uniform bytes (mean 510,
+    variance 4 * (256^2 - 1) / 12), so the alphabet is a unit normal's: mean -0.0017, standard deviation 1.0003 -- which
+    fixes both constants.  Every value is an f16, rounded as numpy rounds f32 to f16 (the oracle converts by hand)."""
+    v = np.array([oracle.ht_value(i) for i in range(65536)], np.float32)
+    assert v[0] == np.float32(-3.453125)
+    assert abs(float(v.mean()) + 0.0017) < 5e-3 and abs(float(v.std()) - 1.0003) < 5e-3
+    assert (v.astype(np.float16).astype(np.float32) == v).all()
+    w = np.arange(65536, dtype=np.uint64)
+    t = (w * np.uint64(0x83DCD12D)) & np.uint64(0xFFFFFFFF)
+    s = (t & 0xFF) + ((t >> 8) & 0xFF) + ((t >> 16) & 0xFF) + (t >> 24)
+    exact = (1024 + s).astype(np.float64) * float(np.float32(1.732421875 / 256)) + (-10.3828125)  # exact in float64
+    assert (np.float32(exact).astype(np.float16).astype(np.float32) == v).all()
+
+
+def test_ht_decode_against_the_reference_encoder(oracle, tmp_path):
+    """The reference's own ht encoder (tools/v2repro/htenc.cc, built as oracle/_ref/htenc) searches the code stream whose
+    decoded values are nearest to a target, in the official tile layout, and prints the mean squared error it reached.
+    Decoding its stream here must give that same error: a wrong tile / granule / row / column index, a window taken from
+    the wrong bits or the wrong neighbouring word would leave the decoded values uncorrelated with the target (relative
+    error 1.4 instead of 0.24)."""
+    import os
+    import shutil
+    import subprocess
+    exe = os.path.join(os.path.dirname(oracle.__file__), "_ref", "htenc")
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/htenc is not built (the reference tree is not here)")
+    shutil.copy(exe, tmp_path / "htenc")  # the encoder reads ht_lut.f32 from its own directory
+    np.array([oracle.ht_value(i) for i in range(65536)], np.float32).tofile(tmp_path / "ht_lut.f32")
+    rng = np.random.default_rng(41)
+    rows, cols = 256, 384  # 2 x 3 tiles
+    G = rng.standard_normal((rows, cols)).astype(np.float32)
+    G.tofile(tmp_path / "t.f32")
+    r = subprocess.run([str(tmp_path / "htenc"), "t.f32", str(rows), str(cols), "o.codes", "16", "2"], cwd=tmp_path,
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    said = float(r.stderr.split("mse")[1].split()[0])
+    got = oracle.ht_decode(np.fromfile(tmp_path / "o.codes", np.uint8), rows, cols)
+    mse = float(((got.astype(np.float64) - G) ** 2).mean())
+    assert abs(mse - said) <= 1e-5 * said, (mse, said)
+    assert mse < 0.08
+
+
+def test_v2_dense_ht_is_the_unrotated_matrix(oracle):
+    """bf16 W of an ht tensor = diag(svh) . H . G . H . diag(suh) / 128 (H = scipy's Sylvester matrix, per 128 x 128 tile),
+    evaluated in float64 from the decoded values: planes on the right sides, both transforms, the scale.  bf16 rounding
+    only (2^-8 relative), an all-zero plane gives (signed) zeros."""
+    from scipy.linalg import hadamard
+    rng = np.random.default_rng(42)
+    rows, cols = 256, 384
+    codes = rng.integers(0, 256, rows * cols // 2, dtype=np.uint8)
+    suh = (rng.uniform(0.5, 1.5, cols) * rng.choice([-1, 1], cols)).astype(np.float16).astype(np.float32)
+    svh = (rng.uniform(0.5, 1.5, rows) * rng.choice([-1, 1], rows)).astype(np.float16).astype(np.float32)
+    G = oracle.ht_decode(codes, rows, cols).astype(np.float64)
+    H = hadamard(128).astype(np.float64)
+    W = np.empty((rows, cols))
+    for r in range(0, rows, 128):
+        for c in range(0, cols, 128):
+            W[r:r + 128, c:c + 128] = H @ G[r:r + 128, c:c + 128] @ H / 128.0
+    W = W * svh[:, None].astype(np.float64) * suh[None, :].astype(np.float64)
+    got = _bf16_to_f64(oracle.v2_dense_bf16(16, codes, rows, cols, suh, svh))
+    assert np.abs(got - W).max() <= 2.0 ** -8 * np.abs(W).max()
+    assert (np.abs(got - W) <= 2.0 ** -8 * np.abs(W) + 1e-6).all()
+    assert not (oracle.v2_dense_bf16(16, codes, rows, cols, suh * 0, svh) & 0x7fff).any()
+
+
+def test_v2_dense_q6g64_closed_form(oracle):
+    """q6g64 rows packed here element by element from the published layout (row stride align16(13 C / 16): C/2 bytes of
+    low nibbles, even column in the low half; C/4 bytes of high bit pairs, column k in byte k/4 at bits 2 (k % 4); C/64
+    x (f16 scale, f16 bias)).  Scale 1 / bias 0: the matrix is the codes themselves (0 .. 63, exact in bf16).  General
+    scales: code * scale + bias in float64 within bf16 rounding."""
+    rng = np.random.default_rng(43)
+    R, Cc = 5, 192
+    st = (13 * Cc // 16 + 15) & ~15
+    code = rng.integers(0, 64, (R, Cc))
+    code[0, :64] = np.arange(64)
+    for unit in (True, False):
+        sc = np.ones((R, Cc // 64), np.float16) if unit else rng.uniform(0.01, 0.05, (R, Cc // 64)).astype(np.float16)
+        bi = np.zeros((R, Cc // 64), np.float16) if unit else rng.uniform(-1, 1, (R, Cc // 64)).astype(np.float16)
+        blob = np.zeros((R, st), np.uint8)
+        for r in range(R):
+            for k in range(Cc):
+                blob[r, k // 2] |= (int(code[r, k]) & 15) << (4 * (k % 2))
+                blob[r, Cc // 2 + k // 4] |= (int(code[r, k]) >> 4) << (2 * (k % 4))
+            for g in range(Cc // 64):
+                blob[r, 3 * Cc // 4 + 4 * g: 3 * Cc // 4 + 4 * g + 2] = np.frombuffer(sc[r, g].tobytes(), np.uint8)
+                blob[r, 3 * Cc // 4 + 4 * g + 2: 3 * Cc // 4 + 4 * g + 4] = np.frombuffer(bi[r, g].tobytes(), np.uint8)
+        got = _bf16_to_f64(oracle.v2_dense_bf16(24, blob, R, Cc))
+        want = code * np.repeat(sc.astype(np.float64), 64, axis=1) + np.repeat(bi.astype(np.float64), 64, axis=1)
+        if unit:
+            assert (got == want).all()
+        else:
+            assert (np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-9).all()
