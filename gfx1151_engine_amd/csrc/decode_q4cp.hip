@@ -436,22 +436,33 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
     const float* wcb = shared ? A.shd.cb : A.dn.cb;
     const uint64_t wss = shared ? A.shd.ss : A.dn.ss;
     const int wgsh = shared ? A.shd.gsh : A.dn.gsh;
-    const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
+    // (an unconditional load -- the shared expert's lanes read slot 0's id and drop it: under a per-lane branch the
+    // compiler waits for the id before it issues anything else.  Indices in 32 bits: a 64-bit product per lane is two
+    // quarter-rate instructions.)
+    const int e_any = ids[tok * id_stride + (shared ? 0 : s)];
+    const uint32_t e = shared ? 0u : (uint32_t)e_any;
     XG x;
     XF xh;
     if (LUT) load_xf(xh, hid_f32 + ((size_t)tok * nslots + s) * mid + (size_t)g * 32);
-    else load_xg(x, hplanes, hmeta, ((size_t)tok * nslots + s) * G + g);
+    else load_xg(x, hplanes, hmeta, (size_t)((tok * nslots + s) * G + g));
     const float* lt = lutmem + (shared ? LUT_DW : 0) + (lane & 31);
     const float a = wcb[1] - wcb[0], b = fmaf(8.f, a, wcb[0]);
-    const uint64_t row0 = (shared ? 0 : (uint64_t)e * d) + r0;
-    const uint8_t* cp = wcodes + row0 * rb + (size_t)g * 16;
-    const uint8_t* sp = wscales + row0 * wss + (g >> wgsh) * 2;
+    const uint32_t row0 = e * (uint32_t)d + (uint32_t)r0;  // < experts * d: the launcher checks that it fits
+    const uint8_t* cp = wcodes + (uint64_t)row0 * (uint32_t)rb + (uint32_t)g * 16;
+    const uint8_t* sp = wscales + (uint64_t)row0 * (uint32_t)wss + (uint32_t)(g >> wgsh) * 2;
     uint4 cw[ROWS];
     __half sc[ROWS];
+    {
+      // (row addresses by repeated addition: wss is a per-lane value, and r * wss as a 64-bit product costs two
+      // quarter-rate instructions per row)
+      const uint8_t *cpr = cp, *spr = sp;
 #pragma unroll
-    for (int r = 0; r < ROWS; r++) {
-      cw[r] = *(const uint4*)(cp + r * rb);
-      sc[r] = *(const __half*)(sp + r * wss);
+      for (int r = 0; r < ROWS; r++) {
+        cw[r] = *(const uint4*)cpr;
+        sc[r] = *(const __half*)spr;
+        cpr += rb;
+        spr += wss;
+      }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first dot product
 #pragma unroll
@@ -648,6 +659,7 @@ int moe_launch_dec_dn_lut(const moe_wview* dn, const moe_wview* sh_down, const f
   A.dn = decw(dn);
   A.shd = decw(sh_down);
   A.sh_logit = sh_logit;
+  if (dn->rows > 0xffffffffull) return MOE_E_UNSUPPORTED;  // (row numbers are 32-bit in the kernel)
   const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
   constexpr int lds = 2 * LUT_DW * 4;
   if (d % MOE_DN_ROWS == 0)
@@ -701,6 +713,7 @@ int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float
   A.sh_logit = sh_logit;
   A.out_sh = out_sh;
   if (!A.dn.cb) return MOE_E_STATE;
+  if (dn->rows > 0xffffffffull) return MOE_E_UNSUPPORTED;  // (row numbers are 32-bit in the kernel)
   const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
   // MOE_DN_ROWS rows per block where that divides d (d = 3072: 512 blocks, two per CU), else 8
   if (d % MOE_DN_ROWS == 0)

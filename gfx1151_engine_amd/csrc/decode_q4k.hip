@@ -262,8 +262,10 @@ __global__ void __launch_bounds__(256) k_dec4k_dn(Dn4kArgs A, const uint32_t* __
     const int s = live ? s_raw : 0, u = live ? u_raw : 0;
     const float mlive = live ? 1.f : 0.f;
     const bool shared = has_shared && s == nslots - 1;
-    const int e = shared ? 0 : ids[(size_t)tok * id_stride + s];
-    const uint8_t* base = (shared ? A.sh_down : A.down + (uint64_t)e * d * rb) + (uint64_t)r0 * rb + (size_t)(u >> 2) * 144;
+    // (an unconditional load: under a per-lane branch the compiler waits for the id before it issues anything else)
+    const int e_any = ids[tok * id_stride + (shared ? 0 : s)];
+    const uint32_t e = shared ? 0u : (uint32_t)e_any;
+    const uint8_t* base = (shared ? A.sh_down : A.down + (uint64_t)(e * (uint32_t)d) * rb) + (uint64_t)r0 * rb + (uint32_t)(u >> 2) * 144;
     const int jj = u & 3;
     XU x;
     load_xu(x, hplanes, hmeta, (((size_t)tok * nslots + s) * U + u) * 2);
@@ -679,8 +681,10 @@ __global__ void __launch_bounds__(320) k_decgg_dn(DnGgArgs A, const uint32_t* __
     const float mlive = live ? 1.f : 0.f;
     const int t = shw ? A.tsh : A.tdn;
     const uint64_t rb = ggu_row_bytes(t, (uint64_t)mid);
-    const int e = shw ? 0 : ids[(size_t)tok * id_stride + s];
-    const uint8_t* base = (shw ? A.sh_down : A.down + (uint64_t)e * d * rb) + (uint64_t)r0 * rb;
+    // (an unconditional load: under a per-lane branch the compiler waits for the id before it issues anything else)
+    const int e_any = ids[tok * id_stride + (shw ? 0 : s)];
+    const uint32_t e = shw ? 0u : (uint32_t)e_any;
+    const uint8_t* base = (shw ? A.sh_down : A.down + (uint64_t)(e * (uint32_t)d) * rb) + (uint64_t)r0 * rb;
     XU x;
     load_xu(x, hplanes, hmeta, (((size_t)tok * nslots + s) * U + ul) * 2);
     GGU_SWITCH(t, ggu_dn_rows<T>(base, mid, ul, mlive, x, u_raw == 0 && okslot, part[s]));
