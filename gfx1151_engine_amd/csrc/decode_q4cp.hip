@@ -191,7 +191,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   __shared__ uint32_t pk[QV4_GROUP_DW];
   __shared__ int sel_ids[64];
   __shared__ float sel_ws[64];
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));  // (a scalar: see e)
   const int G = d / 32;
   int s = blockIdx.y, nslots = gridDim.y - (NPL > 0 ? 1 : 0), e = 0, first = 0, npairs = 1;
   if (NPL > 0 && s == nslots) {
@@ -231,6 +231,9 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     shared = s >= kpt;
     e = shared ? 0 : ids[(size_t)blockIdx.z * id_stride + s];
   }
+  // the expert number is the same in every lane: as a scalar, the row and byte offsets that follow from it are scalar
+  // arithmetic instead of 64-bit products per lane (quarter-rate instructions between the selection and the first load)
+  e = __builtin_amdgcn_readfirstlane(e);
   const DecW Wg = shared ? A.shg : A.gu;  // block-uniform choice, by value
   const DecW Wu = shared ? A.shu : A.gu;
   const float *lutg = lutmem + (lane & 31), *lutu = lutg;

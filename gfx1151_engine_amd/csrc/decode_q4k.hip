@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(512, 4) k_dec4k_gu(Gu4kArgs A, const uint32_t*
     }
     return;
   }
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int U = d / 64;
   const bool shared = s >= kpt;
   const uint64_t rb = (uint64_t)(d / 256) * 144;
@@ -164,6 +164,7 @@ __global__ void __launch_bounds__(512, 4) k_dec4k_gu(Gu4kArgs A, const uint32_t*
   } else if (!shared) {
     e = ids[(size_t)tok * id_stride + s];
   }
+  e = __builtin_amdgcn_readfirstlane(e);  // (the same in every lane: as a scalar, the offsets below are scalar arithmetic)
   const uint8_t* gbase = shared ? A.sh_gate : A.gate + (uint64_t)e * mid * rb;
   const uint8_t* ubase = shared ? A.sh_up : A.up + (uint64_t)e * mid * rb;
   const int r0 = blockIdx.x * G4_ROWS + 4 * wv;
@@ -577,6 +578,7 @@ __global__ void __launch_bounds__(512, 4) k_decgg_gu(GuGgArgs A, const uint32_t*
       e = ids_in[(size_t)tok * id_stride + s];  // (NPL == 0: the ids come from the router's launches)
     }
   }
+  e = __builtin_amdgcn_readfirstlane(e);  // (the same in every lane: as a scalar, the offsets below are scalar arithmetic)
   const int t = shared ? A.tsh : A.tgu;
   const uint64_t rb = ggu_row_bytes(t, (uint64_t)d);
   const uint8_t* gbase = shared ? A.sh_gate : A.gate + (uint64_t)e * mid * rb;
