@@ -38,6 +38,22 @@ PMC_TRAFFIC = {("prefill", "q4cp", 16384): ("prefill_q4cp_T16384_hbm_traffic.txt
                ("prefill", "q4k", 8192): ("prefill_q4k_T8192_hbm_traffic.txt", "k_moe_gemm_q4cp<true", "max")}
 
 
+_timing_capi = False
+
+
+def timing_capi():
+    """A second binding of the C ABI, on the library's timing twin (the same sources built with -DMOE_TIMING_HOOKS, the
+    only build in which a stage's launches can be left out), or None when that library is not there.  Used to time the
+    dominant launch of a small-batch call as the difference of two step loops; the step loop that gives `value` runs
+    on the default library."""
+    global _timing_capi
+    if _timing_capi is False:
+        from gfx1151_engine_amd import LIB_TIMING, capi
+        path = os.environ.get("MI355MOE_LIB_TIMING") or (None if os.environ.get("MI355MOE_LIB") else LIB_TIMING)
+        _timing_capi = capi.second_binding(path) if path and os.path.exists(path) else None
+    return _timing_capi
+
+
 def pmc_traffic(kind, fmt, T):
     """HBM bytes per launch of the workload's dominant kernel from its committed counter summary, or None."""
     ent = PMC_TRAFFIC.get((kind, fmt, T))
@@ -174,22 +190,41 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     # rotating inputs (so no cache level holds the experts).  Three alternations, median.
     up_marginal_ms = None
     if T <= 32:
-        def loop_ms():
-            f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            f0.record()
-            for i in range(steps):
-                step(warmup + i)
-            f1.record()
-            torch.cuda.synchronize()
-            return f0.elapsed_time(f1) / steps
-        diffs = []
-        for _ in range(3):
-            full = loop_ms()
-            m.set_option(5, 3)   # MOE_OPT_TIMING_SKIP_STAGE = 1 + MOE_PROF_UP
-            part = loop_ms()
-            m.set_option(5, 0)
-            diffs.append(full - part)
-        up_marginal_ms = sorted(diffs)[1] / nlayers
+        ct = timing_capi()
+        if ct is not None:
+            # a context of the timing twin over the same device weights (its own scratch); the loops below run on it
+            mt = ct.Moe(d, mid, E, k, layers=nlayers, max_tokens=T)
+            for l, L in enumerate(layers):
+                L.register(mt, l)
+            for o, v in list(LIB_OPTIONS) + list(opts):
+                mt.set_option(o, v)
+
+            def step_t(i):
+                if kind == "stack":
+                    for l in range(nlayers):
+                        mt.forward(l, xs[(i * nlayers + l) % len(xs)], y)
+                else:
+                    mt.forward(0, xs[i % len(xs)], y)
+
+            def loop_ms():
+                f0, f1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                f0.record()
+                for i in range(steps):
+                    step_t(warmup + i)
+                f1.record()
+                torch.cuda.synchronize()
+                return f0.elapsed_time(f1) / steps
+            for i in range(warmup):
+                step_t(i)
+            diffs = []
+            for _ in range(3):
+                full = loop_ms()
+                mt.set_option(5, 3)   # MOE_OPT_TIMING_SKIP_STAGE = 1 + MOE_PROF_UP
+                part = loop_ms()
+                mt.set_option(5, 0)
+                diffs.append(full - part)
+            up_marginal_ms = sorted(diffs)[1] / nlayers
+            mt.close()
 
     # A pair of stage events costs a few microseconds more than the kernels between them take when they run
     # back to back (the event makes the next dispatch wait).  The mean surplus per stage is reported for
@@ -253,6 +288,9 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
             gu_bytes = uniq * 2 * mid * (d // 2 + d // 128 * 2) + 2 * mid * (d // 2 + S.q4cp_scale_stride(d))
         else:
             gu_bytes = 2 * mid * (uniq * W.gg_row_bytes(gg_types[0], d) + W.gg_row_bytes(gg_types[2], d))
+        marginal = up_marginal_ms is not None
+        if not marginal:  # (no timing twin of the library: the event pair around the launch, an upper bound)
+            up_marginal_ms = stage["up"]
         up_s = up_marginal_ms * 1e-3
         od = dict(list(LIB_OPTIONS) + list(opts))
         int_dec = od.get(1, 1) != 0 and not universal  # (a table codebook takes look-up / f32 kernels)
@@ -269,9 +307,11 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
                                                              if fmt == "i4r" else "gate/up GEMV + SwiGLU"),
                                  "achieved": round(gu_bytes / up_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                  "frac": round(gu_bytes / up_s / 1e9 / HBM_PEAK_GBS, 4),
-                                 "timing": "step loop minus the same loop without this launch, HIP events around the "
-                                           "loops (an event pair around the single launch reads %.2f us: the pair's "
-                                           "dispatch latency is of the kernel's size)" % (stage["up"] * 1e3),
+                                 "timing": ("step loop minus the same loop without this launch (on the library's timing "
+                                            "twin, same kernels), HIP events around the loops (an event pair around the "
+                                            "single launch reads %.2f us: the pair's dispatch latency is of the kernel's "
+                                            "size)" % (stage["up"] * 1e3)) if marginal else
+                                           "HIP events around the launch (moe_profile_enable), same stream",
                                  "traffic": pmc_traffic(kind, fmt, T) if int_dec else None}})
         cfg.update({"unique_experts": uniq, "step_bytes": int(step_bytes)})
     res["config"] = cfg
@@ -410,6 +450,22 @@ def main():
         sub("gguf_q5k_q8_0_decode_T1", "ggmix_decode", nd, wd)
         sub("hgn_v2_prefill_T16384", "v2_prefill", a.steps, a.warmup)
         sub("hgn_v2_decode_T1", "v2_decode", nd, wd)
+        sub("universal_codebook_verify_T20", "verify", 128, wd, codebook="universal")
+        # the sub-records' key figures once more as top-level scalars, in front of the records themselves (a reader
+        # that keeps only the head of the line still has every configuration's number)
+        flat = {}
+        for name in [n for n, v in res.items() if isinstance(v, dict) and "ms_per_step" in v]:
+            r = res[name]
+            flat[name + "_ms"] = r["ms_per_step"]
+            if "hbm_frac" in r:
+                flat[name + "_hbm_frac"] = r["hbm_frac"]
+            if "layer_mfma_frac" in r:
+                flat[name + "_layer_mfma_frac"] = r["layer_mfma_frac"]
+            if r.get("roofline"):
+                flat[name + "_kernel_frac"] = r["roofline"]["frac"]
+        subs = {n: res.pop(n) for n in list(res) if isinstance(res[n], dict) and "ms_per_step" in res[n]}
+        res.update(flat)
+        res.update(subs)
     elif a.workload in ("load", "q4k_load"):
         res = measure_load("q4k" if a.workload.startswith("q4k") else "q4cp", min(a.steps, 5), min(a.layers, 2))
     else:

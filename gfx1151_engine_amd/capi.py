@@ -51,6 +51,22 @@ def lib():
     return _lib
 
 
+def second_binding(path):
+    """Another instance of this module, bound to another build of the library at `path` (the benchmark's timing twin):
+    its own library handle, the same classes and helpers.  Device pointers are process-wide, so contexts of both
+    bindings can work on the same weights."""
+    import importlib.util
+    if not os.path.exists(path):
+        raise MoeError(f"{path} is missing")
+    spec = importlib.util.find_spec(__name__)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    mod._lib = C.CDLL(path)
+    mod._lib.moe_version.restype = C.c_char_p
+    mod._lib.moe_status_string.restype = C.c_char_p
+    return mod
+
+
 def check(rc, what=""):
     if rc != 0:
         raise MoeError(f"{what}: status {rc} ({lib().moe_status_string(C.c_int(rc)).decode()})")

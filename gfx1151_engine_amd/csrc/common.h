@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/mi355_moe.h"
 
 #define MOE_API extern "C" __attribute__((visibility("default")))
@@ -24,6 +26,22 @@ static inline hipStream_t moe_s(moe_stream_t s) { return (hipStream_t)s; }
   } while (0)
 
 static inline bool moe_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// Set-up that a launch site needs once per device (hipFuncSetAttribute applies to the current device's copy of the
+// kernel): one bit per device ordinal.  moe_dev_pending is true until moe_dev_done has been called with that device
+// current; two host threads that arrive together both do the (idempotent) set-up.
+struct moe_dev_once {
+  std::atomic<uint64_t> bits[4] = {};
+};
+static inline bool moe_dev_pending(moe_dev_once& o, int* dev_out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 256) dev = 255;  // (unknown ordinal: never marked, set up again every time)
+  *dev_out = dev;
+  return dev == 255 || !(o.bits[dev >> 6].load(std::memory_order_acquire) & (1ull << (dev & 63)));
+}
+static inline void moe_dev_done(moe_dev_once& o, int dev) {
+  if (dev != 255) o.bits[dev >> 6].fetch_or(1ull << (dev & 63), std::memory_order_release);
+}
 
 // q4cp view -> operand pointers (reference: xcodes(), 40_model.inc:1599-1602)
 struct Q4cpOps {

@@ -81,7 +81,8 @@ struct moe_ctx {
   bool uq_gguf = false;       // the same for GGUF layers (off: their per-token kernels measure faster unless most tokens share experts)
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
   bool profile = false;
-  int skip_stage = 0;      // MOE_OPT_TIMING_SKIP_STAGE: 1 + the stage whose launches are left out (0 = none)
+  int skip_stage = 0;      // MOE_OPT_TIMING_SKIP_STAGE: 1 + the stage whose launches are left out (0 = none; builds with MOE_TIMING_HOOKS only)
+  int ran_complete = 0;    // the largest batch of at most small_max tokens that ran with every stage on this context
   hipEvent_t ev[MOE_PROF_STAGES + 1] = {};
   int ev_n = 0;            // events recorded by the last call
   int ev_stage[MOE_PROF_STAGES] = {};
@@ -168,8 +169,12 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   c->layers.resize(cfg->layers);
   const size_t T = (size_t)cfg->max_tokens, E = cfg->experts, S = c->cfg.id_stride;
   hipError_t e = hipMalloc(&c->logits, T * E * 4);
+  // (index-like scratch starts at zero: expert ids, offsets and tile counts are addresses in the making, and nothing
+  //  but a complete call fills them)
   if (e == hipSuccess) e = hipMalloc(&c->ids, T * S * 4);
+  if (e == hipSuccess) e = hipMemset(c->ids, 0, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ws, T * S * 4);
+  if (e == hipSuccess) e = hipMemset(c->ws, 0, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->sh_logit, T * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ticket, 256);
   if (e == hipSuccess) e = hipMemset(c->ticket, 0, 256);
@@ -195,13 +200,20 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
       return rc;
     }
     e = hipMalloc(&c->tokidx, k1 * T * 4);
+    if (e == hipSuccess) e = hipMemset(c->tokidx, 0, k1 * T * 4);
     if (e == hipSuccess) e = hipMalloc(&c->pw, k1 * T * 4);
     if (e == hipSuccess) e = hipMalloc(&c->eoff, (E + 2) * 4);
+    if (e == hipSuccess) e = hipMemset(c->eoff, 0, (E + 2) * 4);
     if (e == hipSuccess) e = hipMalloc(&c->pairids, T * cfg->topk * 4);
+    if (e == hipSuccess) e = hipMemset(c->pairids, 0, T * cfg->topk * 4);
     if (e == hipSuccess) e = hipMalloc(&c->tiles, (size_t)c->max_tiles * sizeof(moe_tile));
+    if (e == hipSuccess) e = hipMemset(c->tiles, 0, (size_t)c->max_tiles * sizeof(moe_tile));
     if (e == hipSuccess) e = hipMalloc(&c->ntiles, 8);
+    if (e == hipSuccess) e = hipMemset(c->ntiles, 0, 8);
     if (e == hipSuccess) e = hipMalloc(&c->tiles_sh, ((T + 127) / 128 + 1) * sizeof(moe_tile));
+    if (e == hipSuccess) e = hipMemset(c->tiles_sh, 0, ((T + 127) / 128 + 1) * sizeof(moe_tile));
     if (e == hipSuccess) e = hipMalloc(&c->ntiles_sh, 8);
+    if (e == hipSuccess) e = hipMemset(c->ntiles_sh, 0, 8);
     if (e == hipSuccess) e = hipMalloc(&c->pairs32, k1 * Ts * (size_t)cfg->d * 4);
   }
   if (e == hipSuccess && T > (size_t)c->small_max) {
@@ -456,9 +468,16 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
       c->gu_topk_max = value;
       return MOE_OK;
     case MOE_OPT_TIMING_SKIP_STAGE:
+#ifdef MOE_TIMING_HOOKS
+      // (the timing twin of the library only; and only once a complete call has filled the scratch that the stages
+      //  behind the skipped one take their indices from)
       if (value < 0 || value > MOE_PROF_STAGES) return MOE_E_INVALID;
+      if (value != 0 && c->ran_complete == 0) return MOE_E_STATE;
       c->skip_stage = value;
       return MOE_OK;
+#else
+      return MOE_E_UNSUPPORTED;  // not part of this build: a call with a stage left out returns wrong results
+#endif
     default: return MOE_E_INVALID;
   }
 }
@@ -826,7 +845,16 @@ static int router_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* o
 // Batches: expert-sorted permutation, MFMA grouped GEMMs over <=128-pair tiles (the shared expert
 // rides along as expert index E over all tokens), f16 pair buffer, deterministic weighted combine.
 // Returns MOE_E_UNSUPPORTED (before enqueuing anything) for shapes / formats the GEMM does not cover.
+static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st, bool* enqueued);
+
 static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
+  bool enqueued = false;
+  const int rc = forward_batch_impl(c, L, x, P, y, st, &enqueued);
+  // "unsupported" promises the caller that nothing ran; past the first launch it is a broken call instead
+  return rc == MOE_E_UNSUPPORTED && enqueued ? MOE_E_STATE : rc;
+}
+
+static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st, bool* enqueued) {
   const moe_config& g = c->cfg;
   const bool q4k = L.has_gguf;  // raw GGUF blocks
   // hgn v2 rotated experts (reference: moe_b_v2, 40_model.inc:4570-4686): the routed launches read rot_in(x, su),
@@ -867,15 +895,17 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     moe_lut_q4cp_view(L.sh_down.data, L.sh_down.rows, L.sh_down.cols, L.sh_down.scale_stride, g.d, 0, &sdn);
   }
   int rc;
-  c->ev_n = 0;
-  prof_mark(c, 0, st);
   const moe_hscale hs{c->xms, L.c_routed, L.c_shared};
   const __half* xh = c->x16_ext ? c->x16_ext : c->x16;  // f16 activations in the GEMM's order
   const int xl = batch_x16_layout(L, g);       // that order (moe_f32_to_f16's layout)
   const bool nat = batch_nat(L);               // table codebooks: natural K order, pair tables
   // gate/up (+ SwiGLU) and down launches over a tile list: routed experts, with_sh: the shared expert as well
   // (tiles whose expert index is >= n_experts)
+  // dry: the launchers run their shape / type / alignment checks and return in front of the launch (a tile capacity
+  // of 0), so that every reason to decline is found before anything is enqueued
+  bool dry = true;
   auto gemm_up = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2) -> int {
+    if (dry) mt = 0;
     if (shd && with_sh)  // the shared expert's own tile list
       return moe_launch_gemm_gg(true, L.sh_dense, L.sh_gate.data, L.sh_up.data, 0, nullptr, nullptr, g.experts, xh,
                                 c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, hs, s2, xl);
@@ -897,7 +927,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
     if (v2 && !with_sh) {  // the routed experts' tiles: plain rows of the fused tensor, then the slot-wise middle
       const int e = moe_launch_gemm_q4cp(false, &gu, nullptr, g.experts, c->v2_x16, c->tokidx, tl, ntl, mt, c->v2_z16,
                                          2 * g.mid, g.d, true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
-      return e ? e : moe_launch_i4r_mid(c->v2_z16, true, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu, L.v2_suh_dn,
+      return e || dry ? e : moe_launch_i4r_mid(c->v2_z16, true, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu, L.v2_suh_dn,
                                         1, c->hid16, (uint64_t)g.mid, 1, 1, nullptr, nullptr, s2);
     }
     if (v2)  // the shared expert's own tile list (q4cp, not rotated; every tile's expert index is >= n_experts)
@@ -907,6 +937,7 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
                                 g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up, 0, q4k && L.gg.tgu == MOE_GGML_Q5_K, nat);
   };
   auto gemm_dn = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2, const moe_comb* cmb) -> int {
+    if (dry) mt = 0;
     if (shd && with_sh)  // (hid rows of the shared tiles were written in natural order by the launch above)
       return moe_launch_gemm_gg(false, L.sh_dense, L.sh_down.data, nullptr, 0, nullptr, nullptr, g.experts, c->hid16,
                                 nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid, hs, s2, 0);
@@ -936,7 +967,28 @@ static int forward_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
                                 0, false, nat);
   };
   const bool fused = c->fused_combine && !c->hc && !(q4k && !kd.r_dn) && !split && !v2;  // the HC write-back belongs to the ordered combine
-  if (v2 || (L.has_shared && (split || (c->shared_aside && !fused)))) {
+  const bool aside = v2 || (L.has_shared && (split || (c->shared_aside && !fused)));
+  {
+    const moe_comb cmb0{y, c->tokidx, c->pw, L.has_shared ? c->sh_logit : nullptr};
+    int pre = MOE_OK;
+    if (aside) {
+      if (L.has_shared) {
+        pre = gemm_up(true, c->tiles_sh, c->ntiles_sh, 0, st);
+        if (!pre) pre = gemm_dn(true, c->tiles_sh, c->ntiles_sh, 0, st, nullptr);
+      }
+      if (!pre) pre = gemm_up(false, c->tiles, c->ntiles, 0, st);
+      if (!pre) pre = gemm_dn(false, c->tiles, c->ntiles, 0, st, nullptr);
+    } else {
+      pre = gemm_up(L.has_shared, c->tiles, c->ntiles, 0, st);
+      if (!pre) pre = gemm_dn(L.has_shared, c->tiles, c->ntiles, 0, st, fused ? &cmb0 : nullptr);
+    }
+    if (pre) return pre;  // nothing has been enqueued
+    dry = false;
+  }
+  *enqueued = true;
+  c->ev_n = 0;
+  prof_mark(c, 0, st);
+  if (aside) {
     // The shared expert does not depend on the routing: its two GEMMs run on the side stream from the start
     // of the call, next to the fp64 router launch and the latency-bound top-k / permutation launches.  The
     // side stream also makes what both streams need first: the per-token mean square of x (range guard) and
@@ -1033,7 +1085,14 @@ MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, 
   if (P > c->cfg.max_tokens) return MOE_E_STATE;
   if (!moe_aligned(x, 16) || !moe_aligned(y, 16)) return MOE_E_INVALID;
   if (P == 0) return MOE_OK;
-  if (P <= c->small_max) return forward_small(c, *L, x, P, y, moe_s(st));
+  if (P <= c->small_max) {
+#ifdef MOE_TIMING_HOOKS
+    if (c->skip_stage != 0 && P > c->ran_complete) return MOE_E_STATE;  // the scratch of a call this size is not filled yet
+#endif
+    const int rs = forward_small(c, *L, x, P, y, moe_s(st));
+    if (rs == MOE_OK && c->skip_stage == 0 && P > c->ran_complete) c->ran_complete = P;
+    return rs;
+  }
   const int rc = forward_batch(c, *L, x, P, y, moe_s(st));
   if (rc != MOE_E_UNSUPPORTED) return rc;
   // formats the grouped GEMM does not cover yet: the in-place path, 32 rows at a time.  Every chunk leaves its

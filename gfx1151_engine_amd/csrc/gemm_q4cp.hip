@@ -914,22 +914,24 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   const int split = sh ? 1 : 0;
 #define GEMM_LAUNCH(UPK, F16, Q, G)                                                                              \
   do {                                                                                                           \
-    static bool attr_done = false;                                                                               \
-    if (!attr_done) {                                                                                            \
+    static moe_dev_once attr_once;                                                                               \
+    int dev_now;                                                                                                 \
+    if (moe_dev_pending(attr_once, &dev_now)) {                                                                  \
       MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<UPK, F16, Q, G>,                                  \
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));                 \
-      attr_done = true;                                                                                          \
+      moe_dev_done(attr_once, dev_now);                                                                          \
     }                                                                                                            \
     k_moe_gemm_q4cp<UPK, F16, Q, G><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
                                                                   m, k, nblk_n, split, hs, cmb);                 \
   } while (0)
 #define GEMM_LAUNCH_NAT(UPK, F16)                                                                                \
   do {                                                                                                           \
-    static bool attr_done = false;                                                                               \
-    if (!attr_done) {                                                                                            \
+    static moe_dev_once attr_once;                                                                               \
+    int dev_now;                                                                                                 \
+    if (moe_dev_pending(attr_once, &dev_now)) {                                                                  \
       MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<UPK, F16, false, 0, false, true>,                 \
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)(SMEM_BYTES + PT_BYTES)));    \
-      attr_done = true;                                                                                          \
+      moe_dev_done(attr_once, dev_now);                                                                          \
     }                                                                                                            \
     k_moe_gemm_q4cp<UPK, F16, false, 0, false, true><<<grid, NT, SMEM_BYTES + PT_BYTES, st>>>(                    \
         R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, split, hs, cmb);                           \
@@ -939,11 +941,12 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
     else if (f16out) GEMM_LAUNCH_NAT(false, true);
     else GEMM_LAUNCH_NAT(false, false);
   } else if (q5k) {
-    static bool attr5 = false;
-    if (!attr5) {
+    static moe_dev_once attr5;
+    int dev_now;
+    if (moe_dev_pending(attr5, &dev_now)) {
       MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<true, true, true, 0, true>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
-      attr5 = true;
+      moe_dev_done(attr5, dev_now);
     }
     k_moe_gemm_q4cp<true, true, true, 0, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out,
                                                                              m, k, nblk_n, split, hs, cmb);

@@ -849,8 +849,9 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
   if (max_tiles == 0) return MOE_OK;
   GgGemmW R{w, w_up, type}, S{sh_w ? sh_w : w, sh_w ? sh_w_up : w_up, sh_w ? tsh : type};
   const dim3 grid((unsigned)(up ? (m + 63) / 64 : (m + GG_BN - 1) / GG_BN), (unsigned)max_tiles);
-  static bool attr_done = false;
-  if (!attr_done) {
+  static moe_dev_once attr_once;
+  int dev_now;
+  if (moe_dev_pending(attr_once, &dev_now)) {
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, GG_PK_Q8_0>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
@@ -861,7 +862,7 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_IQ4_NL>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<true, GG_PK_IQ4_XS>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
     MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_gg<false, GG_PK_IQ4_XS>, hipFuncAttributeMaxDynamicSharedMemorySize, GG_SMEM));
-    attr_done = true;
+    moe_dev_done(attr_once, dev_now);
   }
   // all-Q8_0 / all-Q5_1 launches (4-byte aligned rows: whole pairs of 34-byte blocks, or 24-byte blocks, from a 4-byte
   // aligned base)

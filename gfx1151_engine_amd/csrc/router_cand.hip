@@ -765,10 +765,11 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
     if (bf) k_router_w16<true><<<(Epad + 3) / 4, 256, 0, st>>>(W->data, E, Epad, d, W16, wnorm, counters);
     else k_router_w16<false><<<(Epad + 3) / 4, 256, 0, st>>>(W->data, E, Epad, d, W16, wnorm, counters);
     MOE_LAUNCH_CHECK();
-    static bool attr_done = false;
-    if (!attr_done) {
+    static moe_dev_once attr_once;
+    int dev_now;
+    if (moe_dev_pending(attr_once, &dev_now)) {
       MOE_HIP(hipFuncSetAttribute((const void*)k_router_approx2, hipFuncAttributeMaxDynamicSharedMemorySize, R2_SMEM));
-      attr_done = true;
+      moe_dev_done(attr_once, dev_now);
     }
     const dim3 g2((unsigned)((P + R2_BT - 1) / R2_BT), (unsigned)(Epad / R2_BE));
     k_router_approx2<<<g2, 512, R2_SMEM, st>>>(W16, bias, x, P, E, d, logits, xnorm, out_xms);

@@ -299,10 +299,13 @@ int moe_forward_x16(moe_ctx* ctx, int layer, const float* x, const void* x16, in
  * exact arithmetic over all experts.  Expert ids and their order are the reference's bit for bit; the renormalised
  * weights can differ from it in the last bit or two (the softmax normaliser, which cancels in them up to rounding,
  * contains approximate terms for the experts that were not candidates).  0 = dense fp64 logits and exact weights. */
-/* MOE_OPT_TIMING_SKIP_STAGE (default 0): timing experiments only.  value = 1 + MOE_PROF_* stage: calls with at most 32
- * tokens leave that stage's launches out (the later stages then work on stale scratch and the output is meaningless).
- * The difference between the times of a loop of calls without and with the skip is that stage's cost inside the
- * pipelined stream, without the dispatch latency that an event pair around a 10 us kernel adds. */
+/* MOE_OPT_TIMING_SKIP_STAGE (default 0): NOT in the library's default build, where it returns MOE_E_UNSUPPORTED; only a
+ * build with -DMOE_TIMING_HOOKS (the benchmark's timing twin of the library) takes it.  value = 1 + MOE_PROF_* stage:
+ * calls with at most 32 tokens leave that stage's launches out (the later stages then work on the scratch of the last
+ * complete call and the output is meaningless).  Refused with MOE_E_STATE until a complete call of at least that many
+ * tokens has run on the context.  The difference between the times of a loop of calls without and with the skip is
+ * that stage's cost inside the pipelined stream, without the dispatch latency that an event pair around a 10 us
+ * kernel adds. */
 /* MOE_OPT_GU_TOPK_MAX_TOKENS (default 4: the measured crossover on every weight format): batches of at most this many tokens run the softmax / top-k inside the gate/up launch
  * (every block of a routed slot selects its token's experts itself: one launch less on the latency-bound path);
  * larger batches of the integer-dot kernels take the ids from the router's launches, so that the thousands of blocks

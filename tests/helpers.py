@@ -77,10 +77,13 @@ class HostLayer:
                        gate=O.Mat(self.tgu, self.gate, E * mid, d), up=O.Mat(self.tgu, self.up, E * mid, d), shared=sh,
                        router_bias=self.bias)
 
-    def to_gpu(self, max_tokens=32):
-        """-> (capi.Moe context with this layer registered as layer 0, dict of device tensors)."""
+    def to_gpu(self, max_tokens=32, binding=None):
+        """-> (capi.Moe context with this layer registered as layer 0, dict of device tensors).
+        binding: another binding of the C ABI (capi.second_binding) instead of the default library's."""
         import torch
         from gfx1151_engine_amd import capi
+        if binding is not None:
+            capi = binding
         d, mid, E, k = self.d, self.mid, self.E, self.k
         dev = {}
 

@@ -314,3 +314,35 @@ def test_forward_errors(oracle):
     m.close()
     with pytest.raises(capi.MoeError):  # d not a multiple of 32
         capi.Moe(100, 64, 8, 2)
+
+
+def test_stage_skipping_is_not_in_the_default_build_and_guarded_in_the_timing_twin():
+    """MOE_OPT_TIMING_SKIP_STAGE makes a call return wrong results: the default library refuses it outright; the
+    benchmark's timing twin takes it only once a complete call of that size has filled the scratch that the stages
+    behind the skipped one index with."""
+    import os
+    import torch
+    from gfx1151_engine_amd import LIB_TIMING, capi
+    rng = np.random.default_rng(11)
+    hl = HostLayer(rng, 1024, 256, 16, 4)
+    m, dev = hl.to_gpu(max_tokens=8)
+    with pytest.raises(capi.MoeError, match="unsupported"):
+        m.set_option(capi.OPT_TIMING_SKIP_STAGE, 3)
+    m.close()
+    if not os.path.exists(LIB_TIMING):
+        pytest.skip("timing twin of the library not built")
+    twin = capi.second_binding(LIB_TIMING)
+    mt, dev2 = hl.to_gpu(max_tokens=8, binding=twin)
+    with pytest.raises(twin.MoeError, match="not ready"):
+        mt.set_option(capi.OPT_TIMING_SKIP_STAGE, 3)  # fresh context: nothing has run yet
+    x1 = torch.from_numpy(rng.standard_normal((1, 1024), dtype=np.float32)).cuda()
+    x2 = torch.from_numpy(rng.standard_normal((2, 1024), dtype=np.float32)).cuda()
+    y_full = mt.forward(0, x1).clone()
+    mt.set_option(capi.OPT_TIMING_SKIP_STAGE, 3)
+    mt.forward(0, x1)                       # runs (on the scratch of the complete call)
+    with pytest.raises(twin.MoeError, match="not ready"):
+        mt.forward(0, x2)                   # no complete call of two tokens yet
+    mt.set_option(capi.OPT_TIMING_SKIP_STAGE, 0)
+    assert torch.equal(mt.forward(0, x1), y_full)
+    torch.cuda.synchronize()
+    mt.close()
