@@ -40,6 +40,7 @@ static int codebook_affine(const moe_wview* w, bool* out) {
 }
 
 struct moe_ctx;
+static int pexp_register(moe_ctx* c, int layer, int slot0, const moe_wview* a, const moe_wview* b, int n_experts);
 static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gate, uint64_t gate_stride,
                               const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
                               float* out);
@@ -74,6 +75,10 @@ struct moe_ctx {
   int max_tiles = 0;
   __half* hid16 = nullptr;    // [(k+1)T][mid]
   __half* pairs16 = nullptr;  // [(k+1)T][d]
+  // scaled dequantisation of the grouped GEMM (internal.h): per layer [E gate_up | E down | shared gate/up | shared down]
+  // powers of two, MOE_PEXP_NONE where the form does not apply; span_tmp: the scan's (hi, lo) pairs of one tensor
+  int8_t* pexp = nullptr;
+  int8_t* span_tmp = nullptr;
   float* pairs32 = nullptr;   // [(k+1)min(T,small_max)][d] unweighted pair rows of the unique-expert small-batch path
   bool fused_combine = false; // batch path: the down GEMM adds its weighted rows into y with f32 atomics (no pairs buffer, no reduce launch)
   int uq_min = 24;            // > 0: small batches of at least this many tokens read every distinct expert once
@@ -110,6 +115,32 @@ struct moe_ctx {
   __half* v2_z16 = nullptr;      // [kT][2 mid]
 };
 
+// Scaled dequantisation of the grouped GEMM: the powers of two of the experts of tensor a (and, for a launch that reads
+// two tensors -- a shared expert's gate_proj and up_proj --, of a and b together) into slots slot0 .. of the layer's
+// table.  a == nullptr: the form is switched off for these slots.  Set-up work (a scan of the scale planes, a read-back).
+static int8_t* pexp_slot(moe_ctx* c, int layer, int slot0) {
+  return c->pexp ? c->pexp + (size_t)layer * (2 * (size_t)c->cfg.experts + 2) + slot0 : nullptr;
+}
+static int pexp_register(moe_ctx* c, int layer, int slot0, const moe_wview* a, const moe_wview* b, int n_experts) {
+  int8_t* dst = pexp_slot(c, layer, slot0);
+  if (!dst) return MOE_OK;  // contexts for small batches only have no grouped GEMM
+  std::vector<int8_t> out((size_t)n_experts, (int8_t)MOE_PEXP_NONE);
+  if (a) {
+    std::vector<int8_t> sa((size_t)2 * n_experts), sb;
+    int rc = moe_q4cp_scale_span(a, n_experts, c->span_tmp, nullptr);
+    if (rc) return rc;
+    MOE_HIP(hipMemcpy(sa.data(), c->span_tmp, sa.size(), hipMemcpyDeviceToHost));
+    if (b) {
+      sb.resize(sa.size());
+      if ((rc = moe_q4cp_scale_span(b, n_experts, c->span_tmp, nullptr))) return rc;
+      MOE_HIP(hipMemcpy(sb.data(), c->span_tmp, sb.size(), hipMemcpyDeviceToHost));
+    }
+    for (int e = 0; e < n_experts; e++) out[e] = (int8_t)moe_pexp_from_span(&sa[2 * e], b ? &sb[2 * e] : nullptr);
+  }
+  MOE_HIP(hipMemcpy(dst, out.data(), out.size(), hipMemcpyHostToDevice));
+  return MOE_OK;
+}
+
 static void prof_mark(moe_ctx* c, int stage_done, hipStream_t st) {
   // event i closes stage ev_stage[i-1]; event 0 opens the call
   if (!c->profile || c->ev_n > MOE_PROF_STAGES) return;
@@ -142,7 +173,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->side) (void)hipStreamDestroy(c->side);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->kpart, c->ktickets, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->tiles_sh, c->ntiles_sh, c->hid16, c->pairs16, c->pairs32, c->rc_scratch,
-                  c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16};
+                  c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16, c->pexp, c->span_tmp};
   for (void* b : bufs)
     if (b) {
       hipError_t e = hipFree(b);
@@ -220,6 +251,10 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
     const size_t d = cfg->d, mid = cfg->mid;
     e = hipMalloc(&c->rc_scratch, moe_router_cand_scratch_bytes(cfg->max_tokens, cfg->experts, cfg->d));
     if (e == hipSuccess) e = hipMalloc(&c->x16, T * d * 2);
+    const size_t pe_bytes = (size_t)cfg->layers * (2 * E + 2);
+    if (e == hipSuccess) e = hipMalloc(&c->pexp, pe_bytes);
+    if (e == hipSuccess) e = hipMemset(c->pexp, 0x80, pe_bytes);  // MOE_PEXP_NONE
+    if (e == hipSuccess) e = hipMalloc(&c->span_tmp, 2 * E);
     if (e == hipSuccess) e = hipMalloc(&c->hid16, k1 * T * mid * 2);
     if (e == hipSuccess) e = hipMalloc(&c->pairs16, k1 * T * d * 2);
   }
@@ -268,6 +303,9 @@ MOE_API int moe_set_experts_q4cp(moe_ctx* c, int layer, const moe_wview* gu, con
   L->experts_affine = a1 && a2;
   if ((rc = magnitude_constant(c, 0, 0, gu, (uint64_t)2 * g.mid, gu, (uint64_t)g.mid, dn, g.experts, &L->c_routed)))
     return rc;
+  if ((rc = pexp_register(c, layer, 0, a1 ? gu : nullptr, nullptr, g.experts)) ||
+      (rc = pexp_register(c, layer, g.experts, a2 ? dn : nullptr, nullptr, g.experts)))
+    return rc;
   L->gate_up = *gu;
   L->down = *dn;
   L->has_q4cp = true;
@@ -306,7 +344,7 @@ MOE_API int moe_set_experts_i4r(moe_ctx* c, int layer, const moe_wview* gu, cons
       if (e == hipSuccess) e = hipMalloc(&c->v2_z16, T * g.topk * 2 * (size_t)g.mid * 2);
     }
     if (e != hipSuccess) {
-      void* bufs[] = {c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16};
+      void* bufs[] = {c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16, c->pexp, c->span_tmp};
       for (void* b : bufs)
         if (b) (void)hipFree(b);
       c->v2_zraw = nullptr; c->v2_xplanes = nullptr; c->v2_xmeta = nullptr; c->v2_acc = c->v2_ey = nullptr;
@@ -376,6 +414,14 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
     int rc;
     if ((rc = codebook_affine(g, &a1)) || (rc = codebook_affine(u, &a2)) || (rc = codebook_affine(dn, &a3))) return rc;
     L->shared_affine = a1 && a2 && a3;
+    if ((rc = pexp_register(c, layer, 2 * cf.experts, a1 && a2 ? g : nullptr, u, 1)) ||
+        (rc = pexp_register(c, layer, 2 * cf.experts + 1, a3 ? dn : nullptr, nullptr, 1)))
+      return rc;
+  } else {
+    int rc;
+    if ((rc = pexp_register(c, layer, 2 * cf.experts, nullptr, nullptr, 1)) ||
+        (rc = pexp_register(c, layer, 2 * cf.experts + 1, nullptr, nullptr, 1)))
+      return rc;
   }
   L->c_shared = 0.f;
   {
@@ -899,6 +945,12 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
   const __half* xh = c->x16_ext ? c->x16_ext : c->x16;  // f16 activations in the GEMM's order
   const int xl = batch_x16_layout(L, g);       // that order (moe_f32_to_f16's layout)
   const bool nat = batch_nat(L);               // table codebooks: natural K order, pair tables
+  // scaled dequantisation (affine q4cp codebooks): the powers of two found when the weights were registered
+  const bool pe_r = L.has_q4cp && !v2 && L.experts_affine, pe_s = L.has_shared && !shd && !q4k && L.shared_affine;
+  const int8_t* pe_gu = pe_r ? pexp_slot(c, (int)(&L - c->layers.data()), 0) : nullptr;
+  const int8_t* pe_dn = pe_r ? pexp_slot(c, (int)(&L - c->layers.data()), g.experts) : nullptr;
+  const int8_t* pe_sgu = pe_s ? pexp_slot(c, (int)(&L - c->layers.data()), 2 * g.experts) : nullptr;
+  const int8_t* pe_sdn = pe_s ? pexp_slot(c, (int)(&L - c->layers.data()), 2 * g.experts + 1) : nullptr;
   // gate/up (+ SwiGLU) and down launches over a tile list: routed experts, with_sh: the shared expert as well
   // (tiles whose expert index is >= n_experts)
   // dry: the launchers run their shape / type / alignment checks and return in front of the launch (a tile capacity
@@ -932,9 +984,10 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
     }
     if (v2)  // the shared expert's own tile list (q4cp, not rotated; every tile's expert index is >= n_experts)
       return moe_launch_gemm_q4cp(true, &sgu, &sgu, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, true,
-                                  false, hs, s2, nullptr, sh_cb_up);
+                                  false, hs, s2, nullptr, sh_cb_up, 0, false, false, pe_sgu, pe_sgu);
     return moe_launch_gemm_q4cp(true, &gu, with_sh ? &sgu : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16,
-                                g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up, 0, q4k && L.gg.tgu == MOE_GGML_Q5_K, nat);
+                                g.mid, g.d, true, q4k, hs, s2, nullptr, sh_cb_up, 0, q4k && L.gg.tgu == MOE_GGML_Q5_K, nat,
+                                pe_gu, pe_sgu);
   };
   auto gemm_dn = [&](bool with_sh, const moe_tile* tl, const int* ntl, int mt, hipStream_t s2, const moe_comb* cmb) -> int {
     if (dry) mt = 0;
@@ -961,10 +1014,10 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
                                   true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
     if (v2)
       return moe_launch_gemm_q4cp(false, &sdn, &sdn, g.experts, c->hid16, nullptr, tl, ntl, mt, c->pairs16, g.d, g.mid,
-                                  true, false, hs, s2, nullptr);
+                                  true, false, hs, s2, nullptr, nullptr, 0, false, false, pe_sdn, pe_sdn);
     return moe_launch_gemm_q4cp(false, &dn, with_sh ? &sdn : nullptr, g.experts, c->hid16, nullptr, tl, ntl, mt,
                                 cmb ? (void*)cmb->y : (void*)c->pairs16, g.d, g.mid, cmb == nullptr, q4k, hs, s2, cmb, nullptr,
-                                0, false, nat);
+                                0, false, nat, pe_dn, pe_sdn);
   };
   const bool fused = c->fused_combine && !c->hc && !(q4k && !kd.r_dn) && !split && !v2;  // the HC write-back belongs to the ordered combine
   const bool aside = v2 || (L.has_shared && (split || (c->shared_aside && !fused)));

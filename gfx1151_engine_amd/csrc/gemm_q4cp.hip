@@ -80,6 +80,8 @@ struct LutDev {
   const uint8_t *w, *w_up, *sc, *sc_up;
   const float *cb, *cb_up;  // codebook of the (gate) rows and of the up rows (the same for a fused gate_up tensor)
   int sstride, e_rows, up_off;
+  // per expert: the power of two P of the scaled dequantisation (DN below), or MOE_PEXP_NONE; nullptr = none
+  const int8_t* pexp;
 };
 
 union H8 {
@@ -146,12 +148,26 @@ __device__ __forceinline__ void g2l4(const void* g, uint8_t* lds_base) {
 // MF = live 32-row fragments of the tile (1 .. 4); AFFINE = codebook a*n+b.
 // NF = weight fragments (32 rows) per wave: the block's 16 fragments are split over NW = 16/NF
 // waves, each wave multiplying all MF pair fragments with its own NF weight fragments.
-template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS, bool Q5, bool NAT = false>
+// DN (affine q4cp codebooks, a power of two P known for the expert): two instructions per weight pair instead of three.
+// A masked code pair IS a pair of f16 denormals, n * 2^-24 (nibbles at bits 0-3) or n * 2^-20 (bits 4-7), so one packed
+// FMA with a = f16(cb_a * scale) * 2^(24+P) (or 2^(20+P)) and b = f16(cb_b * scale) * 2^P gives 2^P * f16(n*a' + b'):
+// the weights of the three-instruction form times 2^P, bit for bit wherever the scaled weight is a normal f16 (the
+// product is exact inside the FMA, one rounding).  P is chosen when the weights are registered, from the expert's
+// largest scale, so that the scaled slope stays below 2^15 (an f16 can hold it); the accumulators carry the factor
+// 2^P and the epilogue takes it out (exact).  v_pk_fma_f16 takes denormal operands at full rate on gfx950.
+template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS, bool Q5, bool NAT = false, bool DN = false>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
                                           const float* __restrict__ xms,
-                                          float cmag, const moe_comb& cmb, bool shared) {
+                                          float cmag, const moe_comb& cmb, bool shared, int pexp = 0) {
+  static_assert(!DN || (AFFINE && !Q4K && !Q5 && !NAT), "scaled dequantisation: affine q4cp-style planes");
+  if (DN) {  // the codebook in the scaled units
+    const float s24 = __builtin_ldexpf(1.f, 24 + pexp), sp = __builtin_ldexpf(1.f, pexp);
+    cb_a *= s24; cb_a_up *= s24;
+    cb_b *= sp; cb_b_up *= sp;
+  }
+  const float oscale = DN ? __builtin_ldexpf(1.f, -pexp) : 1.f;  // takes 2^P out of the accumulators
   constexpr int NH = NF / 2;  // gate/up: fragments per half
   static_assert(GS == 0 || (GS == 2 && !Q4K && NSB == 1), "one scale per 128 columns: q4cp-style planes, single scale buffer");
   static_assert(!Q5 || (Q4K && NSB == 1), "Q5_K: the Q4_K stages plus a fifth bit");
@@ -362,6 +378,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   uint4 cw[NF], cw8[NF];  // code words of the stage and the same shifted right by 8 (parts 2, 3)
   constexpr int NS = Q4K ? 2 : 1;  // scale sets per stage (Q4_K: the two sub-blocks of the stage)
   half2v as2[NF][NS], bs2[NF][NS];
+  half2v as20[DN ? NF : 1];  // DN: the slope for code pairs at bits 4-7 (n * 2^-20): as2 / 16
   float scf[NF];
   uint4 hdr[NF];
   uint4 qh4[Q5 ? NF : 1];  // Q5_K: this lane's 16 qh bytes of the current super-block (code bytes 16 h .. 16 h + 15)
@@ -470,6 +487,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         const _Float16 as = (_Float16)((upf ? cb_a_up : cb_a) * scf[nf]), bs = (_Float16)((upf ? cb_b_up : cb_b) * scf[nf]);
         as2[nf][0] = half2v{as, as};
         bs2[nf][0] = half2v{bs, bs};
+        if (DN) as20[nf] = as2[nf][0] * half2v{(_Float16)0.0625f, (_Float16)0.0625f};  // (exact: a power of two, far from underflow)
       }
     }
   };
@@ -478,7 +496,12 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   auto deq_unit = [&](int q, int u, H8* dst) {
     const int nf = u >> 2, part = u & 3;
     const uint32_t w = q == 0 ? cw[nf].x : q == 1 ? cw[nf].y : q == 2 ? cw[nf].z : cw[nf].w;
-    if (AFFINE) {
+    if (DN) {
+      const uint32_t w8 = q == 0 ? cw8[nf].x : q == 1 ? cw8[nf].y : q == 2 ? cw8[nf].z : cw8[nf].w;
+      const uint32_t ws = part >= 2 ? w8 : w;
+      if ((part & 1) == 0) dst[nf].h[part] = as_h2(ws & 0x000f000fu) * as2[nf][0] + bs2[nf][0];
+      else dst[nf].h[part] = as_h2(ws & 0x00f000f0u) * as20[DN ? nf : 0] + bs2[nf][0];
+    } else if (AFFINE) {
       // (Q5_K shifts on the spot: it has no registers to spare for the shifted copies)
       const uint32_t w8 = Q5 ? w >> 8 : q == 0 ? cw8[nf].x : q == 1 ? cw8[nf].y : q == 2 ? cw8[nf].z : cw8[nf].w;
       const uint32_t ws = part >= 2 ? w8 : w;
@@ -636,7 +659,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
 #pragma unroll
         for (int f = 0; f < NH; f++) {
-          const float g = acc[mf][f][r], u = acc[mf][NH + f][r];
+          const float g = DN ? acc[mf][f][r] * oscale : acc[mf][f][r], u = DN ? acc[mf][NH + f][r] * oscale : acc[mf][NH + f][r];
           // hardware reciprocal (1 ulp) instead of the IEEE division sequence: the result is rounded
           // to f16 below, and this epilogue is VALU time during which the matrix pipe idles
           const float hv = g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) * u * rowscale[32 * mf + ml];
@@ -679,7 +702,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
 #pragma unroll
         for (int nf = 0; nf < NF; nf++)
-          *(__half*)(patch + ml * LDP + (32 * nf + n) * 2) = __float2half(acc[mf][nf][r]);
+          *(__half*)(patch + ml * LDP + (32 * nf + n) * 2) = __float2half(DN ? acc[mf][nf][r] * oscale : acc[mf][nf][r]);
       }
       // 32 rows x NC columns -> NC/8 16-byte chunks per row
       constexpr int CPR = NC / 8;
@@ -716,7 +739,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         const int m = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
         if (m >= tile.count) continue;
         float* yrow = cmb.y + (size_t)rowidx[m] * M;
-        const float w = rowscale[m];
+        const float w = rowscale[m] * oscale;
 #pragma unroll
         for (int nf = 0; nf < NF; nf++) {
           const int col = colbase + 32 * nf + n;
@@ -734,7 +757,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
 #pragma unroll
         for (int nf = 0; nf < NF; nf++) {
           const int col = colbase + 32 * nf + n;
-          if (col < M) ((float*)out)[(size_t)(tile.first + m) * M + col] = acc[mf][nf][r];
+          if (col < M) ((float*)out)[(size_t)(tile.first + m) * M + col] = DN ? acc[mf][nf][r] * oscale : acc[mf][nf][r];
         }
       }
     }
@@ -780,7 +803,11 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   L.sstride = shared ? Sh.sstride : R.sstride;
   L.e_rows = shared ? Sh.e_rows : R.e_rows;
   L.up_off = shared ? Sh.up_off : R.up_off;
+  L.pexp = shared ? Sh.pexp : R.pexp;
   const int e = shared ? 0 : tile.expert;
+  // scaled dequantisation: the expert's power of two (requested here, used after the first loads have gone out)
+  int pexp = MOE_PEXP_NONE;
+  if (!Q4K && GS == 0 && !NAT && L.pexp) pexp = L.pexp[e];
   const int tid = threadIdx.x, lane = tid & 63;
 
   // the tile's row indices: requested before the codebook is looked at, so that the two round trips
@@ -829,11 +856,23 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const float cmag = shared ? hs.c_shared : hs.c_routed;
   __syncthreads();  // cbs
   const int mfn = (tile.count + 31) >> 5;
+#define GEMM_ARGS smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if constexpr (NAT) gemm_tile<UP, F16OUT, MF, false, false, 0, false, true>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
-    else if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS, Q5>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
-    else gemm_tile<UP, F16OUT, MF, false, false, GS, false>(smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared); \
+    if constexpr (NAT) gemm_tile<UP, F16OUT, MF, false, false, 0, false, true>(GEMM_ARGS);              \
+    else {                                                                                              \
+      bool scaled = false;                                                                              \
+      if constexpr (!Q4K && GS == 0) {                                                                  \
+        if (affine && pexp != MOE_PEXP_NONE) {                                                          \
+          gemm_tile<UP, F16OUT, MF, true, false, 0, false, false, true>(GEMM_ARGS, pexp);               \
+          scaled = true;                                                                                \
+        }                                                                                               \
+      }                                                                                                 \
+      if (!scaled) {                                                                                    \
+        if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS, Q5>(GEMM_ARGS);                     \
+        else gemm_tile<UP, F16OUT, MF, false, false, GS, false>(GEMM_ARGS);                             \
+      }                                                                                                 \
+    }                                                                                                   \
   } while (0)
   if (mfn <= 1) GEMM_GO(1);
   else if (mfn == 2) GEMM_GO(2);
@@ -843,11 +882,13 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
     if (mfn <= 6) GEMM_GO(6);
     else GEMM_GO(8);
   }
+#undef GEMM_ARGS
 #undef GEMM_GO
 }
 
-LutDev to_dev(const moe_lutw* p, const float* cb_up) {
+LutDev to_dev(const moe_lutw* p, const float* cb_up, const int8_t* pexp) {
   LutDev d{};
+  d.pexp = pexp;
   if (p) {
     d.w = p->w; d.w_up = p->w_up; d.sc = p->sc; d.sc_up = p->sc_up; d.cb = p->cb;
     d.cb_up = cb_up ? cb_up : p->cb;
@@ -875,6 +916,82 @@ bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k, int gs = 0) {
 
 }  // namespace
 
+namespace {
+// One block per expert: hi = exponent of |slope| * (largest |scale| of the expert), lo = exponent of |slope| * (the
+// smallest of the rows' largest scales; rows of zeros left out), as frexp gives them; hi = 127: the scaled
+// dequantisation does not apply (a scale or the slope not finite, slope zero); hi = -127: every scale is zero.
+__global__ void __launch_bounds__(256) k_q4cp_scale_span(const uint8_t* __restrict__ sc, const float* __restrict__ cb,
+                                                         int sstride, int rows, int groups, int8_t* __restrict__ span) {
+  __shared__ float s_hi[256], s_lo[256];
+  __shared__ int s_bad[256];
+  const int e = blockIdx.x, tid = threadIdx.x;
+  const uint8_t* base = sc + (size_t)e * rows * sstride;
+  float hi = 0.f, lo = INFINITY;
+  int bad = 0;
+  for (int r = tid; r < rows; r += 256) {
+    const __half* row = (const __half*)(base + (size_t)r * sstride);
+    float rm = 0.f;
+    for (int g = 0; g < groups; g++) {
+      const float v = fabsf(__half2float(row[g]));
+      if (!(v <= 65504.f)) bad = 1;
+      rm = fmaxf(rm, v);
+    }
+    hi = fmaxf(hi, rm);
+    if (rm > 0.f) lo = fminf(lo, rm);
+  }
+  s_hi[tid] = hi; s_lo[tid] = lo; s_bad[tid] = bad;
+  __syncthreads();
+  for (int o = 128; o; o >>= 1) {
+    if (tid < o) {
+      s_hi[tid] = fmaxf(s_hi[tid], s_hi[tid + o]);
+      s_lo[tid] = fminf(s_lo[tid], s_lo[tid + o]);
+      s_bad[tid] |= s_bad[tid + o];
+    }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    const float a = fabsf(cb[1] - cb[0]);
+    int h = 127, l = 127;
+    if (!s_bad[0] && a > 0.f && a <= 3.0e38f) {
+      if (s_hi[0] == 0.f) {
+        h = l = -127;
+      } else {
+        int eh, el;
+        (void)frexpf(a * s_hi[0], &eh);
+        (void)frexpf(a * s_lo[0], &el);
+        if (a * s_hi[0] <= 3.0e38f && a * s_lo[0] > 0.f && eh < 100 && el > -100) { h = eh; l = el; }
+      }
+    }
+    span[2 * e] = (int8_t)h;
+    span[2 * e + 1] = (int8_t)l;
+  }
+}
+}  // namespace
+
+int moe_q4cp_scale_span(const moe_wview* w, int n_experts, int8_t* span_dev, hipStream_t st) {
+  if (!w || !w->data || !span_dev || n_experts < 1 || w->rows % (uint64_t)n_experts || w->cols % 32) return MOE_E_INVALID;
+  const Q4cpOps o = q4cp_ops(w);
+  k_q4cp_scale_span<<<n_experts, 256, 0, st>>>(o.scales, o.cb, (int)o.scale_stride, (int)(w->rows / n_experts),
+                                               (int)(w->cols / 32), span_dev);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+// hi_lo_b may be null (one tensor)
+int moe_pexp_from_span(const int8_t* a, const int8_t* b) {
+  int hi = a[0], lo = a[1];
+  if (hi == 127) return MOE_PEXP_NONE;
+  if (b) {
+    if (b[0] == 127) return MOE_PEXP_NONE;
+    if (hi == -127) { hi = b[0]; lo = b[1]; }
+    else if (b[0] != -127) { hi = b[0] > hi ? b[0] : hi; lo = b[1] < lo ? b[1] : lo; }
+  }
+  if (hi == -127) return 0;          // nothing but zeros: any power will do
+  if (hi - lo > 5) return MOE_PEXP_NONE;
+  const int P = -9 - hi;             // |slope| * scale * 2^(24+P) < 2^15
+  return P < -100 || P > 100 ? MOE_PEXP_NONE : P;
+}
+
 bool moe_gemm_q5k_fits(uint64_t rows, uint64_t x_rows, int k) {
   const uint64_t lim = (1ull << 32) - (1ull << 16);
   return k > 0 && k % 256 == 0 && rows * (uint64_t)(k / 256 * 176) < lim && x_rows * (uint64_t)k * 2 < lim;
@@ -886,7 +1003,8 @@ bool moe_gemm_q5k_fits(uint64_t rows, uint64_t x_rows, int k) {
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
-                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs, bool q5k, bool nat) {
+                         hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs, bool q5k, bool nat,
+                         const int8_t* pexp_routed, const int8_t* pexp_sh) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
   if (nat && (q4k || q5k || gs != 0)) return MOE_E_UNSUPPORTED;  // (natural K order: q4cp planes through pair tables)
   if (q5k && (!q4k || !up || comb)) return MOE_E_UNSUPPORTED;  // (Q5_K: gate/up tensors, the reference checkpoints' use of it)
@@ -910,7 +1028,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   // per XCD: ceil(routed/8) + ceil(shared/8) <= max_tiles/8 + 2 tile slots
   const int per_xcd = (max_tiles + 7) / 8 + 1;
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
-  LutDev R = to_dev(routed, nullptr), S = to_dev(sh ? sh : routed, sh ? sh_cb_up : nullptr);
+  LutDev R = to_dev(routed, nullptr, pexp_routed), S = to_dev(sh ? sh : routed, sh ? sh_cb_up : nullptr, sh ? pexp_sh : pexp_routed);
   const int split = sh ? 1 : 0;
 #define GEMM_LAUNCH(UPK, F16, Q, G)                                                                              \
   do {                                                                                                           \

@@ -55,7 +55,16 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
                          hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr, int gs = 0,
-                         bool q5k = false, bool nat = false);
+                         bool q5k = false, bool nat = false, const int8_t* pexp_routed = nullptr,
+                         const int8_t* pexp_sh = nullptr);
+// Scaled dequantisation of the grouped GEMM (affine q4cp codebooks): per expert the power of two P with
+// |cb slope| * (largest scale of the expert) * 2^(24+P) in [2^14, 2^15), or MOE_PEXP_NONE where the form does not apply
+// (a scale that is not finite, a zero slope, rows whose largest scale lies more than 2^5 below the expert's: their
+// weights would fall into the f16 denormals of the scaled units).  moe_q4cp_scale_span fills one (hi, lo) pair of
+// exponents per expert for a tensor; moe_pexp_from_span combines the spans of the tensors one launch reads.
+constexpr int MOE_PEXP_NONE = -128;
+int moe_q4cp_scale_span(const moe_wview* w, int n_experts, int8_t* span_dev, hipStream_t st);
+int moe_pexp_from_span(const int8_t* hi_lo_a, const int8_t* hi_lo_b);
 // The Q5_K form addresses weights and activations with 32-bit byte offsets: true when a tensor of `rows` rows of k
 // columns and an activation buffer of `x_rows` rows of k f16 values both stay below 4 GB (the caller of
 // moe_launch_gemm_q4cp(q5k = true) checks it; other layers take the general kernel)
