@@ -46,6 +46,9 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #ifndef MOE_GEMM_NF
 #define MOE_GEMM_NF 2
 #endif
+#ifndef MOE_GEMM_WALK
+#define MOE_GEMM_WALK 3  // column blocks that a block of a down launch walks (at most)
+#endif
 #ifndef MOE_GEMM_WROWS
 #define MOE_GEMM_WROWS 256
 #endif
@@ -160,7 +163,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
                                           const float* __restrict__ xms,
-                                          float cmag, const moe_comb& cmb, bool shared, int pexp = 0) {
+                                          float cmag, const moe_comb& cmb, bool shared, int pexp = 0, int npass = 1) {
+  // npass > 1 (down launches with f16 results): the block walks npass neighbouring column blocks of its pair tile.  The
+  // K stages of all passes form one pipeline -- the first stages of the next column block are requested while the
+  // current one's last stages run, so only the first pass pays for the trip to memory -- and the epilogue of a pass
+  // uses the stage buffer that the pipeline has just left.
+  constexpr bool WALK = !UP && F16OUT && !Q5 && AHEAD == 2;
+  if (!WALK) npass = 1;
   static_assert(!DN || (AFFINE && !Q4K && !Q5 && !NAT), "scaled dequantisation: affine q4cp-style planes");
   if (DN) {  // the codebook in the scaled units
     const float s24 = __builtin_ldexpf(1.f, 24 + pexp), sp = __builtin_ldexpf(1.f, pexp);
@@ -283,8 +292,11 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   const int nstage = K / BK, ngroups = K / 32;
   constexpr int NLOADS = A_LOADS + W_LOADS;  // per stage (+S_LOADS scale loads on every fourth stage)
   // one direct-to-LDS load of stage s: u < A_LOADS activations, then the code loads, then the scale loads
-  auto issue_unit = [&](int s, int u) {
-    const int b = s % NBUF;
+  // bytes from one column block's rows to the next one's (passes of a walk)
+  const size_t wpass = WALK ? (size_t)WROWS * (Q4K ? (size_t)(K / 256 * KBLK) : (size_t)(K / 2)) : 0;
+  const size_t spass = WALK ? (Q4K ? wpass : (size_t)WROWS * (size_t)L.sstride) : 0;
+  // stage s of a pass into buffer b; pw / ps: byte offsets of the pass's code and scale rows from the first pass's
+  auto issue_unit = [&](int s, int b, size_t pw, size_t ps, int u) {
     if (u < A_LOADS) {
       if (Q5) g2l16((const uint8_t*)x + (a_off[Q5 ? u : 0] + (uint32_t)s * (BK * 2)), A0 + b * A_BYTES + a_grp[u] * 1024);
       else g2l16(a_src[u] + (size_t)s * BK, A0 + b * A_BYTES + a_grp[u] * 1024);
@@ -292,13 +304,13 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       const int i = u - A_LOADS;
       const size_t off = Q4K ? (size_t)(s >> 2) * KBLK + KQS + (size_t)(s & 3) * 32 : (size_t)s * 32;
       if (Q5) g2l16(wave_w + (w_off[Q5 ? i : 0] + (uint32_t)off), W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
-      else g2l16(w_src[i] + off, W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
+      else g2l16(w_src[i] + (off + pw), W0 + b * W_BYTES + (W_LOADS * wv + i) * 1024);
     } else {
       // 8 scales (16 B) per row for stages s..s+3; at the end of K the window is pulled back inside the row
       const int i = (u - NLOADS) / SP, pc = (u - NLOADS) % SP;  // row group, 16-byte piece of the row's record
       int g0 = 2 * s;
       g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
-      const size_t off = Q4K ? (size_t)(s >> 2) * KBLK : (size_t)g0 * 2;
+      const size_t off = (Q4K ? (size_t)(s >> 2) * KBLK : (size_t)g0 * 2) + ps;
       if (Q5 && pc == 1)  // this lane's 16 qh bytes of each fragment, into registers
         qhn[0] = *(const uint2*)(L.w + (qh_off0 + (uint32_t)off));
       else if (Q5 && pc == 2)
@@ -310,21 +322,21 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       else if (Q5)
         g2l16(wave_w + (s_off + (uint32_t)off), S0 + wv * 1024);
       else if (GS == 2)  // the two scales of stages s..s+3 (s % 4 == 0: columns 64 s .. 64 s + 255), [row][4 B]
-        g2l4(s_src[i] + (size_t)s, S0 + (S_ROWG * wv + i) * 256);
+        g2l4(s_src[i] + ((size_t)s + ps), S0 + (S_ROWG * wv + i) * 256);
       else  // piece pc of every row: a region of its own, [row][16 B]
         g2l16(s_src[i] + off, S0 + ((s >> 2) & (NSB - 1)) * S_BYTES + (S_ROWG * wv + i) * 1024);
     }
   };
   auto issue_a = [&](int s) {
 #pragma unroll
-    for (int u = 0; u < A_LOADS; u++) issue_unit(s, u);
+    for (int u = 0; u < A_LOADS; u++) issue_unit(s, s % NBUF, 0, 0, u);
   };
   auto issue_w = [&](int s) {  // codes, and the scales on every fourth stage
 #pragma unroll
-    for (int u = A_LOADS; u < NLOADS; u++) issue_unit(s, u);
+    for (int u = A_LOADS; u < NLOADS; u++) issue_unit(s, s % NBUF, 0, 0, u);
     if ((s & 3) == 0) {
 #pragma unroll
-      for (int u = 0; u < S_LOADS; u++) issue_unit(s, NLOADS + u);
+      for (int u = 0; u < S_LOADS; u++) issue_unit(s, s % NBUF, 0, 0, NLOADS + u);
     }
   };
   // s_waitcnt vmcnt(N), N = loads allowed to stay in flight (loads retire in order)
@@ -342,11 +354,12 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   };
   // wait until the loads of every stage before `first` have landed; stages first .. first+AHEAD-2
   // (those that exist) may still be in flight
-  auto wait_loads_before = [&](int first) {
+  // (more: that later stage exists -- in this pass or, on a walk, in the next)
+  auto wait_loads_before = [&](int first, bool more) {
     if (AHEAD == 2) {
       // one later stage can be in flight: none, its NLOADS loads, or those and the scale loads -- three immediates
       // (the general count below compiles to a search tree of scalar branches in every stage)
-      if (first >= nstage) __builtin_amdgcn_s_waitcnt(0x0F70);
+      if (!more) __builtin_amdgcn_s_waitcnt(0x0F70);
       else if ((first & 3) == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | ((NLOADS + S_LOADS) & 15) | (((NLOADS + S_LOADS) >> 4) << 14));
       else __builtin_amdgcn_s_waitcnt(0x0F70 | (NLOADS & 15) | ((NLOADS >> 4) << 14));
       return;
@@ -393,9 +406,9 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // stage takes its own with one 64-bit shift (a choice between four registers by the wave-uniform stage index
   // compiles to a tree of scalar branches in every stage)
   uint32_t scp[NSB == 1 ? NF : 1][2];
-  auto load_codes = [&](int s) {  // raw codes + this lane's scale of stage s (buffers already selected)
+  auto load_codes = [&](int s, int b) {  // raw codes + this lane's scale of stage s, which lies in buffer b
     if (Q5) q5sh = 2 * (s & 3);
-    const uint8_t* Wb = W0 + (s % NBUF) * W_BYTES;
+    const uint8_t* Wb = W0 + b * W_BYTES;
     const uint8_t* Sb = S0 + ((s >> 2) & (NSB - 1)) * S_BYTES;
     int g0 = 2 * (s & ~3);
     g0 = g0 + 8 <= ngroups ? g0 : ngroups - 8;
@@ -575,17 +588,27 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   // stage 0 must have landed; only the activation loads of the later stages may still be in flight
   wait_vm(nstage > 1 ? A_LOADS * (AHEAD - 1) : 0);
   moe_lds_barrier();  // the later stages' loads stay in flight
-  load_codes(0);
+  load_codes(0, 0);
 #pragma unroll
   for (int mf = 0; mf < MF; mf++) load_a1(0, mf, a[0]);
   scale_consts(0);
 #pragma unroll
   for (int u = 0; u < NU; u++) deq_unit(0, u, b[0]);
 
-  for (int s = 0; s < nstage; s++) {
-    Ab = A0 + (s % NBUF) * A_BYTES;
-    const bool pf = s + AHEAD < nstage;        // stage s+AHEAD exists: its loads go out during step 0
-    const bool pf_s = pf && ((s + AHEAD) & 3) == 0;
+  // `epilogue` (below the loop in the source) writes one column block's results; cbuf = the stage buffer that the
+  // pipeline has just left (a walk's patch lives there)
+  auto run = [&](auto&& epilogue) {
+  int s = 0, p = 0, cbuf = 0;  // stage within the pass, pass, the stage's LDS buffer
+  const int nvs = nstage * npass;
+  for (int v = 0; v < nvs; v++) {
+    Ab = A0 + cbuf * A_BYTES;
+    // the stage whose loads go out during step 0: AHEAD stages on, in the next pass where this one ends before
+    int is = s + AHEAD, ip = p;
+    if (is >= nstage) { is -= nstage; ip++; }
+    const bool pf = ip < npass;
+    const bool pf_s = pf && (is & 3) == 0;
+    const int ib = cbuf + AHEAD >= NBUF ? cbuf + AHEAD - NBUF : cbuf + AHEAD;
+    const size_t ipw = (size_t)ip * wpass, ips = (size_t)ip * spass;
 #pragma unroll
     for (int q = 0; q < 3; q++) {
       const int cur = q & 1, nxt = cur ^ 1;
@@ -599,33 +622,35 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         for (int k = 0; k < UPM; k++)
           if (i * UPM + k < NU) deq_unit(q + 1, i * UPM + k, b[nxt]);
         if (q == 0) {
-          // buffer (s+AHEAD)%NBUF was last read in stage s-1: free since the previous barrier
+          // buffer ib was last read in the stage before this one: free since the previous barrier
           constexpr int LPS = (NLOADS + S_LOADS + NM - 1) / NM;  // loads per MFMA slot
 #pragma unroll
           for (int k = 0; k < LPS; k++) {
             const int u = i * LPS + k;
-            if (u < NLOADS) { if (pf) issue_unit(s + AHEAD, u); }
-            else if (u < NLOADS + S_LOADS) { if (pf_s) issue_unit(s + AHEAD, u); }
+            if (u < NLOADS) { if (pf) issue_unit(is, ib, ipw, ips, u); }
+            else if (u < NLOADS + S_LOADS) { if (pf_s) issue_unit(is, ib, ipw, ips, u); }
           }
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // last step: a[1], b[1] hold its operands.  Step 0 of stage s+1 is prepared from the next
-    // buffer meanwhile, so that buffer must be complete and visible: loads of stage s+1 done
-    // (stage s+2's may still fly), then the block barrier.
-    wait_loads_before(s + 2);
+    // last step: a[1], b[1] hold its operands.  Step 0 of the next stage is prepared from the next
+    // buffer meanwhile, so that buffer must be complete and visible: loads of the next stage done
+    // (the one after it may still fly), then the block barrier.
+    const int sn = s + 1 == nstage ? 0 : s + 1;            // the next stage (on a walk: of the next pass after the last)
+    const int nbuf = cbuf + 1 == NBUF ? 0 : cbuf + 1;
+    wait_loads_before(s + 2, v + 2 < nvs);
     moe_lds_barrier();  // (not __syncthreads(): its fence would wait for the loads just issued two stages ahead)
-    Ab = A0 + ((s + 1) % NBUF) * A_BYTES;
+    Ab = A0 + nbuf * A_BYTES;
 #pragma unroll
     for (int i = 0; i < NM; i++) {
       const int mf = i / NF, nf = i % NF;
       mfma16(acc[mf][nf], a[1][mf], b[1][nf].v);
       __builtin_amdgcn_sched_barrier(0);
-      // (past the last stage this reads stale LDS and the result is never used)
-      if (i == 0) load_codes(s + 1);
+      // (past the last stage of the last pass this reads stale LDS and the result is never used)
+      if (i == 0) load_codes(sn, nbuf);
       if (i < MF) load_a1(0, i, a[0]);
-      if (i == X0) scale_consts(s + 1);
+      if (i == X0) scale_consts(sn);
       if (i >= X0) {
 #pragma unroll
         for (int k = 0; k < XPM; k++)
@@ -633,20 +658,41 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    if (WALK && sn == 0) {  // a pass ends: its column block goes out, the accumulators start over
+      epilogue(nb + p, cbuf);
+      p++;
+      // The patch is the wave's quarter of the buffer.  With all four row fragments live those are exactly the bytes
+      // that the wave's own loads write (activation row groups 4 wv .. 4 wv + 3), so whoever runs ahead cannot touch
+      // another wave's patch; a tile with fewer fragments deals its row groups to the waves differently, and the
+      // block has to meet before the next loads into this buffer go out.
+      if (MF < 4 && p < npass) moe_lds_barrier();
+#pragma unroll
+      for (int mf = 0; mf < MF; mf++)
+#pragma unroll
+        for (int nf = 0; nf < NF; nf++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) acc[mf][nf][i] = 0.f;
+    }
+    s = sn;
+    cbuf = nbuf;
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // no LDS-bound load may outlive the block
-  if (UP) {
-    if (tid < BM) rowscale[tid] = xms ? moe_hid_scale(cmag, xms_v) : 1.f;
-    __syncthreads();
+  if (!WALK) {
+    if (UP) {
+      if (tid < BM) rowscale[tid] = xms ? moe_hid_scale(cmag, xms_v) : 1.f;
+      __syncthreads();
+    }
+    epilogue(nb, 0);
   }
+  };
 
   // epilogue.  D[i][j]: j = lane%32 (weight row), i = 8*(r/4) + 4*(lane/32) + r%4 (pair).
   // f16 results go through a per-wave LDS patch (the stage buffers are dead by now) so that global
   // stores are 16 bytes per lane and whole rows are contiguous.
   constexpr int NC = UP ? 32 * NH : 32 * NF;  // output columns of this wave
-  constexpr int LDP = NC * 2 + 16;            // padded row pitch of the patch in bytes
+  auto epilogue = [&](int nb, int cbuf) {     // nb: the column block that the accumulators hold
   const int colbase = UP ? nb * HALF + NC * wv : nb * WROWS + NC * wv;
-  if (UP) {
+  if constexpr (UP) {
     // gate/up: a wave holds 32 of the block's HALF hid columns, 64 bytes of a row -- stored per wave, the two halves of
     // a 128-byte line reach memory separately (measured: 2.3 times the payload written).  So the block's waves put
     // their columns into one patch of whole rows and every store instruction writes complete lines.
@@ -691,30 +737,45 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         if (m < tile.count && col < M) *(uint4*)((__half*)out + (size_t)(tile.first + m) * M + col) = v;
       }
     }
-  } else if (F16OUT) {
+  } else if constexpr (F16OUT) {
     // down: a wave's 64 columns are whole 128-byte lines of a row; a per-wave patch turns the accumulators' layout into
-    // 16-byte stores
-    uint8_t* patch = smem + wv * (32 * LDP);
+    // 16-byte stores.  The patch is the wave's own quarter of the activation buffer that the pipeline has just left,
+    // 32 rows of NC f16 without padding; rows 4..7 of every eight swap their row halves, which puts the two lane
+    // halves of a store (rows m and m + 4, same columns) on different banks.
+    // (Measured and dropped: the two MFMA operands exchanged, which transposes the accumulators so that, after one
+    //  v_permlane32_swap between the lane halves, a lane holds 8 neighbouring f16 of one row and stores them without
+    //  LDS -- 32 bytes of a row per lane pair and instruction: 4 % slower than this patch, whose stores are whole lines.)
+    static_assert(32 * NC * 2 * NW <= A_BYTES && NC * 2 == 128, "the patch is a wave's share of one activation buffer");
+    uint8_t* patch = A0 + cbuf * A_BYTES + wv * (32 * NC * 2);
+    // (the lane's coordinates pass through an opaque copy: on a walk the epilogue sits inside the K loop, and address
+    //  terms derived from the plain values would be computed ahead of the loop and held in registers through it)
+    int lq = lane;
+    asm volatile("" : "+v"(lq));
+    const int nq = lq & 31, hq = lq >> 5;
 #pragma unroll
     for (int mf = 0; mf < MF; mf++) {
+      // row 4 h + ..., column 32 nf + n at byte 2 n + 64 (nf ^ h) of the row
+      static_assert(NF == 2, "two 32-column halves per wave");
+      uint8_t* const wr0 = patch + (4 * hq) * 128 + nq * 2 + 64 * hq;
+      uint8_t* const wr1 = patch + (4 * hq) * 128 + nq * 2 + 64 * (1 - hq);
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
 #pragma unroll
         for (int nf = 0; nf < NF; nf++)
-          *(__half*)(patch + ml * LDP + (32 * nf + n) * 2) = __float2half(DN ? acc[mf][nf][r] * oscale : acc[mf][nf][r]);
+          *(__half*)((nf ? wr1 : wr0) + (8 * (r >> 2) + (r & 3)) * 128) = __float2half(DN ? acc[mf][nf][r] * oscale : acc[mf][nf][r]);
       }
       // 32 rows x NC columns -> NC/8 16-byte chunks per row
       constexpr int CPR = NC / 8;
       constexpr int ITS = (32 * CPR + 63) / 64;
+      static_assert(CPR == 8 && ITS == 4, "eight 16-byte chunks per row, eight rows per instruction");
+      const int ml0 = lq >> 3, c8 = lq & 7;
+      const uint8_t* const rd = patch + ml0 * 128 + ((c8 * 16) ^ (((ml0 >> 2) & 1) << 6));
+      __half* const orow = (__half*)out + (size_t)(tile.first + 32 * mf + ml0) * M + (colbase + c8 * 8);
 #pragma unroll
       for (int it = 0; it < ITS; it++) {
-        const int c = it * 64 + lane, ml = c / CPR, c8 = c % CPR;
-        if (c < 32 * CPR) {
-          const uint4 v = *(const uint4*)(patch + ml * LDP + c8 * 16);
-          const int m = 32 * mf + ml, col = colbase + c8 * 8;
-          if (m < tile.count && col < M) *(uint4*)((__half*)out + (size_t)(tile.first + m) * M + col) = v;
-        }
+        const uint4 v = *(const uint4*)(rd + it * 8 * 128);  // rows ml0 + 8 it: the same halves swapped
+        const int m = 32 * mf + ml0 + 8 * it;
+        if (m < tile.count && colbase + c8 * 8 < M) *(uint4*)(orow + (size_t)(8 * it) * M) = v;
       }
     }
   } else if (cmb.y) {
@@ -762,6 +823,8 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
       }
     }
   }
+  };
+  run(epilogue);
 }
 
 template <bool UP, bool F16OUT, bool Q4K, int GS, bool Q5 = false, bool NAT = false>
@@ -769,7 +832,7 @@ __global__ void __launch_bounds__(NT, WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,
-                moe_hscale hs, moe_comb cmb) {
+                moe_hscale hs, moe_comb cmb, int npass) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
@@ -780,7 +843,7 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   const int nr = split ? ntiles[1] : nt;  // routed tiles come first in the list
   const int wg = blockIdx.x, xcd = wg & 7, j = wg >> 3;
   const int per_r = (nr + 7) >> 3, per_s = (nt - nr + 7) >> 3;
-  const int tl = j / nblk_n, nb = j - tl * nblk_n;
+  const int tl = j / nblk_n, nb = (j - tl * nblk_n) * npass;  // (nblk_n: groups of npass column blocks per tile)
   int ti;
   if (tl < per_r) {
     ti = xcd * per_r + tl;
@@ -857,20 +920,21 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
   __syncthreads();  // cbs
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_ARGS smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared
+#define GEMM_TAIL 0, npass
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if constexpr (NAT) gemm_tile<UP, F16OUT, MF, false, false, 0, false, true>(GEMM_ARGS);              \
+    if constexpr (NAT) gemm_tile<UP, F16OUT, MF, false, false, 0, false, true>(GEMM_ARGS, GEMM_TAIL);   \
     else {                                                                                              \
       bool scaled = false;                                                                              \
       if constexpr (!Q4K && GS == 0) {                                                                  \
         if (affine && pexp != MOE_PEXP_NONE) {                                                          \
-          gemm_tile<UP, F16OUT, MF, true, false, 0, false, false, true>(GEMM_ARGS, pexp);               \
+          gemm_tile<UP, F16OUT, MF, true, false, 0, false, false, true>(GEMM_ARGS, pexp, npass);        \
           scaled = true;                                                                                \
         }                                                                                               \
       }                                                                                                 \
       if (!scaled) {                                                                                    \
-        if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS, Q5>(GEMM_ARGS);                     \
-        else gemm_tile<UP, F16OUT, MF, false, false, GS, false>(GEMM_ARGS);                             \
+        if (Q4K || affine) gemm_tile<UP, F16OUT, MF, true, Q4K, GS, Q5>(GEMM_ARGS, GEMM_TAIL);          \
+        else gemm_tile<UP, F16OUT, MF, false, false, GS, false>(GEMM_ARGS, GEMM_TAIL);                  \
       }                                                                                                 \
     }                                                                                                   \
   } while (0)
@@ -883,6 +947,7 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
     else GEMM_GO(8);
   }
 #undef GEMM_ARGS
+#undef GEMM_TAIL
 #undef GEMM_GO
 }
 
@@ -1024,7 +1089,17 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
   if (q4k && up && m % 64) return MOE_E_UNSUPPORTED;  // hid is written in whole 64-element blocks
   if (!moe_aligned(x, 16) || !moe_aligned(out, 4)) return MOE_E_INVALID;
   if (max_tiles == 0) return MOE_OK;
-  const int nblk_n = up ? (m + HALF - 1) / HALF : (m + WROWS - 1) / WROWS;
+  int nblk_n = up ? (m + HALF - 1) / HALF : (m + WROWS - 1) / WROWS;
+  // down launches with f16 results: a block walks npass neighbouring column blocks of its pair tile (whole column
+  // blocks and whole scale windows only); the largest divisor of the column block count up to the wanted length
+  // (measured at 163840 pairs, K = 768, 12 column blocks: 0.938 / 0.921 / 0.912 / 0.921 / 0.943 / 1.015 ms for walks of
+  //  1 / 2 / 3 / 4 / 6 / 12; a launch with few tiles keeps its blocks short: the shared expert's 1536 blocks next to the
+  //  router's launches took longer as 512 blocks of three passes)
+  int npass = 1;
+  if (!up && f16out && !q5k && !comb && NBUF == 3 && m % WROWS == 0 && k % 256 == 0)
+    for (int c = 1; c <= MOE_GEMM_WALK && c <= nblk_n; c++)
+      if (nblk_n % c == 0 && (int64_t)max_tiles * (nblk_n / c) >= 4096) npass = c;
+  nblk_n /= npass;
   // per XCD: ceil(routed/8) + ceil(shared/8) <= max_tiles/8 + 2 tile slots
   const int per_xcd = (max_tiles + 7) / 8 + 1;
   const unsigned grid = (unsigned)(per_xcd * nblk_n * 8);
@@ -1040,7 +1115,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
       moe_dev_done(attr_once, dev_now);                                                                          \
     }                                                                                                            \
     k_moe_gemm_q4cp<UPK, F16, Q, G><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
-                                                                  m, k, nblk_n, split, hs, cmb);                 \
+                                                                  m, k, nblk_n, split, hs, cmb, npass);          \
   } while (0)
 #define GEMM_LAUNCH_NAT(UPK, F16)                                                                                \
   do {                                                                                                           \
@@ -1052,7 +1127,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
       moe_dev_done(attr_once, dev_now);                                                                          \
     }                                                                                                            \
     k_moe_gemm_q4cp<UPK, F16, false, 0, false, true><<<grid, NT, SMEM_BYTES + PT_BYTES, st>>>(                    \
-        R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, split, hs, cmb);                           \
+        R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, split, hs, cmb, npass);                    \
   } while (0)
   if (nat) {
     if (up) GEMM_LAUNCH_NAT(true, true);
@@ -1067,7 +1142,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
       moe_dev_done(attr5, dev_now);
     }
     k_moe_gemm_q4cp<true, true, true, 0, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out,
-                                                                             m, k, nblk_n, split, hs, cmb);
+                                                                             m, k, nblk_n, split, hs, cmb, npass);
   } else if (gs == 2) {
     GEMM_LAUNCH(false, true, false, 2);
   } else if (q4k) {
