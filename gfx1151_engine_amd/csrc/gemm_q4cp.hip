@@ -553,6 +553,10 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         dst[nf].h[part] = hv;
       }
     }
+    // The unit stays where it is written: without a use in its own block the compiler moves a unit's instructions down
+    // into the block of the MFMA that reads them (past the branches of the load slots, past the stage barrier), where
+    // they run in a row in front of that MFMA instead of one by one behind the earlier ones.
+    asm volatile("" : "+v"(dst[nf].u[part]));
   };
   constexpr int NM = NF * MF;                     // MFMAs per K step
   constexpr int UPM = (NU + NM - 1) / NM;         // dequant units behind each MFMA (steps 0-2)
@@ -745,6 +749,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
     // (Measured and dropped: the two MFMA operands exchanged, which transposes the accumulators so that, after one
     //  v_permlane32_swap between the lane halves, a lane holds 8 neighbouring f16 of one row and stores them without
     //  LDS -- 32 bytes of a row per lane pair and instruction: 4 % slower than this patch, whose stores are whole lines.)
+#if MOE_GEMM_NF == 2 && MOE_GEMM_WROWS == 256
     static_assert(32 * NC * 2 * NW <= A_BYTES && NC * 2 == 128, "the patch is a wave's share of one activation buffer");
     uint8_t* patch = A0 + cbuf * A_BYTES + wv * (32 * NC * 2);
     // (the lane's coordinates pass through an opaque copy: on a walk the epilogue sits inside the K loop, and address
@@ -778,6 +783,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
         if (m < tile.count && colbase + c8 * 8 < M) *(uint4*)(orow + (size_t)(8 * it) * M) = v;
       }
     }
+#endif  // (other fragment counts per wave: timing experiments of the gate/up launch only)
   } else if (cmb.y) {
     // fused weighted combine: the tile's rows are added straight into their tokens' output rows
     // (f32 atomics executed in L2, no value returned), weight = the pair's routing weight (the
@@ -1133,6 +1139,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
     if (up) GEMM_LAUNCH_NAT(true, true);
     else if (f16out) GEMM_LAUNCH_NAT(false, true);
     else GEMM_LAUNCH_NAT(false, false);
+#if MOE_GEMM_NF == 2 && MOE_GEMM_WROWS == 256  // (other block shapes: timing experiments of the q4cp / Q4_K launches only)
   } else if (q5k) {
     static moe_dev_once attr5;
     int dev_now;
@@ -1145,6 +1152,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                                                                              m, k, nblk_n, split, hs, cmb, npass);
   } else if (gs == 2) {
     GEMM_LAUNCH(false, true, false, 2);
+#endif
   } else if (q4k) {
     if (up) GEMM_LAUNCH(true, true, true, 0);
     else if (f16out) GEMM_LAUNCH(false, true, true, 0);
