@@ -13,6 +13,7 @@ struct MoeLayer {
   bool has_router = false, has_q4cp = false, has_gguf = false, has_shared = false;
   moe_wview router{};
   const float* router_bias = nullptr;
+  float router_wmax = 0.f;  // the largest row norm of the router matrix (the bound of the small-batch selection, moe_rfix)
   moe_wview gate_up{}, down{};
   moe_gg_experts gg{};
   moe_wview sh_gate{}, sh_up{}, sh_down{}, sh_sg{};
@@ -53,6 +54,7 @@ struct moe_ctx {
   int* ids = nullptr;         // [T][id_stride]
   float* ws = nullptr;        // [T][id_stride]
   float* sh_logit = nullptr;  // [T]
+  float* rtol = nullptr;      // [min(T, small_max)]: per token, how far the small-batch router's logits can lie from the reference's
   unsigned* ticket = nullptr; // block counter of the fused small-batch router launch (rests at 0)
   double* kpart = nullptr;    // partial tiles and per-row-group tickets (resting at 0) of the column-split router launch
   unsigned* ktickets = nullptr;
@@ -173,7 +175,7 @@ MOE_API int moe_destroy(moe_ctx* c) {
   if (c->side) (void)hipStreamDestroy(c->side);
   void* bufs[] = {c->logits, c->ids, c->ws, c->sh_logit, c->ticket, c->kpart, c->ktickets, c->xms, c->sample, c->hid32, c->xplanes, c->hplanes, c->xmeta, c->hmeta, c->x16, c->tokidx, c->pw, c->eoff,
                   c->pairids, c->tiles, c->ntiles, c->tiles_sh, c->ntiles_sh, c->hid16, c->pairs16, c->pairs32, c->rc_scratch,
-                  c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16, c->pexp, c->span_tmp};
+                  c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16, c->pexp, c->span_tmp, c->rtol};
   for (void* b : bufs)
     if (b) {
       hipError_t e = hipFree(b);
@@ -207,6 +209,7 @@ MOE_API int moe_create(const moe_config* cfg, moe_ctx** out) {
   if (e == hipSuccess) e = hipMalloc(&c->ws, T * S * 4);
   if (e == hipSuccess) e = hipMemset(c->ws, 0, T * S * 4);
   if (e == hipSuccess) e = hipMalloc(&c->sh_logit, T * 4);
+  if (e == hipSuccess) e = hipMalloc(&c->rtol, (T < (size_t)c->small_max ? T : (size_t)c->small_max) * 4);
   if (e == hipSuccess) e = hipMalloc(&c->ticket, 256);
   if (e == hipSuccess) e = hipMemset(c->ticket, 0, 256);
   if (e == hipSuccess) e = hipMalloc(&c->kpart, MOE_ROUTER_KPART_BYTES);
@@ -283,6 +286,8 @@ MOE_API int moe_set_router(moe_ctx* c, int layer, const moe_wview* w, const floa
   if (!L || !w || !w->data) return MOE_E_INVALID;
   if (w->dtype != MOE_DT_F32 && w->dtype != MOE_DT_BF16) return MOE_E_UNSUPPORTED;
   if ((int)w->rows != c->cfg.experts || (int)w->cols != c->cfg.d) return MOE_E_INVALID;
+  const int rn = moe_router_row_norm_max(w, c->sample, &L->router_wmax);
+  if (rn) return rn;
   L->router = *w;
   L->router_bias = bias;
   L->has_router = true;
@@ -344,7 +349,7 @@ MOE_API int moe_set_experts_i4r(moe_ctx* c, int layer, const moe_wview* gu, cons
       if (e == hipSuccess) e = hipMalloc(&c->v2_z16, T * g.topk * 2 * (size_t)g.mid * 2);
     }
     if (e != hipSuccess) {
-      void* bufs[] = {c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16, c->pexp, c->span_tmp};
+      void* bufs[] = {c->v2_zraw, c->v2_xplanes, c->v2_xmeta, c->v2_acc, c->v2_ey, c->v2_x16, c->v2_z16};
       for (void* b : bufs)
         if (b) (void)hipFree(b);
       c->v2_zraw = nullptr; c->v2_xplanes = nullptr; c->v2_xmeta = nullptr; c->v2_acc = c->v2_ey = nullptr;
@@ -575,6 +580,21 @@ static int forward_small(moe_ctx* c, MoeLayer& L, const float* x, int P, float* 
                                        y, st);
 }
 
+// What the selection of a small batch needs to be certain of its expert ids (topk.h, select_certain): the router
+// launch sums the products in a parallel order; |that fp64 sum - the reference's sequential one| <= 2 gamma_d |w||x|
+// for any row w (gamma_d = d u / (1 - d u), u = 2^-53), so tol_scale * |x| bounds it for every logit of a token.
+static moe_rfix router_fix(const moe_ctx* c, const MoeLayer& L, const float* x, bool tol_from_router) {
+  moe_rfix R{};
+  R.W = L.router.data;
+  R.bias = L.router_bias;
+  R.x = x;
+  R.tol = tol_from_router ? c->rtol : nullptr;
+  R.tol_scale = 2.f * (float)(c->cfg.d + 4) * 0x1p-53f * L.router_wmax * 1.05f;
+  R.bf16 = L.router.dtype == MOE_DT_BF16 ? 1 : 0;
+  R.d = c->cfg.d;
+  return R;
+}
+
 // the router and the routed experts (and the shared expert where the kernels take it along as one more slot)
 static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, float* y, hipStream_t st) {
   const moe_config& g = c->cfg;
@@ -617,14 +637,19 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
   const bool gu_topk = ((((use_int && !use_uq) || ((use_int4k || use_intgg) && !use_uq_gg)) && P <= c->gu_topk_max) || use_lut) &&
                        moe_dec_gu_topk_supported(g.experts, g.topk);
+  // (up to 4 tokens the router launch leaves each token's bound for the selection; larger batches: the selecting
+  //  block takes the norm of x itself)
+  const moe_rfix rf = router_fix(c, L, x, P <= 4);
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
+         // (the selection runs in launches of its own here, so that it can be made certain: no top-k inside the logits launch)
          int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
                                          c->sh_logit, (use_int || use_int4k || use_intgg) ? c->xplanes : nullptr, c->xmeta,
-                                         use_int4k || use_intgg, gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk,
-                                         g.id_stride, &fused, st, c->kpart, c->ktickets);
-         if (!e && !fused && !gu_topk)
-           e = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
+                                         use_int4k || use_intgg, nullptr, c->ids, c->ws, g.topk,
+                                         g.id_stride, &fused, st, c->kpart, c->ktickets, nullptr, P <= 4 && rf.W ? c->rtol : nullptr,
+                                         rf.tol_scale);
+         if (!e && !gu_topk)
+           e = moe_launch_router_topk_small(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, &rf, st);
          return e;
        })))
     return rc;
@@ -666,7 +691,7 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
       if ((rc = stage(MOE_PROF_UP, [&]() -> int {
              return gu_topk ? moe_launch_dec_gu_topk(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->logits, g.experts,
                                                      c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes,
-                                                     c->hmeta, nullptr, st)
+                                                     c->hmeta, nullptr, st, nullptr, &rf)
                             : moe_launch_dec_gu(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->ids, g.id_stride, g.topk,
                                                 P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st);
            })))
@@ -679,7 +704,7 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
     if (use_lut) {
       if ((rc = stage(MOE_PROF_UP, [&]() -> int {
              return moe_launch_dec_gu_lut(&L.gate_up, shg, shu, x, c->logits, g.experts, c->ids, c->ws, g.id_stride,
-                                          g.topk, P, g.d, g.mid, c->hid32, st);
+                                          g.topk, P, g.d, g.mid, c->hid32, st, &rf);
            })))
         return rc;
       return stage(MOE_PROF_DOWN, [&]() -> int {
@@ -732,7 +757,7 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
     if ((rc = stage(MOE_PROF_UP, [&]() -> int {
            return gu_topk ? moe_launch_decgg_gu_topk(L.gg.tgu, L.sh_gguf_type, L.gg.gate, L.gg.up, rg, ru, c->xplanes,
                                                      c->xmeta, c->logits, g.experts, c->ids, c->ws, g.id_stride, g.topk,
-                                                     P, g.d, g.mid, c->hplanes, c->hmeta, st)
+                                                     P, g.d, g.mid, c->hplanes, c->hmeta, st, &rf)
                           : moe_launch_decgg_gu(L.gg.tgu, L.sh_gguf_type, L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta,
                                                 c->ids, g.experts, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes, c->hmeta,
                                                 st);
@@ -758,7 +783,7 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
     if ((rc = stage(MOE_PROF_UP, [&]() -> int {
            return gu_topk ? moe_launch_dec4k_gu_topk(L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta, c->logits,
                                                      g.experts, c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid,
-                                                     c->hplanes, c->hmeta, st)
+                                                     c->hplanes, c->hmeta, st, &rf)
                           : moe_launch_dec4k_gu(L.gg.gate, L.gg.up, rg, ru, c->xplanes, c->xmeta, c->ids, g.id_stride,
                                                 g.topk, P, g.d, g.mid, c->hplanes, c->hmeta, st);
          })))
@@ -800,15 +825,16 @@ static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, floa
   if (sh && (L.sh_gguf_type != 0 || !L.shared_affine)) return MOE_E_UNSUPPORTED;
   const int nslots_d = g.topk + (sh ? 1 : 0);
   const bool gu_topk = P <= c->gu_topk_max;
+  const moe_rfix rf = router_fix(c, L, x, P <= 4);
   if ((rc = stage(MOE_PROF_ROUTER, [&]() -> int {
          bool fused = false;
          // (the planes of rot_in(x, su) ride in the router launch's spare blocks)
          const moe_rot_planes rot{L.v2_su, c->v2_xplanes, c->v2_xmeta};
          int e = moe_router_logits_small(&L.router, L.router_bias, L.has_shared ? &L.sh_sg : nullptr, x, P, c->logits,
                                          c->sh_logit, sh ? c->xplanes : nullptr, c->xmeta, false,
-                                         gu_topk ? nullptr : c->ticket, c->ids, c->ws, g.topk, g.id_stride, &fused, st,
-                                         c->kpart, c->ktickets, &rot);
-         if (!e && !fused && !gu_topk) e = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
+                                         nullptr, c->ids, c->ws, g.topk, g.id_stride, &fused, st,
+                                         c->kpart, c->ktickets, &rot, P <= 4 && rf.W ? c->rtol : nullptr, rf.tol_scale);
+         if (!e && !gu_topk) e = moe_launch_router_topk_small(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, &rf, st);
          return e;
        })))
     return rc;
@@ -817,7 +843,7 @@ static int forward_small_v2(moe_ctx* c, MoeLayer& L, const float* x, int P, floa
          const moe_dec_v2 v2{c->v2_zraw, c->v2_xplanes, c->v2_xmeta};
          const int e = gu_topk ? moe_launch_dec_gu_topk(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->logits, g.experts,
                                                         c->ids, c->ws, g.id_stride, g.topk, P, g.d, g.mid, c->hplanes,
-                                                        c->hmeta, nullptr, st, &v2)
+                                                        c->hmeta, nullptr, st, &v2, &rf)
                                : moe_launch_dec_gu(&L.gate_up, shg, shu, c->xplanes, c->xmeta, c->ids, g.id_stride, g.topk,
                                                    P, g.d, g.mid, c->hplanes, c->hmeta, nullptr, st, &v2);
          return e ? e : moe_launch_i4r_mid(c->v2_zraw, false, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu,

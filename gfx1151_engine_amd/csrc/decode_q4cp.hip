@@ -185,7 +185,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
                                                 const moe_tile* __restrict__ tiles, const int* __restrict__ ntiles,
                                                 const int* __restrict__ tokidx, int n_experts,
                                                 const float* __restrict__ logits, int* __restrict__ ids_out,
-                                                float* __restrict__ ws_out, const float* __restrict__ xf32) {
+                                                float* __restrict__ ws_out, const float* __restrict__ xf32, moe_rfix RF) {
   extern __shared__ float lutmem[];
   __shared__ float gs[GU2_ROWS], us[GU2_ROWS];
   __shared__ uint32_t pk[QV4_GROUP_DW];
@@ -198,7 +198,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     // one block of the extra grid row: the exact softmax / top-k (ids, renormalised weights) for the down
     // launch, next to the blocks that stream the weights and only need the ids
     if (blockIdx.x == 0) {
-      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)blockIdx.z * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      select_certain<NPL ? NPL : 8, 512>(logits + (size_t)blockIdx.z * n_experts, RF, (int)blockIdx.z, sel_ids, sel_ws, n_experts, kpt, true);
       __syncthreads();
       if ((int)threadIdx.x < kpt) {
         ids_out[(size_t)blockIdx.z * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
@@ -221,10 +221,7 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
       // the ids by logit order (no exps, no sums); the exact selection only when two of the best logits
       // are too close for that to be certain
       const float* lg = logits + (size_t)blockIdx.z * n_experts;
-      if (!topk_ids_by_logit<NPL ? NPL : 8>(lg, sel_ids, n_experts, kpt)) {
-        topk_block<NPL ? NPL : 8, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
-        __syncthreads();
-      }
+      if (!select_certain<NPL ? NPL : 8, 512>(lg, RF, (int)blockIdx.z, sel_ids, sel_ws, n_experts, kpt, false)) __syncthreads();
       e = sel_ids[s];
     }
   } else {
@@ -598,7 +595,7 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
   if (!A.gu.cb) return MOE_E_STATE;
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
   k_dec_gu<false, 0, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
-                                                  nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr);
+                                                  nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, moe_rfix{});
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -609,7 +606,9 @@ bool moe_dec_gu_topk_supported(int n_experts, int kpt) { return n_experts <= 102
 int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                            const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                            int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
-                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st, const moe_dec_v2* v2) {
+                           uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st, const moe_dec_v2* v2,
+                           const moe_rfix* rf) {
+  const moe_rfix RFV = rf ? *rf : moe_rfix{};
   GuArgs2 A{};
   A.gu = decw(gu);
   A.shg = decw(sh_gate);
@@ -624,10 +623,10 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);  // + the row of the exact top-k block
   if (n_experts <= 512)
     k_dec_gu<false, 8, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
-                                                    hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr);
+                                                    hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr, RFV);
   else
     k_dec_gu<false, 16, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
-                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr);
+                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr, RFV);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -636,8 +635,9 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
 // the launch as above.
 int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up, const float* x,
                           const float* logits, int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d,
-                          int mid, float* hid_f32, hipStream_t st) {
+                          int mid, float* hid_f32, hipStream_t st, const moe_rfix* rf) {
   if (!x || !hid_f32 || !logits || !moe_dec_gu_topk_supported(n_experts, kpt)) return MOE_E_INVALID;
+  const moe_rfix RFV = rf ? *rf : moe_rfix{};
   GuArgs2 A{};
   A.gu = decw(gu);
   A.shg = decw(sh_gate);
@@ -647,10 +647,10 @@ int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const m
   if (lds > 64 * 1024) return MOE_E_UNSUPPORTED;
   if (n_experts <= 512)
     k_dec_gu<false, 8, true><<<grid, 512, lds, st>>>(A, nullptr, nullptr, nullptr, id_stride, kpt, d, mid, nullptr, nullptr,
-                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x);
+                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x, RFV);
   else
     k_dec_gu<false, 16, true><<<grid, 512, lds, st>>>(A, nullptr, nullptr, nullptr, id_stride, kpt, d, mid, nullptr, nullptr,
-                                                      hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x);
+                                                      hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x, RFV);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -688,7 +688,7 @@ int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const mo
   if (max_tiles <= 0) return MOE_OK;
   dim3 grid(mid / GU2_ROWS, max_tiles);
   k_dec_gu<true, 0, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
-                                                 ntiles, tokidx, n_experts, nullptr, nullptr, nullptr, nullptr);
+                                                 ntiles, tokidx, n_experts, nullptr, nullptr, nullptr, nullptr, moe_rfix{});
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

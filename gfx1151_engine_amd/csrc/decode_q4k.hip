@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(512, 4) k_dec4k_gu(Gu4kArgs A, const uint32_t*
                                                      int mid, uint32_t* __restrict__ hplanes,
                                                      float2* __restrict__ hmeta, const float* __restrict__ logits,
                                                      int n_experts, int* __restrict__ ids_out,
-                                                     float* __restrict__ ws_out) {
+                                                     float* __restrict__ ws_out, moe_rfix RF) {
   __shared__ float gs[G4_ROWS], us[G4_ROWS];
   __shared__ uint32_t pk[QV_GROUP_DW];
   __shared__ int sel_ids[64];
@@ -137,7 +137,7 @@ __global__ void __launch_bounds__(512, 4) k_dec4k_gu(Gu4kArgs A, const uint32_t*
     // one block of the extra grid row: the exact softmax / top-k (ids, renormalised weights) for the down
     // launch, next to the blocks that stream the weights and only need the ids
     if (blockIdx.x == 0) {
-      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      select_certain<NPL ? NPL : 8, 512>(logits + (size_t)tok * n_experts, RF, (int)tok, sel_ids, sel_ws, n_experts, kpt, true);
       __syncthreads();
       if ((int)threadIdx.x < kpt) {
         ids_out[(size_t)tok * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
@@ -155,10 +155,7 @@ __global__ void __launch_bounds__(512, 4) k_dec4k_gu(Gu4kArgs A, const uint32_t*
     if (!shared) {
       // the ids by logit order; the exact selection only when two of the best logits are too close
       const float* lg = logits + (size_t)tok * n_experts;
-      if (!topk_ids_by_logit<NPL ? NPL : 8>(lg, sel_ids, n_experts, kpt)) {
-        topk_block<NPL ? NPL : 8, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
-        __syncthreads();
-      }
+      if (!select_certain<NPL ? NPL : 8, 512>(lg, RF, (int)tok, sel_ids, sel_ws, n_experts, kpt, false)) __syncthreads();
       e = sel_ids[s];
     }
   } else if (!shared) {
@@ -545,7 +542,7 @@ __global__ void __launch_bounds__(512, 4) k_decgg_gu(GuGgArgs A, const uint32_t*
                                                      int mid, uint32_t* __restrict__ hplanes,
                                                      float2* __restrict__ hmeta, const float* __restrict__ logits,
                                                      int n_experts, int* __restrict__ ids_out,
-                                                     float* __restrict__ ws_out, const int* __restrict__ ids_in) {
+                                                     float* __restrict__ ws_out, const int* __restrict__ ids_in, moe_rfix RF) {
   __shared__ float gs[G4_ROWS], us[G4_ROWS];
   __shared__ uint32_t pk[QV_GROUP_DW];
   __shared__ int sel_ids[64];
@@ -553,7 +550,7 @@ __global__ void __launch_bounds__(512, 4) k_decgg_gu(GuGgArgs A, const uint32_t*
   const int s = blockIdx.y, tok = blockIdx.z, nslots = gridDim.y - (NPL > 0 ? 1 : 0);
   if (NPL > 0 && s == nslots) {  // the extra grid row: exact softmax / top-k for the down launch
     if (blockIdx.x == 0) {
-      topk_block<NPL ? NPL : 8, false, 512>(logits + (size_t)tok * n_experts, sel_ids, sel_ws, n_experts, kpt);
+      select_certain<NPL ? NPL : 8, 512>(logits + (size_t)tok * n_experts, RF, (int)tok, sel_ids, sel_ws, n_experts, kpt, true);
       __syncthreads();
       if ((int)threadIdx.x < kpt) {
         ids_out[(size_t)tok * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
@@ -569,10 +566,7 @@ __global__ void __launch_bounds__(512, 4) k_decgg_gu(GuGgArgs A, const uint32_t*
   if (!shared) {
     if (NPL > 0) {
       const float* lg = logits + (size_t)tok * n_experts;
-      if (!topk_ids_by_logit<NPL ? NPL : 8>(lg, sel_ids, n_experts, kpt)) {
-        topk_block<NPL ? NPL : 8, false, 512>(lg, sel_ids, sel_ws, n_experts, kpt);
-        __syncthreads();
-      }
+      if (!select_certain<NPL ? NPL : 8, 512>(lg, RF, (int)tok, sel_ids, sel_ws, n_experts, kpt, false)) __syncthreads();
       e = sel_ids[s];
     } else {
       e = ids_in[(size_t)tok * id_stride + s];  // (NPL == 0: the ids come from the router's launches)
@@ -877,7 +871,7 @@ int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* s
   Gu4kArgs A{gate, up, sh_gate, sh_up};
   dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0), P);
   k_dec4k_gu<0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, nullptr, 0,
-                                      nullptr, nullptr);
+                                      nullptr, nullptr, moe_rfix{});
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -887,7 +881,8 @@ int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* s
 int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
                              const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                              int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
-                             uint32_t* hplanes, float2* hmeta, hipStream_t st) {
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st, const moe_rfix* rf) {
+  const moe_rfix RFV = rf ? *rf : moe_rfix{};
   if (!gate || !up || !xplanes || !xmeta || !logits || !ids || !ws || !hplanes || !hmeta || (!sh_gate != !sh_up))
     return MOE_E_INVALID;
   if (!moe_aligned(gate, 16) || !moe_aligned(up, 16) || (sh_gate && (!moe_aligned(sh_gate, 16) || !moe_aligned(sh_up, 16))))
@@ -896,10 +891,10 @@ int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8
   dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);  // + the row of the exact top-k block
   if (n_experts <= 512)
     k_dec4k_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta, logits,
-                                        n_experts, ids, ws);
+                                        n_experts, ids, ws, RFV);
   else
     k_dec4k_gu<16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta, logits,
-                                         n_experts, ids, ws);
+                                         n_experts, ids, ws, RFV);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -935,7 +930,8 @@ static size_t ggu_align(int t) { return t == MOE_GGML_Q8_0 || t == MOE_GGML_IQ4_
 int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
                              const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const float* logits,
                              int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
-                             uint32_t* hplanes, float2* hmeta, hipStream_t st) {
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st, const moe_rfix* rf) {
+  const moe_rfix RFV = rf ? *rf : moe_rfix{};
   if (!gate || !up || !xplanes || !xmeta || !logits || !ids || !ws || !hplanes || !hmeta || (!sh_gate != !sh_up))
     return MOE_E_INVALID;
   if (!moe_decgg_supported(tgu, tgu, tsh, sh_gate != nullptr, d, mid, kpt, n_experts)) return MOE_E_UNSUPPORTED;
@@ -945,9 +941,9 @@ int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_
   GuGgArgs A{gate, up, sh_gate, sh_up, tgu, tsh};
   dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);
   if (n_experts <= 512)
-    k_decgg_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws, nullptr);
+    k_decgg_gu<8><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws, nullptr, RFV);
   else
-    k_decgg_gu<16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws, nullptr);
+    k_decgg_gu<16><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, logits, n_experts, ids, ws, nullptr, RFV);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -964,7 +960,7 @@ int moe_launch_decgg_gu(int tgu, int tsh, const uint8_t* gate, const uint8_t* up
   GuGgArgs A{gate, up, sh_gate, sh_up, tgu, tsh};
   dim3 grid(mid / G4_ROWS, kpt + (sh_gate ? 1 : 0), P);
   k_decgg_gu<0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, id_stride, kpt, d, mid, hplanes, hmeta, nullptr, n_experts, nullptr,
-                                      nullptr, ids);
+                                      nullptr, ids, moe_rfix{});
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

@@ -24,6 +24,22 @@ struct moe_hc {
   uint16_t* R;
 };
 
+// What the small-batch selection needs to make the expert ids certain: the router's operands and the bound tol.
+struct moe_rfix {
+  const void* W;      // router matrix [E][d], f32 or bf16 (nullptr: no check, the logits are taken as they are)
+  const float* bias;  // [E] or nullptr
+  const float* x;     // activations [P][d]
+  const float* tol;   // [P]: bound on |fp64 sum in the router launch's order - the reference's sequential sum| (any logit
+                      // of the token), written by the router launch; nullptr: the selecting block takes the norm of x itself
+  float tol_scale;    // the bound = tol_scale * |x_token|_2: 2 (d + 4) 2^-53 * the largest row norm of W, with a margin
+  int bf16, d;
+};
+// the largest row norm of a router matrix (set-up work: one launch and a read-back through `scratch`, a device float)
+int moe_router_row_norm_max(const moe_wview* W, float* scratch, float* out_host);
+// softmax / top-k of at most 32 tokens, a block per token, with the expert ids made certain (rf may be null)
+int moe_launch_router_topk_small(const float* logits, int* ids, float* ws, int P, int E, int k, int id_stride,
+                                 const moe_rfix* rf, hipStream_t st);
+
 // hgn v2 layers: the small-batch router launch also leaves the digit planes of rot_in(x, pre) (planes / meta [P][d/32])
 struct moe_rot_planes {
   const float* pre;
@@ -33,7 +49,8 @@ struct moe_rot_planes {
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
-                            hipStream_t st, double* kpart, unsigned* ktickets, const moe_rot_planes* rot = nullptr);
+                            hipStream_t st, double* kpart, unsigned* ktickets, const moe_rot_planes* rot = nullptr,
+                            float* tol_out = nullptr, float tol_scale = 0.f);
 // scratch of the column-split router launch (5..32 tokens): fp64 partial tiles of up to 8 splits x 32 tokens
 // for at most MOE_ROUTER_KSPLIT_ROWS rows, and one ticket counter (resting at 0) per 16 rows
 constexpr int MOE_ROUTER_KSPLIT_ROWS = 1040;
@@ -116,14 +133,14 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
                            const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                            int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
                            uint32_t* hplanes, float2* hmeta, float* hid_f32, hipStream_t st,
-                           const moe_dec_v2* v2 = nullptr);
+                           const moe_dec_v2* v2 = nullptr, const moe_rfix* rf = nullptr);
 int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                       const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                       int P, int d, int mid, uint32_t* hplanes, float2* hmeta, float* hid_f32,
                       hipStream_t st, const moe_dec_v2* v2 = nullptr);
 int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up, const float* x,
                           const float* logits, int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d,
-                          int mid, float* hid_f32, hipStream_t st);
+                          int mid, float* hid_f32, hipStream_t st, const moe_rfix* rf = nullptr);
 int moe_launch_dec_dn_lut(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit, const float* hid_f32,
                           const int* ids, const float* ws, int id_stride, int kpt, int P, int d, int mid, float* out,
                           uint64_t out_stride, hipStream_t st);
@@ -140,7 +157,7 @@ bool moe_decgg_supported(int tgu, int tdn, int tsh, bool has_shared, int d, int 
 int moe_launch_decgg_gu_topk(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
                              const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const float* logits,
                              int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
-                             uint32_t* hplanes, float2* hmeta, hipStream_t st);
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st, const moe_rfix* rf = nullptr);
 int moe_launch_decgg_gu(int tgu, int tsh, const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate,
                         const uint8_t* sh_up, const uint32_t* xplanes, const float2* xmeta, const int* ids, int n_experts,
                         int id_stride, int kpt, int P, int d, int mid, uint32_t* hplanes, float2* hmeta, hipStream_t st);
@@ -159,7 +176,7 @@ int moe_launch_decgg_dn_uq(int tdn, int tsh, const uint8_t* down, const uint8_t*
 int moe_launch_dec4k_gu_topk(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
                              const uint32_t* xplanes, const float2* xmeta, const float* logits, int n_experts,
                              int* ids, float* ws, int id_stride, int kpt, int P, int d, int mid,
-                             uint32_t* hplanes, float2* hmeta, hipStream_t st);
+                             uint32_t* hplanes, float2* hmeta, hipStream_t st, const moe_rfix* rf = nullptr);
 int moe_launch_dec4k_gu(const uint8_t* gate, const uint8_t* up, const uint8_t* sh_gate, const uint8_t* sh_up,
                         const uint32_t* xplanes, const float2* xmeta, const int* ids, int id_stride, int kpt,
                         int P, int d, int mid, uint32_t* hplanes, float2* hmeta, hipStream_t st);

@@ -250,7 +250,8 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
                                                       int nrows, uint32_t* __restrict__ planes,
                                                       float2* __restrict__ meta, bool planes_natural,
                                                       unsigned* counter, int* __restrict__ ids,
-                                                      float* __restrict__ ws, int k, int id_stride, moe_rot_planes rot) {
+                                                      float* __restrict__ ws, int k, int id_stride, moe_rot_planes rot,
+                                                      float* __restrict__ tol_out, float tol_scale) {
   __shared__ int s_last;
   // the wave index as a scalar: row, weight type and base address are then wave-uniform values
   // and the bf16 / f32 choice below is a scalar branch, not a divergent one around every load
@@ -267,12 +268,18 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
     const void* Wr = extra ? Wx : W;
     const uint64_t base = extra ? 0 : (uint64_t)row * d;
     const bool bf = extra ? wx_bf16 : BF16;
+    // the wave of row 0 also takes |x|^2 of every token: the selection that follows needs a bound on how far these
+    // sums (lanes, then a tree) can lie from the reference's sequential ones, tol_scale * |x|
+    const bool norms = tol_out && row == 0;
     for (int t0 = 0; t0 < P; t0 += TT) {
       double acc[TT][4];
+      float xs[TT];
 #pragma unroll
-      for (int i = 0; i < TT; i++)
+      for (int i = 0; i < TT; i++) {
+        xs[i] = 0.f;
 #pragma unroll
         for (int q = 0; q < 4; q++) acc[i][q] = 0.0;
+      }
 #pragma unroll 12
       for (int c = lane * 4; c < d; c += 256) {
         float w[4];
@@ -294,6 +301,17 @@ __global__ void __launch_bounds__(256) k_router_small(const void* __restrict__ W
             acc[i][1] = fma((double)w[1], (double)xv.y, acc[i][1]);
             acc[i][2] = fma((double)w[2], (double)xv.z, acc[i][2]);
             acc[i][3] = fma((double)w[3], (double)xv.w, acc[i][3]);
+            if (norms) xs[i] += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+          }
+        }
+      }
+      if (norms) {
+#pragma unroll
+        for (int i = 0; i < TT; i++) {
+          const float n2 = wave_sum(xs[i]);
+          if (lane == 0 && t0 + i < P) {
+            float tl = tol_scale * sqrtf(n2) * 1.01f;
+            tol_out[t0 + i] = tl >= 0.f ? tl : INFINITY;  // (NaN: nothing is certain)
           }
         }
       }
@@ -452,9 +470,33 @@ __global__ void __launch_bounds__(256) k_router_topk(const float* __restrict__ l
 
 template <int NPL>
 __global__ void __launch_bounds__(256) k_router_topk_block(const float* __restrict__ logits, int* __restrict__ ids,
-                                                           float* __restrict__ ws, int E, int k, int id_stride) {
+                                                           float* __restrict__ ws, int E, int k, int id_stride, moe_rfix RF) {
+  __shared__ int sel_ids[64];
+  __shared__ float sel_ws[64];
   const int t = blockIdx.x;
-  topk_block<NPL, false>(logits + (size_t)t * E, ids + (size_t)t * id_stride, ws + (size_t)t * id_stride, E, k);
+  if (!RF.W) {
+    topk_block<NPL, false>(logits + (size_t)t * E, ids + (size_t)t * id_stride, ws + (size_t)t * id_stride, E, k);
+    return;
+  }
+  select_certain<NPL, 256>(logits + (size_t)t * E, RF, t, sel_ids, sel_ws, E, k, true);
+  __syncthreads();
+  if ((int)threadIdx.x < k) {
+    ids[(size_t)t * id_stride + threadIdx.x] = sel_ids[threadIdx.x];
+    ws[(size_t)t * id_stride + threadIdx.x] = sel_ws[threadIdx.x];
+  }
+}
+
+// |row|_2 of every row, the maximum as the bits of a non-negative float
+__global__ void __launch_bounds__(256) k_row_norm_max(const void* __restrict__ W, int bf16, int E, int d, unsigned* __restrict__ out) {
+  const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= E) return;
+  float a = 0.f;
+  for (int c = lane; c < d; c += 64) {
+    const float w = bf16 ? bf16_bits_to_f32(((const uint16_t*)W)[(size_t)row * d + c]) : ((const float*)W)[(size_t)row * d + c];
+    a += w * w;
+  }
+  a = wave_sum(a);
+  if (lane == 0) atomicMax(out, __float_as_uint(a >= 0.f ? sqrtf(a) : INFINITY));
 }
 
 // Launch of the sequential-order kernel: 128-token tiles when there are enough of them to fill the
@@ -672,7 +714,8 @@ int moe_router_logits_seq_if(const moe_wview* W, const float* bias, const moe_wv
 int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x,
                             int P, float* logits, float* out_x, uint32_t* planes, float2* meta,
                             bool planes_natural, unsigned* counter, int* ids, float* ws, int k, int id_stride, bool* fused_topk,
-                            hipStream_t st, double* kpart, unsigned* ktickets, const moe_rot_planes* rotp) {
+                            hipStream_t st, double* kpart, unsigned* ktickets, const moe_rot_planes* rotp,
+                            float* tol_out, float tol_scale) {
   const int E = (int)W->rows, d = (int)W->cols;
   moe_rot_planes rot{nullptr, nullptr, nullptr};
   if (rotp) {  // hgn v2: the planes of rot_in(x, pre) in the same launch
@@ -723,7 +766,7 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   const int qblocks = (planes ? P * ((d / 32 + bs - 1) / bs) : 0) + (rot.planes ? P * ((d / 8 + bs - 1) / bs) : 0);
   dim3 g((nrows + rpb - 1) / rpb + qblocks);
   const void* wx = Wx ? Wx->data : nullptr;
-#define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, bs, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride, rot)
+#define RSM_GO(BF, TT, NPL) k_router_small<BF, TT, NPL><<<g, bs, 0, st>>>(W->data, bias, wx, xbf, x, P, E, d, logits, out_x, nrows, planes, meta, planes_natural, cn, ids, ws, k, id_stride, rot, tol_out, tol_scale)
   if (P == 1 && E <= 512) {
     if (bf) RSM_GO(true, 1, 8); else RSM_GO(false, 1, 8);
   } else if (P <= 4) {
@@ -758,18 +801,33 @@ int moe_router_logits_small(const moe_wview* W, const float* bias, const moe_wvi
   return MOE_OK;
 }
 
+int moe_launch_router_topk_small(const float* logits, int* ids, float* ws, int P, int E, int k, int id_stride,
+                                 const moe_rfix* rf, hipStream_t st) {
+  const moe_rfix R = rf ? *rf : moe_rfix{};
+  if (E <= 512) k_router_topk_block<8><<<P, 256, 0, st>>>(logits, ids, ws, E, k, id_stride, R);
+  else k_router_topk_block<16><<<P, 256, 0, st>>>(logits, ids, ws, E, k, id_stride, R);
+  MOE_LAUNCH_CHECK();
+  return MOE_OK;
+}
+
+int moe_router_row_norm_max(const moe_wview* W, float* scratch, float* out_host) {
+  if (!W || !W->data || !scratch || !out_host) return MOE_E_INVALID;
+  MOE_HIP(hipMemset(scratch, 0, 4));
+  k_row_norm_max<<<(unsigned)((W->rows + 3) / 4), 256, 0, nullptr>>>(W->data, W->dtype == MOE_DT_BF16 ? 1 : 0, (int)W->rows,
+                                                                     (int)W->cols, (unsigned*)scratch);
+  MOE_LAUNCH_CHECK();
+  MOE_HIP(hipMemcpy(out_host, scratch, 4, hipMemcpyDeviceToHost));
+  return MOE_OK;
+}
+
 MOE_API int moe_router_topk(const float* logits, int* ids, float* ws, int P, int E, int k,
                             int id_stride, moe_stream_t st) {
   if (!logits || !ids || !ws) return MOE_E_INVALID;
   if (P < 0 || E < 1 || k < 1 || k > E || k > 64 || id_stride < k) return MOE_E_INVALID;
   if (E > 1024) return MOE_E_UNSUPPORTED;
   if (P == 0) return MOE_OK;
-  if (P <= 32) {  // few tokens: a block per token, the fp64 exps spread over its threads
-    if (E <= 512) k_router_topk_block<8><<<P, 256, 0, moe_s(st)>>>(logits, ids, ws, E, k, id_stride);
-    else k_router_topk_block<16><<<P, 256, 0, moe_s(st)>>>(logits, ids, ws, E, k, id_stride);
-    MOE_LAUNCH_CHECK();
-    return MOE_OK;
-  }
+  if (P <= 32)  // few tokens: a block per token, the fp64 exps spread over its threads
+    return moe_launch_router_topk_small(logits, ids, ws, P, E, k, id_stride, nullptr, moe_s(st));
   dim3 g((P + 3) / 4);
   if (E <= 512) k_router_topk<8><<<g, 256, 0, moe_s(st)>>>(logits, ids, ws, P, E, k, id_stride);
   else k_router_topk<16><<<g, 256, 0, moe_s(st)>>>(logits, ids, ws, P, E, k, id_stride);

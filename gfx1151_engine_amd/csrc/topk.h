@@ -3,6 +3,7 @@
 //  the lower index, weights renormalised over the selected k)
 #pragma once
 #include "common.h"
+#include "internal.h"
 
 __device__ __forceinline__ uint32_t umax(uint32_t a, uint32_t b) { return a > b ? a : b; }
 __device__ __forceinline__ uint32_t umin(uint32_t a, uint32_t b) { return a < b ? a : b; }
@@ -144,9 +145,10 @@ __device__ __forceinline__ void topk_select_lm(uint32_t (&key)[NPL], int lane, i
 // A round is then the wave-wide maximum of the lanes' heads and a pop in the winning lane — the
 // per-lane scan over NPL registers, a chain of dependent compares and selects, leaves the
 // rounds.  The keys' original register indices travel in 4-bit fields of one word.
+// runner_up (optional): the expert ranked k + 1, or -1 when there is none, the same in every lane.
 template <int NPL>
 __device__ __forceinline__ void topk_select_sorted(uint32_t (&key)[NPL], int lane, int k, int* ids_row,
-                                                   float* ws_row) {
+                                                   float* ws_row, int* runner_up = nullptr) {
   static_assert(NPL <= 8, "4-bit index fields in one 32-bit word");
   uint32_t jj[NPL];
 #pragma unroll
@@ -194,6 +196,26 @@ __device__ __forceinline__ void topk_select_sorted(uint32_t (&key)[NPL], int lan
     ids_row[lane] = myid;
     ws_row[lane] = (float)((double)mine / wsum);
   }
+  if (runner_up) {
+    const uint32_t wm = wave_umax(key[0]);
+    const int wl = __builtin_ctzll(__ballot(key[0] == wm));
+    const int wj = __builtin_amdgcn_readlane((int)jw, wl) & 15;
+    *runner_up = wm != 0u ? NPL * wl + wj : -1;
+  }
+}
+
+// Gap that two neighbours among the k + 1 best logits must exceed for their order to be the reference's: 1e-6 (below
+// it two probabilities can round to one float, where the reference orders by index) + twice what a logit can lie
+// from the reference's value (tol: the two fp64 summation orders; 2 ulp: the roundings to f32 and the bias addition).
+// (ulps = 0 for logits that are the reference's own)
+__device__ __forceinline__ float topk_gap_needed(float la, float lb, float tol, float ulps = 4.8e-7f) {
+  return 1e-6f + 2.f * tol + ulps * fmaxf(fabsf(la), fabsf(lb));
+}
+// rows that the ranking by logit handles (block-uniform)
+template <int NPL>
+__device__ __forceinline__ bool topk_fast_handled(const float* lg, int E, int k) {
+  if constexpr (NPL == 8) return E % 4 == 0 && E >= 4 && k < E && k < 63 && ((uintptr_t)lg & 15) == 0;
+  return false;
 }
 
 // The softmax / top-k of one token by one wave (E <= 64 * NPL): lane l holds experts NPL*l .. NPL*l + NPL - 1
@@ -254,8 +276,13 @@ __device__ __forceinline__ void topk_wave(const float* __restrict__ lg, int* __r
 // costly part, are spread over the block; wave 0 then runs the k selection rounds on the keys in
 // LDS.  COH: the logits were written by other blocks of the same launch: read them with
 // device-scope loads.  ids_row / ws_row may point to global memory or LDS.
-template <int NPL, bool COH, int NT = 256>
-__device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, int k) {
+// CHECK: also returns (to every thread; one more barrier) the slack of the k + 1 best logits: the smallest gap between
+// neighbours minus what topk_gap_needed asks for at tol = 0 (-inf: a logit range in which probabilities underflow, or
+// NaNs).  The selection is certain when the slack exceeds 2 tol -- the verdict of topk_ids_by_logit below on the same
+// row, so that blocks which rank by logit and a block which runs this function agree on when to fall back.  Rows
+// that ranking does not handle return +inf (taken as they are).
+template <int NPL, bool COH, int NT = 256, bool CHECK = false>
+__device__ float topk_block(const float* lg, int* ids_row, float* ws_row, int E, int k, float ulps = 4.8e-7f) {
   constexpr int NPT = (64 * NPL + NT - 1) / NT;  // values per thread
   constexpr int NW = NT / 64;
   __shared__ float pb[64 * NPL];
@@ -263,6 +290,8 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
   __shared__ double red[NW];
   __shared__ float redf[NW];
   __shared__ int redx[NW];
+  __shared__ float slack;
+  __shared__ float lgs[CHECK ? 64 * NPL : 1];
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   __syncthreads();  // LDS of a previous token is no longer read
   float v[NPT];
@@ -272,6 +301,7 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
     const int e = tid + NT * j;
     v[j] = -INFINITY;
     if (e < E) v[j] = COH ? __hip_atomic_load(&lg[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
+    if (CHECK && e < 64 * NPL) lgs[e] = v[j];
     mxf = fmaxf(mxf, v[j]);
   }
   // The maximum: every wave reads the whole row itself (NPL values per lane, 16-byte loads; rows
@@ -341,16 +371,41 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
     if (e < 64 * NPL) keys[e] = e < E ? __float_as_uint((float)((double)p[j] / se)) + 1u : 0u;
   }
   __syncthreads();
-  if (wv != 0) return;
-  uint32_t key[NPL];
+  if (wv == 0) {
+    uint32_t key[NPL];
 #pragma unroll
-  for (int j = 0; j < NPL; j++) key[j] = keys[NPL * lane + j];
-#ifdef MOE_TOPK_SCAN
-  topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
-#else
-  if constexpr (NPL <= 8) topk_select_sorted<NPL>(key, lane, k, ids_row, ws_row);
-  else topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
-#endif
+    for (int j = 0; j < NPL; j++) key[j] = keys[NPL * lane + j];
+    if constexpr (NPL <= 8) {
+      int ru = -1;
+      topk_select_sorted<NPL>(key, lane, k, ids_row, ws_row, CHECK ? &ru : nullptr);
+      if constexpr (CHECK) {
+        float sl = INFINITY;
+        if (topk_fast_handled<NPL>(lg, E, k)) {
+          // lane r < k: the expert of rank r (its own write), lane k: the runner-up; each against the next rank
+          const int idr = lane < k ? ids_row[lane] : lane == k ? ru : -1;
+          const float la = idr >= 0 ? lgs[idr] : -INFINITY;
+          const float lb = __shfl_down(la, 1, 64);
+          const float lmax = __shfl(la, 0, 64);
+          float mine = INFINITY;
+          if (lane < k) {
+            const bool fine = idr >= 0 && lb > -INFINITY && lmax - lb < 70.f;  // false for NaNs
+            mine = fine ? (la - lb) - topk_gap_needed(la, lb, 0.f, ulps) : -INFINITY;
+            if (!(mine == mine)) mine = -INFINITY;
+          }
+          sl = -wave_fmax_dpp(-mine);
+        }
+        if (lane == 0) slack = sl;
+      }
+    } else {
+      topk_select_lm<NPL>(key, lane, k, ids_row, ws_row);
+      if (CHECK && lane == 0) slack = INFINITY;
+    }
+  }
+  if constexpr (CHECK) {
+    __syncthreads();
+    return slack;
+  }
+  return INFINITY;
 }
 
 // The k best experts of one token by their LOGITS, without the softmax: wave 0 of the block selects,
@@ -361,15 +416,19 @@ __device__ void topk_block(const float* lg, int* ids_row, float* ws_row, int E, 
 // probabilities whose ratio exceeds 1 + 2^-23 after both roundings, i.e. different floats in the same
 // order.  The function therefore checks the k + 1 best logits: every gap between neighbours above
 // 1e-6 and all of them within 70 of the maximum (probabilities that are normal floats) -> ids_row[0..k) (LDS)
-// holds the reference's ranking and true is returned; otherwise (also: rows it does not handle, NaNs) false,
-// and the caller runs the exact selection.
+// holds the reference's ranking and 1 is returned; 0: the ranking is not certain (also NaNs); -1: a row this
+// function does not handle; in both cases the caller runs the exact selection.
+// tol: how far a logit as it stands in lg can lie from the reference's value (the small-batch router sums the
+// products in a parallel order: a bound on the difference of the two fp64 sums, from the norms of the operands; the
+// roundings to f32 on top are charged here).  Gaps of the k + 1 best above 1e-6 + 2 (tol + 2 ulp) mean that the
+// reference's own logits are more than 1e-6 apart and in the same order.
 template <int NPL>
-__device__ bool topk_ids_by_logit(const float* lg, int* ids_row, int E, int k) {
+__device__ int topk_ids_by_logit(const float* lg, int* ids_row, int E, int k, float tol = 0.f, float ulps = 4.8e-7f) {
   __shared__ int fast_ok;
   const int tid = threadIdx.x, lane = tid & 63;
   bool handled = false;
-  if constexpr (NPL == 8) handled = E % 4 == 0 && E >= 4 && k < E && k < 63 && ((uintptr_t)lg & 15) == 0;
-  if (!handled) return false;  // block-uniform
+  handled = topk_fast_handled<NPL>(lg, E, k);
+  if (!handled) return -1;  // block-uniform
   if constexpr (NPL == 8) {
     if (tid < 64) {
       // lane-major keys: key[j] of lane l = expert 8 l + j; unsigned keys that order like the floats
@@ -430,13 +489,196 @@ __device__ bool topk_ids_by_logit(const float* lg, int* ids_row, int E, int k) {
       // the probabilities go subnormal or to zero, the reference sees ties there and orders them by index, so
       // such rows take the exact selection as well.
       const float lmax = __shfl(la, 0, 64);
-      const bool good = lane >= k || (mykey != 0u && nk != 0u && la - lb > 1e-6f && lmax - lb < 70.f);  // false for NaNs
+      const bool good = lane >= k || (mykey != 0u && nk != 0u && (la - lb) - topk_gap_needed(la, lb, 0.f, ulps) > 2.f * tol && lmax - lb < 70.f);  // false for NaNs; the same arithmetic as topk_block's slack
       const int ok = __all(good);
       if (lane < k) ids_row[lane] = myid;
       if (lane == 0) fast_ok = ok;
     }
     __syncthreads();
-    return fast_ok != 0;
+    return fast_ok != 0 ? 1 : 0;
   }
+  return -1;
+}
+
+// Every logit of token `tok` as the reference computes it (src/ref.cpp:70-77: one fp64 chain over the columns in
+// order, rounded to f32, + bias), a thread per expert, into out[0..E).  The slow, certain path: a block reads the
+// whole router matrix.
+template <int NT>
+__device__ void exact_logits_block(const moe_rfix& R, int tok, int E, float* out) {
+  // Two experts per thread (e and e + NT) as two interleaved chains, 32 columns per step with all of the step's
+  // loads requested before the first of its additions: the chains are bound by the latency of their loads, a thread's
+  // row being read 16 (f32) or 8 (bf16) bytes at a time out of L2.  d % 32 == 0 (moe_create).
+  const float* xr = R.x + (size_t)tok * R.d;
+  for (int e0 = threadIdx.x; e0 < E; e0 += 2 * NT) {
+    const int e1 = e0 + NT < E ? e0 + NT : e0;  // (no second expert: the first again, dropped below)
+    double a0 = 0.0, a1 = 0.0;
+    for (int c = 0; c < R.d; c += 32) {
+      float w0[32], w1[32];
+      if (R.bf16) {
+        const uint16_t* r0 = (const uint16_t*)R.W + (size_t)e0 * R.d + c;
+        const uint16_t* r1 = (const uint16_t*)R.W + (size_t)e1 * R.d + c;
+        uint4 u0[4], u1[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) { u0[i] = ((const uint4*)r0)[i]; u1[i] = ((const uint4*)r1)[i]; }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const uint32_t p0[4] = {u0[i].x, u0[i].y, u0[i].z, u0[i].w}, p1[4] = {u1[i].x, u1[i].y, u1[i].z, u1[i].w};
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            w0[8 * i + 2 * j] = __uint_as_float(p0[j] << 16);
+            w0[8 * i + 2 * j + 1] = __uint_as_float(p0[j] & 0xffff0000u);
+            w1[8 * i + 2 * j] = __uint_as_float(p1[j] << 16);
+            w1[8 * i + 2 * j + 1] = __uint_as_float(p1[j] & 0xffff0000u);
+          }
+        }
+      } else {
+        const float4* r0 = (const float4*)((const float*)R.W + (size_t)e0 * R.d + c);
+        const float4* r1 = (const float4*)((const float*)R.W + (size_t)e1 * R.d + c);
+        float4 f0[8], f1[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) { f0[i] = r0[i]; f1[i] = r1[i]; }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          w0[4 * i] = f0[i].x; w0[4 * i + 1] = f0[i].y; w0[4 * i + 2] = f0[i].z; w0[4 * i + 3] = f0[i].w;
+          w1[4 * i] = f1[i].x; w1[4 * i + 1] = f1[i].y; w1[4 * i + 2] = f1[i].z; w1[4 * i + 3] = f1[i].w;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 32; i++) {
+        const double xv = (double)xr[c + i];
+        a0 = fma((double)w0[i], xv, a0);
+        a1 = fma((double)w1[i], xv, a1);
+      }
+    }
+    float v0 = (float)a0, v1 = (float)a1;
+    if (R.bias) { v0 += R.bias[e0]; v1 += R.bias[e1]; }
+    out[e0] = v0;
+    if (e1 != e0) out[e1] = v1;
+  }
+}
+
+// One logit as the reference computes it, by one thread (32 columns per step, the step's loads requested together).
+__device__ __forceinline__ float exact_logit(const moe_rfix& R, int tok, int e) {
+  const float* xr = R.x + (size_t)tok * R.d;
+  double a0 = 0.0;
+  for (int c = 0; c < R.d; c += 32) {
+    float w0[32];
+    if (R.bf16) {
+      const uint4* r0 = (const uint4*)((const uint16_t*)R.W + (size_t)e * R.d + c);
+      uint4 u0[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) u0[i] = r0[i];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const uint32_t p0[4] = {u0[i].x, u0[i].y, u0[i].z, u0[i].w};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          w0[8 * i + 2 * j] = __uint_as_float(p0[j] << 16);
+          w0[8 * i + 2 * j + 1] = __uint_as_float(p0[j] & 0xffff0000u);
+        }
+      }
+    } else {
+      const float4* r0 = (const float4*)((const float*)R.W + (size_t)e * R.d + c);
+      float4 f0[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) f0[i] = r0[i];
+#pragma unroll
+      for (int i = 0; i < 8; i++) { w0[4 * i] = f0[i].x; w0[4 * i + 1] = f0[i].y; w0[4 * i + 2] = f0[i].z; w0[4 * i + 3] = f0[i].w; }
+    }
+#pragma unroll
+    for (int i = 0; i < 32; i++) a0 = fma((double)w0[i], (double)xr[c + i], a0);
+  }
+  float v = (float)a0;
+  if (R.bias) v += R.bias[e];
+  return v;
+}
+
+// The selection of one token by one block, certain to be the reference's: ids by logit order where the k + 1 best
+// are far enough apart for that (returns true; sel_ws untouched unless want_ws), else the exact softmax / top-k.
+// Where the gaps are within what the router launch's summation order can differ from the reference's by, the logits
+// that can reach the top k are recomputed in the reference's order first; if their exact values are more than 1e-6
+// apart, that settles it, and only a true near tie (where the reference's f32 probabilities decide, and with them
+// the exact normaliser) has the block recompute every logit.  All threads of the block call it; sel_ids / sel_ws are
+// LDS rows of the caller.  Every block of a launch that calls this for a token reaches the same verdicts: they see
+// the same logits and run the same arithmetic.
+template <int NPL, int NT>
+__device__ bool select_certain(const float* lg, const moe_rfix& R, int tok, int* sel_ids, float* sel_ws, int E, int k,
+                               bool want_ws) {
+  __shared__ __attribute__((aligned(16))) float lgfix[64 * NPL];
+  __shared__ float xsq[NT / 64];
+  float tol = 0.f;
+  if (!want_ws) {
+    tol = R.W && R.tol ? R.tol[tok] : 0.f;  // (blocks that only rank take the bound from the router launch)
+    const int r = topk_ids_by_logit<NPL>(lg, sel_ids, E, k, tol);
+    if (r == 1) return true;
+    if (r != 0 || !R.W) {  // rows the ranking does not handle, or no router operands: the logits as they stand
+      topk_block<NPL, false, NT>(lg, sel_ids, sel_ws, E, k);
+      return false;
+    }
+  } else {
+    if (!R.W) {
+      topk_block<NPL, false, NT>(lg, sel_ids, sel_ws, E, k);
+      return false;
+    }
+    // The exact selection on the logits as they stand, with the slack of the k + 1 best on the side.  Without a
+    // bound from the router launch the block takes |x| itself: the loads go out first and are summed after the
+    // selection, whose own loads and barriers they then overlap.
+    constexpr int PRE = 4;  // 16-byte loads per thread held in registers
+    float4 xv[PRE];
+    const bool own = R.tol == nullptr;
+    const float* xr = R.x + (size_t)tok * R.d;
+    if (own) {
+#pragma unroll
+      for (int i = 0; i < PRE; i++) {
+        const int c = 4 * ((int)threadIdx.x + NT * i);
+        xv[i] = c < R.d ? *(const float4*)(xr + c) : float4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    const float sl = topk_block<NPL, false, NT, true>(lg, sel_ids, sel_ws, E, k);
+    if (own) {
+      float a = 0.f;
+#pragma unroll
+      for (int i = 0; i < PRE; i++) a += xv[i].x * xv[i].x + xv[i].y * xv[i].y + xv[i].z * xv[i].z + xv[i].w * xv[i].w;
+      for (int c = 4 * ((int)threadIdx.x + NT * PRE); c < R.d; c += 4 * NT) {
+        const float4 v = *(const float4*)(xr + c);
+        a += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+      }
+      a = wave_sum(a);
+      if ((threadIdx.x & 63) == 0) xsq[threadIdx.x >> 6] = a;
+      __syncthreads();
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < NT / 64; w++) t += xsq[w];
+      tol = R.tol_scale * sqrtf(t) * 1.01f;
+      if (!(tol >= 0.f)) tol = INFINITY;  // (NaN / overflow: nothing is certain, take the slow path)
+    } else {
+      tol = R.tol[tok];
+    }
+    if (sl > 2.f * tol) return false;
+  }
+  // Not certain (block-uniform from here on).  sel_ids[k - 1] is the k-th best by the logits as they stand; an expert
+  // whose logit lies further below it than the margin cannot be among the reference's k best, nor come within 1e-6
+  // of them.
+  __syncthreads();
+  const float lk = lg[sel_ids[k - 1]];
+  const float margin = topk_gap_needed(lk, lk, tol) + 4.8e-7f * 70.f;  // (logits up to 70 above the k-th: their ulps)
+  bool full = !(lk == lk) || !(margin < INFINITY);
+  if (!full) {
+    for (int e = threadIdx.x; e < E; e += NT) {
+      const float v = lg[e];
+      lgfix[e] = v >= lk - margin ? exact_logit(R, tok, e) : v;  // (NaNs stay as they are)
+    }
+    __syncthreads();
+    if (!want_ws) {
+      if (topk_ids_by_logit<NPL>(lgfix, sel_ids, E, k, 0.f, 0.f) == 1) return true;
+      full = true;
+    } else {
+      if (topk_block<NPL, false, NT, true>(lgfix, sel_ids, sel_ws, E, k, 0.f) > 0.f) return false;
+      full = true;
+    }
+  }
+  exact_logits_block<NT>(R, tok, E, lgfix);
+  __syncthreads();
+  topk_block<NPL, false, NT>(lgfix, sel_ids, sel_ws, E, k);
   return false;
 }

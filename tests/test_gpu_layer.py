@@ -346,3 +346,53 @@ def test_stage_skipping_is_not_in_the_default_build_and_guarded_in_the_timing_tw
     assert torch.equal(mt.forward(0, x1), y_full)
     torch.cuda.synchronize()
     mt.close()
+
+
+@pytest.mark.parametrize("fmt,T,int_decode", [("q4cp", 1, 1), ("q4cp", 3, 1), ("q4cp", 7, 1), ("q4cp", 20, 1),
+                                               ("q4cp", 2, 0), ("q4k", 1, 1), ("q4k", 6, 1)])
+def test_small_batch_ids_when_summation_orders_disagree(oracle, fmt, T, int_decode):
+    """The small-batch router sums a logit's products lane-parallel, the reference one after the other
+    (src/ref.cpp:70-77); the two fp64 sums can differ, and with them the f32 logits.  Here they differ by far more
+    than an ulp: token activations with +-2^36 in two columns that cancel in one expert's row, so that the order of
+    the additions decides what is left of the small terms.  A ladder of experts whose logits are pure biases, 1e-5
+    apart, brackets that expert's sequential logit; wherever the parallel sum lands, its rank in the ladder is not
+    the reference's.  The library must notice that the gaps are within what the two orders can differ by (a bound
+    from the norms of the operands), recompute the logits in the reference's order and return the oracle's ids."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(101 + T)
+    d, mid, E, k = 1024, 256, 64, 8
+    bias = np.full(E, -30.0, np.float32)
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt, bias=bias)
+    A = 61                                     # the expert with the ill-conditioned sum (a high index: ties go to lower ones)
+    hl.router[:] = 0.0
+    hl.router[A] = rng.standard_normal(d).astype(np.float32) * np.float32(0.05)
+    hl.router[A, 0] = 1.0
+    hl.router[A, d - 1] = 1.0
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    x[:, 0] = np.float32(2.0 ** 36)
+    x[:, d - 1] = -np.float32(2.0 ** 36)
+    bias[A] = 0.0
+    # the sequential logit of A for token 0, then the ladder around it (every token sees the same ladder; the
+    # tokens' own values of A differ, so A's rank differs from token to token)
+    lgA = oracle.router(hl.oracle_layer().router, x, k, bias=bias)[0][:, A]
+    ladder = [e for e in range(E) if e != A][:40]
+    for j, e in enumerate(ladder):
+        bias[e] = np.float32(np.float64(lgA[0]) + (3.5 - j) * 1e-5)  # four rungs above A's logit, the others below
+    hl.bias = bias
+    ol = hl.oracle_layer()
+    lg, io, wo = oracle.router(ol.router, x, k, bias=bias)
+    # the parallel-order logits of the stateless entry point (the forward call's launches use other splits of the
+    # sum, with other roundings): they must not agree with the sequential ones, or the test tests nothing
+    import torch
+    Wd = torch.from_numpy(hl.router).cuda()
+    lt = capi.router_logits(capi.wview(Wd, capi.F32, E, d), torch.from_numpy(x).cuda(), torch.from_numpy(bias).cuda(), mode=0).cpu().numpy()
+    assert np.abs(lt[:, A].astype(np.float64) - lg[:, A]).max() > 2e-5, "the two summation orders (nearly) agree on this input: nothing to test"
+    m, dev = hl.to_gpu(max_tokens=32)
+    m.set_option(capi.OPT_INT_DECODE, int_decode)
+    y = m.forward(0, torch.from_numpy(x).cuda())
+    ids, ws = m.last_routing(T)
+    torch.cuda.synchronize()
+    ids = ids.cpu().numpy()
+    assert (ids[:, :k] == io[:, :k]).all(), (ids[:, :k], io[:, :k])
+    assert np.isfinite(y.cpu().numpy()).all()
+    m.close()
