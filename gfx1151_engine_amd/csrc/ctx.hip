@@ -63,7 +63,10 @@ struct moe_ctx {
   float* hid32 = nullptr;     // [min(T,small_max)][k+1][mid] f32 (small-batch path)
   uint32_t *xplanes = nullptr, *hplanes = nullptr;  // integer digit planes of x / hid (decode kernels)
   float2 *xmeta = nullptr, *hmeta = nullptr;
-  int small_max = 32;         // batches up to this size take the in-place GEMV path
+#ifndef MOE_SMALL_MAX
+#define MOE_SMALL_MAX 32
+#endif
+  int small_max = MOE_SMALL_MAX;         // batches up to this size take the in-place GEMV path
   bool int_decode = true;     // small batches: integer-dot kernels where they apply (else f32 kernels)
   // expert-sorted permutation (batch path; small batches that de-duplicate experts)
   moe_routing* routing = nullptr;
@@ -84,6 +87,7 @@ struct moe_ctx {
   float* pairs32 = nullptr;   // [(k+1)min(T,small_max)][d] unweighted pair rows of the unique-expert small-batch path
   bool fused_combine = false; // batch path: the down GEMM adds its weighted rows into y with f32 atomics (no pairs buffer, no reduce launch)
   int uq_min = 24;            // > 0: small batches of at least this many tokens read every distinct expert once
+  int lut_max = 5;            // q4cp layers off the integer-dot kernels: batches up to this size take the register-resident f32 down kernel
   int gu_topk_max = 4;        // batches up to this size run the softmax / top-k inside the gate/up launch (else in the router's launches)
   bool uq_gguf = false;       // the same for GGUF layers (off: their per-token kernels measure faster unless most tokens share experts)
   // per-stage timing (the reference's KP("moe:route|up|down|reduce") tags, 07_kprof.inc)
@@ -514,6 +518,10 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
     case MOE_OPT_SHARED_ASIDE: c->shared_aside = value != 0; return MOE_OK;
     case MOE_OPT_ROUTER_CANDIDATES: c->router_cand = value != 0; return MOE_OK;
     case MOE_OPT_UNIQUE_GGUF: c->uq_gguf = value != 0; return MOE_OK;
+    case MOE_OPT_F32_DECODE_MAX_TOKENS:
+      if (value < 0 || value > c->small_max) return MOE_E_INVALID;
+      c->lut_max = value;
+      return MOE_OK;
     case MOE_OPT_GU_TOPK_MAX_TOKENS:
       if (value < 0) return MOE_E_INVALID;
       c->gu_topk_max = value;
@@ -619,10 +627,16 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
                          (!sh || L.sh_gguf_type == MOE_GGML_Q4_K) && moe_dec4k_supported(g.d, g.mid, nslots_d);
   // q4cp codebooks that are not affine (the reference converter's fixed table, trained tables): the same launch
   // structure with look-up arithmetic
-  // (up to 5 tokens: 65 / 107 us against 78 / 119 for the plain f32 kernels at 2 / 4 tokens, but 163 against 141 at 8 --
-  // the look-up kernels win on latency, not on throughput)
-  const bool use_lut = L.has_q4cp && c->int_decode && !use_int && P <= 5 && (!sh || L.sh_gguf_type == 0) &&
+  // (the gate/up launch at every small-batch size -- 138 against 151 us at 20 tokens --, the down launch up to
+  //  lut_max tokens: 35 against 38 us at 4 tokens, but 135 against 91 at 20)
+  const bool use_lut = L.has_q4cp && c->int_decode && !use_int && (!sh || L.sh_gguf_type == 0) &&
                        moe_dec_supported(g.d, g.mid, nslots_d) && moe_dec_gu_topk_supported(g.experts, g.topk);
+  // the integer-dot kernels switched off: for a*n + b codebooks the same launches with f32 arithmetic (every weight a
+  // conversion and an FMA on the f32 activations; against the plain f32 kernels below, a lane keeps its group's
+  // activations in registers over the block's rows and the top-k rides in the gate/up launch)
+  const bool use_f32a = L.has_q4cp && !c->int_decode && L.experts_affine && (!sh || L.shared_affine) &&
+                        (!sh || L.sh_gguf_type == 0) && moe_dec_supported(g.d, g.mid, nslots_d) &&
+                        moe_dec_gu_topk_supported(g.experts, g.topk);
   // GGUF layers in other mixes of Q4_K / Q5_K / Q8_0 / Q5_1 (the reference checkpoints' types): the same integer-dot
   // launches, generalised over the block type
   const bool use_intgg = L.has_gguf && c->int_decode && !use_int4k &&
@@ -635,7 +649,7 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
                          (!sh || L.sh_gguf_type != 0);
   // integer-dot kernels: the gate/up launch runs the softmax / top-k itself (one launch less on the
   // latency-bound path than a top-k kernel, no last-block ticket in the logits launch)
-  const bool gu_topk = ((((use_int && !use_uq) || ((use_int4k || use_intgg) && !use_uq_gg)) && P <= c->gu_topk_max) || use_lut) &&
+  const bool gu_topk = (((use_int && !use_uq) || ((use_int4k || use_intgg) && !use_uq_gg) || use_lut || use_f32a) && P <= c->gu_topk_max) &&
                        moe_dec_gu_topk_supported(g.experts, g.topk);
   // (up to 4 tokens the router launch leaves each token's bound for the selection; larger batches: the selecting
   //  block takes the norm of x itself)
@@ -701,15 +715,20 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
                                  g.d, g.mid, y, (uint64_t)g.d, st);
       });
     }
-    if (use_lut) {
+    if (use_lut || use_f32a) {
       if ((rc = stage(MOE_PROF_UP, [&]() -> int {
-             return moe_launch_dec_gu_lut(&L.gate_up, shg, shu, x, c->logits, g.experts, c->ids, c->ws, g.id_stride,
-                                          g.topk, P, g.d, g.mid, c->hid32, st, &rf);
+             return moe_launch_dec_gu_lut(&L.gate_up, shg, shu, x, gu_topk ? c->logits : nullptr, g.experts, c->ids, c->ws,
+                                          g.id_stride, g.topk, P, g.d, g.mid, c->hid32, st, &rf, use_f32a);
            })))
         return rc;
       return stage(MOE_PROF_DOWN, [&]() -> int {
+        // (the down projection of more than a few tokens: the plain f32 kernel's blocks of 32 rows read a token's
+        //  hidden rows once for all of them and measure faster from about 6 tokens on)
+        if (P > c->lut_max)
+          return moe_launch_gemv_dn(&L.down, shd, c->sh_logit, nullptr, nullptr, c->hid32, c->ids, c->ws, g.id_stride,
+                                    g.topk, P, g.d, y, (uint64_t)g.d, st);
         return moe_launch_dec_dn_lut(&L.down, shd, c->sh_logit, c->hid32, c->ids, c->ws, g.id_stride, g.topk, P, g.d,
-                                     g.mid, y, (uint64_t)g.d, st);
+                                     g.mid, y, (uint64_t)g.d, st, use_f32a);
       });
     }
     if ((rc = stage(MOE_PROF_UP, [&]() -> int {

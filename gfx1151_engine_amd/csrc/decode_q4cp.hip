@@ -149,6 +149,42 @@ __device__ __forceinline__ float lut_dot(const uint4 cw, const XF& x, const floa
   return a0 + a1;
 }
 
+// The same kernels once more for codebooks a*n + b in plain f32 arithmetic (the integer-dot kernels switched off):
+// sum_k n_k * x_k over one group -- two masks per code word turn its even and odd nibbles into bytes, then a
+// byte-to-float conversion and an FMA per weight; the caller adds b * sum(x).
+__device__ __forceinline__ float aff_dot(const uint4 cw, const XF& x) {
+  const uint32_t w[4] = {cw.x, cw.y, cw.z, cw.w};
+  float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t lo = w[i] & 0x0f0f0f0fu, hi = (w[i] >> 4) & 0x0f0f0f0fu;
+    a0 = fmaf((float)(lo & 0xff), x.v[8 * i], a0);
+    a1 = fmaf((float)(hi & 0xff), x.v[8 * i + 1], a1);
+    a0 = fmaf((float)((lo >> 8) & 0xff), x.v[8 * i + 2], a0);
+    a1 = fmaf((float)((hi >> 8) & 0xff), x.v[8 * i + 3], a1);
+    a0 = fmaf((float)((lo >> 16) & 0xff), x.v[8 * i + 4], a0);
+    a1 = fmaf((float)((hi >> 16) & 0xff), x.v[8 * i + 5], a1);
+    a0 = fmaf((float)(lo >> 24), x.v[8 * i + 6], a0);
+    a1 = fmaf((float)(hi >> 24), x.v[8 * i + 7], a1);
+  }
+  return a0 + a1;
+}
+__device__ __forceinline__ float xf_sum(const XF& x) {
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < 32; i += 2) {
+    s0 += x.v[i];
+    s1 += x.v[i + 1];
+  }
+  return s0 + s1;
+}
+// MODE 1: the look-up (any codebook); MODE 2: cb[n] = a n + b0 in f32, sx = the sum of the group's activations
+template <int MODE>
+__device__ __forceinline__ float f32_dot(const uint4 cw, const XF& x, const float* lut_lane, float a, float b0, float sx) {
+  if (MODE == 2) return fmaf(a, aff_dot(cw, x), b0 * sx);
+  return lut_dot(cw, x, lut_lane);
+}
+
 struct GuArgs2 {
   DecW gu;           // fused gate_up [E*2*mid][d]
   DecW shg, shu;     // shared expert gate / up [mid][d] (codes == nullptr: none)
@@ -173,10 +209,11 @@ struct GuArgs2 {
 // ids and weights in every block; cheaper than a last-block ticket in the router launch plus a
 // dependent load of the ids here) and block (0, 0, token) writes ids / weights out for the down
 // kernel.  The shared expert's blocks skip it and have the CU to themselves meanwhile.
-// LUT (not with UQ): table look-up arithmetic (above) for any codebook; xf32 = the tokens' activations [P][d],
+// LUT = 1 (not with UQ): table look-up arithmetic (above) for any codebook; xf32 = the tokens' activations [P][d],
 // dynamic LDS = two tables (gate rows', up rows') and the token's d activations, hid goes out as f32 only.
+// LUT = 2: the same data flow with f32 arithmetic for codebooks a*n + b (no tables).
 constexpr int GU2_ROWS = 32;
-template <bool UQ, int NPL, bool LUT>
+template <bool UQ, int NPL, int LUT>
 __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __restrict__ xplanes,
                                                 const float2* __restrict__ xmeta,
                                                 const int* __restrict__ ids, int id_stride, int kpt, int d,
@@ -235,17 +272,19 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
   const DecW Wu = shared ? A.shu : A.gu;
   const float *lutg = lutmem + (lane & 31), *lutu = lutg;
   if (LUT) {
-    build_lut(lutmem, Wg.cb);
-    if (Wu.cb != Wg.cb) {  // (block-uniform) the shared expert's up_proj is a tensor with a codebook of its own
-      build_lut(lutmem + LUT_DW, Wu.cb);
-      lutu += LUT_DW;
+    if (LUT == 1) {
+      build_lut(lutmem, Wg.cb);
+      if (Wu.cb != Wg.cb) {  // (block-uniform) the shared expert's up_proj is a tensor with a codebook of its own
+        build_lut(lutmem + LUT_DW, Wu.cb);
+        lutu += LUT_DW;
+      }
     }
     // the token's activations, staged once per block: a lane fetches a group's 32 values when it starts on it
     const float4* xr = (const float4*)(xf32 + (size_t)blockIdx.z * d);
-    for (int i = threadIdx.x; i < d / 4; i += blockDim.x) ((float4*)(lutmem + 2 * LUT_DW))[i] = xr[i];
+    for (int i = threadIdx.x; i < d / 4; i += blockDim.x) ((float4*)(lutmem + (LUT == 1 ? 2 * LUT_DW : 0)))[i] = xr[i];
     __syncthreads();
   }
-  const float* xs = lutmem + 2 * LUT_DW;
+  const float* xs = lutmem + (LUT == 1 ? 2 * LUT_DW : 0);
   const uint64_t grow0 = shared ? 0 : (uint64_t)e * 2 * mid;
   const uint64_t urow0 = shared ? 0 : (uint64_t)e * 2 * mid + mid;
   const int r0 = blockIdx.x * GU2_ROWS + 4 * wv;  // first of this wave's 4 gate rows
@@ -300,16 +339,20 @@ __global__ void __launch_bounds__(512, 4) k_dec_gu(GuArgs2 A, const uint32_t* __
     // group gA of all eight rows first, then the tail group: one group's activations in registers at a time
     XF xf;
     load_xf(xf, xs + (size_t)gA * 32);
+    const float g0 = Wg.cb[0], u0 = Wu.cb[0];
+    float sx = LUT == 2 ? xf_sum(xf) : 0.f;
 #pragma unroll
     for (int p = 0; p < 4; p++) {
       const float* lt = p >= 2 ? lutu : lutg;
-      acc[2 * p] = __half2float(sa[p]) * mA * lut_dot(ca[p], xf, lt);
-      acc[2 * p + 1] = __half2float(sb[p]) * mA * lut_dot(cb[p], xf, lt);
+      const float a = p >= 2 ? ua : ga, b0 = p >= 2 ? u0 : g0;
+      acc[2 * p] = __half2float(sa[p]) * mA * f32_dot<LUT>(ca[p], xf, lt, a, b0, sx);
+      acc[2 * p + 1] = __half2float(sb[p]) * mA * f32_dot<LUT>(cb[p], xf, lt, a, b0, sx);
     }
     load_xf(xf, xs + (size_t)gB * 32);
+    sx = LUT == 2 ? xf_sum(xf) : 0.f;
 #pragma unroll
     for (int p = 0; p < 4; p++) {
-      const float vt = __half2float(st[p]) * mB * lut_dot(ct[p], xf, p >= 2 ? lutu : lutg);
+      const float vt = __half2float(st[p]) * mB * f32_dot<LUT>(ct[p], xf, p >= 2 ? lutu : lutg, p >= 2 ? ua : ga, p >= 2 ? u0 : g0, sx);
       if (lane < 32) acc[2 * p] += vt;
       else acc[2 * p + 1] += vt;
     }
@@ -393,9 +436,9 @@ constexpr int DN2_MAXSLOTS = 16;
 #ifndef MOE_DN_ROWS
 #define MOE_DN_ROWS 6
 #endif
-// LUT: table look-up arithmetic for any codebook; hid_f32 = [P][slots][mid], dynamic LDS = two tables (the routed
-// experts' tensor, the shared expert's).
-template <int ROWS, bool LUT>
+// LUT = 1: table look-up arithmetic for any codebook; hid_f32 = [P][slots][mid], dynamic LDS = two tables (the routed
+// experts' tensor, the shared expert's).  LUT = 2: f32 arithmetic for codebooks a*n + b, no tables.
+template <int ROWS, int LUT>
 __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __restrict__ hplanes,
                                                 const float2* __restrict__ hmeta,
                                                 const int* __restrict__ ids, const float* __restrict__ ws,
@@ -412,7 +455,7 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
   const int G = mid / 32, half = lane >> 5;
   const int r0 = blockIdx.x * ROWS;
   const size_t rb = (size_t)mid / 2;
-  if (LUT) {
+  if (LUT == 1) {
     build_lut(lutmem, A.dn.cb);
     if (has_shared) build_lut(lutmem + LUT_DW, A.shd.cb);
     __syncthreads();
@@ -465,9 +508,10 @@ __global__ void __launch_bounds__(512) k_dec_dn(DnArgs2 A, const uint32_t* __res
       }
     }
     __builtin_amdgcn_sched_barrier(0);  // every load is issued before the first dot product
+    const float b0 = LUT == 2 ? wcb[0] : 0.f, sxh = LUT == 2 ? xf_sum(xh) : 0.f;
 #pragma unroll
     for (int r = 0; r < ROWS; r++) {
-      float v = __half2float(sc[r]) * m * (LUT ? lut_dot(cw[r], xh, lt) : chunk_dot(cw[r], x, a, b));
+      float v = __half2float(sc[r]) * m * (LUT ? f32_dot<LUT>(cw[r], xh, lt, a, b0, sxh) : chunk_dot(cw[r], x, a, b));
       v = sum32(v);
       if (g_raw == 0 && s_raw < nslots) part[s_raw][r] = v;
       if ((r & 1) == 1) __builtin_amdgcn_sched_barrier(0);  // rows are consumed in arrival order
@@ -594,7 +638,7 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
   }
   if (!A.gu.cb) return MOE_E_STATE;
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0), P);
-  k_dec_gu<false, 0, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
+  k_dec_gu<false, 0, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, ids, id_stride, kpt, d, mid, hplanes, hmeta, hid_f32,
                                                   nullptr, nullptr, nullptr, 0, nullptr, nullptr, nullptr, nullptr, moe_rfix{});
   MOE_LAUNCH_CHECK();
   return MOE_OK;
@@ -622,10 +666,10 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
   if (!A.gu.cb) return MOE_E_STATE;
   dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);  // + the row of the exact top-k block
   if (n_experts <= 512)
-    k_dec_gu<false, 8, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
+    k_dec_gu<false, 8, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr, RFV);
   else
-    k_dec_gu<false, 16, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
+    k_dec_gu<false, 16, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, id_stride, kpt, d, mid, hplanes, hmeta,
                                                      hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, nullptr, RFV);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
@@ -633,31 +677,41 @@ int moe_launch_dec_gu_topk(const moe_wview* gu, const moe_wview* sh_gate, const 
 
 // The look-up kernels (any codebook): x f32 [P][d] in, hid f32 [P][kpt + shared][mid] out; softmax / top-k inside
 // the launch as above.
+// (affine: every codebook involved is a*n + b -- the f32 arithmetic instead of the look-up.  logits == nullptr: the
+//  ids are given and no selection runs inside the launch.)
 int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up, const float* x,
                           const float* logits, int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d,
-                          int mid, float* hid_f32, hipStream_t st, const moe_rfix* rf) {
-  if (!x || !hid_f32 || !logits || !moe_dec_gu_topk_supported(n_experts, kpt)) return MOE_E_INVALID;
+                          int mid, float* hid_f32, hipStream_t st, const moe_rfix* rf, bool affine) {
+  if (!x || !hid_f32 || !ids || (logits && !moe_dec_gu_topk_supported(n_experts, kpt))) return MOE_E_INVALID;
   const moe_rfix RFV = rf ? *rf : moe_rfix{};
   GuArgs2 A{};
   A.gu = decw(gu);
   A.shg = decw(sh_gate);
   A.shu = decw(sh_up);
-  dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + 1, P);
-  const int lds = 2 * LUT_DW * 4 + d * 4;
+  dim3 grid(mid / GU2_ROWS, kpt + (sh_gate ? 1 : 0) + (logits ? 1 : 0), P);
+  const int lds = (affine ? 0 : 2 * LUT_DW * 4) + d * 4;
   if (lds > 64 * 1024) return MOE_E_UNSUPPORTED;
-  if (n_experts <= 512)
-    k_dec_gu<false, 8, true><<<grid, 512, lds, st>>>(A, nullptr, nullptr, nullptr, id_stride, kpt, d, mid, nullptr, nullptr,
-                                                     hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x, RFV);
-  else
-    k_dec_gu<false, 16, true><<<grid, 512, lds, st>>>(A, nullptr, nullptr, nullptr, id_stride, kpt, d, mid, nullptr, nullptr,
-                                                      hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x, RFV);
+#define DEC_GU_F32(NPL, MODE)                                                                                          \
+  k_dec_gu<false, NPL, MODE><<<grid, 512, lds, st>>>(A, nullptr, nullptr, NPL ? nullptr : ids, id_stride, kpt, d, mid, nullptr, \
+                                                     nullptr, hid_f32, nullptr, nullptr, nullptr, n_experts, logits, ids, ws, x, RFV)
+  if (!logits) {
+    if (affine) DEC_GU_F32(0, 2);
+    else DEC_GU_F32(0, 1);
+  } else if (n_experts <= 512) {
+    if (affine) DEC_GU_F32(8, 2);
+    else DEC_GU_F32(8, 1);
+  } else {
+    if (affine) DEC_GU_F32(16, 2);
+    else DEC_GU_F32(16, 1);
+  }
+#undef DEC_GU_F32
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
 
 int moe_launch_dec_dn_lut(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit, const float* hid_f32,
                           const int* ids, const float* ws, int id_stride, int kpt, int P, int d, int mid, float* out,
-                          uint64_t out_stride, hipStream_t st) {
+                          uint64_t out_stride, hipStream_t st, bool affine) {
   DnArgs2 A{};
   A.dn = decw(dn);
   A.shd = decw(sh_down);
@@ -665,12 +719,17 @@ int moe_launch_dec_dn_lut(const moe_wview* dn, const moe_wview* sh_down, const f
   if (dn->rows > 0xffffffffull) return MOE_E_UNSUPPORTED;  // (row numbers are 32-bit in the kernel)
   const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
   constexpr int lds = 2 * LUT_DW * 4;
-  if (d % MOE_DN_ROWS == 0)
-    k_dec_dn<MOE_DN_ROWS, true><<<dim3(d / MOE_DN_ROWS, P), bs, lds, st>>>(A, nullptr, nullptr, ids, ws, id_stride, kpt, d,
-                                                                           mid, out, out_stride, hid_f32);
-  else
-    k_dec_dn<8, true><<<dim3(d / 8, P), bs, lds, st>>>(A, nullptr, nullptr, ids, ws, id_stride, kpt, d, mid, out,
-                                                       out_stride, hid_f32);
+#define DEC_DN_F32(ROWS, MODE)                                                                                          \
+  k_dec_dn<ROWS, MODE><<<dim3(d / ROWS, P), bs, MODE == 1 ? lds : 0, st>>>(A, nullptr, nullptr, ids, ws, id_stride, kpt, d, mid, \
+                                                                           out, out_stride, hid_f32)
+  if (d % MOE_DN_ROWS == 0) {
+    if (affine) DEC_DN_F32(MOE_DN_ROWS, 2);
+    else DEC_DN_F32(MOE_DN_ROWS, 1);
+  } else {
+    if (affine) DEC_DN_F32(8, 2);
+    else DEC_DN_F32(8, 1);
+  }
+#undef DEC_DN_F32
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -687,7 +746,7 @@ int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const mo
   A.shu = decw(sh_up);
   if (max_tiles <= 0) return MOE_OK;
   dim3 grid(mid / GU2_ROWS, max_tiles);
-  k_dec_gu<true, 0, false><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
+  k_dec_gu<true, 0, 0><<<grid, 512, 0, st>>>(A, xplanes, xmeta, nullptr, 0, 0, d, mid, hplanes, hmeta, nullptr, tiles,
                                                  ntiles, tokidx, n_experts, nullptr, nullptr, nullptr, nullptr, moe_rfix{});
   MOE_LAUNCH_CHECK();
   return MOE_OK;
@@ -720,9 +779,9 @@ int moe_launch_dec_dn(const moe_wview* dn, const moe_wview* sh_down, const float
   const int nslots = kpt + (sh_down ? 1 : 0), bs = 64 * ((nslots + 1) / 2);
   // MOE_DN_ROWS rows per block where that divides d (d = 3072: 512 blocks, two per CU), else 8
   if (d % MOE_DN_ROWS == 0)
-    k_dec_dn<MOE_DN_ROWS, false><<<dim3(d / MOE_DN_ROWS, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride, nullptr);
+    k_dec_dn<MOE_DN_ROWS, 0><<<dim3(d / MOE_DN_ROWS, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride, nullptr);
   else
-    k_dec_dn<8, false><<<dim3(d / 8, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride, nullptr);
+    k_dec_dn<8, 0><<<dim3(d / 8, P), bs, 0, st>>>(A, hplanes, hmeta, ids, ws, id_stride, kpt, d, mid, out, out_stride, nullptr);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }

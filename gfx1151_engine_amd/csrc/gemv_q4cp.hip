@@ -39,14 +39,16 @@ __device__ __forceinline__ float dot32(const uint4 pk, const float4* xv, const f
     const uint32_t v = w[i];
     const float4 x0 = xv[2 * i], x1 = xv[2 * i + 1];
     if (AFFINE) {
-      a0 = fmaf((float)(v & 0xf), x0.x, a0);
-      a1 = fmaf((float)((v >> 4) & 0xf), x0.y, a1);
-      a0 = fmaf((float)((v >> 8) & 0xf), x0.z, a0);
-      a1 = fmaf((float)((v >> 12) & 0xf), x0.w, a1);
-      a0 = fmaf((float)((v >> 16) & 0xf), x1.x, a0);
-      a1 = fmaf((float)((v >> 20) & 0xf), x1.y, a1);
-      a0 = fmaf((float)((v >> 24) & 0xf), x1.z, a0);
-      a1 = fmaf((float)(v >> 28), x1.w, a1);
+      // even and odd nibbles as bytes: two masks, then one byte-to-float conversion per weight
+      const uint32_t lo = v & 0x0f0f0f0fu, hi = (v >> 4) & 0x0f0f0f0fu;
+      a0 = fmaf((float)(lo & 0xff), x0.x, a0);
+      a1 = fmaf((float)(hi & 0xff), x0.y, a1);
+      a0 = fmaf((float)((lo >> 8) & 0xff), x0.z, a0);
+      a1 = fmaf((float)((hi >> 8) & 0xff), x0.w, a1);
+      a0 = fmaf((float)((lo >> 16) & 0xff), x1.x, a0);
+      a1 = fmaf((float)((hi >> 16) & 0xff), x1.y, a1);
+      a0 = fmaf((float)(lo >> 24), x1.z, a0);
+      a1 = fmaf((float)(hi >> 24), x1.w, a1);
     } else {
       a0 = fmaf(cbs[v & 0xf], x0.x, a0);
       a1 = fmaf(cbs[(v >> 4) & 0xf], x0.y, a1);
@@ -60,16 +62,6 @@ __device__ __forceinline__ float dot32(const uint4 pk, const float4* xv, const f
   }
   return a0 + a1;
 }
-__device__ __forceinline__ float sum32(const float4* xv) {
-  float s0 = 0.f, s1 = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; i += 2) {
-    s0 += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
-    s1 += (xv[i + 1].x + xv[i + 1].y) + (xv[i + 1].z + xv[i + 1].w);
-  }
-  return s0 + s1;
-}
-
 struct GuArgs {
   const uint8_t *codes, *scales;  // routed experts: fused gate_up [E*2*mid][d]
   const float* cb;
@@ -80,63 +72,38 @@ struct GuArgs {
   uint64_t sh_scale_stride;
 };
 
-// grid (mid / ROWS, slots per token incl. shared, P); block 256 = 4 waves.
+// grid (mid / rows, slots per token incl. shared, P); block 256 = 4 waves.
 // x of the token lies in LDS as float4 [j][g] (j-th quad of group g) so that lanes of
 // consecutive groups read consecutive 16-byte words.
-constexpr int GU_ROWS = 32;  // gate rows per block (and as many up rows)
-template <bool AFFINE>
-__device__ __forceinline__ void gu_rows(const uint8_t* gc, const uint8_t* gs, const uint8_t* uc,
-                                        const uint8_t* us, uint64_t ss, int d, int r0, int nrows,
-                                        CbInfo cg, CbInfo cu, const float* cbg, const float* cbu,
-                                        const float4* xs, float* hid_out) {
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int G = d / 32;
-  for (int rr = wv; rr < nrows; rr += 4) {
-    const int r = r0 + rr;
-    const uint8_t* grow = gc + (uint64_t)r * (d / 2);
-    const uint8_t* urow = uc + (uint64_t)r * (d / 2);
-    const __half* gsc = (const __half*)(gs + (uint64_t)r * ss);
-    const __half* usc = (const __half*)(us + (uint64_t)r * ss);
-    float ag = 0.f, au = 0.f;
-    for (int g = lane; g < G; g += 64) {
-      const uint4 pg = *(const uint4*)(grow + (size_t)g * 16);
-      const uint4 pu = *(const uint4*)(urow + (size_t)g * 16);
-      const float sg = __half2float(gsc[g]), su = __half2float(usc[g]);
-      float4 xv[8];
-#pragma unroll
-      for (int j = 0; j < 8; j++) xv[j] = xs[j * G + g];
-      float dg = dot32<AFFINE>(pg, xv, cbg), du = dot32<AFFINE>(pu, xv, cbu);
-      if (AFFINE) {
-        const float sx = sum32(xv);
-        dg = fmaf(cg.a, dg, cg.b * sx);
-        du = fmaf(cu.a, du, cu.b * sx);
-      }
-      ag = fmaf(dg, sg, ag);
-      au = fmaf(du, su, au);
-    }
-    ag = wave_sum(ag);
-    au = wave_sum(au);
-    if (lane == 0) hid_out[r] = silu_f(ag) * au;
-  }
-}
+// A wave works on two gate rows (and their up rows) at a time: the 2 G groups of the pair are dealt to the lanes as
+// units (unit u = row u / G, group u % G; 192 units = three per lane and pass), so that a row of 96 groups fills
+// all 64 lanes.  The loads of the next step are in flight while the current one is summed, and a block's first
+// loads leave before it stages x: at one token the launch is a few short blocks per CU, and what bounds it is how
+// many bytes are in flight, not arithmetic.
+constexpr int GU_NI = 3;
+struct GuUnit {
+  uint4 pg, pu;
+  __half sg, su;  // (converted where they are used: a conversion at the load would wait for it there)
+  float m;        // 0 for a unit past the pair's end
+};
 
 __global__ void __launch_bounds__(256) k_q4cp_gemv_gu(GuArgs A, const float* __restrict__ x,
                                                       uint64_t x_stride, const int* __restrict__ ids,
-                                                      int id_stride, int kpt, int d, int mid,
+                                                      int id_stride, int kpt, int d, int mid, int rows_per_block,
                                                       float* __restrict__ hid) {
-  extern __shared__ float4 xs[];  // d/4 float4
+  extern __shared__ float4 xs[];  // d/4 float4, then d/32 group sums of x
   __shared__ float cbg[16], cbu[16];
   const int s = blockIdx.y, tok = blockIdx.z;
   const bool shared = s >= kpt;
   const int G = d / 32;
-  const float* xt = x + (size_t)tok * x_stride;
-  for (int i = threadIdx.x; i < d / 4; i += blockDim.x) xs[(i & 7) * G + (i >> 3)] = ((const float4*)xt)[i];
-  const int r0 = blockIdx.x * GU_ROWS;
-  const int nrows = min(GU_ROWS, mid - r0);
+  float* const xsum = (float*)(xs + d / 4);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int r0 = blockIdx.x * rows_per_block;
+  const int nrows = min(rows_per_block, mid - r0);
   float* ho = hid + ((size_t)tok * gridDim.y + s) * mid;
   const uint8_t *gc, *gs, *uc, *us;
   uint64_t ss;
-  CbInfo cg, cu;
+  const float *cbgp, *cbup;
   if (!shared) {
     const int e = ids[(size_t)tok * id_stride + s];
     const uint64_t gr = (uint64_t)e * 2 * mid;
@@ -145,19 +112,94 @@ __global__ void __launch_bounds__(256) k_q4cp_gemv_gu(GuArgs A, const float* __r
     uc = A.codes + (gr + mid) * (d / 2);
     us = A.scales + (gr + mid) * A.scale_stride;
     ss = A.scale_stride;
-    cg = load_cb(A.cb, cbg);
-    cu = cg;
-    if (threadIdx.x < 16) cbu[threadIdx.x] = A.cb[threadIdx.x];
+    cbgp = cbup = A.cb;
   } else {
     gc = A.sh_gcodes; gs = A.sh_gscales; uc = A.sh_ucodes; us = A.sh_uscales;
     ss = A.sh_scale_stride;
-    cg = load_cb(A.sh_gcb, cbg);
-    cu = load_cb(A.sh_ucb, cbu);
-    if (threadIdx.x < 16) cbu[threadIdx.x] = A.sh_ucb[threadIdx.x];
+    cbgp = A.sh_gcb;
+    cbup = A.sh_ucb;
   }
+  // steps of this wave: (row pair q, pass p) with the pair at rows 2 wv + 8 q, units 192 p .. 192 p + 191
+  const int npass = (2 * G + 64 * GU_NI - 1) / (64 * GU_NI);
+  const int npairs = nrows > 2 * wv ? (nrows - 2 * wv + 7) / 8 : 0;
+  const int nsteps = npairs * npass;
+  auto load = [&](int st, GuUnit* u) {
+    const int q = st / npass, p = st - q * npass;
+    const int rr = 2 * wv + 8 * q;
+    const int lim = min(2, nrows - rr) * G;
+#pragma unroll
+    for (int i = 0; i < GU_NI; i++) {
+      // branch-free: a unit past the pair's end reads unit 0 and gets zero scales (loads under a divergent branch
+      // are waited for one by one; in straight-line code they are all in flight together)
+      const int idx0 = (p * GU_NI + i) * 64 + lane;
+      const bool ok = idx0 < lim;
+      const int idx = ok ? idx0 : 0;
+      const float m = ok ? 1.f : 0.f;
+      const int row = idx >= G ? 1 : 0, g = idx - row * G;
+      const uint64_t r = (uint64_t)(r0 + rr + row);
+      u[i].pg = *(const uint4*)(gc + r * (d / 2) + (size_t)g * 16);
+      u[i].pu = *(const uint4*)(uc + r * (d / 2) + (size_t)g * 16);
+      u[i].sg = ((const __half*)(gs + r * ss))[g];
+      u[i].su = ((const __half*)(us + r * ss))[g];
+      u[i].m = m;
+    }
+  };
+  GuUnit cur[GU_NI], nxt[GU_NI];
+  if (nsteps > 0) load(0, cur);
+  const float* xt = x + (size_t)tok * x_stride;
+  // (d / 4 is a multiple of 8: the eight quads of a group lie with eight neighbouring lanes)
+  for (int i = threadIdx.x; i < d / 4; i += blockDim.x) {
+    const float4 v = ((const float4*)xt)[i];
+    xs[(i & 7) * G + (i >> 3)] = v;
+    float t = (v.x + v.y) + (v.z + v.w);
+    t += __shfl_xor(t, 1, 64);
+    t += __shfl_xor(t, 2, 64);
+    t += __shfl_xor(t, 4, 64);
+    if ((i & 7) == 0) xsum[i >> 3] = t;
+  }
+  const CbInfo cg = load_cb(cbgp, cbg), cu = load_cb(cbup, cbu);
   __syncthreads();
-  if (cg.affine && cu.affine) gu_rows<true>(gc, gs, uc, us, ss, d, r0, nrows, cg, cu, cbg, cbu, xs, ho);
-  else gu_rows<false>(gc, gs, uc, us, ss, d, r0, nrows, cg, cu, cbg, cbu, xs, ho);
+  const bool affine = cg.affine && cu.affine;
+  float ag0 = 0.f, au0 = 0.f, ag1 = 0.f, au1 = 0.f;
+  for (int st = 0; st < nsteps; st++) {
+    if (st + 1 < nsteps) load(st + 1, nxt);
+    const int q = st / npass, p = st - q * npass;
+#pragma unroll
+    for (int i = 0; i < GU_NI; i++) {
+      const int idx = (p * GU_NI + i) * 64 + lane;
+      const int row = idx >= G ? 1 : 0;
+      const int g = min(idx - row * G, G - 1);  // (a unit past the pair's end has zero scales)
+      float4 xv[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) xv[j] = xs[j * G + g];
+      float dg, du;
+      if (affine) {
+        const float sx = xsum[g];
+        dg = fmaf(cg.a, dot32<true>(cur[i].pg, xv, cbg), cg.b * sx);
+        du = fmaf(cu.a, dot32<true>(cur[i].pu, xv, cbu), cu.b * sx);
+      } else {
+        dg = dot32<false>(cur[i].pg, xv, cbg);
+        du = dot32<false>(cur[i].pu, xv, cbu);
+      }
+      dg *= __half2float(cur[i].sg) * cur[i].m;
+      du *= __half2float(cur[i].su) * cur[i].m;
+      ag0 += row ? 0.f : dg;
+      au0 += row ? 0.f : du;
+      ag1 += row ? dg : 0.f;
+      au1 += row ? du : 0.f;
+    }
+    if (p == npass - 1) {
+      const int rr = 2 * wv + 8 * q;
+      ag0 = wave_sum(ag0); au0 = wave_sum(au0); ag1 = wave_sum(ag1); au1 = wave_sum(au1);
+      if (lane == 0) {
+        ho[r0 + rr] = silu_f(ag0) * au0;
+        if (rr + 1 < nrows) ho[r0 + rr + 1] = silu_f(ag1) * au1;
+      }
+      ag0 = au0 = ag1 = au1 = 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < GU_NI; i++) cur[i] = nxt[i];
+  }
 }
 
 struct DnArgs {
@@ -170,6 +212,132 @@ struct DnArgs {
   const float* sh_logit;  // [P] shared-expert gate logit (weight = sigmoid)
   const float *ey, *sg;   // alternative: precomputed shared-expert output [P][d] and gate logit [P]
 };
+
+// Few tokens: grid (d / 8, P); block 256.  hid of all the token's slots in LDS as float4 [slot][j][g].
+// A half-wave per output row, a lane per group (32 groups a pass); a lane has the codes and scales of all the
+// row's slots in flight at once, and a block's first loads leave before it stages hid.  Every slot's partial
+// stays in a register and the weighted sum runs in slot order (= descending router probability), then the shared
+// expert.
+constexpr int DNF_ROWS = 8;
+
+__device__ __forceinline__ float half_wave_sum(float v) {
+#pragma unroll
+  for (int o = 16; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+template <int NS>
+__global__ void __launch_bounds__(256) k_q4cp_gemv_dn_few(DnArgs A, const float* __restrict__ hid,
+                                                      const int* __restrict__ ids,
+                                                      const float* __restrict__ ws, int id_stride,
+                                                      int kpt, int d, int mid, int rows_per_block,
+                                                      float* __restrict__ out, uint64_t out_stride) {
+  extern __shared__ float4 hs[];  // nslots * mid/4 float4, then nslots * mid/32 group sums
+  __shared__ float cbr[16], cbsh[16];
+  const int tok = blockIdx.y;
+  const bool has_shared = A.sh_codes != nullptr;
+  const int nslots = kpt + (has_shared ? 1 : 0);
+  const int G = mid / 32, q = mid / 4;
+  float* const hsum = (float*)(hs + (size_t)nslots * q);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, l32 = lane & 31;
+  const int rb = blockIdx.x * rows_per_block + 2 * wv + (lane >> 5);  // this half-wave's first row; then every 8th
+  const int rend = min(d, (int)(blockIdx.x + 1) * rows_per_block);
+  const int npass = (G + 31) / 32;
+  // steps of this wave: (row pair it, pass p); the wave's lower half decides how many there are
+  const int rb0 = blockIdx.x * rows_per_block + 2 * wv;
+  const int npairs = rend > rb0 ? (rend - rb0 + 7) / 8 : 0;
+  const int nsteps = npairs * npass;
+  uint4 pk[NS];
+  __half sc[NS];  // (converted where they are used: a conversion at the load would wait for it there)
+  auto load = [&](int st) {
+    // branch-free (loads under a divergent branch are waited for one by one): a lane past the row's end, a row past
+    // the block's and a slot past the token's reads a valid address and gets a zero scale
+    const int it = st / npass, p = st - it * npass;
+    const int r = rb + 8 * it;
+    const bool live = r < rend;
+    const int g0 = p * 32 + l32;
+    const int g = g0 < G ? g0 : 0;
+    const uint64_t rr = live ? (uint64_t)r : 0;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+      const int se = s < nslots ? s : 0;
+      const bool sh = has_shared && se == nslots - 1;
+      const uint64_t row = sh ? rr : (uint64_t)ids[(size_t)tok * id_stride + (sh ? 0 : se)] * d + rr;
+      pk[s] = *(const uint4*)((sh ? A.sh_codes : A.codes) + row * (mid / 2) + (size_t)g * 16);
+      sc[s] = ((const __half*)((sh ? A.sh_scales : A.scales) + row * (sh ? A.sh_scale_stride : A.scale_stride)))[g];
+    }
+  };
+  if (nsteps > 0) load(0);
+  const float* ht = hid + (size_t)tok * nslots * mid;
+  for (int s = 0; s < nslots; s++)
+    for (int c = threadIdx.x; c < q; c += blockDim.x) {  // (q is a multiple of 8: a group's quads lie with eight neighbouring lanes)
+      const float4 v = ((const float4*)ht)[(size_t)s * q + c];
+      hs[((size_t)s * 8 + (c & 7)) * G + (c >> 3)] = v;
+      float t = (v.x + v.y) + (v.z + v.w);
+      t += __shfl_xor(t, 1, 64);
+      t += __shfl_xor(t, 2, 64);
+      t += __shfl_xor(t, 4, 64);
+      if ((c & 7) == 0) hsum[s * G + (c >> 3)] = t;
+    }
+  const CbInfo cr = load_cb(A.cb, cbr);
+  CbInfo cs = cr;
+  if (has_shared) cs = load_cb(A.sh_cb, cbsh);
+  __syncthreads();
+  const bool affine = cr.affine && cs.affine;
+  float acc[NS];
+#pragma unroll
+  for (int s = 0; s < NS; s++) acc[s] = 0.f;
+  for (int st = 0; st < nsteps; st++) {
+    const int it = st / npass, p = st - it * npass;
+    const int g = min(p * 32 + l32, G - 1);
+    const float m = (rb + 8 * it < rend && p * 32 + l32 < G) ? 1.f : 0.f;  // a lane past the row's end, a row past the block's
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+      if (s < nslots) {
+        const bool sh = has_shared && s == nslots - 1;
+        float4 xv[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) xv[j] = hs[((size_t)s * 8 + j) * G + g];
+        float dv;
+        if (affine) {
+          const CbInfo c = sh ? cs : cr;
+          dv = fmaf(c.a, dot32<true>(pk[s], xv, cbr), c.b * hsum[s * G + g]);
+        } else {
+          dv = dot32<false>(pk[s], xv, sh ? cbsh : cbr);
+        }
+        acc[s] = fmaf(dv, __half2float(sc[s]) * m, acc[s]);
+      }
+    }
+    if (st + 1 < nsteps) load(st + 1);
+    if (p == npass - 1) {
+      const int r = rb + 8 * it;
+      float y = 0.f;
+#pragma unroll
+      for (int s = 0; s < NS; s++) {
+        if (s < nslots) {
+          const float a = half_wave_sum(acc[s]);
+          const float w = s < kpt ? ws[(size_t)tok * id_stride + s] : sigmoid_f(A.sh_logit[tok]);
+          y += w * a;
+        }
+        acc[s] = 0.f;
+      }
+      if (r < rend && l32 == 0) {
+        if (A.ey) y += sigmoid_f(A.sg[tok]) * A.ey[(size_t)tok * d + r];
+        out[(size_t)tok * out_stride + r] = y;
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ float sum32(const float4* xv) {
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i += 2) {
+    s0 += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+    s1 += (xv[i + 1].x + xv[i + 1].y) + (xv[i + 1].z + xv[i + 1].w);
+  }
+  return s0 + s1;
+}
 
 // grid (d / ROWS, P); block 256.  hid of all the token's slots in LDS as float4 [slot][j][g].
 // Eight lanes per output row; every slot's partial stays in a register and the weighted sum runs
@@ -301,8 +469,11 @@ int moe_launch_gemv_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_
     A.sh_scale_stride = g.scale_stride;
     nslots++;
   }
-  dim3 grid((mid + GU_ROWS - 1) / GU_ROWS, nslots, P);
-  k_q4cp_gemv_gu<<<grid, 256, (size_t)d * 4, st>>>(A, x, x_stride, ids, id_stride, kpt, d, mid, hid);
+  // one row pair per wave where the launch would otherwise leave most of the device idle; more rows per block (one
+  // staging of x for all of them) once there are blocks enough
+  const int rows = (size_t)((mid + 7) / 8) * nslots * P <= 4096 ? 8 : 32;
+  dim3 grid((mid + rows - 1) / rows, nslots, P);
+  k_q4cp_gemv_gu<<<grid, 256, (size_t)d * 4 + (size_t)d / 8, st>>>(A, x, x_stride, ids, id_stride, kpt, d, mid, rows, hid);
   MOE_LAUNCH_CHECK();
   return MOE_OK;
 }
@@ -331,6 +502,16 @@ int moe_launch_gemv_dn(const moe_wview* dn, const moe_wview* sh_down, const floa
     Q4cpOps s = q4cp_ops(sh_down);
     A.sh_codes = s.codes; A.sh_scales = s.scales; A.sh_cb = s.cb; A.sh_scale_stride = s.scale_stride;
     A.sh_logit = sh_logit;
+  }
+  if ((size_t)((d + DNF_ROWS - 1) / DNF_ROWS) * P <= 1024) {
+    // few tokens: 32-row blocks would leave most of the device idle
+    dim3 grid((d + DNF_ROWS - 1) / DNF_ROWS, P);
+    const size_t lds = (size_t)nslots * mid * 4 + (size_t)nslots * mid / 8;
+    if (nslots <= 4) k_q4cp_gemv_dn_few<4><<<grid, 256, lds, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, DNF_ROWS, out, out_stride);
+    else if (nslots <= 11) k_q4cp_gemv_dn_few<11><<<grid, 256, lds, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, DNF_ROWS, out, out_stride);
+    else k_q4cp_gemv_dn_few<16><<<grid, 256, lds, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, DNF_ROWS, out, out_stride);
+    MOE_LAUNCH_CHECK();
+    return MOE_OK;
   }
   dim3 grid((d + DN_ROWS - 1) / DN_ROWS, P);
   const size_t lds = (size_t)nslots * mid * 4;

@@ -140,10 +140,10 @@ int moe_launch_dec_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_w
                       hipStream_t st, const moe_dec_v2* v2 = nullptr);
 int moe_launch_dec_gu_lut(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up, const float* x,
                           const float* logits, int n_experts, int* ids, float* ws, int id_stride, int kpt, int P, int d,
-                          int mid, float* hid_f32, hipStream_t st, const moe_rfix* rf = nullptr);
+                          int mid, float* hid_f32, hipStream_t st, const moe_rfix* rf = nullptr, bool affine = false);
 int moe_launch_dec_dn_lut(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit, const float* hid_f32,
                           const int* ids, const float* ws, int id_stride, int kpt, int P, int d, int mid, float* out,
-                          uint64_t out_stride, hipStream_t st);
+                          uint64_t out_stride, hipStream_t st, bool affine = false);
 int moe_launch_dec_gu_uq(const moe_wview* gu, const moe_wview* sh_gate, const moe_wview* sh_up,
                          const uint32_t* xplanes, const float2* xmeta, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, const int* tokidx, int n_experts, int d, int mid, uint32_t* hplanes,

@@ -310,13 +310,18 @@ int moe_forward_x16(moe_ctx* ctx, int layer, const float* x, const void* x16, in
  * (every block of a routed slot selects its token's experts itself: one launch less on the latency-bound path);
  * larger batches of the integer-dot kernels take the ids from the router's launches, so that the thousands of blocks
  * of such a launch do not each repeat the selection. */
+/* MOE_OPT_F32_DECODE_MAX_TOKENS (default 5; 0 .. 32): q4cp layers that do not run on the integer-dot kernels (a codebook
+ * that is not a*n + b, or MOE_OPT_INT_DECODE = 0) use f32 kernels in which a lane keeps its group's activations in
+ * registers over a block's rows (a look-up per weight for table codebooks, a conversion and an FMA for a*n + b); for
+ * batches of more than this many tokens the down projection goes to the plain f32 GEMV kernel instead, whose blocks of
+ * 32 rows read a token's hidden rows once (the measured crossover is between 4 and 6 tokens). */
 /* MOE_OPT_UNIQUE_GGUF (default 0): 1 = GGUF layers on the integer-dot kernels also take the distinct-expert path for
  * batches of MOE_OPT_UNIQUE_MIN_TOKENS .. 32 tokens (the reference's _uq kernels, 26_kernels_moe_gguf.inc:758-886:
  * every distinct expert's rows are read once per batch).  Off by default: at the benchmark's verify batch (20 tokens,
  * 30 % of the expert picks shared) the per-token kernels measure faster; it pays when most tokens share their experts. */
 enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2, MOE_OPT_FUSED_COMBINE = 3, MOE_OPT_SHARED_ASIDE = 4,
        MOE_OPT_TIMING_SKIP_STAGE = 5, MOE_OPT_ROUTER_CANDIDATES = 6, MOE_OPT_UNIQUE_GGUF = 7,
-       MOE_OPT_GU_TOPK_MAX_TOKENS = 8 };
+       MOE_OPT_GU_TOPK_MAX_TOKENS = 8, MOE_OPT_F32_DECODE_MAX_TOKENS = 9 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP
