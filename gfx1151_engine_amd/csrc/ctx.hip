@@ -14,6 +14,7 @@ struct MoeLayer {
   moe_wview router{};
   const float* router_bias = nullptr;
   float router_wmax = 0.f;  // the largest row norm of the router matrix (the bound of the small-batch selection, moe_rfix)
+  float router_bmax = 0.f;  // the largest |bias| (how far a logit's dot product can lie above the logit itself)
   moe_wview gate_up{}, down{};
   moe_gg_experts gg{};
   moe_wview sh_gate{}, sh_up{}, sh_down{}, sh_sg{};
@@ -292,6 +293,12 @@ MOE_API int moe_set_router(moe_ctx* c, int layer, const moe_wview* w, const floa
   if ((int)w->rows != c->cfg.experts || (int)w->cols != c->cfg.d) return MOE_E_INVALID;
   const int rn = moe_router_row_norm_max(w, c->sample, &L->router_wmax);
   if (rn) return rn;
+  L->router_bmax = 0.f;
+  if (bias) {
+    std::vector<float> hb((size_t)w->rows);
+    MOE_HIP(hipMemcpy(hb.data(), bias, hb.size() * 4, hipMemcpyDeviceToHost));
+    for (float b : hb) L->router_bmax = fmaxf(L->router_bmax, fabsf(b));
+  }
   L->router = *w;
   L->router_bias = bias;
   L->has_router = true;
@@ -927,7 +934,7 @@ static int router_batch(moe_ctx* c, MoeLayer& L, const float* x, int P, float* o
   const moe_wview* wx = L.has_shared ? &L.sh_sg : nullptr;
   if (c->router_cand && c->rc_scratch && moe_router_cand_supported(&L.router, wx, P, g.topk))
     return moe_router_batch_cand(&L.router, L.router_bias, wx, x, P, c->logits, c->sh_logit, out_xms, c->ids, c->ws,
-                                 g.topk, g.id_stride, c->rc_scratch, st);
+                                 g.topk, g.id_stride, c->rc_scratch, st, L.router_bmax);
   int rc = moe_router_logits_seq(&L.router, L.router_bias, wx, x, P, c->logits, c->sh_logit, out_xms, st);
   if (!rc) rc = moe_router_topk(c->logits, c->ids, c->ws, P, g.experts, g.topk, g.id_stride, st);
   return rc;

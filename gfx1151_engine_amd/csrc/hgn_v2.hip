@@ -246,26 +246,37 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {  // the reference
   return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
 }
 
-// One block per 128 x 128 tile (k_ht_deq_bf16, 28_kernels_hgn_v2.inc:386-440): 8 granules of 1 KiB (tile columns
-// 16g .. 16g+15), each of 8 blocks of 128 bytes (tile rows 16q .. 16q+15); word L of a block belongs to row L % 16,
-// column half L / 16, and carries 8 values, windows over the words L-1 (mod 32) : L.  The tile goes to LDS as f32
-// (element (r, c) at r * 128 + (c ^ (r >> 3)): the column pass reads rows 8 apart), is transformed down the columns,
-// then along the rows -- W = diag(svh) . H . G . H . diag(suh) / 128 with the butterflies in ascending stride order,
-// as the reference's fwht128 -- and leaves as bf16(v * (svh[R] / 128) * suh[C]).
+// One block per 128 x 128 tile of 8 KiB (format: k_ht_deq_bf16, 28_kernels_hgn_v2.inc:386-440).  Seen from the matrix
+// side, the tile is 128 rows x 16 column octets and every (row, octet) pair owns exactly one 32-bit word: octet o =
+// columns 8o .. 8o+7 lies in the 1 KiB granule o / 2, a granule holds eight 128-byte groups of 16 rows, and inside a
+// group the words of the even octet come first (word = row % 16), then the odd octet's.  The eight values of a word
+// are 16-bit windows that slide a nibble at a time over the word and its predecessor in the group (cyclically): column
+// 8o + 7 - s is the window at bit 4s of predecessor:word.  A thread takes one row and walks the octets.
+// The tile goes to LDS as f32 (element (r, c) at r * 128 + (c ^ (r >> 3)): the column pass reads rows 8 apart), is
+// transformed down the columns, then along the rows -- W = diag(svh) . H . G . H . diag(suh) / 128 with the
+// butterflies in ascending stride order, as the reference's fwht128 -- and leaves as bf16(v * (svh[R] / 128) * suh[C]).
 __global__ void __launch_bounds__(256) k_ht_to_bf16(const uint8_t* __restrict__ codes, const float* __restrict__ suh,
                                                     const float* __restrict__ svh, uint16_t* __restrict__ out, int K) {
   __shared__ float t[128 * 128];
-  const int ntx = K >> 7;
-  const int tile = blockIdx.x, ty = tile / ntx, tx = tile - ty * ntx;
-  const uint32_t* tb = (const uint32_t*)(codes + (size_t)tile * 8192);
-  const int tid = threadIdx.x, L = tid & 31;
-  for (int it = 0; it < 8; it++) {
-    const int blk = it * 8 + (tid >> 5), g = blk >> 3, q = blk & 7;
-    const uint32_t* bw = tb + g * 256 + q * 32;
-    const uint64_t V = ((uint64_t)bw[(L + 31) & 31] << 32) | bw[L];
-    const int r = q * 16 + (L & 15), c0 = g * 16 + (L >> 4) * 8;
+  const int tiles_across = K / 128;
+  const int ty = (int)blockIdx.x / tiles_across, tx = (int)blockIdx.x % tiles_across;
+  const uint32_t* words = (const uint32_t*)(codes + (size_t)blockIdx.x * 8192);
+  const int tid = threadIdx.x;
+  {
+    const int row = tid & 127;
+    const uint32_t* group = words + (row >> 4) * 32;  // this row's 128-byte group inside a granule
+    for (int octet = tid >> 7; octet < 16; octet += 2) {
+      const uint32_t* gw = group + (octet >> 1) * 256;
+      const int slot = (row & 15) | ((octet & 1) << 4);
+      const uint32_t cur = gw[slot], prev = gw[(slot - 1) & 31];
+      float* dst = t + row * 128;
+      const int swz = row >> 3;
 #pragma unroll
-    for (int e = 0; e < 8; e++) t[r * 128 + ((c0 + e) ^ (r >> 3))] = ht_val((uint32_t)(V >> (28 - 4 * e)) & 0xffffu);
+      for (int sft = 0; sft < 8; sft++) {
+        const uint32_t window = __builtin_amdgcn_alignbit(prev, cur, 4 * sft) & 0xffffu;
+        dst[(8 * octet + 7 - sft) ^ swz] = ht_val(window);
+      }
+    }
   }
   __syncthreads();
   const int j = tid & 15, vec = tid >> 4;  // 16 lanes per 128-vector, 8 elements each

@@ -113,7 +113,7 @@ bool moe_router_cand_supported(const moe_wview* W, const moe_wview* Wx, int P, i
 size_t moe_router_cand_scratch_bytes(int max_tokens, int experts, int d);
 int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
                           float* logits, float* out_x, float* out_xms, int* ids, float* ws, int k, int id_stride,
-                          void* scratch, hipStream_t st);
+                          void* scratch, hipStream_t st, float bias_max);
 
 size_t moe_qvec_plane_bytes(int K);
 size_t moe_qvec_meta_bytes(int K);

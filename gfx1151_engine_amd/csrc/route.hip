@@ -379,12 +379,14 @@ MOE_API int moe_routing_run_static(const int* ids, const float* ws, int* tokidx,
   if (P < 0 || k < 1 || id_stride < k || experts < 1) return MOE_E_INVALID;
   if (experts > RT_MAXE) return MOE_E_UNSUPPORTED;
   if (P > MOE_ROUTING_STATIC_MAX_TOKENS) return MOE_E_STATE;  // beyond the fixed scratch: use moe_routing_create / run
-  if (moe_route_small_supported(P, k, experts))
-    return moe_launch_route_small(ids, ws, tokidx, pw, eoff, pairids, P, k, experts, id_stride, nullptr, nullptr, 0,
-                                  -1, moe_s(st));
+  // (the look-up comes first, whatever the batch size: any call made outside a capture, P = 0 included, sets the
+  //  device up for later calls inside one)
   int* base = nullptr;
   const int rc = scratch_of_current_device(&base);
   if (rc) return rc;
+  if (moe_route_small_supported(P, k, experts))
+    return moe_launch_route_small(ids, ws, tokidx, pw, eoff, pairids, P, k, experts, id_stride, nullptr, nullptr, 0,
+                                  -1, moe_s(st));
   return routing_launch(base, base + (size_t)RT_STATIC_BLOCKS * RT_MAXE, ids, ws, tokidx, pw, eoff, pairids, P, k,
                         experts, id_stride, moe_s(st));
 }

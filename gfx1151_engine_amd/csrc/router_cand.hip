@@ -10,15 +10,17 @@
 //                        [a_e - B_e, a_e + B_e] that holds the exact logit; tau = the k-th largest lower end; every
 //                        expert whose upper end reaches tau - 1e-5 is a candidate (the true top k are among them:
 //                        at least k exact logits are >= tau, and a true top-k logit is >= the k-th largest exact one);
-//   3. k_router_exact_pairs the candidates' logits (typically 12-18 of 512) as the reference's sequential fp64
-//                        chains, one lane per (token, candidate), written over the approximate values;
-//   4. k_router_topk_mixed  ranks the k + 1 best logits; if every gap between neighbours exceeds 1e-6 and all lie
-//                        within 70 of the maximum, the order by logit is the reference's order by f32 probability
-//                        (no two of them can round to one float) and the ids are final; the weights use the exact
-//                        logits of the selected experts and a normaliser in which the non-candidates' terms are
-//                        approximate, which moves a renormalised weight by an ulp or two at most;
+//   3. k_router_pairs_split the candidates' logits (typically 12-18 of 512) as fp64 dot products, eight lanes per
+//                        (token, candidate), written over the approximate values: the reference's float, or in
+//                        rare cases its neighbour (the fp64 sum in another order than the reference's sequential
+//                        one can fall on the other side of a rounding boundary);
+//   4. k_router_topk_mixed  ranks the k + 1 best logits; if every gap between neighbours exceeds 1e-6 plus two ulps
+//                        and all lie within 70 of the maximum, the order by logit is the reference's order by f32
+//                        probability (no two of them can round to one float) and the ids are final; the weights use
+//                        these logits of the selected experts and a normaliser in which the non-candidates' terms
+//                        are approximate, which moves a renormalised weight by an ulp or two at most;
 //   5. tokens that fail any test (near ties, a logit range where probabilities underflow, more candidates than
-//      lanes, non-finite values) are listed and redone exactly: all E logits as fp64 chains and the exact softmax /
+//      lanes, non-finite values) are listed and redone exactly: all E logits as sequential fp64 chains (k_router_exact_pairs) and the exact softmax /
 //      top-k; when more than T/16 tokens are listed the dense fp64 kernel runs for the whole batch instead.
 // Error bound.  a~ = fl32(sum of f16(x_c) * f16(w_c)): |f16(v) - v| <= 2^-11 |v| + 2^-25 (the second term covers
 // f16 subnormals), so sum |x~ w~ - x w| <= 1.001 (2^-10 |x||w| + 2^-25 sqrt(d) (|x| + |w|)) by Cauchy-Schwarz, and
@@ -40,6 +42,7 @@ constexpr int RA_BT = 128, RA_BE = 128, RA_K = 32;
 constexpr int RA_PITCH = 80;   // bytes per LDS row: 32 f16 + 16 B of padding (the 16-byte fragment reads of 8 rows then cover all banks)
 constexpr int RA_CHUNK = 128;  // columns summed in the matrix pipe's f32 accumulators before they are added to the running sums
 constexpr int RC_SLOTS = 32;   // at most 31 candidates per token (+ the shared-expert gate row) in the exact pass
+constexpr int RC_NC_ULP = 1 << 20;  // flag in nc[t]: one of the token's candidate logits may be an ulp off the reference's float
 
 // ---- 1. approximate logits: block = 128 tokens x 128 experts, 4 waves as 2 x 2, wave = 64 x 64 (2 x 2 MFMA tiles) ----
 // The accumulators of the matrix pipe are flushed into running f32 sums every RA_CHUNK columns, which bounds the
@@ -518,41 +521,31 @@ __device__ __forceinline__ double chain_row(const void* wrow, const float* xrow,
   return acc;
 }
 
-// ---- 3. exact logits of the listed (token, row) pairs: a lane per pair, 64 pairs per wave ----
+// ---- 5. exact logits of the listed tokens, every expert: a lane per (token, row) pair, 64 pairs per wave ----
 // f32 weights: a wave stages the 64 weight-row pieces of an iteration (32 columns = one 128-byte line per row)
 // through LDS, so that a load instruction fetches 8 whole lines (8 lanes per row) instead of 16 bytes of 64
 // different lines; lane l of instruction i takes row 8i + l/8, piece (l%8 + l/8) % 8, which lands at byte 16 l of
 // the instruction's 1 KB image, and a lane reads its own row's piece j from slot 8a + (j - a) % 8, a = row % 8:
 // the 8 lanes of an LDS phase then hit 8 different 16-byte bank groups.  Two images per wave (next iteration in
 // flight), waves are independent (no block barrier).  Activations come straight from global memory: the pairs of
-// a token are neighbours in the list, so a wave touches a handful of rows.
-// LISTED = true is step 5: the pairs are (listed token, expert) for every expert, taken from the list of tokens
-// (fb_list, counters[0] entries; nothing to do when the dense kernel takes over) instead of from the pair list.
-template <bool BF16, bool LISTED = false>
+// a token are neighbours, so a wave touches one or two rows.  The pairs are (listed token, expert) for every expert,
+// taken from the list of tokens (fb_list, counters[0] entries; nothing to do when the dense kernel takes over).
+template <bool BF16>
 __global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restrict__ W, const float* __restrict__ bias,
-                                                            const void* __restrict__ Wx, const float* __restrict__ x,
-                                                            int E, int d, const uint32_t* __restrict__ pairs,
-                                                            const int* __restrict__ counters,
-                                                            float* __restrict__ logits, float* __restrict__ out_x,
-                                                            const int* __restrict__ fb_list = nullptr, int dense_above = 0) {
+                                                            const float* __restrict__ x, int E, int d,
+                                                            const int* __restrict__ counters, float* __restrict__ logits,
+                                                            const int* __restrict__ fb_list, int dense_above) {
   __shared__ __attribute__((aligned(16))) uint8_t img[4][2][8192];
-  int np;
-  if (LISTED) {
-    const int nl = counters[0];
-    if (nl == 0 || nl > dense_above) return;
-    np = nl * E;
-  } else {
-    np = counters[1];
-  }
+  const int nl = counters[0];
+  if (nl == 0 || nl > dense_above) return;
+  const int np = nl * E;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int p0 = (blockIdx.x * 4 + wv) * 64;
   if (p0 >= np) return;
   const bool live = p0 + lane < np;
   const int pi = live ? p0 + lane : p0;  // idle lanes repeat the wave's first pair (no extra traffic)
-  const uint32_t pr = LISTED ? ((uint32_t)fb_list[pi / E] << 10) | (uint32_t)(pi % E) : pairs[pi];
-  const int t = (int)(pr >> 10), e = (int)(pr & 1023u);
-  const bool gate = e == E;
-  const uint8_t* wrow = gate ? (const uint8_t*)Wx : (const uint8_t*)W + (size_t)e * d * (BF16 ? 2 : 4);
+  const int t = fb_list[pi / E], e = pi % E;
+  const uint8_t* wrow = (const uint8_t*)W + (size_t)e * d * (BF16 ? 2 : 4);
   const float* xrow = x + (size_t)t * d;
   double acc = 0.0;
   if constexpr (BF16) {
@@ -611,9 +604,92 @@ __global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restri
     }
   }
   if (!live) return;
+  float v = (float)acc;
+  if (bias) v += bias[e];
+  logits[(size_t)t * E + e] = v;
+}
+
+// ---- 3. the candidates' logits with the columns dealt to eight lanes ----
+// What step 4 needs from a candidate's logit is the fp64 dot product rounded to f32.  Summed in any order the fp64
+// value lies within delta = 2 (d + 8) 2^-53 |w||x| of the reference's sequential sum, so it rounds to the reference's
+// float unless a rounding boundary lies within delta of it; the kernel tests exactly that and marks the token
+// (RC_NC_ULP in nc[t], a few in ten thousand pairs) so that step 4 allows for an ulp in that token's gap test.  So
+// the candidates do not need the sequential chain (the listed tokens of step 5, whose ids hang on the last bit, keep it):
+// eight lanes share a pair, lane j takes the 16-byte piece j of every 128-byte line of the weight row (f32: columns
+// 32 i + 4 j ..; bf16: 64 i + 8 j ..) and the matching activations, so that a load instruction covers whole lines
+// without a trip through LDS, a lane's chain is an eighth as long, and a launch has eight times the waves to hide
+// the L2 round trips with.  Two accumulators per lane, then a three-step reduction; the order is fixed.
+template <bool BF16>
+__global__ void __launch_bounds__(256) k_router_pairs_split(const void* __restrict__ W, const float* __restrict__ bias,
+                                                            const void* __restrict__ Wx, const float* __restrict__ x,
+                                                            int E, int d, const uint32_t* __restrict__ pairs,
+                                                            const int* __restrict__ counters,
+                                                            float* __restrict__ logits, float* __restrict__ out_x,
+                                                            const float* __restrict__ wnorm, const float* __restrict__ xnorm,
+                                                            int* __restrict__ nc) {
+  constexpr int U = 8;                  // lines in flight per lane and operand
+  constexpr int LINE = BF16 ? 64 : 32;  // columns per 128-byte line of the weight row
+  constexpr int PIECE = LINE / 8;       // columns per lane and line
+  const int np = counters[1];
+  const int p_wave = (int)((blockIdx.x * 256 + (threadIdx.x & ~63u)) >> 3);
+  if (p_wave >= np) return;
+  const int p_mine = (int)((blockIdx.x * 256 + threadIdx.x) >> 3), j = threadIdx.x & 7;
+  const bool live = p_mine < np;
+  const uint32_t pr = pairs[live ? p_mine : p_wave];  // idle lanes repeat the wave's first pair (no extra traffic)
+  const int t = (int)(pr >> 10), e = (int)(pr & 1023u);
+  const bool gate = e == E;
+  const uint8_t* wrow = gate ? (const uint8_t*)Wx : (const uint8_t*)W + (size_t)e * d * (BF16 ? 2 : 4);
+  const float* xrow = x + (size_t)t * d + PIECE * j;
+  wrow += 16 * j;
+  double a0 = 0.0, a1 = 0.0;
+  auto mac = [&](const uint4 wq, const float4 xa, const float4 xb, double& acc) {
+    if (BF16) {
+      acc = fma((double)__uint_as_float(wq.x << 16), (double)xa.x, acc);
+      acc = fma((double)__uint_as_float(wq.x & 0xffff0000u), (double)xa.y, acc);
+      acc = fma((double)__uint_as_float(wq.y << 16), (double)xa.z, acc);
+      acc = fma((double)__uint_as_float(wq.y & 0xffff0000u), (double)xa.w, acc);
+      acc = fma((double)__uint_as_float(wq.z << 16), (double)xb.x, acc);
+      acc = fma((double)__uint_as_float(wq.z & 0xffff0000u), (double)xb.y, acc);
+      acc = fma((double)__uint_as_float(wq.w << 16), (double)xb.z, acc);
+      acc = fma((double)__uint_as_float(wq.w & 0xffff0000u), (double)xb.w, acc);
+    } else {
+      acc = fma((double)__uint_as_float(wq.x), (double)xa.x, acc);
+      acc = fma((double)__uint_as_float(wq.y), (double)xa.y, acc);
+      acc = fma((double)__uint_as_float(wq.z), (double)xa.z, acc);
+      acc = fma((double)__uint_as_float(wq.w), (double)xa.w, acc);
+    }
+  };
+  int c = 0;
+  for (; c + U * LINE <= d; c += U * LINE) {
+    uint4 wq[U];
+    float4 xa[U], xb[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      wq[u] = *(const uint4*)(wrow + (size_t)(c + u * LINE) * (BF16 ? 2 : 4));
+      xa[u] = *(const float4*)(xrow + c + u * LINE);
+      if (BF16) xb[u] = *(const float4*)(xrow + c + u * LINE + 4);
+      else xb[u] = float4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) mac(wq[u], xa[u], xb[u], (u & 1) ? a1 : a0);
+  }
+  for (; c < d; c += LINE) {  // the last lines (d is a multiple of 32 columns: of a bf16 row's last line, half may be missing)
+    if (c + PIECE * j + PIECE <= d) {
+      const uint4 wq = *(const uint4*)(wrow + (size_t)c * (BF16 ? 2 : 4));
+      const float4 xa = *(const float4*)(xrow + c);
+      const float4 xb = BF16 ? *(const float4*)(xrow + c + 4) : float4{0.f, 0.f, 0.f, 0.f};
+      mac(wq, xa, xb, a0);
+    }
+  }
+  double acc = a0 + a1;
+#pragma unroll
+  for (int o = 1; o < 8; o <<= 1) acc += __shfl_xor(acc, o, 64);
+  if (!live || j != 0) return;
   if (gate) out_x[t] = (float)acc;
   else {
     float v = (float)acc;
+    const double delta = (double)(2.f * (float)(d + 8) * 0x1p-53f * 1.01f) * (double)wnorm[e] * (double)xnorm[t];
+    if ((float)(acc - delta) != v || (float)(acc + delta) != v) atomicOr(&nc[t], RC_NC_ULP);  // (nc[t] < 0, a listed token: stays negative)
     if (bias) v += bias[e];
     logits[(size_t)t * E + e] = v;
   }
@@ -624,7 +700,7 @@ template <int NPL>
 __global__ void __launch_bounds__(256) k_router_topk_mixed(const float* __restrict__ lg, int* __restrict__ ids,
                                                            float* __restrict__ ws, int P, int E, int k, int id_stride,
                                                            const int* __restrict__ nc, int* __restrict__ fb_list,
-                                                           int* __restrict__ counters) {
+                                                           int* __restrict__ counters, float bias_max) {
   static_assert(NPL <= 8, "4-bit index fields in one 32-bit word");
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int t = blockIdx.x * 4 + wv;
@@ -676,7 +752,9 @@ __global__ void __launch_bounds__(256) k_router_topk_mixed(const float* __restri
   const float la = __uint_as_float((mykey & 0x80000000u) ? (mykey ^ 0x80000000u) : ~mykey);
   const float lb = __uint_as_float((nk & 0x80000000u) ? (nk ^ 0x80000000u) : ~nk);
   const float lmax = __shfl(la, 0, 64);
-  const bool good = lane >= k || (mykey != 0u && nk != 0u && la - lb > 1e-6f && lmax - lb < 70.f);  // false for NaNs
+  // (a marked token: either logit's dot product can be an ulp off the reference's float, see step 3; |dot| <= |logit| + |bias|)
+  const float ulp2 = (nc[t] & RC_NC_ULP) ? 0x1p-22f * (fmaxf(fabsf(la), fabsf(lb)) + bias_max) : 0.f;
+  const bool good = lane >= k || (mykey != 0u && nk != 0u && la - lb > 1e-6f + ulp2 && lmax - lb < 70.f);  // false for NaNs
   if (!__all(good)) {
     if (lane == 0) fb_list[atomicAdd(&counters[0], 1)] = t;
     return;
@@ -738,7 +816,7 @@ size_t moe_router_cand_scratch_bytes(int max_tokens, int experts, int d) {
 // up holding exact values for each token's candidates and approximate ones elsewhere.
 int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview* Wx, const float* x, int P,
                           float* logits, float* out_x, float* out_xms, int* ids, float* ws, int k, int id_stride,
-                          void* scratch, hipStream_t st) {
+                          void* scratch, hipStream_t st, float bias_max) {
   const int E = (int)W->rows, d = (int)W->cols;
   if (!moe_router_cand_supported(W, Wx, P, k) || !moe_aligned(x, 16)) return MOE_E_UNSUPPORTED;
   uint8_t* sp = (uint8_t*)scratch;
@@ -783,17 +861,17 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
                                          wx ? 1 : 0);
   MOE_LAUNCH_CHECK();
   // at most 32 pairs per token (31 candidates + the gate row); surplus blocks return at once
-  const unsigned gpair = (unsigned)(((size_t)P * RC_SLOTS + 255) / 256);
-  if (bf) k_router_exact_pairs<true><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x);
-  else k_router_exact_pairs<false><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x);
+  const unsigned gpair = (unsigned)(((size_t)P * RC_SLOTS * 8 + 255) / 256);  // eight lanes per pair
+  if (bf) k_router_pairs_split<true><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, wnorm, xnorm, nc);
+  else k_router_pairs_split<false><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, wnorm, xnorm, nc);
   MOE_LAUNCH_CHECK();
-  k_router_topk_mixed<8><<<gtok, 256, 0, st>>>(logits, ids, ws, P, E, k, id_stride, nc, fb_list, counters);
+  k_router_topk_mixed<8><<<gtok, 256, 0, st>>>(logits, ids, ws, P, E, k, id_stride, nc, fb_list, counters, bias_max);
   MOE_LAUNCH_CHECK();
   // the exact redo of the listed tokens: three launches that return at once when nothing is listed
   // (sized for the most tokens the listed path takes, dense_above of them; surplus blocks return at once)
   const unsigned glist = (unsigned)(((size_t)(dense_above > 0 ? dense_above : 1) * E + 255) / 256);
-  if (bf) k_router_exact_pairs<true, true><<<glist, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, fb_list, dense_above);
-  else k_router_exact_pairs<false, true><<<glist, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, fb_list, dense_above);
+  if (bf) k_router_exact_pairs<true><<<glist, 256, 0, st>>>(W->data, bias, x, E, d, counters, logits, fb_list, dense_above);
+  else k_router_exact_pairs<false><<<glist, 256, 0, st>>>(W->data, bias, x, E, d, counters, logits, fb_list, dense_above);
   MOE_LAUNCH_CHECK();
   int rc = moe_router_logits_seq_if(W, bias, nullptr, x, P, logits, nullptr, nullptr, counters, dense_above, st);
   if (rc) return rc;

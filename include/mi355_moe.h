@@ -116,7 +116,10 @@ int moe_routing_run(moe_routing* r, const int* ids, const float* ws, int* tokidx
  * histograms live in a fixed 1 MiB array inside the library's device image (one copy per GPU, kept until the
  * process ends), so nothing is allocated or freed, at the first call or later.  P <= MOE_ROUTING_STATIC_MAX_TOKENS
  * (MOE_E_STATE beyond it), experts <= 1024.  Every call on a GPU uses that GPU's one array: calls that
- * overlap on the same GPU (two streams or two host threads) race; calls on one stream are ordered. */
+ * overlap on the same GPU (two streams or two host threads) race; calls on one stream are ordered.
+ * The first call on each GPU looks the array's address up (hipGetSymbolAddress, under a mutex: host work, not a
+ * stream operation); make that call outside any stream capture -- one with P = 0 is enough -- and every later
+ * call, captured or not, only launches kernels. */
 enum { MOE_ROUTING_STATIC_MAX_TOKENS = 32768 };
 int moe_routing_run_static(const int* ids, const float* ws, int* tokidx, float* pw, int* eoff, int* pairids,
                            int P, int k, int experts, int id_stride, moe_stream_t st);
