@@ -10,7 +10,7 @@
 //                        [a_e - B_e, a_e + B_e] that holds the exact logit; tau = the k-th largest lower end; every
 //                        expert whose upper end reaches tau - 1e-5 is a candidate (the true top k are among them:
 //                        at least k exact logits are >= tau, and a true top-k logit is >= the k-th largest exact one);
-//   3. k_router_pairs_split the candidates' logits (typically 12-18 of 512) as fp64 dot products, eight lanes per
+//   3. k_router_pairs_token the candidates' logits (typically 12-18 of 512) as fp64 dot products, eight lanes per
 //                        (token, candidate), written over the approximate values: the reference's float, or in
 //                        rare cases its neighbour (the fp64 sum in another order than the reference's sequential
 //                        one can fall on the other side of a rounding boundary);
@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(256, 2) k_router_approx(const void* __restrict
   const int col = q % ncol, tt = (q / ncol) * 8 + xcd;  // the column blocks of a token tile share an XCD (and its L2 copy of x)
   if (b == 0 && tid == 0) {
     counters[0] = 0;  // tokens listed for the exact redo
-    counters[1] = 0;  // (token, row) pairs of the exact pass      (both are first used by later launches)
+    counters[1] = 0;  // (spare)                                   (first used by later launches)
   }
   if (tt >= ntt) return;
   const int e0 = col * RA_BE, t0 = tt * RA_BT;
@@ -189,7 +189,7 @@ __global__ void __launch_bounds__(256) k_router_w16(const void* __restrict__ W, 
   const int row = blockIdx.x * 4 + wv;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     counters[0] = 0;  // tokens listed for the exact redo
-    counters[1] = 0;  // (token, row) pairs of the exact pass      (both are first used by later launches)
+    counters[1] = 0;  // (spare)                                   (first used by later launches)
   }
   if (row >= Epad) return;
   float s2 = 0.f;
@@ -391,7 +391,6 @@ __global__ void __launch_bounds__(1024) k_router_cand(const float* __restrict__ 
                                                      const float* __restrict__ xnorm, int P, int E, int k, float eps,
                                                      float dterm, uint32_t* __restrict__ pairs, int* __restrict__ nc,
                                                      int* __restrict__ fb_list, int* __restrict__ counters, int gate_row) {
-  __shared__ int s_want[16], s_base;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int t = blockIdx.x * 16 + wv;
   const bool tok = t < P;
@@ -445,24 +444,11 @@ __global__ void __launch_bounds__(1024) k_router_cand(const float* __restrict__ 
   }
   const int total = __shfl(inc, 63, 64);
   const bool ok = __all(fin) && total <= RC_SLOTS - 1 && total >= 1 && (maxU - thr) < 60.f && isfinite(tau);
-  // The (token, row) pairs of the exact pass go into one dense list (token << 10 | row; row E = the shared-expert
-  // gate vector, which every token needs).  A token's pairs are contiguous; the order of the tokens in the list
-  // depends on timing, the result of a pair does not.
-  // (one atomic per block of 16 tokens: thousands of atomics on one address would serialise for longer than the
-  // rest of the kernel takes)
-  const int want = tok ? (ok ? total : 0) + gate_row : 0;
-  if (lane == 0) s_want[wv] = want;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int sum = 0;
-    for (int i = 0; i < 16; i++) sum += s_want[i];
-    s_base = sum ? atomicAdd(&counters[1], sum) : 0;
-  }
-  __syncthreads();
+  // The rows whose exact dot products step 3 computes for this token: pairs[t][0 .. n), the shared-expert gate vector
+  // (row E) first where there is one, then the candidates; nc[t] = the number of candidates, -1 for a listed token.
   if (!tok) return;
-  int base = s_base;
-  for (int i = 0; i < wv; i++) base += s_want[i];
-  if (gate_row && lane == 0) pairs[base] = ((uint32_t)t << 10) | (uint32_t)E;
+  uint32_t* mine_out = pairs + (size_t)t * RC_SLOTS;
+  if (gate_row && lane == 0) mine_out[0] = (uint32_t)E;
   if (!ok) {
     if (lane == 0) {
       nc[t] = -1;
@@ -470,10 +456,10 @@ __global__ void __launch_bounds__(1024) k_router_cand(const float* __restrict__ 
     }
     return;
   }
-  int pos = base + gate_row + inc - mine;
+  int pos = gate_row + inc - mine;
 #pragma unroll
   for (int j = 0; j < NPL; j++)
-    if (U[j] >= thr) pairs[pos++] = ((uint32_t)t << 10) | (uint32_t)(NPL * lane + j);
+    if (U[j] >= thr) mine_out[pos++] = (uint32_t)(NPL * lane + j);
   if (lane == 0) nc[t] = total;
 }
 
@@ -609,89 +595,108 @@ __global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restri
   logits[(size_t)t * E + e] = v;
 }
 
-// ---- 3. the candidates' logits with the columns dealt to eight lanes ----
+// ---- 3. the candidates' logits: a wave per token, eight lanes per (token, row) pair ----
 // What step 4 needs from a candidate's logit is the fp64 dot product rounded to f32.  Summed in any order the fp64
 // value lies within delta = 2 (d + 8) 2^-53 |w||x| of the reference's sequential sum, so it rounds to the reference's
 // float unless a rounding boundary lies within delta of it; the kernel tests exactly that and marks the token
 // (RC_NC_ULP in nc[t], a few in ten thousand pairs) so that step 4 allows for an ulp in that token's gap test.  So
-// the candidates do not need the sequential chain (the listed tokens of step 5, whose ids hang on the last bit, keep it):
-// eight lanes share a pair, lane j takes the 16-byte piece j of every 128-byte line of the weight row (f32: columns
-// 32 i + 4 j ..; bf16: 64 i + 8 j ..) and the matching activations, so that a load instruction covers whole lines
-// without a trip through LDS, a lane's chain is an eighth as long, and a launch has eight times the waves to hide
-// the L2 round trips with.  Two accumulators per lane, then a three-step reduction; the order is fixed.
+// the candidates do not need the sequential chain (the listed tokens of step 5, whose ids hang on the last bit, keep it).
+// A wave takes one token and eight of its rows at a time; lane j of a row's eight takes the 16-byte piece j of every
+// 128-byte line of the row, so that a load instruction covers eight whole lines, with no trip through LDS for the
+// weights.  The token's activations are the same for all rows: the wave fetches them once per pass, 256 columns per
+// load instruction, and hands them round through LDS -- loaded per lane like the weights they were half of the load
+// instructions, and the rate of those is what bounds this kernel.  The next chunk's weights are requested before the
+// current chunk is summed.  Two accumulators per lane, a three-step reduction; the order is fixed.
 template <bool BF16>
-__global__ void __launch_bounds__(256) k_router_pairs_split(const void* __restrict__ W, const float* __restrict__ bias,
+__global__ void __launch_bounds__(256) k_router_pairs_token(const void* __restrict__ W, const float* __restrict__ bias,
                                                             const void* __restrict__ Wx, const float* __restrict__ x,
-                                                            int E, int d, const uint32_t* __restrict__ pairs,
-                                                            const int* __restrict__ counters,
+                                                            int P, int E, int d, const uint32_t* __restrict__ pairs,
                                                             float* __restrict__ logits, float* __restrict__ out_x,
                                                             const float* __restrict__ wnorm, const float* __restrict__ xnorm,
-                                                            int* __restrict__ nc) {
-  constexpr int U = 8;                  // lines in flight per lane and operand
-  constexpr int LINE = BF16 ? 64 : 32;  // columns per 128-byte line of the weight row
-  constexpr int PIECE = LINE / 8;       // columns per lane and line
-  const int np = counters[1];
-  const int p_wave = (int)((blockIdx.x * 256 + (threadIdx.x & ~63u)) >> 3);
-  if (p_wave >= np) return;
-  const int p_mine = (int)((blockIdx.x * 256 + threadIdx.x) >> 3), j = threadIdx.x & 7;
-  const bool live = p_mine < np;
-  const uint32_t pr = pairs[live ? p_mine : p_wave];  // idle lanes repeat the wave's first pair (no extra traffic)
-  const int t = (int)(pr >> 10), e = (int)(pr & 1023u);
-  const bool gate = e == E;
-  const uint8_t* wrow = gate ? (const uint8_t*)Wx : (const uint8_t*)W + (size_t)e * d * (BF16 ? 2 : 4);
-  const float* xrow = x + (size_t)t * d + PIECE * j;
-  wrow += 16 * j;
-  double a0 = 0.0, a1 = 0.0;
-  auto mac = [&](const uint4 wq, const float4 xa, const float4 xb, double& acc) {
-    if (BF16) {
-      acc = fma((double)__uint_as_float(wq.x << 16), (double)xa.x, acc);
-      acc = fma((double)__uint_as_float(wq.x & 0xffff0000u), (double)xa.y, acc);
-      acc = fma((double)__uint_as_float(wq.y << 16), (double)xa.z, acc);
-      acc = fma((double)__uint_as_float(wq.y & 0xffff0000u), (double)xa.w, acc);
-      acc = fma((double)__uint_as_float(wq.z << 16), (double)xb.x, acc);
-      acc = fma((double)__uint_as_float(wq.z & 0xffff0000u), (double)xb.y, acc);
-      acc = fma((double)__uint_as_float(wq.w << 16), (double)xb.z, acc);
-      acc = fma((double)__uint_as_float(wq.w & 0xffff0000u), (double)xb.w, acc);
-    } else {
-      acc = fma((double)__uint_as_float(wq.x), (double)xa.x, acc);
-      acc = fma((double)__uint_as_float(wq.y), (double)xa.y, acc);
-      acc = fma((double)__uint_as_float(wq.z), (double)xa.z, acc);
-      acc = fma((double)__uint_as_float(wq.w), (double)xa.w, acc);
-    }
-  };
-  int c = 0;
-  for (; c + U * LINE <= d; c += U * LINE) {
-    uint4 wq[U];
-    float4 xa[U], xb[U];
+                                                            int* __restrict__ nc, int gate_row) {
+  constexpr int CH = 256;                    // columns of x per wave load
+  constexpr int LINE = BF16 ? 64 : 32;       // columns per 128-byte line of a weight row
+  constexpr int NL = CH / LINE;              // lines per chunk
+  constexpr int ESZ = BF16 ? 2 : 4;
+  __shared__ float4 xl[4][2][64];
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + wv;
+  if (t >= P) return;
+  const int ncv = nc[t];
+  const int cnt = (ncv < 0 ? 0 : ncv) + gate_row;  // (the marks of this launch are set after every wave's own read)
+  const int slot = lane >> 3, j = lane & 7;
+  const float* xrow = x + (size_t)t * d;
+  const uint32_t* mine = pairs + (size_t)t * RC_SLOTS;
+  const int nchunk = (d + CH - 1) / CH;
+  // (d is a multiple of 32 columns; a piece past the row's end is read from the row's last 16 bytes instead and meets
+  //  zeros in the activations' chunk)
+  const int last_piece = d * ESZ - 16;
+  for (int p0 = 0; p0 < cnt; p0 += 8) {
+    const bool live = p0 + slot < cnt;
+    const int e = (int)mine[live ? p0 + slot : p0];  // idle slots repeat the pass's first row (no extra traffic)
+    const bool gate = e == E;
+    const uint8_t* wrow = gate ? (const uint8_t*)Wx : (const uint8_t*)W + (size_t)e * d * ESZ;
+    double a0 = 0.0, a1 = 0.0;
+    uint4 wc[NL], wn[NL];
+    auto load_w = [&](int g, uint4* w) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-      wq[u] = *(const uint4*)(wrow + (size_t)(c + u * LINE) * (BF16 ? 2 : 4));
-      xa[u] = *(const float4*)(xrow + c + u * LINE);
-      if (BF16) xb[u] = *(const float4*)(xrow + c + u * LINE + 4);
-      else xb[u] = float4{0.f, 0.f, 0.f, 0.f};
-    }
+      for (int l = 0; l < NL; l++) {
+        const int off = (g * CH + l * LINE) * ESZ + 16 * j;
+        w[l] = *(const uint4*)(wrow + (off < last_piece ? off : last_piece));
+      }
+    };
+    load_w(0, wc);
+    float4 xn = 4 * lane < d ? *(const float4*)(xrow + 4 * lane) : float4{0.f, 0.f, 0.f, 0.f};
+    int buf = 0;
+    for (int g = 0; g < nchunk; g++) {
+      xl[wv][buf][lane] = xn;
+      if (g + 1 < nchunk) {
+        const int c1 = (g + 1) * CH + 4 * lane;
+        xn = c1 < d ? *(const float4*)(xrow + c1) : float4{0.f, 0.f, 0.f, 0.f};
+        load_w(g + 1, wn);
+      }
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the wave's own LDS writes
+      __builtin_amdgcn_wave_barrier();
+      const float4* xs = &xl[wv][buf][0];
 #pragma unroll
-    for (int u = 0; u < U; u++) mac(wq[u], xa[u], xb[u], (u & 1) ? a1 : a0);
-  }
-  for (; c < d; c += LINE) {  // the last lines (d is a multiple of 32 columns: of a bf16 row's last line, half may be missing)
-    if (c + PIECE * j + PIECE <= d) {
-      const uint4 wq = *(const uint4*)(wrow + (size_t)c * (BF16 ? 2 : 4));
-      const float4 xa = *(const float4*)(xrow + c);
-      const float4 xb = BF16 ? *(const float4*)(xrow + c + 4) : float4{0.f, 0.f, 0.f, 0.f};
-      mac(wq, xa, xb, a0);
-    }
-  }
-  double acc = a0 + a1;
+      for (int l = 0; l < NL; l++) {
+        double& acc = (l & 1) ? a1 : a0;
+        const uint4 u = wc[l];
+        if (BF16) {
+          const float4 x0 = xs[l * 16 + 2 * j], x1 = xs[l * 16 + 2 * j + 1];
+          acc = fma((double)__uint_as_float(u.x << 16), (double)x0.x, acc);
+          acc = fma((double)__uint_as_float(u.x & 0xffff0000u), (double)x0.y, acc);
+          acc = fma((double)__uint_as_float(u.y << 16), (double)x0.z, acc);
+          acc = fma((double)__uint_as_float(u.y & 0xffff0000u), (double)x0.w, acc);
+          acc = fma((double)__uint_as_float(u.z << 16), (double)x1.x, acc);
+          acc = fma((double)__uint_as_float(u.z & 0xffff0000u), (double)x1.y, acc);
+          acc = fma((double)__uint_as_float(u.w << 16), (double)x1.z, acc);
+          acc = fma((double)__uint_as_float(u.w & 0xffff0000u), (double)x1.w, acc);
+        } else {
+          const float4 x0 = xs[l * 8 + j];
+          acc = fma((double)__uint_as_float(u.x), (double)x0.x, acc);
+          acc = fma((double)__uint_as_float(u.y), (double)x0.y, acc);
+          acc = fma((double)__uint_as_float(u.z), (double)x0.z, acc);
+          acc = fma((double)__uint_as_float(u.w), (double)x0.w, acc);
+        }
+      }
 #pragma unroll
-  for (int o = 1; o < 8; o <<= 1) acc += __shfl_xor(acc, o, 64);
-  if (!live || j != 0) return;
-  if (gate) out_x[t] = (float)acc;
-  else {
-    float v = (float)acc;
-    const double delta = (double)(2.f * (float)(d + 8) * 0x1p-53f * 1.01f) * (double)wnorm[e] * (double)xnorm[t];
-    if ((float)(acc - delta) != v || (float)(acc + delta) != v) atomicOr(&nc[t], RC_NC_ULP);  // (nc[t] < 0, a listed token: stays negative)
-    if (bias) v += bias[e];
-    logits[(size_t)t * E + e] = v;
+      for (int l = 0; l < NL; l++) wc[l] = wn[l];
+      buf ^= 1;
+    }
+    double acc = a0 + a1;
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) acc += __shfl_xor(acc, o, 64);
+    if (live && j == 0) {
+      if (gate) out_x[t] = (float)acc;
+      else {
+        float v = (float)acc;
+        const double delta = (double)(2.f * (float)(d + 8) * 0x1p-53f * 1.01f) * (double)wnorm[e] * (double)xnorm[t];
+        if ((float)(acc - delta) != v || (float)(acc + delta) != v) atomicOr(&nc[t], RC_NC_ULP);
+        if (bias) v += bias[e];
+        logits[(size_t)t * E + e] = v;
+      }
+    }
   }
 }
 
@@ -860,10 +865,9 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
   k_router_cand<8><<<gtok16, 1024, 0, st>>>(logits, wnorm, xnorm, P, E, k, eps, dterm, pairs, nc, fb_list, counters,
                                          wx ? 1 : 0);
   MOE_LAUNCH_CHECK();
-  // at most 32 pairs per token (31 candidates + the gate row); surplus blocks return at once
-  const unsigned gpair = (unsigned)(((size_t)P * RC_SLOTS * 8 + 255) / 256);  // eight lanes per pair
-  if (bf) k_router_pairs_split<true><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, wnorm, xnorm, nc);
-  else k_router_pairs_split<false><<<gpair, 256, 0, st>>>(W->data, bias, wx, x, E, d, pairs, counters, logits, out_x, wnorm, xnorm, nc);
+  // at most 32 rows per token (31 candidates + the gate row): a wave per token, eight rows a pass
+  if (bf) k_router_pairs_token<true><<<gtok, 256, 0, st>>>(W->data, bias, wx, x, P, E, d, pairs, logits, out_x, wnorm, xnorm, nc, wx ? 1 : 0);
+  else k_router_pairs_token<false><<<gtok, 256, 0, st>>>(W->data, bias, wx, x, P, E, d, pairs, logits, out_x, wnorm, xnorm, nc, wx ? 1 : 0);
   MOE_LAUNCH_CHECK();
   k_router_topk_mixed<8><<<gtok, 256, 0, st>>>(logits, ids, ws, P, E, k, id_stride, nc, fb_list, counters, bias_max);
   MOE_LAUNCH_CHECK();
