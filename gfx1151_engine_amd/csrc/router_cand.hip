@@ -35,6 +35,7 @@
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef double double2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
@@ -512,25 +513,33 @@ __device__ __forceinline__ double chain_row(const void* wrow, const float* xrow,
 // through LDS, so that a load instruction fetches 8 whole lines (8 lanes per row) instead of 16 bytes of 64
 // different lines; lane l of instruction i takes row 8i + l/8, piece (l%8 + l/8) % 8, which lands at byte 16 l of
 // the instruction's 1 KB image, and a lane reads its own row's piece j from slot 8a + (j - a) % 8, a = row % 8:
-// the 8 lanes of an LDS phase then hit 8 different 16-byte bank groups.  Two images per wave (next iteration in
-// flight), waves are independent (no block barrier).  Activations come straight from global memory: the pairs of
-// a token are neighbours, so a wave touches one or two rows.  The pairs are (listed token, expert) for every expert,
-// taken from the list of tokens (fb_list, counters[0] entries; nothing to do when the dense kernel takes over).
+// the 8 lanes of an LDS phase then hit 8 different 16-byte bank groups.  The pairs are (listed token, expert) for
+// every expert, taken from the list of tokens (fb_list, counters[0] entries; nothing to do when the dense kernel
+// takes over).
+// A block is one wave = one listed token and 64 of its experts: with the few tokens that are listed in practice (near
+// ties: a couple in ten thousand) the launch is a handful of waves, and what it takes is the latency of one chain --
+// d / 32 steps of 32 columns, each a trip to L2, 64 f32 -> f64 conversions (quarter rate) and 32 dependent fp64 FMAs.
+// A step's operands are requested three steps ahead: the weight-row pieces (8 KB) and the token's 128 bytes of
+// activations (one load by eight lanes) go global -> LDS, three step buffers, and a step's buffer is re-filled as
+// soon as its operands are in registers.  (Six steps ahead with the next step's operands read during the current
+// step's FMAs measured slower, 65 against 54 us for a handful of tokens: the chain is bound by its own instructions,
+// not by the trips to memory any more; raising the wave's priority changes nothing either.)
 template <bool BF16>
-__global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restrict__ W, const float* __restrict__ bias,
-                                                            const float* __restrict__ x, int E, int d,
-                                                            const int* __restrict__ counters, float* __restrict__ logits,
-                                                            const int* __restrict__ fb_list, int dense_above) {
-  __shared__ __attribute__((aligned(16))) uint8_t img[4][2][8192];
+__global__ void __launch_bounds__(64) k_router_exact_pairs(const void* __restrict__ W, const float* __restrict__ bias,
+                                                           const float* __restrict__ x, int E, int d,
+                                                           const int* __restrict__ counters, float* __restrict__ logits,
+                                                           const int* __restrict__ fb_list, int dense_above, int wpt) {
+  constexpr int XD = 3;           // steps in flight
+  constexpr int SB = 8192 + 128;  // bytes of a step buffer: 64 rows x 128 B of weights, 128 B of activations
+  __shared__ __attribute__((aligned(16))) uint8_t img[XD * SB];
   const int nl = counters[0];
   if (nl == 0 || nl > dense_above) return;
-  const int np = nl * E;
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int p0 = (blockIdx.x * 4 + wv) * 64;
-  if (p0 >= np) return;
-  const bool live = p0 + lane < np;
-  const int pi = live ? p0 + lane : p0;  // idle lanes repeat the wave's first pair (no extra traffic)
-  const int t = fb_list[pi / E], e = pi % E;
+  const int lane = threadIdx.x;
+  const int tl = (int)blockIdx.x / wpt;  // wpt = waves per token = ceil(E / 64)
+  if (tl >= nl) return;
+  const int e_raw = ((int)blockIdx.x - tl * wpt) * 64 + lane;
+  const bool live = e_raw < E;
+  const int t = fb_list[tl], e = live ? e_raw : E - 1;  // (idle lanes repeat the last row)
   const uint8_t* wrow = (const uint8_t*)W + (size_t)e * d * (BF16 ? 2 : 4);
   const float* xrow = x + (size_t)t * d;
   double acc = 0.0;
@@ -547,38 +556,37 @@ __global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restri
       const uint32_t lo = (uint32_t)__shfl((int)(uint32_t)pw, from, 64), hi = (uint32_t)__shfl((int)(uint32_t)(pw >> 32), from, 64);
       src[i] = (const uint8_t*)(((uint64_t)hi << 32) | lo) + piece * 16;
     }
-    uint8_t* const my = &img[wv][0][0];
-    auto issue = [&](int c, int buf) {
+    auto issue = [&](int step, int buf) {  // nine loads
+      const int c = step * 32;
 #pragma unroll
       for (int i = 0; i < 8; i++)
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src[i] + (size_t)c * 4),
-                                         (__attribute__((address_space(3))) void*)(my + buf * 8192 + i * 1024), 16, 0, 0);
-    };
-    float4 xq[8];
-    auto loadx = [&](int c) {
-#pragma unroll
-      for (int i = 0; i < 8; i++) xq[i] = *(const float4*)(xrow + c + 4 * i);
+                                         (__attribute__((address_space(3))) void*)(&img[buf * SB + i * 1024]), 16, 0, 0);
+      if (lane < 8)  // lane l: columns c + 4 l .. of the token's activations, to byte 16 l behind the weights
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xrow + c + 4 * lane),
+                                         (__attribute__((address_space(3))) void*)(&img[buf * SB + 8192]), 16, 0, 0);
     };
     const int ar = lane & 7;
-    const uint8_t* rd = my + (lane >> 3) * 1024 + ar * 128;  // this lane's row inside an image
-    issue(0, 0);
-    loadx(0);
+    const int rd_w = (lane >> 3) * 1024 + ar * 128;  // this lane's row inside a step's weight image
+    const int n = d / 32;
+    for (int st = 0; st < XD && st < n; st++) issue(st, st);
     int buf = 0;
-    for (int c = 0; c < d; c += 32) {
-      float4 xv[8];
+    for (int it = 0; it < n; it++) {
+      // the loads of the steps behind this one stay in flight (nine per step; they retire in order)
+      const int behind = n - 1 - it < XD - 1 ? n - 1 - it : XD - 1;
+      if (behind >= 2) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+      else if (behind == 1) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      float4 w[8], xv[8];
 #pragma unroll
-      for (int i = 0; i < 8; i++) xv[i] = xq[i];
-      const bool more = c + 32 < d;
-      if (more) {
-        issue(c + 32, buf ^ 1);
-        loadx(c + 32);
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // all but the 16 loads just issued have landed (LDS image of this iteration)
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      for (int j = 0; j < 8; j++) {
+        w[j] = *(const float4*)(&img[buf * SB + rd_w + (((j - ar) & 7) << 4)]);
+        xv[j] = *(const float4*)(&img[buf * SB + 8192 + 16 * j]);
       }
-      float4 w[8];
-#pragma unroll
-      for (int j = 0; j < 8; j++) w[j] = *(const float4*)(rd + buf * 8192 + (((j - ar) & 7) << 4));
+      if (it + XD < n) {
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the step's operands are in registers, its buffer is free
+        issue(it + XD, buf);
+      }
 #pragma unroll
       for (int i = 0; i < 8; i++) {
         acc = fma((double)w[i].x, (double)xv[i].x, acc);
@@ -586,7 +594,7 @@ __global__ void __launch_bounds__(256) k_router_exact_pairs(const void* __restri
         acc = fma((double)w[i].z, (double)xv[i].z, acc);
         acc = fma((double)w[i].w, (double)xv[i].w, acc);
       }
-      buf ^= 1;
+      buf = buf + 1 == XD ? 0 : buf + 1;
     }
   }
   if (!live) return;
@@ -618,7 +626,9 @@ __global__ void __launch_bounds__(256) k_router_pairs_token(const void* __restri
   constexpr int LINE = BF16 ? 64 : 32;       // columns per 128-byte line of a weight row
   constexpr int NL = CH / LINE;              // lines per chunk
   constexpr int ESZ = BF16 ? 2 : 4;
-  __shared__ float4 xl[4][2][64];
+  // (the activations lie in LDS widened to f64: f32 -> f64 conversions run at a quarter of the FMA rate, and a lane
+  //  would otherwise convert the same 4 activations per line that the 63 other lanes convert too)
+  __shared__ double2v xl[4][2][128];
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int t = blockIdx.x * 4 + wv;
   if (t >= P) return;
@@ -649,7 +659,8 @@ __global__ void __launch_bounds__(256) k_router_pairs_token(const void* __restri
     float4 xn = 4 * lane < d ? *(const float4*)(xrow + 4 * lane) : float4{0.f, 0.f, 0.f, 0.f};
     int buf = 0;
     for (int g = 0; g < nchunk; g++) {
-      xl[wv][buf][lane] = xn;
+      xl[wv][buf][2 * lane] = double2v{(double)xn.x, (double)xn.y};
+      xl[wv][buf][2 * lane + 1] = double2v{(double)xn.z, (double)xn.w};
       if (g + 1 < nchunk) {
         const int c1 = (g + 1) * CH + 4 * lane;
         xn = c1 < d ? *(const float4*)(xrow + c1) : float4{0.f, 0.f, 0.f, 0.f};
@@ -657,13 +668,14 @@ __global__ void __launch_bounds__(256) k_router_pairs_token(const void* __restri
       }
       __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the wave's own LDS writes
       __builtin_amdgcn_wave_barrier();
-      const float4* xs = &xl[wv][buf][0];
+      const double2v* xs = &xl[wv][buf][0];
 #pragma unroll
       for (int l = 0; l < NL; l++) {
         double& acc = (l & 1) ? a1 : a0;
         const uint4 u = wc[l];
         if (BF16) {
-          const float4 x0 = xs[l * 16 + 2 * j], x1 = xs[l * 16 + 2 * j + 1];
+          const double2v xa = xs[l * 32 + 4 * j], xb = xs[l * 32 + 4 * j + 1], xc = xs[l * 32 + 4 * j + 2], xd = xs[l * 32 + 4 * j + 3];
+          struct { double x, y, z, w; } x0{xa.x, xa.y, xb.x, xb.y}, x1{xc.x, xc.y, xd.x, xd.y};
           acc = fma((double)__uint_as_float(u.x << 16), (double)x0.x, acc);
           acc = fma((double)__uint_as_float(u.x & 0xffff0000u), (double)x0.y, acc);
           acc = fma((double)__uint_as_float(u.y << 16), (double)x0.z, acc);
@@ -673,11 +685,11 @@ __global__ void __launch_bounds__(256) k_router_pairs_token(const void* __restri
           acc = fma((double)__uint_as_float(u.w << 16), (double)x1.z, acc);
           acc = fma((double)__uint_as_float(u.w & 0xffff0000u), (double)x1.w, acc);
         } else {
-          const float4 x0 = xs[l * 8 + j];
-          acc = fma((double)__uint_as_float(u.x), (double)x0.x, acc);
-          acc = fma((double)__uint_as_float(u.y), (double)x0.y, acc);
-          acc = fma((double)__uint_as_float(u.z), (double)x0.z, acc);
-          acc = fma((double)__uint_as_float(u.w), (double)x0.w, acc);
+          const double2v xa = xs[l * 16 + 2 * j], xb = xs[l * 16 + 2 * j + 1];
+          acc = fma((double)__uint_as_float(u.x), xa.x, acc);
+          acc = fma((double)__uint_as_float(u.y), xa.y, acc);
+          acc = fma((double)__uint_as_float(u.z), xb.x, acc);
+          acc = fma((double)__uint_as_float(u.w), xb.y, acc);
         }
       }
 #pragma unroll
@@ -873,9 +885,10 @@ int moe_router_batch_cand(const moe_wview* W, const float* bias, const moe_wview
   MOE_LAUNCH_CHECK();
   // the exact redo of the listed tokens: three launches that return at once when nothing is listed
   // (sized for the most tokens the listed path takes, dense_above of them; surplus blocks return at once)
-  const unsigned glist = (unsigned)(((size_t)(dense_above > 0 ? dense_above : 1) * E + 255) / 256);
-  if (bf) k_router_exact_pairs<true><<<glist, 256, 0, st>>>(W->data, bias, x, E, d, counters, logits, fb_list, dense_above);
-  else k_router_exact_pairs<false><<<glist, 256, 0, st>>>(W->data, bias, x, E, d, counters, logits, fb_list, dense_above);
+  const int wpt = (E + 63) / 64;  // a wave per token and 64 experts
+  const unsigned glist = (unsigned)((dense_above > 0 ? dense_above : 1) * wpt);
+  if (bf) k_router_exact_pairs<true><<<glist, 64, 0, st>>>(W->data, bias, x, E, d, counters, logits, fb_list, dense_above, wpt);
+  else k_router_exact_pairs<false><<<glist, 64, 0, st>>>(W->data, bias, x, E, d, counters, logits, fb_list, dense_above, wpt);
   MOE_LAUNCH_CHECK();
   int rc = moe_router_logits_seq_if(W, bias, nullptr, x, P, logits, nullptr, nullptr, counters, dense_above, st);
   if (rc) return rc;
