@@ -88,6 +88,34 @@ def test_small_batch_table_codebooks(oracle, T, kind):
     m.close()
 
 
+@pytest.mark.parametrize("limit", [0, 3, 32])
+@pytest.mark.parametrize("codebook", ["affine", "universal"])
+def test_f32_decode_token_limit(oracle, limit, codebook):
+    """MOE_OPT_F32_DECODE_MAX_TOKENS moves the batch size at which the f32 path's down launch changes from the
+    register-resident kernel to the plain one: every setting gives the oracle's ids and meets the f32 bar at 2, 4 and
+    20 tokens (affine codebook with the integer-dot kernels off; the converter's table with them on)."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(9100 + limit)
+    d, mid, E, k = 3072, 768, 24, 10
+    hl = HostLayer(rng, d, mid, E, k, codebook=S.UNIVERSAL_CODEBOOK, scale_std=0.05) if codebook == "universal" else \
+        HostLayer(rng, d, mid, E, k)
+    m, dev = hl.to_gpu(max_tokens=32)
+    if codebook == "affine":
+        m.set_option(capi.OPT_INT_DECODE, 0)
+    m.set_option(capi.OPT_F32_DECODE_MAX_TOKENS, limit)
+    for T in (2, 4, 20):
+        x = rng.standard_normal((T, d), dtype=np.float32)
+        yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+        y = m.forward(0, gpu(x)).cpu().numpy()
+        ids, ws = m.last_routing(T)
+        assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all(), T
+        assert np.abs(ws.cpu().numpy()[:, :k] - wo[:, :k]).max() <= 1e-6
+        assert max_abs_rel(y, yo) <= TOL_GEMV, (T, max_abs_rel(y, yo))
+    with pytest.raises(capi.MoeError):
+        m.set_option(capi.OPT_F32_DECODE_MAX_TOKENS, 33)
+    m.close()
+
+
 @pytest.mark.parametrize("fmt,T,rdt", [("q4cp", 3, "f32"), ("q4cp", 32, "f32"), ("q4k", 27, "f32"), ("q4k", 2, "f32"),
                                         ("q4cp", 1, "bf16"), ("q4cp", 4, "bf16"), ("q4cp", 5, "f32"), ("q4cp", 11, "f32"), ("q4cp", 12, "bf16"), ("q4cp", 17, "f32"),
                                         ("q4k", 30, "bf16")])
@@ -105,10 +133,13 @@ def test_small_batch_sizes_and_router_dtypes(oracle, fmt, T, rdt):
     assert max_abs_rel(y, yo) <= tol_small(fmt), max_abs_rel(y, yo)
 
 
-@pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 9), ("q4k", 1), ("q4k", 9)])
+@pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 3), ("q4cp", 5), ("q4cp", 6), ("q4cp", 9), ("q4cp", 32),
+                                   ("q4k", 1), ("q4k", 9)])
 def test_int_decode_switch(oracle, fmt, T):
     """MOE_OPT_INT_DECODE 1 (integer-dot kernels, default) and 0 (f32 kernels) both meet the GEMV bar
-    and select the same experts."""
+    and select the same experts.  (q4cp with the switch at 0: up to 4 tokens the register-resident f32 kernels with
+    the top-k inside the gate/up launch, at 5 with the ids from the router's launches, from 6 on the plain f32 down
+    kernel behind the register-resident gate/up launch.)"""
     from gfx1151_engine_amd import capi
     rng = np.random.default_rng(77 + T)
     d, mid, E, k = 3072, 768, 16, 10
