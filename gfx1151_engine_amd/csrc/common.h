@@ -88,16 +88,33 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 // Range guard of the f16 intermediates of the batch path.  hid = silu(g)*u and the down-projection
 // pairs are kept in f16; for weights with large scales (raw Q4_K blocks with big sub-scales) their
-// magnitude, ~ C * mean(x^2) with C a per-layer constant from the weights' row norms, can pass
-// 65504.  The gate/up epilogue multiplies hid by this power of two (<= 1; exactly 1 while the
-// estimate stays below 16), the pairs inherit it and the combine divides it out in f32: exact
-// except for f16 underflow 2^-14 below the typical value.
-__device__ __forceinline__ float moe_hid_scale(float C, float xms) {
-  const float est = C * xms;
-  if (!(est > 16.f)) return 1.f;
+// magnitude, ~ C.hi * mean(x^2) with C.hi a per-layer constant from the weights' row norms (the larger of
+// hid's and the pairs' typical magnitude at unit activations), can pass 65504.  The gate/up epilogue
+// multiplies hid by this power of two (exactly 1 while the estimate stays below 16), the pairs inherit it
+// and the combine divides it out in f32: exact.  The other side: with very small weights the smaller of the
+// two magnitudes, ~ C.lo * mean(x^2), heads for f16's subnormal range (below 2^-14, where a value keeps fewer
+// than 11 bits); under 2^-10 the factor is a power of two above 1 that brings it to about 2^-6, as far as the
+// larger magnitude stays below 16.  Exactly 1 for ordinary weights (the benchmark's layers: 4 and 4).
+struct moe_cmag {
+  float hi, lo;
+};
+__device__ __forceinline__ float moe_hid_scale(moe_cmag C, float xms) {
+  const float est = C.hi * xms;
   int e;
-  (void)frexpf(est * 0.0625f, &e);  // est/16 = m * 2^e, m in [0.5, 1)
-  return ldexpf(1.f, -e);
+  if (est > 16.f) {
+    (void)frexpf(est * 0.0625f, &e);  // est/16 = m * 2^e, m in [0.5, 1)
+    return ldexpf(1.f, -e);
+  }
+  const float lo = C.lo * xms;
+  if (lo > 0.f && lo < 0x1p-10f) {
+    (void)frexpf(lo, &e);      // lo = m * 2^e, m in [0.5, 1)
+    int up = -6 - e;           // lo * 2^up in [2^-7, 2^-6)
+    int eh;
+    (void)frexpf(est, &eh);    // est < 2^eh
+    up = up < 4 - eh ? up : 4 - eh;  // est * 2^up < 16
+    return up > 0 ? ldexpf(1.f, up) : 1.f;
+  }
+  return 1.f;
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }

@@ -24,7 +24,7 @@ struct MoeLayer {
   bool experts_affine = false, shared_affine = false;
   // f16 range guard of the batch path: typical |hid| (and |pair|) per unit mean-square activation,
   // estimated from sampled weight rows when the weights are registered
-  float c_routed = 0.f, c_shared = 0.f;
+  moe_cmag c_routed{0.f, 0.f}, c_shared{0.f, 0.f};  // f16 range guard constants (common.h), 0 = no guard
   // hgn v2 rotated experts (gate_up / down are MOE_DT_I4R views): the sign-scale planes of the two tensors, f32
   bool has_i4r = false;
   const float *v2_su = nullptr, *v2_svh_gu = nullptr, *v2_suh_dn = nullptr, *v2_svh_dn = nullptr;
@@ -45,7 +45,7 @@ struct moe_ctx;
 static int pexp_register(moe_ctx* c, int layer, int slot0, const moe_wview* a, const moe_wview* b, int n_experts);
 static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gate, uint64_t gate_stride,
                               const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
-                              float* out);
+                              moe_cmag* out);
 
 struct moe_ctx {
   moe_config cfg;
@@ -371,7 +371,7 @@ MOE_API int moe_set_experts_i4r(moe_ctx* c, int layer, const moe_wview* gu, cons
   L->gate_up = *gu;
   L->down = *dn;
   L->v2_su = su; L->v2_svh_gu = svh_gu; L->v2_suh_dn = suh_dn; L->v2_svh_dn = svh_dn;
-  L->c_routed = 0.f;  // (no f16 range guard on these launches: the reference's have none either)
+  L->c_routed = moe_cmag{0.f, 0.f};  // (no f16 range guard on these launches: the reference's have none either)
   L->experts_affine = true;
   L->has_i4r = true;
   L->has_q4cp = false;
@@ -389,7 +389,7 @@ MOE_API int moe_set_experts_gguf(moe_ctx* c, int layer, const moe_gg_experts* gg
   MoeLayer* L = layer_of(c, layer);
   if (!L || !gg || !gg->gate || !gg->up || !gg->down) return MOE_E_INVALID;
   if (!moe_gg_types_supported(gg->tgu, gg->tdn, c->cfg.d, c->cfg.mid)) return MOE_E_UNSUPPORTED;
-  L->c_routed = 0.f;
+  L->c_routed = moe_cmag{0.f, 0.f};
   {  // constant of the f16 range guard of the grouped GEMMs
     const moe_config& g = c->cfg;
     moe_wview gv{0, gg->gate, (uint64_t)g.experts * g.mid, (uint64_t)g.d, 0};
@@ -439,7 +439,7 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
         (rc = pexp_register(c, layer, 2 * cf.experts + 1, nullptr, nullptr, 1)))
       return rc;
   }
-  L->c_shared = 0.f;
+  L->c_shared = moe_cmag{0.f, 0.f};
   {
     const int t = dense ? dense : sh_gguf_type;
     int rc = magnitude_constant(c, t, t, g, (uint64_t)cf.mid, u, 0, dn, 1, &L->c_shared);
@@ -457,14 +457,15 @@ MOE_API int moe_set_shared(moe_ctx* c, int layer, const moe_wview* g, const moe_
 
 // Typical |silu(g)*u| (times the growth through the down projection, if that is > 1) for
 // activations of unit mean square: sigma_gate * sigma_up * max(1, sigma_down), sigma^2 = mean
-// squared row norm over two sampled rows, maximum over up to 16 evenly spaced experts.  Expert e's
+// squared row norm over two sampled rows, maximum over up to 16 evenly spaced experts (out->hi); and the smaller of
+// the two magnitudes, sigma_gate * sigma_up * min(1, sigma_down), minimum over those experts (out->lo).  Expert e's
 // gate rows start at row e*gate_stride of `gate`, its up rows at e*gate_stride + up_first of `up`
 // (the same fused tensor for hgn, a tensor of its own for GGUF), its down rows at e*down->rows/n.
 // Set-up work: dequantises 6 rows per sampled expert on the device and reads them back.
 // tgu / tdn: ggml block types of raw GGUF rows (gate and up; down), a dense code of dense.h, or 0 = q4cp views.
 static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gate, uint64_t gate_stride,
                               const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
-                              float* out) {
+                              moe_cmag* out) {
   const int ns = n_experts < 16 ? n_experts : 16;
   const uint64_t d = gate->cols, mid = down->cols, drows = down->rows / (uint64_t)n_experts;
   const uint64_t pitch = d > mid ? d : mid;
@@ -487,7 +488,7 @@ static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gat
   }
   std::vector<float> h((size_t)ns * 6 * pitch);
   MOE_HIP(hipMemcpy(h.data(), c->sample, h.size() * 4, hipMemcpyDeviceToHost));
-  double best = 0.0;
+  double best = 0.0, least = 1e300;
   for (int i = 0; i < ns; i++) {
     double n2[6];
     for (int r = 0; r < 6; r++) {
@@ -501,8 +502,12 @@ static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gat
                  sd = std::sqrt(0.5 * (n2[4] + n2[5]));
     const double cst = sg * su * (sd > 1.0 ? sd : 1.0);
     if (cst > best) best = cst;
+    // the smaller of the two magnitudes (hid, pairs), smallest over the sampled experts: what can underflow
+    const double low = sg * su * (sd < 1.0 ? sd : 1.0);
+    if (low < least) least = low;
   }
-  *out = (float)best;
+  out->hi = (float)best;
+  out->lo = least < 1e300 ? (float)least : 0.f;
   return MOE_OK;
 }
 
@@ -1137,7 +1142,7 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
     if (ee != hipSuccess) return (int)ee;
     rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
                            L.has_shared ? sh_first : -1, y, P, g.d, g.topk,
-                           v2 ? moe_hscale{L.has_shared ? c->xms : nullptr, 0.f, L.c_shared} : hs, st, c->hc,
+                           v2 ? moe_hscale{L.has_shared ? c->xms : nullptr, moe_cmag{0.f, 0.f}, L.c_shared} : hs, st, c->hc,
                            v2 ? L.v2_svh_dn : nullptr);
     prof_mark(c, MOE_PROF_REDUCE, st);
     return rc;

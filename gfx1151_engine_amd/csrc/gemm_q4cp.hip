@@ -163,7 +163,7 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
                                           const float* __restrict__ xms,
-                                          float cmag, const moe_comb& cmb, bool shared, int pexp = 0, int npass = 1) {
+                                          moe_cmag cmag, const moe_comb& cmb, bool shared, int pexp = 0, int npass = 1) {
   // npass > 1 (down launches with f16 results): the block walks npass neighbouring column blocks of its pair tile.  The
   // K stages of all passes form one pipeline -- the first stages of the next column block are requested while the
   // current one's last stages run, so only the first pass pays for the trip to memory -- and the epilogue of a pass
@@ -922,7 +922,7 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
     cb_b_up = u0;
   }
 
-  const float cmag = shared ? hs.c_shared : hs.c_routed;
+  const moe_cmag cmag = shared ? hs.c_shared : hs.c_routed;
   __syncthreads();  // cbs
   const int mfn = (tile.count + 31) >> 5;
 #define GEMM_ARGS smem, L, e, tile, nb, x, out, M, K, cb_a, cb_b, cb_a_up, cb_b_up, ri, hs.xms, cmag, cmb, shared

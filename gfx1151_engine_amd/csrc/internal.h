@@ -6,7 +6,7 @@
 // (routed experts, shared expert); xms == nullptr switches it off (scale 1).
 struct moe_hscale {
   const float* xms;
-  float c_routed, c_shared;
+  moe_cmag c_routed, c_shared;
 };
 
 // Fused weighted combine of the down launch (f32 results): rows are added into y[tokidx[pair]] with the

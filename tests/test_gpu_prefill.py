@@ -183,6 +183,26 @@ def test_batch_layer_vs_oracle(oracle, d, mid, E, k, T, skew):
     m.close()
 
 
+@pytest.mark.parametrize("cb,sstd", [("universal", 0.002), ("zp8", 0.0003), ("universal", 0.0005)])
+def test_batch_layer_with_very_small_weights(oracle, cb, sstd):
+    """Weights several to thirty times smaller than the benchmark's: the down-projection pair rows (about 3e-6 and
+    below at unit activations) would sit in f16's subnormal range; the range guard scales such rows up by a power of
+    two on their way through f16 and the combine takes it out again."""
+    rng = np.random.default_rng(1039)
+    d, mid, E, k, T = 256, 384, 32, 4, 108
+    hl = HostLayer(rng, d, mid, E, k, codebook=S.UNIVERSAL_CODEBOOK if cb == "universal" else None, scale_std=sstd,
+                   shared=(cb == "zp8"), bias=S.zipf_bias(rng, E, 1.1, 1.0))
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    ids, ws = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    err = max_abs_rel(y, yo)
+    assert err <= TOL_LAYER, err
+    m.close()
+
+
 @pytest.mark.parametrize("kind", ["affine", "table", "mixed"])
 @pytest.mark.parametrize("T", [70, 20])
 def test_shared_expert_with_a_codebook_per_tensor(oracle, kind, T):
