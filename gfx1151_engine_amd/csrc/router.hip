@@ -373,7 +373,8 @@ __global__ void __launch_bounds__(256) k_router_mid(const void* __restrict__ W, 
   }
   // the wave's row as scalar values: the bf16 / f32 choice is then a scalar branch
   const int row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(wv);
-  const bool live = row < nrows, extra = row == E;
+  // (without a gate vector row E is padding like every row past it: it must not take Wx, a null pointer then)
+  const bool live = row < nrows, extra = Wx != nullptr && row == E;
   const void* Wr = extra ? Wx : W;
   const uint64_t base = (extra || !live) ? 0 : (uint64_t)row * d;  // rows past the matrix read row 0, never stored
   const bool bf = extra ? wx_bf16 : BF16;

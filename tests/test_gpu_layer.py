@@ -133,6 +133,24 @@ def test_small_batch_sizes_and_router_dtypes(oracle, fmt, T, rdt):
     assert max_abs_rel(y, yo) <= tol_small(fmt), max_abs_rel(y, yo)
 
 
+@pytest.mark.parametrize("T", [3, 6, 12, 21, 30])
+@pytest.mark.parametrize("rdt", ["f32", "bf16"])
+def test_small_batch_router_without_gate_vector_and_ragged_rows(oracle, T, rdt):
+    """A layer without a shared expert (no gate vector beside the router matrix) whose expert count is not a multiple
+    of the router launch's rows per block, at a width where 5..24 tokens take the row-per-wave launch (d not a
+    multiple of 256): the padding rows of the last block read the router matrix, never the absent gate vector."""
+    rng = np.random.default_rng(3300 + T + (rdt == "bf16"))
+    d, mid, E, k = 320, 256, 33, 4
+    hl = HostLayer(rng, d, mid, E, k, router_dtype=rdt, shared=False,
+                   bias=rng.standard_normal(E).astype(np.float32) * 0.1)
+    x = rng.standard_normal((T, d), dtype=np.float32) * 3
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    y, ids, ws = run_layer(hl, x)
+    assert (ids[:, :k] == io[:, :k]).all(), "router ids must be bit-exact"
+    assert np.abs(ws[:, :k] - wo[:, :k]).max() <= 1e-6
+    assert max_abs_rel(y, yo) <= TOL_INT_Q4CP, max_abs_rel(y, yo)
+
+
 @pytest.mark.parametrize("fmt,T", [("q4cp", 1), ("q4cp", 3), ("q4cp", 5), ("q4cp", 6), ("q4cp", 9), ("q4cp", 32),
                                    ("q4k", 1), ("q4k", 9)])
 def test_int_decode_switch(oracle, fmt, T):
