@@ -46,6 +46,8 @@ static int pexp_register(moe_ctx* c, int layer, int slot0, const moe_wview* a, c
 static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gate, uint64_t gate_stride,
                               const moe_wview* up, uint64_t up_first, const moe_wview* down, int n_experts,
                               moe_cmag* out);
+static int magnitude_constant_i4r(moe_ctx* c, const moe_wview* gu, const moe_wview* dn, const float* su,
+                                  const float* svh_gu, const float* suh_dn, int n_experts, moe_cmag* out);
 
 struct moe_ctx {
   moe_config cfg;
@@ -371,7 +373,11 @@ MOE_API int moe_set_experts_i4r(moe_ctx* c, int layer, const moe_wview* gu, cons
   L->gate_up = *gu;
   L->down = *dn;
   L->v2_su = su; L->v2_svh_gu = svh_gu; L->v2_suh_dn = suh_dn; L->v2_svh_dn = svh_dn;
-  L->c_routed = moe_cmag{0.f, 0.f};  // (no f16 range guard on these launches: the reference's have none either)
+  L->c_routed = moe_cmag{0.f, 0.f};
+  if (c->v2_x16) {  // (the batch path's f16 range guard; the small-batch kernels keep f32 between the projections)
+    const int rm = magnitude_constant_i4r(c, gu, dn, su, svh_gu, suh_dn, g.experts, &L->c_routed);
+    if (rm) return rm;
+  }
   L->experts_affine = true;
   L->has_i4r = true;
   L->has_q4cp = false;
@@ -508,6 +514,61 @@ static int magnitude_constant(moe_ctx* c, int tgu, int tdn, const moe_wview* gat
   }
   out->hi = (float)best;
   out->lo = least < 1e300 ? (float)least : 0.f;
+  return MOE_OK;
+}
+
+// The same two magnitudes for hgn v2 rotated experts, as the batch path's f16 buffers see them: hid in the rotated
+// domain of down_proj, ~ sigma_gate * sigma_up * rms(suh_dn) per unit mean square of x, and the pairs, that times the
+// row norm of the stored down matrix.  The block Hadamard rotations are orthogonal, so the mean squared row norm of
+// W = diag(svh) H G H diag(suh) / 128 is that of the stored G times the mean squares of the two vectors (to the
+// accuracy a guard with factor-of-many margins needs).  Set-up work like magnitude_constant.
+static int magnitude_constant_i4r(moe_ctx* c, const moe_wview* gu, const moe_wview* dn, const float* su,
+                                  const float* svh_gu, const float* suh_dn, int n_experts, moe_cmag* out) {
+  const int ns = n_experts < 16 ? n_experts : 16;
+  const uint64_t d = gu->cols, mid = dn->cols;
+  const uint64_t pitch = d > mid ? d : mid;
+  int rc;
+  for (int i = 0; i < ns; i++) {
+    const uint64_t e = (uint64_t)i * n_experts / ns;
+    float* base = c->sample + (size_t)i * 6 * pitch;
+    const uint64_t g0 = e * 2 * mid, u0 = g0 + mid, d0 = e * d;
+    const uint64_t rows[6] = {g0, g0 + mid / 2, u0, u0 + mid / 2, d0, d0 + d / 2};
+    for (int r = 0; r < 6; r++) {
+      const moe_wview* w = r < 4 ? gu : dn;
+      if ((rc = moe_i4r_dequant_rows(w->data, w->rows, w->cols, rows[r], 1, base + (size_t)r * pitch, nullptr))) return rc;
+    }
+  }
+  std::vector<float> h((size_t)ns * 6 * pitch), vsu(d), vgu(2 * mid), vdn(mid);
+  MOE_HIP(hipMemcpy(h.data(), c->sample, h.size() * 4, hipMemcpyDeviceToHost));
+  MOE_HIP(hipMemcpy(vsu.data(), su, d * 4, hipMemcpyDeviceToHost));
+  MOE_HIP(hipMemcpy(vgu.data(), svh_gu, 2 * mid * 4, hipMemcpyDeviceToHost));
+  MOE_HIP(hipMemcpy(vdn.data(), suh_dn, mid * 4, hipMemcpyDeviceToHost));
+  auto rms = [](const float* v, uint64_t n) {
+    double s = 0.0;
+    for (uint64_t j = 0; j < n; j++) s += (double)v[j] * v[j];
+    return std::sqrt(s / (double)n);
+  };
+  const double r_su = rms(vsu.data(), d), r_g = rms(vgu.data(), mid), r_u = rms(vgu.data() + mid, mid), r_dn = rms(vdn.data(), mid);
+  double best = 0.0, least = 1e300;
+  for (int i = 0; i < ns; i++) {
+    double n2[6];
+    for (int r = 0; r < 6; r++) {
+      const float* v = h.data() + ((size_t)i * 6 + r) * pitch;
+      const uint64_t n = r < 4 ? d : mid;
+      double s = 0.0;
+      for (uint64_t j = 0; j < n; j++) s += (double)v[j] * v[j];
+      n2[r] = s;
+    }
+    const double sg = std::sqrt(0.5 * (n2[0] + n2[1])) * r_su * r_g, sup = std::sqrt(0.5 * (n2[2] + n2[3])) * r_su * r_u,
+                 sd = std::sqrt(0.5 * (n2[4] + n2[5]));
+    const double hid = sg * sup * r_dn;
+    const double cst = hid * (sd > 1.0 ? sd : 1.0), low = hid * (sd < 1.0 ? sd : 1.0);
+    if (cst > best) best = cst;
+    if (low < least) least = low;
+  }
+  if (!(best < 1e30)) best = 0.0;  // (non-finite vectors: no guard rather than a factor of zero)
+  out->hi = (float)best;
+  out->lo = least < 1e300 && best > 0.0 ? (float)least : 0.f;
   return MOE_OK;
 }
 
@@ -1037,7 +1098,7 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
       const int e = moe_launch_gemm_q4cp(false, &gu, nullptr, g.experts, c->v2_x16, c->tokidx, tl, ntl, mt, c->v2_z16,
                                          2 * g.mid, g.d, true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
       return e || dry ? e : moe_launch_i4r_mid(c->v2_z16, true, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu, L.v2_suh_dn,
-                                        1, c->hid16, (uint64_t)g.mid, 1, 1, nullptr, nullptr, s2);
+                                        1, c->hid16, (uint64_t)g.mid, 1, 1, nullptr, nullptr, s2, c->xms, L.c_routed, c->tokidx);
     }
     if (v2)  // the shared expert's own tile list (q4cp, not rotated; every tile's expert index is >= n_experts)
       return moe_launch_gemm_q4cp(true, &sgu, &sgu, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d, true,
@@ -1110,7 +1171,7 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
     MOE_HIP(hipStreamWaitEvent(c->side, c->ev_fork, 0));
     int rs = MOE_OK;
     if (v2) rs = moe_launch_v2_rot(x, (uint64_t)g.d, P, g.d, L.v2_su, nullptr, 1, c->v2_x16, (uint64_t)g.d, nullptr, 0, nullptr, nullptr, c->side);
-    if (!rs && (!v2 || L.has_shared))
+    if (!rs)
       rs = c->x16_ext ? moe_launch_meansq_f16(xh, P, g.d, c->xms, c->side)
                       : moe_launch_f16_rows_meansq(x, c->x16, P, g.d, xl, c->xms, c->side);
     hipError_t ee = hipEventRecord(c->ev_x16, c->side);
@@ -1142,7 +1203,7 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
     if (ee != hipSuccess) return (int)ee;
     rc = moe_launch_reduce(c->pairs16, true, c->pairids, c->pw, nullptr, L.has_shared ? c->sh_logit : nullptr,
                            L.has_shared ? sh_first : -1, y, P, g.d, g.topk,
-                           v2 ? moe_hscale{L.has_shared ? c->xms : nullptr, moe_cmag{0.f, 0.f}, L.c_shared} : hs, st, c->hc,
+                           hs, st, c->hc,
                            v2 ? L.v2_svh_dn : nullptr);
     prof_mark(c, MOE_PROF_REDUCE, st);
     return rc;

@@ -104,11 +104,15 @@ __global__ void __launch_bounds__(256) k_v2_rot(const float* x, uint64_t xs, voi
 // row (s / k) * row_slots + s % k (the decode path keeps a token's slots next to its shared-expert slot).
 // MODE 1 (batches: the result is rounded to f16) takes the hardware's exp2 / reciprocal approximations (1 ulp) in
 // SwiGLU, as the grouped GEMM's fused epilogue does; the other modes the exact expf and division.
+// xms (MODE 1, may be null): the f16 range guard of the batch path -- slot s belongs to token tokidx[s], whose row is
+// multiplied by moe_hid_scale(C, xms[token]) in front of the rotation (a power of two; the combine divides it out).
 template <class TG, int MODE>
 __global__ void __launch_bounds__(256) k_i4r_mid(const TG* __restrict__ z, uint64_t zs, void* out, uint64_t os,
                                                  const float* __restrict__ svh_gu, const float* __restrict__ suh_dn,
                                                  int mid, int nslots, int k, int row_slots,
-                                                 uint32_t* __restrict__ planes, float2* __restrict__ meta) {
+                                                 uint32_t* __restrict__ planes, float2* __restrict__ meta,
+                                                 const float* __restrict__ xms, moe_cmag C,
+                                                 const int* __restrict__ tokidx) {
   const int lane = threadIdx.x & 63;
   const int nb = mid >> 7;
   const int64_t grp = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
@@ -124,6 +128,11 @@ __global__ void __launch_bounds__(256) k_i4r_mid(const TG* __restrict__ z, uint6
     ld8(svh_gu + c, fg);
     ld8(svh_gu + mid + c, fu);
     ld8(suh_dn + c, sd);
+    if (MODE == 1 && xms) {
+      const float f = moe_hid_scale(C, xms[tokidx[slot]]);
+#pragma unroll
+      for (int i = 0; i < 8; i++) sd[i] *= f;
+    }
   }
   moe_fwht128_r8(g, lane);
   moe_fwht128_r8(u, lane);
@@ -210,7 +219,8 @@ int moe_launch_v2_rot(const float* x, uint64_t xs, int P, int n, const float* pr
 // z: [nslots][zs] f32 or f16; output row of slot s: (s / k) * row_slots + s % k (k = row_slots = 1: row s)
 int moe_launch_i4r_mid(const void* z, bool z_f16, uint64_t zs, int nslots, int mid, const float* svh_gu,
                        const float* suh_dn, int mode, void* out, uint64_t os, int k, int row_slots, uint32_t* planes,
-                       float2* meta, hipStream_t st) {
+                       float2* meta, hipStream_t st, const float* xms, moe_cmag C, const int* tokidx) {
+  if (xms && (mode != 1 || !tokidx)) return MOE_E_INVALID;
   if (!z || !svh_gu || !suh_dn || nslots < 0 || mode < 0 || mode > 2 || k < 1 || row_slots < k) return MOE_E_INVALID;
   if (mode == 2 ? (!planes || !meta) : !out) return MOE_E_INVALID;
   if (mid < 128 || mid % 128 || 2 * mid > 2048) return MOE_E_UNSUPPORTED;
@@ -221,7 +231,8 @@ int moe_launch_i4r_mid(const void* z, bool z_f16, uint64_t zs, int nslots, int m
   const int64_t threads = (int64_t)nslots * (mid / 128) * 16;
   const unsigned grid = (unsigned)((threads + 255) / 256);
 #define MID_GO(TG, M) \
-  k_i4r_mid<TG, M><<<grid, 256, 0, st>>>((const TG*)z, zs, out, os, svh_gu, suh_dn, mid, nslots, k, row_slots, planes, meta)
+  k_i4r_mid<TG, M><<<grid, 256, 0, st>>>((const TG*)z, zs, out, os, svh_gu, suh_dn, mid, nslots, k, row_slots, planes, meta, \
+                                         xms, C, tokidx)
   if (z_f16) {
     if (mode == 0) MID_GO(__half, 0); else if (mode == 1) MID_GO(__half, 1); else MID_GO(__half, 2);
   } else {

@@ -195,7 +195,8 @@ int moe_launch_v2_rot(const float* x, uint64_t xs, int P, int n, const float* pr
                       uint64_t ys, const float* add, uint64_t adds, uint32_t* planes, float2* meta, hipStream_t st);
 int moe_launch_i4r_mid(const void* z, bool z_f16, uint64_t zs, int nslots, int mid, const float* svh_gu,
                        const float* suh_dn, int mode, void* out, uint64_t os, int k, int row_slots, uint32_t* planes,
-                       float2* meta, hipStream_t st);
+                       float2* meta, hipStream_t st, const float* xms = nullptr, moe_cmag C = moe_cmag{0.f, 0.f},
+                       const int* tokidx = nullptr);
 // general GEMV kernels for any supported mix of ggml block types (gguf_types.hip)
 int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up, int tsh, const uint8_t* sh_w,
                        const uint8_t* sh_w_up, int n_experts, const __half* x16, const int* tokidx,

@@ -203,6 +203,26 @@ def test_batch_layer_with_very_small_weights(oracle, cb, sstd):
     m.close()
 
 
+@pytest.mark.parametrize("sstd,xs,shared", [(0.0005, 0.3, True), (0.0005, 0.3, False), (0.3, 3.0, True), (0.002, 1.0, False)])
+def test_batch_layer_of_rotated_experts_with_weights_far_off_the_usual_scale(oracle, sstd, xs, shared):
+    """hgn v2 rotated experts twenty times smaller / thirty times larger than usual: the rows between the two
+    projections (rotated hid, pair rows) would leave f16's normal range on either side; the range guard applies to
+    this path as well (a power of two per token in the slot-wise middle, divided out in the combine)."""
+    rng = np.random.default_rng(5032 + int(sstd * 1e4))
+    d, mid, E, k, T = 256, 512, 32, 2, 172
+    hl = HostLayer(rng, d, mid, E, k, fmt="i4r", scale_std=sstd, shared=shared, bias=S.zipf_bias(rng, E, 1.1, 1.0))
+    x = rng.standard_normal((T, d), dtype=np.float32) * xs
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    ids, ws = m.last_routing(T)
+    assert (ids.cpu().numpy()[:, :k] == io[:, :k]).all()
+    assert np.isfinite(y).all()
+    err = max_abs_rel(y, yo)
+    assert err <= TOL_LAYER, err
+    m.close()
+
+
 @pytest.mark.parametrize("kind", ["affine", "table", "mixed"])
 @pytest.mark.parametrize("T", [70, 20])
 def test_shared_expert_with_a_codebook_per_tensor(oracle, kind, T):
