@@ -226,6 +226,7 @@ OPT_ROUTER_CANDIDATES = 6
 OPT_UNIQUE_GGUF = 7
 OPT_GU_TOPK_MAX_TOKENS = 8
 OPT_F32_DECODE_MAX_TOKENS = 9
+OPT_V2_FUSED_MIDDLE = 10
 
 
 def lut_q4cp_view(blob, rows, cols, e_rows, up_off):

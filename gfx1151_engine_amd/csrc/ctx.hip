@@ -110,6 +110,7 @@ struct moe_ctx {
   const moe_hc* hc = nullptr;  // set for the duration of moe_forward_hc: the combine writes into the HC state
   const __half* x16_ext = nullptr;  // set for the duration of moe_forward_x16: the caller's f16 copy of x
   bool shared_aside = true;
+  bool v2_fused_mid = true;   // hgn v2 batches: the slot-wise middle in the gate/up launch's epilogue
   // batch router through candidate selection (exact ids at a fraction of the fp64 work); its scratch
   bool router_cand = true;
   void* rc_scratch = nullptr;
@@ -591,6 +592,7 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
     case MOE_OPT_SHARED_ASIDE: c->shared_aside = value != 0; return MOE_OK;
     case MOE_OPT_ROUTER_CANDIDATES: c->router_cand = value != 0; return MOE_OK;
     case MOE_OPT_UNIQUE_GGUF: c->uq_gguf = value != 0; return MOE_OK;
+    case MOE_OPT_V2_FUSED_MIDDLE: c->v2_fused_mid = value != 0; return MOE_OK;
     case MOE_OPT_F32_DECODE_MAX_TOKENS:
       if (value < 0 || value > c->small_max) return MOE_E_INVALID;
       c->lut_max = value;
@@ -1094,7 +1096,17 @@ static int forward_batch_impl(moe_ctx* c, MoeLayer& L, const float* x, int P, fl
       return moe_launch_gemm_gg(true, L.gg.tgu, L.gg.gate, L.gg.up, L.sh_gguf_type, with_sh ? L.sh_gate.data : nullptr,
                                 with_sh ? L.sh_up.data : nullptr, g.experts, xh, c->tokidx, tl, ntl, mt, c->hid16, g.mid,
                                 g.d, hs, s2, xl);
-    if (v2 && !with_sh) {  // the routed experts' tiles: plain rows of the fused tensor, then the slot-wise middle
+    if (v2 && !with_sh) {
+      // the routed experts' tiles: gate rows and their up rows in one block, the slot-wise middle (rotation back,
+      // SwiGLU, rotation for down_proj) in the launch's epilogue
+      if (c->v2_fused_mid) {
+        moe_lutw gf = gu;
+        gf.up_off = g.mid;
+        const moe_rotv rv{L.v2_svh_gu, L.v2_suh_dn};
+        return moe_launch_gemm_q4cp(true, &gf, nullptr, g.experts, c->v2_x16, c->tokidx, tl, ntl, mt, c->hid16, g.mid, g.d,
+                                    true, false, hs, s2, nullptr, nullptr, 2, false, false, nullptr, nullptr, &rv);
+      }
+      // (the earlier form: plain rows of the fused tensor as f16 sums, then the middle as a launch of its own)
       const int e = moe_launch_gemm_q4cp(false, &gu, nullptr, g.experts, c->v2_x16, c->tokidx, tl, ntl, mt, c->v2_z16,
                                          2 * g.mid, g.d, true, false, moe_hscale{nullptr, 0.f, 0.f}, s2, nullptr, nullptr, 2);
       return e || dry ? e : moe_launch_i4r_mid(c->v2_z16, true, (uint64_t)2 * g.mid, P * g.topk, g.mid, L.v2_svh_gu, L.v2_suh_dn,

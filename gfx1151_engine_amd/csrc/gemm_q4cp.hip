@@ -35,6 +35,7 @@
 // src/gpu/parts/27_kernels_moe_lut.inc:23-29): the four stages between two scale refreshes span exactly two scales,
 // fetched as one 4-byte load per row.
 #include "common.h"
+#include "hv2.h"
 #include "internal.h"
 
 namespace {
@@ -158,12 +159,15 @@ __device__ __forceinline__ void g2l4(const void* g, uint8_t* lds_base) {
 // product is exact inside the FMA, one rounding).  P is chosen when the weights are registered, from the expert's
 // largest scale, so that the scaled slope stays below 2^15 (an f16 can hold it); the accumulators carry the factor
 // 2^P and the epilogue takes it out (exact).  v_pk_fma_f16 takes denormal operands at full rate on gfx950.
-template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS, bool Q5, bool NAT = false, bool DN = false>
+constexpr bool NH_OK = NF == 2;
+template <bool UP, bool F16OUT, int MF, bool AFFINE, bool Q4K, int GS, bool Q5, bool NAT = false, bool DN = false, bool ROT = false>
 __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e, const moe_tile tile, int nb,
                                           const __half* __restrict__ x, void* __restrict__ out, int M,
                                           int K, float cb_a, float cb_b, float cb_a_up, float cb_b_up, int ri,
                                           const float* __restrict__ xms,
-                                          moe_cmag cmag, const moe_comb& cmb, bool shared, int pexp = 0, int npass = 1) {
+                                          moe_cmag cmag, const moe_comb& cmb, bool shared, int pexp = 0, int npass = 1,
+                                          moe_rotv rot = moe_rotv{nullptr, nullptr}) {
+  static_assert(!ROT || (UP && F16OUT && GS == 2 && AFFINE && !DN && HALF == 128 && NH_OK), "rotated experts: gate/up rows of one 128-block per block");
   // npass > 1 (down launches with f16 results): the block walks npass neighbouring column blocks of its pair tile.  The
   // K stages of all passes form one pipeline -- the first stages of the next column block are requested while the
   // current one's last stages run, so only the first pass pays for the trip to memory -- and the epilogue of a pass
@@ -696,7 +700,64 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   constexpr int NC = UP ? 32 * NH : 32 * NF;  // output columns of this wave
   auto epilogue = [&](int nb, int cbuf) {     // nb: the column block that the accumulators hold
   const int colbase = UP ? nb * HALF + NC * wv : nb * WROWS + NC * wv;
-  if constexpr (UP) {
+  if constexpr (ROT) {
+    // hgn v2 rotated experts: the block holds the raw sums of one 128-block of gate columns and of the matching up
+    // columns for its pairs, which is what the slot-wise middle works on -- rot_out, SwiGLU, rot_in of the block
+    // (hgn_v2.hip, k_i4r_mid) -- so it runs here instead of as a launch of its own behind a round trip of the sums
+    // through memory.  The sums cross the waves through LDS as f16 (the rounding that the unfused form's f16 rows
+    // in memory have), then 16 lanes take a pair row each, 8 columns a lane.
+    constexpr int BP = 2 * HALF * 2 + 16;  // [128 gate | 128 up] f16 + padding: rows m and m + 4 on different banks
+    static_assert(BM * BP <= NBUF * (A_BYTES + W_BYTES), "the patch fits the stage buffers");
+    uint8_t* patch = smem;
+#pragma unroll
+    for (int mf = 0; mf < MF; mf++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ml = 8 * (r >> 2) + 4 * h + (r & 3);
+        uint8_t* prow = patch + (32 * mf + ml) * BP + (NC * wv + n) * 2;
+        *(__half*)prow = __float2half(acc[mf][0][r]);
+        *(__half*)(prow + HALF * 2) = __float2half(acc[mf][1][r]);
+      }
+    }
+    __syncthreads();
+    const int j = tid & 15;
+    const int c = nb * HALF + 8 * j;  // this lane's 8 columns of the expert's hid
+    float fg[8], fu[8], sd[8];
+    {
+      const int cc = c < M ? c : 0;
+      const float4* pg = (const float4*)(rot.svh_gu + cc);
+      const float4* pu = (const float4*)(rot.svh_gu + M + cc);
+      const float4* pd = (const float4*)(rot.suh_dn + cc);
+      const float4 a0 = pg[0], a1 = pg[1], b0 = pu[0], b1 = pu[1], d0 = pd[0], d1 = pd[1];
+      fg[0] = a0.x; fg[1] = a0.y; fg[2] = a0.z; fg[3] = a0.w; fg[4] = a1.x; fg[5] = a1.y; fg[6] = a1.z; fg[7] = a1.w;
+      fu[0] = b0.x; fu[1] = b0.y; fu[2] = b0.z; fu[3] = b0.w; fu[4] = b1.x; fu[5] = b1.y; fu[6] = b1.z; fu[7] = b1.w;
+      sd[0] = d0.x; sd[1] = d0.y; sd[2] = d0.z; sd[3] = d0.w; sd[4] = d1.x; sd[5] = d1.y; sd[6] = d1.z; sd[7] = d1.w;
+    }
+#pragma unroll 1
+    for (int m = tid >> 4; m < 32 * MF; m += NT / 16) {
+      const uint4 gq = *(const uint4*)(patch + m * BP + j * 16), uq = *(const uint4*)(patch + m * BP + HALF * 2 + j * 16);
+      const __half2* gh = (const __half2*)&gq;
+      const __half2* uh = (const __half2*)&uq;
+      float g[8], u[8], hv[8];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const float2 a = __half22float2(gh[i]), b = __half22float2(uh[i]);
+        g[2 * i] = a.x; g[2 * i + 1] = a.y; u[2 * i] = b.x; u[2 * i + 1] = b.y;
+      }
+      moe_fwht128_r8(g, lane);
+      moe_fwht128_r8(u, lane);
+      const float rs = rowscale[m];
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const float gv = g[i] * MOE_RS128 * fg[i], uv = u[i] * MOE_RS128 * fu[i];  // (the slot-wise middle's own arithmetic)
+        hv[i] = gv * __builtin_amdgcn_rcpf(1.f + __expf(-gv)) * uv * (sd[i] * rs);
+      }
+      moe_fwht128_r8(hv, lane);
+#pragma unroll
+      for (int i = 0; i < 8; i++) hv[i] *= MOE_RS128;
+      if (m < tile.count && c < M) moe_st8_f16_ilv((__half*)out + (size_t)(tile.first + m) * M + c, hv);
+    }
+  } else if constexpr (UP) {
     // gate/up: a wave holds 32 of the block's HALF hid columns, 64 bytes of a row -- stored per wave, the two halves of
     // a 128-byte line reach memory separately (measured: 2.3 times the payload written).  So the block's waves put
     // their columns into one patch of whole rows and every store instruction writes complete lines.
@@ -833,12 +894,12 @@ __device__ __forceinline__ void gemm_tile(uint8_t* smem, const LutDev& L, int e,
   run(epilogue);
 }
 
-template <bool UP, bool F16OUT, bool Q4K, int GS, bool Q5 = false, bool NAT = false>
+template <bool UP, bool F16OUT, bool Q4K, int GS, bool Q5 = false, bool NAT = false, bool ROT = false>
 __global__ void __launch_bounds__(NT, WPE)
 k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x,
                 const int* __restrict__ tokidx, const moe_tile* __restrict__ tiles,
                 const int* __restrict__ ntiles, void* __restrict__ out, int M, int K, int nblk_n, int split,
-                moe_hscale hs, moe_comb cmb, int npass) {
+                moe_hscale hs, moe_comb cmb, int npass, moe_rotv rot) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* cbs = (float*)(smem + NBUF * (A_BYTES + W_BYTES) + NSB * S_BYTES);
   // XCD-aware order: consecutive workgroup ids go round-robin over the 8 XCDs; give each XCD a
@@ -929,7 +990,8 @@ k_moe_gemm_q4cp(LutDev R, LutDev Sh, int n_experts, const __half* __restrict__ x
 #define GEMM_TAIL 0, npass
 #define GEMM_GO(MF)                                                                                     \
   do {                                                                                                  \
-    if constexpr (NAT) gemm_tile<UP, F16OUT, MF, false, false, 0, false, true>(GEMM_ARGS, GEMM_TAIL);   \
+    if constexpr (ROT) gemm_tile<UP, F16OUT, MF, true, false, GS, false, false, false, true>(GEMM_ARGS, GEMM_TAIL, rot); \
+    else if constexpr (NAT) gemm_tile<UP, F16OUT, MF, false, false, 0, false, true>(GEMM_ARGS, GEMM_TAIL);   \
     else {                                                                                              \
       bool scaled = false;                                                                              \
       if constexpr (!Q4K && GS == 0) {                                                                  \
@@ -970,7 +1032,8 @@ LutDev to_dev(const moe_lutw* p, const float* cb_up, const int8_t* pexp) {
 
 bool lut_ok(const moe_lutw* p, bool pair, int k, bool q4k, int gs = 0) {
   if (gs == 2) {  // one scale per 128 columns, unpadded scale rows; whole 256-column scale windows
-    if (q4k || pair || !p || !p->w || !p->sc || !p->cb || k < 256 || k % 256) return false;
+    if (q4k || !p || !p->w || !p->sc || !p->cb || k < 256 || k % 256) return false;
+    if (pair && (!p->w_up || !p->sc_up || !moe_aligned(p->w_up, 16) || !moe_aligned(p->sc_up, 4))) return false;
     return moe_aligned(p->w, 16) && moe_aligned(p->sc, 4) && p->sstride % 4 == 0 && p->sstride >= k / 128 * 2;
   }
   if (q4k) {  // raw Q4_K rows: only the code pointers are used
@@ -1075,8 +1138,14 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
                          hipStream_t st, const moe_comb* comb, const float* sh_cb_up, int gs, bool q5k, bool nat,
-                         const int8_t* pexp_routed, const int8_t* pexp_sh) {
+                         const int8_t* pexp_routed, const int8_t* pexp_sh, const moe_rotv* rot) {
   if (!x || !tiles || !ntiles || !out || max_tiles < 0) return MOE_E_INVALID;
+  // (the rotated experts' fused form: gate/up rows with one scale per 128 columns, whole 128-blocks of hid, no shared
+  //  expert's tiles in the same launch)
+  if (rot && (!up || gs != 2 || sh || comb || !f16out || m % 128 || !rot->svh_gu || !rot->suh_dn ||
+              !moe_aligned(rot->svh_gu, 16) || !moe_aligned(rot->suh_dn, 16)))
+    return MOE_E_INVALID;
+  if (up && gs == 2 && !rot) return MOE_E_UNSUPPORTED;
   if (nat && (q4k || q5k || gs != 0)) return MOE_E_UNSUPPORTED;  // (natural K order: q4cp planes through pair tables)
   if (q5k && (!q4k || !up || comb)) return MOE_E_UNSUPPORTED;  // (Q5_K: gate/up tensors, the reference checkpoints' use of it)
   // (Q5_K: 32-bit byte offsets into the tensors; the caller vouches for the activation rows, moe_gemm_q5k_fits)
@@ -1084,7 +1153,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
     return MOE_E_UNSUPPORTED;
   if (q5k && sh && sh != routed && !moe_gemm_q5k_fits((uint64_t)sh->e_rows + (uint64_t)sh->up_off + (uint64_t)m, 0, k))
     return MOE_E_UNSUPPORTED;
-  if (gs != 0 && (gs != 2 || up || !f16out || q4k || sh || comb)) return MOE_E_UNSUPPORTED;
+  if (gs != 0 && (gs != 2 || (up && !rot) || !f16out || q4k || sh || comb)) return MOE_E_UNSUPPORTED;
   moe_comb cmb{};
   if (comb) {  // fused combine: down launch with f32 results, out = the (zeroed) token rows
     if (up || f16out || !comb->tokidx || !comb->pw || (sh && !comb->sg) || comb->y != out) return MOE_E_INVALID;
@@ -1121,7 +1190,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
       moe_dev_done(attr_once, dev_now);                                                                          \
     }                                                                                                            \
     k_moe_gemm_q4cp<UPK, F16, Q, G><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out, \
-                                                                  m, k, nblk_n, split, hs, cmb, npass);          \
+                                                                  m, k, nblk_n, split, hs, cmb, npass, moe_rotv{nullptr, nullptr}); \
   } while (0)
 #define GEMM_LAUNCH_NAT(UPK, F16)                                                                                \
   do {                                                                                                           \
@@ -1133,7 +1202,7 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
       moe_dev_done(attr_once, dev_now);                                                                          \
     }                                                                                                            \
     k_moe_gemm_q4cp<UPK, F16, false, 0, false, true><<<grid, NT, SMEM_BYTES + PT_BYTES, st>>>(                    \
-        R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, split, hs, cmb, npass);                    \
+        R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, split, hs, cmb, npass, moe_rotv{nullptr, nullptr}); \
   } while (0)
   if (nat) {
     if (up) GEMM_LAUNCH_NAT(true, true);
@@ -1149,7 +1218,17 @@ int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, in
       moe_dev_done(attr5, dev_now);
     }
     k_moe_gemm_q4cp<true, true, true, 0, true><<<grid, NT, SMEM_BYTES, st>>>(R, S, n_experts, x, tokidx, tiles, ntiles, out,
-                                                                             m, k, nblk_n, split, hs, cmb, npass);
+                                                                             m, k, nblk_n, split, hs, cmb, npass, moe_rotv{nullptr, nullptr});
+  } else if (gs == 2 && up) {
+    static moe_dev_once attr_rot;
+    int dev_now;
+    if (moe_dev_pending(attr_rot, &dev_now)) {
+      MOE_HIP(hipFuncSetAttribute((const void*)k_moe_gemm_q4cp<true, true, false, 2, false, false, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)SMEM_BYTES));
+      moe_dev_done(attr_rot, dev_now);
+    }
+    k_moe_gemm_q4cp<true, true, false, 2, false, false, true><<<grid, NT, SMEM_BYTES, st>>>(
+        R, S, n_experts, x, tokidx, tiles, ntiles, out, m, k, nblk_n, split, hs, cmb, npass, *rot);
   } else if (gs == 2) {
     GEMM_LAUNCH(false, true, false, 2);
 #endif

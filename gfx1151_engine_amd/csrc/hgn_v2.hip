@@ -38,14 +38,7 @@ __device__ __forceinline__ void st8(float* p, const float (&v)[8]) {
   ((float4*)p)[0] = make_float4(v[0], v[1], v[2], v[3]);
   ((float4*)p)[1] = make_float4(v[4], v[5], v[6], v[7]);
 }
-// 8 values as f16 in the order the grouped GEMM keeps its activations in: [e0,e4,e1,e5,e2,e6,e3,e7]
-__device__ __forceinline__ void st8_f16_ilv(__half* p, const float (&v)[8]) {
-  const __half2 a = __floats2half2_rn(v[0], v[4]), b = __floats2half2_rn(v[1], v[5]);
-  const __half2 c = __floats2half2_rn(v[2], v[6]), d = __floats2half2_rn(v[3], v[7]);
-  uint4 o;
-  o.x = *(const uint32_t*)&a; o.y = *(const uint32_t*)&b; o.z = *(const uint32_t*)&c; o.w = *(const uint32_t*)&d;
-  *(uint4*)p = o;
-}
+__device__ __forceinline__ void st8_f16_ilv(__half* p, const float (&v)[8]) { moe_st8_f16_ilv(p, v); }
 // y[p][i] = post[i] * H(pre . x[p])[i] / sqrt(128) (+ add[p][i]) per 128 block; pre / post / add optional.
 // P rows of n values (n % 128 == 0), n/8 lanes per row.  MODE 0: f32 rows; 1: f16 rows in the grouped GEMM's order;
 // 2: digit planes of the decode kernels (planes / meta indexed [p][n/32]).  In place (MODE 0, y == x) is fine.

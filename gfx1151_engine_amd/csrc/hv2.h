@@ -49,6 +49,15 @@ __device__ __forceinline__ void moe_fwht128_r8(float (&v)[8], int lane) {
 #undef MOE_FWHT_STEP
 }
 
+// 8 values as f16 in the order the grouped GEMM keeps its activations in: [e0,e4,e1,e5,e2,e6,e3,e7]
+__device__ __forceinline__ void moe_st8_f16_ilv(__half* p, const float (&v)[8]) {
+  const __half2 a = __floats2half2_rn(v[0], v[4]), b = __floats2half2_rn(v[1], v[5]);
+  const __half2 c = __floats2half2_rn(v[2], v[6]), d = __floats2half2_rn(v[3], v[7]);
+  uint4 o;
+  o.x = *(const uint32_t*)&a; o.y = *(const uint32_t*)&b; o.z = *(const uint32_t*)&c; o.w = *(const uint32_t*)&d;
+  *(uint4*)p = o;
+}
+
 __device__ __forceinline__ float moe_quad_xor1(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
 }

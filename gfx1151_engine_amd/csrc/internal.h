@@ -68,12 +68,16 @@ int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const
                         const float* sh_logit, const float* x, const int* ids, const float* ws,
                         float* hid, float* out, int P, int d, int mid, int kpt, int id_stride,
                         hipStream_t st);
+// hgn v2 rotated experts, gate/up launch with the slot-wise middle in its epilogue (gs = 2, up): svh_gu [2 m], suh_dn [m]
+struct moe_rotv {
+  const float *svh_gu, *suh_dn;
+};
 int moe_launch_gemm_q4cp(bool up, const moe_lutw* routed, const moe_lutw* sh, int n_experts,
                          const __half* x, const int* tokidx, const moe_tile* tiles, const int* ntiles,
                          int max_tiles, void* out, int m, int k, bool f16out, bool q4k, moe_hscale hs,
                          hipStream_t st, const moe_comb* comb, const float* sh_cb_up = nullptr, int gs = 0,
                          bool q5k = false, bool nat = false, const int8_t* pexp_routed = nullptr,
-                         const int8_t* pexp_sh = nullptr);
+                         const int8_t* pexp_sh = nullptr, const moe_rotv* rot = nullptr);
 // Scaled dequantisation of the grouped GEMM (affine q4cp codebooks): per expert the power of two P with
 // |cb slope| * (largest scale of the expert) * 2^(24+P) in [2^14, 2^15), or MOE_PEXP_NONE where the form does not apply
 // (a scale that is not finite, a zero slope, rows whose largest scale lies more than 2^5 below the expert's: their

@@ -162,6 +162,28 @@ def test_v2_batch_layer(oracle, d, mid, E, k, T, shared):
     assert max_abs_rel(y, yo) <= TOL_LAYER, max_abs_rel(y, yo)
 
 
+@pytest.mark.parametrize("d,mid,E,k,T", [(256, 256, 6, 2, 77), (768, 512, 8, 4, 333), (3072, 768, 16, 10, 200), (512, 128, 5, 1, 260)])
+def test_v2_batch_middle_in_the_epilogue_equals_the_separate_launch(oracle, d, mid, E, k, T):
+    """MOE_OPT_V2_FUSED_MIDDLE: the gate/up launch with the slot-wise middle in its epilogue (default) against the
+    gate | up sums in memory + the middle as a launch of its own: the same arithmetic in the same order (the sums cross
+    the block's waves as f16, the rounding the rows in memory have), so the layers' outputs are identical."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(8100 + d + T)
+    hl = HostLayer(rng, d, mid, E, k, fmt="i4r", shared=True)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    y1 = m.forward(0, gpu(x)).cpu().numpy()
+    m.set_option(capi.OPT_V2_FUSED_MIDDLE, 0)
+    y0 = m.forward(0, gpu(x)).cpu().numpy()
+    m.set_option(capi.OPT_V2_FUSED_MIDDLE, 1)
+    y2 = m.forward(0, gpu(x)).cpu().numpy()
+    m.close()
+    assert max_abs_rel(y1, yo) <= TOL_LAYER, max_abs_rel(y1, yo)
+    assert (y1 == y0).all(), float(np.abs(y1 - y0).max())
+    assert (y2 == y1).all()
+
+
 def test_v2_layer_hc_writeback(oracle):
     """moe_forward_hc on an hgn v2 layer (the reference's k_v2_reduce_rot_hc, 28_kernels_hgn_v2.inc:189-230): the
     rotated combine written straight into the bf16 HC state, against the oracle's write-back of the oracle's y."""
