@@ -227,6 +227,7 @@ OPT_UNIQUE_GGUF = 7
 OPT_GU_TOPK_MAX_TOKENS = 8
 OPT_F32_DECODE_MAX_TOKENS = 9
 OPT_V2_FUSED_MIDDLE = 10
+PATH_NONE, PATH_SMALL, PATH_BATCH, PATH_WALKED = 0, 1, 2, 3
 
 
 def lut_q4cp_view(blob, rows, cols, e_rows, up_off):
@@ -436,6 +437,10 @@ class Moe:
 
     def set_option(self, option, value):
         check(lib().moe_set_option(self.h, option, value), "moe_set_option")
+
+    def last_path(self):
+        """PATH_SMALL / PATH_BATCH / PATH_WALKED of the last forward call (moe_last_path)."""
+        return int(lib().moe_last_path(self.h))
 
     def profile(self, on=True):
         check(lib().moe_profile_enable(self.h, 1 if on else 0), "moe_profile_enable")

@@ -111,6 +111,7 @@ struct moe_ctx {
   const __half* x16_ext = nullptr;  // set for the duration of moe_forward_x16: the caller's f16 copy of x
   bool shared_aside = true;
   bool v2_fused_mid = true;   // hgn v2 batches: the slot-wise middle in the gate/up launch's epilogue
+  int last_path = MOE_PATH_NONE;  // which path the last successful moe_forward* call took (moe_last_path)
   // batch router through candidate selection (exact ids at a fraction of the fp64 work); its scratch
   bool router_cand = true;
   void* rc_scratch = nullptr;
@@ -1274,9 +1275,11 @@ MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, 
 #endif
     const int rs = forward_small(c, *L, x, P, y, moe_s(st));
     if (rs == MOE_OK && c->skip_stage == 0 && P > c->ran_complete) c->ran_complete = P;
+    if (rs == MOE_OK) c->last_path = MOE_PATH_SMALL;
     return rs;
   }
   const int rc = forward_batch(c, *L, x, P, y, moe_s(st));
+  if (rc == MOE_OK) c->last_path = MOE_PATH_BATCH;
   if (rc != MOE_E_UNSUPPORTED) return rc;
   // formats the grouped GEMM does not cover yet: the in-place path, 32 rows at a time.  Every chunk leaves its
   // router output in the first rows of ids / ws; the walk runs from the last chunk to the first and moves each
@@ -1291,8 +1294,11 @@ MOE_API int moe_forward(moe_ctx* c, int layer, const float* x, int P, float* y, 
       MOE_HIP(hipMemcpyAsync(c->ws + t0 * stride, c->ws, n * stride * 4, hipMemcpyDeviceToDevice, moe_s(st)));
     }
   }
+  c->last_path = MOE_PATH_WALKED;
   return MOE_OK;
 }
+
+MOE_API int moe_last_path(const moe_ctx* c) { return c ? c->last_path : MOE_E_INVALID; }
 
 // GpuModel::moe_b(l, P, try_hcw = true) (src/gpu/parts/40_model.inc:4018,4082-4094): the batch call with the HC
 // write-back fused into the combine.  MOE_E_UNSUPPORTED (nothing enqueued) where the reference returns false:
@@ -1310,6 +1316,7 @@ MOE_API int moe_forward_hc(moe_ctx* c, int layer, const float* x, int P, const f
   c->hc = &hc;
   const int rc = forward_batch(c, *L, x, P, nullptr, moe_s(st));
   c->hc = nullptr;
+  if (rc == MOE_OK) c->last_path = MOE_PATH_BATCH;
   return rc;
 }
 
@@ -1336,5 +1343,6 @@ MOE_API int moe_forward_x16(moe_ctx* c, int layer, const float* x, const void* x
   c->x16_ext = (const __half*)x16;
   const int rc = forward_batch(c, *L, x, P, y, moe_s(st));
   c->x16_ext = nullptr;
+  if (rc == MOE_OK) c->last_path = MOE_PATH_BATCH;
   return rc;
 }

@@ -343,6 +343,13 @@ int moe_profile_read(moe_ctx* ctx, float* ms);
 /* Copy the last call's router output (the reference keeps it in d_topids / d_topw,
  * 40_model.inc:1811) into caller buffers [P][id_stride] (device memory; async on st). */
 int moe_get_routing(moe_ctx* ctx, int P, int* ids_out, float* ws_out, moe_stream_t st);
+/* Which path the last successful moe_forward / moe_forward_hc / moe_forward_x16 call on the context took (no
+ * counterpart in the reference, whose callers pick the path themselves: 40_model.inc:1959-1996 moe / moe_b).
+ * MOE_PATH_SMALL: the in-place kernels for at most 32 tokens; MOE_PATH_BATCH: the grouped GEMM; MOE_PATH_WALKED: a
+ * batch over 32 tokens of a shape or format outside the grouped GEMM, run through the in-place kernels 32 rows at a
+ * time -- correct, and several times slower than the grouped GEMM, which is why a caller may want to know. */
+enum { MOE_PATH_NONE = 0, MOE_PATH_SMALL = 1, MOE_PATH_BATCH = 2, MOE_PATH_WALKED = 3 };
+int moe_last_path(const moe_ctx* ctx);
 
 /* ---- hgn v2 rotated experts: the stages around the projections ---- */
 /* rows [row0, row0 + nrows) of an i4r tensor as f32, bit-exact (tools/moe_lut_test.cu:936-948) */

@@ -203,6 +203,36 @@ def test_batch_layer_with_very_small_weights(oracle, cb, sstd):
     m.close()
 
 
+@pytest.mark.parametrize("fmt,kw,d,mid,want", [
+    ("q4cp", {}, 512, 256, "batch"), ("q4cp", {"codebook": "universal"}, 512, 256, "batch"),
+    ("q4cp", {"shared": False}, 256, 384, "batch"), ("q4k", {}, 512, 256, "batch"),
+    ("q4k", {"gg_types": (13, 8, 8)}, 512, 256, "batch"), ("q4k", {"gg_types": (23, 20, 12)}, 512, 256, "batch"),
+    ("i4r", {}, 512, 256, "batch"), ("i4r", {"shared": False}, 256, 512, "batch"), ("i4r", {"shared_dense": "bf16"}, 512, 256, "batch"),
+    ("q4cp", {"shared_dense": "q8g64"}, 512, 256, "batch"),
+    ("q4cp", {}, 320, 256, "walked"), ("i4r", {}, 384, 384, "walked")])
+def test_which_shapes_take_the_grouped_gemm(oracle, fmt, kw, d, mid, want):
+    """moe_last_path: batches over 32 tokens of every supported format run on the grouped GEMM (a launch plan that
+    declines silently would send them through the in-place kernels 32 rows at a time -- right results, several times
+    the time); shapes outside the GEMM's tiling are walked; at most 32 tokens take the in-place kernels."""
+    from gfx1151_engine_amd import capi
+    rng = np.random.default_rng(77 + d + mid)
+    kw = dict(kw)
+    if kw.get("codebook") == "universal":
+        kw["codebook"] = S.UNIVERSAL_CODEBOOK
+    E, k, T = 8, 2, 70
+    hl = HostLayer(rng, d, mid, E, k, fmt=fmt, **kw)
+    x = rng.standard_normal((T, d), dtype=np.float32)
+    yo, io, wo = oracle.moe_layer(hl.oracle_layer(), x)
+    m, dev = hl.to_gpu(max_tokens=T)
+    assert m.last_path() == capi.PATH_NONE
+    y = m.forward(0, gpu(x)).cpu().numpy()
+    assert m.last_path() == (capi.PATH_BATCH if want == "batch" else capi.PATH_WALKED)
+    assert max_abs_rel(y, yo) <= TOL_LAYER, max_abs_rel(y, yo)
+    m.forward(0, gpu(x[:7]))
+    assert m.last_path() == capi.PATH_SMALL
+    m.close()
+
+
 @pytest.mark.parametrize("sstd,xs,shared", [(0.0005, 0.3, True), (0.0005, 0.3, False), (0.3, 3.0, True), (0.002, 1.0, False)])
 def test_batch_layer_of_rotated_experts_with_weights_far_off_the_usual_scale(oracle, sstd, xs, shared):
     """hgn v2 rotated experts twenty times smaller / thirty times larger than usual: the rows between the two
