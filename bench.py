@@ -164,6 +164,13 @@ def measure(wl, steps, warmup, tokens=0, nlayers_arg=48, cpu=True, opts=(), cpu_
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
+    # the path the timed calls take: batches over 32 tokens on the grouped GEMM (a batch walked through the in-place
+    # kernels 32 rows at a time would return right results and a meaningless figure)
+    step(0)
+    want = capi.PATH_BATCH if T > 32 else capi.PATH_SMALL
+    if m.last_path() != want:
+        raise SystemExit(f"bench.py: workload {kind!r} at {T} tokens took path {m.last_path()}, expected {want} (moe_last_path)")
+    torch.cuda.synchronize()
     # whole-job timing: K steps between two synchronisations, HIP events on the launch stream
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
