@@ -227,6 +227,7 @@ OPT_UNIQUE_GGUF = 7
 OPT_GU_TOPK_MAX_TOKENS = 8
 OPT_F32_DECODE_MAX_TOKENS = 9
 OPT_V2_FUSED_MIDDLE = 10
+OPT_PAIR_TABLES = 11
 PATH_NONE, PATH_SMALL, PATH_BATCH, PATH_WALKED = 0, 1, 2, 3
 
 

@@ -111,6 +111,7 @@ struct moe_ctx {
   const __half* x16_ext = nullptr;  // set for the duration of moe_forward_x16: the caller's f16 copy of x
   bool shared_aside = true;
   bool v2_fused_mid = true;   // hgn v2 batches: the slot-wise middle in the gate/up launch's epilogue
+  bool pair_tables = true;    // table codebooks, 6..32 tokens: look-ups through pair tables
   int last_path = MOE_PATH_NONE;  // which path the last successful moe_forward* call took (moe_last_path)
   // batch router through candidate selection (exact ids at a fraction of the fp64 work); its scratch
   bool router_cand = true;
@@ -594,6 +595,7 @@ MOE_API int moe_set_option(moe_ctx* c, int option, int value) {
     case MOE_OPT_ROUTER_CANDIDATES: c->router_cand = value != 0; return MOE_OK;
     case MOE_OPT_UNIQUE_GGUF: c->uq_gguf = value != 0; return MOE_OK;
     case MOE_OPT_V2_FUSED_MIDDLE: c->v2_fused_mid = value != 0; return MOE_OK;
+    case MOE_OPT_PAIR_TABLES: c->pair_tables = value != 0; return MOE_OK;
     case MOE_OPT_F32_DECODE_MAX_TOKENS:
       if (value < 0 || value > c->small_max) return MOE_E_INVALID;
       c->lut_max = value;
@@ -792,6 +794,10 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
       });
     }
     if (use_lut || use_f32a) {
+      // table codebooks past the few-token sizes: the plain f32 down kernel looks the routed experts' weights up two
+      // at a time in a pair table (the gate/up kernel was measured with one as well: no gain, its LDS traffic per
+      // weight stays what it is)
+      const bool pair_tabs = use_lut && !use_f32a && c->pair_tables && P > c->lut_max;
       if ((rc = stage(MOE_PROF_UP, [&]() -> int {
              return moe_launch_dec_gu_lut(&L.gate_up, shg, shu, x, gu_topk ? c->logits : nullptr, g.experts, c->ids, c->ws,
                                           g.id_stride, g.topk, P, g.d, g.mid, c->hid32, st, &rf, use_f32a);
@@ -802,7 +808,7 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
         //  hidden rows once for all of them and measure faster from about 6 tokens on)
         if (P > c->lut_max)
           return moe_launch_gemv_dn(&L.down, shd, c->sh_logit, nullptr, nullptr, c->hid32, c->ids, c->ws, g.id_stride,
-                                    g.topk, P, g.d, y, (uint64_t)g.d, st);
+                                    g.topk, P, g.d, y, (uint64_t)g.d, st, pair_tabs);
         return moe_launch_dec_dn_lut(&L.down, shd, c->sh_logit, c->hid32, c->ids, c->ws, g.id_stride, g.topk, P, g.d,
                                      g.mid, y, (uint64_t)g.d, st, use_f32a);
       });
@@ -814,7 +820,7 @@ static int forward_small_routed(moe_ctx* c, MoeLayer& L, const float* x, int P, 
       return rc;
     return stage(MOE_PROF_DOWN, [&]() -> int {
       return moe_launch_gemv_dn(&L.down, shd, c->sh_logit, nullptr, nullptr, c->hid32, c->ids, c->ws, g.id_stride,
-                                g.topk, P, g.d, y, (uint64_t)g.d, st);
+                                g.topk, P, g.d, y, (uint64_t)g.d, st, false);
     });
   }
   if (sh && L.sh_gguf_type == 0) return MOE_E_UNSUPPORTED;

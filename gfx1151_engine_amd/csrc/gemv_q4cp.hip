@@ -62,6 +62,41 @@ __device__ __forceinline__ float dot32(const uint4 pk, const float4* xv, const f
   }
   return a0 + a1;
 }
+// Pair tables (table codebooks, batches of more than a few tokens: the launch is bound by vector instructions): a code
+// byte holds two neighbouring weights; a 256-entry table of (cb[b & 15], cb[b >> 4]) gives both with one 8-byte LDS
+// read.  Sixteen copies side by side (entry b, copy c at dword 32 b + 2 c: 32 KB), a lane reads copy lane % 16: the
+// sixteen lanes that an 8-byte read serves together sit on sixteen different bank pairs whatever their bytes are.
+constexpr int PT_DW = 256 * 32;
+typedef float float2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void build_ptab(float* tab, const float* __restrict__ cb) {
+  for (int i = threadIdx.x; i < 256 * 16; i += blockDim.x) {
+    const int b = i >> 4, c = i & 15;
+    *(float2v*)(tab + b * 32 + c * 2) = float2v{cb[b & 15], cb[b >> 4]};
+  }
+}
+__device__ __forceinline__ float dot32_pairs(const uint4 pk, const float4* xv, const float* tab_lane) {
+  const uint32_t w[4] = {pk.x, pk.y, pk.z, pk.w};
+  float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t v = w[i];
+    const float4 x0 = xv[2 * i], x1 = xv[2 * i + 1];
+    const float2v t0 = *(const float2v*)(tab_lane + (v & 0xff) * 32);
+    const float2v t1 = *(const float2v*)(tab_lane + ((v >> 8) & 0xff) * 32);
+    const float2v t2 = *(const float2v*)(tab_lane + ((v >> 16) & 0xff) * 32);
+    const float2v t3 = *(const float2v*)(tab_lane + (v >> 24) * 32);
+    a0 = fmaf(t0.x, x0.x, a0);
+    a1 = fmaf(t0.y, x0.y, a1);
+    a0 = fmaf(t1.x, x0.z, a0);
+    a1 = fmaf(t1.y, x0.w, a1);
+    a0 = fmaf(t2.x, x1.x, a0);
+    a1 = fmaf(t2.y, x1.y, a1);
+    a0 = fmaf(t3.x, x1.z, a0);
+    a1 = fmaf(t3.y, x1.w, a1);
+  }
+  return a0 + a1;
+}
+
 struct GuArgs {
   const uint8_t *codes, *scales;  // routed experts: fused gate_up [E*2*mid][d]
   const float* cb;
@@ -343,14 +378,17 @@ __device__ __forceinline__ float sum32(const float4* xv) {
 // Eight lanes per output row; every slot's partial stays in a register and the weighted sum runs
 // in slot order (= descending router probability), then the shared expert.
 constexpr int DN_ROWS = 32, DN_MAXSLOTS = 17;
-template <bool AFFINE, int NS>
+// PAIR (not with AFFINE): the routed slots' look-ups through the pair table `ptab` (the shared expert's slot, one of
+// eleven and with a codebook of its own, stays on the 16-entry table)
+template <bool AFFINE, int NS, bool PAIR = false>
 __device__ __forceinline__ void dn_rows(const DnArgs& A, const int* eid, const float* wgt, int nslots,
                                         bool has_shared, int d, int mid, int r0, int nrows, CbInfo cr,
                                         CbInfo cs, const float* cbr, const float* cbsh,
-                                        const float4* hs, int tok, float* out) {
+                                        const float4* hs, int tok, float* out, const float* ptab = nullptr) {
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, sub = lane >> 3, l8 = lane & 7;
   const int G = mid / 32;
-  for (int rr = wv * 8 + sub; rr < nrows; rr += 32) {
+  const float* const tab_lane = PAIR ? ptab + 2 * (lane & 15) : nullptr;
+  for (int rr = wv * 8 + sub; rr < nrows; rr += (int)(blockDim.x >> 3)) {
     const int r = r0 + rr;
     float acc[NS];
 #pragma unroll
@@ -370,7 +408,9 @@ __device__ __forceinline__ void dn_rows(const DnArgs& A, const int* eid, const f
           float4 xv[8];
 #pragma unroll
           for (int j = 0; j < 8; j++) xv[j] = hs[((size_t)s * 8 + j) * G + g];
-          float dv = dot32<AFFINE>(pk, xv, cbl);
+          float dv;
+          if (PAIR && !sh) dv = dot32_pairs(pk, xv, tab_lane);
+          else dv = dot32<AFFINE>(pk, xv, cbl);
           if (AFFINE) dv = fmaf(c.a, dv, c.b * sum32(xv));
           a = fmaf(dv, sc, a);
         }
@@ -391,13 +431,15 @@ __device__ __forceinline__ void dn_rows(const DnArgs& A, const int* eid, const f
   }
 }
 
-template <int NS>
-__global__ void __launch_bounds__(256) k_q4cp_gemv_dn(DnArgs A, const float* __restrict__ hid,
+// PAIR: 512 threads and 64 rows per block, the routed experts' pair table behind hid in LDS (for codebooks that are not
+// a*n + b; the launcher picks it for batches past the few-token sizes)
+template <int NS, bool PAIR = false>
+__global__ void __launch_bounds__(PAIR ? 512 : 256) k_q4cp_gemv_dn(DnArgs A, const float* __restrict__ hid,
                                                       const int* __restrict__ ids,
                                                       const float* __restrict__ ws, int id_stride,
                                                       int kpt, int d, int mid, float* __restrict__ out,
                                                       uint64_t out_stride) {
-  extern __shared__ float4 hs[];  // nslots * mid/4 float4
+  extern __shared__ float4 hs[];  // nslots * mid/4 float4 (PAIR: then the pair table)
   __shared__ float cbr[16], cbsh[16];
   __shared__ int eid[DN_MAXSLOTS];
   __shared__ float wgt[DN_MAXSLOTS];
@@ -423,11 +465,16 @@ __global__ void __launch_bounds__(256) k_q4cp_gemv_dn(DnArgs A, const float* __r
   const CbInfo cr = load_cb(A.cb, cbr);
   CbInfo cs = cr;
   if (has_shared) cs = load_cb(A.sh_cb, cbsh);
+  float* const ptab = (float*)(hs + (size_t)nslots * q);
+  if (PAIR) build_ptab(ptab, A.cb);
   __syncthreads();
-  const int r0 = blockIdx.x * DN_ROWS;
-  const int nrows = min(DN_ROWS, d - r0);
+  const int rows_pb = (int)(blockDim.x >> 3);  // 8 lanes per row: 32 rows (256 threads) or 64 (512)
+  const int r0 = blockIdx.x * rows_pb;
+  const int nrows = min(rows_pb, d - r0);
   float* o = out + (size_t)tok * out_stride;
-  if (cr.affine && cs.affine)
+  if (PAIR)
+    dn_rows<false, NS, true>(A, eid, wgt, nslots, has_shared, d, mid, r0, nrows, cr, cs, cbr, cbsh, hs, tok, o, ptab);
+  else if (cr.affine && cs.affine)
     dn_rows<true, NS>(A, eid, wgt, nslots, has_shared, d, mid, r0, nrows, cr, cs, cbr, cbsh, hs, tok, o);
   else
     dn_rows<false, NS>(A, eid, wgt, nslots, has_shared, d, mid, r0, nrows, cr, cs, cbr, cbsh, hs, tok, o);
@@ -481,7 +528,7 @@ int moe_launch_gemv_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_
 int moe_launch_gemv_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,
                        const float* ey, const float* sg, const float* hid, const int* ids,
                        const float* ws, int id_stride, int kpt, int P, int d, float* out,
-                       uint64_t out_stride, hipStream_t st) {
+                       uint64_t out_stride, hipStream_t st, bool pair_tables) {
   int rc = check_q4cp(dn);
   if (rc) return rc;
   const int mid = (int)dn->cols;
@@ -513,6 +560,29 @@ int moe_launch_gemv_dn(const moe_wview* dn, const moe_wview* sh_down, const floa
     MOE_LAUNCH_CHECK();
     return MOE_OK;
   }
+  if (pair_tables) {
+    // (the caller vouches that the routed experts' codebook is a table; 64 rows per block of 512 threads)
+    const size_t ldp = (size_t)nslots * mid * 4 + (size_t)PT_DW * 4;
+    if (ldp > 96 * 1024) return MOE_E_UNSUPPORTED;
+    dim3 gp((d + 63) / 64, P);
+#define DN_PAIR(N)                                                                                                     \
+  do {                                                                                                                 \
+    static moe_dev_once once;                                                                                          \
+    int dev_now;                                                                                                       \
+    if (moe_dev_pending(once, &dev_now)) {                                                                             \
+      MOE_HIP(hipFuncSetAttribute((const void*)k_q4cp_gemv_dn<N, true>, hipFuncAttributeMaxDynamicSharedMemorySize,   \
+                                  96 * 1024));                                                                         \
+      moe_dev_done(once, dev_now);                                                                                     \
+    }                                                                                                                  \
+    k_q4cp_gemv_dn<N, true><<<gp, 512, ldp, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out, out_stride);           \
+  } while (0)
+    if (nslots <= 4) DN_PAIR(4);
+    else if (nslots <= 11) DN_PAIR(11);
+    else DN_PAIR(16);
+#undef DN_PAIR
+    MOE_LAUNCH_CHECK();
+    return MOE_OK;
+  }
   dim3 grid((d + DN_ROWS - 1) / DN_ROWS, P);
   const size_t lds = (size_t)nslots * mid * 4;
   if (nslots <= 4) k_q4cp_gemv_dn<4><<<grid, 256, lds, st>>>(A, hid, ids, ws, id_stride, kpt, d, mid, out, out_stride);
@@ -534,5 +604,5 @@ MOE_API int moe_q4cp_gemv_down_topk(const moe_wview* dn, const float* hid, const
                                     const float* ey, const float* sg, float* out, uint64_t out_stride,
                                     moe_stream_t st) {
   if (!hid || !ids || !ws || !out) return MOE_E_INVALID;
-  return moe_launch_gemv_dn(dn, nullptr, nullptr, ey, sg, hid, ids, ws, id_stride, kpt, P, d, out, out_stride, moe_s(st));
+  return moe_launch_gemv_dn(dn, nullptr, nullptr, ey, sg, hid, ids, ws, id_stride, kpt, P, d, out, out_stride, moe_s(st), false);
 }

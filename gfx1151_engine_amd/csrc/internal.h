@@ -62,7 +62,7 @@ int moe_launch_gemv_gu(const moe_wview* gu, const moe_wview* sh_gate, const moe_
 int moe_launch_gemv_dn(const moe_wview* dn, const moe_wview* sh_down, const float* sh_logit,
                        const float* ey, const float* sg, const float* hid, const int* ids,
                        const float* ws, int id_stride, int kpt, int P, int d, float* out,
-                       uint64_t out_stride, hipStream_t st);
+                       uint64_t out_stride, hipStream_t st, bool pair_tables = false);
 int moe_launch_q4k_gemv(int phase, const uint8_t* gate, const uint8_t* up, const uint8_t* down,
                         const uint8_t* sh_gate, const uint8_t* sh_up, const uint8_t* sh_down,
                         const float* sh_logit, const float* x, const int* ids, const float* ws,

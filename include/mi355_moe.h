@@ -326,10 +326,13 @@ int moe_forward_x16(moe_ctx* ctx, int layer, const float* x, const void* x16, in
  * an expert's gate rows and the matching up rows into one block and runs the slot-wise middle (rotation back, SwiGLU,
  * rotation for down_proj) in its epilogue; 0 = the gate | up sums as f16 rows in memory and the middle as a launch of
  * its own (the reference's moe_lut_up_raw + k_i4r_mid, 40_model.inc:4600-4618). */
+/* MOE_OPT_PAIR_TABLES (default 1): q4cp layers whose codebook is a table (not a*n + b), batches above
+ * MOE_OPT_F32_DECODE_MAX_TOKENS and up to 32 tokens: the f32 kernels look two neighbouring weights up at a time in
+ * 256-entry pair tables (one per code byte); 0 = one look-up per weight in the 16-entry table, as at a few tokens. */
 enum { MOE_OPT_INT_DECODE = 1, MOE_OPT_UNIQUE_MIN_TOKENS = 2, MOE_OPT_FUSED_COMBINE = 3, MOE_OPT_SHARED_ASIDE = 4,
        MOE_OPT_TIMING_SKIP_STAGE = 5, MOE_OPT_ROUTER_CANDIDATES = 6, MOE_OPT_UNIQUE_GGUF = 7,
        MOE_OPT_GU_TOPK_MAX_TOKENS = 8, MOE_OPT_F32_DECODE_MAX_TOKENS = 9,
-       MOE_OPT_V2_FUSED_MIDDLE = 10 };
+       MOE_OPT_V2_FUSED_MIDDLE = 10, MOE_OPT_PAIR_TABLES = 11 };
 int moe_set_option(moe_ctx* ctx, int option, int value);
 /* Per-stage timing of the last moe_forward, the reference's KP("moe:route|up|down|reduce") tags
  * (src/gpu/parts/07_kprof.inc, 40_model.inc:1749-1782).  While enabled moe_forward records HIP
