@@ -750,6 +750,33 @@ __global__ void __launch_bounds__(256, 2) k_moe_gemm_gg(GgGemmW R, GgGemmW Sh, i
     }
   }
   // D[i][j]: j = lane % 32 (weight row), i = 8 * (r / 4) + 4 * (lane / 32) + r % 4 (pair)
+  if constexpr (!UP) {
+    // down launches: a wave's 64 x 64 results are 128 contiguous bytes of each of its 64 output rows.  Stored straight
+    // from the accumulators they leave as 2-byte pieces, 64 bytes per half-wave and instruction; through a patch of the
+    // wave's own in LDS (the operand tiles are dead: every wave is past the loop's last barrier) they leave as 16-byte
+    // pieces, eight lanes to a whole line.  Rows at a pitch of 144 bytes: the two lane halves write rows m and m + 4,
+    // which then lie 16 banks apart.
+    static_assert(4 * 64 * GG_PITCH <= 4 * GG_TILE_BYTES, "four per-wave patches fit the operand tiles");
+    uint8_t* const patch = gsm + wv * (64 * GG_PITCH);
+#pragma unroll
+    for (int mf = 0; mf < 2; mf++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int ml = 32 * mf + 8 * (r >> 2) + 4 * h + (r & 3);
+#pragma unroll
+        for (int nf = 0; nf < 2; nf++) *(__half*)(patch + ml * GG_PITCH + (32 * nf + n) * 2) = __float2half(acc[mf][nf][r]);
+      }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the wave's own writes
+    __builtin_amdgcn_wave_barrier();
+    const int c8 = lane & 7, col = nb * GG_BN + 64 * wn + 8 * c8;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      const int ml = 8 * it + (lane >> 3), m = wm * 64 + ml;
+      const uint4 v = *(const uint4*)(patch + ml * GG_PITCH + c8 * 16);
+      if (m < tile.count && col < M) *(uint4*)(out + (size_t)(tile.first + m) * M + col) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int mf = 0; mf < 2; mf++)
 #pragma unroll
@@ -846,6 +873,7 @@ int moe_launch_gemm_gg(bool up, int type, const uint8_t* w, const uint8_t* w_up,
   if (!moe_aligned(w, align_of(type)) || (up && !moe_aligned(w_up, align_of(type))) || !moe_aligned(x16, 16) ||
       (sh_w && (!moe_aligned(sh_w, align_of(tsh)) || (up && (!sh_w_up || !moe_aligned(sh_w_up, align_of(tsh)))))))
     return MOE_E_INVALID;
+  if (!up && (m % 8 || !moe_aligned(out, 16))) return MOE_E_UNSUPPORTED;  // (down results leave as 16-byte pieces)
   if (max_tiles == 0) return MOE_OK;
   GgGemmW R{w, w_up, type}, S{sh_w ? sh_w : w, sh_w ? sh_w_up : w_up, sh_w ? tsh : type};
   const dim3 grid((unsigned)(up ? (m + 63) / 64 : (m + GG_BN - 1) / GG_BN), (unsigned)max_tiles);
